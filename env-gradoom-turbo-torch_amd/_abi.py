@@ -1,0 +1,128 @@
+"""ctypes mirror of ``include/gradoom_amd.h`` (struct layouts and field order must match)."""
+
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+SCREEN_WIDTH = 320
+VIEW_HEIGHT = 208
+SCREEN_HEIGHT = 240
+OBS_SIZE = 84
+FRAME_STACK = 4
+
+GD_OK = 0
+GD_E_ARG = -1
+GD_E_HIP = -2
+GD_E_UNSUPPORTED = -3
+
+_P = C.c_void_p
+
+MAP_SCALARS = (
+    "wall_count",
+    "sector_count",
+    "vertex_count",
+    "texture_count",
+    "tex_max_h",
+    "tex_max_w",
+    "sprite_count",
+    "spr_max_h",
+    "spr_max_w",
+    "blocking_count",
+    "neighbor_slots",
+    "direct_neighbors",
+)
+
+# (field, numpy dtype) in header order
+MAP_ARRAYS = (
+    ("walls", np.float32),
+    ("walls_fixed", np.int32),
+    ("wall_sectors", np.int32),
+    ("wall_vertex", np.int32),
+    ("side_tex", np.int32),
+    ("side_off", np.float32),
+    ("wall_len", np.float32),
+    ("endpoint_neighbors", np.int32),
+    ("endpoint_neighbor_starts", np.uint8),
+    ("endpoint_neighbor_ends", np.uint8),
+    ("solid_bridge_start_ofs", np.int32),
+    ("solid_bridge_start_idx", np.int32),
+    ("solid_bridge_end_ofs", np.int32),
+    ("solid_bridge_end_idx", np.int32),
+    ("vertex_wall_ofs", np.int32),
+    ("vertex_wall_idx", np.int32),
+    ("sector_wall_ofs", np.int32),
+    ("sector_wall_idx", np.int32),
+    ("sector_edge_ofs", np.int32),
+    ("sector_edge_idx", np.int32),
+    ("blocking_walls", np.int32),
+    ("sector_heights", np.float32),
+    ("sector_lights", np.float32),
+    ("sector_floor_tex", np.int32),
+    ("sector_ceil_tex", np.int32),
+    ("tex_atlas", np.uint8),
+    ("tex_w", np.int32),
+    ("tex_h", np.int32),
+    ("playpal", np.uint8),
+    ("colormap", np.uint8),
+    ("spr_atlas", np.uint8),
+    ("spr_opaque", np.uint8),
+    ("spr_post_top", np.uint8),
+    ("spr_w", np.int32),
+    ("spr_h", np.int32),
+    ("spr_left", np.int32),
+    ("spr_top", np.int32),
+)
+
+LANE_ARRAYS = (
+    ("x", np.float32),
+    ("y", np.float32),
+    ("angle", np.float32),
+    ("view_z", np.float32),
+    ("x_fixed", np.int64),
+    ("y_fixed", np.int64),
+    ("angle_bam", np.int64),
+    ("pitch_bam", np.int64),
+    ("flash_light", np.int64),
+    ("ray_cos", np.float32),
+    ("ray_sin", np.float32),
+    ("sprite_x", np.float32),
+    ("sprite_y", np.float32),
+    ("sprite_z", np.float32),
+    ("sprite_depth", np.float32),
+    ("sprite_id", np.int32),
+    ("sprite_alive", np.uint8),
+    ("sprite_fullbright", np.uint8),
+)
+
+OUT_FIELDS = ("indexed", "obs", "frames", "reset_mask", "rgb")
+
+
+class MapDesc(C.Structure):
+    _fields_ = [(name, C.c_int32) for name in MAP_SCALARS] + [(name, _P) for name, _ in MAP_ARRAYS]
+
+
+class LanesDesc(C.Structure):
+    _fields_ = [("lane_count", C.c_int32), ("sprite_slots", C.c_int32)] + [(name, _P) for name, _ in LANE_ARRAYS]
+
+
+class FrameOut(C.Structure):
+    _fields_ = [(name, _P) for name in OUT_FIELDS]
+
+
+def host_map_desc(tables: dict) -> tuple[MapDesc, list]:
+    """Build a MapDesc of HOST pointers from ``mapbuild.build_map_tables`` output.
+
+    Returns the struct and the list of arrays that must stay alive while it is used.
+    """
+
+    desc = MapDesc()
+    keep = []
+    for name in MAP_SCALARS:
+        setattr(desc, name, int(tables[name]))
+    for name, dtype in MAP_ARRAYS:
+        array = np.ascontiguousarray(tables[name], dtype=dtype)
+        keep.append(array)
+        setattr(desc, name, array.ctypes.data)
+    return desc, keep

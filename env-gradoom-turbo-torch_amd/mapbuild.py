@@ -1,0 +1,197 @@
+"""Host-side derivation of the map tables the renderer consumes (NumPy only).
+
+Restates, in compact form, what the reference derives once per scenario in
+``DeviceScenario.from_host`` (``/root/reference/src/gradoom/engine.py:721-849``)
+and in ``TorchDeathmatchEngine.__init__`` (``engine.py:1527-1634``).  The
+reference's dense ``[W, W]`` / ``[2, W, W]`` tables do not scale to thousands of
+linedefs; here every pairwise relation is reduced to (a) vertex ids assigned by
+exact float32 equality of endpoints and (b) CSR adjacency lists, from which the
+kernels answer the same queries on the fly.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+
+FIXED_UNIT = 65536
+
+
+def _csr(rows: list[list[int]]) -> tuple[np.ndarray, np.ndarray]:
+    offsets = np.zeros(len(rows) + 1, dtype=np.int32)
+    for i, row in enumerate(rows):
+        offsets[i + 1] = offsets[i] + len(row)
+    flat = [v for row in rows for v in row]
+    return offsets, np.asarray(flat if flat else [0], dtype=np.int32)
+
+
+def build_map_tables(smap) -> dict[str, np.ndarray | int]:
+    """Return contiguous arrays keyed by the field names of ``gd_map_desc``."""
+
+    walls = np.ascontiguousarray(smap.wall_segments, dtype=np.float32)
+    wall_count = len(walls)
+    sectors = np.ascontiguousarray(smap.wall_sectors, dtype=np.int32)
+    sector_count = len(smap.sector_heights)
+    if wall_count == 0 or sector_count == 0:
+        raise ValueError("a map needs at least one linedef and one sector")
+    if np.abs(walls).max() >= 16384:
+        raise ValueError("map coordinates must stay below 16384 units (16.16 in int32)")
+
+    # rint(walls * 65536): engine.py:749-751 (float64) and engine.py:10876 (float32) agree
+    # whenever the product is exact, which the int32 range check above guarantees only for
+    # coordinates with <= 8 fractional bits; verify instead of assuming.
+    fixed32 = np.rint(walls * np.float32(FIXED_UNIT))
+    fixed64 = np.rint(walls.astype(np.float64) * FIXED_UNIT)
+    if not np.array_equal(fixed32.astype(np.float64), fixed64):
+        raise ValueError("linedef coordinates are not exactly representable in 16.16")
+    walls_fixed = fixed64.astype(np.int32)
+
+    # Vertex ids by exact float equality (-0.0 == 0.0), as engine.py:776-781 compares them.
+    vertex_ids: dict[tuple[float, float], int] = {}
+    wall_vertex = np.zeros((wall_count, 2), dtype=np.int32)
+    for w in range(wall_count):
+        for slot in range(2):
+            key = (float(walls[w, 2 * slot]) + 0.0, float(walls[w, 2 * slot + 1]) + 0.0)
+            wall_vertex[w, slot] = vertex_ids.setdefault(key, len(vertex_ids))
+    vertex_count = len(vertex_ids)
+    vertex_rows: list[list[int]] = [[] for _ in range(vertex_count)]
+    for w in range(wall_count):
+        for slot in range(2):
+            v = int(wall_vertex[w, slot])
+            if not vertex_rows[v] or vertex_rows[v][-1] != w:
+                vertex_rows[v].append(w)
+    vertex_wall_ofs, vertex_wall_idx = _csr(vertex_rows)
+
+    one_sided = sectors[:, 1] < 0
+
+    def same_pair(a: int, b: int) -> bool:
+        return (sectors[a, 0] == sectors[b, 0] and sectors[a, 1] == sectors[b, 1]) or (
+            sectors[a, 0] == sectors[b, 1] and sectors[a, 1] == sectors[b, 0]
+        )
+
+    def shares(a: int, slot: int, b: int) -> bool:
+        v = wall_vertex[a, slot]
+        return wall_vertex[b, 0] == v or wall_vertex[b, 1] == v
+
+    # Endpoint neighbours: same sector pair and a shared endpoint (engine.py:769-786, 831-849).
+    neighbor_rows: list[list[int]] = []
+    for w in range(wall_count):
+        near = set()
+        for slot in range(2):
+            v = int(wall_vertex[w, slot])
+            near.update(vertex_rows[v])
+        near.discard(w)
+        neighbor_rows.append(sorted(n for n in near if same_pair(w, n)))
+    slots = max(1, max(len(row) for row in neighbor_rows))
+    endpoint_neighbors = np.repeat(np.arange(wall_count, dtype=np.int32)[:, None], slots, axis=1)
+    neighbor_starts = np.zeros((wall_count, slots), dtype=np.uint8)
+    neighbor_ends = np.zeros((wall_count, slots), dtype=np.uint8)
+    for w, row in enumerate(neighbor_rows):
+        for k, n in enumerate(row):
+            endpoint_neighbors[w, k] = n
+            neighbor_starts[w, k] = shares(w, 0, n)
+            neighbor_ends[w, k] = shares(w, 1, n)
+    direct = bool(np.all(neighbor_starts.sum(axis=1) <= 1) and np.all(neighbor_ends.sum(axis=1) <= 1))
+
+    # One-hop solid bridges (engine.py:787-830): bridge[w] = { k : exists j one-sided,
+    # sharing w's start (resp. end), with sectors[j,0] in sectors[w], and k one-sided,
+    # k != j, sharing any endpoint with j, sectors[k,0] == sectors[j,0] }.
+    def solid_bridges(slot: int) -> list[list[int]]:
+        rows: list[list[int]] = []
+        for w in range(wall_count):
+            found = set()
+            for j in vertex_rows[int(wall_vertex[w, slot])]:
+                if not one_sided[j]:
+                    continue
+                if not (sectors[w, 0] == sectors[j, 0] or sectors[w, 1] == sectors[j, 0]):
+                    continue
+                for jslot in range(2):
+                    for k in vertex_rows[int(wall_vertex[j, jslot])]:
+                        if k != j and one_sided[k] and sectors[k, 0] == sectors[j, 0]:
+                            found.add(k)
+            rows.append(sorted(found))
+        return rows
+
+    solid_bridge_start_ofs, solid_bridge_start_idx = _csr(solid_bridges(0))
+    solid_bridge_end_ofs, solid_bridge_end_idx = _csr(solid_bridges(1))
+
+    sector_wall_rows: list[list[int]] = [[] for _ in range(sector_count)]
+    for w in range(wall_count):
+        front, back = int(sectors[w, 0]), int(sectors[w, 1])
+        if front >= 0:
+            sector_wall_rows[front].append(w)
+        if back >= 0 and back != front:
+            sector_wall_rows[back].append(w)
+    sector_wall_ofs, sector_wall_idx = _csr(sector_wall_rows)
+    edge_mask = np.asarray(smap.sector_edge_mask, dtype=bool)
+    sector_edge_ofs, sector_edge_idx = _csr([np.flatnonzero(edge_mask[s]).tolist() for s in range(sector_count)])
+
+    dx = walls[:, 2] - walls[:, 0]
+    dy = walls[:, 3] - walls[:, 1]
+    wall_len = np.floor(np.sqrt(np.square(dx) + np.square(dy)) + 0.5).astype(np.float32)
+
+    tex_atlas = np.ascontiguousarray(smap.texture_atlas, dtype=np.uint8)
+    tex_w = np.ascontiguousarray(smap.texture_widths, dtype=np.int32)
+    tex_h = np.ascontiguousarray(smap.texture_heights, dtype=np.int32)
+    for name, values in (("width", tex_w), ("height", tex_h)):
+        if np.any(values <= 0) or np.any(values & (values - 1)):
+            raise ValueError(f"texture {name}s must be powers of two")
+
+    spr_atlas = np.ascontiguousarray(smap.sprite_atlas, dtype=np.uint8)
+    spr_opaque = np.ascontiguousarray(smap.sprite_opaque, dtype=np.uint8)
+    # First source row of the opaque post containing each texel (engine.py:14230-14256).
+    prior = np.concatenate((np.zeros_like(spr_opaque[:, :1]), spr_opaque[:, :-1]), axis=1)
+    starts = (spr_opaque != 0) & (prior == 0)
+    rows = np.arange(spr_opaque.shape[1], dtype=np.int64)[None, :, None]
+    spr_post_top = np.maximum.accumulate(np.where(starts, rows, 0), axis=1).astype(np.uint8)
+
+    return dict(
+        wall_count=wall_count,
+        sector_count=sector_count,
+        vertex_count=vertex_count,
+        texture_count=int(tex_atlas.shape[0]),
+        tex_max_h=int(tex_atlas.shape[1]),
+        tex_max_w=int(tex_atlas.shape[2]),
+        sprite_count=int(spr_atlas.shape[0]),
+        spr_max_h=int(spr_atlas.shape[1]),
+        spr_max_w=int(spr_atlas.shape[2]),
+        blocking_count=int(len(smap.blocking_wall_indices)),
+        neighbor_slots=int(slots),
+        direct_neighbors=int(direct),
+        walls=walls,
+        walls_fixed=walls_fixed,
+        wall_sectors=sectors,
+        wall_vertex=wall_vertex,
+        side_tex=np.ascontiguousarray(smap.wall_side_texture_ids, dtype=np.int32),
+        side_off=np.ascontiguousarray(smap.wall_side_texture_offsets, dtype=np.float32),
+        wall_len=wall_len,
+        endpoint_neighbors=endpoint_neighbors,
+        endpoint_neighbor_starts=neighbor_starts,
+        endpoint_neighbor_ends=neighbor_ends,
+        solid_bridge_start_ofs=solid_bridge_start_ofs,
+        solid_bridge_start_idx=solid_bridge_start_idx,
+        solid_bridge_end_ofs=solid_bridge_end_ofs,
+        solid_bridge_end_idx=solid_bridge_end_idx,
+        vertex_wall_ofs=vertex_wall_ofs,
+        vertex_wall_idx=vertex_wall_idx,
+        sector_wall_ofs=sector_wall_ofs,
+        sector_wall_idx=sector_wall_idx,
+        sector_edge_ofs=sector_edge_ofs,
+        sector_edge_idx=sector_edge_idx,
+        blocking_walls=np.ascontiguousarray(smap.blocking_wall_indices, dtype=np.int32),
+        sector_heights=np.ascontiguousarray(smap.sector_heights, dtype=np.float32),
+        sector_lights=np.ascontiguousarray(smap.sector_lights).astype(np.float32),
+        sector_floor_tex=np.ascontiguousarray(smap.sector_floor_texture_ids, dtype=np.int32),
+        sector_ceil_tex=np.ascontiguousarray(smap.sector_ceiling_texture_ids, dtype=np.int32),
+        tex_atlas=tex_atlas,
+        tex_w=tex_w,
+        tex_h=tex_h,
+        playpal=np.ascontiguousarray(smap.playpal, dtype=np.uint8),
+        colormap=np.ascontiguousarray(smap.colormap, dtype=np.uint8),
+        spr_atlas=spr_atlas,
+        spr_opaque=spr_opaque,
+        spr_post_top=spr_post_top,
+        spr_w=np.ascontiguousarray(smap.sprite_widths, dtype=np.int32),
+        spr_h=np.ascontiguousarray(smap.sprite_heights, dtype=np.int32),
+        spr_left=np.ascontiguousarray(smap.sprite_left_offsets, dtype=np.int32),
+        spr_top=np.ascontiguousarray(smap.sprite_top_offsets, dtype=np.int32),
+    )

@@ -1,0 +1,369 @@
+"""Seeded synthetic maps, textures and camera poses for the batched renderer.
+
+The generator emits the subset of the reference's ``CompiledScenario`` schema
+that the native render path reads (``/root/reference/src/gradoom/scenario.py:302-401``):
+linedef segments with exact shared float32 vertices, per-side texture ids in
+(middle, bottom, top) order (``scenario.py:516``), sector heights/lights/flats,
+one shared ``[T, maxH, maxW]`` texture atlas with power-of-two sizes, PLAYPAL,
+COLORMAP and a raw sprite atlas.  Only NumPy is used so the same arrays can be
+fed to the reference (to write golden vectors), to the CPU oracle and to the
+HIP path.
+
+Map shape: a jittered grid of quadrilateral cells.  A seeded subset of cells
+is void (solid rock); every other cell is one sector.  An edge between two
+sectors is a two-sided linedef, an edge between a sector and void/outside is
+one-sided, and edges are split at exact dyadic points until the requested
+linedef count is reached.  The front sector (``wall_sectors[w, 0]``) lies to
+the right of the directed linedef, which is what makes a one-sided wall
+front-facing from inside its sector (``engine.py:10777-10780``).
+"""
+
+from __future__ import annotations
+
+import dataclasses
+import math
+
+import numpy as np
+
+CONFIGS = {
+    # name: lanes, grid, sectors, linedefs, sprites/lane, masked-midtex probability
+    "config1": dict(lanes=16, grid=(9, 6), sectors=48, linedefs=320, sprites=0, midtex=0.0),
+    "config2": dict(lanes=256, grid=(12, 9), sectors=96, linedefs=800, sprites=32, midtex=0.0),
+    "config3": dict(lanes=1024, grid=(15, 15), sectors=200, linedefs=2000, sprites=64, midtex=0.0),
+    "config4": dict(lanes=4096, grid=(21, 21), sectors=400, linedefs=4000, sprites=128, midtex=0.15),
+}
+
+CELL = 256.0
+JITTER = 40
+MAX_SPLIT_DEPTH = 3
+
+
+@dataclasses.dataclass
+class SynthMap:
+    """Host arrays of one synthetic scenario (names follow ``CompiledScenario``)."""
+
+    vertices: np.ndarray  # [V,2] f32
+    wall_segments: np.ndarray  # [W,4] f32 (x1,y1,x2,y2)
+    wall_sectors: np.ndarray  # [W,2] i32 (front, back or -1)
+    wall_side_texture_ids: np.ndarray  # [W,2,3] i32 (middle,bottom,top), -1 none
+    wall_side_texture_offsets: np.ndarray  # [W,2,2] f32
+    blocking_wall_indices: np.ndarray  # [B] i32
+    sector_edge_mask: np.ndarray  # [S,W] bool
+    sector_heights: np.ndarray  # [S,2] f32 (floor, ceiling)
+    sector_lights: np.ndarray  # [S] i16
+    sector_floor_texture_ids: np.ndarray  # [S] i32
+    sector_ceiling_texture_ids: np.ndarray  # [S] i32
+    texture_atlas: np.ndarray  # [T,maxH,maxW] u8
+    texture_widths: np.ndarray  # [T] i32
+    texture_heights: np.ndarray  # [T] i32
+    playpal: np.ndarray  # [256,3] u8
+    colormap: np.ndarray  # [34,256] u8
+    sprite_atlas: np.ndarray  # [P,maxH,maxW] u8, index 0 transparent
+    sprite_widths: np.ndarray  # [P] i32
+    sprite_heights: np.ndarray  # [P] i32
+    sprite_left_offsets: np.ndarray  # [P] i32
+    sprite_top_offsets: np.ndarray  # [P] i32
+    sector_cells: np.ndarray  # [S,2] i32 grid cell of each sector (generator bookkeeping)
+    grid_points: np.ndarray  # [gy+1,gx+1,2] f32 jittered grid vertices
+
+    @property
+    def blocking_segments(self) -> np.ndarray:
+        return self.wall_segments[self.blocking_wall_indices]
+
+    @property
+    def sprite_opaque(self) -> np.ndarray:
+        return self.sprite_atlas != 0
+
+
+@dataclasses.dataclass
+class Poses:
+    """Per-lane camera state, in the reference engine's own tensors' dtypes."""
+
+    x: np.ndarray  # [N] f32
+    y: np.ndarray  # [N] f32
+    angle_bam: np.ndarray  # [N] i64, unsigned 32-bit BAM
+    pitch_bam: np.ndarray  # [N] i64
+    view_z: np.ndarray  # [N] f32
+    flash_light: np.ndarray  # [N] i64 in {0,1,2}
+    sector: np.ndarray  # [N] i32 sector the pose was drawn in (bookkeeping)
+
+
+@dataclasses.dataclass
+class Sprites:
+    """Packed per-lane billboard list (the renderer's sprite input)."""
+
+    x: np.ndarray  # [N,A] f32
+    y: np.ndarray  # [N,A] f32
+    z: np.ndarray  # [N,A] f32
+    sprite: np.ndarray  # [N,A] i32 patch id
+    alive: np.ndarray  # [N,A] bool
+    fullbright: np.ndarray  # [N,A] bool
+
+
+def _split_edges(rng, edges, target):
+    """Split ``edges`` (list of (p, q, front, back, depth)) at midpoints up to ``target``."""
+
+    edges = list(edges)
+    if len(edges) > target:
+        raise ValueError(f"grid already has {len(edges)} linedefs, more than the {target} asked for")
+    while len(edges) < target:
+        order = rng.permutation(len(edges))
+        progressed = False
+        for index in order:
+            if len(edges) >= target:
+                break
+            p, q, front, back, depth = edges[index]
+            if depth >= MAX_SPLIT_DEPTH:
+                continue
+            mid = ((p[0] + q[0]) / 2.0, (p[1] + q[1]) / 2.0)
+            edges[index] = (p, mid, front, back, depth + 1)
+            edges.append((mid, q, front, back, depth + 1))
+            progressed = True
+        if not progressed:
+            raise ValueError("cannot reach the requested linedef count at the split depth limit")
+    return edges
+
+
+def generate_map(
+    seed: int,
+    *,
+    grid: tuple[int, int],
+    sectors: int,
+    linedefs: int,
+    midtex: float = 0.0,
+    wall_textures: int = 64,
+    flats: int = 16,
+    sprite_patches: int = 64,
+) -> SynthMap:
+    rng = np.random.default_rng(seed)
+    gx, gy = grid
+    if sectors > gx * gy:
+        raise ValueError("more sectors than grid cells")
+    origin_x = -gx * CELL / 2.0
+    origin_y = -gy * CELL / 2.0
+    points = np.zeros((gy + 1, gx + 1, 2), dtype=np.float64)
+    for j in range(gy + 1):
+        for i in range(gx + 1):
+            points[j, i, 0] = origin_x + i * CELL + int(rng.integers(-JITTER, JITTER + 1))
+            points[j, i, 1] = origin_y + j * CELL + int(rng.integers(-JITTER, JITTER + 1))
+
+    # Choose which cells are void; every other cell becomes a sector in row-major order.
+    cell_sector = np.full((gy, gx), -1, dtype=np.int64)
+    void = np.zeros(gy * gx, dtype=bool)
+    void[rng.permutation(gy * gx)[: gy * gx - sectors]] = True
+    sector_cells = []
+    for j in range(gy):
+        for i in range(gx):
+            if not void[j * gx + i]:
+                cell_sector[j, i] = len(sector_cells)
+                sector_cells.append((i, j))
+
+    def sector_of(i, j):
+        if 0 <= i < gx and 0 <= j < gy:
+            return int(cell_sector[j, i])
+        return -1
+
+    # Cells are counter-clockwise quads, so the interior is on the LEFT of each
+    # directed boundary edge; a linedef wants its front sector on the RIGHT,
+    # hence every edge is emitted reversed relative to its front cell.
+    edges = []
+
+    def add_edge(p, q, left_sector, right_sector):
+        # left/right relative to the direction p->q.
+        if left_sector < 0 and right_sector < 0:
+            return
+        if right_sector < 0:
+            p, q, left_sector, right_sector = q, p, right_sector, left_sector
+        elif left_sector >= 0 and rng.random() < 0.5:
+            p, q, left_sector, right_sector = q, p, right_sector, left_sector
+        edges.append((tuple(p), tuple(q), right_sector, left_sector, 0))
+
+    for j in range(gy + 1):
+        for i in range(gx):
+            # horizontal edge from (i,j) to (i+1,j): cell above (j) is on the left, below (j-1) on the right
+            add_edge(points[j, i], points[j, i + 1], sector_of(i, j), sector_of(i, j - 1))
+    for j in range(gy):
+        for i in range(gx + 1):
+            # vertical edge from (i,j) to (i,j+1): cell (i-1) is on the left, cell (i) on the right
+            add_edge(points[j, i], points[j + 1, i], sector_of(i - 1, j), sector_of(i, j))
+
+    edges = _split_edges(rng, edges, linedefs)
+    order = rng.permutation(len(edges))
+    edges = [edges[k] for k in order]
+    wall_count = len(edges)
+    wall_segments = np.asarray([(p[0], p[1], q[0], q[1]) for p, q, *_ in edges], dtype=np.float32)
+    wall_sectors = np.asarray([(f, b) for _p, _q, f, b, _d in edges], dtype=np.int32)
+    assert np.all(wall_segments.astype(np.float64) * 8 == np.round(wall_segments.astype(np.float64) * 8))
+    vertices = np.unique(wall_segments.reshape(-1, 2), axis=0).astype(np.float32)
+
+    sector_count = len(sector_cells)
+    floors = rng.integers(0, 13, sector_count) * 8.0
+    ceilings = 160.0 + rng.integers(0, 13, sector_count) * 8.0
+    sector_heights = np.stack((floors, ceilings), axis=1).astype(np.float32)
+    sector_lights = rng.integers(96, 256, sector_count).astype(np.int16)
+    sector_floor_texture_ids = (wall_textures + rng.integers(0, flats, sector_count)).astype(np.int32)
+    sector_ceiling_texture_ids = (wall_textures + rng.integers(0, flats, sector_count)).astype(np.int32)
+
+    side_ids = np.full((wall_count, 2, 3), -1, dtype=np.int32)
+    side_offsets = np.zeros((wall_count, 2, 2), dtype=np.float32)
+    for w in range(wall_count):
+        one_sided = wall_sectors[w, 1] < 0
+        for side in range(1 if one_sided else 2):
+            side_offsets[w, side] = rng.integers(0, 64, 2)
+            if one_sided:
+                side_ids[w, side, 0] = rng.integers(0, wall_textures)
+            else:
+                side_ids[w, side, 1] = rng.integers(0, wall_textures)
+                side_ids[w, side, 2] = rng.integers(0, wall_textures)
+                if midtex > 0.0 and rng.random() < midtex:
+                    side_ids[w, side, 0] = rng.integers(0, wall_textures)
+
+    sector_edge_mask = np.zeros((sector_count, wall_count), dtype=bool)
+    for w in range(wall_count):
+        front, back = wall_sectors[w]
+        if front == back:
+            continue
+        sector_edge_mask[front, w] = True
+        if back >= 0:
+            sector_edge_mask[back, w] = True
+
+    texture_total = wall_textures + flats
+    atlas = np.zeros((texture_total, 128, 64), dtype=np.uint8)
+    atlas[:wall_textures] = rng.integers(0, 256, (wall_textures, 128, 64), dtype=np.uint8)
+    atlas[wall_textures:, :64, :] = rng.integers(0, 256, (flats, 64, 64), dtype=np.uint8)
+    texture_widths = np.full(texture_total, 64, dtype=np.int32)
+    texture_heights = np.concatenate(
+        (np.full(wall_textures, 128, dtype=np.int32), np.full(flats, 64, dtype=np.int32))
+    )
+    playpal = rng.integers(0, 256, (256, 3), dtype=np.uint8)
+    colormap = rng.integers(0, 256, (34, 256), dtype=np.uint8)
+
+    sprite_widths = rng.integers(32, 65, sprite_patches).astype(np.int32)
+    sprite_heights = rng.integers(32, 65, sprite_patches).astype(np.int32)
+    sprite_atlas = np.zeros((sprite_patches, 64, 64), dtype=np.uint8)
+    for p in range(sprite_patches):
+        w, h = int(sprite_widths[p]), int(sprite_heights[p])
+        patch = rng.integers(0, 256, (h, w), dtype=np.uint8)
+        # Carve transparent holes so posts start below row 0 in some columns.
+        holes = rng.random((h, w)) < 0.2
+        patch[holes] = 0
+        sprite_atlas[p, :h, :w] = patch
+    sprite_left_offsets = (sprite_widths // 2).astype(np.int32)
+    sprite_top_offsets = sprite_heights.astype(np.int32)
+
+    return SynthMap(
+        vertices=vertices,
+        wall_segments=wall_segments,
+        wall_sectors=wall_sectors,
+        wall_side_texture_ids=side_ids,
+        wall_side_texture_offsets=side_offsets,
+        blocking_wall_indices=np.flatnonzero(wall_sectors[:, 1] < 0).astype(np.int32),
+        sector_edge_mask=sector_edge_mask,
+        sector_heights=sector_heights,
+        sector_lights=sector_lights,
+        sector_floor_texture_ids=sector_floor_texture_ids,
+        sector_ceiling_texture_ids=sector_ceiling_texture_ids,
+        texture_atlas=atlas,
+        texture_widths=texture_widths,
+        texture_heights=texture_heights,
+        playpal=playpal,
+        colormap=colormap,
+        sprite_atlas=sprite_atlas,
+        sprite_widths=sprite_widths,
+        sprite_heights=sprite_heights,
+        sprite_left_offsets=sprite_left_offsets,
+        sprite_top_offsets=sprite_top_offsets,
+        sector_cells=np.asarray(sector_cells, dtype=np.int32),
+        grid_points=points.astype(np.float32),
+    )
+
+
+def generate_config_map(name: str, seed: int | None = None) -> SynthMap:
+    cfg = CONFIGS[name]
+    if seed is None:
+        seed = 1000 + int(name[-1])
+    return generate_map(
+        seed,
+        grid=cfg["grid"],
+        sectors=cfg["sectors"],
+        linedefs=cfg["linedefs"],
+        midtex=cfg["midtex"],
+    )
+
+
+def _point_in_cell(smap: SynthMap, sector: int, u: float, v: float) -> tuple[float, float]:
+    i, j = smap.sector_cells[sector]
+    p00 = smap.grid_points[j, i].astype(np.float64)
+    p10 = smap.grid_points[j, i + 1].astype(np.float64)
+    p01 = smap.grid_points[j + 1, i].astype(np.float64)
+    p11 = smap.grid_points[j + 1, i + 1].astype(np.float64)
+    point = (1 - u) * (1 - v) * p00 + u * (1 - v) * p10 + (1 - u) * v * p01 + u * v * p11
+    # 1/16 map unit keeps the float32 value and its 16.16 image both exact.
+    return float(np.round(point[0] * 16) / 16), float(np.round(point[1] * 16) / 16)
+
+
+def generate_poses(
+    smap: SynthMap,
+    lanes: int,
+    seed: int,
+    *,
+    pitch: bool = False,
+    flash: bool = False,
+    frame: int = 0,
+) -> Poses:
+    """Random camera poses strictly inside sectors (bilinear margin keeps them off the walls)."""
+
+    x = np.zeros(lanes, dtype=np.float32)
+    y = np.zeros(lanes, dtype=np.float32)
+    angle_bam = np.zeros(lanes, dtype=np.int64)
+    pitch_bam = np.zeros(lanes, dtype=np.int64)
+    view_z = np.zeros(lanes, dtype=np.float32)
+    flash_light = np.zeros(lanes, dtype=np.int64)
+    sector = np.zeros(lanes, dtype=np.int32)
+    sector_count = len(smap.sector_heights)
+    for lane in range(lanes):
+        rng = np.random.default_rng((seed * 65536 + lane) * 4096 + frame)
+        s = int(rng.integers(0, sector_count))
+        u, v = rng.uniform(0.15, 0.85, 2)
+        px, py = _point_in_cell(smap, s, float(u), float(v))
+        x[lane], y[lane] = px, py
+        angle_bam[lane] = int(rng.integers(0, 1 << 32))
+        view_z[lane] = smap.sector_heights[s, 0] + 41.0
+        if pitch:
+            pitch_bam[lane] = int(rng.integers(-10, 11)) * (182 << 16)
+        if flash:
+            flash_light[lane] = int(rng.integers(0, 3))
+        sector[lane] = s
+    return Poses(x, y, angle_bam, pitch_bam, view_z, flash_light, sector)
+
+
+def generate_sprites(smap: SynthMap, lanes: int, count: int, seed: int, frame: int = 0) -> Sprites:
+    """Random billboards standing on sector floors; depths are distinct with probability one."""
+
+    shape = (lanes, max(count, 0))
+    x = np.zeros(shape, dtype=np.float32)
+    y = np.zeros(shape, dtype=np.float32)
+    z = np.zeros(shape, dtype=np.float32)
+    sprite = np.zeros(shape, dtype=np.int32)
+    alive = np.zeros(shape, dtype=bool)
+    fullbright = np.zeros(shape, dtype=bool)
+    sector_count = len(smap.sector_heights)
+    patches = len(smap.sprite_widths)
+    for lane in range(lanes):
+        rng = np.random.default_rng(((seed + 7919) * 65536 + lane) * 4096 + frame)
+        for a in range(count):
+            s = int(rng.integers(0, sector_count))
+            u, v = rng.uniform(0.1, 0.9, 2)
+            px, py = _point_in_cell(smap, s, float(u), float(v))
+            x[lane, a], y[lane, a] = px, py
+            z[lane, a] = smap.sector_heights[s, 0]
+            sprite[lane, a] = int(rng.integers(0, patches))
+            alive[lane, a] = rng.random() < 0.9
+            fullbright[lane, a] = rng.random() < 0.1
+    return Sprites(x, y, z, sprite, alive, fullbright)
+
+
+def bam_to_radians_f32(angle_bam: np.ndarray) -> np.ndarray:
+    """float32 view angle the reference derives from a retained BAM (``engine.py:10651``)."""
+
+    return (angle_bam.astype(np.float32) * np.float32(2.0 * math.pi / float(1 << 32))).astype(np.float32)

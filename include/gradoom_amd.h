@@ -1,0 +1,182 @@
+/*
+ * gradoom_amd.h - C ABI of the MI355X (gfx950) batched software renderer and
+ * observation pipeline that replaces the reference's Torch "reference" render
+ * path behind GraDoomVecEnv (reset_device / step_and_reset_device / render).
+ *
+ * Every pointer in gd_map_desc / gd_lanes_desc / gd_frame_out is a DEVICE
+ * pointer when passed to the gd_* entry points of libgradoom_amd.so, and a
+ * HOST pointer when the same structs are handed to the CPU oracle
+ * (liboracle.so, test infrastructure only).  The structs themselves live in
+ * host memory.  Entry points return 0 on success or a negative GD_E_* code;
+ * gd_last_error() returns a message for the calling thread.
+ *
+ * Names follow the reference's domain: lanes (batched environments), linedefs
+ * ("walls"), sectors, flats, visplanes, drawsegs, sprites, PLAYPAL, COLORMAP.
+ */
+#ifndef GRADOOM_AMD_H
+#define GRADOOM_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GD_SCREEN_WIDTH 320
+#define GD_VIEW_HEIGHT 208   /* world view rows; rows 208..239 are the status bar */
+#define GD_SCREEN_HEIGHT 240
+#define GD_OBS_SIZE 84
+#define GD_FRAME_STACK 4
+
+#define GD_OK 0
+#define GD_E_ARG (-1)       /* bad argument: null pointer, negative count, size over a limit */
+#define GD_E_HIP (-2)       /* a HIP runtime call failed */
+#define GD_E_UNSUPPORTED (-3) /* the map needs a feature this build does not implement */
+
+/*
+ * Immutable map, atlases and look-up tables.
+ * Mirrors the tensors of DeviceScenario (reference src/gradoom/engine.py:607-719)
+ * that the native render path reads, plus compact forms of the derived tables
+ * the reference builds in DeviceScenario.from_host (engine.py:721-849) and in
+ * TorchDeathmatchEngine.__init__ (engine.py:1527-1634).  The reference's dense
+ * [W,W] and [2,W,W] pair/bridge tables are replaced by a vertex -> linedef CSR
+ * from which the same answers are derived on the fly.
+ */
+typedef struct gd_map_desc {
+    int32_t wall_count;      /* W linedefs */
+    int32_t sector_count;    /* S */
+    int32_t vertex_count;    /* V distinct endpoints (exact float32 equality) */
+    int32_t texture_count;   /* T */
+    int32_t tex_max_h, tex_max_w;
+    int32_t sprite_count;    /* P raw sprite patches */
+    int32_t spr_max_h, spr_max_w;
+    int32_t blocking_count;  /* B one-sided / blocking linedefs */
+    int32_t neighbor_slots;  /* K columns of endpoint_neighbors */
+    int32_t direct_neighbors;/* 1: every linedef has <=1 start and <=1 end neighbour (engine.py:1558) */
+
+    const float *walls;              /* [W,4] x1,y1,x2,y2 (portal_walls) */
+    const int32_t *walls_fixed;      /* [W,4] rint(walls*65536) (engine.py:10876) */
+    const int32_t *wall_sectors;     /* [W,2] front, back (-1 = one-sided) */
+    const int32_t *wall_vertex;      /* [W,2] vertex id of start, end */
+    const int32_t *side_tex;         /* [W,2,3] middle,bottom,top texture id or -1 */
+    const float *side_off;           /* [W,2,2] x,y texture offsets */
+    const float *wall_len;           /* [W] floor(len+0.5) (engine.py:737-743) */
+    const int32_t *endpoint_neighbors;      /* [W,K] (engine.py:833-849), self where unused */
+    const uint8_t *endpoint_neighbor_starts;/* [W,K] */
+    const uint8_t *endpoint_neighbor_ends;  /* [W,K] */
+    const int32_t *solid_bridge_start_ofs;  /* [W+1] CSR of engine.py:802-830 */
+    const int32_t *solid_bridge_start_idx;
+    const int32_t *solid_bridge_end_ofs;    /* [W+1] */
+    const int32_t *solid_bridge_end_idx;
+    const int32_t *vertex_wall_ofs;  /* [V+1] CSR vertex -> linedefs touching it, ascending */
+    const int32_t *vertex_wall_idx;
+    const int32_t *sector_wall_ofs;  /* [S+1] CSR sector -> linedefs with that sector on either side */
+    const int32_t *sector_wall_idx;
+    const int32_t *sector_edge_ofs;  /* [S+1] CSR rows of sector_edge_mask (scenario.py:906-916) */
+    const int32_t *sector_edge_idx;
+    const int32_t *blocking_walls;   /* [B] linedef index of each blocking segment, ascending */
+
+    const float *sector_heights;     /* [S,2] floor, ceiling */
+    const float *sector_lights;      /* [S] */
+    const int32_t *sector_floor_tex; /* [S] */
+    const int32_t *sector_ceil_tex;  /* [S] */
+
+    const uint8_t *tex_atlas;        /* [T,tex_max_h,tex_max_w] palette indices */
+    const int32_t *tex_w;            /* [T] power of two */
+    const int32_t *tex_h;            /* [T] power of two */
+    const uint8_t *playpal;          /* [256,3] */
+    const uint8_t *colormap;         /* [34,256] */
+
+    const uint8_t *spr_atlas;        /* [P,spr_max_h,spr_max_w] */
+    const uint8_t *spr_opaque;       /* [P,spr_max_h,spr_max_w] 0/1 */
+    const uint8_t *spr_post_top;     /* [P,spr_max_h,spr_max_w] first row of the opaque run (engine.py:14230) */
+    const int32_t *spr_w, *spr_h, *spr_left, *spr_top; /* [P] */
+} gd_map_desc;
+
+/*
+ * Per-lane camera and sprite list for one frame.
+ * x,y,angle,view_z and the retained fixed-point twins are the engine tensors
+ * of the same names (engine.py:1669, 10648-10687).  ray_cos/ray_sin are
+ * cos/sin(angle + native_ray_offsets) (engine.py:10966-10974) and sprite_depth
+ * is dist*cos(wrap(atan2 - angle)) (engine.py:14684-14688): the host computes
+ * these float32 transcendentals with the same Torch ops the reference uses so
+ * the kernels only do +,-,*,/ and comparisons.
+ */
+typedef struct gd_lanes_desc {
+    int32_t lane_count;       /* N */
+    int32_t sprite_slots;     /* A sprites per lane (0 = none) */
+    const float *x, *y;       /* [N] */
+    const float *angle;       /* [N] radians */
+    const float *view_z;      /* [N] */
+    const int64_t *x_fixed, *y_fixed; /* [N] retained 16.16 */
+    const int64_t *angle_bam; /* [N] retained unsigned 32-bit BAM */
+    const int64_t *pitch_bam; /* [N] */
+    const int64_t *flash_light; /* [N] extralight steps (x16) */
+    const float *ray_cos, *ray_sin; /* [N,320] */
+    const float *sprite_x, *sprite_y, *sprite_z; /* [N,A] */
+    const float *sprite_depth;       /* [N,A] */
+    const int32_t *sprite_id;        /* [N,A] */
+    const uint8_t *sprite_alive;     /* [N,A] */
+    const uint8_t *sprite_fullbright;/* [N,A] */
+} gd_lanes_desc;
+
+/* Output buffers; any pointer may be null to skip that product. */
+typedef struct gd_frame_out {
+    uint8_t *indexed;   /* [N,240,320] palette indices; rows 208..239 = 0 (empty status bar) */
+    uint8_t *obs;       /* [N,84,84] grayscale policy frame (HUD rows masked black) */
+    uint8_t *frames;    /* [N,4,84,84] stack, oldest first: rolled by one and obs appended */
+    const uint8_t *reset_mask; /* [N] or null: lanes whose stack is filled with 4 copies instead */
+    uint8_t *rgb;       /* [N,240,320,3] PLAYPAL expansion of `indexed` */
+} gd_frame_out;
+
+typedef struct gd_renderer gd_renderer;
+
+/* library identification; replaces nothing in the reference */
+const char *gd_version(void);
+const char *gd_last_error(void);
+
+/*
+ * Upload an immutable map (host pointers in `host_map`) to the current HIP
+ * device and size per-lane scratch for `max_lanes`.
+ * Replaces DeviceScenario.from_host + the engine ctor precompute
+ * (engine.py:721-1476, 1527-1634).
+ */
+int gd_renderer_create(const gd_map_desc *host_map, int32_t max_lanes, gd_renderer **out);
+void gd_renderer_destroy(gd_renderer *r);
+
+/*
+ * Render one frame for every lane on `stream` (a hipStream_t, may be null).
+ * All gd_lanes_desc / gd_frame_out pointers are device pointers.
+ * Replaces TorchDeathmatchEngine._render_native_indexed_frame (engine.py:15338-15379)
+ * + render_reference_frame (engine.py:15436-15451) + _finish_observation
+ * (engine.py:9545-9548) / the reset stack fill (engine.py:2443-2450)
+ * + _native_indexed_to_rgb (engine.py:15381-15398, flashes off).
+ * No allocation, no host synchronisation.
+ */
+int gd_render(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_out *out, void *stream);
+
+/*
+ * Observation pipeline alone on an existing indexed frame.
+ * Replaces policy_area_grayscale (_triton_kernels.py:120-203) fused with the
+ * frame-stack update (engine.py:9545-9548, 2443-2450).
+ * indexed: [N,source_rows,320] with source_rows 208 or 240; rows >= source_rows are black.
+ */
+int gd_observe(const uint8_t *indexed, int32_t source_rows, const uint8_t *playpal, int32_t lane_count,
+               uint8_t *obs, uint8_t *frames, const uint8_t *reset_mask, void *stream);
+
+/* PLAYPAL expansion [N,rows,320] -> [N,rows,320,3]; replaces engine.py:15381-15384. */
+int gd_expand_rgb24(const uint8_t *indexed, int32_t rows, const uint8_t *playpal, int32_t lane_count,
+                    uint8_t *rgb, void *stream);
+
+/*
+ * Time `launches` back-to-back gd_render launches with HIP events on `stream`
+ * and return the average milliseconds per launch of each kernel stage in
+ * ms[0..stage_count).  Measurement helper for the benchmark; replaces nothing.
+ */
+int gd_render_timed(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_out *out, void *stream,
+                    int32_t launches, float *ms, int32_t stage_count);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GRADOOM_AMD_H */

@@ -1,0 +1,118 @@
+"""Drive the reference's Torch CPU render path on synthetic maps (build container only).
+
+The reference package cannot be imported as ``gradoom`` here because its
+``__init__``/``env`` modules need ``gymnasium``; the render path itself lives in
+``gradoom.engine`` + ``gradoom.scenario`` which only need torch/numpy.  This
+module registers an empty parent package whose ``__path__`` points at the
+reference sources and imports just those two modules.  It is used only by
+``make_golden.py`` to write fixtures; nothing on the GPU box imports it.
+"""
+
+from __future__ import annotations
+
+import importlib
+import os
+import sys
+import types
+
+import numpy as np
+import torch
+
+REFERENCE_SRC = os.environ.get("GRADOOM_REFERENCE_SRC", "/root/reference/src/gradoom")
+
+
+def load_reference():
+    if "gradoom.engine" in sys.modules:
+        return sys.modules["gradoom.engine"], sys.modules["gradoom.scenario"]
+    if not os.path.isdir(REFERENCE_SRC):
+        raise RuntimeError(f"reference sources not found at {REFERENCE_SRC}")
+    parent = types.ModuleType("gradoom")
+    parent.__path__ = [REFERENCE_SRC]
+    sys.modules["gradoom"] = parent
+    scenario = importlib.import_module("gradoom.scenario")
+    engine = importlib.import_module("gradoom.engine")
+    return engine, scenario
+
+
+def to_compiled_scenario(smap, *, flash_lights: bool = False):
+    """Wrap a SynthMap in the reference's CompiledScenario (``scenario.py:302-401``)."""
+
+    _engine, scenario = load_reference()
+    wall_count = len(smap.wall_segments)
+    sprite_count = len(smap.sprite_widths)
+    # enemy types 0..5 x 4 walk frames x 8 rotations address up to 192 patches
+    # (engine.py:14073); drops use raw_static_sprite_ids[12] (engine.py:14657-14660).
+    enemy_walk = (np.arange(6 * 4 * 8, dtype=np.int32) % sprite_count).reshape(6, 4, 8)
+    raw_static = (np.arange(32, dtype=np.int32) * 5 + 3) % sprite_count
+    kwargs = {}
+    if flash_lights:
+        lights = np.zeros((8, 2, 52), dtype=np.int64)
+        lights[:, :, 1] = 1
+        lights[:, :, 2] = 2
+        kwargs["native_weapon_flash_lights"] = lights
+    return scenario.CompiledScenario(
+        scenario_sha256="s" * 64,
+        iwad_sha256="i" * 64,
+        namespace="zdoom",
+        vertices=smap.vertices,
+        wall_segments=smap.wall_segments,
+        blocking_segments=smap.blocking_segments.copy(),
+        blocking_wall_indices=smap.blocking_wall_indices,
+        wall_texture_ids=np.zeros(wall_count, dtype=np.int32),
+        wall_texture_offsets=np.zeros((wall_count, 2), dtype=np.float32),
+        wall_side_texture_ids=smap.wall_side_texture_ids,
+        wall_side_texture_offsets=smap.wall_side_texture_offsets,
+        wall_sectors=smap.wall_sectors,
+        sector_edge_mask=smap.sector_edge_mask,
+        sector_heights=smap.sector_heights,
+        sector_lights=smap.sector_lights,
+        sector_floor_texture_ids=smap.sector_floor_texture_ids,
+        sector_ceiling_texture_ids=smap.sector_ceiling_texture_ids,
+        player_starts=np.asarray([(float(smap.vertices[0, 0]), float(smap.vertices[0, 1]), 0.0)], dtype=np.float32),
+        item_spawns=np.empty((0, 3), dtype=np.float32),
+        item_types=np.empty((0,), dtype=np.int32),
+        playpal=smap.playpal,
+        texture_names=tuple(f"T{i}" for i in range(len(smap.texture_widths))),
+        texture_atlas=smap.texture_atlas,
+        texture_widths=smap.texture_widths,
+        texture_heights=smap.texture_heights,
+        sprite_names=tuple(f"S{i}" for i in range(sprite_count)),
+        sprite_atlas=smap.sprite_atlas,
+        sprite_opaque=smap.sprite_opaque,
+        sprite_widths=smap.sprite_widths,
+        sprite_heights=smap.sprite_heights,
+        sprite_left_offsets=smap.sprite_left_offsets,
+        sprite_top_offsets=smap.sprite_top_offsets,
+        weapon_sprite_names=tuple(f"W{i}" for i in range(8)),
+        weapon_screen_values=np.zeros((8, 84, 84), dtype=np.float32),
+        weapon_screen_alpha=np.zeros((8, 84, 84), dtype=np.float32),
+        colormap=smap.colormap,
+        enemy_walk_sprite_ids=enemy_walk,
+        raw_static_sprite_ids=raw_static,
+        **kwargs,
+    )
+
+
+def make_engine(smap, lanes: int, *, flash_lights: bool = False):
+    engine_module, _scenario = load_reference()
+    compiled = to_compiled_scenario(smap, flash_lights=flash_lights)
+    return engine_module.TorchDeathmatchEngine(compiled, lanes, device=torch.device("cpu"))
+
+
+def set_poses(engine, poses) -> None:
+    """Overwrite the per-lane camera like the reference's own tests do (tests/test_rendering.py:388-393)."""
+
+    engine_module, _ = load_reference()
+    bam = torch.as_tensor(poses.angle_bam, dtype=torch.int64)
+    engine._angle_bam.copy_(bam)
+    engine.angle.copy_(bam.to(torch.float32) * engine_module._BAM_TO_RADIANS)
+    engine.x.copy_(torch.as_tensor(poses.x))
+    engine.y.copy_(torch.as_tensor(poses.y))
+    engine._x_fixed.copy_(torch.round(engine.x * 65536).to(torch.int64))
+    engine._y_fixed.copy_(torch.round(engine.y * 65536).to(torch.int64))
+    engine._pitch_bam.copy_(torch.as_tensor(poses.pitch_bam, dtype=torch.int64))
+    engine.view_z.copy_(torch.as_tensor(poses.view_z))
+    # flash_light = native_weapon_flash_lights[weapon, parity, cooldown] (engine.py:14949-14967)
+    engine.weapon_state_cooldown.copy_(
+        torch.as_tensor(poses.flash_light).to(engine.weapon_state_cooldown.dtype)
+    )
