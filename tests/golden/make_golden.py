@@ -1,0 +1,166 @@
+"""Write golden vectors from the reference's own Torch CPU render path (build container only).
+
+Usage:  python tests/golden/make_golden.py [--only NAME ...] [--time]
+
+For each case below a seeded synthetic map and pose set is built with
+``synthmap``, rendered by the reference (``/root/reference/src/gradoom/engine.py``,
+imported through ``refdrive``), and the inputs + outputs are stored as
+``tests/golden/fixtures/<name>.npz``:
+
+* lane inputs exactly as ``gd_lanes_desc`` wants them (including the Torch
+  float32 ray tables and sprite depths, so nothing on the GPU box needs the
+  reference or a particular Torch CPU build);
+* ``indexed``  uint8 [N,240,320]  ``_render_native_indexed_frame(include_hud=True)`` (engine.py:15338)
+* ``obs``      uint8 [N,84,84]    ``render_reference_frame()`` CPU float path (engine.py:15436)
+* for ``stages`` cases, lane 0 intermediates of every pipeline stage
+  (geometry, intersections, PrepWall, flats, depth / sprite-clip buffers).
+
+The map itself is regenerated from its seed at test time; ``map_sha256`` guards
+against generator drift.
+"""
+
+from __future__ import annotations
+
+import argparse
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, HERE)
+
+import __graft_entry__ as entry  # noqa: E402
+
+entry.load_package()
+from gradoom_amd import hostmath, synthmap  # noqa: E402
+
+import refdrive  # noqa: E402
+from make_golden_meta import map_digest  # noqa: E402
+
+FIXTURES = os.path.join(HERE, "fixtures")
+
+# name -> generator arguments. Every case is a distinct (map seed, pose seed).
+CASES = {
+    "tiny_stages": dict(map_seed=7, grid=(4, 3), sectors=10, linedefs=48, lanes=4, pose_seed=1, stages=True),
+    "small_pitch": dict(map_seed=11, grid=(4, 3), sectors=10, linedefs=60, lanes=8, pose_seed=1, pitch=True),
+    "small_flash": dict(map_seed=12, grid=(5, 4), sectors=17, linedefs=100, lanes=8, pose_seed=1, flash=True),
+    "small_midtex_sprites": dict(
+        map_seed=22, grid=(6, 5), sectors=26, linedefs=160, lanes=8, pose_seed=1, sprites=128, flash=True,
+        pitch=True, midtex=0.2, stages=True,
+    ),
+    "config1": dict(map_seed=1001, grid=(9, 6), sectors=48, linedefs=320, lanes=16, pose_seed=1),
+    "config1_pitch_flash": dict(
+        map_seed=1001, grid=(9, 6), sectors=48, linedefs=320, lanes=8, pose_seed=2, pitch=True, flash=True
+    ),
+    "config1_midtex": dict(map_seed=2001, grid=(9, 6), sectors=48, linedefs=320, lanes=8, pose_seed=3, midtex=0.2),
+    "config2_subset": dict(map_seed=1002, grid=(12, 9), sectors=96, linedefs=800, lanes=4, pose_seed=1, sprites=32),
+    "config3_subset": dict(
+        map_seed=1003, grid=(15, 15), sectors=200, linedefs=2000, lanes=2, pose_seed=1, sprites=64, flash=True
+    ),
+    "config4_subset": dict(
+        map_seed=1004, grid=(21, 21), sectors=400, linedefs=4000, lanes=2, pose_seed=1, sprites=128, midtex=0.15
+    ),
+}
+
+
+def build_case(name: str, cfg: dict, do_time: bool) -> dict:
+    smap = synthmap.generate_map(
+        cfg["map_seed"], grid=cfg["grid"], sectors=cfg["sectors"], linedefs=cfg["linedefs"], midtex=cfg.get("midtex", 0.0)
+    )
+    lanes = cfg["lanes"]
+    started = time.time()
+    engine = refdrive.make_engine(smap, lanes, flash_lights=cfg.get("flash", False))
+    ctor_seconds = time.time() - started
+    poses = synthmap.generate_poses(
+        smap, lanes, cfg["pose_seed"], pitch=cfg.get("pitch", False), flash=cfg.get("flash", False)
+    )
+    refdrive.set_poses(engine, poses)
+    offsets = hostmath.native_ray_offsets("cpu")
+    assert torch.equal(offsets, engine._native_ray_offsets)
+    ray_cos, ray_sin = hostmath.ray_tables(engine.angle, offsets)
+    data = dict(
+        x=engine.x.numpy().copy(), y=engine.y.numpy().copy(), angle=engine.angle.numpy().copy(),
+        view_z=engine.view_z.numpy().copy(), x_fixed=engine._x_fixed.numpy().copy(),
+        y_fixed=engine._y_fixed.numpy().copy(), angle_bam=engine._angle_bam.numpy().copy(),
+        pitch_bam=engine._pitch_bam.numpy().copy(), flash_light=np.asarray(poses.flash_light, dtype=np.int64),
+        ray_cos=ray_cos.numpy(), ray_sin=ray_sin.numpy(),
+        cosine_correction=hostmath.cosine_correction("cpu").numpy(),
+    )
+    if cfg.get("sprites", 0):
+        sprites = synthmap.generate_sprites(smap, lanes, cfg["sprites"], cfg["pose_seed"])
+        packed = refdrive.set_sprites(engine, sprites, cfg["pose_seed"])
+        data.update(packed)
+        data["sprite_depth"] = hostmath.sprite_depth(
+            engine.x, engine.y, engine.angle, torch.as_tensor(packed["sprite_x"]), torch.as_tensor(packed["sprite_y"])
+        ).numpy()
+    started = time.time()
+    with torch.no_grad():
+        indexed = engine._render_native_indexed_frame(include_hud=True)
+        obs = engine.render_reference_frame()
+        rgb_lane0 = engine.render_native_frame(include_hud=True)[0]
+    render_seconds = time.time() - started
+    data["indexed"] = indexed.numpy()
+    data["obs"] = obs.numpy()
+    data["rgb_lane0"] = rgb_lane0.numpy()
+    if cfg.get("stages", False):
+        with torch.no_grad():
+            geometry = engine._native_wall_projection_geometry()
+            inter = engine._native_portal_intersections(geometry)
+            hoff, vstep = engine._native_wall_texture_mapping()
+            sector = engine._current_sector()
+            flats, surface, scene_surface = engine._native_render_flats(sector, engine.view_z)
+            walls, scene_depth, clip_depth, clip_wall = engine._native_render_portal_walls(
+                flats, engine.view_z, surface, scene_surface
+            )
+        data.update(
+            st_sector=sector.numpy().astype(np.int32),
+            st_geometry=torch.stack(geometry, dim=-1)[0].numpy(),
+            st_distances=inter[0][0].numpy(), st_along=inter[1][0].numpy(), st_geometric=inter[2][0].numpy(),
+            st_projected=inter[3][0].numpy(), st_left_edge=inter[4][0].numpy(), st_visibility=inter[5][0].numpy(),
+            st_hoff=hoff[0].numpy(), st_vstep=vstep[0].numpy(), st_flats=flats[0].numpy(),
+            st_surface_depth=surface[0].numpy(), st_scene_surface_depth=scene_surface[0].numpy(),
+            st_walls=walls[0].numpy(), st_scene_depth=scene_depth[0].numpy(), st_clip_depth=clip_depth[0].numpy(),
+            st_clip_wall=clip_wall[0].numpy().astype(np.int32),
+        )
+    timing = None
+    if do_time:
+        # The CPU-baseline protocol: full indexed frame + observation + stack update per lane.
+        torch.set_num_threads(os.cpu_count())
+        samples = []
+        for _ in range(3):
+            started = time.time()
+            with torch.no_grad():
+                engine._finish_observation(engine.render_reference_frame())
+            samples.append(lanes / (time.time() - started))
+        timing = float(np.median(samples))
+    meta = dict(cfg)
+    meta["map_sha256"] = map_digest(smap)
+    data["meta"] = np.asarray(repr(meta))
+    print(
+        f"{name}: W={cfg['linedefs']} S={cfg['sectors']} lanes={lanes} ctor {ctor_seconds:.1f}s render {render_seconds:.1f}s"
+        + (f" reference CPU {timing:.3f} lane-frames/s on {os.cpu_count()} cores" if timing else ""),
+        flush=True,
+    )
+    return data
+
+
+def main() -> None:
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--only", nargs="*", default=None)
+    parser.add_argument("--time", action="store_true")
+    args = parser.parse_args()
+    os.makedirs(FIXTURES, exist_ok=True)
+    for name, cfg in CASES.items():
+        if args.only and name not in args.only:
+            continue
+        data = build_case(name, cfg, args.time)
+        np.savez_compressed(os.path.join(FIXTURES, f"{name}.npz"), **data)
+
+
+if __name__ == "__main__":
+    main()

@@ -116,3 +116,76 @@ def set_poses(engine, poses) -> None:
     engine.weapon_state_cooldown.copy_(
         torch.as_tensor(poses.flash_light).to(engine.weapon_state_cooldown.dtype)
     )
+
+
+def set_sprites(engine, sprites, seed: int):
+    """Place billboards through the enemy and drop slots (engine.py:14328-14343, 14657-14682).
+
+    Slots [0, 64) of ``sprites`` go to enemy slots, [64, 128) to drop slots.  The
+    patch id an enemy shows depends on its type, walk frame and viewing rotation
+    (engine.py:14011-14077); this function randomises those and then asks the
+    reference which patch, fullbright flag and packed order result, returning the
+    packed per-lane list the renderer consumes (engine.py:14684 onward).
+    """
+
+    count = sprites.x.shape[1]
+    lanes = sprites.x.shape[0]
+    enemy_count = min(count, engine.enemy_slots)
+    drop_count = min(max(count - enemy_count, 0), engine.enemy_slots)
+    generator = torch.Generator().manual_seed(seed)
+    if enemy_count:
+        sl = slice(0, enemy_count)
+        engine.enemy_x[:, sl] = torch.as_tensor(sprites.x[:, :enemy_count])
+        engine.enemy_y[:, sl] = torch.as_tensor(sprites.y[:, :enemy_count])
+        engine.enemy_z[:, sl] = torch.as_tensor(sprites.z[:, :enemy_count])
+        engine.enemy_alive[:, sl] = torch.as_tensor(sprites.alive[:, :enemy_count])
+        engine.enemy_type[:, sl] = torch.randint(0, 6, (lanes, enemy_count), generator=generator)
+        engine.enemy_angle[:, sl] = torch.rand((lanes, enemy_count), generator=generator) * 6.25
+        engine.enemy_animation_tics[:, sl] = torch.randint(
+            0, 64, (lanes, enemy_count), generator=generator
+        ).to(engine.enemy_animation_tics.dtype)
+        # type 3 in attack phase 2/3 is a BRIGHT state (engine.py:14125-14136)
+        bright = torch.as_tensor(sprites.fullbright[:, :enemy_count])
+        engine.enemy_type[:, sl] = torch.where(bright, torch.full_like(engine.enemy_type[:, sl], 3), engine.enemy_type[:, sl])
+        engine.enemy_attack_phase[:, sl] = torch.where(
+            bright, torch.full_like(engine.enemy_attack_phase[:, sl], 3), torch.zeros_like(engine.enemy_attack_phase[:, sl])
+        )
+    if drop_count:
+        src = slice(enemy_count, enemy_count + drop_count)
+        sl = slice(0, drop_count)
+        engine.drop_x[:, sl] = torch.as_tensor(sprites.x[:, src])
+        engine.drop_y[:, sl] = torch.as_tensor(sprites.y[:, src])
+        engine.drop_z[:, sl] = torch.as_tensor(sprites.z[:, src])
+        engine.drop_type[:, sl] = torch.where(torch.as_tensor(sprites.alive[:, src]), 2001, -1)
+        engine.drop_spawned[:, sl] = True
+    return packed_sprites(engine)
+
+
+def packed_sprites(engine):
+    """Replay the reference's slot trimming and concatenation order for enemies and drops."""
+
+    enemy_sprite = engine._native_enemy_sprite_ids()
+    enemy_slots = torch.nonzero(torch.any(engine.enemy_alive, dim=0)).flatten()
+    enemy_type = engine.enemy_type[:, enemy_slots].clamp(0, 5)
+    fullbright = engine._native_enemy_fullbright(
+        enemy_type,
+        engine.enemy_attack_phase[:, enemy_slots],
+        engine.enemy_cooldown[:, enemy_slots],
+        engine._enemy_attack_recovery[enemy_type],
+    )
+    drop_visible = (engine.drop_type >= 0) & engine.drop_spawned
+    static = engine.map.raw_static_sprite_ids
+    drop_sprite = static[12].expand_as(engine.drop_type)
+    drop_sprite = torch.where(engine.drop_type == 2007, static[6], drop_sprite)
+    drop_sprite = torch.where(engine.drop_type == 2002, static[14], drop_sprite)
+    drop_slots = torch.nonzero(torch.any(drop_visible, dim=0)).flatten()
+    return dict(
+        sprite_x=torch.cat((engine.enemy_x[:, enemy_slots], engine.drop_x[:, drop_slots]), dim=1).numpy(),
+        sprite_y=torch.cat((engine.enemy_y[:, enemy_slots], engine.drop_y[:, drop_slots]), dim=1).numpy(),
+        sprite_z=torch.cat((engine.enemy_z[:, enemy_slots], engine.drop_z[:, drop_slots]), dim=1).numpy(),
+        sprite_id=torch.cat((enemy_sprite[:, enemy_slots], drop_sprite[:, drop_slots]), dim=1).numpy().astype(np.int32),
+        sprite_alive=torch.cat((engine.enemy_alive[:, enemy_slots], drop_visible[:, drop_slots]), dim=1).numpy(),
+        sprite_fullbright=torch.cat(
+            (fullbright, torch.zeros_like(drop_visible[:, drop_slots])), dim=1
+        ).numpy(),
+    )

@@ -1,0 +1,73 @@
+"""The CPU oracle against golden vectors written by the reference's own Torch path."""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+
+from conftest import fixture_names, lane_inputs, load_fixture
+
+# Cases whose oracle run takes more than a few seconds on the CPU are trimmed to a lane subset.
+LANE_LIMIT = {"config3_subset": 1, "config4_subset": 1}
+
+
+@pytest.mark.parametrize("name", fixture_names())
+def test_indexed_frame_bit_exact_and_observation_within_one(oracle, name):
+    meta, data, _smap, tables = load_fixture(name)
+    lanes = min(meta["lanes"], LANE_LIMIT.get(name, meta["lanes"]))
+    result = oracle.render(tables, lane_inputs(data), data["cosine_correction"], lane_range=(0, lanes))
+    assert np.array_equal(result["indexed"][:lanes], data["indexed"][:lanes])
+    # rows 208..239: empty status bar on synthetic maps (engine.py:15232-15267 with a zero HUD atlas)
+    assert not result["indexed"][:lanes, 208:].any()
+    # The reference CPU path pools in float32 matmuls; the oracle uses the exact integer
+    # form of the reference's GPU branch. Tolerance from tests/test_rendering.py:138-139.
+    delta = np.abs(result["obs"][:lanes].astype(np.int32) - data["obs"][:lanes].astype(np.int32))
+    assert delta.max() <= 1
+    assert delta.mean() < 0.01
+
+
+@pytest.mark.parametrize("name", [n for n in fixture_names() if "stages" in n or n == "small_midtex_sprites"])
+def test_every_stage_matches_reference_intermediates(oracle, name):
+    _meta, data, _smap, tables = load_fixture(name)
+    if "st_geometry" not in data:
+        pytest.skip("fixture carries no stage taps")
+    result = oracle.render(tables, lane_inputs(data), data["cosine_correction"], lane_range=(0, 1), debug_lane=0)
+    taps = result["debug"]
+    assert result["sector"][0] == data["st_sector"][0]
+
+    def same(ours, ref):
+        ours = np.asarray(ours)
+        ref = np.asarray(ref)
+        if ours.dtype.kind == "f":
+            return bool(np.all((ours == ref) | (np.isnan(ours) & np.isnan(ref))))
+        return bool(np.array_equal(ours, ref))
+
+    assert same(taps["geometry"], data["st_geometry"])
+    assert same(taps["distances"], data["st_distances"])
+    assert same(taps["along"], data["st_along"])
+    assert same(taps["geometric"].astype(bool), data["st_geometric"])
+    assert same(taps["projected"].astype(bool), data["st_projected"])
+    assert same(taps["left_edge"].astype(bool), data["st_left_edge"])
+    assert same(taps["visibility"], data["st_visibility"])
+    assert same(taps["horizontal_offset"], data["st_hoff"])
+    assert same(taps["vertical_step"], data["st_vstep"])
+    assert same(taps["flats_frame"], data["st_flats"])
+    assert same(taps["surface_depth"], data["st_surface_depth"])
+    assert same(taps["scene_surface_depth"], data["st_scene_surface_depth"])
+    assert same(taps["walls_frame"], data["st_walls"])
+    assert same(taps["scene_depth"], data["st_scene_depth"])
+    assert same(taps["sprite_clip_depth"], data["st_clip_depth"])
+    assert same(taps["sprite_clip_wall"], data["st_clip_wall"])
+
+
+def test_sprites_are_actually_drawn_in_the_sprite_fixtures(oracle):
+    _meta, data, _smap, tables = load_fixture("small_midtex_sprites")
+    result = oracle.render(tables, lane_inputs(data), data["cosine_correction"], lane_range=(0, 1), debug_lane=0)
+    changed = int((result["debug"]["walls_frame"] != result["indexed"][0, :208]).sum())
+    assert changed > 200, "sprite layer changed too few pixels for the parity check to mean anything"
+
+
+def test_rgb_expansion_matches_reference(oracle):
+    _meta, data, _smap, tables = load_fixture("tiny_stages")
+    result = oracle.render(tables, lane_inputs(data), data["cosine_correction"], lane_range=(0, 1), want_rgb=True)
+    assert np.array_equal(result["rgb"][0], data["rgb_lane0"])
