@@ -32,7 +32,12 @@ MAP_SCALARS = (
     "blocking_count",
     "neighbor_slots",
     "direct_neighbors",
+    "floor_level_count",
+    "ceil_level_count",
+    "grid_nx",
+    "grid_ny",
 )
+MAP_FLOATS = ("grid_min_x", "grid_min_y", "grid_cell")
 
 # (field, numpy dtype) in header order
 MAP_ARRAYS = (
@@ -57,6 +62,12 @@ MAP_ARRAYS = (
     ("sector_edge_ofs", np.int32),
     ("sector_edge_idx", np.int32),
     ("blocking_walls", np.int32),
+    ("grid_cell_ofs", np.int32),
+    ("grid_item_sector", np.int32),
+    ("grid_item_edge_ofs", np.int32),
+    ("grid_item_edges", np.int32),
+    ("floor_levels", np.float32),
+    ("ceil_levels", np.float32),
     ("sector_heights", np.float32),
     ("sector_lights", np.float32),
     ("sector_floor_tex", np.int32),
@@ -100,7 +111,11 @@ OUT_FIELDS = ("indexed", "obs", "frames", "reset_mask", "rgb")
 
 
 class MapDesc(C.Structure):
-    _fields_ = [(name, C.c_int32) for name in MAP_SCALARS] + [(name, _P) for name, _ in MAP_ARRAYS]
+    _fields_ = (
+        [(name, C.c_int32) for name in MAP_SCALARS]
+        + [(name, C.c_float) for name in MAP_FLOATS]
+        + [(name, _P) for name, _ in MAP_ARRAYS]
+    )
 
 
 class LanesDesc(C.Structure):
@@ -121,6 +136,8 @@ def host_map_desc(tables: dict) -> tuple[MapDesc, list]:
     keep = []
     for name in MAP_SCALARS:
         setattr(desc, name, int(tables[name]))
+    for name in MAP_FLOATS:
+        setattr(desc, name, float(tables[name]))
     for name, dtype in MAP_ARRAYS:
         array = np.ascontiguousarray(tables[name], dtype=dtype)
         keep.append(array)

@@ -1,0 +1,1900 @@
+// MI355X (gfx950) batched software renderer + observation pipeline.
+//
+// One frame for N lanes runs as a short chain of kernels on one stream:
+//
+//   lane_setup     1 thread / lane          view basis, pitch centre, camera sector
+//   wall_setup     1 thread / (lane, wall)  FWallCoords span+depths, span ownership bounds
+//   column_lists   1 thread / (lane, col)   ray x visible-linedef test -> per-column candidate list
+//   flat_select    1 thread / pixel         nearest floor/ceiling sector through the point grid
+//   flat_finish    320 threads / lane       visplane repair (wave ballots) + flat shading
+//   wall_columns   320 threads / lane       portal traversal, tiers, planes, masked mid-textures
+//   sprite_columns 320 threads / lane       billboards far -> near
+//   observe        1 thread / obs pixel     PLAYPAL + exact area pool + gray + 4-frame stack
+//
+// All fixed-point arithmetic is int64 like the reference's Torch code; float32
+// expressions are evaluated operation by operation (-ffp-contract=off) so that
+// palette-index frames are bit-identical to the reference.  Citations name
+// /root/reference/src/gradoom/engine.py unless stated otherwise.
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "../../include/gradoom_amd.h"
+
+namespace {
+
+typedef long long i64;
+typedef unsigned long long u64;
+
+#define SW 320
+#define VH 208
+#define CAND_MAX 64          // candidate linedefs kept per screen column
+#define GD_INF __builtin_inff()
+
+// engine.py:42-51, 139-156
+#define FIXED_UNIT 65536LL
+#define UINT32_MASK 0xFFFFFFFFLL
+#define FINE_ANGLES 8192
+#define ANGLE_90 (1LL << 30)
+#define FOCAL_X_FIXED (160LL * 65536LL)
+#define Y_ASPECT_FIXED ((320LL * 65536LL * 240LL) / (200LL * 320LL))
+#define FOCAL_Y_FIXED (160LL * Y_ASPECT_FIXED)
+#define FLOOR_VISIBILITY_FIXED ((160LL * 65536LL * (8LL * 65536LL)) / FOCAL_Y_FIXED)
+#define WALL_VISIBILITY_FIXED (((FOCAL_Y_FIXED * (320LL * 600LL) / (320LL * 240LL * 3LL)) * (8LL * 65536LL)) >> 16)
+#define SPRITE_MIN_DEPTH_FIXED 8192LL
+
+// candidate flags
+#define CF_GEO 1
+#define CF_PROJ 2
+#define CF_LEDGE 4
+
+// wall record flags
+#define WF_HC 1        // owns at least one column after every span test
+#define WF_FF 2        // front facing (float32 test of engine.py:11376-11381)
+#define WF_SUBPIXEL 4  // two-sided and at most one column wide (engine.py:11589-11591)
+#define WF_ANYGEO 8    // some column ray hits the segment
+
+struct LaneCtx {
+    float x, y, view_z, pitch_offset, fsin, fcos;
+    i64 view_x_fixed, view_y_fixed, vsin, vcos, center_fixed, flash_light;
+    int sector;
+    int visible_count;
+};
+
+struct WallRec {   // one linedef seen from one lane
+    int tx0, tx1, ty0, ty1;  // view-space endpoints, start then end (engine.py:11173-11205)
+    i64 dl, dr;              // clipped endpoint depths (engine.py:10835-10852)
+    i64 sl, sr;              // clipped half-open screen span (engine.py:10825-10868); a rejected
+                             // linedef keeps whatever its projection produced, hence 64 bits
+    short pl, pr;            // span used for ray ownership (engine.py:11347-11427), within [0, 320]
+    int flags;
+};
+
+struct Cand {      // one linedef with a finite ray distance at one column
+    int wall;
+    float dist, along;
+    int flags;
+};
+
+struct DeviceMap {  // device copy of gd_map_desc (device pointers) + fixed tables
+    gd_map_desc d;
+    const i64 *fine_sine;     // [8192]
+    const i64 *fine_tangent;  // [4096]
+    const float *cosine_correction;  // [320] cos(native_ray_offsets), supplied by the host
+};
+
+struct Scratch {    // per-chunk working memory, sized at create
+    LaneCtx *ctx;          // [L]
+    WallRec *rec;          // [L,W]
+    int *visible;          // [L,W] compact list of linedefs that can own a column
+    Cand *cand;            // [L,CAND_MAX,320]
+    unsigned char *cand_count;  // [L,320]
+    unsigned short *flat_sector;// [L,208,320]
+    unsigned char *flat_flags;  // [L,208,320] bit0 unresolved
+    unsigned int *meta;    // [L,208,320] filled | floor | plane_sector+1 | clip_wall+1
+    float *clip_depth;     // [L,208,320]
+    unsigned char *frame;  // [L,240,320] when the caller wants no indexed output
+    int *status;           // [1] sticky overflow flags
+};
+
+#define META_FILLED 0x80000000u
+#define META_FLOOR 0x40000000u
+#define META_SECTOR_SHIFT 16
+#define META_SECTOR_MASK 0x3FFFu
+#define META_WALL_MASK 0xFFFFu
+
+#define STATUS_CAND_OVERFLOW 1
+
+__device__ __forceinline__ i64 mul64(i64 a, i64 b) { return (i64)((u64)a * (u64)b); }
+__device__ __forceinline__ i64 shl64(i64 a, int s) { return (i64)((u64)a << s); }
+__device__ __forceinline__ i64 tdiv(i64 a, i64 b) { return a / b; }
+__device__ __forceinline__ i64 clampi(i64 v, i64 lo, i64 hi) { return v < lo ? lo : (v > hi ? hi : v); }
+__device__ __forceinline__ i64 max64(i64 a, i64 b) { return a > b ? a : b; }
+__device__ __forceinline__ i64 min64(i64 a, i64 b) { return a < b ? a : b; }
+__device__ __forceinline__ i64 round_to_i64(float v) { return (i64)rintf(v); }
+__device__ __forceinline__ i64 f64_to_i64(double v) {
+    // Torch's CPU cast (x86 cvttsd2si): out of range or NaN -> INT64_MIN
+    if (!(v >= -9223372036854775808.0 && v < 9223372036854775808.0)) return (i64)0x8000000000000000ULL;
+    return (i64)v;
+}
+__device__ __forceinline__ int ilog2(int v) { return 31 - __clz(v); }
+__device__ __forceinline__ bool finitef(float v) { return fabsf(v) < GD_INF; }
+__device__ __forceinline__ float tolerance_of(float d) { return fmaxf(fabsf(d) / 128.0f, 4.0f); }
+
+// ---------------------------------------------------------------------------------------------
+// map relations (engine.py:399-484, 1578-1612), answered from vertex ids and the vertex CSR
+// ---------------------------------------------------------------------------------------------
+struct MapView {
+    const gd_map_desc *m;
+    __device__ int sec(int w, int side) const { return m->wall_sectors[2 * w + side]; }
+    __device__ int vert(int w, int slot) const { return m->wall_vertex[2 * w + slot]; }
+    __device__ bool one_sided(int w) const { return m->wall_sectors[2 * w + 1] < 0; }
+    __device__ bool two_sided_distinct(int w) const { return sec(w, 0) >= 0 && sec(w, 1) >= 0 && sec(w, 0) != sec(w, 1); }
+    __device__ bool same_pair(int a, int b) const {
+        int a0 = sec(a, 0), a1 = sec(a, 1), b0 = sec(b, 0), b1 = sec(b, 1);
+        return (a0 == b0 && a1 == b1) || (a0 == b1 && a1 == b0);
+    }
+    __device__ bool shares_any_endpoint(int a, int b) const {
+        int a0 = vert(a, 0), a1 = vert(a, 1), b0 = vert(b, 0), b1 = vert(b, 1);
+        return a0 == b0 || a0 == b1 || a1 == b0 || a1 == b1;
+    }
+    __device__ bool opposing(int a, int b) const {
+        if (!same_pair(a, b) || sec(a, 1) < 0 || sec(b, 1) < 0 || shares_any_endpoint(a, b)) return false;
+        const float *wa = m->walls + 4 * a, *wb = m->walls + 4 * b;
+        float ax = wa[2] - wa[0], ay = wa[3] - wa[1], bx = wb[2] - wb[0], by = wb[3] - wb[1];
+        float dot = ax * bx + ay * by;
+        float cross = ax * by - ay * bx;
+        return dot < 0 && fabsf(cross) < 1e-6f;
+    }
+    __device__ bool triangle_bridge(int vertex, int a, int b, int *index) const {
+        *index = 0;
+        if (!two_sided_distinct(a) || !two_sided_distinct(b)) return false;
+        int a0 = sec(a, 0), a1 = sec(a, 1), b0 = sec(b, 0), b1 = sec(b, 1);
+        int shared_count = (a0 == b0 || a0 == b1) + (a1 == b0 || a1 == b1);
+        if (shared_count != 1) return false;
+        int shared = (a0 == b0 || a0 == b1) ? a0 : a1;
+        int pa = (a0 == shared) ? a1 : a0;
+        int pb = (b0 == shared) ? b1 : b0;
+        int found = -1, count = 0;
+        for (int k = m->vertex_wall_ofs[vertex]; k < m->vertex_wall_ofs[vertex + 1]; ++k) {
+            int w = m->vertex_wall_idx[k];
+            if (w == a || w == b) continue;
+            int s0 = sec(w, 0), s1 = sec(w, 1);
+            if ((s0 == pa && s1 == pb) || (s0 == pb && s1 == pa)) { found = w; ++count; }
+        }
+        if (count != 1) return false;
+        *index = found;
+        return true;
+    }
+    __device__ bool portal_bridge(int slot, int path, int owner, int *index) const {
+        *index = 0;
+        if (owner == path) return false;
+        int v = vert(path, slot);
+        if (vert(owner, 0) != v && vert(owner, 1) != v) return false;
+        return triangle_bridge(v, path, owner, index);
+    }
+    __device__ bool sector_bridge(int slot, int pending, int path, int *index) const {
+        *index = 0;
+        if (path == pending) return false;
+        return triangle_bridge(vert(pending, slot), pending, path, index);
+    }
+};
+
+// Even-odd parity of one sector's edge sub-list around a point (engine.py:9598-9612, 10994-11015).
+__device__ __forceinline__ bool inside_edges(const gd_map_desc *m, int e0, int e1, float px, float py) {
+    int crossings = 0;
+    for (int k = e0; k < e1; ++k) {
+        const float4 e = *reinterpret_cast<const float4 *>(m->walls + 4 * m->grid_item_edges[k]);
+        float dy = e.w - e.y;
+        float safe_dy = fabsf(dy) < 1e-6f ? 1.0f : dy;
+        bool crosses = (e.y > py) != (e.w > py);
+        float crossing_x = e.x + (py - e.y) * (e.z - e.x) / safe_dy;
+        crossings += (crosses && px < crossing_x) ? 1 : 0;
+    }
+    return crossings & 1;
+}
+
+// Cell of the point grid, or -1 when no sector can contain the point.
+__device__ __forceinline__ int grid_cell_of(const gd_map_desc *m, float px, float py) {
+    float fx = floorf((px - m->grid_min_x) / m->grid_cell);
+    float fy = floorf((py - m->grid_min_y) / m->grid_cell);
+    if (!(fy >= 0.0f) || !(fy < (float)m->grid_ny) || !(fx < (float)m->grid_nx)) return -1;
+    int ix = fx < 0.0f ? 0 : (int)fx;   // column 0 also stands for everything left of the grid
+    if (!(fx == fx)) return -1;
+    return (int)fy * m->grid_nx + ix;
+}
+
+// _sector_at (engine.py:9598-9617): first sector with odd parity, 0 when none
+__device__ int sector_at(const gd_map_desc *m, float px, float py) {
+    int cell = grid_cell_of(m, px, py);
+    if (cell < 0) return 0;
+    for (int it = m->grid_cell_ofs[cell]; it < m->grid_cell_ofs[cell + 1]; ++it) {
+        if (inside_edges(m, m->grid_item_edge_ofs[it], m->grid_item_edge_ofs[it + 1], px, py)) return m->grid_item_sector[it];
+    }
+    return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// lane_setup: engine.py:10648-10658, 2122-2133, 9622-9631, 12384-12391, 9619
+// ---------------------------------------------------------------------------------------------
+__global__ void lane_setup_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
+    int local = blockIdx.x * blockDim.x + threadIdx.x;
+    if (local >= lane_count) return;
+    int n = lane_base + local;
+    const float BAM_TO_RADIANS = (float)(2.0 * 3.14159265358979323846 / 4294967296.0);
+    LaneCtx c;
+    c.x = lanes.x[n]; c.y = lanes.y[n]; c.view_z = lanes.view_z[n];
+    float angle = lanes.angle[n];
+    i64 pitch_bam = lanes.pitch_bam[n];
+    c.flash_light = lanes.flash_light ? lanes.flash_light[n] : 0;
+    i64 retained_bam = lanes.angle_bam[n];
+    float visible_angle = (float)retained_bam * BAM_TO_RADIANS;
+    i64 angle_bam = retained_bam;
+    if (angle != visible_angle) {
+        float two_pi = (float)(2.0 * 3.14159265358979323846);
+        float r = fmodf(angle, two_pi);
+        if (r != 0.0f && (r < 0.0f)) r += two_pi;   // torch.remainder with a positive divisor
+        angle_bam = round_to_i64(r / BAM_TO_RADIANS) & UINT32_MASK;
+    }
+    i64 xf = lanes.x_fixed[n], yf = lanes.y_fixed[n];
+    float visible_x = (float)xf / 65536.0f, visible_y = (float)yf / 65536.0f;
+    c.view_x_fixed = (c.x != visible_x) ? round_to_i64(c.x * 65536.0f) : xf;
+    c.view_y_fixed = (c.y != visible_y) ? round_to_i64(c.y * 65536.0f) : yf;
+    int fine = (int)((angle_bam >> 19) & (FINE_ANGLES - 1));
+    c.vsin = dm.fine_sine[fine];
+    c.vcos = dm.fine_sine[(fine + FINE_ANGLES / 4) & (FINE_ANGLES - 1)];
+    c.fsin = (float)c.vsin / 65536.0f;
+    c.fcos = (float)c.vcos / 65536.0f;
+    i64 tangent_index = clampi((ANGLE_90 - pitch_bam) >> 19, 0, FINE_ANGLES / 2 - 1);
+    i64 tangent = dm.fine_tangent[tangent_index];
+    c.center_fixed = (i64)(VH / 2) * FIXED_UNIT + ((FOCAL_Y_FIXED * tangent) >> 16);
+    c.pitch_offset = (float)((tangent * 12582912LL) >> 16) / 65536.0f;
+    c.sector = sector_at(&dm.d, c.x, c.y);
+    c.visible_count = 0;
+    sc.ctx[local] = c;
+}
+
+__device__ __forceinline__ void ray_direction(const LaneCtx &c, int x, float *rx, float *ry) {
+    // engine.py:10660-10670
+    float col = ((float)x - 160.0f) / 160.0f;
+    *rx = c.fcos + c.fsin * col;
+    *ry = c.fsin - c.fcos * col;
+}
+
+// ---------------------------------------------------------------------------------------------
+// wall_setup: engine.py:10747-10869 (FWallCoords) and the per-linedef half of 11304-11451
+// ---------------------------------------------------------------------------------------------
+__global__ void wall_setup_kernel(DeviceMap dm, int lane_count, Scratch sc) {
+    const gd_map_desc *m = &dm.d;
+    int w = blockIdx.x * blockDim.x + threadIdx.x;
+    int local = blockIdx.y;
+    if (w >= m->wall_count || local >= lane_count) return;
+    const LaneCtx &c = sc.ctx[local];
+    const int *wf = m->walls_fixed + 4 * w;
+    i64 rx0 = (i64)wf[0] - c.view_x_fixed, ry0 = (i64)wf[1] - c.view_y_fixed;
+    i64 rx1 = (i64)wf[2] - c.view_x_fixed, ry1 = (i64)wf[3] - c.view_y_fixed;
+    i64 tx0 = (rx0 * c.vsin - ry0 * c.vcos) >> 20, ty0 = (rx0 * c.vcos + ry0 * c.vsin) >> 20;
+    i64 tx1v = (rx1 * c.vsin - ry1 * c.vcos) >> 20, ty1v = (rx1 * c.vcos + ry1 * c.vsin) >> 20;
+    i64 vx = (i64)wf[2] - wf[0], vy = (i64)wf[3] - wf[1];
+    i64 fx = c.view_x_fixed - wf[0], fy = c.view_y_fixed - wf[1];
+    bool front = (vx * fy - vy * fx) < 0;
+    i64 tx1 = front ? tx0 : tx1v, tx2 = front ? tx1v : tx0;
+    i64 ty1 = front ? ty0 : ty1v, ty2 = front ? ty1v : ty0;
+    const i64 center = 160 * FIXED_UNIT;
+    i64 safe_ty1 = ty1 == 0 ? 1 : ty1, safe_ty2 = ty2 == 0 ? 1 : ty2;
+    i64 left_projected = ((center + tdiv(tx1 * center, safe_ty1)) >> 16) + (tx1 >= 0);
+    if (tx1 >= 0) left_projected = min64(left_projected, SW);
+    i64 right_projected = ((center + tdiv(tx2 * center, safe_ty2)) >> 16) + (tx2 >= 0);
+    if (tx2 >= 0) right_projected = min64(right_projected, SW);
+    i64 left_den = tx1 - tx2 - ty2 + ty1, right_den = ty2 - ty1 - tx2 + tx1;
+    i64 safe_left_den = left_den == 0 ? 1 : left_den, safe_right_den = right_den == 0 ? 1 : right_den;
+    bool left_inside = tx1 >= -ty1, right_inside = tx2 <= ty2;
+    i64 sl = left_inside ? left_projected : 0;
+    i64 sr = right_inside ? right_projected : SW;
+    i64 dl = left_inside ? ty1 : ty1 + tdiv((ty2 - ty1) * (tx1 + ty1), safe_left_den);
+    i64 dr = right_inside ? ty2 : ty1 + tdiv((ty2 - ty1) * (tx1 - ty1), safe_right_den);
+    bool invalid_left = (left_inside ? ((tx1 > ty1) || (ty1 == 0)) : ((tx2 < -ty2) || (left_den == 0))) || (dl < 32);
+    bool invalid_right = (right_inside ? ((tx2 < -ty2) || (ty2 == 0)) : ((tx1 > ty1) || (right_den == 0))) || (dr < 32);
+    bool invalid = invalid_left || invalid_right || (sr <= sl);
+    if (invalid) sr = sl;
+
+    // ray x segment over all columns: first / last geometric hit (engine.py:11323-11348)
+    const float4 wl = *reinterpret_cast<const float4 *>(m->walls + 4 * w);
+    float segx = wl.z - wl.x, segy = wl.w - wl.y;
+    float offx = wl.x - c.x, offy = wl.y - c.y;
+    int first = 0, last = SW - 1; bool any = false;
+    float numer_d = offx * segy - offy * segx;
+    for (int x = 0; x < SW; ++x) {
+        float rx, ry; ray_direction(c, x, &rx, &ry);
+        float den = rx * segy - ry * segx;
+        bool ok = fabsf(den) >= 1e-6f;
+        float safe = ok ? den : 1.0f;
+        float d = numer_d / safe;
+        float a = (offx * ry - offy * rx) / safe;
+        bool g = ok && (d > 0) && (a >= 0) && (a <= 1);
+        if (g) { if (!any) first = x; last = x; any = true; }
+    }
+    float vfx = c.x - wl.x, vfy = c.y - wl.y;
+    bool ff = (segx * vfy - segy * vfx) < 0;
+    i64 screen_left = first, screen_right = (i64)last + 1;
+    bool hc = any;
+    i64 ep_col[2]; bool ep_vis[2];
+    i64 txe[2] = {tx0, tx1v}, tye[2] = {ty0, ty1v};
+    for (int e = 0; e < 2; ++e) {
+        i64 safe_ty = tye[e] == 0 ? 1 : tye[e];
+        i64 projected_fixed = center + tdiv(txe[e] * center, safe_ty);
+        ep_col[e] = (projected_fixed >> 16) + (txe[e] >= 0);
+        ep_vis[e] = (tye[e] > 0) && (txe[e] >= -tye[e]) && (txe[e] <= tye[e]) && (ep_col[e] >= 0) && (ep_col[e] <= SW);
+    }
+    for (int e = 0; e < 2; ++e) {
+        bool visible = ep_vis[e] && hc;
+        bool owns_left = ff ? (e == 0) : (e == 1);
+        if (visible && owns_left) screen_left = ep_col[e];
+        if (visible && !owns_left) screen_right = ep_col[e];
+    }
+    if (ep_vis[0] && ep_vis[1]) {
+        screen_left = ff ? ep_col[0] : ep_col[1];
+        screen_right = ff ? ep_col[1] : ep_col[0];
+        hc = screen_right > screen_left;
+    }
+    hc = hc && (sr > sl);
+    bool os = m->wall_sectors[2 * w + 1] < 0;
+    WallRec r;
+    r.tx0 = (int)tx0; r.tx1 = (int)tx1v; r.ty0 = (int)ty0; r.ty1 = (int)ty1v;
+    r.dl = dl; r.dr = dr; r.sl = sl; r.sr = sr;
+    r.pl = (short)screen_left; r.pr = (short)screen_right;
+    r.flags = (hc ? WF_HC : 0) | (ff ? WF_FF : 0) | (((sr - sl <= 1) && !os) ? WF_SUBPIXEL : 0) | (any ? WF_ANYGEO : 0);
+    sc.rec[(size_t)local * m->wall_count + w] = r;
+    // A linedef can have a finite distance at some column only if it owns a span
+    // (projected) or, for two-sided lines, is hit by a ray (engine.py:11446-11451).
+    bool can_be_finite = os ? (hc && ff) : (hc || any);
+    if (can_be_finite) {
+        int slot = atomicAdd(&sc.ctx[local].visible_count, 1);
+        sc.visible[(size_t)local * m->wall_count + slot] = w;
+    }
+}
+
+// distances / along / geometric / projected / left-edge of one linedef at one column
+// (engine.py:11317-11331, 11440-11460)
+__device__ __forceinline__ Cand eval_wall(const gd_map_desc *m, const LaneCtx &c, const WallRec *recs, int x, int w, float rx, float ry) {
+    const float4 wl = *reinterpret_cast<const float4 *>(m->walls + 4 * w);
+    const WallRec &r = recs[w];
+    float segx = wl.z - wl.x, segy = wl.w - wl.y;
+    float offx = wl.x - c.x, offy = wl.y - c.y;
+    float den = rx * segy - ry * segx;
+    bool ok = fabsf(den) >= 1e-6f;
+    float safe = ok ? den : 1.0f;
+    float d = (offx * segy - offy * segx) / safe;
+    float a = (offx * ry - offy * rx) / safe;
+    bool g = ok && (d > 0) && (a >= 0) && (a <= 1);
+    bool screen_valid = (r.flags & WF_HC) && (x >= r.pl) && (x < r.pr);
+    bool p = ok && (d > 0) && screen_valid;
+    bool os = m->wall_sectors[2 * w + 1] < 0;
+    bool valid = os ? (p && (r.flags & WF_FF)) : (g || p);
+    Cand out;
+    out.wall = w;
+    out.dist = valid ? d : GD_INF;
+    out.along = a < 0.0f ? 0.0f : (a > 1.0f ? 1.0f : a);
+    out.flags = (g ? CF_GEO : 0) | (p ? CF_PROJ : 0) | ((x == r.pl) ? CF_LEDGE : 0);
+    return out;
+}
+
+// ---------------------------------------------------------------------------------------------
+// column_lists: finite-distance linedefs of every column, in ascending linedef order is NOT
+// required: every reduction below breaks distance ties on the linedef index explicitly.
+// ---------------------------------------------------------------------------------------------
+__global__ void column_lists_kernel(DeviceMap dm, int lane_count, Scratch sc) {
+    const gd_map_desc *m = &dm.d;
+    int local = blockIdx.x;
+    int x = threadIdx.x;
+    if (local >= lane_count || x >= SW) return;
+    const LaneCtx &c = sc.ctx[local];
+    const WallRec *recs = sc.rec + (size_t)local * m->wall_count;
+    const int *visible = sc.visible + (size_t)local * m->wall_count;
+    Cand *list = sc.cand + (size_t)local * CAND_MAX * SW;
+    float rx, ry; ray_direction(c, x, &rx, &ry);
+    int count = 0;
+    bool overflow = false;
+    const int visible_count = c.visible_count;
+    for (int k = 0; k < visible_count; ++k) {
+        int w = visible[k];
+        Cand cd = eval_wall(m, c, recs, x, w, rx, ry);
+        if (finitef(cd.dist)) {
+            if (count < CAND_MAX) list[(size_t)count * SW + x] = cd;
+            else overflow = true;
+            ++count;
+        }
+    }
+    if (overflow) { atomicOr(sc.status, STATUS_CAND_OVERFLOW); count = CAND_MAX; }
+    sc.cand_count[(size_t)local * SW + x] = (unsigned char)count;
+}
+
+// ---------------------------------------------------------------------------------------------
+// flats: engine.py:10956-11171
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float flat_center(const LaneCtx &c) { return 103.5f + c.pitch_offset; }
+
+// Per pixel: nearest plane among all sectors (engine.py:10981-11024).  Sectors that share a
+// plane height share the candidate point, and the distance grows with the plane height, so the
+// levels are visited nearest first and the scan stops once a farther level cannot win.
+__global__ void flat_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
+    const gd_map_desc *m = &dm.d;
+    int local = blockIdx.y;
+    int pixel = blockIdx.x * blockDim.x + threadIdx.x;
+    if (local >= lane_count || pixel >= VH * SW) return;
+    int y = pixel / SW, x = pixel - y * SW;
+    const LaneCtx &c = sc.ctx[local];
+    int n = lane_base + local;
+    float center = flat_center(c);
+    float delta = (float)y - center;
+    bool is_floor = delta > 0;
+    float denom = fmaxf(fabsf(delta), 0.5f);
+    float cc = dm.cosine_correction[x];
+    float rc = lanes.ray_cos[(size_t)n * SW + x], rs = lanes.ray_sin[(size_t)n * SW + x];
+    const float *levels = is_floor ? m->floor_levels : m->ceil_levels;
+    int level_count = is_floor ? m->floor_level_count : m->ceil_level_count;
+    float best = GD_INF; int best_sector = -1;
+    for (int l = 0; l < level_count; ++l) {
+        float level = levels[l];
+        float plane_height = is_floor ? (c.view_z - level) : (level - c.view_z);
+        if (!(plane_height > 0)) continue;
+        float perpendicular = plane_height * 192.0f / denom;
+        float cd = perpendicular / cc;
+        if (!(finitef(cd) && cd > 0)) continue;
+        if (cd > best) break;           // later levels are at least this far
+        float px = c.x + rc * cd, py = c.y + rs * cd;
+        int cell = grid_cell_of(m, px, py);
+        if (cell < 0) continue;
+        for (int it = m->grid_cell_ofs[cell]; it < m->grid_cell_ofs[cell + 1]; ++it) {
+            int s = m->grid_item_sector[it];
+            float sector_level = m->sector_heights[2 * s + (is_floor ? 0 : 1)];
+            if (sector_level != level) continue;
+            if (cd < best || (cd == best && s < best_sector)) {
+                if (inside_edges(m, m->grid_item_edge_ofs[it], m->grid_item_edge_ofs[it + 1], px, py)) { best = cd; best_sector = s; }
+            }
+        }
+    }
+    size_t i = (size_t)local * VH * SW + pixel;
+    sc.flat_sector[i] = (unsigned short)(best_sector < 0 ? c.sector : best_sector);
+    sc.flat_flags[i] = best_sector < 0 ? 1 : 0;
+}
+
+// engine.py:10879-10954
+__device__ void flat_texture_coordinates(const gd_map_desc *m, const LaneCtx &c, int texture_id, float plane_height, int px, int py, i64 *u, i64 *v) {
+    int width_bits = ilog2(m->tex_w[texture_id]);
+    int height_bits = ilog2(m->tex_h[texture_id]);
+    i64 xscale = shl64(1, 32 - width_bits), yscale = shl64(1, 32 - height_bits);
+    i64 xstep_scale = tdiv(mul64(xscale, c.vsin), FOCAL_X_FIXED);
+    i64 ystep_scale = tdiv(mul64(yscale, c.vcos), FOCAL_X_FIXED);
+    i64 flat_column = (i64)px - (SW / 2 - 1);
+    i64 basexfrac = (mul64(xscale, c.vcos) >> 16) + mul64(flat_column, xstep_scale);
+    i64 baseyfrac = (mul64(yscale, -c.vsin) >> 16) + mul64(flat_column, ystep_scale);
+    i64 pviewx = mul64(xscale, c.view_x_fixed) >> 16;
+    i64 pviewy = mul64(yscale, -c.view_y_fixed) >> 16;
+    i64 center_row = c.center_fixed >> 16;
+    i64 pixel_y_fixed = (i64)py * FIXED_UNIT;
+    i64 den = (py < center_row) ? (c.center_fixed - pixel_y_fixed - FIXED_UNIT / 2) : (pixel_y_fixed - c.center_fixed + FIXED_UNIT / 2);
+    den = max64(den, 1);
+    bool overflow = den <= (FOCAL_Y_FIXED >> 15);
+    i64 yslope = tdiv(FOCAL_Y_FIXED << 16, den);
+    if (overflow) yslope = (1LL << 31) - 1;
+    i64 plane_height_fixed = round_to_i64(plane_height * 65536.0f);
+    i64 distance = mul64(plane_height_fixed, yslope) >> 16;
+    i64 xfrac = ((mul64(distance, basexfrac) >> 16) + pviewx) & UINT32_MASK;
+    i64 yfrac = ((mul64(distance, baseyfrac) >> 16) + pviewy) & UINT32_MASK;
+    *u = xfrac >> (32 - width_bits);
+    *v = yfrac >> (32 - height_bits);
+}
+
+// engine.py:10588-10616
+__device__ unsigned char plane_colormap(const gd_map_desc *m, const LaneCtx &c, unsigned char index, float light, float plane_height, int py) {
+    i64 plane_height_fixed = round_to_i64(plane_height * 65536.0f);
+    i64 glob = min64(tdiv(FLOOR_VISIBILITY_FIXED << 16, max64(plane_height_fixed, 1)), (1LL << 31) - 1);
+    i64 row = c.center_fixed - (i64)py * FIXED_UNIT;
+    if (row < 0) row = -row;
+    i64 visibility = min64(mul64(glob, row) >> 16, 24 * FIXED_UNIT);
+    i64 plane_shade = 64 * FIXED_UNIT - ((i64)light + 12) * (FIXED_UNIT / 4);
+    i64 shade = clampi((plane_shade - visibility) >> 16, 0, 31);
+    return m->colormap[shade * 256 + index];
+}
+
+__device__ unsigned char flat_pixel(const gd_map_desc *m, const LaneCtx &c, int sector, bool is_floor, int px, int py) {
+    float plane_height = is_floor ? (c.view_z - m->sector_heights[2 * sector]) : (m->sector_heights[2 * sector + 1] - c.view_z);
+    int texture = is_floor ? m->sector_floor_tex[sector] : m->sector_ceil_tex[sector];
+    i64 u, v;
+    flat_texture_coordinates(m, c, texture, plane_height, px, py, &u, &v);
+    unsigned char index = m->tex_atlas[((size_t)texture * m->tex_max_h + v) * m->tex_max_w + u];
+    float light = m->sector_lights[sector] + (float)(c.flash_light * 16);
+    return plane_colormap(m, c, index, light, plane_height, py);
+}
+
+// Visplane continuity repair and shading for one lane (engine.py:11026-11171).
+// 320 threads: vertical repair is one thread per column; horizontal repair is one wave per
+// row with 64-column ballots; shading is one thread per column again.
+__global__ void __launch_bounds__(SW) flat_finish_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
+    const gd_map_desc *m = &dm.d;
+    int local = blockIdx.x;
+    if (local >= lane_count) return;
+    const LaneCtx c = sc.ctx[local];
+    unsigned short *sector = sc.flat_sector + (size_t)local * VH * SW;
+    unsigned char *flags = sc.flat_flags + (size_t)local * VH * SW;
+    unsigned char *frame = frame_base + (size_t)local * frame_stride;
+    const int x = threadIdx.x;
+    const float center = flat_center(c);
+    // --- vertical: an unresolved pixel takes the next resolved row below of its own kind.
+    // Floors are repaired first and ceilings read the repaired map (engine.py:11050-11083);
+    // the gathered rows are resolved pixels, which no repair modifies.
+    {
+        int next_floor = VH, next_ceiling = VH;
+        int floor_sector = 0, ceiling_sector = 0;
+        for (int y = VH - 1; y >= 0; --y) {
+            size_t i = (size_t)y * SW + x;
+            bool is_floor = ((float)y - center) > 0;
+            bool unresolved = flags[i] & 1;
+            int s = sector[i];
+            if (!unresolved) {
+                if (is_floor) { next_floor = y; floor_sector = s; } else { next_ceiling = y; ceiling_sector = s; }
+            } else {
+                bool vfloor = is_floor && next_floor < VH;
+                bool vceil = !is_floor && next_ceiling < VH;
+                if (vfloor || vceil) {
+                    int span_sector = vfloor ? floor_sector : ceiling_sector;
+                    sector[i] = (unsigned short)span_sector;
+                    // bit1: vertical span; bit2: its sector differs from the camera's (anchor)
+                    flags[i] = (unsigned char)(1 | 2 | ((span_sector != c.sector) ? 4 : 0));
+                }
+            }
+        }
+    }
+    __syncthreads();
+    // --- horizontal (engine.py:11085-11135): between a left and a right anchor of one sector
+    {
+        const int lane_id = threadIdx.x & 63;
+        const int wave = threadIdx.x >> 6;
+        for (int y = wave; y < VH; y += SW / 64) {
+            unsigned short *row_sector = sector + (size_t)y * SW;
+            unsigned char *row_flags = flags + (size_t)y * SW;
+            u64 anchors[5];
+            unsigned char f[5];
+            for (int k = 0; k < 5; ++k) {
+                f[k] = row_flags[k * 64 + lane_id];
+                bool anchor = !(f[k] & 1) || (f[k] & 4);
+                anchors[k] = __ballot(anchor);
+            }
+            for (int k = 0; k < 5; ++k) {
+                if (!(f[k] & 1)) continue;
+                int col = k * 64 + lane_id;
+                // nearest anchor at or left of col
+                int left = -1;
+                u64 below = anchors[k] & ((lane_id == 63) ? ~0ULL : ((1ULL << (lane_id + 1)) - 1));
+                if (below) left = k * 64 + 63 - __clzll(below);
+                else for (int j = k - 1; j >= 0 && left < 0; --j) if (anchors[j]) left = j * 64 + 63 - __clzll(anchors[j]);
+                int right = SW;
+                u64 above = anchors[k] & ~((1ULL << lane_id) - 1);
+                if (above) right = k * 64 + __ffsll((long long)above) - 1;
+                else for (int j = k + 1; j < 5 && right >= SW; ++j) if (anchors[j]) right = j * 64 + __ffsll((long long)anchors[j]) - 1;
+                if (left >= 0 && right < SW) {
+                    int ls = row_sector[left], rs = row_sector[right];
+                    // anchors are never rewritten by this pass, so reading them while other
+                    // lanes write their own unresolved pixels is race free
+                    if (ls == rs) { row_sector[col] = (unsigned short)ls; row_flags[col] = (unsigned char)(f[k] | 8); }
+                }
+            }
+        }
+    }
+    __syncthreads();
+    // --- shade every view pixel with its selected sector (engine.py:11145-11163)
+    for (int y = 0; y < VH; ++y) {
+        size_t i = (size_t)y * SW + x;
+        bool is_floor = ((float)y - center) > 0;
+        frame[i] = flat_pixel(m, c, sector[i], is_floor, x, y);
+    }
+    for (int y = VH; y < GD_SCREEN_HEIGHT; ++y) frame[(size_t)y * SW + x] = 0;  // empty status bar
+}
+
+// ---------------------------------------------------------------------------------------------
+// walls: engine.py:11462-13745
+// ---------------------------------------------------------------------------------------------
+struct ColumnCtx {
+    const gd_map_desc *m;
+    MapView mv;
+    const LaneCtx *c;
+    const WallRec *recs;
+    const Cand *list;     // this lane's candidate block, entry k of column x at [k*320 + x]
+    int count;
+    int x;
+    float rx, ry;
+    __device__ Cand cand(int k) const { return list[(size_t)k * SW + x]; }
+    __device__ Cand eval(int w) const { return eval_wall(m, *c, recs, x, w, rx, ry); }
+};
+
+// engine.py:11217-11291 for one endpoint order, evaluated at one column
+__device__ i64 wall_visibility(const WallRec &r, int side, int x) {
+    i64 tx1 = side ? r.tx1 : r.tx0, tx2 = side ? r.tx0 : r.tx1;
+    i64 ty1 = side ? r.ty1 : r.ty0, ty2 = side ? r.ty0 : r.ty1;
+    const i64 center = 160 * FIXED_UNIT;
+    i64 safe_ty1 = ty1 == 0 ? 1 : ty1, safe_ty2 = ty2 == 0 ? 1 : ty2;
+    i64 left_projected = ((center + tdiv(tx1 * center, safe_ty1)) >> 16) + (tx1 >= 0);
+    i64 right_projected = ((center + tdiv(tx2 * center, safe_ty2)) >> 16) + (tx2 >= 0);
+    i64 left_den = tx1 - tx2 - ty2 + ty1, right_den = ty2 - ty1 - tx2 + tx1;
+    i64 safe_left_den = left_den == 0 ? 1 : left_den, safe_right_den = right_den == 0 ? 1 : right_den;
+    bool left_inside = tx1 >= -ty1, right_inside = tx2 <= ty2;
+    i64 wsl = left_inside ? left_projected : 0;
+    i64 wsr = right_inside ? right_projected : SW;
+    i64 wdl = left_inside ? ty1 : ty1 + tdiv((ty2 - ty1) * (tx1 + ty1), safe_left_den);
+    i64 wdr = right_inside ? ty2 : ty1 + tdiv((ty2 - ty1) * (tx1 - ty1), safe_right_den);
+    i64 light_left = tdiv(WALL_VISIBILITY_FIXED << 12, max64(wdl, 1));
+    i64 light_right = tdiv(WALL_VISIBILITY_FIXED << 12, max64(wdr, 1));
+    i64 light_step = tdiv(light_right - light_left, max64(wsr - wsl, 1));
+    return light_left + ((i64)x - wsl) * light_step;
+}
+
+// engine.py:10672-10739 (PrepWall) for one (linedef, column)
+__device__ void texture_mapping(const gd_map_desc *m, const WallRec &r, int w, int x, i64 *hoff, i64 *vstep) {
+    const float wall_map_scale = (float)((320 * 200.0 / 320.0 / 240) * 64.0 / (320 / 2.0));
+    i64 tx1 = r.tx0, tx2 = r.tx1, ty1 = r.ty0, ty2 = r.ty1;
+    double u_over_z_origin = (double)((float)tx1 * 160.0f);
+    float u_over_z_step_f = -(float)ty1;
+    double u_over_z_step = (double)u_over_z_step_f;
+    double inv_z_origin = (double)((float)(tx1 - tx2) * 160.0f);
+    float inv_z_step_float = (float)(ty2 - ty1);
+    double inv_z_step = (double)inv_z_step_float;
+    double depth_scale = (double)(inv_z_step_float * wall_map_scale);
+    double depth_origin = (double)(-u_over_z_step_f * wall_map_scale);
+    double repeat = (double)round_to_i64(m->wall_len[w] * 65536.0f);
+    double column = (double)x - 160.0;
+    double top = u_over_z_origin + u_over_z_step * column;
+    double bottom = inv_z_origin + inv_z_step * column;
+    double safe_bottom = bottom == 0 ? 1.0 : bottom;
+    double fraction = top / safe_bottom;
+    *hoff = f64_to_i64(floor(fraction * repeat + 0.5));
+    *vstep = f64_to_i64(floor(fraction * depth_scale + depth_origin + 0.5));
+}
+
+// engine.py:12294-12605 (OWallMost) for one column
+__device__ float project(const LaneCtx &c, const WallRec &g, float world_z, int x) {
+    i64 whole_sl = g.sl, whole_sr = g.sr;
+    i64 whole_dl = max64(g.dl, 1), whole_dr = max64(g.dr, 1);
+    bool has_fragment = (g.sr > g.sl) && (x >= g.sl) && (x < g.sr);
+    i64 screen_left = g.sl, screen_right = g.sr, depth_left = whole_dl, depth_right = whole_dr;
+    i64 relative_z_fixed = round_to_i64((world_z - c.view_z) * 65536.0f);
+    i64 pz = -(relative_z_fixed >> 4);
+    i64 center_fixed = c.center_fixed;
+    i64 px = x;
+    if (!has_fragment) {
+        i64 original_span = max64(whole_sr - whole_sl, 1);
+        i64 opl = tdiv(mul64(pz, FOCAL_Y_FIXED), whole_dl);
+        i64 opr = tdiv(mul64(pz, FOCAL_Y_FIXED), whole_dr);
+        i64 ostep = tdiv(opr - opl, original_span);
+        return (float)clampi((center_fixed + opl + mul64(px - whole_sl, ostep)) >> 16, 0, VH);
+    }
+    i64 upper_clip = tdiv(shl64(-center_fixed, 16), FOCAL_Y_FIXED);
+    i64 lower_clip = tdiv(shl64((i64)VH * FIXED_UNIT - center_fixed, 16), FOCAL_Y_FIXED);
+    i64 upper_left = mul64(upper_clip, depth_left) >> 16, upper_right = mul64(upper_clip, depth_right) >> 16;
+    i64 lower_left = mul64(lower_clip, depth_left) >> 16, lower_right = mul64(lower_clip, depth_right) >> 16;
+    bool above_left = pz < upper_left, above_right = pz < upper_right;
+    bool below_left = pz > lower_left, below_right = pz > lower_right;
+    bool entirely_above = above_left && above_right, entirely_below = below_left && below_right;
+    i64 clipped_left = screen_left, clipped_right = screen_right;
+    i64 clipped_dl = depth_left, clipped_dr = depth_right;
+    bool outside_top = false, outside_bottom = false;
+    bool crosses_top = above_left != above_right;
+    if (crosses_top) {
+        i64 safe_upper_delta = (upper_right != upper_left) ? (upper_right - upper_left) : 1;
+        i64 top_fraction = tdiv(shl64(pz - upper_left, 30), safe_upper_delta);
+        i64 top_depth = depth_left + (mul64(depth_right - depth_left, top_fraction) >> 30);
+        i64 top_cross = screen_left + tdiv(mul64(mul64(depth_right, top_fraction) >> 30, screen_right - screen_left), max64(top_depth, 1));
+        if (above_right && (screen_left <= top_cross)) { clipped_right = top_cross; clipped_dr = top_depth; }
+        outside_top |= above_right && (screen_right > top_cross) && (px >= top_cross) && (px < screen_right);
+        if (above_left && (top_cross <= screen_right)) { clipped_left = top_cross; clipped_dl = top_depth; }
+        outside_top |= above_left && (top_cross > screen_left) && (px >= screen_left) && (px < top_cross);
+    }
+    bool crosses_bottom = below_left != below_right;
+    if (crosses_bottom) {
+        i64 safe_lower_delta = (lower_right != lower_left) ? (lower_right - lower_left) : 1;
+        i64 bottom_fraction = tdiv(shl64(pz - lower_left, 30), safe_lower_delta);
+        i64 bottom_depth = depth_left + (mul64(depth_right - depth_left, bottom_fraction) >> 30);
+        i64 bottom_cross = screen_left + tdiv(mul64(mul64(depth_right, bottom_fraction) >> 30, screen_right - screen_left), max64(bottom_depth, 1));
+        if (below_right && (screen_left <= bottom_cross)) { clipped_right = bottom_cross; clipped_dr = bottom_depth; }
+        outside_bottom |= below_right && (screen_right > bottom_cross) && (px >= bottom_cross) && (px < screen_right);
+        if (below_left && (bottom_cross <= screen_right)) { clipped_left = bottom_cross; clipped_dl = bottom_depth; }
+        outside_bottom |= below_left && (bottom_cross > screen_left) && (px >= screen_left) && (px < bottom_cross);
+    }
+    i64 projected_left = tdiv(mul64(pz, FOCAL_Y_FIXED), max64(clipped_dl, 1));
+    i64 projected_right = tdiv(mul64(pz, FOCAL_Y_FIXED), max64(clipped_dr, 1));
+    i64 span = max64(clipped_right - clipped_left, 1);
+    i64 projected_step = tdiv(projected_right - projected_left, span);
+    i64 projected = clampi((center_fixed + projected_left + mul64(px - clipped_left, projected_step)) >> 16, 0, VH);
+    bool collapsed = (clipped_right == clipped_left) && (px == clipped_left) && !(entirely_above || entirely_below);
+    if (entirely_above || (outside_top && !collapsed)) projected = 0;
+    else if (entirely_below || (outside_bottom && !collapsed)) projected = VH;
+    return (float)projected;
+}
+
+// engine.py:10630-10640
+__device__ __forceinline__ i64 wall_shade(float light, i64 visibility) {
+    i64 shade = 64 * FIXED_UNIT - ((i64)light + 12) * (FIXED_UNIT / 4);
+    return clampi((shade - min64(visibility, 24 * FIXED_UNIT)) >> 16, 0, 31);
+}
+
+// engine.py:11596-11730 for one (column, linedef)
+__device__ void endpoint_owner(const ColumnCtx &cc, int w, const Cand &cw, int *owner_index, float *owner_distance) {
+    const gd_map_desc *m = cc.m;
+    const int K = m->neighbor_slots;
+    const bool subpixel = cc.recs[w].flags & WF_SUBPIXEL;
+    float tol_w = tolerance_of(cw.dist);
+    bool uses_start = cw.along <= 0.5f;
+    int index; float distance; bool valid;
+    if (m->direct_neighbors) {
+        int ss = 0, es = 0; bool hs = false, he = false;
+        for (int k = K - 1; k >= 0; --k) {
+            if (m->endpoint_neighbor_starts[w * K + k]) { ss = k; hs = true; }
+            if (m->endpoint_neighbor_ends[w * K + k]) { es = k; he = true; }
+        }
+        int rslot = uses_start ? ss : es, oslot = uses_start ? es : ss;
+        bool rexists = uses_start ? hs : he, oexists = uses_start ? he : hs;
+        int rn = m->endpoint_neighbors[w * K + rslot], on = m->endpoint_neighbors[w * K + oslot];
+        Cand r = cc.eval(rn);
+        bool r_owns = rexists && (r.flags & CF_PROJ) && (r.flags & CF_LEDGE);
+        Cand o = (on == rn) ? r : cc.eval(on);
+        bool o_owns = subpixel && oexists && (o.flags & CF_PROJ) && (o.flags & CF_LEDGE) && (fabsf(o.dist - cw.dist) <= tol_w);
+        bool use_o = o_owns && (!r_owns || (o.dist < r.dist) || ((o.dist == r.dist) && (oslot < rslot)));
+        index = use_o ? on : rn;
+        distance = use_o ? o.dist : r.dist;
+        valid = r_owns || o_owns;
+    } else {
+        float best = GD_INF; int best_slot = 0;
+        for (int k = 0; k < K; ++k) {
+            int n = m->endpoint_neighbors[w * K + k];
+            bool st = m->endpoint_neighbor_starts[w * K + k], en = m->endpoint_neighbor_ends[w * K + k];
+            Cand nb = cc.eval(n);
+            bool ray_nb = uses_start ? st : en;
+            bool selected = ray_nb || (subpixel && (st || en) && (fabsf(nb.dist - cw.dist) <= tol_w));
+            float v = ((nb.flags & CF_PROJ) && (nb.flags & CF_LEDGE) && selected) ? nb.dist : GD_INF;
+            if (v < best) { best = v; best_slot = k; }
+        }
+        index = m->endpoint_neighbors[w * K + best_slot];
+        distance = best;
+        valid = finitef(best);
+    }
+    bool has = !(cw.flags & CF_PROJ) && valid;
+    *owner_index = has ? index : w;
+    *owner_distance = has ? distance : cw.dist;
+}
+
+struct ColumnState {   // engine.py:11561-11580, 11735-11762
+    int current_sector;
+    float ceiling_clip, floor_clip;
+    float masked_ceiling_clip, masked_floor_clip, masked_distance;
+    int masked_wall;
+    float previous_distance;
+    int pend_po_vertex, pend_ep_vertex, pend_ep_wall, pend_eb_index, pend_pb_index, pend_pb_sector;
+    float pend_pb_exit;
+    int flags;  // bit0 pend_po_boundary, bit1 pend_ep_boundary, bit2 pend_eb_boundary, bit3 pend_pb
+};
+#define ST_PO 1
+#define ST_EP 2
+#define ST_EB 4
+#define ST_PB 8
+
+__device__ __forceinline__ bool same_state(const ColumnState &a, const ColumnState &b) {
+    return a.current_sector == b.current_sector && a.ceiling_clip == b.ceiling_clip && a.floor_clip == b.floor_clip &&
+           a.masked_ceiling_clip == b.masked_ceiling_clip && a.masked_floor_clip == b.masked_floor_clip &&
+           a.masked_distance == b.masked_distance && a.masked_wall == b.masked_wall &&
+           a.previous_distance == b.previous_distance && a.pend_po_vertex == b.pend_po_vertex &&
+           a.pend_ep_vertex == b.pend_ep_vertex && a.pend_ep_wall == b.pend_ep_wall && a.pend_eb_index == b.pend_eb_index &&
+           a.pend_pb_index == b.pend_pb_index && a.pend_pb_sector == b.pend_pb_sector && a.pend_pb_exit == b.pend_pb_exit &&
+           a.flags == b.flags;
+}
+
+struct PassColumn {
+    int wall, side, render_current, other_sector;
+    float distance;
+    i64 visibility;
+    float view_floor, view_ceiling, other_floor, other_ceiling;
+    float clipped_top, clipped_bottom, clipped_upper_bottom, clipped_lower_top;
+    int side_tex[3];
+    int ps_path_index, ps_other, no_path_other, sel_vertex, fb_idx;
+    float ps_path_distance, no_path_distance;
+    int bits;
+};
+#define PB_VALID 0x1
+#define PB_RASTER 0x2
+#define PB_ONE_SIDED 0x4
+#define PB_TIER0 0x8
+#define PB_TIER1 0x10
+#define PB_TIER2 0x20
+#define PB_MARK_CEILING 0x40
+#define PB_MARK_FLOOR 0x80
+#define PB_PS_KEEPS 0x100
+#define PB_NO_KEEPS 0x200
+#define PB_GEOMETRIC 0x400
+#define PB_REPLACE_NP 0x800
+#define PB_PS_FROM_FRONT 0x1000
+#define PB_CONTINUES_PO 0x2000
+#define PB_FORWARD_BRIDGE 0x4000
+#define PB_GEO_FINAL 0x8000
+
+// (distance, linedef) lexicographic minimum: what torch.min(dim) returns on ascending indices
+__device__ __forceinline__ void take_min(float v, int w, float &best, int &best_w) {
+    if (v < best || (v == best && w < best_w && finitef(v))) { best = v; best_w = w; }
+}
+
+// engine.py:11769-12636: selection of the pass's drawseg for one column
+__device__ void pass_select(const ColumnCtx &cc, const ColumnState &c, bool boundary_has_po, PassColumn &r) {
+    const gd_map_desc *m = cc.m;
+    const MapView &mv = cc.mv;
+    const int x = cc.x;
+    const int cs = c.current_sector;
+    const int cur = cs < 0 ? 0 : cs;
+    const float prev = c.previous_distance;
+    const float prev_eps = prev + 1e-3f;
+    auto incident = [&](int w) { return mv.sec(w, 0) == cur || mv.sec(w, 1) == cur; };
+    // a. nearest incident linedef beyond previous_distance (engine.py:11769-11780)
+    float distance = GD_INF; int wi = 0x7fffffff;
+    if (cs >= 0) {
+        for (int k = 0; k < cc.count; ++k) {
+            Cand q = cc.cand(k);
+            if (incident(q.wall) && q.dist > prev) take_min(q.dist, q.wall, distance, wi);
+        }
+        // b. equal-depth solid (engine.py:11784-11807)
+        float sd = GD_INF; int swi = 0x7fffffff;
+        for (int k = 0; k < cc.count; ++k) {
+            Cand q = cc.cand(k);
+            if (incident(q.wall) && q.dist > prev && mv.one_sided(q.wall) && (fabsf(q.dist - distance) <= 1e-3f)) take_min(q.dist, q.wall, sd, swi);
+        }
+        if (finitef(sd)) { distance = sd; wi = swi; }
+    }
+    if (!finitef(distance)) wi = 0;
+    Cand cwi = cc.eval(wi);
+    // c. selected endpoint (engine.py:11815-11871)
+    float sel_along = cwi.along;
+    bool sel_start = sel_along <= 0.5f;
+    int sel_vertex = mv.vert(wi, sel_start ? 0 : 1);
+    auto shares_sel = [&](int w) { return mv.vert(w, 0) == sel_vertex || mv.vert(w, 1) == sel_vertex; };
+    bool continues_po_boundary = (c.flags & ST_PO) && (sel_vertex == c.pend_po_vertex);
+    bool continues_ep_boundary = (c.flags & ST_EP) && (sel_vertex == c.pend_ep_vertex);
+    int sel_slot = sel_along > 0.5f ? 1 : 0;
+    int fb_idx; bool fb_exists = mv.portal_bridge(sel_slot, wi, c.pend_ep_wall, &fb_idx);
+    bool pend_ep_has_forward_bridge = false;
+    if (continues_ep_boundary && fb_exists) pend_ep_has_forward_bridge = cc.eval(fb_idx).dist > distance + 1e-3f;
+    bool completes_pending_endpoint_bridge = (c.flags & ST_EB) && (wi == c.pend_eb_index);
+    bool sel_is_proj = cwi.flags & CF_PROJ;
+    bool sel_excl_right = cc.recs[wi].sr == x;
+    // d. projected solid owner (engine.py:11872-11954)
+    float ps_path_distance = distance; int ps_path_index = wi;
+    bool ps_path_geo = cwi.flags & CF_GEO;
+    float psd = GD_INF; int psi = 0x7fffffff;
+    if (!sel_is_proj) {
+        for (int k = 0; k < cc.count; ++k) {
+            Cand q = cc.cand(k);
+            bool owner = incident(q.wall) && mv.one_sided(q.wall) && (q.flags & CF_PROJ) && (q.flags & CF_LEDGE) && shares_sel(q.wall) && (q.dist > prev_eps);
+            if (owner) take_min(q.dist, q.wall, psd, psi);
+        }
+        if (sel_excl_right) {
+            const int *ofs = sel_start ? m->solid_bridge_start_ofs : m->solid_bridge_end_ofs;
+            const int *idx = sel_start ? m->solid_bridge_start_idx : m->solid_bridge_end_idx;
+            float sbd = GD_INF; int sbi = 0;
+            for (int k = ofs[wi]; k < ofs[wi + 1]; ++k) {
+                int b = idx[k];
+                if (!(incident(b) && mv.one_sided(b))) continue;
+                Cand q = cc.eval(b);
+                bool owner = (q.flags & CF_PROJ) && (q.flags & CF_LEDGE) && (q.dist > prev_eps);
+                float v = owner ? q.dist : GD_INF;
+                if (v < sbd) { sbd = v; sbi = b; }   // list is ascending: first slot wins ties
+            }
+            if (sbd < psd) { psd = sbd; psi = sbi; }
+        }
+    }
+    bool has_ps = finitef(psd);
+    if (has_ps) { distance = psd; wi = psi; cwi = cc.eval(wi); }
+    // e. endpoint owner (engine.py:11960-12001)
+    int eo_idx; float eo_dist;
+    endpoint_owner(cc, wi, cwi, &eo_idx, &eo_dist);
+    bool eo_path_geo = cwi.flags & CF_GEO;
+    bool replace_eo = (eo_idx != wi) && (eo_dist > prev_eps);
+    if (replace_eo) { distance = eo_dist; wi = eo_idx; cwi = cc.eval(wi); }
+    int no_path_index = wi; float no_path_distance = distance;
+    bool no_path_geo = replace_eo ? eo_path_geo : (bool)(cwi.flags & CF_GEO);
+    bool no_from_front = cs == mv.sec(no_path_index, 0);
+    int no_path_other = no_from_front ? mv.sec(no_path_index, 1) : mv.sec(no_path_index, 0);
+    // f. near projected owner (engine.py:12002-12179)
+    bool so_is_proj = cwi.flags & CF_PROJ;
+    const WallRec &so_rec = cc.recs[wi];
+    bool so_excl_right = so_rec.sr == x;
+    i64 so_span = so_rec.sr - so_rec.sl;
+    bool so_short = m->wall_len[wi] <= 32.0f;
+    float npd = GD_INF; int npi = 0x7fffffff;
+    if (!so_is_proj) {
+        for (int k = 0; k < cc.count; ++k) {
+            Cand q = cc.cand(k);
+            int w = q.wall;
+            if (!(incident(w) && !mv.one_sided(w) && (q.flags & CF_PROJ) && (q.dist > prev_eps))) continue;
+            bool le = q.flags & CF_LEDGE;
+            bool close = (mv.same_pair(wi, w) || (le && so_excl_right && ((so_span <= 2) || (shares_sel(w) && so_short)))) &&
+                         (fabsf(q.dist - distance) <= tolerance_of(q.dist));
+            bool topo = false;
+            if (!close && le && so_excl_right && so_span <= 2) { int dummy; topo = mv.sector_bridge(q.along > 0.5f ? 1 : 0, w, no_path_index, &dummy); }
+            if (close || topo) take_min(q.dist, w, npd, npi);
+        }
+    }
+    int pe_wall = c.pend_ep_wall;
+    int pe_s0 = mv.sec(pe_wall, 0), pe_s1 = mv.sec(pe_wall, 1);
+    bool pe_from_current = cs == pe_s0;
+    bool pe_incident = pe_from_current || (cs == pe_s1);
+    int pe_other = pe_from_current ? pe_s1 : pe_s0;
+    bool use_psb = false; int psb_idx = 0;
+    if ((c.flags & ST_EP) && pe_incident && (pe_other >= 0) && (no_path_other >= 0) && no_path_geo && !so_is_proj && so_excl_right &&
+        (cc.recs[pe_wall].sr - cc.recs[pe_wall].sl <= 1)) {
+        int pe_slot = (c.pend_ep_vertex == mv.vert(pe_wall, 1)) ? 1 : 0;
+        bool psb_exists = mv.sector_bridge(pe_slot, pe_wall, no_path_index, &psb_idx);
+        if (psb_exists) {
+            int b0 = mv.sec(psb_idx, 0), b1 = mv.sec(psb_idx, 1);
+            bool matches = (b0 == pe_other && b1 == no_path_other) || (b1 == pe_other && b0 == no_path_other);
+            Cand qb = cc.eval(psb_idx);
+            float pe_tol = tolerance_of(cc.eval(pe_wall).dist);
+            bool psb = matches && (qb.flags & CF_PROJ) && (qb.flags & CF_LEDGE) && (qb.dist > prev - pe_tol) && (qb.dist < no_path_distance);
+            if (psb && qb.dist < npd) { use_psb = true; npd = qb.dist; npi = psb_idx; }
+        }
+    }
+    bool replace_np = finitef(npd);
+    if (replace_np) { distance = npd; wi = npi; cwi = cc.eval(wi); }
+    bool final_proj = cwi.flags & CF_PROJ, final_geo = cwi.flags & CF_GEO;
+    bool completes_poab = (c.flags & ST_EP) && final_proj && !final_geo && mv.opposing(pe_wall, wi);
+    // g. validity (engine.py:12197-12239)
+    bool valid = finitef(distance);
+    bool excl_only = !so_is_proj && so_excl_right && !replace_np && (so_span <= 2) && !boundary_has_po;
+    bool raster_valid = valid && !excl_only && !continues_po_boundary &&
+                        !((pend_ep_has_forward_bridge || completes_pending_endpoint_bridge) && !sel_is_proj && sel_excl_right && !replace_np);
+    bool geometric_intersection = replace_np ? no_path_geo : (replace_eo ? eo_path_geo : final_geo);
+    bool no_keeps = replace_np && no_path_geo && (no_path_other >= 0);
+    // h. sides (engine.py:12240-12292)
+    int front = mv.sec(wi, 0), back = mv.sec(wi, 1);
+    bool from_front = cs == front;
+    int other_sector = from_front ? back : front;
+    int render_current = use_psb ? pe_other : (completes_poab ? other_sector : cur);
+    bool render_from_front = render_current == front;
+    int render_other = render_from_front ? back : front;
+    int side = render_from_front ? 0 : 1;
+    bool ps_from_front = cs == mv.sec(ps_path_index, 0);
+    int ps_other = ps_from_front ? mv.sec(ps_path_index, 1) : mv.sec(ps_path_index, 0);
+    bool ps_keeps = has_ps && ps_path_geo && (ps_other >= 0);
+    int safe_other = render_other < 0 ? 0 : render_other;
+    bool one_sided = other_sector < 0;
+
+    r.wall = wi; r.side = side; r.render_current = render_current; r.other_sector = other_sector;
+    r.distance = distance;
+    const WallRec &wr = cc.recs[wi];
+    r.visibility = wall_visibility(wr, side, x);
+    r.view_floor = m->sector_heights[2 * render_current]; r.view_ceiling = m->sector_heights[2 * render_current + 1];
+    r.other_floor = m->sector_heights[2 * safe_other]; r.other_ceiling = m->sector_heights[2 * safe_other + 1];
+    for (int t = 0; t < 3; ++t) r.side_tex[t] = m->side_tex[(wi * 2 + side) * 3 + t];
+    // j. projection and clipping (engine.py:12607-12620)
+    float one_top = project(*cc.c, wr, r.view_ceiling, x), one_bottom = project(*cc.c, wr, r.view_floor, x);
+    float lower_top = project(*cc.c, wr, r.other_floor, x), upper_bottom = project(*cc.c, wr, r.other_ceiling, x);
+    r.clipped_top = fmaxf(one_top, c.ceiling_clip);
+    r.clipped_bottom = fminf(one_bottom, c.floor_clip);
+    r.clipped_upper_bottom = fmaxf(fminf(upper_bottom, c.floor_clip), r.clipped_top);
+    r.clipped_lower_top = fminf(fmaxf(lower_top, c.ceiling_clip), r.clipped_bottom);
+    // k. plane marks (engine.py:12621-12636)
+    bool light_differs = m->sector_lights[render_current] != m->sector_lights[safe_other];
+    bool mark_ceiling = one_sided || (r.view_ceiling != r.other_ceiling) || (m->sector_ceil_tex[render_current] != m->sector_ceil_tex[safe_other]) || light_differs;
+    bool mark_floor = one_sided || (r.view_floor != r.other_floor) || (m->sector_floor_tex[render_current] != m->sector_floor_tex[safe_other]) || light_differs;
+    bool tier0 = one_sided && raster_valid && (r.side_tex[0] >= 0) && (r.clipped_top < r.clipped_bottom);
+    bool tier1 = !one_sided && raster_valid && (r.view_floor < r.other_floor) && (r.side_tex[1] >= 0) && (r.clipped_lower_top < r.clipped_bottom);
+    bool tier2 = !one_sided && raster_valid && (r.view_ceiling > r.other_ceiling) && (r.side_tex[2] >= 0) && (r.clipped_top < r.clipped_upper_bottom);
+    r.ps_path_index = ps_path_index; r.ps_other = ps_other; r.no_path_other = no_path_other; r.sel_vertex = sel_vertex; r.fb_idx = fb_idx;
+    r.ps_path_distance = ps_path_distance; r.no_path_distance = no_path_distance;
+    r.bits = (valid ? PB_VALID : 0) | (raster_valid ? PB_RASTER : 0) | (one_sided ? PB_ONE_SIDED : 0) | (tier0 ? PB_TIER0 : 0) |
+             (tier1 ? PB_TIER1 : 0) | (tier2 ? PB_TIER2 : 0) | (mark_ceiling ? PB_MARK_CEILING : 0) | (mark_floor ? PB_MARK_FLOOR : 0) |
+             (ps_keeps ? PB_PS_KEEPS : 0) | (no_keeps ? PB_NO_KEEPS : 0) | (geometric_intersection ? PB_GEOMETRIC : 0) |
+             (replace_np ? PB_REPLACE_NP : 0) | (ps_from_front ? PB_PS_FROM_FRONT : 0) | (continues_po_boundary ? PB_CONTINUES_PO : 0) |
+             (pend_ep_has_forward_bridge ? PB_FORWARD_BRIDGE : 0);
+}
+
+struct PixelBuffers {
+    unsigned char *frame;   // [240][320]
+    unsigned int *meta;     // [208][320]
+    float *clip_depth;      // [208][320]
+};
+
+// Silhouette bookkeeping: every row >= bot_row holds a clip depth <= bot_depth, every row
+// < top_row holds a clip depth <= top_depth.  Clip depths only ever decrease, so a silhouette
+// at a depth not below the bound cannot change those rows and they need not be visited.
+struct SilhouetteBounds {
+    int bot_row, top_row;
+    float bot_depth, top_depth;
+};
+
+__device__ void apply_silhouette(PixelBuffers &pb, SilhouetteBounds &sb, int x, bool bottom, bool top, float floor_clip, float ceiling_clip, float distance, int wall) {
+    if (bottom) {
+        int first = floor_clip <= 0.0f ? 0 : (floor_clip >= (float)VH ? VH : (int)floor_clip);   // clips hold integers
+        int last = (distance >= sb.bot_depth) ? (sb.bot_row < VH ? sb.bot_row : VH) : VH;
+        for (int y = first; y < last; ++y) {
+            size_t i = (size_t)y * SW + x;
+            if (distance < pb.clip_depth[i]) { pb.clip_depth[i] = distance; pb.meta[i] = (pb.meta[i] & ~META_WALL_MASK) | (unsigned)(wall + 1); }
+        }
+        sb.bot_row = first < sb.bot_row ? first : sb.bot_row;
+        sb.bot_depth = fmaxf(sb.bot_depth, distance);
+    }
+    if (top) {
+        int end = ceiling_clip <= 0.0f ? 0 : (ceiling_clip >= (float)VH ? VH : (int)ceiling_clip);
+        int start = (distance >= sb.top_depth) ? (sb.top_row > 0 ? sb.top_row : 0) : 0;
+        for (int y = start; y < end; ++y) {
+            size_t i = (size_t)y * SW + x;
+            if (distance < pb.clip_depth[i]) { pb.clip_depth[i] = distance; pb.meta[i] = (pb.meta[i] & ~META_WALL_MASK) | (unsigned)(wall + 1); }
+        }
+        sb.top_row = end > sb.top_row ? end : sb.top_row;
+        sb.top_depth = fmaxf(sb.top_depth, distance);
+    }
+}
+
+// engine.py:12637-12884
+__device__ void pass_paint(const ColumnCtx &cc, const ColumnState &c, const PassColumn &r, PixelBuffers &pb,
+                           const bool group_valid[3], const float group_bottom[3], i64 first_group_visibility) {
+    if (!(r.bits & PB_RASTER)) return;
+    const gd_map_desc *m = cc.m;
+    const LaneCtx &L = *cc.c;
+    const int x = cc.x, wi = r.wall, side = r.side;
+    const bool one_sided = r.bits & PB_ONE_SIDED;
+    const float ceiling_plane_bottom = fminf(r.clipped_top, c.floor_clip);
+    const float floor_plane_top = fmaxf(r.clipped_bottom, c.ceiling_clip);
+    const float *toff = m->side_off + (wi * 2 + side) * 2;
+    i64 h, swall;
+    texture_mapping(m, cc.recs[wi], wi, x, &h, &swall);
+    i64 repeat = round_to_i64(m->wall_len[wi] * 65536.0f);
+    if (side != 0) h = repeat - h;
+    if (cc.recs[wi].sl > 0 && h < 0) h = 0;
+    if (h >= repeat) h = repeat - 1;
+    i64 offx_fixed = round_to_i64(toff[0] * 65536.0f);
+    i64 u_base = (h + offx_fixed) >> 16;
+    const float4 wl = *reinterpret_cast<const float4 *>(m->walls + 4 * wi);
+    bool horizontal = fabsf(wl.w - wl.y) < 1e-6f, vertical = fabsf(wl.z - wl.x) < 1e-6f;
+    float fake_contrast = vertical ? 16.0f : (horizontal ? -16.0f : 0.0f);
+    float light = (m->sector_lights[r.render_current] + (float)(L.flash_light * 16)) + fake_contrast;
+    const i64 shade_own = wall_shade(light, r.visibility);
+    const i64 shade_group = wall_shade(light, first_group_visibility);
+    // every span of this pass lies inside the open window [ceiling_clip, floor_clip)
+    int y0 = c.ceiling_clip <= 0.0f ? 0 : (int)c.ceiling_clip;
+    int y1 = c.floor_clip >= (float)VH ? VH : (int)c.floor_clip;
+    const bool lower_on = !one_sided && (r.view_floor < r.other_floor);
+    const bool upper_on = !one_sided && (r.view_ceiling > r.other_ceiling);
+    for (int y = y0; y < y1; ++y) {
+        const float py = (float)y;
+        const size_t i = (size_t)y * SW + x;
+        unsigned int meta = pb.meta[i];
+        bool ceiling_span = (r.bits & PB_MARK_CEILING) && (py >= c.ceiling_clip) && (py < ceiling_plane_bottom);
+        bool floor_span = (r.bits & PB_MARK_FLOOR) && (py >= floor_plane_top) && (py < c.floor_clip);
+        bool meta_dirty = false;
+        if (((meta >> META_SECTOR_SHIFT) & META_SECTOR_MASK) == 0 && (ceiling_span || floor_span)) {
+            meta |= ((unsigned)(r.render_current + 1) << META_SECTOR_SHIFT) | (floor_span ? META_FLOOR : 0);
+            meta_dirty = true;
+        }
+        bool one_span = one_sided && (py >= r.clipped_top) && (py < r.clipped_bottom);
+        bool lower_span = lower_on && (py >= r.clipped_lower_top) && (py < r.clipped_bottom);
+        bool upper_span = upper_on && (py >= r.clipped_top) && (py < r.clipped_upper_bottom);
+        if (one_span || lower_span || upper_span) {
+            int texture_id = one_span ? r.side_tex[0] : (lower_span ? r.side_tex[1] : r.side_tex[2]);
+            if (texture_id >= 0 && !(meta & META_FILLED)) {
+                bool bottom_tail = (one_span && group_valid[0] && py >= group_bottom[0]) ||
+                                   (lower_span && group_valid[1] && py >= group_bottom[1]) ||
+                                   (upper_span && group_valid[2] && py >= group_bottom[2]);
+                int tw = m->tex_w[texture_id], th = m->tex_h[texture_id];
+                i64 tu = u_base & (i64)(tw - 1);   // floor-mod by a power of two
+                float origin_z = one_span ? r.view_ceiling : (lower_span ? r.other_floor : r.other_ceiling);
+                int height_bits = ilog2(th);
+                i64 vertical_step = mul64(swall, shl64(1, 14 - height_bits));
+                i64 screen_delta = (i64)y * FIXED_UNIT - L.center_fixed + FIXED_UNIT;
+                i64 texture_mid = round_to_i64((origin_z - L.view_z) * 65536.0f + toff[1] * 65536.0f);
+                i64 fraction = shl64(texture_mid, 16 - height_bits) + (mul64(vertical_step, screen_delta) >> 16);
+                i64 tv = (fraction & UINT32_MASK) >> (32 - height_bits);
+                unsigned char texel = m->tex_atlas[((size_t)texture_id * m->tex_max_h + tv) * m->tex_max_w + tu];
+                pb.frame[i] = m->colormap[(bottom_tail ? shade_group : shade_own) * 256 + texel];
+                if (r.distance < pb.clip_depth[i]) { pb.clip_depth[i] = r.distance; meta = (meta & ~META_WALL_MASK) | (unsigned)(wi + 1); }
+                meta |= META_FILLED;
+                meta_dirty = true;
+            }
+        }
+        if (meta_dirty) pb.meta[i] = meta;
+    }
+}
+
+// engine.py:12885-13371
+__device__ bool pass_advance(const ColumnCtx &cc, ColumnState &c, const PassColumn &r, PixelBuffers &pb, SilhouetteBounds &sb) {
+    const gd_map_desc *m = cc.m;
+    const MapView &mv = cc.mv;
+    const LaneCtx &L = *cc.c;
+    const ColumnState before = c;
+    const int x = cc.x;
+    const int cs = c.current_sector;
+    const int cur = cs < 0 ? 0 : cs;
+    const int wi = r.wall;
+    const float distance = r.distance;
+    const bool valid = r.bits & PB_VALID, raster_valid = r.bits & PB_RASTER, one_sided = r.bits & PB_ONE_SIDED;
+    auto incident = [&](int w) { return mv.sec(w, 0) == cur || mv.sec(w, 1) == cur; };
+    // o. clip updates (engine.py:12888-12913)
+    bool draws_upper = (r.view_ceiling > r.other_ceiling) && (r.side_tex[2] >= 0);
+    if (raster_valid && !one_sided && (draws_upper || (r.bits & PB_MARK_CEILING))) c.ceiling_clip = draws_upper ? r.clipped_upper_bottom : r.clipped_top;
+    bool draws_lower = (r.view_floor < r.other_floor) && (r.side_tex[1] >= 0);
+    if (raster_valid && !one_sided && (draws_lower || (r.bits & PB_MARK_FLOOR))) c.floor_clip = draws_lower ? r.clipped_lower_top : r.clipped_bottom;
+    // p. masked drawseg snapshot (engine.py:12914-12939)
+    if (raster_valid && !one_sided && (r.side_tex[0] >= 0) && (distance < c.masked_distance)) {
+        c.masked_ceiling_clip = c.ceiling_clip; c.masked_floor_clip = c.floor_clip; c.masked_distance = distance; c.masked_wall = wi;
+    }
+    // q. sprite silhouettes (engine.py:12943-12964)
+    if (raster_valid && !one_sided) {
+        bool masked_texture = r.side_tex[0] >= 0;
+        bool bottom_sil = (r.view_floor > r.other_floor) || (L.view_z < r.other_floor) || masked_texture;
+        bool top_sil = (r.view_ceiling < r.other_ceiling) || (L.view_z > r.other_ceiling) || masked_texture;
+        apply_silhouette(pb, sb, x, bottom_sil, top_sil, c.floor_clip, c.ceiling_clip, distance, wi);
+    }
+    // r. clips of the geometric portal behind a projected solid (engine.py:12969-13069)
+    if (r.bits & PB_PS_KEEPS) {
+        int path = r.ps_path_index;
+        const WallRec &pr = cc.recs[path];
+        int path_safe_other = r.ps_other < 0 ? 0 : r.ps_other;
+        float pof = m->sector_heights[2 * path_safe_other], poc = m->sector_heights[2 * path_safe_other + 1];
+        int pside = (r.bits & PB_PS_FROM_FRONT) ? 0 : 1;
+        const int *ptex = m->side_tex + (path * 2 + pside) * 3;
+        float path_top = project(L, pr, r.view_ceiling, x), path_bottom = project(L, pr, r.view_floor, x);
+        float path_lower_top = project(L, pr, pof, x), path_upper_bottom = project(L, pr, poc, x);
+        float pct = fmaxf(path_top, c.ceiling_clip);
+        float pcb = fminf(path_bottom, c.floor_clip);
+        float pcub = fmaxf(fminf(path_upper_bottom, c.floor_clip), pct);
+        float pclt = fminf(fmaxf(path_lower_top, c.ceiling_clip), pcb);
+        bool light_differs = m->sector_lights[r.render_current] != m->sector_lights[path_safe_other];
+        bool p_draws_upper = (r.view_ceiling > poc) && (ptex[2] >= 0);
+        bool p_marks_ceiling = (r.view_ceiling != poc) || (m->sector_ceil_tex[r.render_current] != m->sector_ceil_tex[path_safe_other]) || light_differs;
+        bool p_draws_lower = (r.view_floor < pof) && (ptex[1] >= 0);
+        bool p_marks_floor = (r.view_floor != pof) || (m->sector_floor_tex[r.render_current] != m->sector_floor_tex[path_safe_other]) || light_differs;
+        float new_ceiling = c.ceiling_clip, new_floor = c.floor_clip;
+        if (p_draws_upper || p_marks_ceiling) new_ceiling = p_draws_upper ? pcub : pct;
+        if (p_draws_lower || p_marks_floor) new_floor = p_draws_lower ? pclt : pcb;
+        c.ceiling_clip = new_ceiling; c.floor_clip = new_floor;
+        bool pmasked = ptex[0] >= 0;
+        bool pbottom = (r.view_floor > pof) || (L.view_z < pof) || pmasked;
+        bool ptop = (r.view_ceiling < poc) || (L.view_z > poc) || pmasked;
+        apply_silhouette(pb, sb, x, pbottom, ptop, c.floor_clip, c.ceiling_clip, r.ps_path_distance, path);
+    }
+    // s. next sector (engine.py:13070-13241)
+    const float prior = before.previous_distance;
+    const float prior_eps = prior + 1e-3f;
+    const bool geometric_intersection = r.bits & PB_GEOMETRIC;
+    bool endpoint_only_portal = valid && !one_sided && !geometric_intersection;
+    const int other_sector = r.other_sector;
+    float pd = prior;
+    int next_sector = -1;
+    bool endpoint_portal_bridge = false;
+    int ppb_idx = 0, gp_other = -1; float gpd = GD_INF;
+    if (endpoint_only_portal) {
+        auto other_incident = [&](int w) { return mv.sec(w, 0) == other_sector || mv.sec(w, 1) == other_sector; };
+        const float dist_eps = distance + 1e-3f;
+        float cnd = GD_INF, ond = GD_INF; int cni = 0x7fffffff, oni = 0x7fffffff;
+        float csd = GD_INF, osd = GD_INF;
+        int gpi = 0x7fffffff; float gp_along = 0.0f;
+        const int v0 = mv.vert(wi, 0), v1 = mv.vert(wi, 1);
+        for (int k = 0; k < cc.count; ++k) {
+            Cand q = cc.cand(k);
+            int w = q.wall; float d = q.dist;
+            bool os = mv.one_sided(w);
+            bool inc = incident(w), oinc = other_incident(w);
+            bool future = ((q.flags & CF_GEO) || os) && (d > dist_eps);
+            if (future) {
+                if (inc) take_min(d, w, cnd, cni);
+                if (oinc) take_min(d, w, ond, oni);
+            }
+            bool shares_endpoint = mv.vert(w, 0) == v0 || mv.vert(w, 0) == v1 || mv.vert(w, 1) == v0 || mv.vert(w, 1) == v1;
+            bool shared_solid = os && (shares_endpoint || (q.flags & CF_LEDGE)) && (d > prior_eps) && (d <= dist_eps);
+            if (shared_solid) {
+                if (inc && d < csd) csd = d;
+                if (oinc && d < osd) osd = d;
+            }
+            bool sgp = (q.flags & CF_GEO) && inc && shares_endpoint && !os && (d > prior_eps) && (fabsf(d - distance) <= (1.0f / 16.0f));
+            if (sgp && (d < gpd || (d == gpd && w < gpi))) { gpd = d; gpi = w; gp_along = q.along; }
+        }
+        if (!finitef(cnd)) cni = 0;
+        if (!finitef(ond)) oni = 0;
+        bool enters_tied_strip = finitef(cnd) && (cni == oni) && mv.opposing(wi, cni);
+        bool enters_other = (other_sector >= 0) && ((ond < cnd) || enters_tied_strip);
+        bool enters_shared = (other_sector >= 0) && (osd < csd);
+        bool uses_geometric_path = false;
+        if (finitef(gpd)) {
+            bool gp_from_front = cs == mv.sec(gpi, 0);
+            gp_other = gp_from_front ? mv.sec(gpi, 1) : mv.sec(gpi, 0);
+            uses_geometric_path = gp_other >= 0;
+            if (uses_geometric_path) {
+                int pb_slot = gp_along > 0.5f ? 1 : 0;
+                bool ppb_exists = mv.portal_bridge(pb_slot, gpi, wi, &ppb_idx);
+                if (ppb_exists) {
+                    Cand qb = cc.eval(ppb_idx);
+                    endpoint_portal_bridge = (qb.flags & CF_PROJ) && (qb.flags & CF_LEDGE) && (qb.dist > prior_eps) && (fabsf(qb.dist - gpd) <= tolerance_of(gpd));
+                }
+            }
+        }
+        // t. previous_distance (engine.py:13242-13262)
+        if (r.bits & PB_NO_KEEPS) pd = r.no_path_distance;
+        else if (r.bits & PB_PS_KEEPS) pd = r.ps_path_distance;
+        else if (enters_shared && (osd < distance)) pd = prior;
+        else if (uses_geometric_path) pd = gpd;
+        else pd = distance;
+        if (r.bits & PB_NO_KEEPS) next_sector = r.no_path_other;
+        else if (r.bits & PB_PS_KEEPS) next_sector = r.ps_other;
+        else if (uses_geometric_path) next_sector = gp_other;
+        else if (enters_other || enters_shared) next_sector = other_sector;
+        else next_sector = cs;
+    } else {
+        if (valid) {
+            if (r.bits & PB_NO_KEEPS) pd = r.no_path_distance;
+            else if (r.bits & PB_PS_KEEPS) pd = r.ps_path_distance;
+            else pd = distance;
+        }
+        if (r.bits & PB_NO_KEEPS) next_sector = r.no_path_other;
+        else if (r.bits & PB_PS_KEEPS) next_sector = r.ps_other;
+        else if (valid && !one_sided && geometric_intersection) next_sector = other_sector;
+        else next_sector = -1;
+    }
+    bool completes_pending_portal_bridge = valid && (before.flags & ST_PB) && (wi == before.pend_pb_index);
+    if (valid && endpoint_portal_bridge) pd = prior;
+    if (valid && completes_pending_portal_bridge) pd = fmaxf(distance, before.pend_pb_exit);
+    c.previous_distance = pd;
+    // carried state (engine.py:13276-13313, 13355-13371)
+    bool starts_po = r.bits & PB_REPLACE_NP;
+    if (starts_po) c.pend_po_vertex = r.sel_vertex;
+    bool po = starts_po || ((before.flags & ST_PO) && (r.bits & PB_CONTINUES_PO));
+    if (endpoint_only_portal) {
+        Cand cw = cc.eval(wi);
+        c.pend_ep_vertex = mv.vert(wi, cw.along <= 0.5f ? 0 : 1);
+        c.pend_ep_wall = wi;
+    }
+    if (r.bits & PB_FORWARD_BRIDGE) c.pend_eb_index = r.fb_idx;
+    if (endpoint_portal_bridge) next_sector = other_sector;
+    if (completes_pending_portal_bridge) next_sector = before.pend_pb_sector;
+    if (endpoint_portal_bridge) { c.pend_pb_index = ppb_idx; c.pend_pb_sector = gp_other; c.pend_pb_exit = gpd; }
+    c.flags = (po ? ST_PO : 0) | (endpoint_only_portal ? ST_EP : 0) | ((r.bits & PB_FORWARD_BRIDGE) ? ST_EB : 0) | (endpoint_portal_bridge ? ST_PB : 0);
+    c.current_sector = next_sector;
+    return !same_state(before, c);
+}
+
+// engine.py:13424-13744 for one column
+__device__ void masked_midtexture(const ColumnCtx &cc, const ColumnState &c, PixelBuffers &pb) {
+    const gd_map_desc *m = cc.m;
+    const MapView &mv = cc.mv;
+    const LaneCtx &L = *cc.c;
+    const int x = cc.x;
+    float md = GD_INF; int mw = 0x7fffffff; int mside = 0; int cand_flags = 0;
+    for (int k = 0; k < cc.count; ++k) {
+        Cand q = cc.cand(k);
+        int w = q.wall;
+        if (!(q.flags & CF_PROJ) || mv.one_sided(w)) continue;
+        const float4 wl = *reinterpret_cast<const float4 *>(m->walls + 4 * w);
+        float vx = wl.z - wl.x, vy = wl.w - wl.y;
+        float fx = L.x - wl.x, fy = L.y - wl.y;
+        int sidew = ((vx * fy - vy * fx) < 0) ? 0 : 1;
+        if (m->side_tex[(w * 2 + sidew) * 3] < 0) continue;
+        if (q.dist < md || (q.dist == md && w < mw)) { md = q.dist; mw = w; mside = sidew; cand_flags = q.flags; }
+    }
+    if (!finitef(md)) return;
+    int texture_id = m->side_tex[(mw * 2 + mside) * 3];
+    if (texture_id < 0) texture_id = 0;
+    bool left_edge = cand_flags & CF_LEDGE;
+    bool has_saved = c.masked_wall == mw;
+    if (!(has_saved || left_edge)) return;
+    const WallRec &wr = cc.recs[mw];
+    int front_sector = mv.sec(mw, 0), back_sector = mv.sec(mw, 1) < 0 ? 0 : mv.sec(mw, 1);
+    int light_sector = mside == 0 ? front_sector : back_sector;
+    float world_top = fminf(m->sector_heights[2 * front_sector + 1], m->sector_heights[2 * back_sector + 1]);
+    int tw = m->tex_w[texture_id], th = m->tex_h[texture_id];
+    float owall_top = project(L, wr, world_top, x);
+    float owall_bottom = project(L, wr, world_top - (float)th, x);
+    float mceil = fmaxf(owall_top, has_saved ? c.masked_ceiling_clip : 0.0f);
+    float mfloor = fminf(owall_bottom, has_saved ? c.masked_floor_clip : (float)VH);
+    const float *toff = m->side_off + (mw * 2 + mside) * 2;
+    i64 h, swall_cur;
+    texture_mapping(m, wr, mw, x, &h, &swall_cur);
+    i64 repeat = round_to_i64(m->wall_len[mw] * 65536.0f);
+    if (mside != 0) h = repeat - h;
+    i64 msl = wr.sl, msr = wr.sr;
+    if (msl > 0 && h < 0) h = 0;
+    if (h >= repeat) h = repeat - 1;
+    i64 offx = round_to_i64(toff[0] * 65536.0f);
+    i64 mu = ((h + offx) >> 16) & (i64)(tw - 1);
+    int height_bits = ilog2(th);
+    i64 vertical_step = mul64(swall_cur, shl64(1, 14 - height_bits));
+    i64 center_fixed = L.center_fixed;
+    i64 texture_mid = round_to_i64((world_top - L.view_z) * 65536.0f + toff[1] * 65536.0f);
+    int safe_left = (int)clampi(msl, 0, SW - 1), safe_last = (int)clampi(msr - 1, 0, SW - 1);
+    i64 dummy_h, start_swall, end_swall;
+    texture_mapping(m, wr, mw, safe_left, &dummy_h, &start_swall);
+    texture_mapping(m, wr, mw, safe_last, &dummy_h, &end_swall);
+    auto iscale_of = [](i64 swall) {
+        i64 s = mul64(swall, FIXED_UNIT) >> 18;
+        if (s >= 0 && s < 3) return (i64)3;
+        if (s > -3 && s < 0) return (i64)-3;
+        return s;
+    };
+    i64 start_scale = tdiv(1LL << 32, iscale_of(start_swall)), end_scale = tdiv(1LL << 32, iscale_of(end_swall));
+    i64 scale_step = tdiv(end_scale - start_scale, max64(msr - msl, 1));
+    i64 sprite_scale = start_scale + mul64(scale_step, (i64)x - msl);
+    i64 top_screen = center_fixed - (mul64(texture_mid, sprite_scale) >> 16);
+    i64 post_top = top_screen >> 16;
+    i64 post_bottom = ((top_screen + mul64(sprite_scale, th) - FIXED_UNIT) >> 16) + 1;
+    i64 clipped_top = max64(post_top, (i64)mceil);
+    i64 clipped_bottom = min64(post_bottom, (i64)mfloor);
+    i64 dc_iscale = mul64(swall_cur, FIXED_UNIT) >> 18;
+    bool initial_post = clipped_top < clipped_bottom;
+    i64 frac_start = texture_mid + mul64(clipped_top, dc_iscale) - (mul64(center_fixed - FIXED_UNIT, dc_iscale) >> 16);
+    i64 frac_end = frac_start + mul64(clipped_bottom - clipped_top - 1, dc_iscale);
+    bool extends = initial_post && ((float)clipped_bottom < mfloor) && (frac_end < (i64)th * FIXED_UNIT - dc_iscale);
+    clipped_bottom += extends ? 1 : 0;
+    const float4 wl = *reinterpret_cast<const float4 *>(m->walls + 4 * mw);
+    bool horizontal = fabsf(wl.w - wl.y) < 1e-6f, vertical = fabsf(wl.z - wl.x) < 1e-6f;
+    float contrast = vertical ? 16.0f : (horizontal ? -16.0f : 0.0f);
+    float light = (m->sector_lights[light_sector] + (float)(L.flash_light * 16)) + contrast;
+    i64 shade = wall_shade(light, wall_visibility(wr, mside, x));
+    int y0 = (int)clampi(clipped_top, 0, VH), y1 = (int)clampi(clipped_bottom, 0, VH);
+    for (int y = y0; y < y1; ++y) {
+        i64 screen_delta = (i64)y * FIXED_UNIT - center_fixed + FIXED_UNIT;
+        i64 fraction = shl64(texture_mid, 16 - height_bits) + (mul64(vertical_step, screen_delta) >> 16);
+        i64 mv_ = (fraction & UINT32_MASK) >> (32 - height_bits);
+        unsigned char texel = m->tex_atlas[((size_t)texture_id * m->tex_max_h + mv_) * m->tex_max_w + mu];
+        pb.frame[(size_t)y * SW + x] = m->colormap[shade * 256 + texel];
+    }
+}
+
+__global__ void __launch_bounds__(SW) wall_columns_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
+    const gd_map_desc *m = &dm.d;
+    const int local = blockIdx.x;
+    if (local >= lane_count) return;
+    __shared__ LaneCtx lane_ctx;
+    if (threadIdx.x == 0) lane_ctx = sc.ctx[local];
+    __syncthreads();
+    const int x = threadIdx.x;
+    ColumnCtx cc;
+    cc.m = m; cc.mv.m = m; cc.c = &lane_ctx;
+    cc.recs = sc.rec + (size_t)local * m->wall_count;
+    cc.list = sc.cand + (size_t)local * CAND_MAX * SW;
+    cc.count = sc.cand_count[(size_t)local * SW + x];
+    cc.x = x;
+    ray_direction(lane_ctx, x, &cc.rx, &cc.ry);
+    PixelBuffers pb;
+    pb.frame = frame_base + (size_t)local * frame_stride;
+    pb.meta = sc.meta + (size_t)local * VH * SW;
+    pb.clip_depth = sc.clip_depth + (size_t)local * VH * SW;
+    for (int y = 0; y < VH; ++y) { pb.meta[(size_t)y * SW + x] = 0; pb.clip_depth[(size_t)y * SW + x] = GD_INF; }
+    ColumnState st;
+    st.current_sector = lane_ctx.sector;
+    st.ceiling_clip = 0.0f; st.floor_clip = (float)VH;
+    st.masked_ceiling_clip = 0.0f; st.masked_floor_clip = (float)VH; st.masked_distance = GD_INF; st.masked_wall = -1;
+    st.previous_distance = 0.0f;
+    st.pend_po_vertex = -1; st.pend_ep_vertex = -1; st.pend_ep_wall = 0; st.pend_eb_index = 0;
+    st.pend_pb_index = 0; st.pend_pb_sector = -1; st.pend_pb_exit = 0.0f; st.flags = 0;
+    SilhouetteBounds sb; sb.bot_row = VH; sb.top_row = 0; sb.bot_depth = -GD_INF; sb.top_depth = -GD_INF;
+    bool boundary_has_po = false;
+    for (int k = 0; k < cc.count; ++k) if (cc.cand(k).flags & CF_LEDGE) { boundary_has_po = true; break; }
+    PassColumn pc;
+    bool done = false;
+    const int lane_id = threadIdx.x & 63;
+    const int group_base = lane_id & ~3;
+    const int sectors = m->sector_count;
+    for (int pass = 0; pass < sectors; ++pass) {
+        if (!done) pass_select(cc, st, boundary_has_po, pc);
+        // 4-column wallscan groups (engine.py:12688-12761): exchange with the aligned neighbours
+        bool same_group = true;
+        int w0 = __shfl(pc.wall, group_base), s0 = __shfl(pc.side, group_base);
+        bool all_tier[3] = {true, true, true};
+        float common_top[3] = {-GD_INF, -GD_INF, -GD_INF}, common_bottom[3] = {GD_INF, GD_INF, GD_INF};
+        for (int k = 0; k < 4; ++k) {
+            int src = group_base + k;
+            int qw = __shfl(pc.wall, src), qs = __shfl(pc.side, src), qb = __shfl(pc.bits, src);
+            float qt = __shfl(pc.clipped_top, src), qlt = __shfl(pc.clipped_lower_top, src);
+            float qbm = __shfl(pc.clipped_bottom, src), qub = __shfl(pc.clipped_upper_bottom, src);
+            same_group &= (qw == w0) && (qs == s0);
+            all_tier[0] &= (qb & PB_TIER0) != 0; all_tier[1] &= (qb & PB_TIER1) != 0; all_tier[2] &= (qb & PB_TIER2) != 0;
+            common_top[0] = fmaxf(common_top[0], qt); common_top[1] = fmaxf(common_top[1], qlt); common_top[2] = fmaxf(common_top[2], qt);
+            common_bottom[0] = fminf(common_bottom[0], qbm); common_bottom[1] = fminf(common_bottom[1], qbm); common_bottom[2] = fminf(common_bottom[2], qub);
+        }
+        int vis_lo = __shfl((int)(pc.visibility & 0xFFFFFFFFLL), group_base);
+        int vis_hi = __shfl((int)(pc.visibility >> 32), group_base);
+        i64 first_group_visibility = ((i64)vis_hi << 32) | (i64)(unsigned)vis_lo;
+        bool group_valid[3];
+        for (int t = 0; t < 3; ++t) group_valid[t] = same_group && all_tier[t] && (common_top[t] < common_bottom[t]);
+        if (!done) {
+            pass_paint(cc, st, pc, pb, group_valid, common_bottom, first_group_visibility);
+            bool changed = pass_advance(cc, st, pc, pb, sb);
+            // A pass that found nothing and changed nothing repeats identically for ever.
+            if (!(pc.bits & PB_VALID) && !changed) done = true;
+        }
+        if (__ballot(!done) == 0) break;
+    }
+    // exact planes (engine.py:13372-13422)
+    {
+        const float flat_center_px = (103.0f + lane_ctx.pitch_offset) + 0.5f;
+        const unsigned char *fflags = sc.flat_flags + (size_t)local * VH * SW;
+        for (int y = 0; y < VH; ++y) {
+            size_t i = (size_t)y * SW + x;
+            unsigned int meta = pb.meta[i];
+            int ps = (int)((meta >> META_SECTOR_SHIFT) & META_SECTOR_MASK) - 1;
+            if (ps < 0 || (meta & META_FILLED)) continue;
+            bool is_floor = meta & META_FLOOR;
+            pb.frame[i] = flat_pixel(m, lane_ctx, ps, is_floor, x, y);
+            // plane fallback occluder for sprites where the flat ray was unresolved.
+            // Bit 1|8 of flat_flags mark repaired pixels, whose surface depth is infinite.
+            if ((fflags[i] & 1) && !finitef(pb.clip_depth[i])) {
+                float plane_height = is_floor ? (lane_ctx.view_z - m->sector_heights[2 * ps]) : (m->sector_heights[2 * ps + 1] - lane_ctx.view_z);
+                float plane_denominator = fmaxf(fabsf((float)y - flat_center_px), 0.5f);
+                pb.clip_depth[i] = plane_height * 192.0f / plane_denominator;
+            }
+        }
+    }
+    masked_midtexture(cc, st, pb);
+}
+
+// ---------------------------------------------------------------------------------------------
+// sprites: engine.py:10534-10557 (blocking raycast) and 14684-14947
+// ---------------------------------------------------------------------------------------------
+struct SpriteRec {
+    float x, y, depth, light;
+    i64 depth_fixed, left, right, hstep, yscale, top_fixed, texmid, iscale;
+    int id, flags;   // bit0 alive, bit1 fullbright
+};
+
+__global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc,
+                                                            unsigned char *frame_base, size_t frame_stride) {
+    extern __shared__ unsigned char shared_raw[];
+    SpriteRec *sp = reinterpret_cast<SpriteRec *>(shared_raw);
+    const gd_map_desc *m = &dm.d;
+    const int local = blockIdx.x;
+    if (local >= lane_count) return;
+    const int n = lane_base + local;
+    const int A = lanes.sprite_slots;
+    const LaneCtx L = sc.ctx[local];
+    for (int a = threadIdx.x; a < A; a += blockDim.x) {
+        SpriteRec s;
+        size_t k = (size_t)n * A + a;
+        s.x = lanes.sprite_x[k]; s.y = lanes.sprite_y[k];
+        float z = lanes.sprite_z[k];
+        s.depth = lanes.sprite_depth[k]; s.id = lanes.sprite_id[k];
+        s.flags = (lanes.sprite_alive[k] ? 1 : 0) | ((lanes.sprite_fullbright && lanes.sprite_fullbright[k]) ? 2 : 0);
+        i64 ax = round_to_i64(s.x * 65536.0f), ay = round_to_i64(s.y * 65536.0f);
+        i64 rx = ax - L.view_x_fixed, ry = ay - L.view_y_fixed;
+        s.depth_fixed = (rx * L.vcos + ry * L.vsin) >> 20;
+        i64 side_fixed = (rx * L.vsin - ry * L.vcos) >> 16;
+        i64 xscale = tdiv(FOCAL_X_FIXED << 12, max64(s.depth_fixed, SPRITE_MIN_DEPTH_FIXED));
+        i64 left_fixed = side_fixed - (i64)m->spr_left[s.id] * FIXED_UNIT;
+        s.left = SW / 2 + (mul64(left_fixed, xscale) >> 32);
+        i64 right_fixed = left_fixed + (i64)m->spr_w[s.id] * FIXED_UNIT;
+        s.right = SW / 2 + (mul64(right_fixed, xscale) >> 32);
+        s.hstep = tdiv((i64)m->spr_w[s.id] << 16, max64(s.right - s.left, 1));
+        s.yscale = tdiv(FOCAL_Y_FIXED << 12, max64(s.depth_fixed, SPRITE_MIN_DEPTH_FIXED));
+        s.texmid = (i64)m->spr_top[s.id] * FIXED_UNIT - round_to_i64((L.view_z - z) * 65536.0f);
+        s.top_fixed = L.center_fixed - (mul64(s.texmid, s.yscale) >> 16);
+        s.iscale = tdiv(UINT32_MASK, max64(s.yscale, 1));
+        s.light = m->sector_lights[sector_at(m, s.x, s.y)];
+        sp[a] = s;
+    }
+    __syncthreads();
+    const int x = threadIdx.x;
+    const WallRec *recs = sc.rec + (size_t)local * m->wall_count;
+    unsigned char *frame = frame_base + (size_t)local * frame_stride;
+    const unsigned int *meta = sc.meta + (size_t)local * VH * SW;
+    const float *clip_depth = sc.clip_depth + (size_t)local * VH * SW;
+    // nearest blocking linedef of this column (engine.py:10534-10557)
+    float rx, ry; ray_direction(L, x, &rx, &ry);
+    float best = GD_INF; int slot = 0;
+    for (int b = 0; b < m->blocking_count; ++b) {
+        const float4 wl = *reinterpret_cast<const float4 *>(m->walls + 4 * m->blocking_walls[b]);
+        float segx = wl.z - wl.x, segy = wl.w - wl.y;
+        float offx = wl.x - L.x, offy = wl.y - L.y;
+        float den = rx * segy - ry * segx;
+        bool ok = fabsf(den) >= 1e-6f;
+        float safe = ok ? den : 1.0f;
+        float d = (offx * segy - offy * segx) / safe;
+        float a = (offx * ry - offy * rx) / safe;
+        bool valid = ok && (d > 0) && (a >= 0) && (a <= 1);
+        if (valid && d < best) { best = d; slot = b; }
+    }
+    float wall_distance = fminf(fmaxf(best, 1.0f), 4096.0f);
+    int bw = m->blocking_count ? m->blocking_walls[slot] : 0;
+    const WallRec &bg = recs[bw];
+    i64 bnear = min64(bg.dl, bg.dr), bfar = max64(bg.dl, bg.dr);
+    const float4 bl = *reinterpret_cast<const float4 *>(m->walls + 4 * bw);
+    float bdx = bl.z - bl.x, bdy = bl.w - bl.y;
+    bool owns = (x >= bg.sl) && (x < bg.sr);
+    // painter's order far -> near: repeatedly take the farthest candidate nearer than the last one
+    float last_depth = GD_INF; int last_slot = A;
+    for (;;) {
+        float pick_depth = -GD_INF; int pick = -1;
+        for (int a = 0; a < A; ++a) {
+            const SpriteRec &s = sp[a];
+            if (!((s.flags & 1) && (x >= s.left) && (x < s.right) && (s.depth > 0))) continue;
+            // strictly before (last_depth, last_slot) in (depth, slot) order
+            if (!(s.depth < last_depth || (s.depth == last_depth && a < last_slot))) continue;
+            if (s.depth > pick_depth || (s.depth == pick_depth && a > pick)) {
+                bool ray_visible = s.depth < wall_distance;
+                if (!ray_visible) {
+                    float bside = bdx * (s.y - bl.y) - bdy * (s.x - bl.x);
+                    bool behind = (bnear > s.depth_fixed) || ((bfar > s.depth_fixed) && (bside <= 0));
+                    ray_visible = !owns || behind;
+                }
+                if (ray_visible) { pick_depth = s.depth; pick = a; }
+            }
+        }
+        if (pick < 0) break;
+        last_depth = pick_depth; last_slot = pick;
+        const SpriteRec &s = sp[pick];
+        int width = m->spr_w[s.id], height = m->spr_h[s.id];
+        i64 su = mul64((i64)x - s.left, s.hstep) >> 16;
+        if (!(su >= 0 && su < width)) continue;
+        float light = s.light + (float)(L.flash_light * 16);
+        if (s.flags & 2) light = 255.0f;
+        float base_shade = 61.0f - light / 4.0f;
+        float visibility = fminf(1280.0f / fmaxf(s.depth, 1.0f), 24.0f);
+        i64 shade = clampi((i64)floorf(base_shade - visibility), 0, 31);
+        i64 fraction_base = s.texmid - (mul64(L.center_fixed - FIXED_UNIT, s.iscale) >> 16);
+        for (int y = 0; y < VH; ++y) {
+            i64 sv = (fraction_base + mul64((i64)y, s.iscale)) >> 16;
+            if (!(sv >= 0 && sv < height)) continue;
+            size_t i = (size_t)y * SW + x;
+            int cw = (int)(meta[i] & META_WALL_MASK) - 1;
+            bool visible;
+            if (cw >= 0) {
+                const WallRec &cg = recs[cw];
+                i64 cnear = min64(cg.dl, cg.dr), cfar = max64(cg.dl, cg.dr);
+                const float4 cl = *reinterpret_cast<const float4 *>(m->walls + 4 * cw);
+                float side = (cl.z - cl.x) * (s.y - cl.y) - (cl.w - cl.y) * (s.x - cl.x);
+                visible = (cnear > s.depth_fixed) || ((cfar > s.depth_fixed) && (side <= 0));
+            } else {
+                visible = s.depth < clip_depth[i];
+            }
+            if (!visible) continue;
+            size_t t = ((size_t)s.id * m->spr_max_h + sv) * m->spr_max_w + su;
+            if (!m->spr_opaque[t]) continue;
+            i64 post_screen_top = (s.top_fixed + mul64(s.yscale, m->spr_post_top[t])) >> 16;
+            if ((i64)y < post_screen_top) continue;
+            frame[i] = m->colormap[shade * 256 + m->spr_atlas[t]];
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// observation: _triton_kernels.py:120-177 + engine.py:9545-9548 / 2443-2450
+// ---------------------------------------------------------------------------------------------
+__global__ void observe_kernel(const unsigned char *indexed, size_t lane_stride, int source_rows, const unsigned char *playpal,
+                               int lane_count, unsigned char *obs, unsigned char *frames, const unsigned char *reset_mask) {
+    __shared__ unsigned char pal[768];
+    for (int k = threadIdx.x; k < 768; k += blockDim.x) pal[k] = playpal[k];
+    __syncthreads();
+    int pixel = blockIdx.x * blockDim.x + threadIdx.x;
+    int n = blockIdx.y;
+    if (n >= lane_count || pixel >= GD_OBS_SIZE * GD_OBS_SIZE) return;
+    int oy = pixel / GD_OBS_SIZE, ox = pixel - oy * GD_OBS_SIZE;
+    const unsigned char *src = indexed + (size_t)n * lane_stride;
+    int y_start = oy * 240, y_end = y_start + 240, x_start = ox * 320, x_end = x_start + 320;
+    int rs = 0, gs = 0, bs = 0;
+    for (int sy = 0; sy < 4; ++sy) {
+        int source_y = y_start / 84 + sy;
+        int y_overlap = min(y_end, (source_y + 1) * 84) - max(y_start, source_y * 84);
+        if (source_y >= source_rows || y_overlap <= 0) continue;
+        for (int sx = 0; sx < 5; ++sx) {
+            int source_x = x_start / 84 + sx;
+            int x_overlap = min(x_end, (source_x + 1) * 84) - max(x_start, source_x * 84);
+            if (source_x >= 320 || x_overlap <= 0) continue;
+            int weight = (y_overlap * x_overlap) / 48;
+            int p = src[source_y * SW + source_x] * 3;
+            rs += pal[p] * weight; gs += pal[p + 1] * weight; bs += pal[p + 2] * weight;
+        }
+    }
+    int r = (rs + 800) / 1600, g = (gs + 800) / 1600, b = (bs + 800) / 1600;
+    unsigned char gray = (unsigned char)((r * 77 + g * 150 + b * 29 + 128) >> 8);
+    const size_t F = (size_t)GD_OBS_SIZE * GD_OBS_SIZE;
+    if (obs) obs[(size_t)n * F + pixel] = gray;
+    if (frames) {
+        unsigned char *stack = frames + (size_t)n * GD_FRAME_STACK * F + pixel;
+        if (reset_mask && reset_mask[n]) {
+            for (int k = 0; k < GD_FRAME_STACK; ++k) stack[k * F] = gray;
+        } else {
+            for (int k = 0; k < GD_FRAME_STACK - 1; ++k) stack[k * F] = stack[(k + 1) * F];
+            stack[(GD_FRAME_STACK - 1) * F] = gray;
+        }
+    }
+}
+
+// engine.py:15381-15384
+__global__ void expand_rgb_kernel(const unsigned char *indexed, const unsigned char *playpal, size_t pixels, unsigned char *rgb) {
+    __shared__ unsigned char pal[768];
+    for (int k = threadIdx.x; k < 768; k += blockDim.x) pal[k] = playpal[k];
+    __syncthreads();
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= pixels) return;
+    int p = indexed[i] * 3;
+    rgb[i * 3] = pal[p]; rgb[i * 3 + 1] = pal[p + 1]; rgb[i * 3 + 2] = pal[p + 2];
+}
+
+// ---------------------------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------------------------
+thread_local std::string g_error;
+
+int fail(int code, const std::string &message) { g_error = message; return code; }
+
+#define HIP_TRY(expr)                                                                          \
+    do {                                                                                       \
+        hipError_t e_ = (expr);                                                                \
+        if (e_ != hipSuccess) return fail(GD_E_HIP, std::string(#expr) + ": " + hipGetErrorString(e_)); \
+    } while (0)
+
+}  // namespace
+
+struct gd_renderer {
+    DeviceMap dm;
+    Scratch sc;
+    int chunk_lanes;
+    std::vector<void *> allocations;
+    hipEvent_t events[16];
+    bool events_ready;
+};
+
+namespace {
+
+template <typename T>
+int upload(gd_renderer *r, const T *host, size_t count, const T **device) {
+    if (count == 0) count = 1;
+    void *ptr = nullptr;
+    HIP_TRY(hipMalloc(&ptr, count * sizeof(T)));
+    r->allocations.push_back(ptr);
+    if (host) HIP_TRY(hipMemcpy(ptr, host, count * sizeof(T), hipMemcpyHostToDevice));
+    else HIP_TRY(hipMemset(ptr, 0, count * sizeof(T)));
+    *device = static_cast<const T *>(ptr);
+    return GD_OK;
+}
+
+template <typename T>
+int scratch_alloc(gd_renderer *r, size_t count, T **device) {
+    void *ptr = nullptr;
+    HIP_TRY(hipMalloc(&ptr, (count ? count : 1) * sizeof(T)));
+    r->allocations.push_back(ptr);
+    *device = static_cast<T *>(ptr);
+    return GD_OK;
+}
+
+void build_fine_tables(std::vector<i64> &sine, std::vector<i64> &tangent) {
+    // engine.py:309-328
+    const double PI = 3.14159265358979323846;
+    sine.assign(FINE_ANGLES, 0);
+    tangent.assign(FINE_ANGLES / 2, 0);
+    const int quarter = FINE_ANGLES / 4;
+    for (int i = 0; i < quarter; ++i) sine[i] = (i64)std::trunc(std::sin((double)i * (2.0 * PI / FINE_ANGLES)) * 65536.0);
+    for (int i = 0; i < quarter; ++i) sine[quarter + i] = sine[quarter - 1 - i];
+    for (int i = 0; i < 2 * quarter; ++i) sine[2 * quarter + i] = -sine[i];
+    sine[quarter] = 65536;
+    sine[3 * quarter] = -65536;
+    for (int i = 0; i < FINE_ANGLES / 2; ++i) {
+        double phase = ((double)i - FINE_ANGLES / 4) * (2.0 * PI / FINE_ANGLES);
+        if (i == 0) phase += PI / FINE_ANGLES;
+        tangent[i] = (i64)std::trunc(std::tan(phase) * 65536.0 + 0.5);
+    }
+}
+
+const int STAGE_COUNT = 8;
+
+int launch_chunk(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_out *out, int base, int count, hipStream_t stream, bool timed) {
+    const gd_map_desc &m = r->dm.d;
+    unsigned char *frame_base;
+    size_t frame_stride = (size_t)GD_SCREEN_HEIGHT * SW;
+    if (out->indexed) frame_base = out->indexed + (size_t)base * frame_stride;
+    else frame_base = r->sc.frame;
+    int stage = 0;
+    auto mark = [&]() { if (timed) (void)hipEventRecord(r->events[stage], stream); ++stage; };
+    mark();
+    hipLaunchKernelGGL(lane_setup_kernel, dim3((count + 63) / 64), dim3(64), 0, stream, r->dm, *lanes, base, count, r->sc);
+    hipLaunchKernelGGL(wall_setup_kernel, dim3((m.wall_count + 127) / 128, count), dim3(128), 0, stream, r->dm, count, r->sc);
+    mark();
+    hipLaunchKernelGGL(column_lists_kernel, dim3(count), dim3(SW), 0, stream, r->dm, count, r->sc);
+    mark();
+    hipLaunchKernelGGL(flat_select_kernel, dim3((VH * SW + 255) / 256, count), dim3(256), 0, stream, r->dm, *lanes, base, count, r->sc);
+    mark();
+    hipLaunchKernelGGL(flat_finish_kernel, dim3(count), dim3(SW), 0, stream, r->dm, count, r->sc, frame_base, frame_stride);
+    mark();
+    hipLaunchKernelGGL(wall_columns_kernel, dim3(count), dim3(SW), 0, stream, r->dm, count, r->sc, frame_base, frame_stride);
+    mark();
+    if (lanes->sprite_slots > 0 && lanes->sprite_x) {
+        size_t shared = (size_t)lanes->sprite_slots * sizeof(SpriteRec);
+        hipLaunchKernelGGL(sprite_columns_kernel, dim3(count), dim3(SW), shared, stream, r->dm, *lanes, base, count, r->sc, frame_base, frame_stride);
+    }
+    mark();
+    if (out->obs || out->frames) {
+        const size_t F = (size_t)GD_OBS_SIZE * GD_OBS_SIZE;
+        hipLaunchKernelGGL(observe_kernel, dim3((GD_OBS_SIZE * GD_OBS_SIZE + 255) / 256, count), dim3(256), 0, stream,
+                           frame_base, frame_stride, VH, m.playpal, count, out->obs ? out->obs + (size_t)base * F : nullptr,
+                           out->frames ? out->frames + (size_t)base * GD_FRAME_STACK * F : nullptr,
+                           out->reset_mask ? out->reset_mask + base : nullptr);
+    }
+    if (out->rgb) {
+        size_t pixels = (size_t)count * frame_stride;
+        hipLaunchKernelGGL(expand_rgb_kernel, dim3((unsigned)((pixels + 255) / 256)), dim3(256), 0, stream, frame_base, m.playpal, pixels,
+                           out->rgb + (size_t)base * frame_stride * 3);
+    }
+    mark();
+    HIP_TRY(hipGetLastError());
+    return GD_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *gd_version(void) { return "gradoom_amd 0.1.0 (gfx950)"; }
+const char *gd_last_error(void) { return g_error.c_str(); }
+
+int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int32_t max_lanes, gd_renderer **out) {
+    if (!h || !out || !cosine_correction) return fail(GD_E_ARG, "null argument");
+    if (max_lanes <= 0) return fail(GD_E_ARG, "max_lanes must be positive");
+    if (h->wall_count <= 0 || h->sector_count <= 0) return fail(GD_E_ARG, "empty map");
+    if (h->wall_count >= 65535) return fail(GD_E_ARG, "at most 65534 linedefs");
+    if (h->sector_count >= 16383) return fail(GD_E_ARG, "at most 16382 sectors");
+    gd_renderer *r = new (std::nothrow) gd_renderer();
+    if (!r) return fail(GD_E_ARG, "out of host memory");
+    r->events_ready = false;
+    std::memset(&r->sc, 0, sizeof(r->sc));
+    r->dm.d = *h;
+    gd_map_desc &d = r->dm.d;
+    const size_t W = h->wall_count, S = h->sector_count, V = h->vertex_count, K = h->neighbor_slots;
+    int rc = GD_OK;
+#define UP(field, count) if (rc == GD_OK) rc = upload(r, h->field, (size_t)(count), &d.field)
+    UP(walls, W * 4); UP(walls_fixed, W * 4); UP(wall_sectors, W * 2); UP(wall_vertex, W * 2);
+    UP(side_tex, W * 6); UP(side_off, W * 4); UP(wall_len, W);
+    UP(endpoint_neighbors, W * K); UP(endpoint_neighbor_starts, W * K); UP(endpoint_neighbor_ends, W * K);
+    UP(solid_bridge_start_ofs, W + 1); UP(solid_bridge_start_idx, h->solid_bridge_start_ofs[W]);
+    UP(solid_bridge_end_ofs, W + 1); UP(solid_bridge_end_idx, h->solid_bridge_end_ofs[W]);
+    UP(vertex_wall_ofs, V + 1); UP(vertex_wall_idx, h->vertex_wall_ofs[V]);
+    UP(sector_wall_ofs, S + 1); UP(sector_wall_idx, h->sector_wall_ofs[S]);
+    UP(sector_edge_ofs, S + 1); UP(sector_edge_idx, h->sector_edge_ofs[S]);
+    UP(blocking_walls, h->blocking_count);
+    const size_t cells = (size_t)h->grid_nx * h->grid_ny;
+    const size_t items = h->grid_cell_ofs[cells];
+    UP(grid_cell_ofs, cells + 1); UP(grid_item_sector, items); UP(grid_item_edge_ofs, items + 1);
+    UP(grid_item_edges, h->grid_item_edge_ofs[items]);
+    UP(floor_levels, h->floor_level_count); UP(ceil_levels, h->ceil_level_count);
+    UP(sector_heights, S * 2); UP(sector_lights, S); UP(sector_floor_tex, S); UP(sector_ceil_tex, S);
+    const size_t texels = (size_t)h->texture_count * h->tex_max_h * h->tex_max_w;
+    UP(tex_atlas, texels); UP(tex_w, h->texture_count); UP(tex_h, h->texture_count);
+    UP(playpal, 768); UP(colormap, 34 * 256);
+    const size_t sprels = (size_t)h->sprite_count * h->spr_max_h * h->spr_max_w;
+    UP(spr_atlas, sprels); UP(spr_opaque, sprels); UP(spr_post_top, sprels);
+    UP(spr_w, h->sprite_count); UP(spr_h, h->sprite_count); UP(spr_left, h->sprite_count); UP(spr_top, h->sprite_count);
+#undef UP
+    std::vector<i64> sine, tangent;
+    build_fine_tables(sine, tangent);
+    if (rc == GD_OK) rc = upload(r, sine.data(), sine.size(), &r->dm.fine_sine);
+    if (rc == GD_OK) rc = upload(r, tangent.data(), tangent.size(), &r->dm.fine_tangent);
+    if (rc == GD_OK) rc = upload(r, cosine_correction, (size_t)SW, &r->dm.cosine_correction);
+    // Working memory for one chunk of lanes; larger batches are rendered chunk by chunk.
+    const int chunk = max_lanes < 1024 ? max_lanes : 1024;
+    r->chunk_lanes = chunk;
+    const size_t L = chunk, PX = (size_t)VH * SW;
+    if (rc == GD_OK) rc = scratch_alloc(r, L, &r->sc.ctx);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * W, &r->sc.rec);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * W, &r->sc.visible);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * CAND_MAX * SW, &r->sc.cand);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * SW, &r->sc.cand_count);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &r->sc.flat_sector);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &r->sc.flat_flags);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &r->sc.meta);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &r->sc.clip_depth);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)GD_SCREEN_HEIGHT * SW, &r->sc.frame);
+    if (rc == GD_OK) rc = scratch_alloc(r, 1, &r->sc.status);
+    if (rc == GD_OK && hipMemset(r->sc.status, 0, sizeof(int)) != hipSuccess) rc = fail(GD_E_HIP, "hipMemset status");
+    if (rc == GD_OK) {
+        for (int i = 0; i < 16; ++i) if (hipEventCreate(&r->events[i]) != hipSuccess) rc = fail(GD_E_HIP, "hipEventCreate");
+        r->events_ready = rc == GD_OK;
+    }
+    if (rc != GD_OK) { std::string keep = g_error; gd_renderer_destroy(r); g_error = keep; return rc; }
+    *out = r;
+    return GD_OK;
+}
+
+void gd_renderer_destroy(gd_renderer *r) {
+    if (!r) return;
+    for (void *ptr : r->allocations) (void)hipFree(ptr);
+    if (r->events_ready) for (int i = 0; i < 16; ++i) (void)hipEventDestroy(r->events[i]);
+    delete r;
+}
+
+static int check_render_args(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_out *out) {
+    if (!r || !lanes || !out) return fail(GD_E_ARG, "null argument");
+    if (lanes->lane_count < 0) return fail(GD_E_ARG, "negative lane count");
+    if (!lanes->x || !lanes->y || !lanes->angle || !lanes->view_z || !lanes->x_fixed || !lanes->y_fixed || !lanes->angle_bam ||
+        !lanes->pitch_bam || !lanes->ray_cos || !lanes->ray_sin)
+        return fail(GD_E_ARG, "missing lane tensor");
+    if (lanes->sprite_slots < 0 || lanes->sprite_slots > 512) return fail(GD_E_ARG, "sprite_slots must be in [0, 512]");
+    if (lanes->sprite_slots > 0 && lanes->sprite_x &&
+        (!lanes->sprite_y || !lanes->sprite_z || !lanes->sprite_depth || !lanes->sprite_id || !lanes->sprite_alive))
+        return fail(GD_E_ARG, "missing sprite tensor");
+    return GD_OK;
+}
+
+int gd_render(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_out *out, void *stream) {
+    int rc = check_render_args(r, lanes, out);
+    if (rc != GD_OK) return rc;
+    for (int base = 0; base < lanes->lane_count; base += r->chunk_lanes) {
+        int count = lanes->lane_count - base < r->chunk_lanes ? lanes->lane_count - base : r->chunk_lanes;
+        rc = launch_chunk(r, lanes, out, base, count, static_cast<hipStream_t>(stream), false);
+        if (rc != GD_OK) return rc;
+    }
+    return GD_OK;
+}
+
+int gd_render_timed(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_out *out, void *stream, int32_t launches, float *ms, int32_t stage_count) {
+    int rc = check_render_args(r, lanes, out);
+    if (rc != GD_OK) return rc;
+    if (!ms || stage_count < STAGE_COUNT - 1 || launches <= 0) return fail(GD_E_ARG, "ms must hold 7 stage times");
+    for (int s = 0; s < stage_count; ++s) ms[s] = 0.0f;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    for (int it = 0; it < launches; ++it) {
+        for (int base = 0; base < lanes->lane_count; base += r->chunk_lanes) {
+            int count = lanes->lane_count - base < r->chunk_lanes ? lanes->lane_count - base : r->chunk_lanes;
+            rc = launch_chunk(r, lanes, out, base, count, st, true);
+            if (rc != GD_OK) return rc;
+            HIP_TRY(hipEventSynchronize(r->events[STAGE_COUNT - 1]));
+            for (int s = 0; s + 1 < STAGE_COUNT; ++s) {
+                float t = 0.0f;
+                HIP_TRY(hipEventElapsedTime(&t, r->events[s], r->events[s + 1]));
+                ms[s] += t;
+            }
+        }
+    }
+    for (int s = 0; s + 1 < STAGE_COUNT; ++s) ms[s] /= (float)launches;
+    return GD_OK;
+}
+
+/* Sticky status bits of the renderer (synchronises the device): bit0 = a column had more than
+   CAND_MAX candidate linedefs and its list was truncated. Replaces nothing in the reference. */
+int gd_renderer_status(gd_renderer *r, int32_t *status) {
+    if (!r || !status) return fail(GD_E_ARG, "null argument");
+    int value = 0;
+    HIP_TRY(hipMemcpy(&value, r->sc.status, sizeof(int), hipMemcpyDeviceToHost));
+    *status = value;
+    return GD_OK;
+}
+
+int gd_observe(const uint8_t *indexed, int32_t source_rows, const uint8_t *playpal, int32_t lane_count,
+               uint8_t *obs, uint8_t *frames, const uint8_t *reset_mask, void *stream) {
+    if (!indexed || !playpal) return fail(GD_E_ARG, "null argument");
+    if (source_rows != 208 && source_rows != 240) return fail(GD_E_ARG, "indexed must have 208 or 240 rows");
+    if (lane_count < 0) return fail(GD_E_ARG, "negative lane count");
+    if (lane_count == 0 || (!obs && !frames)) return GD_OK;
+    for (int base = 0; base < lane_count; base += 32768) {
+        int count = lane_count - base < 32768 ? lane_count - base : 32768;
+        const size_t F = (size_t)GD_OBS_SIZE * GD_OBS_SIZE;
+        hipLaunchKernelGGL(observe_kernel, dim3((GD_OBS_SIZE * GD_OBS_SIZE + 255) / 256, count), dim3(256), 0, static_cast<hipStream_t>(stream),
+                           indexed + (size_t)base * source_rows * SW, (size_t)source_rows * SW, source_rows, playpal, count,
+                           obs ? obs + (size_t)base * F : nullptr, frames ? frames + (size_t)base * GD_FRAME_STACK * F : nullptr,
+                           reset_mask ? reset_mask + base : nullptr);
+    }
+    HIP_TRY(hipGetLastError());
+    return GD_OK;
+}
+
+int gd_expand_rgb24(const uint8_t *indexed, int32_t rows, const uint8_t *playpal, int32_t lane_count, uint8_t *rgb, void *stream) {
+    if (!indexed || !playpal || !rgb) return fail(GD_E_ARG, "null argument");
+    if (rows <= 0 || lane_count < 0) return fail(GD_E_ARG, "bad shape");
+    size_t pixels = (size_t)lane_count * rows * SW;
+    if (pixels == 0) return GD_OK;
+    const size_t step = (size_t)1 << 30;
+    for (size_t base = 0; base < pixels; base += step) {
+        size_t count = pixels - base < step ? pixels - base : step;
+        hipLaunchKernelGGL(expand_rgb_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                           indexed + base, playpal, count, rgb + base * 3);
+    }
+    HIP_TRY(hipGetLastError());
+    return GD_OK;
+}
+
+}  // extern "C"

@@ -144,7 +144,19 @@ def build_map_tables(smap) -> dict[str, np.ndarray | int]:
     rows = np.arange(spr_opaque.shape[1], dtype=np.int64)[None, :, None]
     spr_post_top = np.maximum.accumulate(np.where(starts, rows, 0), axis=1).astype(np.uint8)
 
+    grid = build_sector_grid(walls, sector_edge_ofs, sector_edge_idx, sector_count)
+    heights = np.ascontiguousarray(smap.sector_heights, dtype=np.float32)
+    # Plane levels in the order that makes plane height (and so ray distance) ascend:
+    # floors from the highest down, ceilings from the lowest up.
+    floor_levels = np.unique(heights[:, 0])[::-1].astype(np.float32).copy()
+    ceil_levels = np.unique(heights[:, 1]).astype(np.float32).copy()
+
     return dict(
+        floor_level_count=int(len(floor_levels)),
+        ceil_level_count=int(len(ceil_levels)),
+        floor_levels=floor_levels,
+        ceil_levels=ceil_levels,
+        **grid,
         wall_count=wall_count,
         sector_count=sector_count,
         vertex_count=vertex_count,
@@ -194,4 +206,84 @@ def build_map_tables(smap) -> dict[str, np.ndarray | int]:
         spr_h=np.ascontiguousarray(smap.sprite_heights, dtype=np.int32),
         spr_left=np.ascontiguousarray(smap.sprite_left_offsets, dtype=np.int32),
         spr_top=np.ascontiguousarray(smap.sprite_top_offsets, dtype=np.int32),
+    )
+
+
+GRID_CELL = 64.0
+GRID_PAD = 0.5
+
+
+def build_sector_grid(walls, sector_edge_ofs, sector_edge_idx, sector_count, cell: float = GRID_CELL) -> dict:
+    """Uniform grid of candidate (sector, edge sub-list) pairs for the even-odd polygon test.
+
+    The reference tests a point against every edge of every sector
+    (``engine.py:9598-9617`` and ``engine.py:10994-11015``).  An edge can only be
+    counted for a point ``(px, py)`` when ``py`` lies between its endpoints' y and
+    ``px < crossing_x <= max(x1, x2)`` (up to float32 rounding, covered by the
+    pad), and a sector whose boundary is a set of closed loops can only have odd
+    parity when ``px`` is not left of all its edges.  A cell therefore lists, per
+    sector whose padded bounding box meets it, exactly the edges that can be
+    counted for points inside the cell; the parity over that sub-list equals the
+    parity over the full edge list.  Sectors with an open boundary are treated
+    as unbounded on the left.
+    """
+
+    all_x = walls[:, (0, 2)]
+    all_y = walls[:, (1, 3)]
+    min_x = float(np.floor(all_x.min() - 2 * GRID_PAD))
+    min_y = float(np.floor(all_y.min() - 2 * GRID_PAD))
+    nx = int(np.ceil((float(all_x.max()) + 2 * GRID_PAD - min_x) / cell)) + 1
+    ny = int(np.ceil((float(all_y.max()) + 2 * GRID_PAD - min_y) / cell)) + 1
+    cell_rows: list[list[tuple[int, list[int]]]] = [[] for _ in range(nx * ny)]
+    for s in range(sector_count):
+        edges = sector_edge_idx[sector_edge_ofs[s] : sector_edge_ofs[s + 1]]
+        if len(edges) == 0:
+            continue
+        ex = walls[edges][:, (0, 2)]
+        ey = walls[edges][:, (1, 3)]
+        degree: dict[tuple[float, float], int] = {}
+        for w in edges:
+            for slot in range(2):
+                key = (float(walls[w, 2 * slot]) + 0.0, float(walls[w, 2 * slot + 1]) + 0.0)
+                degree[key] = degree.get(key, 0) + 1
+        closed = all(count % 2 == 0 for count in degree.values())
+        sx0 = -np.inf if not closed else float(ex.min()) - GRID_PAD
+        sx1 = float(ex.max()) + GRID_PAD
+        sy0 = float(ey.min()) - GRID_PAD
+        sy1 = float(ey.max()) + GRID_PAD
+        ix0 = 0 if not closed else max(int(np.floor((sx0 - min_x) / cell)), 0)
+        ix1 = min(int(np.floor((sx1 - min_x) / cell)), nx - 1)
+        iy0 = max(int(np.floor((sy0 - min_y) / cell)), 0)
+        iy1 = min(int(np.floor((sy1 - min_y) / cell)), ny - 1)
+        edge_max_x = ex.max(axis=1)
+        edge_min_y = ey.min(axis=1)
+        edge_max_y = ey.max(axis=1)
+        for iy in range(iy0, iy1 + 1):
+            cy0 = min_y + iy * cell - GRID_PAD
+            cy1 = min_y + (iy + 1) * cell + GRID_PAD
+            row_mask = (edge_max_y >= cy0) & (edge_min_y <= cy1)
+            for ix in range(ix0, ix1 + 1):
+                cx0 = (min_x + ix * cell - GRID_PAD) if ix > 0 else -np.inf
+                keep = row_mask & (edge_max_x >= cx0)
+                cell_rows[iy * nx + ix].append((s, [int(w) for w in edges[keep]]))
+    cell_ofs = np.zeros(nx * ny + 1, dtype=np.int32)
+    item_sector: list[int] = []
+    item_edge_ofs = [0]
+    item_edges: list[int] = []
+    for c, row in enumerate(cell_rows):
+        for s, sub in row:  # sectors were appended in ascending order
+            item_sector.append(s)
+            item_edges.extend(sub)
+            item_edge_ofs.append(len(item_edges))
+        cell_ofs[c + 1] = len(item_sector)
+    return dict(
+        grid_nx=nx,
+        grid_ny=ny,
+        grid_min_x=min_x,
+        grid_min_y=min_y,
+        grid_cell=float(cell),
+        grid_cell_ofs=cell_ofs,
+        grid_item_sector=np.asarray(item_sector if item_sector else [0], dtype=np.int32),
+        grid_item_edge_ofs=np.asarray(item_edge_ofs, dtype=np.int32),
+        grid_item_edges=np.asarray(item_edges if item_edges else [0], dtype=np.int32),
     )

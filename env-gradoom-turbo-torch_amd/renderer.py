@@ -1,0 +1,235 @@
+"""Torch-facing front end of the HIP renderer.
+
+Mirrors the seam the reference's environment plugs a renderer into
+(``/root/reference/src/gradoom/env.py:444-447``): ``render_frame() -> uint8 [N,84,84]``,
+``render_native_frame(include_hud) -> uint8 [N,240,320,3]``, and the engine-owned
+``frames`` stack updated by ``_finish_observation`` (``engine.py:9545-9548``) or filled
+on reset (``engine.py:2443-2450``).  Tensors stay Torch (ROCm) tensors; this module only
+passes their device pointers and the current stream through the C ABI.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import dataclasses
+
+import numpy as np
+import torch
+
+from . import _abi, _lib, hostmath, mapbuild
+
+STAGES = ("wall_setup", "column_lists", "flat_select", "flat_finish", "wall_columns", "sprite_columns", "observe")
+
+
+@dataclasses.dataclass
+class LaneState:
+    """Per-lane camera tensors, named like the reference engine's own attributes."""
+
+    x: torch.Tensor  # f32 [N]
+    y: torch.Tensor
+    angle: torch.Tensor
+    view_z: torch.Tensor
+    x_fixed: torch.Tensor  # i64 [N] (engine._x_fixed)
+    y_fixed: torch.Tensor
+    angle_bam: torch.Tensor  # i64 [N] (engine._angle_bam)
+    pitch_bam: torch.Tensor
+    flash_light: torch.Tensor  # i64 [N]
+    sprite_x: torch.Tensor | None = None  # f32 [N,A]
+    sprite_y: torch.Tensor | None = None
+    sprite_z: torch.Tensor | None = None
+    sprite_id: torch.Tensor | None = None  # i32 [N,A]
+    sprite_alive: torch.Tensor | None = None  # bool/u8 [N,A]
+    sprite_fullbright: torch.Tensor | None = None
+    # Optional overrides of the Torch-computed float32 inputs (golden fixtures carry the
+    # reference's own CPU values so that parity is independent of the Torch build).
+    ray_cos: torch.Tensor | None = None
+    ray_sin: torch.Tensor | None = None
+    sprite_depth: torch.Tensor | None = None
+
+    @classmethod
+    def from_numpy(cls, arrays: dict, device) -> "LaneState":
+        def get(name, dtype):
+            value = arrays.get(name)
+            if value is None:
+                return None
+            return torch.as_tensor(np.ascontiguousarray(value)).to(device=device, dtype=dtype).contiguous()
+
+        return cls(
+            x=get("x", torch.float32), y=get("y", torch.float32), angle=get("angle", torch.float32),
+            view_z=get("view_z", torch.float32), x_fixed=get("x_fixed", torch.int64), y_fixed=get("y_fixed", torch.int64),
+            angle_bam=get("angle_bam", torch.int64), pitch_bam=get("pitch_bam", torch.int64),
+            flash_light=get("flash_light", torch.int64), sprite_x=get("sprite_x", torch.float32),
+            sprite_y=get("sprite_y", torch.float32), sprite_z=get("sprite_z", torch.float32),
+            sprite_id=get("sprite_id", torch.int32), sprite_alive=get("sprite_alive", torch.uint8),
+            sprite_fullbright=get("sprite_fullbright", torch.uint8), ray_cos=get("ray_cos", torch.float32),
+            ray_sin=get("ray_sin", torch.float32), sprite_depth=get("sprite_depth", torch.float32),
+        )
+
+
+def _require(tensor: torch.Tensor, name: str, dtype, shape, device) -> torch.Tensor:
+    # Same error classes as the reference's tensor validation (env.py:711-728).
+    if not isinstance(tensor, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if tensor.device != device:
+        raise TypeError(f"{name} must be on {device}, got {tensor.device}")
+    if tensor.dtype != dtype:
+        raise TypeError(f"{name} must have dtype {dtype}, got {tensor.dtype}")
+    if tuple(tensor.shape) != tuple(shape):
+        raise ValueError(f"{name} must have shape {tuple(shape)}, got {tuple(tensor.shape)}")
+    if not tensor.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    return tensor
+
+
+class HipRenderer:
+    """Owns a ``gd_renderer`` for one map on one device."""
+
+    def __init__(self, smap, max_lanes: int, device="cuda:0", *, cosine_correction=None, tables=None):
+        self.device = torch.device(device)
+        if self.device.type != "cuda":
+            raise RuntimeError("HipRenderer needs a ROCm device; there is no CPU fallback")
+        self._lib = _lib.library()
+        self.tables = mapbuild.build_map_tables(smap) if tables is None else tables
+        self.max_lanes = int(max_lanes)
+        if cosine_correction is None:
+            cosine_correction = hostmath.cosine_correction("cpu").numpy()
+        self._cosine = np.ascontiguousarray(cosine_correction, dtype=np.float32)
+        if self._cosine.shape != (_abi.SCREEN_WIDTH,):
+            raise ValueError("cosine_correction must hold 320 floats")
+        self.ray_offsets = hostmath.native_ray_offsets("cpu").to(self.device)
+        self.playpal = torch.as_tensor(self.tables["playpal"]).to(self.device).contiguous()
+        desc, keep = _abi.host_map_desc(self.tables)
+        handle = C.c_void_p()
+        with torch.cuda.device(self.device):
+            _lib.check(self._lib.gd_renderer_create(C.byref(desc), self._cosine.ctypes.data, self.max_lanes, C.byref(handle)))
+        del keep
+        self._handle = handle
+
+    def close(self) -> None:
+        if getattr(self, "_handle", None):
+            self._lib.gd_renderer_destroy(self._handle)
+            self._handle = None
+
+    def __del__(self):  # pragma: no cover
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def status(self) -> int:
+        value = C.c_int32()
+        _lib.check(self._lib.gd_renderer_status(self._handle, C.byref(value)))
+        return int(value.value)
+
+    # ------------------------------------------------------------------ descriptors
+    def _lanes_desc(self, lanes: LaneState):
+        count = int(lanes.x.shape[0])
+        device = self.device
+        keep = []
+        desc = _abi.LanesDesc()
+        desc.lane_count = count
+        for name in ("x", "y", "angle", "view_z"):
+            setattr(desc, name, _require(getattr(lanes, name), name, torch.float32, (count,), device).data_ptr())
+        for name in ("x_fixed", "y_fixed", "angle_bam", "pitch_bam", "flash_light"):
+            setattr(desc, name, _require(getattr(lanes, name), name, torch.int64, (count,), device).data_ptr())
+        if lanes.ray_cos is None or lanes.ray_sin is None:
+            ray_cos, ray_sin = hostmath.ray_tables(lanes.angle, self.ray_offsets)
+        else:
+            ray_cos, ray_sin = lanes.ray_cos, lanes.ray_sin
+        keep += [ray_cos, ray_sin]
+        desc.ray_cos = _require(ray_cos, "ray_cos", torch.float32, (count, 320), device).data_ptr()
+        desc.ray_sin = _require(ray_sin, "ray_sin", torch.float32, (count, 320), device).data_ptr()
+        desc.sprite_slots = 0
+        if lanes.sprite_x is not None and lanes.sprite_x.shape[1] > 0:
+            slots = int(lanes.sprite_x.shape[1])
+            desc.sprite_slots = slots
+            for name in ("sprite_x", "sprite_y", "sprite_z"):
+                setattr(desc, name, _require(getattr(lanes, name), name, torch.float32, (count, slots), device).data_ptr())
+            desc.sprite_id = _require(lanes.sprite_id, "sprite_id", torch.int32, (count, slots), device).data_ptr()
+            alive = lanes.sprite_alive
+            if alive.dtype == torch.bool:
+                alive = alive.to(torch.uint8)
+            keep.append(alive)
+            desc.sprite_alive = _require(alive, "sprite_alive", torch.uint8, (count, slots), device).data_ptr()
+            if lanes.sprite_fullbright is not None:
+                bright = lanes.sprite_fullbright
+                if bright.dtype == torch.bool:
+                    bright = bright.to(torch.uint8)
+                keep.append(bright)
+                desc.sprite_fullbright = _require(bright, "sprite_fullbright", torch.uint8, (count, slots), device).data_ptr()
+            depth = lanes.sprite_depth
+            if depth is None:
+                depth = hostmath.sprite_depth(lanes.x, lanes.y, lanes.angle, lanes.sprite_x, lanes.sprite_y)
+            keep.append(depth)
+            desc.sprite_depth = _require(depth, "sprite_depth", torch.float32, (count, slots), device).data_ptr()
+        return desc, keep
+
+    def _out_desc(self, count, indexed, obs, frames, reset_mask, rgb):
+        device = self.device
+        out = _abi.FrameOut()
+        keep = []
+        if indexed is not None:
+            out.indexed = _require(indexed, "indexed", torch.uint8, (count, 240, 320), device).data_ptr()
+        if obs is not None:
+            out.obs = _require(obs, "obs", torch.uint8, (count, 84, 84), device).data_ptr()
+        if frames is not None:
+            out.frames = _require(frames, "frames", torch.uint8, (count, 4, 84, 84), device).data_ptr()
+        if reset_mask is not None:
+            mask = reset_mask.to(torch.uint8) if reset_mask.dtype == torch.bool else reset_mask
+            keep.append(mask)
+            out.reset_mask = _require(mask, "reset_mask", torch.uint8, (count,), device).data_ptr()
+        if rgb is not None:
+            out.rgb = _require(rgb, "rgb", torch.uint8, (count, 240, 320, 3), device).data_ptr()
+        return out, keep
+
+    # ------------------------------------------------------------------ entry points
+    def render(self, lanes: LaneState, *, indexed=None, obs=None, frames=None, reset_mask=None, rgb=None) -> None:
+        """One frame for every lane, written into the given (preallocated) tensors."""
+
+        if self._handle is None:
+            raise RuntimeError("renderer is closed")
+        desc, keep_lanes = self._lanes_desc(lanes)
+        out, keep_out = self._out_desc(desc.lane_count, indexed, obs, frames, reset_mask, rgb)
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        _lib.check(self._lib.gd_render(self._handle, C.byref(desc), C.byref(out), C.c_void_p(stream)))
+        del keep_lanes, keep_out
+
+    def render_timed(self, lanes: LaneState, launches: int, *, indexed=None, obs=None, frames=None) -> dict[str, float]:
+        """Average milliseconds per launch of each kernel stage (HIP events on the current stream)."""
+
+        desc, keep_lanes = self._lanes_desc(lanes)
+        out, keep_out = self._out_desc(desc.lane_count, indexed, obs, frames, None, None)
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        times = (C.c_float * len(STAGES))()
+        _lib.check(
+            self._lib.gd_render_timed(self._handle, C.byref(desc), C.byref(out), C.c_void_p(stream), int(launches), times, len(STAGES))
+        )
+        del keep_lanes, keep_out
+        return {name: float(times[i]) for i, name in enumerate(STAGES)}
+
+    def observe(self, indexed: torch.Tensor, *, obs=None, frames=None, reset_mask=None) -> None:
+        """Observation pipeline on an existing ``[N,208|240,320]`` indexed frame."""
+
+        if indexed.ndim != 3 or tuple(indexed.shape[1:]) not in ((208, 320), (240, 320)):
+            raise ValueError("indexed must have shape (N, 208, 320) or (N, 240, 320)")
+        if indexed.dtype != torch.uint8:
+            raise TypeError("indexed must be a uint8 tensor")
+        count, rows = int(indexed.shape[0]), int(indexed.shape[1])
+        out, keep = self._out_desc(count, None, obs, frames, reset_mask, None)
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        _lib.check(
+            self._lib.gd_observe(
+                indexed.contiguous().data_ptr(), rows, self.playpal.data_ptr(), count, out.obs, out.frames, out.reset_mask,
+                C.c_void_p(stream),
+            )
+        )
+        del keep
+
+    def expand_rgb24(self, indexed: torch.Tensor, rgb: torch.Tensor) -> None:
+        count, rows = int(indexed.shape[0]), int(indexed.shape[1])
+        _require(indexed, "indexed", torch.uint8, (count, rows, 320), self.device)
+        _require(rgb, "rgb", torch.uint8, (count, rows, 320, 3), self.device)
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        _lib.check(
+            self._lib.gd_expand_rgb24(indexed.data_ptr(), rows, self.playpal.data_ptr(), count, rgb.data_ptr(), C.c_void_p(stream))
+        )

@@ -53,6 +53,9 @@ typedef struct gd_map_desc {
     int32_t blocking_count;  /* B one-sided / blocking linedefs */
     int32_t neighbor_slots;  /* K columns of endpoint_neighbors */
     int32_t direct_neighbors;/* 1: every linedef has <=1 start and <=1 end neighbour (engine.py:1558) */
+    int32_t floor_level_count, ceil_level_count; /* distinct plane heights */
+    int32_t grid_nx, grid_ny;/* point-location grid (cells of grid_cell map units) */
+    float grid_min_x, grid_min_y, grid_cell;
 
     const float *walls;              /* [W,4] x1,y1,x2,y2 (portal_walls) */
     const int32_t *walls_fixed;      /* [W,4] rint(walls*65536) (engine.py:10876) */
@@ -75,6 +78,14 @@ typedef struct gd_map_desc {
     const int32_t *sector_edge_ofs;  /* [S+1] CSR rows of sector_edge_mask (scenario.py:906-916) */
     const int32_t *sector_edge_idx;
     const int32_t *blocking_walls;   /* [B] linedef index of each blocking segment, ascending */
+    /* Point-location grid: the even-odd polygon tests of engine.py:9598-9617 and
+       10994-11015 restricted, per cell, to the sectors and edges that can count there. */
+    const int32_t *grid_cell_ofs;    /* [nx*ny+1] -> items */
+    const int32_t *grid_item_sector; /* [items] ascending sector id within a cell */
+    const int32_t *grid_item_edge_ofs;/* [items+1] -> grid_item_edges */
+    const int32_t *grid_item_edges;  /* linedef ids */
+    const float *floor_levels;       /* [floor_level_count] distinct floor heights, descending */
+    const float *ceil_levels;        /* [ceil_level_count] distinct ceiling heights, ascending */
 
     const float *sector_heights;     /* [S,2] floor, ceiling */
     const float *sector_lights;      /* [S] */
@@ -136,12 +147,15 @@ const char *gd_version(void);
 const char *gd_last_error(void);
 
 /*
- * Upload an immutable map (host pointers in `host_map`) to the current HIP
- * device and size per-lane scratch for `max_lanes`.
+ * Upload an immutable map (HOST pointers in `host_map`) to the current HIP
+ * device and allocate working memory for batches of up to `max_lanes` lanes
+ * (larger batches are rendered in chunks).  `cosine_correction` is a host
+ * array of 320 floats, cos(native_ray_offsets) (engine.py:10967), computed by
+ * the caller with Torch like every other float32 transcendental input.
  * Replaces DeviceScenario.from_host + the engine ctor precompute
  * (engine.py:721-1476, 1527-1634).
  */
-int gd_renderer_create(const gd_map_desc *host_map, int32_t max_lanes, gd_renderer **out);
+int gd_renderer_create(const gd_map_desc *host_map, const float *cosine_correction, int32_t max_lanes, gd_renderer **out);
 void gd_renderer_destroy(gd_renderer *r);
 
 /*
@@ -154,6 +168,13 @@ void gd_renderer_destroy(gd_renderer *r);
  * No allocation, no host synchronisation.
  */
 int gd_render(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_out *out, void *stream);
+
+/*
+ * Sticky status bits (synchronises the device).  bit0: some screen column had
+ * more candidate linedefs than the library keeps and was truncated - the frame
+ * of that lane is not trustworthy.  Replaces nothing in the reference.
+ */
+int gd_renderer_status(gd_renderer *r, int32_t *status);
 
 /*
  * Observation pipeline alone on an existing indexed frame.

@@ -23,6 +23,9 @@
 #include "../include/gradoom_amd.h"
 
 #include <algorithm>
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
 #include <cmath>
 #include <cstdint>
 #include <cstring>
@@ -1501,7 +1504,11 @@ int gdo_render(const gd_map_desc *map, const gd_lanes_desc *lanes, const gd_fram
     const size_t W = map->wall_count;
     std::vector<uint8_t> obs(size_t(GD_OBS_SIZE) * GD_OBS_SIZE);
     std::vector<uint8_t> full(size_t(GD_SCREEN_HEIGHT) * SW);
+    const bool profile = std::getenv("GDO_PROFILE") != nullptr;
+    double t_setup = 0, t_flats = 0, t_walls = 0, t_sprites = 0, t_obs = 0;
+    auto now = [] { return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count(); };
     for (int n = lane_begin; n < lane_end; ++n) {
+        double t0 = now();
         o.setup_lane(lanes, n);
         for (int w = 0; w < o.W; ++w) {
             o.wall_geometry(w);
@@ -1510,7 +1517,9 @@ int gdo_render(const gd_map_desc *map, const gd_lanes_desc *lanes, const gd_fram
         }
         o.portal_intersections();
         o.texture_mapping();
+        double t1 = now();
         o.render_flats(lanes->ray_cos + size_t(n) * SW, lanes->ray_sin + size_t(n) * SW, cosine_correction);
+        double t2 = now();
         const bool tap = dbg && dbg->debug_lane == n;
         if (dbg && dbg->sector) dbg->sector[n] = o.L.sector;
         if (tap) {
@@ -1532,7 +1541,9 @@ int gdo_render(const gd_map_desc *map, const gd_lanes_desc *lanes, const gd_fram
             if (dbg->visibility) for (int x = 0; x < SW; ++x) for (size_t w = 0; w < W; ++w) for (int s = 0; s < 2; ++s)
                 dbg->visibility[(size_t(x) * W + w) * 2 + s] = o.visibility_at(int(w), s, x);
         }
+        double t3 = now();
         o.render_portal_walls();
+        double t4 = now();
         if (tap) {
             const size_t PX = size_t(VH) * SW;
             if (dbg->scene_depth) std::memcpy(dbg->scene_depth, o.scene_depth.data(), PX * 4);
@@ -1540,7 +1551,10 @@ int gdo_render(const gd_map_desc *map, const gd_lanes_desc *lanes, const gd_fram
             if (dbg->sprite_clip_wall) std::memcpy(dbg->sprite_clip_wall, o.sprite_clip_wall.data(), PX * 4);
             if (dbg->walls_frame) std::memcpy(dbg->walls_frame, o.frame.data(), PX);
         }
+        double t5 = now();
         o.render_sprites(lanes, n);
+        double t6 = now();
+        t_setup += t1 - t0; t_flats += t2 - t1; t_walls += t4 - t3; t_sprites += t6 - t5;
         std::memcpy(full.data(), o.frame.data(), size_t(VH) * SW);
         std::memset(full.data() + size_t(VH) * SW, 0, size_t(GD_SCREEN_HEIGHT - VH) * SW);
         if (out->indexed) std::memcpy(out->indexed + size_t(n) * full.size(), full.data(), full.size());
@@ -1554,6 +1568,7 @@ int gdo_render(const gd_map_desc *map, const gd_lanes_desc *lanes, const gd_fram
             for (size_t i = 0; i < full.size(); ++i) for (int c = 0; c < 3; ++c) rgb[i * 3 + c] = map->playpal[full[i] * 3 + c];
         }
     }
+    if (profile) std::fprintf(stderr, "oracle lanes %d: setup %.3fs flats %.3fs walls %.3fs sprites %.3fs\n", lane_end - lane_begin, t_setup, t_flats, t_walls, t_sprites);
     return GD_OK;
 }
 

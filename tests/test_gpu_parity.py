@@ -1,0 +1,77 @@
+"""HIP path against the reference's golden vectors and against the CPU oracle (needs an MI355X)."""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import fixture_names, lane_inputs, load_fixture
+
+pytestmark = pytest.mark.gpu
+
+
+def _renderer(name):
+    from gradoom_amd.renderer import HipRenderer, LaneState
+
+    meta, data, smap, tables = load_fixture(name)
+    renderer = HipRenderer(smap, meta["lanes"], "cuda:0", cosine_correction=data["cosine_correction"], tables=tables)
+    lanes = LaneState.from_numpy(lane_inputs(data), "cuda:0")
+    return meta, data, tables, renderer, lanes
+
+
+@pytest.mark.parametrize("name", fixture_names())
+def test_indexed_frame_bit_exact_vs_reference_golden(name):
+    print(f"case {name}", flush=True)
+    meta, data, _tables, renderer, lanes = _renderer(name)
+    count = meta["lanes"]
+    indexed = torch.zeros((count, 240, 320), dtype=torch.uint8, device="cuda:0")
+    obs = torch.zeros((count, 84, 84), dtype=torch.uint8, device="cuda:0")
+    renderer.render(lanes, indexed=indexed, obs=obs)
+    torch.cuda.synchronize()
+    assert renderer.status() == 0
+    ours = indexed.cpu().numpy()
+    mismatched = int((ours != data["indexed"]).sum())
+    assert mismatched == 0, f"{mismatched} palette indices differ from the reference"
+    delta = np.abs(obs.cpu().numpy().astype(np.int32) - data["obs"].astype(np.int32))
+    assert delta.max() <= 1 and delta.mean() < 0.01  # tolerance: tests/test_rendering.py:138-139
+    renderer.close()
+
+
+@pytest.mark.parametrize("name", ["config1", "small_midtex_sprites"])
+def test_observation_and_stack_bit_exact_vs_oracle(oracle, name):
+    meta, data, tables, renderer, lanes = _renderer(name)
+    count = meta["lanes"]
+    rng = np.random.default_rng(3)
+    start = rng.integers(0, 256, (count, 4, 84, 84), dtype=np.uint8)
+    mask = (rng.random(count) < 0.4).astype(np.uint8)
+    expected = oracle.render(tables, lane_inputs(data), data["cosine_correction"], frames=start, reset_mask=mask, want_rgb=True)
+    indexed = torch.zeros((count, 240, 320), dtype=torch.uint8, device="cuda:0")
+    obs = torch.zeros((count, 84, 84), dtype=torch.uint8, device="cuda:0")
+    frames = torch.as_tensor(start).to("cuda:0")
+    rgb = torch.zeros((count, 240, 320, 3), dtype=torch.uint8, device="cuda:0")
+    renderer.render(lanes, indexed=indexed, obs=obs, frames=frames, reset_mask=torch.as_tensor(mask).to("cuda:0"), rgb=rgb)
+    torch.cuda.synchronize()
+    assert np.array_equal(indexed.cpu().numpy(), expected["indexed"])
+    assert np.array_equal(obs.cpu().numpy(), expected["obs"])
+    assert np.array_equal(frames.cpu().numpy(), expected["frames"])
+    assert np.array_equal(rgb.cpu().numpy(), expected["rgb"])
+    assert np.array_equal(rgb[0].cpu().numpy(), data["rgb_lane0"])
+    renderer.close()
+
+
+def test_observe_entry_point_matches_oracle(oracle):
+    _meta, _data, _tables, renderer, _lanes = _renderer("tiny_stages")
+    rng = np.random.default_rng(11)
+    for rows in (208, 240):
+        indexed = rng.integers(0, 256, (5, rows, 320), dtype=np.uint8)
+        start = rng.integers(0, 256, (5, 4, 84, 84), dtype=np.uint8)
+        mask = np.asarray([1, 0, 0, 1, 0], dtype=np.uint8)
+        expected_obs, expected_frames = oracle.observe(indexed, renderer.tables["playpal"], frames=start, reset_mask=mask)
+        obs = torch.zeros((5, 84, 84), dtype=torch.uint8, device="cuda:0")
+        frames = torch.as_tensor(start).to("cuda:0")
+        renderer.observe(torch.as_tensor(indexed).to("cuda:0"), obs=obs, frames=frames, reset_mask=torch.as_tensor(mask).to("cuda:0"))
+        torch.cuda.synchronize()
+        assert np.array_equal(obs.cpu().numpy(), expected_obs)
+        assert np.array_equal(frames.cpu().numpy(), expected_frames)
+    renderer.close()
