@@ -1,0 +1,165 @@
+"""Headline benchmark: rendered lane-frames/s (320x240 indexed + 84x84x4 observation) on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config4] [--lanes N] [--no-cpu]
+
+A step is one pass of the whole hot path over one batch of lanes whose inputs already sit in
+HBM: sector-light flicker update, the Torch float32 ray / sprite-depth tables, the render
+kernel chain and the fused observation + frame-stack update.  Camera poses and sprite lists
+change every step.  One JSON line is printed (see README of the contract in DESIGN.md).
+"""
+
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+POSE_SETS = 4
+
+
+def algorithmic_bytes_per_lane_frame(sprites: int, map_bytes: int, lanes: int) -> float:
+    # 320x240 u8 frame write + 4x84x84 stack write + 3 older stack frames read
+    # + lane pose (64 B) + 24 B per sprite + the shared map/atlas bytes once per launch.
+    return 76800 + 28224 + 21168 + 64 + 24 * sprites + map_bytes / lanes
+
+
+def main() -> int:
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=10)
+    parser.add_argument("--warmup", type=int, default=2)
+    parser.add_argument("--workload", default="config4")
+    parser.add_argument("--lanes", type=int, default=None)
+    parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    parser.add_argument("--cpu-lanes", type=int, default=12, help="lanes of the same workload the CPU baseline renders")
+    args = parser.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: lanes are independent and this build has no multi-GPU path; run with --gpus 1", file=sys.stderr)
+        return 2
+
+    import torch
+
+    import __graft_entry__ as entry
+
+    entry.load_package()
+    from gradoom_amd import hostmath, mapbuild, synthmap
+    from gradoom_amd.renderer import STAGES, HipRenderer, LaneState
+    from gradoom_amd.selfcheck import make_lane_arrays
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a ROCm device", file=sys.stderr)
+        return 2
+    device = torch.device("cuda:0")
+    cfg = synthmap.CONFIGS[args.workload]
+    lanes = args.lanes or cfg["lanes"]
+    sprites = cfg["sprites"]
+    smap = synthmap.generate_config_map(args.workload)
+    tables = mapbuild.build_map_tables(smap)
+    cosine = hostmath.cosine_correction("cpu").numpy()
+    renderer = HipRenderer(smap, lanes, device, cosine_correction=cosine, tables=tables)
+
+    # Resident inputs: a few pose/sprite sets cycled step by step, plus flicker light vectors.
+    states = []
+    for k in range(POSE_SETS):
+        poses = synthmap.generate_poses_batch(smap, lanes, 100 + k, flash=True)
+        spr = synthmap.generate_sprites_batch(smap, lanes, sprites, 100 + k) if sprites else None
+        bam = torch.as_tensor(poses.angle_bam, dtype=torch.int64)
+        arrays = dict(
+            x=poses.x, y=poses.y, angle=hostmath.angle_from_bam(bam).numpy(), view_z=poses.view_z,
+            x_fixed=np.rint(poses.x.astype(np.float64) * 65536).astype(np.int64),
+            y_fixed=np.rint(poses.y.astype(np.float64) * 65536).astype(np.int64),
+            angle_bam=poses.angle_bam, pitch_bam=poses.pitch_bam, flash_light=poses.flash_light,
+        )
+        if spr is not None:
+            arrays.update(sprite_x=spr.x, sprite_y=spr.y, sprite_z=spr.z, sprite_id=spr.sprite,
+                          sprite_alive=spr.alive.astype(np.uint8), sprite_fullbright=spr.fullbright.astype(np.uint8))
+        states.append(LaneState.from_numpy(arrays, device))
+    rng = np.random.default_rng(7)
+    base_lights = tables["sector_lights"]
+    flicker = [
+        torch.as_tensor(np.clip(base_lights + rng.integers(-16, 17, len(base_lights)), 0, 255).astype(np.float32)).to(device)
+        for _ in range(POSE_SETS)
+    ]
+    indexed = torch.zeros((lanes, 240, 320), dtype=torch.uint8, device=device)
+    obs = torch.zeros((lanes, 84, 84), dtype=torch.uint8, device=device)
+    frames = torch.zeros((lanes, 4, 84, 84), dtype=torch.uint8, device=device)
+
+    def step(k: int) -> None:
+        renderer.set_sector_lights(flicker[k % POSE_SETS])
+        renderer.render(states[k % POSE_SETS], indexed=indexed, obs=obs, frames=frames)
+
+    for k in range(args.warmup):
+        step(k)
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    for k in range(args.steps):
+        step(args.warmup + k)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - started
+    if renderer.status() != 0:
+        print("renderer reported truncated column lists: result invalid", file=sys.stderr)
+        return 1
+    value = lanes * args.steps / elapsed
+
+    # Per-kernel durations with HIP events on the launch stream, same inputs, same region.
+    stage_launches = max(2, min(args.steps, 5))
+    stage_ms = renderer.render_timed(states[0], stage_launches, indexed=indexed, obs=obs, frames=frames)
+    torch.cuda.synchronize()
+    dominant = max(stage_ms, key=stage_ms.get)
+    chunk = min(lanes, 1024)
+    chunks = (lanes + chunk - 1) // chunk
+    map_bytes = sum(int(np.asarray(v).nbytes) for v in tables.values() if isinstance(v, np.ndarray))
+    bytes_per_lane = algorithmic_bytes_per_lane_frame(sprites, map_bytes, lanes)
+    # render_timed sums a stage over the chunks of one frame; one launch handles `chunk` lanes
+    launch_ms = stage_ms[dominant] / chunks
+    achieved = bytes_per_lane * chunk / (launch_ms * 1e-3) / 1e9 if launch_ms > 0 else 0.0
+    roofline = dict(
+        bound="hbm", kernel=dominant + "_kernel", achieved=round(achieved, 3), peak=HBM_PEAK_GBPS, unit="GB/s",
+        frac=round(achieved / HBM_PEAK_GBPS, 6), traffic=None, launch_ms=round(launch_ms, 4),
+        stage_ms_per_frame={name: round(ms, 4) for name, ms in stage_ms.items()},
+        whole_path_frac=round(value * bytes_per_lane / 1e9 / HBM_PEAK_GBPS, 6),
+        bytes_per_lane_frame=round(bytes_per_lane, 1),
+    )
+
+    cpu_baseline = None
+    if not args.no_cpu:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import oracle  # CPU restatement of the reference algorithm: the reported baseline only
+
+        sample = max(1, min(args.cpu_lanes, lanes))
+        poses = synthmap.generate_poses_batch(smap, sample, 100, flash=True)
+        spr = synthmap.generate_sprites_batch(smap, sample, sprites, 100) if sprites else None
+        arrays = make_lane_arrays(smap, poses, spr)
+        oracle.library()
+        cpu_started = time.perf_counter()
+        oracle.render(tables, arrays, cosine, frames=np.zeros((sample, 4, 84, 84), np.uint8))
+        cpu_elapsed = time.perf_counter() - cpu_started
+        cpu_baseline = dict(
+            value=round(sample / cpu_elapsed, 3), unit="lane-frames/s", cores=1, kind="port",
+            sample=f"{sample} lanes of {args.workload} (one frame each), scalar C++ restatement of the reference algorithm, {cpu_elapsed:.1f} s",
+        )
+
+    line = dict(
+        metric="rendered lane-frames/sec (320x240 + 84x84x4 obs)", value=round(value, 1), unit="lane-frames/s", n_gpus=1,
+        steps=args.steps, warmup=args.warmup, ms_per_step=round(elapsed / args.steps * 1e3, 3), higher_is_better=True,
+        scaling="weak", vs_baseline=None, dtype="int64+f32", data="synthetic",
+        config=dict(workload=f"{args.workload}: {lanes} lanes, {cfg['sectors']} sectors, {cfg['linedefs']} linedefs, "
+                    f"{sprites} sprites/lane, masked midtex p={cfg['midtex']}, per-step sector-light flicker"),
+        roofline=roofline, cpu_baseline=cpu_baseline,
+    )
+    print(json.dumps(line))
+    renderer.close()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -17,6 +17,7 @@ SYMBOLS = (
     "gd_renderer_create",
     "gd_renderer_destroy",
     "gd_renderer_status",
+    "gd_renderer_set_sector_lights",
     "gd_render",
     "gd_render_timed",
     "gd_observe",
@@ -47,6 +48,8 @@ def library() -> C.CDLL:
     lib.gd_renderer_destroy.argtypes = [C.c_void_p]
     lib.gd_renderer_status.restype = C.c_int
     lib.gd_renderer_status.argtypes = [C.c_void_p, C.POINTER(C.c_int32)]
+    lib.gd_renderer_set_sector_lights.restype = C.c_int
+    lib.gd_renderer_set_sector_lights.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
     lib.gd_render.restype = C.c_int
     lib.gd_render.argtypes = [C.c_void_p, C.POINTER(_abi.LanesDesc), C.POINTER(_abi.FrameOut), C.c_void_p]
     lib.gd_render_timed.restype = C.c_int

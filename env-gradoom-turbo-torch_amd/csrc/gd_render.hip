@@ -1461,7 +1461,9 @@ __global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lan
         s.x = lanes.sprite_x[k]; s.y = lanes.sprite_y[k];
         float z = lanes.sprite_z[k];
         s.depth = lanes.sprite_depth[k]; s.id = lanes.sprite_id[k];
-        s.flags = (lanes.sprite_alive[k] ? 1 : 0) | ((lanes.sprite_fullbright && lanes.sprite_fullbright[k]) ? 2 : 0);
+        const bool known_patch = s.id >= 0 && s.id < m->sprite_count;   // an unknown patch id is never drawn
+        if (!known_patch) s.id = 0;
+        s.flags = ((lanes.sprite_alive[k] && known_patch) ? 1 : 0) | ((lanes.sprite_fullbright && lanes.sprite_fullbright[k]) ? 2 : 0);
         i64 ax = round_to_i64(s.x * 65536.0f), ay = round_to_i64(s.y * 65536.0f);
         i64 rx = ax - L.view_x_fixed, ry = ay - L.view_y_fixed;
         s.depth_fixed = (rx * L.vcos + ry * L.vsin) >> 20;
@@ -1861,6 +1863,13 @@ int gd_renderer_status(gd_renderer *r, int32_t *status) {
     int value = 0;
     HIP_TRY(hipMemcpy(&value, r->sc.status, sizeof(int), hipMemcpyDeviceToHost));
     *status = value;
+    return GD_OK;
+}
+
+int gd_renderer_set_sector_lights(gd_renderer *r, const float *lights, void *stream) {
+    if (!r || !lights) return fail(GD_E_ARG, "null argument");
+    HIP_TRY(hipMemcpyAsync(const_cast<float *>(r->dm.d.sector_lights), lights, (size_t)r->dm.d.sector_count * sizeof(float),
+                           hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream)));
     return GD_OK;
 }
 

@@ -121,6 +121,14 @@ class HipRenderer:
         _lib.check(self._lib.gd_renderer_status(self._handle, C.byref(value)))
         return int(value.value)
 
+    def set_sector_lights(self, lights: torch.Tensor) -> None:
+        """Replace the per-sector light levels (float32 [S] on the device) for later frames."""
+
+        count = int(self.tables["sector_count"])
+        _require(lights, "lights", torch.float32, (count,), self.device)
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        _lib.check(self._lib.gd_renderer_set_sector_lights(self._handle, lights.data_ptr(), C.c_void_p(stream)))
+
     # ------------------------------------------------------------------ descriptors
     def _lanes_desc(self, lanes: LaneState):
         count = int(lanes.x.shape[0])

@@ -367,3 +367,44 @@ def bam_to_radians_f32(angle_bam: np.ndarray) -> np.ndarray:
     """float32 view angle the reference derives from a retained BAM (``engine.py:10651``)."""
 
     return (angle_bam.astype(np.float32) * np.float32(2.0 * math.pi / float(1 << 32))).astype(np.float32)
+
+
+def _points_in_cells(smap: SynthMap, sectors: np.ndarray, u: np.ndarray, v: np.ndarray):
+    """Vectorised ``_point_in_cell`` (same bilinear map, same 1/16-unit snapping)."""
+
+    i = smap.sector_cells[sectors, 0]
+    j = smap.sector_cells[sectors, 1]
+    grid = smap.grid_points.astype(np.float64)
+    p00, p10, p01, p11 = grid[j, i], grid[j, i + 1], grid[j + 1, i], grid[j + 1, i + 1]
+    u = u[..., None]
+    v = v[..., None]
+    point = (1 - u) * (1 - v) * p00 + u * (1 - v) * p10 + (1 - u) * v * p01 + u * v * p11
+    point = np.round(point * 16) / 16
+    return point[..., 0].astype(np.float32), point[..., 1].astype(np.float32)
+
+
+def generate_poses_batch(smap: SynthMap, lanes: int, seed: int, *, pitch: bool = False, flash: bool = False) -> Poses:
+    """Same distribution as ``generate_poses`` from one generator (for large batches)."""
+
+    rng = np.random.default_rng(seed)
+    sector = rng.integers(0, len(smap.sector_heights), lanes)
+    x, y = _points_in_cells(smap, sector, rng.uniform(0.15, 0.85, lanes), rng.uniform(0.15, 0.85, lanes))
+    angle_bam = rng.integers(0, 1 << 32, lanes).astype(np.int64)
+    pitch_bam = (rng.integers(-10, 11, lanes) * (182 << 16)).astype(np.int64) if pitch else np.zeros(lanes, np.int64)
+    flash_light = rng.integers(0, 3, lanes).astype(np.int64) if flash else np.zeros(lanes, np.int64)
+    view_z = (smap.sector_heights[sector, 0] + 41.0).astype(np.float32)
+    return Poses(x, y, angle_bam, pitch_bam, view_z, flash_light, sector.astype(np.int32))
+
+
+def generate_sprites_batch(smap: SynthMap, lanes: int, count: int, seed: int) -> Sprites:
+    """Same distribution as ``generate_sprites`` from one generator (for large batches)."""
+
+    rng = np.random.default_rng(seed + 7919)
+    shape = (lanes, count)
+    sector = rng.integers(0, len(smap.sector_heights), shape)
+    x, y = _points_in_cells(smap, sector, rng.uniform(0.1, 0.9, shape), rng.uniform(0.1, 0.9, shape))
+    z = smap.sector_heights[sector, 0].astype(np.float32)
+    sprite = rng.integers(0, len(smap.sprite_widths), shape).astype(np.int32)
+    alive = rng.random(shape) < 0.9
+    fullbright = rng.random(shape) < 0.1
+    return Sprites(x, y, z, sprite, alive, fullbright)

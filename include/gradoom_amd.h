@@ -177,6 +177,14 @@ int gd_render(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_out *ou
 int gd_renderer_status(gd_renderer *r, int32_t *status);
 
 /*
+ * Replace the map-wide sector light levels (device pointer to S floats) for the frames
+ * that follow on `stream`; the copy is asynchronous.  The reference keeps one
+ * sector_lights tensor per map (engine.py:640, 1277-1279); this is how a caller
+ * animates it (light flicker) between frames.
+ */
+int gd_renderer_set_sector_lights(gd_renderer *r, const float *lights, void *stream);
+
+/*
  * Observation pipeline alone on an existing indexed frame.
  * Replaces policy_area_grayscale (_triton_kernels.py:120-203) fused with the
  * frame-stack update (engine.py:9545-9548, 2443-2450).

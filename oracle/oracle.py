@@ -54,7 +54,8 @@ def library():
     global _LIB
     if _LIB is None:
         path = os.path.join(_HERE, "_build", "liboracle.so")
-        if not os.path.exists(path):
+        sources = [os.path.join(_HERE, "gd_oracle.cpp"), os.path.join(_ROOT, "include", "gradoom_amd.h")]
+        if not os.path.exists(path) or any(os.path.getmtime(src) > os.path.getmtime(path) for src in sources):
             subprocess.run(["make", "-C", _HERE, "-s"], check=True)
         lib = C.CDLL(path)
         lib.gdo_render.restype = C.c_int
