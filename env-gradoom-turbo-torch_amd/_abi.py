@@ -12,6 +12,9 @@ SCREEN_HEIGHT = 240
 OBS_SIZE = 84
 FRAME_STACK = 4
 
+STACK_STEP = 0
+STACK_RESET = 1
+
 GD_OK = 0
 GD_E_ARG = -1
 GD_E_HIP = -2
@@ -123,7 +126,7 @@ class LanesDesc(C.Structure):
 
 
 class FrameOut(C.Structure):
-    _fields_ = [(name, _P) for name in OUT_FIELDS]
+    _fields_ = [(name, _P) for name in OUT_FIELDS] + [("stack_mode", C.c_int32)]
 
 
 def host_map_desc(tables: dict) -> tuple[MapDesc, list]:

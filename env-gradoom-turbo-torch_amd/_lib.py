@@ -57,7 +57,7 @@ def library() -> C.CDLL:
         C.c_void_p, C.POINTER(_abi.LanesDesc), C.POINTER(_abi.FrameOut), C.c_void_p, C.c_int32, C.POINTER(C.c_float), C.c_int32,
     ]
     lib.gd_observe.restype = C.c_int
-    lib.gd_observe.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+    lib.gd_observe.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]
     lib.gd_expand_rgb24.restype = C.c_int
     lib.gd_expand_rgb24.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p]
     _LIBRARY = lib

@@ -1569,7 +1569,7 @@ __global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lan
 // observation: _triton_kernels.py:120-177 + engine.py:9545-9548 / 2443-2450
 // ---------------------------------------------------------------------------------------------
 __global__ void observe_kernel(const unsigned char *indexed, size_t lane_stride, int source_rows, const unsigned char *playpal,
-                               int lane_count, unsigned char *obs, unsigned char *frames, const unsigned char *reset_mask) {
+                               int lane_count, unsigned char *obs, unsigned char *frames, const unsigned char *reset_mask, int stack_mode) {
     __shared__ unsigned char pal[768];
     for (int k = threadIdx.x; k < 768; k += blockDim.x) pal[k] = playpal[k];
     __syncthreads();
@@ -1601,7 +1601,7 @@ __global__ void observe_kernel(const unsigned char *indexed, size_t lane_stride,
         unsigned char *stack = frames + (size_t)n * GD_FRAME_STACK * F + pixel;
         if (reset_mask && reset_mask[n]) {
             for (int k = 0; k < GD_FRAME_STACK; ++k) stack[k * F] = gray;
-        } else {
+        } else if (stack_mode == GD_STACK_STEP) {
             for (int k = 0; k < GD_FRAME_STACK - 1; ++k) stack[k * F] = stack[(k + 1) * F];
             stack[(GD_FRAME_STACK - 1) * F] = gray;
         }
@@ -1716,7 +1716,7 @@ int launch_chunk(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_out 
         hipLaunchKernelGGL(observe_kernel, dim3((GD_OBS_SIZE * GD_OBS_SIZE + 255) / 256, count), dim3(256), 0, stream,
                            frame_base, frame_stride, VH, m.playpal, count, out->obs ? out->obs + (size_t)base * F : nullptr,
                            out->frames ? out->frames + (size_t)base * GD_FRAME_STACK * F : nullptr,
-                           out->reset_mask ? out->reset_mask + base : nullptr);
+                           out->reset_mask ? out->reset_mask + base : nullptr, out->stack_mode);
     }
     if (out->rgb) {
         size_t pixels = (size_t)count * frame_stride;
@@ -1815,6 +1815,7 @@ static int check_render_args(gd_renderer *r, const gd_lanes_desc *lanes, const g
     if (!lanes->x || !lanes->y || !lanes->angle || !lanes->view_z || !lanes->x_fixed || !lanes->y_fixed || !lanes->angle_bam ||
         !lanes->pitch_bam || !lanes->ray_cos || !lanes->ray_sin)
         return fail(GD_E_ARG, "missing lane tensor");
+    if (out->stack_mode != GD_STACK_STEP && out->stack_mode != GD_STACK_RESET) return fail(GD_E_ARG, "unknown stack_mode");
     if (lanes->sprite_slots < 0 || lanes->sprite_slots > 512) return fail(GD_E_ARG, "sprite_slots must be in [0, 512]");
     if (lanes->sprite_slots > 0 && lanes->sprite_x &&
         (!lanes->sprite_y || !lanes->sprite_z || !lanes->sprite_depth || !lanes->sprite_id || !lanes->sprite_alive))
@@ -1874,8 +1875,9 @@ int gd_renderer_set_sector_lights(gd_renderer *r, const float *lights, void *str
 }
 
 int gd_observe(const uint8_t *indexed, int32_t source_rows, const uint8_t *playpal, int32_t lane_count,
-               uint8_t *obs, uint8_t *frames, const uint8_t *reset_mask, void *stream) {
+               uint8_t *obs, uint8_t *frames, const uint8_t *reset_mask, int32_t stack_mode, void *stream) {
     if (!indexed || !playpal) return fail(GD_E_ARG, "null argument");
+    if (stack_mode != GD_STACK_STEP && stack_mode != GD_STACK_RESET) return fail(GD_E_ARG, "unknown stack_mode");
     if (source_rows != 208 && source_rows != 240) return fail(GD_E_ARG, "indexed must have 208 or 240 rows");
     if (lane_count < 0) return fail(GD_E_ARG, "negative lane count");
     if (lane_count == 0 || (!obs && !frames)) return GD_OK;
@@ -1885,7 +1887,7 @@ int gd_observe(const uint8_t *indexed, int32_t source_rows, const uint8_t *playp
         hipLaunchKernelGGL(observe_kernel, dim3((GD_OBS_SIZE * GD_OBS_SIZE + 255) / 256, count), dim3(256), 0, static_cast<hipStream_t>(stream),
                            indexed + (size_t)base * source_rows * SW, (size_t)source_rows * SW, source_rows, playpal, count,
                            obs ? obs + (size_t)base * F : nullptr, frames ? frames + (size_t)base * GD_FRAME_STACK * F : nullptr,
-                           reset_mask ? reset_mask + base : nullptr);
+                           reset_mask ? reset_mask + base : nullptr, stack_mode);
     }
     HIP_TRY(hipGetLastError());
     return GD_OK;

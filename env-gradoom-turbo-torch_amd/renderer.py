@@ -172,9 +172,10 @@ class HipRenderer:
             desc.sprite_depth = _require(depth, "sprite_depth", torch.float32, (count, slots), device).data_ptr()
         return desc, keep
 
-    def _out_desc(self, count, indexed, obs, frames, reset_mask, rgb):
+    def _out_desc(self, count, indexed, obs, frames, reset_mask, rgb, stack_only_masked=False):
         device = self.device
         out = _abi.FrameOut()
+        out.stack_mode = _abi.STACK_RESET if stack_only_masked else _abi.STACK_STEP
         keep = []
         if indexed is not None:
             out.indexed = _require(indexed, "indexed", torch.uint8, (count, 240, 320), device).data_ptr()
@@ -191,13 +192,19 @@ class HipRenderer:
         return out, keep
 
     # ------------------------------------------------------------------ entry points
-    def render(self, lanes: LaneState, *, indexed=None, obs=None, frames=None, reset_mask=None, rgb=None) -> None:
-        """One frame for every lane, written into the given (preallocated) tensors."""
+    def render(self, lanes: LaneState, *, indexed=None, obs=None, frames=None, reset_mask=None, rgb=None,
+               stack_only_masked: bool = False) -> None:
+        """One frame for every lane, written into the given (preallocated) tensors.
+
+        ``frames`` is rolled by one and the new observation appended (``engine.py:9545-9548``); lanes
+        whose ``reset_mask`` is set get four copies instead (``engine.py:2443-2450``).  With
+        ``stack_only_masked`` the unmasked lanes' stacks are left untouched (the reset call).
+        """
 
         if self._handle is None:
             raise RuntimeError("renderer is closed")
         desc, keep_lanes = self._lanes_desc(lanes)
-        out, keep_out = self._out_desc(desc.lane_count, indexed, obs, frames, reset_mask, rgb)
+        out, keep_out = self._out_desc(desc.lane_count, indexed, obs, frames, reset_mask, rgb, stack_only_masked)
         stream = torch.cuda.current_stream(self.device).cuda_stream
         _lib.check(self._lib.gd_render(self._handle, C.byref(desc), C.byref(out), C.c_void_p(stream)))
         del keep_lanes, keep_out
@@ -215,7 +222,7 @@ class HipRenderer:
         del keep_lanes, keep_out
         return {name: float(times[i]) for i, name in enumerate(STAGES)}
 
-    def observe(self, indexed: torch.Tensor, *, obs=None, frames=None, reset_mask=None) -> None:
+    def observe(self, indexed: torch.Tensor, *, obs=None, frames=None, reset_mask=None, stack_only_masked: bool = False) -> None:
         """Observation pipeline on an existing ``[N,208|240,320]`` indexed frame."""
 
         if indexed.ndim != 3 or tuple(indexed.shape[1:]) not in ((208, 320), (240, 320)):
@@ -223,12 +230,12 @@ class HipRenderer:
         if indexed.dtype != torch.uint8:
             raise TypeError("indexed must be a uint8 tensor")
         count, rows = int(indexed.shape[0]), int(indexed.shape[1])
-        out, keep = self._out_desc(count, None, obs, frames, reset_mask, None)
+        out, keep = self._out_desc(count, None, obs, frames, reset_mask, None, stack_only_masked)
         stream = torch.cuda.current_stream(self.device).cuda_stream
         _lib.check(
             self._lib.gd_observe(
                 indexed.contiguous().data_ptr(), rows, self.playpal.data_ptr(), count, out.obs, out.frames, out.reset_mask,
-                C.c_void_p(stream),
+                out.stack_mode, C.c_void_p(stream),
             )
         )
         del keep

@@ -28,6 +28,10 @@ extern "C" {
 #define GD_OBS_SIZE 84
 #define GD_FRAME_STACK 4
 
+/* gd_frame_out.stack_mode */
+#define GD_STACK_STEP 0   /* every lane: roll by one, append (engine.py:9545-9548); lanes with reset_mask set: 4 copies */
+#define GD_STACK_RESET 1  /* lanes with reset_mask set: 4 copies (engine.py:2443-2450); other lanes untouched */
+
 #define GD_OK 0
 #define GD_E_ARG (-1)       /* bad argument: null pointer, negative count, size over a limit */
 #define GD_E_HIP (-2)       /* a HIP runtime call failed */
@@ -138,6 +142,7 @@ typedef struct gd_frame_out {
     uint8_t *frames;    /* [N,4,84,84] stack, oldest first: rolled by one and obs appended */
     const uint8_t *reset_mask; /* [N] or null: lanes whose stack is filled with 4 copies instead */
     uint8_t *rgb;       /* [N,240,320,3] PLAYPAL expansion of `indexed` */
+    int32_t stack_mode; /* GD_STACK_STEP or GD_STACK_RESET */
 } gd_frame_out;
 
 typedef struct gd_renderer gd_renderer;
@@ -191,7 +196,7 @@ int gd_renderer_set_sector_lights(gd_renderer *r, const float *lights, void *str
  * indexed: [N,source_rows,320] with source_rows 208 or 240; rows >= source_rows are black.
  */
 int gd_observe(const uint8_t *indexed, int32_t source_rows, const uint8_t *playpal, int32_t lane_count,
-               uint8_t *obs, uint8_t *frames, const uint8_t *reset_mask, void *stream);
+               uint8_t *obs, uint8_t *frames, const uint8_t *reset_mask, int32_t stack_mode, void *stream);
 
 /* PLAYPAL expansion [N,rows,320] -> [N,rows,320,3]; replaces engine.py:15381-15384. */
 int gd_expand_rgb24(const uint8_t *indexed, int32_t rows, const uint8_t *playpal, int32_t lane_count,

@@ -1458,11 +1458,11 @@ void observe_lane(const uint8_t *indexed, int source_rows, const uint8_t *playpa
 }
 
 // engine.py:9545-9548 (roll + append) and engine.py:2443-2450 (reset fill)
-void stack_lane(const uint8_t *obs, uint8_t *frames, bool reset) {
+void stack_lane(const uint8_t *obs, uint8_t *frames, bool reset, int stack_mode) {
     const size_t F = size_t(GD_OBS_SIZE) * GD_OBS_SIZE;
     if (reset) {
         for (int k = 0; k < GD_FRAME_STACK; ++k) std::memcpy(frames + k * F, obs, F);
-    } else {
+    } else if (stack_mode == GD_STACK_STEP) {
         std::memmove(frames, frames + F, (GD_FRAME_STACK - 1) * F);
         std::memcpy(frames + (GD_FRAME_STACK - 1) * F, obs, F);
     }
@@ -1561,7 +1561,7 @@ int gdo_render(const gd_map_desc *map, const gd_lanes_desc *lanes, const gd_fram
         if (out->obs || out->frames) {
             observe_lane(full.data(), VH, map->playpal, obs.data());  // HUD rows masked black
             if (out->obs) std::memcpy(out->obs + size_t(n) * obs.size(), obs.data(), obs.size());
-            if (out->frames) stack_lane(obs.data(), out->frames + size_t(n) * GD_FRAME_STACK * obs.size(), out->reset_mask && out->reset_mask[n]);
+            if (out->frames) stack_lane(obs.data(), out->frames + size_t(n) * GD_FRAME_STACK * obs.size(), out->reset_mask && out->reset_mask[n], out->stack_mode);
         }
         if (out->rgb) {
             uint8_t *rgb = out->rgb + size_t(n) * full.size() * 3;
@@ -1573,15 +1573,34 @@ int gdo_render(const gd_map_desc *map, const gd_lanes_desc *lanes, const gd_fram
 }
 
 int gdo_observe(const uint8_t *indexed, int32_t source_rows, const uint8_t *playpal, int32_t lane_count,
-                uint8_t *obs, uint8_t *frames, const uint8_t *reset_mask) {
+                uint8_t *obs, uint8_t *frames, const uint8_t *reset_mask, int32_t stack_mode) {
     if (!indexed || !playpal || (source_rows != 208 && source_rows != 240)) { g_error = "bad argument"; return GD_E_ARG; }
     std::vector<uint8_t> one(size_t(GD_OBS_SIZE) * GD_OBS_SIZE);
     for (int n = 0; n < lane_count; ++n) {
         observe_lane(indexed + size_t(n) * source_rows * SW, source_rows, playpal, one.data());
         if (obs) std::memcpy(obs + size_t(n) * one.size(), one.data(), one.size());
-        if (frames) stack_lane(one.data(), frames + size_t(n) * GD_FRAME_STACK * one.size(), reset_mask && reset_mask[n]);
+        if (frames) stack_lane(one.data(), frames + size_t(n) * GD_FRAME_STACK * one.size(), reset_mask && reset_mask[n], stack_mode);
     }
     return GD_OK;
+}
+
+// Dense forms of the pair/bridge relations the reference precomputes (engine.py:399-484, 1597-1612),
+// evaluated through the same on-the-fly functions the render loop uses. Arrays are [W,W] / [2,W,W].
+void gdo_relation_tables(const gd_map_desc *map, uint8_t *same_pair, uint8_t *opposing, int64_t *portal_bridge_index,
+                         uint8_t *portal_bridge_mask, int64_t *sector_bridge_index, uint8_t *sector_bridge_mask) {
+    Oracle o(map);
+    const size_t W = map->wall_count;
+    for (size_t a = 0; a < W; ++a) for (size_t b = 0; b < W; ++b) {
+        same_pair[a * W + b] = o.same_pair(int(a), int(b));
+        opposing[a * W + b] = o.opposing(int(a), int(b));
+        for (int slot = 0; slot < 2; ++slot) {
+            int index;
+            portal_bridge_mask[(slot * W + a) * W + b] = o.portal_bridge(slot, int(a), int(b), &index);
+            portal_bridge_index[(slot * W + a) * W + b] = index;
+            sector_bridge_mask[(slot * W + a) * W + b] = o.sector_bridge(slot, int(a), int(b), &index);
+            sector_bridge_index[(slot * W + a) * W + b] = index;
+        }
+    }
 }
 
 void gdo_fine_tables(int64_t *fine_sine, int64_t *fine_tangent) {

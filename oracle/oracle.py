@@ -93,7 +93,7 @@ def lanes_desc(lanes: dict):
 
 
 def render(tables: dict, lanes: dict, cosine_correction, *, lane_range=None, frames=None, reset_mask=None,
-           want_rgb=False, debug_lane=None):
+           want_rgb=False, debug_lane=None, stack_mode=0):
     """Render lanes on the CPU. Returns dict(indexed, obs, frames, rgb, debug...)."""
 
     lib = library()
@@ -106,6 +106,7 @@ def render(tables: dict, lanes: dict, cosine_correction, *, lane_range=None, fra
     out = _abi.FrameOut()
     out.indexed = indexed.ctypes.data
     out.obs = obs.ctypes.data
+    out.stack_mode = int(stack_mode)
     result = {"indexed": indexed, "obs": obs}
     if frames is not None:
         frames = np.ascontiguousarray(frames, dtype=np.uint8).copy()
@@ -159,7 +160,7 @@ def render(tables: dict, lanes: dict, cosine_correction, *, lane_range=None, fra
     return result
 
 
-def observe(indexed, playpal, *, frames=None, reset_mask=None):
+def observe(indexed, playpal, *, frames=None, reset_mask=None, stack_mode=0):
     lib = library()
     indexed = np.ascontiguousarray(indexed, dtype=np.uint8)
     count, rows, _ = indexed.shape
@@ -175,8 +176,28 @@ def observe(indexed, playpal, *, frames=None, reset_mask=None):
         mask_ptr = reset_mask.ctypes.data_as(C.c_void_p)
     code = lib.gdo_observe(
         indexed.ctypes.data_as(C.c_void_p), C.c_int32(rows), playpal.ctypes.data_as(C.c_void_p), C.c_int32(count),
-        obs.ctypes.data_as(C.c_void_p), frames_ptr, mask_ptr,
+        obs.ctypes.data_as(C.c_void_p), frames_ptr, mask_ptr, C.c_int32(stack_mode),
     )
     if code != 0:
         raise RuntimeError(f"oracle observe failed ({code})")
     return obs, frames
+
+
+def relation_tables(tables: dict) -> dict:
+    """Dense [W,W] / [2,W,W] relation tables from the oracle's on-the-fly functions (small maps only)."""
+
+    lib = library()
+    map_desc, keep = _abi.host_map_desc(tables)
+    walls = int(tables["wall_count"])
+    out = dict(
+        same_pair=np.zeros((walls, walls), np.uint8), opposing=np.zeros((walls, walls), np.uint8),
+        portal_bridge_index=np.zeros((2, walls, walls), np.int64), portal_bridge_mask=np.zeros((2, walls, walls), np.uint8),
+        sector_bridge_index=np.zeros((2, walls, walls), np.int64), sector_bridge_mask=np.zeros((2, walls, walls), np.uint8),
+    )
+    lib.gdo_relation_tables.restype = None
+    lib.gdo_relation_tables(
+        C.byref(map_desc), *(out[name].ctypes.data_as(C.c_void_p) for name in (
+            "same_pair", "opposing", "portal_bridge_index", "portal_bridge_mask", "sector_bridge_index", "sector_bridge_mask")),
+    )
+    del keep
+    return out

@@ -127,6 +127,28 @@ def build_case(name: str, cfg: dict, do_time: bool) -> dict:
             st_walls=walls[0].numpy(), st_scene_depth=scene_depth[0].numpy(), st_clip_depth=clip_depth[0].numpy(),
             st_clip_wall=clip_wall[0].numpy().astype(np.int32),
         )
+        # derived map tables (engine.py:721-849, 1527-1634)
+        dmap = engine.map
+        data.update(
+            ref_wall_lengths=dmap.portal_wall_lengths.numpy(),
+            ref_endpoint_neighbors=dmap.portal_endpoint_neighbors.numpy(),
+            ref_endpoint_neighbor_starts=dmap.portal_endpoint_neighbor_starts.numpy(),
+            ref_endpoint_neighbor_ends=dmap.portal_endpoint_neighbor_ends.numpy(),
+            ref_solid_bridge_start_indices=dmap.portal_endpoint_solid_bridge_start_indices.numpy(),
+            ref_solid_bridge_start_mask=dmap.portal_endpoint_solid_bridge_start_mask.numpy(),
+            ref_solid_bridge_end_indices=dmap.portal_endpoint_solid_bridge_end_indices.numpy(),
+            ref_solid_bridge_end_mask=dmap.portal_endpoint_solid_bridge_end_mask.numpy(),
+            ref_direct_neighbors=np.asarray(engine._native_direct_endpoint_neighbors is not None),
+            ref_same_pair=engine._native_same_portal_sector_pairs.numpy(),
+            ref_opposing=engine._native_opposing_portal_pairs.numpy(),
+            ref_portal_bridge_index=engine._native_projected_portal_bridge_indices.numpy(),
+            ref_portal_bridge_mask=engine._native_projected_portal_bridge_mask.numpy(),
+            ref_sector_bridge_index=engine._native_projected_sector_bridge_indices.numpy(),
+            ref_sector_bridge_mask=engine._native_projected_sector_bridge_mask.numpy(),
+            ref_walls_fixed=torch.round(dmap.portal_walls * 65536).to(torch.int64).numpy(),
+            ref_blocking_wall_indices=engine._native_blocking_wall_indices.numpy(),
+            ref_sector_lights=dmap.sector_lights.numpy(),
+        )
     timing = None
     if do_time:
         # The CPU-baseline protocol: full indexed frame + observation + stack update per lane.

@@ -1,0 +1,121 @@
+"""Host logic of the vector-env front end with a recording stand-in for the renderer (CPU only)."""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import load_fixture
+
+
+class RecordingRenderer:
+    """Writes a lane-dependent constant so ownership and masking can be observed without a GPU."""
+
+    def __init__(self):
+        self.calls = []
+
+    def render(self, lanes, *, indexed=None, obs=None, frames=None, reset_mask=None, rgb=None, stack_only_masked=False):
+        self.calls.append(dict(reset=stack_only_masked, mask=None if reset_mask is None else reset_mask.clone()))
+        value = (lanes.x.abs().to(torch.int64) % 251).to(torch.uint8)
+        if frames is not None:
+            new = value[:, None, None].expand(-1, 84, 84)
+            for lane in range(frames.shape[0]):
+                if reset_mask is not None and bool(reset_mask[lane]):
+                    frames[lane] = new[lane]
+                elif not stack_only_masked:
+                    frames[lane] = torch.roll(frames[lane], -1, 0)
+                    frames[lane, -1] = new[lane]
+        if rgb is not None:
+            rgb.copy_(value[:, None, None, None].expand_as(rgb))
+
+    def close(self):
+        self.closed = True
+
+
+@pytest.fixture
+def env():
+    from gradoom_amd.env import GraDoomVecEnv
+
+    _meta, _data, smap, _tables = load_fixture("tiny_stages")
+    return GraDoomVecEnv(smap, 4, device="cpu", render_mode="rgb_array", renderer=RecordingRenderer(), episode_timeout=3)
+
+
+def test_argument_validation_matches_reference_error_classes(env):
+    mask = torch.ones(4, dtype=torch.bool)
+    seeds = torch.arange(4)
+    with pytest.raises(TypeError, match="mask must be a Torch tensor"):
+        env.reset_device([True] * 4, seeds)
+    with pytest.raises(TypeError, match="mask must have dtype torch.bool"):
+        env.reset_device(mask.to(torch.uint8), seeds)
+    with pytest.raises(ValueError, match="seeds must have shape"):
+        env.reset_device(mask, seeds[:3])
+    with pytest.raises(TypeError, match="seeds must have dtype"):
+        env.reset_device(mask, seeds.to(torch.float32))
+    with pytest.raises(TypeError, match="actions must have dtype"):
+        env.step_device(torch.zeros(4))
+
+
+def test_observations_are_the_engine_owned_stack_and_finals_are_clones(env):
+    obs, signals = env.reset_device(torch.ones(4, dtype=torch.bool), torch.arange(4))
+    assert obs.data_ptr() == env.frames.data_ptr() and signals.data_ptr() == env.signal_buffer.data_ptr()
+    assert obs.shape == (4, 4, 84, 84) and obs.dtype == torch.uint8
+    # reset fills four identical frames (engine.py:2443-2450)
+    assert torch.equal(obs[:, 0], obs[:, 3])
+    transition = env.step_and_reset_device(torch.zeros(4, dtype=torch.int64), torch.arange(4))
+    assert transition.observations.data_ptr() == env.frames.data_ptr()
+    assert transition.final_observations.data_ptr() != env.frames.data_ptr()
+    assert torch.equal(transition.final_observations, transition.observations)
+    assert not bool(transition.truncated.any())
+    # no lane done -> no reset render (tests/test_env.py:187-210)
+    assert [call["reset"] for call in env._renderer.calls] == [True, False]
+
+
+def test_done_lanes_are_reset_and_terminal_observation_is_retained(env):
+    env.reset_device(torch.ones(4, dtype=torch.bool), torch.arange(4))
+    actions = torch.zeros(4, dtype=torch.int64)
+    env.step_and_reset_device(actions, torch.arange(4))
+    env.step_and_reset_device(actions, torch.arange(4))
+    env._dynamics.episode_time[2:] = 0  # only lanes 0 and 1 reach the timeout next step
+    transition = env.step_and_reset_device(actions, torch.tensor([9, 8, 7, 6]))
+    assert transition.truncated.tolist() == [True, True, False, False]
+    last = env._renderer.calls[-1]
+    assert last["reset"] and last["mask"].tolist() == [True, True, False, False]
+    # reset lanes show four copies of their new frame, the others kept their rolled stack
+    assert torch.equal(transition.observations[0, 0], transition.observations[0, 3])
+    assert torch.equal(transition.observations[2], transition.final_observations[2])
+    assert not torch.equal(transition.observations[0], transition.final_observations[0])
+    assert env._latest_reset_seeds.tolist()[:2] == [9, 8]
+
+
+def test_hwc_layout_is_a_permuted_view():
+    from gradoom_amd.env import GraDoomVecEnv
+
+    _meta, _data, smap, _tables = load_fixture("tiny_stages")
+    env = GraDoomVecEnv(smap, 2, device="cpu", obs_layout="hwc", renderer=RecordingRenderer())
+    obs, _ = env.reset_device(torch.ones(2, dtype=torch.bool), torch.zeros(2, dtype=torch.int64))
+    assert obs.shape == (2, 84, 84, 4) and obs.data_ptr() == env.frames.data_ptr()
+
+
+def test_render_contract(env):
+    env.reset_device(torch.ones(4, dtype=torch.bool), torch.arange(4))
+    image = env.render()
+    assert isinstance(image, np.ndarray) and image.shape == (240, 320, 3) and image.dtype == np.uint8
+    assert len(env.get_images()) == 4
+    with pytest.raises(TypeError):
+        env.render_lane(True)
+    with pytest.raises(IndexError):
+        env.render_lane(4)
+    env.close()
+    with pytest.raises(RuntimeError, match="closed"):
+        env.render()
+    with pytest.raises(RuntimeError, match="closed"):
+        env.step_device(torch.zeros(4, dtype=torch.int64))
+
+
+def test_render_mode_none_returns_none():
+    from gradoom_amd.env import GraDoomVecEnv
+
+    _meta, _data, smap, _tables = load_fixture("tiny_stages")
+    env = GraDoomVecEnv(smap, 2, device="cpu", renderer=RecordingRenderer())
+    assert env.render() is None and env.get_images() == [None, None]

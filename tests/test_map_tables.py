@@ -1,0 +1,83 @@
+"""Derived map tables (mapbuild + the on-the-fly relations) against the reference's own tables."""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+
+from conftest import load_fixture
+
+CASES = ["tiny_stages", "small_midtex_sprites"]
+
+
+@pytest.mark.parametrize("name", CASES)
+def test_compact_tables_equal_reference(name):
+    _meta, data, _smap, tables = load_fixture(name)
+    walls = tables["wall_count"]
+    assert np.array_equal(tables["wall_len"], data["ref_wall_lengths"])
+    assert np.array_equal(tables["walls_fixed"].astype(np.int64), data["ref_walls_fixed"])
+    assert np.array_equal(tables["blocking_walls"], data["ref_blocking_wall_indices"])
+    assert np.array_equal(tables["sector_lights"], data["ref_sector_lights"])
+    assert bool(tables["direct_neighbors"]) == bool(data["ref_direct_neighbors"])
+    # endpoint neighbours: same compact [W,K] layout, ascending, self-padded (engine.py:833-849)
+    assert np.array_equal(tables["endpoint_neighbors"], data["ref_endpoint_neighbors"])
+    assert np.array_equal(tables["endpoint_neighbor_starts"].astype(bool), data["ref_endpoint_neighbor_starts"])
+    assert np.array_equal(tables["endpoint_neighbor_ends"].astype(bool), data["ref_endpoint_neighbor_ends"])
+    # solid bridges: CSR rows equal the masked prefix of the reference's padded rows (engine.py:811-830)
+    for side in ("start", "end"):
+        ofs, idx = tables[f"solid_bridge_{side}_ofs"], tables[f"solid_bridge_{side}_idx"]
+        ref_idx, ref_mask = data[f"ref_solid_bridge_{side}_indices"], data[f"ref_solid_bridge_{side}_mask"]
+        for w in range(walls):
+            ours = idx[ofs[w] : ofs[w + 1]].tolist()
+            assert ours == ref_idx[w][ref_mask[w]].tolist()
+            assert not ref_mask[w][len(ours) :].any()
+
+
+@pytest.mark.parametrize("name", CASES)
+def test_on_the_fly_relations_equal_reference_dense_tables(oracle, name):
+    _meta, data, _smap, tables = load_fixture(name)
+    ours = oracle.relation_tables(tables)
+    assert np.array_equal(ours["same_pair"].astype(bool), data["ref_same_pair"])
+    assert np.array_equal(ours["opposing"].astype(bool), data["ref_opposing"])
+    for kind in ("portal", "sector"):
+        mask = ours[f"{kind}_bridge_mask"].astype(bool)
+        assert np.array_equal(mask, data[f"ref_{kind}_bridge_mask"])
+        assert np.array_equal(ours[f"{kind}_bridge_index"], data[f"ref_{kind}_bridge_index"])
+
+
+def test_sector_grid_lists_every_edge_that_can_count():
+    # brute force: for random points, parity over the cell's edge sub-list == parity over the full edge list
+    _meta, _data, smap, tables = load_fixture("small_midtex_sprites")
+    rng = np.random.default_rng(1)
+    walls = tables["walls"]
+    lo = walls[:, (0, 2)].min() - 50, walls[:, (1, 3)].min() - 50
+    hi = walls[:, (0, 2)].max() + 50, walls[:, (1, 3)].max() + 50
+    nx, ny = tables["grid_nx"], tables["grid_ny"]
+
+    def parity(edges, px, py):
+        count = 0
+        for w in edges:
+            x1, y1, x2, y2 = (np.float32(v) for v in walls[w])
+            dy = np.float32(y2 - y1)
+            safe = np.float32(1.0) if abs(dy) < 1e-6 else dy
+            crossing = np.float32(x1 + np.float32(np.float32(np.float32(py - y1) * np.float32(x2 - x1)) / safe))
+            if ((y1 > py) != (y2 > py)) and px < crossing:
+                count += 1
+        return count & 1
+
+    for _ in range(400):
+        px = np.float32(rng.uniform(lo[0], hi[0]))
+        py = np.float32(rng.uniform(lo[1], hi[1]))
+        fx = np.floor(np.float32(np.float32(px - np.float32(tables["grid_min_x"])) / np.float32(tables["grid_cell"])))
+        fy = np.floor(np.float32(np.float32(py - np.float32(tables["grid_min_y"])) / np.float32(tables["grid_cell"])))
+        listed = {}
+        if 0 <= fy < ny and fx < nx:
+            cell = int(fy) * nx + max(int(fx), 0)
+            for item in range(tables["grid_cell_ofs"][cell], tables["grid_cell_ofs"][cell + 1]):
+                e0, e1 = tables["grid_item_edge_ofs"][item], tables["grid_item_edge_ofs"][item + 1]
+                listed[int(tables["grid_item_sector"][item])] = tables["grid_item_edges"][e0:e1]
+        for s in range(tables["sector_count"]):
+            full = tables["sector_edge_idx"][tables["sector_edge_ofs"][s] : tables["sector_edge_ofs"][s + 1]]
+            expected = parity(full, px, py)
+            got = parity(listed[s], px, py) if s in listed else 0
+            assert got == expected
