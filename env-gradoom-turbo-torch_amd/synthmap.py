@@ -65,6 +65,7 @@ class SynthMap:
     sprite_top_offsets: np.ndarray  # [P] i32
     sector_cells: np.ndarray  # [S,2] i32 grid cell of each sector (generator bookkeeping)
     grid_points: np.ndarray  # [gy+1,gx+1,2] f32 jittered grid vertices
+    sector_quads: np.ndarray | None = None  # [S,4,2] f64 corners p00,p10,p01,p11 used to place cameras/sprites
 
     @property
     def blocking_segments(self) -> np.ndarray:
@@ -134,7 +135,16 @@ def generate_map(
     wall_textures: int = 64,
     flats: int = 16,
     sprite_patches: int = 64,
+    layout: str = "grid",
+    islands: int = 0,
 ) -> SynthMap:
+    if layout == "brick":
+        return _generate_brick_map(
+            seed, grid=grid, sectors=sectors, linedefs=linedefs, midtex=midtex, wall_textures=wall_textures,
+            flats=flats, sprite_patches=sprite_patches, islands=islands,
+        )
+    if layout != "grid":
+        raise ValueError("layout must be 'grid' or 'brick'")
     rng = np.random.default_rng(seed)
     gx, gy = grid
     if sectors > gx * gy:
@@ -187,6 +197,47 @@ def generate_map(
             # vertical edge from (i,j) to (i,j+1): cell (i-1) is on the left, cell (i) on the right
             add_edge(points[j, i], points[j + 1, i], sector_of(i - 1, j), sector_of(i, j))
 
+    quads = np.zeros((len(sector_cells), 4, 2), dtype=np.float64)
+    for index, (i, j) in enumerate(sector_cells):
+        quads[index] = (points[j, i], points[j, i + 1], points[j + 1, i], points[j + 1, i + 1])
+    return _finish_map(
+        rng, edges, sector_cells, points, quads, linedefs=linedefs, midtex=midtex, wall_textures=wall_textures,
+        flats=flats, sprite_patches=sprite_patches, islands=islands,
+    )
+
+
+def _add_islands(rng, edges, sector_cells, sector_quads, count):
+    """Nest an axis-aligned rectangular sector in the middle of `count` cells.
+
+    Opposite sides of an island bound the same sector pair with anti-parallel directions and no
+    shared endpoint, the configuration the reference calls opposing portals (``engine.py:1605-1612``).
+    """
+
+    hosts = rng.permutation(len(sector_cells))[:count]
+    quads = list(sector_quads)
+    cells = list(sector_cells)
+    for host in hosts:
+        centre = np.round(np.mean(sector_quads[host], axis=0))
+        half_w = float(rng.integers(3, 7) * 8)
+        half_h = float(rng.integers(3, 7) * 8)
+        x0, x1, y0, y1 = centre[0] - half_w, centre[0] + half_w, centre[1] - half_h, centre[1] + half_h
+        island = len(cells)
+        cells.append(tuple(sector_cells[host]))
+        quads.append(np.asarray([(x0, y0), (x1, y0), (x0, y1), (x1, y1)], dtype=np.float64))
+        # counter-clockwise loop: the island is on the left, so it is the back sector
+        corners = [(x0, y0), (x1, y0), (x1, y1), (x0, y1)]
+        for k in range(4):
+            p, q = corners[k], corners[(k + 1) % 4]
+            if rng.random() < 0.5:
+                edges.append((p, q, int(host), island, MAX_SPLIT_DEPTH))
+            else:
+                edges.append((q, p, island, int(host), MAX_SPLIT_DEPTH))
+    return edges, cells, np.asarray(quads, dtype=np.float64)
+
+
+def _finish_map(rng, edges, sector_cells, points, sector_quads, *, linedefs, midtex, wall_textures, flats, sprite_patches, islands=0):
+    if islands:
+        edges, sector_cells, sector_quads = _add_islands(rng, edges, sector_cells, sector_quads, islands)
     edges = _split_edges(rng, edges, linedefs)
     order = rng.permutation(len(edges))
     edges = [edges[k] for k in order]
@@ -274,7 +325,98 @@ def generate_map(
         sprite_left_offsets=sprite_left_offsets,
         sprite_top_offsets=sprite_top_offsets,
         sector_cells=np.asarray(sector_cells, dtype=np.int32),
-        grid_points=points.astype(np.float32),
+        grid_points=np.asarray(points, dtype=np.float32),
+        sector_quads=sector_quads,
+    )
+
+
+
+def _generate_brick_map(seed, *, grid, sectors, linedefs, midtex, wall_textures, flats, sprite_patches, islands=0):
+    """Staggered rows: odd rows are shifted by half a cell, so every interior vertex joins three sectors.
+
+    At such a T-junction all three pairwise linedefs exist, which is what the reference's
+    three-sector "bridge" tables (``engine.py:399-484``) index; the plain grid never produces one.
+    """
+
+    rng = np.random.default_rng(seed)
+    gx, gy = grid
+    jitter = 24
+    origin_x = -gx * CELL / 2.0
+    origin_y = -gy * CELL / 2.0
+
+    def row_boundaries(j):
+        if j % 2 == 0:
+            return [origin_x + i * CELL for i in range(gx + 1)]
+        return [origin_x] + [origin_x + (i + 0.5) * CELL for i in range(gx)] + [origin_x + gx * CELL]
+
+    # vertices on horizontal line j (between rows j-1 and j), keyed by nominal x
+    line_points: list[dict[float, tuple[float, float]]] = []
+    for j in range(gy + 1):
+        xs = set()
+        if j < gy:
+            xs.update(row_boundaries(j))
+        if j > 0:
+            xs.update(row_boundaries(j - 1))
+        line = {}
+        for x in sorted(xs):
+            line[x] = (x + int(rng.integers(-jitter, jitter + 1)), origin_y + j * CELL + int(rng.integers(-jitter, jitter + 1)))
+        line_points.append(line)
+
+    cells = [(i, j) for j in range(gy) for i in range(len(row_boundaries(j)) - 1)]
+    if sectors > len(cells):
+        raise ValueError("more sectors than brick cells")
+    void = np.zeros(len(cells), dtype=bool)
+    void[rng.permutation(len(cells))[: len(cells) - sectors]] = True
+    cell_sector = {}
+    sector_cells = []
+    for index, cell in enumerate(cells):
+        if not void[index]:
+            cell_sector[cell] = len(sector_cells)
+            sector_cells.append(cell)
+
+    def sector_of_x(j, x):
+        """Sector of the row-j cell whose nominal x-range contains x (x is an interval midpoint)."""
+        if not 0 <= j < gy:
+            return -1
+        bounds = row_boundaries(j)
+        for i in range(len(bounds) - 1):
+            if bounds[i] < x < bounds[i + 1]:
+                return cell_sector.get((i, j), -1)
+        return -1
+
+    edges = []
+
+    def add_edge(p, q, left_sector, right_sector):
+        if left_sector < 0 and right_sector < 0:
+            return
+        if right_sector < 0:
+            p, q, left_sector, right_sector = q, p, right_sector, left_sector
+        elif left_sector >= 0 and rng.random() < 0.5:
+            p, q, left_sector, right_sector = q, p, right_sector, left_sector
+        edges.append((tuple(p), tuple(q), right_sector, left_sector, 0))
+
+    for j in range(gy + 1):
+        xs = sorted(line_points[j])
+        for a, b in zip(xs[:-1], xs[1:]):
+            mid = (a + b) / 2.0
+            # direction +x: the row above (j) is on the left, the row below (j-1) on the right
+            add_edge(line_points[j][a], line_points[j][b], sector_of_x(j, mid), sector_of_x(j - 1, mid))
+    for j in range(gy):
+        bounds = row_boundaries(j)
+        for i, x in enumerate(bounds):
+            left = cell_sector.get((i - 1, j), -1) if i > 0 else -1
+            right = cell_sector.get((i, j), -1) if i < len(bounds) - 1 else -1
+            # direction +y: the cell at smaller x is on the left
+            add_edge(line_points[j][x], line_points[j + 1][x], left, right)
+
+    quads = np.zeros((len(sector_cells), 4, 2), dtype=np.float64)
+    for index, (i, j) in enumerate(sector_cells):
+        bounds = row_boundaries(j)
+        quads[index] = (line_points[j][bounds[i]], line_points[j][bounds[i + 1]], line_points[j + 1][bounds[i]], line_points[j + 1][bounds[i + 1]])
+    points = np.zeros((1, 1, 2), dtype=np.float64)
+    return _finish_map(
+        rng, edges, sector_cells, points, quads, linedefs=linedefs, midtex=midtex, wall_textures=wall_textures,
+        flats=flats, sprite_patches=sprite_patches, islands=islands,
     )
 
 
@@ -292,11 +434,7 @@ def generate_config_map(name: str, seed: int | None = None) -> SynthMap:
 
 
 def _point_in_cell(smap: SynthMap, sector: int, u: float, v: float) -> tuple[float, float]:
-    i, j = smap.sector_cells[sector]
-    p00 = smap.grid_points[j, i].astype(np.float64)
-    p10 = smap.grid_points[j, i + 1].astype(np.float64)
-    p01 = smap.grid_points[j + 1, i].astype(np.float64)
-    p11 = smap.grid_points[j + 1, i + 1].astype(np.float64)
+    p00, p10, p01, p11 = smap.sector_quads[sector]
     point = (1 - u) * (1 - v) * p00 + u * (1 - v) * p10 + (1 - u) * v * p01 + u * v * p11
     # 1/16 map unit keeps the float32 value and its 16.16 image both exact.
     return float(np.round(point[0] * 16) / 16), float(np.round(point[1] * 16) / 16)
@@ -372,10 +510,8 @@ def bam_to_radians_f32(angle_bam: np.ndarray) -> np.ndarray:
 def _points_in_cells(smap: SynthMap, sectors: np.ndarray, u: np.ndarray, v: np.ndarray):
     """Vectorised ``_point_in_cell`` (same bilinear map, same 1/16-unit snapping)."""
 
-    i = smap.sector_cells[sectors, 0]
-    j = smap.sector_cells[sectors, 1]
-    grid = smap.grid_points.astype(np.float64)
-    p00, p10, p01, p11 = grid[j, i], grid[j, i + 1], grid[j + 1, i], grid[j + 1, i + 1]
+    quads = smap.sector_quads[sectors]
+    p00, p10, p01, p11 = quads[..., 0, :], quads[..., 1, :], quads[..., 2, :], quads[..., 3, :]
     u = u[..., None]
     v = v[..., None]
     point = (1 - u) * (1 - v) * p00 + u * (1 - v) * p10 + (1 - u) * v * p01 + u * v * p11

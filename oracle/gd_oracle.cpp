@@ -95,6 +95,17 @@ inline i64 f64_to_i64(double v) {
 }
 inline int ilog2(int v) { int b = 0; while ((1 << (b + 1)) <= v) ++b; return b; }
 
+// Rule coverage counters (how often each ownership rule fired), reported through gdo_coverage.
+enum {
+    COV_PASSES, COV_VALID, COV_EQUAL_DEPTH_SOLID, COV_PROJECTED_SOLID, COV_SOLID_BRIDGE, COV_ENDPOINT_OWNER, COV_NEAR_PROJECTED,
+    COV_TOPOLOGICAL_OWNER, COV_SECTOR_BRIDGE, COV_OPPOSING_BOUNDARY, COV_EXCLUDED_RIGHT_EDGE, COV_CONTINUES_OWNER_BOUNDARY,
+    COV_FORWARD_BRIDGE, COV_COMPLETES_ENDPOINT_BRIDGE, COV_ENDPOINT_ONLY_PORTAL, COV_TIED_STRIP, COV_ENTERS_OTHER, COV_ENTERS_SHARED,
+    COV_GEOMETRIC_PATH, COV_PORTAL_BRIDGE, COV_COMPLETES_PORTAL_BRIDGE, COV_PS_KEEPS_PATH, COV_NO_KEEPS_PATH, COV_BOTTOM_TAIL,
+    COV_MASKED_COLUMN, COV_MASKED_EXTENDS, COV_DEAD_COLUMN_REVIVED, COV_COUNT
+};
+long long g_coverage[COV_COUNT];
+#define COVER(name, cond) do { if (cond) ++g_coverage[name]; } while (0)
+
 struct Lane {
     float x, y, angle, view_z;
     i64 view_x_fixed, view_y_fixed, angle_bam, pitch_bam, flash_light;
@@ -827,7 +838,8 @@ struct Oracle {
                 float vv = eds ? v : INF;
                 if (vv < sd) { sd = vv; swi = w; }
             }
-            if (std::isfinite(sd)) { distance = sd; wi = swi; }
+            COVER(COV_EQUAL_DEPTH_SOLID, std::isfinite(sd) && swi != wi);
+        if (std::isfinite(sd)) { distance = sd; wi = swi; }
         }
         // c. selected endpoint (engine.py:11815-11871)
         float sel_along = AL[wi];
@@ -862,15 +874,18 @@ struct Oracle {
                 float v = owner ? D[b] : INF;
                 if (v < sbd) { sbd = v; sbi = b; }
             }
+            COVER(COV_SOLID_BRIDGE, sbd < psd);
             if (sbd < psd) { psd = sbd; psi = sbi; }
         }
         bool has_ps = std::isfinite(psd);
+        COVER(COV_PROJECTED_SOLID, has_ps);
         if (has_ps) { distance = psd; wi = psi; }
         // e. endpoint owner (engine.py:11960-12001)
         int eo_idx; float eo_dist;
         endpoint_owner(x, wi, &eo_idx, &eo_dist);
         bool eo_path_geo = G[wi];
         bool replace_eo = (eo_idx != wi) && (eo_dist > prev_eps);
+        COVER(COV_ENDPOINT_OWNER, replace_eo);
         if (replace_eo) { distance = eo_dist; wi = eo_idx; }
         int no_path_index = wi; float no_path_distance = distance;
         bool no_path_geo = replace_eo ? eo_path_geo : (bool)G[wi];
@@ -891,6 +906,7 @@ struct Oracle {
                 int dummy; topo = sector_bridge(AL[w] > 0.5f ? 1 : 0, w, no_path_index, &dummy);
             }
             if (!(close || topo)) continue;
+            COVER(COV_TOPOLOGICAL_OWNER, topo);
             if (D[w] < npd) { npd = D[w]; npi = w; }
         }
         int pe_s0 = sec(c.pend_ep_wall, 0), pe_s1 = sec(c.pend_ep_wall, 1);
@@ -910,6 +926,8 @@ struct Oracle {
         bool use_psb = psb_dist < npd;
         if (use_psb) { npd = psb_dist; npi = psb_idx; }
         bool replace_np = std::isfinite(npd);
+        COVER(COV_SECTOR_BRIDGE, use_psb);
+        COVER(COV_NEAR_PROJECTED, replace_np);
         if (replace_np) { distance = npd; wi = npi; }
         bool final_proj = P[wi], final_geo = G[wi];
         bool completes_poab = c.pend_ep_boundary && opposing(c.pend_ep_wall, wi) && final_proj && !final_geo;
@@ -920,6 +938,15 @@ struct Oracle {
                             !((pend_ep_has_forward_bridge || completes_pending_endpoint_bridge) && !sel_is_proj && sel_excl_right && !replace_np);
         bool geometric_intersection = replace_np ? no_path_geo : (replace_eo ? eo_path_geo : (bool)G[wi]);
         bool no_keeps = replace_np && no_path_geo && (no_path_other >= 0);
+        ++g_coverage[COV_PASSES];
+        COVER(COV_VALID, valid);
+        COVER(COV_DEAD_COLUMN_REVIVED, valid && cs < 0);
+        COVER(COV_OPPOSING_BOUNDARY, completes_poab);
+        COVER(COV_EXCLUDED_RIGHT_EDGE, valid && excl_only);
+        COVER(COV_CONTINUES_OWNER_BOUNDARY, valid && continues_po_boundary);
+        COVER(COV_FORWARD_BRIDGE, pend_ep_has_forward_bridge);
+        COVER(COV_COMPLETES_ENDPOINT_BRIDGE, valid && completes_pending_endpoint_bridge);
+        COVER(COV_NO_KEEPS_PATH, no_keeps);
         // h. sides (engine.py:12240-12292)
         int front = sec(wi, 0), back = sec(wi, 1);
         bool from_front = cs == front;
@@ -931,6 +958,7 @@ struct Oracle {
         bool ps_from_front = cs == sec(ps_path_index, 0);
         int ps_other = ps_from_front ? sec(ps_path_index, 1) : sec(ps_path_index, 0);
         bool ps_keeps = has_ps && G[ps_path_index] && (ps_other >= 0);
+        COVER(COV_PS_KEEPS_PATH, ps_keeps);
         int safe_other = std::max(render_other, 0);
 
         r.valid = valid; r.raster_valid = raster_valid; r.one_sided = other_sector < 0;
@@ -1034,6 +1062,7 @@ struct Oracle {
             i64 fraction = shl64(texture_mid, 16 - height_bits) + (mul64(vertical_step, screen_delta) >> 16);
             i64 tv = (fraction & UINT32_MASK) >> (32 - height_bits);
             uint8_t texel = m->tex_atlas[(size_t(texture_id) * m->tex_max_h + tv) * m->tex_max_w + tu];
+            COVER(COV_BOTTOM_TAIL, bottom_tail && first_group_visibility != r.visibility);
             i64 shade = wall_shade(light, bottom_tail ? first_group_visibility : r.visibility);
             frame[i] = m->colormap[shade * 256 + texel];
             scene_depth[i] = r.distance;
@@ -1157,6 +1186,13 @@ struct Oracle {
         bool endpoint_portal_bridge = uses_geometric_path && ppb_exists && P[ppb_idx] && LE[ppb_idx] && (ppb_dist > prior_eps) &&
                                       (std::fabs(ppb_dist - gpd) <= gp_tol);
         bool completes_pending_portal_bridge = r.valid && c.pend_pb && (wi == c.pend_pb_index);
+        COVER(COV_ENDPOINT_ONLY_PORTAL, endpoint_only_portal);
+        COVER(COV_TIED_STRIP, enters_tied_strip);
+        COVER(COV_ENTERS_OTHER, enters_other);
+        COVER(COV_ENTERS_SHARED, enters_shared);
+        COVER(COV_GEOMETRIC_PATH, uses_geometric_path);
+        COVER(COV_PORTAL_BRIDGE, endpoint_portal_bridge);
+        COVER(COV_COMPLETES_PORTAL_BRIDGE, completes_pending_portal_bridge);
         // t. previous_distance (engine.py:13242-13275)
         float pd = prior;
         if (r.valid) {
@@ -1289,6 +1325,8 @@ struct Oracle {
             bool extends = initial_post && (float(clipped_bottom) < mfloor) && (frac_end < i64(th) * FIXED_UNIT - dc_iscale);
             clipped_bottom += extends;
             if (!(has_saved || left_edge)) continue;
+            ++g_coverage[COV_MASKED_COLUMN];
+            COVER(COV_MASKED_EXTENDS, extends);
             const float *wl = m->walls + 4 * mw;
             bool horizontal = std::fabs(wl[3] - wl[1]) < 1e-6f, vertical = std::fabs(wl[2] - wl[0]) < 1e-6f;
             float contrast = vertical ? 16.0f : (horizontal ? -16.0f : 0.0f);
@@ -1601,6 +1639,14 @@ void gdo_relation_tables(const gd_map_desc *map, uint8_t *same_pair, uint8_t *op
             sector_bridge_index[(slot * W + a) * W + b] = index;
         }
     }
+}
+
+// Copies the rule-coverage counters (COV_COUNT values) and optionally clears them.
+int gdo_coverage(long long *out, int capacity, int reset) {
+    int n = capacity < COV_COUNT ? capacity : COV_COUNT;
+    for (int i = 0; i < n; ++i) out[i] = g_coverage[i];
+    if (reset) std::memset(g_coverage, 0, sizeof(g_coverage));
+    return COV_COUNT;
 }
 
 void gdo_fine_tables(int64_t *fine_sine, int64_t *fine_tangent) {

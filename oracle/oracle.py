@@ -201,3 +201,21 @@ def relation_tables(tables: dict) -> dict:
     )
     del keep
     return out
+
+
+COVERAGE_NAMES = (
+    "passes", "valid", "equal_depth_solid", "projected_solid", "solid_bridge", "endpoint_owner", "near_projected",
+    "topological_owner", "sector_bridge", "opposing_boundary", "excluded_right_edge", "continues_owner_boundary",
+    "forward_bridge", "completes_endpoint_bridge", "endpoint_only_portal", "tied_strip", "enters_other", "enters_shared",
+    "geometric_path", "portal_bridge", "completes_portal_bridge", "ps_keeps_path", "no_keeps_path", "bottom_tail",
+    "masked_column", "masked_extends", "dead_column_revived",
+)
+
+
+def coverage(reset: bool = False) -> dict:
+    """How often each ownership rule of the wall traversal fired since the last reset."""
+
+    values = (C.c_longlong * len(COVERAGE_NAMES))()
+    count = library().gdo_coverage(values, len(COVERAGE_NAMES), int(reset))
+    assert count == len(COVERAGE_NAMES)
+    return {name: int(values[i]) for i, name in enumerate(COVERAGE_NAMES)}

@@ -58,6 +58,16 @@ CASES = {
         map_seed=1001, grid=(9, 6), sectors=48, linedefs=320, lanes=8, pose_seed=2, pitch=True, flash=True
     ),
     "config1_midtex": dict(map_seed=2001, grid=(9, 6), sectors=48, linedefs=320, lanes=8, pose_seed=3, midtex=0.2),
+    "brick_islands": dict(
+        map_seed=61, grid=(5, 4), sectors=18, linedefs=170, lanes=8, pose_seed=1, layout="brick", islands=6, midtex=0.2
+    ),
+    "grid_islands_sprites": dict(
+        map_seed=62, grid=(6, 5), sectors=26, linedefs=200, lanes=8, pose_seed=1, islands=10, pitch=True, flash=True,
+        sprites=32,
+    ),
+    "brick_islands_320": dict(
+        map_seed=63, grid=(8, 6), sectors=44, linedefs=360, lanes=12, pose_seed=2, layout="brick", islands=16, midtex=0.15
+    ),
     "config2_subset": dict(map_seed=1002, grid=(12, 9), sectors=96, linedefs=800, lanes=4, pose_seed=1, sprites=32),
     "config3_subset": dict(
         map_seed=1003, grid=(15, 15), sectors=200, linedefs=2000, lanes=2, pose_seed=1, sprites=64, flash=True
@@ -70,7 +80,8 @@ CASES = {
 
 def build_case(name: str, cfg: dict, do_time: bool) -> dict:
     smap = synthmap.generate_map(
-        cfg["map_seed"], grid=cfg["grid"], sectors=cfg["sectors"], linedefs=cfg["linedefs"], midtex=cfg.get("midtex", 0.0)
+        cfg["map_seed"], grid=cfg["grid"], sectors=cfg["sectors"], linedefs=cfg["linedefs"], midtex=cfg.get("midtex", 0.0),
+        layout=cfg.get("layout", "grid"), islands=cfg.get("islands", 0),
     )
     lanes = cfg["lanes"]
     started = time.time()
