@@ -115,7 +115,7 @@ def main() -> int:
     stage_ms = renderer.render_timed(states[0], stage_launches, indexed=indexed, obs=obs, frames=frames)
     torch.cuda.synchronize()
     dominant = max(stage_ms, key=stage_ms.get)
-    chunk = min(lanes, 1024)
+    chunk = renderer.chunk_lanes
     chunks = (lanes + chunk - 1) // chunk
     map_bytes = sum(int(np.asarray(v).nbytes) for v in tables.values() if isinstance(v, np.ndarray))
     bytes_per_lane = algorithmic_bytes_per_lane_frame(sprites, map_bytes, lanes)

@@ -54,6 +54,7 @@ MAP_ARRAYS = (
     ("endpoint_neighbors", np.int32),
     ("endpoint_neighbor_starts", np.uint8),
     ("endpoint_neighbor_ends", np.uint8),
+    ("direct_neighbor_table", np.int32),
     ("solid_bridge_start_ofs", np.int32),
     ("solid_bridge_start_idx", np.int32),
     ("solid_bridge_end_ofs", np.int32),

@@ -3,8 +3,8 @@
 // One frame for N lanes runs as a short chain of kernels on one stream:
 //
 //   lane_setup     1 thread / lane          view basis, pitch centre, camera sector
-//   wall_setup     1 thread / (lane, wall)  FWallCoords span+depths, span ownership bounds
-//   column_lists   1 thread / (lane, col)   ray x visible-linedef test -> per-column candidate list
+//   wall_setup     1 thread / (lane, wall)  FWallCoords span+depths, span ownership bounds, and the
+//                                           linedef's entry in the candidate list of every column it can own
 //   flat_select    1 thread / pixel         nearest floor/ceiling sector through the point grid
 //   flat_finish    320 threads / lane       visplane repair (wave ballots) + flat shading
 //   wall_columns   320 threads / lane       portal traversal, tiers, planes, masked mid-textures
@@ -54,6 +54,8 @@ typedef unsigned long long u64;
 #define CF_GEO 1
 #define CF_PROJ 2
 #define CF_LEDGE 4
+#define CF_ALONG_HI 8   // along > 0.5: the ray is nearer the linedef's end vertex
+#define CF_FF 16        // camera on the front side of the linedef (float32 test)
 
 // wall record flags
 #define WF_HC 1        // owns at least one column after every span test
@@ -65,7 +67,7 @@ struct LaneCtx {
     float x, y, view_z, pitch_offset, fsin, fcos;
     i64 view_x_fixed, view_y_fixed, vsin, vcos, center_fixed, flash_light;
     int sector;
-    int visible_count;
+    int pad;
 };
 
 struct WallRec {   // one linedef seen from one lane
@@ -77,9 +79,17 @@ struct WallRec {   // one linedef seen from one lane
     int flags;
 };
 
-struct Cand {      // one linedef with a finite ray distance at one column
-    int wall;
-    float dist, along;
+struct Cand {      // one linedef with a finite ray distance at one column, with the static
+                   // linedef facts every scan needs packed in so that scans do no gathers
+    unsigned short wall, flags;
+    short s0, s1;            // front / back sector (-1 = none)
+    unsigned short v0, v1;   // vertex ids of start / end
+    float dist;
+};
+
+struct Eval {      // distances/along/geometric/projected/left-edge of one linedef at one column;
+                   // CF_ALONG_HI in flags carries (along > 0.5), the only use the traversal makes of along
+    float dist;
     int flags;
 };
 
@@ -93,9 +103,8 @@ struct DeviceMap {  // device copy of gd_map_desc (device pointers) + fixed tabl
 struct Scratch {    // per-chunk working memory, sized at create
     LaneCtx *ctx;          // [L]
     WallRec *rec;          // [L,W]
-    int *visible;          // [L,W] compact list of linedefs that can own a column
     Cand *cand;            // [L,CAND_MAX,320]
-    unsigned char *cand_count;  // [L,320]
+    int *cand_count;       // [L,320] (may exceed CAND_MAX when a list overflowed)
     unsigned short *flat_sector;// [L,208,320]
     unsigned char *flat_flags;  // [L,208,320] bit0 unresolved
     unsigned int *meta;    // [L,208,320] filled | floor | plane_sector+1 | clip_wall+1
@@ -114,7 +123,19 @@ struct Scratch {    // per-chunk working memory, sized at create
 
 __device__ __forceinline__ i64 mul64(i64 a, i64 b) { return (i64)((u64)a * (u64)b); }
 __device__ __forceinline__ i64 shl64(i64 a, int s) { return (i64)((u64)a << s); }
-__device__ __forceinline__ i64 tdiv(i64 a, i64 b) { return a / b; }
+// C truncating division (engine.py:3115-3118).  gfx950 has no 64-bit integer divider; when both
+// magnitudes are below 2^52 the quotient estimated in float64 is within one of the true quotient
+// and one remainder check makes it exact.  Larger operands take the compiler's long division.
+__device__ __forceinline__ i64 tdiv(i64 a, i64 b) {
+    u64 ua = a < 0 ? (u64)0 - (u64)a : (u64)a;
+    u64 ub = b < 0 ? (u64)0 - (u64)b : (u64)b;
+    if (((ua | ub) >> 52) != 0 || ub == 0) return b == 0 ? 0 : a / b;
+    u64 uq = (u64)((double)ua / (double)ub);
+    u64 prod = uq * ub;
+    if (prod > ua) --uq;
+    else if (ua - prod >= ub) ++uq;
+    return ((a < 0) != (b < 0)) ? -(i64)uq : (i64)uq;
+}
 __device__ __forceinline__ i64 clampi(i64 v, i64 lo, i64 hi) { return v < lo ? lo : (v > hi ? hi : v); }
 __device__ __forceinline__ i64 max64(i64 a, i64 b) { return a > b ? a : b; }
 __device__ __forceinline__ i64 min64(i64 a, i64 b) { return a < b ? a : b; }
@@ -257,8 +278,9 @@ __global__ void lane_setup_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_ba
     c.center_fixed = (i64)(VH / 2) * FIXED_UNIT + ((FOCAL_Y_FIXED * tangent) >> 16);
     c.pitch_offset = (float)((tangent * 12582912LL) >> 16) / 65536.0f;
     c.sector = sector_at(&dm.d, c.x, c.y);
-    c.visible_count = 0;
+    c.pad = 0;
     sc.ctx[local] = c;
+    for (int x = 0; x < SW; ++x) sc.cand_count[(size_t)local * SW + x] = 0;
 }
 
 __device__ __forceinline__ void ray_direction(const LaneCtx &c, int x, float *rx, float *ry) {
@@ -266,6 +288,32 @@ __device__ __forceinline__ void ray_direction(const LaneCtx &c, int x, float *rx
     float col = ((float)x - 160.0f) / 160.0f;
     *rx = c.fcos + c.fsin * col;
     *ry = c.fsin - c.fcos * col;
+}
+
+// distances / along / geometric / projected / left-edge of one linedef at one column
+// (engine.py:11317-11331, 11440-11460)
+__device__ __forceinline__ Eval eval_segment(const float4 wl, const WallRec &r, bool os, const LaneCtx &c, int x, float rx, float ry) {
+    float segx = wl.z - wl.x, segy = wl.w - wl.y;
+    float offx = wl.x - c.x, offy = wl.y - c.y;
+    float den = rx * segy - ry * segx;
+    bool ok = fabsf(den) >= 1e-6f;
+    float safe = ok ? den : 1.0f;
+    float d = (offx * segy - offy * segx) / safe;
+    float a = (offx * ry - offy * rx) / safe;
+    bool g = ok && (d > 0) && (a >= 0) && (a <= 1);
+    bool screen_valid = (r.flags & WF_HC) && (x >= r.pl) && (x < r.pr);
+    bool p = ok && (d > 0) && screen_valid;
+    bool valid = os ? (p && (r.flags & WF_FF)) : (g || p);
+    Eval out;
+    out.dist = valid ? d : GD_INF;
+    out.flags = (g ? CF_GEO : 0) | (p ? CF_PROJ : 0) | ((x == r.pl) ? CF_LEDGE : 0) | ((a > 0.5f) ? CF_ALONG_HI : 0) |
+                ((r.flags & WF_FF) ? CF_FF : 0);
+    return out;
+}
+
+__device__ __forceinline__ Eval eval_wall(const gd_map_desc *m, const LaneCtx &c, const WallRec *recs, int x, int w, float rx, float ry) {
+    const float4 wl = *reinterpret_cast<const float4 *>(m->walls + 4 * w);
+    return eval_segment(wl, recs[w], m->wall_sectors[2 * w + 1] < 0, c, x, rx, ry);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -305,13 +353,33 @@ __global__ void wall_setup_kernel(DeviceMap dm, int lane_count, Scratch sc) {
     bool invalid = invalid_left || invalid_right || (sr <= sl);
     if (invalid) sr = sl;
 
-    // ray x segment over all columns: first / last geometric hit (engine.py:11323-11348)
+    // Ray x segment: first / last column whose ray hits the segment (engine.py:11323-11348).
+    // A ray of column parameter col = (x-160)/160 is forward + col*right; an endpoint with view
+    // coordinates (f, r) lies on it when r = col*f.  The float test below can only pass where the
+    // two endpoints are not both clearly (> half a map unit) on one side of the ray, so for a
+    // segment wholly in front of the camera only the columns between its endpoint columns
+    // (padded) are examined; segments reaching behind the camera get the full scan.
     const float4 wl = *reinterpret_cast<const float4 *>(m->walls + 4 * w);
     float segx = wl.z - wl.x, segy = wl.w - wl.y;
     float offx = wl.x - c.x, offy = wl.y - c.y;
+    int scan_lo = 0, scan_hi = SW - 1;
+    {
+        float e1x = offx + segx, e1y = offy + segy;
+        float f0 = offx * c.fcos + offy * c.fsin, r0 = offx * c.fsin - offy * c.fcos;
+        float f1 = e1x * c.fcos + e1y * c.fsin, r1 = e1x * c.fsin - e1y * c.fcos;
+        if (f0 > 1.0f && f1 > 1.0f) {
+            float c0 = r0 / f0, c1 = r1 / f1, p0 = 0.5f / f0, p1 = 0.5f / f1;
+            float lo = fminf(c0 - p0, c1 - p1), hi = fmaxf(c0 + p0, c1 + p1);
+            float xlo = floorf(160.0f + 160.0f * lo) - 1.0f, xhi = ceilf(160.0f + 160.0f * hi) + 1.0f;
+            scan_lo = xlo < 0.0f ? 0 : (xlo > 320.0f ? 320 : (int)xlo);
+            scan_hi = xhi > 319.0f ? 319 : (xhi < -1.0f ? -1 : (int)xhi);
+        } else if (f0 < -1.0f && f1 < -1.0f) {
+            scan_lo = 1; scan_hi = 0;   // wholly behind the camera: no ray reaches it
+        }
+    }
     int first = 0, last = SW - 1; bool any = false;
     float numer_d = offx * segy - offy * segx;
-    for (int x = 0; x < SW; ++x) {
+    for (int x = scan_lo; x <= scan_hi; ++x) {
         float rx, ry; ray_direction(c, x, &rx, &ry);
         float den = rx * segy - ry * segx;
         bool ok = fabsf(den) >= 1e-6f;
@@ -345,75 +413,42 @@ __global__ void wall_setup_kernel(DeviceMap dm, int lane_count, Scratch sc) {
         hc = screen_right > screen_left;
     }
     hc = hc && (sr > sl);
-    bool os = m->wall_sectors[2 * w + 1] < 0;
+    const int s0 = m->wall_sectors[2 * w], s1 = m->wall_sectors[2 * w + 1];
+    bool os = s1 < 0;
     WallRec r;
     r.tx0 = (int)tx0; r.tx1 = (int)tx1v; r.ty0 = (int)ty0; r.ty1 = (int)ty1v;
     r.dl = dl; r.dr = dr; r.sl = sl; r.sr = sr;
     r.pl = (short)screen_left; r.pr = (short)screen_right;
     r.flags = (hc ? WF_HC : 0) | (ff ? WF_FF : 0) | (((sr - sl <= 1) && !os) ? WF_SUBPIXEL : 0) | (any ? WF_ANYGEO : 0);
     sc.rec[(size_t)local * m->wall_count + w] = r;
-    // A linedef can have a finite distance at some column only if it owns a span
-    // (projected) or, for two-sided lines, is hit by a ray (engine.py:11446-11451).
-    bool can_be_finite = os ? (hc && ff) : (hc || any);
-    if (can_be_finite) {
-        int slot = atomicAdd(&sc.ctx[local].visible_count, 1);
-        sc.visible[(size_t)local * m->wall_count + slot] = w;
-    }
-}
-
-// distances / along / geometric / projected / left-edge of one linedef at one column
-// (engine.py:11317-11331, 11440-11460)
-__device__ __forceinline__ Cand eval_wall(const gd_map_desc *m, const LaneCtx &c, const WallRec *recs, int x, int w, float rx, float ry) {
-    const float4 wl = *reinterpret_cast<const float4 *>(m->walls + 4 * w);
-    const WallRec &r = recs[w];
-    float segx = wl.z - wl.x, segy = wl.w - wl.y;
-    float offx = wl.x - c.x, offy = wl.y - c.y;
-    float den = rx * segy - ry * segx;
-    bool ok = fabsf(den) >= 1e-6f;
-    float safe = ok ? den : 1.0f;
-    float d = (offx * segy - offy * segx) / safe;
-    float a = (offx * ry - offy * rx) / safe;
-    bool g = ok && (d > 0) && (a >= 0) && (a <= 1);
-    bool screen_valid = (r.flags & WF_HC) && (x >= r.pl) && (x < r.pr);
-    bool p = ok && (d > 0) && screen_valid;
-    bool os = m->wall_sectors[2 * w + 1] < 0;
-    bool valid = os ? (p && (r.flags & WF_FF)) : (g || p);
-    Cand out;
-    out.wall = w;
-    out.dist = valid ? d : GD_INF;
-    out.along = a < 0.0f ? 0.0f : (a > 1.0f ? 1.0f : a);
-    out.flags = (g ? CF_GEO : 0) | (p ? CF_PROJ : 0) | ((x == r.pl) ? CF_LEDGE : 0);
-    return out;
-}
-
-// ---------------------------------------------------------------------------------------------
-// column_lists: finite-distance linedefs of every column, in ascending linedef order is NOT
-// required: every reduction below breaks distance ties on the linedef index explicitly.
-// ---------------------------------------------------------------------------------------------
-__global__ void column_lists_kernel(DeviceMap dm, int lane_count, Scratch sc) {
-    const gd_map_desc *m = &dm.d;
-    int local = blockIdx.x;
-    int x = threadIdx.x;
-    if (local >= lane_count || x >= SW) return;
-    const LaneCtx &c = sc.ctx[local];
-    const WallRec *recs = sc.rec + (size_t)local * m->wall_count;
-    const int *visible = sc.visible + (size_t)local * m->wall_count;
-    Cand *list = sc.cand + (size_t)local * CAND_MAX * SW;
-    float rx, ry; ray_direction(c, x, &rx, &ry);
-    int count = 0;
-    bool overflow = false;
-    const int visible_count = c.visible_count;
-    for (int k = 0; k < visible_count; ++k) {
-        int w = visible[k];
-        Cand cd = eval_wall(m, c, recs, x, w, rx, ry);
-        if (finitef(cd.dist)) {
-            if (count < CAND_MAX) list[(size_t)count * SW + x] = cd;
-            else overflow = true;
-            ++count;
+    // Enter the linedef in the candidate list of every column where its distance can be
+    // finite: its owned span (projected) and, for two-sided lines, the columns its rays hit
+    // (engine.py:11446-11451).  List order is irrelevant: scans break ties on the linedef index.
+    int a_lo = SW, a_hi = 0;
+    if (hc && (!os || ff)) { a_lo = r.pl; a_hi = r.pr; }
+    if (!os && any) { a_lo = a_lo < first ? a_lo : first; a_hi = a_hi > last + 1 ? a_hi : last + 1; }
+    a_lo = a_lo < 0 ? 0 : a_lo; a_hi = a_hi > SW ? SW : a_hi;
+    if (a_lo < a_hi) {
+        Cand *list = sc.cand + (size_t)local * CAND_MAX * SW;
+        int *counts = sc.cand_count + (size_t)local * SW;
+        Cand entry;
+        entry.wall = (unsigned short)w; entry.s0 = (short)s0; entry.s1 = (short)s1;
+        entry.v0 = (unsigned short)m->wall_vertex[2 * w]; entry.v1 = (unsigned short)m->wall_vertex[2 * w + 1];
+        for (int x = a_lo; x < a_hi; ++x) {
+            float rx, ry; ray_direction(c, x, &rx, &ry);
+            Eval e = eval_segment(wl, r, os, c, x, rx, ry);
+            if (finitef(e.dist)) {
+                int slot = atomicAdd(&counts[x], 1);
+                if (slot < CAND_MAX) {
+                    entry.flags = (unsigned short)e.flags;
+                    entry.dist = e.dist;
+                    list[(size_t)slot * SW + x] = entry;
+                } else {
+                    atomicOr(sc.status, STATUS_CAND_OVERFLOW);
+                }
+            }
         }
     }
-    if (overflow) { atomicOr(sc.status, STATUS_CAND_OVERFLOW); count = CAND_MAX; }
-    sc.cand_count[(size_t)local * SW + x] = (unsigned char)count;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -612,7 +647,7 @@ struct ColumnCtx {
     int x;
     float rx, ry;
     __device__ Cand cand(int k) const { return list[(size_t)k * SW + x]; }
-    __device__ Cand eval(int w) const { return eval_wall(m, *c, recs, x, w, rx, ry); }
+    __device__ Eval eval(int w) const { return eval_wall(m, *c, recs, x, w, rx, ry); }
 };
 
 // engine.py:11217-11291 for one endpoint order, evaluated at one column
@@ -725,25 +760,23 @@ __device__ __forceinline__ i64 wall_shade(float light, i64 visibility) {
 }
 
 // engine.py:11596-11730 for one (column, linedef)
-__device__ void endpoint_owner(const ColumnCtx &cc, int w, const Cand &cw, int *owner_index, float *owner_distance) {
+__device__ void endpoint_owner(const ColumnCtx &cc, int w, const Eval &cw, int *owner_index, float *owner_distance) {
     const gd_map_desc *m = cc.m;
     const int K = m->neighbor_slots;
     const bool subpixel = cc.recs[w].flags & WF_SUBPIXEL;
     float tol_w = tolerance_of(cw.dist);
-    bool uses_start = cw.along <= 0.5f;
+    bool uses_start = !(cw.flags & CF_ALONG_HI);
     int index; float distance; bool valid;
     if (m->direct_neighbors) {
-        int ss = 0, es = 0; bool hs = false, he = false;
-        for (int k = K - 1; k >= 0; --k) {
-            if (m->endpoint_neighbor_starts[w * K + k]) { ss = k; hs = true; }
-            if (m->endpoint_neighbor_ends[w * K + k]) { es = k; he = true; }
-        }
+        // {start neighbour, end neighbour, start slot | end slot << 8 | has start << 16 | has end << 17}
+        const int4 nb = *reinterpret_cast<const int4 *>(m->direct_neighbor_table + 4 * w);
+        int ss = nb.z & 0xFF, es = (nb.z >> 8) & 0xFF; bool hs = (nb.z >> 16) & 1, he = (nb.z >> 17) & 1;
         int rslot = uses_start ? ss : es, oslot = uses_start ? es : ss;
         bool rexists = uses_start ? hs : he, oexists = uses_start ? he : hs;
-        int rn = m->endpoint_neighbors[w * K + rslot], on = m->endpoint_neighbors[w * K + oslot];
-        Cand r = cc.eval(rn);
+        int rn = uses_start ? nb.x : nb.y, on = uses_start ? nb.y : nb.x;
+        Eval r = cc.eval(rn);
         bool r_owns = rexists && (r.flags & CF_PROJ) && (r.flags & CF_LEDGE);
-        Cand o = (on == rn) ? r : cc.eval(on);
+        Eval o = (on == rn) ? r : cc.eval(on);
         bool o_owns = subpixel && oexists && (o.flags & CF_PROJ) && (o.flags & CF_LEDGE) && (fabsf(o.dist - cw.dist) <= tol_w);
         bool use_o = o_owns && (!r_owns || (o.dist < r.dist) || ((o.dist == r.dist) && (oslot < rslot)));
         index = use_o ? on : rn;
@@ -754,7 +787,7 @@ __device__ void endpoint_owner(const ColumnCtx &cc, int w, const Cand &cw, int *
         for (int k = 0; k < K; ++k) {
             int n = m->endpoint_neighbors[w * K + k];
             bool st = m->endpoint_neighbor_starts[w * K + k], en = m->endpoint_neighbor_ends[w * K + k];
-            Cand nb = cc.eval(n);
+            Eval nb = cc.eval(n);
             bool ray_nb = uses_start ? st : en;
             bool selected = ray_nb || (subpixel && (st || en) && (fabsf(nb.dist - cw.dist) <= tol_w));
             float v = ((nb.flags & CF_PROJ) && (nb.flags & CF_LEDGE) && selected) ? nb.dist : GD_INF;
@@ -820,7 +853,7 @@ struct PassColumn {
 #define PB_PS_FROM_FRONT 0x1000
 #define PB_CONTINUES_PO 0x2000
 #define PB_FORWARD_BRIDGE 0x4000
-#define PB_GEO_FINAL 0x8000
+#define PB_FINAL_ALONG_HI 0x8000
 
 // (distance, linedef) lexicographic minimum: what torch.min(dim) returns on ascending indices
 __device__ __forceinline__ void take_min(float v, int w, float &best, int &best_w) {
@@ -837,31 +870,32 @@ __device__ void pass_select(const ColumnCtx &cc, const ColumnState &c, bool boun
     const float prev = c.previous_distance;
     const float prev_eps = prev + 1e-3f;
     auto incident = [&](int w) { return mv.sec(w, 0) == cur || mv.sec(w, 1) == cur; };
+    auto incident_c = [&](const Cand &q) { return q.s0 == cur || q.s1 == cur; };
     // a. nearest incident linedef beyond previous_distance (engine.py:11769-11780)
     float distance = GD_INF; int wi = 0x7fffffff;
+    Eval cwi;
     if (cs >= 0) {
-        for (int k = 0; k < cc.count; ++k) {
-            Cand q = cc.cand(k);
-            if (incident(q.wall) && q.dist > prev) take_min(q.dist, q.wall, distance, wi);
-        }
-        // b. equal-depth solid (engine.py:11784-11807)
+        // b. equal-depth solid (engine.py:11784-11807): the nearest one-sided candidate replaces
+        // the selection when it lies within 1e-3 of the nearest candidate, found in the same scan.
         float sd = GD_INF; int swi = 0x7fffffff;
+        int wi_flags = 0, swi_flags = 0;
         for (int k = 0; k < cc.count; ++k) {
             Cand q = cc.cand(k);
-            if (incident(q.wall) && q.dist > prev && mv.one_sided(q.wall) && (fabsf(q.dist - distance) <= 1e-3f)) take_min(q.dist, q.wall, sd, swi);
+            if (!(incident_c(q) && q.dist > prev)) continue;
+            if (q.dist < distance || (q.dist == distance && (int)q.wall < wi)) { distance = q.dist; wi = q.wall; wi_flags = q.flags; }
+            if ((q.s1 < 0) && (q.dist < sd || (q.dist == sd && (int)q.wall < swi))) { sd = q.dist; swi = q.wall; swi_flags = q.flags; }
         }
-        if (finitef(sd)) { distance = sd; wi = swi; }
+        if (finitef(sd) && (fabsf(sd - distance) <= 1e-3f)) { distance = sd; wi = swi; wi_flags = swi_flags; }
+        cwi.dist = distance; cwi.flags = wi_flags;
     }
-    if (!finitef(distance)) wi = 0;
-    Cand cwi = cc.eval(wi);
+    if (!finitef(distance)) { wi = 0; cwi = cc.eval(0); }
     // c. selected endpoint (engine.py:11815-11871)
-    float sel_along = cwi.along;
-    bool sel_start = sel_along <= 0.5f;
+    bool sel_start = !(cwi.flags & CF_ALONG_HI);
     int sel_vertex = mv.vert(wi, sel_start ? 0 : 1);
-    auto shares_sel = [&](int w) { return mv.vert(w, 0) == sel_vertex || mv.vert(w, 1) == sel_vertex; };
+    auto shares_sel_c = [&](const Cand &q) { return (int)q.v0 == sel_vertex || (int)q.v1 == sel_vertex; };
     bool continues_po_boundary = (c.flags & ST_PO) && (sel_vertex == c.pend_po_vertex);
     bool continues_ep_boundary = (c.flags & ST_EP) && (sel_vertex == c.pend_ep_vertex);
-    int sel_slot = sel_along > 0.5f ? 1 : 0;
+    int sel_slot = sel_start ? 0 : 1;
     int fb_idx; bool fb_exists = mv.portal_bridge(sel_slot, wi, c.pend_ep_wall, &fb_idx);
     bool pend_ep_has_forward_bridge = false;
     if (continues_ep_boundary && fb_exists) pend_ep_has_forward_bridge = cc.eval(fb_idx).dist > distance + 1e-3f;
@@ -871,30 +905,30 @@ __device__ void pass_select(const ColumnCtx &cc, const ColumnState &c, bool boun
     // d. projected solid owner (engine.py:11872-11954)
     float ps_path_distance = distance; int ps_path_index = wi;
     bool ps_path_geo = cwi.flags & CF_GEO;
-    float psd = GD_INF; int psi = 0x7fffffff;
+    float psd = GD_INF; int psi = 0x7fffffff; int psi_flags = 0;
     if (!sel_is_proj) {
         for (int k = 0; k < cc.count; ++k) {
             Cand q = cc.cand(k);
-            bool owner = incident(q.wall) && mv.one_sided(q.wall) && (q.flags & CF_PROJ) && (q.flags & CF_LEDGE) && shares_sel(q.wall) && (q.dist > prev_eps);
-            if (owner) take_min(q.dist, q.wall, psd, psi);
+            bool owner = incident_c(q) && (q.s1 < 0) && (q.flags & CF_PROJ) && (q.flags & CF_LEDGE) && shares_sel_c(q) && (q.dist > prev_eps);
+            if (owner && (q.dist < psd || (q.dist == psd && (int)q.wall < psi))) { psd = q.dist; psi = q.wall; psi_flags = q.flags; }
         }
         if (sel_excl_right) {
             const int *ofs = sel_start ? m->solid_bridge_start_ofs : m->solid_bridge_end_ofs;
             const int *idx = sel_start ? m->solid_bridge_start_idx : m->solid_bridge_end_idx;
-            float sbd = GD_INF; int sbi = 0;
+            float sbd = GD_INF; int sbi = 0; int sbi_flags = 0;
             for (int k = ofs[wi]; k < ofs[wi + 1]; ++k) {
                 int b = idx[k];
                 if (!(incident(b) && mv.one_sided(b))) continue;
-                Cand q = cc.eval(b);
+                Eval q = cc.eval(b);
                 bool owner = (q.flags & CF_PROJ) && (q.flags & CF_LEDGE) && (q.dist > prev_eps);
                 float v = owner ? q.dist : GD_INF;
-                if (v < sbd) { sbd = v; sbi = b; }   // list is ascending: first slot wins ties
+                if (v < sbd) { sbd = v; sbi = b; sbi_flags = q.flags; }   // list is ascending: first slot wins ties
             }
-            if (sbd < psd) { psd = sbd; psi = sbi; }
+            if (sbd < psd) { psd = sbd; psi = sbi; psi_flags = sbi_flags; }
         }
     }
     bool has_ps = finitef(psd);
-    if (has_ps) { distance = psd; wi = psi; cwi = cc.eval(wi); }
+    if (has_ps) { distance = psd; wi = psi; cwi.dist = psd; cwi.flags = psi_flags; }
     // e. endpoint owner (engine.py:11960-12001)
     int eo_idx; float eo_dist;
     endpoint_owner(cc, wi, cwi, &eo_idx, &eo_dist);
@@ -911,18 +945,20 @@ __device__ void pass_select(const ColumnCtx &cc, const ColumnState &c, bool boun
     bool so_excl_right = so_rec.sr == x;
     i64 so_span = so_rec.sr - so_rec.sl;
     bool so_short = m->wall_len[wi] <= 32.0f;
-    float npd = GD_INF; int npi = 0x7fffffff;
+    float npd = GD_INF; int npi = 0x7fffffff; int npi_flags = 0;
+    const int so_s0 = mv.sec(wi, 0), so_s1 = mv.sec(wi, 1);
     if (!so_is_proj) {
         for (int k = 0; k < cc.count; ++k) {
             Cand q = cc.cand(k);
             int w = q.wall;
-            if (!(incident(w) && !mv.one_sided(w) && (q.flags & CF_PROJ) && (q.dist > prev_eps))) continue;
+            if (!(incident_c(q) && (q.s1 >= 0) && (q.flags & CF_PROJ) && (q.dist > prev_eps))) continue;
             bool le = q.flags & CF_LEDGE;
-            bool close = (mv.same_pair(wi, w) || (le && so_excl_right && ((so_span <= 2) || (shares_sel(w) && so_short)))) &&
+            bool same_pair = (q.s0 == so_s0 && q.s1 == so_s1) || (q.s0 == so_s1 && q.s1 == so_s0);
+            bool close = (same_pair || (le && so_excl_right && ((so_span <= 2) || (shares_sel_c(q) && so_short)))) &&
                          (fabsf(q.dist - distance) <= tolerance_of(q.dist));
             bool topo = false;
-            if (!close && le && so_excl_right && so_span <= 2) { int dummy; topo = mv.sector_bridge(q.along > 0.5f ? 1 : 0, w, no_path_index, &dummy); }
-            if (close || topo) take_min(q.dist, w, npd, npi);
+            if (!close && le && so_excl_right && so_span <= 2) { int dummy; topo = mv.sector_bridge((q.flags & CF_ALONG_HI) ? 1 : 0, w, no_path_index, &dummy); }
+            if ((close || topo) && (q.dist < npd || (q.dist == npd && w < npi))) { npd = q.dist; npi = w; npi_flags = q.flags; }
         }
     }
     int pe_wall = c.pend_ep_wall;
@@ -938,14 +974,14 @@ __device__ void pass_select(const ColumnCtx &cc, const ColumnState &c, bool boun
         if (psb_exists) {
             int b0 = mv.sec(psb_idx, 0), b1 = mv.sec(psb_idx, 1);
             bool matches = (b0 == pe_other && b1 == no_path_other) || (b1 == pe_other && b0 == no_path_other);
-            Cand qb = cc.eval(psb_idx);
+            Eval qb = cc.eval(psb_idx);
             float pe_tol = tolerance_of(cc.eval(pe_wall).dist);
             bool psb = matches && (qb.flags & CF_PROJ) && (qb.flags & CF_LEDGE) && (qb.dist > prev - pe_tol) && (qb.dist < no_path_distance);
-            if (psb && qb.dist < npd) { use_psb = true; npd = qb.dist; npi = psb_idx; }
+            if (psb && qb.dist < npd) { use_psb = true; npd = qb.dist; npi = psb_idx; npi_flags = qb.flags; }
         }
     }
     bool replace_np = finitef(npd);
-    if (replace_np) { distance = npd; wi = npi; cwi = cc.eval(wi); }
+    if (replace_np) { distance = npd; wi = npi; cwi.dist = npd; cwi.flags = npi_flags; }
     bool final_proj = cwi.flags & CF_PROJ, final_geo = cwi.flags & CF_GEO;
     bool completes_poab = (c.flags & ST_EP) && final_proj && !final_geo && mv.opposing(pe_wall, wi);
     // g. validity (engine.py:12197-12239)
@@ -996,7 +1032,7 @@ __device__ void pass_select(const ColumnCtx &cc, const ColumnState &c, bool boun
              (tier1 ? PB_TIER1 : 0) | (tier2 ? PB_TIER2 : 0) | (mark_ceiling ? PB_MARK_CEILING : 0) | (mark_floor ? PB_MARK_FLOOR : 0) |
              (ps_keeps ? PB_PS_KEEPS : 0) | (no_keeps ? PB_NO_KEEPS : 0) | (geometric_intersection ? PB_GEOMETRIC : 0) |
              (replace_np ? PB_REPLACE_NP : 0) | (ps_from_front ? PB_PS_FROM_FRONT : 0) | (continues_po_boundary ? PB_CONTINUES_PO : 0) |
-             (pend_ep_has_forward_bridge ? PB_FORWARD_BRIDGE : 0);
+             (pend_ep_has_forward_bridge ? PB_FORWARD_BRIDGE : 0) | ((cwi.flags & CF_ALONG_HI) ? PB_FINAL_ALONG_HI : 0);
 }
 
 struct PixelBuffers {
@@ -1037,8 +1073,14 @@ __device__ void apply_silhouette(PixelBuffers &pb, SilhouetteBounds &sb, int x, 
 }
 
 // engine.py:12637-12884
+// `window_dirty` says whether some pixel inside the open window [ceiling_clip, floor_clip) may
+// already be filled, plane-owned or carry a sprite-clip depth.  A two-sided drawseg only writes
+// rows that its own clip update then removes from the window, so the window stays untouched
+// until a one-sided drawseg (which leaves the clips alone) has painted; until then painting
+// needs no reads and visits only the rows it writes.
 __device__ void pass_paint(const ColumnCtx &cc, const ColumnState &c, const PassColumn &r, PixelBuffers &pb,
-                           const bool group_valid[3], const float group_bottom[3], i64 first_group_visibility) {
+                           const bool group_valid[3], const float group_bottom[3], i64 first_group_visibility,
+                           const unsigned char *colormap, bool &window_dirty) {
     if (!(r.bits & PB_RASTER)) return;
     const gd_map_desc *m = cc.m;
     const LaneCtx &L = *cc.c;
@@ -1066,6 +1108,50 @@ __device__ void pass_paint(const ColumnCtx &cc, const ColumnState &c, const Pass
     int y1 = c.floor_clip >= (float)VH ? VH : (int)c.floor_clip;
     const bool lower_on = !one_sided && (r.view_floor < r.other_floor);
     const bool upper_on = !one_sided && (r.view_ceiling > r.other_ceiling);
+    if (!window_dirty) {
+        // clips and projections hold integers in [0, 208]
+        const unsigned claim = (unsigned)(r.render_current + 1) << META_SECTOR_SHIFT;
+        if (r.bits & PB_MARK_CEILING) {
+            int e = (int)ceiling_plane_bottom;
+            for (int y = y0; y < e; ++y) pb.meta[(size_t)y * SW + x] = claim;
+        }
+        if (r.bits & PB_MARK_FLOOR) {
+            int b = (int)floor_plane_top;
+            for (int y = b; y < y1; ++y) pb.meta[(size_t)y * SW + x] = claim | META_FLOOR;
+        }
+        int t0 = VH, t1 = 0;
+        if (one_sided) { t0 = (int)r.clipped_top; t1 = (int)r.clipped_bottom; }
+        if (lower_on) { t0 = min(t0, (int)r.clipped_lower_top); t1 = max(t1, (int)r.clipped_bottom); }
+        if (upper_on) { t0 = min(t0, (int)r.clipped_top); t1 = max(t1, (int)r.clipped_upper_bottom); }
+        for (int y = t0; y < t1; ++y) {
+            const float py = (float)y;
+            bool one_span = one_sided && (py >= r.clipped_top) && (py < r.clipped_bottom);
+            bool lower_span = lower_on && (py >= r.clipped_lower_top) && (py < r.clipped_bottom);
+            bool upper_span = upper_on && (py >= r.clipped_top) && (py < r.clipped_upper_bottom);
+            if (!(one_span || lower_span || upper_span)) continue;
+            int texture_id = one_span ? r.side_tex[0] : (lower_span ? r.side_tex[1] : r.side_tex[2]);
+            if (texture_id < 0) continue;
+            bool bottom_tail = (one_span && group_valid[0] && py >= group_bottom[0]) ||
+                               (lower_span && group_valid[1] && py >= group_bottom[1]) ||
+                               (upper_span && group_valid[2] && py >= group_bottom[2]);
+            int tw = m->tex_w[texture_id], th = m->tex_h[texture_id];
+            i64 tu = u_base & (i64)(tw - 1);
+            float origin_z = one_span ? r.view_ceiling : (lower_span ? r.other_floor : r.other_ceiling);
+            int height_bits = ilog2(th);
+            i64 vertical_step = mul64(swall, shl64(1, 14 - height_bits));
+            i64 screen_delta = (i64)y * FIXED_UNIT - L.center_fixed + FIXED_UNIT;
+            i64 texture_mid = round_to_i64((origin_z - L.view_z) * 65536.0f + toff[1] * 65536.0f);
+            i64 fraction = shl64(texture_mid, 16 - height_bits) + (mul64(vertical_step, screen_delta) >> 16);
+            i64 tv = (fraction & UINT32_MASK) >> (32 - height_bits);
+            unsigned char texel = m->tex_atlas[((size_t)texture_id * m->tex_max_h + tv) * m->tex_max_w + tu];
+            const size_t i = (size_t)y * SW + x;
+            pb.frame[i] = colormap[(bottom_tail ? shade_group : shade_own) * 256 + texel];
+            pb.clip_depth[i] = r.distance;
+            pb.meta[i] = META_FILLED | (unsigned)(wi + 1);
+        }
+        if (one_sided) window_dirty = true;
+        return;
+    }
     for (int y = y0; y < y1; ++y) {
         const float py = (float)y;
         const size_t i = (size_t)y * SW + x;
@@ -1096,7 +1182,7 @@ __device__ void pass_paint(const ColumnCtx &cc, const ColumnState &c, const Pass
                 i64 fraction = shl64(texture_mid, 16 - height_bits) + (mul64(vertical_step, screen_delta) >> 16);
                 i64 tv = (fraction & UINT32_MASK) >> (32 - height_bits);
                 unsigned char texel = m->tex_atlas[((size_t)texture_id * m->tex_max_h + tv) * m->tex_max_w + tu];
-                pb.frame[i] = m->colormap[(bottom_tail ? shade_group : shade_own) * 256 + texel];
+                pb.frame[i] = colormap[(bottom_tail ? shade_group : shade_own) * 256 + texel];
                 if (r.distance < pb.clip_depth[i]) { pb.clip_depth[i] = r.distance; meta = (meta & ~META_WALL_MASK) | (unsigned)(wi + 1); }
                 meta |= META_FILLED;
                 meta_dirty = true;
@@ -1174,30 +1260,29 @@ __device__ bool pass_advance(const ColumnCtx &cc, ColumnState &c, const PassColu
     bool endpoint_portal_bridge = false;
     int ppb_idx = 0, gp_other = -1; float gpd = GD_INF;
     if (endpoint_only_portal) {
-        auto other_incident = [&](int w) { return mv.sec(w, 0) == other_sector || mv.sec(w, 1) == other_sector; };
         const float dist_eps = distance + 1e-3f;
         float cnd = GD_INF, ond = GD_INF; int cni = 0x7fffffff, oni = 0x7fffffff;
         float csd = GD_INF, osd = GD_INF;
-        int gpi = 0x7fffffff; float gp_along = 0.0f;
+        int gpi = 0x7fffffff; bool gp_along_hi = false;
         const int v0 = mv.vert(wi, 0), v1 = mv.vert(wi, 1);
         for (int k = 0; k < cc.count; ++k) {
             Cand q = cc.cand(k);
             int w = q.wall; float d = q.dist;
-            bool os = mv.one_sided(w);
-            bool inc = incident(w), oinc = other_incident(w);
+            bool os = q.s1 < 0;
+            bool inc = (q.s0 == cur || q.s1 == cur), oinc = (q.s0 == other_sector || q.s1 == other_sector);
             bool future = ((q.flags & CF_GEO) || os) && (d > dist_eps);
             if (future) {
                 if (inc) take_min(d, w, cnd, cni);
                 if (oinc) take_min(d, w, ond, oni);
             }
-            bool shares_endpoint = mv.vert(w, 0) == v0 || mv.vert(w, 0) == v1 || mv.vert(w, 1) == v0 || mv.vert(w, 1) == v1;
+            bool shares_endpoint = (int)q.v0 == v0 || (int)q.v0 == v1 || (int)q.v1 == v0 || (int)q.v1 == v1;
             bool shared_solid = os && (shares_endpoint || (q.flags & CF_LEDGE)) && (d > prior_eps) && (d <= dist_eps);
             if (shared_solid) {
                 if (inc && d < csd) csd = d;
                 if (oinc && d < osd) osd = d;
             }
             bool sgp = (q.flags & CF_GEO) && inc && shares_endpoint && !os && (d > prior_eps) && (fabsf(d - distance) <= (1.0f / 16.0f));
-            if (sgp && (d < gpd || (d == gpd && w < gpi))) { gpd = d; gpi = w; gp_along = q.along; }
+            if (sgp && (d < gpd || (d == gpd && w < gpi))) { gpd = d; gpi = w; gp_along_hi = (q.flags & CF_ALONG_HI) != 0; }
         }
         if (!finitef(cnd)) cni = 0;
         if (!finitef(ond)) oni = 0;
@@ -1210,10 +1295,10 @@ __device__ bool pass_advance(const ColumnCtx &cc, ColumnState &c, const PassColu
             gp_other = gp_from_front ? mv.sec(gpi, 1) : mv.sec(gpi, 0);
             uses_geometric_path = gp_other >= 0;
             if (uses_geometric_path) {
-                int pb_slot = gp_along > 0.5f ? 1 : 0;
+                int pb_slot = gp_along_hi ? 1 : 0;
                 bool ppb_exists = mv.portal_bridge(pb_slot, gpi, wi, &ppb_idx);
                 if (ppb_exists) {
-                    Cand qb = cc.eval(ppb_idx);
+                    Eval qb = cc.eval(ppb_idx);
                     endpoint_portal_bridge = (qb.flags & CF_PROJ) && (qb.flags & CF_LEDGE) && (qb.dist > prior_eps) && (fabsf(qb.dist - gpd) <= tolerance_of(gpd));
                 }
             }
@@ -1249,8 +1334,7 @@ __device__ bool pass_advance(const ColumnCtx &cc, ColumnState &c, const PassColu
     if (starts_po) c.pend_po_vertex = r.sel_vertex;
     bool po = starts_po || ((before.flags & ST_PO) && (r.bits & PB_CONTINUES_PO));
     if (endpoint_only_portal) {
-        Cand cw = cc.eval(wi);
-        c.pend_ep_vertex = mv.vert(wi, cw.along <= 0.5f ? 0 : 1);
+        c.pend_ep_vertex = mv.vert(wi, (r.bits & PB_FINAL_ALONG_HI) ? 1 : 0);
         c.pend_ep_wall = wi;
     }
     if (r.bits & PB_FORWARD_BRIDGE) c.pend_eb_index = r.fb_idx;
@@ -1272,11 +1356,8 @@ __device__ void masked_midtexture(const ColumnCtx &cc, const ColumnState &c, Pix
     for (int k = 0; k < cc.count; ++k) {
         Cand q = cc.cand(k);
         int w = q.wall;
-        if (!(q.flags & CF_PROJ) || mv.one_sided(w)) continue;
-        const float4 wl = *reinterpret_cast<const float4 *>(m->walls + 4 * w);
-        float vx = wl.z - wl.x, vy = wl.w - wl.y;
-        float fx = L.x - wl.x, fy = L.y - wl.y;
-        int sidew = ((vx * fy - vy * fx) < 0) ? 0 : 1;
+        if (!(q.flags & CF_PROJ) || (q.s1 < 0)) continue;
+        int sidew = (q.flags & CF_FF) ? 0 : 1;   // engine.py:13436-13444, the float32 facing test
         if (m->side_tex[(w * 2 + sidew) * 3] < 0) continue;
         if (q.dist < md || (q.dist == md && w < mw)) { md = q.dist; mw = w; mside = sidew; cand_flags = q.flags; }
     }
@@ -1353,14 +1434,18 @@ __global__ void __launch_bounds__(SW) wall_columns_kernel(DeviceMap dm, int lane
     const int local = blockIdx.x;
     if (local >= lane_count) return;
     __shared__ LaneCtx lane_ctx;
+    __shared__ unsigned char colormap_lds[32 * 256];   // shade rows 0..31 are the only ones indexed
     if (threadIdx.x == 0) lane_ctx = sc.ctx[local];
+    for (int k = threadIdx.x; k < 32 * 256 / 4; k += SW) reinterpret_cast<unsigned int *>(colormap_lds)[k] = reinterpret_cast<const unsigned int *>(m->colormap)[k];
     __syncthreads();
     const int x = threadIdx.x;
+    bool window_dirty = false;
     ColumnCtx cc;
     cc.m = m; cc.mv.m = m; cc.c = &lane_ctx;
     cc.recs = sc.rec + (size_t)local * m->wall_count;
     cc.list = sc.cand + (size_t)local * CAND_MAX * SW;
     cc.count = sc.cand_count[(size_t)local * SW + x];
+    if (cc.count > CAND_MAX) cc.count = CAND_MAX;
     cc.x = x;
     ray_direction(lane_ctx, x, &cc.rx, &cc.ry);
     PixelBuffers pb;
@@ -1406,7 +1491,7 @@ __global__ void __launch_bounds__(SW) wall_columns_kernel(DeviceMap dm, int lane
         bool group_valid[3];
         for (int t = 0; t < 3; ++t) group_valid[t] = same_group && all_tier[t] && (common_top[t] < common_bottom[t]);
         if (!done) {
-            pass_paint(cc, st, pc, pb, group_valid, common_bottom, first_group_visibility);
+            pass_paint(cc, st, pc, pb, group_valid, common_bottom, first_group_visibility, colormap_lds, window_dirty);
             bool changed = pass_advance(cc, st, pc, pb, sb);
             // A pass that found nothing and changed nothing repeats identically for ever.
             if (!(pc.bits & PB_VALID) && !changed) done = true;
@@ -1698,7 +1783,6 @@ int launch_chunk(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_out 
     hipLaunchKernelGGL(lane_setup_kernel, dim3((count + 63) / 64), dim3(64), 0, stream, r->dm, *lanes, base, count, r->sc);
     hipLaunchKernelGGL(wall_setup_kernel, dim3((m.wall_count + 127) / 128, count), dim3(128), 0, stream, r->dm, count, r->sc);
     mark();
-    hipLaunchKernelGGL(column_lists_kernel, dim3(count), dim3(SW), 0, stream, r->dm, count, r->sc);
     mark();
     hipLaunchKernelGGL(flat_select_kernel, dim3((VH * SW + 255) / 256, count), dim3(256), 0, stream, r->dm, *lanes, base, count, r->sc);
     mark();
@@ -1741,6 +1825,7 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     if (h->wall_count <= 0 || h->sector_count <= 0) return fail(GD_E_ARG, "empty map");
     if (h->wall_count >= 65535) return fail(GD_E_ARG, "at most 65534 linedefs");
     if (h->sector_count >= 16383) return fail(GD_E_ARG, "at most 16382 sectors");
+    if (h->vertex_count >= 65536) return fail(GD_E_ARG, "at most 65535 distinct vertices");
     gd_renderer *r = new (std::nothrow) gd_renderer();
     if (!r) return fail(GD_E_ARG, "out of host memory");
     r->events_ready = false;
@@ -1753,6 +1838,7 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     UP(walls, W * 4); UP(walls_fixed, W * 4); UP(wall_sectors, W * 2); UP(wall_vertex, W * 2);
     UP(side_tex, W * 6); UP(side_off, W * 4); UP(wall_len, W);
     UP(endpoint_neighbors, W * K); UP(endpoint_neighbor_starts, W * K); UP(endpoint_neighbor_ends, W * K);
+    UP(direct_neighbor_table, W * 4);
     UP(solid_bridge_start_ofs, W + 1); UP(solid_bridge_start_idx, h->solid_bridge_start_ofs[W]);
     UP(solid_bridge_end_ofs, W + 1); UP(solid_bridge_end_idx, h->solid_bridge_end_ofs[W]);
     UP(vertex_wall_ofs, V + 1); UP(vertex_wall_idx, h->vertex_wall_ofs[V]);
@@ -1778,12 +1864,11 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     if (rc == GD_OK) rc = upload(r, tangent.data(), tangent.size(), &r->dm.fine_tangent);
     if (rc == GD_OK) rc = upload(r, cosine_correction, (size_t)SW, &r->dm.cosine_correction);
     // Working memory for one chunk of lanes; larger batches are rendered chunk by chunk.
-    const int chunk = max_lanes < 1024 ? max_lanes : 1024;
+    const int chunk = max_lanes < 4096 ? max_lanes : 4096;
     r->chunk_lanes = chunk;
     const size_t L = chunk, PX = (size_t)VH * SW;
     if (rc == GD_OK) rc = scratch_alloc(r, L, &r->sc.ctx);
     if (rc == GD_OK) rc = scratch_alloc(r, L * W, &r->sc.rec);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * W, &r->sc.visible);
     if (rc == GD_OK) rc = scratch_alloc(r, L * CAND_MAX * SW, &r->sc.cand);
     if (rc == GD_OK) rc = scratch_alloc(r, L * SW, &r->sc.cand_count);
     if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &r->sc.flat_sector);

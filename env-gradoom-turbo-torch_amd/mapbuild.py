@@ -92,6 +92,17 @@ def build_map_tables(smap) -> dict[str, np.ndarray | int]:
             neighbor_ends[w, k] = shares(w, 1, n)
     direct = bool(np.all(neighbor_starts.sum(axis=1) <= 1) and np.all(neighbor_ends.sum(axis=1) <= 1))
 
+    # engine.py:1558-1575: argmax over the start / end flags picks the first set slot (0 when none)
+    direct_table = np.zeros((wall_count, 4), dtype=np.int32)
+    for w in range(wall_count):
+        start_slot = int(np.argmax(neighbor_starts[w]))
+        end_slot = int(np.argmax(neighbor_ends[w]))
+        direct_table[w, 0] = endpoint_neighbors[w, start_slot]
+        direct_table[w, 1] = endpoint_neighbors[w, end_slot]
+        direct_table[w, 2] = (
+            start_slot | (end_slot << 8) | (int(neighbor_starts[w].any()) << 16) | (int(neighbor_ends[w].any()) << 17)
+        )
+
     # One-hop solid bridges (engine.py:787-830): bridge[w] = { k : exists j one-sided,
     # sharing w's start (resp. end), with sectors[j,0] in sectors[w], and k one-sided,
     # k != j, sharing any endpoint with j, sectors[k,0] == sectors[j,0] }.
@@ -179,6 +190,7 @@ def build_map_tables(smap) -> dict[str, np.ndarray | int]:
         endpoint_neighbors=endpoint_neighbors,
         endpoint_neighbor_starts=neighbor_starts,
         endpoint_neighbor_ends=neighbor_ends,
+        direct_neighbor_table=direct_table,
         solid_bridge_start_ofs=solid_bridge_start_ofs,
         solid_bridge_start_idx=solid_bridge_start_idx,
         solid_bridge_end_ofs=solid_bridge_end_ofs,

@@ -91,6 +91,7 @@ class HipRenderer:
         self._lib = _lib.library()
         self.tables = mapbuild.build_map_tables(smap) if tables is None else tables
         self.max_lanes = int(max_lanes)
+        self.chunk_lanes = min(self.max_lanes, 4096)  # lanes per kernel launch (library working-memory chunk)
         if cosine_correction is None:
             cosine_correction = hostmath.cosine_correction("cpu").numpy()
         self._cosine = np.ascontiguousarray(cosine_correction, dtype=np.float32)

@@ -71,6 +71,8 @@ typedef struct gd_map_desc {
     const int32_t *endpoint_neighbors;      /* [W,K] (engine.py:833-849), self where unused */
     const uint8_t *endpoint_neighbor_starts;/* [W,K] */
     const uint8_t *endpoint_neighbor_ends;  /* [W,K] */
+    const int32_t *direct_neighbor_table;   /* [W,4] engine.py:1558-1575 packed: start neighbour, end neighbour,
+                                               start slot | end slot<<8 | has start<<16 | has end<<17, 0 */
     const int32_t *solid_bridge_start_ofs;  /* [W+1] CSR of engine.py:802-830 */
     const int32_t *solid_bridge_start_idx;
     const int32_t *solid_bridge_end_ofs;    /* [W+1] */
