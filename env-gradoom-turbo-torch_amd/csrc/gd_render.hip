@@ -113,11 +113,12 @@ struct Scratch {    // per-chunk working memory, sized at create
     int *status;           // [1] sticky overflow flags
 };
 
-#define META_FILLED 0x80000000u
-#define META_FLOOR 0x40000000u
+#define META_FILLED 0x80000000u   // an opaque wall tier owns the pixel
+#define META_FLOOR 0x40000000u    // the owning plane is a floor
+#define META_MASKED 0x20000000u   // a masked mid-texture was drawn over the pixel
 #define META_SECTOR_SHIFT 16
-#define META_SECTOR_MASK 0x3FFFu
-#define META_WALL_MASK 0xFFFFu
+#define META_SECTOR_MASK 0x1FFFu  // plane sector + 1
+#define META_WALL_MASK 0xFFFFu    // sprite-clip linedef + 1
 
 #define STATUS_CAND_OVERFLOW 1
 
@@ -126,14 +127,30 @@ __device__ __forceinline__ i64 shl64(i64 a, int s) { return (i64)((u64)a << s); 
 // C truncating division (engine.py:3115-3118).  gfx950 has no 64-bit integer divider; when both
 // magnitudes are below 2^52 the quotient estimated in float64 is within one of the true quotient
 // and one remainder check makes it exact.  Larger operands take the compiler's long division.
+// The rare large-operand case is a compact shift-subtract loop rather than the compiler's
+// unrolled long division, which would be replicated at every call site and push the kernels
+// far past the instruction cache.
+__device__ __forceinline__ u64 udiv_long(u64 n, u64 d) {
+    u64 q = 0, r = 0;
+#pragma unroll 1
+    for (int i = 63; i >= 0; --i) {
+        r = (r << 1) | ((n >> i) & 1);
+        if (r >= d) { r -= d; q |= 1ULL << i; }
+    }
+    return q;
+}
 __device__ __forceinline__ i64 tdiv(i64 a, i64 b) {
     u64 ua = a < 0 ? (u64)0 - (u64)a : (u64)a;
     u64 ub = b < 0 ? (u64)0 - (u64)b : (u64)b;
-    if (((ua | ub) >> 52) != 0 || ub == 0) return b == 0 ? 0 : a / b;
-    u64 uq = (u64)((double)ua / (double)ub);
-    u64 prod = uq * ub;
-    if (prod > ua) --uq;
-    else if (ua - prod >= ub) ++uq;
+    u64 uq;
+    if (((ua | ub) >> 52) != 0 || ub == 0) {
+        uq = ub == 0 ? 0 : udiv_long(ua, ub);
+    } else {
+        uq = (u64)((double)ua / (double)ub);
+        u64 prod = uq * ub;
+        if (prod > ua) --uq;
+        else if (ua - prod >= ub) ++uq;
+    }
     return ((a < 0) != (b < 0)) ? -(i64)uq : (i64)uq;
 }
 __device__ __forceinline__ i64 clampi(i64 v, i64 lo, i64 hi) { return v < lo ? lo : (v > hi ? hi : v); }
@@ -501,10 +518,43 @@ __global__ void flat_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
     sc.flat_flags[i] = best_sector < 0 ? 1 : 0;
 }
 
+// Small per-sector / per-texture tables staged in LDS by the kernels whose inner loops chase
+// them (a dependent global gather costs ~500 cycles, an LDS read ~60).  Sectors or textures
+// beyond the staged count fall back to the global arrays.
+#define LDS_SECTORS 512
+#define LDS_TEXTURES 256
+struct Tables {
+    const gd_map_desc *m;
+    const float4 *sector;          // floor, ceiling, light, bits(floor_tex | ceil_tex << 16)
+    const unsigned char *tex_bits; // log2 width | log2 height << 4
+    int sector_cached, tex_cached;
+    __device__ __forceinline__ float floor_h(int s) const { return s < sector_cached ? sector[s].x : m->sector_heights[2 * s]; }
+    __device__ __forceinline__ float ceil_h(int s) const { return s < sector_cached ? sector[s].y : m->sector_heights[2 * s + 1]; }
+    __device__ __forceinline__ float light(int s) const { return s < sector_cached ? sector[s].z : m->sector_lights[s]; }
+    __device__ __forceinline__ int floor_tex(int s) const { return s < sector_cached ? (int)(__float_as_uint(sector[s].w) & 0xFFFFu) : m->sector_floor_tex[s]; }
+    __device__ __forceinline__ int ceil_tex(int s) const { return s < sector_cached ? (int)(__float_as_uint(sector[s].w) >> 16) : m->sector_ceil_tex[s]; }
+    __device__ __forceinline__ int width_bits(int t) const { return t < tex_cached ? (tex_bits[t] & 15) : ilog2(m->tex_w[t]); }
+    __device__ __forceinline__ int height_bits(int t) const { return t < tex_cached ? (tex_bits[t] >> 4) : ilog2(m->tex_h[t]); }
+};
+
+// Cooperative fill of the LDS tables by the whole block (call before a __syncthreads()).
+__device__ __forceinline__ void stage_tables(const gd_map_desc *m, float4 *sector_lds, unsigned char *tex_lds, Tables &tb) {
+    int sectors = m->sector_count < LDS_SECTORS ? m->sector_count : LDS_SECTORS;
+    int textures = m->texture_count < LDS_TEXTURES ? m->texture_count : LDS_TEXTURES;
+    for (int s = threadIdx.x; s < sectors; s += blockDim.x) {
+        float4 v;
+        v.x = m->sector_heights[2 * s]; v.y = m->sector_heights[2 * s + 1]; v.z = m->sector_lights[s];
+        v.w = __uint_as_float(((unsigned)m->sector_floor_tex[s] & 0xFFFFu) | ((unsigned)m->sector_ceil_tex[s] << 16));
+        sector_lds[s] = v;
+    }
+    for (int t = threadIdx.x; t < textures; t += blockDim.x) tex_lds[t] = (unsigned char)(ilog2(m->tex_w[t]) | (ilog2(m->tex_h[t]) << 4));
+    tb.m = m; tb.sector = sector_lds; tb.tex_bits = tex_lds; tb.sector_cached = sectors; tb.tex_cached = textures;
+}
+
 // engine.py:10879-10954
-__device__ void flat_texture_coordinates(const gd_map_desc *m, const LaneCtx &c, int texture_id, float plane_height, int px, int py, i64 *u, i64 *v) {
-    int width_bits = ilog2(m->tex_w[texture_id]);
-    int height_bits = ilog2(m->tex_h[texture_id]);
+__device__ __forceinline__ void flat_texture_coordinates(const Tables &tb, const LaneCtx &c, int texture_id, float plane_height, int px, int py, i64 *u, i64 *v) {
+    int width_bits = tb.width_bits(texture_id);
+    int height_bits = tb.height_bits(texture_id);
     i64 xscale = shl64(1, 32 - width_bits), yscale = shl64(1, 32 - height_bits);
     i64 xstep_scale = tdiv(mul64(xscale, c.vsin), FOCAL_X_FIXED);
     i64 ystep_scale = tdiv(mul64(yscale, c.vcos), FOCAL_X_FIXED);
@@ -529,7 +579,7 @@ __device__ void flat_texture_coordinates(const gd_map_desc *m, const LaneCtx &c,
 }
 
 // engine.py:10588-10616
-__device__ unsigned char plane_colormap(const gd_map_desc *m, const LaneCtx &c, unsigned char index, float light, float plane_height, int py) {
+__device__ __forceinline__ unsigned char plane_colormap(const unsigned char *colormap, const LaneCtx &c, unsigned char index, float light, float plane_height, int py) {
     i64 plane_height_fixed = round_to_i64(plane_height * 65536.0f);
     i64 glob = min64(tdiv(FLOOR_VISIBILITY_FIXED << 16, max64(plane_height_fixed, 1)), (1LL << 31) - 1);
     i64 row = c.center_fixed - (i64)py * FIXED_UNIT;
@@ -537,17 +587,18 @@ __device__ unsigned char plane_colormap(const gd_map_desc *m, const LaneCtx &c, 
     i64 visibility = min64(mul64(glob, row) >> 16, 24 * FIXED_UNIT);
     i64 plane_shade = 64 * FIXED_UNIT - ((i64)light + 12) * (FIXED_UNIT / 4);
     i64 shade = clampi((plane_shade - visibility) >> 16, 0, 31);
-    return m->colormap[shade * 256 + index];
+    return colormap[shade * 256 + index];
 }
 
-__device__ unsigned char flat_pixel(const gd_map_desc *m, const LaneCtx &c, int sector, bool is_floor, int px, int py) {
-    float plane_height = is_floor ? (c.view_z - m->sector_heights[2 * sector]) : (m->sector_heights[2 * sector + 1] - c.view_z);
-    int texture = is_floor ? m->sector_floor_tex[sector] : m->sector_ceil_tex[sector];
+__device__ __forceinline__ unsigned char flat_pixel(const Tables &tb, const unsigned char *colormap, const LaneCtx &c, int sector, bool is_floor, int px, int py) {
+    const gd_map_desc *m = tb.m;
+    float plane_height = is_floor ? (c.view_z - tb.floor_h(sector)) : (tb.ceil_h(sector) - c.view_z);
+    int texture = is_floor ? tb.floor_tex(sector) : tb.ceil_tex(sector);
     i64 u, v;
-    flat_texture_coordinates(m, c, texture, plane_height, px, py, &u, &v);
+    flat_texture_coordinates(tb, c, texture, plane_height, px, py, &u, &v);
     unsigned char index = m->tex_atlas[((size_t)texture * m->tex_max_h + v) * m->tex_max_w + u];
-    float light = m->sector_lights[sector] + (float)(c.flash_light * 16);
-    return plane_colormap(m, c, index, light, plane_height, py);
+    float light = tb.light(sector) + (float)(c.flash_light * 16);
+    return plane_colormap(colormap, c, index, light, plane_height, py);
 }
 
 // Visplane continuity repair and shading for one lane (engine.py:11026-11171).
@@ -624,13 +675,7 @@ __global__ void __launch_bounds__(SW) flat_finish_kernel(DeviceMap dm, int lane_
             }
         }
     }
-    __syncthreads();
-    // --- shade every view pixel with its selected sector (engine.py:11145-11163)
-    for (int y = 0; y < VH; ++y) {
-        size_t i = (size_t)y * SW + x;
-        bool is_floor = ((float)y - center) > 0;
-        frame[i] = flat_pixel(m, c, sector[i], is_floor, x, y);
-    }
+    // shading happens once per pixel in plane_shade_kernel, after the walls have claimed theirs
     for (int y = VH; y < GD_SCREEN_HEIGHT; ++y) frame[(size_t)y * SW + x] = 0;  // empty status bar
 }
 
@@ -638,6 +683,7 @@ __global__ void __launch_bounds__(SW) flat_finish_kernel(DeviceMap dm, int lane_
 // walls: engine.py:11462-13745
 // ---------------------------------------------------------------------------------------------
 struct ColumnCtx {
+    const Tables *tb;
     const gd_map_desc *m;
     MapView mv;
     const LaneCtx *c;
@@ -694,7 +740,7 @@ __device__ void texture_mapping(const gd_map_desc *m, const WallRec &r, int w, i
 }
 
 // engine.py:12294-12605 (OWallMost) for one column
-__device__ float project(const LaneCtx &c, const WallRec &g, float world_z, int x) {
+__device__ __forceinline__ float project(const LaneCtx &c, const WallRec &g, float world_z, int x) {
     i64 whole_sl = g.sl, whole_sr = g.sr;
     i64 whole_dl = max64(g.dl, 1), whole_dr = max64(g.dr, 1);
     bool has_fragment = (g.sr > g.sl) && (x >= g.sl) && (x < g.sr);
@@ -760,11 +806,13 @@ __device__ __forceinline__ i64 wall_shade(float light, i64 visibility) {
 }
 
 // engine.py:11596-11730 for one (column, linedef)
-__device__ void endpoint_owner(const ColumnCtx &cc, int w, const Eval &cw, int *owner_index, float *owner_distance) {
+__device__ __forceinline__ void endpoint_owner(const ColumnCtx &cc, int w, const Eval &cw, int *owner_index, float *owner_distance) {
     const gd_map_desc *m = cc.m;
     const int K = m->neighbor_slots;
     const bool subpixel = cc.recs[w].flags & WF_SUBPIXEL;
     float tol_w = tolerance_of(cw.dist);
+    // the owner only matters for a linedef that does not own this column itself (engine.py:11716)
+    if (cw.flags & CF_PROJ) { *owner_index = w; *owner_distance = cw.dist; return; }
     bool uses_start = !(cw.flags & CF_ALONG_HI);
     int index; float distance; bool valid;
     if (m->direct_neighbors) {
@@ -801,6 +849,17 @@ __device__ void endpoint_owner(const ColumnCtx &cc, int w, const Eval &cw, int *
     *owner_index = has ? index : w;
     *owner_distance = has ? distance : cw.dist;
 }
+
+#ifdef GD_PROFILE
+__device__ unsigned long long g_profile[16];
+#define PROF_T(var) long long var = wall_clock64()
+#define PROF_ADD(slot, t0, t1) prof_acc[slot] += (t1) - (t0)
+#define PROF_MARK(slot, tprev) do { long long tn_ = wall_clock64(); if (threadIdx.x == 0) atomicAdd(&g_profile[slot], (unsigned long long)(tn_ - tprev)); tprev = tn_; } while (0)
+#else
+#define PROF_T(var)
+#define PROF_ADD(slot, t0, t1)
+#define PROF_MARK(slot, tprev)
+#endif
 
 struct ColumnState {   // engine.py:11561-11580, 11735-11762
     int current_sector;
@@ -861,7 +920,7 @@ __device__ __forceinline__ void take_min(float v, int w, float &best, int &best_
 }
 
 // engine.py:11769-12636: selection of the pass's drawseg for one column
-__device__ void pass_select(const ColumnCtx &cc, const ColumnState &c, bool boundary_has_po, PassColumn &r) {
+__device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnState &c, bool boundary_has_po, PassColumn &r) {
     const gd_map_desc *m = cc.m;
     const MapView &mv = cc.mv;
     const int x = cc.x;
@@ -871,6 +930,9 @@ __device__ void pass_select(const ColumnCtx &cc, const ColumnState &c, bool boun
     const float prev_eps = prev + 1e-3f;
     auto incident = [&](int w) { return mv.sec(w, 0) == cur || mv.sec(w, 1) == cur; };
     auto incident_c = [&](const Cand &q) { return q.s0 == cur || q.s1 == cur; };
+#ifdef GD_PROFILE
+    long long tsub = wall_clock64();
+#endif
     // a. nearest incident linedef beyond previous_distance (engine.py:11769-11780)
     float distance = GD_INF; int wi = 0x7fffffff;
     Eval cwi;
@@ -889,6 +951,7 @@ __device__ void pass_select(const ColumnCtx &cc, const ColumnState &c, bool boun
         cwi.dist = distance; cwi.flags = wi_flags;
     }
     if (!finitef(distance)) { wi = 0; cwi = cc.eval(0); }
+    PROF_MARK(8, tsub);
     // c. selected endpoint (engine.py:11815-11871)
     bool sel_start = !(cwi.flags & CF_ALONG_HI);
     int sel_vertex = mv.vert(wi, sel_start ? 0 : 1);
@@ -896,9 +959,11 @@ __device__ void pass_select(const ColumnCtx &cc, const ColumnState &c, bool boun
     bool continues_po_boundary = (c.flags & ST_PO) && (sel_vertex == c.pend_po_vertex);
     bool continues_ep_boundary = (c.flags & ST_EP) && (sel_vertex == c.pend_ep_vertex);
     int sel_slot = sel_start ? 0 : 1;
-    int fb_idx; bool fb_exists = mv.portal_bridge(sel_slot, wi, c.pend_ep_wall, &fb_idx);
+    // the forward bridge only matters while an endpoint-projected boundary continues
+    int fb_idx = 0;
     bool pend_ep_has_forward_bridge = false;
-    if (continues_ep_boundary && fb_exists) pend_ep_has_forward_bridge = cc.eval(fb_idx).dist > distance + 1e-3f;
+    if (continues_ep_boundary && mv.portal_bridge(sel_slot, wi, c.pend_ep_wall, &fb_idx))
+        pend_ep_has_forward_bridge = cc.eval(fb_idx).dist > distance + 1e-3f;
     bool completes_pending_endpoint_bridge = (c.flags & ST_EB) && (wi == c.pend_eb_index);
     bool sel_is_proj = cwi.flags & CF_PROJ;
     bool sel_excl_right = cc.recs[wi].sr == x;
@@ -929,6 +994,7 @@ __device__ void pass_select(const ColumnCtx &cc, const ColumnState &c, bool boun
     }
     bool has_ps = finitef(psd);
     if (has_ps) { distance = psd; wi = psi; cwi.dist = psd; cwi.flags = psi_flags; }
+    PROF_MARK(9, tsub);
     // e. endpoint owner (engine.py:11960-12001)
     int eo_idx; float eo_dist;
     endpoint_owner(cc, wi, cwi, &eo_idx, &eo_dist);
@@ -984,6 +1050,7 @@ __device__ void pass_select(const ColumnCtx &cc, const ColumnState &c, bool boun
     if (replace_np) { distance = npd; wi = npi; cwi.dist = npd; cwi.flags = npi_flags; }
     bool final_proj = cwi.flags & CF_PROJ, final_geo = cwi.flags & CF_GEO;
     bool completes_poab = (c.flags & ST_EP) && final_proj && !final_geo && mv.opposing(pe_wall, wi);
+    PROF_MARK(10, tsub);
     // g. validity (engine.py:12197-12239)
     bool valid = finitef(distance);
     bool excl_only = !so_is_proj && so_excl_right && !replace_np && (so_span <= 2) && !boundary_has_po;
@@ -1009,20 +1076,28 @@ __device__ void pass_select(const ColumnCtx &cc, const ColumnState &c, bool boun
     r.distance = distance;
     const WallRec &wr = cc.recs[wi];
     r.visibility = wall_visibility(wr, side, x);
-    r.view_floor = m->sector_heights[2 * render_current]; r.view_ceiling = m->sector_heights[2 * render_current + 1];
-    r.other_floor = m->sector_heights[2 * safe_other]; r.other_ceiling = m->sector_heights[2 * safe_other + 1];
+    const Tables &tb = *cc.tb;
+    r.view_floor = tb.floor_h(render_current); r.view_ceiling = tb.ceil_h(render_current);
+    r.other_floor = tb.floor_h(safe_other); r.other_ceiling = tb.ceil_h(safe_other);
     for (int t = 0; t < 3; ++t) r.side_tex[t] = m->side_tex[(wi * 2 + side) * 3 + t];
+    PROF_MARK(11, tsub);
     // j. projection and clipping (engine.py:12607-12620)
-    float one_top = project(*cc.c, wr, r.view_ceiling, x), one_bottom = project(*cc.c, wr, r.view_floor, x);
-    float lower_top = project(*cc.c, wr, r.other_floor, x), upper_bottom = project(*cc.c, wr, r.other_ceiling, x);
+    float one_top = 0, one_bottom = 0, lower_top = 0, upper_bottom = 0;
+#pragma unroll 1
+    for (int k = 0; k < 4; ++k) {   // one copy of the projection code, four heights
+        float z = k == 0 ? r.view_ceiling : (k == 1 ? r.view_floor : (k == 2 ? r.other_floor : r.other_ceiling));
+        float v = project(*cc.c, wr, z, x);
+        if (k == 0) one_top = v; else if (k == 1) one_bottom = v; else if (k == 2) lower_top = v; else upper_bottom = v;
+    }
     r.clipped_top = fmaxf(one_top, c.ceiling_clip);
     r.clipped_bottom = fminf(one_bottom, c.floor_clip);
     r.clipped_upper_bottom = fmaxf(fminf(upper_bottom, c.floor_clip), r.clipped_top);
     r.clipped_lower_top = fminf(fmaxf(lower_top, c.ceiling_clip), r.clipped_bottom);
+    PROF_MARK(12, tsub);
     // k. plane marks (engine.py:12621-12636)
-    bool light_differs = m->sector_lights[render_current] != m->sector_lights[safe_other];
-    bool mark_ceiling = one_sided || (r.view_ceiling != r.other_ceiling) || (m->sector_ceil_tex[render_current] != m->sector_ceil_tex[safe_other]) || light_differs;
-    bool mark_floor = one_sided || (r.view_floor != r.other_floor) || (m->sector_floor_tex[render_current] != m->sector_floor_tex[safe_other]) || light_differs;
+    bool light_differs = tb.light(render_current) != tb.light(safe_other);
+    bool mark_ceiling = one_sided || (r.view_ceiling != r.other_ceiling) || (tb.ceil_tex(render_current) != tb.ceil_tex(safe_other)) || light_differs;
+    bool mark_floor = one_sided || (r.view_floor != r.other_floor) || (tb.floor_tex(render_current) != tb.floor_tex(safe_other)) || light_differs;
     bool tier0 = one_sided && raster_valid && (r.side_tex[0] >= 0) && (r.clipped_top < r.clipped_bottom);
     bool tier1 = !one_sided && raster_valid && (r.view_floor < r.other_floor) && (r.side_tex[1] >= 0) && (r.clipped_lower_top < r.clipped_bottom);
     bool tier2 = !one_sided && raster_valid && (r.view_ceiling > r.other_ceiling) && (r.side_tex[2] >= 0) && (r.clipped_top < r.clipped_upper_bottom);
@@ -1049,7 +1124,7 @@ struct SilhouetteBounds {
     float bot_depth, top_depth;
 };
 
-__device__ void apply_silhouette(PixelBuffers &pb, SilhouetteBounds &sb, int x, bool bottom, bool top, float floor_clip, float ceiling_clip, float distance, int wall) {
+__device__ __forceinline__ void apply_silhouette(PixelBuffers &pb, SilhouetteBounds &sb, int x, bool bottom, bool top, float floor_clip, float ceiling_clip, float distance, int wall) {
     if (bottom) {
         int first = floor_clip <= 0.0f ? 0 : (floor_clip >= (float)VH ? VH : (int)floor_clip);   // clips hold integers
         int last = (distance >= sb.bot_depth) ? (sb.bot_row < VH ? sb.bot_row : VH) : VH;
@@ -1078,7 +1153,7 @@ __device__ void apply_silhouette(PixelBuffers &pb, SilhouetteBounds &sb, int x, 
 // rows that its own clip update then removes from the window, so the window stays untouched
 // until a one-sided drawseg (which leaves the clips alone) has painted; until then painting
 // needs no reads and visits only the rows it writes.
-__device__ void pass_paint(const ColumnCtx &cc, const ColumnState &c, const PassColumn &r, PixelBuffers &pb,
+__device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnState &c, const PassColumn &r, PixelBuffers &pb,
                            const bool group_valid[3], const float group_bottom[3], i64 first_group_visibility,
                            const unsigned char *colormap, bool &window_dirty) {
     if (!(r.bits & PB_RASTER)) return;
@@ -1100,7 +1175,8 @@ __device__ void pass_paint(const ColumnCtx &cc, const ColumnState &c, const Pass
     const float4 wl = *reinterpret_cast<const float4 *>(m->walls + 4 * wi);
     bool horizontal = fabsf(wl.w - wl.y) < 1e-6f, vertical = fabsf(wl.z - wl.x) < 1e-6f;
     float fake_contrast = vertical ? 16.0f : (horizontal ? -16.0f : 0.0f);
-    float light = (m->sector_lights[r.render_current] + (float)(L.flash_light * 16)) + fake_contrast;
+    const Tables &tb = *cc.tb;
+    float light = (tb.light(r.render_current) + (float)(L.flash_light * 16)) + fake_contrast;
     const i64 shade_own = wall_shade(light, r.visibility);
     const i64 shade_group = wall_shade(light, first_group_visibility);
     // every span of this pass lies inside the open window [ceiling_clip, floor_clip)
@@ -1134,10 +1210,9 @@ __device__ void pass_paint(const ColumnCtx &cc, const ColumnState &c, const Pass
             bool bottom_tail = (one_span && group_valid[0] && py >= group_bottom[0]) ||
                                (lower_span && group_valid[1] && py >= group_bottom[1]) ||
                                (upper_span && group_valid[2] && py >= group_bottom[2]);
-            int tw = m->tex_w[texture_id], th = m->tex_h[texture_id];
-            i64 tu = u_base & (i64)(tw - 1);
+            i64 tu = u_base & (i64)((1 << tb.width_bits(texture_id)) - 1);
             float origin_z = one_span ? r.view_ceiling : (lower_span ? r.other_floor : r.other_ceiling);
-            int height_bits = ilog2(th);
+            int height_bits = tb.height_bits(texture_id);
             i64 vertical_step = mul64(swall, shl64(1, 14 - height_bits));
             i64 screen_delta = (i64)y * FIXED_UNIT - L.center_fixed + FIXED_UNIT;
             i64 texture_mid = round_to_i64((origin_z - L.view_z) * 65536.0f + toff[1] * 65536.0f);
@@ -1172,10 +1247,9 @@ __device__ void pass_paint(const ColumnCtx &cc, const ColumnState &c, const Pass
                 bool bottom_tail = (one_span && group_valid[0] && py >= group_bottom[0]) ||
                                    (lower_span && group_valid[1] && py >= group_bottom[1]) ||
                                    (upper_span && group_valid[2] && py >= group_bottom[2]);
-                int tw = m->tex_w[texture_id], th = m->tex_h[texture_id];
-                i64 tu = u_base & (i64)(tw - 1);   // floor-mod by a power of two
+                i64 tu = u_base & (i64)((1 << tb.width_bits(texture_id)) - 1);   // floor-mod by a power of two
                 float origin_z = one_span ? r.view_ceiling : (lower_span ? r.other_floor : r.other_ceiling);
-                int height_bits = ilog2(th);
+                int height_bits = tb.height_bits(texture_id);
                 i64 vertical_step = mul64(swall, shl64(1, 14 - height_bits));
                 i64 screen_delta = (i64)y * FIXED_UNIT - L.center_fixed + FIXED_UNIT;
                 i64 texture_mid = round_to_i64((origin_z - L.view_z) * 65536.0f + toff[1] * 65536.0f);
@@ -1193,7 +1267,7 @@ __device__ void pass_paint(const ColumnCtx &cc, const ColumnState &c, const Pass
 }
 
 // engine.py:12885-13371
-__device__ bool pass_advance(const ColumnCtx &cc, ColumnState &c, const PassColumn &r, PixelBuffers &pb, SilhouetteBounds &sb) {
+__device__ __forceinline__ bool pass_advance(const ColumnCtx &cc, ColumnState &c, const PassColumn &r, PixelBuffers &pb, SilhouetteBounds &sb) {
     const gd_map_desc *m = cc.m;
     const MapView &mv = cc.mv;
     const LaneCtx &L = *cc.c;
@@ -1226,20 +1300,26 @@ __device__ bool pass_advance(const ColumnCtx &cc, ColumnState &c, const PassColu
         int path = r.ps_path_index;
         const WallRec &pr = cc.recs[path];
         int path_safe_other = r.ps_other < 0 ? 0 : r.ps_other;
-        float pof = m->sector_heights[2 * path_safe_other], poc = m->sector_heights[2 * path_safe_other + 1];
+        const Tables &tb = *cc.tb;
+        float pof = tb.floor_h(path_safe_other), poc = tb.ceil_h(path_safe_other);
         int pside = (r.bits & PB_PS_FROM_FRONT) ? 0 : 1;
         const int *ptex = m->side_tex + (path * 2 + pside) * 3;
-        float path_top = project(L, pr, r.view_ceiling, x), path_bottom = project(L, pr, r.view_floor, x);
-        float path_lower_top = project(L, pr, pof, x), path_upper_bottom = project(L, pr, poc, x);
+        float path_top = 0, path_bottom = 0, path_lower_top = 0, path_upper_bottom = 0;
+#pragma unroll 1
+        for (int k = 0; k < 4; ++k) {
+            float z = k == 0 ? r.view_ceiling : (k == 1 ? r.view_floor : (k == 2 ? pof : poc));
+            float v = project(L, pr, z, x);
+            if (k == 0) path_top = v; else if (k == 1) path_bottom = v; else if (k == 2) path_lower_top = v; else path_upper_bottom = v;
+        }
         float pct = fmaxf(path_top, c.ceiling_clip);
         float pcb = fminf(path_bottom, c.floor_clip);
         float pcub = fmaxf(fminf(path_upper_bottom, c.floor_clip), pct);
         float pclt = fminf(fmaxf(path_lower_top, c.ceiling_clip), pcb);
-        bool light_differs = m->sector_lights[r.render_current] != m->sector_lights[path_safe_other];
+        bool light_differs = tb.light(r.render_current) != tb.light(path_safe_other);
         bool p_draws_upper = (r.view_ceiling > poc) && (ptex[2] >= 0);
-        bool p_marks_ceiling = (r.view_ceiling != poc) || (m->sector_ceil_tex[r.render_current] != m->sector_ceil_tex[path_safe_other]) || light_differs;
+        bool p_marks_ceiling = (r.view_ceiling != poc) || (tb.ceil_tex(r.render_current) != tb.ceil_tex(path_safe_other)) || light_differs;
         bool p_draws_lower = (r.view_floor < pof) && (ptex[1] >= 0);
-        bool p_marks_floor = (r.view_floor != pof) || (m->sector_floor_tex[r.render_current] != m->sector_floor_tex[path_safe_other]) || light_differs;
+        bool p_marks_floor = (r.view_floor != pof) || (tb.floor_tex(r.render_current) != tb.floor_tex(path_safe_other)) || light_differs;
         float new_ceiling = c.ceiling_clip, new_floor = c.floor_clip;
         if (p_draws_upper || p_marks_ceiling) new_ceiling = p_draws_upper ? pcub : pct;
         if (p_draws_lower || p_marks_floor) new_floor = p_draws_lower ? pclt : pcb;
@@ -1347,7 +1427,7 @@ __device__ bool pass_advance(const ColumnCtx &cc, ColumnState &c, const PassColu
 }
 
 // engine.py:13424-13744 for one column
-__device__ void masked_midtexture(const ColumnCtx &cc, const ColumnState &c, PixelBuffers &pb) {
+__device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const ColumnState &c, PixelBuffers &pb) {
     const gd_map_desc *m = cc.m;
     const MapView &mv = cc.mv;
     const LaneCtx &L = *cc.c;
@@ -1370,10 +1450,15 @@ __device__ void masked_midtexture(const ColumnCtx &cc, const ColumnState &c, Pix
     const WallRec &wr = cc.recs[mw];
     int front_sector = mv.sec(mw, 0), back_sector = mv.sec(mw, 1) < 0 ? 0 : mv.sec(mw, 1);
     int light_sector = mside == 0 ? front_sector : back_sector;
-    float world_top = fminf(m->sector_heights[2 * front_sector + 1], m->sector_heights[2 * back_sector + 1]);
-    int tw = m->tex_w[texture_id], th = m->tex_h[texture_id];
-    float owall_top = project(L, wr, world_top, x);
-    float owall_bottom = project(L, wr, world_top - (float)th, x);
+    const Tables &tb = *cc.tb;
+    float world_top = fminf(tb.ceil_h(front_sector), tb.ceil_h(back_sector));
+    int tw = 1 << tb.width_bits(texture_id), th = 1 << tb.height_bits(texture_id);
+    float owall_top = 0, owall_bottom = 0;
+#pragma unroll 1
+    for (int k = 0; k < 2; ++k) {
+        float v = project(L, wr, k == 0 ? world_top : world_top - (float)th, x);
+        if (k == 0) owall_top = v; else owall_bottom = v;
+    }
     float mceil = fmaxf(owall_top, has_saved ? c.masked_ceiling_clip : 0.0f);
     float mfloor = fminf(owall_bottom, has_saved ? c.masked_floor_clip : (float)VH);
     const float *toff = m->side_off + (mw * 2 + mside) * 2;
@@ -1391,9 +1476,13 @@ __device__ void masked_midtexture(const ColumnCtx &cc, const ColumnState &c, Pix
     i64 center_fixed = L.center_fixed;
     i64 texture_mid = round_to_i64((world_top - L.view_z) * 65536.0f + toff[1] * 65536.0f);
     int safe_left = (int)clampi(msl, 0, SW - 1), safe_last = (int)clampi(msr - 1, 0, SW - 1);
-    i64 dummy_h, start_swall, end_swall;
-    texture_mapping(m, wr, mw, safe_left, &dummy_h, &start_swall);
-    texture_mapping(m, wr, mw, safe_last, &dummy_h, &end_swall);
+    i64 dummy_h, start_swall = 0, end_swall = 0;
+#pragma unroll 1
+    for (int k = 0; k < 2; ++k) {
+        i64 sw;
+        texture_mapping(m, wr, mw, k == 0 ? safe_left : safe_last, &dummy_h, &sw);
+        if (k == 0) start_swall = sw; else end_swall = sw;
+    }
     auto iscale_of = [](i64 swall) {
         i64 s = mul64(swall, FIXED_UNIT) >> 18;
         if (s >= 0 && s < 3) return (i64)3;
@@ -1417,7 +1506,7 @@ __device__ void masked_midtexture(const ColumnCtx &cc, const ColumnState &c, Pix
     const float4 wl = *reinterpret_cast<const float4 *>(m->walls + 4 * mw);
     bool horizontal = fabsf(wl.w - wl.y) < 1e-6f, vertical = fabsf(wl.z - wl.x) < 1e-6f;
     float contrast = vertical ? 16.0f : (horizontal ? -16.0f : 0.0f);
-    float light = (m->sector_lights[light_sector] + (float)(L.flash_light * 16)) + contrast;
+    float light = (tb.light(light_sector) + (float)(L.flash_light * 16)) + contrast;
     i64 shade = wall_shade(light, wall_visibility(wr, mside, x));
     int y0 = (int)clampi(clipped_top, 0, VH), y1 = (int)clampi(clipped_bottom, 0, VH);
     for (int y = y0; y < y1; ++y) {
@@ -1426,22 +1515,29 @@ __device__ void masked_midtexture(const ColumnCtx &cc, const ColumnState &c, Pix
         i64 mv_ = (fraction & UINT32_MASK) >> (32 - height_bits);
         unsigned char texel = m->tex_atlas[((size_t)texture_id * m->tex_max_h + mv_) * m->tex_max_w + mu];
         pb.frame[(size_t)y * SW + x] = m->colormap[shade * 256 + texel];
+        pb.meta[(size_t)y * SW + x] |= META_MASKED;
     }
 }
 
-__global__ void __launch_bounds__(SW) wall_columns_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
+// One wavefront per (lane, 64-column strip): strips of one lane share nothing but read-only
+// tables, so each is its own work-group and leaves the CU as soon as its own columns finish.
+__global__ void __launch_bounds__(64) wall_columns_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
     const gd_map_desc *m = &dm.d;
-    const int local = blockIdx.x;
+    const int local = blockIdx.y;
     if (local >= lane_count) return;
     __shared__ LaneCtx lane_ctx;
     __shared__ unsigned char colormap_lds[32 * 256];   // shade rows 0..31 are the only ones indexed
+    __shared__ float4 sector_lds[LDS_SECTORS];
+    __shared__ unsigned char tex_lds[LDS_TEXTURES];
+    Tables tb;
+    stage_tables(m, sector_lds, tex_lds, tb);
     if (threadIdx.x == 0) lane_ctx = sc.ctx[local];
-    for (int k = threadIdx.x; k < 32 * 256 / 4; k += SW) reinterpret_cast<unsigned int *>(colormap_lds)[k] = reinterpret_cast<const unsigned int *>(m->colormap)[k];
+    for (int k = threadIdx.x; k < 32 * 256 / 4; k += 64) reinterpret_cast<unsigned int *>(colormap_lds)[k] = reinterpret_cast<const unsigned int *>(m->colormap)[k];
     __syncthreads();
-    const int x = threadIdx.x;
+    const int x = blockIdx.x * 64 + threadIdx.x;
     bool window_dirty = false;
     ColumnCtx cc;
-    cc.m = m; cc.mv.m = m; cc.c = &lane_ctx;
+    cc.tb = &tb; cc.m = m; cc.mv.m = m; cc.c = &lane_ctx;
     cc.recs = sc.rec + (size_t)local * m->wall_count;
     cc.list = sc.cand + (size_t)local * CAND_MAX * SW;
     cc.count = sc.cand_count[(size_t)local * SW + x];
@@ -1465,11 +1561,18 @@ __global__ void __launch_bounds__(SW) wall_columns_kernel(DeviceMap dm, int lane
     for (int k = 0; k < cc.count; ++k) if (cc.cand(k).flags & CF_LEDGE) { boundary_has_po = true; break; }
     PassColumn pc;
     bool done = false;
+#ifdef GD_PROFILE
+    long long prof_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    long long prof_start = wall_clock64();
+#endif
     const int lane_id = threadIdx.x & 63;
     const int group_base = lane_id & ~3;
     const int sectors = m->sector_count;
     for (int pass = 0; pass < sectors; ++pass) {
+        PROF_T(t0);
         if (!done) pass_select(cc, st, boundary_has_po, pc);
+        PROF_T(t1);
+        PROF_ADD(0, t0, t1);
         // 4-column wallscan groups (engine.py:12688-12761): exchange with the aligned neighbours
         bool same_group = true;
         int w0 = __shfl(pc.wall, group_base), s0 = __shfl(pc.side, group_base);
@@ -1491,34 +1594,73 @@ __global__ void __launch_bounds__(SW) wall_columns_kernel(DeviceMap dm, int lane
         bool group_valid[3];
         for (int t = 0; t < 3; ++t) group_valid[t] = same_group && all_tier[t] && (common_top[t] < common_bottom[t]);
         if (!done) {
+            PROF_T(t2);
             pass_paint(cc, st, pc, pb, group_valid, common_bottom, first_group_visibility, colormap_lds, window_dirty);
+            PROF_T(t3);
+            PROF_ADD(1, t2, t3);
             bool changed = pass_advance(cc, st, pc, pb, sb);
+            PROF_T(t4);
+            PROF_ADD(2, t3, t4);
+#ifdef GD_PROFILE
+            prof_acc[5] += 1;
+#endif
             // A pass that found nothing and changed nothing repeats identically for ever.
             if (!(pc.bits & PB_VALID) && !changed) done = true;
         }
         if (__ballot(!done) == 0) break;
     }
-    // exact planes (engine.py:13372-13422)
-    {
-        const float flat_center_px = (103.0f + lane_ctx.pitch_offset) + 0.5f;
-        const unsigned char *fflags = sc.flat_flags + (size_t)local * VH * SW;
-        for (int y = 0; y < VH; ++y) {
-            size_t i = (size_t)y * SW + x;
-            unsigned int meta = pb.meta[i];
-            int ps = (int)((meta >> META_SECTOR_SHIFT) & META_SECTOR_MASK) - 1;
-            if (ps < 0 || (meta & META_FILLED)) continue;
-            bool is_floor = meta & META_FLOOR;
-            pb.frame[i] = flat_pixel(m, lane_ctx, ps, is_floor, x, y);
-            // plane fallback occluder for sprites where the flat ray was unresolved.
-            // Bit 1|8 of flat_flags mark repaired pixels, whose surface depth is infinite.
-            if ((fflags[i] & 1) && !finitef(pb.clip_depth[i])) {
-                float plane_height = is_floor ? (lane_ctx.view_z - m->sector_heights[2 * ps]) : (m->sector_heights[2 * ps + 1] - lane_ctx.view_z);
-                float plane_denominator = fmaxf(fabsf((float)y - flat_center_px), 0.5f);
-                pb.clip_depth[i] = plane_height * 192.0f / plane_denominator;
-            }
-        }
-    }
+    PROF_T(t5);
+    PROF_T(t6);
     masked_midtexture(cc, st, pb);
+#ifdef GD_PROFILE
+    long long t7 = wall_clock64();
+    prof_acc[3] += t6 - t5; prof_acc[4] += t7 - t6; prof_acc[6] += t7 - prof_start;
+    if ((threadIdx.x & 63) == 0) {   // one sample per wave: phases are wave-synchronous
+        for (int k = 0; k < 7; ++k) atomicAdd(&g_profile[k], (unsigned long long)prof_acc[k]);
+        atomicAdd(&g_profile[7], 1ULL);
+    }
+#endif
+}
+
+// ---------------------------------------------------------------------------------------------
+// plane shading, one thread per view pixel.  A pixel no wall tier owns shows a flat: the
+// visplane the wall traversal marked for it (engine.py:13372-13405) or, where no drawseg marked
+// one, the sector the per-pixel plane rays selected (engine.py:11145-11163).  Doing both here
+// shades every pixel once, in a kernel light enough to run at full occupancy.
+// ---------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) plane_shade_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
+    const gd_map_desc *m = &dm.d;
+    __shared__ float4 sector_lds[LDS_SECTORS];
+    __shared__ unsigned char tex_lds[LDS_TEXTURES];
+    __shared__ unsigned char colormap_lds[32 * 256];
+    Tables tb;
+    stage_tables(m, sector_lds, tex_lds, tb);
+    for (int k = threadIdx.x; k < 32 * 256 / 4; k += blockDim.x) reinterpret_cast<unsigned int *>(colormap_lds)[k] = reinterpret_cast<const unsigned int *>(m->colormap)[k];
+    __syncthreads();
+    const int local = blockIdx.y;
+    const int pixel = blockIdx.x * blockDim.x + threadIdx.x;
+    if (local >= lane_count || pixel >= VH * SW) return;
+    const int y = pixel / SW, x = pixel - y * SW;
+    const LaneCtx &c = sc.ctx[local];
+    const size_t i = (size_t)local * VH * SW + pixel;
+    const unsigned int meta = sc.meta[i];
+    if (meta & META_FILLED) return;
+    const int ps = (int)((meta >> META_SECTOR_SHIFT) & META_SECTOR_MASK) - 1;
+    unsigned char *frame = frame_base + (size_t)local * frame_stride;
+    if (ps >= 0) {
+        const bool is_floor = meta & META_FLOOR;
+        if (!(meta & META_MASKED)) frame[pixel] = flat_pixel(tb, colormap_lds, c, ps, is_floor, x, y);
+        // plane fallback occluder for sprites where the flat ray was unresolved (engine.py:13417-13422)
+        if ((sc.flat_flags[i] & 1) && !finitef(sc.clip_depth[i])) {
+            const float flat_center_px = (103.0f + c.pitch_offset) + 0.5f;
+            float plane_height = is_floor ? (c.view_z - tb.floor_h(ps)) : (tb.ceil_h(ps) - c.view_z);
+            float plane_denominator = fmaxf(fabsf((float)y - flat_center_px), 0.5f);
+            sc.clip_depth[i] = plane_height * 192.0f / plane_denominator;
+        }
+    } else if (!(meta & META_MASKED)) {
+        const bool is_floor = ((float)y - flat_center(c)) > 0;
+        frame[pixel] = flat_pixel(tb, colormap_lds, c, sc.flat_sector[i], is_floor, x, y);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1783,12 +1925,13 @@ int launch_chunk(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_out 
     hipLaunchKernelGGL(lane_setup_kernel, dim3((count + 63) / 64), dim3(64), 0, stream, r->dm, *lanes, base, count, r->sc);
     hipLaunchKernelGGL(wall_setup_kernel, dim3((m.wall_count + 127) / 128, count), dim3(128), 0, stream, r->dm, count, r->sc);
     mark();
-    mark();
     hipLaunchKernelGGL(flat_select_kernel, dim3((VH * SW + 255) / 256, count), dim3(256), 0, stream, r->dm, *lanes, base, count, r->sc);
     mark();
     hipLaunchKernelGGL(flat_finish_kernel, dim3(count), dim3(SW), 0, stream, r->dm, count, r->sc, frame_base, frame_stride);
     mark();
-    hipLaunchKernelGGL(wall_columns_kernel, dim3(count), dim3(SW), 0, stream, r->dm, count, r->sc, frame_base, frame_stride);
+    hipLaunchKernelGGL(wall_columns_kernel, dim3(SW / 64, count), dim3(64), 0, stream, r->dm, count, r->sc, frame_base, frame_stride);
+    mark();
+    hipLaunchKernelGGL(plane_shade_kernel, dim3((VH * SW + 255) / 256, count), dim3(256), 0, stream, r->dm, count, r->sc, frame_base, frame_stride);
     mark();
     if (lanes->sprite_slots > 0 && lanes->sprite_x) {
         size_t shared = (size_t)lanes->sprite_slots * sizeof(SpriteRec);
@@ -1824,7 +1967,7 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     if (max_lanes <= 0) return fail(GD_E_ARG, "max_lanes must be positive");
     if (h->wall_count <= 0 || h->sector_count <= 0) return fail(GD_E_ARG, "empty map");
     if (h->wall_count >= 65535) return fail(GD_E_ARG, "at most 65534 linedefs");
-    if (h->sector_count >= 16383) return fail(GD_E_ARG, "at most 16382 sectors");
+    if (h->sector_count >= 8191) return fail(GD_E_ARG, "at most 8190 sectors");
     if (h->vertex_count >= 65536) return fail(GD_E_ARG, "at most 65535 distinct vertices");
     gd_renderer *r = new (std::nothrow) gd_renderer();
     if (!r) return fail(GD_E_ARG, "out of host memory");
@@ -1958,6 +2101,15 @@ int gd_renderer_set_sector_lights(gd_renderer *r, const float *lights, void *str
                            hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream)));
     return GD_OK;
 }
+
+#ifdef GD_PROFILE
+/* profiling build only: cumulative per-wave clock ticks of the wall kernel's phases */
+int gd_profile_read(unsigned long long *out, int reset) {
+    HIP_TRY(hipMemcpyFromSymbol(out, HIP_SYMBOL(g_profile), sizeof(unsigned long long) * 16));
+    if (reset) { unsigned long long zero[16] = {0}; HIP_TRY(hipMemcpyToSymbol(HIP_SYMBOL(g_profile), zero, sizeof(zero))); }
+    return GD_OK;
+}
+#endif
 
 int gd_observe(const uint8_t *indexed, int32_t source_rows, const uint8_t *playpal, int32_t lane_count,
                uint8_t *obs, uint8_t *frames, const uint8_t *reset_mask, int32_t stack_mode, void *stream) {

@@ -18,7 +18,7 @@ import torch
 
 from . import _abi, _lib, hostmath, mapbuild
 
-STAGES = ("wall_setup", "column_lists", "flat_select", "flat_finish", "wall_columns", "sprite_columns", "observe")
+STAGES = ("wall_setup", "flat_select", "flat_repair", "wall_columns", "plane_shade", "sprite_columns", "observe")
 
 
 @dataclasses.dataclass
