@@ -39,8 +39,10 @@ MAP_SCALARS = (
     "ceil_level_count",
     "grid_nx",
     "grid_ny",
+    "fine_nx",
+    "fine_ny",
 )
-MAP_FLOATS = ("grid_min_x", "grid_min_y", "grid_cell")
+MAP_FLOATS = ("grid_min_x", "grid_min_y", "grid_cell", "fine_cell")
 
 # (field, numpy dtype) in header order
 MAP_ARRAYS = (
@@ -70,6 +72,7 @@ MAP_ARRAYS = (
     ("grid_item_sector", np.int32),
     ("grid_item_edge_ofs", np.int32),
     ("grid_item_edges", np.int32),
+    ("fine_sector", np.uint16),
     ("floor_levels", np.float32),
     ("ceil_levels", np.float32),
     ("sector_heights", np.float32),

@@ -225,6 +225,10 @@ struct MapView {
     }
 };
 
+#define LDS_SECTORS 512
+#define LDS_TEXTURES 256
+#define GRID_ALWAYS_INSIDE (1 << 30)   // grid item flag: the whole cell lies inside the sector
+
 // Even-odd parity of one sector's edge sub-list around a point (engine.py:9598-9612, 10994-11015).
 __device__ __forceinline__ bool inside_edges(const gd_map_desc *m, int e0, int e1, float px, float py) {
     int crossings = 0;
@@ -249,12 +253,29 @@ __device__ __forceinline__ int grid_cell_of(const gd_map_desc *m, float px, floa
     return (int)fy * m->grid_nx + ix;
 }
 
+#define FINE_MIXED 0xFFFF   // fine cell where the crossing test has to decide
+#define FINE_EMPTY 0xFFFE   // fine cell outside every sector
+
+// Fine raster lookup: the one sector that contains the point, FINE_EMPTY, or FINE_MIXED when the
+// raster cannot tell (near an edge, overlapping sectors, outside the raster, non-finite point).
+__device__ __forceinline__ int fine_lookup(const gd_map_desc *m, float px, float py) {
+    float inv = 1.0f / m->fine_cell;   // a reciprocal is fine here: cells are padded far beyond its rounding
+    float fx = floorf((px - m->grid_min_x) * inv), fy = floorf((py - m->grid_min_y) * inv);
+    if (!(fx >= 0.0f && fx < (float)m->fine_nx && fy >= 0.0f && fy < (float)m->fine_ny)) return FINE_MIXED;
+    return m->fine_sector[(int)fy * m->fine_nx + (int)fx];
+}
+
 // _sector_at (engine.py:9598-9617): first sector with odd parity, 0 when none
 __device__ int sector_at(const gd_map_desc *m, float px, float py) {
+    int fine = fine_lookup(m, px, py);
+    if (fine == FINE_EMPTY) return 0;
+    if (fine != FINE_MIXED) return fine;
     int cell = grid_cell_of(m, px, py);
     if (cell < 0) return 0;
     for (int it = m->grid_cell_ofs[cell]; it < m->grid_cell_ofs[cell + 1]; ++it) {
-        if (inside_edges(m, m->grid_item_edge_ofs[it], m->grid_item_edge_ofs[it + 1], px, py)) return m->grid_item_sector[it];
+        int item = m->grid_item_sector[it];
+        if ((item & GRID_ALWAYS_INSIDE) || inside_edges(m, m->grid_item_edge_ofs[it], m->grid_item_edge_ofs[it + 1], px, py))
+            return item & ~GRID_ALWAYS_INSIDE;
     }
     return 0;
 }
@@ -309,7 +330,7 @@ __device__ __forceinline__ void ray_direction(const LaneCtx &c, int x, float *rx
 
 // distances / along / geometric / projected / left-edge of one linedef at one column
 // (engine.py:11317-11331, 11440-11460)
-__device__ __forceinline__ Eval eval_segment(const float4 wl, const WallRec &r, bool os, const LaneCtx &c, int x, float rx, float ry) {
+__device__ __forceinline__ Eval eval_segment(const float4 wl, int rec_flags, int rec_pl, int rec_pr, bool os, const LaneCtx &c, int x, float rx, float ry) {
     float segx = wl.z - wl.x, segy = wl.w - wl.y;
     float offx = wl.x - c.x, offy = wl.y - c.y;
     float den = rx * segy - ry * segx;
@@ -318,29 +339,38 @@ __device__ __forceinline__ Eval eval_segment(const float4 wl, const WallRec &r, 
     float d = (offx * segy - offy * segx) / safe;
     float a = (offx * ry - offy * rx) / safe;
     bool g = ok && (d > 0) && (a >= 0) && (a <= 1);
-    bool screen_valid = (r.flags & WF_HC) && (x >= r.pl) && (x < r.pr);
+    bool screen_valid = (rec_flags & WF_HC) && (x >= rec_pl) && (x < rec_pr);
     bool p = ok && (d > 0) && screen_valid;
-    bool valid = os ? (p && (r.flags & WF_FF)) : (g || p);
+    bool valid = os ? (p && (rec_flags & WF_FF)) : (g || p);
     Eval out;
     out.dist = valid ? d : GD_INF;
-    out.flags = (g ? CF_GEO : 0) | (p ? CF_PROJ : 0) | ((x == r.pl) ? CF_LEDGE : 0) | ((a > 0.5f) ? CF_ALONG_HI : 0) |
-                ((r.flags & WF_FF) ? CF_FF : 0);
+    out.flags = (g ? CF_GEO : 0) | (p ? CF_PROJ : 0) | ((x == rec_pl) ? CF_LEDGE : 0) | ((a > 0.5f) ? CF_ALONG_HI : 0) |
+                ((rec_flags & WF_FF) ? CF_FF : 0);
     return out;
 }
 
 __device__ __forceinline__ Eval eval_wall(const gd_map_desc *m, const LaneCtx &c, const WallRec *recs, int x, int w, float rx, float ry) {
     const float4 wl = *reinterpret_cast<const float4 *>(m->walls + 4 * w);
-    return eval_segment(wl, recs[w], m->wall_sectors[2 * w + 1] < 0, c, x, rx, ry);
+    const WallRec &r = recs[w];
+    return eval_segment(wl, r.flags, r.pl, r.pr, m->wall_sectors[2 * w + 1] < 0, c, x, rx, ry);
 }
 
 // ---------------------------------------------------------------------------------------------
 // wall_setup: engine.py:10747-10869 (FWallCoords) and the per-linedef half of 11304-11451
 // ---------------------------------------------------------------------------------------------
-__global__ void wall_setup_kernel(DeviceMap dm, int lane_count, Scratch sc) {
+//
+// One thread owns one linedef for the per-linedef arithmetic.  The two per-column loops have
+// wildly different trip counts per linedef (none for most, up to 320 for a few), so they are
+// run by the whole wavefront together: the linedefs with a non-empty column range take turns,
+// their parameters are broadcast from the owning lane, and the 64 lanes each take one column.
+__global__ void __launch_bounds__(128) wall_setup_kernel(DeviceMap dm, int lane_count, Scratch sc) {
     const gd_map_desc *m = &dm.d;
-    int w = blockIdx.x * blockDim.x + threadIdx.x;
-    int local = blockIdx.y;
-    if (w >= m->wall_count || local >= lane_count) return;
+    const int slot_in_wave = threadIdx.x & 63;
+    const int w_raw = blockIdx.x * blockDim.x + threadIdx.x;
+    const int local = blockIdx.y;
+    if (local >= lane_count) return;          // uniform over the block
+    const bool live = w_raw < m->wall_count;  // dead lanes still help with the column loops
+    const int w = live ? w_raw : 0;
     const LaneCtx &c = sc.ctx[local];
     const int *wf = m->walls_fixed + 4 * w;
     i64 rx0 = (i64)wf[0] - c.view_x_fixed, ry0 = (i64)wf[1] - c.view_y_fixed;
@@ -394,17 +424,31 @@ __global__ void wall_setup_kernel(DeviceMap dm, int lane_count, Scratch sc) {
             scan_lo = 1; scan_hi = 0;   // wholly behind the camera: no ray reaches it
         }
     }
+    if (!live) { scan_lo = 1; scan_hi = 0; }
     int first = 0, last = SW - 1; bool any = false;
     float numer_d = offx * segy - offy * segx;
-    for (int x = scan_lo; x <= scan_hi; ++x) {
-        float rx, ry; ray_direction(c, x, &rx, &ry);
-        float den = rx * segy - ry * segx;
-        bool ok = fabsf(den) >= 1e-6f;
-        float safe = ok ? den : 1.0f;
-        float d = numer_d / safe;
-        float a = (offx * ry - offy * rx) / safe;
-        bool g = ok && (d > 0) && (a >= 0) && (a <= 1);
-        if (g) { if (!any) first = x; last = x; any = true; }
+    for (u64 pending = __ballot(scan_lo <= scan_hi); pending; pending &= pending - 1) {
+        const int owner = __ffsll((long long)pending) - 1;
+        const float b_segx = __shfl(segx, owner), b_segy = __shfl(segy, owner);
+        const float b_offx = __shfl(offx, owner), b_offy = __shfl(offy, owner), b_numer = __shfl(numer_d, owner);
+        const int b_lo = __shfl(scan_lo, owner), b_hi = __shfl(scan_hi, owner);
+        int hit_first = SW, hit_last = -1;
+        for (int x0 = b_lo; x0 <= b_hi; x0 += 64) {
+            const int x = x0 + slot_in_wave;
+            float rx, ry; ray_direction(c, x, &rx, &ry);
+            float den = rx * b_segy - ry * b_segx;
+            bool ok = fabsf(den) >= 1e-6f;
+            float safe = ok ? den : 1.0f;
+            float d = b_numer / safe;
+            float a = (b_offx * ry - b_offy * rx) / safe;
+            bool g = x <= b_hi && ok && (d > 0) && (a >= 0) && (a <= 1);
+            const u64 hits = __ballot(g);
+            if (hits) {
+                if (hit_last < 0) hit_first = x0 + __ffsll((long long)hits) - 1;
+                hit_last = x0 + 63 - __clzll((long long)hits);
+            }
+        }
+        if (slot_in_wave == owner && hit_last >= 0) { first = hit_first; last = hit_last; any = true; }
     }
     float vfx = c.x - wl.x, vfy = c.y - wl.y;
     bool ff = (segx * vfy - segy * vfx) < 0;
@@ -437,7 +481,7 @@ __global__ void wall_setup_kernel(DeviceMap dm, int lane_count, Scratch sc) {
     r.dl = dl; r.dr = dr; r.sl = sl; r.sr = sr;
     r.pl = (short)screen_left; r.pr = (short)screen_right;
     r.flags = (hc ? WF_HC : 0) | (ff ? WF_FF : 0) | (((sr - sl <= 1) && !os) ? WF_SUBPIXEL : 0) | (any ? WF_ANYGEO : 0);
-    sc.rec[(size_t)local * m->wall_count + w] = r;
+    if (live) sc.rec[(size_t)local * m->wall_count + w] = r;
     // Enter the linedef in the candidate list of every column where its distance can be
     // finite: its owned span (projected) and, for two-sided lines, the columns its rays hit
     // (engine.py:11446-11451).  List order is irrelevant: scans break ties on the linedef index.
@@ -445,15 +489,27 @@ __global__ void wall_setup_kernel(DeviceMap dm, int lane_count, Scratch sc) {
     if (hc && (!os || ff)) { a_lo = r.pl; a_hi = r.pr; }
     if (!os && any) { a_lo = a_lo < first ? a_lo : first; a_hi = a_hi > last + 1 ? a_hi : last + 1; }
     a_lo = a_lo < 0 ? 0 : a_lo; a_hi = a_hi > SW ? SW : a_hi;
-    if (a_lo < a_hi) {
-        Cand *list = sc.cand + (size_t)local * CAND_MAX * SW;
-        int *counts = sc.cand_count + (size_t)local * SW;
+    if (!live) { a_lo = SW; a_hi = 0; }
+    Cand *list = sc.cand + (size_t)local * CAND_MAX * SW;
+    int *counts = sc.cand_count + (size_t)local * SW;
+    const int packed_sectors = (s0 & 0xFFFF) | (s1 << 16);
+    const int packed_vertices = (int)(((unsigned)m->wall_vertex[2 * w] & 0xFFFFu) | ((unsigned)m->wall_vertex[2 * w + 1] << 16));
+    const int packed_span = (r.flags & 0xFF) | (os ? 0x100 : 0);
+    const int rec_pl = r.pl, rec_pr = r.pr;
+    for (u64 pending = __ballot(a_lo < a_hi); pending; pending &= pending - 1) {
+        const int owner = __ffsll((long long)pending) - 1;
+        float4 b_wl;
+        b_wl.x = __shfl(wl.x, owner); b_wl.y = __shfl(wl.y, owner); b_wl.z = __shfl(wl.z, owner); b_wl.w = __shfl(wl.w, owner);
+        const int b_span = __shfl(packed_span, owner), b_pl = __shfl(rec_pl, owner), b_pr = __shfl(rec_pr, owner);
+        const int b_sectors = __shfl(packed_sectors, owner), b_vertices = __shfl(packed_vertices, owner);
+        const int b_lo = __shfl(a_lo, owner), b_hi = __shfl(a_hi, owner);
         Cand entry;
-        entry.wall = (unsigned short)w; entry.s0 = (short)s0; entry.s1 = (short)s1;
-        entry.v0 = (unsigned short)m->wall_vertex[2 * w]; entry.v1 = (unsigned short)m->wall_vertex[2 * w + 1];
-        for (int x = a_lo; x < a_hi; ++x) {
+        entry.wall = (unsigned short)__shfl(w, owner);
+        entry.s0 = (short)(b_sectors & 0xFFFF); entry.s1 = (short)(b_sectors >> 16);
+        entry.v0 = (unsigned short)(b_vertices & 0xFFFF); entry.v1 = (unsigned short)((unsigned)b_vertices >> 16);
+        for (int x = b_lo + slot_in_wave; x < b_hi; x += 64) {
             float rx, ry; ray_direction(c, x, &rx, &ry);
-            Eval e = eval_segment(wl, r, os, c, x, rx, ry);
+            Eval e = eval_segment(b_wl, b_span & 0xFF, b_pl, b_pr, (b_span & 0x100) != 0, c, x, rx, ry);
             if (finitef(e.dist)) {
                 int slot = atomicAdd(&counts[x], 1);
                 if (slot < CAND_MAX) {
@@ -480,6 +536,10 @@ __global__ void flat_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
     const gd_map_desc *m = &dm.d;
     int local = blockIdx.y;
     int pixel = blockIdx.x * blockDim.x + threadIdx.x;
+    __shared__ float2 heights_lds[LDS_SECTORS];
+    const int staged = m->sector_count < LDS_SECTORS ? m->sector_count : LDS_SECTORS;
+    for (int s = threadIdx.x; s < staged; s += blockDim.x) heights_lds[s] = *reinterpret_cast<const float2 *>(m->sector_heights + 2 * s);
+    __syncthreads();
     if (local >= lane_count || pixel >= VH * SW) return;
     int y = pixel / SW, x = pixel - y * SW;
     const LaneCtx &c = sc.ctx[local];
@@ -502,14 +562,22 @@ __global__ void flat_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
         if (!(finitef(cd) && cd > 0)) continue;
         if (cd > best) break;           // later levels are at least this far
         float px = c.x + rc * cd, py = c.y + rs * cd;
+        int fine = fine_lookup(m, px, py);
+        if (fine == FINE_EMPTY) continue;
+        if (fine != FINE_MIXED) {
+            float2 h = fine < staged ? heights_lds[fine] : *reinterpret_cast<const float2 *>(m->sector_heights + 2 * fine);
+            if ((is_floor ? h.x : h.y) == level && (cd < best || (cd == best && fine < best_sector))) { best = cd; best_sector = fine; }
+            continue;
+        }
         int cell = grid_cell_of(m, px, py);
         if (cell < 0) continue;
         for (int it = m->grid_cell_ofs[cell]; it < m->grid_cell_ofs[cell + 1]; ++it) {
-            int s = m->grid_item_sector[it];
-            float sector_level = m->sector_heights[2 * s + (is_floor ? 0 : 1)];
-            if (sector_level != level) continue;
+            int item = m->grid_item_sector[it];
+            int s = item & ~GRID_ALWAYS_INSIDE;
+            float2 h = s < staged ? heights_lds[s] : *reinterpret_cast<const float2 *>(m->sector_heights + 2 * s);
+            if ((is_floor ? h.x : h.y) != level) continue;
             if (cd < best || (cd == best && s < best_sector)) {
-                if (inside_edges(m, m->grid_item_edge_ofs[it], m->grid_item_edge_ofs[it + 1], px, py)) { best = cd; best_sector = s; }
+                if ((item & GRID_ALWAYS_INSIDE) || inside_edges(m, m->grid_item_edge_ofs[it], m->grid_item_edge_ofs[it + 1], px, py)) { best = cd; best_sector = s; }
             }
         }
     }
@@ -521,8 +589,6 @@ __global__ void flat_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
 // Small per-sector / per-texture tables staged in LDS by the kernels whose inner loops chase
 // them (a dependent global gather costs ~500 cycles, an LDS read ~60).  Sectors or textures
 // beyond the staged count fall back to the global arrays.
-#define LDS_SECTORS 512
-#define LDS_TEXTURES 256
 struct Tables {
     const gd_map_desc *m;
     const float4 *sector;          // floor, ceiling, light, bits(floor_tex | ceil_tex << 16)
@@ -1969,6 +2035,7 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     if (h->wall_count >= 65535) return fail(GD_E_ARG, "at most 65534 linedefs");
     if (h->sector_count >= 8191) return fail(GD_E_ARG, "at most 8190 sectors");
     if (h->vertex_count >= 65536) return fail(GD_E_ARG, "at most 65535 distinct vertices");
+    if (h->fine_nx <= 0 || h->fine_ny <= 0 || !(h->fine_cell > 0.0f) || !h->fine_sector) return fail(GD_E_ARG, "missing fine point-location raster");
     gd_renderer *r = new (std::nothrow) gd_renderer();
     if (!r) return fail(GD_E_ARG, "out of host memory");
     r->events_ready = false;
@@ -1992,6 +2059,7 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     const size_t items = h->grid_cell_ofs[cells];
     UP(grid_cell_ofs, cells + 1); UP(grid_item_sector, items); UP(grid_item_edge_ofs, items + 1);
     UP(grid_item_edges, h->grid_item_edge_ofs[items]);
+    UP(fine_sector, (size_t)h->fine_nx * h->fine_ny);
     UP(floor_levels, h->floor_level_count); UP(ceil_levels, h->ceil_level_count);
     UP(sector_heights, S * 2); UP(sector_lights, S); UP(sector_floor_tex, S); UP(sector_ceil_tex, S);
     const size_t texels = (size_t)h->texture_count * h->tex_max_h * h->tex_max_w;

@@ -156,6 +156,7 @@ def build_map_tables(smap) -> dict[str, np.ndarray | int]:
     spr_post_top = np.maximum.accumulate(np.where(starts, rows, 0), axis=1).astype(np.uint8)
 
     grid = build_sector_grid(walls, sector_edge_ofs, sector_edge_idx, sector_count)
+    grid.update(build_fine_grid(walls, sector_edge_ofs, sector_edge_idx, sector_count, grid["grid_min_x"], grid["grid_min_y"]))
     heights = np.ascontiguousarray(smap.sector_heights, dtype=np.float32)
     # Plane levels in the order that makes plane height (and so ray distance) ascend:
     # floors from the highest down, ceilings from the lowest up.
@@ -223,6 +224,118 @@ def build_map_tables(smap) -> dict[str, np.ndarray | int]:
 
 GRID_CELL = 64.0
 GRID_PAD = 0.5
+GRID_ALWAYS_INSIDE = 1 << 30  # flag on a grid item: every point of the cell is inside that sector
+
+
+def _any_segment_near_box(segments: np.ndarray, x0: float, y0: float, x1: float, y1: float) -> bool:
+    """True when some segment [x1,y1,x2,y2] intersects the axis-aligned box (Liang-Barsky clip)."""
+
+    px, py = segments[:, 0], segments[:, 1]
+    dx, dy = segments[:, 2] - px, segments[:, 3] - py
+    t0 = np.zeros(len(segments))
+    t1 = np.ones(len(segments))
+    alive = np.ones(len(segments), dtype=bool)
+    for p, q in ((-dx, px - x0), (dx, x1 - px), (-dy, py - y0), (dy, y1 - py)):
+        parallel = p == 0
+        alive &= ~(parallel & (q < 0))
+        with np.errstate(divide="ignore", invalid="ignore"):
+            r = np.where(parallel, 0.0, q / np.where(parallel, 1.0, p))
+        entering = (p < 0) & ~parallel
+        leaving = (p > 0) & ~parallel
+        t0 = np.where(entering, np.maximum(t0, r), t0)
+        t1 = np.where(leaving, np.minimum(t1, r), t1)
+    return bool(np.any(alive & (t0 <= t1)))
+
+
+FINE_CELL = 8.0
+FINE_MAX_CELLS = 1 << 21
+FINE_MIXED = 0xFFFF  # fine cell near an edge, in several sectors or otherwise undecided: run the crossing test
+FINE_EMPTY = 0xFFFE  # fine cell wholly outside every sector
+
+
+def build_fine_grid(walls, sector_edge_ofs, sector_edge_idx, sector_count, min_x: float, min_y: float) -> dict:
+    """Fine raster of the even-odd point location (``engine.py:9598-9617``, ``10994-11015``).
+
+    A cell that no linedef comes within ``GRID_PAD`` of is wholly inside or wholly outside
+    each sector, and the float32 crossing test agrees with exact geometry there (its error is
+    orders of magnitude below the pad).  Such a cell stores the one sector that contains its
+    centre, or ``FINE_EMPTY``; every other cell stores ``FINE_MIXED`` and the caller falls back
+    to the crossing test.  The grid shares its origin with the coarse point-location grid.
+    """
+
+    walls64 = np.asarray(walls, dtype=np.float64)
+    max_x = float(walls64[:, (0, 2)].max()) + 2 * GRID_PAD
+    max_y = float(walls64[:, (1, 3)].max()) + 2 * GRID_PAD
+    cell = FINE_CELL
+    while (np.ceil((max_x - min_x) / cell) + 1) * (np.ceil((max_y - min_y) / cell) + 1) > FINE_MAX_CELLS:
+        cell *= 2.0
+    nx = int(np.ceil((max_x - min_x) / cell)) + 1
+    ny = int(np.ceil((max_y - min_y) / cell)) + 1
+    mixed = np.zeros((ny, nx), dtype=bool)
+    used = np.unique(sector_edge_idx[: sector_edge_ofs[sector_count]])
+    for w in used:
+        x1, y1, x2, y2 = walls64[w]
+        ix0 = max(int(np.floor((min(x1, x2) - GRID_PAD - min_x) / cell)), 0)
+        ix1 = min(int(np.floor((max(x1, x2) + GRID_PAD - min_x) / cell)), nx - 1)
+        iy0 = max(int(np.floor((min(y1, y2) - GRID_PAD - min_y) / cell)), 0)
+        iy1 = min(int(np.floor((max(y1, y2) + GRID_PAD - min_y) / cell)), ny - 1)
+        if ix1 < ix0 or iy1 < iy0:
+            continue
+        if ix0 == ix1 or iy0 == iy1 or x1 == x2 or y1 == y2:
+            mixed[iy0 : iy1 + 1, ix0 : ix1 + 1] = True
+            continue
+        # Liang-Barsky clip of the one segment against every padded cell box of its bounding box
+        bx0 = (min_x + np.arange(ix0, ix1 + 1) * cell - GRID_PAD)[None, :]
+        by0 = (min_y + np.arange(iy0, iy1 + 1) * cell - GRID_PAD)[:, None]
+        bx1 = bx0 + cell + 2 * GRID_PAD
+        by1 = by0 + cell + 2 * GRID_PAD
+        dx, dy = x2 - x1, y2 - y1
+        tx_a, tx_b = (bx0 - x1) / dx, (bx1 - x1) / dx
+        ty_a, ty_b = (by0 - y1) / dy, (by1 - y1) / dy
+        t_in = np.maximum(np.maximum(np.minimum(tx_a, tx_b), np.minimum(ty_a, ty_b)), 0.0)
+        t_out = np.minimum(np.minimum(np.maximum(tx_a, tx_b), np.maximum(ty_a, ty_b)), 1.0)
+        mixed[iy0 : iy1 + 1, ix0 : ix1 + 1] |= t_in <= t_out
+    owners = np.zeros((ny, nx), dtype=np.int32)
+    owner = np.full((ny, nx), FINE_EMPTY, dtype=np.uint16)
+    for s in range(sector_count):
+        edges = sector_edge_idx[sector_edge_ofs[s] : sector_edge_ofs[s + 1]]
+        if len(edges) == 0:
+            continue
+        seg = walls64[edges]
+        ends = np.concatenate([seg[:, 0:2], seg[:, 2:4]]) + 0.0
+        _, counts = np.unique(ends, axis=0, return_counts=True)
+        closed = bool(np.all(counts % 2 == 0))
+        ix0 = 0 if not closed else max(int(np.floor((seg[:, (0, 2)].min() - GRID_PAD - min_x) / cell)), 0)
+        ix1 = min(int(np.floor((seg[:, (0, 2)].max() + GRID_PAD - min_x) / cell)), nx - 1)
+        iy0 = max(int(np.floor((seg[:, (1, 3)].min() - GRID_PAD - min_y) / cell)), 0)
+        iy1 = min(int(np.floor((seg[:, (1, 3)].max() + GRID_PAD - min_y) / cell)), ny - 1)
+        if ix1 < ix0 or iy1 < iy0:
+            continue
+        if not closed:  # an open boundary can give odd parity anywhere to its left
+            mixed[iy0 : iy1 + 1, ix0 : ix1 + 1] = True
+            continue
+        cx = (min_x + (np.arange(ix0, ix1 + 1) + 0.5) * cell)[None, :, None]
+        cy = (min_y + (np.arange(iy0, iy1 + 1) + 0.5) * cell)[:, None, None]
+        ex1, ey1, ex2, ey2 = (seg[:, k][None, None, :] for k in range(4))
+        crosses = (ey1 > cy) != (ey2 > cy)
+        with np.errstate(divide="ignore", invalid="ignore"):
+            crossing_x = ex1 + (cy - ey1) * (ex2 - ex1) / np.where(ey2 == ey1, 1.0, ey2 - ey1)
+        inside = (np.count_nonzero(crosses & (cx < crossing_x), axis=2) & 1).astype(bool)
+        view_owners = owners[iy0 : iy1 + 1, ix0 : ix1 + 1]
+        view_owner = owner[iy0 : iy1 + 1, ix0 : ix1 + 1]
+        view_owner[inside & (view_owners == 0)] = s
+        view_owners += inside
+    mixed |= owners > 1
+    owner[mixed] = FINE_MIXED
+    return dict(fine_nx=nx, fine_ny=ny, fine_cell=float(cell), fine_sector=np.ascontiguousarray(owner.reshape(-1)))
+
+
+def _point_in_polygon(segments: np.ndarray, x: float, y: float) -> bool:
+    x1, y1, x2, y2 = segments[:, 0], segments[:, 1], segments[:, 2], segments[:, 3]
+    crosses = (y1 > y) != (y2 > y)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        crossing_x = x1 + (y - y1) * (x2 - x1) / np.where(y2 == y1, 1.0, y2 - y1)
+    return bool(np.count_nonzero(crosses & (x < crossing_x)) & 1)
 
 
 def build_sector_grid(walls, sector_edge_ofs, sector_edge_idx, sector_count, cell: float = GRID_CELL) -> dict:
@@ -270,13 +383,24 @@ def build_sector_grid(walls, sector_edge_ofs, sector_edge_idx, sector_count, cel
         edge_max_x = ex.max(axis=1)
         edge_min_y = ey.min(axis=1)
         edge_max_y = ey.max(axis=1)
+        segments = walls[edges].astype(np.float64)
         for iy in range(iy0, iy1 + 1):
             cy0 = min_y + iy * cell - GRID_PAD
             cy1 = min_y + (iy + 1) * cell + GRID_PAD
             row_mask = (edge_max_y >= cy0) & (edge_min_y <= cy1)
             for ix in range(ix0, ix1 + 1):
                 cx0 = (min_x + ix * cell - GRID_PAD) if ix > 0 else -np.inf
+                cx1 = min_x + (ix + 1) * cell + GRID_PAD
                 keep = row_mask & (edge_max_x >= cx0)
+                # A cell that no edge of the sector comes near (padded by GRID_PAD, far more than the
+                # float32 error of the crossing test) lies wholly inside or wholly outside the sector:
+                # decide once at its centre and spare the kernels every edge test there.
+                if closed and ix > 0 and not _any_segment_near_box(segments, cx0, cy0, cx1, cy1):
+                    centre_x = min_x + (ix + 0.5) * cell
+                    centre_y = min_y + (iy + 0.5) * cell
+                    if _point_in_polygon(segments, centre_x, centre_y):
+                        cell_rows[iy * nx + ix].append((s | GRID_ALWAYS_INSIDE, []))
+                    continue
                 cell_rows[iy * nx + ix].append((s, [int(w) for w in edges[keep]]))
     cell_ofs = np.zeros(nx * ny + 1, dtype=np.int32)
     item_sector: list[int] = []
@@ -295,7 +419,7 @@ def build_sector_grid(walls, sector_edge_ofs, sector_edge_idx, sector_count, cel
         grid_min_y=min_y,
         grid_cell=float(cell),
         grid_cell_ofs=cell_ofs,
-        grid_item_sector=np.asarray(item_sector if item_sector else [0], dtype=np.int32),
+        grid_item_sector=np.asarray(item_sector if item_sector else [0], dtype=np.int32),  # | GRID_ALWAYS_INSIDE
         grid_item_edge_ofs=np.asarray(item_edge_ofs, dtype=np.int32),
         grid_item_edges=np.asarray(item_edges if item_edges else [0], dtype=np.int32),
     )

@@ -59,7 +59,8 @@ typedef struct gd_map_desc {
     int32_t direct_neighbors;/* 1: every linedef has <=1 start and <=1 end neighbour (engine.py:1558) */
     int32_t floor_level_count, ceil_level_count; /* distinct plane heights */
     int32_t grid_nx, grid_ny;/* point-location grid (cells of grid_cell map units) */
-    float grid_min_x, grid_min_y, grid_cell;
+    int32_t fine_nx, fine_ny;/* fine point-location raster (cells of fine_cell map units, same origin) */
+    float grid_min_x, grid_min_y, grid_cell, fine_cell;
 
     const float *walls;              /* [W,4] x1,y1,x2,y2 (portal_walls) */
     const int32_t *walls_fixed;      /* [W,4] rint(walls*65536) (engine.py:10876) */
@@ -87,9 +88,12 @@ typedef struct gd_map_desc {
     /* Point-location grid: the even-odd polygon tests of engine.py:9598-9617 and
        10994-11015 restricted, per cell, to the sectors and edges that can count there. */
     const int32_t *grid_cell_ofs;    /* [nx*ny+1] -> items */
-    const int32_t *grid_item_sector; /* [items] ascending sector id within a cell */
+    const int32_t *grid_item_sector; /* [items] ascending sector id within a cell; bit 30 set = the whole
+                                        cell lies inside that sector (no edge list, no crossing test) */
     const int32_t *grid_item_edge_ofs;/* [items+1] -> grid_item_edges */
     const int32_t *grid_item_edges;  /* linedef ids */
+    const uint16_t *fine_sector;     /* [fine_ny*fine_nx] the one sector containing the whole cell, 0xFFFE =
+                                        outside every sector, 0xFFFF = undecided (run the crossing test) */
     const float *floor_levels;       /* [floor_level_count] distinct floor heights, descending */
     const float *ceil_levels;        /* [ceil_level_count] distinct ceiling heights, ascending */
 

@@ -65,7 +65,7 @@ def test_sector_grid_lists_every_edge_that_can_count():
                 count += 1
         return count & 1
 
-    for _ in range(400):
+    for _ in range(1500):
         px = np.float32(rng.uniform(lo[0], hi[0]))
         py = np.float32(rng.uniform(lo[1], hi[1]))
         fx = np.floor(np.float32(np.float32(px - np.float32(tables["grid_min_x"])) / np.float32(tables["grid_cell"])))
@@ -75,9 +75,50 @@ def test_sector_grid_lists_every_edge_that_can_count():
             cell = int(fy) * nx + max(int(fx), 0)
             for item in range(tables["grid_cell_ofs"][cell], tables["grid_cell_ofs"][cell + 1]):
                 e0, e1 = tables["grid_item_edge_ofs"][item], tables["grid_item_edge_ofs"][item + 1]
-                listed[int(tables["grid_item_sector"][item])] = tables["grid_item_edges"][e0:e1]
+                entry = int(tables["grid_item_sector"][item])
+                listed[entry & ~(1 << 30)] = None if entry & (1 << 30) else tables["grid_item_edges"][e0:e1]
         for s in range(tables["sector_count"]):
             full = tables["sector_edge_idx"][tables["sector_edge_ofs"][s] : tables["sector_edge_ofs"][s + 1]]
             expected = parity(full, px, py)
-            got = parity(listed[s], px, py) if s in listed else 0
+            got = (1 if listed[s] is None else parity(listed[s], px, py)) if s in listed else 0
             assert got == expected
+
+
+@pytest.mark.parametrize("fixture", ["small_midtex_sprites", "brick_islands"])
+def test_fine_raster_agrees_with_the_crossing_test(fixture):
+    # every decided cell of the fine raster must name exactly the set of sectors with odd float32 parity;
+    # points are drawn uniformly and also snapped close to linedefs, where a wrong "decided" cell would show
+    _meta, _data, smap, tables = load_fixture(fixture)
+    rng = np.random.default_rng(2)
+    walls = tables["walls"].astype(np.float32)
+    S = tables["sector_count"]
+    count = 6000
+    px = rng.uniform(walls[:, (0, 2)].min() - 30, walls[:, (0, 2)].max() + 30, count)
+    py = rng.uniform(walls[:, (1, 3)].min() - 30, walls[:, (1, 3)].max() + 30, count)
+    pick = rng.integers(0, len(walls), count // 2)
+    t = rng.uniform(0, 1, count // 2)
+    px[: count // 2] = walls[pick, 0] + t * (walls[pick, 2] - walls[pick, 0]) + rng.uniform(-1.5, 1.5, count // 2)
+    py[: count // 2] = walls[pick, 1] + t * (walls[pick, 3] - walls[pick, 1]) + rng.uniform(-1.5, 1.5, count // 2)
+    px, py = px.astype(np.float32), py.astype(np.float32)
+    inv = np.float32(1.0) / np.float32(tables["fine_cell"])
+    fx = np.floor((px - np.float32(tables["grid_min_x"])) * inv)
+    fy = np.floor((py - np.float32(tables["grid_min_y"])) * inv)
+    inside_raster = (fx >= 0) & (fx < tables["fine_nx"]) & (fy >= 0) & (fy < tables["fine_ny"])
+    entry = np.full(count, 0xFFFF, dtype=np.int64)
+    entry[inside_raster] = tables["fine_sector"][fy[inside_raster].astype(int) * tables["fine_nx"] + fx[inside_raster].astype(int)]
+    parity = np.zeros((count, S), dtype=bool)
+    for s in range(S):
+        e = walls[tables["sector_edge_idx"][tables["sector_edge_ofs"][s] : tables["sector_edge_ofs"][s + 1]]]
+        x1, y1, x2, y2 = (e[:, k][None, :] for k in range(4))
+        dy = y2 - y1
+        safe = np.where(np.abs(dy) < 1e-6, np.float32(1.0), dy)
+        crossing = x1 + (py[:, None] - y1) * (x2 - x1) / safe
+        assert crossing.dtype == np.float32
+        parity[:, s] = np.count_nonzero(((y1 > py[:, None]) != (y2 > py[:, None])) & (px[:, None] < crossing), axis=1) & 1
+    decided = entry != 0xFFFF
+    assert decided.mean() > 0.3  # the raster must actually decide a good share of the points
+    empty = entry == 0xFFFE
+    assert not parity[empty].any()
+    owned = decided & ~empty
+    assert np.array_equal(parity[owned].sum(axis=1), np.ones(owned.sum(), dtype=int))
+    assert np.array_equal(parity[owned].argmax(axis=1), entry[owned])
