@@ -72,7 +72,7 @@ MAP_ARRAYS = (
     ("grid_item_sector", np.int32),
     ("grid_item_edge_ofs", np.int32),
     ("grid_item_edges", np.int32),
-    ("fine_sector", np.uint16),
+    ("fine_sector", np.uint32),
     ("floor_levels", np.float32),
     ("ceil_levels", np.float32),
     ("sector_heights", np.float32),

@@ -153,6 +153,9 @@ __device__ __forceinline__ i64 tdiv(i64 a, i64 b) {
     }
     return ((a < 0) != (b < 0)) ? -(i64)uq : (i64)uq;
 }
+// Value of `v` in lane `lane` of the wavefront; `lane` must be the same in every active lane.
+__device__ __forceinline__ int bcast(int v, int lane) { return __builtin_amdgcn_readlane(v, lane); }
+__device__ __forceinline__ float bcast(float v, int lane) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane)); }
 __device__ __forceinline__ i64 clampi(i64 v, i64 lo, i64 hi) { return v < lo ? lo : (v > hi ? hi : v); }
 __device__ __forceinline__ i64 max64(i64 a, i64 b) { return a > b ? a : b; }
 __device__ __forceinline__ i64 min64(i64 a, i64 b) { return a < b ? a : b; }
@@ -253,24 +256,34 @@ __device__ __forceinline__ int grid_cell_of(const gd_map_desc *m, float px, floa
     return (int)fy * m->grid_nx + ix;
 }
 
-#define FINE_MIXED 0xFFFF   // fine cell where the crossing test has to decide
-#define FINE_EMPTY 0xFFFE   // fine cell outside every sector
+// Fine raster entries (top two bits): a decided sector, empty, or undecided with / without the
+// masks of plane levels that can win in the cell.
+#define FINE_KIND(v) ((unsigned)(v) >> 30)
+#define FINE_DECIDED 0u
+#define FINE_EMPTY 1u
+#define FINE_MIXED 2u
+#define FINE_UNKNOWN 3u
+#define FINE_MASK_LEVELS 15
 
-// Fine raster lookup: the one sector that contains the point, FINE_EMPTY, or FINE_MIXED when the
-// raster cannot tell (near an edge, overlapping sectors, outside the raster, non-finite point).
-__device__ __forceinline__ int fine_lookup(const gd_map_desc *m, float px, float py) {
-    float inv = 1.0f / m->fine_cell;   // a reciprocal is fine here: cells are padded far beyond its rounding
-    float fx = floorf((px - m->grid_min_x) * inv), fy = floorf((py - m->grid_min_y) * inv);
-    if (!(fx >= 0.0f && fx < (float)m->fine_nx && fy >= 0.0f && fy < (float)m->fine_ny)) return FINE_MIXED;
-    return m->fine_sector[(int)fy * m->fine_nx + (int)fx];
+// Fine raster lookup.  Points outside the raster (or not finite) report FINE_UNKNOWN with a
+// negative cell, and the caller locates them with grid_cell_of.  The coarse cell of a point
+// inside the raster is (iy >> 3) * grid_nx + (ix >> 3): grid_cell is 8 * fine_cell and both
+// grids pad their cells far beyond the rounding of either index computation.
+__device__ __forceinline__ unsigned fine_lookup(const gd_map_desc *m, float inv_cell, float px, float py, int *coarse_cell) {
+    int ix = (int)floorf((px - m->grid_min_x) * inv_cell), iy = (int)floorf((py - m->grid_min_y) * inv_cell);
+    *coarse_cell = -1;
+    if ((unsigned)ix >= (unsigned)m->fine_nx || (unsigned)iy >= (unsigned)m->fine_ny || !(px == px) || !(py == py)) return 0xC0000000u;
+    *coarse_cell = (iy >> 3) * m->grid_nx + (ix >> 3);
+    return m->fine_sector[iy * m->fine_nx + ix];
 }
 
 // _sector_at (engine.py:9598-9617): first sector with odd parity, 0 when none
 __device__ int sector_at(const gd_map_desc *m, float px, float py) {
-    int fine = fine_lookup(m, px, py);
-    if (fine == FINE_EMPTY) return 0;
-    if (fine != FINE_MIXED) return fine;
-    int cell = grid_cell_of(m, px, py);
+    int cell;
+    unsigned fine = fine_lookup(m, 1.0f / m->fine_cell, px, py, &cell);
+    if (FINE_KIND(fine) == FINE_EMPTY) return 0;
+    if (FINE_KIND(fine) == FINE_DECIDED) return (int)(fine & 0xFFFFu);
+    if (cell < 0) cell = grid_cell_of(m, px, py);
     if (cell < 0) return 0;
     for (int it = m->grid_cell_ofs[cell]; it < m->grid_cell_ofs[cell + 1]; ++it) {
         int item = m->grid_item_sector[it];
@@ -429,9 +442,9 @@ __global__ void __launch_bounds__(128) wall_setup_kernel(DeviceMap dm, int lane_
     float numer_d = offx * segy - offy * segx;
     for (u64 pending = __ballot(scan_lo <= scan_hi); pending; pending &= pending - 1) {
         const int owner = __ffsll((long long)pending) - 1;
-        const float b_segx = __shfl(segx, owner), b_segy = __shfl(segy, owner);
-        const float b_offx = __shfl(offx, owner), b_offy = __shfl(offy, owner), b_numer = __shfl(numer_d, owner);
-        const int b_lo = __shfl(scan_lo, owner), b_hi = __shfl(scan_hi, owner);
+        const float b_segx = bcast(segx, owner), b_segy = bcast(segy, owner);
+        const float b_offx = bcast(offx, owner), b_offy = bcast(offy, owner), b_numer = bcast(numer_d, owner);
+        const int b_lo = bcast(scan_lo, owner), b_hi = bcast(scan_hi, owner);
         int hit_first = SW, hit_last = -1;
         for (int x0 = b_lo; x0 <= b_hi; x0 += 64) {
             const int x = x0 + slot_in_wave;
@@ -499,12 +512,12 @@ __global__ void __launch_bounds__(128) wall_setup_kernel(DeviceMap dm, int lane_
     for (u64 pending = __ballot(a_lo < a_hi); pending; pending &= pending - 1) {
         const int owner = __ffsll((long long)pending) - 1;
         float4 b_wl;
-        b_wl.x = __shfl(wl.x, owner); b_wl.y = __shfl(wl.y, owner); b_wl.z = __shfl(wl.z, owner); b_wl.w = __shfl(wl.w, owner);
-        const int b_span = __shfl(packed_span, owner), b_pl = __shfl(rec_pl, owner), b_pr = __shfl(rec_pr, owner);
-        const int b_sectors = __shfl(packed_sectors, owner), b_vertices = __shfl(packed_vertices, owner);
-        const int b_lo = __shfl(a_lo, owner), b_hi = __shfl(a_hi, owner);
+        b_wl.x = bcast(wl.x, owner); b_wl.y = bcast(wl.y, owner); b_wl.z = bcast(wl.z, owner); b_wl.w = bcast(wl.w, owner);
+        const int b_span = bcast(packed_span, owner), b_pl = bcast(rec_pl, owner), b_pr = bcast(rec_pr, owner);
+        const int b_sectors = bcast(packed_sectors, owner), b_vertices = bcast(packed_vertices, owner);
+        const int b_lo = bcast(a_lo, owner), b_hi = bcast(a_hi, owner);
         Cand entry;
-        entry.wall = (unsigned short)__shfl(w, owner);
+        entry.wall = (unsigned short)bcast(w, owner);
         entry.s0 = (short)(b_sectors & 0xFFFF); entry.s1 = (short)(b_sectors >> 16);
         entry.v0 = (unsigned short)(b_vertices & 0xFFFF); entry.v1 = (unsigned short)((unsigned)b_vertices >> 16);
         for (int x = b_lo + slot_in_wave; x < b_hi; x += 64) {
@@ -536,10 +549,6 @@ __global__ void flat_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
     const gd_map_desc *m = &dm.d;
     int local = blockIdx.y;
     int pixel = blockIdx.x * blockDim.x + threadIdx.x;
-    __shared__ float2 heights_lds[LDS_SECTORS];
-    const int staged = m->sector_count < LDS_SECTORS ? m->sector_count : LDS_SECTORS;
-    for (int s = threadIdx.x; s < staged; s += blockDim.x) heights_lds[s] = *reinterpret_cast<const float2 *>(m->sector_heights + 2 * s);
-    __syncthreads();
     if (local >= lane_count || pixel >= VH * SW) return;
     int y = pixel / SW, x = pixel - y * SW;
     const LaneCtx &c = sc.ctx[local];
@@ -550,34 +559,69 @@ __global__ void flat_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
     float denom = fmaxf(fabsf(delta), 0.5f);
     float cc = dm.cosine_correction[x];
     float rc = lanes.ray_cos[(size_t)n * SW + x], rs = lanes.ray_sin[(size_t)n * SW + x];
-    const float *levels = is_floor ? m->floor_levels : m->ceil_levels;
-    int level_count = is_floor ? m->floor_level_count : m->ceil_level_count;
+    // A wavefront covers 64 pixels of one row (320 = 5 * 64), so the plane side and everything
+    // that depends only on (row, level) is the same in all its lanes.
+    const bool floor_uniform = __builtin_amdgcn_readfirstlane((int)is_floor) != 0;
+    const float *levels = floor_uniform ? m->floor_levels : m->ceil_levels;
+    const int level_count = floor_uniform ? m->floor_level_count : m->ceil_level_count;
+    const int mask_shift = floor_uniform ? 0 : FINE_MASK_LEVELS;
+    const int index_shift = floor_uniform ? 16 : 20;
+    // cd = perpendicular / cc below is the hot division.  With y = RN(1 / cc), q = RN(p * y) is within
+    // one ulp of p / cc, and RN(q + RN(p - cc * q) * y) is then the correctly rounded quotient
+    // (Markstein's theorem; the inner product is exact in an FMA) as long as nothing over- or
+    // underflows, which the range tests on both operands ensure.
+    const float inv_cc = 1.0f / cc;
+    const bool cc_plain = cc >= 0.5f && cc <= 1.0f;
+    const float inv_fine = 1.0f / m->fine_cell;   // a reciprocal is fine here: see fine_lookup
+    const int slot_in_wave = threadIdx.x & 63;
     float best = GD_INF; int best_sector = -1;
-    for (int l = 0; l < level_count; ++l) {
-        float level = levels[l];
-        float plane_height = is_floor ? (c.view_z - level) : (level - c.view_z);
-        if (!(plane_height > 0)) continue;
-        float perpendicular = plane_height * 192.0f / denom;
-        float cd = perpendicular / cc;
-        if (!(finitef(cd) && cd > 0)) continue;
-        if (cd > best) break;           // later levels are at least this far
-        float px = c.x + rc * cd, py = c.y + rs * cd;
-        int fine = fine_lookup(m, px, py);
-        if (fine == FINE_EMPTY) continue;
-        if (fine != FINE_MIXED) {
-            float2 h = fine < staged ? heights_lds[fine] : *reinterpret_cast<const float2 *>(m->sector_heights + 2 * fine);
-            if ((is_floor ? h.x : h.y) == level && (cd < best || (cd == best && fine < best_sector))) { best = cd; best_sector = fine; }
-            continue;
-        }
-        int cell = grid_cell_of(m, px, py);
-        if (cell < 0) continue;
-        for (int it = m->grid_cell_ofs[cell]; it < m->grid_cell_ofs[cell + 1]; ++it) {
-            int item = m->grid_item_sector[it];
-            int s = item & ~GRID_ALWAYS_INSIDE;
-            float2 h = s < staged ? heights_lds[s] : *reinterpret_cast<const float2 *>(m->sector_heights + 2 * s);
-            if ((is_floor ? h.x : h.y) != level) continue;
-            if (cd < best || (cd == best && s < best_sector)) {
-                if ((item & GRID_ALWAYS_INSIDE) || inside_edges(m, m->grid_item_edge_ofs[it], m->grid_item_edge_ofs[it + 1], px, py)) { best = cd; best_sector = s; }
+    bool done = false;
+    for (int base = 0; base < level_count && !done; base += 64) {
+        // lane k works out level base+k: its height and perpendicular distance (one division for
+        // the wavefront instead of one per level per lane); a level the plane cannot show gets -1
+        const int mine = base + slot_in_wave;
+        const float my_level = mine < level_count ? levels[mine] : 0.0f;
+        const float my_height = floor_uniform ? (c.view_z - my_level) : (my_level - c.view_z);
+        const float my_perpendicular = (mine < level_count && my_height > 0) ? my_height * 192.0f / denom : -1.0f;
+        const int chunk = level_count - base < 64 ? level_count - base : 64;
+        for (int k = 0; k < chunk; ++k) {
+            const float perpendicular = bcast(my_perpendicular, k);
+            const float level = bcast(my_level, k);
+            if (!(perpendicular > 0)) continue;              // the same in every lane
+            float cd;
+            if (cc_plain && perpendicular >= 1e-18f && perpendicular <= 1e18f) {
+                const float q = perpendicular * inv_cc;
+                cd = __builtin_fmaf(__builtin_fmaf(-cc, q, perpendicular), inv_cc, q);
+            } else {
+                cd = perpendicular / cc;
+            }
+            if (!(finitef(cd) && cd > 0)) continue;
+            if (cd > best) { done = true; break; }           // later levels are at least this far
+            float px = c.x + rc * cd, py = c.y + rs * cd;
+            int cell;
+            unsigned fine = fine_lookup(m, inv_fine, px, py, &cell);
+            unsigned kind = FINE_KIND(fine);
+            if (kind == FINE_EMPTY) continue;
+            if (kind == FINE_DECIDED) {
+                const int s = (int)(fine & 0xFFFFu);
+                const unsigned listed = (fine >> index_shift) & 15u;   // the sector's level index, 15 = not recorded
+                bool same_level = listed == (unsigned)(base + k);
+                if (listed == 15u) {
+                    same_level = m->sector_heights[2 * s + (floor_uniform ? 0 : 1)] == level;
+                }
+                if (same_level && (cd < best || (cd == best && s < best_sector))) { best = cd; best_sector = s; }
+                continue;
+            }
+            if (kind == FINE_MIXED && !((fine >> (mask_shift + base + k)) & 1u)) continue;   // no sector here has this level
+            if (cell < 0) cell = grid_cell_of(m, px, py);
+            if (cell < 0) continue;
+            for (int it = m->grid_cell_ofs[cell]; it < m->grid_cell_ofs[cell + 1]; ++it) {
+                int item = m->grid_item_sector[it];
+                int s = item & ~GRID_ALWAYS_INSIDE;
+                if (m->sector_heights[2 * s + (floor_uniform ? 0 : 1)] != level) continue;
+                if (cd < best || (cd == best && s < best_sector)) {
+                    if ((item & GRID_ALWAYS_INSIDE) || inside_edges(m, m->grid_item_edge_ofs[it], m->grid_item_edge_ofs[it + 1], px, py)) { best = cd; best_sector = s; }
+                }
             }
         }
     }
@@ -2036,6 +2080,8 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     if (h->sector_count >= 8191) return fail(GD_E_ARG, "at most 8190 sectors");
     if (h->vertex_count >= 65536) return fail(GD_E_ARG, "at most 65535 distinct vertices");
     if (h->fine_nx <= 0 || h->fine_ny <= 0 || !(h->fine_cell > 0.0f) || !h->fine_sector) return fail(GD_E_ARG, "missing fine point-location raster");
+    if (h->grid_cell != 8.0f * h->fine_cell || (h->fine_nx + 7) / 8 > h->grid_nx || (h->fine_ny + 7) / 8 > h->grid_ny)
+        return fail(GD_E_ARG, "grid_cell must be 8 * fine_cell and the coarse grid must cover the fine raster");
     gd_renderer *r = new (std::nothrow) gd_renderer();
     if (!r) return fail(GD_E_ARG, "out of host memory");
     r->events_ready = false;

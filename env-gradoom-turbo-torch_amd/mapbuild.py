@@ -155,13 +155,15 @@ def build_map_tables(smap) -> dict[str, np.ndarray | int]:
     rows = np.arange(spr_opaque.shape[1], dtype=np.int64)[None, :, None]
     spr_post_top = np.maximum.accumulate(np.where(starts, rows, 0), axis=1).astype(np.uint8)
 
-    grid = build_sector_grid(walls, sector_edge_ofs, sector_edge_idx, sector_count)
-    grid.update(build_fine_grid(walls, sector_edge_ofs, sector_edge_idx, sector_count, grid["grid_min_x"], grid["grid_min_y"]))
     heights = np.ascontiguousarray(smap.sector_heights, dtype=np.float32)
     # Plane levels in the order that makes plane height (and so ray distance) ascend:
     # floors from the highest down, ceilings from the lowest up.
     floor_levels = np.unique(heights[:, 0])[::-1].astype(np.float32).copy()
     ceil_levels = np.unique(heights[:, 1]).astype(np.float32).copy()
+    fine_cell = fine_cell_size(walls)
+    grid = build_sector_grid(walls, sector_edge_ofs, sector_edge_idx, sector_count, cell=fine_cell * FINE_PER_COARSE)
+    grid.update(build_fine_grid(walls, sector_edge_ofs, sector_edge_idx, sector_count, grid["grid_min_x"], grid["grid_min_y"],
+                                fine_cell, heights, floor_levels, ceil_levels))
 
     return dict(
         floor_level_count=int(len(floor_levels)),
@@ -248,59 +250,60 @@ def _any_segment_near_box(segments: np.ndarray, x0: float, y0: float, x1: float,
 
 
 FINE_CELL = 8.0
+FINE_PER_COARSE = 8         # the coarse grid cell is this many fine cells wide, same origin
 FINE_MAX_CELLS = 1 << 21
-FINE_MIXED = 0xFFFF  # fine cell near an edge, in several sectors or otherwise undecided: run the crossing test
-FINE_EMPTY = 0xFFFE  # fine cell wholly outside every sector
+FINE_EMPTY = 0x40000000     # fine cell wholly outside every sector
+FINE_MIXED = 0x80000000     # crossing test needed; bits 0..14 / 15..29 = floor / ceiling levels that can win there
+FINE_UNKNOWN = 0xC0000000   # crossing test needed, nothing known about the levels
+FINE_MASK_LEVELS = 15
 
 
-def build_fine_grid(walls, sector_edge_ofs, sector_edge_idx, sector_count, min_x: float, min_y: float) -> dict:
+def fine_cell_size(walls) -> float:
+    """Fine raster cell: FINE_CELL map units, doubled until the raster stays below FINE_MAX_CELLS."""
+
+    walls64 = np.asarray(walls, dtype=np.float64)
+    width = float(walls64[:, (0, 2)].max() - walls64[:, (0, 2)].min()) + 4 * GRID_PAD + 1
+    height = float(walls64[:, (1, 3)].max() - walls64[:, (1, 3)].min()) + 4 * GRID_PAD + 1
+    cell = FINE_CELL
+    while (np.ceil(width / cell) + 1) * (np.ceil(height / cell) + 1) > FINE_MAX_CELLS:
+        cell *= 2.0
+    return cell
+
+
+def build_fine_grid(walls, sector_edge_ofs, sector_edge_idx, sector_count, min_x: float, min_y: float, cell: float,
+                    sector_heights, floor_levels, ceil_levels) -> dict:
     """Fine raster of the even-odd point location (``engine.py:9598-9617``, ``10994-11015``).
 
     A cell that no linedef comes within ``GRID_PAD`` of is wholly inside or wholly outside
     each sector, and the float32 crossing test agrees with exact geometry there (its error is
     orders of magnitude below the pad).  Such a cell stores the one sector that contains its
-    centre, or ``FINE_EMPTY``; every other cell stores ``FINE_MIXED`` and the caller falls back
-    to the crossing test.  The grid shares its origin with the coarse point-location grid.
+    centre (with the indices of its floor and ceiling in the level lists), or ``FINE_EMPTY``.  Every other cell is ``FINE_MIXED`` and the caller falls back to
+    the crossing test; it carries the plane levels of the sectors that can contain one of its
+    points (those with an edge near the cell or containing its centre), so a probe for any other
+    level is a miss without testing.  The raster shares its origin with the coarse grid.
     """
 
     walls64 = np.asarray(walls, dtype=np.float64)
     max_x = float(walls64[:, (0, 2)].max()) + 2 * GRID_PAD
     max_y = float(walls64[:, (1, 3)].max()) + 2 * GRID_PAD
-    cell = FINE_CELL
-    while (np.ceil((max_x - min_x) / cell) + 1) * (np.ceil((max_y - min_y) / cell) + 1) > FINE_MAX_CELLS:
-        cell *= 2.0
     nx = int(np.ceil((max_x - min_x) / cell)) + 1
     ny = int(np.ceil((max_y - min_y) / cell)) + 1
+    masks_known = len(floor_levels) <= FINE_MASK_LEVELS and len(ceil_levels) <= FINE_MASK_LEVELS
     mixed = np.zeros((ny, nx), dtype=bool)
-    used = np.unique(sector_edge_idx[: sector_edge_ofs[sector_count]])
-    for w in used:
-        x1, y1, x2, y2 = walls64[w]
-        ix0 = max(int(np.floor((min(x1, x2) - GRID_PAD - min_x) / cell)), 0)
-        ix1 = min(int(np.floor((max(x1, x2) + GRID_PAD - min_x) / cell)), nx - 1)
-        iy0 = max(int(np.floor((min(y1, y2) - GRID_PAD - min_y) / cell)), 0)
-        iy1 = min(int(np.floor((max(y1, y2) + GRID_PAD - min_y) / cell)), ny - 1)
-        if ix1 < ix0 or iy1 < iy0:
-            continue
-        if ix0 == ix1 or iy0 == iy1 or x1 == x2 or y1 == y2:
-            mixed[iy0 : iy1 + 1, ix0 : ix1 + 1] = True
-            continue
-        # Liang-Barsky clip of the one segment against every padded cell box of its bounding box
-        bx0 = (min_x + np.arange(ix0, ix1 + 1) * cell - GRID_PAD)[None, :]
-        by0 = (min_y + np.arange(iy0, iy1 + 1) * cell - GRID_PAD)[:, None]
-        bx1 = bx0 + cell + 2 * GRID_PAD
-        by1 = by0 + cell + 2 * GRID_PAD
-        dx, dy = x2 - x1, y2 - y1
-        tx_a, tx_b = (bx0 - x1) / dx, (bx1 - x1) / dx
-        ty_a, ty_b = (by0 - y1) / dy, (by1 - y1) / dy
-        t_in = np.maximum(np.maximum(np.minimum(tx_a, tx_b), np.minimum(ty_a, ty_b)), 0.0)
-        t_out = np.minimum(np.minimum(np.maximum(tx_a, tx_b), np.maximum(ty_a, ty_b)), 1.0)
-        mixed[iy0 : iy1 + 1, ix0 : ix1 + 1] |= t_in <= t_out
+    level_bits = np.zeros((ny, nx), dtype=np.uint32)
     owners = np.zeros((ny, nx), dtype=np.int32)
-    owner = np.full((ny, nx), FINE_EMPTY, dtype=np.uint16)
+    owner = np.full((ny, nx), FINE_EMPTY, dtype=np.uint32)
     for s in range(sector_count):
         edges = sector_edge_idx[sector_edge_ofs[s] : sector_edge_ofs[s + 1]]
         if len(edges) == 0:
             continue
+        bits = np.uint32(0)
+        level_index = np.uint32(0xFF << 16)  # decided cells: floor / ceiling level index in bits 16..19 / 20..23, 15 = unknown
+        if masks_known:
+            floor_index = int(np.nonzero(floor_levels == sector_heights[s, 0])[0][0])
+            ceil_index = int(np.nonzero(ceil_levels == sector_heights[s, 1])[0][0])
+            bits = np.uint32((1 << floor_index) | (1 << (FINE_MASK_LEVELS + ceil_index)))
+            level_index = np.uint32((floor_index << 16) | (ceil_index << 20))
         seg = walls64[edges]
         ends = np.concatenate([seg[:, 0:2], seg[:, 2:4]]) + 0.0
         _, counts = np.unique(ends, axis=0, return_counts=True)
@@ -313,20 +316,47 @@ def build_fine_grid(walls, sector_edge_ofs, sector_edge_idx, sector_count, min_x
             continue
         if not closed:  # an open boundary can give odd parity anywhere to its left
             mixed[iy0 : iy1 + 1, ix0 : ix1 + 1] = True
+            level_bits[iy0 : iy1 + 1, ix0 : ix1 + 1] |= bits
             continue
+        # cells that an edge of this sector comes near
+        for x1, y1, x2, y2 in seg:
+            ex0 = max(int(np.floor((min(x1, x2) - GRID_PAD - min_x) / cell)), 0)
+            ex1 = min(int(np.floor((max(x1, x2) + GRID_PAD - min_x) / cell)), nx - 1)
+            ey0 = max(int(np.floor((min(y1, y2) - GRID_PAD - min_y) / cell)), 0)
+            ey1 = min(int(np.floor((max(y1, y2) + GRID_PAD - min_y) / cell)), ny - 1)
+            if ex1 < ex0 or ey1 < ey0:
+                continue
+            if ex0 == ex1 or ey0 == ey1 or x1 == x2 or y1 == y2:
+                near = np.ones((ey1 - ey0 + 1, ex1 - ex0 + 1), dtype=bool)
+            else:
+                # Liang-Barsky clip of the segment against every padded cell box of its bounding box
+                bx0 = (min_x + np.arange(ex0, ex1 + 1) * cell - GRID_PAD)[None, :]
+                by0 = (min_y + np.arange(ey0, ey1 + 1) * cell - GRID_PAD)[:, None]
+                bx1 = bx0 + cell + 2 * GRID_PAD
+                by1 = by0 + cell + 2 * GRID_PAD
+                dx, dy = x2 - x1, y2 - y1
+                tx_a, tx_b = (bx0 - x1) / dx, (bx1 - x1) / dx
+                ty_a, ty_b = (by0 - y1) / dy, (by1 - y1) / dy
+                t_in = np.maximum(np.maximum(np.minimum(tx_a, tx_b), np.minimum(ty_a, ty_b)), 0.0)
+                t_out = np.minimum(np.minimum(np.maximum(tx_a, tx_b), np.maximum(ty_a, ty_b)), 1.0)
+                near = t_in <= t_out
+            mixed[ey0 : ey1 + 1, ex0 : ex1 + 1] |= near
+            level_bits[ey0 : ey1 + 1, ex0 : ex1 + 1] |= np.where(near, bits, np.uint32(0))
+        # cells whose centre the sector contains
         cx = (min_x + (np.arange(ix0, ix1 + 1) + 0.5) * cell)[None, :, None]
         cy = (min_y + (np.arange(iy0, iy1 + 1) + 0.5) * cell)[:, None, None]
-        ex1, ey1, ex2, ey2 = (seg[:, k][None, None, :] for k in range(4))
-        crosses = (ey1 > cy) != (ey2 > cy)
+        ex1_, ey1_, ex2_, ey2_ = (seg[:, k][None, None, :] for k in range(4))
+        crosses = (ey1_ > cy) != (ey2_ > cy)
         with np.errstate(divide="ignore", invalid="ignore"):
-            crossing_x = ex1 + (cy - ey1) * (ex2 - ex1) / np.where(ey2 == ey1, 1.0, ey2 - ey1)
+            crossing_x = ex1_ + (cy - ey1_) * (ex2_ - ex1_) / np.where(ey2_ == ey1_, 1.0, ey2_ - ey1_)
         inside = (np.count_nonzero(crosses & (cx < crossing_x), axis=2) & 1).astype(bool)
         view_owners = owners[iy0 : iy1 + 1, ix0 : ix1 + 1]
         view_owner = owner[iy0 : iy1 + 1, ix0 : ix1 + 1]
-        view_owner[inside & (view_owners == 0)] = s
+        view_owner[inside & (view_owners == 0)] = np.uint32(s) | level_index
         view_owners += inside
+        level_bits[iy0 : iy1 + 1, ix0 : ix1 + 1] |= np.where(inside, bits, np.uint32(0))
     mixed |= owners > 1
-    owner[mixed] = FINE_MIXED
+    owner[mixed] = (np.uint32(FINE_MIXED) | level_bits[mixed]) if masks_known else np.uint32(FINE_UNKNOWN)
     return dict(fine_nx=nx, fine_ny=ny, fine_cell=float(cell), fine_sector=np.ascontiguousarray(owner.reshape(-1)))
 
 

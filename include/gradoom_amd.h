@@ -92,8 +92,12 @@ typedef struct gd_map_desc {
                                         cell lies inside that sector (no edge list, no crossing test) */
     const int32_t *grid_item_edge_ofs;/* [items+1] -> grid_item_edges */
     const int32_t *grid_item_edges;  /* linedef ids */
-    const uint16_t *fine_sector;     /* [fine_ny*fine_nx] the one sector containing the whole cell, 0xFFFE =
-                                        outside every sector, 0xFFFF = undecided (run the crossing test) */
+    const uint32_t *fine_sector;     /* [fine_ny*fine_nx] bits 31..30: 0 = bits 0..15 name the one sector that
+                                        contains the whole cell, bits 16..19 / 20..23 its index in floor_levels /
+                                        ceil_levels (15 = not recorded); 1 = outside every sector; 2 = undecided
+                                        (run the crossing test), bits 0..14 / 15..29 flag the floor_levels /
+                                        ceil_levels entries that can win in the cell; 3 = undecided, levels
+                                        unknown.  grid_cell must be 8 * fine_cell. */
     const float *floor_levels;       /* [floor_level_count] distinct floor heights, descending */
     const float *ceil_levels;        /* [ceil_level_count] distinct ceiling heights, ascending */
 

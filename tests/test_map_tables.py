@@ -104,8 +104,9 @@ def test_fine_raster_agrees_with_the_crossing_test(fixture):
     fx = np.floor((px - np.float32(tables["grid_min_x"])) * inv)
     fy = np.floor((py - np.float32(tables["grid_min_y"])) * inv)
     inside_raster = (fx >= 0) & (fx < tables["fine_nx"]) & (fy >= 0) & (fy < tables["fine_ny"])
-    entry = np.full(count, 0xFFFF, dtype=np.int64)
+    entry = np.full(count, 0xC0000000, dtype=np.int64)
     entry[inside_raster] = tables["fine_sector"][fy[inside_raster].astype(int) * tables["fine_nx"] + fx[inside_raster].astype(int)]
+    kind = entry >> 30
     parity = np.zeros((count, S), dtype=bool)
     for s in range(S):
         e = walls[tables["sector_edge_idx"][tables["sector_edge_ofs"][s] : tables["sector_edge_ofs"][s + 1]]]
@@ -115,10 +116,24 @@ def test_fine_raster_agrees_with_the_crossing_test(fixture):
         crossing = x1 + (py[:, None] - y1) * (x2 - x1) / safe
         assert crossing.dtype == np.float32
         parity[:, s] = np.count_nonzero(((y1 > py[:, None]) != (y2 > py[:, None])) & (px[:, None] < crossing), axis=1) & 1
-    decided = entry != 0xFFFF
+    decided = kind <= 1
     assert decided.mean() > 0.3  # the raster must actually decide a good share of the points
-    empty = entry == 0xFFFE
+    empty = kind == 1
     assert not parity[empty].any()
-    owned = decided & ~empty
+    owned = kind == 0
     assert np.array_equal(parity[owned].sum(axis=1), np.ones(owned.sum(), dtype=int))
-    assert np.array_equal(parity[owned].argmax(axis=1), entry[owned])
+    assert np.array_equal(parity[owned].argmax(axis=1), entry[owned] & 0xFFFF)
+    sector_of = entry[owned] & 0xFFFF
+    assert np.array_equal(tables["floor_levels"][(entry[owned] >> 16) & 15], tables["sector_heights"][sector_of, 0])
+    assert np.array_equal(tables["ceil_levels"][(entry[owned] >> 20) & 15], tables["sector_heights"][sector_of, 1])
+    # undecided cells with level masks: every sector that contains the point has its levels flagged
+    heights = tables["sector_heights"]
+    floor_index = {float(v): k for k, v in enumerate(tables["floor_levels"])}
+    ceil_index = {float(v): k for k, v in enumerate(tables["ceil_levels"])}
+    masked = np.nonzero(kind == 2)[0]
+    assert len(masked) > 100
+    for i in masked:
+        for s in np.nonzero(parity[i])[0]:
+            assert (entry[i] >> floor_index[float(heights[s, 0])]) & 1
+            assert (entry[i] >> (15 + ceil_index[float(heights[s, 1])])) & 1
+    assert tables["grid_cell"] == 8 * tables["fine_cell"]
