@@ -1629,22 +1629,29 @@ __device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const Col
     }
 }
 
-// One wavefront per (lane, 64-column strip): strips of one lane share nothing but read-only
-// tables, so each is its own work-group and leaves the CU as soon as its own columns finish.
-__global__ void __launch_bounds__(64) wall_columns_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
+// One wavefront per (lane, 64-column strip).  Strips share nothing but read-only tables; a
+// work-group is WALL_STRIPS_PER_GROUP consecutive strips only so that the LDS copies of those
+// tables are paid once per group rather than once per wavefront (which would cap the CU at a
+// couple of wavefronts per SIMD).  After the staging barrier the wavefronts never meet again.
+#define WALL_STRIPS_PER_GROUP 2
+__global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amdgpu_waves_per_eu(4, 4))) wall_columns_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
     const gd_map_desc *m = &dm.d;
-    const int local = blockIdx.y;
-    if (local >= lane_count) return;
-    __shared__ LaneCtx lane_ctx;
+    __shared__ LaneCtx lane_ctxs[WALL_STRIPS_PER_GROUP];
     __shared__ unsigned char colormap_lds[32 * 256];   // shade rows 0..31 are the only ones indexed
     __shared__ float4 sector_lds[LDS_SECTORS];
     __shared__ unsigned char tex_lds[LDS_TEXTURES];
+    const int wave_in_group = threadIdx.x >> 6;
+    const int strip_index = blockIdx.x * WALL_STRIPS_PER_GROUP + wave_in_group;
+    const int local = strip_index / (SW / 64);
+    const bool live = local < lane_count;
     Tables tb;
     stage_tables(m, sector_lds, tex_lds, tb);
-    if (threadIdx.x == 0) lane_ctx = sc.ctx[local];
-    for (int k = threadIdx.x; k < 32 * 256 / 4; k += 64) reinterpret_cast<unsigned int *>(colormap_lds)[k] = reinterpret_cast<const unsigned int *>(m->colormap)[k];
+    if ((threadIdx.x & 63) == 0 && live) lane_ctxs[wave_in_group] = sc.ctx[local];
+    for (int k = threadIdx.x; k < 32 * 256 / 4; k += blockDim.x) reinterpret_cast<unsigned int *>(colormap_lds)[k] = reinterpret_cast<const unsigned int *>(m->colormap)[k];
     __syncthreads();
-    const int x = blockIdx.x * 64 + threadIdx.x;
+    if (!live) return;
+    const LaneCtx &lane_ctx = lane_ctxs[wave_in_group];
+    const int x = (strip_index - local * (SW / 64)) * 64 + (threadIdx.x & 63);
     bool window_dirty = false;
     ColumnCtx cc;
     cc.tb = &tb; cc.m = m; cc.mv.m = m; cc.c = &lane_ctx;
@@ -1971,6 +1978,11 @@ int fail(int code, const std::string &message) { g_error = message; return code;
 
 }  // namespace
 
+// The flat kernels (bound by the vector ALU) and the wall kernels (bound by memory latency) of a
+// chunk are independent until plane shading, so the flats run on a side stream forked from the
+// caller's stream and joined back before plane shading.  (Cutting a batch into smaller chunks
+// pipelined over several streams measured slower: the wall traversal has a long per-wavefront
+// critical path and wants as many lanes per launch as possible.)
 struct gd_renderer {
     DeviceMap dm;
     Scratch sc;
@@ -1978,6 +1990,9 @@ struct gd_renderer {
     std::vector<void *> allocations;
     hipEvent_t events[16];
     bool events_ready;
+    hipStream_t side_stream;
+    hipEvent_t fork_event, flat_event;
+    bool side_ready;
 };
 
 namespace {
@@ -2023,29 +2038,39 @@ void build_fine_tables(std::vector<i64> &sine, std::vector<i64> &tangent) {
 
 const int STAGE_COUNT = 8;
 
-int launch_chunk(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_out *out, int base, int count, hipStream_t stream, bool timed) {
+// `side` (optional) is a second stream for the flat kernels of this chunk.
+int launch_chunk(gd_renderer *r, Scratch &sc, const gd_lanes_desc *lanes, const gd_frame_out *out, int base, int count, hipStream_t stream, hipStream_t side, bool timed) {
     const gd_map_desc &m = r->dm.d;
     unsigned char *frame_base;
     size_t frame_stride = (size_t)GD_SCREEN_HEIGHT * SW;
     if (out->indexed) frame_base = out->indexed + (size_t)base * frame_stride;
-    else frame_base = r->sc.frame;
+    else frame_base = sc.frame;
     int stage = 0;
     auto mark = [&]() { if (timed) (void)hipEventRecord(r->events[stage], stream); ++stage; };
+    // Stage timing needs the kernels one after another; otherwise the flats run on the side stream.
+    const bool overlap = !timed && side != nullptr;
+    hipStream_t flat_stream = overlap ? side : stream;
     mark();
-    hipLaunchKernelGGL(lane_setup_kernel, dim3((count + 63) / 64), dim3(64), 0, stream, r->dm, *lanes, base, count, r->sc);
-    hipLaunchKernelGGL(wall_setup_kernel, dim3((m.wall_count + 127) / 128, count), dim3(128), 0, stream, r->dm, count, r->sc);
+    hipLaunchKernelGGL(lane_setup_kernel, dim3((count + 63) / 64), dim3(64), 0, stream, r->dm, *lanes, base, count, sc);
+    if (overlap) {
+        HIP_TRY(hipEventRecord(r->fork_event, stream));
+        HIP_TRY(hipStreamWaitEvent(side, r->fork_event, 0));
+    }
+    hipLaunchKernelGGL(wall_setup_kernel, dim3((m.wall_count + 127) / 128, count), dim3(128), 0, stream, r->dm, count, sc);
     mark();
-    hipLaunchKernelGGL(flat_select_kernel, dim3((VH * SW + 255) / 256, count), dim3(256), 0, stream, r->dm, *lanes, base, count, r->sc);
+    hipLaunchKernelGGL(flat_select_kernel, dim3((VH * SW + 255) / 256, count), dim3(256), 0, flat_stream, r->dm, *lanes, base, count, sc);
     mark();
-    hipLaunchKernelGGL(flat_finish_kernel, dim3(count), dim3(SW), 0, stream, r->dm, count, r->sc, frame_base, frame_stride);
+    hipLaunchKernelGGL(flat_finish_kernel, dim3(count), dim3(SW), 0, flat_stream, r->dm, count, sc, frame_base, frame_stride);
     mark();
-    hipLaunchKernelGGL(wall_columns_kernel, dim3(SW / 64, count), dim3(64), 0, stream, r->dm, count, r->sc, frame_base, frame_stride);
+    if (overlap) HIP_TRY(hipEventRecord(r->flat_event, side));
+    hipLaunchKernelGGL(wall_columns_kernel, dim3((count * (SW / 64) + WALL_STRIPS_PER_GROUP - 1) / WALL_STRIPS_PER_GROUP), dim3(64 * WALL_STRIPS_PER_GROUP), 0, stream, r->dm, count, sc, frame_base, frame_stride);
     mark();
-    hipLaunchKernelGGL(plane_shade_kernel, dim3((VH * SW + 255) / 256, count), dim3(256), 0, stream, r->dm, count, r->sc, frame_base, frame_stride);
+    if (overlap) HIP_TRY(hipStreamWaitEvent(stream, r->flat_event, 0));
+    hipLaunchKernelGGL(plane_shade_kernel, dim3((VH * SW + 255) / 256, count), dim3(256), 0, stream, r->dm, count, sc, frame_base, frame_stride);
     mark();
     if (lanes->sprite_slots > 0 && lanes->sprite_x) {
         size_t shared = (size_t)lanes->sprite_slots * sizeof(SpriteRec);
-        hipLaunchKernelGGL(sprite_columns_kernel, dim3(count), dim3(SW), shared, stream, r->dm, *lanes, base, count, r->sc, frame_base, frame_stride);
+        hipLaunchKernelGGL(sprite_columns_kernel, dim3(count), dim3(SW), shared, stream, r->dm, *lanes, base, count, sc, frame_base, frame_stride);
     }
     mark();
     if (out->obs || out->frames) {
@@ -2085,6 +2110,7 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     gd_renderer *r = new (std::nothrow) gd_renderer();
     if (!r) return fail(GD_E_ARG, "out of host memory");
     r->events_ready = false;
+    r->side_ready = false;
     std::memset(&r->sc, 0, sizeof(r->sc));
     r->dm.d = *h;
     gd_map_desc &d = r->dm.d;
@@ -2124,20 +2150,28 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     const int chunk = max_lanes < 4096 ? max_lanes : 4096;
     r->chunk_lanes = chunk;
     const size_t L = chunk, PX = (size_t)VH * SW;
-    if (rc == GD_OK) rc = scratch_alloc(r, L, &r->sc.ctx);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * W, &r->sc.rec);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * CAND_MAX * SW, &r->sc.cand);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * SW, &r->sc.cand_count);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &r->sc.flat_sector);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &r->sc.flat_flags);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &r->sc.meta);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &r->sc.clip_depth);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)GD_SCREEN_HEIGHT * SW, &r->sc.frame);
-    if (rc == GD_OK) rc = scratch_alloc(r, 1, &r->sc.status);
-    if (rc == GD_OK && hipMemset(r->sc.status, 0, sizeof(int)) != hipSuccess) rc = fail(GD_E_HIP, "hipMemset status");
+    Scratch &sc = r->sc;
+    if (rc == GD_OK) rc = scratch_alloc(r, L, &sc.ctx);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * W, &sc.rec);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * CAND_MAX * SW, &sc.cand);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * SW, &sc.cand_count);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.flat_sector);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.flat_flags);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.meta);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.clip_depth);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)GD_SCREEN_HEIGHT * SW, &sc.frame);
+    if (rc == GD_OK) rc = scratch_alloc(r, 1, &sc.status);
+    if (rc == GD_OK && hipMemset(sc.status, 0, sizeof(int)) != hipSuccess) rc = fail(GD_E_HIP, "hipMemset status");
     if (rc == GD_OK) {
         for (int i = 0; i < 16; ++i) if (hipEventCreate(&r->events[i]) != hipSuccess) rc = fail(GD_E_HIP, "hipEventCreate");
         r->events_ready = rc == GD_OK;
+    }
+    if (rc == GD_OK) {
+        // default priority, as every stream of this library
+        if (hipStreamCreateWithFlags(&r->side_stream, hipStreamNonBlocking) != hipSuccess) rc = fail(GD_E_HIP, "hipStreamCreateWithFlags");
+        else if (hipEventCreateWithFlags(&r->fork_event, hipEventDisableTiming) != hipSuccess) { (void)hipStreamDestroy(r->side_stream); rc = fail(GD_E_HIP, "hipEventCreateWithFlags"); }
+        else if (hipEventCreateWithFlags(&r->flat_event, hipEventDisableTiming) != hipSuccess) { (void)hipEventDestroy(r->fork_event); (void)hipStreamDestroy(r->side_stream); rc = fail(GD_E_HIP, "hipEventCreateWithFlags"); }
+        else r->side_ready = true;
     }
     if (rc != GD_OK) { std::string keep = g_error; gd_renderer_destroy(r); g_error = keep; return rc; }
     *out = r;
@@ -2146,6 +2180,7 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
 
 void gd_renderer_destroy(gd_renderer *r) {
     if (!r) return;
+    if (r->side_ready) { (void)hipStreamSynchronize(r->side_stream); (void)hipEventDestroy(r->fork_event); (void)hipEventDestroy(r->flat_event); (void)hipStreamDestroy(r->side_stream); }
     for (void *ptr : r->allocations) (void)hipFree(ptr);
     if (r->events_ready) for (int i = 0; i < 16; ++i) (void)hipEventDestroy(r->events[i]);
     delete r;
@@ -2168,9 +2203,10 @@ static int check_render_args(gd_renderer *r, const gd_lanes_desc *lanes, const g
 int gd_render(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_out *out, void *stream) {
     int rc = check_render_args(r, lanes, out);
     if (rc != GD_OK) return rc;
+    hipStream_t caller = static_cast<hipStream_t>(stream);
     for (int base = 0; base < lanes->lane_count; base += r->chunk_lanes) {
         int count = lanes->lane_count - base < r->chunk_lanes ? lanes->lane_count - base : r->chunk_lanes;
-        rc = launch_chunk(r, lanes, out, base, count, static_cast<hipStream_t>(stream), false);
+        rc = launch_chunk(r, r->sc, lanes, out, base, count, caller, r->side_ready ? r->side_stream : nullptr, false);
         if (rc != GD_OK) return rc;
     }
     return GD_OK;
@@ -2185,7 +2221,7 @@ int gd_render_timed(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_o
     for (int it = 0; it < launches; ++it) {
         for (int base = 0; base < lanes->lane_count; base += r->chunk_lanes) {
             int count = lanes->lane_count - base < r->chunk_lanes ? lanes->lane_count - base : r->chunk_lanes;
-            rc = launch_chunk(r, lanes, out, base, count, st, true);
+            rc = launch_chunk(r, r->sc, lanes, out, base, count, st, nullptr, true);
             if (rc != GD_OK) return rc;
             HIP_TRY(hipEventSynchronize(r->events[STAGE_COUNT - 1]));
             for (int s = 0; s + 1 < STAGE_COUNT; ++s) {

@@ -75,3 +75,25 @@ def test_observe_entry_point_matches_oracle(oracle):
         assert np.array_equal(obs.cpu().numpy(), expected_obs)
         assert np.array_equal(frames.cpu().numpy(), expected_frames)
     renderer.close()
+
+
+def test_chunked_batches_render_every_lane_like_the_golden():
+    # a renderer made for a few lanes given more than that renders chunk by chunk, the last one short
+    from gradoom_amd.renderer import HipRenderer, LaneState
+
+    meta, data, smap, tables = load_fixture("small_midtex_sprites")
+    base = lane_inputs(data)
+    count = meta["lanes"]
+    for max_lanes, total in ((4, 11), (16, 40)):
+        picks = np.arange(total) % count
+        arrays = {k: np.ascontiguousarray(v[picks]) for k, v in base.items()}
+        renderer = HipRenderer(smap, max_lanes, "cuda:0", cosine_correction=data["cosine_correction"], tables=tables)
+        lanes = LaneState.from_numpy(arrays, "cuda:0")
+        indexed = torch.zeros((total, 240, 320), dtype=torch.uint8, device="cuda:0")
+        for _ in range(2):  # the second frame reuses every working set
+            indexed.zero_()
+            renderer.render(lanes, indexed=indexed)
+            torch.cuda.synchronize()
+            assert renderer.status() == 0
+            assert np.array_equal(indexed.cpu().numpy(), data["indexed"][picks])
+        renderer.close()
