@@ -22,6 +22,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <map>
 #include <new>
 #include <string>
 #include <vector>
@@ -98,6 +99,11 @@ struct DeviceMap {  // device copy of gd_map_desc (device pointers) + fixed tabl
     const i64 *fine_sine;     // [8192]
     const i64 *fine_tangent;  // [4096]
     const float *cosine_correction;  // [320] cos(native_ray_offsets), supplied by the host
+    // Sectors grouped by plane level, floors (in floor_levels order) then ceilings: CSR over
+    // floor_level_count + ceil_level_count rows into level_boxes, one padded bounding box
+    // (x0, y0, x1, y1) per sector outside which no point tests inside that sector.
+    const int *level_box_ofs;
+    const float4 *level_boxes;
 };
 
 struct Scratch {    // per-chunk working memory, sized at create
@@ -111,6 +117,8 @@ struct Scratch {    // per-chunk working memory, sized at create
     float *clip_depth;     // [L,208,320]
     unsigned char *frame;  // [L,240,320] when the caller wants no indexed output
     int *status;           // [1] sticky overflow flags
+    float *level_reach;    // [L, floor levels + ceiling levels] lower bound of the distance from the
+                           // camera to any point inside a sector with that plane level
 };
 
 #define META_FILLED 0x80000000u   // an opaque wall tier owns the pixel
@@ -291,6 +299,26 @@ __device__ int sector_at(const gd_map_desc *m, float px, float py) {
             return item & ~GRID_ALWAYS_INSIDE;
     }
     return 0;
+}
+
+// Per lane and plane level: how far the camera is, at least, from every sector at that level.
+// A flat probe nearer than that cannot land in such a sector (engine.py:10981-11024 tests the
+// point against every sector; here the far ones are ruled out by their bounding boxes).
+__global__ void level_reach_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
+    const int local = blockIdx.x;
+    const int levels = dm.d.floor_level_count + dm.d.ceil_level_count;
+    if (local >= lane_count) return;
+    const float cx = lanes.x[lane_base + local], cy = lanes.y[lane_base + local];
+    for (int l = threadIdx.x; l < levels; l += blockDim.x) {
+        float reach = GD_INF;
+        for (int k = dm.level_box_ofs[l]; k < dm.level_box_ofs[l + 1]; ++k) {
+            const float4 box = dm.level_boxes[k];
+            float dx = fmaxf(fmaxf(box.x - cx, cx - box.z), 0.0f), dy = fmaxf(fmaxf(box.y - cy, cy - box.w), 0.0f);
+            reach = fminf(reach, sqrtf(dx * dx + dy * dy));
+        }
+        // margin: the probe point is camera + unit ray * distance in float32, far inside 0.1%
+        sc.level_reach[(size_t)local * levels + l] = reach * 0.999f - 0.5f;
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -566,6 +594,7 @@ __global__ void flat_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
     const int level_count = floor_uniform ? m->floor_level_count : m->ceil_level_count;
     const int mask_shift = floor_uniform ? 0 : FINE_MASK_LEVELS;
     const int index_shift = floor_uniform ? 16 : 20;
+    const float *reach = sc.level_reach + (size_t)local * (m->floor_level_count + m->ceil_level_count) + (floor_uniform ? 0 : m->floor_level_count);
     // cd = perpendicular / cc below is the hot division.  With y = RN(1 / cc), q = RN(p * y) is within
     // one ulp of p / cc, and RN(q + RN(p - cc * q) * y) is then the correctly rounded quotient
     // (Markstein's theorem; the inner product is exact in an FMA) as long as nothing over- or
@@ -581,12 +610,14 @@ __global__ void flat_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
         // the wavefront instead of one per level per lane); a level the plane cannot show gets -1
         const int mine = base + slot_in_wave;
         const float my_level = mine < level_count ? levels[mine] : 0.0f;
+        const float my_reach = mine < level_count ? reach[mine] : 0.0f;
         const float my_height = floor_uniform ? (c.view_z - my_level) : (my_level - c.view_z);
         const float my_perpendicular = (mine < level_count && my_height > 0) ? my_height * 192.0f / denom : -1.0f;
         const int chunk = level_count - base < 64 ? level_count - base : 64;
         for (int k = 0; k < chunk; ++k) {
             const float perpendicular = bcast(my_perpendicular, k);
             const float level = bcast(my_level, k);
+            const float nearest = bcast(my_reach, k);
             if (!(perpendicular > 0)) continue;              // the same in every lane
             float cd;
             if (cc_plain && perpendicular >= 1e-18f && perpendicular <= 1e18f) {
@@ -597,6 +628,7 @@ __global__ void flat_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
             }
             if (!(finitef(cd) && cd > 0)) continue;
             if (cd > best) { done = true; break; }           // later levels are at least this far
+            if (cd < nearest) continue;                      // every sector at this level is farther away
             float px = c.x + rc * cd, py = c.y + rs * cd;
             int cell;
             unsigned fine = fine_lookup(m, inv_fine, px, py, &cell);
@@ -2018,6 +2050,43 @@ int scratch_alloc(gd_renderer *r, size_t count, T **device) {
     return GD_OK;
 }
 
+// Bounding boxes of the sectors, grouped by plane level (floors first).  The box of a sector is
+// that of its edges padded by half a map unit; the even-odd test of engine.py:9598-9617 counts
+// edges to the right of the point, so a sector whose boundary is not a set of closed loops can
+// also test inside anywhere to the left of its edges and its box is open on that side.
+void build_level_boxes(const gd_map_desc *h, std::vector<int> &ofs, std::vector<float4> &boxes) {
+    const int S = h->sector_count;
+    std::vector<float4> sector_box(S);
+    std::vector<char> has_box(S, 0);
+    for (int s = 0; s < S; ++s) {
+        float x0 = GD_INF, y0 = GD_INF, x1 = -GD_INF, y1 = -GD_INF;
+        std::map<std::pair<float, float>, int> degree;
+        for (int k = h->sector_edge_ofs[s]; k < h->sector_edge_ofs[s + 1]; ++k) {
+            const float *w = h->walls + 4 * h->sector_edge_idx[k];
+            for (int e = 0; e < 2; ++e) {
+                float x = w[2 * e] + 0.0f, y = w[2 * e + 1] + 0.0f;
+                x0 = std::fmin(x0, x); x1 = std::fmax(x1, x); y0 = std::fmin(y0, y); y1 = std::fmax(y1, y);
+                ++degree[std::make_pair(x, y)];
+            }
+            has_box[s] = 1;
+        }
+        bool closed = true;
+        for (const auto &entry : degree) closed = closed && (entry.second % 2 == 0);
+        if (!closed) x0 = -GD_INF;
+        sector_box[s] = make_float4(x0 - 0.5f, y0 - 0.5f, x1 + 0.5f, y1 + 0.5f);
+    }
+    ofs.assign(1, 0);
+    for (int side = 0; side < 2; ++side) {
+        const float *levels = side == 0 ? h->floor_levels : h->ceil_levels;
+        const int count = side == 0 ? h->floor_level_count : h->ceil_level_count;
+        for (int l = 0; l < count; ++l) {
+            for (int s = 0; s < S; ++s)
+                if (has_box[s] && h->sector_heights[2 * s + side] == levels[l]) boxes.push_back(sector_box[s]);
+            ofs.push_back((int)boxes.size());
+        }
+    }
+}
+
 void build_fine_tables(std::vector<i64> &sine, std::vector<i64> &tangent) {
     // engine.py:309-328
     const double PI = 3.14159265358979323846;
@@ -2058,6 +2127,7 @@ int launch_chunk(gd_renderer *r, Scratch &sc, const gd_lanes_desc *lanes, const 
     }
     hipLaunchKernelGGL(wall_setup_kernel, dim3((m.wall_count + 127) / 128, count), dim3(128), 0, stream, r->dm, count, sc);
     mark();
+    hipLaunchKernelGGL(level_reach_kernel, dim3(count), dim3(64), 0, flat_stream, r->dm, *lanes, base, count, sc);
     hipLaunchKernelGGL(flat_select_kernel, dim3((VH * SW + 255) / 256, count), dim3(256), 0, flat_stream, r->dm, *lanes, base, count, sc);
     mark();
     hipLaunchKernelGGL(flat_finish_kernel, dim3(count), dim3(SW), 0, flat_stream, r->dm, count, sc, frame_base, frame_stride);
@@ -2146,6 +2216,13 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     if (rc == GD_OK) rc = upload(r, sine.data(), sine.size(), &r->dm.fine_sine);
     if (rc == GD_OK) rc = upload(r, tangent.data(), tangent.size(), &r->dm.fine_tangent);
     if (rc == GD_OK) rc = upload(r, cosine_correction, (size_t)SW, &r->dm.cosine_correction);
+    {
+        std::vector<int> box_ofs;
+        std::vector<float4> boxes;
+        build_level_boxes(h, box_ofs, boxes);
+        if (rc == GD_OK) rc = upload(r, box_ofs.data(), box_ofs.size(), &r->dm.level_box_ofs);
+        if (rc == GD_OK) rc = upload(r, boxes.data(), boxes.size(), &r->dm.level_boxes);
+    }
     // Working memory for one chunk of lanes; larger batches are rendered chunk by chunk.
     const int chunk = max_lanes < 4096 ? max_lanes : 4096;
     r->chunk_lanes = chunk;
@@ -2160,6 +2237,7 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.meta);
     if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.clip_depth);
     if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)GD_SCREEN_HEIGHT * SW, &sc.frame);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)(h->floor_level_count + h->ceil_level_count), &sc.level_reach);
     if (rc == GD_OK) rc = scratch_alloc(r, 1, &sc.status);
     if (rc == GD_OK && hipMemset(sc.status, 0, sizeof(int)) != hipSuccess) rc = fail(GD_E_HIP, "hipMemset status");
     if (rc == GD_OK) {
