@@ -104,6 +104,8 @@ struct DeviceMap {  // device copy of gd_map_desc (device pointers) + fixed tabl
     // (x0, y0, x1, y1) per sector outside which no point tests inside that sector.
     const int *level_box_ofs;
     const float4 *level_boxes;
+    const unsigned short *sector_level;  // [S] index of the floor in floor_levels | index of the ceiling in
+                                         // ceil_levels << 8; null when a level list is longer than PLANE_LEVELS
 };
 
 struct Scratch {    // per-chunk working memory, sized at create
@@ -119,7 +121,11 @@ struct Scratch {    // per-chunk working memory, sized at create
     int *status;           // [1] sticky overflow flags
     float *level_reach;    // [L, floor levels + ceiling levels] lower bound of the distance from the
                            // camera to any point inside a sector with that plane level
+    i64 *level_plane;      // [L, floor levels + ceiling levels, 2] plane height (16.16) and its visibility factor
+    i64 *row_slope;        // [L, 208] plane distance per unit of plane height on each view row
+    i64 *step_scale;       // [L, 2, 16] flat texture steps per column for every log2 texture size
 };
+#define PLANE_LEVELS 64    // level lists up to this long are shaded from the per-lane tables
 
 #define META_FILLED 0x80000000u   // an opaque wall tier owns the pixel
 #define META_FLOOR 0x40000000u    // the owning plane is a floor
@@ -301,13 +307,20 @@ __device__ int sector_at(const gd_map_desc *m, float px, float py) {
     return 0;
 }
 
-// Per lane and plane level: how far the camera is, at least, from every sector at that level.
-// A flat probe nearer than that cannot land in such a sector (engine.py:10981-11024 tests the
-// point against every sector; here the far ones are ruled out by their bounding boxes).
-__global__ void level_reach_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
+// Per-lane tables for the flat kernels, one block per lane (after lane_setup):
+//  * per plane level, how far the camera is, at least, from every sector at that level: a flat
+//    probe nearer than that cannot land in such a sector (engine.py:10981-11024 tests the point
+//    against every sector; here the far ones are ruled out by their bounding boxes);
+//  * per plane level, the fixed-point plane height and visibility factor (engine.py:10588-10600);
+//  * per view row, the plane distance slope (engine.py:10917-10931);
+//  * per log2 texture size, the per-column texture steps (engine.py:10895-10902).
+// The last three only depend on (lane, level), (lane, row) and (lane, size), so dividing once
+// here spares plane shading four 64-bit divisions per pixel.
+__global__ void lane_tables_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
     const int local = blockIdx.x;
-    const int levels = dm.d.floor_level_count + dm.d.ceil_level_count;
+    const int floors = dm.d.floor_level_count, levels = floors + dm.d.ceil_level_count;
     if (local >= lane_count) return;
+    const LaneCtx &c = sc.ctx[local];
     const float cx = lanes.x[lane_base + local], cy = lanes.y[lane_base + local];
     for (int l = threadIdx.x; l < levels; l += blockDim.x) {
         float reach = GD_INF;
@@ -318,6 +331,23 @@ __global__ void level_reach_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
         }
         // margin: the probe point is camera + unit ray * distance in float32, far inside 0.1%
         sc.level_reach[(size_t)local * levels + l] = reach * 0.999f - 0.5f;
+        const float plane_height = l < floors ? (c.view_z - dm.d.floor_levels[l]) : (dm.d.ceil_levels[l - floors] - c.view_z);
+        const i64 plane_height_fixed = round_to_i64(plane_height * 65536.0f);
+        sc.level_plane[((size_t)local * levels + l) * 2] = plane_height_fixed;
+        sc.level_plane[((size_t)local * levels + l) * 2 + 1] = min64(tdiv(FLOOR_VISIBILITY_FIXED << 16, max64(plane_height_fixed, 1)), (1LL << 31) - 1);
+    }
+    for (int py = threadIdx.x; py < VH; py += blockDim.x) {
+        i64 center_row = c.center_fixed >> 16;
+        i64 pixel_y_fixed = (i64)py * FIXED_UNIT;
+        i64 den = (py < center_row) ? (c.center_fixed - pixel_y_fixed - FIXED_UNIT / 2) : (pixel_y_fixed - c.center_fixed + FIXED_UNIT / 2);
+        den = max64(den, 1);
+        bool overflow = den <= (FOCAL_Y_FIXED >> 15);
+        i64 yslope = tdiv(FOCAL_Y_FIXED << 16, den);
+        sc.row_slope[(size_t)local * VH + py] = overflow ? (1LL << 31) - 1 : yslope;
+    }
+    for (int k = threadIdx.x; k < 32; k += blockDim.x) {
+        const i64 basis = k < 16 ? c.vsin : c.vcos;
+        sc.step_scale[(size_t)local * 32 + k] = tdiv(shl64(basis, 32 - (k & 15)), FOCAL_X_FIXED);
     }
 }
 
@@ -741,6 +771,41 @@ __device__ __forceinline__ unsigned char flat_pixel(const Tables &tb, const unsi
     unsigned char index = m->tex_atlas[((size_t)texture * m->tex_max_h + v) * m->tex_max_w + u];
     float light = tb.light(sector) + (float)(c.flash_light * 16);
     return plane_colormap(colormap, c, index, light, plane_height, py);
+}
+
+// flat_pixel with every division looked up: the lane's per-level, per-row and per-size tables
+// hold exactly the quotients flat_texture_coordinates and plane_colormap would compute, and a
+// product with a power-of-two texture scale is a shift.
+struct LaneTables {
+    const i64 *level_plane;   // this lane's [levels][2]
+    const i64 *step_scale;    // this lane's [2][16]
+    int floors;
+};
+__device__ __forceinline__ unsigned char flat_pixel_tabled(const Tables &tb, const unsigned char *colormap, const LaneCtx &c, const LaneTables &lt,
+                                                           i64 yslope, int level_index, int sector, bool is_floor, int px, int py) {
+    const gd_map_desc *m = tb.m;
+    const int texture = is_floor ? tb.floor_tex(sector) : tb.ceil_tex(sector);
+    const int width_bits = tb.width_bits(texture), height_bits = tb.height_bits(texture);
+    const i64 *plane = lt.level_plane + 2 * (is_floor ? level_index : lt.floors + level_index);
+    const i64 plane_height_fixed = plane[0], glob = plane[1];
+    const i64 xstep_scale = lt.step_scale[width_bits], ystep_scale = lt.step_scale[16 + height_bits];
+    const i64 flat_column = (i64)px - (SW / 2 - 1);
+    const i64 basexfrac = (shl64(c.vcos, 32 - width_bits) >> 16) + mul64(flat_column, xstep_scale);
+    const i64 baseyfrac = (shl64(-c.vsin, 32 - height_bits) >> 16) + mul64(flat_column, ystep_scale);
+    const i64 pviewx = shl64(c.view_x_fixed, 32 - width_bits) >> 16;
+    const i64 pviewy = shl64(-c.view_y_fixed, 32 - height_bits) >> 16;
+    const i64 distance = mul64(plane_height_fixed, yslope) >> 16;
+    const i64 xfrac = ((mul64(distance, basexfrac) >> 16) + pviewx) & UINT32_MASK;
+    const i64 yfrac = ((mul64(distance, baseyfrac) >> 16) + pviewy) & UINT32_MASK;
+    const i64 u = xfrac >> (32 - width_bits), v = yfrac >> (32 - height_bits);
+    const unsigned char index = m->tex_atlas[((size_t)texture * m->tex_max_h + v) * m->tex_max_w + u];
+    const float light = tb.light(sector) + (float)(c.flash_light * 16);
+    i64 row = c.center_fixed - (i64)py * FIXED_UNIT;
+    if (row < 0) row = -row;
+    const i64 visibility = min64(mul64(glob, row) >> 16, 24 * FIXED_UNIT);
+    const i64 plane_shade = 64 * FIXED_UNIT - ((i64)light + 12) * (FIXED_UNIT / 4);
+    const i64 shade = clampi((plane_shade - visibility) >> 16, 0, 31);
+    return colormap[shade * 256 + index];
 }
 
 // Visplane continuity repair and shading for one lane (engine.py:11026-11171).
@@ -1777,38 +1842,58 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
 // one, the sector the per-pixel plane rays selected (engine.py:11145-11163).  Doing both here
 // shades every pixel once, in a kernel light enough to run at full occupancy.
 // ---------------------------------------------------------------------------------------------
+#define SHADE_TILES 13   // 256-pixel tiles per block: 260 tiles per view = 20 blocks per lane
 __global__ void __launch_bounds__(256) plane_shade_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
     const gd_map_desc *m = &dm.d;
     __shared__ float4 sector_lds[LDS_SECTORS];
+    __shared__ unsigned short sector_level_lds[LDS_SECTORS];
     __shared__ unsigned char tex_lds[LDS_TEXTURES];
     __shared__ unsigned char colormap_lds[32 * 256];
+    __shared__ i64 level_plane_lds[2 * PLANE_LEVELS * 2];
+    __shared__ i64 step_scale_lds[32];
+    const int local = blockIdx.y;
+    if (local >= lane_count) return;     // uniform over the block
     Tables tb;
     stage_tables(m, sector_lds, tex_lds, tb);
     for (int k = threadIdx.x; k < 32 * 256 / 4; k += blockDim.x) reinterpret_cast<unsigned int *>(colormap_lds)[k] = reinterpret_cast<const unsigned int *>(m->colormap)[k];
+    const int floors = m->floor_level_count, levels = floors + m->ceil_level_count;
+    const bool tabled = dm.sector_level != nullptr;   // implies both level lists fit PLANE_LEVELS
+    if (tabled) {
+        for (int s = threadIdx.x; s < tb.sector_cached; s += blockDim.x) sector_level_lds[s] = dm.sector_level[s];
+        for (int k = threadIdx.x; k < 2 * levels; k += blockDim.x) level_plane_lds[k] = sc.level_plane[(size_t)local * levels * 2 + k];
+        if (threadIdx.x < 32) step_scale_lds[threadIdx.x] = sc.step_scale[(size_t)local * 32 + threadIdx.x];
+    }
     __syncthreads();
-    const int local = blockIdx.y;
-    const int pixel = blockIdx.x * blockDim.x + threadIdx.x;
-    if (local >= lane_count || pixel >= VH * SW) return;
-    const int y = pixel / SW, x = pixel - y * SW;
+    LaneTables lt; lt.level_plane = level_plane_lds; lt.step_scale = step_scale_lds; lt.floors = floors;
     const LaneCtx &c = sc.ctx[local];
-    const size_t i = (size_t)local * VH * SW + pixel;
-    const unsigned int meta = sc.meta[i];
-    if (meta & META_FILLED) return;
-    const int ps = (int)((meta >> META_SECTOR_SHIFT) & META_SECTOR_MASK) - 1;
     unsigned char *frame = frame_base + (size_t)local * frame_stride;
-    if (ps >= 0) {
-        const bool is_floor = meta & META_FLOOR;
-        if (!(meta & META_MASKED)) frame[pixel] = flat_pixel(tb, colormap_lds, c, ps, is_floor, x, y);
+    for (int tile = 0; tile < SHADE_TILES; ++tile) {
+        const int pixel = (blockIdx.x * SHADE_TILES + tile) * 256 + threadIdx.x;
+        if (pixel >= VH * SW) break;
+        const int y = pixel / SW, x = pixel - y * SW;
+        const size_t i = (size_t)local * VH * SW + pixel;
+        const unsigned int meta = sc.meta[i];
+        if (meta & META_FILLED) continue;
+        const int ps = (int)((meta >> META_SECTOR_SHIFT) & META_SECTOR_MASK) - 1;
+        const bool claimed = ps >= 0;
+        const bool is_floor = claimed ? (meta & META_FLOOR) != 0 : ((float)y - flat_center(c)) > 0;
+        const int sector = claimed ? ps : (int)sc.flat_sector[i];
+        if (!(meta & META_MASKED)) {
+            if (tabled) {
+                const unsigned short pair = sector < tb.sector_cached ? sector_level_lds[sector] : dm.sector_level[sector];
+                frame[pixel] = flat_pixel_tabled(tb, colormap_lds, c, lt, sc.row_slope[(size_t)local * VH + y], is_floor ? (pair & 0xFF) : (pair >> 8),
+                                                 sector, is_floor, x, y);
+            } else {
+                frame[pixel] = flat_pixel(tb, colormap_lds, c, sector, is_floor, x, y);
+            }
+        }
         // plane fallback occluder for sprites where the flat ray was unresolved (engine.py:13417-13422)
-        if ((sc.flat_flags[i] & 1) && !finitef(sc.clip_depth[i])) {
+        if (claimed && (sc.flat_flags[i] & 1) && !finitef(sc.clip_depth[i])) {
             const float flat_center_px = (103.0f + c.pitch_offset) + 0.5f;
             float plane_height = is_floor ? (c.view_z - tb.floor_h(ps)) : (tb.ceil_h(ps) - c.view_z);
             float plane_denominator = fmaxf(fabsf((float)y - flat_center_px), 0.5f);
             sc.clip_depth[i] = plane_height * 192.0f / plane_denominator;
         }
-    } else if (!(meta & META_MASKED)) {
-        const bool is_floor = ((float)y - flat_center(c)) > 0;
-        frame[pixel] = flat_pixel(tb, colormap_lds, c, sc.flat_sector[i], is_floor, x, y);
     }
 }
 
@@ -2127,7 +2212,7 @@ int launch_chunk(gd_renderer *r, Scratch &sc, const gd_lanes_desc *lanes, const 
     }
     hipLaunchKernelGGL(wall_setup_kernel, dim3((m.wall_count + 127) / 128, count), dim3(128), 0, stream, r->dm, count, sc);
     mark();
-    hipLaunchKernelGGL(level_reach_kernel, dim3(count), dim3(64), 0, flat_stream, r->dm, *lanes, base, count, sc);
+    hipLaunchKernelGGL(lane_tables_kernel, dim3(count), dim3(256), 0, flat_stream, r->dm, *lanes, base, count, sc);
     hipLaunchKernelGGL(flat_select_kernel, dim3((VH * SW + 255) / 256, count), dim3(256), 0, flat_stream, r->dm, *lanes, base, count, sc);
     mark();
     hipLaunchKernelGGL(flat_finish_kernel, dim3(count), dim3(SW), 0, flat_stream, r->dm, count, sc, frame_base, frame_stride);
@@ -2136,7 +2221,7 @@ int launch_chunk(gd_renderer *r, Scratch &sc, const gd_lanes_desc *lanes, const 
     hipLaunchKernelGGL(wall_columns_kernel, dim3((count * (SW / 64) + WALL_STRIPS_PER_GROUP - 1) / WALL_STRIPS_PER_GROUP), dim3(64 * WALL_STRIPS_PER_GROUP), 0, stream, r->dm, count, sc, frame_base, frame_stride);
     mark();
     if (overlap) HIP_TRY(hipStreamWaitEvent(stream, r->flat_event, 0));
-    hipLaunchKernelGGL(plane_shade_kernel, dim3((VH * SW + 255) / 256, count), dim3(256), 0, stream, r->dm, count, sc, frame_base, frame_stride);
+    hipLaunchKernelGGL(plane_shade_kernel, dim3(((VH * SW + 255) / 256 + SHADE_TILES - 1) / SHADE_TILES, count), dim3(256), 0, stream, r->dm, count, sc, frame_base, frame_stride);
     mark();
     if (lanes->sprite_slots > 0 && lanes->sprite_x) {
         size_t shared = (size_t)lanes->sprite_slots * sizeof(SpriteRec);
@@ -2222,6 +2307,20 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
         build_level_boxes(h, box_ofs, boxes);
         if (rc == GD_OK) rc = upload(r, box_ofs.data(), box_ofs.size(), &r->dm.level_box_ofs);
         if (rc == GD_OK) rc = upload(r, boxes.data(), boxes.size(), &r->dm.level_boxes);
+        r->dm.sector_level = nullptr;
+        if (h->floor_level_count <= PLANE_LEVELS && h->ceil_level_count <= PLANE_LEVELS) {
+            std::vector<unsigned short> pairs(S, 0);
+            bool listed = true;
+            for (size_t s = 0; s < S; ++s) {
+                int fi = -1, ci = -1;
+                for (int l = 0; l < h->floor_level_count; ++l) if (h->floor_levels[l] == h->sector_heights[2 * s]) fi = l;
+                for (int l = 0; l < h->ceil_level_count; ++l) if (h->ceil_levels[l] == h->sector_heights[2 * s + 1]) ci = l;
+                listed = listed && fi >= 0 && ci >= 0;
+                pairs[s] = (unsigned short)((fi & 0xFF) | ((ci & 0xFF) << 8));
+            }
+            // a sector whose height is missing from the level lists keeps the per-pixel divisions
+            if (listed && rc == GD_OK) rc = upload(r, pairs.data(), pairs.size(), &r->dm.sector_level);
+        }
     }
     // Working memory for one chunk of lanes; larger batches are rendered chunk by chunk.
     const int chunk = max_lanes < 4096 ? max_lanes : 4096;
@@ -2238,6 +2337,9 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.clip_depth);
     if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)GD_SCREEN_HEIGHT * SW, &sc.frame);
     if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)(h->floor_level_count + h->ceil_level_count), &sc.level_reach);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)(h->floor_level_count + h->ceil_level_count) * 2, &sc.level_plane);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)VH, &sc.row_slope);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * 32, &sc.step_scale);
     if (rc == GD_OK) rc = scratch_alloc(r, 1, &sc.status);
     if (rc == GD_OK && hipMemset(sc.status, 0, sizeof(int)) != hipSuccess) rc = fail(GD_E_HIP, "hipMemset status");
     if (rc == GD_OK) {
