@@ -104,6 +104,7 @@ struct DeviceMap {  // device copy of gd_map_desc (device pointers) + fixed tabl
     // (x0, y0, x1, y1) per sector outside which no point tests inside that sector.
     const int *level_box_ofs;
     const float4 *level_boxes;
+    const int *wall_blocking_slot;       // [W] position of the linedef in blocking_walls, -1 when it does not block
     const unsigned short *sector_level;  // [S] index of the floor in floor_levels | index of the ceiling in
                                          // ceil_levels << 8; null when a level list is longer than PLANE_LEVELS
 };
@@ -118,6 +119,8 @@ struct Scratch {    // per-chunk working memory, sized at create
     unsigned int *meta;    // [L,208,320] filled | floor | plane_sector+1 | clip_wall+1
     float *clip_depth;     // [L,208,320]
     unsigned char *frame;  // [L,240,320] when the caller wants no indexed output
+    u64 *block_hit;        // [L,320] nearest blocking linedef of the column ray: float bits of the distance << 32 |
+                           // slot in blocking_walls, all ones when no ray hits (engine.py:10534-10557)
     int *status;           // [1] sticky overflow flags
     float *level_reach;    // [L, floor levels + ceiling levels] lower bound of the distance from the
                            // camera to any point inside a sector with that plane level
@@ -389,7 +392,7 @@ __global__ void lane_setup_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_ba
     c.sector = sector_at(&dm.d, c.x, c.y);
     c.pad = 0;
     sc.ctx[local] = c;
-    for (int x = 0; x < SW; ++x) sc.cand_count[(size_t)local * SW + x] = 0;
+    for (int x = 0; x < SW; ++x) { sc.cand_count[(size_t)local * SW + x] = 0; sc.block_hit[(size_t)local * SW + x] = ~0ULL; }
 }
 
 __device__ __forceinline__ void ray_direction(const LaneCtx &c, int x, float *rx, float *ry) {
@@ -496,6 +499,8 @@ __global__ void __launch_bounds__(128) wall_setup_kernel(DeviceMap dm, int lane_
         }
     }
     if (!live) { scan_lo = 1; scan_hi = 0; }
+    const int blocking_slot = dm.wall_blocking_slot[w];
+    u64 *block_hits = sc.block_hit + (size_t)local * SW;
     int first = 0, last = SW - 1; bool any = false;
     float numer_d = offx * segy - offy * segx;
     for (u64 pending = __ballot(scan_lo <= scan_hi); pending; pending &= pending - 1) {
@@ -503,6 +508,7 @@ __global__ void __launch_bounds__(128) wall_setup_kernel(DeviceMap dm, int lane_
         const float b_segx = bcast(segx, owner), b_segy = bcast(segy, owner);
         const float b_offx = bcast(offx, owner), b_offy = bcast(offy, owner), b_numer = bcast(numer_d, owner);
         const int b_lo = bcast(scan_lo, owner), b_hi = bcast(scan_hi, owner);
+        const int b_block = bcast(blocking_slot, owner);
         int hit_first = SW, hit_last = -1;
         for (int x0 = b_lo; x0 <= b_hi; x0 += 64) {
             const int x = x0 + slot_in_wave;
@@ -513,6 +519,8 @@ __global__ void __launch_bounds__(128) wall_setup_kernel(DeviceMap dm, int lane_
             float d = b_numer / safe;
             float a = (b_offx * ry - b_offy * rx) / safe;
             bool g = x <= b_hi && ok && (d > 0) && (a >= 0) && (a <= 1);
+            // the sprite pass wants the nearest blocking linedef each column ray hits, lowest slot on ties
+            if (g && b_block >= 0) atomicMin(&block_hits[x], ((u64)__float_as_uint(d) << 32) | (u64)(unsigned)b_block);
             const u64 hits = __ballot(g);
             if (hits) {
                 if (hit_last < 0) hit_first = x0 + __ffsll((long long)hits) - 1;
@@ -1948,21 +1956,10 @@ __global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lan
     unsigned char *frame = frame_base + (size_t)local * frame_stride;
     const unsigned int *meta = sc.meta + (size_t)local * VH * SW;
     const float *clip_depth = sc.clip_depth + (size_t)local * VH * SW;
-    // nearest blocking linedef of this column (engine.py:10534-10557)
-    float rx, ry; ray_direction(L, x, &rx, &ry);
-    float best = GD_INF; int slot = 0;
-    for (int b = 0; b < m->blocking_count; ++b) {
-        const float4 wl = *reinterpret_cast<const float4 *>(m->walls + 4 * m->blocking_walls[b]);
-        float segx = wl.z - wl.x, segy = wl.w - wl.y;
-        float offx = wl.x - L.x, offy = wl.y - L.y;
-        float den = rx * segy - ry * segx;
-        bool ok = fabsf(den) >= 1e-6f;
-        float safe = ok ? den : 1.0f;
-        float d = (offx * segy - offy * segx) / safe;
-        float a = (offx * ry - offy * rx) / safe;
-        bool valid = ok && (d > 0) && (a >= 0) && (a <= 1);
-        if (valid && d < best) { best = d; slot = b; }
-    }
+    // nearest blocking linedef of this column (engine.py:10534-10557), gathered by wall_setup
+    const u64 hit = sc.block_hit[(size_t)local * SW + x];
+    float best = hit == ~0ULL ? GD_INF : __uint_as_float((unsigned)(hit >> 32));
+    int slot = finitef(best) ? (int)(hit & 0xFFFFFFFFu) : 0;
     float wall_distance = fminf(fmaxf(best, 1.0f), 4096.0f);
     int bw = m->blocking_count ? m->blocking_walls[slot] : 0;
     const WallRec &bg = recs[bw];
@@ -2307,6 +2304,13 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
         build_level_boxes(h, box_ofs, boxes);
         if (rc == GD_OK) rc = upload(r, box_ofs.data(), box_ofs.size(), &r->dm.level_box_ofs);
         if (rc == GD_OK) rc = upload(r, boxes.data(), boxes.size(), &r->dm.level_boxes);
+        std::vector<int> blocking_slot(W, -1);
+        for (int b = 0; b < h->blocking_count; ++b) {
+            const int w = h->blocking_walls[b];
+            if (w < 0 || (size_t)w >= W) { if (rc == GD_OK) rc = fail(GD_E_ARG, "blocking_walls holds a linedef index out of range"); continue; }
+            if (blocking_slot[w] < 0) blocking_slot[w] = b;   // the first slot wins ties, like the scan it replaces
+        }
+        if (rc == GD_OK) rc = upload(r, blocking_slot.data(), blocking_slot.size(), &r->dm.wall_blocking_slot);
         r->dm.sector_level = nullptr;
         if (h->floor_level_count <= PLANE_LEVELS && h->ceil_level_count <= PLANE_LEVELS) {
             std::vector<unsigned short> pairs(S, 0);
@@ -2340,6 +2344,7 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)(h->floor_level_count + h->ceil_level_count) * 2, &sc.level_plane);
     if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)VH, &sc.row_slope);
     if (rc == GD_OK) rc = scratch_alloc(r, L * 32, &sc.step_scale);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * SW, &sc.block_hit);
     if (rc == GD_OK) rc = scratch_alloc(r, 1, &sc.status);
     if (rc == GD_OK && hipMemset(sc.status, 0, sizeof(int)) != hipSuccess) rc = fail(GD_E_HIP, "hipMemset status");
     if (rc == GD_OK) {
