@@ -80,7 +80,7 @@ struct WallRec {   // one linedef seen from one lane
     int flags;
 };
 
-struct Cand {      // one linedef with a finite ray distance at one column, with the static
+struct __align__(16) Cand {      // one linedef with a finite ray distance at one column, with the static
                    // linedef facts every scan needs packed in so that scans do no gathers
     unsigned short wall, flags;
     short s0, s1;            // front / back sector (-1 = none)
@@ -281,6 +281,7 @@ __device__ __forceinline__ int grid_cell_of(const gd_map_desc *m, float px, floa
 #define FINE_MIXED 2u
 #define FINE_UNKNOWN 3u
 #define FINE_MASK_LEVELS 15
+#define FLAT_BATCH 4       // plane levels probed together in flat_select
 
 // Fine raster lookup.  Points outside the raster (or not finite) report FINE_UNKNOWN with a
 // negative cell, and the caller locates them with grid_cell_of.  The coarse cell of a point
@@ -652,45 +653,64 @@ __global__ void flat_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
         const float my_height = floor_uniform ? (c.view_z - my_level) : (my_level - c.view_z);
         const float my_perpendicular = (mine < level_count && my_height > 0) ? my_height * 192.0f / denom : -1.0f;
         const int chunk = level_count - base < 64 ? level_count - base : 64;
-        for (int k = 0; k < chunk; ++k) {
-            const float perpendicular = bcast(my_perpendicular, k);
-            const float level = bcast(my_level, k);
-            const float nearest = bcast(my_reach, k);
-            if (!(perpendicular > 0)) continue;              // the same in every lane
-            float cd;
-            if (cc_plain && perpendicular >= 1e-18f && perpendicular <= 1e18f) {
-                const float q = perpendicular * inv_cc;
-                cd = __builtin_fmaf(__builtin_fmaf(-cc, q, perpendicular), inv_cc, q);
-            } else {
-                cd = perpendicular / cc;
-            }
-            if (!(finitef(cd) && cd > 0)) continue;
-            if (cd > best) { done = true; break; }           // later levels are at least this far
-            if (cd < nearest) continue;                      // every sector at this level is farther away
-            float px = c.x + rc * cd, py = c.y + rs * cd;
-            int cell;
-            unsigned fine = fine_lookup(m, inv_fine, px, py, &cell);
-            unsigned kind = FINE_KIND(fine);
-            if (kind == FINE_EMPTY) continue;
-            if (kind == FINE_DECIDED) {
-                const int s = (int)(fine & 0xFFFFu);
-                const unsigned listed = (fine >> index_shift) & 15u;   // the sector's level index, 15 = not recorded
-                bool same_level = listed == (unsigned)(base + k);
-                if (listed == 15u) {
-                    same_level = m->sector_heights[2 * s + (floor_uniform ? 0 : 1)] == level;
+        // Levels are taken FLAT_BATCH at a time: first the probe points and raster loads of the whole
+        // batch (independent, so their memory latencies overlap), then the decisions in level order.
+        // A load for a level past the one that ends the scan is wasted, never wrong.
+        for (int k0 = 0; k0 < chunk && !done; k0 += FLAT_BATCH) {
+            float cdv[FLAT_BATCH], pxv[FLAT_BATCH], pyv[FLAT_BATCH];
+            unsigned finev[FLAT_BATCH];
+            int cellv[FLAT_BATCH];
+#pragma unroll
+            for (int j = 0; j < FLAT_BATCH; ++j) {
+                const int k = k0 + j;
+                cdv[j] = -1.0f; pxv[j] = 0.0f; pyv[j] = 0.0f; finev[j] = 0x40000000u; cellv[j] = -1;
+                if (k >= chunk) continue;                        // the same in every lane
+                const float perpendicular = bcast(my_perpendicular, k);
+                const float nearest = bcast(my_reach, k);
+                if (!(perpendicular > 0)) continue;              // the same in every lane
+                float cd;
+                if (cc_plain && perpendicular >= 1e-18f && perpendicular <= 1e18f) {
+                    const float q = perpendicular * inv_cc;
+                    cd = __builtin_fmaf(__builtin_fmaf(-cc, q, perpendicular), inv_cc, q);
+                } else {
+                    cd = perpendicular / cc;
                 }
-                if (same_level && (cd < best || (cd == best && s < best_sector))) { best = cd; best_sector = s; }
-                continue;
+                cdv[j] = cd;
+                if (!(finitef(cd) && cd > 0) || cd > best || cd < nearest) continue;   // cd < nearest: every sector at this level is farther away
+                pxv[j] = c.x + rc * cd; pyv[j] = c.y + rs * cd;
+                finev[j] = fine_lookup(m, inv_fine, pxv[j], pyv[j], &cellv[j]);
             }
-            if (kind == FINE_MIXED && !((fine >> (mask_shift + base + k)) & 1u)) continue;   // no sector here has this level
-            if (cell < 0) cell = grid_cell_of(m, px, py);
-            if (cell < 0) continue;
-            for (int it = m->grid_cell_ofs[cell]; it < m->grid_cell_ofs[cell + 1]; ++it) {
-                int item = m->grid_item_sector[it];
-                int s = item & ~GRID_ALWAYS_INSIDE;
-                if (m->sector_heights[2 * s + (floor_uniform ? 0 : 1)] != level) continue;
-                if (cd < best || (cd == best && s < best_sector)) {
-                    if ((item & GRID_ALWAYS_INSIDE) || inside_edges(m, m->grid_item_edge_ofs[it], m->grid_item_edge_ofs[it + 1], px, py)) { best = cd; best_sector = s; }
+#pragma unroll
+            for (int j = 0; j < FLAT_BATCH; ++j) {
+                const int k = k0 + j;
+                if (k >= chunk || done) continue;
+                const float cd = cdv[j];
+                if (!(finitef(cd) && cd > 0)) continue;
+                if (cd > best) { done = true; continue; }        // later levels are at least this far
+                const unsigned fine = finev[j];
+                const unsigned kind = FINE_KIND(fine);
+                if (kind == FINE_EMPTY) continue;                // also levels skipped above
+                const float level = bcast(my_level, k);
+                if (kind == FINE_DECIDED) {
+                    const int s = (int)(fine & 0xFFFFu);
+                    const unsigned listed = (fine >> index_shift) & 15u;   // the sector's level index, 15 = not recorded
+                    bool same_level = listed == (unsigned)(base + k);
+                    if (listed == 15u) same_level = m->sector_heights[2 * s + (floor_uniform ? 0 : 1)] == level;
+                    if (same_level && (cd < best || (cd == best && s < best_sector))) { best = cd; best_sector = s; }
+                    continue;
+                }
+                if (kind == FINE_MIXED && !((fine >> (mask_shift + base + k)) & 1u)) continue;   // no sector here has this level
+                const float px = pxv[j], py = pyv[j];
+                int cell = cellv[j];
+                if (cell < 0) cell = grid_cell_of(m, px, py);
+                if (cell < 0) continue;
+                for (int it = m->grid_cell_ofs[cell]; it < m->grid_cell_ofs[cell + 1]; ++it) {
+                    int item = m->grid_item_sector[it];
+                    int s = item & ~GRID_ALWAYS_INSIDE;
+                    if (m->sector_heights[2 * s + (floor_uniform ? 0 : 1)] != level) continue;
+                    if (cd < best || (cd == best && s < best_sector)) {
+                        if ((item & GRID_ALWAYS_INSIDE) || inside_edges(m, m->grid_item_edge_ofs[it], m->grid_item_edge_ofs[it + 1], px, py)) { best = cd; best_sector = s; }
+                    }
                 }
             }
         }
@@ -897,6 +917,7 @@ __global__ void __launch_bounds__(SW) flat_finish_kernel(DeviceMap dm, int lane_
 // ---------------------------------------------------------------------------------------------
 // walls: engine.py:11462-13745
 // ---------------------------------------------------------------------------------------------
+#define CAND_BATCH 4
 struct ColumnCtx {
     const Tables *tb;
     const gd_map_desc *m;
@@ -907,7 +928,17 @@ struct ColumnCtx {
     int count;
     int x;
     float rx, ry;
-    __device__ Cand cand(int k) const { return list[(size_t)k * SW + x]; }
+    __device__ __forceinline__ Cand cand(int k) const {
+        union { uint4 raw; Cand c; } u;
+        u.raw = *reinterpret_cast<const uint4 *>(list + (size_t)k * SW + x);   // one 16-byte load
+        return u.c;
+    }
+    // Entries k0 .. k0+CAND_BATCH-1 of this column's list, loaded together so that their memory
+    // latencies overlap; slots past the end repeat the last entry (callers skip them).
+    __device__ __forceinline__ void cand_batch(int k0, Cand (&out)[CAND_BATCH]) const {
+#pragma unroll
+        for (int j = 0; j < CAND_BATCH; ++j) out[j] = cand(k0 + j < count ? k0 + j : count - 1);
+    }
     __device__ Eval eval(int w) const { return eval_wall(m, *c, recs, x, w, rx, ry); }
 };
 
@@ -1156,11 +1187,17 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
         // the selection when it lies within 1e-3 of the nearest candidate, found in the same scan.
         float sd = GD_INF; int swi = 0x7fffffff;
         int wi_flags = 0, swi_flags = 0;
-        for (int k = 0; k < cc.count; ++k) {
-            Cand q = cc.cand(k);
-            if (!(incident_c(q) && q.dist > prev)) continue;
-            if (q.dist < distance || (q.dist == distance && (int)q.wall < wi)) { distance = q.dist; wi = q.wall; wi_flags = q.flags; }
-            if ((q.s1 < 0) && (q.dist < sd || (q.dist == sd && (int)q.wall < swi))) { sd = q.dist; swi = q.wall; swi_flags = q.flags; }
+        for (int k0 = 0; k0 < cc.count; k0 += CAND_BATCH) {
+            Cand batch[CAND_BATCH];
+            cc.cand_batch(k0, batch);
+#pragma unroll
+            for (int j = 0; j < CAND_BATCH; ++j) {
+                if (k0 + j >= cc.count) continue;
+                const Cand q = batch[j];
+                if (!(incident_c(q) && q.dist > prev)) continue;
+                if (q.dist < distance || (q.dist == distance && (int)q.wall < wi)) { distance = q.dist; wi = q.wall; wi_flags = q.flags; }
+                if ((q.s1 < 0) && (q.dist < sd || (q.dist == sd && (int)q.wall < swi))) { sd = q.dist; swi = q.wall; swi_flags = q.flags; }
+            }
         }
         if (finitef(sd) && (fabsf(sd - distance) <= 1e-3f)) { distance = sd; wi = swi; wi_flags = swi_flags; }
         cwi.dist = distance; cwi.flags = wi_flags;
@@ -1187,10 +1224,16 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
     bool ps_path_geo = cwi.flags & CF_GEO;
     float psd = GD_INF; int psi = 0x7fffffff; int psi_flags = 0;
     if (!sel_is_proj) {
-        for (int k = 0; k < cc.count; ++k) {
-            Cand q = cc.cand(k);
-            bool owner = incident_c(q) && (q.s1 < 0) && (q.flags & CF_PROJ) && (q.flags & CF_LEDGE) && shares_sel_c(q) && (q.dist > prev_eps);
-            if (owner && (q.dist < psd || (q.dist == psd && (int)q.wall < psi))) { psd = q.dist; psi = q.wall; psi_flags = q.flags; }
+        for (int k0 = 0; k0 < cc.count; k0 += CAND_BATCH) {
+            Cand batch[CAND_BATCH];
+            cc.cand_batch(k0, batch);
+#pragma unroll
+            for (int j = 0; j < CAND_BATCH; ++j) {
+                if (k0 + j >= cc.count) continue;
+                const Cand q = batch[j];
+                bool owner = incident_c(q) && (q.s1 < 0) && (q.flags & CF_PROJ) && (q.flags & CF_LEDGE) && shares_sel_c(q) && (q.dist > prev_eps);
+                if (owner && (q.dist < psd || (q.dist == psd && (int)q.wall < psi))) { psd = q.dist; psi = q.wall; psi_flags = q.flags; }
+            }
         }
         if (sel_excl_right) {
             const int *ofs = sel_start ? m->solid_bridge_start_ofs : m->solid_bridge_end_ofs;
@@ -1229,17 +1272,23 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
     float npd = GD_INF; int npi = 0x7fffffff; int npi_flags = 0;
     const int so_s0 = mv.sec(wi, 0), so_s1 = mv.sec(wi, 1);
     if (!so_is_proj) {
-        for (int k = 0; k < cc.count; ++k) {
-            Cand q = cc.cand(k);
-            int w = q.wall;
-            if (!(incident_c(q) && (q.s1 >= 0) && (q.flags & CF_PROJ) && (q.dist > prev_eps))) continue;
-            bool le = q.flags & CF_LEDGE;
-            bool same_pair = (q.s0 == so_s0 && q.s1 == so_s1) || (q.s0 == so_s1 && q.s1 == so_s0);
-            bool close = (same_pair || (le && so_excl_right && ((so_span <= 2) || (shares_sel_c(q) && so_short)))) &&
-                         (fabsf(q.dist - distance) <= tolerance_of(q.dist));
-            bool topo = false;
-            if (!close && le && so_excl_right && so_span <= 2) { int dummy; topo = mv.sector_bridge((q.flags & CF_ALONG_HI) ? 1 : 0, w, no_path_index, &dummy); }
-            if ((close || topo) && (q.dist < npd || (q.dist == npd && w < npi))) { npd = q.dist; npi = w; npi_flags = q.flags; }
+        for (int k0 = 0; k0 < cc.count; k0 += CAND_BATCH) {
+            Cand batch[CAND_BATCH];
+            cc.cand_batch(k0, batch);
+#pragma unroll
+            for (int j = 0; j < CAND_BATCH; ++j) {
+                if (k0 + j >= cc.count) continue;
+                const Cand q = batch[j];
+                int w = q.wall;
+                if (!(incident_c(q) && (q.s1 >= 0) && (q.flags & CF_PROJ) && (q.dist > prev_eps))) continue;
+                bool le = q.flags & CF_LEDGE;
+                bool same_pair = (q.s0 == so_s0 && q.s1 == so_s1) || (q.s0 == so_s1 && q.s1 == so_s0);
+                bool close = (same_pair || (le && so_excl_right && ((so_span <= 2) || (shares_sel_c(q) && so_short)))) &&
+                             (fabsf(q.dist - distance) <= tolerance_of(q.dist));
+                bool topo = false;
+                if (!close && le && so_excl_right && so_span <= 2) { int dummy; topo = mv.sector_bridge((q.flags & CF_ALONG_HI) ? 1 : 0, w, no_path_index, &dummy); }
+                if ((close || topo) && (q.dist < npd || (q.dist == npd && w < npi))) { npd = q.dist; npi = w; npi_flags = q.flags; }
+            }
         }
     }
     int pe_wall = c.pend_ep_wall;
@@ -1560,24 +1609,30 @@ __device__ __forceinline__ bool pass_advance(const ColumnCtx &cc, ColumnState &c
         float csd = GD_INF, osd = GD_INF;
         int gpi = 0x7fffffff; bool gp_along_hi = false;
         const int v0 = mv.vert(wi, 0), v1 = mv.vert(wi, 1);
-        for (int k = 0; k < cc.count; ++k) {
-            Cand q = cc.cand(k);
-            int w = q.wall; float d = q.dist;
-            bool os = q.s1 < 0;
-            bool inc = (q.s0 == cur || q.s1 == cur), oinc = (q.s0 == other_sector || q.s1 == other_sector);
-            bool future = ((q.flags & CF_GEO) || os) && (d > dist_eps);
-            if (future) {
-                if (inc) take_min(d, w, cnd, cni);
-                if (oinc) take_min(d, w, ond, oni);
+        for (int k0 = 0; k0 < cc.count; k0 += CAND_BATCH) {
+            Cand batch[CAND_BATCH];
+            cc.cand_batch(k0, batch);
+#pragma unroll
+            for (int j = 0; j < CAND_BATCH; ++j) {
+                if (k0 + j >= cc.count) continue;
+                const Cand q = batch[j];
+                int w = q.wall; float d = q.dist;
+                bool os = q.s1 < 0;
+                bool inc = (q.s0 == cur || q.s1 == cur), oinc = (q.s0 == other_sector || q.s1 == other_sector);
+                bool future = ((q.flags & CF_GEO) || os) && (d > dist_eps);
+                if (future) {
+                    if (inc) take_min(d, w, cnd, cni);
+                    if (oinc) take_min(d, w, ond, oni);
+                }
+                bool shares_endpoint = (int)q.v0 == v0 || (int)q.v0 == v1 || (int)q.v1 == v0 || (int)q.v1 == v1;
+                bool shared_solid = os && (shares_endpoint || (q.flags & CF_LEDGE)) && (d > prior_eps) && (d <= dist_eps);
+                if (shared_solid) {
+                    if (inc && d < csd) csd = d;
+                    if (oinc && d < osd) osd = d;
+                }
+                bool sgp = (q.flags & CF_GEO) && inc && shares_endpoint && !os && (d > prior_eps) && (fabsf(d - distance) <= (1.0f / 16.0f));
+                if (sgp && (d < gpd || (d == gpd && w < gpi))) { gpd = d; gpi = w; gp_along_hi = (q.flags & CF_ALONG_HI) != 0; }
             }
-            bool shares_endpoint = (int)q.v0 == v0 || (int)q.v0 == v1 || (int)q.v1 == v0 || (int)q.v1 == v1;
-            bool shared_solid = os && (shares_endpoint || (q.flags & CF_LEDGE)) && (d > prior_eps) && (d <= dist_eps);
-            if (shared_solid) {
-                if (inc && d < csd) csd = d;
-                if (oinc && d < osd) osd = d;
-            }
-            bool sgp = (q.flags & CF_GEO) && inc && shares_endpoint && !os && (d > prior_eps) && (fabsf(d - distance) <= (1.0f / 16.0f));
-            if (sgp && (d < gpd || (d == gpd && w < gpi))) { gpd = d; gpi = w; gp_along_hi = (q.flags & CF_ALONG_HI) != 0; }
         }
         if (!finitef(cnd)) cni = 0;
         if (!finitef(ond)) oni = 0;
@@ -1648,13 +1703,19 @@ __device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const Col
     const LaneCtx &L = *cc.c;
     const int x = cc.x;
     float md = GD_INF; int mw = 0x7fffffff; int mside = 0; int cand_flags = 0;
-    for (int k = 0; k < cc.count; ++k) {
-        Cand q = cc.cand(k);
-        int w = q.wall;
-        if (!(q.flags & CF_PROJ) || (q.s1 < 0)) continue;
-        int sidew = (q.flags & CF_FF) ? 0 : 1;   // engine.py:13436-13444, the float32 facing test
-        if (m->side_tex[(w * 2 + sidew) * 3] < 0) continue;
-        if (q.dist < md || (q.dist == md && w < mw)) { md = q.dist; mw = w; mside = sidew; cand_flags = q.flags; }
+    for (int k0 = 0; k0 < cc.count; k0 += CAND_BATCH) {
+        Cand batch[CAND_BATCH];
+        cc.cand_batch(k0, batch);
+#pragma unroll
+        for (int j = 0; j < CAND_BATCH; ++j) {
+            if (k0 + j >= cc.count) continue;
+            const Cand q = batch[j];
+            int w = q.wall;
+            if (!(q.flags & CF_PROJ) || (q.s1 < 0)) continue;
+            int sidew = (q.flags & CF_FF) ? 0 : 1;   // engine.py:13436-13444, the float32 facing test
+            if (m->side_tex[(w * 2 + sidew) * 3] < 0) continue;
+            if (q.dist < md || (q.dist == md && w < mw)) { md = q.dist; mw = w; mside = sidew; cand_flags = q.flags; }
+        }
     }
     if (!finitef(md)) return;
     int texture_id = m->side_tex[(mw * 2 + mside) * 3];
