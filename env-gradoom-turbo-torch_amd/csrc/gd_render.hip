@@ -1388,24 +1388,37 @@ struct SilhouetteBounds {
     float bot_depth, top_depth;
 };
 
+// Rows [first, last) of one column take `distance` / `wall` as their sprite clip where it is nearer
+// than what they hold.  Four rows at a time, loads first, so the rows' memory latencies overlap.
+__device__ __forceinline__ void clip_rows(PixelBuffers &pb, int x, int first, int last, float distance, int wall) {
+    for (int y0 = first; y0 < last; y0 += 4) {
+        float held[4]; unsigned int meta[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const size_t i = (size_t)(y0 + j < last ? y0 + j : last - 1) * SW + x;
+            held[j] = pb.clip_depth[i]; meta[j] = pb.meta[i];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (y0 + j >= last || !(distance < held[j])) continue;
+            const size_t i = (size_t)(y0 + j) * SW + x;
+            pb.clip_depth[i] = distance; pb.meta[i] = (meta[j] & ~META_WALL_MASK) | (unsigned)(wall + 1);
+        }
+    }
+}
+
 __device__ __forceinline__ void apply_silhouette(PixelBuffers &pb, SilhouetteBounds &sb, int x, bool bottom, bool top, float floor_clip, float ceiling_clip, float distance, int wall) {
     if (bottom) {
         int first = floor_clip <= 0.0f ? 0 : (floor_clip >= (float)VH ? VH : (int)floor_clip);   // clips hold integers
         int last = (distance >= sb.bot_depth) ? (sb.bot_row < VH ? sb.bot_row : VH) : VH;
-        for (int y = first; y < last; ++y) {
-            size_t i = (size_t)y * SW + x;
-            if (distance < pb.clip_depth[i]) { pb.clip_depth[i] = distance; pb.meta[i] = (pb.meta[i] & ~META_WALL_MASK) | (unsigned)(wall + 1); }
-        }
+        clip_rows(pb, x, first, last, distance, wall);
         sb.bot_row = first < sb.bot_row ? first : sb.bot_row;
         sb.bot_depth = fmaxf(sb.bot_depth, distance);
     }
     if (top) {
         int end = ceiling_clip <= 0.0f ? 0 : (ceiling_clip >= (float)VH ? VH : (int)ceiling_clip);
         int start = (distance >= sb.top_depth) ? (sb.top_row > 0 ? sb.top_row : 0) : 0;
-        for (int y = start; y < end; ++y) {
-            size_t i = (size_t)y * SW + x;
-            if (distance < pb.clip_depth[i]) { pb.clip_depth[i] = distance; pb.meta[i] = (pb.meta[i] & ~META_WALL_MASK) | (unsigned)(wall + 1); }
-        }
+        clip_rows(pb, x, start, end, distance, wall);
         sb.top_row = end > sb.top_row ? end : sb.top_row;
         sb.top_depth = fmaxf(sb.top_depth, distance);
     }
@@ -1463,30 +1476,48 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
         if (one_sided) { t0 = (int)r.clipped_top; t1 = (int)r.clipped_bottom; }
         if (lower_on) { t0 = min(t0, (int)r.clipped_lower_top); t1 = max(t1, (int)r.clipped_bottom); }
         if (upper_on) { t0 = min(t0, (int)r.clipped_top); t1 = max(t1, (int)r.clipped_upper_bottom); }
-        for (int y = t0; y < t1; ++y) {
-            const float py = (float)y;
-            bool one_span = one_sided && (py >= r.clipped_top) && (py < r.clipped_bottom);
-            bool lower_span = lower_on && (py >= r.clipped_lower_top) && (py < r.clipped_bottom);
-            bool upper_span = upper_on && (py >= r.clipped_top) && (py < r.clipped_upper_bottom);
-            if (!(one_span || lower_span || upper_span)) continue;
-            int texture_id = one_span ? r.side_tex[0] : (lower_span ? r.side_tex[1] : r.side_tex[2]);
-            if (texture_id < 0) continue;
-            bool bottom_tail = (one_span && group_valid[0] && py >= group_bottom[0]) ||
-                               (lower_span && group_valid[1] && py >= group_bottom[1]) ||
-                               (upper_span && group_valid[2] && py >= group_bottom[2]);
-            i64 tu = u_base & (i64)((1 << tb.width_bits(texture_id)) - 1);
-            float origin_z = one_span ? r.view_ceiling : (lower_span ? r.other_floor : r.other_ceiling);
-            int height_bits = tb.height_bits(texture_id);
-            i64 vertical_step = mul64(swall, shl64(1, 14 - height_bits));
-            i64 screen_delta = (i64)y * FIXED_UNIT - L.center_fixed + FIXED_UNIT;
-            i64 texture_mid = round_to_i64((origin_z - L.view_z) * 65536.0f + toff[1] * 65536.0f);
-            i64 fraction = shl64(texture_mid, 16 - height_bits) + (mul64(vertical_step, screen_delta) >> 16);
-            i64 tv = (fraction & UINT32_MASK) >> (32 - height_bits);
-            unsigned char texel = m->tex_atlas[((size_t)texture_id * m->tex_max_h + tv) * m->tex_max_w + tu];
-            const size_t i = (size_t)y * SW + x;
-            pb.frame[i] = colormap[(bottom_tail ? shade_group : shade_own) * 256 + texel];
-            pb.clip_depth[i] = r.distance;
-            pb.meta[i] = META_FILLED | (unsigned)(wi + 1);
+        // what the three tiers need per row, worked out once: texture, column, vertical mapping
+        int tier_tex[3]; i64 tier_tu[3], tier_step[3], tier_base[3]; int tier_bits[3];
+        const float tier_origin[3] = {r.view_ceiling, r.other_floor, r.other_ceiling};
+        const float toff_y = toff[1] * 65536.0f;
+#pragma unroll
+        for (int t = 0; t < 3; ++t) {
+            tier_tex[t] = r.side_tex[t];
+            const int id = tier_tex[t] < 0 ? 0 : tier_tex[t];
+            tier_bits[t] = tb.height_bits(id);
+            tier_tu[t] = u_base & (i64)((1 << tb.width_bits(id)) - 1);
+            tier_step[t] = mul64(swall, shl64(1, 14 - tier_bits[t]));
+            tier_base[t] = shl64(round_to_i64((tier_origin[t] - L.view_z) * 65536.0f + toff_y), 16 - tier_bits[t]);
+        }
+        // four rows at a time: texel loads first, so their latencies overlap, then the stores
+        for (int yb = t0; yb < t1; yb += 4) {
+            unsigned char texel[4]; bool draw[4], tail[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int y = yb + j;
+                const float py = (float)y;
+                const bool one_span = one_sided && (py >= r.clipped_top) && (py < r.clipped_bottom);
+                const bool lower_span = lower_on && (py >= r.clipped_lower_top) && (py < r.clipped_bottom);
+                const bool upper_span = upper_on && (py >= r.clipped_top) && (py < r.clipped_upper_bottom);
+                const int t = one_span ? 0 : (lower_span ? 1 : 2);
+                draw[j] = y < t1 && (one_span || lower_span || upper_span) && tier_tex[t] >= 0;
+                tail[j] = group_valid[t] && py >= group_bottom[t];
+                texel[j] = 0;
+                if (draw[j]) {
+                    const i64 screen_delta = (i64)y * FIXED_UNIT - L.center_fixed + FIXED_UNIT;
+                    const i64 fraction = tier_base[t] + (mul64(tier_step[t], screen_delta) >> 16);
+                    const i64 tv = (fraction & UINT32_MASK) >> (32 - tier_bits[t]);
+                    texel[j] = m->tex_atlas[((size_t)tier_tex[t] * m->tex_max_h + tv) * m->tex_max_w + tier_tu[t]];
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (!draw[j]) continue;
+                const size_t i = (size_t)(yb + j) * SW + x;
+                pb.frame[i] = colormap[(tail[j] ? shade_group : shade_own) * 256 + texel[j]];
+                pb.clip_depth[i] = r.distance;
+                pb.meta[i] = META_FILLED | (unsigned)(wi + 1);
+            }
         }
         if (one_sided) window_dirty = true;
         return;
