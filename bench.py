@@ -24,6 +24,13 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 POSE_SETS = 4
+# HBM bytes one launch of a kernel moves, per lane, on the config4 workload: rocprofv3 FETCH_SIZE + WRITE_SIZE
+# of a 4096-lane launch, each scaled by what the same counter reads for a 1 GiB copy
+# (profiles/render_chain_config4_4096lanes.md).  Measured offline; other workloads report null.
+MEASURED_TRAFFIC_PER_LANE = {
+    ("config4", "wall_columns"): 1.503e10 / 4096,
+    ("config4", "flat_select"): 9.356e8 / 4096,
+}
 
 
 def algorithmic_bytes_per_lane_frame(sprites: int, map_bytes: int, lanes: int) -> float:
@@ -41,6 +48,9 @@ def main() -> int:
     parser.add_argument("--lanes", type=int, default=None)
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     parser.add_argument("--cpu-lanes", type=int, default=12, help="lanes of the same workload the CPU baseline renders")
+    parser.add_argument("--copy-probe-mib", type=int, default=0,
+                        help="after the timed region, copy this many MiB device to device once (a kernel of known "
+                             "traffic that scales the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: lanes are independent and this build has no multi-GPU path; run with --gpus 1", file=sys.stderr)
@@ -122,13 +132,21 @@ def main() -> int:
     # render_timed sums a stage over the chunks of one frame; one launch handles `chunk` lanes
     launch_ms = stage_ms[dominant] / chunks
     achieved = bytes_per_lane * chunk / (launch_ms * 1e-3) / 1e9 if launch_ms > 0 else 0.0
+    per_lane_traffic = MEASURED_TRAFFIC_PER_LANE.get((args.workload, dominant))
+    traffic = None if per_lane_traffic is None else round(per_lane_traffic * chunk)
     roofline = dict(
         bound="hbm", kernel=dominant + "_kernel", achieved=round(achieved, 3), peak=HBM_PEAK_GBPS, unit="GB/s",
-        frac=round(achieved / HBM_PEAK_GBPS, 6), traffic=None, launch_ms=round(launch_ms, 4),
+        frac=round(achieved / HBM_PEAK_GBPS, 6), traffic=traffic, launch_ms=round(launch_ms, 4),
         stage_ms_per_frame={name: round(ms, 4) for name, ms in stage_ms.items()},
         whole_path_frac=round(value * bytes_per_lane / 1e9 / HBM_PEAK_GBPS, 6),
         bytes_per_lane_frame=round(bytes_per_lane, 1),
     )
+
+    if args.copy_probe_mib > 0:
+        probe_src = torch.ones(args.copy_probe_mib << 20, dtype=torch.uint8, device=device)
+        probe_dst = torch.empty_like(probe_src)
+        probe_dst.copy_(probe_src)
+        torch.cuda.synchronize()
 
     cpu_baseline = None
     if not args.no_cpu:

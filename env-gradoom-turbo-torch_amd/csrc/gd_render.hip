@@ -1831,7 +1831,7 @@ __device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const Col
 // tables are paid once per group rather than once per wavefront (which would cap the CU at a
 // couple of wavefronts per SIMD).  After the staging barrier the wavefronts never meet again.
 #define WALL_STRIPS_PER_GROUP 2
-__global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amdgpu_waves_per_eu(4, 4))) wall_columns_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
+__global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amdgpu_waves_per_eu(3, 3))) wall_columns_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
     const gd_map_desc *m = &dm.d;
     __shared__ LaneCtx lane_ctxs[WALL_STRIPS_PER_GROUP];
     __shared__ unsigned char colormap_lds[32 * 256];   // shade rows 0..31 are the only ones indexed
