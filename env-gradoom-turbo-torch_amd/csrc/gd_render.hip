@@ -855,21 +855,31 @@ __global__ void __launch_bounds__(SW) flat_finish_kernel(DeviceMap dm, int lane_
     {
         int next_floor = VH, next_ceiling = VH;
         int floor_sector = 0, ceiling_sector = 0;
-        for (int y = VH - 1; y >= 0; --y) {
-            size_t i = (size_t)y * SW + x;
-            bool is_floor = ((float)y - center) > 0;
-            bool unresolved = flags[i] & 1;
-            int s = sector[i];
-            if (!unresolved) {
-                if (is_floor) { next_floor = y; floor_sector = s; } else { next_ceiling = y; ceiling_sector = s; }
-            } else {
-                bool vfloor = is_floor && next_floor < VH;
-                bool vceil = !is_floor && next_ceiling < VH;
-                if (vfloor || vceil) {
-                    int span_sector = vfloor ? floor_sector : ceiling_sector;
-                    sector[i] = (unsigned short)span_sector;
-                    // bit1: vertical span; bit2: its sector differs from the camera's (anchor)
-                    flags[i] = (unsigned char)(1 | 2 | ((span_sector != c.sector) ? 4 : 0));
+        // eight rows per step, loads first (a row only depends on rows below it through the four
+        // carried values, never through memory), so the loads of a step overlap
+        static_assert(VH % 8 == 0, "row batches");
+        for (int yb = VH - 8; yb >= 0; yb -= 8) {
+            unsigned char row_flags[8]; unsigned short row_sector[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) { row_flags[j] = flags[(size_t)(yb + j) * SW + x]; row_sector[j] = sector[(size_t)(yb + j) * SW + x]; }
+#pragma unroll
+            for (int j = 7; j >= 0; --j) {
+                const int y = yb + j;
+                const size_t i = (size_t)y * SW + x;
+                bool is_floor = ((float)y - center) > 0;
+                bool unresolved = row_flags[j] & 1;
+                int s = row_sector[j];
+                if (!unresolved) {
+                    if (is_floor) { next_floor = y; floor_sector = s; } else { next_ceiling = y; ceiling_sector = s; }
+                } else {
+                    bool vfloor = is_floor && next_floor < VH;
+                    bool vceil = !is_floor && next_ceiling < VH;
+                    if (vfloor || vceil) {
+                        int span_sector = vfloor ? floor_sector : ceiling_sector;
+                        sector[i] = (unsigned short)span_sector;
+                        // bit1: vertical span; bit2: its sector differs from the camera's (anchor)
+                        flags[i] = (unsigned char)(1 | 2 | ((span_sector != c.sector) ? 4 : 0));
+                    }
                 }
             }
         }
@@ -884,8 +894,10 @@ __global__ void __launch_bounds__(SW) flat_finish_kernel(DeviceMap dm, int lane_
             unsigned char *row_flags = flags + (size_t)y * SW;
             u64 anchors[5];
             unsigned char f[5];
+#pragma unroll
+            for (int k = 0; k < 5; ++k) f[k] = row_flags[k * 64 + lane_id];
+#pragma unroll
             for (int k = 0; k < 5; ++k) {
-                f[k] = row_flags[k * 64 + lane_id];
                 bool anchor = !(f[k] & 1) || (f[k] & 4);
                 anchors[k] = __ballot(anchor);
             }
@@ -2130,16 +2142,34 @@ __global__ void observe_kernel(const unsigned char *indexed, size_t lane_stride,
     const unsigned char *src = indexed + (size_t)n * lane_stride;
     int y_start = oy * 240, y_end = y_start + 240, x_start = ox * 320, x_end = x_start + 320;
     int rs = 0, gs = 0, bs = 0;
+    // up to 4 x 5 source pixels overlap one observation pixel; all of them are loaded first (taps
+    // outside the overlap read a clamped address and weigh nothing), then accumulated
+    int y_overlap[4], x_overlap[5], row_offset[4], column[5];
+#pragma unroll
     for (int sy = 0; sy < 4; ++sy) {
-        int source_y = y_start / 84 + sy;
-        int y_overlap = min(y_end, (source_y + 1) * 84) - max(y_start, source_y * 84);
-        if (source_y >= source_rows || y_overlap <= 0) continue;
+        const int source_y = y_start / 84 + sy;
+        const int overlap = min(y_end, (source_y + 1) * 84) - max(y_start, source_y * 84);
+        y_overlap[sy] = (source_y >= source_rows || overlap <= 0) ? 0 : overlap;
+        row_offset[sy] = min(source_y, source_rows - 1) * SW;
+    }
+#pragma unroll
+    for (int sx = 0; sx < 5; ++sx) {
+        const int source_x = x_start / 84 + sx;
+        const int overlap = min(x_end, (source_x + 1) * 84) - max(x_start, source_x * 84);
+        x_overlap[sx] = (source_x >= SW || overlap <= 0) ? 0 : overlap;
+        column[sx] = min(source_x, SW - 1);
+    }
+    unsigned char tap[4][5];
+#pragma unroll
+    for (int sy = 0; sy < 4; ++sy)
+#pragma unroll
+        for (int sx = 0; sx < 5; ++sx) tap[sy][sx] = src[row_offset[sy] + column[sx]];
+#pragma unroll
+    for (int sy = 0; sy < 4; ++sy) {
+#pragma unroll
         for (int sx = 0; sx < 5; ++sx) {
-            int source_x = x_start / 84 + sx;
-            int x_overlap = min(x_end, (source_x + 1) * 84) - max(x_start, source_x * 84);
-            if (source_x >= 320 || x_overlap <= 0) continue;
-            int weight = (y_overlap * x_overlap) / 48;
-            int p = src[source_y * SW + source_x] * 3;
+            const int weight = (y_overlap[sy] * x_overlap[sx]) / 48;
+            const int p = tap[sy][sx] * 3;
             rs += pal[p] * weight; gs += pal[p + 1] * weight; bs += pal[p + 2] * weight;
         }
     }
