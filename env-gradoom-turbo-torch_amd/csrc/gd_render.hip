@@ -104,6 +104,13 @@ struct DeviceMap {  // device copy of gd_map_desc (device pointers) + fixed tabl
     // (x0, y0, x1, y1) per sector outside which no point tests inside that sector.
     const int *level_box_ofs;
     const float4 *level_boxes;
+    // The coarse grid repacked for the crossing test of flat selection: per cell its item range, per
+    // item one 16-byte record, per item edge a copy of the linedef's endpoints, so that a test is
+    // three dependent loads (range, record, edges) instead of six.
+    const int2 *cell_range;              // [cells] first item, one past the last
+    const int4 *cell_item;               // [items] sector | GRID_ALWAYS_INSIDE, floor level index | ceiling level
+                                         // index << 8 (or -1 when not recorded), first edge, one past the last
+    const float4 *cell_edge;             // [item edges] x1, y1, x2, y2
     const int *wall_blocking_slot;       // [W] position of the linedef in blocking_walls, -1 when it does not block
     const unsigned short *sector_level;  // [S] index of the floor in floor_levels | index of the ceiling in
                                          // ceil_levels << 8; null when a level list is longer than PLANE_LEVELS
@@ -263,6 +270,24 @@ __device__ __forceinline__ bool inside_edges(const gd_map_desc *m, int e0, int e
     return crossings & 1;
 }
 
+// inside_edges over the repacked edge copies, two edges per step
+__device__ __forceinline__ bool inside_edge_copies(const float4 *edges, int e0, int e1, float px, float py) {
+    int crossings = 0;
+    for (int k = e0; k < e1; k += 2) {
+        const float4 a = edges[k], b = edges[k + 1 < e1 ? k + 1 : k];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const float4 e = j == 0 ? a : b;
+            float dy = e.w - e.y;
+            float safe_dy = fabsf(dy) < 1e-6f ? 1.0f : dy;
+            bool crosses = (e.y > py) != (e.w > py);
+            float crossing_x = e.x + (py - e.y) * (e.z - e.x) / safe_dy;
+            crossings += (k + j < e1 && crosses && px < crossing_x) ? 1 : 0;
+        }
+    }
+    return crossings & 1;
+}
+
 // Cell of the point grid, or -1 when no sector can contain the point.
 __device__ __forceinline__ int grid_cell_of(const gd_map_desc *m, float px, float py) {
     float fx = floorf((px - m->grid_min_x) / m->grid_cell);
@@ -281,12 +306,21 @@ __device__ __forceinline__ int grid_cell_of(const gd_map_desc *m, float px, floa
 #define FINE_MIXED 2u
 #define FINE_UNKNOWN 3u
 #define FINE_MASK_LEVELS 15
-#define FLAT_BATCH 4       // plane levels probed together in flat_select
+#define FLAT_BATCH 2       // plane levels probed together in flat_select
 
 // Fine raster lookup.  Points outside the raster (or not finite) report FINE_UNKNOWN with a
 // negative cell, and the caller locates them with grid_cell_of.  The coarse cell of a point
 // inside the raster is (iy >> 3) * grid_nx + (ix >> 3): grid_cell is 8 * fine_cell and both
 // grids pad their cells far beyond the rounding of either index computation.
+// (fx, fy) is the point in raster cell units; anything within a small fraction of a cell of the
+// true position will do, because decided cells keep a margin of half a map unit.
+__device__ __forceinline__ unsigned fine_lookup_cells(const gd_map_desc *m, float fx, float fy, int *coarse_cell) {
+    int ix = (int)floorf(fx), iy = (int)floorf(fy);
+    *coarse_cell = -1;
+    if ((unsigned)ix >= (unsigned)m->fine_nx || (unsigned)iy >= (unsigned)m->fine_ny || !(fx == fx) || !(fy == fy)) return 0xC0000000u;
+    *coarse_cell = (iy >> 3) * m->grid_nx + (ix >> 3);
+    return m->fine_sector[iy * m->fine_nx + ix];
+}
 __device__ __forceinline__ unsigned fine_lookup(const gd_map_desc *m, float inv_cell, float px, float py, int *coarse_cell) {
     int ix = (int)floorf((px - m->grid_min_x) * inv_cell), iy = (int)floorf((py - m->grid_min_y) * inv_cell);
     *coarse_cell = -1;
@@ -641,7 +675,16 @@ __global__ void flat_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
     const float inv_cc = 1.0f / cc;
     const bool cc_plain = cc >= 0.5f && cc <= 1.0f;
     const float inv_fine = 1.0f / m->fine_cell;   // a reciprocal is fine here: see fine_lookup
+    // the probe point camera + ray * cd in raster cell units, as one multiply-add per axis
+    const float cell_x0 = (c.x - m->grid_min_x) * inv_fine, cell_y0 = (c.y - m->grid_min_y) * inv_fine;
+    const float cell_dx = rc * inv_fine, cell_dy = rs * inv_fine;
     const int slot_in_wave = threadIdx.x & 63;
+    // cd <= perpendicular / (smallest cc of the wavefront): with it a level whose every sector is
+    // farther than that from the camera is dropped for the whole wavefront at once
+    float cc_floor = cc;
+#pragma unroll
+    for (int step = 1; step < 64; step <<= 1) cc_floor = fminf(cc_floor, __shfl_xor(cc_floor, step));
+    const float reach_scale = cc_floor > 0.0f ? 1.001f / cc_floor : GD_INF;
     float best = GD_INF; int best_sector = -1;
     bool done = false;
     for (int base = 0; base < level_count && !done; base += 64) {
@@ -657,17 +700,18 @@ __global__ void flat_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
         // batch (independent, so their memory latencies overlap), then the decisions in level order.
         // A load for a level past the one that ends the scan is wasted, never wrong.
         for (int k0 = 0; k0 < chunk && !done; k0 += FLAT_BATCH) {
-            float cdv[FLAT_BATCH], pxv[FLAT_BATCH], pyv[FLAT_BATCH];
+            float cdv[FLAT_BATCH];
             unsigned finev[FLAT_BATCH];
             int cellv[FLAT_BATCH];
 #pragma unroll
             for (int j = 0; j < FLAT_BATCH; ++j) {
                 const int k = k0 + j;
-                cdv[j] = -1.0f; pxv[j] = 0.0f; pyv[j] = 0.0f; finev[j] = 0x40000000u; cellv[j] = -1;
+                cdv[j] = -1.0f; finev[j] = 0x40000000u; cellv[j] = -1;
                 if (k >= chunk) continue;                        // the same in every lane
                 const float perpendicular = bcast(my_perpendicular, k);
                 const float nearest = bcast(my_reach, k);
                 if (!(perpendicular > 0)) continue;              // the same in every lane
+                if (perpendicular * reach_scale < nearest) continue;   // the same in every lane: no lane can reach the level
                 float cd;
                 if (cc_plain && perpendicular >= 1e-18f && perpendicular <= 1e18f) {
                     const float q = perpendicular * inv_cc;
@@ -677,8 +721,7 @@ __global__ void flat_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
                 }
                 cdv[j] = cd;
                 if (!(finitef(cd) && cd > 0) || cd > best || cd < nearest) continue;   // cd < nearest: every sector at this level is farther away
-                pxv[j] = c.x + rc * cd; pyv[j] = c.y + rs * cd;
-                finev[j] = fine_lookup(m, inv_fine, pxv[j], pyv[j], &cellv[j]);
+                finev[j] = fine_lookup_cells(m, __builtin_fmaf(cd, cell_dx, cell_x0), __builtin_fmaf(cd, cell_dy, cell_y0), &cellv[j]);
             }
 #pragma unroll
             for (int j = 0; j < FLAT_BATCH; ++j) {
@@ -700,16 +743,19 @@ __global__ void flat_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
                     continue;
                 }
                 if (kind == FINE_MIXED && !((fine >> (mask_shift + base + k)) & 1u)) continue;   // no sector here has this level
-                const float px = pxv[j], py = pyv[j];
+                const float px = c.x + rc * cd, py = c.y + rs * cd;
                 int cell = cellv[j];
                 if (cell < 0) cell = grid_cell_of(m, px, py);
                 if (cell < 0) continue;
-                for (int it = m->grid_cell_ofs[cell]; it < m->grid_cell_ofs[cell + 1]; ++it) {
-                    int item = m->grid_item_sector[it];
-                    int s = item & ~GRID_ALWAYS_INSIDE;
-                    if (m->sector_heights[2 * s + (floor_uniform ? 0 : 1)] != level) continue;
+                const int2 range = dm.cell_range[cell];
+                for (int it = range.x; it < range.y; ++it) {
+                    const int4 item = dm.cell_item[it];
+                    const int s = item.x & ~GRID_ALWAYS_INSIDE;
+                    const bool same_level = item.y >= 0 ? ((floor_uniform ? (item.y & 0xFF) : (item.y >> 8)) == base + k)
+                                                        : (m->sector_heights[2 * s + (floor_uniform ? 0 : 1)] == level);
+                    if (!same_level) continue;
                     if (cd < best || (cd == best && s < best_sector)) {
-                        if ((item & GRID_ALWAYS_INSIDE) || inside_edges(m, m->grid_item_edge_ofs[it], m->grid_item_edge_ofs[it + 1], px, py)) { best = cd; best_sector = s; }
+                        if ((item.x & GRID_ALWAYS_INSIDE) || inside_edge_copies(dm.cell_edge, item.z, item.w, px, py)) { best = cd; best_sector = s; }
                     }
                 }
             }
@@ -2434,9 +2480,10 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
         }
         if (rc == GD_OK) rc = upload(r, blocking_slot.data(), blocking_slot.size(), &r->dm.wall_blocking_slot);
         r->dm.sector_level = nullptr;
+        std::vector<unsigned short> pairs(S, 0);
+        bool listed = false;
         if (h->floor_level_count <= PLANE_LEVELS && h->ceil_level_count <= PLANE_LEVELS) {
-            std::vector<unsigned short> pairs(S, 0);
-            bool listed = true;
+            listed = true;
             for (size_t s = 0; s < S; ++s) {
                 int fi = -1, ci = -1;
                 for (int l = 0; l < h->floor_level_count; ++l) if (h->floor_levels[l] == h->sector_heights[2 * s]) fi = l;
@@ -2447,6 +2494,25 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
             // a sector whose height is missing from the level lists keeps the per-pixel divisions
             if (listed && rc == GD_OK) rc = upload(r, pairs.data(), pairs.size(), &r->dm.sector_level);
         }
+        std::vector<int2> cell_range(cells);
+        std::vector<int4> cell_item(items);
+        std::vector<float4> cell_edge;
+        for (size_t c = 0; c < cells; ++c) cell_range[c] = make_int2(h->grid_cell_ofs[c], h->grid_cell_ofs[c + 1]);
+        for (size_t it = 0; it < items; ++it) {
+            const int entry = h->grid_item_sector[it];
+            const size_t s = (size_t)(entry & ~GRID_ALWAYS_INSIDE);
+            if (s >= S) { if (rc == GD_OK) rc = fail(GD_E_ARG, "grid_item_sector holds a sector index out of range"); continue; }
+            const int first = (int)cell_edge.size();
+            for (int k = h->grid_item_edge_ofs[it]; k < h->grid_item_edge_ofs[it + 1]; ++k) {
+                const int w = h->grid_item_edges[k];
+                if (w < 0 || (size_t)w >= W) { if (rc == GD_OK) rc = fail(GD_E_ARG, "grid_item_edges holds a linedef index out of range"); continue; }
+                cell_edge.push_back(make_float4(h->walls[4 * w], h->walls[4 * w + 1], h->walls[4 * w + 2], h->walls[4 * w + 3]));
+            }
+            cell_item[it] = make_int4(entry, listed ? (int)pairs[s] : -1, first, (int)cell_edge.size());
+        }
+        if (rc == GD_OK) rc = upload(r, cell_range.data(), cell_range.size(), &r->dm.cell_range);
+        if (rc == GD_OK) rc = upload(r, cell_item.data(), cell_item.size(), &r->dm.cell_item);
+        if (rc == GD_OK) rc = upload(r, cell_edge.data(), cell_edge.size(), &r->dm.cell_edge);
     }
     // Working memory for one chunk of lanes; larger batches are rendered chunk by chunk.
     const int chunk = max_lanes < 4096 ? max_lanes : 4096;
