@@ -2148,27 +2148,53 @@ __global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lan
         float visibility = fminf(1280.0f / fmaxf(s.depth, 1.0f), 24.0f);
         i64 shade = clampi((i64)floorf(base_shade - visibility), 0, 31);
         i64 fraction_base = s.texmid - (mul64(L.center_fixed - FIXED_UNIT, s.iscale) >> 16);
-        for (int y = 0; y < VH; ++y) {
-            i64 sv = (fraction_base + mul64((i64)y, s.iscale)) >> 16;
-            if (!(sv >= 0 && sv < height)) continue;
-            size_t i = (size_t)y * SW + x;
-            int cw = (int)(meta[i] & META_WALL_MASK) - 1;
-            bool visible;
-            if (cw >= 0) {
-                const WallRec &cg = recs[cw];
-                i64 cnear = min64(cg.dl, cg.dr), cfar = max64(cg.dl, cg.dr);
-                const float4 cl = *reinterpret_cast<const float4 *>(m->walls + 4 * cw);
-                float side = (cl.z - cl.x) * (s.y - cl.y) - (cl.w - cl.y) * (s.x - cl.x);
-                visible = (cnear > s.depth_fixed) || ((cfar > s.depth_fixed) && (side <= 0));
-            } else {
-                visible = s.depth < clip_depth[i];
+        // Rows whose source row sv = (fraction_base + y * iscale) >> 16 can fall inside the patch:
+        // a bracket from two divisions, a row too wide on either side; the exact test stays per row.
+        int y_lo = 0, y_hi = VH;
+        if (s.iscale > 0) {
+            y_lo = (int)clampi(tdiv(-fraction_base, s.iscale) - 1, 0, VH);
+            y_hi = (int)clampi(tdiv(((i64)height << 16) - fraction_base, s.iscale) + 2, 0, VH);
+        }
+        // four rows per step, each stage's loads issued together so that their latencies overlap
+        for (int yb = y_lo; yb < y_hi; yb += 4) {
+            i64 sv[4]; bool live[4]; unsigned int row_meta[4]; float row_clip[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int y = yb + j;
+                sv[j] = (fraction_base + mul64((i64)y, s.iscale)) >> 16;
+                live[j] = y < y_hi && sv[j] >= 0 && sv[j] < height;
+                const size_t i = (size_t)(y < VH ? y : VH - 1) * SW + x;
+                row_meta[j] = meta[i]; row_clip[j] = clip_depth[i];
             }
-            if (!visible) continue;
-            size_t t = ((size_t)s.id * m->spr_max_h + sv) * m->spr_max_w + su;
-            if (!m->spr_opaque[t]) continue;
-            i64 post_screen_top = (s.top_fixed + mul64(s.yscale, m->spr_post_top[t])) >> 16;
-            if ((i64)y < post_screen_top) continue;
-            frame[i] = m->colormap[shade * 256 + m->spr_atlas[t]];
+            unsigned char opaque[4], post_top[4], texel[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                opaque[j] = 0; post_top[j] = 0; texel[j] = 0;
+                if (!live[j]) continue;
+                const int cw = (int)(row_meta[j] & META_WALL_MASK) - 1;
+                bool visible;
+                if (cw >= 0) {
+                    const WallRec &cg = recs[cw];
+                    i64 cnear = min64(cg.dl, cg.dr), cfar = max64(cg.dl, cg.dr);
+                    const float4 cl = *reinterpret_cast<const float4 *>(m->walls + 4 * cw);
+                    float side = (cl.z - cl.x) * (s.y - cl.y) - (cl.w - cl.y) * (s.x - cl.x);
+                    visible = (cnear > s.depth_fixed) || ((cfar > s.depth_fixed) && (side <= 0));
+                } else {
+                    visible = s.depth < row_clip[j];
+                }
+                live[j] = visible;
+                if (!visible) continue;
+                const size_t t = ((size_t)s.id * m->spr_max_h + sv[j]) * m->spr_max_w + su;
+                opaque[j] = m->spr_opaque[t]; post_top[j] = m->spr_post_top[t]; texel[j] = m->spr_atlas[t];
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (!live[j] || !opaque[j]) continue;
+                const int y = yb + j;
+                i64 post_screen_top = (s.top_fixed + mul64(s.yscale, post_top[j])) >> 16;
+                if ((i64)y < post_screen_top) continue;
+                frame[(size_t)y * SW + x] = m->colormap[shade * 256 + texel[j]];
+            }
         }
     }
 }
