@@ -2117,23 +2117,40 @@ __global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lan
     const float4 bl = *reinterpret_cast<const float4 *>(m->walls + 4 * bw);
     float bdx = bl.z - bl.x, bdy = bl.w - bl.y;
     bool owns = (x >= bg.sl) && (x < bg.sr);
+    // The sprites that can show in this column at all (alive, in front, horizontally covering it and
+    // not hidden by the column's blocking linedef), as a bit set: the painter's loop below runs once
+    // per drawn sprite and would otherwise test every slot each time.
+    u64 cover[8] = {0, 0, 0, 0, 0, 0, 0, 0};   // sprite_slots <= 512
+#pragma unroll
+    for (int word = 0; word < 8; ++word) {
+        if (word * 64 >= A) continue;          // the same in every thread
+        u64 bits = 0;
+        const int end = A - word * 64 < 64 ? A - word * 64 : 64;
+        for (int b = 0; b < end; ++b) {
+            const SpriteRec &s = sp[word * 64 + b];
+            if (!((s.flags & 1) && (x >= s.left) && (x < s.right) && (s.depth > 0))) continue;
+            bool ray_visible = s.depth < wall_distance;
+            if (!ray_visible) {
+                float bside = bdx * (s.y - bl.y) - bdy * (s.x - bl.x);
+                bool behind = (bnear > s.depth_fixed) || ((bfar > s.depth_fixed) && (bside <= 0));
+                ray_visible = !owns || behind;
+            }
+            if (ray_visible) bits |= 1ULL << b;
+        }
+        cover[word] = bits;
+    }
     // painter's order far -> near: repeatedly take the farthest candidate nearer than the last one
     float last_depth = GD_INF; int last_slot = A;
     for (;;) {
         float pick_depth = -GD_INF; int pick = -1;
-        for (int a = 0; a < A; ++a) {
-            const SpriteRec &s = sp[a];
-            if (!((s.flags & 1) && (x >= s.left) && (x < s.right) && (s.depth > 0))) continue;
-            // strictly before (last_depth, last_slot) in (depth, slot) order
-            if (!(s.depth < last_depth || (s.depth == last_depth && a < last_slot))) continue;
-            if (s.depth > pick_depth || (s.depth == pick_depth && a > pick)) {
-                bool ray_visible = s.depth < wall_distance;
-                if (!ray_visible) {
-                    float bside = bdx * (s.y - bl.y) - bdy * (s.x - bl.x);
-                    bool behind = (bnear > s.depth_fixed) || ((bfar > s.depth_fixed) && (bside <= 0));
-                    ray_visible = !owns || behind;
-                }
-                if (ray_visible) { pick_depth = s.depth; pick = a; }
+#pragma unroll
+        for (int word = 0; word < 8; ++word) {
+            for (u64 bits = cover[word]; bits; bits &= bits - 1) {
+                const int a = word * 64 + __ffsll((long long)bits) - 1;
+                const float depth = sp[a].depth;
+                // strictly before (last_depth, last_slot) in (depth, slot) order
+                if (!(depth < last_depth || (depth == last_depth && a < last_slot))) continue;
+                if (depth > pick_depth || (depth == pick_depth && a > pick)) { pick_depth = depth; pick = a; }
             }
         }
         if (pick < 0) break;
