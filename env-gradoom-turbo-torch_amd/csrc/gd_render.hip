@@ -128,6 +128,8 @@ struct Scratch {    // per-chunk working memory, sized at create
     unsigned char *frame;  // [L,240,320] when the caller wants no indexed output
     u64 *block_hit;        // [L,320] nearest blocking linedef of the column ray: float bits of the distance << 32 |
                            // slot in blocking_walls, all ones when no ray hits (engine.py:10534-10557)
+    unsigned char *strip_key;  // [L*5] expected traversal length of each (lane, 64-column strip)
+    int *strip_order;      // [L*5] strips, longest expected traversal first
     int *status;           // [1] sticky overflow flags
     float *level_reach;    // [L, floor levels + ceiling levels] lower bound of the distance from the
                            // camera to any point inside a sector with that plane level
@@ -1156,6 +1158,7 @@ __device__ __forceinline__ void endpoint_owner(const ColumnCtx &cc, int w, const
 
 #ifdef GD_PROFILE
 __device__ unsigned long long g_profile[16];
+__device__ unsigned int g_wave_log[3 * 32768];   // per strip: clock ticks, candidate total, passes
 #define PROF_T(var) long long var = wall_clock64()
 #define PROF_ADD(slot, t0, t1) prof_acc[slot] += (t1) - (t0)
 #define PROF_MARK(slot, tprev) do { long long tn_ = wall_clock64(); if (threadIdx.x == 0) atomicAdd(&g_profile[slot], (unsigned long long)(tn_ - tprev)); tprev = tn_; } while (0)
@@ -1884,6 +1887,51 @@ __device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const Col
     }
 }
 
+// How long a strip's traversal runs is set by the column that crosses the most portals: the
+// two-sided linedefs its ray hits before the nearest blocking one.  Strips differ by a factor of
+// ten, and a launch ends with its longest wavefront, so the traversal takes the strips longest
+// first: strip_key_kernel counts (one wavefront per strip, one lane per column, a walk over the
+// column's candidate list), strip_order_kernel sorts the counts (one block, counting sort).
+__global__ void __launch_bounds__(256) strip_key_kernel(int lane_count, Scratch sc) {
+    const int strip = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int local = strip / (SW / 64);
+    if (local >= lane_count) return;
+    const int x = (strip - local * (SW / 64)) * 64 + (threadIdx.x & 63);
+    const u64 hit = sc.block_hit[(size_t)local * SW + x];
+    const float solid = hit == ~0ULL ? GD_INF : __uint_as_float((unsigned)(hit >> 32));
+    const Cand *list = sc.cand + (size_t)local * CAND_MAX * SW + x;
+    int count = sc.cand_count[(size_t)local * SW + x];
+    if (count > CAND_MAX) count = CAND_MAX;
+    int portals = 0;
+    for (int k0 = 0; k0 < count; k0 += 4) {
+        uint4 raw[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) raw[j] = *reinterpret_cast<const uint4 *>(list + (size_t)(k0 + j < count ? k0 + j : count - 1) * SW);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            union { uint4 r; Cand c; } u; u.r = raw[j];
+            portals += (k0 + j < count && u.c.s1 >= 0 && (u.c.flags & CF_GEO) && u.c.dist < solid) ? 1 : 0;
+        }
+    }
+#pragma unroll
+    for (int step = 1; step < 64; step <<= 1) portals = max(portals, __shfl_xor(portals, step));
+    if ((threadIdx.x & 63) == 0) sc.strip_key[strip] = (unsigned char)portals;   // at most CAND_MAX
+}
+
+__global__ void __launch_bounds__(1024) strip_order_kernel(int strips, Scratch sc) {
+    __shared__ int histogram[CAND_MAX + 1], position[CAND_MAX + 1];
+    for (int k = threadIdx.x; k <= CAND_MAX; k += blockDim.x) histogram[k] = 0;
+    __syncthreads();
+    for (int s = threadIdx.x; s < strips; s += blockDim.x) atomicAdd(&histogram[sc.strip_key[s]], 1);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int running = 0;
+        for (int k = CAND_MAX; k >= 0; --k) { position[k] = running; running += histogram[k]; }
+    }
+    __syncthreads();
+    for (int s = threadIdx.x; s < strips; s += blockDim.x) sc.strip_order[atomicAdd(&position[sc.strip_key[s]], 1)] = s;
+}
+
 // One wavefront per (lane, 64-column strip).  Strips share nothing but read-only tables; a
 // work-group is WALL_STRIPS_PER_GROUP consecutive strips only so that the LDS copies of those
 // tables are paid once per group rather than once per wavefront (which would cap the CU at a
@@ -1896,9 +1944,10 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
     __shared__ float4 sector_lds[LDS_SECTORS];
     __shared__ unsigned char tex_lds[LDS_TEXTURES];
     const int wave_in_group = threadIdx.x >> 6;
-    const int strip_index = blockIdx.x * WALL_STRIPS_PER_GROUP + wave_in_group;
+    const int strip_slot = blockIdx.x * WALL_STRIPS_PER_GROUP + wave_in_group;
+    const bool live = strip_slot < lane_count * (SW / 64);
+    const int strip_index = live ? sc.strip_order[strip_slot] : 0;
     const int local = strip_index / (SW / 64);
-    const bool live = local < lane_count;
     Tables tb;
     stage_tables(m, sector_lds, tex_lds, tb);
     if ((threadIdx.x & 63) == 0 && live) lane_ctxs[wave_in_group] = sc.ctx[local];
@@ -1942,6 +1991,9 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
     const int sectors = m->sector_count;
     for (int pass = 0; pass < sectors; ++pass) {
         PROF_T(t0);
+#ifdef GD_PROFILE
+        prof_acc[7] += 1;
+#endif
         if (!done) pass_select(cc, st, boundary_has_po, pc);
         PROF_T(t1);
         PROF_ADD(0, t0, t1);
@@ -1986,10 +2038,17 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
     masked_midtexture(cc, st, pb);
 #ifdef GD_PROFILE
     long long t7 = wall_clock64();
+    int prof_cands = cc.count;
+    for (int step = 1; step < 64; step <<= 1) prof_cands += __shfl_xor(prof_cands, step);
     prof_acc[3] += t6 - t5; prof_acc[4] += t7 - t6; prof_acc[6] += t7 - prof_start;
     if ((threadIdx.x & 63) == 0) {   // one sample per wave: phases are wave-synchronous
         for (int k = 0; k < 7; ++k) atomicAdd(&g_profile[k], (unsigned long long)prof_acc[k]);
         atomicAdd(&g_profile[7], 1ULL);
+        if (strip_index < 32768) {
+            g_wave_log[3 * strip_index] = (unsigned int)prof_acc[6];
+            g_wave_log[3 * strip_index + 1] = (unsigned int)prof_cands;
+            g_wave_log[3 * strip_index + 2] = (unsigned int)prof_acc[7];
+        }
     }
 #endif
 }
@@ -2426,6 +2485,8 @@ int launch_chunk(gd_renderer *r, Scratch &sc, const gd_lanes_desc *lanes, const 
     hipLaunchKernelGGL(flat_finish_kernel, dim3(count), dim3(SW), 0, flat_stream, r->dm, count, sc, frame_base, frame_stride);
     mark();
     if (overlap) HIP_TRY(hipEventRecord(r->flat_event, side));
+    hipLaunchKernelGGL(strip_key_kernel, dim3((count * (SW / 64) + 3) / 4), dim3(256), 0, stream, count, sc);
+    hipLaunchKernelGGL(strip_order_kernel, dim3(1), dim3(1024), 0, stream, count * (SW / 64), sc);
     hipLaunchKernelGGL(wall_columns_kernel, dim3((count * (SW / 64) + WALL_STRIPS_PER_GROUP - 1) / WALL_STRIPS_PER_GROUP), dim3(64 * WALL_STRIPS_PER_GROUP), 0, stream, r->dm, count, sc, frame_base, frame_stride);
     mark();
     if (overlap) HIP_TRY(hipStreamWaitEvent(stream, r->flat_event, 0));
@@ -2576,6 +2637,8 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)VH, &sc.row_slope);
     if (rc == GD_OK) rc = scratch_alloc(r, L * 32, &sc.step_scale);
     if (rc == GD_OK) rc = scratch_alloc(r, L * SW, &sc.block_hit);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * (SW / 64), &sc.strip_key);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * (SW / 64), &sc.strip_order);
     if (rc == GD_OK) rc = scratch_alloc(r, 1, &sc.status);
     if (rc == GD_OK && hipMemset(sc.status, 0, sizeof(int)) != hipSuccess) rc = fail(GD_E_HIP, "hipMemset status");
     if (rc == GD_OK) {
@@ -2670,6 +2733,10 @@ int gd_renderer_set_sector_lights(gd_renderer *r, const float *lights, void *str
 
 #ifdef GD_PROFILE
 /* profiling build only: cumulative per-wave clock ticks of the wall kernel's phases */
+int gd_wave_log_read(unsigned int *out) {
+    HIP_TRY(hipMemcpyFromSymbol(out, HIP_SYMBOL(g_wave_log), sizeof(unsigned int) * 3 * 32768));
+    return GD_OK;
+}
 int gd_profile_read(unsigned long long *out, int reset) {
     HIP_TRY(hipMemcpyFromSymbol(out, HIP_SYMBOL(g_profile), sizeof(unsigned long long) * 16));
     if (reset) { unsigned long long zero[16] = {0}; HIP_TRY(hipMemcpyToSymbol(HIP_SYMBOL(g_profile), zero, sizeof(zero))); }
