@@ -857,8 +857,10 @@ struct LaneTables {
     const i64 *step_scale;    // this lane's [2][16]
     int floors;
 };
-__device__ __forceinline__ unsigned char flat_pixel_tabled(const Tables &tb, const unsigned char *colormap, const LaneCtx &c, const LaneTables &lt,
-                                                           i64 yslope, int level_index, int sector, bool is_floor, int px, int py) {
+// Returns the texel's offset in the texture atlas and the colormap row, so that a caller can
+// have several texel loads in flight before it needs any of them.
+__device__ __forceinline__ size_t flat_sample_tabled(const Tables &tb, const LaneCtx &c, const LaneTables &lt,
+                                                     i64 yslope, int level_index, int sector, bool is_floor, int px, int py, int *colormap_row) {
     const gd_map_desc *m = tb.m;
     const int texture = is_floor ? tb.floor_tex(sector) : tb.ceil_tex(sector);
     const int width_bits = tb.width_bits(texture), height_bits = tb.height_bits(texture);
@@ -874,14 +876,13 @@ __device__ __forceinline__ unsigned char flat_pixel_tabled(const Tables &tb, con
     const i64 xfrac = ((mul64(distance, basexfrac) >> 16) + pviewx) & UINT32_MASK;
     const i64 yfrac = ((mul64(distance, baseyfrac) >> 16) + pviewy) & UINT32_MASK;
     const i64 u = xfrac >> (32 - width_bits), v = yfrac >> (32 - height_bits);
-    const unsigned char index = m->tex_atlas[((size_t)texture * m->tex_max_h + v) * m->tex_max_w + u];
     const float light = tb.light(sector) + (float)(c.flash_light * 16);
     i64 row = c.center_fixed - (i64)py * FIXED_UNIT;
     if (row < 0) row = -row;
     const i64 visibility = min64(mul64(glob, row) >> 16, 24 * FIXED_UNIT);
     const i64 plane_shade = 64 * FIXED_UNIT - ((i64)light + 12) * (FIXED_UNIT / 4);
-    const i64 shade = clampi((plane_shade - visibility) >> 16, 0, 31);
-    return colormap[shade * 256 + index];
+    *colormap_row = (int)clampi((plane_shade - visibility) >> 16, 0, 31);
+    return ((size_t)texture * m->tex_max_h + v) * m->tex_max_w + u;
 }
 
 // Visplane continuity repair and shading for one lane (engine.py:11026-11171).
@@ -2059,7 +2060,8 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
 // one, the sector the per-pixel plane rays selected (engine.py:11145-11163).  Doing both here
 // shades every pixel once, in a kernel light enough to run at full occupancy.
 // ---------------------------------------------------------------------------------------------
-#define SHADE_TILES 13   // 256-pixel tiles per block: 260 tiles per view = 20 blocks per lane
+#define SHADE_TILES 12   // 256-pixel tiles per block: 260 tiles per view = 22 blocks per lane
+#define SHADE_GROUP 4    // tiles per step
 __global__ void __launch_bounds__(256) plane_shade_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
     const gd_map_desc *m = &dm.d;
     __shared__ float4 sector_lds[LDS_SECTORS];
@@ -2084,32 +2086,53 @@ __global__ void __launch_bounds__(256) plane_shade_kernel(DeviceMap dm, int lane
     LaneTables lt; lt.level_plane = level_plane_lds; lt.step_scale = step_scale_lds; lt.floors = floors;
     const LaneCtx &c = sc.ctx[local];
     unsigned char *frame = frame_base + (size_t)local * frame_stride;
-    for (int tile = 0; tile < SHADE_TILES; ++tile) {
-        const int pixel = (blockIdx.x * SHADE_TILES + tile) * 256 + threadIdx.x;
-        if (pixel >= VH * SW) break;
-        const int y = pixel / SW, x = pixel - y * SW;
-        const size_t i = (size_t)local * VH * SW + pixel;
-        const unsigned int meta = sc.meta[i];
-        if (meta & META_FILLED) continue;
-        const int ps = (int)((meta >> META_SECTOR_SHIFT) & META_SECTOR_MASK) - 1;
-        const bool claimed = ps >= 0;
-        const bool is_floor = claimed ? (meta & META_FLOOR) != 0 : ((float)y - flat_center(c)) > 0;
-        const int sector = claimed ? ps : (int)sc.flat_sector[i];
-        if (!(meta & META_MASKED)) {
-            if (tabled) {
-                const unsigned short pair = sector < tb.sector_cached ? sector_level_lds[sector] : dm.sector_level[sector];
-                frame[pixel] = flat_pixel_tabled(tb, colormap_lds, c, lt, sc.row_slope[(size_t)local * VH + y], is_floor ? (pair & 0xFF) : (pair >> 8),
-                                                 sector, is_floor, x, y);
-            } else {
-                frame[pixel] = flat_pixel(tb, colormap_lds, c, sector, is_floor, x, y);
-            }
+    // SHADE_GROUP tiles per step and three stages per step (per-pixel words, texels, stores), each
+    // stage's loads issued together so that their latencies overlap
+    for (int tile0 = 0; tile0 < SHADE_TILES; tile0 += SHADE_GROUP) {
+        unsigned int meta[SHADE_GROUP]; unsigned short flat_sector[SHADE_GROUP]; unsigned char flat_flags[SHADE_GROUP];
+        int pixels[SHADE_GROUP];
+#pragma unroll
+        for (int j = 0; j < SHADE_GROUP; ++j) {
+            const int pixel = (blockIdx.x * SHADE_TILES + tile0 + j) * 256 + threadIdx.x;
+            pixels[j] = (tile0 + j < SHADE_TILES && pixel < VH * SW) ? pixel : -1;
+            const size_t i = (size_t)local * VH * SW + (pixels[j] < 0 ? 0 : pixels[j]);
+            meta[j] = sc.meta[i]; flat_sector[j] = sc.flat_sector[i]; flat_flags[j] = sc.flat_flags[i];
         }
-        // plane fallback occluder for sprites where the flat ray was unresolved (engine.py:13417-13422)
-        if (claimed && (sc.flat_flags[i] & 1) && !finitef(sc.clip_depth[i])) {
-            const float flat_center_px = (103.0f + c.pitch_offset) + 0.5f;
-            float plane_height = is_floor ? (c.view_z - tb.floor_h(ps)) : (tb.ceil_h(ps) - c.view_z);
-            float plane_denominator = fmaxf(fabsf((float)y - flat_center_px), 0.5f);
-            sc.clip_depth[i] = plane_height * 192.0f / plane_denominator;
+        size_t texel_at[SHADE_GROUP]; int colormap_row[SHADE_GROUP]; unsigned char texel[SHADE_GROUP];
+        bool shade[SHADE_GROUP];
+#pragma unroll
+        for (int j = 0; j < SHADE_GROUP; ++j) {
+            const int pixel = pixels[j];
+            shade[j] = tabled && pixel >= 0 && !(meta[j] & (META_FILLED | META_MASKED));
+            texel[j] = 0; colormap_row[j] = 0; texel_at[j] = 0;
+            if (!shade[j]) continue;
+            const int y = pixel / SW, x = pixel - y * SW;
+            const int ps = (int)((meta[j] >> META_SECTOR_SHIFT) & META_SECTOR_MASK) - 1;
+            const bool is_floor = ps >= 0 ? (meta[j] & META_FLOOR) != 0 : ((float)y - flat_center(c)) > 0;
+            const int sector = ps >= 0 ? ps : (int)flat_sector[j];
+            const unsigned short pair = sector < tb.sector_cached ? sector_level_lds[sector] : dm.sector_level[sector];
+            texel_at[j] = flat_sample_tabled(tb, c, lt, sc.row_slope[(size_t)local * VH + y], is_floor ? (pair & 0xFF) : (pair >> 8),
+                                             sector, is_floor, x, y, &colormap_row[j]);
+            texel[j] = m->tex_atlas[texel_at[j]];
+        }
+#pragma unroll
+        for (int j = 0; j < SHADE_GROUP; ++j) {
+            const int pixel = pixels[j];
+            if (pixel < 0 || (meta[j] & META_FILLED)) continue;
+            const int y = pixel / SW, x = pixel - y * SW;
+            const size_t i = (size_t)local * VH * SW + pixel;
+            const int ps = (int)((meta[j] >> META_SECTOR_SHIFT) & META_SECTOR_MASK) - 1;
+            const bool claimed = ps >= 0;
+            const bool is_floor = claimed ? (meta[j] & META_FLOOR) != 0 : ((float)y - flat_center(c)) > 0;
+            if (shade[j]) frame[pixel] = colormap_lds[colormap_row[j] * 256 + texel[j]];
+            else if (!(meta[j] & META_MASKED)) frame[pixel] = flat_pixel(tb, colormap_lds, c, claimed ? ps : (int)flat_sector[j], is_floor, x, y);
+            // plane fallback occluder for sprites where the flat ray was unresolved (engine.py:13417-13422)
+            if (claimed && (flat_flags[j] & 1) && !finitef(sc.clip_depth[i])) {
+                const float flat_center_px = (103.0f + c.pitch_offset) + 0.5f;
+                float plane_height = is_floor ? (c.view_z - tb.floor_h(ps)) : (tb.ceil_h(ps) - c.view_z);
+                float plane_denominator = fmaxf(fabsf((float)y - flat_center_px), 0.5f);
+                sc.clip_depth[i] = plane_height * 192.0f / plane_denominator;
+            }
         }
     }
 }
