@@ -99,6 +99,9 @@ struct DeviceMap {  // device copy of gd_map_desc (device pointers) + fixed tabl
     const i64 *fine_sine;     // [8192]
     const i64 *fine_tangent;  // [4096]
     const float *cosine_correction;  // [320] cos(native_ray_offsets), supplied by the host
+    const float *inverse_cosine;     // [320] 1 / cosine_correction, correctly rounded
+    float strip_reach_scale[SW / 64];// per 64-column strip: 1.001 / (its smallest cosine_correction), inf if not positive
+    float fine_inverse;              // 1 / fine_cell
     // Sectors grouped by plane level, floors (in floor_levels order) then ceilings: CSR over
     // floor_level_count + ceil_level_count rows into level_boxes, one padded bounding box
     // (x0, y0, x1, y1) per sector outside which no point tests inside that sector.
@@ -674,19 +677,16 @@ __global__ void flat_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
     // one ulp of p / cc, and RN(q + RN(p - cc * q) * y) is then the correctly rounded quotient
     // (Markstein's theorem; the inner product is exact in an FMA) as long as nothing over- or
     // underflows, which the range tests on both operands ensure.
-    const float inv_cc = 1.0f / cc;
+    const float inv_cc = dm.inverse_cosine[x];
     const bool cc_plain = cc >= 0.5f && cc <= 1.0f;
-    const float inv_fine = 1.0f / m->fine_cell;   // a reciprocal is fine here: see fine_lookup
+    const float inv_fine = dm.fine_inverse;       // a reciprocal is fine here: see fine_lookup_cells
     // the probe point camera + ray * cd in raster cell units, as one multiply-add per axis
     const float cell_x0 = (c.x - m->grid_min_x) * inv_fine, cell_y0 = (c.y - m->grid_min_y) * inv_fine;
     const float cell_dx = rc * inv_fine, cell_dy = rs * inv_fine;
     const int slot_in_wave = threadIdx.x & 63;
     // cd <= perpendicular / (smallest cc of the wavefront): with it a level whose every sector is
     // farther than that from the camera is dropped for the whole wavefront at once
-    float cc_floor = cc;
-#pragma unroll
-    for (int step = 1; step < 64; step <<= 1) cc_floor = fminf(cc_floor, __shfl_xor(cc_floor, step));
-    const float reach_scale = cc_floor > 0.0f ? 1.001f / cc_floor : GD_INF;
+    const float reach_scale = dm.strip_reach_scale[__builtin_amdgcn_readfirstlane(x >> 6)];
     float best = GD_INF; int best_sector = -1;
     bool done = false;
     for (int base = 0; base < level_count && !done; base += 64) {
@@ -2593,6 +2593,17 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     if (rc == GD_OK) rc = upload(r, sine.data(), sine.size(), &r->dm.fine_sine);
     if (rc == GD_OK) rc = upload(r, tangent.data(), tangent.size(), &r->dm.fine_tangent);
     if (rc == GD_OK) rc = upload(r, cosine_correction, (size_t)SW, &r->dm.cosine_correction);
+    {
+        std::vector<float> inverse(SW);
+        for (int x = 0; x < SW; ++x) inverse[x] = 1.0f / cosine_correction[x];   // IEEE division, as on the device
+        if (rc == GD_OK) rc = upload(r, inverse.data(), inverse.size(), &r->dm.inverse_cosine);
+        for (int strip = 0; strip < SW / 64; ++strip) {
+            float smallest = cosine_correction[strip * 64];
+            for (int x = strip * 64; x < strip * 64 + 64; ++x) smallest = std::fmin(smallest, cosine_correction[x]);
+            r->dm.strip_reach_scale[strip] = smallest > 0.0f ? 1.001f / smallest : GD_INF;
+        }
+        r->dm.fine_inverse = 1.0f / h->fine_cell;
+    }
     {
         std::vector<int> box_ofs;
         std::vector<float4> boxes;
