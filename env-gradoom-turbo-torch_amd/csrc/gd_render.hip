@@ -1937,7 +1937,11 @@ __global__ void __launch_bounds__(1024) strip_order_kernel(int strips, Scratch s
 // work-group is WALL_STRIPS_PER_GROUP consecutive strips only so that the LDS copies of those
 // tables are paid once per group rather than once per wavefront (which would cap the CU at a
 // couple of wavefronts per SIMD).  After the staging barrier the wavefronts never meet again.
-#define WALL_STRIPS_PER_GROUP 2
+#define WALL_STRIPS_PER_GROUP 1
+// Unused LDS that caps the kernel at two wavefronts per SIMD: its 166 registers per lane would
+// otherwise fill the register file with three, and the flat kernels on the side stream could not
+// run beside it at all.
+#define WALL_LDS_PAD 3072
 __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amdgpu_waves_per_eu(3, 3))) wall_columns_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
     const gd_map_desc *m = &dm.d;
     __shared__ LaneCtx lane_ctxs[WALL_STRIPS_PER_GROUP];
@@ -2387,9 +2391,8 @@ int fail(int code, const std::string &message) { g_error = message; return code;
 
 // The flat kernels (bound by the vector ALU) and the wall kernels (bound by memory latency) of a
 // chunk are independent until plane shading, so the flats run on a side stream forked from the
-// caller's stream and joined back before plane shading.  (Cutting a batch into smaller chunks
-// pipelined over several streams measured slower: the wall traversal has a long per-wavefront
-// critical path and wants as many lanes per launch as possible.)
+// caller's stream and joined back before plane shading.  (Cutting a batch into chunks or halves
+// pipelined over more streams measured no faster: the kernels already share the machine.)
 struct gd_renderer {
     DeviceMap dm;
     Scratch sc;
@@ -2510,7 +2513,7 @@ int launch_chunk(gd_renderer *r, Scratch &sc, const gd_lanes_desc *lanes, const 
     if (overlap) HIP_TRY(hipEventRecord(r->flat_event, side));
     hipLaunchKernelGGL(strip_key_kernel, dim3((count * (SW / 64) + 3) / 4), dim3(256), 0, stream, count, sc);
     hipLaunchKernelGGL(strip_order_kernel, dim3(1), dim3(1024), 0, stream, count * (SW / 64), sc);
-    hipLaunchKernelGGL(wall_columns_kernel, dim3((count * (SW / 64) + WALL_STRIPS_PER_GROUP - 1) / WALL_STRIPS_PER_GROUP), dim3(64 * WALL_STRIPS_PER_GROUP), 0, stream, r->dm, count, sc, frame_base, frame_stride);
+    hipLaunchKernelGGL(wall_columns_kernel, dim3((count * (SW / 64) + WALL_STRIPS_PER_GROUP - 1) / WALL_STRIPS_PER_GROUP), dim3(64 * WALL_STRIPS_PER_GROUP), WALL_LDS_PAD, stream, r->dm, count, sc, frame_base, frame_stride);
     mark();
     if (overlap) HIP_TRY(hipStreamWaitEvent(stream, r->flat_event, 0));
     hipLaunchKernelGGL(plane_shade_kernel, dim3(((VH * SW + 255) / 256 + SHADE_TILES - 1) / SHADE_TILES, count), dim3(256), 0, stream, r->dm, count, sc, frame_base, frame_stride);
