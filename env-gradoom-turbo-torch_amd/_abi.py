@@ -114,7 +114,7 @@ LANE_ARRAYS = (
     ("sprite_fullbright", np.uint8),
 )
 
-OUT_FIELDS = ("indexed", "obs", "frames", "reset_mask", "rgb")
+OUT_FIELDS = ("indexed", "obs", "frames", "reset_mask", "rgb", "final_frames")
 
 
 class MapDesc(C.Structure):

@@ -2306,7 +2306,8 @@ __global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lan
 // observation: _triton_kernels.py:120-177 + engine.py:9545-9548 / 2443-2450
 // ---------------------------------------------------------------------------------------------
 __global__ void observe_kernel(const unsigned char *indexed, size_t lane_stride, int source_rows, const unsigned char *playpal,
-                               int lane_count, unsigned char *obs, unsigned char *frames, const unsigned char *reset_mask, int stack_mode) {
+                               int lane_count, unsigned char *obs, unsigned char *frames, const unsigned char *reset_mask, int stack_mode,
+                               unsigned char *final_frames) {
     __shared__ unsigned char pal[768];
     for (int k = threadIdx.x; k < 768; k += blockDim.x) pal[k] = playpal[k];
     __syncthreads();
@@ -2354,11 +2355,21 @@ __global__ void observe_kernel(const unsigned char *indexed, size_t lane_stride,
     if (obs) obs[(size_t)n * F + pixel] = gray;
     if (frames) {
         unsigned char *stack = frames + (size_t)n * GD_FRAME_STACK * F + pixel;
+        unsigned char *copy = final_frames ? final_frames + (size_t)n * GD_FRAME_STACK * F + pixel : nullptr;
         if (reset_mask && reset_mask[n]) {
             for (int k = 0; k < GD_FRAME_STACK; ++k) stack[k * F] = gray;
+            if (copy) for (int k = 0; k < GD_FRAME_STACK; ++k) copy[k * F] = gray;
         } else if (stack_mode == GD_STACK_STEP) {
-            for (int k = 0; k < GD_FRAME_STACK - 1; ++k) stack[k * F] = stack[(k + 1) * F];
+            unsigned char kept[GD_FRAME_STACK - 1];
+            for (int k = 0; k < GD_FRAME_STACK - 1; ++k) kept[k] = stack[(k + 1) * F];
+            for (int k = 0; k < GD_FRAME_STACK - 1; ++k) stack[k * F] = kept[k];
             stack[(GD_FRAME_STACK - 1) * F] = gray;
+            if (copy) {
+                for (int k = 0; k < GD_FRAME_STACK - 1; ++k) copy[k * F] = kept[k];
+                copy[(GD_FRAME_STACK - 1) * F] = gray;
+            }
+        } else if (copy) {
+            for (int k = 0; k < GD_FRAME_STACK; ++k) copy[k * F] = stack[k * F];   // lane left as it was
         }
     }
 }
@@ -2523,12 +2534,14 @@ int launch_chunk(gd_renderer *r, Scratch &sc, const gd_lanes_desc *lanes, const 
         hipLaunchKernelGGL(sprite_columns_kernel, dim3(count), dim3(SW), shared, stream, r->dm, *lanes, base, count, sc, frame_base, frame_stride);
     }
     mark();
+    if (out->final_frames && !out->frames) return fail(GD_E_ARG, "final_frames needs frames");
     if (out->obs || out->frames) {
         const size_t F = (size_t)GD_OBS_SIZE * GD_OBS_SIZE;
         hipLaunchKernelGGL(observe_kernel, dim3((GD_OBS_SIZE * GD_OBS_SIZE + 255) / 256, count), dim3(256), 0, stream,
                            frame_base, frame_stride, VH, m.playpal, count, out->obs ? out->obs + (size_t)base * F : nullptr,
                            out->frames ? out->frames + (size_t)base * GD_FRAME_STACK * F : nullptr,
-                           out->reset_mask ? out->reset_mask + base : nullptr, out->stack_mode);
+                           out->reset_mask ? out->reset_mask + base : nullptr, out->stack_mode,
+                           out->final_frames ? out->final_frames + (size_t)base * GD_FRAME_STACK * F : nullptr);
     }
     if (out->rgb) {
         size_t pixels = (size_t)count * frame_stride;
@@ -2794,7 +2807,7 @@ int gd_observe(const uint8_t *indexed, int32_t source_rows, const uint8_t *playp
         hipLaunchKernelGGL(observe_kernel, dim3((GD_OBS_SIZE * GD_OBS_SIZE + 255) / 256, count), dim3(256), 0, static_cast<hipStream_t>(stream),
                            indexed + (size_t)base * source_rows * SW, (size_t)source_rows * SW, source_rows, playpal, count,
                            obs ? obs + (size_t)base * F : nullptr, frames ? frames + (size_t)base * GD_FRAME_STACK * F : nullptr,
-                           reset_mask ? reset_mask + base : nullptr, stack_mode);
+                           reset_mask ? reset_mask + base : nullptr, stack_mode, nullptr);
     }
     HIP_TRY(hipGetLastError());
     return GD_OK;

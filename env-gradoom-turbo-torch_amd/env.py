@@ -189,11 +189,14 @@ class GraDoomVecEnv:
         return self._device_observations(self.frames), self.signal_buffer
 
     def step_device(self, actions: torch.Tensor) -> DeviceTransition:
+        return self._step(actions, None)
+
+    def _step(self, actions: torch.Tensor, final_frames) -> DeviceTransition:
         if self.closed:
             raise RuntimeError("cannot step a closed environment")
         indices = self._require_device_tensor(actions, "actions", shape=(self.num_envs,), dtypes=INDEX_DTYPES).to(torch.int64)
         rewards, terminated, truncated = self._dynamics.step(indices)
-        self._renderer.render(self._dynamics.lane_state(), frames=self.frames)
+        self._renderer.render(self._dynamics.lane_state(), frames=self.frames, final_frames=final_frames)
         self._update_signals()
         return DeviceTransition(
             observations=self._device_observations(self.frames), rewards=rewards, terminated=terminated, truncated=truncated,
@@ -201,8 +204,10 @@ class GraDoomVecEnv:
         )
 
     def step_and_reset_device(self, actions: torch.Tensor, reset_seeds: torch.Tensor) -> DeviceAutoResetTransition:
-        transition = self.step_device(actions)
-        final_observations = transition.observations.clone()
+        # the final-observation clone (env.py:915) is written by the observation kernel of the step
+        final_frames = torch.empty_like(self.frames)
+        transition = self._step(actions, final_frames)
+        final_observations = self._device_observations(final_frames)
         final_signals = transition.signals.clone()
         final_info_histories = transition.info_histories.clone()
         done = transition.terminated | transition.truncated

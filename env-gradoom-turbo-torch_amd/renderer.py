@@ -173,7 +173,7 @@ class HipRenderer:
             desc.sprite_depth = _require(depth, "sprite_depth", torch.float32, (count, slots), device).data_ptr()
         return desc, keep
 
-    def _out_desc(self, count, indexed, obs, frames, reset_mask, rgb, stack_only_masked=False):
+    def _out_desc(self, count, indexed, obs, frames, reset_mask, rgb, stack_only_masked=False, final_frames=None):
         device = self.device
         out = _abi.FrameOut()
         out.stack_mode = _abi.STACK_RESET if stack_only_masked else _abi.STACK_STEP
@@ -190,22 +190,29 @@ class HipRenderer:
             out.reset_mask = _require(mask, "reset_mask", torch.uint8, (count,), device).data_ptr()
         if rgb is not None:
             out.rgb = _require(rgb, "rgb", torch.uint8, (count, 240, 320, 3), device).data_ptr()
+        if final_frames is not None:
+            if frames is None:
+                raise ValueError("final_frames needs frames")
+            out.final_frames = _require(final_frames, "final_frames", torch.uint8, (count, 4, 84, 84), device).data_ptr()
         return out, keep
 
     # ------------------------------------------------------------------ entry points
     def render(self, lanes: LaneState, *, indexed=None, obs=None, frames=None, reset_mask=None, rgb=None,
-               stack_only_masked: bool = False) -> None:
+               stack_only_masked: bool = False, final_frames=None) -> None:
         """One frame for every lane, written into the given (preallocated) tensors.
 
         ``frames`` is rolled by one and the new observation appended (``engine.py:9545-9548``); lanes
         whose ``reset_mask`` is set get four copies instead (``engine.py:2443-2450``).  With
         ``stack_only_masked`` the unmasked lanes' stacks are left untouched (the reset call).
+        ``final_frames`` also receives every lane's stack as the call leaves it: the clone that
+        ``step_and_reset_device`` returns as ``final_observations`` (``env.py:915-917``), written by
+        the observation kernel itself.
         """
 
         if self._handle is None:
             raise RuntimeError("renderer is closed")
         desc, keep_lanes = self._lanes_desc(lanes)
-        out, keep_out = self._out_desc(desc.lane_count, indexed, obs, frames, reset_mask, rgb, stack_only_masked)
+        out, keep_out = self._out_desc(desc.lane_count, indexed, obs, frames, reset_mask, rgb, stack_only_masked, final_frames)
         stream = torch.cuda.current_stream(self.device).cuda_stream
         _lib.check(self._lib.gd_render(self._handle, C.byref(desc), C.byref(out), C.c_void_p(stream)))
         del keep_lanes, keep_out

@@ -152,6 +152,9 @@ typedef struct gd_frame_out {
     uint8_t *frames;    /* [N,4,84,84] stack, oldest first: rolled by one and obs appended */
     const uint8_t *reset_mask; /* [N] or null: lanes whose stack is filled with 4 copies instead */
     uint8_t *rgb;       /* [N,240,320,3] PLAYPAL expansion of `indexed` */
+    uint8_t *final_frames; /* [N,4,84,84] or null: also receives every lane's stack as this call leaves it,
+                              the clone step_and_reset_device hands out as final_observations
+                              (env.py:915-917), written by the same kernel instead of a second pass */
     int32_t stack_mode; /* GD_STACK_STEP or GD_STACK_RESET */
 } gd_frame_out;
 

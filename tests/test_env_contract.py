@@ -15,7 +15,7 @@ class RecordingRenderer:
     def __init__(self):
         self.calls = []
 
-    def render(self, lanes, *, indexed=None, obs=None, frames=None, reset_mask=None, rgb=None, stack_only_masked=False):
+    def render(self, lanes, *, indexed=None, obs=None, frames=None, reset_mask=None, rgb=None, stack_only_masked=False, final_frames=None):
         self.calls.append(dict(reset=stack_only_masked, mask=None if reset_mask is None else reset_mask.clone()))
         value = (lanes.x.abs().to(torch.int64) % 251).to(torch.uint8)
         if frames is not None:
@@ -26,6 +26,8 @@ class RecordingRenderer:
                 elif not stack_only_masked:
                     frames[lane] = torch.roll(frames[lane], -1, 0)
                     frames[lane, -1] = new[lane]
+            if final_frames is not None:
+                final_frames.copy_(frames)
         if rgb is not None:
             rgb.copy_(value[:, None, None, None].expand_as(rgb))
 

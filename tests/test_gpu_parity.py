@@ -97,3 +97,23 @@ def test_chunked_batches_render_every_lane_like_the_golden():
             assert renderer.status() == 0
             assert np.array_equal(indexed.cpu().numpy(), data["indexed"][picks])
         renderer.close()
+
+
+def test_final_frames_receive_the_stack_the_call_leaves(oracle):
+    # the fused final-observation clone: step mode, reset mode with untouched lanes, and masked lanes
+    meta, data, tables, renderer, lanes = _renderer("config1")
+    count = meta["lanes"]
+    rng = np.random.default_rng(5)
+    start = rng.integers(0, 256, (count, 4, 84, 84), dtype=np.uint8)
+    mask = torch.as_tensor((rng.random(count) < 0.5).astype(np.uint8)).to("cuda:0")
+    for kwargs in (dict(), dict(reset_mask=mask), dict(reset_mask=mask, stack_only_masked=True)):
+        frames = torch.as_tensor(start).to("cuda:0")
+        plain = torch.as_tensor(start).to("cuda:0")
+        final = torch.full((count, 4, 84, 84), 7, dtype=torch.uint8, device="cuda:0")
+        renderer.render(lanes, frames=frames, final_frames=final, **kwargs)
+        renderer.render(lanes, frames=plain, **kwargs)
+        torch.cuda.synchronize()
+        assert torch.equal(frames, plain)          # the extra output changes nothing else
+        assert torch.equal(final, frames)          # and equals a clone taken after the call
+        assert final.data_ptr() != frames.data_ptr()
+    renderer.close()
