@@ -117,3 +117,43 @@ def test_final_frames_receive_the_stack_the_call_leaves(oracle):
         assert torch.equal(final, frames)          # and equals a clone taken after the call
         assert final.data_ptr() != frames.data_ptr()
     renderer.close()
+
+
+@pytest.mark.parametrize("case", ["many_sectors", "twenty_levels", "eighty_levels"])
+def test_maps_beyond_the_fast_paths_match_the_oracle(oracle, case):
+    # more sectors than the LDS tables hold, more plane levels than the raster's level masks
+    # (15) and than the per-lane plane tables (64): the general paths, checked against the oracle
+    from gradoom_amd import hostmath, mapbuild, synthmap
+    from gradoom_amd.renderer import HipRenderer, LaneState
+    from gradoom_amd.selfcheck import make_lane_arrays
+
+    print(f"case {case}", flush=True)
+    if case == "many_sectors":
+        smap = synthmap.generate_map(77, grid=(25, 24), sectors=600, linedefs=1300, midtex=0.1)
+    else:
+        smap = synthmap.generate_map(78, grid=(12, 12), sectors=144, linedefs=320, midtex=0.1)
+        levels = 20 if case == "twenty_levels" else 400
+        rng = np.random.default_rng(9)
+        count = len(smap.sector_heights)
+        smap.sector_heights[:, 0] = (rng.integers(0, levels, count) * (96.0 / levels)).astype(np.float32)
+        smap.sector_heights[:, 1] = (160.0 + rng.integers(0, levels, count) * (96.0 / levels)).astype(np.float32)
+    tables = mapbuild.build_map_tables(smap)
+    if case == "many_sectors":
+        assert tables["sector_count"] > 512
+    else:
+        assert tables["floor_level_count"] > (15 if case == "twenty_levels" else 64)
+    lanes = 3
+    poses = synthmap.generate_poses(smap, lanes, 31, flash=True)
+    sprites = synthmap.generate_sprites(smap, lanes, 8, 31)
+    arrays = make_lane_arrays(smap, poses, sprites)
+    cosine = hostmath.cosine_correction("cpu").numpy()
+    expected = oracle.render(tables, arrays, cosine, frames=np.zeros((lanes, 4, 84, 84), np.uint8))
+    renderer = HipRenderer(smap, lanes, "cuda:0", cosine_correction=cosine, tables=tables)
+    indexed = torch.zeros((lanes, 240, 320), dtype=torch.uint8, device="cuda:0")
+    frames = torch.zeros((lanes, 4, 84, 84), dtype=torch.uint8, device="cuda:0")
+    renderer.render(LaneState.from_numpy(arrays, "cuda:0"), indexed=indexed, frames=frames)
+    torch.cuda.synchronize()
+    assert renderer.status() == 0
+    assert np.array_equal(indexed.cpu().numpy(), expected["indexed"])
+    assert np.array_equal(frames.cpu().numpy(), expected["frames"])
+    renderer.close()
