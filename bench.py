@@ -33,10 +33,15 @@ MEASURED_TRAFFIC_PER_LANE = {
 }
 
 
-def algorithmic_bytes_per_lane_frame(sprites: int, map_bytes: int, lanes: int) -> float:
+def algorithmic_bytes_per_lane_frame(sprites: int, map_bytes: int, lanes: int, mode: str) -> float:
     # 320x240 u8 frame write + 4x84x84 stack write + 3 older stack frames read
     # + lane pose (64 B) + 24 B per sprite + the shared map/atlas bytes once per launch.
-    return 76800 + 28224 + 21168 + 64 + 24 * sprites + map_bytes / lanes
+    state = 64 + 24 * sprites + map_bytes / lanes
+    if mode == "obs-only":      # no 320x240 frame handed out
+        return 28224 + 21168 + state
+    if mode == "rgb":           # palette-expanded RGB24 frame beside the indexed one
+        return 230400 + 76800 + state
+    return 76800 + 28224 + 21168 + state
 
 
 def main() -> int:
@@ -46,6 +51,9 @@ def main() -> int:
     parser.add_argument("--warmup", type=int, default=2)
     parser.add_argument("--workload", default="config4")
     parser.add_argument("--lanes", type=int, default=None)
+    parser.add_argument("--mode", choices=("full", "obs-only", "rgb"), default="full",
+                        help="full: indexed frame + observation stack (the headline metric); obs-only: observation stack "
+                             "only, no 320x240 frame handed to the caller; rgb: indexed + RGB24 frame, no observation")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     parser.add_argument("--cpu-lanes", type=int, default=12, help="lanes of the same workload the CPU baseline renders")
     parser.add_argument("--copy-probe-mib", type=int, default=0,
@@ -99,13 +107,18 @@ def main() -> int:
         torch.as_tensor(np.clip(base_lights + rng.integers(-16, 17, len(base_lights)), 0, 255).astype(np.float32)).to(device)
         for _ in range(POSE_SETS)
     ]
-    indexed = torch.zeros((lanes, 240, 320), dtype=torch.uint8, device=device)
-    obs = torch.zeros((lanes, 84, 84), dtype=torch.uint8, device=device)
-    frames = torch.zeros((lanes, 4, 84, 84), dtype=torch.uint8, device=device)
+    indexed = obs = frames = rgb = None
+    if args.mode != "obs-only":
+        indexed = torch.zeros((lanes, 240, 320), dtype=torch.uint8, device=device)
+    if args.mode != "rgb":
+        obs = torch.zeros((lanes, 84, 84), dtype=torch.uint8, device=device)
+        frames = torch.zeros((lanes, 4, 84, 84), dtype=torch.uint8, device=device)
+    else:
+        rgb = torch.zeros((lanes, 240, 320, 3), dtype=torch.uint8, device=device)
 
     def step(k: int) -> None:
         renderer.set_sector_lights(flicker[k % POSE_SETS])
-        renderer.render(states[k % POSE_SETS], indexed=indexed, obs=obs, frames=frames)
+        renderer.render(states[k % POSE_SETS], indexed=indexed, obs=obs, frames=frames, rgb=rgb)
 
     for k in range(args.warmup):
         step(k)
@@ -128,7 +141,7 @@ def main() -> int:
     chunk = renderer.chunk_lanes
     chunks = (lanes + chunk - 1) // chunk
     map_bytes = sum(int(np.asarray(v).nbytes) for v in tables.values() if isinstance(v, np.ndarray))
-    bytes_per_lane = algorithmic_bytes_per_lane_frame(sprites, map_bytes, lanes)
+    bytes_per_lane = algorithmic_bytes_per_lane_frame(sprites, map_bytes, lanes, args.mode)
     # render_timed sums a stage over the chunks of one frame; one launch handles `chunk` lanes
     launch_ms = stage_ms[dominant] / chunks
     achieved = bytes_per_lane * chunk / (launch_ms * 1e-3) / 1e9 if launch_ms > 0 else 0.0
@@ -167,10 +180,11 @@ def main() -> int:
         )
 
     line = dict(
-        metric="rendered lane-frames/sec (320x240 + 84x84x4 obs)", value=round(value, 1), unit="lane-frames/s", n_gpus=1,
+        metric={"full": "rendered lane-frames/sec (320x240 + 84x84x4 obs)", "obs-only": "rendered lane-frames/sec (84x84x4 obs only)",
+                "rgb": "rendered lane-frames/sec (320x240 indexed + RGB24)"}[args.mode], value=round(value, 1), unit="lane-frames/s", n_gpus=1,
         steps=args.steps, warmup=args.warmup, ms_per_step=round(elapsed / args.steps * 1e3, 3), higher_is_better=True,
         scaling="weak", vs_baseline=None, dtype="int64+f32", data="synthetic",
-        config=dict(workload=f"{args.workload}: {lanes} lanes, {cfg['sectors']} sectors, {cfg['linedefs']} linedefs, "
+        config=dict(mode=args.mode, workload=f"{args.workload}: {lanes} lanes, {cfg['sectors']} sectors, {cfg['linedefs']} linedefs, "
                     f"{sprites} sprites/lane, masked midtex p={cfg['midtex']}, per-step sector-light flicker"),
         roofline=roofline, cpu_baseline=cpu_baseline,
     )
