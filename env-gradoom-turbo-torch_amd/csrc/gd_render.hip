@@ -978,7 +978,8 @@ __global__ void __launch_bounds__(SW) flat_finish_kernel(DeviceMap dm, int lane_
 // ---------------------------------------------------------------------------------------------
 // walls: engine.py:11462-13745
 // ---------------------------------------------------------------------------------------------
-#define CAND_BATCH 4
+#define CAND_BATCH 8
+#define WALL_ROWS 8          // rows painted / clipped per step of the wall traversal
 struct ColumnCtx {
     const Tables *tb;
     const gd_map_desc *m;
@@ -1451,17 +1452,17 @@ struct SilhouetteBounds {
 };
 
 // Rows [first, last) of one column take `distance` / `wall` as their sprite clip where it is nearer
-// than what they hold.  Four rows at a time, loads first, so the rows' memory latencies overlap.
+// than what they hold.  WALL_ROWS rows at a time, loads first, so the rows' memory latencies overlap.
 __device__ __forceinline__ void clip_rows(PixelBuffers &pb, int x, int first, int last, float distance, int wall) {
-    for (int y0 = first; y0 < last; y0 += 4) {
-        float held[4]; unsigned int meta[4];
+    for (int y0 = first; y0 < last; y0 += WALL_ROWS) {
+        float held[WALL_ROWS]; unsigned int meta[WALL_ROWS];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < WALL_ROWS; ++j) {
             const size_t i = (size_t)(y0 + j < last ? y0 + j : last - 1) * SW + x;
             held[j] = pb.clip_depth[i]; meta[j] = pb.meta[i];
         }
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < WALL_ROWS; ++j) {
             if (y0 + j >= last || !(distance < held[j])) continue;
             const size_t i = (size_t)(y0 + j) * SW + x;
             pb.clip_depth[i] = distance; pb.meta[i] = (meta[j] & ~META_WALL_MASK) | (unsigned)(wall + 1);
@@ -1551,11 +1552,11 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
             tier_step[t] = mul64(swall, shl64(1, 14 - tier_bits[t]));
             tier_base[t] = shl64(round_to_i64((tier_origin[t] - L.view_z) * 65536.0f + toff_y), 16 - tier_bits[t]);
         }
-        // four rows at a time: texel loads first, so their latencies overlap, then the stores
-        for (int yb = t0; yb < t1; yb += 4) {
-            unsigned char texel[4]; bool draw[4], tail[4];
+        // WALL_ROWS rows at a time: texel loads first, so their latencies overlap, then the stores
+        for (int yb = t0; yb < t1; yb += WALL_ROWS) {
+            unsigned char texel[WALL_ROWS]; bool draw[WALL_ROWS], tail[WALL_ROWS];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < WALL_ROWS; ++j) {
                 const int y = yb + j;
                 const float py = (float)y;
                 const bool one_span = one_sided && (py >= r.clipped_top) && (py < r.clipped_bottom);
@@ -1573,7 +1574,7 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
                 }
             }
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < WALL_ROWS; ++j) {
                 if (!draw[j]) continue;
                 const size_t i = (size_t)(yb + j) * SW + x;
                 pb.frame[i] = colormap[(tail[j] ? shade_group : shade_own) * 256 + texel[j]];
