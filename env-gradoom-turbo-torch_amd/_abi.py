@@ -112,6 +112,8 @@ LANE_ARRAYS = (
     ("sprite_id", np.int32),
     ("sprite_alive", np.uint8),
     ("sprite_fullbright", np.uint8),
+    ("weapon_state", np.int64),
+    ("hud_state", np.int32),
 )
 
 OUT_FIELDS = ("indexed", "obs", "frames", "reset_mask", "rgb", "final_frames")
@@ -127,6 +129,54 @@ class MapDesc(C.Structure):
 
 class LanesDesc(C.Structure):
     _fields_ = [("lane_count", C.c_int32), ("sprite_slots", C.c_int32)] + [(name, _P) for name, _ in LANE_ARRAYS]
+
+
+OVERLAY_SCALARS = ("weapon_patch_count", "weapon_max_h", "weapon_max_w", "hud_patch_count", "hud_max_h", "hud_max_w")
+OVERLAY_ARRAYS = (
+    ("weapon_atlas", np.uint8),
+    ("weapon_opaque", np.uint8),
+    ("weapon_w", np.int32),
+    ("weapon_h", np.int32),
+    ("weapon_left", np.int32),
+    ("weapon_top", np.int32),
+    ("hud_atlas", np.uint8),
+    ("hud_opaque", np.uint8),
+    ("hud_w", np.int32),
+    ("hud_h", np.int32),
+    ("hud_left", np.int32),
+    ("hud_top", np.int32),
+)
+
+
+class OverlayDesc(C.Structure):
+    _fields_ = [(name, C.c_int32) for name in OVERLAY_SCALARS] + [(name, _P) for name, _ in OVERLAY_ARRAYS]
+
+
+def host_overlay_desc(overlays: dict) -> tuple[OverlayDesc, list]:
+    """OverlayDesc of HOST pointers from a dict of arrays named like ``gd_overlay_desc``'s fields.
+
+    ``weapon_atlas`` / ``hud_atlas`` are ``[patches, max_h, max_w]``; counts and sizes come from them.
+    """
+
+    desc = OverlayDesc()
+    keep = []
+    for prefix in ("weapon", "hud"):
+        atlas = np.ascontiguousarray(overlays[f"{prefix}_atlas"], dtype=np.uint8)
+        if atlas.ndim != 3:
+            raise ValueError(f"{prefix}_atlas must be [patches, height, width]")
+        setattr(desc, f"{prefix}_patch_count", atlas.shape[0])
+        setattr(desc, f"{prefix}_max_h", atlas.shape[1])
+        setattr(desc, f"{prefix}_max_w", atlas.shape[2])
+        if np.asarray(overlays[f"{prefix}_opaque"]).shape != atlas.shape:
+            raise ValueError(f"{prefix}_opaque must have the shape of {prefix}_atlas")
+        for field in ("w", "h", "left", "top"):
+            if np.asarray(overlays[f"{prefix}_{field}"]).shape != (atlas.shape[0],):
+                raise ValueError(f"{prefix}_{field} must hold one value per patch")
+    for name, dtype in OVERLAY_ARRAYS:
+        array = np.ascontiguousarray(overlays[name], dtype=dtype)
+        keep.append(array)
+        setattr(desc, name, array.ctypes.data)
+    return desc, keep
 
 
 class FrameOut(C.Structure):

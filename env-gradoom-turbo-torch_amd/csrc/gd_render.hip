@@ -119,6 +119,10 @@ struct DeviceMap {  // device copy of gd_map_desc (device pointers) + fixed tabl
                                          // ceil_levels << 8; null when a level list is longer than PLANE_LEVELS
 };
 
+struct Overlays {   // device copy of gd_overlay_desc; count 0 = layer not loaded
+    gd_overlay_desc d;
+};
+
 struct Scratch {    // per-chunk working memory, sized at create
     LaneCtx *ctx;          // [L]
     WallRec *rec;          // [L,W]
@@ -2304,6 +2308,123 @@ __global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lan
 }
 
 // ---------------------------------------------------------------------------------------------
+// overlay layers drawn after the sprites
+// ---------------------------------------------------------------------------------------------
+// One psprite patch over one pixel (engine.py:14997-15049, _triton_kernels.py:2611-2634).
+__device__ __forceinline__ bool psprite_texel(const gd_overlay_desc &o, i64 patch, i64 horizontal_fixed, i64 vertical_fixed, int px, int py, unsigned char *value) {
+    if (patch < 0 || patch >= o.weapon_patch_count) return false;
+    const i64 width = o.weapon_w[patch], height = o.weapon_h[patch];
+    const i64 screen_left = (horizontal_fixed - (i64)o.weapon_left[patch] * FIXED_UNIT) >> 16;
+    const i64 source_x = (i64)px - screen_left;
+    // BASEYCENTER 100, weapon top 32 + 0x6000/65536, reciprocal of the 240/200 vertical scale
+    const i64 weapon_top_fixed = 32 * FIXED_UNIT + 0x6000;
+    const i64 texture_mid = 100 * FIXED_UNIT - weapon_top_fixed - vertical_fixed + (i64)o.weapon_top[patch] * FIXED_UNIT;
+    const i64 y_scale = ((i64)GD_SCREEN_HEIGHT * FIXED_UNIT) / 200;
+    const i64 y_iscale = UINT32_MASK / y_scale;
+    const i64 source_y = (texture_mid + ((i64)py - (VH / 2 - 1)) * y_iscale) >> 16;
+    if (source_x < 0 || source_x >= width || source_y < 0 || source_y >= height) return false;
+    if (source_x >= o.weapon_max_w || source_y >= o.weapon_max_h) return false;   // sizes beyond the atlas: malformed patch
+    const size_t t = ((size_t)patch * o.weapon_max_h + (size_t)source_y) * o.weapon_max_w + (size_t)source_x;
+    if (!o.weapon_opaque[t]) return false;
+    *value = o.weapon_atlas[t];
+    return true;
+}
+
+// _native_render_weapon (engine.py:15051-15110): the weapon patch, then its muzzle flash on top
+__global__ void __launch_bounds__(256) weapon_overlay_kernel(Overlays ov, const int64_t *weapon_state, int lane_base, int lane_count,
+                                                             unsigned char *frame_base, size_t frame_stride) {
+    const int local = blockIdx.y;
+    const int pixel = blockIdx.x * blockDim.x + threadIdx.x;
+    if (local >= lane_count || pixel >= VH * SW) return;
+    const int64_t *state = weapon_state + (size_t)(lane_base + local) * 5;
+    if (state[4] == 0) return;                    // player dead: no psprite
+    const int py = pixel / SW, px = pixel - py * SW;
+    unsigned char value;
+    bool drawn = psprite_texel(ov.d, state[0], state[2], state[3], px, py, &value);
+    unsigned char flash;
+    if (state[1] >= 0 && psprite_texel(ov.d, state[1], state[2], state[3], px, py, &flash)) { value = flash; drawn = true; }
+    if (drawn) frame_base[(size_t)local * frame_stride + pixel] = value;
+}
+
+// _native_render_hud (engine.py:15153-15267): the status bar is a short list of patches drawn in
+// order, later ones over earlier ones.  One block per lane: thread 0 writes the list, then every
+// thread resolves its pixels by walking the list backwards to the first opaque texel.
+#define HUD_ROWS (GD_SCREEN_HEIGHT - VH)
+#define HUD_LIST_MAX 48
+struct HudEntry { int patch, x, y; };
+
+// _native_draw_hud_number (engine.py:15186-15207); note that the glyph offsets are applied here and
+// again by the patch draw, as in the reference
+__device__ void hud_number(const gd_overlay_desc &o, HudEntry *list, int *count, int value, int right, int y, bool small) {
+    value = value < -99 ? -99 : (value > 999 ? 999 : value);
+    const int digit_width = small ? 4 : 14, base = small ? 28 : 2;
+    const bool negative = value < 0;
+    int magnitude = negative ? -value : value;
+    int digits[3], length = 0;
+    do { digits[length++] = magnitude % 10; magnitude /= 10; } while (magnitude > 0);
+    int x = right - (length + (negative ? 1 : 0)) * digit_width;
+    if (negative) x += digit_width;               // the sign takes a cell and draws nothing
+    for (int k = length - 1; k >= 0; --k) {
+        const int patch = base + digits[k];
+        if (patch < o.hud_patch_count && *count < HUD_LIST_MAX) {
+            HudEntry e; e.patch = patch; e.x = x - o.hud_left[patch]; e.y = y - o.hud_top[patch];
+            list[(*count)++] = e;
+        }
+        x += digit_width;
+    }
+}
+
+__global__ void __launch_bounds__(256) hud_kernel(Overlays ov, const int *hud_state, int lane_base, int lane_count,
+                                                  unsigned char *frame_base, size_t frame_stride) {
+    const gd_overlay_desc &o = ov.d;
+    __shared__ HudEntry list[HUD_LIST_MAX];
+    __shared__ int list_count;
+    const int local = blockIdx.x;
+    if (local >= lane_count) return;
+    if (threadIdx.x == 0) {
+        const int *state = hud_state + (size_t)(lane_base + local) * 9;
+        int count = 0;
+        auto patch_at = [&](int patch, int x, int y) {
+            if (patch >= 0 && patch < o.hud_patch_count && count < HUD_LIST_MAX) { HudEntry e; e.patch = patch; e.x = x; e.y = y; list[count++] = e; }
+        };
+        patch_at(0, 0, 0);
+        patch_at(1, 104, 0);
+        hud_number(o, list, &count, state[0], 44, 3, false);
+        hud_number(o, list, &count, state[1], 90, 3, false);
+        patch_at(12, 90, 3);
+        hud_number(o, list, &count, state[2], 221, 3, false);
+        patch_at(12, 221, 3);
+        patch_at(state[3], 143, 0);
+        const int arms_x[6] = {111, 123, 135, 111, 123, 135}, arms_y[6] = {4, 4, 4, 14, 14, 14};
+        for (int k = 0; k < 6; ++k) {
+            const bool owned = k < 5 && ((state[4] >> k) & 1);
+            patch_at(owned ? 30 + k : 38 + k, arms_x[k], arms_y[k]);
+        }
+        const int maximum[4] = {200, 50, 50, 300};
+        for (int row = 0; row < 4; ++row) {
+            hud_number(o, list, &count, state[5 + row], 288, 5 + row * 6, true);
+            hud_number(o, list, &count, maximum[row], 314, 5 + row * 6, true);
+        }
+        list_count = count;
+    }
+    __syncthreads();
+    unsigned char *bar = frame_base + (size_t)local * frame_stride + (size_t)VH * SW;
+    for (int p = threadIdx.x; p < HUD_ROWS * SW; p += blockDim.x) {
+        const int cy = p / SW, cx = p - cy * SW;
+        unsigned char value = 0;
+        for (int k = list_count - 1; k >= 0; --k) {
+            const HudEntry e = list[k];
+            // _native_draw_hud_patch (engine.py:15153-15184): position minus the patch's own offsets, clipped
+            const int sx = cx - (e.x - o.hud_left[e.patch]), sy = cy - (e.y - o.hud_top[e.patch]);
+            if (sx < 0 || sy < 0 || sx >= o.hud_w[e.patch] || sy >= o.hud_h[e.patch] || sx >= o.hud_max_w || sy >= o.hud_max_h) continue;
+            const size_t t = ((size_t)e.patch * o.hud_max_h + sy) * o.hud_max_w + sx;
+            if (o.hud_opaque[t]) { value = o.hud_atlas[t]; break; }
+        }
+        bar[p] = value;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // observation: _triton_kernels.py:120-177 + engine.py:9545-9548 / 2443-2450
 // ---------------------------------------------------------------------------------------------
 __global__ void observe_kernel(const unsigned char *indexed, size_t lane_stride, int source_rows, const unsigned char *playpal,
@@ -2415,6 +2536,8 @@ struct gd_renderer {
     hipStream_t side_stream;
     hipEvent_t fork_event, flat_event;
     bool side_ready;
+    Overlays overlays;                       // device pointers, counts 0 until gd_renderer_set_overlays
+    std::vector<void *> overlay_allocations;
 };
 
 namespace {
@@ -2534,6 +2657,11 @@ int launch_chunk(gd_renderer *r, Scratch &sc, const gd_lanes_desc *lanes, const 
         size_t shared = (size_t)lanes->sprite_slots * sizeof(SpriteRec);
         hipLaunchKernelGGL(sprite_columns_kernel, dim3(count), dim3(SW), shared, stream, r->dm, *lanes, base, count, sc, frame_base, frame_stride);
     }
+    if (lanes->weapon_state && r->overlays.d.weapon_patch_count > 0)
+        hipLaunchKernelGGL(weapon_overlay_kernel, dim3((VH * SW + 255) / 256, count), dim3(256), 0, stream, r->overlays, lanes->weapon_state, base, count,
+                           frame_base, frame_stride);
+    if (lanes->hud_state && r->overlays.d.hud_patch_count > 0)
+        hipLaunchKernelGGL(hud_kernel, dim3(count), dim3(256), 0, stream, r->overlays, lanes->hud_state, base, count, frame_base, frame_stride);
     mark();
     if (out->final_frames && !out->frames) return fail(GD_E_ARG, "final_frames needs frames");
     if (out->obs || out->frames) {
@@ -2576,6 +2704,7 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     r->events_ready = false;
     r->side_ready = false;
     std::memset(&r->sc, 0, sizeof(r->sc));
+    std::memset(&r->overlays, 0, sizeof(r->overlays));
     r->dm.d = *h;
     gd_map_desc &d = r->dm.d;
     const size_t W = h->wall_count, S = h->sector_count, V = h->vertex_count, K = h->neighbor_slots;
@@ -2712,6 +2841,7 @@ void gd_renderer_destroy(gd_renderer *r) {
     if (!r) return;
     if (r->side_ready) { (void)hipStreamSynchronize(r->side_stream); (void)hipEventDestroy(r->fork_event); (void)hipEventDestroy(r->flat_event); (void)hipStreamDestroy(r->side_stream); }
     for (void *ptr : r->allocations) (void)hipFree(ptr);
+    for (void *ptr : r->overlay_allocations) (void)hipFree(ptr);
     if (r->events_ready) for (int i = 0; i < 16; ++i) (void)hipEventDestroy(r->events[i]);
     delete r;
 }
@@ -2772,6 +2902,43 @@ int gd_renderer_status(gd_renderer *r, int32_t *status) {
     int value = 0;
     HIP_TRY(hipMemcpy(&value, r->sc.status, sizeof(int), hipMemcpyDeviceToHost));
     *status = value;
+    return GD_OK;
+}
+
+int gd_renderer_set_overlays(gd_renderer *r, const gd_overlay_desc *h) {
+    if (!r || !h) return fail(GD_E_ARG, "null argument");
+    if (h->weapon_patch_count < 0 || h->hud_patch_count < 0 || h->weapon_max_h < 0 || h->weapon_max_w < 0 || h->hud_max_h < 0 || h->hud_max_w < 0)
+        return fail(GD_E_ARG, "negative overlay size");
+    if (h->weapon_patch_count > 0 && (!h->weapon_atlas || !h->weapon_opaque || !h->weapon_w || !h->weapon_h || !h->weapon_left || !h->weapon_top))
+        return fail(GD_E_ARG, "missing weapon patch array");
+    if (h->hud_patch_count > 0 && (!h->hud_atlas || !h->hud_opaque || !h->hud_w || !h->hud_h || !h->hud_left || !h->hud_top))
+        return fail(GD_E_ARG, "missing status bar patch array");
+    HIP_TRY(hipDeviceSynchronize());              // no frame may still be reading the old patches
+    for (void *ptr : r->overlay_allocations) (void)hipFree(ptr);
+    r->overlay_allocations.clear();
+    std::memset(&r->overlays, 0, sizeof(r->overlays));
+    gd_overlay_desc d = *h;
+    auto copy = [&](const void *host, size_t bytes, const void **device) -> int {
+        void *ptr = nullptr;
+        HIP_TRY(hipMalloc(&ptr, bytes ? bytes : 1));
+        r->overlay_allocations.push_back(ptr);
+        if (bytes) HIP_TRY(hipMemcpy(ptr, host, bytes, hipMemcpyHostToDevice));
+        *device = ptr;
+        return GD_OK;
+    };
+    int rc = GD_OK;
+    const size_t wp = h->weapon_patch_count, wt = wp * h->weapon_max_h * h->weapon_max_w;
+    const size_t hp = h->hud_patch_count, ht = hp * h->hud_max_h * h->hud_max_w;
+#define OV(field, bytes) if (rc == GD_OK) rc = copy(h->field, (bytes), reinterpret_cast<const void **>(&d.field))
+    OV(weapon_atlas, wt); OV(weapon_opaque, wt); OV(weapon_w, wp * 4); OV(weapon_h, wp * 4); OV(weapon_left, wp * 4); OV(weapon_top, wp * 4);
+    OV(hud_atlas, ht); OV(hud_opaque, ht); OV(hud_w, hp * 4); OV(hud_h, hp * 4); OV(hud_left, hp * 4); OV(hud_top, hp * 4);
+#undef OV
+    if (rc != GD_OK) {
+        for (void *ptr : r->overlay_allocations) (void)hipFree(ptr);
+        r->overlay_allocations.clear();
+        return rc;
+    }
+    r->overlays.d = d;
     return GD_OK;
 }
 

@@ -45,6 +45,9 @@ class LaneState:
     ray_cos: torch.Tensor | None = None
     ray_sin: torch.Tensor | None = None
     sprite_depth: torch.Tensor | None = None
+    # Overlay layers (see overlay_inputs.py); drawn when the renderer holds overlay patches.
+    weapon_state: torch.Tensor | None = None  # i64 [N,5]
+    hud_state: torch.Tensor | None = None  # i32 [N,9]
 
     @classmethod
     def from_numpy(cls, arrays: dict, device) -> "LaneState":
@@ -63,6 +66,7 @@ class LaneState:
             sprite_id=get("sprite_id", torch.int32), sprite_alive=get("sprite_alive", torch.uint8),
             sprite_fullbright=get("sprite_fullbright", torch.uint8), ray_cos=get("ray_cos", torch.float32),
             ray_sin=get("ray_sin", torch.float32), sprite_depth=get("sprite_depth", torch.float32),
+            weapon_state=get("weapon_state", torch.int64), hud_state=get("hud_state", torch.int32),
         )
 
 
@@ -122,6 +126,20 @@ class HipRenderer:
         _lib.check(self._lib.gd_renderer_status(self._handle, C.byref(value)))
         return int(value.value)
 
+    def set_overlays(self, overlays: dict) -> None:
+        """Upload the weapon and status bar patches (NumPy arrays named like ``gd_overlay_desc``'s fields).
+
+        Afterwards lanes that carry ``weapon_state`` / ``hud_state`` get the psprite over the view and
+        the status bar in rows 208..239 (``engine.py:15051-15110``, ``15232-15267``).
+        """
+
+        if self._handle is None:
+            raise RuntimeError("renderer is closed")
+        desc, keep = _abi.host_overlay_desc(overlays)
+        with torch.cuda.device(self.device):
+            _lib.check(self._lib.gd_renderer_set_overlays(self._handle, C.byref(desc)))
+        del keep
+
     def set_sector_lights(self, lights: torch.Tensor) -> None:
         """Replace the per-sector light levels (float32 [S] on the device) for later frames."""
 
@@ -171,6 +189,10 @@ class HipRenderer:
                 depth = hostmath.sprite_depth(lanes.x, lanes.y, lanes.angle, lanes.sprite_x, lanes.sprite_y)
             keep.append(depth)
             desc.sprite_depth = _require(depth, "sprite_depth", torch.float32, (count, slots), device).data_ptr()
+        if lanes.weapon_state is not None:
+            desc.weapon_state = _require(lanes.weapon_state, "weapon_state", torch.int64, (count, 5), device).data_ptr()
+        if lanes.hud_state is not None:
+            desc.hud_state = _require(lanes.hud_state, "hud_state", torch.int32, (count, 9), device).data_ptr()
         return desc, keep
 
     def _out_desc(self, count, indexed, obs, frames, reset_mask, rgb, stack_only_masked=False, final_frames=None):

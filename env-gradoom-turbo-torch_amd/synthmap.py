@@ -544,3 +544,61 @@ def generate_sprites_batch(smap: SynthMap, lanes: int, count: int, seed: int) ->
     alive = rng.random(shape) < 0.9
     fullbright = rng.random(shape) < 0.1
     return Sprites(x, y, z, sprite, alive, fullbright)
+
+
+def generate_overlays(seed: int, *, weapon_patches: int = 12, cooldowns: int = 8) -> dict:
+    """Seeded weapon psprite and status bar patches, named like ``gd_overlay_desc``'s fields.
+
+    Shapes follow the reference's assets: psprite patches with the negative offsets Doom uses
+    to place them (``engine.py:14997-15020``), a 320x32 status bar, an arms panel, 14-pixel big
+    digits, 4-pixel small digits, faces, owned / missing weapon numbers (patch ids as in
+    ``engine.py:15186-15259``).  Also the ``[8, 2, cooldowns]`` weapon frame / flash / flash
+    light tables of ``engine.py:14949-14967``.
+    """
+
+    rng = np.random.default_rng(seed)
+    wh, ww = 112, 160
+    weapon_atlas = np.zeros((weapon_patches, wh, ww), dtype=np.uint8)
+    weapon_opaque = np.zeros((weapon_patches, wh, ww), dtype=np.uint8)
+    weapon_w = rng.integers(40, ww + 1, weapon_patches).astype(np.int32)
+    weapon_h = rng.integers(40, wh + 1, weapon_patches).astype(np.int32)
+    weapon_left = -rng.integers(60, 200, weapon_patches).astype(np.int32)
+    weapon_top = -rng.integers(40, 150, weapon_patches).astype(np.int32)
+    for p in range(weapon_patches):
+        w, h = int(weapon_w[p]), int(weapon_h[p])
+        weapon_atlas[p, :h, :w] = rng.integers(1, 256, (h, w), dtype=np.uint8)
+        weapon_opaque[p, :h, :w] = rng.random((h, w)) < 0.8
+    hud_patches = 70
+    hh, hw = 32, 320
+    hud_w = np.zeros(hud_patches, dtype=np.int32)
+    hud_h = np.zeros(hud_patches, dtype=np.int32)
+    hud_left = np.zeros(hud_patches, dtype=np.int32)
+    hud_top = np.zeros(hud_patches, dtype=np.int32)
+    for p in range(hud_patches):
+        if p == 0:
+            size, offsets = (320, 32), (0, 0)
+        elif p == 1:
+            size, offsets = (40, 32), (0, 0)
+        elif 2 <= p <= 12:
+            size, offsets = (14, 16), (int(rng.integers(-2, 3)), int(rng.integers(-2, 3)))
+        elif 28 <= p <= 43:
+            size, offsets = (4, 6), (int(rng.integers(-1, 2)), int(rng.integers(-1, 2)))
+        else:  # faces
+            size, offsets = (int(rng.integers(22, 27)), int(rng.integers(27, 32))), (int(rng.integers(-3, 4)), int(rng.integers(-3, 2)))
+        hud_w[p], hud_h[p] = size
+        hud_left[p], hud_top[p] = offsets
+    hud_atlas = np.zeros((hud_patches, hh, hw), dtype=np.uint8)
+    hud_opaque = np.zeros((hud_patches, hh, hw), dtype=np.uint8)
+    for p in range(hud_patches):
+        w, h = int(hud_w[p]), int(hud_h[p])
+        hud_atlas[p, :h, :w] = rng.integers(1, 256, (h, w), dtype=np.uint8)
+        hud_opaque[p, :h, :w] = rng.random((h, w)) < 0.85
+    frame_ids = rng.integers(0, weapon_patches, (8, 2, cooldowns)).astype(np.int32)
+    flash_ids = np.where(rng.random((8, 2, cooldowns)) < 0.4, rng.integers(0, weapon_patches, (8, 2, cooldowns)), -1).astype(np.int32)
+    flash_lights = np.where(flash_ids >= 0, rng.integers(1, 3, (8, 2, cooldowns)), 0).astype(np.int64)
+    return dict(
+        weapon_atlas=weapon_atlas, weapon_opaque=weapon_opaque, weapon_w=weapon_w, weapon_h=weapon_h,
+        weapon_left=weapon_left, weapon_top=weapon_top, hud_atlas=hud_atlas, hud_opaque=hud_opaque, hud_w=hud_w,
+        hud_h=hud_h, hud_left=hud_left, hud_top=hud_top, weapon_frame_ids=frame_ids, weapon_flash_ids=flash_ids,
+        weapon_flash_lights=flash_lights,
+    )

@@ -143,7 +143,35 @@ typedef struct gd_lanes_desc {
     const int32_t *sprite_id;        /* [N,A] */
     const uint8_t *sprite_alive;     /* [N,A] */
     const uint8_t *sprite_fullbright;/* [N,A] */
+    /* Overlay layers, drawn after the sprites when the renderer holds overlay patches
+       (gd_renderer_set_overlays); either pointer may be null to skip that layer. */
+    const int64_t *weapon_state;    /* [N,5] psprite of engine.py:15051-15110: patch id, muzzle flash patch id
+                                       (-1 = none), horizontal offset (bob) 16.16, vertical offset 16.16,
+                                       visible (0/1) */
+    const int32_t *hud_state;       /* [N,9] status bar of engine.py:15232-15267: ready ammo, health, armor,
+                                       face patch id, owned weapon bits (bit k = weapon k+1, k < 5),
+                                       four ammo counts */
 } gd_lanes_desc;
+
+/*
+ * Weapon psprite and status bar patches (HOST pointers; gd_renderer_set_overlays
+ * uploads them).  Replaces map.native_weapon_patch_* (engine.py:14997-15049,
+ * _triton_kernels.py:2571-2670) and map.hud_patch_* (engine.py:15153-15267).
+ * Patch atlases are [patches, max_h, max_w] with per-patch sizes and offsets.
+ * Status bar patch numbering follows the reference: 0 bar, 1 arms panel,
+ * 2..11 big digits, 12 percent sign, 13.. faces, 28..37 small digits,
+ * 30..35 owned weapon numbers, 38..43 missing weapon numbers (engine.py:15186-15259).
+ */
+typedef struct gd_overlay_desc {
+    int32_t weapon_patch_count, weapon_max_h, weapon_max_w;
+    int32_t hud_patch_count, hud_max_h, hud_max_w;
+    const uint8_t *weapon_atlas;    /* [Pw,Hw,Ww] palette indices */
+    const uint8_t *weapon_opaque;   /* [Pw,Hw,Ww] 0/1 */
+    const int32_t *weapon_w, *weapon_h, *weapon_left, *weapon_top; /* [Pw] */
+    const uint8_t *hud_atlas;       /* [Ph,Hh,Wh] */
+    const uint8_t *hud_opaque;      /* [Ph,Hh,Wh] */
+    const int32_t *hud_w, *hud_h, *hud_left, *hud_top;             /* [Ph] */
+} gd_overlay_desc;
 
 /* Output buffers; any pointer may be null to skip that product. */
 typedef struct gd_frame_out {
@@ -201,6 +229,16 @@ int gd_renderer_status(gd_renderer *r, int32_t *status);
  * animates it (light flicker) between frames.
  */
 int gd_renderer_set_sector_lights(gd_renderer *r, const float *lights, void *stream);
+
+/*
+ * Upload (or replace) the weapon and status bar patches.  With them a gd_render call
+ * whose lanes carry weapon_state draws the psprite and its muzzle flash over the view
+ * after the sprites (_native_render_weapon, engine.py:15051-15110, fixed-point path), and
+ * one whose lanes carry hud_state draws the status bar into rows 208..239
+ * (_native_render_hud, engine.py:15232-15267); without them those rows stay 0.
+ * Synchronises the device; call it between frames.
+ */
+int gd_renderer_set_overlays(gd_renderer *r, const gd_overlay_desc *overlays);
 
 /*
  * Observation pipeline alone on an existing indexed frame.

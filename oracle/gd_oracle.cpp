@@ -1534,6 +1534,104 @@ typedef struct gdo_debug {
     uint8_t *walls_frame;        // [208,320] frame after walls/planes/masked, before sprites
 } gdo_debug;
 
+// ---------------------------------------------------------------------------------------------
+// Overlay layers: weapon psprite (engine.py:14997-15110) and status bar (engine.py:15153-15267),
+// restated as the reference's CPU path does them: whole-patch composites in draw order.
+// ---------------------------------------------------------------------------------------------
+static gd_overlay_desc g_overlays;
+static bool g_overlays_set = false;
+
+int gdo_set_overlays(const gd_overlay_desc *overlays) {
+    g_overlays_set = overlays != nullptr;
+    if (overlays) g_overlays = *overlays;     // host pointers, kept by the caller
+    return GD_OK;
+}
+
+// _native_composite_weapon_patch (engine.py:14997-15049) over the 320x208 view of one lane
+static void composite_weapon_patch(uint8_t *view, int64_t patch, int64_t horizontal_fixed, int64_t vertical_fixed, bool visible) {
+    const gd_overlay_desc &o = g_overlays;
+    if (!visible) return;
+    const int64_t FIXED = 65536;
+    const int64_t width = o.weapon_w[patch], height = o.weapon_h[patch];
+    const int64_t left_offset = o.weapon_left[patch], top_offset = o.weapon_top[patch];
+    const int64_t screen_left = (horizontal_fixed - left_offset * FIXED) >> 16;
+    const int64_t weapon_top_fixed = 32 * FIXED + 0x6000;
+    const int64_t texture_mid_fixed = 100 * FIXED - weapon_top_fixed - vertical_fixed + top_offset * FIXED;
+    const int64_t psprite_y_scale_fixed = int64_t(GD_SCREEN_HEIGHT) * FIXED / 200;
+    const int64_t psprite_y_iscale_fixed = int64_t(0xFFFFFFFFLL) / psprite_y_scale_fixed;
+    for (int y = 0; y < VH; ++y) {
+        const int64_t screen_delta = int64_t(y) - (VH / 2 - 1);
+        const int64_t source_y = (texture_mid_fixed + screen_delta * psprite_y_iscale_fixed) >> 16;
+        for (int x = 0; x < SW; ++x) {
+            const int64_t source_x = int64_t(x) - screen_left;
+            const bool inside = source_x >= 0 && source_x < width && source_y >= 0 && source_y < height;
+            if (!inside) continue;
+            const int64_t cx = std::min<int64_t>(std::max<int64_t>(source_x, 0), o.weapon_max_w - 1);
+            const int64_t cy = std::min<int64_t>(std::max<int64_t>(source_y, 0), o.weapon_max_h - 1);
+            const size_t t = (size_t(patch) * o.weapon_max_h + size_t(cy)) * o.weapon_max_w + size_t(cx);
+            if (o.weapon_opaque[t]) view[size_t(y) * SW + x] = o.weapon_atlas[t];
+        }
+    }
+}
+
+// _native_draw_hud_patch (engine.py:15153-15184) on a [32,320] canvas
+static void draw_hud_patch(uint8_t *canvas, int patch, int x, int y) {
+    const gd_overlay_desc &o = g_overlays;
+    const int rows = GD_SCREEN_HEIGHT - VH;
+    x -= o.hud_left[patch];
+    y -= o.hud_top[patch];
+    const int width = o.hud_w[patch], height = o.hud_h[patch];
+    if (width <= 0 || height <= 0) return;
+    const int source_x = std::max(-x, 0), source_y = std::max(-y, 0);
+    const int target_x = std::max(x, 0), target_y = std::max(y, 0);
+    const int copy_width = std::min(width - source_x, SW - target_x);
+    const int copy_height = std::min(height - source_y, rows - target_y);
+    if (copy_width <= 0 || copy_height <= 0) return;
+    for (int r = 0; r < copy_height; ++r) for (int c = 0; c < copy_width; ++c) {
+        const size_t t = (size_t(patch) * o.hud_max_h + size_t(source_y + r)) * o.hud_max_w + size_t(source_x + c);
+        if (o.hud_opaque[t]) canvas[size_t(target_y + r) * SW + target_x + c] = o.hud_atlas[t];
+    }
+}
+
+// _native_draw_hud_number (engine.py:15186-15207)
+static void draw_hud_number(uint8_t *canvas, int value, int right, int y, bool small) {
+    const gd_overlay_desc &o = g_overlays;
+    char text[16];
+    std::snprintf(text, sizeof(text), "%d", std::max(-99, std::min(value, 999)));
+    const int digit_width = small ? 4 : 14, base = small ? 28 : 2;
+    int x = right - int(std::strlen(text)) * digit_width;
+    for (const char *c = text; *c; ++c) {
+        if (*c == '-') { x += digit_width; continue; }
+        const int patch = base + (*c - '0');
+        const int glyph_x = x - o.hud_left[patch], glyph_y = y - o.hud_top[patch];
+        draw_hud_patch(canvas, patch, glyph_x, glyph_y);
+        x += digit_width;
+    }
+}
+
+// _native_render_hud (engine.py:15232-15267) for one lane; `state` as gd_lanes_desc.hud_state
+static void render_hud(uint8_t *canvas, const int32_t *state) {
+    draw_hud_patch(canvas, 0, 0, 0);
+    draw_hud_patch(canvas, 1, 104, 0);
+    draw_hud_number(canvas, state[0], 44, 3, false);
+    draw_hud_number(canvas, state[1], 90, 3, false);
+    draw_hud_patch(canvas, 12, 90, 3);
+    draw_hud_number(canvas, state[2], 221, 3, false);
+    draw_hud_patch(canvas, 12, 221, 3);
+    draw_hud_patch(canvas, state[3], 143, 0);
+    const int positions[6][2] = {{111, 4}, {123, 4}, {135, 4}, {111, 14}, {123, 14}, {135, 14}};
+    for (int weapon_index = 0; weapon_index < 6; ++weapon_index) {
+        const bool owned = weapon_index < 5 && ((state[4] >> weapon_index) & 1);
+        draw_hud_patch(canvas, owned ? 28 + weapon_index + 2 : 38 + weapon_index, positions[weapon_index][0], positions[weapon_index][1]);
+    }
+    const int maximum[4] = {200, 50, 50, 300};
+    for (int row = 0; row < 4; ++row) {
+        const int y = 5 + row * 6;
+        draw_hud_number(canvas, state[5 + row], 288, y, true);
+        draw_hud_number(canvas, maximum[row], 314, y, true);
+    }
+}
+
 // Full frame for lanes [lane_begin, lane_end): indexed, obs, stack, rgb as in gd_render.
 int gdo_render(const gd_map_desc *map, const gd_lanes_desc *lanes, const gd_frame_out *out,
                int32_t lane_begin, int32_t lane_end, const float *cosine_correction, const gdo_debug *dbg) {
@@ -1595,6 +1693,13 @@ int gdo_render(const gd_map_desc *map, const gd_lanes_desc *lanes, const gd_fram
         t_setup += t1 - t0; t_flats += t2 - t1; t_walls += t4 - t3; t_sprites += t6 - t5;
         std::memcpy(full.data(), o.frame.data(), size_t(VH) * SW);
         std::memset(full.data() + size_t(VH) * SW, 0, size_t(GD_SCREEN_HEIGHT - VH) * SW);
+        if (g_overlays_set && lanes->weapon_state && g_overlays.weapon_patch_count > 0) {
+            const int64_t *state = lanes->weapon_state + size_t(n) * 5;
+            composite_weapon_patch(full.data(), state[0], state[2], state[3], state[4] != 0);
+            composite_weapon_patch(full.data(), std::max<int64_t>(state[1], 0), state[2], state[3], state[4] != 0 && state[1] >= 0);
+        }
+        if (g_overlays_set && lanes->hud_state && g_overlays.hud_patch_count > 0)
+            render_hud(full.data() + size_t(VH) * SW, lanes->hud_state + size_t(n) * 9);
         if (out->indexed) std::memcpy(out->indexed + size_t(n) * full.size(), full.data(), full.size());
         if (out->obs || out->frames) {
             observe_lane(full.data(), VH, map->playpal, obs.data());  // HUD rows masked black

@@ -65,6 +65,23 @@ def library():
     return _LIB
 
 
+_OVERLAY_KEEP = None
+
+
+def set_overlays(overlays: dict | None) -> None:
+    """Weapon and status bar patches for later ``render`` calls (``None`` removes them)."""
+
+    global _OVERLAY_KEEP
+    lib = library()
+    if overlays is None:
+        lib.gdo_set_overlays(None)
+        _OVERLAY_KEEP = None
+        return
+    desc, keep = _abi.host_overlay_desc(overlays)
+    lib.gdo_set_overlays(C.byref(desc))
+    _OVERLAY_KEEP = (desc, keep)
+
+
 def fine_tables():
     sine = np.zeros(8192, dtype=np.int64)
     tangent = np.zeros(4096, dtype=np.int64)

@@ -52,7 +52,16 @@ def load_fixture(name: str):
 LANE_KEYS = (
     "x", "y", "angle", "view_z", "x_fixed", "y_fixed", "angle_bam", "pitch_bam", "flash_light", "ray_cos", "ray_sin",
     "sprite_x", "sprite_y", "sprite_z", "sprite_depth", "sprite_id", "sprite_alive", "sprite_fullbright",
+    "weapon_state", "hud_state",
 )
+
+
+def fixture_overlays(meta: dict):
+    """The seeded weapon / status bar patches of a case that has them, else None."""
+
+    from gradoom_amd import synthmap
+
+    return synthmap.generate_overlays(meta["overlays"]) if meta.get("overlays") else None
 
 
 def lane_inputs(data: dict) -> dict:

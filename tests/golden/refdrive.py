@@ -34,7 +34,7 @@ def load_reference():
     return engine, scenario
 
 
-def to_compiled_scenario(smap, *, flash_lights: bool = False):
+def to_compiled_scenario(smap, *, flash_lights: bool = False, overlays: dict | None = None):
     """Wrap a SynthMap in the reference's CompiledScenario (``scenario.py:302-401``)."""
 
     _engine, scenario = load_reference()
@@ -50,6 +50,19 @@ def to_compiled_scenario(smap, *, flash_lights: bool = False):
         lights[:, :, 1] = 1
         lights[:, :, 2] = 2
         kwargs["native_weapon_flash_lights"] = lights
+    if overlays is not None:
+        # raw psprite and status bar patches (scenario.py:382-397)
+        kwargs.update(
+            native_weapon_patch_atlas=overlays["weapon_atlas"], native_weapon_patch_opaque=overlays["weapon_opaque"].astype(bool),
+            native_weapon_patch_widths=overlays["weapon_w"], native_weapon_patch_heights=overlays["weapon_h"],
+            native_weapon_patch_left_offsets=overlays["weapon_left"], native_weapon_patch_top_offsets=overlays["weapon_top"],
+            native_weapon_frame_ids=overlays["weapon_frame_ids"], native_weapon_flash_ids=overlays["weapon_flash_ids"],
+            native_weapon_flash_lights=overlays["weapon_flash_lights"],
+            hud_patch_names=tuple(f"H{i}" for i in range(len(overlays["hud_w"]))),
+            hud_patch_atlas=overlays["hud_atlas"], hud_patch_opaque=overlays["hud_opaque"].astype(bool),
+            hud_patch_widths=overlays["hud_w"], hud_patch_heights=overlays["hud_h"],
+            hud_patch_left_offsets=overlays["hud_left"], hud_patch_top_offsets=overlays["hud_top"],
+        )
     return scenario.CompiledScenario(
         scenario_sha256="s" * 64,
         iwad_sha256="i" * 64,
@@ -93,9 +106,9 @@ def to_compiled_scenario(smap, *, flash_lights: bool = False):
     )
 
 
-def make_engine(smap, lanes: int, *, flash_lights: bool = False):
+def make_engine(smap, lanes: int, *, flash_lights: bool = False, overlays: dict | None = None):
     engine_module, _scenario = load_reference()
-    compiled = to_compiled_scenario(smap, flash_lights=flash_lights)
+    compiled = to_compiled_scenario(smap, flash_lights=flash_lights, overlays=overlays)
     return engine_module.TorchDeathmatchEngine(compiled, lanes, device=torch.device("cpu"))
 
 
@@ -188,4 +201,58 @@ def packed_sprites(engine):
         sprite_fullbright=torch.cat(
             (fullbright, torch.zeros_like(drop_visible[:, drop_slots])), dim=1
         ).numpy(),
+    )
+
+
+def set_overlay_state(engine, seed: int) -> None:
+    """Randomise the gameplay tensors the weapon and status bar layers read (engine.py:14949-15267)."""
+
+    n = engine.num_envs
+    g = torch.Generator().manual_seed(seed)
+
+    def integers(low, high, dtype):
+        return torch.randint(low, high, (n,), generator=g).to(dtype)
+
+    cooldowns = engine.map.native_weapon_frame_ids.shape[2]
+    engine.selected_weapon.copy_(integers(0, engine._slot_base_weapon.shape[0], torch.int64))
+    engine.selected_weapon_variant.copy_(integers(0, 2, torch.bool))
+    engine.weapon_state_cooldown.copy_(integers(0, cooldowns + 1, torch.int32))
+    engine.weapon_state_cooldown[::3] = 0
+    engine.weapon_fire_count.copy_(integers(0, 9, torch.int32))
+    engine.weapon_ready_tics.copy_(integers(0, 40, torch.int32))
+    engine.weapon_raise_cooldown.copy_(integers(0, 8, torch.int32))
+    engine.weapon_raise_cooldown[::2] = 0
+    engine.weapon_lower_cooldown.copy_(integers(0, 20, torch.int32))
+    engine.pending_weapon.copy_(torch.where(torch.rand(n, generator=g) < 0.3, integers(0, 7, torch.int64), torch.full((n,), -1)))
+    engine.episode_time.copy_(integers(1, 400, torch.int32))
+    engine.episode_time[0] = 3   # spawn raise still running
+    engine._player_bob_fixed.copy_(integers(0, 16 * 65536, torch.int64))
+    engine.health.copy_(integers(-20, 201, torch.float32) + 0.5)
+    engine.health[1] = 0.0
+    engine.player_dead.copy_(engine.health <= 0)
+    engine.armor.copy_(integers(0, 250, torch.float32) + 0.25)
+    engine.hud_ready_ammo.copy_(integers(0, 1100, torch.float32))
+    engine.weapons.copy_((torch.rand((n, engine.weapons.shape[1]), generator=g) < 0.5).to(engine.weapons.dtype))
+    engine.hud_ammo_counts.copy_(torch.randint(0, 400, (n, 4), generator=g).to(engine.hud_ammo_counts.dtype))
+    engine.mugshot_face_index.copy_(integers(0, 3, torch.int64))
+    engine.mugshot_grin_tics.copy_(torch.where(torch.rand(n, generator=g) < 0.2, integers(1, 9, torch.int32), torch.zeros(n, dtype=torch.int32)))
+    engine.mugshot_pain_tics.copy_(torch.where(torch.rand(n, generator=g) < 0.4, integers(1, 9, torch.int32), torch.zeros(n, dtype=torch.int32)))
+    engine.mugshot_ouch.copy_(integers(0, 2, torch.bool))
+    engine.mugshot_pain_direction.copy_(integers(0, 3, torch.int64))
+    engine.attack_held_tics.copy_(torch.where(torch.rand(n, generator=g) < 0.3, integers(70, 100, torch.int32), integers(0, 70, torch.int32)))
+
+
+def overlay_engine_tensors(engine) -> dict:
+    """The engine tensors ``overlay_inputs.weapon_state`` / ``hud_state`` take, by their argument names."""
+
+    return dict(
+        active_weapon=engine._active_weapon(), weapon_state_cooldown=engine.weapon_state_cooldown,
+        weapon_fire_count=engine.weapon_fire_count, weapon_ready_tics=engine.weapon_ready_tics,
+        weapon_lower_cooldown=engine.weapon_lower_cooldown, weapon_raise_cooldown=engine.weapon_raise_cooldown,
+        pending_weapon=engine.pending_weapon, episode_time=engine.episode_time, player_bob_fixed=engine._player_bob_fixed,
+        player_dead=engine.player_dead, weapon_ammo_slot=engine._weapon_ammo_slot, hud_ready_ammo=engine.hud_ready_ammo,
+        health=engine.health, armor=engine.armor, weapons=engine.weapons, hud_ammo_counts=engine.hud_ammo_counts,
+        mugshot_face_index=engine.mugshot_face_index, mugshot_grin_tics=engine.mugshot_grin_tics,
+        mugshot_pain_tics=engine.mugshot_pain_tics, mugshot_ouch=engine.mugshot_ouch,
+        mugshot_pain_direction=engine.mugshot_pain_direction, attack_held_tics=engine.attack_held_tics,
     )

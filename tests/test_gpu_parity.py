@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 import torch
 
-from conftest import fixture_names, lane_inputs, load_fixture
+from conftest import fixture_names, fixture_overlays, lane_inputs, load_fixture
 
 pytestmark = pytest.mark.gpu
 
@@ -16,6 +16,9 @@ def _renderer(name):
 
     meta, data, smap, tables = load_fixture(name)
     renderer = HipRenderer(smap, meta["lanes"], "cuda:0", cosine_correction=data["cosine_correction"], tables=tables)
+    overlays = fixture_overlays(meta)
+    if overlays is not None:
+        renderer.set_overlays(overlays)
     lanes = LaneState.from_numpy(lane_inputs(data), "cuda:0")
     return meta, data, tables, renderer, lanes
 

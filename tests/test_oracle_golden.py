@@ -5,7 +5,7 @@ from __future__ import annotations
 import numpy as np
 import pytest
 
-from conftest import fixture_names, lane_inputs, load_fixture
+from conftest import fixture_names, fixture_overlays, lane_inputs, load_fixture
 
 # Cases whose oracle run takes more than a few seconds on the CPU are trimmed to a lane subset.
 LANE_LIMIT = {"config3_subset": 1, "config4_subset": 1}
@@ -15,10 +15,16 @@ LANE_LIMIT = {"config3_subset": 1, "config4_subset": 1}
 def test_indexed_frame_bit_exact_and_observation_within_one(oracle, name):
     meta, data, _smap, tables = load_fixture(name)
     lanes = min(meta["lanes"], LANE_LIMIT.get(name, meta["lanes"]))
-    result = oracle.render(tables, lane_inputs(data), data["cosine_correction"], lane_range=(0, lanes))
+    overlays = fixture_overlays(meta)
+    oracle.set_overlays(overlays)
+    try:
+        result = oracle.render(tables, lane_inputs(data), data["cosine_correction"], lane_range=(0, lanes))
+    finally:
+        oracle.set_overlays(None)
     assert np.array_equal(result["indexed"][:lanes], data["indexed"][:lanes])
-    # rows 208..239: empty status bar on synthetic maps (engine.py:15232-15267 with a zero HUD atlas)
-    assert not result["indexed"][:lanes, 208:].any()
+    # rows 208..239: empty status bar without status bar patches (engine.py:15232-15267 with a zero HUD
+    # atlas), the drawn bar with them
+    assert bool(result["indexed"][:lanes, 208:].any()) == (overlays is not None)
     # The reference CPU path pools in float32 matmuls; the oracle uses the exact integer
     # form of the reference's GPU branch. Tolerance from tests/test_rendering.py:138-139.
     delta = np.abs(result["obs"][:lanes].astype(np.int32) - data["obs"][:lanes].astype(np.int32))
