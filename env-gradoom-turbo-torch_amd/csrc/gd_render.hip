@@ -2639,6 +2639,8 @@ int launch_chunk(gd_renderer *r, Scratch &sc, const gd_lanes_desc *lanes, const 
         HIP_TRY(hipStreamWaitEvent(side, r->fork_event, 0));
     }
     hipLaunchKernelGGL(wall_setup_kernel, dim3((m.wall_count + 127) / 128, count), dim3(128), 0, stream, r->dm, count, sc);
+    hipLaunchKernelGGL(strip_key_kernel, dim3((count * (SW / 64) + 3) / 4), dim3(256), 0, stream, count, sc);
+    hipLaunchKernelGGL(strip_order_kernel, dim3(1), dim3(1024), 0, stream, count * (SW / 64), sc);
     mark();
     hipLaunchKernelGGL(lane_tables_kernel, dim3(count), dim3(256), 0, flat_stream, r->dm, *lanes, base, count, sc);
     hipLaunchKernelGGL(flat_select_kernel, dim3((VH * SW + 255) / 256, count), dim3(256), 0, flat_stream, r->dm, *lanes, base, count, sc);
@@ -2646,8 +2648,6 @@ int launch_chunk(gd_renderer *r, Scratch &sc, const gd_lanes_desc *lanes, const 
     hipLaunchKernelGGL(flat_finish_kernel, dim3(count), dim3(SW), 0, flat_stream, r->dm, count, sc, frame_base, frame_stride);
     mark();
     if (overlap) HIP_TRY(hipEventRecord(r->flat_event, side));
-    hipLaunchKernelGGL(strip_key_kernel, dim3((count * (SW / 64) + 3) / 4), dim3(256), 0, stream, count, sc);
-    hipLaunchKernelGGL(strip_order_kernel, dim3(1), dim3(1024), 0, stream, count * (SW / 64), sc);
     hipLaunchKernelGGL(wall_columns_kernel, dim3((count * (SW / 64) + WALL_STRIPS_PER_GROUP - 1) / WALL_STRIPS_PER_GROUP), dim3(64 * WALL_STRIPS_PER_GROUP), WALL_LDS_PAD, stream, r->dm, count, sc, frame_base, frame_stride);
     mark();
     if (overlap) HIP_TRY(hipStreamWaitEvent(stream, r->flat_event, 0));
