@@ -1,15 +1,22 @@
 // MI355X (gfx950) batched software renderer + observation pipeline.
 //
-// One frame for N lanes runs as a short chain of kernels on one stream:
+// One frame for N lanes runs as a short chain of kernels on two streams (walls on the caller's stream, flats
+// on a side stream that forks after lane_setup and joins before plane_shade):
 //
-//   lane_setup     1 thread / lane          view basis, pitch centre, camera sector
-//   wall_setup     1 thread / (lane, wall)  FWallCoords span+depths, span ownership bounds, and the
-//                                           linedef's entry in the candidate list of every column it can own
-//   flat_select    1 thread / pixel         nearest floor/ceiling sector through the point grid
-//   flat_finish    320 threads / lane       visplane repair (wave ballots) + flat shading
-//   wall_columns   320 threads / lane       portal traversal, tiers, planes, masked mid-textures
-//   sprite_columns 320 threads / lane       billboards far -> near
-//   observe        1 thread / obs pixel     PLAYPAL + exact area pool + gray + 4-frame stack
+//   lane_setup      1 thread / lane           view basis, pitch centre, camera sector
+//   wall_setup      1 wave-slot / (lane,wall) FWallCoords span+depths, span ownership bounds, the linedef's
+//                                             entry in the candidate list of every column it can own, and the
+//                                             nearest blocking hit of every column (64-bit atomicMin)
+//   strip_key/order 1 thread / 64-col strip   longest strip first (counting sort on the blocking distance)
+//   lane_tables     1 thread / (lane, row)    per-lane reach of every height level, plane rows, row slopes
+//   flat_select     1 thread / pixel          nearest floor/ceiling sector through the fine point raster
+//   flat_finish     320 threads / lane        visplane repair (wave ballots), status bar rows cleared
+//   wall_columns    1 wave / strip            portal traversal, tiers, planes, masked mid-textures
+//   plane_shade     1 thread / 4 pixels       flat texel + light for every pixel a wall did not cover
+//   sprite_columns  320 threads / lane        billboards far -> near
+//   weapon_overlay, hud                       player weapon, muzzle flash and status bar patches
+//   observe         1 thread / obs pixel      PLAYPAL + exact area pool + gray + 4-frame stack
+//   expand_rgb      1 thread / pixel          PLAYPAL expansion for callers that want RGB24 frames
 //
 // All fixed-point arithmetic is int64 like the reference's Torch code; float32
 // expressions are evaluated operation by operation (-ffp-contract=off) so that

@@ -448,9 +448,31 @@ def generate_poses(
     pitch: bool = False,
     flash: bool = False,
     frame: int = 0,
+    margin: float = 0.15,
 ) -> Poses:
-    """Random camera poses strictly inside sectors (bilinear margin keeps them off the walls)."""
+    """Random camera poses strictly inside sectors (bilinear margin keeps them off the walls).
 
+    A small ``margin`` puts cameras close to walls and vertices, where linedefs are seen edge-on and
+    the thin-span ownership rules of the wall traversal come into play.
+    """
+
+    return generate_picked_poses(
+        smap, [(seed, lane) for lane in range(lanes)], pitch=pitch, flash=flash, frame=frame, margin=margin
+    )
+
+
+def generate_picked_poses(
+    smap: SynthMap,
+    picks,
+    *,
+    pitch: bool = False,
+    flash: bool = False,
+    frame: int = 0,
+    margin: float = 0.15,
+) -> Poses:
+    """The poses ``generate_poses`` gives lane ``lane`` under ``seed``, for a list of (seed, lane) pairs."""
+
+    lanes = len(picks)
     x = np.zeros(lanes, dtype=np.float32)
     y = np.zeros(lanes, dtype=np.float32)
     angle_bam = np.zeros(lanes, dtype=np.int64)
@@ -459,19 +481,19 @@ def generate_poses(
     flash_light = np.zeros(lanes, dtype=np.int64)
     sector = np.zeros(lanes, dtype=np.int32)
     sector_count = len(smap.sector_heights)
-    for lane in range(lanes):
+    for slot, (seed, lane) in enumerate(picks):
         rng = np.random.default_rng((seed * 65536 + lane) * 4096 + frame)
         s = int(rng.integers(0, sector_count))
-        u, v = rng.uniform(0.15, 0.85, 2)
+        u, v = rng.uniform(margin, 1.0 - margin, 2)
         px, py = _point_in_cell(smap, s, float(u), float(v))
-        x[lane], y[lane] = px, py
-        angle_bam[lane] = int(rng.integers(0, 1 << 32))
-        view_z[lane] = smap.sector_heights[s, 0] + 41.0
+        x[slot], y[slot] = px, py
+        angle_bam[slot] = int(rng.integers(0, 1 << 32))
+        view_z[slot] = smap.sector_heights[s, 0] + 41.0
         if pitch:
-            pitch_bam[lane] = int(rng.integers(-10, 11)) * (182 << 16)
+            pitch_bam[slot] = int(rng.integers(-10, 11)) * (182 << 16)
         if flash:
-            flash_light[lane] = int(rng.integers(0, 3))
-        sector[lane] = s
+            flash_light[slot] = int(rng.integers(0, 3))
+        sector[slot] = s
     return Poses(x, y, angle_bam, pitch_bam, view_z, flash_light, sector)
 
 

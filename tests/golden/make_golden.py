@@ -73,6 +73,21 @@ CASES = {
     "overlays": dict(
         map_seed=12, grid=(5, 4), sectors=17, linedefs=100, lanes=12, pose_seed=4, pitch=True, sprites=16, overlays=71
     ),
+    # Single-column events found by searching seeded maps and poses with the oracle's rule counters: the
+    # equal-depth solid replacement, the solid bridge, the sector bridge and the tied-strip rule fire on
+    # the picked (pose seed, lane) pairs; the other lanes are close-to-wall poses of the same maps.
+    "rare_rules_brick26": dict(
+        map_seed=3001, grid=(6, 5), sectors=26, linedefs=260, lanes=6, layout="brick", islands=10, midtex=0.1,
+        picks=[(1, 14), (5, 1), (8, 8), (1, 0), (5, 0), (8, 0)], pose_seed=1,
+    ),
+    "rare_rules_brick18": dict(
+        map_seed=3023, grid=(5, 4), sectors=18, linedefs=170, lanes=4, layout="brick", islands=6, midtex=0.1,
+        picks=[(3, 10), (3, 0), (3, 1), (3, 2)], pose_seed=3,
+    ),
+    "grazing_brick26": dict(
+        map_seed=3001, grid=(6, 5), sectors=26, linedefs=260, lanes=8, layout="brick", islands=10, midtex=0.1,
+        picks=[(1, 10), (3, 1), (1, 0), (1, 1), (1, 2), (3, 0), (3, 2), (3, 3)], margin=0.02, pose_seed=1, pitch=True,
+    ),
     "config2_subset": dict(map_seed=1002, grid=(12, 9), sectors=96, linedefs=800, lanes=4, pose_seed=1, sprites=32),
     "config3_subset": dict(
         map_seed=1003, grid=(15, 15), sectors=200, linedefs=2000, lanes=2, pose_seed=1, sprites=64, flash=True
@@ -93,8 +108,10 @@ def build_case(name: str, cfg: dict, do_time: bool) -> dict:
     overlays = synthmap.generate_overlays(cfg["overlays"]) if cfg.get("overlays") else None
     engine = refdrive.make_engine(smap, lanes, flash_lights=cfg.get("flash", False), overlays=overlays)
     ctor_seconds = time.time() - started
-    poses = synthmap.generate_poses(
-        smap, lanes, cfg["pose_seed"], pitch=cfg.get("pitch", False), flash=cfg.get("flash", False)
+    picks = cfg.get("picks") or [(cfg["pose_seed"], lane) for lane in range(lanes)]
+    assert len(picks) == lanes
+    poses = synthmap.generate_picked_poses(
+        smap, picks, pitch=cfg.get("pitch", False), flash=cfg.get("flash", False), margin=cfg.get("margin", 0.15)
     )
     refdrive.set_poses(engine, poses)
     offsets = hostmath.native_ray_offsets("cpu")

@@ -9,10 +9,11 @@ EXERCISED = (
     "projected_solid", "endpoint_owner", "near_projected", "topological_owner", "opposing_boundary", "excluded_right_edge",
     "continues_owner_boundary", "forward_bridge", "completes_endpoint_bridge", "endpoint_only_portal", "enters_other",
     "enters_shared", "geometric_path", "portal_bridge", "completes_portal_bridge", "ps_keeps_path", "no_keeps_path",
-    "bottom_tail", "masked_column", "masked_extends", "dead_column_revived",
+    "bottom_tail", "masked_column", "masked_extends", "dead_column_revived", "equal_depth_solid", "solid_bridge",
+    "sector_bridge", "tied_strip",
 )
-# Rules no fixture reaches yet; parity of these branches rests on reading alone.
-NOT_EXERCISED = ("equal_depth_solid", "solid_bridge", "sector_bridge", "tied_strip")
+# Rules no fixture reaches; parity of such branches would rest on reading alone.
+NOT_EXERCISED = ()
 
 
 def test_fixture_set_fires_the_listed_rules(oracle):
