@@ -66,6 +66,7 @@ class SynthMap:
     sector_cells: np.ndarray  # [S,2] i32 grid cell of each sector (generator bookkeeping)
     grid_points: np.ndarray  # [gy+1,gx+1,2] f32 jittered grid vertices
     sector_quads: np.ndarray | None = None  # [S,4,2] f64 corners p00,p10,p01,p11 used to place cameras/sprites
+    void_boxes: np.ndarray | None = None  # [B,4] f64 x0,y0,x1,y1 of void pillars inside sectors (no camera goes there)
 
     @property
     def blocking_segments(self) -> np.ndarray:
@@ -137,11 +138,12 @@ def generate_map(
     sprite_patches: int = 64,
     layout: str = "grid",
     islands: int = 0,
+    pillars: int = 0,
 ) -> SynthMap:
     if layout == "brick":
         return _generate_brick_map(
             seed, grid=grid, sectors=sectors, linedefs=linedefs, midtex=midtex, wall_textures=wall_textures,
-            flats=flats, sprite_patches=sprite_patches, islands=islands,
+            flats=flats, sprite_patches=sprite_patches, islands=islands, pillars=pillars,
         )
     if layout != "grid":
         raise ValueError("layout must be 'grid' or 'brick'")
@@ -202,7 +204,7 @@ def generate_map(
         quads[index] = (points[j, i], points[j, i + 1], points[j + 1, i], points[j + 1, i + 1])
     return _finish_map(
         rng, edges, sector_cells, points, quads, linedefs=linedefs, midtex=midtex, wall_textures=wall_textures,
-        flats=flats, sprite_patches=sprite_patches, islands=islands,
+        flats=flats, sprite_patches=sprite_patches, islands=islands, pillars=pillars,
     )
 
 
@@ -235,9 +237,45 @@ def _add_islands(rng, edges, sector_cells, sector_quads, count):
     return edges, cells, np.asarray(quads, dtype=np.float64)
 
 
-def _finish_map(rng, edges, sector_cells, points, sector_quads, *, linedefs, midtex, wall_textures, flats, sprite_patches, islands=0):
+def _add_pinched_pillars(rng, edges, sector_quads, hosts):
+    """Two square void pillars that touch at one corner, in the middle of every host cell.
+
+    Four one-sided linedefs of the same sector meet at the shared corner, so each of them has more than
+    one endpoint neighbour there: the reference then drops its direct neighbour tables and takes the
+    general neighbour-slot search (``engine.py:1558-1577``, ``engine.py:11672-11712``).
+    """
+
+    boxes = []
+    for host in hosts:
+        cx, cy = (float(v) for v in np.round(np.mean(sector_quads[host], axis=0)))
+        a = float(rng.integers(2, 5) * 8)
+        b = float(rng.integers(2, 5) * 8)
+        for x0, y0, x1, y1 in ((cx - a, cy - a, cx, cy), (cx, cy, cx + b, cy + b)):
+            corners = [(x0, y0), (x1, y0), (x1, y1), (x0, y1)]  # counter-clockwise: the void is on the left
+            for k in range(4):
+                edges.append((corners[k], corners[(k + 1) % 4], int(host), -1, MAX_SPLIT_DEPTH))
+            boxes.append((x0, y0, x1, y1))
+    return edges, np.asarray(boxes, dtype=np.float64)
+
+
+def _finish_map(
+    rng, edges, sector_cells, points, sector_quads, *, linedefs, midtex, wall_textures, flats, sprite_patches, islands=0,
+    pillars=0,
+):
+    void_boxes = None
+    if pillars:
+        if islands + pillars > len(sector_cells):
+            raise ValueError("more islands and pillars than cells")
+        # hosts the islands (which draw the same permutation first) will not use
+        state = rng.bit_generator.state
+        island_hosts = set(int(h) for h in rng.permutation(len(sector_cells))[:islands]) if islands else set()
+        rng.bit_generator.state = state
+        free = [h for h in range(len(sector_cells)) if h not in island_hosts]
     if islands:
         edges, sector_cells, sector_quads = _add_islands(rng, edges, sector_cells, sector_quads, islands)
+    if pillars:
+        hosts = [free[int(k)] for k in rng.permutation(len(free))[:pillars]]
+        edges, void_boxes = _add_pinched_pillars(rng, edges, sector_quads, hosts)
     edges = _split_edges(rng, edges, linedefs)
     order = rng.permutation(len(edges))
     edges = [edges[k] for k in order]
@@ -327,11 +365,11 @@ def _finish_map(rng, edges, sector_cells, points, sector_quads, *, linedefs, mid
         sector_cells=np.asarray(sector_cells, dtype=np.int32),
         grid_points=np.asarray(points, dtype=np.float32),
         sector_quads=sector_quads,
+        void_boxes=void_boxes,
     )
 
 
-
-def _generate_brick_map(seed, *, grid, sectors, linedefs, midtex, wall_textures, flats, sprite_patches, islands=0):
+def _generate_brick_map(seed, *, grid, sectors, linedefs, midtex, wall_textures, flats, sprite_patches, islands=0, pillars=0):
     """Staggered rows: odd rows are shifted by half a cell, so every interior vertex joins three sectors.
 
     At such a T-junction all three pairwise linedefs exist, which is what the reference's
@@ -416,7 +454,7 @@ def _generate_brick_map(seed, *, grid, sectors, linedefs, midtex, wall_textures,
     points = np.zeros((1, 1, 2), dtype=np.float64)
     return _finish_map(
         rng, edges, sector_cells, points, quads, linedefs=linedefs, midtex=midtex, wall_textures=wall_textures,
-        flats=flats, sprite_patches=sprite_patches, islands=islands,
+        flats=flats, sprite_patches=sprite_patches, islands=islands, pillars=pillars,
     )
 
 
@@ -484,8 +522,14 @@ def generate_picked_poses(
     for slot, (seed, lane) in enumerate(picks):
         rng = np.random.default_rng((seed * 65536 + lane) * 4096 + frame)
         s = int(rng.integers(0, sector_count))
-        u, v = rng.uniform(margin, 1.0 - margin, 2)
-        px, py = _point_in_cell(smap, s, float(u), float(v))
+        while True:
+            u, v = rng.uniform(margin, 1.0 - margin, 2)
+            px, py = _point_in_cell(smap, s, float(u), float(v))
+            if smap.void_boxes is None or not np.any(
+                (px > smap.void_boxes[:, 0] - 4) & (px < smap.void_boxes[:, 2] + 4)
+                & (py > smap.void_boxes[:, 1] - 4) & (py < smap.void_boxes[:, 3] + 4)
+            ):
+                break
         x[slot], y[slot] = px, py
         angle_bam[slot] = int(rng.integers(0, 1 << 32))
         view_z[slot] = smap.sector_heights[s, 0] + 41.0

@@ -43,6 +43,7 @@ def load_fixture(name: str):
     smap = synthmap.generate_map(
         meta["map_seed"], grid=tuple(meta["grid"]), sectors=meta["sectors"], linedefs=meta["linedefs"],
         midtex=meta.get("midtex", 0.0), layout=meta.get("layout", "grid"), islands=meta.get("islands", 0),
+        pillars=meta.get("pillars", 0),
     )
     assert map_digest(smap) == meta["map_sha256"], "synthetic map generator drifted from the golden fixtures"
     tables = mapbuild.build_map_tables(smap)

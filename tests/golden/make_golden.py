@@ -88,6 +88,12 @@ CASES = {
         map_seed=3001, grid=(6, 5), sectors=26, linedefs=260, lanes=8, layout="brick", islands=10, midtex=0.1,
         picks=[(1, 10), (3, 1), (1, 0), (1, 1), (1, 2), (3, 0), (3, 2), (3, 3)], margin=0.02, pose_seed=1, pitch=True,
     ),
+    # Two void pillars touching at a corner put four same-sector one-sided linedefs on one vertex: the
+    # reference drops its direct endpoint-neighbour tables and searches the neighbour slots instead.
+    "pinched_pillars": dict(
+        map_seed=41, grid=(4, 3), sectors=10, linedefs=120, lanes=8, pose_seed=1, islands=2, pillars=4, midtex=0.1,
+        pitch=True, flash=True, stages=True,
+    ),
     "config2_subset": dict(map_seed=1002, grid=(12, 9), sectors=96, linedefs=800, lanes=4, pose_seed=1, sprites=32),
     "config3_subset": dict(
         map_seed=1003, grid=(15, 15), sectors=200, linedefs=2000, lanes=2, pose_seed=1, sprites=64, flash=True
@@ -101,7 +107,7 @@ CASES = {
 def build_case(name: str, cfg: dict, do_time: bool) -> dict:
     smap = synthmap.generate_map(
         cfg["map_seed"], grid=cfg["grid"], sectors=cfg["sectors"], linedefs=cfg["linedefs"], midtex=cfg.get("midtex", 0.0),
-        layout=cfg.get("layout", "grid"), islands=cfg.get("islands", 0),
+        layout=cfg.get("layout", "grid"), islands=cfg.get("islands", 0), pillars=cfg.get("pillars", 0),
     )
     lanes = cfg["lanes"]
     started = time.time()

@@ -27,3 +27,12 @@ def test_fixture_set_fires_the_listed_rules(oracle):
     assert not missing, f"rules no longer exercised by the fixtures: {missing}"
     newly = [rule for rule in NOT_EXERCISED if counts[rule] > 0]
     assert not newly, f"rules now exercised, move them to EXERCISED: {newly}"
+
+
+def test_one_fixture_takes_the_general_endpoint_neighbour_search():
+    """Every other case has at most one neighbour per endpoint and uses the direct tables (engine.py:1558-1577)."""
+
+    _meta, _data, _smap, tables = load_fixture("pinched_pillars")
+    assert tables["direct_neighbors"] == 0 and tables["neighbor_slots"] >= 3
+    _meta, _data, _smap, tables = load_fixture("config1")
+    assert tables["direct_neighbors"] == 1
