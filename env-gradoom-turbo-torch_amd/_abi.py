@@ -41,6 +41,8 @@ MAP_SCALARS = (
     "grid_ny",
     "fine_nx",
     "fine_ny",
+    "fragment_slots",
+    "split_count",
 )
 MAP_FLOATS = ("grid_min_x", "grid_min_y", "grid_cell", "fine_cell")
 
@@ -68,6 +70,9 @@ MAP_ARRAYS = (
     ("sector_edge_ofs", np.int32),
     ("sector_edge_idx", np.int32),
     ("blocking_walls", np.int32),
+    ("wall_split_slot", np.int32),
+    ("split_fragments_fixed", np.int32),
+    ("split_fragment_mask", np.uint8),
     ("grid_cell_ofs", np.int32),
     ("grid_item_sector", np.int32),
     ("grid_item_edge_ofs", np.int32),

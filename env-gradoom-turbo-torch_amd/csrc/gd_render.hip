@@ -70,6 +70,7 @@ typedef unsigned long long u64;
 #define WF_FF 2        // front facing (float32 test of engine.py:11376-11381)
 #define WF_SUBPIXEL 4  // two-sided and at most one column wide (engine.py:11589-11591)
 #define WF_ANYGEO 8    // some column ray hits the segment
+#define WF_SPLIT 16    // projects through BSP fragments (engine.py:11472-11545, 12310-12380)
 
 struct LaneCtx {
     float x, y, view_z, pitch_offset, fsin, fcos;
@@ -133,6 +134,7 @@ struct Overlays {   // device copy of gd_overlay_desc; count 0 = layer not loade
 struct Scratch {    // per-chunk working memory, sized at create
     LaneCtx *ctx;          // [L]
     WallRec *rec;          // [L,W]
+    WallRec *frag_rec;     // [L,split_count,fragment_slots] FWallCoords of the BSP fragments of split linedefs
     Cand *cand;            // [L,CAND_MAX,320]
     int *cand_count;       // [L,320] (may exceed CAND_MAX when a list overflowed)
     unsigned short *flat_sector;// [L,208,320]
@@ -483,21 +485,9 @@ __device__ __forceinline__ Eval eval_wall(const gd_map_desc *m, const LaneCtx &c
 // ---------------------------------------------------------------------------------------------
 // wall_setup: engine.py:10747-10869 (FWallCoords) and the per-linedef half of 11304-11451
 // ---------------------------------------------------------------------------------------------
-//
-// One thread owns one linedef for the per-linedef arithmetic.  The two per-column loops have
-// wildly different trip counts per linedef (none for most, up to 320 for a few), so they are
-// run by the whole wavefront together: the linedefs with a non-empty column range take turns,
-// their parameters are broadcast from the owning lane, and the 64 lanes each take one column.
-__global__ void __launch_bounds__(128) wall_setup_kernel(DeviceMap dm, int lane_count, Scratch sc) {
-    const gd_map_desc *m = &dm.d;
-    const int slot_in_wave = threadIdx.x & 63;
-    const int w_raw = blockIdx.x * blockDim.x + threadIdx.x;
-    const int local = blockIdx.y;
-    if (local >= lane_count) return;          // uniform over the block
-    const bool live = w_raw < m->wall_count;  // dead lanes still help with the column loops
-    const int w = live ? w_raw : 0;
-    const LaneCtx &c = sc.ctx[local];
-    const int *wf = m->walls_fixed + 4 * w;
+// FWallCoords of one fixed-point segment seen from one lane (engine.py:10747-10869): view-space
+// endpoints, clipped half-open screen span and clipped endpoint depths.
+__device__ __forceinline__ void wall_coords(const LaneCtx &c, const int *wf, WallRec &r) {
     i64 rx0 = (i64)wf[0] - c.view_x_fixed, ry0 = (i64)wf[1] - c.view_y_fixed;
     i64 rx1 = (i64)wf[2] - c.view_x_fixed, ry1 = (i64)wf[3] - c.view_y_fixed;
     i64 tx0 = (rx0 * c.vsin - ry0 * c.vcos) >> 20, ty0 = (rx0 * c.vcos + ry0 * c.vsin) >> 20;
@@ -524,6 +514,42 @@ __global__ void __launch_bounds__(128) wall_setup_kernel(DeviceMap dm, int lane_
     bool invalid_right = (right_inside ? ((tx2 < -ty2) || (ty2 == 0)) : ((tx1 > ty1) || (right_den == 0))) || (dr < 32);
     bool invalid = invalid_left || invalid_right || (sr <= sl);
     if (invalid) sr = sl;
+    r.tx0 = (int)tx0; r.tx1 = (int)tx1v; r.ty0 = (int)ty0; r.ty1 = (int)ty1v;
+    r.dl = dl; r.dr = dr; r.sl = sl; r.sr = sr;
+}
+
+// Every fragment of every split linedef of one lane (engine.py:11472-11500).
+__global__ void fragment_setup_kernel(DeviceMap dm, int lane_count, Scratch sc) {
+    const gd_map_desc *m = &dm.d;
+    const int per_lane = m->split_count * m->fragment_slots;
+    const int k = blockIdx.x * blockDim.x + threadIdx.x;
+    const int local = blockIdx.y;
+    if (local >= lane_count || k >= per_lane) return;
+    WallRec r;
+    wall_coords(sc.ctx[local], m->split_fragments_fixed + 4 * (size_t)k, r);
+    r.pl = 0; r.pr = 0; r.flags = 0;
+    sc.frag_rec[(size_t)local * per_lane + k] = r;
+}
+
+// One thread owns one linedef for the per-linedef arithmetic.  The two per-column loops have
+// wildly different trip counts per linedef (none for most, up to 320 for a few), so they are
+// run by the whole wavefront together: the linedefs with a non-empty column range take turns,
+// their parameters are broadcast from the owning lane, and the 64 lanes each take one column.
+__global__ void __launch_bounds__(128) wall_setup_kernel(DeviceMap dm, int lane_count, Scratch sc) {
+    const gd_map_desc *m = &dm.d;
+    const int slot_in_wave = threadIdx.x & 63;
+    const int w_raw = blockIdx.x * blockDim.x + threadIdx.x;
+    const int local = blockIdx.y;
+    if (local >= lane_count) return;          // uniform over the block
+    const bool live = w_raw < m->wall_count;  // dead lanes still help with the column loops
+    const int w = live ? w_raw : 0;
+    const LaneCtx &c = sc.ctx[local];
+    const int *wf = m->walls_fixed + 4 * w;
+    WallRec r;
+    wall_coords(c, wf, r);
+    const i64 tx0 = r.tx0, tx1v = r.tx1, ty0 = r.ty0, ty1v = r.ty1;
+    const i64 sl = r.sl, sr = r.sr;
+    const i64 center = 160 * FIXED_UNIT;
 
     // Ray x segment: first / last column whose ray hits the segment (engine.py:11323-11348).
     // A ray of column parameter col = (x-160)/160 is forward + col*right; an endpoint with view
@@ -606,11 +632,9 @@ __global__ void __launch_bounds__(128) wall_setup_kernel(DeviceMap dm, int lane_
     hc = hc && (sr > sl);
     const int s0 = m->wall_sectors[2 * w], s1 = m->wall_sectors[2 * w + 1];
     bool os = s1 < 0;
-    WallRec r;
-    r.tx0 = (int)tx0; r.tx1 = (int)tx1v; r.ty0 = (int)ty0; r.ty1 = (int)ty1v;
-    r.dl = dl; r.dr = dr; r.sl = sl; r.sr = sr;
     r.pl = (short)screen_left; r.pr = (short)screen_right;
-    r.flags = (hc ? WF_HC : 0) | (ff ? WF_FF : 0) | (((sr - sl <= 1) && !os) ? WF_SUBPIXEL : 0) | (any ? WF_ANYGEO : 0);
+    r.flags = (hc ? WF_HC : 0) | (ff ? WF_FF : 0) | (((sr - sl <= 1) && !os) ? WF_SUBPIXEL : 0) | (any ? WF_ANYGEO : 0) |
+              (m->wall_split_slot[w] >= 0 ? WF_SPLIT : 0);
     if (live) sc.rec[(size_t)local * m->wall_count + w] = r;
     // Enter the linedef in the candidate list of every column where its distance can be
     // finite: its owned span (projected) and, for two-sided lines, the columns its rays hit
@@ -997,6 +1021,7 @@ struct ColumnCtx {
     MapView mv;
     const LaneCtx *c;
     const WallRec *recs;
+    const WallRec *frags; // this lane's [split_count, fragment_slots] fragment records
     const Cand *list;     // this lane's candidate block, entry k of column x at [k*320 + x]
     int count;
     int x;
@@ -1014,6 +1039,35 @@ struct ColumnCtx {
     }
     __device__ Eval eval(int w) const { return eval_wall(m, *c, recs, x, w, rx, ry); }
 };
+
+// The projection fragment of a linedef at one column (engine.py:11511-11529, 12324-12376): the first
+// present fragment whose half-open span holds the column.  A linedef that was never split is its own
+// fragment.  `has` is false where no fragment holds the column (OWallMost then falls back to the whole
+// linedef, engine.py:12598-12604); `lights` tells whether wallscan light interpolates over the fragment,
+// which only linedefs with several fragments do (engine.py:11530-11545).
+struct FragmentChoice {
+    const WallRec *rec;
+    bool has, lights;
+};
+__device__ __forceinline__ FragmentChoice choose_fragment(const gd_map_desc *m, const WallRec *frags, const WallRec &whole, int w, int x) {
+    FragmentChoice f;
+    f.rec = &whole; f.lights = false;
+    f.has = (whole.sr > whole.sl) && (x >= whole.sl) && (x < whole.sr);
+    if (whole.flags & WF_SPLIT) {
+        const int F = m->fragment_slots, row = m->wall_split_slot[w];
+        int count = 0;
+        f.has = false;
+        for (int k = 0; k < F; ++k) {
+            if (!m->split_fragment_mask[row * F + k]) continue;
+            ++count;
+            const WallRec &g = frags[row * F + k];
+            if (!f.has && (g.sr > g.sl) && (x >= g.sl) && (x < g.sr)) { f.rec = &g; f.has = true; }
+        }
+        f.lights = f.has && count > 1;
+        if (!f.has) f.rec = &whole;
+    }
+    return f;
+}
 
 // engine.py:11217-11291 for one endpoint order, evaluated at one column
 __device__ i64 wall_visibility(const WallRec &r, int side, int x) {
@@ -1059,11 +1113,12 @@ __device__ void texture_mapping(const gd_map_desc *m, const WallRec &r, int w, i
 }
 
 // engine.py:12294-12605 (OWallMost) for one column
-__device__ __forceinline__ float project(const LaneCtx &c, const WallRec &g, float world_z, int x) {
+__device__ __forceinline__ float project(const LaneCtx &c, const WallRec &g, const FragmentChoice &fragment, float world_z, int x) {
     i64 whole_sl = g.sl, whole_sr = g.sr;
     i64 whole_dl = max64(g.dl, 1), whole_dr = max64(g.dr, 1);
-    bool has_fragment = (g.sr > g.sl) && (x >= g.sl) && (x < g.sr);
-    i64 screen_left = g.sl, screen_right = g.sr, depth_left = whole_dl, depth_right = whole_dr;
+    const bool has_fragment = fragment.has;
+    const WallRec &f = *fragment.rec;
+    i64 screen_left = f.sl, screen_right = f.sr, depth_left = max64(f.dl, 1), depth_right = max64(f.dr, 1);
     i64 relative_z_fixed = round_to_i64((world_z - c.view_z) * 65536.0f);
     i64 pz = -(relative_z_fixed >> 4);
     i64 center_fixed = c.center_fixed;
@@ -1413,7 +1468,8 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
     r.wall = wi; r.side = side; r.render_current = render_current; r.other_sector = other_sector;
     r.distance = distance;
     const WallRec &wr = cc.recs[wi];
-    r.visibility = wall_visibility(wr, side, x);
+    const FragmentChoice wr_fragment = choose_fragment(m, cc.frags, wr, wi, x);
+    r.visibility = wall_visibility(wr_fragment.lights ? *wr_fragment.rec : wr, side, x);
     const Tables &tb = *cc.tb;
     r.view_floor = tb.floor_h(render_current); r.view_ceiling = tb.ceil_h(render_current);
     r.other_floor = tb.floor_h(safe_other); r.other_ceiling = tb.ceil_h(safe_other);
@@ -1424,7 +1480,7 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
 #pragma unroll 1
     for (int k = 0; k < 4; ++k) {   // one copy of the projection code, four heights
         float z = k == 0 ? r.view_ceiling : (k == 1 ? r.view_floor : (k == 2 ? r.other_floor : r.other_ceiling));
-        float v = project(*cc.c, wr, z, x);
+        float v = project(*cc.c, wr, wr_fragment, z, x);
         if (k == 0) one_top = v; else if (k == 1) one_bottom = v; else if (k == 2) lower_top = v; else upper_bottom = v;
     }
     r.clipped_top = fmaxf(one_top, c.ceiling_clip);
@@ -1668,6 +1724,7 @@ __device__ __forceinline__ bool pass_advance(const ColumnCtx &cc, ColumnState &c
     if (r.bits & PB_PS_KEEPS) {
         int path = r.ps_path_index;
         const WallRec &pr = cc.recs[path];
+        const FragmentChoice pr_fragment = choose_fragment(m, cc.frags, pr, path, x);
         int path_safe_other = r.ps_other < 0 ? 0 : r.ps_other;
         const Tables &tb = *cc.tb;
         float pof = tb.floor_h(path_safe_other), poc = tb.ceil_h(path_safe_other);
@@ -1677,7 +1734,7 @@ __device__ __forceinline__ bool pass_advance(const ColumnCtx &cc, ColumnState &c
 #pragma unroll 1
         for (int k = 0; k < 4; ++k) {
             float z = k == 0 ? r.view_ceiling : (k == 1 ? r.view_floor : (k == 2 ? pof : poc));
-            float v = project(L, pr, z, x);
+            float v = project(L, pr, pr_fragment, z, x);
             if (k == 0) path_top = v; else if (k == 1) path_bottom = v; else if (k == 2) path_lower_top = v; else path_upper_bottom = v;
         }
         float pct = fmaxf(path_top, c.ceiling_clip);
@@ -1829,6 +1886,7 @@ __device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const Col
     bool has_saved = c.masked_wall == mw;
     if (!(has_saved || left_edge)) return;
     const WallRec &wr = cc.recs[mw];
+    const FragmentChoice wr_fragment = choose_fragment(m, cc.frags, wr, mw, x);
     int front_sector = mv.sec(mw, 0), back_sector = mv.sec(mw, 1) < 0 ? 0 : mv.sec(mw, 1);
     int light_sector = mside == 0 ? front_sector : back_sector;
     const Tables &tb = *cc.tb;
@@ -1837,7 +1895,7 @@ __device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const Col
     float owall_top = 0, owall_bottom = 0;
 #pragma unroll 1
     for (int k = 0; k < 2; ++k) {
-        float v = project(L, wr, k == 0 ? world_top : world_top - (float)th, x);
+        float v = project(L, wr, wr_fragment, k == 0 ? world_top : world_top - (float)th, x);
         if (k == 0) owall_top = v; else owall_bottom = v;
     }
     float mceil = fmaxf(owall_top, has_saved ? c.masked_ceiling_clip : 0.0f);
@@ -1888,7 +1946,7 @@ __device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const Col
     bool horizontal = fabsf(wl.w - wl.y) < 1e-6f, vertical = fabsf(wl.z - wl.x) < 1e-6f;
     float contrast = vertical ? 16.0f : (horizontal ? -16.0f : 0.0f);
     float light = (tb.light(light_sector) + (float)(L.flash_light * 16)) + contrast;
-    i64 shade = wall_shade(light, wall_visibility(wr, mside, x));
+    i64 shade = wall_shade(light, wall_visibility(wr_fragment.lights ? *wr_fragment.rec : wr, mside, x));
     int y0 = (int)clampi(clipped_top, 0, VH), y1 = (int)clampi(clipped_bottom, 0, VH);
     for (int y = y0; y < y1; ++y) {
         i64 screen_delta = (i64)y * FIXED_UNIT - center_fixed + FIXED_UNIT;
@@ -1977,6 +2035,7 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
     ColumnCtx cc;
     cc.tb = &tb; cc.m = m; cc.mv.m = m; cc.c = &lane_ctx;
     cc.recs = sc.rec + (size_t)local * m->wall_count;
+    cc.frags = sc.frag_rec + (size_t)local * m->split_count * m->fragment_slots;
     cc.list = sc.cand + (size_t)local * CAND_MAX * SW;
     cc.count = sc.cand_count[(size_t)local * SW + x];
     if (cc.count > CAND_MAX) cc.count = CAND_MAX;
@@ -2646,6 +2705,8 @@ int launch_chunk(gd_renderer *r, Scratch &sc, const gd_lanes_desc *lanes, const 
         HIP_TRY(hipStreamWaitEvent(side, r->fork_event, 0));
     }
     hipLaunchKernelGGL(wall_setup_kernel, dim3((m.wall_count + 127) / 128, count), dim3(128), 0, stream, r->dm, count, sc);
+    if (m.split_count > 0)
+        hipLaunchKernelGGL(fragment_setup_kernel, dim3((m.split_count * m.fragment_slots + 63) / 64, count), dim3(64), 0, stream, r->dm, count, sc);
     hipLaunchKernelGGL(strip_key_kernel, dim3((count * (SW / 64) + 3) / 4), dim3(256), 0, stream, count, sc);
     hipLaunchKernelGGL(strip_order_kernel, dim3(1), dim3(1024), 0, stream, count * (SW / 64), sc);
     mark();
@@ -2706,6 +2767,12 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     if (h->fine_nx <= 0 || h->fine_ny <= 0 || !(h->fine_cell > 0.0f) || !h->fine_sector) return fail(GD_E_ARG, "missing fine point-location raster");
     if (h->grid_cell != 8.0f * h->fine_cell || (h->fine_nx + 7) / 8 > h->grid_nx || (h->fine_ny + 7) / 8 > h->grid_ny)
         return fail(GD_E_ARG, "grid_cell must be 8 * fine_cell and the coarse grid must cover the fine raster");
+    if (h->fragment_slots < 1 || h->split_count < 0 || h->split_count > h->wall_count || !h->wall_split_slot ||
+        (h->split_count > 0 && (!h->split_fragments_fixed || !h->split_fragment_mask)))
+        return fail(GD_E_ARG, "invalid projection fragment tables");
+    for (int w = 0; w < h->wall_count; ++w)
+        if (h->wall_split_slot[w] < -1 || h->wall_split_slot[w] >= h->split_count)
+            return fail(GD_E_ARG, "wall_split_slot names a row outside the fragment tables");
     gd_renderer *r = new (std::nothrow) gd_renderer();
     if (!r) return fail(GD_E_ARG, "out of host memory");
     r->events_ready = false;
@@ -2727,6 +2794,12 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     UP(sector_wall_ofs, S + 1); UP(sector_wall_idx, h->sector_wall_ofs[S]);
     UP(sector_edge_ofs, S + 1); UP(sector_edge_idx, h->sector_edge_ofs[S]);
     UP(blocking_walls, h->blocking_count);
+    {
+        const size_t fragments = (size_t)(h->split_count > 0 ? h->split_count : 1) * h->fragment_slots;
+        UP(wall_split_slot, W);
+        if (h->split_count > 0) { UP(split_fragments_fixed, fragments * 4); UP(split_fragment_mask, fragments); }
+        else { d.split_fragments_fixed = nullptr; d.split_fragment_mask = nullptr; }
+    }
     const size_t cells = (size_t)h->grid_nx * h->grid_ny;
     const size_t items = h->grid_cell_ofs[cells];
     UP(grid_cell_ofs, cells + 1); UP(grid_item_sector, items); UP(grid_item_edge_ofs, items + 1);
@@ -2812,6 +2885,7 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     Scratch &sc = r->sc;
     if (rc == GD_OK) rc = scratch_alloc(r, L, &sc.ctx);
     if (rc == GD_OK) rc = scratch_alloc(r, L * W, &sc.rec);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)(h->split_count > 0 ? h->split_count * h->fragment_slots : 1), &sc.frag_rec);
     if (rc == GD_OK) rc = scratch_alloc(r, L * CAND_MAX * SW, &sc.cand);
     if (rc == GD_OK) rc = scratch_alloc(r, L * SW, &sc.cand_count);
     if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.flat_sector);

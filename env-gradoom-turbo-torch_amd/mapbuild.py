@@ -24,6 +24,44 @@ def _csr(rows: list[list[int]]) -> tuple[np.ndarray, np.ndarray]:
     return offsets, np.asarray(flat if flat else [0], dtype=np.int32)
 
 
+def build_split_tables(smap, walls_fixed: np.ndarray) -> dict[str, np.ndarray | int]:
+    """Projection fragments of the linedefs a BSP builder split (scenario.py:420-454).
+
+    A linedef whose only fragment is the linedef itself needs no row: the renderer then projects with
+    the linedef's own FWallCoords, which is what the reference computes for it (engine.py:12310-12380).
+    """
+
+    fragments = getattr(smap, "wall_projection_fragments_fixed", None)
+    mask = getattr(smap, "wall_projection_fragment_mask", None)
+    wall_count = len(walls_fixed)
+    if (fragments is None) != (mask is None):
+        raise ValueError("wall projection fragments and their mask must be provided together")
+    if fragments is None:
+        fragments = walls_fixed.astype(np.int64)[:, None, :]
+        mask = np.ones((wall_count, 1), dtype=bool)
+    fragments = np.asarray(fragments, dtype=np.int64)
+    mask = np.asarray(mask, dtype=bool)
+    if fragments.shape[:2] != mask.shape or fragments.shape[2:] != (4,) or len(fragments) != wall_count:
+        raise ValueError("invalid wall projection fragment arrays")
+    if np.abs(fragments).max(initial=0) >= 2**31:
+        raise ValueError("projection fragment coordinates do not fit 16.16 in int32")
+    slots = max(1, mask.shape[1])
+    plain = mask[:, 0] & ~mask[:, 1:].any(axis=1) & np.all(fragments[:, 0] == walls_fixed, axis=1)
+    rows = np.flatnonzero(~plain)
+    wall_split_slot = np.full(wall_count, -1, dtype=np.int32)
+    wall_split_slot[rows] = np.arange(len(rows), dtype=np.int32)
+    if len(rows):
+        split_fragments = np.ascontiguousarray(fragments[rows], dtype=np.int32)
+        split_mask = np.ascontiguousarray(mask[rows], dtype=np.uint8)
+    else:
+        split_fragments = np.zeros((1, slots, 4), dtype=np.int32)
+        split_mask = np.zeros((1, slots), dtype=np.uint8)
+    return dict(
+        fragment_slots=int(slots), split_count=int(len(rows)), wall_split_slot=wall_split_slot,
+        split_fragments_fixed=split_fragments, split_fragment_mask=split_mask,
+    )
+
+
 def build_map_tables(smap) -> dict[str, np.ndarray | int]:
     """Return contiguous arrays keyed by the field names of ``gd_map_desc``."""
 
@@ -165,7 +203,10 @@ def build_map_tables(smap) -> dict[str, np.ndarray | int]:
     grid.update(build_fine_grid(walls, sector_edge_ofs, sector_edge_idx, sector_count, grid["grid_min_x"], grid["grid_min_y"],
                                 fine_cell, heights, floor_levels, ceil_levels))
 
+    split = build_split_tables(smap, walls_fixed)
+
     return dict(
+        **split,
         floor_level_count=int(len(floor_levels)),
         ceil_level_count=int(len(ceil_levels)),
         floor_levels=floor_levels,

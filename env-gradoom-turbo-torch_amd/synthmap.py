@@ -67,6 +67,8 @@ class SynthMap:
     grid_points: np.ndarray  # [gy+1,gx+1,2] f32 jittered grid vertices
     sector_quads: np.ndarray | None = None  # [S,4,2] f64 corners p00,p10,p01,p11 used to place cameras/sprites
     void_boxes: np.ndarray | None = None  # [B,4] f64 x0,y0,x1,y1 of void pillars inside sectors (no camera goes there)
+    wall_projection_fragments_fixed: np.ndarray | None = None  # [W,F,4] i64 16.16 BSP fragments (scenario.py:400)
+    wall_projection_fragment_mask: np.ndarray | None = None  # [W,F] bool
 
     @property
     def blocking_segments(self) -> np.ndarray:
@@ -235,6 +237,30 @@ def _add_islands(rng, edges, sector_cells, sector_quads, count):
             else:
                 edges.append((q, p, island, int(host), MAX_SPLIT_DEPTH))
     return edges, cells, np.asarray(quads, dtype=np.float64)
+
+
+def split_linedefs(smap: SynthMap, seed: int, share: float = 0.2, slots: int = 3) -> SynthMap:
+    """Give a share of the linedefs two or three BSP projection fragments (scenario.py:420-454).
+
+    A node builder splits a linedef at points rounded to 16.16, a hair off the line; the copy
+    returned carries such fragments, the linedefs themselves stay as they are.
+    """
+
+    rng = np.random.default_rng(seed)
+    walls_fixed = np.rint(smap.wall_segments.astype(np.float64) * 65536.0).astype(np.int64)
+    wall_count = len(walls_fixed)
+    fragments = np.zeros((wall_count, slots, 4), dtype=np.int64)
+    mask = np.zeros((wall_count, slots), dtype=bool)
+    for w in range(wall_count):
+        start, end = walls_fixed[w, :2], walls_fixed[w, 2:]
+        pieces = int(rng.integers(2, slots + 1)) if rng.random() < share else 1
+        cuts = np.sort(rng.uniform(0.1, 0.9, pieces - 1))
+        points = [start] + [np.rint(start + (end - start) * t).astype(np.int64) for t in cuts] + [end]
+        for k in range(pieces):
+            fragments[w, k, :2] = points[k]
+            fragments[w, k, 2:] = points[k + 1]
+            mask[w, k] = True
+    return dataclasses.replace(smap, wall_projection_fragments_fixed=fragments, wall_projection_fragment_mask=mask)
 
 
 def _add_pinched_pillars(rng, edges, sector_quads, hosts):

@@ -60,6 +60,8 @@ typedef struct gd_map_desc {
     int32_t floor_level_count, ceil_level_count; /* distinct plane heights */
     int32_t grid_nx, grid_ny;/* point-location grid (cells of grid_cell map units) */
     int32_t fine_nx, fine_ny;/* fine point-location raster (cells of fine_cell map units, same origin) */
+    int32_t fragment_slots;  /* F >= 1 projection fragments per split linedef (engine.py:620-621) */
+    int32_t split_count;     /* SP linedefs whose projection fragments differ from the linedef itself */
     float grid_min_x, grid_min_y, grid_cell, fine_cell;
 
     const float *walls;              /* [W,4] x1,y1,x2,y2 (portal_walls) */
@@ -85,6 +87,12 @@ typedef struct gd_map_desc {
     const int32_t *sector_edge_ofs;  /* [S+1] CSR rows of sector_edge_mask (scenario.py:906-916) */
     const int32_t *sector_edge_idx;
     const int32_t *blocking_walls;   /* [B] linedef index of each blocking segment, ascending */
+    /* BSP fragments of split linedefs (scenario.py:420-454, portal_projection_fragments_fixed / _mask):
+       OWallMost projects with the fragment that owns the column (engine.py:12310-12380) and wallscan
+       light interpolates over it when the linedef has more than one (engine.py:11495-11545). */
+    const int32_t *wall_split_slot;      /* [W] row of the linedef in the two tables below, -1 = not split */
+    const int32_t *split_fragments_fixed;/* [SP,F,4] 16.16 x1,y1,x2,y2 */
+    const uint8_t *split_fragment_mask;  /* [SP,F] 1 = fragment present */
     /* Point-location grid: the even-odd polygon tests of engine.py:9598-9617 and
        10994-11015 restricted, per cell, to the sectors and edges that can count there. */
     const int32_t *grid_cell_ofs;    /* [nx*ny+1] -> items */

@@ -139,6 +139,9 @@ struct Oracle {
     std::vector<WallGeom> geom;
     std::vector<WallVis> vis;      // [W][2]
     std::vector<i64> tx, ty;       // [W][2] view coordinates (engine.py:11173-11205)
+    // BSP projection fragments of split linedefs (engine.py:11472-11545): FWallCoords and wallscan light
+    std::vector<WallGeom> frag_geom;  // [SP][F]
+    std::vector<WallVis> frag_vis;    // [SP][F][2]
     std::vector<uint8_t> front_facing_f32;  // engine.py:11376-11381
     std::vector<float> dist, along;        // [320][W]
     std::vector<uint8_t> geo, proj, ledge; // [320][W]
@@ -176,6 +179,8 @@ struct Oracle {
             has_start[w] = sc > 0; has_end[w] = ec > 0;
         }
         geom.resize(W); vis.resize(2 * W); tx.resize(2 * W); ty.resize(2 * W);
+        frag_geom.resize(size_t(m->split_count) * m->fragment_slots);
+        frag_vis.resize(2 * size_t(m->split_count) * m->fragment_slots);
         front_facing_f32.resize(W); subpixel_two_sided.resize(W);
         dist.resize(size_t(SW) * W); along.resize(size_t(SW) * W);
         geo.resize(size_t(SW) * W); proj.resize(size_t(SW) * W); ledge.resize(size_t(SW) * W);
@@ -303,13 +308,40 @@ struct Oracle {
     }
 
     // engine.py:10747-10869 for one linedef (whole-linedef fragment)
-    void wall_geometry(int w) {
-        const int32_t *wf = m->walls_fixed + 4 * w;
+    void wall_geometry(int w) { geom[w] = wall_coords(m->walls_fixed + 4 * w, &tx[2 * w], &ty[2 * w]); }
+
+    // engine.py:11472-11500: the same for every fragment of the split linedefs
+    void fragment_geometry() {
+        const int F = m->fragment_slots;
+        for (int k = 0; k < m->split_count * F; ++k) {
+            i64 ftx[2], fty[2];
+            frag_geom[k] = wall_coords(m->split_fragments_fixed + 4 * size_t(k), ftx, fty);
+            frag_vis[2 * k] = wall_visibility_side(ftx[0], ftx[1], fty[0], fty[1]);
+            frag_vis[2 * k + 1] = wall_visibility_side(ftx[1], ftx[0], fty[1], fty[0]);
+        }
+    }
+
+    // engine.py:11511-11529 / 12324-12333: the first present fragment whose half-open span holds the
+    // column; -1 if none.  *fragments receives how many fragments the linedef has.
+    int owning_fragment(int w, int x, int *fragments) const {
+        const int F = m->fragment_slots, row = m->wall_split_slot[w];
+        int owner = -1, count = 0;
+        for (int k = 0; k < F; ++k) {
+            if (!m->split_fragment_mask[row * F + k]) continue;
+            ++count;
+            const WallGeom &g = frag_geom[size_t(row) * F + k];
+            if (owner < 0 && (g.sr > g.sl) && (x >= g.sl) && (x < g.sr)) owner = row * F + k;
+        }
+        *fragments = count;
+        return owner;
+    }
+
+    WallGeom wall_coords(const int32_t *wf, i64 *tx_out, i64 *ty_out) const {
         i64 rx0 = wf[0] - L.view_x_fixed, ry0 = wf[1] - L.view_y_fixed;
         i64 rx1 = wf[2] - L.view_x_fixed, ry1 = wf[3] - L.view_y_fixed;
         i64 tx0 = (rx0 * L.vsin - ry0 * L.vcos) >> 20, ty0 = (rx0 * L.vcos + ry0 * L.vsin) >> 20;
         i64 tx1v = (rx1 * L.vsin - ry1 * L.vcos) >> 20, ty1v = (rx1 * L.vcos + ry1 * L.vsin) >> 20;
-        tx[2 * w] = tx0; tx[2 * w + 1] = tx1v; ty[2 * w] = ty0; ty[2 * w + 1] = ty1v;
+        tx_out[0] = tx0; tx_out[1] = tx1v; ty_out[0] = ty0; ty_out[1] = ty1v;
         i64 vx = i64(wf[2]) - wf[0], vy = i64(wf[3]) - wf[1];
         i64 fx = L.view_x_fixed - wf[0], fy = L.view_y_fixed - wf[1];
         bool front = (vx * fy - vy * fx) < 0;
@@ -334,7 +366,7 @@ struct Oracle {
         bool invalid_right = (right_inside ? ((tx2 < -ty2) || (ty2 == 0)) : ((tx1 > ty1) || (right_den == 0))) || (dr < 32);
         bool invalid = invalid_left || invalid_right || (sr <= sl);
         if (invalid) sr = sl;
-        geom[w] = WallGeom{sl, sr, dl, dr};
+        return WallGeom{sl, sr, dl, dr};
     }
 
     // engine.py:11217-11291 for one endpoint order
@@ -356,7 +388,12 @@ struct Oracle {
         return WallVis{light_left, light_step, wsl};
     }
     i64 visibility_at(int w, int side, int x) const {
-        const WallVis &v = vis[2 * w + side];
+        const WallVis *chosen = &vis[2 * w + side];
+        if (m->wall_split_slot[w] >= 0) {   // engine.py:11530-11545: only linedefs with several fragments
+            int fragments, owner = owning_fragment(w, x, &fragments);
+            if (owner >= 0 && fragments > 1) chosen = &frag_vis[2 * size_t(owner) + side];
+        }
+        const WallVis &v = *chosen;
         return v.light_left + (i64(x) - v.screen_left) * v.light_step;
     }
 
@@ -676,8 +713,18 @@ struct Oracle {
         i64 whole_sl = g.sl, whole_sr = g.sr;
         i64 whole_dl = std::max<i64>(g.dl, 1), whole_dr = std::max<i64>(g.dr, 1);
         bool has_fragment = (g.sr > g.sl) && (x >= g.sl) && (x < g.sr);
-        // argmax over an all-false single-fragment axis still selects fragment 0
+        // argmax over an all-false fragment axis still selects fragment 0, but every use of the
+        // selection is then overridden by the whole-linedef projection (engine.py:12598-12604)
         i64 screen_left = g.sl, screen_right = g.sr, depth_left = whole_dl, depth_right = whole_dr;
+        if (m->wall_split_slot[w] >= 0) {
+            int fragments, owner = owning_fragment(w, x, &fragments);
+            has_fragment = owner >= 0;
+            if (has_fragment) {
+                const WallGeom &f = frag_geom[owner];
+                screen_left = f.sl; screen_right = f.sr;
+                depth_left = std::max<i64>(f.dl, 1); depth_right = std::max<i64>(f.dr, 1);
+            }
+        }
         i64 relative_z_fixed = round_to_i64((world_z - L.view_z) * float(FIXED_UNIT));
         i64 pz = -(relative_z_fixed >> 4);
         i64 center_fixed = L.center_fixed;
@@ -1651,6 +1698,7 @@ int gdo_render(const gd_map_desc *map, const gd_lanes_desc *lanes, const gd_fram
             o.vis[2 * w] = o.wall_visibility_side(o.tx[2 * w], o.tx[2 * w + 1], o.ty[2 * w], o.ty[2 * w + 1]);
             o.vis[2 * w + 1] = o.wall_visibility_side(o.tx[2 * w + 1], o.tx[2 * w], o.ty[2 * w + 1], o.ty[2 * w]);
         }
+        o.fragment_geometry();
         o.portal_intersections();
         o.texture_mapping();
         double t1 = now();
@@ -1675,7 +1723,10 @@ int gdo_render(const gd_map_desc *map, const gd_lanes_desc *lanes, const gd_fram
             if (dbg->horizontal_offset) std::memcpy(dbg->horizontal_offset, o.hoff.data(), SW * W * 8);
             if (dbg->vertical_step) std::memcpy(dbg->vertical_step, o.vstep.data(), SW * W * 8);
             if (dbg->visibility) for (int x = 0; x < SW; ++x) for (size_t w = 0; w < W; ++w) for (int s = 0; s < 2; ++s)
-                dbg->visibility[(size_t(x) * W + w) * 2 + s] = o.visibility_at(int(w), s, x);
+                {   // the tap is _native_portal_intersections' own tensor, before fragments replace split linedefs
+                    const WallVis &v = o.vis[2 * w + s];
+                    dbg->visibility[(size_t(x) * W + w) * 2 + s] = v.light_left + (i64(x) - v.screen_left) * v.light_step;
+                }
         }
         double t3 = now();
         o.render_portal_walls();

@@ -36,7 +36,7 @@ def load_fixture(name: str):
     from gradoom_amd import mapbuild, synthmap
 
     sys.path.insert(0, os.path.join(ROOT, "tests", "golden"))
-    from make_golden_meta import map_digest
+    from make_golden_meta import fragment_digest, map_digest
 
     data = dict(np.load(os.path.join(FIXTURE_DIR, f"{name}.npz")))
     meta = ast.literal_eval(str(data.pop("meta")))
@@ -46,6 +46,9 @@ def load_fixture(name: str):
         pillars=meta.get("pillars", 0),
     )
     assert map_digest(smap) == meta["map_sha256"], "synthetic map generator drifted from the golden fixtures"
+    if meta.get("split_seed"):
+        smap = synthmap.split_linedefs(smap, meta["split_seed"])
+        assert fragment_digest(smap) == meta["fragment_sha256"], "linedef splitter drifted from the golden fixtures"
     tables = mapbuild.build_map_tables(smap)
     return meta, data, smap, tables
 

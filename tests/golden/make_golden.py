@@ -40,7 +40,7 @@ entry.load_package()
 from gradoom_amd import hostmath, overlay_inputs, synthmap  # noqa: E402
 
 import refdrive  # noqa: E402
-from make_golden_meta import map_digest  # noqa: E402
+from make_golden_meta import fragment_digest, map_digest  # noqa: E402
 
 FIXTURES = os.path.join(HERE, "fixtures")
 
@@ -94,6 +94,16 @@ CASES = {
         map_seed=41, grid=(4, 3), sectors=10, linedefs=120, lanes=8, pose_seed=1, islands=2, pillars=4, midtex=0.1,
         pitch=True, flash=True, stages=True,
     ),
+    # A fifth of the linedefs carry two or three BSP projection fragments (scenario.py:420-454): OWallMost and
+    # the wallscan light then work from the fragment that owns the column.
+    "split_linedefs": dict(
+        map_seed=22, grid=(6, 5), sectors=26, linedefs=160, lanes=8, pose_seed=2, sprites=32, pitch=True, flash=True,
+        midtex=0.2, split_seed=5, stages=True,
+    ),
+    "split_linedefs_grazing": dict(
+        map_seed=3001, grid=(6, 5), sectors=26, linedefs=260, lanes=6, layout="brick", islands=10, midtex=0.1,
+        pose_seed=7, margin=0.02, split_seed=9,
+    ),
     "config2_subset": dict(map_seed=1002, grid=(12, 9), sectors=96, linedefs=800, lanes=4, pose_seed=1, sprites=32),
     "config3_subset": dict(
         map_seed=1003, grid=(15, 15), sectors=200, linedefs=2000, lanes=2, pose_seed=1, sprites=64, flash=True
@@ -109,6 +119,8 @@ def build_case(name: str, cfg: dict, do_time: bool) -> dict:
         cfg["map_seed"], grid=cfg["grid"], sectors=cfg["sectors"], linedefs=cfg["linedefs"], midtex=cfg.get("midtex", 0.0),
         layout=cfg.get("layout", "grid"), islands=cfg.get("islands", 0), pillars=cfg.get("pillars", 0),
     )
+    if cfg.get("split_seed"):
+        smap = synthmap.split_linedefs(smap, cfg["split_seed"])
     lanes = cfg["lanes"]
     started = time.time()
     overlays = synthmap.generate_overlays(cfg["overlays"]) if cfg.get("overlays") else None
@@ -232,6 +244,8 @@ def build_case(name: str, cfg: dict, do_time: bool) -> dict:
         timing = float(np.median(samples))
     meta = dict(cfg)
     meta["map_sha256"] = map_digest(smap)
+    if cfg.get("split_seed"):
+        meta["fragment_sha256"] = fragment_digest(smap)
     data["meta"] = np.asarray(repr(meta))
     print(
         f"{name}: W={cfg['linedefs']} S={cfg['sectors']} lanes={lanes} ctor {ctor_seconds:.1f}s render {render_seconds:.1f}s"

@@ -18,3 +18,10 @@ def map_digest(smap) -> str:
     for name in DIGEST_FIELDS:
         digest.update(np.ascontiguousarray(getattr(smap, name)).tobytes())
     return digest.hexdigest()
+
+
+def fragment_digest(smap) -> str:
+    digest = hashlib.sha256()
+    digest.update(np.ascontiguousarray(smap.wall_projection_fragments_fixed, dtype=np.int64).tobytes())
+    digest.update(np.ascontiguousarray(smap.wall_projection_fragment_mask, dtype=np.uint8).tobytes())
+    return digest.hexdigest()

@@ -102,6 +102,8 @@ def to_compiled_scenario(smap, *, flash_lights: bool = False, overlays: dict | N
         colormap=smap.colormap,
         enemy_walk_sprite_ids=enemy_walk,
         raw_static_sprite_ids=raw_static,
+        wall_projection_fragments_fixed=smap.wall_projection_fragments_fixed,
+        wall_projection_fragment_mask=smap.wall_projection_fragment_mask,
         **kwargs,
     )
 

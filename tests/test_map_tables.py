@@ -137,3 +137,48 @@ def test_fine_raster_agrees_with_the_crossing_test(fixture):
             assert (entry[i] >> floor_index[float(heights[s, 0])]) & 1
             assert (entry[i] >> (15 + ceil_index[float(heights[s, 1])])) & 1
     assert tables["grid_cell"] == 8 * tables["fine_cell"]
+
+
+def test_split_tables_hold_only_linedefs_whose_fragments_differ_from_the_linedef():
+    """scenario.py:420-454: every linedef has a fragment row; only split ones need a row on the device."""
+
+    import dataclasses
+
+    import pytest
+
+    from gradoom_amd import mapbuild, synthmap
+
+    smap = synthmap.generate_map(7, grid=(4, 3), sectors=10, linedefs=48)
+    plain = mapbuild.build_map_tables(smap)
+    assert plain["split_count"] == 0 and plain["fragment_slots"] == 1
+    assert np.all(plain["wall_split_slot"] == -1)
+
+    split = synthmap.split_linedefs(smap, 5, share=0.3)
+    tables = mapbuild.build_map_tables(split)
+    mask = split.wall_projection_fragment_mask
+    expected_rows = np.flatnonzero(mask.sum(axis=1) > 1)
+    assert tables["split_count"] == len(expected_rows) > 0
+    assert tables["fragment_slots"] == mask.shape[1]
+    assert np.array_equal(np.flatnonzero(tables["wall_split_slot"] >= 0), expected_rows)
+    for row, w in enumerate(expected_rows):
+        assert tables["wall_split_slot"][w] == row
+        assert np.array_equal(tables["split_fragments_fixed"][row], split.wall_projection_fragments_fixed[w])
+        assert np.array_equal(tables["split_fragment_mask"][row].astype(bool), mask[w])
+        pieces = split.wall_projection_fragments_fixed[w][mask[w]]
+        # consecutive fragments chain from the linedef's start to its end
+        assert np.array_equal(pieces[0, :2], tables["walls_fixed"][w, :2])
+        assert np.array_equal(pieces[-1, 2:], tables["walls_fixed"][w, 2:])
+        assert np.array_equal(pieces[1:, :2], pieces[:-1, 2:])
+
+    # a single fragment that is not the linedef itself still needs its row; so does a linedef with none
+    moved = dataclasses.replace(
+        smap,
+        wall_projection_fragments_fixed=tables["walls_fixed"].astype(np.int64)[:, None, :] + np.asarray([0, 0, 0, 1])[None, None, :] * (np.arange(len(tables["walls_fixed"])) == 3)[:, None, None],
+        wall_projection_fragment_mask=(np.arange(len(tables["walls_fixed"])) != 5)[:, None],
+    )
+    rows = mapbuild.build_map_tables(moved)
+    assert rows["split_count"] == 2
+    assert list(np.flatnonzero(rows["wall_split_slot"] >= 0)) == [3, 5]
+
+    with pytest.raises(ValueError):
+        mapbuild.build_map_tables(dataclasses.replace(smap, wall_projection_fragments_fixed=np.zeros((48, 1, 4), np.int64)))
