@@ -96,6 +96,8 @@ MAP_ARRAYS = (
     ("spr_h", np.int32),
     ("spr_left", np.int32),
     ("spr_top", np.int32),
+    ("additive_luts", np.uint8),
+    ("translucent_lut", np.uint8),
 )
 
 LANE_ARRAYS = (
@@ -119,6 +121,7 @@ LANE_ARRAYS = (
     ("sprite_fullbright", np.uint8),
     ("weapon_state", np.int64),
     ("hud_state", np.int32),
+    ("sprite_style", np.int8),
 )
 
 OUT_FIELDS = ("indexed", "obs", "frames", "reset_mask", "rgb", "final_frames")

@@ -2218,7 +2218,7 @@ __global__ void __launch_bounds__(256) plane_shade_kernel(DeviceMap dm, int lane
 struct SpriteRec {
     float x, y, depth, light;
     i64 depth_fixed, left, right, hstep, yscale, top_fixed, texmid, iscale;
-    int id, flags;   // bit0 alive, bit1 fullbright
+    int id, flags;   // bit0 alive, bit1 fullbright, bits 8..15 style (signed: -1 opaque, -2 translucent, >= 0 additive)
 };
 
 __global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc,
@@ -2240,6 +2240,7 @@ __global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lan
         const bool known_patch = s.id >= 0 && s.id < m->sprite_count;   // an unknown patch id is never drawn
         if (!known_patch) s.id = 0;
         s.flags = ((lanes.sprite_alive[k] && known_patch) ? 1 : 0) | ((lanes.sprite_fullbright && lanes.sprite_fullbright[k]) ? 2 : 0);
+        s.flags |= ((lanes.sprite_style ? (int)lanes.sprite_style[k] : -1) & 0xFF) << 8;
         i64 ax = round_to_i64(s.x * 65536.0f), ay = round_to_i64(s.y * 65536.0f);
         i64 rx = ax - L.view_x_fixed, ry = ay - L.view_y_fixed;
         s.depth_fixed = (rx * L.vcos + ry * L.vsin) >> 20;
@@ -2316,6 +2317,7 @@ __global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lan
         int width = m->spr_w[s.id], height = m->spr_h[s.id];
         i64 su = mul64((i64)x - s.left, s.hstep) >> 16;
         if (!(su >= 0 && su < width)) continue;
+        const int style = (int)(signed char)(s.flags >> 8);
         float light = s.light + (float)(L.flash_light * 16);
         if (s.flags & 2) light = 255.0f;
         float base_shade = 61.0f - light / 4.0f;
@@ -2367,7 +2369,12 @@ __global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lan
                 const int y = yb + j;
                 i64 post_screen_top = (s.top_fixed + mul64(s.yscale, post_top[j])) >> 16;
                 if ((i64)y < post_screen_top) continue;
-                frame[(size_t)y * SW + x] = m->colormap[shade * 256 + texel[j]];
+                // engine.py:14914-14939: opaque, additive table or translucent table over the pixel below
+                unsigned char lit = m->colormap[shade * 256 + texel[j]];
+                unsigned char *pixel = frame + (size_t)y * SW + x;
+                if (style == -2) lit = m->translucent_lut[(size_t)*pixel * 256 + lit];
+                else if (style >= 0) lit = m->additive_luts[((size_t)(style > 1 ? 1 : style) * 256 + *pixel) * 256 + lit];
+                *pixel = lit;
             }
         }
     }
@@ -2773,6 +2780,7 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     for (int w = 0; w < h->wall_count; ++w)
         if (h->wall_split_slot[w] < -1 || h->wall_split_slot[w] >= h->split_count)
             return fail(GD_E_ARG, "wall_split_slot names a row outside the fragment tables");
+    if (!h->additive_luts || !h->translucent_lut) return fail(GD_E_ARG, "missing sprite blend tables");
     gd_renderer *r = new (std::nothrow) gd_renderer();
     if (!r) return fail(GD_E_ARG, "out of host memory");
     r->events_ready = false;
@@ -2813,6 +2821,7 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     const size_t sprels = (size_t)h->sprite_count * h->spr_max_h * h->spr_max_w;
     UP(spr_atlas, sprels); UP(spr_opaque, sprels); UP(spr_post_top, sprels);
     UP(spr_w, h->sprite_count); UP(spr_h, h->sprite_count); UP(spr_left, h->sprite_count); UP(spr_top, h->sprite_count);
+    UP(additive_luts, 2 * 256 * 256); UP(translucent_lut, 256 * 256);
 #undef UP
     std::vector<i64> sine, tangent;
     build_fine_tables(sine, tangent);

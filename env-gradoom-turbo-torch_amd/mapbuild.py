@@ -24,6 +24,23 @@ def _csr(rows: list[list[int]]) -> tuple[np.ndarray, np.ndarray]:
     return offsets, np.asarray(flat if flat else [0], dtype=np.int32)
 
 
+def build_blend_tables(smap) -> dict[str, np.ndarray]:
+    """Blend tables of styled sprites, with the reference's defaults when the map has none (engine.py:1017-1032):
+    the additive default shows the lit texel, the translucent default the pixel under the sprite."""
+
+    additive = getattr(smap, "projectile_additive_luts", None)
+    translucent = getattr(smap, "sprite_translucent_lut", None)
+    if additive is None:
+        additive = np.broadcast_to(np.arange(256, dtype=np.uint8)[None, None, :], (2, 256, 256))
+    if translucent is None:
+        translucent = np.broadcast_to(np.arange(256, dtype=np.uint8)[:, None], (256, 256))
+    additive = np.ascontiguousarray(additive, dtype=np.uint8)
+    translucent = np.ascontiguousarray(translucent, dtype=np.uint8)
+    if additive.shape != (2, 256, 256) or translucent.shape != (256, 256):
+        raise ValueError("projectile_additive_luts must be [2,256,256] and sprite_translucent_lut [256,256]")
+    return dict(additive_luts=additive, translucent_lut=translucent)
+
+
 def build_split_tables(smap, walls_fixed: np.ndarray) -> dict[str, np.ndarray | int]:
     """Projection fragments of the linedefs a BSP builder split (scenario.py:420-454).
 
@@ -262,6 +279,7 @@ def build_map_tables(smap) -> dict[str, np.ndarray | int]:
         spr_h=np.ascontiguousarray(smap.sprite_heights, dtype=np.int32),
         spr_left=np.ascontiguousarray(smap.sprite_left_offsets, dtype=np.int32),
         spr_top=np.ascontiguousarray(smap.sprite_top_offsets, dtype=np.int32),
+        **build_blend_tables(smap),
     )
 
 

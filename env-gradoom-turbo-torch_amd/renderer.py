@@ -48,6 +48,7 @@ class LaneState:
     # Overlay layers (see overlay_inputs.py); drawn when the renderer holds overlay patches.
     weapon_state: torch.Tensor | None = None  # i64 [N,5]
     hud_state: torch.Tensor | None = None  # i32 [N,9]
+    sprite_style: torch.Tensor | None = None  # i8 [N,A]: -1 opaque, -2 translucent, >= 0 additive table
 
     @classmethod
     def from_numpy(cls, arrays: dict, device) -> "LaneState":
@@ -67,6 +68,7 @@ class LaneState:
             sprite_fullbright=get("sprite_fullbright", torch.uint8), ray_cos=get("ray_cos", torch.float32),
             ray_sin=get("ray_sin", torch.float32), sprite_depth=get("sprite_depth", torch.float32),
             weapon_state=get("weapon_state", torch.int64), hud_state=get("hud_state", torch.int32),
+            sprite_style=get("sprite_style", torch.int8),
         )
 
 
@@ -184,6 +186,8 @@ class HipRenderer:
                     bright = bright.to(torch.uint8)
                 keep.append(bright)
                 desc.sprite_fullbright = _require(bright, "sprite_fullbright", torch.uint8, (count, slots), device).data_ptr()
+            if lanes.sprite_style is not None:
+                desc.sprite_style = _require(lanes.sprite_style, "sprite_style", torch.int8, (count, slots), device).data_ptr()
             depth = lanes.sprite_depth
             if depth is None:
                 depth = hostmath.sprite_depth(lanes.x, lanes.y, lanes.angle, lanes.sprite_x, lanes.sprite_y)

@@ -69,6 +69,8 @@ class SynthMap:
     void_boxes: np.ndarray | None = None  # [B,4] f64 x0,y0,x1,y1 of void pillars inside sectors (no camera goes there)
     wall_projection_fragments_fixed: np.ndarray | None = None  # [W,F,4] i64 16.16 BSP fragments (scenario.py:400)
     wall_projection_fragment_mask: np.ndarray | None = None  # [W,F] bool
+    projectile_additive_luts: np.ndarray | None = None  # [2,256,256] u8 (scenario.py:367)
+    sprite_translucent_lut: np.ndarray | None = None  # [256,256] u8 (scenario.py:368)
 
     @property
     def blocking_segments(self) -> np.ndarray:
@@ -102,6 +104,7 @@ class Sprites:
     sprite: np.ndarray  # [N,A] i32 patch id
     alive: np.ndarray  # [N,A] bool
     fullbright: np.ndarray  # [N,A] bool
+    style: np.ndarray | None = None  # [N,A] i8: -1 opaque, -2 translucent, >= 0 additive table (engine.py:14343)
 
 
 def _split_edges(rng, edges, target):
@@ -237,6 +240,17 @@ def _add_islands(rng, edges, sector_cells, sector_quads, count):
             else:
                 edges.append((q, p, island, int(host), MAX_SPLIT_DEPTH))
     return edges, cells, np.asarray(quads, dtype=np.float64)
+
+
+def with_blend_tables(smap: SynthMap, seed: int) -> SynthMap:
+    """A copy of the map with seeded random additive / translucent blend tables (scenario.py:367-368)."""
+
+    rng = np.random.default_rng(seed)
+    return dataclasses.replace(
+        smap,
+        projectile_additive_luts=rng.integers(0, 256, (2, 256, 256), dtype=np.uint8),
+        sprite_translucent_lut=rng.integers(0, 256, (256, 256), dtype=np.uint8),
+    )
 
 
 def split_linedefs(smap: SynthMap, seed: int, share: float = 0.2, slots: int = 3) -> SynthMap:

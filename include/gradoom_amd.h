@@ -124,6 +124,9 @@ typedef struct gd_map_desc {
     const uint8_t *spr_opaque;       /* [P,spr_max_h,spr_max_w] 0/1 */
     const uint8_t *spr_post_top;     /* [P,spr_max_h,spr_max_w] first row of the opaque run (engine.py:14230) */
     const int32_t *spr_w, *spr_h, *spr_left, *spr_top; /* [P] */
+    /* Blend tables of styled sprites (engine.py:14920-14939): [style][pixel under the sprite][lit texel]. */
+    const uint8_t *additive_luts;    /* [2,256,256] projectile_additive_luts */
+    const uint8_t *translucent_lut;  /* [256,256] sprite_translucent_lut */
 } gd_map_desc;
 
 /*
@@ -159,6 +162,8 @@ typedef struct gd_lanes_desc {
     const int32_t *hud_state;       /* [N,9] status bar of engine.py:15232-15267: ready ammo, health, armor,
                                        face patch id, owned weapon bits (bit k = weapon k+1, k < 5),
                                        four ammo counts */
+    const int8_t *sprite_style;     /* [N,A] or NULL (all -1): -1 opaque, -2 translucent_lut, s >= 0
+                                       additive_luts[min(s, 1)] (actor_additive_style, engine.py:14343-14682) */
 } gd_lanes_desc;
 
 /*

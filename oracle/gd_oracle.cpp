@@ -1425,7 +1425,7 @@ struct Oracle {
         std::vector<float> wall_distance(SW); std::vector<int> blocking_wall(SW);
         blocking_raycast(wall_distance.data(), blocking_wall.data());
         struct Spr {
-            float x, y, z, depth; int id; bool alive, fullbright;
+            float x, y, z, depth; int id; bool alive, fullbright; int style;
             i64 depth_fixed, left, right, hstep, yscale, top_fixed, texmid, iscale; float light;
         };
         std::vector<Spr> sp(A);
@@ -1435,6 +1435,7 @@ struct Oracle {
             s.x = lanes->sprite_x[k]; s.y = lanes->sprite_y[k]; s.z = lanes->sprite_z[k];
             s.depth = lanes->sprite_depth[k]; s.id = lanes->sprite_id[k];
             s.alive = lanes->sprite_alive[k]; s.fullbright = lanes->sprite_fullbright ? lanes->sprite_fullbright[k] : 0;
+            s.style = lanes->sprite_style ? lanes->sprite_style[k] : -1;
             // engine.py:14174-14198
             i64 ax = round_to_i64(s.x * float(FIXED_UNIT)), ay = round_to_i64(s.y * float(FIXED_UNIT));
             i64 rx = ax - L.view_x_fixed, ry = ay - L.view_y_fixed;
@@ -1510,7 +1511,11 @@ struct Oracle {
                     if (!m->spr_opaque[t]) continue;
                     i64 post_screen_top = (s.top_fixed + mul64(s.yscale, m->spr_post_top[t])) >> 16;
                     if (i64(y) < post_screen_top) continue;
-                    frame[i] = m->colormap[shade * 256 + m->spr_atlas[t]];
+                    // engine.py:14914-14939: opaque, additive table or translucent table over the pixel below
+                    uint8_t lit = m->colormap[shade * 256 + m->spr_atlas[t]];
+                    if (s.style == -2) lit = m->translucent_lut[size_t(frame[i]) * 256 + lit];
+                    else if (s.style >= 0) lit = m->additive_luts[(size_t(s.style > 1 ? 1 : s.style) * 256 + frame[i]) * 256 + lit];
+                    frame[i] = lit;
                 }
             }
         }

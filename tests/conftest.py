@@ -46,6 +46,8 @@ def load_fixture(name: str):
         pillars=meta.get("pillars", 0),
     )
     assert map_digest(smap) == meta["map_sha256"], "synthetic map generator drifted from the golden fixtures"
+    if meta.get("blend_seed"):
+        smap = synthmap.with_blend_tables(smap, meta["blend_seed"])
     if meta.get("split_seed"):
         smap = synthmap.split_linedefs(smap, meta["split_seed"])
         assert fragment_digest(smap) == meta["fragment_sha256"], "linedef splitter drifted from the golden fixtures"
@@ -56,7 +58,7 @@ def load_fixture(name: str):
 LANE_KEYS = (
     "x", "y", "angle", "view_z", "x_fixed", "y_fixed", "angle_bam", "pitch_bam", "flash_light", "ray_cos", "ray_sin",
     "sprite_x", "sprite_y", "sprite_z", "sprite_depth", "sprite_id", "sprite_alive", "sprite_fullbright",
-    "weapon_state", "hud_state",
+    "weapon_state", "hud_state", "sprite_style",
 )
 
 

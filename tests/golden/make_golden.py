@@ -104,6 +104,12 @@ CASES = {
         map_seed=3001, grid=(6, 5), sectors=26, linedefs=260, lanes=6, layout="brick", islands=10, midtex=0.1,
         pose_seed=7, margin=0.02, split_seed=9,
     ),
+    # Styled billboards among opaque ones: plasma balls (additive table 0), teleport fog (additive table 1) and
+    # bullet puffs (translucent table) blend over whatever lies under them through seeded random tables.
+    "styled_sprites": dict(
+        map_seed=22, grid=(6, 5), sectors=26, linedefs=160, lanes=8, pose_seed=3, sprites=48, effects=60, blend_seed=13,
+        pitch=True, flash=True, midtex=0.2,
+    ),
     "config2_subset": dict(map_seed=1002, grid=(12, 9), sectors=96, linedefs=800, lanes=4, pose_seed=1, sprites=32),
     "config3_subset": dict(
         map_seed=1003, grid=(15, 15), sectors=200, linedefs=2000, lanes=2, pose_seed=1, sprites=64, flash=True
@@ -121,6 +127,8 @@ def build_case(name: str, cfg: dict, do_time: bool) -> dict:
     )
     if cfg.get("split_seed"):
         smap = synthmap.split_linedefs(smap, cfg["split_seed"])
+    if cfg.get("blend_seed"):
+        smap = synthmap.with_blend_tables(smap, cfg["blend_seed"])
     lanes = cfg["lanes"]
     started = time.time()
     overlays = synthmap.generate_overlays(cfg["overlays"]) if cfg.get("overlays") else None
@@ -145,7 +153,8 @@ def build_case(name: str, cfg: dict, do_time: bool) -> dict:
     )
     if cfg.get("sprites", 0):
         sprites = synthmap.generate_sprites(smap, lanes, cfg["sprites"], cfg["pose_seed"])
-        packed = refdrive.set_sprites(engine, sprites, cfg["pose_seed"])
+        effects = synthmap.generate_sprites(smap, lanes, cfg["effects"], cfg["pose_seed"] + 50) if cfg.get("effects") else None
+        packed = refdrive.set_sprites(engine, sprites, cfg["pose_seed"], effects)
         data.update(packed)
         data["sprite_depth"] = hostmath.sprite_depth(
             engine.x, engine.y, engine.angle, torch.as_tensor(packed["sprite_x"]), torch.as_tensor(packed["sprite_y"])

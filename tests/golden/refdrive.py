@@ -50,6 +50,14 @@ def to_compiled_scenario(smap, *, flash_lights: bool = False, overlays: dict | N
         lights[:, :, 1] = 1
         lights[:, :, 2] = 2
         kwargs["native_weapon_flash_lights"] = lights
+    if smap.projectile_additive_luts is not None:
+        # styled sprites: blend tables and the patches of the effects that use them (scenario.py:361-369)
+        kwargs.update(
+            projectile_additive_luts=smap.projectile_additive_luts, sprite_translucent_lut=smap.sprite_translucent_lut,
+            raw_projectile_flight_sprite_ids=((np.arange(3 * 2 * 8, dtype=np.int32) * 7 + 1) % sprite_count).reshape(3, 2, 8),
+            raw_teleport_fog_sprite_ids=(np.arange(12, dtype=np.int32) * 3 + 2) % sprite_count,
+            raw_bullet_puff_sprite_ids=(np.arange(4, dtype=np.int32) * 11 + 5) % sprite_count,
+        )
     if overlays is not None:
         # raw psprite and status bar patches (scenario.py:382-397)
         kwargs.update(
@@ -133,7 +141,7 @@ def set_poses(engine, poses) -> None:
     )
 
 
-def set_sprites(engine, sprites, seed: int):
+def set_sprites(engine, sprites, seed: int, effects=None):
     """Place billboards through the enemy and drop slots (engine.py:14328-14343, 14657-14682).
 
     Slots [0, 64) of ``sprites`` go to enemy slots, [64, 128) to drop slots.  The
@@ -173,11 +181,46 @@ def set_sprites(engine, sprites, seed: int):
         engine.drop_z[:, sl] = torch.as_tensor(sprites.z[:, src])
         engine.drop_type[:, sl] = torch.where(torch.as_tensor(sprites.alive[:, src]), 2001, -1)
         engine.drop_spawned[:, sl] = True
+    if effects is not None:
+        set_effect_sprites(engine, effects, seed + 1)
     return packed_sprites(engine)
 
 
+def set_effect_sprites(engine, sprites, seed: int):
+    """Place styled billboards: plasma balls and rockets in flight (additive table 0 / opaque,
+    engine.py:14410-14460), teleport fog (additive table 1, engine.py:14577-14595) and bullet puffs
+    (translucent, engine.py:14597-14630).  A third of ``sprites`` goes to each kind."""
+
+    lanes, count = sprites.x.shape
+    third = count // 3
+    generator = torch.Generator().manual_seed(seed)
+    x, y, z = (torch.as_tensor(v) for v in (sprites.x, sprites.y, sprites.z))
+    alive = torch.as_tensor(sprites.alive)
+    flight = slice(0, min(third, engine.player_projectile_slots))
+    n = flight.stop
+    engine.projectile_x[:, :n], engine.projectile_y[:, :n], engine.projectile_z[:, :n] = x[:, flight], y[:, flight], z[:, flight]
+    engine.projectile_alive[:, :n] = alive[:, flight]
+    engine.projectile_type[:, :n] = torch.randint(0, 2, (lanes, n), generator=generator)
+    engine.projectile_age[:, :n] = torch.randint(0, 40, (lanes, n), generator=generator).to(engine.projectile_age.dtype)
+    engine.projectile_velocity_x[:, :n] = torch.rand((lanes, n), generator=generator) * 20 - 10
+    engine.projectile_velocity_y[:, :n] = torch.rand((lanes, n), generator=generator) * 20 - 10
+    fog = slice(third, third + min(third, engine.enemy_slots))
+    n = fog.stop - fog.start
+    engine.teleport_fog_x[:, :n], engine.teleport_fog_y[:, :n], engine.teleport_fog_z[:, :n] = x[:, fog], y[:, fog], z[:, fog]
+    tics = torch.randint(1, 73, (lanes, n), generator=generator)
+    engine.teleport_fog_tics[:, :n] = torch.where(alive[:, fog], tics, torch.zeros_like(tics)).to(engine.teleport_fog_tics.dtype)
+    puff = slice(2 * third, 2 * third + min(count - 2 * third, engine.hitscan_puff_slots))
+    n = puff.stop - puff.start
+    engine.hitscan_puff_x[:, :n], engine.hitscan_puff_y[:, :n], engine.hitscan_puff_z[:, :n] = x[:, puff], y[:, puff], z[:, puff]
+    tics = torch.randint(1, 17, (lanes, n), generator=generator)
+    engine.hitscan_puff_tics[:, :n] = torch.where(alive[:, puff], tics, torch.zeros_like(tics)).to(engine.hitscan_puff_tics.dtype)
+
+
 def packed_sprites(engine):
-    """Replay the reference's slot trimming and concatenation order for enemies and drops."""
+    """Replay the reference's slot trimming and concatenation order (engine.py:14328-14682) for the kinds
+    this driver places: enemies, player projectiles in flight, teleport fog, bullet puffs and drops."""
+
+    engine_module, _scenario = load_reference()
 
     enemy_sprite = engine._native_enemy_sprite_ids()
     enemy_slots = torch.nonzero(torch.any(engine.enemy_alive, dim=0)).flatten()
@@ -194,15 +237,51 @@ def packed_sprites(engine):
     drop_sprite = torch.where(engine.drop_type == 2007, static[6], drop_sprite)
     drop_sprite = torch.where(engine.drop_type == 2002, static[14], drop_sprite)
     drop_slots = torch.nonzero(torch.any(drop_visible, dim=0)).flatten()
+    opaque = lambda like: torch.full_like(like, -1, dtype=torch.int64)  # noqa: E731
+    kinds = [  # x, y, z, patch, alive, fullbright, style
+        (engine.enemy_x[:, enemy_slots], engine.enemy_y[:, enemy_slots], engine.enemy_z[:, enemy_slots],
+         enemy_sprite[:, enemy_slots], engine.enemy_alive[:, enemy_slots], fullbright, opaque(enemy_sprite[:, enemy_slots])),
+    ]
+    # player projectiles in flight (engine.py:14410-14460)
+    flight_type = engine.projectile_type.clamp(0, 1)
+    rotation = engine._doom_sprite_rotation(
+        torch.atan2(engine.y[:, None] - engine.projectile_y, engine.x[:, None] - engine.projectile_x),
+        torch.atan2(engine.projectile_velocity_y, engine.projectile_velocity_x),
+    )
+    flight_frame = torch.where(flight_type == 1, torch.remainder(engine.projectile_age // 6, 2).to(torch.int64), torch.zeros_like(flight_type))
+    flight_sprite = engine.map.raw_projectile_flight_sprite_ids[flight_type, flight_frame, rotation]
+    slots = torch.nonzero(torch.any(engine.projectile_alive, dim=0)).flatten()
+    if slots.numel():
+        alive = engine.projectile_alive[:, slots]
+        kinds.append((engine.projectile_x[:, slots], engine.projectile_y[:, slots], engine.projectile_z[:, slots],
+                      flight_sprite[:, slots], alive, alive,
+                      torch.where(flight_type[:, slots] == 1, torch.zeros_like(flight_type[:, slots]), opaque(flight_type[:, slots]))))
+    # teleport fog (engine.py:14577-14595)
+    slots = torch.nonzero(torch.any(engine.teleport_fog_tics > 0, dim=0)).flatten()
+    if slots.numel():
+        tics = engine.teleport_fog_tics[:, slots]
+        frame = torch.clamp((engine_module._TELEPORT_FOG_TOTAL_TICS - tics.to(torch.int64)) // 6, max=11)
+        patch = engine.map.raw_teleport_fog_sprite_ids[frame]
+        kinds.append((engine.teleport_fog_x[:, slots], engine.teleport_fog_y[:, slots], engine.teleport_fog_z[:, slots],
+                      patch, tics > 0, tics > 0, torch.ones_like(patch, dtype=torch.int64)))
+    # bullet puffs (engine.py:14597-14630)
+    slots = torch.nonzero(torch.any(engine.hitscan_puff_tics > 0, dim=0)).flatten()
+    if slots.numel():
+        tics = engine.hitscan_puff_tics[:, slots]
+        step = engine_module._BULLET_PUFF_FRAME_TICS
+        frame = torch.where(tics > 3 * step, 0, torch.where(tics > 2 * step, 1, torch.where(tics > step, 2, 3))).to(torch.int64)
+        patch = engine.map.raw_bullet_puff_sprite_ids[frame]
+        kinds.append((engine.hitscan_puff_x[:, slots], engine.hitscan_puff_y[:, slots], engine.hitscan_puff_z[:, slots],
+                      patch, tics > 0, frame == 0, torch.full_like(patch, -2, dtype=torch.int64)))
+    if drop_slots.numel():
+        kinds.append((engine.drop_x[:, drop_slots], engine.drop_y[:, drop_slots], engine.drop_z[:, drop_slots],
+                      drop_sprite[:, drop_slots], drop_visible[:, drop_slots], torch.zeros_like(drop_visible[:, drop_slots]),
+                      opaque(drop_sprite[:, drop_slots])))
+    columns = [torch.cat([kind[k] for kind in kinds], dim=1) for k in range(7)]
     return dict(
-        sprite_x=torch.cat((engine.enemy_x[:, enemy_slots], engine.drop_x[:, drop_slots]), dim=1).numpy(),
-        sprite_y=torch.cat((engine.enemy_y[:, enemy_slots], engine.drop_y[:, drop_slots]), dim=1).numpy(),
-        sprite_z=torch.cat((engine.enemy_z[:, enemy_slots], engine.drop_z[:, drop_slots]), dim=1).numpy(),
-        sprite_id=torch.cat((enemy_sprite[:, enemy_slots], drop_sprite[:, drop_slots]), dim=1).numpy().astype(np.int32),
-        sprite_alive=torch.cat((engine.enemy_alive[:, enemy_slots], drop_visible[:, drop_slots]), dim=1).numpy(),
-        sprite_fullbright=torch.cat(
-            (fullbright, torch.zeros_like(drop_visible[:, drop_slots])), dim=1
-        ).numpy(),
+        sprite_x=columns[0].numpy(), sprite_y=columns[1].numpy(), sprite_z=columns[2].numpy(),
+        sprite_id=columns[3].numpy().astype(np.int32), sprite_alive=columns[4].numpy(),
+        sprite_fullbright=columns[5].numpy(), sprite_style=columns[6].numpy().astype(np.int8),
     )
 
 
