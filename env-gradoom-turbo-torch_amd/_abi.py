@@ -121,6 +121,7 @@ LANE_ARRAYS = (
     ("sprite_fullbright", np.uint8),
     ("weapon_state", np.int64),
     ("hud_state", np.int32),
+    ("screen_blend", np.float32),
     ("sprite_style", np.int8),
 )
 

@@ -2500,14 +2500,34 @@ __global__ void __launch_bounds__(256) hud_kernel(Overlays ov, const int *hud_st
 // ---------------------------------------------------------------------------------------------
 // observation: _triton_kernels.py:120-177 + engine.py:9545-9548 / 2443-2450
 // ---------------------------------------------------------------------------------------------
+// One PLAYPAL channel after the pickup (gold) and damage (red) screen blends, evaluated in float32 one
+// operation at a time and truncated to a byte (engine.py:15385-15397).
+__device__ __forceinline__ unsigned char blended_channel(unsigned char value, int channel, float bonus, float flash) {
+    const float gold = channel == 0 ? 215.0f : (channel == 1 ? 186.0f : 69.0f);
+    const float red = channel == 0 ? 255.0f : 0.0f;
+    float v = (float)value * (1.0f - bonus) + gold * bonus;
+    v = v * (1.0f - flash) + red * flash;
+    return (unsigned char)fminf(fmaxf(v, 0.0f), 255.0f);
+}
+
+// `blend` points at the first lane's (bonus, damage) alphas, or is null for plain PLAYPAL colours.
+__device__ __forceinline__ void stage_palette(unsigned char *pal, const unsigned char *playpal, const float *blend, int lane) {
+    if (blend) {
+        const float bonus = blend[2 * lane], flash = blend[2 * lane + 1];
+        for (int k = threadIdx.x; k < 768; k += blockDim.x) pal[k] = blended_channel(playpal[k], k % 3, bonus, flash);
+    } else {
+        for (int k = threadIdx.x; k < 768; k += blockDim.x) pal[k] = playpal[k];
+    }
+    __syncthreads();
+}
+
 __global__ void observe_kernel(const unsigned char *indexed, size_t lane_stride, int source_rows, const unsigned char *playpal,
                                int lane_count, unsigned char *obs, unsigned char *frames, const unsigned char *reset_mask, int stack_mode,
-                               unsigned char *final_frames) {
+                               unsigned char *final_frames, const float *blend) {
     __shared__ unsigned char pal[768];
-    for (int k = threadIdx.x; k < 768; k += blockDim.x) pal[k] = playpal[k];
-    __syncthreads();
     int pixel = blockIdx.x * blockDim.x + threadIdx.x;
     int n = blockIdx.y;
+    stage_palette(pal, playpal, blend, n < lane_count ? n : 0);
     if (n >= lane_count || pixel >= GD_OBS_SIZE * GD_OBS_SIZE) return;
     int oy = pixel / GD_OBS_SIZE, ox = pixel - oy * GD_OBS_SIZE;
     const unsigned char *src = indexed + (size_t)n * lane_stride;
@@ -2570,10 +2590,11 @@ __global__ void observe_kernel(const unsigned char *indexed, size_t lane_stride,
 }
 
 // engine.py:15381-15384
-__global__ void expand_rgb_kernel(const unsigned char *indexed, const unsigned char *playpal, size_t pixels, unsigned char *rgb) {
+// A block of 256 pixels never straddles two lanes when lane_pixels is a multiple of 256 (240 x 320 is).
+__global__ void expand_rgb_kernel(const unsigned char *indexed, const unsigned char *playpal, size_t pixels, unsigned char *rgb,
+                                  const float *blend, size_t lane_pixels) {
     __shared__ unsigned char pal[768];
-    for (int k = threadIdx.x; k < 768; k += blockDim.x) pal[k] = playpal[k];
-    __syncthreads();
+    stage_palette(pal, playpal, blend, blend ? (int)(((size_t)blockIdx.x * blockDim.x) / lane_pixels) : 0);
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= pixels) return;
     int p = indexed[i] * 3;
@@ -2745,12 +2766,15 @@ int launch_chunk(gd_renderer *r, Scratch &sc, const gd_lanes_desc *lanes, const 
                            frame_base, frame_stride, VH, m.playpal, count, out->obs ? out->obs + (size_t)base * F : nullptr,
                            out->frames ? out->frames + (size_t)base * GD_FRAME_STACK * F : nullptr,
                            out->reset_mask ? out->reset_mask + base : nullptr, out->stack_mode,
-                           out->final_frames ? out->final_frames + (size_t)base * GD_FRAME_STACK * F : nullptr);
+                           out->final_frames ? out->final_frames + (size_t)base * GD_FRAME_STACK * F : nullptr,
+                           lanes->screen_blend ? lanes->screen_blend + 2 * (size_t)base : nullptr);
     }
     if (out->rgb) {
         size_t pixels = (size_t)count * frame_stride;
+        static_assert((GD_SCREEN_HEIGHT * SW) % 256 == 0, "expand_rgb_kernel: one lane per block");
         hipLaunchKernelGGL(expand_rgb_kernel, dim3((unsigned)((pixels + 255) / 256)), dim3(256), 0, stream, frame_base, m.playpal, pixels,
-                           out->rgb + (size_t)base * frame_stride * 3);
+                           out->rgb + (size_t)base * frame_stride * 3,
+                           lanes->screen_blend ? lanes->screen_blend + 2 * (size_t)base : nullptr, (size_t)GD_SCREEN_HEIGHT * SW);
     }
     mark();
     HIP_TRY(hipGetLastError());
@@ -3065,7 +3089,7 @@ int gd_observe(const uint8_t *indexed, int32_t source_rows, const uint8_t *playp
         hipLaunchKernelGGL(observe_kernel, dim3((GD_OBS_SIZE * GD_OBS_SIZE + 255) / 256, count), dim3(256), 0, static_cast<hipStream_t>(stream),
                            indexed + (size_t)base * source_rows * SW, (size_t)source_rows * SW, source_rows, playpal, count,
                            obs ? obs + (size_t)base * F : nullptr, frames ? frames + (size_t)base * GD_FRAME_STACK * F : nullptr,
-                           reset_mask ? reset_mask + base : nullptr, stack_mode, nullptr);
+                           reset_mask ? reset_mask + base : nullptr, stack_mode, nullptr, nullptr);
     }
     HIP_TRY(hipGetLastError());
     return GD_OK;
@@ -3080,7 +3104,7 @@ int gd_expand_rgb24(const uint8_t *indexed, int32_t rows, const uint8_t *playpal
     for (size_t base = 0; base < pixels; base += step) {
         size_t count = pixels - base < step ? pixels - base : step;
         hipLaunchKernelGGL(expand_rgb_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
-                           indexed + base, playpal, count, rgb + base * 3);
+                           indexed + base, playpal, count, rgb + base * 3, nullptr, (size_t)1);
     }
     HIP_TRY(hipGetLastError());
     return GD_OK;

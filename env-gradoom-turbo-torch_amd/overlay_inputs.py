@@ -145,3 +145,15 @@ def hud_state(
     counts = hud_ammo_counts.to(torch.int64)
     columns = (ammo, health_int, armor_int, face, owned, counts[:, 0], counts[:, 1], counts[:, 2], counts[:, 3])
     return torch.stack(columns, dim=1).to(torch.int32).contiguous()
+
+
+def screen_blend(bonus_count: torch.Tensor, damage_count: torch.Tensor, damage_to_alpha: torch.Tensor) -> torch.Tensor:
+    """f32 [N,2]: the pickup and damage alphas of ``_native_indexed_to_rgb`` (engine.py:15385-15394).
+
+    ``damage_to_alpha`` is the engine's 114-entry ``_damage_to_alpha`` table.  Lanes carrying this
+    tensor get PLAYPAL mixed with gold and then red before the RGB24 frame and the observation.
+    """
+
+    bonus = torch.minimum(bonus_count.to(torch.float32) * 8.0, torch.full_like(bonus_count, 128.0, dtype=torch.float32))
+    flash = damage_to_alpha.to(torch.float32)[damage_count.clamp(0, 113).to(torch.int64)]
+    return torch.stack((bonus / 255.0, flash / 255.0), dim=1).contiguous()

@@ -49,6 +49,7 @@ class LaneState:
     weapon_state: torch.Tensor | None = None  # i64 [N,5]
     hud_state: torch.Tensor | None = None  # i32 [N,9]
     sprite_style: torch.Tensor | None = None  # i8 [N,A]: -1 opaque, -2 translucent, >= 0 additive table
+    screen_blend: torch.Tensor | None = None  # f32 [N,2] bonus / damage alphas (overlay_inputs.screen_blend)
 
     @classmethod
     def from_numpy(cls, arrays: dict, device) -> "LaneState":
@@ -68,7 +69,7 @@ class LaneState:
             sprite_fullbright=get("sprite_fullbright", torch.uint8), ray_cos=get("ray_cos", torch.float32),
             ray_sin=get("ray_sin", torch.float32), sprite_depth=get("sprite_depth", torch.float32),
             weapon_state=get("weapon_state", torch.int64), hud_state=get("hud_state", torch.int32),
-            sprite_style=get("sprite_style", torch.int8),
+            sprite_style=get("sprite_style", torch.int8), screen_blend=get("screen_blend", torch.float32),
         )
 
 
@@ -195,6 +196,8 @@ class HipRenderer:
             desc.sprite_depth = _require(depth, "sprite_depth", torch.float32, (count, slots), device).data_ptr()
         if lanes.weapon_state is not None:
             desc.weapon_state = _require(lanes.weapon_state, "weapon_state", torch.int64, (count, 5), device).data_ptr()
+        if lanes.screen_blend is not None:
+            desc.screen_blend = _require(lanes.screen_blend, "screen_blend", torch.float32, (count, 2), device).data_ptr()
         if lanes.hud_state is not None:
             desc.hud_state = _require(lanes.hud_state, "hud_state", torch.int32, (count, 9), device).data_ptr()
         return desc, keep

@@ -162,6 +162,10 @@ typedef struct gd_lanes_desc {
     const int32_t *hud_state;       /* [N,9] status bar of engine.py:15232-15267: ready ammo, health, armor,
                                        face patch id, owned weapon bits (bit k = weapon k+1, k < 5),
                                        four ammo counts */
+    const float *screen_blend;      /* [N,2] or NULL (no blend): bonus alpha min(bonus_count*8, 128)/255 and damage
+                                       alpha damage_to_alpha[clamp(damage_count, 0, 113)]/255; PLAYPAL colours are
+                                       mixed with gold and then red before the RGB24 frame and the observation
+                                       (_native_indexed_to_rgb with render_screen_flashes, engine.py:15381-15398) */
     const int8_t *sprite_style;     /* [N,A] or NULL (all -1): -1 opaque, -2 translucent_lut, s >= 0
                                        additive_luts[min(s, 1)] (actor_additive_style, engine.py:14343-14682) */
 } gd_lanes_desc;

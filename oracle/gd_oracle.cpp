@@ -1523,6 +1523,18 @@ struct Oracle {
 };
 
 // _policy_area_grayscale_kernel (_triton_kernels.py:120-177) for one lane
+// engine.py:15385-15397: PLAYPAL after the pickup (gold) and damage (red) screen blends, float32 op by op
+void blended_palette(const uint8_t *playpal, const float *blend, uint8_t *out) {
+    static const float gold[3] = {215.0f, 186.0f, 69.0f}, red[3] = {255.0f, 0.0f, 0.0f};
+    for (int k = 0; k < 768; ++k) {
+        if (!blend) { out[k] = playpal[k]; continue; }
+        float v = float(playpal[k]) * (1.0f - blend[0]) + gold[k % 3] * blend[0];
+        v = v * (1.0f - blend[1]) + red[k % 3] * blend[1];
+        float clamped = std::min(std::max(v, 0.0f), 255.0f);
+        out[k] = uint8_t(clamped);
+    }
+}
+
 void observe_lane(const uint8_t *indexed, int source_rows, const uint8_t *playpal, uint8_t *obs) {
     for (int oy = 0; oy < GD_OBS_SIZE; ++oy) {
         for (int ox = 0; ox < GD_OBS_SIZE; ++ox) {
@@ -1757,14 +1769,16 @@ int gdo_render(const gd_map_desc *map, const gd_lanes_desc *lanes, const gd_fram
         if (g_overlays_set && lanes->hud_state && g_overlays.hud_patch_count > 0)
             render_hud(full.data() + size_t(VH) * SW, lanes->hud_state + size_t(n) * 9);
         if (out->indexed) std::memcpy(out->indexed + size_t(n) * full.size(), full.data(), full.size());
+        uint8_t palette[768];
+        blended_palette(map->playpal, lanes->screen_blend ? lanes->screen_blend + 2 * size_t(n) : nullptr, palette);
         if (out->obs || out->frames) {
-            observe_lane(full.data(), VH, map->playpal, obs.data());  // HUD rows masked black
+            observe_lane(full.data(), VH, palette, obs.data());  // HUD rows masked black
             if (out->obs) std::memcpy(out->obs + size_t(n) * obs.size(), obs.data(), obs.size());
             if (out->frames) stack_lane(obs.data(), out->frames + size_t(n) * GD_FRAME_STACK * obs.size(), out->reset_mask && out->reset_mask[n], out->stack_mode);
         }
         if (out->rgb) {
             uint8_t *rgb = out->rgb + size_t(n) * full.size() * 3;
-            for (size_t i = 0; i < full.size(); ++i) for (int c = 0; c < 3; ++c) rgb[i * 3 + c] = map->playpal[full[i] * 3 + c];
+            for (size_t i = 0; i < full.size(); ++i) for (int c = 0; c < 3; ++c) rgb[i * 3 + c] = palette[full[i] * 3 + c];
         }
     }
     if (profile) std::fprintf(stderr, "oracle lanes %d: setup %.3fs flats %.3fs walls %.3fs sprites %.3fs\n", lane_end - lane_begin, t_setup, t_flats, t_walls, t_sprites);

@@ -110,6 +110,11 @@ CASES = {
         map_seed=22, grid=(6, 5), sectors=26, linedefs=160, lanes=8, pose_seed=3, sprites=48, effects=60, blend_seed=13,
         pitch=True, flash=True, midtex=0.2,
     ),
+    # render_screen_flashes: PLAYPAL mixed with gold (pickups) and red (damage) per lane before the RGB24 frame
+    # and the observation (engine.py:15381-15398)
+    "screen_flashes": dict(
+        map_seed=12, grid=(5, 4), sectors=17, linedefs=100, lanes=4, pose_seed=6, sprites=16, screen_flashes=29
+    ),
     "config2_subset": dict(map_seed=1002, grid=(12, 9), sectors=96, linedefs=800, lanes=4, pose_seed=1, sprites=32),
     "config3_subset": dict(
         map_seed=1003, grid=(15, 15), sectors=200, linedefs=2000, lanes=2, pose_seed=1, sprites=64, flash=True
@@ -132,7 +137,9 @@ def build_case(name: str, cfg: dict, do_time: bool) -> dict:
     lanes = cfg["lanes"]
     started = time.time()
     overlays = synthmap.generate_overlays(cfg["overlays"]) if cfg.get("overlays") else None
-    engine = refdrive.make_engine(smap, lanes, flash_lights=cfg.get("flash", False), overlays=overlays)
+    engine = refdrive.make_engine(
+        smap, lanes, flash_lights=cfg.get("flash", False), overlays=overlays, screen_flashes=bool(cfg.get("screen_flashes"))
+    )
     ctor_seconds = time.time() - started
     picks = cfg.get("picks") or [(cfg["pose_seed"], lane) for lane in range(lanes)]
     assert len(picks) == lanes
@@ -189,6 +196,17 @@ def build_case(name: str, cfg: dict, do_time: bool) -> dict:
             [engine._native_mugshot_patch_index(lane, int(engine.health[lane].clamp(0, 999).item())) for lane in range(lanes)],
             dtype=np.int64,
         )
+    if cfg.get("screen_flashes"):
+        # pickup and damage counters as gameplay leaves them; lane 0 keeps both at zero (blend = identity)
+        generator = torch.Generator().manual_seed(cfg["screen_flashes"])
+        engine.bonus_count[:] = torch.randint(0, 24, (lanes,), generator=generator).to(engine.bonus_count.dtype)
+        engine.damage_count[:] = torch.randint(0, 130, (lanes,), generator=generator).to(engine.damage_count.dtype)
+        engine.bonus_count[0] = 0
+        engine.damage_count[0] = 0
+        engine.damage_count[1] = 0
+        data["screen_blend"] = overlay_inputs.screen_blend(engine.bonus_count, engine.damage_count, engine._damage_to_alpha).numpy()
+        with torch.no_grad():
+            data["rgb_all"] = engine.render_native_frame(include_hud=True).numpy()
     started = time.time()
     with torch.no_grad():
         indexed = engine._render_native_indexed_frame(include_hud=True)

@@ -116,10 +116,12 @@ def to_compiled_scenario(smap, *, flash_lights: bool = False, overlays: dict | N
     )
 
 
-def make_engine(smap, lanes: int, *, flash_lights: bool = False, overlays: dict | None = None):
+def make_engine(smap, lanes: int, *, flash_lights: bool = False, overlays: dict | None = None, screen_flashes: bool = False):
     engine_module, _scenario = load_reference()
     compiled = to_compiled_scenario(smap, flash_lights=flash_lights, overlays=overlays)
-    return engine_module.TorchDeathmatchEngine(compiled, lanes, device=torch.device("cpu"))
+    return engine_module.TorchDeathmatchEngine(
+        compiled, lanes, device=torch.device("cpu"), render_screen_flashes=screen_flashes
+    )
 
 
 def set_poses(engine, poses) -> None:

@@ -41,7 +41,7 @@ def test_indexed_frame_bit_exact_vs_reference_golden(name):
     renderer.close()
 
 
-@pytest.mark.parametrize("name", ["config1", "small_midtex_sprites"])
+@pytest.mark.parametrize("name", ["config1", "small_midtex_sprites", "screen_flashes"])
 def test_observation_and_stack_bit_exact_vs_oracle(oracle, name):
     meta, data, tables, renderer, lanes = _renderer(name)
     count = meta["lanes"]
@@ -60,6 +60,8 @@ def test_observation_and_stack_bit_exact_vs_oracle(oracle, name):
     assert np.array_equal(frames.cpu().numpy(), expected["frames"])
     assert np.array_equal(rgb.cpu().numpy(), expected["rgb"])
     assert np.array_equal(rgb[0].cpu().numpy(), data["rgb_lane0"])
+    if "rgb_all" in data:   # the case with per-lane screen blends carries every lane's reference RGB24 frame
+        assert np.array_equal(rgb.cpu().numpy(), data["rgb_all"][:count])
     renderer.close()
 
 

@@ -80,3 +80,14 @@ def test_rgb_expansion_matches_reference(oracle):
     _meta, data, _smap, tables = load_fixture("tiny_stages")
     result = oracle.render(tables, lane_inputs(data), data["cosine_correction"], lane_range=(0, 1), want_rgb=True)
     assert np.array_equal(result["rgb"][0], data["rgb_lane0"])
+
+
+def test_screen_flashes_blend_the_palette_per_lane(oracle):
+    """render_screen_flashes (engine.py:15381-15398): RGB24 bit-exact, lane 0 (both counters zero) unblended."""
+
+    _meta, data, _smap, tables = load_fixture("screen_flashes")
+    result = oracle.render(tables, lane_inputs(data), data["cosine_correction"], want_rgb=True)
+    assert np.array_equal(result["rgb"], data["rgb_all"])
+    playpal = tables["playpal"].reshape(256, 3)
+    assert np.array_equal(result["rgb"][0], playpal[result["indexed"][0]])
+    assert not np.array_equal(result["rgb"][2], playpal[result["indexed"][2]])
