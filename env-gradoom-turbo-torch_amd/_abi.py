@@ -121,6 +121,8 @@ LANE_ARRAYS = (
     ("sprite_fullbright", np.uint8),
     ("weapon_state", np.int64),
     ("hud_state", np.int32),
+    ("decal_state", np.int32),
+    ("decal_geom", np.float32),
     ("screen_blend", np.float32),
     ("sprite_style", np.int8),
 )
@@ -137,7 +139,9 @@ class MapDesc(C.Structure):
 
 
 class LanesDesc(C.Structure):
-    _fields_ = [("lane_count", C.c_int32), ("sprite_slots", C.c_int32)] + [(name, _P) for name, _ in LANE_ARRAYS]
+    _fields_ = [("lane_count", C.c_int32), ("sprite_slots", C.c_int32), ("decal_slots", C.c_int32)] + [
+        (name, _P) for name, _ in LANE_ARRAYS
+    ]
 
 
 OVERLAY_SCALARS = ("weapon_patch_count", "weapon_max_h", "weapon_max_w", "hud_patch_count", "hud_max_h", "hud_max_w")
@@ -157,8 +161,22 @@ OVERLAY_ARRAYS = (
 )
 
 
+DECAL_SCALARS = ("decal_variant_count", "decal_max_h", "decal_max_w", "decal_black_rows")
+DECAL_ARRAYS = (
+    ("decal_atlas", np.uint8),
+    ("decal_h", np.int32),
+    ("decal_left", np.int32),
+    ("decal_top", np.int32),
+    ("decal_opacity_lut", np.uint8),
+    ("decal_black_lut", np.uint8),
+)
+
+
 class OverlayDesc(C.Structure):
-    _fields_ = [(name, C.c_int32) for name in OVERLAY_SCALARS] + [(name, _P) for name, _ in OVERLAY_ARRAYS]
+    _fields_ = (
+        [(name, C.c_int32) for name in OVERLAY_SCALARS] + [(name, _P) for name, _ in OVERLAY_ARRAYS]
+        + [(name, C.c_int32) for name in DECAL_SCALARS] + [(name, _P) for name, _ in DECAL_ARRAYS]
+    )
 
 
 def host_overlay_desc(overlays: dict) -> tuple[OverlayDesc, list]:
@@ -185,6 +203,21 @@ def host_overlay_desc(overlays: dict) -> tuple[OverlayDesc, list]:
         array = np.ascontiguousarray(overlays[name], dtype=dtype)
         keep.append(array)
         setattr(desc, name, array.ctypes.data)
+    if overlays.get("decal_atlas") is not None:
+        atlas = np.ascontiguousarray(overlays["decal_atlas"], dtype=np.uint8)
+        if atlas.ndim != 3 or atlas.shape[0] != 5:
+            raise ValueError("decal_atlas must be [5, height, width]")
+        black = np.ascontiguousarray(overlays["decal_black_lut"], dtype=np.uint8)
+        if np.asarray(overlays["decal_opacity_lut"]).shape != (32, 256) or black.ndim != 2 or black.shape[1] != 256:
+            raise ValueError("decal_opacity_lut must be [32,256] and decal_black_lut [rows,256]")
+        desc.decal_variant_count, desc.decal_max_h, desc.decal_max_w = atlas.shape
+        desc.decal_black_rows = black.shape[0]
+        for name, dtype in DECAL_ARRAYS:
+            array = np.ascontiguousarray(overlays[name], dtype=dtype)
+            if name in ("decal_h", "decal_left", "decal_top") and array.shape != (5,):
+                raise ValueError(f"{name} must hold one value per variant")
+            keep.append(array)
+            setattr(desc, name, array.ctypes.data)
     return desc, keep
 
 

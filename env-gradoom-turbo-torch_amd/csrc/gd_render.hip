@@ -13,7 +13,9 @@
 //   flat_finish     320 threads / lane        visplane repair (wave ballots), status bar rows cleared
 //   wall_columns    1 wave / strip            portal traversal, tiers, planes, masked mid-textures
 //   plane_shade     1 thread / 4 pixels       flat texel + light for every pixel a wall did not cover
-//   sprite_columns  320 threads / lane        billboards far -> near
+//   decal           320 threads / lane        bullet chips on the wall tiers they hit (frames that carry decals
+//                                             also keep a per-pixel scene depth: wall_columns<true>, plane_shade<true>)
+//   sprite_columns  320 threads / lane        billboards far -> near, opaque / additive / translucent
 //   weapon_overlay, hud                       player weapon, muzzle flash and status bar patches
 //   observe         1 thread / obs pixel      PLAYPAL + exact area pool + gray + 4-frame stack
 //   expand_rgb      1 thread / pixel          PLAYPAL expansion for callers that want RGB24 frames
@@ -135,6 +137,8 @@ struct Scratch {    // per-chunk working memory, sized at create
     LaneCtx *ctx;          // [L]
     WallRec *rec;          // [L,W]
     WallRec *frag_rec;     // [L,split_count,fragment_slots] FWallCoords of the BSP fragments of split linedefs
+    float *scene_depth;    // [L,208,320] depth of the surface each pixel shows (engine.py:11553, 12700, 13411, 13740),
+                           // kept only for frames that draw wall decals, else null
     Cand *cand;            // [L,CAND_MAX,320]
     int *cand_count;       // [L,320] (may exceed CAND_MAX when a list overflowed)
     unsigned short *flat_sector;// [L,208,320]
@@ -1508,6 +1512,7 @@ struct PixelBuffers {
     unsigned char *frame;   // [240][320]
     unsigned int *meta;     // [208][320]
     float *clip_depth;      // [208][320]
+    float *scene_depth;     // [208][320] or null
 };
 
 // Silhouette bookkeeping: every row >= bot_row holds a clip depth <= bot_depth, every row
@@ -1560,6 +1565,7 @@ __device__ __forceinline__ void apply_silhouette(PixelBuffers &pb, SilhouetteBou
 // rows that its own clip update then removes from the window, so the window stays untouched
 // until a one-sided drawseg (which leaves the clips alone) has painted; until then painting
 // needs no reads and visits only the rows it writes.
+template <bool DEPTH>
 __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnState &c, const PassColumn &r, PixelBuffers &pb,
                            const bool group_valid[3], const float group_bottom[3], i64 first_group_visibility,
                            const unsigned char *colormap, bool &window_dirty) {
@@ -1646,6 +1652,7 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
                 const size_t i = (size_t)(yb + j) * SW + x;
                 pb.frame[i] = colormap[(tail[j] ? shade_group : shade_own) * 256 + texel[j]];
                 pb.clip_depth[i] = r.distance;
+                if (DEPTH) pb.scene_depth[i] = r.distance;
                 pb.meta[i] = META_FILLED | (unsigned)(wi + 1);
             }
         }
@@ -1682,6 +1689,7 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
                 i64 tv = (fraction & UINT32_MASK) >> (32 - height_bits);
                 unsigned char texel = m->tex_atlas[((size_t)texture_id * m->tex_max_h + tv) * m->tex_max_w + tu];
                 pb.frame[i] = colormap[(bottom_tail ? shade_group : shade_own) * 256 + texel];
+                if (DEPTH) pb.scene_depth[i] = r.distance;
                 if (r.distance < pb.clip_depth[i]) { pb.clip_depth[i] = r.distance; meta = (meta & ~META_WALL_MASK) | (unsigned)(wi + 1); }
                 meta |= META_FILLED;
                 meta_dirty = true;
@@ -1859,6 +1867,7 @@ __device__ __forceinline__ bool pass_advance(const ColumnCtx &cc, ColumnState &c
 }
 
 // engine.py:13424-13744 for one column
+template <bool DEPTH>
 __device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const ColumnState &c, PixelBuffers &pb) {
     const gd_map_desc *m = cc.m;
     const MapView &mv = cc.mv;
@@ -1955,6 +1964,7 @@ __device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const Col
         unsigned char texel = m->tex_atlas[((size_t)texture_id * m->tex_max_h + mv_) * m->tex_max_w + mu];
         pb.frame[(size_t)y * SW + x] = m->colormap[shade * 256 + texel];
         pb.meta[(size_t)y * SW + x] |= META_MASKED;
+        if (DEPTH) pb.scene_depth[(size_t)y * SW + x] = md;
     }
 }
 
@@ -2012,6 +2022,8 @@ __global__ void __launch_bounds__(1024) strip_order_kernel(int strips, Scratch s
 // otherwise fill the register file with three, and the flat kernels on the side stream could not
 // run beside it at all.
 #define WALL_LDS_PAD 3072
+// DEPTH: also keep the depth of every wall pixel (frames that draw decals).
+template <bool DEPTH>
 __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amdgpu_waves_per_eu(3, 3))) wall_columns_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
     const gd_map_desc *m = &dm.d;
     __shared__ LaneCtx lane_ctxs[WALL_STRIPS_PER_GROUP];
@@ -2045,6 +2057,7 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
     pb.frame = frame_base + (size_t)local * frame_stride;
     pb.meta = sc.meta + (size_t)local * VH * SW;
     pb.clip_depth = sc.clip_depth + (size_t)local * VH * SW;
+    pb.scene_depth = DEPTH ? sc.scene_depth + (size_t)local * VH * SW : nullptr;
     for (int y = 0; y < VH; ++y) { pb.meta[(size_t)y * SW + x] = 0; pb.clip_depth[(size_t)y * SW + x] = GD_INF; }
     ColumnState st;
     st.current_sector = lane_ctx.sector;
@@ -2095,7 +2108,7 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
         for (int t = 0; t < 3; ++t) group_valid[t] = same_group && all_tier[t] && (common_top[t] < common_bottom[t]);
         if (!done) {
             PROF_T(t2);
-            pass_paint(cc, st, pc, pb, group_valid, common_bottom, first_group_visibility, colormap_lds, window_dirty);
+            pass_paint<DEPTH>(cc, st, pc, pb, group_valid, common_bottom, first_group_visibility, colormap_lds, window_dirty);
             PROF_T(t3);
             PROF_ADD(1, t2, t3);
             bool changed = pass_advance(cc, st, pc, pb, sb);
@@ -2111,7 +2124,7 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
     }
     PROF_T(t5);
     PROF_T(t6);
-    masked_midtexture(cc, st, pb);
+    masked_midtexture<DEPTH>(cc, st, pb);
 #ifdef GD_PROFILE
     long long t7 = wall_clock64();
     int prof_cands = cc.count;
@@ -2137,6 +2150,7 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
 // ---------------------------------------------------------------------------------------------
 #define SHADE_TILES 12   // 256-pixel tiles per block: 260 tiles per view = 22 blocks per lane
 #define SHADE_GROUP 4    // tiles per step
+template <bool DEPTH>   // DEPTH: also keep the depth of every pixel no wall tier covers (frames that draw decals)
 __global__ void __launch_bounds__(256) plane_shade_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
     const gd_map_desc *m = &dm.d;
     __shared__ float4 sector_lds[LDS_SECTORS];
@@ -2201,6 +2215,24 @@ __global__ void __launch_bounds__(256) plane_shade_kernel(DeviceMap dm, int lane
             const bool is_floor = claimed ? (meta[j] & META_FLOOR) != 0 : ((float)y - flat_center(c)) > 0;
             if (shade[j]) frame[pixel] = colormap_lds[colormap_row[j] * 256 + texel[j]];
             else if (!(meta[j] & META_MASKED)) frame[pixel] = flat_pixel(tb, colormap_lds, c, claimed ? ps : (int)flat_sector[j], is_floor, x, y);
+            if (DEPTH && !(meta[j] & META_MASKED)) {
+                float depth;
+                if (claimed) {   // exact plane depth (engine.py:13406-13416)
+                    const float flat_center_px = (103.0f + c.pitch_offset) + 0.5f;
+                    const float plane_height = is_floor ? (c.view_z - tb.floor_h(ps)) : (tb.ceil_h(ps) - c.view_z);
+                    depth = plane_height * 192.0f / fmaxf(fabsf((float)y - flat_center_px), 0.5f);
+                } else {         // what the flat pass left (engine.py:11140-11166)
+                    const int s = flat_sector[j];
+                    const float delta = (float)y - flat_center(c);
+                    const float plane_height = delta > 0 ? (c.view_z - tb.floor_h(s)) : (tb.ceil_h(s) - c.view_z);
+                    const float perpendicular = plane_height * 192.0f / fmaxf(fabsf(delta), 0.5f);
+                    const float cosine = dm.cosine_correction[x];
+                    if (flat_flags[j] & (2 | 8)) depth = perpendicular;             // repaired: its visplane's depth
+                    else if (flat_flags[j] & 1) depth = GD_INF;                    // no sector found along the ray
+                    else depth = (perpendicular / cosine) * cosine;                // ray distance of the hit, corrected back
+                }
+                sc.scene_depth[i] = depth;
+            }
             // plane fallback occluder for sprites where the flat ray was unresolved (engine.py:13417-13422)
             if (claimed && (flat_flags[j] & 1) && !finitef(sc.clip_depth[i])) {
                 const float flat_center_px = (103.0f + c.pitch_offset) + 0.5f;
@@ -2376,6 +2408,100 @@ __global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lan
                 else if (style >= 0) lit = m->additive_luts[((size_t)(style > 1 ? 1 : style) * 256 + *pixel) * 256 + lit];
                 *pixel = lit;
             }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// wall decals: engine.py:13747-13991, drawn after the walls and before the sprites
+// ---------------------------------------------------------------------------------------------
+// One thread per screen column; a lane's decals are painted oldest first, each only where the scene
+// depth is the decal's own ray distance (which ties it to the wall tier it sits on).
+__global__ void __launch_bounds__(SW) decal_kernel(DeviceMap dm, Overlays ov, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc,
+                                                   unsigned char *frame_base, size_t frame_stride) {
+    const gd_map_desc *m = &dm.d;
+    const gd_overlay_desc &o = ov.d;
+    const int local = blockIdx.x;
+    if (local >= lane_count) return;
+    const int n = lane_base + local;
+    const int x = threadIdx.x;
+    const LaneCtx &L = sc.ctx[local];
+    const int D = lanes.decal_slots;
+    const int width = o.decal_max_w;
+    const float center = 104.0f + L.pitch_offset;
+    unsigned char *frame = frame_base + (size_t)local * frame_stride;
+    const float *scene_depth = sc.scene_depth + (size_t)local * VH * SW;
+    float rx, ry; ray_direction(L, x, &rx, &ry);
+    for (int k = 0; k < D; ++k) {
+        const int *state = lanes.decal_state + ((size_t)n * D + k) * 3;
+        const float *geom = lanes.decal_geom + ((size_t)n * D + k) * 4;
+        if (!state[2]) continue;
+        const int wall_index = (int)clampi(state[0], 0, m->wall_count - 1);
+        const int style = state[1];
+        const int variant = style % 5;
+        const bool flip_x = (style / 5) % 2, flip_y = (style / 10) % 2;
+        const int side = style / 20;
+        const float along_wall = geom[0], impact_z = geom[1], tangent_x = geom[2], tangent_y = geom[3];
+        const float4 wl = *reinterpret_cast<const float4 *>(m->walls + 4 * wall_index);
+        const float wvx = wl.z - wl.x, wvy = wl.w - wl.y;
+        const float viewer_cross = wvx * (L.y - wl.y) - wvy * (L.x - wl.x);
+        if ((viewer_cross > 0 ? 1 : 0) != side) continue;
+        const float impact_x = wl.x + along_wall * wvx, impact_y = wl.y + along_wall * wvy;
+        const float left_offset = (float)o.decal_left[variant];
+        const float back = left_offset * 0.5f, forth = ((float)width - left_offset) * 0.5f;
+        const float left_x = impact_x - tangent_x * back, left_y = impact_y - tangent_y * back;
+        const float right_x = impact_x + tangent_x * forth, right_y = impact_y + tangent_y * forth;
+        const float seg_x = right_x - left_x, seg_y = right_y - left_y;
+        // FWallCoords::Init on the two fixed-point endpoints (engine.py:13836-13887)
+        const i64 lx = round_to_i64(left_x * 65536.0f) - L.view_x_fixed, ly = round_to_i64(left_y * 65536.0f) - L.view_y_fixed;
+        const i64 qx = round_to_i64(right_x * 65536.0f) - L.view_x_fixed, qy = round_to_i64(right_y * 65536.0f) - L.view_y_fixed;
+        const i64 tx1 = (lx * L.vsin - ly * L.vcos) >> 20, ty1 = (lx * L.vcos + ly * L.vsin) >> 20;
+        const i64 tx2 = (qx * L.vsin - qy * L.vcos) >> 20, ty2 = (qx * L.vcos + qy * L.vsin) >> 20;
+        const i64 center_fixed = 160 * FIXED_UNIT;
+        const i64 projected_left = ((center_fixed + tdiv(tx1 * center_fixed, ty1 == 0 ? 1 : ty1)) >> 16) + (tx1 >= 0);
+        const i64 projected_right = ((center_fixed + tdiv(tx2 * center_fixed, ty2 == 0 ? 1 : ty2)) >> 16) + (tx2 >= 0);
+        const i64 left_den = tx1 - tx2 - ty2 + ty1, right_den = ty2 - ty1 - tx2 + tx1;
+        const bool left_inside = (tx1 >= -ty1) && (tx1 <= ty1) && (ty1 != 0);
+        const bool right_inside = (tx2 <= ty2) && (tx2 >= -ty2) && (ty2 != 0);
+        const bool left_clipped = (tx1 < -ty1) && (tx2 >= -ty2) && (left_den != 0);
+        const bool right_clipped = (tx2 > ty2) && (tx1 <= ty1) && (right_den != 0);
+        const i64 screen_left = left_inside ? clampi(projected_left, 0, SW) : 0;
+        const i64 screen_right = right_inside ? clampi(projected_right, 0, SW) : SW;
+        if (!((left_inside || left_clipped) && (right_inside || right_clipped) && (screen_right > screen_left))) continue;
+        if (!(x >= screen_left && x < screen_right)) continue;
+        const float off_x = left_x - L.x, off_y = left_y - L.y;
+        const float den = rx * seg_y - ry * seg_x;
+        if (!(fabsf(den) >= 1e-6f)) continue;
+        const float distance = (off_x * seg_y - off_y * seg_x) / den;
+        const float decal_along = (off_x * ry - off_y * rx) / den;
+        if (!(distance > 0)) continue;
+        i64 tu = clampi((i64)floorf(decal_along * (float)width), 0, width - 1);
+        if (flip_x) tu = width - 1 - tu;
+        const float safe_distance = fmaxf(distance, 1e-6f);
+        const float vertical_scale = 96.0f / safe_distance;
+        const float top = center - ((impact_z + (float)o.decal_top[variant] * 0.5f) - L.view_z) * 192.0f / safe_distance;
+        int sector = m->wall_sectors[2 * wall_index + (side > 1 ? 1 : side)];
+        if (sector < 0) sector = 0;
+        const bool horizontal = fabsf(wvy) < 1e-6f, vertical = fabsf(wvx) < 1e-6f;
+        float light = m->sector_lights[sector] + (vertical ? 16.0f : (horizontal ? -16.0f : 0.0f));
+        light = light + (float)(L.flash_light * 16);
+        const i64 depth_fixed = round_to_i64(safe_distance * 4096.0f);
+        const i64 shade = wall_shade(light, tdiv(WALL_VISIBILITY_FIXED << 12, max64(depth_fixed, 1)));
+        const int height = o.decal_h[variant];
+        // rows whose source row floor((y - top) / vertical_scale) can fall inside the patch, a row wider
+        // on either side; the exact test stays per row
+        int y_lo = (int)fminf(fmaxf(floorf(top) - 1.0f, 0.0f), (float)VH);
+        int y_hi = (int)fminf(fmaxf(ceilf(top + (float)height * vertical_scale) + 2.0f, 0.0f), (float)VH);
+        for (int y = y_lo; y < y_hi; ++y) {
+            i64 tv = (i64)floorf(((float)y - top) / vertical_scale);
+            if (!(tv >= 0 && tv < height)) continue;
+            if (flip_y) tv = height - 1 - tv;
+            const size_t i = (size_t)y * SW + x;
+            if (!(fabsf(scene_depth[i] - distance) <= 1e-3f)) continue;
+            const unsigned char source = o.decal_atlas[((size_t)variant * o.decal_max_h + tv) * o.decal_max_w + tu];
+            if (source == 0) continue;
+            const unsigned char opacity = o.decal_opacity_lut[shade * 256 + source];
+            frame[i] = o.decal_black_lut[(size_t)opacity * 256 + frame[i]];
         }
     }
 }
@@ -2715,8 +2841,9 @@ void build_fine_tables(std::vector<i64> &sine, std::vector<i64> &tangent) {
 const int STAGE_COUNT = 8;
 
 // `side` (optional) is a second stream for the flat kernels of this chunk.
-int launch_chunk(gd_renderer *r, Scratch &sc, const gd_lanes_desc *lanes, const gd_frame_out *out, int base, int count, hipStream_t stream, hipStream_t side, bool timed) {
+int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_desc *lanes, const gd_frame_out *out, int base, int count, hipStream_t stream, hipStream_t side, bool timed) {
     const gd_map_desc &m = r->dm.d;
+    Scratch sc = chunk_scratch;
     unsigned char *frame_base;
     size_t frame_stride = (size_t)GD_SCREEN_HEIGHT * SW;
     if (out->indexed) frame_base = out->indexed + (size_t)base * frame_stride;
@@ -2724,7 +2851,10 @@ int launch_chunk(gd_renderer *r, Scratch &sc, const gd_lanes_desc *lanes, const 
     int stage = 0;
     auto mark = [&]() { if (timed) (void)hipEventRecord(r->events[stage], stream); ++stage; };
     // Stage timing needs the kernels one after another; otherwise the flats run on the side stream.
-    const bool overlap = !timed && side != nullptr;
+    const bool decals = lanes->decal_slots > 0 && lanes->decal_state && lanes->decal_geom && r->overlays.d.decal_variant_count > 0;
+    if (!decals) sc.scene_depth = nullptr;
+    // With decals every pass writes the scene depth in turn (flats, walls, planes), so nothing overlaps.
+    const bool overlap = !timed && side != nullptr && !decals;
     hipStream_t flat_stream = overlap ? side : stream;
     mark();
     hipLaunchKernelGGL(lane_setup_kernel, dim3((count + 63) / 64), dim3(64), 0, stream, r->dm, *lanes, base, count, sc);
@@ -2744,11 +2874,21 @@ int launch_chunk(gd_renderer *r, Scratch &sc, const gd_lanes_desc *lanes, const 
     hipLaunchKernelGGL(flat_finish_kernel, dim3(count), dim3(SW), 0, flat_stream, r->dm, count, sc, frame_base, frame_stride);
     mark();
     if (overlap) HIP_TRY(hipEventRecord(r->flat_event, side));
-    hipLaunchKernelGGL(wall_columns_kernel, dim3((count * (SW / 64) + WALL_STRIPS_PER_GROUP - 1) / WALL_STRIPS_PER_GROUP), dim3(64 * WALL_STRIPS_PER_GROUP), WALL_LDS_PAD, stream, r->dm, count, sc, frame_base, frame_stride);
+    {
+        const dim3 grid((count * (SW / 64) + WALL_STRIPS_PER_GROUP - 1) / WALL_STRIPS_PER_GROUP), block(64 * WALL_STRIPS_PER_GROUP);
+        if (decals) hipLaunchKernelGGL(wall_columns_kernel<true>, grid, block, WALL_LDS_PAD, stream, r->dm, count, sc, frame_base, frame_stride);
+        else hipLaunchKernelGGL(wall_columns_kernel<false>, grid, block, WALL_LDS_PAD, stream, r->dm, count, sc, frame_base, frame_stride);
+    }
     mark();
     if (overlap) HIP_TRY(hipStreamWaitEvent(stream, r->flat_event, 0));
-    hipLaunchKernelGGL(plane_shade_kernel, dim3(((VH * SW + 255) / 256 + SHADE_TILES - 1) / SHADE_TILES, count), dim3(256), 0, stream, r->dm, count, sc, frame_base, frame_stride);
+    {
+        const dim3 grid(((VH * SW + 255) / 256 + SHADE_TILES - 1) / SHADE_TILES, count);
+        if (decals) hipLaunchKernelGGL(plane_shade_kernel<true>, grid, dim3(256), 0, stream, r->dm, count, sc, frame_base, frame_stride);
+        else hipLaunchKernelGGL(plane_shade_kernel<false>, grid, dim3(256), 0, stream, r->dm, count, sc, frame_base, frame_stride);
+    }
     mark();
+    if (decals)
+        hipLaunchKernelGGL(decal_kernel, dim3(count), dim3(SW), 0, stream, r->dm, r->overlays, *lanes, base, count, sc, frame_base, frame_stride);
     if (lanes->sprite_slots > 0 && lanes->sprite_x) {
         size_t shared = (size_t)lanes->sprite_slots * sizeof(SpriteRec);
         hipLaunchKernelGGL(sprite_columns_kernel, dim3(count), dim3(SW), shared, stream, r->dm, *lanes, base, count, sc, frame_base, frame_stride);
@@ -2968,6 +3108,9 @@ static int check_render_args(gd_renderer *r, const gd_lanes_desc *lanes, const g
         return fail(GD_E_ARG, "missing lane tensor");
     if (out->stack_mode != GD_STACK_STEP && out->stack_mode != GD_STACK_RESET) return fail(GD_E_ARG, "unknown stack_mode");
     if (lanes->sprite_slots < 0 || lanes->sprite_slots > 512) return fail(GD_E_ARG, "sprite_slots must be in [0, 512]");
+    if (lanes->decal_slots < 0) return fail(GD_E_ARG, "negative decal_slots");
+    if (lanes->decal_slots > 0 && (lanes->decal_state != nullptr) != (lanes->decal_geom != nullptr))
+        return fail(GD_E_ARG, "decal_state and decal_geom go together");
     if (lanes->sprite_slots > 0 && lanes->sprite_x &&
         (!lanes->sprite_y || !lanes->sprite_z || !lanes->sprite_depth || !lanes->sprite_id || !lanes->sprite_alive))
         return fail(GD_E_ARG, "missing sprite tensor");
@@ -3025,6 +3168,16 @@ int gd_renderer_set_overlays(gd_renderer *r, const gd_overlay_desc *h) {
         return fail(GD_E_ARG, "negative overlay size");
     if (h->weapon_patch_count > 0 && (!h->weapon_atlas || !h->weapon_opaque || !h->weapon_w || !h->weapon_h || !h->weapon_left || !h->weapon_top))
         return fail(GD_E_ARG, "missing weapon patch array");
+    if (h->decal_variant_count != 0 &&
+        (h->decal_variant_count != 5 || h->decal_max_h <= 0 || h->decal_max_w <= 0 || h->decal_black_rows <= 0 || !h->decal_atlas ||
+         !h->decal_h || !h->decal_left || !h->decal_top || !h->decal_opacity_lut || !h->decal_black_lut))
+        return fail(GD_E_ARG, "decal patches need 5 variants, their sizes and both tables");
+    if (h->decal_variant_count == 5) {
+        for (int v = 0; v < 5; ++v)
+            if (h->decal_h[v] < 0 || h->decal_h[v] > h->decal_max_h) return fail(GD_E_ARG, "decal height outside the atlas");
+        for (int k = 0; k < 32 * 256; ++k)
+            if (h->decal_opacity_lut[k] >= h->decal_black_rows) return fail(GD_E_ARG, "decal_opacity_lut names a row outside decal_black_lut");
+    }
     if (h->hud_patch_count > 0 && (!h->hud_atlas || !h->hud_opaque || !h->hud_w || !h->hud_h || !h->hud_left || !h->hud_top))
         return fail(GD_E_ARG, "missing status bar patch array");
     HIP_TRY(hipDeviceSynchronize());              // no frame may still be reading the old patches
@@ -3046,10 +3199,21 @@ int gd_renderer_set_overlays(gd_renderer *r, const gd_overlay_desc *h) {
 #define OV(field, bytes) if (rc == GD_OK) rc = copy(h->field, (bytes), reinterpret_cast<const void **>(&d.field))
     OV(weapon_atlas, wt); OV(weapon_opaque, wt); OV(weapon_w, wp * 4); OV(weapon_h, wp * 4); OV(weapon_left, wp * 4); OV(weapon_top, wp * 4);
     OV(hud_atlas, ht); OV(hud_opaque, ht); OV(hud_w, hp * 4); OV(hud_h, hp * 4); OV(hud_left, hp * 4); OV(hud_top, hp * 4);
+    r->sc.scene_depth = nullptr;
+    if (h->decal_variant_count == 5) {
+        OV(decal_atlas, (size_t)5 * h->decal_max_h * h->decal_max_w); OV(decal_h, 5 * 4); OV(decal_left, 5 * 4); OV(decal_top, 5 * 4);
+        OV(decal_opacity_lut, 32 * 256); OV(decal_black_lut, (size_t)h->decal_black_rows * 256);
+        if (rc == GD_OK) {   // the depth buffer decals test against, for one chunk of lanes
+            void *ptr = nullptr;
+            if (hipMalloc(&ptr, (size_t)r->chunk_lanes * VH * SW * sizeof(float)) != hipSuccess) rc = fail(GD_E_HIP, "out of device memory for the decal depth buffer");
+            else { r->overlay_allocations.push_back(ptr); r->sc.scene_depth = static_cast<float *>(ptr); }
+        }
+    }
 #undef OV
     if (rc != GD_OK) {
         for (void *ptr : r->overlay_allocations) (void)hipFree(ptr);
         r->overlay_allocations.clear();
+        r->sc.scene_depth = nullptr;
         return rc;
     }
     r->overlays.d = d;

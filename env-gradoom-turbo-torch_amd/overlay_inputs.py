@@ -157,3 +157,40 @@ def screen_blend(bonus_count: torch.Tensor, damage_count: torch.Tensor, damage_t
     bonus = torch.minimum(bonus_count.to(torch.float32) * 8.0, torch.full_like(bonus_count, 128.0, dtype=torch.float32))
     flash = damage_to_alpha.to(torch.float32)[damage_count.clamp(0, 113).to(torch.int64)]
     return torch.stack((bonus / 255.0, flash / 255.0), dim=1).contiguous()
+
+
+def decal_inputs(serial, wall, along, impact_z, style, portal_walls, fine_sine_fixed):
+    """Pack the wall decals of every lane in paint order (engine.py:13756-13829).
+
+    ``serial, wall, along, impact_z, style`` are the engine's ``hitscan_decal_*`` tensors ``[N, slots]``
+    (serial < 0 = free slot), ``portal_walls`` the map's ``[W,4]`` linedefs and ``fine_sine_fixed`` the
+    8192-entry fine sine table (``fine_sine_fixed()``).  Returns ``(decal_state i32 [N,D,3], decal_geom
+    f32 [N,D,4])`` with D the largest number of live decals in a lane, or ``None`` when no lane has one.
+    Older impacts come first so that a later chip shades an earlier one at the same texels.
+    """
+
+    active_slots = torch.nonzero(torch.any(serial >= 0, dim=0)).flatten()
+    if not active_slots.numel():
+        return None
+    serial = serial[:, active_slots].to(torch.int64)
+    active = serial >= 0
+    layers = int(torch.amax(torch.sum(active, dim=1)).item())
+    order = torch.argsort(torch.where(active, serial, torch.full_like(serial, torch.iinfo(torch.int32).max)), dim=1)
+    order = order[:, :layers]
+    pick = lambda tensor: tensor[:, active_slots].gather(1, order)  # noqa: E731
+    alive = active.gather(1, order)
+    wall_index = pick(wall).to(torch.int64).clamp(0, portal_walls.shape[0] - 1)
+    style_index = pick(style).to(torch.int64)
+    side = style_index // 20
+    segment = portal_walls[wall_index]
+    vector = segment[..., 2:] - segment[..., :2]
+    # the seg runs backwards on sidedef 1; its direction goes through the fine-angle table
+    oriented = torch.where((side == 0)[..., None], vector, -vector)
+    angle = torch.atan2(oriented[..., 1], oriented[..., 0])
+    fine = torch.floor(torch.remainder(angle, 2.0 * math.pi) * (8192 / (2.0 * math.pi))).to(torch.int64) & 8191
+    table = torch.as_tensor(fine_sine_fixed, dtype=torch.int64).to(serial.device)
+    sine = table[fine].to(torch.float32) / 65536
+    cosine = table[(fine + 2048) & 8191].to(torch.float32) / 65536
+    state = torch.stack((wall_index, style_index, alive.to(torch.int64)), dim=-1).to(torch.int32).contiguous()
+    geom = torch.stack((pick(along).to(torch.float32), pick(impact_z).to(torch.float32), cosine, sine), dim=-1).contiguous()
+    return state, geom

@@ -50,6 +50,8 @@ class LaneState:
     hud_state: torch.Tensor | None = None  # i32 [N,9]
     sprite_style: torch.Tensor | None = None  # i8 [N,A]: -1 opaque, -2 translucent, >= 0 additive table
     screen_blend: torch.Tensor | None = None  # f32 [N,2] bonus / damage alphas (overlay_inputs.screen_blend)
+    decal_state: torch.Tensor | None = None  # i32 [N,D,3] packed wall decals (overlay_inputs.decal_inputs)
+    decal_geom: torch.Tensor | None = None  # f32 [N,D,4]
 
     @classmethod
     def from_numpy(cls, arrays: dict, device) -> "LaneState":
@@ -70,6 +72,7 @@ class LaneState:
             ray_sin=get("ray_sin", torch.float32), sprite_depth=get("sprite_depth", torch.float32),
             weapon_state=get("weapon_state", torch.int64), hud_state=get("hud_state", torch.int32),
             sprite_style=get("sprite_style", torch.int8), screen_blend=get("screen_blend", torch.float32),
+            decal_state=get("decal_state", torch.int32), decal_geom=get("decal_geom", torch.float32),
         )
 
 
@@ -196,6 +199,12 @@ class HipRenderer:
             desc.sprite_depth = _require(depth, "sprite_depth", torch.float32, (count, slots), device).data_ptr()
         if lanes.weapon_state is not None:
             desc.weapon_state = _require(lanes.weapon_state, "weapon_state", torch.int64, (count, 5), device).data_ptr()
+        desc.decal_slots = 0
+        if lanes.decal_state is not None and lanes.decal_state.shape[1] > 0:
+            slots = int(lanes.decal_state.shape[1])
+            desc.decal_slots = slots
+            desc.decal_state = _require(lanes.decal_state, "decal_state", torch.int32, (count, slots, 3), device).data_ptr()
+            desc.decal_geom = _require(lanes.decal_geom, "decal_geom", torch.float32, (count, slots, 4), device).data_ptr()
         if lanes.screen_blend is not None:
             desc.screen_blend = _require(lanes.screen_blend, "screen_blend", torch.float32, (count, 2), device).data_ptr()
         if lanes.hud_state is not None:

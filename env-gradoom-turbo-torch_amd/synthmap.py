@@ -702,9 +702,22 @@ def generate_overlays(seed: int, *, weapon_patches: int = 12, cooldowns: int = 8
     frame_ids = rng.integers(0, weapon_patches, (8, 2, cooldowns)).astype(np.int32)
     flash_ids = np.where(rng.random((8, 2, cooldowns)) < 0.4, rng.integers(0, weapon_patches, (8, 2, cooldowns)), -1).astype(np.int32)
     flash_lights = np.where(flash_ids >= 0, rng.integers(1, 3, (8, 2, cooldowns)), 0).astype(np.int64)
+    # bullet chip decals (scenario.py:370-375): five variants of one width, transparent where 0
+    dh, dw = 16, 12
+    decal_h = rng.integers(8, dh + 1, 5).astype(np.int32)
+    decal_atlas = np.zeros((5, dh, dw), dtype=np.uint8)
+    for v in range(5):
+        patch = rng.integers(1, 256, (int(decal_h[v]), dw), dtype=np.uint8)
+        patch[rng.random(patch.shape) < 0.25] = 0
+        decal_atlas[v, : decal_h[v]] = patch
+    decal_left = rng.integers(3, 9, 5).astype(np.int32)
+    decal_top = rng.integers(3, 12, 5).astype(np.int32)
+    decal_opacity_lut = rng.integers(0, 65, (32, 256), dtype=np.uint8)
+    decal_black_lut = rng.integers(0, 256, (65, 256), dtype=np.uint8)
     return dict(
         weapon_atlas=weapon_atlas, weapon_opaque=weapon_opaque, weapon_w=weapon_w, weapon_h=weapon_h,
         weapon_left=weapon_left, weapon_top=weapon_top, hud_atlas=hud_atlas, hud_opaque=hud_opaque, hud_w=hud_w,
         hud_h=hud_h, hud_left=hud_left, hud_top=hud_top, weapon_frame_ids=frame_ids, weapon_flash_ids=flash_ids,
-        weapon_flash_lights=flash_lights,
+        weapon_flash_lights=flash_lights, decal_atlas=decal_atlas, decal_h=decal_h, decal_left=decal_left,
+        decal_top=decal_top, decal_opacity_lut=decal_opacity_lut, decal_black_lut=decal_black_lut,
     )

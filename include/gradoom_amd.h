@@ -141,6 +141,7 @@ typedef struct gd_map_desc {
 typedef struct gd_lanes_desc {
     int32_t lane_count;       /* N */
     int32_t sprite_slots;     /* A sprites per lane (0 = none) */
+    int32_t decal_slots;      /* D packed wall decals per lane (0 = none) */
     const float *x, *y;       /* [N] */
     const float *angle;       /* [N] radians */
     const float *view_z;      /* [N] */
@@ -162,6 +163,13 @@ typedef struct gd_lanes_desc {
     const int32_t *hud_state;       /* [N,9] status bar of engine.py:15232-15267: ready ammo, health, armor,
                                        face patch id, owned weapon bits (bit k = weapon k+1, k < 5),
                                        four ammo counts */
+    /* Wall decals in paint order, oldest first (_native_render_hitscan_decals, engine.py:13747-13991; the
+       host sorts the active slots by serial, engine.py:13756-13776).  Drawn after the walls and before the
+       sprites when the renderer holds decal patches. */
+    const int32_t *decal_state;     /* [N,D,3] linedef index, style (variant + 5*flip_x + 10*flip_y + 20*side), alive */
+    const float *decal_geom;        /* [N,D,4] along the linedef 0..1, impact height, and the linedef's direction
+                                       on the decal's side quantised through the fine sine table: cos, sin
+                                       (engine.py:13822-13829) */
     const float *screen_blend;      /* [N,2] or NULL (no blend): bonus alpha min(bonus_count*8, 128)/255 and damage
                                        alpha damage_to_alpha[clamp(damage_count, 0, 113)]/255; PLAYPAL colours are
                                        mixed with gold and then red before the RGB24 frame and the observation
@@ -188,6 +196,13 @@ typedef struct gd_overlay_desc {
     const uint8_t *hud_atlas;       /* [Ph,Hh,Wh] */
     const uint8_t *hud_opaque;      /* [Ph,Hh,Wh] */
     const int32_t *hud_w, *hud_h, *hud_left, *hud_top;             /* [Ph] */
+    /* Bullet chip decals (map.bullet_decal_*, engine.py:690-695, 1038-1070); decal_variant_count 0 = none.
+       The reference indexes variants with style % 5, so a non-empty set has exactly 5. */
+    int32_t decal_variant_count, decal_max_h, decal_max_w, decal_black_rows;
+    const uint8_t *decal_atlas;        /* [5,Hd,Wd] 0 = transparent; every variant is Wd wide */
+    const int32_t *decal_h, *decal_left, *decal_top; /* [5] */
+    const uint8_t *decal_opacity_lut;  /* [32,256] colormap row x atlas value -> row of decal_black_lut */
+    const uint8_t *decal_black_lut;    /* [decal_black_rows,256] opacity x pixel under the decal -> pixel */
 } gd_overlay_desc;
 
 /* Output buffers; any pointer may be null to skip that product. */

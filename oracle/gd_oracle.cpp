@@ -1522,6 +1522,97 @@ struct Oracle {
     }
 };
 
+// _native_render_hitscan_decals (engine.py:13747-13991) for one lane: decals in paint order over the
+// wall pass's picture, each drawn only where the scene depth is the decal's own ray distance.
+void render_decals(Oracle &o, const gd_overlay_desc &ov, const gd_lanes_desc *lanes, int n) {
+    const gd_map_desc *m = o.m;
+    const Lane &L = o.L;
+    const int D = lanes->decal_slots;
+    const float focal_length = 192.0f;
+    const float center = 104.0f + L.pitch_offset;
+    const int width = ov.decal_max_w;
+    for (int k = 0; k < D; ++k) {
+        const int32_t *state = lanes->decal_state + (size_t(n) * D + k) * 3;
+        const float *geom = lanes->decal_geom + (size_t(n) * D + k) * 4;
+        const bool alive = state[2] != 0;
+        const int wall_index = int(clampi(state[0], 0, o.W - 1));
+        const int style = state[1];
+        const int variant = style % 5;
+        const bool flip_x = (style / 5) % 2, flip_y = (style / 10) % 2;
+        const int side = style / 20;
+        const float along_wall = geom[0], impact_z = geom[1], tangent_x = geom[2], tangent_y = geom[3];
+        const float *wl = m->walls + 4 * wall_index;
+        const float wvx = wl[2] - wl[0], wvy = wl[3] - wl[1];
+        const float impact_x = wl[0] + along_wall * wvx, impact_y = wl[1] + along_wall * wvy;
+        const float left_offset = float(ov.decal_left[variant]);
+        const float back = left_offset * 0.5f, forth = (float(width) - left_offset) * 0.5f;
+        const float left_x = impact_x - tangent_x * back, left_y = impact_y - tangent_y * back;
+        const float right_x = impact_x + tangent_x * forth, right_y = impact_y + tangent_y * forth;
+        const float seg_x = right_x - left_x, seg_y = right_y - left_y;
+        // FWallCoords::Init on the two fixed-point endpoints (engine.py:13836-13887)
+        i64 ex[2] = {round_to_i64(left_x * float(FIXED_UNIT)), round_to_i64(right_x * float(FIXED_UNIT))};
+        i64 ey[2] = {round_to_i64(left_y * float(FIXED_UNIT)), round_to_i64(right_y * float(FIXED_UNIT))};
+        i64 tx[2], ty[2];
+        for (int e = 0; e < 2; ++e) {
+            i64 rx = ex[e] - L.view_x_fixed, ry = ey[e] - L.view_y_fixed;
+            tx[e] = (rx * L.vsin - ry * L.vcos) >> 20;
+            ty[e] = (rx * L.vcos + ry * L.vsin) >> 20;
+        }
+        const i64 tx1 = tx[0], tx2 = tx[1], ty1 = ty[0], ty2 = ty[1];
+        const i64 center_fixed = 160 * FIXED_UNIT;
+        i64 projected_left = ((center_fixed + tdiv(tx1 * center_fixed, ty1 == 0 ? 1 : ty1)) >> 16) + (tx1 >= 0);
+        i64 projected_right = ((center_fixed + tdiv(tx2 * center_fixed, ty2 == 0 ? 1 : ty2)) >> 16) + (tx2 >= 0);
+        i64 left_den = tx1 - tx2 - ty2 + ty1, right_den = ty2 - ty1 - tx2 + tx1;
+        bool left_inside = (tx1 >= -ty1) && (tx1 <= ty1) && (ty1 != 0);
+        bool right_inside = (tx2 <= ty2) && (tx2 >= -ty2) && (ty2 != 0);
+        bool left_clipped = (tx1 < -ty1) && (tx2 >= -ty2) && (left_den != 0);
+        bool right_clipped = (tx2 > ty2) && (tx1 <= ty1) && (right_den != 0);
+        i64 screen_left = left_inside ? clampi(projected_left, 0, SW) : 0;
+        i64 screen_right = right_inside ? clampi(projected_right, 0, SW) : SW;
+        bool projected = alive && (left_inside || left_clipped) && (right_inside || right_clipped) && (screen_right > screen_left);
+        float viewer_cross = wvx * (L.y - wl[1]) - wvy * (L.x - wl[0]);
+        bool side_visible = (viewer_cross > 0 ? 1 : 0) == side;
+        int sector = m->wall_sectors[2 * wall_index + (side < 0 ? 0 : (side > 1 ? 1 : side))];
+        if (sector < 0) sector = 0;
+        bool horizontal = std::fabs(wvy) < 1e-6f, vertical = std::fabs(wvx) < 1e-6f;
+        float light = m->sector_lights[sector] + (vertical ? 16.0f : (horizontal ? -16.0f : 0.0f));
+        light = light + float(L.flash_light * 16);
+        const int height = ov.decal_h[variant];
+        const float top_offset = float(ov.decal_top[variant]);
+        if (!(projected && side_visible)) continue;
+        for (int x = 0; x < SW; ++x) {
+            float col = (float(x) - 160.0f) / 160.0f;
+            float rx = L.fcos + L.fsin * col, ry = L.fsin - L.fcos * col;
+            float off_x = left_x - L.x, off_y = left_y - L.y;
+            float den = rx * seg_y - ry * seg_x;
+            float safe = std::fabs(den) < 1e-6f ? 1.0f : den;
+            float distance = (off_x * seg_y - off_y * seg_x) / safe;
+            float decal_along = (off_x * ry - off_y * rx) / safe;
+            bool inside_column = (x >= screen_left) && (x < screen_right) && (std::fabs(den) >= 1e-6f) && (distance > 0);
+            if (!inside_column) continue;
+            i64 tu = clampi(i64(std::floor(decal_along * float(width))), 0, width - 1);
+            if (flip_x) tu = width - 1 - tu;
+            float safe_distance = std::max(distance, 1e-6f);
+            float vertical_scale = 96.0f / safe_distance;
+            float top = center - ((impact_z + top_offset * 0.5f) - L.view_z) * focal_length / safe_distance;
+            i64 depth_fixed = round_to_i64(safe_distance * 4096.0f);
+            i64 visibility = tdiv(WALL_VISIBILITY_FIXED << 12, std::max<i64>(depth_fixed, 1));
+            i64 shade = Oracle::wall_shade(light, visibility);
+            for (int y = 0; y < VH; ++y) {
+                i64 tv = i64(std::floor((float(y) - top) / vertical_scale));
+                if (!(tv >= 0 && tv < height)) continue;
+                if (flip_y) tv = height - 1 - tv;
+                size_t i = size_t(y) * SW + x;
+                if (!(std::fabs(o.scene_depth[i] - distance) <= 1e-3f)) continue;
+                uint8_t source = ov.decal_atlas[(size_t(variant) * ov.decal_max_h + tv) * ov.decal_max_w + tu];
+                if (source == 0) continue;
+                uint8_t opacity = ov.decal_opacity_lut[shade * 256 + source];
+                o.frame[i] = ov.decal_black_lut[size_t(opacity) * 256 + o.frame[i]];
+            }
+        }
+    }
+}
+
 // _policy_area_grayscale_kernel (_triton_kernels.py:120-177) for one lane
 // engine.py:15385-15397: PLAYPAL after the pickup (gold) and damage (red) screen blends, float32 op by op
 void blended_palette(const uint8_t *playpal, const float *blend, uint8_t *out) {
@@ -1756,6 +1847,8 @@ int gdo_render(const gd_map_desc *map, const gd_lanes_desc *lanes, const gd_fram
             if (dbg->walls_frame) std::memcpy(dbg->walls_frame, o.frame.data(), PX);
         }
         double t5 = now();
+        if (g_overlays_set && g_overlays.decal_variant_count > 0 && lanes->decal_slots > 0 && lanes->decal_state && lanes->decal_geom)
+            render_decals(o, g_overlays, lanes, n);
         o.render_sprites(lanes, n);
         double t6 = now();
         t_setup += t1 - t0; t_flats += t2 - t1; t_walls += t4 - t3; t_sprites += t6 - t5;

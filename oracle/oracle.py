@@ -98,6 +98,8 @@ def lanes_desc(lanes: dict):
     desc.lane_count = count
     sprite_x = lanes.get("sprite_x")
     desc.sprite_slots = 0 if sprite_x is None else int(np.asarray(sprite_x).shape[1])
+    decal_state = lanes.get("decal_state")
+    desc.decal_slots = 0 if decal_state is None else int(np.asarray(decal_state).shape[1])
     for name, dtype in _abi.LANE_ARRAYS:
         value = lanes.get(name)
         if value is None:

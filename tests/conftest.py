@@ -58,7 +58,7 @@ def load_fixture(name: str):
 LANE_KEYS = (
     "x", "y", "angle", "view_z", "x_fixed", "y_fixed", "angle_bam", "pitch_bam", "flash_light", "ray_cos", "ray_sin",
     "sprite_x", "sprite_y", "sprite_z", "sprite_depth", "sprite_id", "sprite_alive", "sprite_fullbright",
-    "weapon_state", "hud_state", "sprite_style", "screen_blend",
+    "weapon_state", "hud_state", "sprite_style", "screen_blend", "decal_state", "decal_geom",
 )
 
 

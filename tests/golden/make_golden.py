@@ -115,6 +115,12 @@ CASES = {
     "screen_flashes": dict(
         map_seed=12, grid=(5, 4), sectors=17, linedefs=100, lanes=4, pose_seed=6, sprites=16, screen_flashes=29
     ),
+    # Bullet chip decals on the linedefs the cameras look at (engine.py:13747-13991), under sprites, the weapon
+    # and the status bar; the reference's scene depth buffer and its picture right after the decal pass ride along.
+    "decals": dict(
+        map_seed=22, grid=(6, 5), sectors=26, linedefs=160, lanes=8, pose_seed=5, sprites=24, pitch=True, flash=True,
+        midtex=0.2, overlays=83, decals=17,
+    ),
     "config2_subset": dict(map_seed=1002, grid=(12, 9), sectors=96, linedefs=800, lanes=4, pose_seed=1, sprites=32),
     "config3_subset": dict(
         map_seed=1003, grid=(15, 15), sectors=200, linedefs=2000, lanes=2, pose_seed=1, sprites=64, flash=True
@@ -196,6 +202,18 @@ def build_case(name: str, cfg: dict, do_time: bool) -> dict:
             [engine._native_mugshot_patch_index(lane, int(engine.health[lane].clamp(0, 999).item())) for lane in range(lanes)],
             dtype=np.int64,
         )
+    if cfg.get("decals"):
+        refdrive.set_decals(engine, smap, cfg["decals"])
+        packed_decals = overlay_inputs.decal_inputs(
+            engine.hitscan_decal_serial, engine.hitscan_decal_wall, engine.hitscan_decal_along, engine.hitscan_decal_z,
+            engine.hitscan_decal_style, engine.map.portal_walls, overlay_inputs.fine_sine_fixed(),
+        )
+        data["decal_state"], data["decal_geom"] = (value.numpy() for value in packed_decals)
+        with torch.no_grad():
+            background = engine._render_native_background()
+            data["ref_scene_depth"] = background[1].numpy()
+            data["ref_decal_frame"] = engine._native_render_hitscan_decals(background[0], engine.view_z, background[1]).numpy()
+            data["ref_background_frame"] = background[0].numpy()
     if cfg.get("screen_flashes"):
         # pickup and damage counters as gameplay leaves them; lane 0 keeps both at zero (blend = identity)
         generator = torch.Generator().manual_seed(cfg["screen_flashes"])

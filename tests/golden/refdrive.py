@@ -71,6 +71,12 @@ def to_compiled_scenario(smap, *, flash_lights: bool = False, overlays: dict | N
             hud_patch_widths=overlays["hud_w"], hud_patch_heights=overlays["hud_h"],
             hud_patch_left_offsets=overlays["hud_left"], hud_patch_top_offsets=overlays["hud_top"],
         )
+        if overlays.get("decal_atlas") is not None:
+            kwargs.update(
+                bullet_decal_atlas=overlays["decal_atlas"], bullet_decal_heights=overlays["decal_h"],
+                bullet_decal_left_offsets=overlays["decal_left"], bullet_decal_top_offsets=overlays["decal_top"],
+                bullet_decal_opacity_lut=overlays["decal_opacity_lut"], bullet_decal_black_lut=overlays["decal_black_lut"],
+            )
     return scenario.CompiledScenario(
         scenario_sha256="s" * 64,
         iwad_sha256="i" * 64,
@@ -186,6 +192,55 @@ def set_sprites(engine, sprites, seed: int, effects=None):
     if effects is not None:
         set_effect_sprites(engine, effects, seed + 1)
     return packed_sprites(engine)
+
+
+def set_decals(engine, smap, seed: int, per_lane: int = 40):
+    """Bullet chips where rays from each camera meet the nearest linedef (engine.py:1868-1885 state).
+
+    Most chips face the camera, some sit on the far side; two share a spot so that the newer shades
+    the older; slots and serials are shuffled so that paint order differs from slot order.
+    """
+
+    rng = np.random.default_rng(seed)
+    lanes = engine.num_envs
+    segments = smap.wall_segments.astype(np.float64)
+    slots = engine.hitscan_decal_slots
+    for lane in range(lanes):
+        px, py, angle = float(engine.x[lane]), float(engine.y[lane]), float(engine.angle[lane])
+        view_z = float(engine.view_z[lane])
+        chips = []
+        for _ in range(per_lane):
+            theta = angle + rng.uniform(-0.7, 0.7)
+            dx, dy = np.cos(theta), np.sin(theta)
+            sx, sy = segments[:, 2] - segments[:, 0], segments[:, 3] - segments[:, 1]
+            ox, oy = segments[:, 0] - px, segments[:, 1] - py
+            den = dx * sy - dy * sx
+            safe = np.where(np.abs(den) < 1e-9, 1.0, den)
+            dist = (ox * sy - oy * sx) / safe
+            along = (ox * dy - oy * dx) / safe
+            hit = (np.abs(den) >= 1e-9) & (dist > 1.0) & (along >= 0.05) & (along <= 0.95)
+            if not hit.any():
+                continue
+            w = int(np.argmin(np.where(hit, dist, np.inf)))
+            cross = sx[w] * (py - segments[w, 1]) - sy[w] * (px - segments[w, 0])
+            side = 1 if cross > 0 else 0
+            if smap.wall_sectors[w, 1] < 0:
+                side = 0 if rng.random() < 0.9 else 1 - side * 0  # one-sided linedefs only have side 0
+            elif rng.random() < 0.15:
+                side = 1 - side
+            style = int(rng.integers(0, 5)) + 5 * int(rng.integers(0, 2)) + 10 * int(rng.integers(0, 2)) + 20 * side
+            chips.append((w, float(along[w]), view_z + float(rng.uniform(-35.0, 45.0)), style))
+        if chips:
+            w, a, z, style = chips[0]
+            chips.append((w, a + 0.004, z + 1.5, (style // 20) * 20 + int(rng.integers(0, 20))))
+        chosen = rng.choice(slots, size=len(chips), replace=False)
+        serials = rng.permutation(len(chips)) + int(rng.integers(0, 1000))
+        for (w, a, z, style), slot, serial in zip(chips, chosen, serials):
+            engine.hitscan_decal_wall[lane, slot] = w
+            engine.hitscan_decal_along[lane, slot] = a
+            engine.hitscan_decal_z[lane, slot] = z
+            engine.hitscan_decal_style[lane, slot] = style
+            engine.hitscan_decal_serial[lane, slot] = int(serial)
 
 
 def set_effect_sprites(engine, sprites, seed: int):

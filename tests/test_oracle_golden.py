@@ -91,3 +91,15 @@ def test_screen_flashes_blend_the_palette_per_lane(oracle):
     playpal = tables["playpal"].reshape(256, 3)
     assert np.array_equal(result["rgb"][0], playpal[result["indexed"][0]])
     assert not np.array_equal(result["rgb"][2], playpal[result["indexed"][2]])
+
+
+def test_scene_depth_under_the_decals_matches_the_reference(oracle):
+    """Decals are drawn where |scene depth - decal distance| <= 1e-3 (engine.py:13930-13933), so the depth
+    buffer itself has to be the reference's, bit for bit, on every kind of pixel."""
+
+    _meta, data, _smap, tables = load_fixture("decals")
+    for lane in (0, 3, 7):
+        taps = oracle.render(tables, lane_inputs(data), data["cosine_correction"], lane_range=(lane, lane + 1), debug_lane=lane)["debug"]
+        ours, ref = np.asarray(taps["scene_depth"]), data["ref_scene_depth"][lane]
+        assert np.array_equal(ours, ref)
+        assert np.isfinite(ref).mean() > 0.9
