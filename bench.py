@@ -5,7 +5,8 @@
 A step is one pass of the whole hot path over one batch of lanes whose inputs already sit in
 HBM: sector-light flicker update, the Torch float32 ray / sprite-depth tables, the render
 kernel chain and the fused observation + frame-stack update.  Camera poses and sprite lists
-change every step.  One JSON line is printed (see README of the contract in DESIGN.md).
+change every step.  One JSON line is printed: metric, value, timing, the roofline of the slowest
+kernel (algorithmic bytes over its launch duration, measured here with HIP events) and a CPU baseline.
 """
 
 from __future__ import annotations
