@@ -29,7 +29,7 @@ POSE_SETS = 4
 # of a 4096-lane launch, each scaled by what the same counter reads for a 1 GiB copy
 # (profiles/render_chain_config4_4096lanes.md).  Measured offline; other workloads report null.
 MEASURED_TRAFFIC_PER_LANE = {
-    ("config4", "wall_columns"): 1.442e10 / 4096,
+    ("config4", "wall_columns"): 1.461e10 / 4096,
     ("config4", "flat_select"): 1.002e9 / 4096,
 }
 
@@ -56,7 +56,7 @@ def main() -> int:
                         help="full: indexed frame + observation stack (the headline metric); obs-only: observation stack "
                              "only, no 320x240 frame handed to the caller; rgb: indexed + RGB24 frame, no observation")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    parser.add_argument("--cpu-lanes", type=int, default=12, help="lanes of the same workload the CPU baseline renders")
+    parser.add_argument("--cpu-lanes", type=int, default=32, help="lanes of the same workload the CPU baseline renders")
     parser.add_argument("--copy-probe-mib", type=int, default=0,
                         help="after the timed region, copy this many MiB device to device once (a kernel of known "
                              "traffic that scales the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
