@@ -1053,11 +1053,13 @@ struct FragmentChoice {
     const WallRec *rec;
     bool has, lights;
 };
+// SPLIT is false for maps without split linedefs, whose kernels then carry none of the search.
+template <bool SPLIT>
 __device__ __forceinline__ FragmentChoice choose_fragment(const gd_map_desc *m, const WallRec *frags, const WallRec &whole, int w, int x) {
     FragmentChoice f;
     f.rec = &whole; f.lights = false;
     f.has = (whole.sr > whole.sl) && (x >= whole.sl) && (x < whole.sr);
-    if (whole.flags & WF_SPLIT) {
+    if (SPLIT && (whole.flags & WF_SPLIT)) {
         const int F = m->fragment_slots, row = m->wall_split_slot[w];
         int count = 0;
         f.has = false;
@@ -1299,6 +1301,7 @@ __device__ __forceinline__ void take_min(float v, int w, float &best, int &best_
 }
 
 // engine.py:11769-12636: selection of the pass's drawseg for one column
+template <bool SPLIT>
 __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnState &c, bool boundary_has_po, PassColumn &r) {
     const gd_map_desc *m = cc.m;
     const MapView &mv = cc.mv;
@@ -1472,7 +1475,7 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
     r.wall = wi; r.side = side; r.render_current = render_current; r.other_sector = other_sector;
     r.distance = distance;
     const WallRec &wr = cc.recs[wi];
-    const FragmentChoice wr_fragment = choose_fragment(m, cc.frags, wr, wi, x);
+    const FragmentChoice wr_fragment = choose_fragment<SPLIT>(m, cc.frags, wr, wi, x);
     r.visibility = wall_visibility(wr_fragment.lights ? *wr_fragment.rec : wr, side, x);
     const Tables &tb = *cc.tb;
     r.view_floor = tb.floor_h(render_current); r.view_ceiling = tb.ceil_h(render_current);
@@ -1700,6 +1703,7 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
 }
 
 // engine.py:12885-13371
+template <bool SPLIT>
 __device__ __forceinline__ bool pass_advance(const ColumnCtx &cc, ColumnState &c, const PassColumn &r, PixelBuffers &pb, SilhouetteBounds &sb) {
     const gd_map_desc *m = cc.m;
     const MapView &mv = cc.mv;
@@ -1732,7 +1736,7 @@ __device__ __forceinline__ bool pass_advance(const ColumnCtx &cc, ColumnState &c
     if (r.bits & PB_PS_KEEPS) {
         int path = r.ps_path_index;
         const WallRec &pr = cc.recs[path];
-        const FragmentChoice pr_fragment = choose_fragment(m, cc.frags, pr, path, x);
+        const FragmentChoice pr_fragment = choose_fragment<SPLIT>(m, cc.frags, pr, path, x);
         int path_safe_other = r.ps_other < 0 ? 0 : r.ps_other;
         const Tables &tb = *cc.tb;
         float pof = tb.floor_h(path_safe_other), poc = tb.ceil_h(path_safe_other);
@@ -1867,7 +1871,7 @@ __device__ __forceinline__ bool pass_advance(const ColumnCtx &cc, ColumnState &c
 }
 
 // engine.py:13424-13744 for one column
-template <bool DEPTH>
+template <bool DEPTH, bool SPLIT>
 __device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const ColumnState &c, PixelBuffers &pb) {
     const gd_map_desc *m = cc.m;
     const MapView &mv = cc.mv;
@@ -1895,7 +1899,7 @@ __device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const Col
     bool has_saved = c.masked_wall == mw;
     if (!(has_saved || left_edge)) return;
     const WallRec &wr = cc.recs[mw];
-    const FragmentChoice wr_fragment = choose_fragment(m, cc.frags, wr, mw, x);
+    const FragmentChoice wr_fragment = choose_fragment<SPLIT>(m, cc.frags, wr, mw, x);
     int front_sector = mv.sec(mw, 0), back_sector = mv.sec(mw, 1) < 0 ? 0 : mv.sec(mw, 1);
     int light_sector = mside == 0 ? front_sector : back_sector;
     const Tables &tb = *cc.tb;
@@ -2022,8 +2026,9 @@ __global__ void __launch_bounds__(1024) strip_order_kernel(int strips, Scratch s
 // otherwise fill the register file with three, and the flat kernels on the side stream could not
 // run beside it at all.
 #define WALL_LDS_PAD 3072
-// DEPTH: also keep the depth of every wall pixel (frames that draw decals).
-template <bool DEPTH>
+// DEPTH: also keep the depth of every wall pixel (frames that draw decals).  SPLIT: the map has linedefs with
+// BSP projection fragments.
+template <bool DEPTH, bool SPLIT>
 __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amdgpu_waves_per_eu(3, 3))) wall_columns_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
     const gd_map_desc *m = &dm.d;
     __shared__ LaneCtx lane_ctxs[WALL_STRIPS_PER_GROUP];
@@ -2083,7 +2088,7 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
 #ifdef GD_PROFILE
         prof_acc[7] += 1;
 #endif
-        if (!done) pass_select(cc, st, boundary_has_po, pc);
+        if (!done) pass_select<SPLIT>(cc, st, boundary_has_po, pc);
         PROF_T(t1);
         PROF_ADD(0, t0, t1);
         // 4-column wallscan groups (engine.py:12688-12761): exchange with the aligned neighbours
@@ -2111,7 +2116,7 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
             pass_paint<DEPTH>(cc, st, pc, pb, group_valid, common_bottom, first_group_visibility, colormap_lds, window_dirty);
             PROF_T(t3);
             PROF_ADD(1, t2, t3);
-            bool changed = pass_advance(cc, st, pc, pb, sb);
+            bool changed = pass_advance<SPLIT>(cc, st, pc, pb, sb);
             PROF_T(t4);
             PROF_ADD(2, t3, t4);
 #ifdef GD_PROFILE
@@ -2124,7 +2129,7 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
     }
     PROF_T(t5);
     PROF_T(t6);
-    masked_midtexture<DEPTH>(cc, st, pb);
+    masked_midtexture<DEPTH, SPLIT>(cc, st, pb);
 #ifdef GD_PROFILE
     long long t7 = wall_clock64();
     int prof_cands = cc.count;
@@ -2876,8 +2881,10 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     if (overlap) HIP_TRY(hipEventRecord(r->flat_event, side));
     {
         const dim3 grid((count * (SW / 64) + WALL_STRIPS_PER_GROUP - 1) / WALL_STRIPS_PER_GROUP), block(64 * WALL_STRIPS_PER_GROUP);
-        if (decals) hipLaunchKernelGGL(wall_columns_kernel<true>, grid, block, WALL_LDS_PAD, stream, r->dm, count, sc, frame_base, frame_stride);
-        else hipLaunchKernelGGL(wall_columns_kernel<false>, grid, block, WALL_LDS_PAD, stream, r->dm, count, sc, frame_base, frame_stride);
+        const bool split = m.split_count > 0;
+        auto kernel = decals ? (split ? wall_columns_kernel<true, true> : wall_columns_kernel<true, false>)
+                             : (split ? wall_columns_kernel<false, true> : wall_columns_kernel<false, false>);
+        hipLaunchKernelGGL(kernel, grid, block, WALL_LDS_PAD, stream, r->dm, count, sc, frame_base, frame_stride);
     }
     mark();
     if (overlap) HIP_TRY(hipStreamWaitEvent(stream, r->flat_event, 0));
