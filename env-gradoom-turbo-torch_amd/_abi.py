@@ -242,3 +242,116 @@ def host_map_desc(tables: dict) -> tuple[MapDesc, list]:
         keep.append(array)
         setattr(desc, name, array.ctypes.data)
     return desc, keep
+
+
+ACTOR_SCALARS = (
+    "lane_count",
+    "enemy_slots",
+    "doll_count",
+    "player_projectile_slots",
+    "enemy_projectile_slots",
+    "fog_slots",
+    "puff_slots",
+    "item_count",
+    "drop_slots",
+    "attack_frames",
+    "death_frames",
+    "xdeath_frames",
+    "explosion_frames",
+)
+ACTOR_ARRAYS = (
+    ("enemy_x", np.float32),
+    ("enemy_y", np.float32),
+    ("enemy_z", np.float32),
+    ("enemy_alive", np.uint8),
+    ("enemy_type", np.int64),
+    ("enemy_rotation", np.uint8),
+    ("enemy_animation_tics", np.int32),
+    ("enemy_target_slot", np.int64),
+    ("enemy_attack_phase", np.int32),
+    ("enemy_cooldown", np.int32),
+    ("enemy_pain_tics", np.int32),
+    ("enemy_death_tics", np.int32),
+    ("enemy_death_type", np.int64),
+    ("enemy_death_elapsed", np.int32),
+    ("enemy_death_extreme", np.uint8),
+    ("doll_x", np.float32),
+    ("doll_y", np.float32),
+    ("doll_z", np.float32),
+    ("doll_rotation", np.uint8),
+    ("player_dead", np.uint8),
+    ("projectile_x", np.float32),
+    ("projectile_y", np.float32),
+    ("projectile_z", np.float32),
+    ("projectile_alive", np.uint8),
+    ("projectile_type", np.int64),
+    ("projectile_age", np.int32),
+    ("projectile_rotation", np.uint8),
+    ("projectile_impact_type", np.int64),
+    ("projectile_impact_tics", np.int32),
+    ("enemy_projectile_x", np.float32),
+    ("enemy_projectile_y", np.float32),
+    ("enemy_projectile_z", np.float32),
+    ("enemy_projectile_alive", np.uint8),
+    ("enemy_projectile_age", np.int32),
+    ("enemy_projectile_rotation", np.uint8),
+    ("enemy_projectile_impact_tics", np.int32),
+    ("teleport_fog_x", np.float32),
+    ("teleport_fog_y", np.float32),
+    ("teleport_fog_z", np.float32),
+    ("teleport_fog_tics", np.int32),
+    ("hitscan_puff_x", np.float32),
+    ("hitscan_puff_y", np.float32),
+    ("hitscan_puff_z", np.float32),
+    ("hitscan_puff_tics", np.int32),
+    ("item_x", np.float32),
+    ("item_y", np.float32),
+    ("item_z", np.float32),
+    ("item_types", np.int64),
+    ("item_raw_visual_types", np.int64),
+    ("item_available", np.uint8),
+    ("item_animation_initial_tics", np.int32),
+    ("episode_time", np.int32),
+    ("drop_x", np.float32),
+    ("drop_y", np.float32),
+    ("drop_z", np.float32),
+    ("drop_type", np.int64),
+    ("drop_spawned", np.uint8),
+    ("enemy_walk_frame_tics", np.int32),
+    ("enemy_idle_frame_tics", np.int32),
+    ("enemy_attack_recovery", np.int32),
+    ("enemy_walk_sprite_ids", np.int64),
+    ("enemy_attack_sprite_ids", np.int64),
+    ("enemy_pain_sprite_ids", np.int64),
+    ("enemy_death_sprite_ids", np.int64),
+    ("enemy_death_frame_durations", np.int64),
+    ("enemy_death_frame_counts", np.int64),
+    ("enemy_xdeath_sprite_ids", np.int64),
+    ("enemy_xdeath_frame_durations", np.int64),
+    ("enemy_xdeath_frame_counts", np.int64),
+    ("projectile_explosion_total_tics", np.int64),
+    ("projectile_explosion_frame_durations", np.int64),
+    ("projectile_explosion_frame_counts", np.int64),
+    ("raw_projectile_explosion_sprite_ids", np.int64),
+    ("raw_projectile_flight_sprite_ids", np.int64),
+    ("raw_teleport_fog_sprite_ids", np.int64),
+    ("raw_bullet_puff_sprite_ids", np.int64),
+    ("raw_static_sprite_ids", np.int64),
+    ("raw_item_animation_sprite_ids", np.int64),
+)
+ACTOR_OUTPUTS = (
+    ("sprite_x", np.float32),
+    ("sprite_y", np.float32),
+    ("sprite_z", np.float32),
+    ("sprite_id", np.int32),
+    ("sprite_alive", np.uint8),
+    ("sprite_fullbright", np.uint8),
+    ("sprite_style", np.int8),
+)
+
+
+class ActorDesc(C.Structure):
+    _fields_ = (
+        [(name, C.c_int32) for name in ACTOR_SCALARS] + [(name, _P) for name, _ in ACTOR_ARRAYS]
+        + [(name, _P) for name, _ in ACTOR_OUTPUTS]
+    )

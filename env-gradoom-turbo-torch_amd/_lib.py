@@ -23,6 +23,7 @@ SYMBOLS = (
     "gd_render_timed",
     "gd_observe",
     "gd_expand_rgb24",
+    "gd_pack_actors",
 )
 
 _LIBRARY = None
@@ -63,6 +64,8 @@ def library() -> C.CDLL:
     lib.gd_observe.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]
     lib.gd_expand_rgb24.restype = C.c_int
     lib.gd_expand_rgb24.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p]
+    lib.gd_pack_actors.restype = C.c_int
+    lib.gd_pack_actors.argtypes = [C.POINTER(_abi.ActorDesc), C.c_void_p]
     _LIBRARY = lib
     return lib
 

@@ -2733,6 +2733,145 @@ __global__ void expand_rgb_kernel(const unsigned char *indexed, const unsigned c
 }
 
 // ---------------------------------------------------------------------------------------------
+// actor packing: engine.py:14328-14682 with the sprite-id helpers of 14011-14136 and 14258-14317
+// ---------------------------------------------------------------------------------------------
+// Index of the animation frame showing after `elapsed` tics: the number of frames whose running end has
+// passed, held on the last one (engine.py:14084-14091, 14117-14122).
+__device__ __forceinline__ int frame_after(i64 elapsed, const int64_t *durations, int frames, i64 count) {
+    i64 end = 0; int frame = 0;
+    for (int k = 0; k < frames; ++k) { end += durations[k]; frame += elapsed >= end ? 1 : 0; }
+    const i64 last = count - 1;
+    return (int)(frame < last ? frame : last);
+}
+
+__device__ __forceinline__ i64 clamp_type(i64 v, i64 hi) { return v < 0 ? 0 : (v > hi ? hi : v); }
+
+__device__ __forceinline__ i64 explosion_patch(const gd_actor_desc &a, i64 kind, i64 remaining) {
+    kind = clamp_type(kind, 2);
+    const int F = a.explosion_frames;
+    const i64 elapsed = a.projectile_explosion_total_tics[kind] - remaining;
+    const int frame = frame_after(elapsed, a.projectile_explosion_frame_durations + kind * F, F, a.projectile_explosion_frame_counts[kind]);
+    return a.raw_projectile_explosion_sprite_ids[kind * F + frame];
+}
+
+__global__ void __launch_bounds__(64) pack_actors_kernel(gd_actor_desc a, int width) {
+    const int slot = blockIdx.x * blockDim.x + threadIdx.x;
+    const int n = blockIdx.y;
+    if (slot >= width || n >= a.lane_count) return;
+    float x = 0, y = 0, z = 0; i64 patch = 0; bool alive = false, bright = false; int style = -1;
+    int k = slot;
+    const int Se = a.enemy_slots, Sd = a.doll_count, Sp = a.player_projectile_slots, Sq = a.enemy_projectile_slots;
+    if (k < Se) {                                   // monsters (engine.py:14011-14077, 14125-14136)
+        const size_t i = (size_t)n * Se + k;
+        x = a.enemy_x[i]; y = a.enemy_y[i]; z = a.enemy_z[i]; alive = a.enemy_alive[i] != 0;
+        const i64 kind = clamp_type(a.enemy_type[i], 5);
+        const int facing = a.enemy_rotation[i];
+        const int tics = a.enemy_animation_tics[i];
+        int walking = (tics / a.enemy_walk_frame_tics[kind]) % 4;
+        int idling = (tics / a.enemy_idle_frame_tics[kind]) % 2;
+        if (kind == 2) idling = 0;
+        if (a.enemy_target_slot[i] < -1) walking = idling;
+        const int phase = a.enemy_attack_phase[i], cooldown = a.enemy_cooldown[i];
+        const bool recovering = cooldown > a.enemy_attack_recovery[kind] / 2;
+        const bool hitscanner = kind == 0 || kind == 1, melee = kind == 4 || kind == 5;
+        int attacking = 0;
+        if (hitscanner && phase == 2) attacking = recovering ? 1 : 0;
+        if (melee && phase == 1) attacking = cooldown <= 8 ? 1 : 0;
+        if (melee && phase == 2) attacking = 2;
+        if (kind == 3 && (phase == 4 || phase == 2)) attacking = 1;
+        if (kind == 3 && phase == 3) attacking = 2;
+        patch = phase > 0 ? a.enemy_attack_sprite_ids[(kind * a.attack_frames + attacking) * 8 + facing]
+                          : a.enemy_walk_sprite_ids[(kind * 4 + walking) * 8 + facing];
+        if (a.enemy_pain_tics[i] > 0) patch = a.enemy_pain_sprite_ids[kind * 8 + facing];
+        bright = (kind == 1 && phase == 2 && recovering) || (kind == 3 && (phase == 2 || phase == 3));
+    } else if ((k -= Se) < Sd) {                    // the other players' start dolls (engine.py:14345-14379)
+        x = a.doll_x[k]; y = a.doll_y[k]; z = a.doll_z[k]; alive = a.player_dead[n] == 0;
+        patch = a.enemy_walk_sprite_ids[(2 * 4 + 0) * 8 + a.doll_rotation[(size_t)n * Sd + k]];
+    } else if ((k -= Sd) < Se) {                    // corpses (engine.py:14079-14106)
+        const size_t i = (size_t)n * Se + k;
+        x = a.enemy_x[i]; y = a.enemy_y[i]; z = a.enemy_z[i]; alive = a.enemy_death_tics[i] > 0;
+        const i64 kind = clamp_type(a.enemy_death_type[i], 5);
+        const i64 elapsed = a.enemy_death_elapsed[i];
+        if (a.enemy_death_extreme[i]) {
+            const int F = a.xdeath_frames;
+            patch = a.enemy_xdeath_sprite_ids[kind * F + frame_after(elapsed, a.enemy_xdeath_frame_durations + kind * F, F, a.enemy_xdeath_frame_counts[kind])];
+        } else {
+            const int F = a.death_frames;
+            patch = a.enemy_death_sprite_ids[kind * F + frame_after(elapsed, a.enemy_death_frame_durations + kind * F, F, a.enemy_death_frame_counts[kind])];
+        }
+    } else if ((k -= Se) < Sp) {                    // rockets and plasma balls in flight (engine.py:14410-14460)
+        const size_t i = (size_t)n * Sp + k;
+        x = a.projectile_x[i]; y = a.projectile_y[i]; z = a.projectile_z[i]; alive = a.projectile_alive[i] != 0;
+        const i64 shot = clamp_type(a.projectile_type[i], 1);
+        const int frame = shot == 1 ? (a.projectile_age[i] / 6) % 2 : 0;
+        patch = a.raw_projectile_flight_sprite_ids[(shot * 2 + frame) * 8 + a.projectile_rotation[i]];
+        bright = alive; style = shot == 1 ? 0 : -1;
+    } else if ((k -= Sp) < Sq) {                    // monster fireballs in flight (engine.py:14462-14510)
+        const size_t i = (size_t)n * Sq + k;
+        x = a.enemy_projectile_x[i]; y = a.enemy_projectile_y[i]; z = a.enemy_projectile_z[i]; alive = a.enemy_projectile_alive[i] != 0;
+        const int frame = (a.enemy_projectile_age[i] / 4) % 2;
+        patch = a.raw_projectile_flight_sprite_ids[(2 * 2 + frame) * 8 + a.enemy_projectile_rotation[i]];
+        bright = alive; style = 1;
+    } else if ((k -= Sq) < Sp) {                    // the player's explosions (engine.py:14512-14541)
+        const size_t i = (size_t)n * Sp + k;
+        x = a.projectile_x[i]; y = a.projectile_y[i]; z = a.projectile_z[i]; alive = a.projectile_impact_tics[i] > 0;
+        patch = explosion_patch(a, a.projectile_impact_type[i], a.projectile_impact_tics[i]);
+        bright = alive; style = a.projectile_impact_type[i] == 1 ? 0 : -1;
+    } else if ((k -= Sp) < Sq) {                    // fireball explosions (engine.py:14543-14573)
+        const size_t i = (size_t)n * Sq + k;
+        x = a.enemy_projectile_x[i]; y = a.enemy_projectile_y[i]; z = a.enemy_projectile_z[i]; alive = a.enemy_projectile_impact_tics[i] > 0;
+        patch = explosion_patch(a, 2, a.enemy_projectile_impact_tics[i]);
+        bright = alive; style = 1;
+    } else if ((k -= Sq) < a.fog_slots) {           // teleport fog: 12 frames of 6 tics out of 72 (engine.py:14577-14595)
+        const size_t i = (size_t)n * a.fog_slots + k;
+        x = a.teleport_fog_x[i]; y = a.teleport_fog_y[i]; z = a.teleport_fog_z[i];
+        const int tics = a.teleport_fog_tics[i];
+        alive = tics > 0;
+        const int elapsed = 72 - tics;
+        int frame = elapsed >= 0 ? elapsed / 6 : -((-elapsed + 5) / 6);   // floor division, like Torch's //
+        if (frame > 11) frame = 11;
+        if (frame < 0) frame += 12;                                      // a negative index counts from the end
+        patch = a.raw_teleport_fog_sprite_ids[frame];
+        bright = alive; style = 1;
+    } else if ((k -= a.fog_slots) < a.puff_slots) { // bullet puffs: 4 frames of 4 tics (engine.py:14597-14630)
+        const size_t i = (size_t)n * a.puff_slots + k;
+        x = a.hitscan_puff_x[i]; y = a.hitscan_puff_y[i]; z = a.hitscan_puff_z[i];
+        const int tics = a.hitscan_puff_tics[i];
+        alive = tics > 0;
+        const int frame = tics > 12 ? 0 : (tics > 8 ? 1 : (tics > 4 ? 2 : 3));
+        patch = a.raw_bullet_puff_sprite_ids[frame];
+        bright = frame == 0; style = -2;
+    } else if ((k -= a.puff_slots) < a.item_count) {   // map items (engine.py:14258-14317, 14632-14655)
+        const size_t i = (size_t)n * a.item_count + k;
+        x = a.item_x[k]; y = a.item_y[k]; z = a.item_z[k]; alive = a.item_available[i] != 0;
+        const i64 kind = a.item_types[k];
+        const i64 elapsed = (i64)a.episode_time[n] + (6 - (i64)a.item_animation_initial_tics[i]);
+        const i64 sixth = elapsed >= 0 ? elapsed / 6 : -((-elapsed + 5) / 6);
+        const int phase = (int)(((sixth % 6) + 6) % 6);
+        const int swing = phase == 0 ? -1 : (phase <= 3 ? phase - 1 : 5 - phase);   // A, then B C D C B
+        patch = a.item_raw_visual_types[k];
+        if (kind == 2014 && swing >= 0) patch = a.raw_item_animation_sprite_ids[swing];
+        if (kind == 2015 && swing >= 0) patch = a.raw_item_animation_sprite_ids[3 + swing];
+        const bool green = kind == 2018 && (((elapsed % 13) + 13) % 13) >= 6;
+        const bool blue = kind == 2019 && (((elapsed % 12) + 12) % 12) >= 6;
+        if (green) patch = a.raw_item_animation_sprite_ids[6];
+        if (blue) patch = a.raw_item_animation_sprite_ids[7];
+        bright = green || blue;
+    } else {                                        // what monsters drop (engine.py:14657-14682)
+        k -= a.item_count;
+        const size_t i = (size_t)n * a.drop_slots + k;
+        x = a.drop_x[i]; y = a.drop_y[i]; z = a.drop_z[i];
+        const i64 kind = a.drop_type[i];
+        alive = kind >= 0 && a.drop_spawned[i] != 0;
+        patch = a.raw_static_sprite_ids[kind == 2002 ? 14 : (kind == 2007 ? 6 : 12)];
+    }
+    const size_t out = (size_t)n * width + slot;
+    a.sprite_x[out] = x; a.sprite_y[out] = y; a.sprite_z[out] = z;
+    a.sprite_id[out] = (int)patch;
+    a.sprite_alive[out] = alive ? 1 : 0; a.sprite_fullbright[out] = bright ? 1 : 0; a.sprite_style[out] = (signed char)style;
+}
+
+// ---------------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------------
 thread_local std::string g_error;
@@ -3277,6 +3416,31 @@ int gd_expand_rgb24(const uint8_t *indexed, int32_t rows, const uint8_t *playpal
         hipLaunchKernelGGL(expand_rgb_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
                            indexed + base, playpal, count, rgb + base * 3, nullptr, (size_t)1);
     }
+    HIP_TRY(hipGetLastError());
+    return GD_OK;
+}
+
+int gd_pack_actors(const gd_actor_desc *a, void *stream) {
+    if (!a) return fail(GD_E_ARG, "null argument");
+    const int32_t counts[] = {a->lane_count, a->enemy_slots, a->doll_count, a->player_projectile_slots, a->enemy_projectile_slots,
+                              a->fog_slots, a->puff_slots, a->item_count, a->drop_slots};
+    for (int32_t v : counts) if (v < 0) return fail(GD_E_ARG, "negative count");
+    if (a->attack_frames < 3 || a->death_frames < 1 || a->xdeath_frames < 1 || a->explosion_frames < 1)
+        return fail(GD_E_ARG, "animation tables need at least 3 attack frames and 1 frame of every other kind");
+    // every pointer of the descriptor sits between the scalars and the end of the struct
+    const void *const *first = reinterpret_cast<const void *const *>(&a->enemy_x);
+    const void *const *last = reinterpret_cast<const void *const *>(&a->sprite_style);
+    for (const void *const *p = first; p <= last; ++p) {
+        const bool doll = p >= reinterpret_cast<const void *const *>(&a->doll_x) && p <= reinterpret_cast<const void *const *>(&a->doll_rotation);
+        const bool item = p >= reinterpret_cast<const void *const *>(&a->item_x) && p <= reinterpret_cast<const void *const *>(&a->item_animation_initial_tics);
+        if (!*p && !(doll && a->doll_count == 0) && !(item && a->item_count == 0)) return fail(GD_E_ARG, "null tensor in gd_actor_desc");
+    }
+    const long long width = 2LL * a->enemy_slots + a->doll_count + 2LL * a->player_projectile_slots + 2LL * a->enemy_projectile_slots +
+                            a->fog_slots + a->puff_slots + a->item_count + a->drop_slots;
+    if (a->lane_count == 0 || width == 0) return GD_OK;
+    if (width > 65535 * 64LL || a->lane_count > 65535) return fail(GD_E_ARG, "too many slots or lanes for one launch");
+    hipLaunchKernelGGL(pack_actors_kernel, dim3((unsigned)((width + 63) / 64), (unsigned)a->lane_count), dim3(64), 0,
+                       static_cast<hipStream_t>(stream), *a, (int)width);
     HIP_TRY(hipGetLastError());
     return GD_OK;
 }

@@ -286,6 +286,114 @@ int gd_expand_rgb24(const uint8_t *indexed, int32_t rows, const uint8_t *playpal
                     uint8_t *rgb, void *stream);
 
 /*
+ * Gameplay state -> packed billboard list, one thread per (lane, slot), nothing trimmed, no host round trip.
+ * Replaces the list building at the head of _native_render_sprites (engine.py:14328-14682) with its helpers
+ * _native_enemy_sprite_ids, _native_enemy_death_sprite_ids, _native_projectile_explosion_sprite_ids,
+ * _native_enemy_fullbright and _native_item_sprite_ids (engine.py:14011-14136, 14258-14317): the same kinds of
+ * actor in the same order, every slot kept and unused ones marked dead instead of the per-kind nonzero() trims
+ * (list order breaks ties between equally distant sprites and is unchanged by trimming).  All pointers are
+ * DEVICE pointers to the engine's own tensors (bool tensors as bytes); fields are the engine / map attributes of
+ * the same names.  The *_rotation arrays are _doom_sprite_rotation (engine.py:13994-14009) of the camera-to-actor
+ * angle and the actor's heading, which the host evaluates with the reference's own float32 Torch ops (atan2).
+ * Output width A = 2 * enemy_slots + doll_count + 2 * player_projectile_slots + 2 * enemy_projectile_slots +
+ * fog_slots + puff_slots + item_count + drop_slots, in the order: monsters, dolls, corpses, player projectiles in
+ * flight, fireballs in flight, player explosions, fireball explosions, teleport fog, bullet puffs, map items,
+ * drops.  Returns GD_E_ARG for a null pointer or a negative count.
+ */
+typedef struct gd_actor_desc {
+    int32_t lane_count, enemy_slots, doll_count, player_projectile_slots, enemy_projectile_slots, fog_slots, puff_slots,
+        item_count, drop_slots, attack_frames, death_frames, xdeath_frames, explosion_frames;
+    const float *enemy_x;  /* [N,Se] */
+    const float *enemy_y;
+    const float *enemy_z;
+    const uint8_t *enemy_alive;  /* bool */
+    const int64_t *enemy_type;
+    const uint8_t *enemy_rotation;  /* 0..7, see above */
+    const int32_t *enemy_animation_tics;
+    const int64_t *enemy_target_slot;
+    const int32_t *enemy_attack_phase;
+    const int32_t *enemy_cooldown;
+    const int32_t *enemy_pain_tics;
+    const int32_t *enemy_death_tics;
+    const int64_t *enemy_death_type;
+    const int32_t *enemy_death_elapsed;
+    const uint8_t *enemy_death_extreme;  /* bool */
+    const float *doll_x;  /* [Sd] player_starts[:-1] */
+    const float *doll_y;
+    const float *doll_z;  /* _player_start_z[:-1] */
+    const uint8_t *doll_rotation;  /* [N,Sd] */
+    const uint8_t *player_dead;  /* [N] bool */
+    const float *projectile_x;  /* [N,Sp] */
+    const float *projectile_y;
+    const float *projectile_z;
+    const uint8_t *projectile_alive;  /* bool */
+    const int64_t *projectile_type;
+    const int32_t *projectile_age;
+    const uint8_t *projectile_rotation;
+    const int64_t *projectile_impact_type;
+    const int32_t *projectile_impact_tics;
+    const float *enemy_projectile_x;  /* [N,Sq] */
+    const float *enemy_projectile_y;
+    const float *enemy_projectile_z;
+    const uint8_t *enemy_projectile_alive;  /* bool */
+    const int32_t *enemy_projectile_age;
+    const uint8_t *enemy_projectile_rotation;
+    const int32_t *enemy_projectile_impact_tics;
+    const float *teleport_fog_x;  /* [N,Sg] */
+    const float *teleport_fog_y;
+    const float *teleport_fog_z;
+    const int32_t *teleport_fog_tics;
+    const float *hitscan_puff_x;  /* [N,Sf] */
+    const float *hitscan_puff_y;
+    const float *hitscan_puff_z;
+    const int32_t *hitscan_puff_tics;
+    const float *item_x;  /* [Si] item_spawns[:,0] */
+    const float *item_y;  /* item_spawns[:,1] */
+    const float *item_z;  /* _item_z */
+    const int64_t *item_types;  /* [Si] */
+    const int64_t *item_raw_visual_types;  /* [Si] */
+    const uint8_t *item_available;  /* [N,Si] bool */
+    const int32_t *item_animation_initial_tics;  /* [N,Si] */
+    const int32_t *episode_time;  /* [N] */
+    const float *drop_x;  /* [N,Sr] */
+    const float *drop_y;
+    const float *drop_z;
+    const int64_t *drop_type;
+    const uint8_t *drop_spawned;  /* bool */
+    const int32_t *enemy_walk_frame_tics;  /* [6] */
+    const int32_t *enemy_idle_frame_tics;  /* [6] */
+    const int32_t *enemy_attack_recovery;  /* [6] */
+    const int64_t *enemy_walk_sprite_ids;  /* [6,4,8] */
+    const int64_t *enemy_attack_sprite_ids;  /* [6,attack_frames,8] */
+    const int64_t *enemy_pain_sprite_ids;  /* [6,8] */
+    const int64_t *enemy_death_sprite_ids;  /* [6,death_frames] */
+    const int64_t *enemy_death_frame_durations;  /* [6,death_frames] */
+    const int64_t *enemy_death_frame_counts;  /* [6] */
+    const int64_t *enemy_xdeath_sprite_ids;  /* [6,xdeath_frames] */
+    const int64_t *enemy_xdeath_frame_durations;  /* [6,xdeath_frames] */
+    const int64_t *enemy_xdeath_frame_counts;  /* [6] */
+    const int64_t *projectile_explosion_total_tics;  /* [3] */
+    const int64_t *projectile_explosion_frame_durations;  /* [3,explosion_frames] */
+    const int64_t *projectile_explosion_frame_counts;  /* [3] */
+    const int64_t *raw_projectile_explosion_sprite_ids;  /* [3,explosion_frames] */
+    const int64_t *raw_projectile_flight_sprite_ids;  /* [3,2,8] */
+    const int64_t *raw_teleport_fog_sprite_ids;  /* [12] */
+    const int64_t *raw_bullet_puff_sprite_ids;  /* [4] */
+    const int64_t *raw_static_sprite_ids;  /* [>=15] */
+    const int64_t *raw_item_animation_sprite_ids;  /* [8] */
+    /* outputs, [N,A] each: the sprite_* fields of gd_lanes_desc */
+    float *sprite_x;
+    float *sprite_y;
+    float *sprite_z;
+    int32_t *sprite_id;
+    uint8_t *sprite_alive;
+    uint8_t *sprite_fullbright;
+    int8_t *sprite_style;
+} gd_actor_desc;
+
+int gd_pack_actors(const gd_actor_desc *actors, void *stream);
+
+/*
  * Time `launches` back-to-back gd_render launches with HIP events on `stream`
  * and return the average milliseconds per launch of each kernel stage in
  * ms[0..stage_count).  Measurement helper for the benchmark; replaces nothing.

@@ -121,6 +121,13 @@ CASES = {
         map_seed=22, grid=(6, 5), sectors=26, linedefs=160, lanes=8, pose_seed=5, sprites=24, pitch=True, flash=True,
         midtex=0.2, overlays=83, decals=17,
     ),
+    # Every kind of actor the sprite pass shows (monsters in all their states, start dolls, corpses, projectiles and
+    # explosions of both sides, teleport fog, bullet puffs, animated map items, drops) from randomised gameplay
+    # tensors; the list the renderer gets is actor_inputs.pack_actors(engine), 556 fixed slots per lane.
+    "actors": dict(
+        map_seed=22, grid=(6, 5), sectors=26, linedefs=160, lanes=8, pose_seed=7, pitch=True, flash=True, midtex=0.1,
+        blend_seed=19, actors=31,
+    ),
     "config2_subset": dict(map_seed=1002, grid=(12, 9), sectors=96, linedefs=800, lanes=4, pose_seed=1, sprites=32),
     "config3_subset": dict(
         map_seed=1003, grid=(15, 15), sectors=200, linedefs=2000, lanes=2, pose_seed=1, sprites=64, flash=True
@@ -144,7 +151,8 @@ def build_case(name: str, cfg: dict, do_time: bool) -> dict:
     started = time.time()
     overlays = synthmap.generate_overlays(cfg["overlays"]) if cfg.get("overlays") else None
     engine = refdrive.make_engine(
-        smap, lanes, flash_lights=cfg.get("flash", False), overlays=overlays, screen_flashes=bool(cfg.get("screen_flashes"))
+        smap, lanes, flash_lights=cfg.get("flash", False), overlays=overlays, screen_flashes=bool(cfg.get("screen_flashes")),
+        actors=cfg.get("actors", 0),
     )
     ctor_seconds = time.time() - started
     picks = cfg.get("picks") or [(cfg["pose_seed"], lane) for lane in range(lanes)]
@@ -164,6 +172,21 @@ def build_case(name: str, cfg: dict, do_time: bool) -> dict:
         ray_cos=ray_cos.numpy(), ray_sin=ray_sin.numpy(),
         cosine_correction=hostmath.cosine_correction("cpu").numpy(),
     )
+    if cfg.get("actors"):
+        # every kind of actor from randomised gameplay tensors, packed at full width by actor_inputs.pack_actors
+        from gradoom_amd import actor_inputs
+
+        refdrive.set_actor_state(engine, smap, cfg["actors"])
+        packed = {key: value.numpy() for key, value in actor_inputs.pack_actors(engine).items()}
+        data.update(packed)
+        # the tensors the packing read, so that it can be re-run without the reference
+        for field in actor_inputs.ENGINE_FIELDS:
+            data[f"actor_engine_{field}"] = getattr(engine, field).numpy().copy()
+        for field in actor_inputs.MAP_FIELDS:
+            data[f"actor_map_{field}"] = getattr(engine.map, field).numpy().copy()
+        data["sprite_depth"] = hostmath.sprite_depth(
+            engine.x, engine.y, engine.angle, torch.as_tensor(packed["sprite_x"]), torch.as_tensor(packed["sprite_y"])
+        ).numpy()
     if cfg.get("sprites", 0):
         sprites = synthmap.generate_sprites(smap, lanes, cfg["sprites"], cfg["pose_seed"])
         effects = synthmap.generate_sprites(smap, lanes, cfg["effects"], cfg["pose_seed"] + 50) if cfg.get("effects") else None

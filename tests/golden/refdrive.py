@@ -34,7 +34,37 @@ def load_reference():
     return engine, scenario
 
 
-def to_compiled_scenario(smap, *, flash_lights: bool = False, overlays: dict | None = None):
+def actor_tables(smap, seed: int) -> dict:
+    """Seeded patch-id and animation tables for every kind of actor, plus map items and player starts
+    (``scenario.py:346-378``); the ids only need to name existing patches."""
+
+    rng = np.random.default_rng(seed)
+    patches = len(smap.sprite_widths)
+    ids = lambda *shape: rng.integers(0, patches, shape).astype(np.int32)  # noqa: E731
+    death_frames = 6
+    death_counts = rng.integers(3, death_frames + 1, 6).astype(np.int32)
+    xdeath_counts = rng.integers(3, death_frames + 1, 6).astype(np.int32)
+    durations = lambda counts: np.where(np.arange(death_frames)[None, :] < counts[:, None], rng.integers(3, 9, (6, death_frames)), 0).astype(np.int32)  # noqa: E731
+    death_durations, xdeath_durations = durations(death_counts), durations(xdeath_counts)
+    sectors = rng.permutation(len(smap.sector_quads))
+    centre = lambda s, du, dv: (1 - du) * (1 - dv) * smap.sector_quads[s][0] + du * (1 - dv) * smap.sector_quads[s][1] + (1 - du) * dv * smap.sector_quads[s][2] + du * dv * smap.sector_quads[s][3]  # noqa: E731
+    starts = [(*np.round(centre(int(s), 0.5, 0.5)), float(rng.integers(0, 8) * 45)) for s in sectors[:4]]
+    item_count = 24
+    item_kinds = rng.choice(np.array([2011, 2012, 2014, 2015, 2018, 2019, 2007, 2048, 2001, 2002]), item_count)
+    spots = [(*np.round(centre(int(sectors[k % len(sectors)]), rng.uniform(0.2, 0.8), rng.uniform(0.2, 0.8))), 0.0) for k in range(item_count)]
+    return dict(
+        enemy_walk_sprite_ids=ids(6, 4, 8), enemy_attack_sprite_ids=ids(6, 3, 8), enemy_pain_sprite_ids=ids(6, 8),
+        enemy_death_sprite_ids=ids(6, death_frames), enemy_death_frame_counts=death_counts, enemy_death_frame_durations=death_durations,
+        enemy_xdeath_sprite_ids=ids(6, death_frames), enemy_xdeath_frame_counts=xdeath_counts, enemy_xdeath_frame_durations=xdeath_durations,
+        raw_projectile_flight_sprite_ids=ids(3, 2, 8), raw_projectile_explosion_sprite_ids=ids(3, 5),
+        raw_teleport_fog_sprite_ids=ids(12), raw_bullet_puff_sprite_ids=ids(4), raw_static_sprite_ids=ids(32),
+        raw_item_animation_sprite_ids=ids(8),
+        player_starts=np.asarray(starts, dtype=np.float32), item_spawns=np.asarray(spots, dtype=np.float32),
+        item_types=item_kinds.astype(np.int32),
+    )
+
+
+def to_compiled_scenario(smap, *, flash_lights: bool = False, overlays: dict | None = None, actors: int = 0):
     """Wrap a SynthMap in the reference's CompiledScenario (``scenario.py:302-401``)."""
 
     _engine, scenario = load_reference()
@@ -77,6 +107,16 @@ def to_compiled_scenario(smap, *, flash_lights: bool = False, overlays: dict | N
                 bullet_decal_left_offsets=overlays["decal_left"], bullet_decal_top_offsets=overlays["decal_top"],
                 bullet_decal_opacity_lut=overlays["decal_opacity_lut"], bullet_decal_black_lut=overlays["decal_black_lut"],
             )
+    fields = dict(
+        player_starts=np.asarray([(float(smap.vertices[0, 0]), float(smap.vertices[0, 1]), 0.0)], dtype=np.float32),
+        item_spawns=np.empty((0, 3), dtype=np.float32),
+        item_types=np.empty((0,), dtype=np.int32),
+        enemy_walk_sprite_ids=enemy_walk,
+        raw_static_sprite_ids=raw_static,
+    )
+    if actors:
+        fields.update(actor_tables(smap, actors))
+    fields.update(kwargs)
     return scenario.CompiledScenario(
         scenario_sha256="s" * 64,
         iwad_sha256="i" * 64,
@@ -95,9 +135,6 @@ def to_compiled_scenario(smap, *, flash_lights: bool = False, overlays: dict | N
         sector_lights=smap.sector_lights,
         sector_floor_texture_ids=smap.sector_floor_texture_ids,
         sector_ceiling_texture_ids=smap.sector_ceiling_texture_ids,
-        player_starts=np.asarray([(float(smap.vertices[0, 0]), float(smap.vertices[0, 1]), 0.0)], dtype=np.float32),
-        item_spawns=np.empty((0, 3), dtype=np.float32),
-        item_types=np.empty((0,), dtype=np.int32),
         playpal=smap.playpal,
         texture_names=tuple(f"T{i}" for i in range(len(smap.texture_widths))),
         texture_atlas=smap.texture_atlas,
@@ -114,17 +151,16 @@ def to_compiled_scenario(smap, *, flash_lights: bool = False, overlays: dict | N
         weapon_screen_values=np.zeros((8, 84, 84), dtype=np.float32),
         weapon_screen_alpha=np.zeros((8, 84, 84), dtype=np.float32),
         colormap=smap.colormap,
-        enemy_walk_sprite_ids=enemy_walk,
-        raw_static_sprite_ids=raw_static,
         wall_projection_fragments_fixed=smap.wall_projection_fragments_fixed,
         wall_projection_fragment_mask=smap.wall_projection_fragment_mask,
-        **kwargs,
+        **fields,
     )
 
 
-def make_engine(smap, lanes: int, *, flash_lights: bool = False, overlays: dict | None = None, screen_flashes: bool = False):
+def make_engine(smap, lanes: int, *, flash_lights: bool = False, overlays: dict | None = None, screen_flashes: bool = False,
+                actors: int = 0):
     engine_module, _scenario = load_reference()
-    compiled = to_compiled_scenario(smap, flash_lights=flash_lights, overlays=overlays)
+    compiled = to_compiled_scenario(smap, flash_lights=flash_lights, overlays=overlays, actors=actors)
     return engine_module.TorchDeathmatchEngine(
         compiled, lanes, device=torch.device("cpu"), render_screen_flashes=screen_flashes
     )
@@ -241,6 +277,83 @@ def set_decals(engine, smap, seed: int, per_lane: int = 40):
             engine.hitscan_decal_z[lane, slot] = z
             engine.hitscan_decal_style[lane, slot] = style
             engine.hitscan_decal_serial[lane, slot] = int(serial)
+
+
+def set_actor_state(engine, smap, seed: int):
+    """Randomise every kind of actor the sprite pass shows (state tensors of ``engine.py:1745-1925``)."""
+
+    from gradoom_amd import synthmap
+
+    generator = torch.Generator().manual_seed(seed)
+    lanes = engine.num_envs
+
+    def rand(low, high, shape, like):
+        return torch.randint(low, high, shape, generator=generator).to(like.dtype)
+
+    def place(count, offset):
+        spots = synthmap.generate_sprites(smap, lanes, count, seed + offset)
+        return (torch.as_tensor(v) for v in (spots.x, spots.y, spots.z, spots.alive))
+
+    # monsters: alive, dying or absent
+    n = engine.enemy_slots
+    x, y, z, used = place(n, 1)
+    engine.enemy_x[:], engine.enemy_y[:], engine.enemy_z[:] = x, y, z
+    dying = used & (torch.rand((lanes, n), generator=generator) < 0.3)
+    engine.enemy_alive[:] = used & ~dying
+    engine.enemy_type[:] = rand(0, 6, (lanes, n), engine.enemy_type)
+    engine.enemy_angle[:] = torch.rand((lanes, n), generator=generator) * 6.25
+    engine.enemy_animation_tics[:] = rand(0, 200, (lanes, n), engine.enemy_animation_tics)
+    engine.enemy_target_slot[:] = rand(-2, 4, (lanes, n), engine.enemy_target_slot)
+    engine.enemy_attack_phase[:] = rand(0, 5, (lanes, n), engine.enemy_attack_phase)
+    engine.enemy_cooldown[:] = rand(0, 40, (lanes, n), engine.enemy_cooldown)
+    engine.enemy_pain_tics[:] = torch.where(torch.rand((lanes, n), generator=generator) < 0.2, 3, 0).to(engine.enemy_pain_tics.dtype)
+    engine.enemy_death_tics[:] = torch.where(dying, 9, 0).to(engine.enemy_death_tics.dtype)
+    engine.enemy_death_type[:] = rand(0, 6, (lanes, n), engine.enemy_death_type)
+    engine.enemy_death_elapsed[:] = rand(0, 60, (lanes, n), engine.enemy_death_elapsed)
+    engine.enemy_death_extreme[:] = torch.rand((lanes, n), generator=generator) < 0.4
+    engine.player_dead[:] = torch.rand((lanes,), generator=generator) < 0.25
+    # the player's projectiles: flying or exploding
+    n = engine.player_projectile_slots
+    x, y, z, used = place(n, 2)
+    engine.projectile_x[:], engine.projectile_y[:], engine.projectile_z[:] = x, y, z
+    bursting = used & (torch.rand((lanes, n), generator=generator) < 0.4)
+    engine.projectile_alive[:] = used & ~bursting
+    engine.projectile_type[:] = rand(0, 2, (lanes, n), engine.projectile_type)
+    engine.projectile_age[:] = rand(0, 40, (lanes, n), engine.projectile_age)
+    engine.projectile_velocity_x[:] = torch.rand((lanes, n), generator=generator) * 20 - 10
+    engine.projectile_velocity_y[:] = torch.rand((lanes, n), generator=generator) * 20 - 10
+    engine.projectile_impact_type[:] = rand(0, 2, (lanes, n), engine.projectile_impact_type)
+    engine.projectile_impact_tics[:] = torch.where(bursting, rand(1, 18, (lanes, n), engine.projectile_impact_tics), 0).to(engine.projectile_impact_tics.dtype)
+    # monster fireballs
+    n = engine.enemy_projectile_slots
+    x, y, z, used = place(n, 3)
+    engine.enemy_projectile_x[:], engine.enemy_projectile_y[:], engine.enemy_projectile_z[:] = x, y, z
+    bursting = used & (torch.rand((lanes, n), generator=generator) < 0.4)
+    engine.enemy_projectile_alive[:] = used & ~bursting
+    engine.enemy_projectile_age[:] = rand(0, 40, (lanes, n), engine.enemy_projectile_age)
+    engine.enemy_projectile_velocity_x[:] = torch.rand((lanes, n), generator=generator) * 20 - 10
+    engine.enemy_projectile_velocity_y[:] = torch.rand((lanes, n), generator=generator) * 20 - 10
+    engine.enemy_projectile_impact_tics[:] = torch.where(bursting, rand(1, 18, (lanes, n), engine.enemy_projectile_impact_tics), 0).to(engine.enemy_projectile_impact_tics.dtype)
+    # teleport fog, bullet puffs, drops
+    n = engine.enemy_slots
+    x, y, z, used = place(n, 4)
+    engine.teleport_fog_x[:], engine.teleport_fog_y[:], engine.teleport_fog_z[:] = x, y, z
+    engine.teleport_fog_tics[:] = torch.where(used, rand(1, 73, (lanes, n), engine.teleport_fog_tics), 0).to(engine.teleport_fog_tics.dtype)
+    n = engine.hitscan_puff_slots
+    x, y, z, used = place(n, 5)
+    engine.hitscan_puff_x[:], engine.hitscan_puff_y[:], engine.hitscan_puff_z[:] = x, y, z
+    engine.hitscan_puff_tics[:] = torch.where(used, rand(1, 17, (lanes, n), engine.hitscan_puff_tics), 0).to(engine.hitscan_puff_tics.dtype)
+    n = engine.enemy_slots
+    x, y, z, used = place(n, 6)
+    engine.drop_x[:], engine.drop_y[:], engine.drop_z[:] = x, y, z
+    kinds = torch.tensor((2001, 2002, 2007, 2048))[torch.randint(0, 4, (lanes, n), generator=generator)]
+    engine.drop_type[:] = torch.where(used, kinds, -1)
+    engine.drop_spawned[:] = torch.rand((lanes, n), generator=generator) < 0.8
+    # map items
+    items = len(engine.map.item_types)
+    engine.item_available[:] = torch.rand((lanes, items), generator=generator) < 0.7
+    engine.item_animation_initial_tics[:] = rand(1, 7, (lanes, items), engine.item_animation_initial_tics)
+    engine.episode_time[:] = rand(0, 500, (lanes,), engine.episode_time)
 
 
 def set_effect_sprites(engine, sprites, seed: int):

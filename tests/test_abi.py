@@ -58,3 +58,5 @@ def test_struct_layouts_match_header_field_order():
     assert fields("gd_map_desc") == [name for name, _ in _abi.MapDesc._fields_]
     assert fields("gd_lanes_desc") == [name for name, _ in _abi.LanesDesc._fields_]
     assert fields("gd_frame_out") == [name for name, _ in _abi.FrameOut._fields_]
+    assert fields("gd_overlay_desc") == [name for name, _ in _abi.OverlayDesc._fields_]
+    assert fields("gd_actor_desc") == [name for name, _ in _abi.ActorDesc._fields_]
