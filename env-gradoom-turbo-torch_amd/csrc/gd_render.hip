@@ -77,6 +77,7 @@ typedef unsigned long long u64;
 struct LaneCtx {
     float x, y, view_z, pitch_offset, fsin, fcos;
     i64 view_x_fixed, view_y_fixed, vsin, vcos, center_fixed, flash_light;
+    i64 upper_clip, lower_clip;   // OWallMost's view-frustum slopes at the top and bottom row (engine.py:12402-12413)
     int sector;
     int pad;
 };
@@ -445,6 +446,8 @@ __global__ void lane_setup_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_ba
     i64 tangent_index = clampi((ANGLE_90 - pitch_bam) >> 19, 0, FINE_ANGLES / 2 - 1);
     i64 tangent = dm.fine_tangent[tangent_index];
     c.center_fixed = (i64)(VH / 2) * FIXED_UNIT + ((FOCAL_Y_FIXED * tangent) >> 16);
+    c.upper_clip = tdiv(shl64(-c.center_fixed, 16), FOCAL_Y_FIXED);
+    c.lower_clip = tdiv(shl64((i64)VH * FIXED_UNIT - c.center_fixed, 16), FOCAL_Y_FIXED);
     c.pitch_offset = (float)((tangent * 12582912LL) >> 16) / 65536.0f;
     c.sector = sector_at(&dm.d, c.x, c.y);
     c.pad = 0;
@@ -1136,8 +1139,7 @@ __device__ __forceinline__ float project(const LaneCtx &c, const WallRec &g, con
         i64 ostep = tdiv(opr - opl, original_span);
         return (float)clampi((center_fixed + opl + mul64(px - whole_sl, ostep)) >> 16, 0, VH);
     }
-    i64 upper_clip = tdiv(shl64(-center_fixed, 16), FOCAL_Y_FIXED);
-    i64 lower_clip = tdiv(shl64((i64)VH * FIXED_UNIT - center_fixed, 16), FOCAL_Y_FIXED);
+    const i64 upper_clip = c.upper_clip, lower_clip = c.lower_clip;
     i64 upper_left = mul64(upper_clip, depth_left) >> 16, upper_right = mul64(upper_clip, depth_right) >> 16;
     i64 lower_left = mul64(lower_clip, depth_left) >> 16, lower_right = mul64(lower_clip, depth_right) >> 16;
     bool above_left = pz < upper_left, above_right = pz < upper_right;
