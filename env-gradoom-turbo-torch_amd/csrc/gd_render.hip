@@ -1486,8 +1486,11 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
     PROF_MARK(11, tsub);
     // j. projection and clipping (engine.py:12607-12620)
     float one_top = 0, one_bottom = 0, lower_top = 0, upper_bottom = 0;
+    // one copy of the projection code, four heights; the back sector's two only matter across a
+    // two-sided linedef (every use of them is behind !one_sided)
+    const int heights = one_sided ? 2 : 4;
 #pragma unroll 1
-    for (int k = 0; k < 4; ++k) {   // one copy of the projection code, four heights
+    for (int k = 0; k < heights; ++k) {
         float z = k == 0 ? r.view_ceiling : (k == 1 ? r.view_floor : (k == 2 ? r.other_floor : r.other_ceiling));
         float v = project(*cc.c, wr, wr_fragment, z, x);
         if (k == 0) one_top = v; else if (k == 1) one_bottom = v; else if (k == 2) lower_top = v; else upper_bottom = v;
