@@ -2272,6 +2272,12 @@ __global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lan
     if (local >= lane_count) return;
     const int n = lane_base + local;
     const int A = lanes.sprite_slots;
+    // the slots that can reach the screen at all (alive, in front, some column between left and right): the
+    // per-column loops below only walk these.  Their order in the list is irrelevant, ties go by slot number.
+    unsigned short *on_screen = reinterpret_cast<unsigned short *>(sp + A);
+    __shared__ int on_screen_count;
+    if (threadIdx.x == 0) on_screen_count = 0;
+    __syncthreads();
     const LaneCtx L = sc.ctx[local];
     for (int a = threadIdx.x; a < A; a += blockDim.x) {
         SpriteRec s;
@@ -2297,8 +2303,10 @@ __global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lan
         s.texmid = (i64)m->spr_top[s.id] * FIXED_UNIT - round_to_i64((L.view_z - z) * 65536.0f);
         s.top_fixed = L.center_fixed - (mul64(s.texmid, s.yscale) >> 16);
         s.iscale = tdiv(UINT32_MASK, max64(s.yscale, 1));
-        s.light = m->sector_lights[sector_at(m, s.x, s.y)];
+        const bool reaches = (s.flags & 1) && (s.depth > 0) && (s.right > 0) && (s.left < SW) && (s.right > s.left);
+        s.light = reaches ? m->sector_lights[sector_at(m, s.x, s.y)] : 0.0f;
         sp[a] = s;
+        if (reaches) on_screen[atomicAdd(&on_screen_count, 1)] = (unsigned short)a;
     }
     __syncthreads();
     const int x = threadIdx.x;
@@ -2320,15 +2328,16 @@ __global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lan
     // The sprites that can show in this column at all (alive, in front, horizontally covering it and
     // not hidden by the column's blocking linedef), as a bit set: the painter's loop below runs once
     // per drawn sprite and would otherwise test every slot each time.
-    u64 cover[8] = {0, 0, 0, 0, 0, 0, 0, 0};   // sprite_slots <= 512
+    const int listed = on_screen_count;
+    u64 cover[8] = {0, 0, 0, 0, 0, 0, 0, 0};   // sprite_slots <= 512; bit p of the set = on_screen[p]
 #pragma unroll
     for (int word = 0; word < 8; ++word) {
-        if (word * 64 >= A) continue;          // the same in every thread
+        if (word * 64 >= listed) continue;     // the same in every thread
         u64 bits = 0;
-        const int end = A - word * 64 < 64 ? A - word * 64 : 64;
+        const int end = listed - word * 64 < 64 ? listed - word * 64 : 64;
         for (int b = 0; b < end; ++b) {
-            const SpriteRec &s = sp[word * 64 + b];
-            if (!((s.flags & 1) && (x >= s.left) && (x < s.right) && (s.depth > 0))) continue;
+            const SpriteRec &s = sp[on_screen[word * 64 + b]];
+            if (!((x >= s.left) && (x < s.right))) continue;
             bool ray_visible = s.depth < wall_distance;
             if (!ray_visible) {
                 float bside = bdx * (s.y - bl.y) - bdy * (s.x - bl.x);
@@ -2346,7 +2355,7 @@ __global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lan
 #pragma unroll
         for (int word = 0; word < 8; ++word) {
             for (u64 bits = cover[word]; bits; bits &= bits - 1) {
-                const int a = word * 64 + __ffsll((long long)bits) - 1;
+                const int a = on_screen[word * 64 + __ffsll((long long)bits) - 1];
                 const float depth = sp[a].depth;
                 // strictly before (last_depth, last_slot) in (depth, slot) order
                 if (!(depth < last_depth || (depth == last_depth && a < last_slot))) continue;
@@ -3041,7 +3050,7 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     if (decals)
         hipLaunchKernelGGL(decal_kernel, dim3(count), dim3(SW), 0, stream, r->dm, r->overlays, *lanes, base, count, sc, frame_base, frame_stride);
     if (lanes->sprite_slots > 0 && lanes->sprite_x) {
-        size_t shared = (size_t)lanes->sprite_slots * sizeof(SpriteRec);
+        size_t shared = (size_t)lanes->sprite_slots * (sizeof(SpriteRec) + sizeof(unsigned short));
         hipLaunchKernelGGL(sprite_columns_kernel, dim3(count), dim3(SW), shared, stream, r->dm, *lanes, base, count, sc, frame_base, frame_stride);
     }
     if (lanes->weapon_state && r->overlays.d.weapon_patch_count > 0)
