@@ -144,6 +144,8 @@ struct Scratch {    // per-chunk working memory, sized at create
     int *cand_count;       // [L,320] (may exceed CAND_MAX when a list overflowed)
     unsigned short *flat_sector;// [L,208,320]
     unsigned char *flat_flags;  // [L,208,320] bit0 unresolved
+    int *flat_span;        // [L,4] first / last row of the ceiling half, then of the floor half, that holds a shown
+                           // pixel the flat pass could not resolve (208, -1 = none): the rows the repairs work on
     unsigned int *meta;    // [L,208,320] filled | floor | plane_sector+1 | clip_wall+1
     float *clip_depth;     // [L,208,320]
     unsigned char *frame;  // [L,240,320] when the caller wants no indexed output
@@ -452,6 +454,8 @@ __global__ void lane_setup_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_ba
     c.sector = sector_at(&dm.d, c.x, c.y);
     c.pad = 0;
     sc.ctx[local] = c;
+    int *span = sc.flat_span + (size_t)local * 4;
+    span[0] = VH; span[1] = -1; span[2] = VH; span[3] = -1;
     for (int x = 0; x < SW; ++x) { sc.cand_count[(size_t)local * SW + x] = 0; sc.block_hit[(size_t)local * SW + x] = ~0ULL; }
 }
 
@@ -693,17 +697,60 @@ __device__ __forceinline__ float flat_center(const LaneCtx &c) { return 103.5f +
 // Per pixel: nearest plane among all sectors (engine.py:10981-11024).  Sectors that share a
 // plane height share the candidate point, and the distance grows with the plane height, so the
 // levels are visited nearest first and the scan stops once a farther level cannot win.
-__global__ void flat_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
+//
+// Does the point lie in some sector whose floor (ceiling) is at `level`?  The even-odd test of
+// engine.py:10994-11015 over the sectors the point-location grid lists for the point's cell.
+__device__ bool flat_level_hit(const DeviceMap &dm, bool is_floor, float level, float px, float py) {
     const gd_map_desc *m = &dm.d;
-    int local = blockIdx.y;
-    int pixel = blockIdx.x * blockDim.x + threadIdx.x;
-    if (local >= lane_count || pixel >= VH * SW) return;
-    int y = pixel / SW, x = pixel - y * SW;
+    int cell;
+    const unsigned fine = fine_lookup(m, dm.fine_inverse, px, py, &cell);
+    const unsigned kind = FINE_KIND(fine);
+    if (kind == FINE_EMPTY) return false;
+    if (kind == FINE_DECIDED) return m->sector_heights[2 * (int)(fine & 0xFFFFu) + (is_floor ? 0 : 1)] == level;
+    if (cell < 0) cell = grid_cell_of(m, px, py);
+    if (cell < 0) return false;
+    const int2 range = dm.cell_range[cell];
+    for (int it = range.x; it < range.y; ++it) {
+        const int4 item = dm.cell_item[it];
+        const int s = item.x & ~GRID_ALWAYS_INSIDE;
+        if (m->sector_heights[2 * s + (is_floor ? 0 : 1)] != level) continue;
+        if ((item.x & GRID_ALWAYS_INSIDE) || inside_edge_copies(dm.cell_edge, item.z, item.w, px, py)) return true;
+    }
+    return false;
+}
+//
+// Does the flat ray of one pixel resolve at all, i.e. does the probe point of some plane level lie in a
+// sector of that level (engine.py:10981-11024)?  `plane` is the sector whose plane the wall pass shows at the
+// pixel: its own level nearly always answers yes at once.
+__device__ bool flat_ray_resolves(const DeviceMap &dm, const LaneCtx &c, float rc, float rs, float cc, int y, int plane) {
+    const gd_map_desc *m = &dm.d;
+    const float delta = (float)y - flat_center(c);
+    const bool is_floor = delta > 0;
+    const float denom = fmaxf(fabsf(delta), 0.5f);
+    const float *levels = is_floor ? m->floor_levels : m->ceil_levels;
+    const int level_count = is_floor ? m->floor_level_count : m->ceil_level_count;
+    const float own = m->sector_heights[2 * plane + (is_floor ? 0 : 1)];
+    for (int k = -1; k < level_count; ++k) {
+        const float level = k < 0 ? own : levels[k];
+        if (k >= 0 && level == own) continue;
+        const float height = is_floor ? (c.view_z - level) : (level - c.view_z);
+        if (!(height > 0)) continue;
+        const float cd = (height * 192.0f / denom) / cc;
+        if (!(finitef(cd) && cd > 0)) continue;
+        if (flat_level_hit(dm, is_floor, level, c.x + rc * cd, c.y + rs * cd)) return true;
+    }
+    return false;
+}
+//
+// flat_select_pixel is called by whole wavefronts whose 64 lanes look at 64 pixels of ONE row of one lane's
+// screen (wanted or not: every lane takes part in the level broadcasts); it returns the sector, -1 if no
+// level's probe point lies in a sector of that level.
+__device__ __forceinline__ int flat_select_pixel(const DeviceMap &dm, const Scratch &sc, const gd_lanes_desc &lanes, int local, int n,
+                                                 int x, int y, bool wanted) {
+    const gd_map_desc *m = &dm.d;
     const LaneCtx &c = sc.ctx[local];
-    int n = lane_base + local;
-    float center = flat_center(c);
-    float delta = (float)y - center;
-    bool is_floor = delta > 0;
+    const float delta = (float)y - flat_center(c);
+    const bool is_floor = delta > 0;
     float denom = fmaxf(fabsf(delta), 0.5f);
     float cc = dm.cosine_correction[x];
     float rc = lanes.ray_cos[(size_t)n * SW + x], rs = lanes.ray_sin[(size_t)n * SW + x];
@@ -730,8 +777,9 @@ __global__ void flat_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
     // farther than that from the camera is dropped for the whole wavefront at once
     const float reach_scale = dm.strip_reach_scale[__builtin_amdgcn_readfirstlane(x >> 6)];
     float best = GD_INF; int best_sector = -1;
-    bool done = false;
-    for (int base = 0; base < level_count && !done; base += 64) {
+    bool done = !wanted;
+    for (int base = 0; base < level_count; base += 64) {
+        if (__ballot(!done) == 0) break;   // every lane takes part in the level broadcasts below, wanted or not
         // lane k works out level base+k: its height and perpendicular distance (one division for
         // the wavefront instead of one per level per lane); a level the plane cannot show gets -1
         const int mine = base + slot_in_wave;
@@ -790,7 +838,10 @@ __global__ void flat_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
                 const float px = c.x + rc * cd, py = c.y + rs * cd;
                 int cell = cellv[j];
                 if (cell < 0) cell = grid_cell_of(m, px, py);
-                if (cell < 0) continue;
+                // Outside the grid (above, below or right of every linedef) no sector holds the point, and the
+                // probe points of the levels still to come lie farther along the same ray, which has left
+                // that convex region for good.
+                if (cell < 0) { done = true; continue; }
                 const int2 range = dm.cell_range[cell];
                 for (int it = range.x; it < range.y; ++it) {
                     const int4 item = dm.cell_item[it];
@@ -805,10 +856,45 @@ __global__ void flat_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
             }
         }
     }
-    size_t i = (size_t)local * VH * SW + pixel;
-    sc.flat_sector[i] = (unsigned short)(best_sector < 0 ? c.sector : best_sector);
-    sc.flat_flags[i] = best_sector < 0 ? 1 : 0;
+    return best_sector;
 }
+
+// The pass runs after the walls and only where its result can matter.  A pixel a wall tier filled never
+// shows it; a pixel a plane of the wall pass claimed only asks whether the flat ray resolved at all, and only
+// where a sprite stands behind the plane with no sprite clip recorded, which the sprite pass finds out for
+// itself (flat_ray_resolves); the few pixels left (columns whose traversal left a gap) show the flat pass's
+// picture.  This kernel handles exactly those pixels and notes, per lane and screen half, the rows where a shown
+// pixel stayed unresolved: flat_span_select_kernel and flat_span_finish_kernel select and repair those rows.
+__global__ void flat_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc,
+                                   unsigned char *frame_base, size_t frame_stride) {
+    const gd_map_desc *m = &dm.d;
+    int local = blockIdx.y;
+    int pixel = blockIdx.x * blockDim.x + threadIdx.x;
+    if (local >= lane_count || pixel >= VH * SW) return;
+    if (pixel < (GD_SCREEN_HEIGHT - VH) * SW)   // the empty status bar, rows 208..239
+        frame_base[(size_t)local * frame_stride + (size_t)VH * SW + pixel] = 0;
+    const int y = pixel / SW, x = pixel - y * SW;
+    const int n = lane_base + local;
+    const size_t i = (size_t)local * VH * SW + pixel;
+    const unsigned meta_word = sc.meta[i];
+    const bool filled = meta_word & META_FILLED;
+    const int plane = (int)((meta_word >> META_SECTOR_SHIFT) & META_SECTOR_MASK) - 1;
+    const bool shown = !filled && plane < 0 && !(meta_word & META_MASKED);
+    if (__ballot(shown) == 0) return;              // the whole wavefront (64 pixels of one row) has nothing to find
+    const bool wanted = shown;
+    const int best_sector = flat_select_pixel(dm, sc, lanes, local, n, x, y, wanted);
+    if (wanted) {
+        sc.flat_sector[i] = (unsigned short)(best_sector < 0 ? sc.ctx[local].sector : best_sector);
+        sc.flat_flags[i] = best_sector < 0 ? 1 : 0;
+    }
+    if (__ballot(shown && best_sector < 0) != 0 && (threadIdx.x & 63) == 0) {
+        const bool floor_row = ((float)y - flat_center(sc.ctx[local])) > 0;
+        int *span = sc.flat_span + (size_t)local * 4 + (floor_row ? 2 : 0);
+        atomicMin(&span[0], y);
+        atomicMax(&span[1], y);
+    }
+}
+
 
 // Small per-sector / per-texture tables staged in LDS by the kernels whose inner loops chase
 // them (a dependent global gather costs ~500 cycles, an LDS read ~60).  Sectors or textures
@@ -927,51 +1013,66 @@ __device__ __forceinline__ size_t flat_sample_tabled(const Tables &tb, const Lan
     return ((size_t)texture * m->tex_max_h + v) * m->tex_max_w + u;
 }
 
-// Visplane continuity repair and shading for one lane (engine.py:11026-11171).
-// 320 threads: vertical repair is one thread per column; horizontal repair is one wave per
-// row with 64-column ballots; shading is one thread per column again.
-__global__ void __launch_bounds__(SW) flat_finish_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
-    const gd_map_desc *m = &dm.d;
-    int local = blockIdx.x;
+// Visplane repair (engine.py:11026-11135) of the row ranges flat_select_kernel noted, one block per lane, one
+// wavefront per 64 columns.  Every pixel of those rows is selected first (the repairs read whole rows and
+// columns).  Vertical: an unresolved pixel takes the sector of the next resolved pixel below it in its half of
+// the screen; rows below the noted range are selected one at a time until every column that still looks for
+// one has found it.  Horizontal: an unresolved pixel between a left and a right anchor of one sector takes
+// that sector.  Pixels outside the noted rows need none of this: no shown pixel there is unresolved, and
+// resolved pixels are never repaired.
+#define SPAN_ROW_SLOTS 16
+// Every pixel of the noted rows, block j of a lane taking rows j, j + SPAN_ROW_SLOTS, ... of both ranges.
+__global__ void __launch_bounds__(SW) flat_span_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
+    const int local = blockIdx.y;
     if (local >= lane_count) return;
+    const int *span = sc.flat_span + (size_t)local * 4;
+    const int lo[2] = {span[0], span[2]}, hi[2] = {span[1], span[3]};
+    const int rows0 = hi[0] < lo[0] ? 0 : hi[0] - lo[0] + 1, rows1 = hi[1] < lo[1] ? 0 : hi[1] - lo[1] + 1;
+    const int n = lane_base + local;
+    const int x = threadIdx.x;
+    for (int r = blockIdx.x; r < rows0 + rows1; r += SPAN_ROW_SLOTS) {
+        const int y = r < rows0 ? lo[0] + r : lo[1] + (r - rows0);
+        const int s = flat_select_pixel(dm, sc, lanes, local, n, x, y, true);
+        const size_t i = (size_t)local * VH * SW + (size_t)y * SW + x;
+        sc.flat_sector[i] = (unsigned short)(s < 0 ? sc.ctx[local].sector : s);
+        sc.flat_flags[i] = s < 0 ? 1 : 0;
+    }
+}
+
+__global__ void __launch_bounds__(SW) flat_span_finish_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
+    const int local = blockIdx.x;
+    if (local >= lane_count) return;
+    const int *span = sc.flat_span + (size_t)local * 4;
+    const int lo[2] = {span[0], span[2]}, hi[2] = {span[1], span[3]};
+    if (hi[0] < lo[0] && hi[1] < lo[1]) return;      // the same in every thread
     const LaneCtx c = sc.ctx[local];
+    const int n = lane_base + local;
     unsigned short *sector = sc.flat_sector + (size_t)local * VH * SW;
     unsigned char *flags = sc.flat_flags + (size_t)local * VH * SW;
-    unsigned char *frame = frame_base + (size_t)local * frame_stride;
     const int x = threadIdx.x;
     const float center = flat_center(c);
-    // --- vertical: an unresolved pixel takes the next resolved row below of its own kind.
-    // Floors are repaired first and ceilings read the repaired map (engine.py:11050-11083);
-    // the gathered rows are resolved pixels, which no repair modifies.
-    {
-        int next_floor = VH, next_ceiling = VH;
-        int floor_sector = 0, ceiling_sector = 0;
-        // eight rows per step, loads first (a row only depends on rows below it through the four
-        // carried values, never through memory), so the loads of a step overlap
-        static_assert(VH % 8 == 0, "row batches");
-        for (int yb = VH - 8; yb >= 0; yb -= 8) {
-            unsigned char row_flags[8]; unsigned short row_sector[8];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) { row_flags[j] = flags[(size_t)(yb + j) * SW + x]; row_sector[j] = sector[(size_t)(yb + j) * SW + x]; }
-#pragma unroll
-            for (int j = 7; j >= 0; --j) {
-                const int y = yb + j;
-                const size_t i = (size_t)y * SW + x;
-                bool is_floor = ((float)y - center) > 0;
-                bool unresolved = row_flags[j] & 1;
-                int s = row_sector[j];
-                if (!unresolved) {
-                    if (is_floor) { next_floor = y; floor_sector = s; } else { next_ceiling = y; ceiling_sector = s; }
-                } else {
-                    bool vfloor = is_floor && next_floor < VH;
-                    bool vceil = !is_floor && next_ceiling < VH;
-                    if (vfloor || vceil) {
-                        int span_sector = vfloor ? floor_sector : ceiling_sector;
-                        sector[i] = (unsigned short)span_sector;
-                        // bit1: vertical span; bit2: its sector differs from the camera's (anchor)
-                        flags[i] = (unsigned char)(1 | 2 | ((span_sector != c.sector) ? 4 : 0));
-                    }
-                }
+    int last_ceiling_row = -1;                       // rows 0 .. last_ceiling_row look at ceilings
+    for (int y = 0; y < VH; ++y) if (!(((float)y - center) > 0)) last_ceiling_row = y;
+    // --- vertical (engine.py:11026-11083): floors and ceilings alike look downwards, within their own half
+    for (int half = 0; half < 2; ++half) {
+        if (hi[half] < lo[half]) continue;           // the same in every thread
+        const int half_end = half ? VH - 1 : last_ceiling_row;
+        // a column whose pixel in the range's last row is unresolved looks further down for a resolved one;
+        // each wavefront goes on, a row at a time, while any of its 64 columns is still looking
+        bool looking = flags[(size_t)hi[half] * SW + x] & 1;
+        bool found = false;
+        int span_sector = 0;
+        for (int y = hi[half] + 1; y <= half_end && __ballot(looking) != 0; ++y) {
+            const int s = flat_select_pixel(dm, sc, lanes, local, n, x, y, looking);
+            if (looking && s >= 0) { looking = false; found = true; span_sector = s; }
+        }
+        for (int y = hi[half]; y >= lo[half]; --y) {
+            const size_t i = (size_t)y * SW + x;
+            if (!(flags[i] & 1)) { found = true; span_sector = sector[i]; }
+            else if (found) {
+                sector[i] = (unsigned short)span_sector;
+                // bit1: vertical span; bit2: its sector differs from the camera's (anchor)
+                flags[i] = (unsigned char)(1 | 2 | ((span_sector != c.sector) ? 4 : 0));
             }
         }
     }
@@ -980,7 +1081,9 @@ __global__ void __launch_bounds__(SW) flat_finish_kernel(DeviceMap dm, int lane_
     {
         const int lane_id = threadIdx.x & 63;
         const int wave = threadIdx.x >> 6;
-        for (int y = wave; y < VH; y += SW / 64) {
+        const int rows0 = hi[0] < lo[0] ? 0 : hi[0] - lo[0] + 1, rows1 = hi[1] < lo[1] ? 0 : hi[1] - lo[1] + 1;
+        for (int r = wave; r < rows0 + rows1; r += SW / 64) {
+            const int y = r < rows0 ? lo[0] + r : lo[1] + (r - rows0);
             unsigned short *row_sector = sector + (size_t)y * SW;
             unsigned char *row_flags = flags + (size_t)y * SW;
             u64 anchors[5];
@@ -1005,16 +1108,14 @@ __global__ void __launch_bounds__(SW) flat_finish_kernel(DeviceMap dm, int lane_
                 if (above) right = k * 64 + __ffsll((long long)above) - 1;
                 else for (int j = k + 1; j < 5 && right >= SW; ++j) if (anchors[j]) right = j * 64 + __ffsll((long long)anchors[j]) - 1;
                 if (left >= 0 && right < SW) {
-                    int ls = row_sector[left], rs = row_sector[right];
+                    int ls = row_sector[left], rs_ = row_sector[right];
                     // anchors are never rewritten by this pass, so reading them while other
                     // lanes write their own unresolved pixels is race free
-                    if (ls == rs) { row_sector[col] = (unsigned short)ls; row_flags[col] = (unsigned char)(f[k] | 8); }
+                    if (ls == rs_) { row_sector[col] = (unsigned short)ls; row_flags[col] = (unsigned char)(f[k] | 8); }
                 }
             }
         }
     }
-    // shading happens once per pixel in plane_shade_kernel, after the walls have claimed theirs
-    for (int y = VH; y < GD_SCREEN_HEIGHT; ++y) frame[(size_t)y * SW + x] = 0;  // empty status bar
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -2243,13 +2344,6 @@ __global__ void __launch_bounds__(256) plane_shade_kernel(DeviceMap dm, int lane
                 }
                 sc.scene_depth[i] = depth;
             }
-            // plane fallback occluder for sprites where the flat ray was unresolved (engine.py:13417-13422)
-            if (claimed && (flat_flags[j] & 1) && !finitef(sc.clip_depth[i])) {
-                const float flat_center_px = (103.0f + c.pitch_offset) + 0.5f;
-                float plane_height = is_floor ? (c.view_z - tb.floor_h(ps)) : (tb.ceil_h(ps) - c.view_z);
-                float plane_denominator = fmaxf(fabsf((float)y - flat_center_px), 0.5f);
-                sc.clip_depth[i] = plane_height * 192.0f / plane_denominator;
-            }
         }
     }
 }
@@ -2408,6 +2502,19 @@ __global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lan
                     visible = (cnear > s.depth_fixed) || ((cfar > s.depth_fixed) && (side <= 0));
                 } else {
                     visible = s.depth < row_clip[j];
+                    // No clip recorded, but a plane of the wall pass shows here: where the flat ray did not
+                    // resolve, the plane's own depth clips sprites (engine.py:13417-13422).  Only a sprite
+                    // standing behind the plane needs to know.
+                    const int plane = (int)((row_meta[j] >> META_SECTOR_SHIFT) & META_SECTOR_MASK) - 1;
+                    if (visible && plane >= 0 && !(row_meta[j] & META_FILLED) && !finitef(row_clip[j])) {
+                        const int y = yb + j;
+                        const bool plane_floor = (row_meta[j] & META_FLOOR) != 0;
+                        const float plane_height = plane_floor ? (L.view_z - m->sector_heights[2 * plane]) : (m->sector_heights[2 * plane + 1] - L.view_z);
+                        const float plane_depth = plane_height * 192.0f / fmaxf(fabsf((float)y - ((103.0f + L.pitch_offset) + 0.5f)), 0.5f);
+                        if (!(s.depth < plane_depth))
+                            visible = flat_ray_resolves(dm, L, lanes.ray_cos[(size_t)n * SW + x], lanes.ray_sin[(size_t)n * SW + x],
+                                                        dm.cosine_correction[x], y, plane);
+                    }
                 }
                 live[j] = visible;
                 if (!visible) continue;
@@ -3008,30 +3115,17 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     else frame_base = sc.frame;
     int stage = 0;
     auto mark = [&]() { if (timed) (void)hipEventRecord(r->events[stage], stream); ++stage; };
-    // Stage timing needs the kernels one after another; otherwise the flats run on the side stream.
     const bool decals = lanes->decal_slots > 0 && lanes->decal_state && lanes->decal_geom && r->overlays.d.decal_variant_count > 0;
     if (!decals) sc.scene_depth = nullptr;
-    // With decals every pass writes the scene depth in turn (flats, walls, planes), so nothing overlaps.
-    const bool overlap = !timed && side != nullptr && !decals;
-    hipStream_t flat_stream = overlap ? side : stream;
     mark();
     hipLaunchKernelGGL(lane_setup_kernel, dim3((count + 63) / 64), dim3(64), 0, stream, r->dm, *lanes, base, count, sc);
-    if (overlap) {
-        HIP_TRY(hipEventRecord(r->fork_event, stream));
-        HIP_TRY(hipStreamWaitEvent(side, r->fork_event, 0));
-    }
+    hipLaunchKernelGGL(lane_tables_kernel, dim3(count), dim3(256), 0, stream, r->dm, *lanes, base, count, sc);
     hipLaunchKernelGGL(wall_setup_kernel, dim3((m.wall_count + 127) / 128, count), dim3(128), 0, stream, r->dm, count, sc);
     if (m.split_count > 0)
         hipLaunchKernelGGL(fragment_setup_kernel, dim3((m.split_count * m.fragment_slots + 63) / 64, count), dim3(64), 0, stream, r->dm, count, sc);
     hipLaunchKernelGGL(strip_key_kernel, dim3((count * (SW / 64) + 3) / 4), dim3(256), 0, stream, count, sc);
     hipLaunchKernelGGL(strip_order_kernel, dim3(1), dim3(1024), 0, stream, count * (SW / 64), sc);
     mark();
-    hipLaunchKernelGGL(lane_tables_kernel, dim3(count), dim3(256), 0, flat_stream, r->dm, *lanes, base, count, sc);
-    hipLaunchKernelGGL(flat_select_kernel, dim3((VH * SW + 255) / 256, count), dim3(256), 0, flat_stream, r->dm, *lanes, base, count, sc);
-    mark();
-    hipLaunchKernelGGL(flat_finish_kernel, dim3(count), dim3(SW), 0, flat_stream, r->dm, count, sc, frame_base, frame_stride);
-    mark();
-    if (overlap) HIP_TRY(hipEventRecord(r->flat_event, side));
     {
         const dim3 grid((count * (SW / 64) + WALL_STRIPS_PER_GROUP - 1) / WALL_STRIPS_PER_GROUP), block(64 * WALL_STRIPS_PER_GROUP);
         const bool split = m.split_count > 0;
@@ -3040,7 +3134,12 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
         hipLaunchKernelGGL(kernel, grid, block, WALL_LDS_PAD, stream, r->dm, count, sc, frame_base, frame_stride);
     }
     mark();
-    if (overlap) HIP_TRY(hipStreamWaitEvent(stream, r->flat_event, 0));
+    // the flat pass, where the walls left it something to decide
+    hipLaunchKernelGGL(flat_select_kernel, dim3((VH * SW + 255) / 256, count), dim3(256), 0, stream, r->dm, *lanes, base, count, sc, frame_base, frame_stride);
+    mark();
+    hipLaunchKernelGGL(flat_span_select_kernel, dim3(SPAN_ROW_SLOTS, count), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
+    hipLaunchKernelGGL(flat_span_finish_kernel, dim3(count), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
+    mark();
     {
         const dim3 grid(((VH * SW + 255) / 256 + SHADE_TILES - 1) / SHADE_TILES, count);
         if (decals) hipLaunchKernelGGL(plane_shade_kernel<true>, grid, dim3(256), 0, stream, r->dm, count, sc, frame_base, frame_stride);
@@ -3223,6 +3322,7 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     if (rc == GD_OK) rc = scratch_alloc(r, L * SW, &sc.cand_count);
     if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.flat_sector);
     if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.flat_flags);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * 4, &sc.flat_span);
     if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.meta);
     if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.clip_depth);
     if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)GD_SCREEN_HEIGHT * SW, &sc.frame);
