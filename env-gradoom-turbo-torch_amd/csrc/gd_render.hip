@@ -2128,10 +2128,6 @@ __global__ void __launch_bounds__(1024) strip_order_kernel(int strips, Scratch s
 // tables are paid once per group rather than once per wavefront (which would cap the CU at a
 // couple of wavefronts per SIMD).  After the staging barrier the wavefronts never meet again.
 #define WALL_STRIPS_PER_GROUP 1
-// Unused LDS that caps the kernel at two wavefronts per SIMD: its 166 registers per lane would
-// otherwise fill the register file with three, and the flat kernels on the side stream could not
-// run beside it at all.
-#define WALL_LDS_PAD 3072
 // DEPTH: also keep the depth of every wall pixel (frames that draw decals).  SPLIT: the map has linedefs with
 // BSP projection fragments.
 template <bool DEPTH, bool SPLIT>
@@ -3131,7 +3127,7 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
         const bool split = m.split_count > 0;
         auto kernel = decals ? (split ? wall_columns_kernel<true, true> : wall_columns_kernel<true, false>)
                              : (split ? wall_columns_kernel<false, true> : wall_columns_kernel<false, false>);
-        hipLaunchKernelGGL(kernel, grid, block, WALL_LDS_PAD, stream, r->dm, count, sc, frame_base, frame_stride);
+        hipLaunchKernelGGL(kernel, grid, block, 0, stream, r->dm, count, sc, frame_base, frame_stride);
     }
     mark();
     // the flat pass, where the walls left it something to decide
