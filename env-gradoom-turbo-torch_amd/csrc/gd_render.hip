@@ -144,6 +144,9 @@ struct Scratch {    // per-chunk working memory, sized at create
     int *cand_count;       // [L,320] (may exceed CAND_MAX when a list overflowed)
     unsigned short *flat_sector;// [L,208,320]
     unsigned char *flat_flags;  // [L,208,320] bit0 unresolved
+    int *flat_list;        // [L,FLAT_LIST_MAX] view pixels no wall tier, plane or masked texture covers: they show the
+                           // flat pass's picture.  Found by plane_shade_kernel.
+    int *flat_list_count;  // [L] how many there are (more than FLAT_LIST_MAX: the lane is handled pixel by pixel)
     int *flat_span;        // [L,4] first / last row of the ceiling half, then of the floor half, that holds a shown
                            // pixel the flat pass could not resolve (208, -1 = none): the rows the repairs work on
     unsigned int *meta;    // [L,208,320] filled | floor | plane_sector+1 | clip_wall+1
@@ -160,6 +163,7 @@ struct Scratch {    // per-chunk working memory, sized at create
     i64 *row_slope;        // [L, 208] plane distance per unit of plane height on each view row
     i64 *step_scale;       // [L, 2, 16] flat texture steps per column for every log2 texture size
 };
+#define FLAT_LIST_MAX 1024 // listed gap pixels per lane (a gap is typically one column wide)
 #define PLANE_LEVELS 64    // level lists up to this long are shaded from the per-lane tables
 
 #define META_FILLED 0x80000000u   // an opaque wall tier owns the pixel
@@ -456,6 +460,7 @@ __global__ void lane_setup_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_ba
     sc.ctx[local] = c;
     int *span = sc.flat_span + (size_t)local * 4;
     span[0] = VH; span[1] = -1; span[2] = VH; span[3] = -1;
+    sc.flat_list_count[local] = 0;
     for (int x = 0; x < SW; ++x) { sc.cand_count[(size_t)local * SW + x] = 0; sc.block_hit[(size_t)local * SW + x] = ~0ULL; }
 }
 
@@ -777,6 +782,7 @@ __device__ __forceinline__ int flat_select_pixel(const DeviceMap &dm, const Scra
     // farther than that from the camera is dropped for the whole wavefront at once
     const float reach_scale = dm.strip_reach_scale[__builtin_amdgcn_readfirstlane(x >> 6)];
     float best = GD_INF; int best_sector = -1;
+    const bool camera_in_grid = grid_cell_of(m, c.x, c.y) >= 0;
     bool done = !wanted;
     for (int base = 0; base < level_count; base += 64) {
         if (__ballot(!done) == 0) break;   // every lane takes part in the level broadcasts below, wanted or not
@@ -838,10 +844,10 @@ __device__ __forceinline__ int flat_select_pixel(const DeviceMap &dm, const Scra
                 const float px = c.x + rc * cd, py = c.y + rs * cd;
                 int cell = cellv[j];
                 if (cell < 0) cell = grid_cell_of(m, px, py);
-                // Outside the grid (above, below or right of every linedef) no sector holds the point, and the
-                // probe points of the levels still to come lie farther along the same ray, which has left
-                // that convex region for good.
-                if (cell < 0) { done = true; continue; }
+                // Outside the grid (above, below or right of every linedef) no sector holds the point.  Seen from a
+                // camera inside that convex region, the probe points of the levels still to come lie farther
+                // along the same ray, which has left the region for good.
+                if (cell < 0) { done = camera_in_grid; continue; }
                 const int2 range = dm.cell_range[cell];
                 for (int it = range.x; it < range.y; ++it) {
                     const int4 item = dm.cell_item[it];
@@ -859,39 +865,89 @@ __device__ __forceinline__ int flat_select_pixel(const DeviceMap &dm, const Scra
     return best_sector;
 }
 
-// The pass runs after the walls and only where its result can matter.  A pixel a wall tier filled never
+// One pixel's flat ray on its own (flat_select_pixel shares work between the 64 pixels of a row): the sector of
+// the nearest plane level whose probe point lies in a sector of that level, -1 if there is none
+// (engine.py:10981-11024).
+__device__ int flat_probe_pixel(const DeviceMap &dm, const LaneCtx &c, float rc, float rs, float cc, int y) {
+    const gd_map_desc *m = &dm.d;
+    const float delta = (float)y - flat_center(c);
+    const bool is_floor = delta > 0;
+    const float denom = fmaxf(fabsf(delta), 0.5f);
+    const float *levels = is_floor ? m->floor_levels : m->ceil_levels;
+    const int level_count = is_floor ? m->floor_level_count : m->ceil_level_count;
+    float best = GD_INF; int best_sector = -1;
+    const bool camera_in_grid = grid_cell_of(m, c.x, c.y) >= 0;
+    for (int k = 0; k < level_count; ++k) {
+        const float level = levels[k];
+        const float height = is_floor ? (c.view_z - level) : (level - c.view_z);
+        if (!(height > 0)) continue;
+        const float cd = (height * 192.0f / denom) / cc;
+        if (!(finitef(cd) && cd > 0)) continue;
+        if (cd > best) break;                                   // later levels are at least this far
+        const float px = c.x + rc * cd, py = c.y + rs * cd;
+        int cell;
+        const unsigned fine = fine_lookup(m, dm.fine_inverse, px, py, &cell);
+        const unsigned kind = FINE_KIND(fine);
+        if (kind == FINE_EMPTY) continue;
+        if (kind == FINE_DECIDED) {
+            const int s = (int)(fine & 0xFFFFu);
+            if (m->sector_heights[2 * s + (is_floor ? 0 : 1)] == level && (cd < best || (cd == best && s < best_sector))) { best = cd; best_sector = s; }
+            continue;
+        }
+        if (cell < 0) cell = grid_cell_of(m, px, py);
+        if (cell < 0) {                                         // outside the grid no sector holds the point
+            if (camera_in_grid) break;                          // and this ray has left that convex region for good
+            continue;
+        }
+        const int2 range = dm.cell_range[cell];
+        for (int it = range.x; it < range.y; ++it) {
+            const int4 item = dm.cell_item[it];
+            const int s = item.x & ~GRID_ALWAYS_INSIDE;
+            if (m->sector_heights[2 * s + (is_floor ? 0 : 1)] != level) continue;
+            if (cd < best || (cd == best && s < best_sector)) {
+                if ((item.x & GRID_ALWAYS_INSIDE) || inside_edge_copies(dm.cell_edge, item.z, item.w, px, py)) { best = cd; best_sector = s; }
+            }
+        }
+    }
+    return best_sector;
+}
+
+// The flat pass runs after the walls and only where its result can matter.  A pixel a wall tier filled never
 // shows it; a pixel a plane of the wall pass claimed only asks whether the flat ray resolved at all, and only
 // where a sprite stands behind the plane with no sprite clip recorded, which the sprite pass finds out for
 // itself (flat_ray_resolves); the few pixels left (columns whose traversal left a gap) show the flat pass's
-// picture.  This kernel handles exactly those pixels and notes, per lane and screen half, the rows where a shown
-// pixel stayed unresolved: flat_span_select_kernel and flat_span_finish_kernel select and repair those rows.
-__global__ void flat_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc,
-                                   unsigned char *frame_base, size_t frame_stride) {
-    const gd_map_desc *m = &dm.d;
-    int local = blockIdx.y;
-    int pixel = blockIdx.x * blockDim.x + threadIdx.x;
-    if (local >= lane_count || pixel >= VH * SW) return;
-    if (pixel < (GD_SCREEN_HEIGHT - VH) * SW)   // the empty status bar, rows 208..239
-        frame_base[(size_t)local * frame_stride + (size_t)VH * SW + pixel] = 0;
-    const int y = pixel / SW, x = pixel - y * SW;
-    const int n = lane_base + local;
-    const size_t i = (size_t)local * VH * SW + pixel;
-    const unsigned meta_word = sc.meta[i];
-    const bool filled = meta_word & META_FILLED;
-    const int plane = (int)((meta_word >> META_SECTOR_SHIFT) & META_SECTOR_MASK) - 1;
-    const bool shown = !filled && plane < 0 && !(meta_word & META_MASKED);
-    if (__ballot(shown) == 0) return;              // the whole wavefront (64 pixels of one row) has nothing to find
-    const bool wanted = shown;
-    const int best_sector = flat_select_pixel(dm, sc, lanes, local, n, x, y, wanted);
-    if (wanted) {
-        sc.flat_sector[i] = (unsigned short)(best_sector < 0 ? sc.ctx[local].sector : best_sector);
-        sc.flat_flags[i] = best_sector < 0 ? 1 : 0;
+// picture.  plane_shade_kernel lists those; this kernel selects them, one thread per listed pixel, and notes,
+// per lane and screen half, the rows where one stayed unresolved: flat_span_select_kernel and
+// flat_span_finish_kernel select and repair those rows, flat_shade_kernel paints the listed pixels.
+__global__ void __launch_bounds__(64) flat_list_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
+    const int local = blockIdx.y;
+    if (local >= lane_count) return;
+    const int listed = sc.flat_list_count[local];
+    const int slot = blockIdx.x * blockDim.x + threadIdx.x;
+    const LaneCtx &c = sc.ctx[local];
+    int *span = sc.flat_span + (size_t)local * 4;
+    if (listed > FLAT_LIST_MAX) {
+        // too many to list (a camera outside the map, say): every row of both halves is selected and repaired
+        if (slot == 0) {
+            int last_ceiling_row = -1;
+            for (int y = 0; y < VH; ++y) if (!(((float)y - flat_center(c)) > 0)) last_ceiling_row = y;
+            if (last_ceiling_row >= 0) { span[0] = 0; span[1] = last_ceiling_row; }
+            if (last_ceiling_row + 1 < VH) { span[2] = last_ceiling_row + 1; span[3] = VH - 1; }
+        }
+        return;
     }
-    if (__ballot(shown && best_sector < 0) != 0 && (threadIdx.x & 63) == 0) {
-        const bool floor_row = ((float)y - flat_center(sc.ctx[local])) > 0;
-        int *span = sc.flat_span + (size_t)local * 4 + (floor_row ? 2 : 0);
-        atomicMin(&span[0], y);
-        atomicMax(&span[1], y);
+    if (slot >= listed) return;
+    const int n = lane_base + local;
+    const int pixel = sc.flat_list[(size_t)local * FLAT_LIST_MAX + slot];
+    const int y = pixel / SW, x = pixel - y * SW;
+    const int s = flat_probe_pixel(dm, c, lanes.ray_cos[(size_t)n * SW + x], lanes.ray_sin[(size_t)n * SW + x], dm.cosine_correction[x], y);
+    const size_t i = (size_t)local * VH * SW + pixel;
+    sc.flat_sector[i] = (unsigned short)(s < 0 ? c.sector : s);
+    sc.flat_flags[i] = s < 0 ? 1 : 0;
+    if (s < 0) {
+        const bool floor_row = ((float)y - flat_center(c)) > 0;
+        atomicMin(&span[floor_row ? 2 : 0], y);
+        atomicMax(&span[floor_row ? 3 : 1], y);
     }
 }
 
@@ -2285,27 +2341,28 @@ __global__ void __launch_bounds__(256) plane_shade_kernel(DeviceMap dm, int lane
     // SHADE_GROUP tiles per step and three stages per step (per-pixel words, texels, stores), each
     // stage's loads issued together so that their latencies overlap
     for (int tile0 = 0; tile0 < SHADE_TILES; tile0 += SHADE_GROUP) {
-        unsigned int meta[SHADE_GROUP]; unsigned short flat_sector[SHADE_GROUP]; unsigned char flat_flags[SHADE_GROUP];
+        unsigned int meta[SHADE_GROUP];
         int pixels[SHADE_GROUP];
 #pragma unroll
         for (int j = 0; j < SHADE_GROUP; ++j) {
             const int pixel = (blockIdx.x * SHADE_TILES + tile0 + j) * 256 + threadIdx.x;
             pixels[j] = (tile0 + j < SHADE_TILES && pixel < VH * SW) ? pixel : -1;
             const size_t i = (size_t)local * VH * SW + (pixels[j] < 0 ? 0 : pixels[j]);
-            meta[j] = sc.meta[i]; flat_sector[j] = sc.flat_sector[i]; flat_flags[j] = sc.flat_flags[i];
+            meta[j] = sc.meta[i];
+            if (pixels[j] >= 0 && pixels[j] < (GD_SCREEN_HEIGHT - VH) * SW) frame[(size_t)VH * SW + pixels[j]] = 0;   // the empty status bar, rows 208..239
         }
         size_t texel_at[SHADE_GROUP]; int colormap_row[SHADE_GROUP]; unsigned char texel[SHADE_GROUP];
         bool shade[SHADE_GROUP];
 #pragma unroll
         for (int j = 0; j < SHADE_GROUP; ++j) {
             const int pixel = pixels[j];
-            shade[j] = tabled && pixel >= 0 && !(meta[j] & (META_FILLED | META_MASKED));
+            const int ps = (int)((meta[j] >> META_SECTOR_SHIFT) & META_SECTOR_MASK) - 1;
+            shade[j] = tabled && pixel >= 0 && ps >= 0 && !(meta[j] & (META_FILLED | META_MASKED));
             texel[j] = 0; colormap_row[j] = 0; texel_at[j] = 0;
             if (!shade[j]) continue;
             const int y = pixel / SW, x = pixel - y * SW;
-            const int ps = (int)((meta[j] >> META_SECTOR_SHIFT) & META_SECTOR_MASK) - 1;
-            const bool is_floor = ps >= 0 ? (meta[j] & META_FLOOR) != 0 : ((float)y - flat_center(c)) > 0;
-            const int sector = ps >= 0 ? ps : (int)flat_sector[j];
+            const bool is_floor = (meta[j] & META_FLOOR) != 0;
+            const int sector = ps;
             const unsigned short pair = sector < tb.sector_cached ? sector_level_lds[sector] : dm.sector_level[sector];
             texel_at[j] = flat_sample_tabled(tb, c, lt, sc.row_slope[(size_t)local * VH + y], is_floor ? (pair & 0xFF) : (pair >> 8),
                                              sector, is_floor, x, y, &colormap_row[j]);
@@ -2318,29 +2375,66 @@ __global__ void __launch_bounds__(256) plane_shade_kernel(DeviceMap dm, int lane
             const int y = pixel / SW, x = pixel - y * SW;
             const size_t i = (size_t)local * VH * SW + pixel;
             const int ps = (int)((meta[j] >> META_SECTOR_SHIFT) & META_SECTOR_MASK) - 1;
-            const bool claimed = ps >= 0;
-            const bool is_floor = claimed ? (meta[j] & META_FLOOR) != 0 : ((float)y - flat_center(c)) > 0;
-            if (shade[j]) frame[pixel] = colormap_lds[colormap_row[j] * 256 + texel[j]];
-            else if (!(meta[j] & META_MASKED)) frame[pixel] = flat_pixel(tb, colormap_lds, c, claimed ? ps : (int)flat_sector[j], is_floor, x, y);
-            if (DEPTH && !(meta[j] & META_MASKED)) {
-                float depth;
-                if (claimed) {   // exact plane depth (engine.py:13406-13416)
-                    const float flat_center_px = (103.0f + c.pitch_offset) + 0.5f;
-                    const float plane_height = is_floor ? (c.view_z - tb.floor_h(ps)) : (tb.ceil_h(ps) - c.view_z);
-                    depth = plane_height * 192.0f / fmaxf(fabsf((float)y - flat_center_px), 0.5f);
-                } else {         // what the flat pass left (engine.py:11140-11166)
-                    const int s = flat_sector[j];
-                    const float delta = (float)y - flat_center(c);
-                    const float plane_height = delta > 0 ? (c.view_z - tb.floor_h(s)) : (tb.ceil_h(s) - c.view_z);
-                    const float perpendicular = plane_height * 192.0f / fmaxf(fabsf(delta), 0.5f);
-                    const float cosine = dm.cosine_correction[x];
-                    if (flat_flags[j] & (2 | 8)) depth = perpendicular;             // repaired: its visplane's depth
-                    else if (flat_flags[j] & 1) depth = GD_INF;                    // no sector found along the ray
-                    else depth = (perpendicular / cosine) * cosine;                // ray distance of the hit, corrected back
+            if (ps < 0) {
+                // neither tier nor plane: the flat pass's picture shows here (unless a masked texture covers it);
+                // flat_shade_kernel paints the pixel once that pass has run
+                if (!(meta[j] & META_MASKED)) {
+                    const int slot = atomicAdd(&sc.flat_list_count[local], 1);
+                    if (slot < FLAT_LIST_MAX) sc.flat_list[(size_t)local * FLAT_LIST_MAX + slot] = pixel;
                 }
-                sc.scene_depth[i] = depth;
+                continue;
+            }
+            const bool is_floor = (meta[j] & META_FLOOR) != 0;
+            if (shade[j]) frame[pixel] = colormap_lds[colormap_row[j] * 256 + texel[j]];
+            else if (!(meta[j] & META_MASKED)) frame[pixel] = flat_pixel(tb, colormap_lds, c, ps, is_floor, x, y);
+            if (DEPTH && !(meta[j] & META_MASKED)) {   // exact plane depth (engine.py:13406-13416)
+                const float flat_center_px = (103.0f + c.pitch_offset) + 0.5f;
+                const float plane_height = is_floor ? (c.view_z - tb.floor_h(ps)) : (tb.ceil_h(ps) - c.view_z);
+                sc.scene_depth[i] = plane_height * 192.0f / fmaxf(fabsf((float)y - flat_center_px), 0.5f);
             }
         }
+    }
+}
+
+// The listed gap pixels, painted with the flat the flat pass settled on (engine.py:11145-11163); frames that
+// draw decals also keep the depth that pass leaves there (engine.py:11140-11166).
+__device__ void flat_shade_pixel(const DeviceMap &dm, const Scratch &sc, const LaneCtx &c, int local, int pixel, unsigned char *frame) {
+    const gd_map_desc *m = &dm.d;
+    Tables tb; tb.m = m; tb.sector = nullptr; tb.tex_bits = nullptr; tb.sector_cached = 0; tb.tex_cached = 0;
+    const int y = pixel / SW, x = pixel - y * SW;
+    const size_t i = (size_t)local * VH * SW + pixel;
+    const int s = sc.flat_sector[i];
+    const float delta = (float)y - flat_center(c);
+    frame[pixel] = flat_pixel(tb, m->colormap, c, s, delta > 0, x, y);
+    if (sc.scene_depth) {
+        const unsigned char flags = sc.flat_flags[i];
+        const float plane_height = delta > 0 ? (c.view_z - tb.floor_h(s)) : (tb.ceil_h(s) - c.view_z);
+        const float perpendicular = plane_height * 192.0f / fmaxf(fabsf(delta), 0.5f);
+        const float cosine = dm.cosine_correction[x];
+        float depth;
+        if (flags & (2 | 8)) depth = perpendicular;             // repaired: its visplane's depth
+        else if (flags & 1) depth = GD_INF;                    // no sector found along the ray
+        else depth = (perpendicular / cosine) * cosine;        // ray distance of the hit, corrected back
+        sc.scene_depth[i] = depth;
+    }
+}
+
+__global__ void __launch_bounds__(64) flat_shade_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
+    const int local = blockIdx.y;
+    if (local >= lane_count) return;
+    const int listed = sc.flat_list_count[local];
+    const LaneCtx &c = sc.ctx[local];
+    unsigned char *frame = frame_base + (size_t)local * frame_stride;
+    const int slot = blockIdx.x * blockDim.x + threadIdx.x;
+    if (listed <= FLAT_LIST_MAX) {
+        if (slot < listed) flat_shade_pixel(dm, sc, c, local, sc.flat_list[(size_t)local * FLAT_LIST_MAX + slot], frame);
+        return;
+    }
+    // a lane with more gap pixels than the list holds: every pixel is looked at
+    for (int pixel = slot; pixel < VH * SW; pixel += gridDim.x * blockDim.x) {
+        const unsigned int meta = sc.meta[(size_t)local * VH * SW + pixel];
+        if (!(meta & (META_FILLED | META_MASKED)) && ((meta >> META_SECTOR_SHIFT) & META_SECTOR_MASK) == 0)
+            flat_shade_pixel(dm, sc, c, local, pixel, frame);
     }
 }
 
@@ -3130,17 +3224,18 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
         hipLaunchKernelGGL(kernel, grid, block, 0, stream, r->dm, count, sc, frame_base, frame_stride);
     }
     mark();
-    // the flat pass, where the walls left it something to decide
-    hipLaunchKernelGGL(flat_select_kernel, dim3((VH * SW + 255) / 256, count), dim3(256), 0, stream, r->dm, *lanes, base, count, sc, frame_base, frame_stride);
-    mark();
-    hipLaunchKernelGGL(flat_span_select_kernel, dim3(SPAN_ROW_SLOTS, count), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
-    hipLaunchKernelGGL(flat_span_finish_kernel, dim3(count), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
-    mark();
     {
         const dim3 grid(((VH * SW + 255) / 256 + SHADE_TILES - 1) / SHADE_TILES, count);
         if (decals) hipLaunchKernelGGL(plane_shade_kernel<true>, grid, dim3(256), 0, stream, r->dm, count, sc, frame_base, frame_stride);
         else hipLaunchKernelGGL(plane_shade_kernel<false>, grid, dim3(256), 0, stream, r->dm, count, sc, frame_base, frame_stride);
     }
+    mark();
+    // the flat pass, where the walls left it something to decide
+    hipLaunchKernelGGL(flat_list_kernel, dim3(FLAT_LIST_MAX / 64, count), dim3(64), 0, stream, r->dm, *lanes, base, count, sc);
+    hipLaunchKernelGGL(flat_span_select_kernel, dim3(SPAN_ROW_SLOTS, count), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
+    mark();
+    hipLaunchKernelGGL(flat_span_finish_kernel, dim3(count), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
+    hipLaunchKernelGGL(flat_shade_kernel, dim3(FLAT_LIST_MAX / 64, count), dim3(64), 0, stream, r->dm, count, sc, frame_base, frame_stride);
     mark();
     if (decals)
         hipLaunchKernelGGL(decal_kernel, dim3(count), dim3(SW), 0, stream, r->dm, r->overlays, *lanes, base, count, sc, frame_base, frame_stride);
@@ -3319,6 +3414,8 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.flat_sector);
     if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.flat_flags);
     if (rc == GD_OK) rc = scratch_alloc(r, L * 4, &sc.flat_span);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * FLAT_LIST_MAX, &sc.flat_list);
+    if (rc == GD_OK) rc = scratch_alloc(r, L, &sc.flat_list_count);
     if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.meta);
     if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.clip_depth);
     if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)GD_SCREEN_HEIGHT * SW, &sc.frame);

@@ -61,3 +61,40 @@ def test_random_maps_and_grazing_poses_match_the_oracle(oracle, first_seed):
         assert np.array_equal(indexed.cpu().numpy(), expected["indexed"]), f"seed {seed}"
         assert np.array_equal(obs.cpu().numpy(), expected["obs"]), f"seed {seed}"
         renderer.close()
+
+
+def test_cameras_outside_the_map_match_the_oracle(oracle):
+    """Cameras in the void beside the map: no wall pass claims most of the screen, so nearly every pixel shows the
+    flat pass's picture (far more than the per-lane gap pixel list holds) and most of them stay unresolved."""
+    from gradoom_amd import hostmath, mapbuild, synthmap
+    from gradoom_amd.renderer import HipRenderer, LaneState
+    from gradoom_amd.selfcheck import make_lane_arrays
+
+    cosine = hostmath.cosine_correction("cpu").numpy()
+    smap = synthmap.generate_map(7001, grid=(5, 4), sectors=17, linedefs=140, layout="grid", islands=4, pillars=2, midtex=0.1)
+    tables = mapbuild.build_map_tables(smap)
+    poses = synthmap.generate_poses(smap, LANES, 11, pitch=True)
+    segments = np.asarray(smap.wall_segments, dtype=np.float64)
+    low = np.array([segments[:, [0, 2]].min(), segments[:, [1, 3]].min()])
+    high = np.array([segments[:, [0, 2]].max(), segments[:, [1, 3]].max()])
+    rng = np.random.default_rng(5)
+    for lane in range(LANES):
+        along, away = rng.uniform(0.1, 0.9), rng.uniform(8, 200)
+        side = lane % 4
+        if side < 2:
+            poses.x[lane] = low[0] - away if side == 0 else high[0] + away
+            poses.y[lane] = low[1] + along * (high[1] - low[1])
+        else:
+            poses.x[lane] = low[0] + along * (high[0] - low[0])
+            poses.y[lane] = low[1] - away if side == 2 else high[1] + away
+    arrays = make_lane_arrays(smap, poses, synthmap.generate_sprites(smap, LANES, 24, 12))
+    expected = oracle.render(tables, arrays, cosine)
+    renderer = HipRenderer(smap, LANES, "cuda:0", cosine_correction=cosine, tables=tables)
+    indexed = torch.zeros((LANES, 240, 320), dtype=torch.uint8, device="cuda:0")
+    obs = torch.zeros((LANES, 84, 84), dtype=torch.uint8, device="cuda:0")
+    renderer.render(LaneState.from_numpy(arrays, "cuda:0"), indexed=indexed, obs=obs)
+    torch.cuda.synchronize()
+    assert renderer.status() == 0
+    assert np.array_equal(indexed.cpu().numpy(), expected["indexed"])
+    assert np.array_equal(obs.cpu().numpy(), expected["obs"])
+    renderer.close()
