@@ -112,6 +112,7 @@ struct DeviceMap {  // device copy of gd_map_desc (device pointers) + fixed tabl
     const float *cosine_correction;  // [320] cos(native_ray_offsets), supplied by the host
     const float *inverse_cosine;     // [320] 1 / cosine_correction, correctly rounded
     float strip_reach_scale[SW / 64];// per 64-column strip: 1.001 / (its smallest cosine_correction), inf if not positive
+    float strip_far_scale[SW / 64];  // per 64-column strip: 0.999 / (its largest cosine_correction), 0 if any is not positive
     float fine_inverse;              // 1 / fine_cell
     // Sectors grouped by plane level, floors (in floor_levels order) then ceilings: CSR over
     // floor_level_count + ceil_level_count rows into level_boxes, one padded bounding box
@@ -147,6 +148,8 @@ struct Scratch {    // per-chunk working memory, sized at create
     int *flat_list;        // [L,FLAT_LIST_MAX] view pixels no wall tier, plane or masked texture covers: they show the
                            // flat pass's picture.  Found by plane_shade_kernel.
     int *flat_list_count;  // [L] how many there are (more than FLAT_LIST_MAX: the lane is handled pixel by pixel)
+    int *flat_tail;        // [L,2,320] per screen half and column: the sector of the first resolved pixel below the
+                           // half's noted rows, -1 if the column was not looking for one or found none
     int *flat_span;        // [L,4] first / last row of the ceiling half, then of the floor half, that holds a shown
                            // pixel the flat pass could not resolve (208, -1 = none): the rows the repairs work on
     unsigned int *meta;    // [L,208,320] filled | floor | plane_sector+1 | clip_wall+1
@@ -159,6 +162,7 @@ struct Scratch {    // per-chunk working memory, sized at create
     int *status;           // [1] sticky overflow flags
     float *level_reach;    // [L, floor levels + ceiling levels] lower bound of the distance from the
                            // camera to any point inside a sector with that plane level
+    float *level_far;      // [L, floor levels + ceiling levels] upper bound of that distance
     i64 *level_plane;      // [L, floor levels + ceiling levels, 2] plane height (16.16) and its visibility factor
     i64 *row_slope;        // [L, 208] plane distance per unit of plane height on each view row
     i64 *step_scale;       // [L, 2, 16] flat texture steps per column for every log2 texture size
@@ -390,14 +394,17 @@ __global__ void lane_tables_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
     const LaneCtx &c = sc.ctx[local];
     const float cx = lanes.x[lane_base + local], cy = lanes.y[lane_base + local];
     for (int l = threadIdx.x; l < levels; l += blockDim.x) {
-        float reach = GD_INF;
+        float reach = GD_INF, far = 0.0f;
         for (int k = dm.level_box_ofs[l]; k < dm.level_box_ofs[l + 1]; ++k) {
             const float4 box = dm.level_boxes[k];
             float dx = fmaxf(fmaxf(box.x - cx, cx - box.z), 0.0f), dy = fmaxf(fmaxf(box.y - cy, cy - box.w), 0.0f);
             reach = fminf(reach, sqrtf(dx * dx + dy * dy));
+            dx = fmaxf(fabsf(box.x - cx), fabsf(box.z - cx)); dy = fmaxf(fabsf(box.y - cy), fabsf(box.w - cy));
+            far = fmaxf(far, sqrtf(dx * dx + dy * dy));
         }
         // margin: the probe point is camera + unit ray * distance in float32, far inside 0.1%
         sc.level_reach[(size_t)local * levels + l] = reach * 0.999f - 0.5f;
+        sc.level_far[(size_t)local * levels + l] = far * 1.001f + 0.5f;
         const float plane_height = l < floors ? (c.view_z - dm.d.floor_levels[l]) : (dm.d.ceil_levels[l - floors] - c.view_z);
         const i64 plane_height_fixed = round_to_i64(plane_height * 65536.0f);
         sc.level_plane[((size_t)local * levels + l) * 2] = plane_height_fixed;
@@ -767,6 +774,7 @@ __device__ __forceinline__ int flat_select_pixel(const DeviceMap &dm, const Scra
     const int mask_shift = floor_uniform ? 0 : FINE_MASK_LEVELS;
     const int index_shift = floor_uniform ? 16 : 20;
     const float *reach = sc.level_reach + (size_t)local * (m->floor_level_count + m->ceil_level_count) + (floor_uniform ? 0 : m->floor_level_count);
+    const float *far = sc.level_far + (size_t)local * (m->floor_level_count + m->ceil_level_count) + (floor_uniform ? 0 : m->floor_level_count);
     // cd = perpendicular / cc below is the hot division.  With y = RN(1 / cc), q = RN(p * y) is within
     // one ulp of p / cc, and RN(q + RN(p - cc * q) * y) is then the correctly rounded quotient
     // (Markstein's theorem; the inner product is exact in an FMA) as long as nothing over- or
@@ -781,6 +789,8 @@ __device__ __forceinline__ int flat_select_pixel(const DeviceMap &dm, const Scra
     // cd <= perpendicular / (smallest cc of the wavefront): with it a level whose every sector is
     // farther than that from the camera is dropped for the whole wavefront at once
     const float reach_scale = dm.strip_reach_scale[__builtin_amdgcn_readfirstlane(x >> 6)];
+    // and cd >= perpendicular / (largest cc of the wavefront): a level whose every sector ends nearer than that
+    const float far_scale = dm.strip_far_scale[__builtin_amdgcn_readfirstlane(x >> 6)];
     float best = GD_INF; int best_sector = -1;
     const bool camera_in_grid = grid_cell_of(m, c.x, c.y) >= 0;
     bool done = !wanted;
@@ -791,6 +801,7 @@ __device__ __forceinline__ int flat_select_pixel(const DeviceMap &dm, const Scra
         const int mine = base + slot_in_wave;
         const float my_level = mine < level_count ? levels[mine] : 0.0f;
         const float my_reach = mine < level_count ? reach[mine] : 0.0f;
+        const float my_far = mine < level_count ? far[mine] : GD_INF;
         const float my_height = floor_uniform ? (c.view_z - my_level) : (my_level - c.view_z);
         const float my_perpendicular = (mine < level_count && my_height > 0) ? my_height * 192.0f / denom : -1.0f;
         const int chunk = level_count - base < 64 ? level_count - base : 64;
@@ -810,6 +821,7 @@ __device__ __forceinline__ int flat_select_pixel(const DeviceMap &dm, const Scra
                 const float nearest = bcast(my_reach, k);
                 if (!(perpendicular > 0)) continue;              // the same in every lane
                 if (perpendicular * reach_scale < nearest) continue;   // the same in every lane: no lane can reach the level
+                if (perpendicular * far_scale > bcast(my_far, k)) continue;   // the same in every lane: every lane looks past the level
                 float cd;
                 if (cc_plain && perpendicular >= 1e-18f && perpendicular <= 1e18f) {
                     const float q = perpendicular * inv_cc;
@@ -868,13 +880,17 @@ __device__ __forceinline__ int flat_select_pixel(const DeviceMap &dm, const Scra
 // One pixel's flat ray on its own (flat_select_pixel shares work between the 64 pixels of a row): the sector of
 // the nearest plane level whose probe point lies in a sector of that level, -1 if there is none
 // (engine.py:10981-11024).
-__device__ int flat_probe_pixel(const DeviceMap &dm, const LaneCtx &c, float rc, float rs, float cc, int y) {
+__device__ int flat_probe_pixel(const DeviceMap &dm, const Scratch &sc, int local, float rc, float rs, float cc, int y) {
+    const LaneCtx &c = sc.ctx[local];
     const gd_map_desc *m = &dm.d;
     const float delta = (float)y - flat_center(c);
     const bool is_floor = delta > 0;
     const float denom = fmaxf(fabsf(delta), 0.5f);
     const float *levels = is_floor ? m->floor_levels : m->ceil_levels;
     const int level_count = is_floor ? m->floor_level_count : m->ceil_level_count;
+    // per lane and level: bounds of the distance from the camera to the sectors of that level
+    const size_t bounds_at = (size_t)local * (m->floor_level_count + m->ceil_level_count) + (is_floor ? 0 : m->floor_level_count);
+    const float *reach = sc.level_reach + bounds_at, *far = sc.level_far + bounds_at;
     float best = GD_INF; int best_sector = -1;
     const bool camera_in_grid = grid_cell_of(m, c.x, c.y) >= 0;
     for (int k = 0; k < level_count; ++k) {
@@ -884,6 +900,7 @@ __device__ int flat_probe_pixel(const DeviceMap &dm, const LaneCtx &c, float rc,
         const float cd = (height * 192.0f / denom) / cc;
         if (!(finitef(cd) && cd > 0)) continue;
         if (cd > best) break;                                   // later levels are at least this far
+        if (cd < reach[k] || cd > far[k]) continue;            // no sector of this level lies at that distance
         const float px = c.x + rc * cd, py = c.y + rs * cd;
         int cell;
         const unsigned fine = fine_lookup(m, dm.fine_inverse, px, py, &cell);
@@ -919,16 +936,15 @@ __device__ int flat_probe_pixel(const DeviceMap &dm, const LaneCtx &c, float rc,
 // picture.  plane_shade_kernel lists those; this kernel selects them, one thread per listed pixel, and notes,
 // per lane and screen half, the rows where one stayed unresolved: flat_span_select_kernel and
 // flat_span_finish_kernel select and repair those rows, flat_shade_kernel paints the listed pixels.
-__global__ void __launch_bounds__(64) flat_list_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
-    const int local = blockIdx.y;
+__global__ void __launch_bounds__(128) flat_list_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
+    const int local = blockIdx.x;
     if (local >= lane_count) return;
     const int listed = sc.flat_list_count[local];
-    const int slot = blockIdx.x * blockDim.x + threadIdx.x;
     const LaneCtx &c = sc.ctx[local];
     int *span = sc.flat_span + (size_t)local * 4;
     if (listed > FLAT_LIST_MAX) {
         // too many to list (a camera outside the map, say): every row of both halves is selected and repaired
-        if (slot == 0) {
+        if (threadIdx.x == 0) {
             int last_ceiling_row = -1;
             for (int y = 0; y < VH; ++y) if (!(((float)y - flat_center(c)) > 0)) last_ceiling_row = y;
             if (last_ceiling_row >= 0) { span[0] = 0; span[1] = last_ceiling_row; }
@@ -936,18 +952,19 @@ __global__ void __launch_bounds__(64) flat_list_kernel(DeviceMap dm, gd_lanes_de
         }
         return;
     }
-    if (slot >= listed) return;
     const int n = lane_base + local;
-    const int pixel = sc.flat_list[(size_t)local * FLAT_LIST_MAX + slot];
-    const int y = pixel / SW, x = pixel - y * SW;
-    const int s = flat_probe_pixel(dm, c, lanes.ray_cos[(size_t)n * SW + x], lanes.ray_sin[(size_t)n * SW + x], dm.cosine_correction[x], y);
-    const size_t i = (size_t)local * VH * SW + pixel;
-    sc.flat_sector[i] = (unsigned short)(s < 0 ? c.sector : s);
-    sc.flat_flags[i] = s < 0 ? 1 : 0;
-    if (s < 0) {
-        const bool floor_row = ((float)y - flat_center(c)) > 0;
-        atomicMin(&span[floor_row ? 2 : 0], y);
-        atomicMax(&span[floor_row ? 3 : 1], y);
+    for (int slot = threadIdx.x; slot < listed; slot += blockDim.x) {
+        const int pixel = sc.flat_list[(size_t)local * FLAT_LIST_MAX + slot];
+        const int y = pixel / SW, x = pixel - y * SW;
+        const int s = flat_probe_pixel(dm, sc, local, lanes.ray_cos[(size_t)n * SW + x], lanes.ray_sin[(size_t)n * SW + x], dm.cosine_correction[x], y);
+        const size_t i = (size_t)local * VH * SW + pixel;
+        sc.flat_sector[i] = (unsigned short)(s < 0 ? c.sector : s);
+        sc.flat_flags[i] = s < 0 ? 1 : 0;
+        if (s < 0) {
+            const bool floor_row = ((float)y - flat_center(c)) > 0;
+            atomicMin(&span[floor_row ? 2 : 0], y);
+            atomicMax(&span[floor_row ? 3 : 1], y);
+        }
     }
 }
 
@@ -1076,7 +1093,7 @@ __device__ __forceinline__ size_t flat_sample_tabled(const Tables &tb, const Lan
 // one has found it.  Horizontal: an unresolved pixel between a left and a right anchor of one sector takes
 // that sector.  Pixels outside the noted rows need none of this: no shown pixel there is unresolved, and
 // resolved pixels are never repaired.
-#define SPAN_ROW_SLOTS 16
+#define SPAN_ROW_SLOTS 8
 // Every pixel of the noted rows, block j of a lane taking rows j, j + SPAN_ROW_SLOTS, ... of both ranges.
 __global__ void __launch_bounds__(SW) flat_span_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
     const int local = blockIdx.y;
@@ -1092,6 +1109,47 @@ __global__ void __launch_bounds__(SW) flat_span_select_kernel(DeviceMap dm, gd_l
         const size_t i = (size_t)local * VH * SW + (size_t)y * SW + x;
         sc.flat_sector[i] = (unsigned short)(s < 0 ? sc.ctx[local].sector : s);
         sc.flat_flags[i] = s < 0 ? 1 : 0;
+    }
+}
+
+// A column whose pixel in the last noted row of a half is unresolved looks further down for a resolved one
+// (engine.py:11026-11083).  One block per (lane, 64-column strip); its TAIL_ROWS wavefronts select that many rows
+// at a time, while any of the strip's columns is still looking.
+#define TAIL_ROWS 4
+__global__ void __launch_bounds__(64 * TAIL_ROWS) flat_tail_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
+    __shared__ int found_lds[TAIL_ROWS][64];
+    const int local = blockIdx.y;
+    if (local >= lane_count) return;
+    const int *span = sc.flat_span + (size_t)local * 4;
+    const int lo[2] = {span[0], span[2]}, hi[2] = {span[1], span[3]};
+    if (hi[0] < lo[0] && hi[1] < lo[1]) return;      // the same in every thread
+    const int n = lane_base + local;
+    const int slot = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int x = blockIdx.x * 64 + slot;
+    const float center = flat_center(sc.ctx[local]);
+    int last_ceiling_row = -1;                       // rows 0 .. last_ceiling_row look at ceilings
+    for (int y = 0; y < VH; ++y) if (!(((float)y - center) > 0)) last_ceiling_row = y;
+    for (int half = 0; half < 2; ++half) {
+        if (hi[half] < lo[half]) continue;           // the same in every thread
+        const int half_end = half ? VH - 1 : last_ceiling_row;
+        bool looking = sc.flat_flags[(size_t)local * VH * SW + (size_t)hi[half] * SW + x] & 1;
+        int found = -1;
+        for (int y0 = hi[half] + 1; y0 <= half_end; y0 += TAIL_ROWS) {
+            if (!__syncthreads_or(looking)) break;   // also keeps the rows of the previous step apart from this one's
+            const int y = y0 + wave;
+            int s = -1;
+            if (y <= half_end) s = flat_select_pixel(dm, sc, lanes, local, n, x, y, looking);   // the same in a whole wavefront
+            found_lds[wave][slot] = s;
+            __syncthreads();
+            if (looking) {
+                for (int j = 0; j < TAIL_ROWS; ++j) {
+                    const int below = found_lds[j][slot];
+                    if (below >= 0) { looking = false; found = below; break; }
+                }
+            }
+        }
+        __syncthreads();
+        if (wave == 0) sc.flat_tail[((size_t)local * 2 + half) * SW + x] = found;
     }
 }
 
@@ -1113,15 +1171,10 @@ __global__ void __launch_bounds__(SW) flat_span_finish_kernel(DeviceMap dm, gd_l
     for (int half = 0; half < 2; ++half) {
         if (hi[half] < lo[half]) continue;           // the same in every thread
         const int half_end = half ? VH - 1 : last_ceiling_row;
-        // a column whose pixel in the range's last row is unresolved looks further down for a resolved one;
-        // each wavefront goes on, a row at a time, while any of its 64 columns is still looking
-        bool looking = flags[(size_t)hi[half] * SW + x] & 1;
-        bool found = false;
-        int span_sector = 0;
-        for (int y = hi[half] + 1; y <= half_end && __ballot(looking) != 0; ++y) {
-            const int s = flat_select_pixel(dm, sc, lanes, local, n, x, y, looking);
-            if (looking && s >= 0) { looking = false; found = true; span_sector = s; }
-        }
+        // what flat_tail_kernel found below the range for a column whose pixel in the range's last row is unresolved
+        const int below = sc.flat_tail[((size_t)local * 2 + half) * SW + x];
+        bool found = below >= 0;
+        int span_sector = found ? below : 0;
         for (int y = hi[half]; y >= lo[half]; --y) {
             const size_t i = (size_t)y * SW + x;
             if (!(flags[i] & 1)) { found = true; span_sector = sector[i]; }
@@ -1676,7 +1729,7 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
 struct PixelBuffers {
     unsigned char *frame;   // [240][320]
     unsigned int *meta;     // [208][320]
-    float *clip_depth;      // [208][320]
+    float *clip_depth;      // [208][320], only meaningful where the meta word names a clip linedef
     float *scene_depth;     // [208][320] or null
 };
 
@@ -1697,6 +1750,7 @@ __device__ __forceinline__ void clip_rows(PixelBuffers &pb, int x, int first, in
         for (int j = 0; j < WALL_ROWS; ++j) {
             const size_t i = (size_t)(y0 + j < last ? y0 + j : last - 1) * SW + x;
             held[j] = pb.clip_depth[i]; meta[j] = pb.meta[i];
+            if (!(meta[j] & META_WALL_MASK)) held[j] = GD_INF;   // no clip recorded yet
         }
 #pragma unroll
         for (int j = 0; j < WALL_ROWS; ++j) {
@@ -1855,7 +1909,8 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
                 unsigned char texel = m->tex_atlas[((size_t)texture_id * m->tex_max_h + tv) * m->tex_max_w + tu];
                 pb.frame[i] = colormap[(bottom_tail ? shade_group : shade_own) * 256 + texel];
                 if (DEPTH) pb.scene_depth[i] = r.distance;
-                if (r.distance < pb.clip_depth[i]) { pb.clip_depth[i] = r.distance; meta = (meta & ~META_WALL_MASK) | (unsigned)(wi + 1); }
+                const float held = (meta & META_WALL_MASK) ? pb.clip_depth[i] : GD_INF;   // no clip recorded yet
+                if (r.distance < held) { pb.clip_depth[i] = r.distance; meta = (meta & ~META_WALL_MASK) | (unsigned)(wi + 1); }
                 meta |= META_FILLED;
                 meta_dirty = true;
             }
@@ -2221,7 +2276,7 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
     pb.meta = sc.meta + (size_t)local * VH * SW;
     pb.clip_depth = sc.clip_depth + (size_t)local * VH * SW;
     pb.scene_depth = DEPTH ? sc.scene_depth + (size_t)local * VH * SW : nullptr;
-    for (int y = 0; y < VH; ++y) { pb.meta[(size_t)y * SW + x] = 0; pb.clip_depth[(size_t)y * SW + x] = GD_INF; }
+    for (int y = 0; y < VH; ++y) pb.meta[(size_t)y * SW + x] = 0;   // no owner, no plane, no clip linedef (clip depth: infinite)
     ColumnState st;
     st.current_sector = lane_ctx.sector;
     st.ceiling_clip = 0.0f; st.floor_clip = (float)VH;
@@ -2419,19 +2474,19 @@ __device__ void flat_shade_pixel(const DeviceMap &dm, const Scratch &sc, const L
     }
 }
 
-__global__ void __launch_bounds__(64) flat_shade_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
-    const int local = blockIdx.y;
+__global__ void __launch_bounds__(128) flat_shade_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
+    const int local = blockIdx.x;
     if (local >= lane_count) return;
     const int listed = sc.flat_list_count[local];
     const LaneCtx &c = sc.ctx[local];
     unsigned char *frame = frame_base + (size_t)local * frame_stride;
-    const int slot = blockIdx.x * blockDim.x + threadIdx.x;
     if (listed <= FLAT_LIST_MAX) {
-        if (slot < listed) flat_shade_pixel(dm, sc, c, local, sc.flat_list[(size_t)local * FLAT_LIST_MAX + slot], frame);
+        for (int slot = threadIdx.x; slot < listed; slot += blockDim.x)
+            flat_shade_pixel(dm, sc, c, local, sc.flat_list[(size_t)local * FLAT_LIST_MAX + slot], frame);
         return;
     }
     // a lane with more gap pixels than the list holds: every pixel is looked at
-    for (int pixel = slot; pixel < VH * SW; pixel += gridDim.x * blockDim.x) {
+    for (int pixel = threadIdx.x; pixel < VH * SW; pixel += blockDim.x) {
         const unsigned int meta = sc.meta[(size_t)local * VH * SW + pixel];
         if (!(meta & (META_FILLED | META_MASKED)) && ((meta >> META_SECTOR_SHIFT) & META_SECTOR_MASK) == 0)
             flat_shade_pixel(dm, sc, c, local, pixel, frame);
@@ -2497,7 +2552,6 @@ __global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lan
     const WallRec *recs = sc.rec + (size_t)local * m->wall_count;
     unsigned char *frame = frame_base + (size_t)local * frame_stride;
     const unsigned int *meta = sc.meta + (size_t)local * VH * SW;
-    const float *clip_depth = sc.clip_depth + (size_t)local * VH * SW;
     // nearest blocking linedef of this column (engine.py:10534-10557), gathered by wall_setup
     const u64 hit = sc.block_hit[(size_t)local * SW + x];
     float best = hit == ~0ULL ? GD_INF : __uint_as_float((unsigned)(hit >> 32));
@@ -2568,14 +2622,14 @@ __global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lan
         }
         // four rows per step, each stage's loads issued together so that their latencies overlap
         for (int yb = y_lo; yb < y_hi; yb += 4) {
-            i64 sv[4]; bool live[4]; unsigned int row_meta[4]; float row_clip[4];
+            i64 sv[4]; bool live[4]; unsigned int row_meta[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int y = yb + j;
                 sv[j] = (fraction_base + mul64((i64)y, s.iscale)) >> 16;
                 live[j] = y < y_hi && sv[j] >= 0 && sv[j] < height;
                 const size_t i = (size_t)(y < VH ? y : VH - 1) * SW + x;
-                row_meta[j] = meta[i]; row_clip[j] = clip_depth[i];
+                row_meta[j] = meta[i];
             }
             unsigned char opaque[4], post_top[4], texel[4];
 #pragma unroll
@@ -2591,12 +2645,12 @@ __global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lan
                     float side = (cl.z - cl.x) * (s.y - cl.y) - (cl.w - cl.y) * (s.x - cl.x);
                     visible = (cnear > s.depth_fixed) || ((cfar > s.depth_fixed) && (side <= 0));
                 } else {
-                    visible = s.depth < row_clip[j];
+                    visible = s.depth < GD_INF;   // no clip linedef: the clip depth is infinite
                     // No clip recorded, but a plane of the wall pass shows here: where the flat ray did not
                     // resolve, the plane's own depth clips sprites (engine.py:13417-13422).  Only a sprite
                     // standing behind the plane needs to know.
                     const int plane = (int)((row_meta[j] >> META_SECTOR_SHIFT) & META_SECTOR_MASK) - 1;
-                    if (visible && plane >= 0 && !(row_meta[j] & META_FILLED) && !finitef(row_clip[j])) {
+                    if (visible && plane >= 0 && !(row_meta[j] & META_FILLED)) {
                         const int y = yb + j;
                         const bool plane_floor = (row_meta[j] & META_FLOOR) != 0;
                         const float plane_height = plane_floor ? (L.view_z - m->sector_heights[2 * plane]) : (m->sector_heights[2 * plane + 1] - L.view_z);
@@ -3231,11 +3285,12 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     }
     mark();
     // the flat pass, where the walls left it something to decide
-    hipLaunchKernelGGL(flat_list_kernel, dim3(FLAT_LIST_MAX / 64, count), dim3(64), 0, stream, r->dm, *lanes, base, count, sc);
+    hipLaunchKernelGGL(flat_list_kernel, dim3(count), dim3(128), 0, stream, r->dm, *lanes, base, count, sc);
     hipLaunchKernelGGL(flat_span_select_kernel, dim3(SPAN_ROW_SLOTS, count), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
     mark();
+    hipLaunchKernelGGL(flat_tail_kernel, dim3(SW / 64, count), dim3(64 * TAIL_ROWS), 0, stream, r->dm, *lanes, base, count, sc);
     hipLaunchKernelGGL(flat_span_finish_kernel, dim3(count), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
-    hipLaunchKernelGGL(flat_shade_kernel, dim3(FLAT_LIST_MAX / 64, count), dim3(64), 0, stream, r->dm, count, sc, frame_base, frame_stride);
+    hipLaunchKernelGGL(flat_shade_kernel, dim3(count), dim3(128), 0, stream, r->dm, count, sc, frame_base, frame_stride);
     mark();
     if (decals)
         hipLaunchKernelGGL(decal_kernel, dim3(count), dim3(SW), 0, stream, r->dm, r->overlays, *lanes, base, count, sc, frame_base, frame_stride);
@@ -3350,6 +3405,9 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
             float smallest = cosine_correction[strip * 64];
             for (int x = strip * 64; x < strip * 64 + 64; ++x) smallest = std::fmin(smallest, cosine_correction[x]);
             r->dm.strip_reach_scale[strip] = smallest > 0.0f ? 1.001f / smallest : GD_INF;
+            float largest = cosine_correction[strip * 64];
+            for (int x = strip * 64; x < strip * 64 + 64; ++x) largest = std::fmax(largest, cosine_correction[x]);
+            r->dm.strip_far_scale[strip] = smallest > 0.0f && std::isfinite(largest) ? 0.999f / largest : 0.0f;
         }
         r->dm.fine_inverse = 1.0f / h->fine_cell;
     }
@@ -3414,12 +3472,14 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.flat_sector);
     if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.flat_flags);
     if (rc == GD_OK) rc = scratch_alloc(r, L * 4, &sc.flat_span);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * 2 * SW, &sc.flat_tail);
     if (rc == GD_OK) rc = scratch_alloc(r, L * FLAT_LIST_MAX, &sc.flat_list);
     if (rc == GD_OK) rc = scratch_alloc(r, L, &sc.flat_list_count);
     if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.meta);
     if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.clip_depth);
     if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)GD_SCREEN_HEIGHT * SW, &sc.frame);
     if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)(h->floor_level_count + h->ceil_level_count), &sc.level_reach);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)(h->floor_level_count + h->ceil_level_count), &sc.level_far);
     if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)(h->floor_level_count + h->ceil_level_count) * 2, &sc.level_plane);
     if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)VH, &sc.row_slope);
     if (rc == GD_OK) rc = scratch_alloc(r, L * 32, &sc.step_scale);
