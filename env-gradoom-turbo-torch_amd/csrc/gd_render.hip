@@ -170,7 +170,8 @@ struct Scratch {    // per-chunk working memory, sized at create
 #define FLAT_LIST_MAX 1024 // listed gap pixels per lane (a gap is typically one column wide)
 #define PLANE_LEVELS 64    // level lists up to this long are shaded from the per-lane tables
 
-#define META_FILLED 0x80000000u   // an opaque wall tier owns the pixel
+#define META_FILLED 0x80000000u   // an opaque wall tier owns the pixel; its palette index sits in the low byte of the
+                                  // plane sector field (plane shading, which writes every other view pixel, stores it)
 #define META_FLOOR 0x40000000u    // the owning plane is a floor
 #define META_MASKED 0x20000000u   // a masked mid-texture was drawn over the pixel
 #define META_SECTOR_SHIFT 16
@@ -1869,10 +1870,10 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
             for (int j = 0; j < WALL_ROWS; ++j) {
                 if (!draw[j]) continue;
                 const size_t i = (size_t)(yb + j) * SW + x;
-                pb.frame[i] = colormap[(tail[j] ? shade_group : shade_own) * 256 + texel[j]];
+                const unsigned colour = colormap[(tail[j] ? shade_group : shade_own) * 256 + texel[j]];
                 pb.clip_depth[i] = r.distance;
                 if (DEPTH) pb.scene_depth[i] = r.distance;
-                pb.meta[i] = META_FILLED | (unsigned)(wi + 1);
+                pb.meta[i] = META_FILLED | (colour << META_SECTOR_SHIFT) | (unsigned)(wi + 1);
             }
         }
         if (one_sided) window_dirty = true;
@@ -1885,7 +1886,7 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
         bool ceiling_span = (r.bits & PB_MARK_CEILING) && (py >= c.ceiling_clip) && (py < ceiling_plane_bottom);
         bool floor_span = (r.bits & PB_MARK_FLOOR) && (py >= floor_plane_top) && (py < c.floor_clip);
         bool meta_dirty = false;
-        if (((meta >> META_SECTOR_SHIFT) & META_SECTOR_MASK) == 0 && (ceiling_span || floor_span)) {
+        if (!(meta & META_FILLED) && ((meta >> META_SECTOR_SHIFT) & META_SECTOR_MASK) == 0 && (ceiling_span || floor_span)) {
             meta |= ((unsigned)(r.render_current + 1) << META_SECTOR_SHIFT) | (floor_span ? META_FLOOR : 0);
             meta_dirty = true;
         }
@@ -1907,11 +1908,11 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
                 i64 fraction = shl64(texture_mid, 16 - height_bits) + (mul64(vertical_step, screen_delta) >> 16);
                 i64 tv = (fraction & UINT32_MASK) >> (32 - height_bits);
                 unsigned char texel = m->tex_atlas[((size_t)texture_id * m->tex_max_h + tv) * m->tex_max_w + tu];
-                pb.frame[i] = colormap[(bottom_tail ? shade_group : shade_own) * 256 + texel];
+                const unsigned colour = colormap[(bottom_tail ? shade_group : shade_own) * 256 + texel];
                 if (DEPTH) pb.scene_depth[i] = r.distance;
                 const float held = (meta & META_WALL_MASK) ? pb.clip_depth[i] : GD_INF;   // no clip recorded yet
                 if (r.distance < held) { pb.clip_depth[i] = r.distance; meta = (meta & ~META_WALL_MASK) | (unsigned)(wi + 1); }
-                meta |= META_FILLED;
+                meta = (meta & ~(META_SECTOR_MASK << META_SECTOR_SHIFT)) | (colour << META_SECTOR_SHIFT) | META_FILLED;
                 meta_dirty = true;
             }
         }
@@ -2426,7 +2427,11 @@ __global__ void __launch_bounds__(256) plane_shade_kernel(DeviceMap dm, int lane
 #pragma unroll
         for (int j = 0; j < SHADE_GROUP; ++j) {
             const int pixel = pixels[j];
-            if (pixel < 0 || (meta[j] & META_FILLED)) continue;
+            if (pixel < 0) continue;
+            if (meta[j] & META_FILLED) {   // a wall tier's pixel, unless a masked texture went over it
+                if (!(meta[j] & META_MASKED)) frame[pixel] = (unsigned char)(meta[j] >> META_SECTOR_SHIFT);
+                continue;
+            }
             const int y = pixel / SW, x = pixel - y * SW;
             const size_t i = (size_t)local * VH * SW + pixel;
             const int ps = (int)((meta[j] >> META_SECTOR_SHIFT) & META_SECTOR_MASK) - 1;
