@@ -1,18 +1,20 @@
 // MI355X (gfx950) batched software renderer + observation pipeline.
 //
-// One frame for N lanes runs as a short chain of kernels on two streams (walls on the caller's stream, flats
-// on a side stream that forks after lane_setup and joins before plane_shade):
+// One frame for N lanes runs as a short chain of kernels on the caller's stream:
 //
 //   lane_setup      1 thread / lane           view basis, pitch centre, camera sector
+//   lane_tables     1 thread / (lane, row)    per-lane distance bounds of every height level, plane rows, row slopes
 //   wall_setup      1 wave-slot / (lane,wall) FWallCoords span+depths, span ownership bounds, the linedef's
 //                                             entry in the candidate list of every column it can own, and the
 //                                             nearest blocking hit of every column (64-bit atomicMin)
 //   strip_key/order 1 thread / 64-col strip   longest strip first (counting sort on the blocking distance)
-//   lane_tables     1 thread / (lane, row)    per-lane reach of every height level, plane rows, row slopes
-//   flat_select     1 thread / pixel          nearest floor/ceiling sector through the fine point raster
-//   flat_finish     320 threads / lane        visplane repair (wave ballots), status bar rows cleared
 //   wall_columns    1 wave / strip            portal traversal, tiers, planes, masked mid-textures
-//   plane_shade     1 thread / 4 pixels       flat texel + light for every pixel a wall did not cover
+//   plane_shade     1 thread / 12 pixels      flat texel + light for every pixel a plane of the wall pass shows,
+//                                             the wall tiers' palette indices, the list of gap pixels
+//   flat_list       128 threads / lane        per-pixel plane rays (fine point raster) for the listed gap pixels
+//   flat_span_select, flat_tail, flat_span_finish
+//                                             visplane repair of the rows where a gap pixel stayed unresolved
+//   flat_shade      128 threads / lane        the gap pixels' flats
 //   decal           320 threads / lane        bullet chips on the wall tiers they hit (frames that carry decals
 //                                             also keep a per-pixel scene depth: wall_columns<true>, plane_shade<true>)
 //   sprite_columns  320 threads / lane        billboards far -> near, opaque / additive / translucent
@@ -3156,10 +3158,8 @@ int fail(int code, const std::string &message) { g_error = message; return code;
 
 }  // namespace
 
-// The flat kernels (bound by the vector ALU) and the wall kernels (bound by memory latency) of a
-// chunk are independent until plane shading, so the flats run on a side stream forked from the
-// caller's stream and joined back before plane shading.  (Cutting a batch into chunks or halves
-// pipelined over more streams measured no faster: the kernels already share the machine.)
+// Every kernel of a frame runs on the caller's stream.  (Cutting a batch into chunks or halves pipelined over
+// more streams measured no faster: the kernels already fill the machine.)
 struct gd_renderer {
     DeviceMap dm;
     Scratch sc;
@@ -3167,9 +3167,6 @@ struct gd_renderer {
     std::vector<void *> allocations;
     hipEvent_t events[16];
     bool events_ready;
-    hipStream_t side_stream;
-    hipEvent_t fork_event, flat_event;
-    bool side_ready;
     Overlays overlays;                       // device pointers, counts 0 until gd_renderer_set_overlays
     std::vector<void *> overlay_allocations;
 };
@@ -3254,8 +3251,7 @@ void build_fine_tables(std::vector<i64> &sine, std::vector<i64> &tangent) {
 
 const int STAGE_COUNT = 8;
 
-// `side` (optional) is a second stream for the flat kernels of this chunk.
-int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_desc *lanes, const gd_frame_out *out, int base, int count, hipStream_t stream, hipStream_t side, bool timed) {
+int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_desc *lanes, const gd_frame_out *out, int base, int count, hipStream_t stream, bool timed) {
     const gd_map_desc &m = r->dm.d;
     Scratch sc = chunk_scratch;
     unsigned char *frame_base;
@@ -3358,7 +3354,6 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     gd_renderer *r = new (std::nothrow) gd_renderer();
     if (!r) return fail(GD_E_ARG, "out of host memory");
     r->events_ready = false;
-    r->side_ready = false;
     std::memset(&r->sc, 0, sizeof(r->sc));
     std::memset(&r->overlays, 0, sizeof(r->overlays));
     r->dm.d = *h;
@@ -3497,13 +3492,6 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
         for (int i = 0; i < 16; ++i) if (hipEventCreate(&r->events[i]) != hipSuccess) rc = fail(GD_E_HIP, "hipEventCreate");
         r->events_ready = rc == GD_OK;
     }
-    if (rc == GD_OK) {
-        // default priority, as every stream of this library
-        if (hipStreamCreateWithFlags(&r->side_stream, hipStreamNonBlocking) != hipSuccess) rc = fail(GD_E_HIP, "hipStreamCreateWithFlags");
-        else if (hipEventCreateWithFlags(&r->fork_event, hipEventDisableTiming) != hipSuccess) { (void)hipStreamDestroy(r->side_stream); rc = fail(GD_E_HIP, "hipEventCreateWithFlags"); }
-        else if (hipEventCreateWithFlags(&r->flat_event, hipEventDisableTiming) != hipSuccess) { (void)hipEventDestroy(r->fork_event); (void)hipStreamDestroy(r->side_stream); rc = fail(GD_E_HIP, "hipEventCreateWithFlags"); }
-        else r->side_ready = true;
-    }
     if (rc != GD_OK) { std::string keep = g_error; gd_renderer_destroy(r); g_error = keep; return rc; }
     *out = r;
     return GD_OK;
@@ -3511,7 +3499,6 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
 
 void gd_renderer_destroy(gd_renderer *r) {
     if (!r) return;
-    if (r->side_ready) { (void)hipStreamSynchronize(r->side_stream); (void)hipEventDestroy(r->fork_event); (void)hipEventDestroy(r->flat_event); (void)hipStreamDestroy(r->side_stream); }
     for (void *ptr : r->allocations) (void)hipFree(ptr);
     for (void *ptr : r->overlay_allocations) (void)hipFree(ptr);
     if (r->events_ready) for (int i = 0; i < 16; ++i) (void)hipEventDestroy(r->events[i]);
@@ -3541,7 +3528,7 @@ int gd_render(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_out *ou
     hipStream_t caller = static_cast<hipStream_t>(stream);
     for (int base = 0; base < lanes->lane_count; base += r->chunk_lanes) {
         int count = lanes->lane_count - base < r->chunk_lanes ? lanes->lane_count - base : r->chunk_lanes;
-        rc = launch_chunk(r, r->sc, lanes, out, base, count, caller, r->side_ready ? r->side_stream : nullptr, false);
+        rc = launch_chunk(r, r->sc, lanes, out, base, count, caller, false);
         if (rc != GD_OK) return rc;
     }
     return GD_OK;
@@ -3556,7 +3543,7 @@ int gd_render_timed(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_o
     for (int it = 0; it < launches; ++it) {
         for (int base = 0; base < lanes->lane_count; base += r->chunk_lanes) {
             int count = lanes->lane_count - base < r->chunk_lanes ? lanes->lane_count - base : r->chunk_lanes;
-            rc = launch_chunk(r, r->sc, lanes, out, base, count, st, nullptr, true);
+            rc = launch_chunk(r, r->sc, lanes, out, base, count, st, true);
             if (rc != GD_OK) return rc;
             HIP_TRY(hipEventSynchronize(r->events[STAGE_COUNT - 1]));
             for (int s = 0; s + 1 < STAGE_COUNT; ++s) {
