@@ -68,6 +68,7 @@ typedef unsigned long long u64;
 #define CF_LEDGE 4
 #define CF_ALONG_HI 8   // along > 0.5: the ray is nearer the linedef's end vertex
 #define CF_FF 16        // camera on the front side of the linedef (float32 test)
+#define CF_MASKED 32    // candidate entries only: the side facing the camera carries a masked mid-texture
 
 // wall record flags
 #define WF_HC 1        // owns at least one column after every span test
@@ -567,6 +568,13 @@ __global__ void __launch_bounds__(128) wall_setup_kernel(DeviceMap dm, int lane_
     const int w_raw = blockIdx.x * blockDim.x + threadIdx.x;
     const int local = blockIdx.y;
     if (local >= lane_count) return;          // uniform over the block
+    {
+        // The traversal starts from a cleared meta plane (no owner, no plane, no clip linedef).  This kernel is
+        // bound by its arithmetic, so the fill rides along here instead of heading wall_columns_kernel.
+        uint4 *plane = reinterpret_cast<uint4 *>(sc.meta + (size_t)local * VH * SW);
+        const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+        for (int k = w_raw; k < VH * SW / 4; k += gridDim.x * blockDim.x) plane[k] = zero;
+    }
     const bool live = w_raw < m->wall_count;  // dead lanes still help with the column loops
     const int w = live ? w_raw : 0;
     const LaneCtx &c = sc.ctx[local];
@@ -674,7 +682,8 @@ __global__ void __launch_bounds__(128) wall_setup_kernel(DeviceMap dm, int lane_
     int *counts = sc.cand_count + (size_t)local * SW;
     const int packed_sectors = (s0 & 0xFFFF) | (s1 << 16);
     const int packed_vertices = (int)(((unsigned)m->wall_vertex[2 * w] & 0xFFFFu) | ((unsigned)m->wall_vertex[2 * w + 1] << 16));
-    const int packed_span = (r.flags & 0xFF) | (os ? 0x100 : 0);
+    const bool masked_side = !os && m->side_tex[(w * 2 + (ff ? 0 : 1)) * 3] >= 0;
+    const int packed_span = (r.flags & 0xFF) | (os ? 0x100 : 0) | (masked_side ? 0x200 : 0);
     const int rec_pl = r.pl, rec_pr = r.pr;
     for (u64 pending = __ballot(a_lo < a_hi); pending; pending &= pending - 1) {
         const int owner = __ffsll((long long)pending) - 1;
@@ -693,7 +702,7 @@ __global__ void __launch_bounds__(128) wall_setup_kernel(DeviceMap dm, int lane_
             if (finitef(e.dist)) {
                 int slot = atomicAdd(&counts[x], 1);
                 if (slot < CAND_MAX) {
-                    entry.flags = (unsigned short)e.flags;
+                    entry.flags = (unsigned short)(e.flags | ((b_span & 0x200) ? CF_MASKED : 0));
                     entry.dist = e.dist;
                     list[(size_t)slot * SW + x] = entry;
                 } else {
@@ -1257,6 +1266,17 @@ struct ColumnCtx {
 #pragma unroll
         for (int j = 0; j < CAND_BATCH; ++j) out[j] = cand(k0 + j < count ? k0 + j : count - 1);
     }
+    // The next CAND_BATCH entries named by the bits of `rest` (list positions, ascending), loaded together;
+    // slot j is absent where at[j] < 0.
+    __device__ __forceinline__ void cand_batch_of(u64 &rest, Cand (&out)[CAND_BATCH], int (&at)[CAND_BATCH]) const {
+#pragma unroll
+        for (int j = 0; j < CAND_BATCH; ++j) {
+            at[j] = rest ? __ffsll((long long)rest) - 1 : -1;
+            rest &= rest - 1;
+        }
+#pragma unroll
+        for (int j = 0; j < CAND_BATCH; ++j) out[j] = cand(at[j] < 0 ? 0 : at[j]);
+    }
     __device__ Eval eval(int w) const { return eval_wall(m, *c, recs, x, w, rx, ry); }
 };
 
@@ -1533,7 +1553,11 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
     // a. nearest incident linedef beyond previous_distance (engine.py:11769-11780)
     float distance = GD_INF; int wi = 0x7fffffff;
     Eval cwi;
+    // List positions of the candidates incident to the current sector and beyond previous_distance: the later
+    // scans of this pass ask for both (and more), so they only visit these.  Without a current sector: all.
+    u64 incident_beyond = cc.count >= 64 ? ~0ULL : ((1ULL << cc.count) - 1);
     if (cs >= 0) {
+        incident_beyond = 0;
         // b. equal-depth solid (engine.py:11784-11807): the nearest one-sided candidate replaces
         // the selection when it lies within 1e-3 of the nearest candidate, found in the same scan.
         float sd = GD_INF; int swi = 0x7fffffff;
@@ -1546,6 +1570,7 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
                 if (k0 + j >= cc.count) continue;
                 const Cand q = batch[j];
                 if (!(incident_c(q) && q.dist > prev)) continue;
+                incident_beyond |= 1ULL << (k0 + j);
                 if (q.dist < distance || (q.dist == distance && (int)q.wall < wi)) { distance = q.dist; wi = q.wall; wi_flags = q.flags; }
                 if ((q.s1 < 0) && (q.dist < sd || (q.dist == sd && (int)q.wall < swi))) { sd = q.dist; swi = q.wall; swi_flags = q.flags; }
             }
@@ -1575,12 +1600,12 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
     bool ps_path_geo = cwi.flags & CF_GEO;
     float psd = GD_INF; int psi = 0x7fffffff; int psi_flags = 0;
     if (!sel_is_proj) {
-        for (int k0 = 0; k0 < cc.count; k0 += CAND_BATCH) {
-            Cand batch[CAND_BATCH];
-            cc.cand_batch(k0, batch);
+        for (u64 rest = incident_beyond; rest;) {
+            Cand batch[CAND_BATCH]; int at[CAND_BATCH];
+            cc.cand_batch_of(rest, batch, at);
 #pragma unroll
             for (int j = 0; j < CAND_BATCH; ++j) {
-                if (k0 + j >= cc.count) continue;
+                if (at[j] < 0) continue;
                 const Cand q = batch[j];
                 bool owner = incident_c(q) && (q.s1 < 0) && (q.flags & CF_PROJ) && (q.flags & CF_LEDGE) && shares_sel_c(q) && (q.dist > prev_eps);
                 if (owner && (q.dist < psd || (q.dist == psd && (int)q.wall < psi))) { psd = q.dist; psi = q.wall; psi_flags = q.flags; }
@@ -1623,12 +1648,12 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
     float npd = GD_INF; int npi = 0x7fffffff; int npi_flags = 0;
     const int so_s0 = mv.sec(wi, 0), so_s1 = mv.sec(wi, 1);
     if (!so_is_proj) {
-        for (int k0 = 0; k0 < cc.count; k0 += CAND_BATCH) {
-            Cand batch[CAND_BATCH];
-            cc.cand_batch(k0, batch);
+        for (u64 rest = incident_beyond; rest;) {
+            Cand batch[CAND_BATCH]; int at[CAND_BATCH];
+            cc.cand_batch_of(rest, batch, at);
 #pragma unroll
             for (int j = 0; j < CAND_BATCH; ++j) {
-                if (k0 + j >= cc.count) continue;
+                if (at[j] < 0) continue;
                 const Cand q = batch[j];
                 int w = q.wall;
                 if (!(incident_c(q) && (q.s1 >= 0) && (q.flags & CF_PROJ) && (q.dist > prev_eps))) continue;
@@ -2108,7 +2133,7 @@ __device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const Col
             int w = q.wall;
             if (!(q.flags & CF_PROJ) || (q.s1 < 0)) continue;
             int sidew = (q.flags & CF_FF) ? 0 : 1;   // engine.py:13436-13444, the float32 facing test
-            if (m->side_tex[(w * 2 + sidew) * 3] < 0) continue;
+            if (!(q.flags & CF_MASKED)) continue;     // no mid-texture on that side
             if (q.dist < md || (q.dist == md && w < mw)) { md = q.dist; mw = w; mside = sidew; cand_flags = q.flags; }
         }
     }
@@ -2279,7 +2304,7 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
     pb.meta = sc.meta + (size_t)local * VH * SW;
     pb.clip_depth = sc.clip_depth + (size_t)local * VH * SW;
     pb.scene_depth = DEPTH ? sc.scene_depth + (size_t)local * VH * SW : nullptr;
-    for (int y = 0; y < VH; ++y) pb.meta[(size_t)y * SW + x] = 0;   // no owner, no plane, no clip linedef (clip depth: infinite)
+    // the meta plane arrives cleared (wall_setup_kernel): no owner, no plane, no clip linedef (clip depth: infinite)
     ColumnState st;
     st.current_sector = lane_ctx.sector;
     st.ceiling_clip = 0.0f; st.floor_clip = (float)VH;
@@ -2924,16 +2949,56 @@ __device__ __forceinline__ void stage_palette(unsigned char *pal, const unsigned
     __syncthreads();
 }
 
-__global__ void observe_kernel(const unsigned char *indexed, size_t lane_stride, int source_rows, const unsigned char *playpal,
+// One block per lane and OBS_BLOCK_ROWS observation rows.  The source rows they overlap are staged in LDS with
+// word loads (a byte load per tap keeps the address units busy for 64 lanes each); taps then read LDS.
+#define OBS_BLOCK_ROWS 3
+#define OBS_TILE_ROWS 11   // source rows that OBS_BLOCK_ROWS observation rows can overlap (10), and one to spare
+static_assert(GD_OBS_SIZE % OBS_BLOCK_ROWS == 0 && OBS_BLOCK_ROWS * GD_OBS_SIZE <= 256, "observe_kernel: rows per block");
+__global__ void __launch_bounds__(256) observe_kernel(const unsigned char *indexed, size_t lane_stride, int source_rows, const unsigned char *playpal,
                                int lane_count, unsigned char *obs, unsigned char *frames, const unsigned char *reset_mask, int stack_mode,
                                unsigned char *final_frames, const float *blend) {
-    __shared__ unsigned char pal[768];
-    int pixel = blockIdx.x * blockDim.x + threadIdx.x;
+    __shared__ unsigned int pal[256];   // PLAYPAL after the lane's screen blend, one word per colour (red | green << 8 | blue << 16)
+    __shared__ unsigned int tile[OBS_TILE_ROWS * (SW / 4)];
     int n = blockIdx.y;
-    stage_palette(pal, playpal, blend, n < lane_count ? n : 0);
-    if (n >= lane_count || pixel >= GD_OBS_SIZE * GD_OBS_SIZE) return;
-    int oy = pixel / GD_OBS_SIZE, ox = pixel - oy * GD_OBS_SIZE;
+    if (n >= lane_count) return;                   // the same in the whole block
     const unsigned char *src = indexed + (size_t)n * lane_stride;
+    const int first_row = blockIdx.x * OBS_BLOCK_ROWS;
+    const int tile_first = (first_row * 240) / 84;
+    // Everything the block reads from memory is asked for up front (palette entry, tile words, the stack words
+    // that the roll keeps), so that the block waits for memory once.
+    const size_t F = (size_t)GD_OBS_SIZE * GD_OBS_SIZE / 4;     // words per observation
+    const size_t word = (size_t)first_row * GD_OBS_SIZE / 4 + threadIdx.x;
+    const bool rolls = threadIdx.x < OBS_BLOCK_ROWS * GD_OBS_SIZE / 4;
+    const bool stack_aligned = ((reinterpret_cast<size_t>(frames) | reinterpret_cast<size_t>(final_frames)) & 3) == 0;
+    unsigned char *stack_bytes = frames ? frames + ((size_t)n * GD_FRAME_STACK * F + word) * 4 : nullptr;
+    auto load_word = [](const unsigned char *p, bool aligned) -> unsigned int {
+        if (aligned) return *reinterpret_cast<const unsigned int *>(p);
+        return (unsigned)p[0] | ((unsigned)p[1] << 8) | ((unsigned)p[2] << 16) | ((unsigned)p[3] << 24);
+    };
+    const bool resets = reset_mask && reset_mask[n];
+    unsigned int kept[GD_FRAME_STACK];
+    for (int k = 0; k < GD_FRAME_STACK; ++k) kept[k] = (rolls && frames && !resets) ? load_word(stack_bytes + k * F * 4, stack_aligned) : 0u;
+    {
+        const int k = threadIdx.x;   // 256 threads, 256 colours
+        unsigned int r = playpal[3 * k], g = playpal[3 * k + 1], b = playpal[3 * k + 2];
+        if (blend) {
+            const float bonus = blend[2 * n], flash = blend[2 * n + 1];
+            r = blended_channel((unsigned char)r, 0, bonus, flash); g = blended_channel((unsigned char)g, 1, bonus, flash); b = blended_channel((unsigned char)b, 2, bonus, flash);
+        }
+        pal[k] = r | (g << 8) | (b << 16);
+    }
+    {
+        const bool aligned = (reinterpret_cast<size_t>(src) & 3) == 0;
+        for (int k = threadIdx.x; k < OBS_TILE_ROWS * (SW / 4); k += blockDim.x) {
+            const int r = k / (SW / 4), c = k - r * (SW / 4);
+            tile[k] = load_word(src + (size_t)min(tile_first + r, source_rows - 1) * SW + 4 * c, aligned);
+        }
+    }
+    __syncthreads();
+    __shared__ unsigned int gray_words[OBS_BLOCK_ROWS * GD_OBS_SIZE / 4];
+    const int row_in_block = min((int)threadIdx.x / GD_OBS_SIZE, OBS_BLOCK_ROWS - 1);   // the last few threads only help staging
+    const int oy = first_row + row_in_block, ox = min((int)threadIdx.x - row_in_block * GD_OBS_SIZE, GD_OBS_SIZE - 1);
+    const unsigned char *staged = reinterpret_cast<const unsigned char *>(tile);
     int y_start = oy * 240, y_end = y_start + 240, x_start = ox * 320, x_end = x_start + 320;
     int rs = 0, gs = 0, bs = 0;
     // up to 4 x 5 source pixels overlap one observation pixel; all of them are loaded first (taps
@@ -2944,7 +3009,7 @@ __global__ void observe_kernel(const unsigned char *indexed, size_t lane_stride,
         const int source_y = y_start / 84 + sy;
         const int overlap = min(y_end, (source_y + 1) * 84) - max(y_start, source_y * 84);
         y_overlap[sy] = (source_y >= source_rows || overlap <= 0) ? 0 : overlap;
-        row_offset[sy] = min(source_y, source_rows - 1) * SW;
+        row_offset[sy] = min(source_y - tile_first, OBS_TILE_ROWS - 1) * SW;   // rows past the tile weigh nothing
     }
 #pragma unroll
     for (int sx = 0; sx < 5; ++sx) {
@@ -2957,37 +3022,50 @@ __global__ void observe_kernel(const unsigned char *indexed, size_t lane_stride,
 #pragma unroll
     for (int sy = 0; sy < 4; ++sy)
 #pragma unroll
-        for (int sx = 0; sx < 5; ++sx) tap[sy][sx] = src[row_offset[sy] + column[sx]];
+        for (int sx = 0; sx < 5; ++sx) tap[sy][sx] = staged[row_offset[sy] + column[sx]];
 #pragma unroll
     for (int sy = 0; sy < 4; ++sy) {
 #pragma unroll
         for (int sx = 0; sx < 5; ++sx) {
             const int weight = (y_overlap[sy] * x_overlap[sx]) / 48;
-            const int p = tap[sy][sx] * 3;
-            rs += pal[p] * weight; gs += pal[p + 1] * weight; bs += pal[p + 2] * weight;
+            const unsigned int colour = pal[tap[sy][sx]];
+            rs += (int)(colour & 0xFFu) * weight; gs += (int)((colour >> 8) & 0xFFu) * weight; bs += (int)(colour >> 16) * weight;
         }
     }
     int r = (rs + 800) / 1600, g = (gs + 800) / 1600, b = (bs + 800) / 1600;
     unsigned char gray = (unsigned char)((r * 77 + g * 150 + b * 29 + 128) >> 8);
-    const size_t F = (size_t)GD_OBS_SIZE * GD_OBS_SIZE;
-    if (obs) obs[(size_t)n * F + pixel] = gray;
+    // The block's pixels are contiguous in the observation; they go out, and the stack is rolled, a word (four
+    // pixels) per thread.
+    if (threadIdx.x < OBS_BLOCK_ROWS * GD_OBS_SIZE) reinterpret_cast<unsigned char *>(gray_words)[threadIdx.x] = gray;
+    __syncthreads();
+    static_assert((GD_OBS_SIZE * GD_OBS_SIZE) % 4 == 0 && (OBS_BLOCK_ROWS * GD_OBS_SIZE) % 4 == 0, "observe_kernel: whole words");
+    if (!rolls) return;
+    const unsigned int grays = gray_words[threadIdx.x];
+    if (obs) {
+        unsigned char *out = obs + ((size_t)n * F + word) * 4;
+        if ((reinterpret_cast<size_t>(obs) & 3) == 0) *reinterpret_cast<unsigned int *>(out) = grays;
+        else for (int k = 0; k < 4; ++k) out[k] = (unsigned char)(grays >> (8 * k));
+    }
     if (frames) {
-        unsigned char *stack = frames + (size_t)n * GD_FRAME_STACK * F + pixel;
-        unsigned char *copy = final_frames ? final_frames + (size_t)n * GD_FRAME_STACK * F + pixel : nullptr;
-        if (reset_mask && reset_mask[n]) {
-            for (int k = 0; k < GD_FRAME_STACK; ++k) stack[k * F] = gray;
-            if (copy) for (int k = 0; k < GD_FRAME_STACK; ++k) copy[k * F] = gray;
+        // a stack is [4][84][84] bytes, so word access only needs the tensors themselves word aligned
+        unsigned char *copy_bytes = final_frames ? final_frames + ((size_t)n * GD_FRAME_STACK * F + word) * 4 : nullptr;
+        auto store = [&](unsigned char *p, unsigned int v) {
+            if (stack_aligned) *reinterpret_cast<unsigned int *>(p) = v;
+            else for (int k = 0; k < 4; ++k) p[k] = (unsigned char)(v >> (8 * k));
+        };
+        const size_t plane = F * 4;   // bytes per stacked observation
+        if (resets) {
+            for (int k = 0; k < GD_FRAME_STACK; ++k) store(stack_bytes + k * plane, grays);
+            if (copy_bytes) for (int k = 0; k < GD_FRAME_STACK; ++k) store(copy_bytes + k * plane, grays);
         } else if (stack_mode == GD_STACK_STEP) {
-            unsigned char kept[GD_FRAME_STACK - 1];
-            for (int k = 0; k < GD_FRAME_STACK - 1; ++k) kept[k] = stack[(k + 1) * F];
-            for (int k = 0; k < GD_FRAME_STACK - 1; ++k) stack[k * F] = kept[k];
-            stack[(GD_FRAME_STACK - 1) * F] = gray;
-            if (copy) {
-                for (int k = 0; k < GD_FRAME_STACK - 1; ++k) copy[k * F] = kept[k];
-                copy[(GD_FRAME_STACK - 1) * F] = gray;
+            for (int k = 0; k < GD_FRAME_STACK - 1; ++k) store(stack_bytes + k * plane, kept[k + 1]);
+            store(stack_bytes + (GD_FRAME_STACK - 1) * plane, grays);
+            if (copy_bytes) {
+                for (int k = 0; k < GD_FRAME_STACK - 1; ++k) store(copy_bytes + k * plane, kept[k + 1]);
+                store(copy_bytes + (GD_FRAME_STACK - 1) * plane, grays);
             }
-        } else if (copy) {
-            for (int k = 0; k < GD_FRAME_STACK; ++k) copy[k * F] = stack[k * F];   // lane left as it was
+        } else if (copy_bytes) {
+            for (int k = 0; k < GD_FRAME_STACK; ++k) store(copy_bytes + k * plane, kept[k]);   // lane left as it was
         }
     }
 }
@@ -3308,7 +3386,7 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     if (out->final_frames && !out->frames) return fail(GD_E_ARG, "final_frames needs frames");
     if (out->obs || out->frames) {
         const size_t F = (size_t)GD_OBS_SIZE * GD_OBS_SIZE;
-        hipLaunchKernelGGL(observe_kernel, dim3((GD_OBS_SIZE * GD_OBS_SIZE + 255) / 256, count), dim3(256), 0, stream,
+        hipLaunchKernelGGL(observe_kernel, dim3(GD_OBS_SIZE / OBS_BLOCK_ROWS, count), dim3(256), 0, stream,
                            frame_base, frame_stride, VH, m.playpal, count, out->obs ? out->obs + (size_t)base * F : nullptr,
                            out->frames ? out->frames + (size_t)base * GD_FRAME_STACK * F : nullptr,
                            out->reset_mask ? out->reset_mask + base : nullptr, out->stack_mode,
@@ -3655,7 +3733,7 @@ int gd_observe(const uint8_t *indexed, int32_t source_rows, const uint8_t *playp
     for (int base = 0; base < lane_count; base += 32768) {
         int count = lane_count - base < 32768 ? lane_count - base : 32768;
         const size_t F = (size_t)GD_OBS_SIZE * GD_OBS_SIZE;
-        hipLaunchKernelGGL(observe_kernel, dim3((GD_OBS_SIZE * GD_OBS_SIZE + 255) / 256, count), dim3(256), 0, static_cast<hipStream_t>(stream),
+        hipLaunchKernelGGL(observe_kernel, dim3(GD_OBS_SIZE / OBS_BLOCK_ROWS, count), dim3(256), 0, static_cast<hipStream_t>(stream),
                            indexed + (size_t)base * source_rows * SW, (size_t)source_rows * SW, source_rows, playpal, count,
                            obs ? obs + (size_t)base * F : nullptr, frames ? frames + (size_t)base * GD_FRAME_STACK * F : nullptr,
                            reset_mask ? reset_mask + base : nullptr, stack_mode, nullptr, nullptr);
