@@ -1789,21 +1789,31 @@ __device__ __forceinline__ void clip_rows(PixelBuffers &pb, int x, int first, in
     }
 }
 
-__device__ __forceinline__ void apply_silhouette(PixelBuffers &pb, SilhouetteBounds &sb, int x, bool bottom, bool top, float floor_clip, float ceiling_clip, float distance, int wall) {
+// `done_from` / `done_to`: rows [done_from, done_to) already carry this silhouette (pass_paint wrote it with
+// the rows the pass took out of a window nothing had touched); an empty range otherwise.
+__device__ __forceinline__ void apply_silhouette(PixelBuffers &pb, SilhouetteBounds &sb, int x, bool bottom, bool top, float floor_clip, float ceiling_clip, float distance, int wall,
+                                                 int done_from, int done_to) {
     if (bottom) {
         int first = floor_clip <= 0.0f ? 0 : (floor_clip >= (float)VH ? VH : (int)floor_clip);   // clips hold integers
         int last = (distance >= sb.bot_depth) ? (sb.bot_row < VH ? sb.bot_row : VH) : VH;
-        clip_rows(pb, x, first, last, distance, wall);
+        clip_rows(pb, x, (done_to > first && done_from <= first) ? done_to : first, last, distance, wall);
         sb.bot_row = first < sb.bot_row ? first : sb.bot_row;
         sb.bot_depth = fmaxf(sb.bot_depth, distance);
     }
     if (top) {
         int end = ceiling_clip <= 0.0f ? 0 : (ceiling_clip >= (float)VH ? VH : (int)ceiling_clip);
         int start = (distance >= sb.top_depth) ? (sb.top_row > 0 ? sb.top_row : 0) : 0;
-        clip_rows(pb, x, start, end, distance, wall);
+        clip_rows(pb, x, start, (done_from < end && done_to >= end) ? done_from : end, distance, wall);
         sb.top_row = end > sb.top_row ? end : sb.top_row;
         sb.top_depth = fmaxf(sb.top_depth, distance);
     }
+}
+
+// May pass_paint write a two-sided pass's sprite silhouettes along with the rows the pass takes out of an untouched
+// window?  Only while its lower and upper tier do not overlap on screen.
+__device__ __forceinline__ bool silhouette_folds(const PassColumn &r) {
+    const bool lower_on = r.view_floor < r.other_floor, upper_on = r.view_ceiling > r.other_ceiling;
+    return !(lower_on && upper_on && r.clipped_lower_top < r.clipped_upper_bottom);
 }
 
 // engine.py:12637-12884
@@ -1847,13 +1857,40 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
     if (!window_dirty) {
         // clips and projections hold integers in [0, 208]
         const unsigned claim = (unsigned)(r.render_current + 1) << META_SECTOR_SHIFT;
-        if (r.bits & PB_MARK_CEILING) {
-            int e = (int)ceiling_plane_bottom;
-            for (int y = y0; y < e; ++y) pb.meta[(size_t)y * SW + x] = claim;
+        // The sprite silhouettes of a two-sided drawseg (engine.py:12943-12964) give every row that this pass
+        // takes out of the window the pass's own (distance, linedef) as sprite clip.  Those rows are untouched
+        // so far, so what this pass writes there carries the clip along and pass_advance need not revisit them:
+        // tier rows hold it anyway, plane rows get it with their claim, rows left bare get it alone.
+        // (Not where the lower and the upper tier overlap, a closed door say: a row of both that the lower tier
+        // leaves undrawn for want of a texture would be missed.  silhouette_folds() is asked here and there.)
+        const bool masked_texture = r.side_tex[0] >= 0;
+        const bool folds = !one_sided && silhouette_folds(r);
+        const bool sil_bottom = folds && ((r.view_floor > r.other_floor) || (L.view_z < r.other_floor) || masked_texture);
+        const bool sil_top = folds && ((r.view_ceiling < r.other_ceiling) || (L.view_z > r.other_ceiling) || masked_texture);
+        const unsigned clip_word = (unsigned)(wi + 1);
+        {
+            const bool claims = r.bits & PB_MARK_CEILING;
+            const bool bare = !claims && sil_top && upper_on && (r.side_tex[2] >= 0);   // the upper tier lowers the clip past these rows
+            if (claims || bare) {
+                const int e = (int)ceiling_plane_bottom;
+                const unsigned word = (claims ? claim : 0u) | (sil_top ? clip_word : 0u);
+                for (int y = y0 < 0 ? 0 : y0; y < e; ++y) {
+                    pb.meta[(size_t)y * SW + x] = word;
+                    if (sil_top) pb.clip_depth[(size_t)y * SW + x] = r.distance;
+                }
+            }
         }
-        if (r.bits & PB_MARK_FLOOR) {
-            int b = (int)floor_plane_top;
-            for (int y = b; y < y1; ++y) pb.meta[(size_t)y * SW + x] = claim | META_FLOOR;
+        {
+            const bool claims = r.bits & PB_MARK_FLOOR;
+            const bool bare = !claims && sil_bottom && lower_on && (r.side_tex[1] >= 0);   // the lower tier raises the clip past these rows
+            if (claims || bare) {
+                const int b = (int)floor_plane_top;
+                const unsigned word = (claims ? (claim | META_FLOOR) : 0u) | (sil_bottom ? clip_word : 0u);
+                for (int y = b < 0 ? 0 : b; y < y1; ++y) {
+                    pb.meta[(size_t)y * SW + x] = word;
+                    if (sil_bottom) pb.clip_depth[(size_t)y * SW + x] = r.distance;
+                }
+            }
         }
         int t0 = VH, t1 = 0;
         if (one_sided) { t0 = (int)r.clipped_top; t1 = (int)r.clipped_bottom; }
@@ -1949,7 +1986,7 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
 
 // engine.py:12885-13371
 template <bool SPLIT>
-__device__ __forceinline__ bool pass_advance(const ColumnCtx &cc, ColumnState &c, const PassColumn &r, PixelBuffers &pb, SilhouetteBounds &sb) {
+__device__ __forceinline__ bool pass_advance(const ColumnCtx &cc, ColumnState &c, const PassColumn &r, PixelBuffers &pb, SilhouetteBounds &sb, bool window_untouched) {
     const gd_map_desc *m = cc.m;
     const MapView &mv = cc.mv;
     const LaneCtx &L = *cc.c;
@@ -1975,7 +2012,17 @@ __device__ __forceinline__ bool pass_advance(const ColumnCtx &cc, ColumnState &c
         bool masked_texture = r.side_tex[0] >= 0;
         bool bottom_sil = (r.view_floor > r.other_floor) || (L.view_z < r.other_floor) || masked_texture;
         bool top_sil = (r.view_ceiling < r.other_ceiling) || (L.view_z > r.other_ceiling) || masked_texture;
-        apply_silhouette(pb, sb, x, bottom_sil, top_sil, c.floor_clip, c.ceiling_clip, distance, wi);
+        // pass_paint, finding the window untouched, has written the silhouette into the rows that this pass took out
+        // of it: [new floor clip, old floor clip) at the bottom, [old ceiling clip, new ceiling clip) at the top
+        auto row_of = [](float clip) { return clip <= 0.0f ? 0 : (clip >= (float)VH ? VH : (int)clip); };
+        const int old_floor = row_of(before.floor_clip), old_ceiling = row_of(before.ceiling_clip);
+        if (window_untouched && silhouette_folds(r)) {
+            // one call per side: the rows already done differ
+            apply_silhouette(pb, sb, x, bottom_sil, false, c.floor_clip, c.ceiling_clip, distance, wi, row_of(c.floor_clip), old_floor);
+            apply_silhouette(pb, sb, x, false, top_sil, c.floor_clip, c.ceiling_clip, distance, wi, old_ceiling, row_of(c.ceiling_clip));
+        } else {
+            apply_silhouette(pb, sb, x, bottom_sil, top_sil, c.floor_clip, c.ceiling_clip, distance, wi, 0, 0);
+        }
     }
     // r. clips of the geometric portal behind a projected solid (engine.py:12969-13069)
     if (r.bits & PB_PS_KEEPS) {
@@ -2010,7 +2057,7 @@ __device__ __forceinline__ bool pass_advance(const ColumnCtx &cc, ColumnState &c
         bool pmasked = ptex[0] >= 0;
         bool pbottom = (r.view_floor > pof) || (L.view_z < pof) || pmasked;
         bool ptop = (r.view_ceiling < poc) || (L.view_z > poc) || pmasked;
-        apply_silhouette(pb, sb, x, pbottom, ptop, c.floor_clip, c.ceiling_clip, r.ps_path_distance, path);
+        apply_silhouette(pb, sb, x, pbottom, ptop, c.floor_clip, c.ceiling_clip, r.ps_path_distance, path, 0, 0);
     }
     // s. next sector (engine.py:13070-13241)
     const float prior = before.previous_distance;
@@ -2357,7 +2404,7 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
             pass_paint<DEPTH>(cc, st, pc, pb, group_valid, common_bottom, first_group_visibility, colormap_lds, window_dirty);
             PROF_T(t3);
             PROF_ADD(1, t2, t3);
-            bool changed = pass_advance<SPLIT>(cc, st, pc, pb, sb);
+            bool changed = pass_advance<SPLIT>(cc, st, pc, pb, sb, !window_dirty);
             PROF_T(t4);
             PROF_ADD(2, t3, t4);
 #ifdef GD_PROFILE
