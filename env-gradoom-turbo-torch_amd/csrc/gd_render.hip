@@ -614,7 +614,55 @@ __global__ void __launch_bounds__(128) wall_setup_kernel(DeviceMap dm, int lane_
     u64 *block_hits = sc.block_hit + (size_t)local * SW;
     int first = 0, last = SW - 1; bool any = false;
     float numer_d = offx * segy - offy * segx;
-    for (u64 pending = __ballot(scan_lo <= scan_hi); pending; pending &= pending - 1) {
+    // Most scan ranges are a few columns wide, so several linedefs share a turn (eight lanes each for eight of
+    // them, sixteen for four, thirty-two for two); a wider range has the wavefront to itself.
+    const int scan_width = scan_hi - scan_lo + 1;
+    auto shared_scans = [&](bool member, int lanes_each) {
+        const int group = slot_in_wave / lanes_each, group_lane = slot_in_wave - group * lanes_each;
+        const int groups = 64 / lanes_each;
+        const u64 group_mask = (lanes_each == 64 ? ~0ULL : ((1ULL << lanes_each) - 1)) << (group * lanes_each);
+        for (u64 pending = __ballot(member); pending;) {
+            int owners[8];
+            int owner = -1;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                owners[k] = -1;
+                if (k >= groups) continue;               // the same in every lane
+                owners[k] = pending ? __ffsll((long long)pending) - 1 : -1;
+                pending &= pending - 1;
+                if (group == k) owner = owners[k];
+            }
+            const int source = owner < 0 ? 0 : owner;
+            const float b_segx = __shfl(segx, source), b_segy = __shfl(segy, source);
+            const float b_offx = __shfl(offx, source), b_offy = __shfl(offy, source), b_numer = __shfl(numer_d, source);
+            const int b_lo = __shfl(scan_lo, source), b_hi = __shfl(scan_hi, source);
+            const int b_block = __shfl(blocking_slot, source);
+            const int x = b_lo + group_lane;
+            float rx, ry; ray_direction(c, x, &rx, &ry);
+            float den = rx * b_segy - ry * b_segx;
+            bool ok = fabsf(den) >= 1e-6f;
+            float safe = ok ? den : 1.0f;
+            float d = b_numer / safe;
+            float a = (b_offx * ry - b_offy * rx) / safe;
+            bool g = owner >= 0 && x <= b_hi && ok && (d > 0) && (a >= 0) && (a <= 1);
+            if (g && b_block >= 0) atomicMin(&block_hits[x], ((u64)__float_as_uint(d) << 32) | (u64)(unsigned)b_block);
+            const u64 hits = __ballot(g) & group_mask;
+            // every lane of a group holds its linedef's first / last hit column; the linedef's own lane fetches them
+            const int group_first = hits ? b_lo + (__ffsll((long long)hits) - 1 - group * lanes_each) : SW;
+            const int group_last = hits ? b_lo + (63 - __clzll((long long)hits) - group * lanes_each) : -1;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                if (k >= groups || owners[k] < 0) continue;   // the same in every lane
+                const int k_first = bcast(group_first, k * lanes_each), k_last = bcast(group_last, k * lanes_each);
+                if (slot_in_wave == owners[k] && k_last >= 0) { first = k_first; last = k_last; any = true; }
+            }
+        }
+    };
+    const bool scans = scan_lo <= scan_hi;
+    shared_scans(scans && scan_width <= 8, 8);
+    shared_scans(scans && scan_width > 8 && scan_width <= 16, 16);
+    shared_scans(scans && scan_width > 16 && scan_width <= 32, 32);
+    for (u64 pending = __ballot(scans && scan_width > 32); pending; pending &= pending - 1) {
         const int owner = __ffsll((long long)pending) - 1;
         const float b_segx = bcast(segx, owner), b_segy = bcast(segy, owner);
         const float b_offx = bcast(offx, owner), b_offy = bcast(offy, owner), b_numer = bcast(numer_d, owner);
@@ -685,7 +733,52 @@ __global__ void __launch_bounds__(128) wall_setup_kernel(DeviceMap dm, int lane_
     const bool masked_side = !os && m->side_tex[(w * 2 + (ff ? 0 : 1)) * 3] >= 0;
     const int packed_span = (r.flags & 0xFF) | (os ? 0x100 : 0) | (masked_side ? 0x200 : 0);
     const int rec_pl = r.pl, rec_pr = r.pr;
-    for (u64 pending = __ballot(a_lo < a_hi); pending; pending &= pending - 1) {
+    // Most linedefs cover a few columns only, so several of them share a turn: eight with eight lanes each, then
+    // four with sixteen, then two with thirty-two; a wider one has the wavefront to itself.
+    const bool listed = a_lo < a_hi;
+    const bool narrow = listed && (a_hi - a_lo <= 32);
+    auto shared_turns = [&](bool member, int lanes_each) {
+        const int group = slot_in_wave / lanes_each, group_lane = slot_in_wave - group * lanes_each;
+        const int groups = 64 / lanes_each;
+        for (u64 pending = __ballot(member); pending;) {
+            int owner = -1;
+#pragma unroll
+            for (int g = 0; g < 8; ++g) {
+                if (g >= groups) break;                  // the same in every lane
+                const int next = pending ? __ffsll((long long)pending) - 1 : -1;
+                pending &= pending - 1;
+                if (group == g) owner = next;
+            }
+            const int source = owner < 0 ? 0 : owner;
+            float4 b_wl;
+            b_wl.x = __shfl(wl.x, source); b_wl.y = __shfl(wl.y, source); b_wl.z = __shfl(wl.z, source); b_wl.w = __shfl(wl.w, source);
+            const int b_span = __shfl(packed_span, source), b_pl = __shfl(rec_pl, source), b_pr = __shfl(rec_pr, source);
+            const int b_sectors = __shfl(packed_sectors, source), b_vertices = __shfl(packed_vertices, source);
+            const int b_lo = __shfl(a_lo, source), b_hi = __shfl(a_hi, source);
+            const int b_wall = __shfl(w, source);
+            const int x = b_lo + group_lane;
+            if (owner < 0 || x >= b_hi) continue;
+            float rx, ry; ray_direction(c, x, &rx, &ry);
+            const Eval e = eval_segment(b_wl, b_span & 0xFF, b_pl, b_pr, (b_span & 0x100) != 0, c, x, rx, ry);
+            if (!finitef(e.dist)) continue;
+            const int slot = atomicAdd(&counts[x], 1);
+            if (slot < CAND_MAX) {
+                Cand entry;
+                entry.wall = (unsigned short)b_wall;
+                entry.s0 = (short)(b_sectors & 0xFFFF); entry.s1 = (short)(b_sectors >> 16);
+                entry.v0 = (unsigned short)(b_vertices & 0xFFFF); entry.v1 = (unsigned short)((unsigned)b_vertices >> 16);
+                entry.flags = (unsigned short)(e.flags | ((b_span & 0x200) ? CF_MASKED : 0));
+                entry.dist = e.dist;
+                list[(size_t)slot * SW + x] = entry;
+            } else {
+                atomicOr(sc.status, STATUS_CAND_OVERFLOW);
+            }
+        }
+    };
+    shared_turns(listed && (a_hi - a_lo <= 8), 8);
+    shared_turns(listed && (a_hi - a_lo > 8) && (a_hi - a_lo <= 16), 16);
+    shared_turns(listed && (a_hi - a_lo > 16) && (a_hi - a_lo <= 32), 32);
+    for (u64 pending = __ballot(listed && !narrow); pending; pending &= pending - 1) {
         const int owner = __ffsll((long long)pending) - 1;
         float4 b_wl;
         b_wl.x = bcast(wl.x, owner); b_wl.y = bcast(wl.y, owner); b_wl.z = bcast(wl.z, owner); b_wl.w = bcast(wl.w, owner);
