@@ -2534,7 +2534,7 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
 // one, the sector the per-pixel plane rays selected (engine.py:11145-11163).  Doing both here
 // shades every pixel once, in a kernel light enough to run at full occupancy.
 // ---------------------------------------------------------------------------------------------
-#define SHADE_TILES 12   // 256-pixel tiles per block: 260 tiles per view = 22 blocks per lane
+#define SHADE_TILES 52   // 256-pixel tiles per block: 260 tiles per view = 5 blocks per lane (each block stages the tables once)
 #define SHADE_GROUP 4    // tiles per step
 template <bool DEPTH>   // DEPTH: also keep the depth of every pixel no wall tier covers (frames that draw decals)
 __global__ void __launch_bounds__(256) plane_shade_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
@@ -2668,6 +2668,7 @@ __global__ void __launch_bounds__(128) flat_shade_kernel(DeviceMap dm, int lane_
 // ---------------------------------------------------------------------------------------------
 // sprites: engine.py:10534-10557 (blocking raycast) and 14684-14947
 // ---------------------------------------------------------------------------------------------
+#define SPRITE_ROWS 4   // rows of a sprite column in flight together
 struct SpriteRec {
     float x, y, depth, light;
     i64 depth_fixed, left, right, hstep, yscale, top_fixed, texmid, iscale;
@@ -2758,6 +2759,7 @@ __global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lan
         }
         cover[word] = bits;
     }
+    int clip_wall = -1; i64 clip_near = 0, clip_far = 0; float4 clip_line = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     // painter's order far -> near: repeatedly take the farthest candidate nearer than the last one
     float last_depth = GD_INF; int last_slot = A;
     for (;;) {
@@ -2792,30 +2794,41 @@ __global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lan
             y_lo = (int)clampi(tdiv(-fraction_base, s.iscale) - 1, 0, VH);
             y_hi = (int)clampi(tdiv(((i64)height << 16) - fraction_base, s.iscale) + 2, 0, VH);
         }
-        // four rows per step, each stage's loads issued together so that their latencies overlap
-        for (int yb = y_lo; yb < y_hi; yb += 4) {
-            i64 sv[4]; bool live[4]; unsigned int row_meta[4];
+        // SPRITE_ROWS rows per step, each stage's loads issued together so that their latencies overlap
+        for (int yb = y_lo; yb < y_hi; yb += SPRITE_ROWS) {
+            i64 sv[SPRITE_ROWS]; bool live[SPRITE_ROWS]; unsigned int row_meta[SPRITE_ROWS];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < SPRITE_ROWS; ++j) {
                 const int y = yb + j;
                 sv[j] = (fraction_base + mul64((i64)y, s.iscale)) >> 16;
                 live[j] = y < y_hi && sv[j] >= 0 && sv[j] < height;
                 const size_t i = (size_t)(y < VH ? y : VH - 1) * SW + x;
                 row_meta[j] = meta[i];
             }
-            unsigned char opaque[4], post_top[4], texel[4];
+            // the patch texels do not wait for the clip test: asked for now, they arrive with the meta words
+            unsigned char opaque[SPRITE_ROWS], post_top[SPRITE_ROWS], texel[SPRITE_ROWS];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < SPRITE_ROWS; ++j) {
                 opaque[j] = 0; post_top[j] = 0; texel[j] = 0;
+                if (!live[j]) continue;
+                const size_t t = ((size_t)s.id * m->spr_max_h + sv[j]) * m->spr_max_w + su;
+                opaque[j] = m->spr_opaque[t]; post_top[j] = m->spr_post_top[t]; texel[j] = m->spr_atlas[t];
+            }
+#pragma unroll
+            for (int j = 0; j < SPRITE_ROWS; ++j) {
                 if (!live[j]) continue;
                 const int cw = (int)(row_meta[j] & META_WALL_MASK) - 1;
                 bool visible;
                 if (cw >= 0) {
-                    const WallRec &cg = recs[cw];
-                    i64 cnear = min64(cg.dl, cg.dr), cfar = max64(cg.dl, cg.dr);
-                    const float4 cl = *reinterpret_cast<const float4 *>(m->walls + 4 * cw);
-                    float side = (cl.z - cl.x) * (s.y - cl.y) - (cl.w - cl.y) * (s.x - cl.x);
-                    visible = (cnear > s.depth_fixed) || ((cfar > s.depth_fixed) && (side <= 0));
+                    // runs of rows share their clip linedef: its depths and line are kept from row to row
+                    if (cw != clip_wall) {
+                        const WallRec &cg = recs[cw];
+                        clip_near = min64(cg.dl, cg.dr); clip_far = max64(cg.dl, cg.dr);
+                        clip_line = *reinterpret_cast<const float4 *>(m->walls + 4 * cw);
+                        clip_wall = cw;
+                    }
+                    float side = (clip_line.z - clip_line.x) * (s.y - clip_line.y) - (clip_line.w - clip_line.y) * (s.x - clip_line.x);
+                    visible = (clip_near > s.depth_fixed) || ((clip_far > s.depth_fixed) && (side <= 0));
                 } else {
                     visible = s.depth < GD_INF;   // no clip linedef: the clip depth is infinite
                     // No clip recorded, but a plane of the wall pass shows here: where the flat ray did not
@@ -2833,12 +2846,9 @@ __global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lan
                     }
                 }
                 live[j] = visible;
-                if (!visible) continue;
-                const size_t t = ((size_t)s.id * m->spr_max_h + sv[j]) * m->spr_max_w + su;
-                opaque[j] = m->spr_opaque[t]; post_top[j] = m->spr_post_top[t]; texel[j] = m->spr_atlas[t];
             }
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < SPRITE_ROWS; ++j) {
                 if (!live[j] || !opaque[j]) continue;
                 const int y = yb + j;
                 i64 post_screen_top = (s.top_fixed + mul64(s.yscale, post_top[j])) >> 16;
