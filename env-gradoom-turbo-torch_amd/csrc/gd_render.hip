@@ -2257,7 +2257,7 @@ __device__ __forceinline__ bool pass_advance(const ColumnCtx &cc, ColumnState &c
 
 // engine.py:13424-13744 for one column
 template <bool DEPTH, bool SPLIT>
-__device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const ColumnState &c, PixelBuffers &pb) {
+__device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const ColumnState &c, PixelBuffers &pb, const unsigned char *colormap) {
     const gd_map_desc *m = cc.m;
     const MapView &mv = cc.mv;
     const LaneCtx &L = *cc.c;
@@ -2346,14 +2346,27 @@ __device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const Col
     float light = (tb.light(light_sector) + (float)(L.flash_light * 16)) + contrast;
     i64 shade = wall_shade(light, wall_visibility(wr_fragment.lights ? *wr_fragment.rec : wr, mside, x));
     int y0 = (int)clampi(clipped_top, 0, VH), y1 = (int)clampi(clipped_bottom, 0, VH);
-    for (int y = y0; y < y1; ++y) {
-        i64 screen_delta = (i64)y * FIXED_UNIT - center_fixed + FIXED_UNIT;
-        i64 fraction = shl64(texture_mid, 16 - height_bits) + (mul64(vertical_step, screen_delta) >> 16);
-        i64 mv_ = (fraction & UINT32_MASK) >> (32 - height_bits);
-        unsigned char texel = m->tex_atlas[((size_t)texture_id * m->tex_max_h + mv_) * m->tex_max_w + mu];
-        pb.frame[(size_t)y * SW + x] = m->colormap[shade * 256 + texel];
-        pb.meta[(size_t)y * SW + x] |= META_MASKED;
-        if (DEPTH) pb.scene_depth[(size_t)y * SW + x] = md;
+    // WALL_ROWS rows at a time: texels and meta words are asked for together, then the stores
+    const i64 fraction_base = shl64(texture_mid, 16 - height_bits);
+    for (int yb = y0; yb < y1; yb += WALL_ROWS) {
+        unsigned char texel[WALL_ROWS]; unsigned int word[WALL_ROWS];
+#pragma unroll
+        for (int j = 0; j < WALL_ROWS; ++j) {
+            const int y = yb + j < y1 ? yb + j : y1 - 1;
+            i64 screen_delta = (i64)y * FIXED_UNIT - center_fixed + FIXED_UNIT;
+            i64 fraction = fraction_base + (mul64(vertical_step, screen_delta) >> 16);
+            i64 mv_ = (fraction & UINT32_MASK) >> (32 - height_bits);
+            texel[j] = m->tex_atlas[((size_t)texture_id * m->tex_max_h + mv_) * m->tex_max_w + mu];
+            word[j] = pb.meta[(size_t)y * SW + x];
+        }
+#pragma unroll
+        for (int j = 0; j < WALL_ROWS; ++j) {
+            const int y = yb + j;
+            if (y >= y1) continue;
+            pb.frame[(size_t)y * SW + x] = colormap[shade * 256 + texel[j]];
+            pb.meta[(size_t)y * SW + x] = word[j] | META_MASKED;
+            if (DEPTH) pb.scene_depth[(size_t)y * SW + x] = md;
+        }
     }
 }
 
@@ -2510,7 +2523,7 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
     }
     PROF_T(t5);
     PROF_T(t6);
-    masked_midtexture<DEPTH, SPLIT>(cc, st, pb);
+    masked_midtexture<DEPTH, SPLIT>(cc, st, pb, colormap_lds);
 #ifdef GD_PROFILE
     long long t7 = wall_clock64();
     int prof_cands = cc.count;
