@@ -2416,10 +2416,11 @@ __global__ void __launch_bounds__(1024) strip_order_kernel(int strips, Scratch s
 }
 
 // One wavefront per (lane, 64-column strip).  Strips share nothing but read-only tables; a
-// work-group is WALL_STRIPS_PER_GROUP consecutive strips only so that the LDS copies of those
-// tables are paid once per group rather than once per wavefront (which would cap the CU at a
-// couple of wavefronts per SIMD).  After the staging barrier the wavefronts never meet again.
-#define WALL_STRIPS_PER_GROUP 1
+// work-group is WALL_STRIPS_PER_GROUP strips (neighbours in the longest-first order) only so that the
+// LDS copies of those tables, 16.7 KB, are held once per group rather than once per wavefront: a CU has
+// 160 KB of LDS and room for twelve of these wavefronts (166 registers), so one strip per group would stop
+// at nine.  After the staging barrier the wavefronts never meet again.
+#define WALL_STRIPS_PER_GROUP 2
 // DEPTH: also keep the depth of every wall pixel (frames that draw decals).  SPLIT: the map has linedefs with
 // BSP projection fragments.
 template <bool DEPTH, bool SPLIT>
