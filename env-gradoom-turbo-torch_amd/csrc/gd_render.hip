@@ -1200,7 +1200,7 @@ __device__ __forceinline__ size_t flat_sample_tabled(const Tables &tb, const Lan
 // resolved pixels are never repaired.
 #define SPAN_ROW_SLOTS 8
 // Every pixel of the noted rows, block j of a lane taking rows j, j + SPAN_ROW_SLOTS, ... of both ranges.
-__global__ void __launch_bounds__(SW) flat_span_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
+__global__ void __launch_bounds__(SW) __attribute__((amdgpu_waves_per_eu(8, 8))) flat_span_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
     const int local = blockIdx.y;
     if (local >= lane_count) return;
     const int *span = sc.flat_span + (size_t)local * 4;
@@ -2551,7 +2551,7 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
 #define SHADE_TILES 52   // 256-pixel tiles per block: 260 tiles per view = 5 blocks per lane (each block stages the tables once)
 #define SHADE_GROUP 4    // tiles per step
 template <bool DEPTH>   // DEPTH: also keep the depth of every pixel no wall tier covers (frames that draw decals)
-__global__ void __launch_bounds__(256) plane_shade_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) plane_shade_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
     const gd_map_desc *m = &dm.d;
     __shared__ float4 sector_lds[LDS_SECTORS];
     __shared__ unsigned short sector_level_lds[LDS_SECTORS];
@@ -2689,7 +2689,7 @@ struct SpriteRec {
     int id, flags;   // bit0 alive, bit1 fullbright, bits 8..15 style (signed: -1 opaque, -2 translucent, >= 0 additive)
 };
 
-__global__ void __launch_bounds__(SW) sprite_columns_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc,
+__global__ void __launch_bounds__(SW) __attribute__((amdgpu_waves_per_eu(5, 5))) sprite_columns_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc,
                                                             unsigned char *frame_base, size_t frame_stride) {
     extern __shared__ unsigned char shared_raw[];
     SpriteRec *sp = reinterpret_cast<SpriteRec *>(shared_raw);
