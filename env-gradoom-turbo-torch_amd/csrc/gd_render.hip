@@ -1990,17 +1990,25 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
         if (lower_on) { t0 = min(t0, (int)r.clipped_lower_top); t1 = max(t1, (int)r.clipped_bottom); }
         if (upper_on) { t0 = min(t0, (int)r.clipped_top); t1 = max(t1, (int)r.clipped_upper_bottom); }
         // what the three tiers need per row, worked out once: texture, column, vertical mapping
-        int tier_tex[3]; i64 tier_tu[3], tier_step[3], tier_base[3]; int tier_bits[3];
+        // The texture row of screen row y is bits 32-height_bits .. 31 of
+        //   fraction(y) = (texture_mid << (16 - height_bits)) + ((step * (y * 65536 + 65536 - center)) >> 16).
+        // step * y * 65536 has no low 16 bits, so it shifts out of the floor unchanged, and only the low 32 bits of
+        // the sum are looked at: they advance by the low 32 bits of step per row, whatever the 64-bit terms wrap to.
+        int tier_tex[3]; unsigned tier_frac[3], tier_step[3], tier_shift[3]; size_t tier_texel[3];
         const float tier_origin[3] = {r.view_ceiling, r.other_floor, r.other_ceiling};
         const float toff_y = toff[1] * 65536.0f;
+        const unsigned atlas_w = (unsigned)m->tex_max_w;
 #pragma unroll
         for (int t = 0; t < 3; ++t) {
             tier_tex[t] = r.side_tex[t];
             const int id = tier_tex[t] < 0 ? 0 : tier_tex[t];
-            tier_bits[t] = tb.height_bits(id);
-            tier_tu[t] = u_base & (i64)((1 << tb.width_bits(id)) - 1);
-            tier_step[t] = mul64(swall, shl64(1, 14 - tier_bits[t]));
-            tier_base[t] = shl64(round_to_i64((tier_origin[t] - L.view_z) * 65536.0f + toff_y), 16 - tier_bits[t]);
+            const int bits = tb.height_bits(id);
+            const i64 step = mul64(swall, shl64(1, 14 - bits));
+            const i64 base = shl64(round_to_i64((tier_origin[t] - L.view_z) * 65536.0f + toff_y), 16 - bits);
+            tier_shift[t] = (unsigned)(31 - bits);   // a one-row texture (bits == 0) must shift everything out: two shifts
+            tier_step[t] = (unsigned)step;
+            tier_frac[t] = (unsigned)(base + (mul64(step, FIXED_UNIT - L.center_fixed) >> 16)) + (unsigned)step * (unsigned)t0;
+            tier_texel[t] = (size_t)id * m->tex_max_h * m->tex_max_w + (size_t)(u_base & (i64)((1 << tb.width_bits(id)) - 1));
         }
         // WALL_ROWS rows at a time: texel loads first, so their latencies overlap, then the stores
         for (int yb = t0; yb < t1; yb += WALL_ROWS) {
@@ -2017,11 +2025,11 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
                 tail[j] = group_valid[t] && py >= group_bottom[t];
                 texel[j] = 0;
                 if (draw[j]) {
-                    const i64 screen_delta = (i64)y * FIXED_UNIT - L.center_fixed + FIXED_UNIT;
-                    const i64 fraction = tier_base[t] + (mul64(tier_step[t], screen_delta) >> 16);
-                    const i64 tv = (fraction & UINT32_MASK) >> (32 - tier_bits[t]);
-                    texel[j] = m->tex_atlas[((size_t)tier_tex[t] * m->tex_max_h + tv) * m->tex_max_w + tier_tu[t]];
+                    const unsigned tv = (tier_frac[t] >> tier_shift[t]) >> 1;
+                    texel[j] = m->tex_atlas[tier_texel[t] + __umul24(tv, atlas_w)];
                 }
+#pragma unroll
+                for (int k = 0; k < 3; ++k) tier_frac[k] += tier_step[k];
             }
 #pragma unroll
             for (int j = 0; j < WALL_ROWS; ++j) {
@@ -2347,16 +2355,19 @@ __device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const Col
     i64 shade = wall_shade(light, wall_visibility(wr_fragment.lights ? *wr_fragment.rec : wr, mside, x));
     int y0 = (int)clampi(clipped_top, 0, VH), y1 = (int)clampi(clipped_bottom, 0, VH);
     // WALL_ROWS rows at a time: texels and meta words are asked for together, then the stores
-    const i64 fraction_base = shl64(texture_mid, 16 - height_bits);
+    // as in pass_paint: only the low 32 bits of the row fraction matter, and they advance by the step's low 32 bits
+    const unsigned row_step = (unsigned)vertical_step;
+    const unsigned row_base = (unsigned)(shl64(texture_mid, 16 - height_bits) + (mul64(vertical_step, FIXED_UNIT - center_fixed) >> 16));
+    const size_t texel_base = (size_t)texture_id * m->tex_max_h * m->tex_max_w + (size_t)mu;
+    const unsigned atlas_w = (unsigned)m->tex_max_w;
     for (int yb = y0; yb < y1; yb += WALL_ROWS) {
         unsigned char texel[WALL_ROWS]; unsigned int word[WALL_ROWS];
 #pragma unroll
         for (int j = 0; j < WALL_ROWS; ++j) {
             const int y = yb + j < y1 ? yb + j : y1 - 1;
-            i64 screen_delta = (i64)y * FIXED_UNIT - center_fixed + FIXED_UNIT;
-            i64 fraction = fraction_base + (mul64(vertical_step, screen_delta) >> 16);
-            i64 mv_ = (fraction & UINT32_MASK) >> (32 - height_bits);
-            texel[j] = m->tex_atlas[((size_t)texture_id * m->tex_max_h + mv_) * m->tex_max_w + mu];
+            const unsigned fraction = row_base + row_step * (unsigned)y;
+            const unsigned mv_ = (fraction >> (31 - height_bits)) >> 1;
+            texel[j] = m->tex_atlas[texel_base + __umul24(mv_, atlas_w)];
             word[j] = pb.meta[(size_t)y * SW + x];
         }
 #pragma unroll
