@@ -154,7 +154,11 @@ struct Scratch {    // per-chunk working memory, sized at create
     int *flat_tail;        // [L,2,320] per screen half and column: the sector of the first resolved pixel below the
                            // half's noted rows, -1 if the column was not looking for one or found none
     int *flat_span;        // [L,4] first / last row of the ceiling half, then of the floor half, that holds a shown
-                           // pixel the flat pass could not resolve (208, -1 = none): the rows the repairs work on
+                           // pixel the flat pass could not resolve and whose repair reads its row (208, -1 = none):
+                           // the rows the row repairs work on
+    int *flat_col_top;     // [L,2,320] per screen half and column: the topmost shown pixel the flat pass could not
+                           // resolve (any value >= 208: none).  flat_list_kernel lowers it, flat_gap_column_kernel
+                           // reads it and puts "none" back, so it is filled once, when the renderer is created.
     unsigned int *meta;    // [L,208,320] filled | floor | plane_sector+1 | clip_wall+1
     float *clip_depth;     // [L,208,320]
     unsigned char *frame;  // [L,240,320] when the caller wants no indexed output
@@ -1067,8 +1071,73 @@ __global__ void __launch_bounds__(128) flat_list_kernel(DeviceMap dm, gd_lanes_d
         sc.flat_flags[i] = s < 0 ? 1 : 0;
         if (s < 0) {
             const bool floor_row = ((float)y - flat_center(c)) > 0;
-            atomicMin(&span[floor_row ? 2 : 0], y);
-            atomicMax(&span[floor_row ? 3 : 1], y);
+            atomicMin(&sc.flat_col_top[((size_t)local * 2 + (floor_row ? 1 : 0)) * SW + x], y);
+        }
+    }
+}
+
+// The vertical repair (engine.py:11026-11083) of the listed pixels, column by column.  An unresolved pixel takes
+// the sector of the next resolved pixel below it in its half of the screen; when that sector is not the camera's,
+// the pixel is its own left and right anchor in the horizontal repair (engine.py:11085-11135), which then leaves
+// it as it is: such a pixel is settled here and its row needs no further work.  Only the rows of the others (no
+// resolved pixel below, or the camera's own sector) are noted for the row kernels.  One block per lane; a
+// wavefront takes the columns of its 64-column strip that hold an unresolved listed pixel one after another,
+// its lanes probing 64 rows of the column at a time, from the bottom of the half up to the column's topmost
+// unresolved listed pixel.
+__global__ void __launch_bounds__(SW) flat_gap_column_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
+    const int local = blockIdx.x;
+    if (local >= lane_count) return;
+    const LaneCtx &c = sc.ctx[local];
+    const int n = lane_base + local;
+    const int lane_id = threadIdx.x & 63;
+    int *span = sc.flat_span + (size_t)local * 4;
+    const float center = flat_center(c);
+    int last_ceiling_row = -1;                       // rows 0 .. last_ceiling_row look at ceilings
+    for (int y = 0; y < VH; ++y) if (!(((float)y - center) > 0)) last_ceiling_row = y;
+    const unsigned int *meta = sc.meta + (size_t)local * VH * SW;
+    for (int half = 0; half < 2; ++half) {
+        int *top_at = sc.flat_col_top + ((size_t)local * 2 + half) * SW + threadIdx.x;
+        const int top = *top_at;
+        if (top < VH) *top_at = VH;
+        const int half_end = half ? VH - 1 : last_ceiling_row;
+        for (u64 columns = __ballot(top < VH); columns; columns &= columns - 1) {
+            const int source = __ffsll((long long)columns) - 1;
+            const int x = (threadIdx.x & ~63) + source;
+            const int first = bcast(top, source);
+            const float rc = lanes.ray_cos[(size_t)n * SW + x], rs = lanes.ray_sin[(size_t)n * SW + x], cc = dm.cosine_correction[x];
+            // chunks of 64 rows, the lowest first: what a chunk finds serves the chunks above it
+            bool below_found = false; int below_sector = 0;
+            const int chunks = (half_end - first) / 64 + 1;
+            for (int chunk = chunks - 1; chunk >= 0; --chunk) {
+                const int y = first + chunk * 64 + lane_id;
+                const bool live = y <= half_end;
+                const int s = live ? flat_probe_pixel(dm, sc, local, rc, rs, cc, y) : -1;
+                const u64 resolved = __ballot(live && s >= 0);
+                const u64 lower = lane_id == 63 ? 0 : resolved & ~((2ULL << lane_id) - 1);   // resolved rows of this chunk below this one
+                const int from = lower ? __ffsll((long long)lower) - 1 : lane_id;
+                const int taken = __shfl(s, from);
+                const bool found = lower ? true : below_found;
+                const int sector = lower ? taken : below_sector;
+                if (live && s < 0) {
+                    const size_t i = (size_t)y * SW + x;
+                    const unsigned int word = meta[i];
+                    const bool listed = !(word & (META_FILLED | META_MASKED)) && ((word >> META_SECTOR_SHIFT) & META_SECTOR_MASK) == 0;
+                    if (listed) {
+                        if (found && sector != c.sector) {
+                            sc.flat_sector[(size_t)local * VH * SW + i] = (unsigned short)sector;
+                            sc.flat_flags[(size_t)local * VH * SW + i] = (unsigned char)(1 | 2 | 4 | 8);
+                        } else {
+                            atomicMin(&span[half ? 2 : 0], y);
+                            atomicMax(&span[half ? 3 : 1], y);
+                        }
+                    }
+                }
+                if (resolved) {
+                    const int first_resolved = __ffsll((long long)resolved) - 1;
+                    below_sector = __shfl(s, first_resolved);
+                    below_found = true;
+                }
+            }
         }
     }
 }
@@ -3540,6 +3609,7 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     mark();
     // the flat pass, where the walls left it something to decide
     hipLaunchKernelGGL(flat_list_kernel, dim3(count), dim3(128), 0, stream, r->dm, *lanes, base, count, sc);
+    hipLaunchKernelGGL(flat_gap_column_kernel, dim3(count), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
     hipLaunchKernelGGL(flat_span_select_kernel, dim3(SPAN_ROW_SLOTS, count), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
     mark();
     hipLaunchKernelGGL(flat_tail_kernel, dim3(SW / 64, count), dim3(64 * TAIL_ROWS), 0, stream, r->dm, *lanes, base, count, sc);
@@ -3726,6 +3796,8 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.flat_flags);
     if (rc == GD_OK) rc = scratch_alloc(r, L * 4, &sc.flat_span);
     if (rc == GD_OK) rc = scratch_alloc(r, L * 2 * SW, &sc.flat_tail);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * 2 * SW, &sc.flat_col_top);
+    if (rc == GD_OK && hipMemset(sc.flat_col_top, 0x7f, L * 2 * SW * sizeof(int)) != hipSuccess) rc = fail(GD_E_HIP, "hipMemset flat_col_top");
     if (rc == GD_OK) rc = scratch_alloc(r, L * FLAT_LIST_MAX, &sc.flat_list);
     if (rc == GD_OK) rc = scratch_alloc(r, L, &sc.flat_list_count);
     if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.meta);
