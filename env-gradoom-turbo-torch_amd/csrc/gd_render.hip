@@ -1081,8 +1081,7 @@ __global__ void __launch_bounds__(128) flat_list_kernel(DeviceMap dm, gd_lanes_d
 // the pixel is its own left and right anchor in the horizontal repair (engine.py:11085-11135), which then leaves
 // it as it is: such a pixel is settled here and its row needs no further work.  Only the rows of the others (no
 // resolved pixel below, or the camera's own sector) are noted for the row kernels.  One block per lane; a
-// wavefront takes the columns of its 64-column strip that hold an unresolved listed pixel one after another,
-// its lanes probing 64 rows of the column at a time, from the bottom of the half up to the column's topmost
+// wavefront takes one column that holds an unresolved listed pixel after another, its lanes probing 64 rows of the column at a time, from the bottom of the half up to the column's topmost
 // unresolved listed pixel.
 __global__ void __launch_bounds__(SW) flat_gap_column_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
     const int local = blockIdx.x;
@@ -1095,53 +1094,62 @@ __global__ void __launch_bounds__(SW) flat_gap_column_kernel(DeviceMap dm, gd_la
     int last_ceiling_row = -1;                       // rows 0 .. last_ceiling_row look at ceilings
     for (int y = 0; y < VH; ++y) if (!(((float)y - center) > 0)) last_ceiling_row = y;
     const unsigned int *meta = sc.meta + (size_t)local * VH * SW;
+    // the block's columns with work, both halves together, dealt out to its wavefronts in turn (the columns of a
+    // gap are neighbours: taken strip by strip, one wavefront would do them all)
+    __shared__ int column_list[2 * SW];
+    __shared__ int column_count;
+    if (threadIdx.x == 0) column_count = 0;
+    __syncthreads();
     for (int half = 0; half < 2; ++half) {
         int *top_at = sc.flat_col_top + ((size_t)local * 2 + half) * SW + threadIdx.x;
         const int top = *top_at;
-        if (top < VH) *top_at = VH;
+        if (top < VH) {
+            *top_at = VH;
+            column_list[atomicAdd(&column_count, 1)] = (int)threadIdx.x | (top << 9) | (half << 17);
+        }
+    }
+    __syncthreads();
+    const int columns = column_count;
+    for (int entry = threadIdx.x >> 6; entry < columns; entry += SW / 64) {
+        const int packed = column_list[entry];
+        const int x = packed & 511, first = (packed >> 9) & 255, half = packed >> 17;
         const int half_end = half ? VH - 1 : last_ceiling_row;
-        for (u64 columns = __ballot(top < VH); columns; columns &= columns - 1) {
-            const int source = __ffsll((long long)columns) - 1;
-            const int x = (threadIdx.x & ~63) + source;
-            const int first = bcast(top, source);
-            const float rc = lanes.ray_cos[(size_t)n * SW + x], rs = lanes.ray_sin[(size_t)n * SW + x], cc = dm.cosine_correction[x];
-            // chunks of 64 rows, the lowest first: what a chunk finds serves the chunks above it
-            bool below_found = false; int below_sector = 0;
-            const int chunks = (half_end - first) / 64 + 1;
-            for (int chunk = chunks - 1; chunk >= 0; --chunk) {
-                const int y = first + chunk * 64 + lane_id;
-                const bool live = y <= half_end;
-                const int s = live ? flat_probe_pixel(dm, sc, local, rc, rs, cc, y) : -1;
-                const u64 resolved = __ballot(live && s >= 0);
-                const u64 lower = lane_id == 63 ? 0 : resolved & ~((2ULL << lane_id) - 1);   // resolved rows of this chunk below this one
-                const int from = lower ? __ffsll((long long)lower) - 1 : lane_id;
-                const int taken = __shfl(s, from);
-                const bool found = lower ? true : below_found;
-                const int sector = lower ? taken : below_sector;
-                if (live && s < 0) {
-                    const size_t i = (size_t)y * SW + x;
-                    const unsigned int word = meta[i];
-                    const bool listed = !(word & (META_FILLED | META_MASKED)) && ((word >> META_SECTOR_SHIFT) & META_SECTOR_MASK) == 0;
-                    if (listed) {
-                        if (found && sector != c.sector) {
-                            sc.flat_sector[(size_t)local * VH * SW + i] = (unsigned short)sector;
-                            sc.flat_flags[(size_t)local * VH * SW + i] = (unsigned char)(1 | 2 | 4 | 8);
-                        } else {
-                            atomicMin(&span[half ? 2 : 0], y);
-                            atomicMax(&span[half ? 3 : 1], y);
-                        }
+        const float rc = lanes.ray_cos[(size_t)n * SW + x], rs = lanes.ray_sin[(size_t)n * SW + x], cc = dm.cosine_correction[x];
+        // chunks of 64 rows, the lowest first: what a chunk finds serves the chunks above it
+        bool below_found = false; int below_sector = 0;
+        const int chunks = (half_end - first) / 64 + 1;
+        for (int chunk = chunks - 1; chunk >= 0; --chunk) {
+            const int y = first + chunk * 64 + lane_id;
+            const bool live = y <= half_end;
+            const int s = live ? flat_probe_pixel(dm, sc, local, rc, rs, cc, y) : -1;
+            const u64 resolved = __ballot(live && s >= 0);
+            const u64 lower = resolved & ~((2ULL << lane_id) - 1);   // resolved rows of this chunk below this one (none for lane 63)
+            const int from = lower ? __ffsll((long long)lower) - 1 : lane_id;
+            const int taken = __shfl(s, from);
+            const bool found = lower ? true : below_found;
+            const int sector = lower ? taken : below_sector;
+            if (live && s < 0) {
+                const size_t i = (size_t)y * SW + x;
+                const unsigned int word = meta[i];
+                const bool listed = !(word & (META_FILLED | META_MASKED)) && ((word >> META_SECTOR_SHIFT) & META_SECTOR_MASK) == 0;
+                if (listed) {
+                    if (found && sector != c.sector) {
+                        sc.flat_sector[(size_t)local * VH * SW + i] = (unsigned short)sector;
+                        sc.flat_flags[(size_t)local * VH * SW + i] = (unsigned char)(1 | 2 | 4 | 8);
+                    } else {
+                        atomicMin(&span[half ? 2 : 0], y);
+                        atomicMax(&span[half ? 3 : 1], y);
                     }
                 }
-                if (resolved) {
-                    const int first_resolved = __ffsll((long long)resolved) - 1;
-                    below_sector = __shfl(s, first_resolved);
-                    below_found = true;
-                }
+            }
+            if (resolved) {
+                const int first_resolved = __ffsll((long long)resolved) - 1;
+                below_sector = __shfl(s, first_resolved);
+                below_found = true;
             }
         }
     }
 }
-
 
 // Small per-sector / per-texture tables staged in LDS by the kernels whose inner loops chase
 // them (a dependent global gather costs ~500 cycles, an LDS read ~60).  Sectors or textures
