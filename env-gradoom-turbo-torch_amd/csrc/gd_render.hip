@@ -1297,7 +1297,7 @@ __global__ void __launch_bounds__(SW) __attribute__((amdgpu_waves_per_eu(8, 8)))
 // A column whose pixel in the last noted row of a half is unresolved looks further down for a resolved one
 // (engine.py:11026-11083).  One block per (lane, 64-column strip); its TAIL_ROWS wavefronts select that many rows
 // at a time, while any of the strip's columns is still looking.
-#define TAIL_ROWS 4
+#define TAIL_ROWS 8
 __global__ void __launch_bounds__(64 * TAIL_ROWS) flat_tail_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
     __shared__ int found_lds[TAIL_ROWS][64];
     const int local = blockIdx.y;
@@ -1942,20 +1942,30 @@ struct SilhouetteBounds {
 // Rows [first, last) of one column take `distance` / `wall` as their sprite clip where it is nearer
 // than what they hold.  WALL_ROWS rows at a time, loads first, so the rows' memory latencies overlap.
 __device__ __forceinline__ void clip_rows(PixelBuffers &pb, int x, int first, int last, float distance, int wall) {
-    for (int y0 = first; y0 < last; y0 += WALL_ROWS) {
-        float held[WALL_ROWS]; unsigned int meta[WALL_ROWS];
+    // one batch ahead: the next rows are asked for before this batch's stores (the rows of two batches are distinct)
+    auto load_rows = [&](int y0, float (&held)[WALL_ROWS], unsigned int (&meta)[WALL_ROWS]) {
 #pragma unroll
         for (int j = 0; j < WALL_ROWS; ++j) {
             const size_t i = (size_t)(y0 + j < last ? y0 + j : last - 1) * SW + x;
             held[j] = pb.clip_depth[i]; meta[j] = pb.meta[i];
-            if (!(meta[j] & META_WALL_MASK)) held[j] = GD_INF;   // no clip recorded yet
         }
+    };
+    float held[WALL_ROWS]; unsigned int meta[WALL_ROWS];
+    if (first < last) load_rows(first, held, meta);
+    for (int y0 = first; y0 < last; y0 += WALL_ROWS) {
+        float next_held[WALL_ROWS]; unsigned int next_meta[WALL_ROWS];
+#pragma unroll
+        for (int j = 0; j < WALL_ROWS; ++j) { next_held[j] = 0.0f; next_meta[j] = 0u; }
+        if (y0 + WALL_ROWS < last) load_rows(y0 + WALL_ROWS, next_held, next_meta);
 #pragma unroll
         for (int j = 0; j < WALL_ROWS; ++j) {
-            if (y0 + j >= last || !(distance < held[j])) continue;
+            const float depth = (meta[j] & META_WALL_MASK) ? held[j] : GD_INF;   // no clip recorded yet: infinite
+            if (y0 + j >= last || !(distance < depth)) continue;
             const size_t i = (size_t)(y0 + j) * SW + x;
             pb.clip_depth[i] = distance; pb.meta[i] = (meta[j] & ~META_WALL_MASK) | (unsigned)(wall + 1);
         }
+#pragma unroll
+        for (int j = 0; j < WALL_ROWS; ++j) { held[j] = next_held[j]; meta[j] = next_meta[j]; }
     }
 }
 
@@ -2087,9 +2097,10 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
             tier_frac[t] = (unsigned)(base + (mul64(step, FIXED_UNIT - L.center_fixed) >> 16)) + (unsigned)step * (unsigned)t0;
             tier_texel[t] = (size_t)id * m->tex_max_h * m->tex_max_w + (size_t)(u_base & (i64)((1 << tb.width_bits(id)) - 1));
         }
-        // WALL_ROWS rows at a time: texel loads first, so their latencies overlap, then the stores
-        for (int yb = t0; yb < t1; yb += WALL_ROWS) {
-            unsigned char texel[WALL_ROWS]; bool draw[WALL_ROWS], tail[WALL_ROWS];
+        // WALL_ROWS rows at a time, one batch ahead: the texels of the next batch are asked for before the rows of
+        // this one are stored, so that a step waits for memory once, not for its stores and then for its loads
+        auto load_rows = [&](int yb, unsigned char (&texel)[WALL_ROWS], unsigned &draw, unsigned &tail) {
+            draw = 0; tail = 0;
 #pragma unroll
             for (int j = 0; j < WALL_ROWS; ++j) {
                 const int y = yb + j;
@@ -2098,25 +2109,37 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
                 const bool lower_span = lower_on && (py >= r.clipped_lower_top) && (py < r.clipped_bottom);
                 const bool upper_span = upper_on && (py >= r.clipped_top) && (py < r.clipped_upper_bottom);
                 const int t = one_span ? 0 : (lower_span ? 1 : 2);
-                draw[j] = y < t1 && (one_span || lower_span || upper_span) && tier_tex[t] >= 0;
-                tail[j] = group_valid[t] && py >= group_bottom[t];
+                const bool draws = y < t1 && (one_span || lower_span || upper_span) && tier_tex[t] >= 0;
+                if (draws) draw |= 1u << j;
+                if (group_valid[t] && py >= group_bottom[t]) tail |= 1u << j;
                 texel[j] = 0;
-                if (draw[j]) {
+                if (draws) {
                     const unsigned tv = (tier_frac[t] >> tier_shift[t]) >> 1;
                     texel[j] = m->tex_atlas[tier_texel[t] + __umul24(tv, atlas_w)];
                 }
 #pragma unroll
                 for (int k = 0; k < 3; ++k) tier_frac[k] += tier_step[k];
             }
+        };
+        unsigned char texel[WALL_ROWS]; unsigned draw = 0, tail = 0;
+        if (t0 < t1) load_rows(t0, texel, draw, tail);
+        for (int yb = t0; yb < t1; yb += WALL_ROWS) {
+            unsigned char next_texel[WALL_ROWS]; unsigned next_draw = 0, next_tail = 0;
+#pragma unroll
+            for (int j = 0; j < WALL_ROWS; ++j) next_texel[j] = 0;
+            if (yb + WALL_ROWS < t1) load_rows(yb + WALL_ROWS, next_texel, next_draw, next_tail);
 #pragma unroll
             for (int j = 0; j < WALL_ROWS; ++j) {
-                if (!draw[j]) continue;
+                if (!(draw & (1u << j))) continue;
                 const size_t i = (size_t)(yb + j) * SW + x;
-                const unsigned colour = colormap[(tail[j] ? shade_group : shade_own) * 256 + texel[j]];
+                const unsigned colour = colormap[((tail & (1u << j)) ? shade_group : shade_own) * 256 + texel[j]];
                 pb.clip_depth[i] = r.distance;
                 if (DEPTH) pb.scene_depth[i] = r.distance;
                 pb.meta[i] = META_FILLED | (colour << META_SECTOR_SHIFT) | (unsigned)(wi + 1);
             }
+#pragma unroll
+            for (int j = 0; j < WALL_ROWS; ++j) texel[j] = next_texel[j];
+            draw = next_draw; tail = next_tail;
         }
         if (one_sided) window_dirty = true;
         return;
