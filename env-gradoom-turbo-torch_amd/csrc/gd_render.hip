@@ -191,7 +191,7 @@ __device__ __forceinline__ i64 mul64(i64 a, i64 b) { return (i64)((u64)a * (u64)
 __device__ __forceinline__ i64 shl64(i64 a, int s) { return (i64)((u64)a << s); }
 // C truncating division (engine.py:3115-3118).  gfx950 has no 64-bit integer divider; when both
 // magnitudes are below 2^52 the quotient estimated in float64 is within one of the true quotient
-// and one remainder check makes it exact.  Larger operands take the compiler's long division.
+// and one remainder check, also in float64, makes it exact.  Larger operands take the compiler's long division.
 // The rare large-operand case is a compact shift-subtract loop rather than the compiler's
 // unrolled long division, which would be replicated at every call site and push the kernels
 // far past the instruction cache.
@@ -207,16 +207,20 @@ __device__ __forceinline__ u64 udiv_long(u64 n, u64 d) {
 __device__ __forceinline__ i64 tdiv(i64 a, i64 b) {
     u64 ua = a < 0 ? (u64)0 - (u64)a : (u64)a;
     u64 ub = b < 0 ? (u64)0 - (u64)b : (u64)b;
-    u64 uq;
     if (((ua | ub) >> 52) != 0 || ub == 0) {
-        uq = ub == 0 ? 0 : udiv_long(ua, ub);
-    } else {
-        uq = (u64)((double)ua / (double)ub);
-        u64 prod = uq * ub;
-        if (prod > ua) --uq;
-        else if (ua - prod >= ub) ++uq;
+        const u64 uq = ub == 0 ? 0 : udiv_long(ua, ub);
+        return ((a < 0) != (b < 0)) ? -(i64)uq : (i64)uq;
     }
-    return ((a < 0) != (b < 0)) ? -(i64)uq : (i64)uq;
+    // Both conversions are exact.  The rounded quotient, truncated, is the true quotient or one above it; the
+    // remainder a - q * b is an integer below 2^53 in magnitude, so the fused multiply-add returns it exactly and its
+    // sign tells which.  (The int64 product and compare this replaces cost three quarter-rate multiplies.)
+    const double ad = fabs((double)a), bd = fabs((double)b);
+    double q = trunc(ad / bd);
+    const double r = __builtin_fma(-q, bd, ad);
+    if (r < 0.0) q -= 1.0;
+    else if (r >= bd) q += 1.0;
+    if ((a < 0) != (b < 0)) q = -q;
+    return (i64)q;
 }
 // Value of `v` in lane `lane` of the wavefront; `lane` must be the same in every active lane.
 __device__ __forceinline__ int bcast(int v, int lane) { return __builtin_amdgcn_readlane(v, lane); }
