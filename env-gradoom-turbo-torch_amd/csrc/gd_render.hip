@@ -172,7 +172,8 @@ struct Scratch {    // per-chunk working memory, sized at create
     float *level_far;      // [L, floor levels + ceiling levels] upper bound of that distance
     i64 *level_plane;      // [L, floor levels + ceiling levels, 2] plane height (16.16) and its visibility factor
     i64 *row_slope;        // [L, 208] plane distance per unit of plane height on each view row
-    i64 *step_scale;       // [L, 2, 16] flat texture steps per column for every log2 texture size
+    i64 *step_scale;       // [L, 3, 2, 16] per log2 texture size (widths, then heights): the flat texture step per
+                           // column, the fraction at screen column 0, the camera's offset
 };
 #define FLAT_LIST_MAX 1024 // listed gap pixels per lane (a gap is typically one column wide)
 #define PLANE_LEVELS 64    // level lists up to this long are shaded from the per-lane tables
@@ -186,9 +187,20 @@ struct Scratch {    // per-chunk working memory, sized at create
 #define META_WALL_MASK 0xFFFFu    // sprite-clip linedef + 1
 
 #define STATUS_CAND_OVERFLOW 1
+#define STEP_TABLE 96   // int64 entries per lane of Scratch::step_scale
 
 __device__ __forceinline__ i64 mul64(i64 a, i64 b) { return (i64)((u64)a * (u64)b); }
 __device__ __forceinline__ i64 shl64(i64 a, int s) { return (i64)((u64)a << s); }
+// a * b for a multiplier known to fit 32 unsigned bits: two 32-bit multiplies instead of three
+__device__ __forceinline__ i64 mul64_u32(i64 a, unsigned b) { return (i64)((u64)a * (u64)b); }
+// Bits 16..47 of a * b, all that `((a * b) >> 16) & 0xFFFFFFFF` ever looks at: the low words' full product, and of the
+// two cross products only their low 16 bits, which 24-bit multiplies of the operands' low halves give at full rate.
+__device__ __forceinline__ unsigned mul64_bits_16_47(i64 a, i64 b) {
+    const unsigned al = (unsigned)a, ah = (unsigned)((u64)a >> 32), bl = (unsigned)b, bh = (unsigned)((u64)b >> 32);
+    const u64 low = (u64)al * (u64)bl;
+    const unsigned cross = __umul24(al & 0xFFFFu, bh & 0xFFFFu) + __umul24(ah & 0xFFFFu, bl & 0xFFFFu);
+    return (unsigned)(low >> 16) + (cross << 16);
+}
 // C truncating division (engine.py:3115-3118).  gfx950 has no 64-bit integer divider; when both
 // magnitudes are below 2^52 the quotient estimated in float64 is within one of the true quotient
 // and one remainder check, also in float64, makes it exact.  Larger operands take the compiler's long division.
@@ -433,7 +445,13 @@ __global__ void lane_tables_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
     }
     for (int k = threadIdx.x; k < 32; k += blockDim.x) {
         const i64 basis = k < 16 ? c.vsin : c.vcos;
-        sc.step_scale[(size_t)local * 32 + k] = tdiv(shl64(basis, 32 - (k & 15)), FOCAL_X_FIXED);
+        const i64 step = tdiv(shl64(basis, 32 - (k & 15)), FOCAL_X_FIXED);
+        i64 *entry = sc.step_scale + (size_t)local * STEP_TABLE;
+        entry[k] = step;
+        // the texture fraction of screen column 0 (column px is (px - 159) steps from the view axis), and the
+        // camera's own offset in the texture, for the same log2 size
+        entry[32 + k] = (shl64(k < 16 ? c.vcos : -c.vsin, 32 - (k & 15)) >> 16) - mul64(SW / 2 - 1, step);
+        entry[64 + k] = shl64(k < 16 ? c.view_x_fixed : -c.view_y_fixed, 32 - (k & 15)) >> 16;
     }
 }
 
@@ -1241,7 +1259,7 @@ __device__ __forceinline__ unsigned char flat_pixel(const Tables &tb, const unsi
 // product with a power-of-two texture scale is a shift.
 struct LaneTables {
     const i64 *level_plane;   // this lane's [levels][2]
-    const i64 *step_scale;    // this lane's [2][16]
+    const i64 *step_scale;    // this lane's [3][2][16]
     int floors;
 };
 // Returns the texel's offset in the texture atlas and the colormap row, so that a caller can
@@ -1253,23 +1271,24 @@ __device__ __forceinline__ size_t flat_sample_tabled(const Tables &tb, const Lan
     const int width_bits = tb.width_bits(texture), height_bits = tb.height_bits(texture);
     const i64 *plane = lt.level_plane + 2 * (is_floor ? level_index : lt.floors + level_index);
     const i64 plane_height_fixed = plane[0], glob = plane[1];
+    // The same integers as flat_texture_coordinates, with narrower multiplies: base + (px - 159) * step is
+    // (base - 159 * step) + px * step; the row slope and the visibility factor are below 2^31 and not negative
+    // (lane_tables_kernel clamps both); of distance * basefrac only bits 16..47 reach the texel coordinate.
     const i64 xstep_scale = lt.step_scale[width_bits], ystep_scale = lt.step_scale[16 + height_bits];
-    const i64 flat_column = (i64)px - (SW / 2 - 1);
-    const i64 basexfrac = (shl64(c.vcos, 32 - width_bits) >> 16) + mul64(flat_column, xstep_scale);
-    const i64 baseyfrac = (shl64(-c.vsin, 32 - height_bits) >> 16) + mul64(flat_column, ystep_scale);
-    const i64 pviewx = shl64(c.view_x_fixed, 32 - width_bits) >> 16;
-    const i64 pviewy = shl64(-c.view_y_fixed, 32 - height_bits) >> 16;
-    const i64 distance = mul64(plane_height_fixed, yslope) >> 16;
-    const i64 xfrac = ((mul64(distance, basexfrac) >> 16) + pviewx) & UINT32_MASK;
-    const i64 yfrac = ((mul64(distance, baseyfrac) >> 16) + pviewy) & UINT32_MASK;
-    const i64 u = xfrac >> (32 - width_bits), v = yfrac >> (32 - height_bits);
+    const i64 basexfrac = lt.step_scale[32 + width_bits] + mul64_u32(xstep_scale, (unsigned)px);
+    const i64 baseyfrac = lt.step_scale[48 + height_bits] + mul64_u32(ystep_scale, (unsigned)px);
+    const unsigned pviewx = (unsigned)lt.step_scale[64 + width_bits], pviewy = (unsigned)lt.step_scale[80 + height_bits];
+    const i64 distance = mul64_u32(plane_height_fixed, (unsigned)yslope) >> 16;
+    const unsigned xfrac = mul64_bits_16_47(distance, basexfrac) + pviewx;
+    const unsigned yfrac = mul64_bits_16_47(distance, baseyfrac) + pviewy;
+    const unsigned u = (xfrac >> (31 - width_bits)) >> 1, v = (yfrac >> (31 - height_bits)) >> 1;   // two shifts: a size of one shifts by 32
     const float light = tb.light(sector) + (float)(c.flash_light * 16);
     i64 row = c.center_fixed - (i64)py * FIXED_UNIT;
     if (row < 0) row = -row;
-    const i64 visibility = min64(mul64(glob, row) >> 16, 24 * FIXED_UNIT);
+    const i64 visibility = min64(mul64_u32(row, (unsigned)glob) >> 16, 24 * FIXED_UNIT);
     const i64 plane_shade = 64 * FIXED_UNIT - ((i64)light + 12) * (FIXED_UNIT / 4);
     *colormap_row = (int)clampi((plane_shade - visibility) >> 16, 0, 31);
-    return ((size_t)texture * m->tex_max_h + v) * m->tex_max_w + u;
+    return (size_t)(((unsigned)texture * (unsigned)m->tex_max_h + v) * (unsigned)m->tex_max_w + u);   // the atlas is below 4 GiB (checked at create)
 }
 
 // Visplane repair (engine.py:11026-11135) of the row ranges flat_select_kernel noted, one block per lane, one
@@ -2673,7 +2692,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))
     __shared__ unsigned char tex_lds[LDS_TEXTURES];
     __shared__ unsigned char colormap_lds[32 * 256];
     __shared__ i64 level_plane_lds[2 * PLANE_LEVELS * 2];
-    __shared__ i64 step_scale_lds[32];
+    __shared__ i64 step_scale_lds[STEP_TABLE];
     const int local = blockIdx.y;
     if (local >= lane_count) return;     // uniform over the block
     Tables tb;
@@ -2684,7 +2703,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))
     if (tabled) {
         for (int s = threadIdx.x; s < tb.sector_cached; s += blockDim.x) sector_level_lds[s] = dm.sector_level[s];
         for (int k = threadIdx.x; k < 2 * levels; k += blockDim.x) level_plane_lds[k] = sc.level_plane[(size_t)local * levels * 2 + k];
-        if (threadIdx.x < 32) step_scale_lds[threadIdx.x] = sc.step_scale[(size_t)local * 32 + threadIdx.x];
+        if (threadIdx.x < STEP_TABLE) step_scale_lds[threadIdx.x] = sc.step_scale[(size_t)local * STEP_TABLE + threadIdx.x];
     }
     __syncthreads();
     LaneTables lt; lt.level_plane = level_plane_lds; lt.step_scale = step_scale_lds; lt.floors = floors;
@@ -3709,6 +3728,8 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
         if (h->wall_split_slot[w] < -1 || h->wall_split_slot[w] >= h->split_count)
             return fail(GD_E_ARG, "wall_split_slot names a row outside the fragment tables");
     if (!h->additive_luts || !h->translucent_lut) return fail(GD_E_ARG, "missing sprite blend tables");
+    if ((unsigned long long)h->texture_count * (unsigned long long)h->tex_max_h * (unsigned long long)h->tex_max_w >= (1ULL << 32))
+        return fail(GD_E_ARG, "the texture atlas must stay below 4 GiB");
     gd_renderer *r = new (std::nothrow) gd_renderer();
     if (!r) return fail(GD_E_ARG, "out of host memory");
     r->events_ready = false;
@@ -3842,7 +3863,7 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)(h->floor_level_count + h->ceil_level_count), &sc.level_far);
     if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)(h->floor_level_count + h->ceil_level_count) * 2, &sc.level_plane);
     if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)VH, &sc.row_slope);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * 32, &sc.step_scale);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * STEP_TABLE, &sc.step_scale);
     if (rc == GD_OK) rc = scratch_alloc(r, L * SW, &sc.block_hit);
     if (rc == GD_OK) rc = scratch_alloc(r, L * (SW / 64), &sc.strip_key);
     if (rc == GD_OK) rc = scratch_alloc(r, L * (SW / 64), &sc.strip_order);
