@@ -3325,9 +3325,11 @@ __global__ void __launch_bounds__(256) observe_kernel(const unsigned char *index
     for (int sy = 0; sy < 4; ++sy) {
 #pragma unroll
         for (int sx = 0; sx < 5; ++sx) {
-            const int weight = (y_overlap[sy] * x_overlap[sx]) / 48;
+            // overlaps are at most 84, so the product stays below 7226 and (p * 5462) >> 18 is p / 48 exactly; every
+            // factor here fits 24 bits, and 24-bit multiplies run at full rate where 32-bit ones take four times as long
+            const unsigned weight = __umul24(__umul24((unsigned)y_overlap[sy], (unsigned)x_overlap[sx]), 5462u) >> 18;
             const unsigned int colour = pal[tap[sy][sx]];
-            rs += (int)(colour & 0xFFu) * weight; gs += (int)((colour >> 8) & 0xFFu) * weight; bs += (int)(colour >> 16) * weight;
+            rs += (int)__umul24(colour & 0xFFu, weight); gs += (int)__umul24((colour >> 8) & 0xFFu, weight); bs += (int)__umul24(colour >> 16, weight);
         }
     }
     int r = (rs + 800) / 1600, g = (gs + 800) / 1600, b = (bs + 800) / 1600;
