@@ -156,6 +156,8 @@ struct Scratch {    // per-chunk working memory, sized at create
     int *flat_span;        // [L,4] first / last row of the ceiling half, then of the floor half, that holds a shown
                            // pixel the flat pass could not resolve and whose repair reads its row (208, -1 = none):
                            // the rows the row repairs work on
+    int *flat_rows;        // [L*208] the noted rows of every lane as one work list, entry = lane << 8 | row
+    int *flat_row_count;   // [1] its length (cleared by lane_setup_kernel, filled by flat_gap_column_kernel)
     int *flat_col_top;     // [L,2,320] per screen half and column: the topmost shown pixel the flat pass could not
                            // resolve (any value >= 208: none).  flat_list_kernel lowers it, flat_gap_column_kernel
                            // reads it and puts "none" back, so it is filled once, when the renderer is created.
@@ -187,6 +189,7 @@ struct Scratch {    // per-chunk working memory, sized at create
 #define META_WALL_MASK 0xFFFFu    // sprite-clip linedef + 1
 
 #define STATUS_CAND_OVERFLOW 1
+#define SPAN_SELECT_BLOCKS 1536   // flat_span_select_kernel's grid: what 256 compute units hold at eight wavefronts per SIMD
 #define STEP_TABLE 96   // int64 entries per lane of Scratch::step_scale
 
 __device__ __forceinline__ i64 mul64(i64 a, i64 b) { return (i64)((u64)a * (u64)b); }
@@ -498,6 +501,7 @@ __global__ void lane_setup_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_ba
     int *span = sc.flat_span + (size_t)local * 4;
     span[0] = VH; span[1] = -1; span[2] = VH; span[3] = -1;
     sc.flat_list_count[local] = 0;
+    if (local == 0) *sc.flat_row_count = 0;
     for (int x = 0; x < SW; ++x) { sc.cand_count[(size_t)local * SW + x] = 0; sc.block_hit[(size_t)local * SW + x] = ~0ULL; }
 }
 
@@ -1171,6 +1175,17 @@ __global__ void __launch_bounds__(SW) flat_gap_column_kernel(DeviceMap dm, gd_la
             }
         }
     }
+    // The lane's row ranges are final now (only this block touches them): its rows join the work list that
+    // flat_span_select_kernel deals out evenly, whichever lanes they come from.
+    __syncthreads();
+    __shared__ int list_base;
+    const int lo0 = atomicAdd(&span[0], 0), hi0 = atomicAdd(&span[1], 0), lo1 = atomicAdd(&span[2], 0), hi1 = atomicAdd(&span[3], 0);   // read where the atomics above wrote
+    const int rows0 = hi0 < lo0 ? 0 : hi0 - lo0 + 1, rows1 = hi1 < lo1 ? 0 : hi1 - lo1 + 1;
+    if (rows0 + rows1 == 0) return;                  // the same in every thread
+    if (threadIdx.x == 0) list_base = atomicAdd(sc.flat_row_count, rows0 + rows1);
+    __syncthreads();
+    for (int r = threadIdx.x; r < rows0 + rows1; r += blockDim.x)
+        sc.flat_rows[list_base + r] = (local << 8) | (r < rows0 ? lo0 + r : lo1 + (r - rows0));
 }
 
 // Small per-sector / per-texture tables staged in LDS by the kernels whose inner loops chase
@@ -1298,19 +1313,15 @@ __device__ __forceinline__ size_t flat_sample_tabled(const Tables &tb, const Lan
 // one has found it.  Horizontal: an unresolved pixel between a left and a right anchor of one sector takes
 // that sector.  Pixels outside the noted rows need none of this: no shown pixel there is unresolved, and
 // resolved pixels are never repaired.
-#define SPAN_ROW_SLOTS 8
-// Every pixel of the noted rows, block j of a lane taking rows j, j + SPAN_ROW_SLOTS, ... of both ranges.
+// Every pixel of the noted rows: the blocks take the rows of the work list in turn, so that lanes with many rows
+// and lanes with none load the chip alike.  One block per row at a time, one wavefront per 64 columns.
 __global__ void __launch_bounds__(SW) __attribute__((amdgpu_waves_per_eu(8, 8))) flat_span_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
-    const int local = blockIdx.y;
-    if (local >= lane_count) return;
-    const int *span = sc.flat_span + (size_t)local * 4;
-    const int lo[2] = {span[0], span[2]}, hi[2] = {span[1], span[3]};
-    const int rows0 = hi[0] < lo[0] ? 0 : hi[0] - lo[0] + 1, rows1 = hi[1] < lo[1] ? 0 : hi[1] - lo[1] + 1;
-    const int n = lane_base + local;
+    const int total = *sc.flat_row_count;
     const int x = threadIdx.x;
-    for (int r = blockIdx.x; r < rows0 + rows1; r += SPAN_ROW_SLOTS) {
-        const int y = r < rows0 ? lo[0] + r : lo[1] + (r - rows0);
-        const int s = flat_select_pixel(dm, sc, lanes, local, n, x, y, true);
+    for (int entry = blockIdx.x; entry < total; entry += gridDim.x) {
+        const int packed = sc.flat_rows[entry];
+        const int local = packed >> 8, y = packed & 255;
+        const int s = flat_select_pixel(dm, sc, lanes, local, lane_base + local, x, y, true);
         const size_t i = (size_t)local * VH * SW + (size_t)y * SW + x;
         sc.flat_sector[i] = (unsigned short)(s < 0 ? sc.ctx[local].sector : s);
         sc.flat_flags[i] = s < 0 ? 1 : 0;
@@ -3666,7 +3677,7 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     // the flat pass, where the walls left it something to decide
     hipLaunchKernelGGL(flat_list_kernel, dim3(count), dim3(128), 0, stream, r->dm, *lanes, base, count, sc);
     hipLaunchKernelGGL(flat_gap_column_kernel, dim3(count), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
-    hipLaunchKernelGGL(flat_span_select_kernel, dim3(SPAN_ROW_SLOTS, count), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
+    hipLaunchKernelGGL(flat_span_select_kernel, dim3(SPAN_SELECT_BLOCKS), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
     mark();
     hipLaunchKernelGGL(flat_tail_kernel, dim3(SW / 64, count), dim3(64 * TAIL_ROWS), 0, stream, r->dm, *lanes, base, count, sc);
     hipLaunchKernelGGL(flat_span_finish_kernel, dim3(count), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
@@ -3854,6 +3865,8 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.flat_flags);
     if (rc == GD_OK) rc = scratch_alloc(r, L * 4, &sc.flat_span);
     if (rc == GD_OK) rc = scratch_alloc(r, L * 2 * SW, &sc.flat_tail);
+    if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)VH, &sc.flat_rows);
+    if (rc == GD_OK) rc = scratch_alloc(r, 1, &sc.flat_row_count);
     if (rc == GD_OK) rc = scratch_alloc(r, L * 2 * SW, &sc.flat_col_top);
     if (rc == GD_OK && hipMemset(sc.flat_col_top, 0x7f, L * 2 * SW * sizeof(int)) != hipSuccess) rc = fail(GD_E_HIP, "hipMemset flat_col_top");
     if (rc == GD_OK) rc = scratch_alloc(r, L * FLAT_LIST_MAX, &sc.flat_list);
