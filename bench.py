@@ -29,7 +29,7 @@ POSE_SETS = 4
 # of a 4096-lane launch, each scaled by what the same counter reads for a 1 GiB copy
 # (profiles/render_chain_config4_4096lanes.md).  Measured offline; other workloads report null.
 MEASURED_TRAFFIC_PER_LANE = {
-    ("config4", "wall_columns"): 1.061e10 / 4096,
+    ("config4", "wall_columns"): 1.064e10 / 4096,
 }
 
 

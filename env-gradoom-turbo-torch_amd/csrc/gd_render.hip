@@ -189,7 +189,8 @@ struct Scratch {    // per-chunk working memory, sized at create
 #define META_WALL_MASK 0xFFFFu    // sprite-clip linedef + 1
 
 #define STATUS_CAND_OVERFLOW 1
-#define SPAN_SELECT_BLOCKS 1536   // flat_span_select_kernel's grid: what 256 compute units hold at eight wavefronts per SIMD
+#define SPAN_SELECT_BLOCKS 6144   // flat_span_select_kernel's grid: four times what 256 compute units hold at eight wavefronts per
+                                  // SIMD, so that rows of unequal cost even out
 #define STEP_TABLE 96   // int64 entries per lane of Scratch::step_scale
 
 __device__ __forceinline__ i64 mul64(i64 a, i64 b) { return (i64)((u64)a * (u64)b); }
