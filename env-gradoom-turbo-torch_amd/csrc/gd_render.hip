@@ -2829,21 +2829,25 @@ __global__ void __launch_bounds__(128) flat_shade_kernel(DeviceMap dm, int lane_
 // sprites: engine.py:10534-10557 (blocking raycast) and 14684-14947
 // ---------------------------------------------------------------------------------------------
 #define SPRITE_ROWS 4   // rows of a sprite column in flight together
+// Columns per block.  A block lasts as long as its slowest column, so three blocks of 128 (the last one 64 wide) pack
+// the chip better than one of 320; each lists only the sprites that reach its own columns.
+#define SPRITE_COLUMNS 128
 struct SpriteRec {
     float x, y, depth, light;
     i64 depth_fixed, left, right, hstep, yscale, top_fixed, texmid, iscale;
     int id, flags;   // bit0 alive, bit1 fullbright, bits 8..15 style (signed: -1 opaque, -2 translucent, >= 0 additive)
 };
 
-__global__ void __launch_bounds__(SW) __attribute__((amdgpu_waves_per_eu(5, 5))) sprite_columns_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc,
+__global__ void __launch_bounds__(SPRITE_COLUMNS) __attribute__((amdgpu_waves_per_eu(5, 5))) sprite_columns_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc,
                                                             unsigned char *frame_base, size_t frame_stride) {
     extern __shared__ unsigned char shared_raw[];
     SpriteRec *sp = reinterpret_cast<SpriteRec *>(shared_raw);
     const gd_map_desc *m = &dm.d;
-    const int local = blockIdx.x;
+    const int local = blockIdx.y;
     if (local >= lane_count) return;
     const int n = lane_base + local;
     const int A = lanes.sprite_slots;
+    const int x_first = blockIdx.x * SPRITE_COLUMNS, x_end = x_first + SPRITE_COLUMNS < SW ? x_first + SPRITE_COLUMNS : SW;
     // the slots that can reach the screen at all (alive, in front, some column between left and right): the
     // per-column loops below only walk these.  Their order in the list is irrelevant, ties go by slot number.
     unsigned short *on_screen = reinterpret_cast<unsigned short *>(sp + A);
@@ -2875,13 +2879,14 @@ __global__ void __launch_bounds__(SW) __attribute__((amdgpu_waves_per_eu(5, 5)))
         s.texmid = (i64)m->spr_top[s.id] * FIXED_UNIT - round_to_i64((L.view_z - z) * 65536.0f);
         s.top_fixed = L.center_fixed - (mul64(s.texmid, s.yscale) >> 16);
         s.iscale = tdiv(UINT32_MASK, max64(s.yscale, 1));
-        const bool reaches = (s.flags & 1) && (s.depth > 0) && (s.right > 0) && (s.left < SW) && (s.right > s.left);
+        const bool reaches = (s.flags & 1) && (s.depth > 0) && (s.right > x_first) && (s.left < x_end) && (s.right > s.left);
         s.light = reaches ? m->sector_lights[sector_at(m, s.x, s.y)] : 0.0f;
         sp[a] = s;
         if (reaches) on_screen[atomicAdd(&on_screen_count, 1)] = (unsigned short)a;
     }
     __syncthreads();
-    const int x = threadIdx.x;
+    const int x = x_first + threadIdx.x;
+    if (x >= x_end) return;
     const WallRec *recs = sc.rec + (size_t)local * m->wall_count;
     unsigned char *frame = frame_base + (size_t)local * frame_stride;
     const unsigned int *meta = sc.meta + (size_t)local * VH * SW;
@@ -3688,7 +3693,7 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
         hipLaunchKernelGGL(decal_kernel, dim3(count), dim3(SW), 0, stream, r->dm, r->overlays, *lanes, base, count, sc, frame_base, frame_stride);
     if (lanes->sprite_slots > 0 && lanes->sprite_x) {
         size_t shared = (size_t)lanes->sprite_slots * (sizeof(SpriteRec) + sizeof(unsigned short));
-        hipLaunchKernelGGL(sprite_columns_kernel, dim3(count), dim3(SW), shared, stream, r->dm, *lanes, base, count, sc, frame_base, frame_stride);
+        hipLaunchKernelGGL(sprite_columns_kernel, dim3((SW + SPRITE_COLUMNS - 1) / SPRITE_COLUMNS, count), dim3(SPRITE_COLUMNS), shared, stream, r->dm, *lanes, base, count, sc, frame_base, frame_stride);
     }
     if (lanes->weapon_state && r->overlays.d.weapon_patch_count > 0)
         hipLaunchKernelGGL(weapon_overlay_kernel, dim3((VH * SW + 255) / 256, count), dim3(256), 0, stream, r->overlays, lanes->weapon_state, base, count,
