@@ -545,7 +545,9 @@ __device__ __forceinline__ Eval eval_wall(const gd_map_desc *m, const LaneCtx &c
 // ---------------------------------------------------------------------------------------------
 // FWallCoords of one fixed-point segment seen from one lane (engine.py:10747-10869): view-space
 // endpoints, clipped half-open screen span and clipped endpoint depths.
-__device__ __forceinline__ void wall_coords(const LaneCtx &c, const int *wf, WallRec &r) {
+// `endpoint_quotient`, when asked for, receives tx * center / ty (ty == 0 counted as 1) of the linedef's two endpoints
+// in map order: the projections below divide exactly these, whichever endpoint the facing puts first.
+__device__ __forceinline__ void wall_coords(const LaneCtx &c, const int *wf, WallRec &r, i64 *endpoint_quotient = nullptr) {
     i64 rx0 = (i64)wf[0] - c.view_x_fixed, ry0 = (i64)wf[1] - c.view_y_fixed;
     i64 rx1 = (i64)wf[2] - c.view_x_fixed, ry1 = (i64)wf[3] - c.view_y_fixed;
     i64 tx0 = (rx0 * c.vsin - ry0 * c.vcos) >> 20, ty0 = (rx0 * c.vcos + ry0 * c.vsin) >> 20;
@@ -556,10 +558,11 @@ __device__ __forceinline__ void wall_coords(const LaneCtx &c, const int *wf, Wal
     i64 tx1 = front ? tx0 : tx1v, tx2 = front ? tx1v : tx0;
     i64 ty1 = front ? ty0 : ty1v, ty2 = front ? ty1v : ty0;
     const i64 center = 160 * FIXED_UNIT;
-    i64 safe_ty1 = ty1 == 0 ? 1 : ty1, safe_ty2 = ty2 == 0 ? 1 : ty2;
-    i64 left_projected = ((center + tdiv(tx1 * center, safe_ty1)) >> 16) + (tx1 >= 0);
+    const i64 quotient0 = tdiv(tx0 * center, ty0 == 0 ? 1 : ty0), quotient1 = tdiv(tx1v * center, ty1v == 0 ? 1 : ty1v);
+    if (endpoint_quotient) { endpoint_quotient[0] = quotient0; endpoint_quotient[1] = quotient1; }
+    i64 left_projected = ((center + (front ? quotient0 : quotient1)) >> 16) + (tx1 >= 0);
     if (tx1 >= 0) left_projected = min64(left_projected, SW);
-    i64 right_projected = ((center + tdiv(tx2 * center, safe_ty2)) >> 16) + (tx2 >= 0);
+    i64 right_projected = ((center + (front ? quotient1 : quotient0)) >> 16) + (tx2 >= 0);
     if (tx2 >= 0) right_projected = min64(right_projected, SW);
     i64 left_den = tx1 - tx2 - ty2 + ty1, right_den = ty2 - ty1 - tx2 + tx1;
     i64 safe_left_den = left_den == 0 ? 1 : left_den, safe_right_den = right_den == 0 ? 1 : right_den;
@@ -611,7 +614,8 @@ __global__ void __launch_bounds__(128) wall_setup_kernel(DeviceMap dm, int lane_
     const LaneCtx &c = sc.ctx[local];
     const int *wf = m->walls_fixed + 4 * w;
     WallRec r;
-    wall_coords(c, wf, r);
+    i64 endpoint_quotient[2];
+    wall_coords(c, wf, r, endpoint_quotient);
     const i64 tx0 = r.tx0, tx1v = r.tx1, ty0 = r.ty0, ty1v = r.ty1;
     const i64 sl = r.sl, sr = r.sr;
     const i64 center = 160 * FIXED_UNIT;
@@ -726,8 +730,7 @@ __global__ void __launch_bounds__(128) wall_setup_kernel(DeviceMap dm, int lane_
     i64 ep_col[2]; bool ep_vis[2];
     i64 txe[2] = {tx0, tx1v}, tye[2] = {ty0, ty1v};
     for (int e = 0; e < 2; ++e) {
-        i64 safe_ty = tye[e] == 0 ? 1 : tye[e];
-        i64 projected_fixed = center + tdiv(txe[e] * center, safe_ty);
+        i64 projected_fixed = center + endpoint_quotient[e];   // tx * center / ty, as wall_coords divided it
         ep_col[e] = (projected_fixed >> 16) + (txe[e] >= 0);
         ep_vis[e] = (tye[e] > 0) && (txe[e] >= -tye[e]) && (txe[e] <= tye[e]) && (ep_col[e] >= 0) && (ep_col[e] <= SW);
     }
