@@ -1113,7 +1113,7 @@ __global__ void __launch_bounds__(128) flat_list_kernel(DeviceMap dm, gd_lanes_d
 // resolved pixel below, or the camera's own sector) are noted for the row kernels.  One block per lane; a
 // wavefront takes one column that holds an unresolved listed pixel after another, its lanes probing 64 rows of the column at a time, from the bottom of the half up to the column's topmost
 // unresolved listed pixel.
-__global__ void __launch_bounds__(SW) flat_gap_column_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
+__global__ void __launch_bounds__(SW) __attribute__((amdgpu_waves_per_eu(8, 8))) flat_gap_column_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
     const int local = blockIdx.x;
     if (local >= lane_count) return;
     const LaneCtx &c = sc.ctx[local];
