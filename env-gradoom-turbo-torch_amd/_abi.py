@@ -16,6 +16,8 @@ STACK_STEP = 0
 STACK_RESET = 1
 
 GD_OK = 0
+STATIC_SCRATCH_MIB = 64  # gd_render_static: the fixed per-GPU working memory
+STATIC_MAX_LANES = 65536
 GD_E_ARG = -1
 GD_E_HIP = -2
 GD_E_UNSUPPORTED = -3

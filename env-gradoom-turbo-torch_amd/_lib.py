@@ -20,6 +20,7 @@ SYMBOLS = (
     "gd_renderer_set_sector_lights",
     "gd_renderer_set_overlays",
     "gd_render",
+    "gd_render_static",
     "gd_render_timed",
     "gd_observe",
     "gd_expand_rgb24",
@@ -56,6 +57,8 @@ def library() -> C.CDLL:
     lib.gd_renderer_set_sector_lights.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
     lib.gd_render.restype = C.c_int
     lib.gd_render.argtypes = [C.c_void_p, C.POINTER(_abi.LanesDesc), C.POINTER(_abi.FrameOut), C.c_void_p]
+    lib.gd_render_static.restype = C.c_int
+    lib.gd_render_static.argtypes = [C.c_void_p, C.POINTER(_abi.LanesDesc), C.POINTER(_abi.FrameOut), C.c_void_p]
     lib.gd_render_timed.restype = C.c_int
     lib.gd_render_timed.argtypes = [
         C.c_void_p, C.POINTER(_abi.LanesDesc), C.POINTER(_abi.FrameOut), C.c_void_p, C.c_int32, C.POINTER(C.c_float), C.c_int32,

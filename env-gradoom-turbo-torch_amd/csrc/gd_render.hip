@@ -36,6 +36,7 @@
 #include <map>
 #include <new>
 #include <string>
+#include <type_traits>
 #include <vector>
 
 #include "../../include/gradoom_amd.h"
@@ -3571,6 +3572,76 @@ struct gd_renderer {
 
 namespace {
 
+// Working memory of callers that may not allocate (gd_render_static): one array per device, held until the
+// process ends.  In host code the array's name only stands for the symbol; its address on the current
+// device comes from hipGetSymbolAddress, once per device.
+#define STATIC_SCRATCH_BYTES ((size_t)GD_STATIC_SCRATCH_MIB << 20)
+#define STATIC_SCRATCH_DEVICES 64
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+namespace {
+unsigned char *g_static_scratch[STATIC_SCRATCH_DEVICES];
+
+int static_scratch_address(unsigned char **out) {
+    int device = 0;
+    HIP_TRY(hipGetDevice(&device));
+    if (device < 0 || device >= STATIC_SCRATCH_DEVICES) return fail(GD_E_ARG, "device ordinal beyond the static working memory table");
+    if (!g_static_scratch[device]) {
+        unsigned char *ptr = nullptr;
+        HIP_TRY(hipGetSymbolAddress(reinterpret_cast<void **>(&ptr), HIP_SYMBOL(scratch)));
+        if (!ptr) return fail(GD_E_HIP, "hipGetSymbolAddress returned no address for the static working memory");
+        g_static_scratch[device] = ptr;
+    }
+    if (out) *out = g_static_scratch[device];
+    return GD_OK;
+}
+
+__global__ void fill_words_kernel(unsigned int *words, size_t count, unsigned int value) {
+    for (size_t k = (size_t)blockIdx.x * blockDim.x + threadIdx.x; k < count; k += (size_t)gridDim.x * blockDim.x) words[k] = value;
+}
+
+// Lay the per-chunk buffers of `sc` out in one block of device memory for `L` lanes of map `h` (every buffer
+// 256-byte aligned) and return the bytes the layout takes; with a null `base` nothing is assigned and the call
+// only measures.  `status` is not part of the block: the renderer keeps it.  `depth`: also the scene depth plane
+// of frames that draw decals.
+size_t carve_scratch(Scratch &sc, unsigned char *base, size_t L, const gd_map_desc &h, bool depth) {
+    size_t used = 0;
+    auto take = [&](auto **field, size_t count) {
+        typedef typename std::remove_reference<decltype(**field)>::type T;
+        used = (used + 255) & ~(size_t)255;
+        if (base) *field = reinterpret_cast<T *>(base + used);
+        used += (count ? count : 1) * sizeof(T);
+    };
+    const size_t W = h.wall_count, PX = (size_t)VH * SW, levels = (size_t)(h.floor_level_count + h.ceil_level_count);
+    take(&sc.ctx, L);
+    take(&sc.rec, L * W);
+    take(&sc.frag_rec, L * (size_t)(h.split_count > 0 ? h.split_count * h.fragment_slots : 1));
+    take(&sc.cand, L * CAND_MAX * SW);
+    take(&sc.cand_count, L * SW);
+    take(&sc.flat_sector, L * PX);
+    take(&sc.flat_flags, L * PX);
+    take(&sc.flat_span, L * 4);
+    take(&sc.flat_tail, L * 2 * SW);
+    take(&sc.flat_rows, L * (size_t)VH);
+    take(&sc.flat_row_count, 1);
+    take(&sc.flat_col_top, L * 2 * SW);
+    take(&sc.flat_list, L * FLAT_LIST_MAX);
+    take(&sc.flat_list_count, L);
+    take(&sc.meta, L * PX);
+    take(&sc.clip_depth, L * PX);
+    take(&sc.frame, L * (size_t)GD_SCREEN_HEIGHT * SW);
+    take(&sc.level_reach, L * levels);
+    take(&sc.level_far, L * levels);
+    take(&sc.level_plane, L * levels * 2);
+    take(&sc.row_slope, L * (size_t)VH);
+    take(&sc.step_scale, L * STEP_TABLE);
+    take(&sc.block_hit, L * SW);
+    take(&sc.strip_key, L * (SW / 64));
+    take(&sc.strip_order, L * (SW / 64));
+    if (depth) take(&sc.scene_depth, L * PX);
+    return (used + 255) & ~(size_t)255;
+}
+
 template <typename T>
 int upload(gd_renderer *r, const T *host, size_t count, const T **device) {
     if (count == 0) count = 1;
@@ -3735,7 +3806,7 @@ const char *gd_last_error(void) { return g_error.c_str(); }
 
 int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int32_t max_lanes, gd_renderer **out) {
     if (!h || !out || !cosine_correction) return fail(GD_E_ARG, "null argument");
-    if (max_lanes <= 0) return fail(GD_E_ARG, "max_lanes must be positive");
+    if (max_lanes < 0) return fail(GD_E_ARG, "max_lanes must not be negative");
     if (h->wall_count <= 0 || h->sector_count <= 0) return fail(GD_E_ARG, "empty map");
     if (h->wall_count >= 65535) return fail(GD_E_ARG, "at most 65534 linedefs");
     if (h->sector_count >= 8191) return fail(GD_E_ARG, "at most 8190 sectors");
@@ -3860,39 +3931,24 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
         if (rc == GD_OK) rc = upload(r, cell_item.data(), cell_item.size(), &r->dm.cell_item);
         if (rc == GD_OK) rc = upload(r, cell_edge.data(), cell_edge.size(), &r->dm.cell_edge);
     }
-    // Working memory for one chunk of lanes; larger batches are rendered chunk by chunk.
+    // Working memory for one chunk of lanes; larger batches are rendered chunk by chunk.  A renderer made for no
+    // lanes holds the map only and renders through gd_render_static.
     const int chunk = max_lanes < 4096 ? max_lanes : 4096;
     r->chunk_lanes = chunk;
-    const size_t L = chunk, PX = (size_t)VH * SW;
     Scratch &sc = r->sc;
-    if (rc == GD_OK) rc = scratch_alloc(r, L, &sc.ctx);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * W, &sc.rec);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)(h->split_count > 0 ? h->split_count * h->fragment_slots : 1), &sc.frag_rec);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * CAND_MAX * SW, &sc.cand);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * SW, &sc.cand_count);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.flat_sector);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.flat_flags);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * 4, &sc.flat_span);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * 2 * SW, &sc.flat_tail);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)VH, &sc.flat_rows);
-    if (rc == GD_OK) rc = scratch_alloc(r, 1, &sc.flat_row_count);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * 2 * SW, &sc.flat_col_top);
-    if (rc == GD_OK && hipMemset(sc.flat_col_top, 0x7f, L * 2 * SW * sizeof(int)) != hipSuccess) rc = fail(GD_E_HIP, "hipMemset flat_col_top");
-    if (rc == GD_OK) rc = scratch_alloc(r, L * FLAT_LIST_MAX, &sc.flat_list);
-    if (rc == GD_OK) rc = scratch_alloc(r, L, &sc.flat_list_count);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.meta);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * PX, &sc.clip_depth);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)GD_SCREEN_HEIGHT * SW, &sc.frame);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)(h->floor_level_count + h->ceil_level_count), &sc.level_reach);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)(h->floor_level_count + h->ceil_level_count), &sc.level_far);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)(h->floor_level_count + h->ceil_level_count) * 2, &sc.level_plane);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * (size_t)VH, &sc.row_slope);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * STEP_TABLE, &sc.step_scale);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * SW, &sc.block_hit);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * (SW / 64), &sc.strip_key);
-    if (rc == GD_OK) rc = scratch_alloc(r, L * (SW / 64), &sc.strip_order);
+    if (rc == GD_OK && chunk > 0) {
+        unsigned char *block = nullptr;
+        const size_t bytes = carve_scratch(sc, nullptr, (size_t)chunk, *h, false);
+        rc = scratch_alloc(r, bytes, &block);
+        if (rc == GD_OK) {
+            carve_scratch(sc, block, (size_t)chunk, *h, false);
+            hipLaunchKernelGGL(fill_words_kernel, dim3(256), dim3(256), 0, 0, reinterpret_cast<unsigned int *>(sc.flat_col_top), (size_t)chunk * 2 * SW, 0x7f7f7f7fu);
+            if (hipDeviceSynchronize() != hipSuccess) rc = fail(GD_E_HIP, "filling flat_col_top");
+        }
+    }
     if (rc == GD_OK) rc = scratch_alloc(r, 1, &sc.status);
     if (rc == GD_OK && hipMemset(sc.status, 0, sizeof(int)) != hipSuccess) rc = fail(GD_E_HIP, "hipMemset status");
+    if (rc == GD_OK) rc = static_scratch_address(nullptr);   // looked up once per device, outside any stream capture
     if (rc == GD_OK) {
         for (int i = 0; i < 16; ++i) if (hipEventCreate(&r->events[i]) != hipSuccess) rc = fail(GD_E_HIP, "hipEventCreate");
         r->events_ready = rc == GD_OK;
@@ -3930,6 +3986,7 @@ static int check_render_args(gd_renderer *r, const gd_lanes_desc *lanes, const g
 int gd_render(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_out *out, void *stream) {
     int rc = check_render_args(r, lanes, out);
     if (rc != GD_OK) return rc;
+    if (r->chunk_lanes <= 0) return fail(GD_E_ARG, "this renderer was created for 0 lanes and holds no working memory: use gd_render_static");
     hipStream_t caller = static_cast<hipStream_t>(stream);
     for (int base = 0; base < lanes->lane_count; base += r->chunk_lanes) {
         int count = lanes->lane_count - base < r->chunk_lanes ? lanes->lane_count - base : r->chunk_lanes;
@@ -3939,9 +3996,41 @@ int gd_render(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_out *ou
     return GD_OK;
 }
 
+int gd_render_static(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_out *out, void *stream) {
+    int rc = check_render_args(r, lanes, out);
+    if (rc != GD_OK) return rc;
+    unsigned char *block = nullptr;
+    rc = static_scratch_address(&block);
+    if (rc != GD_OK) return rc;
+    const gd_map_desc &m = r->dm.d;
+    const bool decals = lanes->decal_slots > 0 && lanes->decal_state && lanes->decal_geom && r->overlays.d.decal_variant_count > 0;
+    Scratch sc = r->sc;   // keeps the renderer's status word
+    const size_t one = carve_scratch(sc, nullptr, 1, m, decals), two = carve_scratch(sc, nullptr, 2, m, decals);
+    if (one > STATIC_SCRATCH_BYTES)
+        return fail(GD_E_ARG, "map too large for gd_render_static: one lane needs " + std::to_string(one) + " bytes of working memory, the static block holds " +
+                                  std::to_string(STATIC_SCRATCH_BYTES));
+    // the layout grows by a fixed amount per lane, up to the padding between its buffers
+    size_t fit = 1 + (STATIC_SCRATCH_BYTES - one) / (two - one);
+    while (fit > 1 && carve_scratch(sc, nullptr, fit, m, decals) > STATIC_SCRATCH_BYTES) --fit;
+    const int chunk = fit > 4096 ? 4096 : (int)fit;
+    if (lanes->lane_count > GD_STATIC_MAX_LANES)
+        return fail(GD_E_ARG, "gd_render_static renders at most " + std::to_string(GD_STATIC_MAX_LANES) + " lanes per call");
+    carve_scratch(sc, block, (size_t)chunk, m, decals);
+    hipStream_t caller = static_cast<hipStream_t>(stream);
+    // the block keeps whatever the last call left: the one buffer the kernels expect to find ready is filled here
+    hipLaunchKernelGGL(fill_words_kernel, dim3(64), dim3(256), 0, caller, reinterpret_cast<unsigned int *>(sc.flat_col_top), (size_t)chunk * 2 * SW, 0x7f7f7f7fu);
+    for (int base = 0; base < lanes->lane_count; base += chunk) {
+        const int count = lanes->lane_count - base < chunk ? lanes->lane_count - base : chunk;
+        rc = launch_chunk(r, sc, lanes, out, base, count, caller, false);
+        if (rc != GD_OK) return rc;
+    }
+    return GD_OK;
+}
+
 int gd_render_timed(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_out *out, void *stream, int32_t launches, float *ms, int32_t stage_count) {
     int rc = check_render_args(r, lanes, out);
     if (rc != GD_OK) return rc;
+    if (r->chunk_lanes <= 0) return fail(GD_E_ARG, "this renderer was created for 0 lanes and holds no working memory");
     if (!ms || stage_count < STAGE_COUNT - 1 || launches <= 0) return fail(GD_E_ARG, "ms must hold 7 stage times");
     for (int s = 0; s < stage_count; ++s) ms[s] = 0.0f;
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -4015,7 +4104,7 @@ int gd_renderer_set_overlays(gd_renderer *r, const gd_overlay_desc *h) {
         OV(decal_opacity_lut, 32 * 256); OV(decal_black_lut, (size_t)h->decal_black_rows * 256);
         if (rc == GD_OK) {   // the depth buffer decals test against, for one chunk of lanes
             void *ptr = nullptr;
-            if (hipMalloc(&ptr, (size_t)r->chunk_lanes * VH * SW * sizeof(float)) != hipSuccess) rc = fail(GD_E_HIP, "out of device memory for the decal depth buffer");
+            if (hipMalloc(&ptr, (size_t)(r->chunk_lanes > 0 ? r->chunk_lanes : 1) * VH * SW * sizeof(float)) != hipSuccess) rc = fail(GD_E_HIP, "out of device memory for the decal depth buffer");
             else { r->overlay_allocations.push_back(ptr); r->sc.scene_depth = static_cast<float *>(ptr); }
         }
     }

@@ -255,6 +255,20 @@ class HipRenderer:
         _lib.check(self._lib.gd_render(self._handle, C.byref(desc), C.byref(out), C.c_void_p(stream)))
         del keep_lanes, keep_out
 
+    def render_static(self, lanes: LaneState, *, indexed=None, obs=None, frames=None, reset_mask=None, rgb=None,
+                      stack_only_masked: bool = False, final_frames=None) -> None:
+        """``render`` through the entry point that allocates nothing (``gd_render_static``): the working memory is
+        the library's fixed per-GPU array, so a renderer created with ``max_lanes=0`` can call it.  Calls that
+        overlap on one GPU race; ``ValueError`` when one lane of the map does not fit the array."""
+
+        if self._handle is None:
+            raise RuntimeError("renderer is closed")
+        desc, keep_lanes = self._lanes_desc(lanes)
+        out, keep_out = self._out_desc(desc.lane_count, indexed, obs, frames, reset_mask, rgb, stack_only_masked, final_frames)
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        _lib.check(self._lib.gd_render_static(self._handle, C.byref(desc), C.byref(out), C.c_void_p(stream)))
+        del keep_lanes, keep_out
+
     def render_timed(self, lanes: LaneState, launches: int, *, indexed=None, obs=None, frames=None) -> dict[str, float]:
         """Average milliseconds per launch of each kernel stage (HIP events on the current stream)."""
 

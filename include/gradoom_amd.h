@@ -227,7 +227,7 @@ const char *gd_last_error(void);
 /*
  * Upload an immutable map (HOST pointers in `host_map`) to the current HIP
  * device and allocate working memory for batches of up to `max_lanes` lanes
- * (larger batches are rendered in chunks).  `cosine_correction` is a host
+ * (larger batches are rendered in chunks; 0 = none, for gd_render_static only).  `cosine_correction` is a host
  * array of 320 floats, cos(native_ray_offsets) (engine.py:10967), computed by
  * the caller with Torch like every other float32 transcendental input.
  * Replaces DeviceScenario.from_host + the engine ctor precompute
@@ -246,6 +246,19 @@ void gd_renderer_destroy(gd_renderer *r);
  * No allocation, no host synchronisation.
  */
 int gd_render(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_out *out, void *stream);
+
+/*
+ * gd_render for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The
+ * working memory comes from one fixed array of GD_STATIC_SCRATCH_MIB MiB that the library holds on every
+ * GPU it runs on, so `r` may be a renderer created with max_lanes 0 (the map only).  Lanes are rendered
+ * in as many chunks as the array needs; GD_E_ARG when one lane of the map alone does not fit, or
+ * for more than GD_STATIC_MAX_LANES lanes.  Calls no hipMalloc / hipFree.  Every call on a GPU uses that
+ * GPU's one array: calls that overlap on one GPU (two streams, two threads) race.
+ */
+#define GD_STATIC_SCRATCH_MIB 64
+#define GD_STATIC_MAX_LANES 65536
+int gd_render_static(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_out *out, void *stream);
 
 /*
  * Sticky status bits (synchronises the device).  bit0: some screen column had

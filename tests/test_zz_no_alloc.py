@@ -1,0 +1,76 @@
+"""gd_render_static, the entry point that allocates nothing, against gd_render (needs an MI355X)."""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import lane_inputs, load_fixture
+
+pytestmark = pytest.mark.gpu
+
+
+def _render(renderer, call, lanes, count, start, mask):
+    indexed = torch.zeros((count, 240, 320), dtype=torch.uint8, device="cuda:0")
+    obs = torch.zeros((count, 84, 84), dtype=torch.uint8, device="cuda:0")
+    frames = torch.as_tensor(start).to("cuda:0")
+    rgb = torch.zeros((count, 240, 320, 3), dtype=torch.uint8, device="cuda:0")
+    call(lanes, indexed=indexed, obs=obs, frames=frames, reset_mask=torch.as_tensor(mask).to("cuda:0"), rgb=rgb)
+    torch.cuda.synchronize()
+    assert renderer.status() == 0
+    return [t.cpu().numpy() for t in (indexed, obs, frames, rgb)]
+
+
+def test_static_entry_point_equals_gd_render_on_two_calls_in_a_row():
+    # the second call is smaller than the first and finds the array as the first left it
+    from gradoom_amd.renderer import HipRenderer, LaneState
+
+    meta, data, smap, tables = load_fixture("small_midtex_sprites")
+    base = lane_inputs(data)
+    count = meta["lanes"]
+    plain = HipRenderer(smap, 64, "cuda:0", cosine_correction=data["cosine_correction"], tables=tables)
+    bare = HipRenderer(smap, 0, "cuda:0", cosine_correction=data["cosine_correction"], tables=tables)   # the map only
+    rng = np.random.default_rng(17)
+    for total in (61, 7):
+        print(f"static entry point: {total} lanes", flush=True)
+        picks = rng.permutation(total) % count
+        arrays = {k: np.ascontiguousarray(v[picks]) for k, v in base.items()}
+        lanes = LaneState.from_numpy(arrays, "cuda:0")
+        start = rng.integers(0, 256, (total, 4, 84, 84), dtype=np.uint8)
+        mask = (rng.random(total) < 0.4).astype(np.uint8)
+        expected = _render(plain, plain.render, lanes, total, start, mask)
+        ours = _render(bare, bare.render_static, lanes, total, start, mask)
+        for name, a, b in zip(("indexed", "obs", "frames", "rgb"), ours, expected):
+            assert np.array_equal(a, b), name
+        assert np.array_equal(ours[0], data["indexed"][picks])   # and both equal the reference's golden frames
+    with pytest.raises(ValueError):
+        bare.render(lanes, indexed=torch.zeros((total, 240, 320), dtype=torch.uint8, device="cuda:0"))   # no working memory of its own
+    plain.close()
+    bare.close()
+
+
+def test_static_entry_point_rejects_more_lanes_than_its_limit():
+    import ctypes as C
+
+    from gradoom_amd import _abi, _lib, hostmath, mapbuild, synthmap
+    from gradoom_amd.renderer import HipRenderer, LaneState
+    from gradoom_amd.selfcheck import make_lane_arrays
+
+    smap = synthmap.generate_map(31, grid=(6, 5), sectors=26, linedefs=160)
+    tables = mapbuild.build_map_tables(smap)
+    cosine = hostmath.cosine_correction("cpu").numpy()
+    renderer = HipRenderer(smap, 0, "cuda:0", cosine_correction=cosine, tables=tables)
+    lanes = LaneState.from_numpy(make_lane_arrays(smap, synthmap.generate_poses(smap, 2, 5)), "cuda:0")
+    indexed = torch.zeros((2, 240, 320), dtype=torch.uint8, device="cuda:0")
+    renderer.render_static(lanes, indexed=indexed)   # two lanes fit
+    torch.cuda.synchronize()
+    assert int(indexed[:, :208].amax()) > 0
+    # the limit is checked before anything is launched, so claiming more lanes than the tensors hold is safe here
+    desc, keep = renderer._lanes_desc(lanes)
+    desc.lane_count = _abi.STATIC_MAX_LANES + 1
+    out, keep_out = renderer._out_desc(2, indexed, None, None, None, None)
+    with pytest.raises(ValueError, match="at most"):
+        _lib.check(renderer._lib.gd_render_static(renderer._handle, C.byref(desc), C.byref(out), None))
+    del keep, keep_out
+    renderer.close()
