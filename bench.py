@@ -1,12 +1,15 @@
 """Headline benchmark: rendered lane-frames/s (320x240 indexed + 84x84x4 observation) on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config4] [--lanes N] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--repeats R] [--workload config4] [--heights quantised|uniform]
+                    [--lanes N] [--mode full|obs-only|rgb] [--no-cpu]
 
 A step is one pass of the whole hot path over one batch of lanes whose inputs already sit in
 HBM: sector-light flicker update, the Torch float32 ray / sprite-depth tables, the render
 kernel chain and the fused observation + frame-stack update.  Camera poses and sprite lists
-change every step.  One JSON line is printed: metric, value, timing, the roofline of the slowest
-kernel (algorithmic bytes over its launch duration, measured here with HIP events) and a CPU baseline.
+change every step.  After W warm-up steps, R repeats of K steps each are timed (device synchronised around every
+repeat); the value is the median repeat and every sample is listed.  One JSON line is printed: metric, value,
+timing, the roofline of the slowest kernel (algorithmic bytes over its launch duration, measured here with HIP
+events) and a CPU baseline (the scalar C++ restatement of the reference algorithm on every host core).
 """
 
 from __future__ import annotations
@@ -29,7 +32,7 @@ POSE_SETS = 4
 # of a 4096-lane launch, each scaled by what the same counter reads for a 1 GiB copy
 # (profiles/render_chain_config4_4096lanes.md).  Measured offline; other workloads report null.
 MEASURED_TRAFFIC_PER_LANE = {
-    ("config4", "wall_columns"): 1.064e10 / 4096,
+    # (workload, heights, kernel stage)
 }
 
 
@@ -49,13 +52,18 @@ def main() -> int:
     parser.add_argument("--gpus", type=int, default=1)
     parser.add_argument("--steps", type=int, default=10)
     parser.add_argument("--warmup", type=int, default=2)
+    parser.add_argument("--repeats", type=int, default=5, help="timed repeats of --steps steps each; the median is reported")
     parser.add_argument("--workload", default="config4")
+    parser.add_argument("--heights", choices=("quantised", "uniform"), default="quantised",
+                        help="sector heights: the map generator's (floors 0..96 and ceilings 160..256 in steps of 8: 13 plane levels "
+                             "each way) or uniform (floors 0..255, ceilings 64..256 above, whole units: a plane level per sector)")
     parser.add_argument("--lanes", type=int, default=None)
     parser.add_argument("--mode", choices=("full", "obs-only", "rgb"), default="full",
                         help="full: indexed frame + observation stack (the headline metric); obs-only: observation stack "
                              "only, no 320x240 frame handed to the caller; rgb: indexed + RGB24 frame, no observation")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    parser.add_argument("--cpu-lanes", type=int, default=32, help="lanes of the same workload the CPU baseline renders")
+    parser.add_argument("--cpu-lanes", type=int, default=0, help="lanes of the same workload the CPU baseline renders (0: 24 per thread)")
+    parser.add_argument("--cpu-threads", type=int, default=0, help="host threads of the CPU baseline (0: every core this process may use, at most 16)")
     parser.add_argument("--copy-probe-mib", type=int, default=0,
                         help="after the timed region, copy this many MiB device to device once (a kernel of known "
                              "traffic that scales the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -81,6 +89,8 @@ def main() -> int:
     lanes = args.lanes or cfg["lanes"]
     sprites = cfg["sprites"]
     smap = synthmap.generate_config_map(args.workload)
+    if args.heights == "uniform":
+        smap = synthmap.with_variant(smap, 5, heights="uniform")
     tables = mapbuild.build_map_tables(smap)
     cosine = hostmath.cosine_correction("cpu").numpy()
     renderer = HipRenderer(smap, lanes, device, cosine_correction=cosine, tables=tables)
@@ -123,15 +133,19 @@ def main() -> int:
     for k in range(args.warmup):
         step(k)
     torch.cuda.synchronize()
-    started = time.perf_counter()
-    for k in range(args.steps):
-        step(args.warmup + k)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - started
+    repeat_seconds = []
+    for repeat in range(max(1, args.repeats)):
+        started = time.perf_counter()
+        for k in range(args.steps):
+            step(args.warmup + repeat * args.steps + k)
+        torch.cuda.synchronize()
+        repeat_seconds.append(time.perf_counter() - started)
     if renderer.status() != 0:
         print("renderer reported truncated column lists: result invalid", file=sys.stderr)
         return 1
+    elapsed = float(np.median(repeat_seconds))
     value = lanes * args.steps / elapsed
+    samples = [round(lanes * args.steps / seconds, 1) for seconds in repeat_seconds]
 
     # Per-kernel durations with HIP events on the launch stream, same inputs, same region.
     stage_launches = max(2, min(args.steps, 5))
@@ -145,7 +159,7 @@ def main() -> int:
     # render_timed sums a stage over the chunks of one frame; one launch handles `chunk` lanes
     launch_ms = stage_ms[dominant] / chunks
     achieved = bytes_per_lane * chunk / (launch_ms * 1e-3) / 1e9 if launch_ms > 0 else 0.0
-    per_lane_traffic = MEASURED_TRAFFIC_PER_LANE.get((args.workload, dominant))
+    per_lane_traffic = MEASURED_TRAFFIC_PER_LANE.get((args.workload, args.heights, dominant)) if lanes >= chunk else None
     traffic = None if per_lane_traffic is None else round(per_lane_traffic * chunk)
     roofline = dict(
         bound="hbm", kernel=dominant + "_kernel", achieved=round(achieved, 3), peak=HBM_PEAK_GBPS, unit="GB/s",
@@ -166,26 +180,31 @@ def main() -> int:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import oracle  # CPU restatement of the reference algorithm: the reported baseline only
 
-        sample = max(1, min(args.cpu_lanes, lanes))
+        threads = args.cpu_threads or min(len(os.sched_getaffinity(0)), 16)
+        sample = max(1, min(args.cpu_lanes or 24 * threads, lanes))
         poses = synthmap.generate_poses_batch(smap, sample, 100, flash=True)
         spr = synthmap.generate_sprites_batch(smap, sample, sprites, 100) if sprites else None
         arrays = make_lane_arrays(smap, poses, spr)
         oracle.library()
         cpu_started = time.perf_counter()
-        oracle.render(tables, arrays, cosine, frames=np.zeros((sample, 4, 84, 84), np.uint8))
+        oracle.render_parallel(tables, arrays, cosine, threads)
         cpu_elapsed = time.perf_counter() - cpu_started
         cpu_baseline = dict(
-            value=round(sample / cpu_elapsed, 3), unit="lane-frames/s", cores=1, kind="port",
-            sample=f"{sample} lanes of {args.workload} (one frame each), scalar C++ restatement of the reference algorithm, {cpu_elapsed:.1f} s",
+            value=round(sample / cpu_elapsed, 3), unit="lane-frames/s", cores=threads, kind="port",
+            sample=f"{sample} lanes of {args.workload} (one frame each: indexed frame, observation, stack), scalar C++ restatement of the "
+                   f"reference algorithm on {threads} host threads, {cpu_elapsed:.1f} s",
         )
 
     line = dict(
         metric={"full": "rendered lane-frames/sec (320x240 + 84x84x4 obs)", "obs-only": "rendered lane-frames/sec (84x84x4 obs only)",
                 "rgb": "rendered lane-frames/sec (320x240 indexed + RGB24)"}[args.mode], value=round(value, 1), unit="lane-frames/s", n_gpus=1,
-        steps=args.steps, warmup=args.warmup, ms_per_step=round(elapsed / args.steps * 1e3, 3), higher_is_better=True,
+        steps=args.steps, warmup=args.warmup, repeats=len(repeat_seconds), samples=samples,
+        ms_per_step=round(elapsed / args.steps * 1e3, 3), higher_is_better=True,
         scaling="weak", vs_baseline=None, dtype="int64+f32", data="synthetic",
         config=dict(mode=args.mode, workload=f"{args.workload}: {lanes} lanes, {cfg['sectors']} sectors, {cfg['linedefs']} linedefs, "
-                    f"{sprites} sprites/lane, masked midtex p={cfg['midtex']}, per-step sector-light flicker"),
+                    f"{sprites} sprites/lane, masked midtex p={cfg['midtex']}, per-step sector-light flicker, "
+                    + ("sector heights quantised (floors 0..96, ceilings 160..256, steps of 8)" if args.heights == "quantised"
+                       else "sector heights uniform (floors 0..255, ceilings 64..256 above, whole units)")),
         roofline=roofline, cpu_baseline=cpu_baseline,
     )
     print(json.dumps(line))

@@ -22,7 +22,18 @@ GD_E_ARG = -1
 GD_E_HIP = -2
 GD_E_UNSUPPORTED = -3
 
+ABI_VERSION = 2  # GD_ABI_VERSION
+
 _P = C.c_void_p
+
+
+class _Sized(C.Structure):
+    """A descriptor whose first field carries its own size (checked by every entry point)."""
+
+    def __init__(self, *args, **kwargs):
+        super().__init__(*args, **kwargs)
+        self.struct_size = C.sizeof(self)
+
 
 MAP_SCALARS = (
     "wall_count",
@@ -132,16 +143,17 @@ LANE_ARRAYS = (
 OUT_FIELDS = ("indexed", "obs", "frames", "reset_mask", "rgb", "final_frames")
 
 
-class MapDesc(C.Structure):
+class MapDesc(_Sized):
     _fields_ = (
-        [(name, C.c_int32) for name in MAP_SCALARS]
+        [("struct_size", C.c_uint32)]
+        + [(name, C.c_int32) for name in MAP_SCALARS]
         + [(name, C.c_float) for name in MAP_FLOATS]
         + [(name, _P) for name, _ in MAP_ARRAYS]
     )
 
 
-class LanesDesc(C.Structure):
-    _fields_ = [("lane_count", C.c_int32), ("sprite_slots", C.c_int32), ("decal_slots", C.c_int32)] + [
+class LanesDesc(_Sized):
+    _fields_ = [("struct_size", C.c_uint32), ("lane_count", C.c_int32), ("sprite_slots", C.c_int32), ("decal_slots", C.c_int32)] + [
         (name, _P) for name, _ in LANE_ARRAYS
     ]
 
@@ -174,9 +186,10 @@ DECAL_ARRAYS = (
 )
 
 
-class OverlayDesc(C.Structure):
+class OverlayDesc(_Sized):
     _fields_ = (
-        [(name, C.c_int32) for name in OVERLAY_SCALARS] + [(name, _P) for name, _ in OVERLAY_ARRAYS]
+        [("struct_size", C.c_uint32)]
+        + [(name, C.c_int32) for name in OVERLAY_SCALARS] + [(name, _P) for name, _ in OVERLAY_ARRAYS]
         + [(name, C.c_int32) for name in DECAL_SCALARS] + [(name, _P) for name, _ in DECAL_ARRAYS]
     )
 
@@ -223,8 +236,8 @@ def host_overlay_desc(overlays: dict) -> tuple[OverlayDesc, list]:
     return desc, keep
 
 
-class FrameOut(C.Structure):
-    _fields_ = [(name, _P) for name in OUT_FIELDS] + [("stack_mode", C.c_int32)]
+class FrameOut(_Sized):
+    _fields_ = [("struct_size", C.c_uint32)] + [(name, _P) for name in OUT_FIELDS] + [("stack_mode", C.c_int32), ("obs_source_rows", C.c_int32)]
 
 
 def host_map_desc(tables: dict) -> tuple[MapDesc, list]:
@@ -352,8 +365,9 @@ ACTOR_OUTPUTS = (
 )
 
 
-class ActorDesc(C.Structure):
+class ActorDesc(_Sized):
     _fields_ = (
-        [(name, C.c_int32) for name in ACTOR_SCALARS] + [(name, _P) for name, _ in ACTOR_ARRAYS]
+        [("struct_size", C.c_uint32)]
+        + [(name, C.c_int32) for name in ACTOR_SCALARS] + [(name, _P) for name, _ in ACTOR_ARRAYS]
         + [(name, _P) for name, _ in ACTOR_OUTPUTS]
     )

@@ -13,6 +13,7 @@ from . import _abi, _build
 
 SYMBOLS = (
     "gd_version",
+    "gd_abi_version",
     "gd_last_error",
     "gd_renderer_create",
     "gd_renderer_destroy",
@@ -44,6 +45,11 @@ def library() -> C.CDLL:
     if missing:
         raise RuntimeError(f"{path} does not export {missing}")
     lib.gd_version.restype = C.c_char_p
+    lib.gd_abi_version.restype = C.c_uint32
+    if lib.gd_abi_version() != _abi.ABI_VERSION:
+        raise RuntimeError(
+            f"{path} was built with struct layout version {lib.gd_abi_version()}, this package expects {_abi.ABI_VERSION}: rebuild it"
+        )
     lib.gd_last_error.restype = C.c_char_p
     lib.gd_renderer_create.restype = C.c_int
     lib.gd_renderer_create.argtypes = [C.POINTER(_abi.MapDesc), C.c_void_p, C.c_int32, C.POINTER(C.c_void_p)]

@@ -1199,7 +1199,7 @@ __global__ void __launch_bounds__(SW) __attribute__((amdgpu_waves_per_eu(8, 8)))
 struct Tables {
     const gd_map_desc *m;
     const float4 *sector;          // floor, ceiling, light, bits(floor_tex | ceil_tex << 16)
-    const unsigned char *tex_bits; // log2 width | log2 height << 4
+    const unsigned short *tex_bits; // floor(log2 width) | floor(log2 height) << 4 | (width is no power of two) << 8
     int sector_cached, tex_cached;
     __device__ __forceinline__ float floor_h(int s) const { return s < sector_cached ? sector[s].x : m->sector_heights[2 * s]; }
     __device__ __forceinline__ float ceil_h(int s) const { return s < sector_cached ? sector[s].y : m->sector_heights[2 * s + 1]; }
@@ -1207,11 +1207,20 @@ struct Tables {
     __device__ __forceinline__ int floor_tex(int s) const { return s < sector_cached ? (int)(__float_as_uint(sector[s].w) & 0xFFFFu) : m->sector_floor_tex[s]; }
     __device__ __forceinline__ int ceil_tex(int s) const { return s < sector_cached ? (int)(__float_as_uint(sector[s].w) >> 16) : m->sector_ceil_tex[s]; }
     __device__ __forceinline__ int width_bits(int t) const { return t < tex_cached ? (tex_bits[t] & 15) : ilog2(m->tex_w[t]); }
-    __device__ __forceinline__ int height_bits(int t) const { return t < tex_cached ? (tex_bits[t] >> 4) : ilog2(m->tex_h[t]); }
+    __device__ __forceinline__ int height_bits(int t) const { return t < tex_cached ? ((tex_bits[t] >> 4) & 15) : ilog2(m->tex_h[t]); }
+    // Texture column of a wall: torch.remainder(u, width) (engine.py:12792-12798).  Widths are powers of two
+    // on most maps, where the remainder is a mask; WAD textures of other widths take the division.
+    __device__ __forceinline__ i64 wrap_column(int t, i64 u) const {
+        const bool odd = t < tex_cached ? (tex_bits[t] >> 8) != 0 : (m->tex_w[t] & (m->tex_w[t] - 1)) != 0;
+        if (!odd) return u & (i64)((1 << width_bits(t)) - 1);
+        const i64 width = m->tex_w[t];
+        const i64 r = u - tdiv(u, width) * width;
+        return r < 0 ? r + width : r;
+    }
 };
 
 // Cooperative fill of the LDS tables by the whole block (call before a __syncthreads()).
-__device__ __forceinline__ void stage_tables(const gd_map_desc *m, float4 *sector_lds, unsigned char *tex_lds, Tables &tb) {
+__device__ __forceinline__ void stage_tables(const gd_map_desc *m, float4 *sector_lds, unsigned short *tex_lds, Tables &tb) {
     int sectors = m->sector_count < LDS_SECTORS ? m->sector_count : LDS_SECTORS;
     int textures = m->texture_count < LDS_TEXTURES ? m->texture_count : LDS_TEXTURES;
     for (int s = threadIdx.x; s < sectors; s += blockDim.x) {
@@ -1220,7 +1229,10 @@ __device__ __forceinline__ void stage_tables(const gd_map_desc *m, float4 *secto
         v.w = __uint_as_float(((unsigned)m->sector_floor_tex[s] & 0xFFFFu) | ((unsigned)m->sector_ceil_tex[s] << 16));
         sector_lds[s] = v;
     }
-    for (int t = threadIdx.x; t < textures; t += blockDim.x) tex_lds[t] = (unsigned char)(ilog2(m->tex_w[t]) | (ilog2(m->tex_h[t]) << 4));
+    for (int t = threadIdx.x; t < textures; t += blockDim.x) {
+        const int w = m->tex_w[t];
+        tex_lds[t] = (unsigned short)(ilog2(w) | (ilog2(m->tex_h[t]) << 4) | ((w & (w - 1)) ? 0x100 : 0));
+    }
     tb.m = m; tb.sector = sector_lds; tb.tex_bits = tex_lds; tb.sector_cached = sectors; tb.tex_cached = textures;
 }
 
@@ -2134,7 +2146,7 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
             tier_shift[t] = (unsigned)(31 - bits);   // a one-row texture (bits == 0) must shift everything out: two shifts
             tier_step[t] = (unsigned)step;
             tier_frac[t] = (unsigned)(base + (mul64(step, FIXED_UNIT - L.center_fixed) >> 16)) + (unsigned)step * (unsigned)t0;
-            tier_texel[t] = (size_t)id * m->tex_max_h * m->tex_max_w + (size_t)(u_base & (i64)((1 << tb.width_bits(id)) - 1));
+            tier_texel[t] = (size_t)id * m->tex_max_h * m->tex_max_w + (size_t)tb.wrap_column(id, u_base);
         }
         // WALL_ROWS rows at a time, one batch ahead: the texels of the next batch are asked for before the rows of
         // this one are stored, so that a step waits for memory once, not for its stores and then for its loads
@@ -2203,7 +2215,7 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
                 bool bottom_tail = (one_span && group_valid[0] && py >= group_bottom[0]) ||
                                    (lower_span && group_valid[1] && py >= group_bottom[1]) ||
                                    (upper_span && group_valid[2] && py >= group_bottom[2]);
-                i64 tu = u_base & (i64)((1 << tb.width_bits(texture_id)) - 1);   // floor-mod by a power of two
+                i64 tu = tb.wrap_column(texture_id, u_base);
                 float origin_z = one_span ? r.view_ceiling : (lower_span ? r.other_floor : r.other_ceiling);
                 int height_bits = tb.height_bits(texture_id);
                 i64 vertical_step = mul64(swall, shl64(1, 14 - height_bits));
@@ -2436,7 +2448,7 @@ __device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const Col
     int light_sector = mside == 0 ? front_sector : back_sector;
     const Tables &tb = *cc.tb;
     float world_top = fminf(tb.ceil_h(front_sector), tb.ceil_h(back_sector));
-    int tw = 1 << tb.width_bits(texture_id), th = 1 << tb.height_bits(texture_id);
+    const int th = m->tex_h[texture_id];   // the texture's own height, whatever its row mask (engine.py:13480-13483)
     float owall_top = 0, owall_bottom = 0;
 #pragma unroll 1
     for (int k = 0; k < 2; ++k) {
@@ -2454,7 +2466,7 @@ __device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const Col
     if (msl > 0 && h < 0) h = 0;
     if (h >= repeat) h = repeat - 1;
     i64 offx = round_to_i64(toff[0] * 65536.0f);
-    i64 mu = ((h + offx) >> 16) & (i64)(tw - 1);
+    i64 mu = tb.wrap_column(texture_id, (h + offx) >> 16);
     int height_bits = ilog2(th);
     i64 vertical_step = mul64(swall_cur, shl64(1, 14 - height_bits));
     i64 center_fixed = L.center_fixed;
@@ -2579,7 +2591,7 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
     __shared__ LaneCtx lane_ctxs[WALL_STRIPS_PER_GROUP];
     __shared__ unsigned char colormap_lds[32 * 256];   // shade rows 0..31 are the only ones indexed
     __shared__ float4 sector_lds[LDS_SECTORS];
-    __shared__ unsigned char tex_lds[LDS_TEXTURES];
+    __shared__ unsigned short tex_lds[LDS_TEXTURES];
     const int wave_in_group = threadIdx.x >> 6;
     const int strip_slot = blockIdx.x * WALL_STRIPS_PER_GROUP + wave_in_group;
     const bool live = strip_slot < lane_count * (SW / 64);
@@ -2705,7 +2717,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))
     const gd_map_desc *m = &dm.d;
     __shared__ float4 sector_lds[LDS_SECTORS];
     __shared__ unsigned short sector_level_lds[LDS_SECTORS];
-    __shared__ unsigned char tex_lds[LDS_TEXTURES];
+    __shared__ unsigned short tex_lds[LDS_TEXTURES];
     __shared__ unsigned char colormap_lds[32 * 256];
     __shared__ i64 level_plane_lds[2 * PLANE_LEVELS * 2];
     __shared__ i64 step_scale_lds[STEP_TABLE];
@@ -3555,6 +3567,14 @@ int fail(int code, const std::string &message) { g_error = message; return code;
         if (e_ != hipSuccess) return fail(GD_E_HIP, std::string(#expr) + ": " + hipGetErrorString(e_)); \
     } while (0)
 
+// A descriptor filled in against another version of the header is refused before any of its fields is trusted.
+#define SIZE_CHECK(ptr, type)                                                                  \
+    do {                                                                                       \
+        if ((ptr)->struct_size != sizeof(type))                                                \
+            return fail(GD_E_ARG, #type ".struct_size is " + std::to_string((ptr)->struct_size) + ", this library expects " + \
+                                      std::to_string(sizeof(type)) + ": the caller was built against another gradoom_amd.h"); \
+    } while (0)
+
 }  // namespace
 
 // Every kernel of a frame runs on the caller's stream.  (Cutting a batch into chunks or halves pipelined over
@@ -3718,6 +3738,68 @@ void build_fine_tables(std::vector<i64> &sine, std::vector<i64> &tangent) {
     }
 }
 
+// Host-side check of a map descriptor before anything is uploaded: every index a kernel follows must land inside
+// its table (a bad one would be a wild device read), and inputs the renderer does not reproduce are refused.
+int validate_map(const gd_map_desc *h) {
+    const int W = h->wall_count, S = h->sector_count, V = h->vertex_count, T = h->texture_count, K = h->neighbor_slots;
+    const void *const needed[] = {h->walls, h->walls_fixed, h->wall_sectors, h->wall_vertex, h->side_tex, h->side_off, h->wall_len,
+                                  h->direct_neighbor_table, h->solid_bridge_start_ofs, h->solid_bridge_end_ofs, h->vertex_wall_ofs,
+                                  h->sector_wall_ofs, h->sector_edge_ofs, h->grid_cell_ofs, h->grid_item_edge_ofs, h->floor_levels,
+                                  h->ceil_levels, h->sector_heights, h->sector_lights, h->sector_floor_tex, h->sector_ceil_tex,
+                                  h->tex_atlas, h->tex_w, h->tex_h, h->playpal, h->colormap};
+    for (const void *p : needed) if (!p) return fail(GD_E_ARG, "gd_map_desc holds a null table");
+    if (V <= 0 || T <= 0 || K < 0 || h->tex_max_h <= 0 || h->tex_max_w <= 0 || h->blocking_count < 0 || h->sprite_count < 0 ||
+        h->floor_level_count <= 0 || h->ceil_level_count <= 0 || h->grid_nx <= 0 || h->grid_ny <= 0)
+        return fail(GD_E_ARG, "gd_map_desc holds a count out of range");
+    if (K > 0 && (!h->endpoint_neighbors || !h->endpoint_neighbor_starts || !h->endpoint_neighbor_ends)) return fail(GD_E_ARG, "missing endpoint neighbour tables");
+    if (h->blocking_count > 0 && !h->blocking_walls) return fail(GD_E_ARG, "missing blocking_walls");
+    if (h->sprite_count > 0 && (!h->spr_atlas || !h->spr_opaque || !h->spr_post_top || !h->spr_w || !h->spr_h || !h->spr_left || !h->spr_top))
+        return fail(GD_E_ARG, "missing sprite patch tables");
+    for (int s = 0; s < S; ++s) {
+        const float floor_z = h->sector_heights[2 * s], ceiling_z = h->sector_heights[2 * s + 1];
+        if (!(floor_z == floor_z) || !(ceiling_z == ceiling_z)) return fail(GD_E_ARG, "sector_heights holds a NaN");
+        if (ceiling_z < floor_z)
+            return fail(GD_E_UNSUPPORTED, "sector " + std::to_string(s) + " has its ceiling below its floor: such sectors are not rendered like the reference");
+        if (h->sector_floor_tex[s] < 0 || h->sector_floor_tex[s] >= T || h->sector_ceil_tex[s] < 0 || h->sector_ceil_tex[s] >= T)
+            return fail(GD_E_ARG, "a sector's flat names a texture out of range");
+    }
+    for (int t = 0; t < T; ++t)
+        if (h->tex_w[t] <= 0 || h->tex_w[t] > h->tex_max_w || h->tex_h[t] <= 0 || h->tex_h[t] > h->tex_max_h || h->tex_w[t] > 32768 || h->tex_h[t] > 32768)
+            return fail(GD_E_ARG, "a texture size lies outside 1..32768 or outside the atlas");
+    for (int p = 0; p < h->sprite_count; ++p)
+        if (h->spr_w[p] < 0 || h->spr_w[p] > h->spr_max_w || h->spr_h[p] < 0 || h->spr_h[p] > h->spr_max_h)
+            return fail(GD_E_ARG, "a sprite patch is larger than its atlas");
+    for (int w = 0; w < W; ++w) {
+        const int front = h->wall_sectors[2 * w], back = h->wall_sectors[2 * w + 1];
+        if (front < 0 || front >= S || back < -1 || back >= S) return fail(GD_E_ARG, "wall_sectors names a sector out of range");
+        for (int e = 0; e < 2; ++e) if (h->wall_vertex[2 * w + e] < 0 || h->wall_vertex[2 * w + e] >= V) return fail(GD_E_ARG, "wall_vertex names a vertex out of range");
+        for (int k = 0; k < 6; ++k) if (h->side_tex[6 * w + k] < -1 || h->side_tex[6 * w + k] >= T) return fail(GD_E_ARG, "side_tex names a texture out of range");
+        for (int k = 0; k < K; ++k) if (h->endpoint_neighbors[(size_t)w * K + k] < 0 || h->endpoint_neighbors[(size_t)w * K + k] >= W) return fail(GD_E_ARG, "endpoint_neighbors names a linedef out of range");
+        for (int k = 0; k < 2; ++k) if (h->direct_neighbor_table[4 * w + k] < 0 || h->direct_neighbor_table[4 * w + k] >= W) return fail(GD_E_ARG, "direct_neighbor_table names a linedef out of range");
+    }
+    struct Csr { const int *ofs, *idx; int rows, limit; const char *name; };
+    const Csr lists[] = {{h->solid_bridge_start_ofs, h->solid_bridge_start_idx, W, W, "solid_bridge_start"}, {h->solid_bridge_end_ofs, h->solid_bridge_end_idx, W, W, "solid_bridge_end"},
+                         {h->vertex_wall_ofs, h->vertex_wall_idx, V, W, "vertex_wall"}, {h->sector_wall_ofs, h->sector_wall_idx, S, W, "sector_wall"},
+                         {h->sector_edge_ofs, h->sector_edge_idx, S, W, "sector_edge"}};
+    for (const Csr &c : lists) {
+        if (c.ofs[0] != 0) return fail(GD_E_ARG, std::string(c.name) + "_ofs must start at 0");
+        for (int r = 0; r < c.rows; ++r) if (c.ofs[r + 1] < c.ofs[r]) return fail(GD_E_ARG, std::string(c.name) + "_ofs must not decrease");
+        if (c.ofs[c.rows] > 0 && !c.idx) return fail(GD_E_ARG, std::string(c.name) + "_idx is missing");
+        for (int k = 0; k < c.ofs[c.rows]; ++k) if (c.idx[k] < 0 || c.idx[k] >= c.limit) return fail(GD_E_ARG, std::string(c.name) + "_idx names a linedef out of range");
+    }
+    const size_t cells = (size_t)h->grid_nx * h->grid_ny;
+    if (h->grid_cell_ofs[0] != 0) return fail(GD_E_ARG, "grid_cell_ofs must start at 0");
+    for (size_t c = 0; c < cells; ++c) if (h->grid_cell_ofs[c + 1] < h->grid_cell_ofs[c]) return fail(GD_E_ARG, "grid_cell_ofs must not decrease");
+    const int items = h->grid_cell_ofs[cells];
+    if (items > 0 && (!h->grid_item_sector || (h->grid_item_edge_ofs[items] > 0 && !h->grid_item_edges))) return fail(GD_E_ARG, "missing grid item tables");
+    if (h->grid_item_edge_ofs[0] != 0) return fail(GD_E_ARG, "grid_item_edge_ofs must start at 0");
+    for (int it = 0; it < items; ++it) if (h->grid_item_edge_ofs[it + 1] < h->grid_item_edge_ofs[it]) return fail(GD_E_ARG, "grid_item_edge_ofs must not decrease");
+    const size_t fine_cells = (size_t)h->fine_nx * h->fine_ny;
+    for (size_t k = 0; k < fine_cells; ++k)
+        if (FINE_KIND(h->fine_sector[k]) == FINE_DECIDED && (int)(h->fine_sector[k] & 0xFFFFu) >= S) return fail(GD_E_ARG, "fine_sector names a sector out of range");
+    return GD_OK;
+}
+
 const int STAGE_COUNT = 8;
 
 int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_desc *lanes, const gd_frame_out *out, int base, int count, hipStream_t stream, bool timed) {
@@ -3779,7 +3861,7 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     if (out->obs || out->frames) {
         const size_t F = (size_t)GD_OBS_SIZE * GD_OBS_SIZE;
         hipLaunchKernelGGL(observe_kernel, dim3(GD_OBS_SIZE / OBS_BLOCK_ROWS, count), dim3(256), 0, stream,
-                           frame_base, frame_stride, VH, m.playpal, count, out->obs ? out->obs + (size_t)base * F : nullptr,
+                           frame_base, frame_stride, out->obs_source_rows == GD_SCREEN_HEIGHT ? GD_SCREEN_HEIGHT : VH, m.playpal, count, out->obs ? out->obs + (size_t)base * F : nullptr,
                            out->frames ? out->frames + (size_t)base * GD_FRAME_STACK * F : nullptr,
                            out->reset_mask ? out->reset_mask + base : nullptr, out->stack_mode,
                            out->final_frames ? out->final_frames + (size_t)base * GD_FRAME_STACK * F : nullptr,
@@ -3801,11 +3883,13 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
 
 extern "C" {
 
-const char *gd_version(void) { return "gradoom_amd 0.1.0 (gfx950)"; }
+const char *gd_version(void) { return "gradoom_amd 0.2.0 (gfx950)"; }
+uint32_t gd_abi_version(void) { return GD_ABI_VERSION; }
 const char *gd_last_error(void) { return g_error.c_str(); }
 
 int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int32_t max_lanes, gd_renderer **out) {
     if (!h || !out || !cosine_correction) return fail(GD_E_ARG, "null argument");
+    SIZE_CHECK(h, gd_map_desc);
     if (max_lanes < 0) return fail(GD_E_ARG, "max_lanes must not be negative");
     if (h->wall_count <= 0 || h->sector_count <= 0) return fail(GD_E_ARG, "empty map");
     if (h->wall_count >= 65535) return fail(GD_E_ARG, "at most 65534 linedefs");
@@ -3823,6 +3907,7 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     if (!h->additive_luts || !h->translucent_lut) return fail(GD_E_ARG, "missing sprite blend tables");
     if ((unsigned long long)h->texture_count * (unsigned long long)h->tex_max_h * (unsigned long long)h->tex_max_w >= (1ULL << 32))
         return fail(GD_E_ARG, "the texture atlas must stay below 4 GiB");
+    if (int bad = validate_map(h)) return bad;
     gd_renderer *r = new (std::nothrow) gd_renderer();
     if (!r) return fail(GD_E_ARG, "out of host memory");
     r->events_ready = false;
@@ -3968,6 +4053,10 @@ void gd_renderer_destroy(gd_renderer *r) {
 
 static int check_render_args(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_out *out) {
     if (!r || !lanes || !out) return fail(GD_E_ARG, "null argument");
+    SIZE_CHECK(lanes, gd_lanes_desc);
+    SIZE_CHECK(out, gd_frame_out);
+    if (out->obs_source_rows != 0 && out->obs_source_rows != VH && out->obs_source_rows != GD_SCREEN_HEIGHT)
+        return fail(GD_E_ARG, "obs_source_rows must be 208 (or 0) or 240");
     if (lanes->lane_count < 0) return fail(GD_E_ARG, "negative lane count");
     if (!lanes->x || !lanes->y || !lanes->angle || !lanes->view_z || !lanes->x_fixed || !lanes->y_fixed || !lanes->angle_bam ||
         !lanes->pitch_bam || !lanes->ray_cos || !lanes->ray_sin)
@@ -4063,6 +4152,7 @@ int gd_renderer_status(gd_renderer *r, int32_t *status) {
 
 int gd_renderer_set_overlays(gd_renderer *r, const gd_overlay_desc *h) {
     if (!r || !h) return fail(GD_E_ARG, "null argument");
+    SIZE_CHECK(h, gd_overlay_desc);
     if (h->weapon_patch_count < 0 || h->hud_patch_count < 0 || h->weapon_max_h < 0 || h->weapon_max_w < 0 || h->hud_max_h < 0 || h->hud_max_w < 0)
         return fail(GD_E_ARG, "negative overlay size");
     if (h->weapon_patch_count > 0 && (!h->weapon_atlas || !h->weapon_opaque || !h->weapon_w || !h->weapon_h || !h->weapon_left || !h->weapon_top))
@@ -4175,6 +4265,7 @@ int gd_expand_rgb24(const uint8_t *indexed, int32_t rows, const uint8_t *playpal
 
 int gd_pack_actors(const gd_actor_desc *a, void *stream) {
     if (!a) return fail(GD_E_ARG, "null argument");
+    SIZE_CHECK(a, gd_actor_desc);
     const int32_t counts[] = {a->lane_count, a->enemy_slots, a->doll_count, a->player_projectile_slots, a->enemy_projectile_slots,
                               a->fog_slots, a->puff_slots, a->item_count, a->drop_slots};
     for (int32_t v : counts) if (v < 0) return fail(GD_E_ARG, "negative count");

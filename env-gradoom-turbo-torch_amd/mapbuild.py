@@ -204,9 +204,13 @@ def build_map_tables(smap) -> dict[str, np.ndarray | int]:
     tex_atlas = np.ascontiguousarray(smap.texture_atlas, dtype=np.uint8)
     tex_w = np.ascontiguousarray(smap.texture_widths, dtype=np.int32)
     tex_h = np.ascontiguousarray(smap.texture_heights, dtype=np.int32)
+    # Any size from 1 to 32768: wall columns wrap modulo the width, rows and flats modulo 2^floor(log2(size))
+    # (engine.py:12792-12843, 10886-10889), so sizes need not be powers of two.
     for name, values in (("width", tex_w), ("height", tex_h)):
-        if np.any(values <= 0) or np.any(values & (values - 1)):
-            raise ValueError(f"texture {name}s must be powers of two")
+        if np.any(values <= 0) or np.any(values > 32768):
+            raise ValueError(f"texture {name}s must lie in 1..32768")
+    if np.any(tex_w > tex_atlas.shape[2]) or np.any(tex_h > tex_atlas.shape[1]):
+        raise ValueError("a texture is larger than the atlas")
 
     spr_atlas = np.ascontiguousarray(smap.sprite_atlas, dtype=np.uint8)
     spr_opaque = np.ascontiguousarray(smap.sprite_opaque, dtype=np.uint8)

@@ -211,10 +211,13 @@ class HipRenderer:
             desc.hud_state = _require(lanes.hud_state, "hud_state", torch.int32, (count, 9), device).data_ptr()
         return desc, keep
 
-    def _out_desc(self, count, indexed, obs, frames, reset_mask, rgb, stack_only_masked=False, final_frames=None):
+    def _out_desc(self, count, indexed, obs, frames, reset_mask, rgb, stack_only_masked=False, final_frames=None, obs_source_rows=208):
         device = self.device
         out = _abi.FrameOut()
         out.stack_mode = _abi.STACK_RESET if stack_only_masked else _abi.STACK_STEP
+        if obs_source_rows not in (208, 240):
+            raise ValueError("obs_source_rows must be 208 (status bar masked) or 240 (status bar pooled)")
+        out.obs_source_rows = int(obs_source_rows)
         keep = []
         if indexed is not None:
             out.indexed = _require(indexed, "indexed", torch.uint8, (count, 240, 320), device).data_ptr()
@@ -236,7 +239,7 @@ class HipRenderer:
 
     # ------------------------------------------------------------------ entry points
     def render(self, lanes: LaneState, *, indexed=None, obs=None, frames=None, reset_mask=None, rgb=None,
-               stack_only_masked: bool = False, final_frames=None) -> None:
+               stack_only_masked: bool = False, final_frames=None, obs_source_rows: int = 208) -> None:
         """One frame for every lane, written into the given (preallocated) tensors.
 
         ``frames`` is rolled by one and the new observation appended (``engine.py:9545-9548``); lanes
@@ -244,13 +247,15 @@ class HipRenderer:
         ``stack_only_masked`` the unmasked lanes' stacks are left untouched (the reset call).
         ``final_frames`` also receives every lane's stack as the call leaves it: the clone that
         ``step_and_reset_device`` returns as ``final_observations`` (``env.py:915-917``), written by
-        the observation kernel itself.
+        the observation kernel itself.  ``obs_source_rows=240`` pools the status bar rows into the observation
+        instead of masking them black, as an environment made with ``obs_crop=None`` does (``env.py:441``,
+        ``engine.py:15440``).
         """
 
         if self._handle is None:
             raise RuntimeError("renderer is closed")
         desc, keep_lanes = self._lanes_desc(lanes)
-        out, keep_out = self._out_desc(desc.lane_count, indexed, obs, frames, reset_mask, rgb, stack_only_masked, final_frames)
+        out, keep_out = self._out_desc(desc.lane_count, indexed, obs, frames, reset_mask, rgb, stack_only_masked, final_frames, obs_source_rows)
         stream = torch.cuda.current_stream(self.device).cuda_stream
         _lib.check(self._lib.gd_render(self._handle, C.byref(desc), C.byref(out), C.c_void_p(stream)))
         del keep_lanes, keep_out

@@ -253,6 +253,60 @@ def with_blend_tables(smap: SynthMap, seed: int) -> SynthMap:
     )
 
 
+def with_variant(smap: SynthMap, seed: int, *, heights: str | None = None, textures: str | None = None, lights: bool = False) -> SynthMap:
+    """A copy of the map with other sector heights, texture sizes or sector lights (same geometry, same texture ids).
+
+    ``heights="uniform"``: floors uniform in 0..255, ceilings 64..256 above their floor, whole map units (so
+    neighbouring sectors may not overlap vertically at all, and a map has as many plane levels as sectors).
+    ``heights="doors"``: the quantised heights of ``generate_map`` with an eighth of the sectors closed (ceiling
+    at the floor) and a tenth crawl spaces 8..24 units high.
+    ``textures="mixed"``: wall textures of every power-of-two size from 8 to 256 either way, flats 64x64 or 64x128.
+    ``textures="npot"``: half the wall textures have sizes that are no powers of two (WAD textures keep their
+    native size, ``textures.py:209-218``): columns wrap modulo the width, rows modulo 2^floor(log2(height))
+    (``engine.py:12792-12843``).
+    ``lights``: other sector light levels.
+    """
+
+    rng = np.random.default_rng(seed)
+    changes = {}
+    count = len(smap.sector_heights)
+    if heights == "uniform":
+        floors = rng.integers(0, 256, count).astype(np.float32)
+        changes["sector_heights"] = np.stack((floors, floors + rng.integers(64, 257, count).astype(np.float32)), axis=1)
+    elif heights == "doors":
+        sector_heights = smap.sector_heights.copy()
+        kind = rng.random(count)
+        closed = kind < 0.125
+        crawl = (kind >= 0.125) & (kind < 0.225)
+        sector_heights[closed, 1] = sector_heights[closed, 0]
+        sector_heights[crawl, 1] = sector_heights[crawl, 0] + 8.0 * rng.integers(1, 4, int(crawl.sum()))
+        changes["sector_heights"] = sector_heights.astype(np.float32)
+    elif heights is not None:
+        raise ValueError("heights must be 'uniform' or 'doors'")
+    if textures in ("mixed", "npot"):
+        total = len(smap.texture_widths)
+        walls = int(np.min(np.concatenate((smap.sector_floor_texture_ids, smap.sector_ceiling_texture_ids))))   # flats follow the wall textures
+        widths = smap.texture_widths.copy()
+        tex_heights = smap.texture_heights.copy()
+        widths[:walls] = 1 << rng.integers(3, 9, walls)
+        tex_heights[:walls] = 1 << rng.integers(3, 9, walls)
+        if textures == "npot":
+            odd = rng.random(walls) < 0.5
+            widths[:walls][odd] = rng.choice(np.asarray([24, 40, 72, 96, 100, 160, 200]), int(odd.sum()))
+            odd = rng.random(walls) < 0.5
+            tex_heights[:walls][odd] = rng.choice(np.asarray([24, 72, 96, 100, 136, 160, 200]), int(odd.sum()))
+        tex_heights[walls:] = np.where(rng.random(total - walls) < 0.5, 64, 128)
+        atlas = np.zeros((total, int(tex_heights.max()), int(widths.max())), dtype=np.uint8)
+        for t in range(total):
+            atlas[t, : tex_heights[t], : widths[t]] = rng.integers(0, 256, (int(tex_heights[t]), int(widths[t])), dtype=np.uint8)
+        changes.update(texture_atlas=atlas, texture_widths=widths.astype(np.int32), texture_heights=tex_heights.astype(np.int32))
+    elif textures is not None:
+        raise ValueError("textures must be 'mixed' or 'npot'")
+    if lights:
+        changes["sector_lights"] = rng.integers(96, 256, count).astype(np.int16)
+    return dataclasses.replace(smap, **changes)
+
+
 def split_linedefs(smap: SynthMap, seed: int, share: float = 0.2, slots: int = 3) -> SynthMap:
     """Give a share of the linedefs two or three BSP projection fragments (scenario.py:420-454).
 
@@ -527,6 +581,7 @@ def generate_poses(
     flash: bool = False,
     frame: int = 0,
     margin: float = 0.15,
+    eye: str = "standing",
 ) -> Poses:
     """Random camera poses strictly inside sectors (bilinear margin keeps them off the walls).
 
@@ -535,7 +590,7 @@ def generate_poses(
     """
 
     return generate_picked_poses(
-        smap, [(seed, lane) for lane in range(lanes)], pitch=pitch, flash=flash, frame=frame, margin=margin
+        smap, [(seed, lane) for lane in range(lanes)], pitch=pitch, flash=flash, frame=frame, margin=margin, eye=eye
     )
 
 
@@ -547,8 +602,13 @@ def generate_picked_poses(
     flash: bool = False,
     frame: int = 0,
     margin: float = 0.15,
+    eye: str = "standing",
 ) -> Poses:
-    """The poses ``generate_poses`` gives lane ``lane`` under ``seed``, for a list of (seed, lane) pairs."""
+    """The poses ``generate_poses`` gives lane ``lane`` under ``seed``, for a list of (seed, lane) pairs.
+
+    Cameras stand in sectors at least 56 units high, eyes 41 units above the floor (``eye="standing"``) or anywhere
+    from 8 units above the floor to 8 below the ceiling (``eye="any"``: crouching, falling, on a lift).
+    """
 
     lanes = len(picks)
     x = np.zeros(lanes, dtype=np.float32)
@@ -562,6 +622,8 @@ def generate_picked_poses(
     for slot, (seed, lane) in enumerate(picks):
         rng = np.random.default_rng((seed * 65536 + lane) * 4096 + frame)
         s = int(rng.integers(0, sector_count))
+        while smap.sector_heights[s, 1] - smap.sector_heights[s, 0] < 56.0:   # no room to stand (closed doors, crawl spaces)
+            s = int(rng.integers(0, sector_count))
         while True:
             u, v = rng.uniform(margin, 1.0 - margin, 2)
             px, py = _point_in_cell(smap, s, float(u), float(v))
@@ -577,6 +639,11 @@ def generate_picked_poses(
             pitch_bam[slot] = int(rng.integers(-10, 11)) * (182 << 16)
         if flash:
             flash_light[slot] = int(rng.integers(0, 3))
+        if eye == "any":
+            headroom = int(smap.sector_heights[s, 1] - smap.sector_heights[s, 0])
+            view_z[slot] = smap.sector_heights[s, 0] + float(rng.integers(8, headroom - 7))
+        elif eye != "standing":
+            raise ValueError("eye must be 'standing' or 'any'")
         sector[slot] = s
     return Poses(x, y, angle_bam, pitch_bam, view_z, flash_light, sector)
 

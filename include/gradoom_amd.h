@@ -32,6 +32,12 @@ extern "C" {
 #define GD_STACK_STEP 0   /* every lane: roll by one, append (engine.py:9545-9548); lanes with reset_mask set: 4 copies */
 #define GD_STACK_RESET 1  /* lanes with reset_mask set: 4 copies (engine.py:2443-2450); other lanes untouched */
 
+/*
+ * Layout version of the structs below.  Every descriptor also starts with its own sizeof, which each entry
+ * point checks: a caller built against another header gets GD_E_ARG instead of a wild read.
+ */
+#define GD_ABI_VERSION 2
+
 #define GD_OK 0
 #define GD_E_ARG (-1)       /* bad argument: null pointer, negative count, size over a limit */
 #define GD_E_HIP (-2)       /* a HIP runtime call failed */
@@ -47,6 +53,7 @@ extern "C" {
  * from which the same answers are derived on the fly.
  */
 typedef struct gd_map_desc {
+    uint32_t struct_size;    /* sizeof(gd_map_desc) of the header the caller was built with */
     int32_t wall_count;      /* W linedefs */
     int32_t sector_count;    /* S */
     int32_t vertex_count;    /* V distinct endpoints (exact float32 equality) */
@@ -139,6 +146,7 @@ typedef struct gd_map_desc {
  * the kernels only do +,-,*,/ and comparisons.
  */
 typedef struct gd_lanes_desc {
+    uint32_t struct_size;    /* sizeof(gd_lanes_desc) of the header the caller was built with */
     int32_t lane_count;       /* N */
     int32_t sprite_slots;     /* A sprites per lane (0 = none) */
     int32_t decal_slots;      /* D packed wall decals per lane (0 = none) */
@@ -188,6 +196,7 @@ typedef struct gd_lanes_desc {
  * 30..35 owned weapon numbers, 38..43 missing weapon numbers (engine.py:15186-15259).
  */
 typedef struct gd_overlay_desc {
+    uint32_t struct_size;    /* sizeof(gd_overlay_desc) of the header the caller was built with */
     int32_t weapon_patch_count, weapon_max_h, weapon_max_w;
     int32_t hud_patch_count, hud_max_h, hud_max_w;
     const uint8_t *weapon_atlas;    /* [Pw,Hw,Ww] palette indices */
@@ -207,6 +216,7 @@ typedef struct gd_overlay_desc {
 
 /* Output buffers; any pointer may be null to skip that product. */
 typedef struct gd_frame_out {
+    uint32_t struct_size;    /* sizeof(gd_frame_out) of the header the caller was built with */
     uint8_t *indexed;   /* [N,240,320] palette indices; rows 208..239 = 0 (empty status bar) */
     uint8_t *obs;       /* [N,84,84] grayscale policy frame (HUD rows masked black) */
     uint8_t *frames;    /* [N,4,84,84] stack, oldest first: rolled by one and obs appended */
@@ -216,12 +226,17 @@ typedef struct gd_frame_out {
                               the clone step_and_reset_device hands out as final_observations
                               (env.py:915-917), written by the same kernel instead of a second pass */
     int32_t stack_mode; /* GD_STACK_STEP or GD_STACK_RESET */
+    int32_t obs_source_rows; /* rows of the frame the observation pools: 208 (or 0) = the world view, status bar rows
+                                black (render_reference_frame with mask_hud, engine.py:15444-15450); 240 = the status bar
+                                too, as the reference does when the environment is made with obs_crop=None
+                                (env.py:441, engine.py:15440) */
 } gd_frame_out;
 
 typedef struct gd_renderer gd_renderer;
 
 /* library identification; replaces nothing in the reference */
 const char *gd_version(void);
+uint32_t gd_abi_version(void);   /* GD_ABI_VERSION of the header the library was built with */
 const char *gd_last_error(void);
 
 /*
@@ -314,6 +329,7 @@ int gd_expand_rgb24(const uint8_t *indexed, int32_t rows, const uint8_t *playpal
  * drops.  Returns GD_E_ARG for a null pointer or a negative count.
  */
 typedef struct gd_actor_desc {
+    uint32_t struct_size;    /* sizeof(gd_actor_desc) of the header the caller was built with */
     int32_t lane_count, enemy_slots, doll_count, player_projectile_slots, enemy_projectile_slots, fog_slots, puff_slots,
         item_count, drop_slots, attack_frames, death_frames, xdeath_frames, explosion_frames;
     const float *enemy_x;  /* [N,Se] */

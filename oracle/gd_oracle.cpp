@@ -16,9 +16,9 @@
 // synthetic maps (tests/golden/*.npz); functions without such a pin are listed
 // in the header of each section as "parity unpinned".
 //
-// Limits of this restatement (checked, GD_E_UNSUPPORTED otherwise):
-//   * one projection fragment per linedef, equal to the linedef (engine.py:745-755);
-//   * texture sizes are powers of two (engine.py:10888, 12808).
+// Linedefs may carry BSP projection fragments (engine.py:745-767, 11472-11545) and textures may have
+// any size: wall columns wrap modulo the width, rows and flats modulo 2^floor(log2(size))
+// (engine.py:10888, 12792-12843), both as in the reference and both covered by golden cases.
 
 #include "../include/gradoom_amd.h"
 
@@ -30,7 +30,9 @@
 #include <cstdint>
 #include <cstring>
 #include <limits>
+#include <mutex>
 #include <string>
+#include <thread>
 #include <vector>
 
 namespace {
@@ -60,11 +62,10 @@ const float BAM_TO_RADIANS = float(2.0 * M_PI / 4294967296.0);
 
 i64 g_fine_sine[FINE_ANGLES];
 i64 g_fine_tangent[FINE_ANGLES / 2];
-bool g_tables_ready = false;
+std::once_flag g_tables_once;
 
 // engine.py:309-328 (ZDoom R_InitTables)
-void build_tables() {
-    if (g_tables_ready) return;
+void fill_tables() {
     const int quarter = FINE_ANGLES / 4;
     for (int i = 0; i < quarter; ++i) {
         double phase = double(i) * (2.0 * M_PI / FINE_ANGLES);
@@ -80,8 +81,8 @@ void build_tables() {
         if (i == 0) phase += M_PI / FINE_ANGLES;
         g_fine_tangent[i] = (i64)std::trunc(std::tan(phase) * double(FIXED_UNIT) + 0.5);
     }
-    g_tables_ready = true;
 }
+void build_tables() { std::call_once(g_tables_once, fill_tables); }
 
 inline i64 mul64(i64 a, i64 b) { return (i64)((u64)a * (u64)b); }
 inline i64 shl64(i64 a, int s) { return (i64)((u64)a << s); }
@@ -103,7 +104,7 @@ enum {
     COV_GEOMETRIC_PATH, COV_PORTAL_BRIDGE, COV_COMPLETES_PORTAL_BRIDGE, COV_PS_KEEPS_PATH, COV_NO_KEEPS_PATH, COV_BOTTOM_TAIL,
     COV_MASKED_COLUMN, COV_MASKED_EXTENDS, COV_DEAD_COLUMN_REVIVED, COV_COUNT
 };
-long long g_coverage[COV_COUNT];
+thread_local long long g_coverage[COV_COUNT];   // per thread: lanes may be rendered by several threads at once
 #define COVER(name, cond) do { if (cond) ++g_coverage[name]; } while (0)
 
 struct Lane {
@@ -1791,6 +1792,12 @@ static void render_hud(uint8_t *canvas, const int32_t *state) {
 int gdo_render(const gd_map_desc *map, const gd_lanes_desc *lanes, const gd_frame_out *out,
                int32_t lane_begin, int32_t lane_end, const float *cosine_correction, const gdo_debug *dbg) {
     if (!map || !lanes || !out || !cosine_correction) { g_error = "null argument"; return GD_E_ARG; }
+    if (map->struct_size != sizeof(gd_map_desc) || lanes->struct_size != sizeof(gd_lanes_desc) || out->struct_size != sizeof(gd_frame_out)) {
+        g_error = "a descriptor's struct_size does not match this build of the header";
+        return GD_E_ARG;
+    }
+    if (out->obs_source_rows != 0 && out->obs_source_rows != VH && out->obs_source_rows != GD_SCREEN_HEIGHT) { g_error = "obs_source_rows"; return GD_E_ARG; }
+    const int source_rows = out->obs_source_rows == GD_SCREEN_HEIGHT ? GD_SCREEN_HEIGHT : VH;
     Oracle o(map);
     const size_t W = map->wall_count;
     std::vector<uint8_t> obs(size_t(GD_OBS_SIZE) * GD_OBS_SIZE);
@@ -1865,7 +1872,7 @@ int gdo_render(const gd_map_desc *map, const gd_lanes_desc *lanes, const gd_fram
         uint8_t palette[768];
         blended_palette(map->playpal, lanes->screen_blend ? lanes->screen_blend + 2 * size_t(n) : nullptr, palette);
         if (out->obs || out->frames) {
-            observe_lane(full.data(), VH, palette, obs.data());  // HUD rows masked black
+            observe_lane(full.data(), source_rows, palette, obs.data());  // 208: HUD rows masked black (engine.py:15444-15450)
             if (out->obs) std::memcpy(out->obs + size_t(n) * obs.size(), obs.data(), obs.size());
             if (out->frames) stack_lane(obs.data(), out->frames + size_t(n) * GD_FRAME_STACK * obs.size(), out->reset_mask && out->reset_mask[n], out->stack_mode);
         }
@@ -1875,6 +1882,29 @@ int gdo_render(const gd_map_desc *map, const gd_lanes_desc *lanes, const gd_fram
         }
     }
     if (profile) std::fprintf(stderr, "oracle lanes %d: setup %.3fs flats %.3fs walls %.3fs sprites %.3fs\n", lane_end - lane_begin, t_setup, t_flats, t_walls, t_sprites);
+    return GD_OK;
+}
+
+// gdo_render with the lanes dealt out to `threads` host threads (lanes are independent; every thread renders a
+// contiguous share into its own rows of the outputs).  Debug taps are not available here.  The CPU baseline of the
+// benchmark: the same scalar restatement on all the host's cores.
+int gdo_render_parallel(const gd_map_desc *map, const gd_lanes_desc *lanes, const gd_frame_out *out,
+                        int32_t lane_begin, int32_t lane_end, const float *cosine_correction, int32_t threads) {
+    if (threads < 1 || lane_end < lane_begin) { g_error = "bad thread count or lane range"; return GD_E_ARG; }
+    const int total = lane_end - lane_begin;
+    if (threads > total) threads = total > 0 ? total : 1;
+    std::vector<int> codes(threads, GD_OK);
+    std::vector<std::string> errors(threads);
+    std::vector<std::thread> pool;
+    for (int t = 0; t < threads; ++t) {
+        const int first = lane_begin + (int)((long long)total * t / threads), last = lane_begin + (int)((long long)total * (t + 1) / threads);
+        pool.emplace_back([=, &codes, &errors] {
+            codes[t] = gdo_render(map, lanes, out, first, last, cosine_correction, nullptr);
+            if (codes[t] != GD_OK) errors[t] = g_error;
+        });
+    }
+    for (std::thread &worker : pool) worker.join();
+    for (int t = 0; t < threads; ++t) if (codes[t] != GD_OK) { g_error = errors[t]; return codes[t]; }
     return GD_OK;
 }
 

@@ -112,7 +112,7 @@ def lanes_desc(lanes: dict):
 
 
 def render(tables: dict, lanes: dict, cosine_correction, *, lane_range=None, frames=None, reset_mask=None,
-           want_rgb=False, debug_lane=None, stack_mode=0):
+           want_rgb=False, debug_lane=None, stack_mode=0, obs_source_rows=208):
     """Render lanes on the CPU. Returns dict(indexed, obs, frames, rgb, debug...)."""
 
     lib = library()
@@ -126,6 +126,7 @@ def render(tables: dict, lanes: dict, cosine_correction, *, lane_range=None, fra
     out.indexed = indexed.ctypes.data
     out.obs = obs.ctypes.data
     out.stack_mode = int(stack_mode)
+    out.obs_source_rows = int(obs_source_rows)
     result = {"indexed": indexed, "obs": obs}
     if frames is not None:
         frames = np.ascontiguousarray(frames, dtype=np.uint8).copy()
@@ -177,6 +178,30 @@ def render(tables: dict, lanes: dict, cosine_correction, *, lane_range=None, fra
         raise RuntimeError(f"oracle render failed ({code}): {lib.gdo_last_error().decode()}")
     del keep_map, keep_lanes, mask
     return result
+
+
+def render_parallel(tables: dict, lanes: dict, cosine_correction, threads: int) -> dict:
+    """``render`` (frame and observation only) with the lanes dealt out to ``threads`` host threads."""
+
+    lib = library()
+    lib.gdo_render_parallel.restype = C.c_int
+    map_desc, keep_map = _abi.host_map_desc(tables)
+    lane_desc, keep_lanes = lanes_desc(lanes)
+    count = lane_desc.lane_count
+    indexed = np.zeros((count, 240, 320), dtype=np.uint8)
+    obs = np.zeros((count, 84, 84), dtype=np.uint8)
+    frames = np.zeros((count, 4, 84, 84), dtype=np.uint8)
+    out = _abi.FrameOut()
+    out.indexed, out.obs, out.frames = indexed.ctypes.data, obs.ctypes.data, frames.ctypes.data
+    correction = np.ascontiguousarray(cosine_correction, dtype=np.float32)
+    code = lib.gdo_render_parallel(
+        C.byref(map_desc), C.byref(lane_desc), C.byref(out), C.c_int32(0), C.c_int32(count),
+        correction.ctypes.data_as(C.c_void_p), C.c_int32(threads),
+    )
+    if code != 0:
+        raise RuntimeError(f"oracle render failed ({code}): {lib.gdo_last_error().decode()}")
+    del keep_map, keep_lanes
+    return {"indexed": indexed, "obs": obs, "frames": frames}
 
 
 def observe(indexed, playpal, *, frames=None, reset_mask=None, stack_mode=0):

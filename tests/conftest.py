@@ -46,6 +46,9 @@ def load_fixture(name: str):
         pillars=meta.get("pillars", 0),
     )
     assert map_digest(smap) == meta["map_sha256"], "synthetic map generator drifted from the golden fixtures"
+    if meta.get("variant"):
+        smap = synthmap.with_variant(smap, **meta["variant"])
+        assert map_digest(smap) == meta["variant_sha256"], "map variant generator drifted from the golden fixtures"
     if meta.get("blend_seed"):
         smap = synthmap.with_blend_tables(smap, meta["blend_seed"])
     if meta.get("split_seed"):

@@ -128,6 +128,39 @@ CASES = {
         map_seed=22, grid=(6, 5), sectors=26, linedefs=160, lanes=8, pose_seed=7, pitch=True, flash=True, midtex=0.1,
         blend_seed=19, actors=31,
     ),
+    # Inputs beyond the generator's defaults (heights in multiples of 8, 64x128 wall textures, eyes 41 above the floor):
+    # heights uniform over whole map units with ceilings 64..256 above their floors, so that neighbours may miss each
+    # other vertically altogether and every sector is a plane level of its own;
+    "uniform_heights": dict(
+        map_seed=1001, grid=(9, 6), sectors=48, linedefs=320, lanes=10, pose_seed=4, pitch=True, flash=True, sprites=24,
+        midtex=0.15, variant=dict(seed=5, heights="uniform"), eye="any",
+    ),
+    # the same on a map with more plane levels than any table of the renderer holds (96 sectors)
+    "uniform_heights_96": dict(
+        map_seed=1002, grid=(12, 9), sectors=96, linedefs=800, lanes=6, pose_seed=3, sprites=16, midtex=0.1,
+        variant=dict(seed=6, heights="uniform"), eye="any",
+    ),
+    # closed doors (ceiling at the floor) and crawl spaces 8..24 units high among ordinary rooms
+    "doors": dict(
+        map_seed=22, grid=(6, 5), sectors=26, linedefs=160, lanes=12, pose_seed=8, pitch=True, flash=True, sprites=24,
+        midtex=0.2, variant=dict(seed=7, heights="doors"),
+    ),
+    "doors_brick": dict(
+        map_seed=3001, grid=(6, 5), sectors=26, linedefs=260, lanes=10, pose_seed=9, layout="brick", islands=10, midtex=0.1,
+        variant=dict(seed=8, heights="doors"), margin=0.05, eye="any",
+    ),
+    # wall textures of every power-of-two size from 8 to 256 either way, flats 64 or 128 rows
+    "mixed_textures": dict(
+        map_seed=22, grid=(6, 5), sectors=26, linedefs=160, lanes=10, pose_seed=10, pitch=True, midtex=0.2,
+        variant=dict(seed=9, textures="mixed"), eye="any",
+    ),
+    # and sizes that are no powers of two, as WAD textures have (24, 72, 96, 100, 136, 160, 200)
+    "npot_textures": dict(
+        map_seed=22, grid=(6, 5), sectors=26, linedefs=160, lanes=10, pose_seed=11, pitch=True, flash=True, midtex=0.25,
+        sprites=8, variant=dict(seed=10, textures="npot"),
+    ),
+    # config1's cameras again after every sector light changed: what gd_renderer_set_sector_lights must produce
+    "config1_relit": dict(map_seed=1001, grid=(9, 6), sectors=48, linedefs=320, lanes=16, pose_seed=1, variant=dict(seed=11, lights=True)),
     "config2_subset": dict(map_seed=1002, grid=(12, 9), sectors=96, linedefs=800, lanes=4, pose_seed=1, sprites=32),
     "config3_subset": dict(
         map_seed=1003, grid=(15, 15), sectors=200, linedefs=2000, lanes=2, pose_seed=1, sprites=64, flash=True
@@ -143,6 +176,9 @@ def build_case(name: str, cfg: dict, do_time: bool) -> dict:
         cfg["map_seed"], grid=cfg["grid"], sectors=cfg["sectors"], linedefs=cfg["linedefs"], midtex=cfg.get("midtex", 0.0),
         layout=cfg.get("layout", "grid"), islands=cfg.get("islands", 0), pillars=cfg.get("pillars", 0),
     )
+    base_digest = map_digest(smap)
+    if cfg.get("variant"):
+        smap = synthmap.with_variant(smap, **cfg["variant"])
     if cfg.get("split_seed"):
         smap = synthmap.split_linedefs(smap, cfg["split_seed"])
     if cfg.get("blend_seed"):
@@ -158,7 +194,8 @@ def build_case(name: str, cfg: dict, do_time: bool) -> dict:
     picks = cfg.get("picks") or [(cfg["pose_seed"], lane) for lane in range(lanes)]
     assert len(picks) == lanes
     poses = synthmap.generate_picked_poses(
-        smap, picks, pitch=cfg.get("pitch", False), flash=cfg.get("flash", False), margin=cfg.get("margin", 0.15)
+        smap, picks, pitch=cfg.get("pitch", False), flash=cfg.get("flash", False), margin=cfg.get("margin", 0.15),
+        eye=cfg.get("eye", "standing"),
     )
     refdrive.set_poses(engine, poses)
     offsets = hostmath.native_ray_offsets("cpu")
@@ -221,6 +258,12 @@ def build_case(name: str, cfg: dict, do_time: bool) -> dict:
         frame_id, flash_id, _light = engine._native_weapon_frame_selection()
         data["ref_weapon_frame_id"] = frame_id.numpy().astype(np.int64)
         data["ref_weapon_flash_id"] = flash_id.numpy().astype(np.int64)
+        # the observation of an environment made with obs_crop=None: the status bar is pooled, not masked
+        # (env.py:441, engine.py:15440)
+        engine.mask_hud = False
+        with torch.no_grad():
+            data["obs_with_hud"] = engine.render_reference_frame().numpy()
+        engine.mask_hud = True
         data["ref_face_patch"] = np.asarray(
             [engine._native_mugshot_patch_index(lane, int(engine.health[lane].clamp(0, 999).item())) for lane in range(lanes)],
             dtype=np.int64,
@@ -311,7 +354,9 @@ def build_case(name: str, cfg: dict, do_time: bool) -> dict:
             samples.append(lanes / (time.time() - started))
         timing = float(np.median(samples))
     meta = dict(cfg)
-    meta["map_sha256"] = map_digest(smap)
+    meta["map_sha256"] = base_digest
+    if cfg.get("variant"):
+        meta["variant_sha256"] = map_digest(smap)
     if cfg.get("split_seed"):
         meta["fragment_sha256"] = fragment_digest(smap)
     data["meta"] = np.asarray(repr(meta))

@@ -85,3 +85,66 @@ def test_observation_is_a_function_of_the_frame(full_size):
     # status bar rows hold index 0 and the view rows are not blank
     assert int(full_size["indexed"][:, 208:].max()) == 0
     assert int((full_size["indexed"][:, :208].amax(dim=(1, 2)) > 0).sum()) == LANES
+
+
+# The other shapes of the benchmark list at their full lane counts: 256 lanes on the 800-linedef map with 32 sprites,
+# 1024 lanes on the 2000-linedef map with 64 sprites and per-lane light offsets, and on the 4000-linedef map 16384 lanes
+# with the observation stack as the only output (four chunks of 4096) and 512 lanes with an RGB24 frame.
+SHAPES = {
+    "config2_256": dict(config="config2", lanes=256, outputs=("indexed", "frames"), probes=(0, 101, 255)),
+    "config3_1024": dict(config="config3", lanes=1024, outputs=("indexed", "frames"), probes=(0, 517, 1023)),
+    "config5_obs_only_16384": dict(config="config4", lanes=16384, outputs=("frames",), probes=(0, 4095, 4096, 9999, 16383)),
+    "config5_rgb_512": dict(config="config4", lanes=512, outputs=("indexed", "rgb"), probes=(0, 300, 511)),
+}
+
+
+@pytest.mark.parametrize("shape", list(SHAPES))
+def test_other_benchmark_shapes_at_full_lane_count(oracle, shape):
+    from gradoom_amd import hostmath, mapbuild, synthmap
+    from gradoom_amd.renderer import HipRenderer, LaneState
+    from gradoom_amd.selfcheck import make_lane_arrays
+
+    spec = SHAPES[shape]
+    count = spec["lanes"]
+    print(f"shape {shape}: building the map and {count} poses", flush=True)
+    smap = synthmap.generate_config_map(spec["config"])
+    tables = mapbuild.build_map_tables(smap)
+    cosine = hostmath.cosine_correction("cpu").numpy()
+    poses = synthmap.generate_poses_batch(smap, count, 77, flash=True)
+    sprites = synthmap.generate_sprites_batch(smap, count, synthmap.CONFIGS[spec["config"]]["sprites"], 77)
+    arrays = make_lane_arrays(smap, poses, sprites)
+    renderer = HipRenderer(smap, count, "cuda:0", cosine_correction=cosine, tables=tables)
+    lanes = LaneState.from_numpy(arrays, "cuda:0")
+    rng = np.random.default_rng(23)
+    start = rng.integers(0, 256, (count, 4, 84, 84), dtype=np.uint8)
+
+    def render(state, n, first):
+        out = {}
+        if "indexed" in spec["outputs"]:
+            out["indexed"] = torch.zeros((n, 240, 320), dtype=torch.uint8, device="cuda:0")
+        if "frames" in spec["outputs"]:
+            out["frames"] = torch.as_tensor(first).to("cuda:0")
+        if "rgb" in spec["outputs"]:
+            out["rgb"] = torch.zeros((n, 240, 320, 3), dtype=torch.uint8, device="cuda:0")
+        renderer.render(state, **out)
+        torch.cuda.synchronize()
+        assert renderer.status() == 0
+        return out
+
+    print(f"shape {shape}: rendering", flush=True)
+    full = render(lanes, count, start)
+    # probe lanes equal the CPU oracle bit for bit: frame, RGB24 expansion and rolled stack
+    probes = list(spec["probes"])
+    expected = oracle.render(tables, _subset(arrays, probes), cosine, frames=start[probes], want_rgb=True)
+    for name, ours in full.items():
+        assert np.array_equal(ours[probes].cpu().numpy(), expected[name]), name
+    # lanes are independent of their batch: a shuffled sample rendered alone gives the same bytes
+    picks = rng.permutation(count)[:64]
+    alone = render(LaneState.from_numpy(_subset(arrays, picks), "cuda:0"), len(picks), start[picks])
+    index = torch.as_tensor(picks, device="cuda:0")
+    for name, ours in alone.items():
+        assert torch.equal(ours, full[name][index]), name
+    if "frames" in full:   # the stack rolled: three older frames kept, no lane left blank
+        assert torch.equal(full["frames"][:, :3].cpu(), torch.as_tensor(start[:, 1:]))
+        assert int((full["frames"][:, 3].amax(dim=(1, 2)) > 0).sum()) == count
+    renderer.close()

@@ -104,23 +104,116 @@ def test_chunked_batches_render_every_lane_like_the_golden():
         renderer.close()
 
 
-def test_final_frames_receive_the_stack_the_call_leaves(oracle):
-    # the fused final-observation clone: step mode, reset mode with untouched lanes, and masked lanes
+def test_final_frames_and_stack_modes_match_the_oracle(oracle):
+    # the three ways a call leaves the stack (step; step with some lanes reset; reset of the masked lanes only), each
+    # against the oracle's stack, with the fused final-observation clone (env.py:915-917) equal to it
     meta, data, tables, renderer, lanes = _renderer("config1")
     count = meta["lanes"]
     rng = np.random.default_rng(5)
     start = rng.integers(0, 256, (count, 4, 84, 84), dtype=np.uint8)
-    mask = torch.as_tensor((rng.random(count) < 0.5).astype(np.uint8)).to("cuda:0")
-    for kwargs in (dict(), dict(reset_mask=mask), dict(reset_mask=mask, stack_only_masked=True)):
+    mask_np = (rng.random(count) < 0.5).astype(np.uint8)
+    assert 0 < mask_np.sum() < count
+    mask = torch.as_tensor(mask_np).to("cuda:0")
+    for mode, kwargs, oracle_kwargs in (
+        ("step", dict(), dict(stack_mode=0)),
+        ("step+reset", dict(reset_mask=mask), dict(stack_mode=0, reset_mask=mask_np)),
+        ("reset", dict(reset_mask=mask, stack_only_masked=True), dict(stack_mode=1, reset_mask=mask_np)),
+    ):
+        print(f"stack mode {mode}", flush=True)
+        expected = oracle.render(tables, lane_inputs(data), data["cosine_correction"], frames=start, **oracle_kwargs)
         frames = torch.as_tensor(start).to("cuda:0")
-        plain = torch.as_tensor(start).to("cuda:0")
         final = torch.full((count, 4, 84, 84), 7, dtype=torch.uint8, device="cuda:0")
-        renderer.render(lanes, frames=frames, final_frames=final, **kwargs)
-        renderer.render(lanes, frames=plain, **kwargs)
+        obs = torch.zeros((count, 84, 84), dtype=torch.uint8, device="cuda:0")
+        renderer.render(lanes, frames=frames, final_frames=final, obs=obs, **kwargs)
         torch.cuda.synchronize()
-        assert torch.equal(frames, plain)          # the extra output changes nothing else
-        assert torch.equal(final, frames)          # and equals a clone taken after the call
+        ours = frames.cpu().numpy()
+        assert np.array_equal(ours, expected["frames"]), mode
+        assert np.array_equal(final.cpu().numpy(), expected["frames"]), mode
+        assert np.array_equal(obs.cpu().numpy(), expected["obs"]), mode
         assert final.data_ptr() != frames.data_ptr()
+        if mode == "step":
+            assert np.array_equal(ours[:, :3], start[:, 1:]) and np.array_equal(ours[:, 3], expected["obs"])
+        if mode == "reset":   # lanes outside the mask keep the stack they had
+            keep = mask_np == 0
+            assert np.array_equal(ours[keep], start[keep])
+            assert np.array_equal(ours[~keep], np.repeat(expected["obs"][~keep, None], 4, axis=1))
+    renderer.close()
+
+
+def test_sector_lights_replaced_between_frames_match_the_reference():
+    # config1 under its own lights, then under the lights of config1_relit (same map, same cameras): the second frame
+    # must be the reference's frame of the relit map, and going back must give the first again
+    meta, data, tables, renderer, lanes = _renderer("config1")
+    _meta2, relit, _smap2, relit_tables = load_fixture("config1_relit")
+    assert np.array_equal(relit["x"], data["x"]) and not np.array_equal(relit_tables["sector_lights"], tables["sector_lights"])
+    count = meta["lanes"]
+    indexed = torch.zeros((count, 240, 320), dtype=torch.uint8, device="cuda:0")
+    obs = torch.zeros((count, 84, 84), dtype=torch.uint8, device="cuda:0")
+    for lights, golden in ((None, data), (relit_tables["sector_lights"], relit), (tables["sector_lights"], data)):
+        if lights is not None:
+            renderer.set_sector_lights(torch.as_tensor(np.asarray(lights, dtype=np.float32)).to("cuda:0"))
+        renderer.render(lanes, indexed=indexed, obs=obs)
+        torch.cuda.synchronize()
+        assert np.array_equal(indexed.cpu().numpy(), golden["indexed"])
+        delta = np.abs(obs.cpu().numpy().astype(np.int32) - golden["obs"].astype(np.int32))
+        assert delta.max() <= 1 and delta.mean() < 0.01
+    assert (relit["indexed"] != data["indexed"]).mean() > 0.3   # the two light vectors really give different pictures
+    renderer.close()
+
+
+def test_status_bar_rows_pooled_into_the_observation(oracle):
+    # obs_source_rows=240 (an environment made with obs_crop=None, engine.py:15440): within 1 of the reference's float
+    # pooling, equal to the oracle's integer pooling, and equal to gd_observe over all 240 rows of the frame
+    meta, data, tables, renderer, lanes = _renderer("overlays")
+    count = meta["lanes"]
+    indexed = torch.zeros((count, 240, 320), dtype=torch.uint8, device="cuda:0")
+    obs = torch.zeros((count, 84, 84), dtype=torch.uint8, device="cuda:0")
+    renderer.render(lanes, indexed=indexed, obs=obs, obs_source_rows=240)
+    again = torch.zeros_like(obs)
+    renderer.observe(indexed, obs=again)
+    torch.cuda.synchronize()
+    delta = np.abs(obs.cpu().numpy().astype(np.int32) - data["obs_with_hud"].astype(np.int32))
+    assert delta.max() <= 1 and delta.mean() < 0.01
+    assert torch.equal(obs, again)
+    oracle.set_overlays(fixture_overlays(meta))
+    try:
+        expected = oracle.render(tables, lane_inputs(data), data["cosine_correction"], obs_source_rows=240)
+    finally:
+        oracle.set_overlays(None)
+    assert np.array_equal(obs.cpu().numpy(), expected["obs"])
+    renderer.close()
+
+
+def test_render_replays_from_a_captured_graph():
+    # the reference replays its background pass as a CUDA graph (engine.py:15308-15336, tests/test_rendering.py:142-171):
+    # gd_render neither allocates nor synchronises, so a caller can capture it; replays after the lane tensors were
+    # rewritten in place must give the frames of the new poses, each checked against the reference's golden frames
+    import dataclasses
+
+    meta, data, tables, renderer, lanes = _renderer("small_midtex_sprites")
+    count = meta["lanes"]
+    base = lane_inputs(data)
+    indexed = torch.zeros((count, 240, 320), dtype=torch.uint8, device="cuda:0")
+    frames = torch.zeros((count, 4, 84, 84), dtype=torch.uint8, device="cuda:0")
+    eager = torch.zeros_like(indexed)
+    eager_frames = torch.zeros_like(frames)
+    renderer.render(lanes, indexed=eager, frames=eager_frames)   # warm-up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        renderer.render(lanes, indexed=indexed, frames=frames)
+    fields = [f.name for f in dataclasses.fields(lanes) if isinstance(getattr(lanes, f.name), torch.Tensor)]
+    for replay, shift in enumerate((0, 3, 5, 0)):
+        picks = (np.arange(count) + shift) % count
+        for name in fields:   # new poses, written into the very tensors the graph reads
+            getattr(lanes, name).copy_(torch.as_tensor(np.ascontiguousarray(base[name][picks])).to("cuda:0"))
+        eager_frames.copy_(frames)
+        graph.replay()
+        renderer.render(lanes, indexed=eager, frames=eager_frames)   # the program's own eager work between replays
+        torch.cuda.synchronize()
+        assert np.array_equal(indexed.cpu().numpy(), data["indexed"][picks]), f"replay {replay}"
+        assert torch.equal(indexed, eager) and torch.equal(frames, eager_frames), f"replay {replay}"
+    assert renderer.status() == 0
     renderer.close()
 
 

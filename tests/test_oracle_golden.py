@@ -103,3 +103,19 @@ def test_scene_depth_under_the_decals_matches_the_reference(oracle):
         ours, ref = np.asarray(taps["scene_depth"]), data["ref_scene_depth"][lane]
         assert np.array_equal(ours, ref)
         assert np.isfinite(ref).mean() > 0.9
+
+
+def test_observation_with_the_status_bar_pooled_matches_the_reference(oracle):
+    """An environment made with obs_crop=None pools all 240 rows (env.py:441, engine.py:15440)."""
+
+    meta, data, _smap, tables = load_fixture("overlays")
+    oracle.set_overlays(fixture_overlays(meta))
+    try:
+        result = oracle.render(tables, lane_inputs(data), data["cosine_correction"], obs_source_rows=240)
+        masked = oracle.render(tables, lane_inputs(data), data["cosine_correction"])
+    finally:
+        oracle.set_overlays(None)
+    delta = np.abs(result["obs"].astype(np.int32) - data["obs_with_hud"].astype(np.int32))
+    assert delta.max() <= 1 and delta.mean() < 0.01   # tolerance: tests/test_rendering.py:138-139
+    assert (data["obs_with_hud"][:, 74:] != data["obs"][:, 74:]).mean() > 0.5   # the bar really shows in the last rows
+    assert np.array_equal(result["obs"][:, :72], masked["obs"][:, :72])   # rows that pool view rows only are unchanged
