@@ -18,6 +18,7 @@ SYMBOLS = (
     "gd_renderer_create",
     "gd_renderer_destroy",
     "gd_renderer_status",
+    "gd_renderer_scribble",
     "gd_renderer_set_sector_lights",
     "gd_renderer_set_overlays",
     "gd_render",
@@ -57,6 +58,8 @@ def library() -> C.CDLL:
     lib.gd_renderer_destroy.argtypes = [C.c_void_p]
     lib.gd_renderer_status.restype = C.c_int
     lib.gd_renderer_status.argtypes = [C.c_void_p, C.POINTER(C.c_int32)]
+    lib.gd_renderer_scribble.restype = C.c_int
+    lib.gd_renderer_scribble.argtypes = [C.c_void_p, C.c_int32, C.c_void_p]
     lib.gd_renderer_set_overlays.restype = C.c_int
     lib.gd_renderer_set_overlays.argtypes = [C.c_void_p, C.POINTER(_abi.OverlayDesc)]
     lib.gd_renderer_set_sector_lights.restype = C.c_int

@@ -10,7 +10,7 @@
 //   strip_key/order 1 thread / 64-col strip   longest strip first (counting sort on the blocking distance)
 //   wall_columns    1 wave / strip            portal traversal, tiers, planes, masked mid-textures
 //   plane_shade     1 thread / 12 pixels      flat texel + light for every pixel a plane of the wall pass shows,
-//                                             the wall tiers' palette indices, the list of gap pixels
+//                                             the wall tiers' palette indices
 //   flat_list       128 threads / lane        per-pixel plane rays (fine point raster) for the listed gap pixels
 //   flat_span_select, flat_tail, flat_span_finish
 //                                             visplane repair of the rows where a gap pixel stayed unresolved
@@ -95,6 +95,12 @@ struct WallRec {   // one linedef seen from one lane
     int flags;
 };
 
+struct RecSpan {   // what a ray test of one linedef needs (eval_segment), kept for every linedef of the map; the full record
+                   // above exists only for the linedefs the camera can see at all
+    short pl, pr;
+    int flags;
+};
+
 struct __align__(16) Cand {      // one linedef with a finite ray distance at one column, with the static
                    // linedef facts every scan needs packed in so that scans do no gathers
     unsigned short wall, flags;
@@ -141,7 +147,8 @@ struct Overlays {   // device copy of gd_overlay_desc; count 0 = layer not loade
 
 struct Scratch {    // per-chunk working memory, sized at create
     LaneCtx *ctx;          // [L]
-    WallRec *rec;          // [L,W]
+    WallRec *rec;          // [L,W] written for the linedefs wall_setup_kernel does not cull; never read for the others
+    RecSpan *span;         // [L,W] every linedef
     WallRec *frag_rec;     // [L,split_count,fragment_slots] FWallCoords of the BSP fragments of split linedefs
     float *scene_depth;    // [L,208,320] depth of the surface each pixel shows (engine.py:11553, 12700, 13411, 13740),
                            // kept only for frames that draw wall decals, else null
@@ -150,7 +157,7 @@ struct Scratch {    // per-chunk working memory, sized at create
     unsigned short *flat_sector;// [L,208,320]
     unsigned char *flat_flags;  // [L,208,320] bit0 unresolved
     int *flat_list;        // [L,FLAT_LIST_MAX] view pixels no wall tier, plane or masked texture covers: they show the
-                           // flat pass's picture.  Found by plane_shade_kernel.
+                           // flat pass's picture.  Listed by wall_columns_kernel, column by column.
     int *flat_list_count;  // [L] how many there are (more than FLAT_LIST_MAX: the lane is handled pixel by pixel)
     int *flat_tail;        // [L,2,320] per screen half and column: the sector of the first resolved pixel below the
                            // half's noted rows, -1 if the column was not looking for one or found none
@@ -315,7 +322,7 @@ struct MapView {
 };
 
 #define LDS_SECTORS 512
-#define LDS_TEXTURES 256
+#define LDS_TEXTURES 224   // textures whose size bits are staged in LDS (a multiple of 32); later ones read the global arrays
 #define GRID_ALWAYS_INSIDE (1 << 30)   // grid item flag: the whole cell lies inside the sector
 
 // Even-odd parity of one sector's edge sub-list around a point (engine.py:9598-9612, 10994-11015).
@@ -535,9 +542,9 @@ __device__ __forceinline__ Eval eval_segment(const float4 wl, int rec_flags, int
     return out;
 }
 
-__device__ __forceinline__ Eval eval_wall(const gd_map_desc *m, const LaneCtx &c, const WallRec *recs, int x, int w, float rx, float ry) {
+__device__ __forceinline__ Eval eval_wall(const gd_map_desc *m, const LaneCtx &c, const RecSpan *spans, int x, int w, float rx, float ry) {
     const float4 wl = *reinterpret_cast<const float4 *>(m->walls + 4 * w);
-    const WallRec &r = recs[w];
+    const RecSpan r = spans[w];
     return eval_segment(wl, r.flags, r.pl, r.pr, m->wall_sectors[2 * w + 1] < 0, c, x, rx, ry);
 }
 
@@ -597,22 +604,53 @@ __global__ void fragment_setup_kernel(DeviceMap dm, int lane_count, Scratch sc) 
 // wildly different trip counts per linedef (none for most, up to 320 for a few), so they are
 // run by the whole wavefront together: the linedefs with a non-empty column range take turns,
 // their parameters are broadcast from the owning lane, and the 64 lanes each take one column.
-__global__ void __launch_bounds__(128) wall_setup_kernel(DeviceMap dm, int lane_count, Scratch sc) {
+//
+// Three quarters of a map's linedefs lie wholly behind the camera or wholly to one side of its view: no
+// column ray can hit such a linedef and FWallCoords rejects it, so nothing of it is ever looked at beyond
+// the ray-test facts of RecSpan (no owned span).  A block first sorts its SETUP_WALLS linedefs into those and the
+// rest, and only the rest, packed into as few wavefronts as they fill, get the arithmetic below.
+#define SETUP_WALLS 256
+__global__ void __launch_bounds__(SETUP_WALLS) wall_setup_kernel(DeviceMap dm, int lane_count, Scratch sc) {
     const gd_map_desc *m = &dm.d;
+    __shared__ int alive_list[SETUP_WALLS];
+    __shared__ int alive_count;
     const int slot_in_wave = threadIdx.x & 63;
-    const int w_raw = blockIdx.x * blockDim.x + threadIdx.x;
     const int local = blockIdx.y;
     if (local >= lane_count) return;          // uniform over the block
-    {
-        // The traversal starts from a cleared meta plane (no owner, no plane, no clip linedef).  This kernel is
-        // bound by its arithmetic, so the fill rides along here instead of heading wall_columns_kernel.
-        uint4 *plane = reinterpret_cast<uint4 *>(sc.meta + (size_t)local * VH * SW);
-        const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
-        for (int k = w_raw; k < VH * SW / 4; k += gridDim.x * blockDim.x) plane[k] = zero;
-    }
-    const bool live = w_raw < m->wall_count;  // dead lanes still help with the column loops
-    const int w = live ? w_raw : 0;
     const LaneCtx &c = sc.ctx[local];
+    if (threadIdx.x == 0) alive_count = 0;
+    __syncthreads();
+    {
+        const int w = blockIdx.x * SETUP_WALLS + threadIdx.x;
+        if (w < m->wall_count) {
+            const float4 wl = *reinterpret_cast<const float4 *>(m->walls + 4 * w);
+            const float ax = wl.x - c.x, ay = wl.y - c.y, bx = wl.z - c.x, by = wl.w - c.y;
+            // forward and rightward view coordinates of both endpoints; a column ray is forward + col * right, |col| <= 1
+            const float f0 = ax * c.fcos + ay * c.fsin, r0 = ax * c.fsin - ay * c.fcos;
+            const float f1 = bx * c.fcos + by * c.fsin, r1 = bx * c.fsin - by * c.fcos;
+            // wholly in one of the half planes behind the camera, right of the right view edge, left of the left one (a map
+            // unit to spare, far more than float32 and 16.16 coordinates can disagree): no ray reaches it, FWallCoords finds
+            // no span.  Linedef 0 and the first blocking linedef stand in where a scan finds nothing, and are always kept.
+            const bool unseen = (f0 < -1.0f && f1 < -1.0f) || (r0 > f0 + 1.0f && r1 > f1 + 1.0f) || (r0 < -f0 - 1.0f && r1 < -f1 - 1.0f);
+            const bool kept = !unseen || w == 0 || (m->blocking_count > 0 && w == m->blocking_walls[0]);
+            if (kept) {
+                alive_list[atomicAdd(&alive_count, 1)] = w;
+            } else {
+                const float vfx = c.x - wl.x, vfy = c.y - wl.y;
+                const bool ff = ((wl.z - wl.x) * vfy - (wl.w - wl.y) * vfx) < 0;
+                RecSpan span;
+                span.pl = 0; span.pr = 0;
+                // an unseen linedef has an empty span (sr == sl), so a two-sided one counts as at most one column wide
+                span.flags = (ff ? WF_FF : 0) | (m->wall_sectors[2 * w + 1] < 0 ? 0 : WF_SUBPIXEL) | (m->wall_split_slot[w] >= 0 ? WF_SPLIT : 0);
+                sc.span[(size_t)local * m->wall_count + w] = span;
+            }
+        }
+    }
+    __syncthreads();
+    const int alive = alive_count;
+    if ((int)(threadIdx.x & ~63u) >= alive) return;   // whole wavefronts beyond the kept linedefs leave
+    const bool live = (int)threadIdx.x < alive;  // dead lanes of the last wavefront still help with the column loops
+    const int w = live ? alive_list[threadIdx.x] : 0;
     const int *wf = m->walls_fixed + 4 * w;
     WallRec r;
     i64 endpoint_quotient[2];
@@ -752,7 +790,12 @@ __global__ void __launch_bounds__(128) wall_setup_kernel(DeviceMap dm, int lane_
     r.pl = (short)screen_left; r.pr = (short)screen_right;
     r.flags = (hc ? WF_HC : 0) | (ff ? WF_FF : 0) | (((sr - sl <= 1) && !os) ? WF_SUBPIXEL : 0) | (any ? WF_ANYGEO : 0) |
               (m->wall_split_slot[w] >= 0 ? WF_SPLIT : 0);
-    if (live) sc.rec[(size_t)local * m->wall_count + w] = r;
+    if (live) {
+        sc.rec[(size_t)local * m->wall_count + w] = r;
+        RecSpan span;
+        span.pl = r.pl; span.pr = r.pr; span.flags = r.flags;
+        sc.span[(size_t)local * m->wall_count + w] = span;
+    }
     // Enter the linedef in the candidate list of every column where its distance can be
     // finite: its owned span (projected) and, for two-sided lines, the columns its rays hit
     // (engine.py:11446-11451).  List order is irrelevant: scans break ties on the linedef index.
@@ -1199,7 +1242,8 @@ __global__ void __launch_bounds__(SW) __attribute__((amdgpu_waves_per_eu(8, 8)))
 struct Tables {
     const gd_map_desc *m;
     const float4 *sector;          // floor, ceiling, light, bits(floor_tex | ceil_tex << 16)
-    const unsigned short *tex_bits; // floor(log2 width) | floor(log2 height) << 4 | (width is no power of two) << 8
+    const unsigned char *tex_bits; // floor(log2 width) | floor(log2 height) << 4
+    const unsigned int *tex_odd;   // bit t: the width of texture t is no power of two
     int sector_cached, tex_cached;
     __device__ __forceinline__ float floor_h(int s) const { return s < sector_cached ? sector[s].x : m->sector_heights[2 * s]; }
     __device__ __forceinline__ float ceil_h(int s) const { return s < sector_cached ? sector[s].y : m->sector_heights[2 * s + 1]; }
@@ -1207,11 +1251,11 @@ struct Tables {
     __device__ __forceinline__ int floor_tex(int s) const { return s < sector_cached ? (int)(__float_as_uint(sector[s].w) & 0xFFFFu) : m->sector_floor_tex[s]; }
     __device__ __forceinline__ int ceil_tex(int s) const { return s < sector_cached ? (int)(__float_as_uint(sector[s].w) >> 16) : m->sector_ceil_tex[s]; }
     __device__ __forceinline__ int width_bits(int t) const { return t < tex_cached ? (tex_bits[t] & 15) : ilog2(m->tex_w[t]); }
-    __device__ __forceinline__ int height_bits(int t) const { return t < tex_cached ? ((tex_bits[t] >> 4) & 15) : ilog2(m->tex_h[t]); }
+    __device__ __forceinline__ int height_bits(int t) const { return t < tex_cached ? (tex_bits[t] >> 4) : ilog2(m->tex_h[t]); }
     // Texture column of a wall: torch.remainder(u, width) (engine.py:12792-12798).  Widths are powers of two
     // on most maps, where the remainder is a mask; WAD textures of other widths take the division.
     __device__ __forceinline__ i64 wrap_column(int t, i64 u) const {
-        const bool odd = t < tex_cached ? (tex_bits[t] >> 8) != 0 : (m->tex_w[t] & (m->tex_w[t] - 1)) != 0;
+        const bool odd = t < tex_cached ? ((tex_odd[t >> 5] >> (t & 31)) & 1u) != 0 : (m->tex_w[t] & (m->tex_w[t] - 1)) != 0;
         if (!odd) return u & (i64)((1 << width_bits(t)) - 1);
         const i64 width = m->tex_w[t];
         const i64 r = u - tdiv(u, width) * width;
@@ -1220,7 +1264,8 @@ struct Tables {
 };
 
 // Cooperative fill of the LDS tables by the whole block (call before a __syncthreads()).
-__device__ __forceinline__ void stage_tables(const gd_map_desc *m, float4 *sector_lds, unsigned short *tex_lds, Tables &tb) {
+struct TexLds { unsigned char bits[LDS_TEXTURES]; unsigned int odd[LDS_TEXTURES / 32]; };   // 252 bytes: plane_shade_kernel's LDS budget is exact
+__device__ __forceinline__ void stage_tables(const gd_map_desc *m, float4 *sector_lds, TexLds *tex_lds, Tables &tb) {
     int sectors = m->sector_count < LDS_SECTORS ? m->sector_count : LDS_SECTORS;
     int textures = m->texture_count < LDS_TEXTURES ? m->texture_count : LDS_TEXTURES;
     for (int s = threadIdx.x; s < sectors; s += blockDim.x) {
@@ -1229,11 +1274,13 @@ __device__ __forceinline__ void stage_tables(const gd_map_desc *m, float4 *secto
         v.w = __uint_as_float(((unsigned)m->sector_floor_tex[s] & 0xFFFFu) | ((unsigned)m->sector_ceil_tex[s] << 16));
         sector_lds[s] = v;
     }
-    for (int t = threadIdx.x; t < textures; t += blockDim.x) {
-        const int w = m->tex_w[t];
-        tex_lds[t] = (unsigned short)(ilog2(w) | (ilog2(m->tex_h[t]) << 4) | ((w & (w - 1)) ? 0x100 : 0));
+    for (int t = threadIdx.x; t < textures; t += blockDim.x) tex_lds->bits[t] = (unsigned char)(ilog2(m->tex_w[t]) | (ilog2(m->tex_h[t]) << 4));
+    for (int k = threadIdx.x; k < LDS_TEXTURES / 32; k += blockDim.x) {
+        unsigned int odd = 0;
+        for (int t = 32 * k; t < 32 * k + 32 && t < textures; ++t) odd |= (m->tex_w[t] & (m->tex_w[t] - 1)) ? 1u << (t & 31) : 0u;
+        tex_lds->odd[k] = odd;
     }
-    tb.m = m; tb.sector = sector_lds; tb.tex_bits = tex_lds; tb.sector_cached = sectors; tb.tex_cached = textures;
+    tb.m = m; tb.sector = sector_lds; tb.tex_bits = tex_lds->bits; tb.tex_odd = tex_lds->odd; tb.sector_cached = sectors; tb.tex_cached = textures;
 }
 
 // engine.py:10879-10954
@@ -1471,6 +1518,7 @@ struct ColumnCtx {
     MapView mv;
     const LaneCtx *c;
     const WallRec *recs;
+    const RecSpan *spans; // this lane's ray-test facts of every linedef
     const WallRec *frags; // this lane's [split_count, fragment_slots] fragment records
     const Cand *list;     // this lane's candidate block, entry k of column x at [k*320 + x]
     int count;
@@ -1498,7 +1546,7 @@ struct ColumnCtx {
 #pragma unroll
         for (int j = 0; j < CAND_BATCH; ++j) out[j] = cand(at[j] < 0 ? 0 : at[j]);
     }
-    __device__ Eval eval(int w) const { return eval_wall(m, *c, recs, x, w, rx, ry); }
+    __device__ Eval eval(int w) const { return eval_wall(m, *c, spans, x, w, rx, ry); }
 };
 
 // The projection fragment of a linedef at one column (engine.py:11511-11529, 12324-12376): the first
@@ -1645,7 +1693,7 @@ __device__ __forceinline__ i64 wall_shade(float light, i64 visibility) {
 __device__ __forceinline__ void endpoint_owner(const ColumnCtx &cc, int w, const Eval &cw, int *owner_index, float *owner_distance) {
     const gd_map_desc *m = cc.m;
     const int K = m->neighbor_slots;
-    const bool subpixel = cc.recs[w].flags & WF_SUBPIXEL;
+    const bool subpixel = cc.spans[w].flags & WF_SUBPIXEL;
     float tol_w = tolerance_of(cw.dist);
     // the owner only matters for a linedef that does not own this column itself (engine.py:11716)
     if (cw.flags & CF_PROJ) { *owner_index = w; *owner_distance = cw.dist; return; }
@@ -2047,6 +2095,22 @@ __device__ __forceinline__ bool silhouette_folds(const PassColumn &r) {
     return !(lower_on && upper_on && r.clipped_lower_top < r.clipped_upper_bottom);
 }
 
+// The meta plane is never cleared between frames.  Instead the traversal keeps every row of its column that lies
+// outside the open window [ceiling_clip, floor_clip) written (with a claim, a tier, or an explicit zero), reads no row
+// inside the window until a one-sided drawseg has painted all of it, and zeroes what is left of the window when the
+// column ends.  Rows that received such a zero are the only ones that can end up without an owner: the column keeps
+// their range and lists the ownerless ones as gap pixels for the flat pass.
+struct GapRange {
+    int lo, hi;   // rows [lo, hi) hold every zero this column wrote
+};
+__device__ __forceinline__ void zero_rows(PixelBuffers &pb, GapRange &gaps, int x, int first, int last) {
+    first = first < 0 ? 0 : first; last = last > VH ? VH : last;
+    if (first >= last) return;
+    for (int y = first; y < last; ++y) pb.meta[(size_t)y * SW + x] = 0u;
+    gaps.lo = first < gaps.lo ? first : gaps.lo;
+    gaps.hi = last > gaps.hi ? last : gaps.hi;
+}
+
 // engine.py:12637-12884
 // `window_dirty` says whether some pixel inside the open window [ceiling_clip, floor_clip) may
 // already be filled, plane-owned or carry a sprite-clip depth.  A two-sided drawseg only writes
@@ -2056,7 +2120,7 @@ __device__ __forceinline__ bool silhouette_folds(const PassColumn &r) {
 template <bool DEPTH>
 __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnState &c, const PassColumn &r, PixelBuffers &pb,
                            const bool group_valid[3], const float group_bottom[3], i64 first_group_visibility,
-                           const unsigned char *colormap, bool &window_dirty) {
+                           const unsigned char *colormap, bool &window_dirty, GapRange &gaps) {
     if (!(r.bits & PB_RASTER)) return;
     const gd_map_desc *m = cc.m;
     const LaneCtx &L = *cc.c;
@@ -2123,6 +2187,11 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
                 }
             }
         }
+        // Rows that leave the window without being written: those the upper tier covers but that belong to a lower
+        // tier without a texture (the lower tier has the say there), and a one-sided drawseg's own rows when it has none.
+        if (lower_on && upper_on && r.side_tex[1] < 0 && r.side_tex[2] >= 0)
+            zero_rows(pb, gaps, x, max((int)r.clipped_top, (int)r.clipped_lower_top), min((int)r.clipped_upper_bottom, (int)r.clipped_bottom));
+        if (one_sided && r.side_tex[0] < 0) zero_rows(pb, gaps, x, max((int)r.clipped_top, y0), min((int)r.clipped_bottom, y1));
         int t0 = VH, t1 = 0;
         if (one_sided) { t0 = (int)r.clipped_top; t1 = (int)r.clipped_bottom; }
         if (lower_on) { t0 = min(t0, (int)r.clipped_lower_top); t1 = max(t1, (int)r.clipped_bottom); }
@@ -2591,14 +2660,14 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
     __shared__ LaneCtx lane_ctxs[WALL_STRIPS_PER_GROUP];
     __shared__ unsigned char colormap_lds[32 * 256];   // shade rows 0..31 are the only ones indexed
     __shared__ float4 sector_lds[LDS_SECTORS];
-    __shared__ unsigned short tex_lds[LDS_TEXTURES];
+    __shared__ TexLds tex_lds;
     const int wave_in_group = threadIdx.x >> 6;
     const int strip_slot = blockIdx.x * WALL_STRIPS_PER_GROUP + wave_in_group;
     const bool live = strip_slot < lane_count * (SW / 64);
     const int strip_index = live ? sc.strip_order[strip_slot] : 0;
     const int local = strip_index / (SW / 64);
     Tables tb;
-    stage_tables(m, sector_lds, tex_lds, tb);
+    stage_tables(m, sector_lds, &tex_lds, tb);
     if ((threadIdx.x & 63) == 0 && live) lane_ctxs[wave_in_group] = sc.ctx[local];
     for (int k = threadIdx.x; k < 32 * 256 / 4; k += blockDim.x) reinterpret_cast<unsigned int *>(colormap_lds)[k] = reinterpret_cast<const unsigned int *>(m->colormap)[k];
     __syncthreads();
@@ -2606,9 +2675,11 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
     const LaneCtx &lane_ctx = lane_ctxs[wave_in_group];
     const int x = (strip_index - local * (SW / 64)) * 64 + (threadIdx.x & 63);
     bool window_dirty = false;
+    GapRange gaps; gaps.lo = VH; gaps.hi = 0;
     ColumnCtx cc;
     cc.tb = &tb; cc.m = m; cc.mv.m = m; cc.c = &lane_ctx;
     cc.recs = sc.rec + (size_t)local * m->wall_count;
+    cc.spans = sc.span + (size_t)local * m->wall_count;
     cc.frags = sc.frag_rec + (size_t)local * m->split_count * m->fragment_slots;
     cc.list = sc.cand + (size_t)local * CAND_MAX * SW;
     cc.count = sc.cand_count[(size_t)local * SW + x];
@@ -2620,7 +2691,7 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
     pb.meta = sc.meta + (size_t)local * VH * SW;
     pb.clip_depth = sc.clip_depth + (size_t)local * VH * SW;
     pb.scene_depth = DEPTH ? sc.scene_depth + (size_t)local * VH * SW : nullptr;
-    // the meta plane arrives cleared (wall_setup_kernel): no owner, no plane, no clip linedef (clip depth: infinite)
+    // the meta plane arrives with whatever the last frame left: see GapRange for how every row gets written
     ColumnState st;
     st.current_sector = lane_ctx.sector;
     st.ceiling_clip = 0.0f; st.floor_clip = (float)VH;
@@ -2670,7 +2741,7 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
         for (int t = 0; t < 3; ++t) group_valid[t] = same_group && all_tier[t] && (common_top[t] < common_bottom[t]);
         if (!done) {
             PROF_T(t2);
-            pass_paint<DEPTH>(cc, st, pc, pb, group_valid, common_bottom, first_group_visibility, colormap_lds, window_dirty);
+            pass_paint<DEPTH>(cc, st, pc, pb, group_valid, common_bottom, first_group_visibility, colormap_lds, window_dirty, gaps);
             PROF_T(t3);
             PROF_ADD(1, t2, t3);
             bool changed = pass_advance<SPLIT>(cc, st, pc, pb, sb, !window_dirty);
@@ -2686,7 +2757,17 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
     }
     PROF_T(t5);
     PROF_T(t6);
+    // what is left of a window no one-sided drawseg closed shows the flat pass's picture
+    if (!window_dirty) zero_rows(pb, gaps, x, st.ceiling_clip <= 0.0f ? 0 : (int)st.ceiling_clip, st.floor_clip >= (float)VH ? VH : (int)st.floor_clip);
     masked_midtexture<DEPTH, SPLIT>(cc, st, pb, colormap_lds);
+    // The view pixels no wall tier, plane or masked texture covers: the flat pass selects them (flat_list_kernel) and
+    // flat_shade_kernel paints them.  More than the list holds: the lane is handled pixel by pixel.
+    for (int y = gaps.lo; y < gaps.hi; ++y) {
+        const unsigned int word = pb.meta[(size_t)y * SW + x];
+        if ((word & (META_FILLED | META_MASKED)) || ((word >> META_SECTOR_SHIFT) & META_SECTOR_MASK) != 0) continue;
+        const int slot = atomicAdd(&sc.flat_list_count[local], 1);
+        if (slot < FLAT_LIST_MAX) sc.flat_list[(size_t)local * FLAT_LIST_MAX + slot] = y * SW + x;
+    }
 #ifdef GD_PROFILE
     long long t7 = wall_clock64();
     int prof_cands = cc.count;
@@ -2717,14 +2798,14 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))
     const gd_map_desc *m = &dm.d;
     __shared__ float4 sector_lds[LDS_SECTORS];
     __shared__ unsigned short sector_level_lds[LDS_SECTORS];
-    __shared__ unsigned short tex_lds[LDS_TEXTURES];
+    __shared__ TexLds tex_lds;
     __shared__ unsigned char colormap_lds[32 * 256];
     __shared__ i64 level_plane_lds[2 * PLANE_LEVELS * 2];
     __shared__ i64 step_scale_lds[STEP_TABLE];
     const int local = blockIdx.y;
     if (local >= lane_count) return;     // uniform over the block
     Tables tb;
-    stage_tables(m, sector_lds, tex_lds, tb);
+    stage_tables(m, sector_lds, &tex_lds, tb);
     for (int k = threadIdx.x; k < 32 * 256 / 4; k += blockDim.x) reinterpret_cast<unsigned int *>(colormap_lds)[k] = reinterpret_cast<const unsigned int *>(m->colormap)[k];
     const int floors = m->floor_level_count, levels = floors + m->ceil_level_count;
     const bool tabled = dm.sector_level != nullptr;   // implies both level lists fit PLANE_LEVELS
@@ -2781,10 +2862,6 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))
             if (ps < 0) {
                 // neither tier nor plane: the flat pass's picture shows here (unless a masked texture covers it);
                 // flat_shade_kernel paints the pixel once that pass has run
-                if (!(meta[j] & META_MASKED)) {
-                    const int slot = atomicAdd(&sc.flat_list_count[local], 1);
-                    if (slot < FLAT_LIST_MAX) sc.flat_list[(size_t)local * FLAT_LIST_MAX + slot] = pixel;
-                }
                 continue;
             }
             const bool is_floor = (meta[j] & META_FLOOR) != 0;
@@ -2803,7 +2880,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))
 // draw decals also keep the depth that pass leaves there (engine.py:11140-11166).
 __device__ void flat_shade_pixel(const DeviceMap &dm, const Scratch &sc, const LaneCtx &c, int local, int pixel, unsigned char *frame) {
     const gd_map_desc *m = &dm.d;
-    Tables tb; tb.m = m; tb.sector = nullptr; tb.tex_bits = nullptr; tb.sector_cached = 0; tb.tex_cached = 0;
+    Tables tb; tb.m = m; tb.sector = nullptr; tb.tex_bits = nullptr; tb.tex_odd = nullptr; tb.sector_cached = 0; tb.tex_cached = 0;
     const int y = pixel / SW, x = pixel - y * SW;
     const size_t i = (size_t)local * VH * SW + pixel;
     const int s = sc.flat_sector[i];
@@ -2902,7 +2979,7 @@ __global__ void __launch_bounds__(SPRITE_COLUMNS) __attribute__((amdgpu_waves_pe
     }
     __syncthreads();
     const int x = x_first + threadIdx.x;
-    if (x >= x_end) return;
+    if (x < x_end) {
     const WallRec *recs = sc.rec + (size_t)local * m->wall_count;
     unsigned char *frame = frame_base + (size_t)local * frame_stride;
     const unsigned int *meta = sc.meta + (size_t)local * VH * SW;
@@ -3042,6 +3119,7 @@ __global__ void __launch_bounds__(SPRITE_COLUMNS) __attribute__((amdgpu_waves_pe
                 *pixel = lit;
             }
         }
+    }
     }
 }
 
@@ -3583,6 +3661,8 @@ struct gd_renderer {
     DeviceMap dm;
     Scratch sc;
     int chunk_lanes;
+    unsigned char *scratch_block;            // the one allocation `sc` is laid out in (null for a renderer made for 0 lanes)
+    size_t scratch_bytes;
     std::vector<void *> allocations;
     hipEvent_t events[16];
     bool events_ready;
@@ -3635,6 +3715,7 @@ size_t carve_scratch(Scratch &sc, unsigned char *base, size_t L, const gd_map_de
     const size_t W = h.wall_count, PX = (size_t)VH * SW, levels = (size_t)(h.floor_level_count + h.ceil_level_count);
     take(&sc.ctx, L);
     take(&sc.rec, L * W);
+    take(&sc.span, L * W);
     take(&sc.frag_rec, L * (size_t)(h.split_count > 0 ? h.split_count * h.fragment_slots : 1));
     take(&sc.cand, L * CAND_MAX * SW);
     take(&sc.cand_count, L * SW);
@@ -3816,7 +3897,7 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     mark();
     hipLaunchKernelGGL(lane_setup_kernel, dim3((count + 63) / 64), dim3(64), 0, stream, r->dm, *lanes, base, count, sc);
     hipLaunchKernelGGL(lane_tables_kernel, dim3(count), dim3(256), 0, stream, r->dm, *lanes, base, count, sc);
-    hipLaunchKernelGGL(wall_setup_kernel, dim3((m.wall_count + 127) / 128, count), dim3(128), 0, stream, r->dm, count, sc);
+    hipLaunchKernelGGL(wall_setup_kernel, dim3((m.wall_count + SETUP_WALLS - 1) / SETUP_WALLS, count), dim3(SETUP_WALLS), 0, stream, r->dm, count, sc);
     if (m.split_count > 0)
         hipLaunchKernelGGL(fragment_setup_kernel, dim3((m.split_count * m.fragment_slots + 63) / 64, count), dim3(64), 0, stream, r->dm, count, sc);
     hipLaunchKernelGGL(strip_key_kernel, dim3((count * (SW / 64) + 3) / 4), dim3(256), 0, stream, count, sc);
@@ -3911,6 +3992,7 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     gd_renderer *r = new (std::nothrow) gd_renderer();
     if (!r) return fail(GD_E_ARG, "out of host memory");
     r->events_ready = false;
+    r->scratch_block = nullptr; r->scratch_bytes = 0;
     std::memset(&r->sc, 0, sizeof(r->sc));
     std::memset(&r->overlays, 0, sizeof(r->overlays));
     r->dm.d = *h;
@@ -4027,6 +4109,7 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
         rc = scratch_alloc(r, bytes, &block);
         if (rc == GD_OK) {
             carve_scratch(sc, block, (size_t)chunk, *h, false);
+            r->scratch_block = block; r->scratch_bytes = bytes;
             hipLaunchKernelGGL(fill_words_kernel, dim3(256), dim3(256), 0, 0, reinterpret_cast<unsigned int *>(sc.flat_col_top), (size_t)chunk * 2 * SW, 0x7f7f7f7fu);
             if (hipDeviceSynchronize() != hipSuccess) rc = fail(GD_E_HIP, "filling flat_col_top");
         }
@@ -4147,6 +4230,19 @@ int gd_renderer_status(gd_renderer *r, int32_t *status) {
     int value = 0;
     HIP_TRY(hipMemcpy(&value, r->sc.status, sizeof(int), hipMemcpyDeviceToHost));
     *status = value;
+    return GD_OK;
+}
+
+/* Fill the renderer's working memory with one byte value (then put back the one buffer the kernels expect ready).
+   Frames must not depend on what that memory held; this lets a caller check it.  Replaces nothing in the reference. */
+int gd_renderer_scribble(gd_renderer *r, int32_t value, void *stream) {
+    if (!r) return fail(GD_E_ARG, "null argument");
+    if (!r->scratch_block) return GD_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const unsigned int byte = (unsigned int)value & 0xFFu, word = byte * 0x01010101u;
+    hipLaunchKernelGGL(fill_words_kernel, dim3(4096), dim3(256), 0, st, reinterpret_cast<unsigned int *>(r->scratch_block), r->scratch_bytes / 4, word);
+    hipLaunchKernelGGL(fill_words_kernel, dim3(256), dim3(256), 0, st, reinterpret_cast<unsigned int *>(r->sc.flat_col_top), (size_t)r->chunk_lanes * 2 * SW, 0x7f7f7f7fu);
+    HIP_TRY(hipGetLastError());
     return GD_OK;
 }
 

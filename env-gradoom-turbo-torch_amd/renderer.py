@@ -132,6 +132,12 @@ class HipRenderer:
         _lib.check(self._lib.gd_renderer_status(self._handle, C.byref(value)))
         return int(value.value)
 
+    def scribble(self, value: int) -> None:
+        """Fill the working memory with one byte value (diagnostic: later frames must not depend on it)."""
+
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        _lib.check(self._lib.gd_renderer_scribble(self._handle, int(value), C.c_void_p(stream)))
+
     def set_overlays(self, overlays: dict) -> None:
         """Upload the weapon and status bar patches (NumPy arrays named like ``gd_overlay_desc``'s fields).
 

@@ -283,6 +283,12 @@ int gd_render_static(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_
 int gd_renderer_status(gd_renderer *r, int32_t *status);
 
 /*
+ * Fill the renderer's working memory with one byte value, asynchronously on `stream` (diagnostic: the frames
+ * that follow must not depend on what the memory held before).  Replaces nothing in the reference.
+ */
+int gd_renderer_scribble(gd_renderer *r, int32_t value, void *stream);
+
+/*
  * Replace the map-wide sector light levels (device pointer to S floats) for the frames
  * that follow on `stream`; the copy is asynchronous.  The reference keeps one
  * sector_lights tensor per map (engine.py:640, 1277-1279); this is how a caller

@@ -30,14 +30,19 @@ def test_indexed_frame_bit_exact_vs_reference_golden(name):
     count = meta["lanes"]
     indexed = torch.zeros((count, 240, 320), dtype=torch.uint8, device="cuda:0")
     obs = torch.zeros((count, 84, 84), dtype=torch.uint8, device="cuda:0")
-    renderer.render(lanes, indexed=indexed, obs=obs)
-    torch.cuda.synchronize()
-    assert renderer.status() == 0
-    ours = indexed.cpu().numpy()
-    mismatched = int((ours != data["indexed"]).sum())
-    assert mismatched == 0, f"{mismatched} palette indices differ from the reference"
-    delta = np.abs(obs.cpu().numpy().astype(np.int32) - data["obs"].astype(np.int32))
-    assert delta.max() <= 1 and delta.mean() < 0.01  # tolerance: tests/test_rendering.py:138-139
+    for fill in (None, 0xFF):   # fresh working memory, then the same memory filled with ones: nothing is cleared between frames
+        if fill is not None:
+            renderer.scribble(fill)
+            indexed.zero_()
+            obs.zero_()
+        renderer.render(lanes, indexed=indexed, obs=obs)
+        torch.cuda.synchronize()
+        assert renderer.status() == 0
+        ours = indexed.cpu().numpy()
+        mismatched = int((ours != data["indexed"]).sum())
+        assert mismatched == 0, f"{mismatched} palette indices differ from the reference (working memory fill {fill})"
+        delta = np.abs(obs.cpu().numpy().astype(np.int32) - data["obs"].astype(np.int32))
+        assert delta.max() <= 1 and delta.mean() < 0.01  # tolerance: tests/test_rendering.py:138-139
     renderer.close()
 
 

@@ -63,6 +63,45 @@ def test_random_maps_and_grazing_poses_match_the_oracle(oracle, first_seed):
         renderer.close()
 
 
+@pytest.mark.parametrize("first_seed", [9000, 9006])
+def test_random_maps_with_other_heights_and_textures_whatever_the_working_memory_held(oracle, first_seed):
+    # doors and crawl spaces, uniform heights, odd texture sizes and eyes at any height, each rendered three times: into
+    # fresh working memory, then after it was filled with 0xFF and with 0xA5 (no frame may depend on what an earlier
+    # frame, or nobody, left there: the kernels clear nothing between frames)
+    from gradoom_amd import hostmath, mapbuild, synthmap
+    from gradoom_amd.renderer import HipRenderer, LaneState
+    from gradoom_amd.selfcheck import make_lane_arrays
+
+    cosine = hostmath.cosine_correction("cpu").numpy()
+    variants = (dict(heights="doors"), dict(heights="uniform"), dict(heights="doors", textures="npot"), dict(textures="mixed"),
+                dict(heights="uniform", textures="npot"), dict(heights="doors"))
+    for seed in range(first_seed, first_seed + 6):
+        print(f"variant case {seed}", flush=True)
+        rng = np.random.default_rng(seed)
+        layout, grid, sectors, linedefs, islands, pillars = SHAPES[seed % len(SHAPES)]
+        smap = synthmap.generate_map(seed, grid=grid, sectors=sectors, linedefs=linedefs, layout=layout, islands=islands,
+                                     pillars=pillars, midtex=float(rng.choice([0.0, 0.2])))
+        smap = synthmap.with_variant(smap, seed + 1, **variants[seed % len(variants)])
+        poses = synthmap.generate_poses(smap, LANES, seed + 3, pitch=bool(rng.random() < 0.5), flash=True,
+                                        margin=float(rng.choice([0.02, 0.15])), eye="any")
+        arrays = make_lane_arrays(smap, poses, synthmap.generate_sprites(smap, LANES, 16, seed + 4))
+        tables = mapbuild.build_map_tables(smap)
+        expected = oracle.render(tables, arrays, cosine)
+        renderer = HipRenderer(smap, LANES, "cuda:0", cosine_correction=cosine, tables=tables)
+        lanes = LaneState.from_numpy(arrays, "cuda:0")
+        for fill in (None, 0xFF, 0xA5):
+            if fill is not None:
+                renderer.scribble(fill)
+            indexed = torch.zeros((LANES, 240, 320), dtype=torch.uint8, device="cuda:0")
+            obs = torch.zeros((LANES, 84, 84), dtype=torch.uint8, device="cuda:0")
+            renderer.render(lanes, indexed=indexed, obs=obs)
+            torch.cuda.synchronize()
+            assert renderer.status() == 0
+            assert np.array_equal(indexed.cpu().numpy(), expected["indexed"]), f"seed {seed} fill {fill}"
+            assert np.array_equal(obs.cpu().numpy(), expected["obs"]), f"seed {seed} fill {fill}"
+        renderer.close()
+
+
 def test_cameras_outside_the_map_match_the_oracle(oracle):
     """Cameras in the void beside the map: no wall pass claims most of the screen, so nearly every pixel shows the
     flat pass's picture (far more than the per-lane gap pixel list holds) and most of them stay unresolved."""
