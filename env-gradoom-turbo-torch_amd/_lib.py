@@ -19,6 +19,7 @@ SYMBOLS = (
     "gd_renderer_destroy",
     "gd_renderer_status",
     "gd_renderer_scribble",
+    "gd_renderer_set_assembly",
     "gd_renderer_set_sector_lights",
     "gd_renderer_set_overlays",
     "gd_render",
@@ -58,6 +59,8 @@ def library() -> C.CDLL:
     lib.gd_renderer_destroy.argtypes = [C.c_void_p]
     lib.gd_renderer_status.restype = C.c_int
     lib.gd_renderer_status.argtypes = [C.c_void_p, C.POINTER(C.c_int32)]
+    lib.gd_renderer_set_assembly.restype = C.c_int
+    lib.gd_renderer_set_assembly.argtypes = [C.c_void_p, C.c_int32]
     lib.gd_renderer_scribble.restype = C.c_int
     lib.gd_renderer_scribble.argtypes = [C.c_void_p, C.c_int32, C.c_void_p]
     lib.gd_renderer_set_overlays.restype = C.c_int

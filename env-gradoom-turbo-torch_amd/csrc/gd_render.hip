@@ -2594,7 +2594,11 @@ __device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const Col
         for (int j = 0; j < WALL_ROWS; ++j) {
             const int y = yb + j;
             if (y >= y1) continue;
-            pb.frame[(size_t)y * SW + x] = colormap[shade * 256 + texel[j]];
+            // the texel goes to the frame where there is one; otherwise it waits in the sprite clip plane, which nothing
+            // reads any more once a column's traversal is over, for the kernel that assembles the frame
+            const unsigned char colour = colormap[shade * 256 + texel[j]];
+            if (pb.frame) pb.frame[(size_t)y * SW + x] = colour;
+            else pb.clip_depth[(size_t)y * SW + x] = __uint_as_float((unsigned)colour);
             pb.meta[(size_t)y * SW + x] = word[j] | META_MASKED;
             if (DEPTH) pb.scene_depth[(size_t)y * SW + x] = md;
         }
@@ -2687,7 +2691,7 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
     cc.x = x;
     ray_direction(lane_ctx, x, &cc.rx, &cc.ry);
     PixelBuffers pb;
-    pb.frame = frame_base + (size_t)local * frame_stride;
+    pb.frame = frame_base ? frame_base + (size_t)local * frame_stride : nullptr;
     pb.meta = sc.meta + (size_t)local * VH * SW;
     pb.clip_depth = sc.clip_depth + (size_t)local * VH * SW;
     pb.scene_depth = DEPTH ? sc.scene_depth + (size_t)local * VH * SW : nullptr;
@@ -2931,23 +2935,19 @@ struct SpriteRec {
     int id, flags;   // bit0 alive, bit1 fullbright, bits 8..15 style (signed: -1 opaque, -2 translucent, >= 0 additive)
 };
 
-__global__ void __launch_bounds__(SPRITE_COLUMNS) __attribute__((amdgpu_waves_per_eu(5, 5))) sprite_columns_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc,
-                                                            unsigned char *frame_base, size_t frame_stride) {
-    extern __shared__ unsigned char shared_raw[];
-    SpriteRec *sp = reinterpret_cast<SpriteRec *>(shared_raw);
+// A frame some kernel paints into: all of a lane's 320x240 frame in device memory, or the rows a work-group keeps in LDS.
+struct GlobalFrame {
+    unsigned char *base;     // row 0, column 0 of the lane's frame
+    __device__ __forceinline__ unsigned char *at(int y, int x) const { return base + (size_t)y * SW + x; }
+};
+
+// The billboards of one lane, worked out once per work-group (engine.py:14684-14760): `sp[a]` for every slot, and in
+// `on_screen` the slots that can reach columns [x_first, x_end) at all (alive, in front, some column between left and
+// right): the per-column loops only walk these.  Their order in the list is irrelevant, ties go by slot number.
+__device__ __forceinline__ void stage_sprites(const DeviceMap &dm, const gd_lanes_desc &lanes, int n, const LaneCtx &L, int x_first, int x_end,
+                                              int row_first, int row_end, SpriteRec *sp, unsigned short *on_screen, int *on_screen_count) {
     const gd_map_desc *m = &dm.d;
-    const int local = blockIdx.y;
-    if (local >= lane_count) return;
-    const int n = lane_base + local;
     const int A = lanes.sprite_slots;
-    const int x_first = blockIdx.x * SPRITE_COLUMNS, x_end = x_first + SPRITE_COLUMNS < SW ? x_first + SPRITE_COLUMNS : SW;
-    // the slots that can reach the screen at all (alive, in front, some column between left and right): the
-    // per-column loops below only walk these.  Their order in the list is irrelevant, ties go by slot number.
-    unsigned short *on_screen = reinterpret_cast<unsigned short *>(sp + A);
-    __shared__ int on_screen_count;
-    if (threadIdx.x == 0) on_screen_count = 0;
-    __syncthreads();
-    const LaneCtx L = sc.ctx[local];
     for (int a = threadIdx.x; a < A; a += blockDim.x) {
         SpriteRec s;
         size_t k = (size_t)n * A + a;
@@ -2972,16 +2972,27 @@ __global__ void __launch_bounds__(SPRITE_COLUMNS) __attribute__((amdgpu_waves_pe
         s.texmid = (i64)m->spr_top[s.id] * FIXED_UNIT - round_to_i64((L.view_z - z) * 65536.0f);
         s.top_fixed = L.center_fixed - (mul64(s.texmid, s.yscale) >> 16);
         s.iscale = tdiv(UINT32_MASK, max64(s.yscale, 1));
-        const bool reaches = (s.flags & 1) && (s.depth > 0) && (s.right > x_first) && (s.left < x_end) && (s.right > s.left);
+        bool reaches = (s.flags & 1) && (s.depth > 0) && (s.right > x_first) && (s.left < x_end) && (s.right > s.left);
+        if (reaches && s.iscale > 0 && (row_first > 0 || row_end < VH)) {
+            // the rows whose source row can fall inside the patch (the bracket sprite_column works with, a row to spare)
+            const i64 fraction_base = s.texmid - (mul64(L.center_fixed - FIXED_UNIT, s.iscale) >> 16);
+            const i64 y_lo = tdiv(-fraction_base, s.iscale) - 1, y_hi = tdiv(((i64)m->spr_h[s.id] << 16) - fraction_base, s.iscale) + 2;
+            reaches = y_hi > row_first && y_lo < row_end;
+        }
         s.light = reaches ? m->sector_lights[sector_at(m, s.x, s.y)] : 0.0f;
         sp[a] = s;
-        if (reaches) on_screen[atomicAdd(&on_screen_count, 1)] = (unsigned short)a;
+        if (reaches) on_screen[atomicAdd(on_screen_count, 1)] = (unsigned short)a;
     }
-    __syncthreads();
-    const int x = x_first + threadIdx.x;
-    if (x < x_end) {
+}
+
+// Every billboard that shows in column x, rows [row_first, row_end), far -> near (engine.py:14762-14947).
+template <typename Frame>
+__device__ __forceinline__ void sprite_column(const DeviceMap &dm, const gd_lanes_desc &lanes, const Scratch &sc, int local, int n, const LaneCtx &L,
+                                              const SpriteRec *sp, const unsigned short *on_screen, int listed, int x, int row_first, int row_end,
+                                              const Frame &frame) {
+    const gd_map_desc *m = &dm.d;
+    const int A = lanes.sprite_slots;
     const WallRec *recs = sc.rec + (size_t)local * m->wall_count;
-    unsigned char *frame = frame_base + (size_t)local * frame_stride;
     const unsigned int *meta = sc.meta + (size_t)local * VH * SW;
     // nearest blocking linedef of this column (engine.py:10534-10557), gathered by wall_setup
     const u64 hit = sc.block_hit[(size_t)local * SW + x];
@@ -2997,7 +3008,6 @@ __global__ void __launch_bounds__(SPRITE_COLUMNS) __attribute__((amdgpu_waves_pe
     // The sprites that can show in this column at all (alive, in front, horizontally covering it and
     // not hidden by the column's blocking linedef), as a bit set: the painter's loop below runs once
     // per drawn sprite and would otherwise test every slot each time.
-    const int listed = on_screen_count;
     u64 cover[8] = {0, 0, 0, 0, 0, 0, 0, 0};   // sprite_slots <= 512; bit p of the set = on_screen[p]
 #pragma unroll
     for (int word = 0; word < 8; ++word) {
@@ -3047,10 +3057,10 @@ __global__ void __launch_bounds__(SPRITE_COLUMNS) __attribute__((amdgpu_waves_pe
         i64 fraction_base = s.texmid - (mul64(L.center_fixed - FIXED_UNIT, s.iscale) >> 16);
         // Rows whose source row sv = (fraction_base + y * iscale) >> 16 can fall inside the patch:
         // a bracket from two divisions, a row too wide on either side; the exact test stays per row.
-        int y_lo = 0, y_hi = VH;
+        int y_lo = row_first, y_hi = row_end;
         if (s.iscale > 0) {
-            y_lo = (int)clampi(tdiv(-fraction_base, s.iscale) - 1, 0, VH);
-            y_hi = (int)clampi(tdiv(((i64)height << 16) - fraction_base, s.iscale) + 2, 0, VH);
+            y_lo = (int)clampi(tdiv(-fraction_base, s.iscale) - 1, row_first, row_end);
+            y_hi = (int)clampi(tdiv(((i64)height << 16) - fraction_base, s.iscale) + 2, row_first, row_end);
         }
         // SPRITE_ROWS rows per step, each stage's loads issued together so that their latencies overlap
         for (int yb = y_lo; yb < y_hi; yb += SPRITE_ROWS) {
@@ -3113,14 +3123,35 @@ __global__ void __launch_bounds__(SPRITE_COLUMNS) __attribute__((amdgpu_waves_pe
                 if ((i64)y < post_screen_top) continue;
                 // engine.py:14914-14939: opaque, additive table or translucent table over the pixel below
                 unsigned char lit = m->colormap[shade * 256 + texel[j]];
-                unsigned char *pixel = frame + (size_t)y * SW + x;
+                unsigned char *pixel = frame.at(y, x);
                 if (style == -2) lit = m->translucent_lut[(size_t)*pixel * 256 + lit];
                 else if (style >= 0) lit = m->additive_luts[((size_t)(style > 1 ? 1 : style) * 256 + *pixel) * 256 + lit];
                 *pixel = lit;
             }
         }
     }
-    }
+}
+
+__global__ void __launch_bounds__(SPRITE_COLUMNS) __attribute__((amdgpu_waves_per_eu(5, 5))) sprite_columns_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc,
+                                                            unsigned char *frame_base, size_t frame_stride) {
+    extern __shared__ unsigned char shared_raw[];
+    SpriteRec *sp = reinterpret_cast<SpriteRec *>(shared_raw);
+    const int local = blockIdx.y;
+    if (local >= lane_count) return;
+    const int n = lane_base + local;
+    const int A = lanes.sprite_slots;
+    const int x_first = blockIdx.x * SPRITE_COLUMNS, x_end = x_first + SPRITE_COLUMNS < SW ? x_first + SPRITE_COLUMNS : SW;
+    unsigned short *on_screen = reinterpret_cast<unsigned short *>(sp + A);
+    __shared__ int on_screen_count;
+    if (threadIdx.x == 0) on_screen_count = 0;
+    __syncthreads();
+    const LaneCtx L = sc.ctx[local];
+    stage_sprites(dm, lanes, n, L, x_first, x_end, 0, VH, sp, on_screen, &on_screen_count);
+    __syncthreads();
+    const int x = x_first + threadIdx.x;
+    if (x >= x_end) return;
+    GlobalFrame frame; frame.base = frame_base + (size_t)local * frame_stride;
+    sprite_column(dm, lanes, sc, local, n, L, sp, on_screen, on_screen_count, x, 0, VH, frame);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -3284,6 +3315,46 @@ __device__ void hud_number(const gd_overlay_desc &o, HudEntry *list, int *count,
     }
 }
 
+// The status bar's patches in drawing order (engine.py:15232-15267), written by one thread.
+__device__ int build_hud_list(const gd_overlay_desc &o, const int *state, HudEntry *list) {
+    int count = 0;
+    auto patch_at = [&](int patch, int x, int y) {
+        if (patch >= 0 && patch < o.hud_patch_count && count < HUD_LIST_MAX) { HudEntry e; e.patch = patch; e.x = x; e.y = y; list[count++] = e; }
+    };
+    patch_at(0, 0, 0);
+    patch_at(1, 104, 0);
+    hud_number(o, list, &count, state[0], 44, 3, false);
+    hud_number(o, list, &count, state[1], 90, 3, false);
+    patch_at(12, 90, 3);
+    hud_number(o, list, &count, state[2], 221, 3, false);
+    patch_at(12, 221, 3);
+    patch_at(state[3], 143, 0);
+    const int arms_x[6] = {111, 123, 135, 111, 123, 135}, arms_y[6] = {4, 4, 4, 14, 14, 14};
+    for (int k = 0; k < 6; ++k) {
+        const bool owned = k < 5 && ((state[4] >> k) & 1);
+        patch_at(owned ? 30 + k : 38 + k, arms_x[k], arms_y[k]);
+    }
+    const int maximum[4] = {200, 50, 50, 300};
+    for (int row = 0; row < 4; ++row) {
+        hud_number(o, list, &count, state[5 + row], 288, 5 + row * 6, true);
+        hud_number(o, list, &count, maximum[row], 314, 5 + row * 6, true);
+    }
+    return count;
+}
+
+// One pixel of the status bar (cx, cy relative to row 208): the last listed patch with an opaque texel there.
+__device__ __forceinline__ unsigned char hud_pixel(const gd_overlay_desc &o, const HudEntry *list, int count, int cx, int cy) {
+    for (int k = count - 1; k >= 0; --k) {
+        const HudEntry e = list[k];
+        // _native_draw_hud_patch (engine.py:15153-15184): position minus the patch's own offsets, clipped
+        const int sx = cx - (e.x - o.hud_left[e.patch]), sy = cy - (e.y - o.hud_top[e.patch]);
+        if (sx < 0 || sy < 0 || sx >= o.hud_w[e.patch] || sy >= o.hud_h[e.patch] || sx >= o.hud_max_w || sy >= o.hud_max_h) continue;
+        const size_t t = ((size_t)e.patch * o.hud_max_h + sy) * o.hud_max_w + sx;
+        if (o.hud_opaque[t]) return o.hud_atlas[t];
+    }
+    return 0;
+}
+
 __global__ void __launch_bounds__(256) hud_kernel(Overlays ov, const int *hud_state, int lane_base, int lane_count,
                                                   unsigned char *frame_base, size_t frame_stride) {
     const gd_overlay_desc &o = ov.d;
@@ -3291,47 +3362,10 @@ __global__ void __launch_bounds__(256) hud_kernel(Overlays ov, const int *hud_st
     __shared__ int list_count;
     const int local = blockIdx.x;
     if (local >= lane_count) return;
-    if (threadIdx.x == 0) {
-        const int *state = hud_state + (size_t)(lane_base + local) * 9;
-        int count = 0;
-        auto patch_at = [&](int patch, int x, int y) {
-            if (patch >= 0 && patch < o.hud_patch_count && count < HUD_LIST_MAX) { HudEntry e; e.patch = patch; e.x = x; e.y = y; list[count++] = e; }
-        };
-        patch_at(0, 0, 0);
-        patch_at(1, 104, 0);
-        hud_number(o, list, &count, state[0], 44, 3, false);
-        hud_number(o, list, &count, state[1], 90, 3, false);
-        patch_at(12, 90, 3);
-        hud_number(o, list, &count, state[2], 221, 3, false);
-        patch_at(12, 221, 3);
-        patch_at(state[3], 143, 0);
-        const int arms_x[6] = {111, 123, 135, 111, 123, 135}, arms_y[6] = {4, 4, 4, 14, 14, 14};
-        for (int k = 0; k < 6; ++k) {
-            const bool owned = k < 5 && ((state[4] >> k) & 1);
-            patch_at(owned ? 30 + k : 38 + k, arms_x[k], arms_y[k]);
-        }
-        const int maximum[4] = {200, 50, 50, 300};
-        for (int row = 0; row < 4; ++row) {
-            hud_number(o, list, &count, state[5 + row], 288, 5 + row * 6, true);
-            hud_number(o, list, &count, maximum[row], 314, 5 + row * 6, true);
-        }
-        list_count = count;
-    }
+    if (threadIdx.x == 0) list_count = build_hud_list(o, hud_state + (size_t)(lane_base + local) * 9, list);
     __syncthreads();
     unsigned char *bar = frame_base + (size_t)local * frame_stride + (size_t)VH * SW;
-    for (int p = threadIdx.x; p < HUD_ROWS * SW; p += blockDim.x) {
-        const int cy = p / SW, cx = p - cy * SW;
-        unsigned char value = 0;
-        for (int k = list_count - 1; k >= 0; --k) {
-            const HudEntry e = list[k];
-            // _native_draw_hud_patch (engine.py:15153-15184): position minus the patch's own offsets, clipped
-            const int sx = cx - (e.x - o.hud_left[e.patch]), sy = cy - (e.y - o.hud_top[e.patch]);
-            if (sx < 0 || sy < 0 || sx >= o.hud_w[e.patch] || sy >= o.hud_h[e.patch] || sx >= o.hud_max_w || sy >= o.hud_max_h) continue;
-            const size_t t = ((size_t)e.patch * o.hud_max_h + sy) * o.hud_max_w + sx;
-            if (o.hud_opaque[t]) { value = o.hud_atlas[t]; break; }
-        }
-        bar[p] = value;
-    }
+    for (int p = threadIdx.x; p < HUD_ROWS * SW; p += blockDim.x) bar[p] = hud_pixel(o, list, list_count, p % SW, p / SW);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -3491,6 +3525,267 @@ __global__ void expand_rgb_kernel(const unsigned char *indexed, const unsigned c
     if (i >= pixels) return;
     int p = indexed[i] * 3;
     rgb[i * 3] = pal[p]; rgb[i * 3 + 1] = pal[p + 1]; rgb[i * 3 + 2] = pal[p + 2];
+}
+
+// ---------------------------------------------------------------------------------------------
+// finish: everything after the wall traversal and the flat selection, for one band of one lane's frame at a time,
+// with the band held in LDS from the first shaded pixel to the pooled observation: plane and tier pixels
+// (engine.py:13372-13405), the flat pass's pixels where nothing else shows (engine.py:11145-11163), billboards
+// (engine.py:14762-14947), weapon and status bar (engine.py:15051-15110, 15232-15267), PLAYPAL expansion
+// (engine.py:15381-15398), area pooling and the frame stack (_triton_kernels.py:120-177, engine.py:9545-9548).
+// The 320x240 frame only goes to device memory when the caller asks for it.
+// ---------------------------------------------------------------------------------------------
+// A band is 80 frame rows: 28 observation rows pool exactly those (84 observation rows x 240 / 84 source rows each).
+#define BAND_ROWS 80
+#define BAND_COUNT (GD_SCREEN_HEIGHT / BAND_ROWS)
+#define BAND_OBS_ROWS (BAND_ROWS * GD_OBS_SIZE / GD_SCREEN_HEIGHT)
+#define BAND_THREADS 512   // sixteen wavefronts a compute unit when two work-groups share it: four per SIMD, none left over
+static_assert(BAND_COUNT * BAND_ROWS == GD_SCREEN_HEIGHT && BAND_OBS_ROWS * BAND_COUNT == GD_OBS_SIZE, "bands tile the frame and the observation");
+static_assert(BAND_THREADS >= SW && (BAND_OBS_ROWS * GD_OBS_SIZE) % 4 == 0, "band_finish_kernel: thread layout");
+
+struct BandFrame {   // the rows [row0, row0 + BAND_ROWS) of a lane's frame, in LDS
+    unsigned char *rows;
+    int row0;
+    __device__ __forceinline__ unsigned char *at(int y, int x) const { return rows + (y - row0) * SW + x; }
+};
+
+struct FinishOut {   // device pointers of the chunk's first lane; null = not wanted
+    unsigned char *indexed, *rgb, *obs, *frames, *final_frames;
+    const unsigned char *reset_mask;
+    const float *blend;
+    int stack_mode, source_rows;
+};
+
+__global__ void __launch_bounds__(BAND_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) band_finish_kernel(DeviceMap dm, Overlays ov, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc, FinishOut out) {
+    extern __shared__ unsigned char shared_raw[];                // billboard records, when there are too many to reuse the tables' LDS
+    __shared__ unsigned int band_words[BAND_ROWS * SW / 4];
+    // the sector table and the colormap serve the shading phase only; the billboard records take their place afterwards
+    __shared__ struct { float4 sector[LDS_SECTORS]; unsigned char colormap[32 * 256]; } shading_lds;
+    float4 *sector_lds = shading_lds.sector;
+    unsigned char *colormap_lds = shading_lds.colormap;
+    __shared__ unsigned short sector_level_lds[LDS_SECTORS];
+    __shared__ TexLds tex_lds;
+    __shared__ i64 level_plane_lds[2 * PLANE_LEVELS * 2];
+    __shared__ i64 step_scale_lds[STEP_TABLE];
+    __shared__ unsigned int pal[256];                            // PLAYPAL after the lane's screen blend: red | green << 8 | blue << 16
+    __shared__ unsigned int gray_words[BAND_OBS_ROWS * GD_OBS_SIZE / 4];
+    __shared__ HudEntry hud_list[HUD_LIST_MAX];
+    __shared__ int hud_count, on_screen_count;
+    const gd_map_desc *m = &dm.d;
+    const int band = blockIdx.x, local = blockIdx.y;
+    if (local >= lane_count) return;     // uniform over the block
+    const int n = lane_base + local;
+    const int tid = threadIdx.x;
+    const int row0 = band * BAND_ROWS;
+    const int view_rows = row0 >= VH ? 0 : (row0 + BAND_ROWS <= VH ? BAND_ROWS : VH - row0);   // the rest are status bar rows
+    unsigned char *band_bytes = reinterpret_cast<unsigned char *>(band_words);
+    BandFrame frame; frame.rows = band_bytes; frame.row0 = row0;
+    Tables tb;
+    stage_tables(m, sector_lds, &tex_lds, tb);
+    for (int k = tid; k < 32 * 256 / 4; k += BAND_THREADS) reinterpret_cast<unsigned int *>(colormap_lds)[k] = reinterpret_cast<const unsigned int *>(m->colormap)[k];
+    const int floors = m->floor_level_count, levels = floors + m->ceil_level_count;
+    const bool tabled = dm.sector_level != nullptr;   // implies both level lists fit PLANE_LEVELS
+    if (tabled) {
+        for (int s = tid; s < tb.sector_cached; s += BAND_THREADS) sector_level_lds[s] = dm.sector_level[s];
+        for (int k = tid; k < 2 * levels; k += BAND_THREADS) level_plane_lds[k] = sc.level_plane[(size_t)local * levels * 2 + k];
+        if (tid < STEP_TABLE) step_scale_lds[tid] = sc.step_scale[(size_t)local * STEP_TABLE + tid];
+    }
+    if (tid < 256) {
+        unsigned int r = m->playpal[3 * tid], g = m->playpal[3 * tid + 1], b = m->playpal[3 * tid + 2];
+        if (out.blend) {
+            const float bonus = out.blend[2 * local], flash = out.blend[2 * local + 1];
+            r = blended_channel((unsigned char)r, 0, bonus, flash); g = blended_channel((unsigned char)g, 1, bonus, flash); b = blended_channel((unsigned char)b, 2, bonus, flash);
+        }
+        pal[tid] = r | (g << 8) | (b << 16);
+    }
+    if (tid == 0) {
+        on_screen_count = 0;
+        hud_count = (view_rows < BAND_ROWS && lanes.hud_state && ov.d.hud_patch_count > 0) ? build_hud_list(ov.d, lanes.hud_state + (size_t)n * 9, hud_list) : 0;
+    }
+    __syncthreads();
+    const LaneCtx L = sc.ctx[local];
+    LaneTables lt; lt.level_plane = level_plane_lds; lt.step_scale = step_scale_lds; lt.floors = floors;
+    // --- the status bar rows of this band (engine.py:15232-15267); empty without status bar patches
+    for (int p = tid; p < (BAND_ROWS - view_rows) * SW; p += BAND_THREADS)
+        band_bytes[view_rows * SW + p] = hud_count > 0 ? hud_pixel(ov.d, hud_list, hud_count, p % SW, row0 + view_rows + p / SW - VH) : (unsigned char)0;
+    // --- every view pixel of the band once: a wall tier's palette index, a visplane's flat, a masked mid-texture's texel, or
+    // the flat pass's pick.  A wavefront takes a row at a time, its lanes the row's five groups of 64 columns: what depends
+    // on the row alone is worked out once per row, and each stage's loads are issued together.
+    const size_t lane_pixels = (size_t)local * VH * SW;
+    const int wave = tid >> 6, lane_id = tid & 63;
+    constexpr int ROW_GROUPS = SW / 64;
+    for (int py = wave; py < view_rows; py += BAND_THREADS / 64) {
+        const int y = row0 + py;
+        const size_t row_at = lane_pixels + (size_t)y * SW;
+        const i64 yslope = sc.row_slope[(size_t)local * VH + y];
+        unsigned int meta[ROW_GROUPS];
+#pragma unroll
+        for (int j = 0; j < ROW_GROUPS; ++j) meta[j] = sc.meta[row_at + j * 64 + lane_id];
+        int colormap_row[ROW_GROUPS]; unsigned char texel[ROW_GROUPS];
+        bool shade[ROW_GROUPS];
+#pragma unroll
+        for (int j = 0; j < ROW_GROUPS; ++j) {
+            const int ps = (int)((meta[j] >> META_SECTOR_SHIFT) & META_SECTOR_MASK) - 1;
+            shade[j] = tabled && ps >= 0 && !(meta[j] & (META_FILLED | META_MASKED));
+            texel[j] = 0; colormap_row[j] = 0;
+            if (!shade[j]) continue;
+            const bool is_floor = (meta[j] & META_FLOOR) != 0;
+            const unsigned short pair = ps < tb.sector_cached ? sector_level_lds[ps] : dm.sector_level[ps];
+            const size_t texel_at = flat_sample_tabled(tb, L, lt, yslope, is_floor ? (pair & 0xFF) : (pair >> 8), ps, is_floor, j * 64 + lane_id, y, &colormap_row[j]);
+            texel[j] = m->tex_atlas[texel_at];
+        }
+#pragma unroll
+        for (int j = 0; j < ROW_GROUPS; ++j) {
+            const int x = j * 64 + lane_id;
+            const int ps = (int)((meta[j] >> META_SECTOR_SHIFT) & META_SECTOR_MASK) - 1;
+            unsigned char colour;
+            if (meta[j] & META_MASKED) colour = (unsigned char)__float_as_uint(sc.clip_depth[row_at + x]);   // left there by masked_midtexture
+            else if (meta[j] & META_FILLED) colour = (unsigned char)(meta[j] >> META_SECTOR_SHIFT);
+            else if (shade[j]) colour = colormap_lds[colormap_row[j] * 256 + texel[j]];
+            else if (ps >= 0) colour = flat_pixel(tb, colormap_lds, L, ps, (meta[j] & META_FLOOR) != 0, x, y);
+            else colour = flat_pixel(tb, colormap_lds, L, sc.flat_sector[row_at + x], ((float)y - flat_center(L)) > 0, x, y);   // the flat pass's picture
+            band_bytes[py * SW + x] = colour;
+        }
+    }
+    // --- billboards, one thread per screen column
+    if (lanes.sprite_slots > 0 && lanes.sprite_x && view_rows > 0) {
+        __syncthreads();                  // every shaded pixel is in place, and the shading tables are free
+        const bool fits = (size_t)lanes.sprite_slots * (sizeof(SpriteRec) + sizeof(unsigned short)) <= sizeof(shading_lds);
+        SpriteRec *sp = reinterpret_cast<SpriteRec *>(fits ? reinterpret_cast<unsigned char *>(&shading_lds) : shared_raw);
+        unsigned short *on_screen = reinterpret_cast<unsigned short *>(sp + lanes.sprite_slots);
+        stage_sprites(dm, lanes, n, L, 0, SW, row0, row0 + view_rows, sp, on_screen, &on_screen_count);
+        __syncthreads();
+        if (tid < SW && on_screen_count > 0) sprite_column(dm, lanes, sc, local, n, L, sp, on_screen, on_screen_count, tid, row0, row0 + view_rows, frame);
+    }
+    __syncthreads();
+    // --- the player's weapon and its muzzle flash (engine.py:15051-15110)
+    if (lanes.weapon_state && ov.d.weapon_patch_count > 0) {
+        const int64_t *state = lanes.weapon_state + (size_t)n * 5;
+        if (state[4] != 0) {
+            for (int p = tid; p < view_rows * SW; p += BAND_THREADS) {
+                const int py = p / SW, px = p - py * SW;
+                unsigned char value;
+                bool drawn = psprite_texel(ov.d, state[0], state[2], state[3], px, row0 + py, &value);
+                unsigned char flash;
+                if (state[1] >= 0 && psprite_texel(ov.d, state[1], state[2], state[3], px, row0 + py, &flash)) { value = flash; drawn = true; }
+                if (drawn) band_bytes[p] = value;
+            }
+        }
+        __syncthreads();
+    }
+    // --- what the caller asked for
+    if (out.indexed) {
+        uint4 *rows = reinterpret_cast<uint4 *>(out.indexed + ((size_t)local * GD_SCREEN_HEIGHT + row0) * SW);
+        const bool aligned = (reinterpret_cast<size_t>(out.indexed) & 15) == 0;
+        if (aligned) {
+            for (int k = tid; k < BAND_ROWS * SW / 16; k += BAND_THREADS) rows[k] = reinterpret_cast<const uint4 *>(band_words)[k];
+        } else {
+            unsigned char *bytes = out.indexed + ((size_t)local * GD_SCREEN_HEIGHT + row0) * SW;
+            for (int k = tid; k < BAND_ROWS * SW; k += BAND_THREADS) bytes[k] = band_bytes[k];
+        }
+    }
+    if (out.rgb) {   // four pixels, twelve bytes, three words per step
+        unsigned char *rows = out.rgb + ((size_t)local * GD_SCREEN_HEIGHT + row0) * SW * 3;
+        const bool aligned = (reinterpret_cast<size_t>(out.rgb) & 3) == 0;
+        for (int k = tid; k < BAND_ROWS * SW / 4; k += BAND_THREADS) {
+            const unsigned int four = band_words[k];
+            const unsigned int c0 = pal[four & 0xFFu], c1 = pal[(four >> 8) & 0xFFu], c2 = pal[(four >> 16) & 0xFFu], c3 = pal[four >> 24];
+            const unsigned int w0 = c0 | (c1 << 24), w1 = (c1 >> 8) | (c2 << 16), w2 = (c2 >> 16) | (c3 << 8);
+            if (aligned) {
+                unsigned int *words = reinterpret_cast<unsigned int *>(rows) + 3 * k;
+                words[0] = w0; words[1] = w1; words[2] = w2;
+            } else {
+                unsigned char *bytes = rows + 12 * k;
+                for (int q = 0; q < 4; ++q) { bytes[q] = (unsigned char)(w0 >> (8 * q)); bytes[4 + q] = (unsigned char)(w1 >> (8 * q)); bytes[8 + q] = (unsigned char)(w2 >> (8 * q)); }
+            }
+        }
+    }
+    if (!out.obs && !out.frames) return;
+    // --- the band's observation rows, pooled from LDS (_triton_kernels.py:120-177).  An observation pixel covers 240/84 source
+    // rows and 320/84 source columns; its weights (y_overlap * x_overlap) // 48 are exactly (y_overlap / 12) * (x_overlap / 4),
+    // since row overlaps are multiples of 12 and column overlaps multiples of 4 (84 = 12 * 7 = 4 * 21, 240 = 12 * 20,
+    // 320 = 4 * 80): the weighted sum factors into a pass along the rows and one down the columns, all in integers.
+    // Seven observation rows pool exactly twenty source rows; rows at or past source_rows are black.
+    constexpr int OBS_GROUP = 7, SRC_GROUP = OBS_GROUP * GD_SCREEN_HEIGHT / GD_OBS_SIZE;   // 7 and 20
+    static_assert(BAND_OBS_ROWS % OBS_GROUP == 0 && SRC_GROUP * GD_OBS_SIZE == OBS_GROUP * GD_SCREEN_HEIGHT, "observation rows group by seven");
+    // per source row and observation column: the three channel sums along the row, 16 bits each (at most 80 * 255)
+    unsigned short *along = reinterpret_cast<unsigned short *>(&shading_lds);
+    static_assert(sizeof(shading_lds) >= (size_t)SRC_GROUP * GD_OBS_SIZE * 3 * sizeof(unsigned short), "row sums fit the shading tables' LDS");
+    const int first_obs_row = band * BAND_OBS_ROWS;
+    for (int group = 0; group < BAND_OBS_ROWS / OBS_GROUP; ++group) {
+        __syncthreads();   // the billboard records (first round) or the last group's row sums are no longer needed
+        for (int q = tid; q < SRC_GROUP * GD_OBS_SIZE; q += BAND_THREADS) {
+            const int sy = q / GD_OBS_SIZE, ox = q - sy * GD_OBS_SIZE;
+            const int band_row = group * SRC_GROUP + sy;
+            const unsigned char *row = band_bytes + band_row * SW;
+            const int x_start = ox * 320, x_end = x_start + 320, first_x = x_start / 84;
+            unsigned int rs = 0, gs = 0, bs = 0;
+            if (row0 + band_row < out.source_rows) {
+#pragma unroll
+                for (int sx = 0; sx < 5; ++sx) {
+                    const int source_x = first_x + sx;
+                    const int over = min(x_end, (source_x + 1) * 84) - max(x_start, source_x * 84);
+                    const unsigned weight = (source_x >= SW || over <= 0) ? 0u : (unsigned)over >> 2;
+                    const unsigned int colour = pal[row[min(source_x, SW - 1)]];
+                    rs += __umul24(colour & 0xFFu, weight); gs += __umul24((colour >> 8) & 0xFFu, weight); bs += __umul24(colour >> 16, weight);
+                }
+            }
+            along[3 * q] = (unsigned short)rs; along[3 * q + 1] = (unsigned short)gs; along[3 * q + 2] = (unsigned short)bs;
+        }
+        __syncthreads();
+        for (int q = tid; q < OBS_GROUP * GD_OBS_SIZE; q += BAND_THREADS) {
+            const int row_in_group = q / GD_OBS_SIZE, ox = q - row_in_group * GD_OBS_SIZE;
+            const int y_start = row_in_group * 240, y_end = y_start + 240, first_y = y_start / 84;   // relative to the group's first source row
+            unsigned int rs = 0, gs = 0, bs = 0;
+#pragma unroll
+            for (int sy = 0; sy < 4; ++sy) {
+                const int source_y = first_y + sy;
+                const int over = min(y_end, (source_y + 1) * 84) - max(y_start, source_y * 84);
+                const unsigned weight = (source_y >= SRC_GROUP || over <= 0) ? 0u : (unsigned)over / 12u;
+                const unsigned short *sums = along + 3 * (min(source_y, SRC_GROUP - 1) * GD_OBS_SIZE + ox);
+                rs += __umul24(sums[0], weight); gs += __umul24(sums[1], weight); bs += __umul24(sums[2], weight);
+            }
+            const unsigned r = (rs + 800u) / 1600u, g = (gs + 800u) / 1600u, b = (bs + 800u) / 1600u;
+            reinterpret_cast<unsigned char *>(gray_words)[group * OBS_GROUP * GD_OBS_SIZE + q] = (unsigned char)((r * 77u + g * 150u + b * 29u + 128u) >> 8);
+        }
+    }
+    __syncthreads();
+    // the band's pixels are contiguous in the observation; they go out, and the stack is rolled, a word (four pixels) per thread
+    const size_t F = (size_t)GD_OBS_SIZE * GD_OBS_SIZE / 4;     // words per observation
+    const bool stack_aligned = ((reinterpret_cast<size_t>(out.frames) | reinterpret_cast<size_t>(out.final_frames)) & 3) == 0;
+    const bool resets = out.reset_mask && out.reset_mask[local];
+    auto load_word = [](const unsigned char *p, bool aligned) -> unsigned int {
+        if (aligned) return *reinterpret_cast<const unsigned int *>(p);
+        return (unsigned)p[0] | ((unsigned)p[1] << 8) | ((unsigned)p[2] << 16) | ((unsigned)p[3] << 24);
+    };
+    auto store_word = [](unsigned char *p, unsigned int v, bool aligned) {
+        if (aligned) *reinterpret_cast<unsigned int *>(p) = v;
+        else for (int k = 0; k < 4; ++k) p[k] = (unsigned char)(v >> (8 * k));
+    };
+    for (int k = tid; k < BAND_OBS_ROWS * GD_OBS_SIZE / 4; k += BAND_THREADS) {
+        const size_t word = (size_t)first_obs_row * GD_OBS_SIZE / 4 + k;
+        const unsigned int grays = gray_words[k];
+        if (out.obs) store_word(out.obs + ((size_t)local * F + word) * 4, grays, (reinterpret_cast<size_t>(out.obs) & 3) == 0);
+        if (!out.frames) continue;
+        unsigned char *stack = out.frames + ((size_t)local * GD_FRAME_STACK * F + word) * 4;
+        unsigned char *copy = out.final_frames ? out.final_frames + ((size_t)local * GD_FRAME_STACK * F + word) * 4 : nullptr;
+        const size_t plane = F * 4;   // bytes per stacked observation
+        if (resets) {
+            for (int f = 0; f < GD_FRAME_STACK; ++f) store_word(stack + f * plane, grays, stack_aligned);
+            if (copy) for (int f = 0; f < GD_FRAME_STACK; ++f) store_word(copy + f * plane, grays, stack_aligned);
+        } else if (out.stack_mode == GD_STACK_STEP) {
+            unsigned int kept[GD_FRAME_STACK];
+            for (int f = 1; f < GD_FRAME_STACK; ++f) kept[f] = load_word(stack + f * plane, stack_aligned);
+            for (int f = 0; f < GD_FRAME_STACK - 1; ++f) store_word(stack + f * plane, kept[f + 1], stack_aligned);
+            store_word(stack + (GD_FRAME_STACK - 1) * plane, grays, stack_aligned);
+            if (copy) {
+                for (int f = 0; f < GD_FRAME_STACK - 1; ++f) store_word(copy + f * plane, kept[f + 1], stack_aligned);
+                store_word(copy + (GD_FRAME_STACK - 1) * plane, grays, stack_aligned);
+            }
+        } else if (copy) {
+            for (int f = 0; f < GD_FRAME_STACK; ++f) store_word(copy + f * plane, load_word(stack + f * plane, stack_aligned), stack_aligned);   // lane left as it was
+        }
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -3661,6 +3956,7 @@ struct gd_renderer {
     DeviceMap dm;
     Scratch sc;
     int chunk_lanes;
+    int assembly;                            // GD_ASSEMBLY_*: how frames are put together after the walls (see launch_chunk)
     unsigned char *scratch_block;            // the one allocation `sc` is laid out in (null for a renderer made for 0 lanes)
     size_t scratch_bytes;
     std::vector<void *> allocations;
@@ -3730,7 +4026,6 @@ size_t carve_scratch(Scratch &sc, unsigned char *base, size_t L, const gd_map_de
     take(&sc.flat_list_count, L);
     take(&sc.meta, L * PX);
     take(&sc.clip_depth, L * PX);
-    take(&sc.frame, L * (size_t)GD_SCREEN_HEIGHT * SW);
     take(&sc.level_reach, L * levels);
     take(&sc.level_far, L * levels);
     take(&sc.level_plane, L * levels * 2);
@@ -3739,7 +4034,10 @@ size_t carve_scratch(Scratch &sc, unsigned char *base, size_t L, const gd_map_de
     take(&sc.block_hit, L * SW);
     take(&sc.strip_key, L * (SW / 64));
     take(&sc.strip_order, L * (SW / 64));
-    if (depth) take(&sc.scene_depth, L * PX);
+    if (depth) {   // frames that draw decals: a scene depth plane, and a frame when the caller wants none
+        take(&sc.scene_depth, L * PX);
+        take(&sc.frame, L * (size_t)GD_SCREEN_HEIGHT * SW);
+    }
     return (used + 255) & ~(size_t)255;
 }
 
@@ -3886,14 +4184,26 @@ const int STAGE_COUNT = 8;
 int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_desc *lanes, const gd_frame_out *out, int base, int count, hipStream_t stream, bool timed) {
     const gd_map_desc &m = r->dm.d;
     Scratch sc = chunk_scratch;
-    unsigned char *frame_base;
-    size_t frame_stride = (size_t)GD_SCREEN_HEIGHT * SW;
-    if (out->indexed) frame_base = out->indexed + (size_t)base * frame_stride;
-    else frame_base = sc.frame;
+    if (out->final_frames && !out->frames) return fail(GD_E_ARG, "final_frames needs frames");
+    const size_t frame_stride = (size_t)GD_SCREEN_HEIGHT * SW;
+    const size_t F = (size_t)GD_OBS_SIZE * GD_OBS_SIZE;
+    const int source_rows = out->obs_source_rows == GD_SCREEN_HEIGHT ? GD_SCREEN_HEIGHT : VH;
     int stage = 0;
     auto mark = [&]() { if (timed) (void)hipEventRecord(r->events[stage], stream); ++stage; };
+    // After the walls and the flat selection a frame is put together in one of two ways.  Kernel by kernel through the
+    // 320x240 frame in device memory (shade, paint the flat pass's pixels, decals, billboards, overlays, then pool the
+    // observation from it): the faster way when the caller wants that frame anyway, and the only one for frames that draw
+    // wall decals, which need a per-pixel scene depth.  Or band by band in LDS (band_finish_kernel), the frame never
+    // reaching device memory: what a caller that only wants observations gets.
     const bool decals = lanes->decal_slots > 0 && lanes->decal_state && lanes->decal_geom && r->overlays.d.decal_variant_count > 0;
     if (!decals) sc.scene_depth = nullptr;
+    if (decals && (!sc.scene_depth || !sc.frame)) return fail(GD_E_ARG, "decal working memory missing");
+    const bool fused = !decals && (r->assembly == GD_ASSEMBLY_FUSED || (r->assembly == GD_ASSEMBLY_AUTO && !out->indexed));
+    unsigned char *frame_base = nullptr;
+    if (!fused) {
+        frame_base = out->indexed ? out->indexed + (size_t)base * frame_stride : sc.frame;
+        if (!frame_base) return fail(GD_E_ARG, "assembling the frame kernel by kernel needs an indexed output");
+    }
     mark();
     hipLaunchKernelGGL(lane_setup_kernel, dim3((count + 63) / 64), dim3(64), 0, stream, r->dm, *lanes, base, count, sc);
     hipLaunchKernelGGL(lane_tables_kernel, dim3(count), dim3(256), 0, stream, r->dm, *lanes, base, count, sc);
@@ -3911,7 +4221,7 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
         hipLaunchKernelGGL(kernel, grid, block, 0, stream, r->dm, count, sc, frame_base, frame_stride);
     }
     mark();
-    {
+    if (!fused) {
         const dim3 grid(((VH * SW + 255) / 256 + SHADE_TILES - 1) / SHADE_TILES, count);
         if (decals) hipLaunchKernelGGL(plane_shade_kernel<true>, grid, dim3(256), 0, stream, r->dm, count, sc, frame_base, frame_stride);
         else hipLaunchKernelGGL(plane_shade_kernel<false>, grid, dim3(256), 0, stream, r->dm, count, sc, frame_base, frame_stride);
@@ -3924,8 +4234,29 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     mark();
     hipLaunchKernelGGL(flat_tail_kernel, dim3(SW / 64, count), dim3(64 * TAIL_ROWS), 0, stream, r->dm, *lanes, base, count, sc);
     hipLaunchKernelGGL(flat_span_finish_kernel, dim3(count), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
-    hipLaunchKernelGGL(flat_shade_kernel, dim3(count), dim3(128), 0, stream, r->dm, count, sc, frame_base, frame_stride);
+    if (!fused) hipLaunchKernelGGL(flat_shade_kernel, dim3(count), dim3(128), 0, stream, r->dm, count, sc, frame_base, frame_stride);
     mark();
+    const float *blend = lanes->screen_blend ? lanes->screen_blend + 2 * (size_t)base : nullptr;
+    if (fused) {
+        FinishOut finish;
+        finish.indexed = out->indexed ? out->indexed + (size_t)base * frame_stride : nullptr;
+        finish.rgb = out->rgb ? out->rgb + (size_t)base * frame_stride * 3 : nullptr;
+        finish.obs = out->obs ? out->obs + (size_t)base * F : nullptr;
+        finish.frames = out->frames ? out->frames + (size_t)base * GD_FRAME_STACK * F : nullptr;
+        finish.final_frames = out->final_frames ? out->final_frames + (size_t)base * GD_FRAME_STACK * F : nullptr;
+        finish.reset_mask = out->reset_mask ? out->reset_mask + base : nullptr;
+        finish.blend = blend;
+        finish.stack_mode = out->stack_mode;
+        finish.source_rows = source_rows;
+        const bool sprites = lanes->sprite_slots > 0 && lanes->sprite_x;
+        size_t shared = sprites ? (size_t)lanes->sprite_slots * (sizeof(SpriteRec) + sizeof(unsigned short)) : 0;
+        if (shared <= (size_t)LDS_SECTORS * sizeof(float4) + 32 * 256) shared = 0;   // the records reuse the shading tables' LDS
+        hipLaunchKernelGGL(band_finish_kernel, dim3(BAND_COUNT, count), dim3(BAND_THREADS), shared, stream, r->dm, r->overlays, *lanes, base, count, sc, finish);
+        mark();
+        mark();
+        HIP_TRY(hipGetLastError());
+        return GD_OK;
+    }
     if (decals)
         hipLaunchKernelGGL(decal_kernel, dim3(count), dim3(SW), 0, stream, r->dm, r->overlays, *lanes, base, count, sc, frame_base, frame_stride);
     if (lanes->sprite_slots > 0 && lanes->sprite_x) {
@@ -3938,22 +4269,18 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     if (lanes->hud_state && r->overlays.d.hud_patch_count > 0)
         hipLaunchKernelGGL(hud_kernel, dim3(count), dim3(256), 0, stream, r->overlays, lanes->hud_state, base, count, frame_base, frame_stride);
     mark();
-    if (out->final_frames && !out->frames) return fail(GD_E_ARG, "final_frames needs frames");
     if (out->obs || out->frames) {
-        const size_t F = (size_t)GD_OBS_SIZE * GD_OBS_SIZE;
         hipLaunchKernelGGL(observe_kernel, dim3(GD_OBS_SIZE / OBS_BLOCK_ROWS, count), dim3(256), 0, stream,
-                           frame_base, frame_stride, out->obs_source_rows == GD_SCREEN_HEIGHT ? GD_SCREEN_HEIGHT : VH, m.playpal, count, out->obs ? out->obs + (size_t)base * F : nullptr,
+                           frame_base, frame_stride, source_rows, m.playpal, count, out->obs ? out->obs + (size_t)base * F : nullptr,
                            out->frames ? out->frames + (size_t)base * GD_FRAME_STACK * F : nullptr,
                            out->reset_mask ? out->reset_mask + base : nullptr, out->stack_mode,
-                           out->final_frames ? out->final_frames + (size_t)base * GD_FRAME_STACK * F : nullptr,
-                           lanes->screen_blend ? lanes->screen_blend + 2 * (size_t)base : nullptr);
+                           out->final_frames ? out->final_frames + (size_t)base * GD_FRAME_STACK * F : nullptr, blend);
     }
     if (out->rgb) {
         size_t pixels = (size_t)count * frame_stride;
         static_assert((GD_SCREEN_HEIGHT * SW) % 256 == 0, "expand_rgb_kernel: one lane per block");
         hipLaunchKernelGGL(expand_rgb_kernel, dim3((unsigned)((pixels + 255) / 256)), dim3(256), 0, stream, frame_base, m.playpal, pixels,
-                           out->rgb + (size_t)base * frame_stride * 3,
-                           lanes->screen_blend ? lanes->screen_blend + 2 * (size_t)base : nullptr, (size_t)GD_SCREEN_HEIGHT * SW);
+                           out->rgb + (size_t)base * frame_stride * 3, blend, (size_t)GD_SCREEN_HEIGHT * SW);
     }
     mark();
     HIP_TRY(hipGetLastError());
@@ -3993,6 +4320,7 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     if (!r) return fail(GD_E_ARG, "out of host memory");
     r->events_ready = false;
     r->scratch_block = nullptr; r->scratch_bytes = 0;
+    r->assembly = GD_ASSEMBLY_AUTO;
     std::memset(&r->sc, 0, sizeof(r->sc));
     std::memset(&r->overlays, 0, sizeof(r->overlays));
     r->dm.d = *h;
@@ -4246,6 +4574,13 @@ int gd_renderer_scribble(gd_renderer *r, int32_t value, void *stream) {
     return GD_OK;
 }
 
+int gd_renderer_set_assembly(gd_renderer *r, int32_t assembly) {
+    if (!r) return fail(GD_E_ARG, "null argument");
+    if (assembly != GD_ASSEMBLY_AUTO && assembly != GD_ASSEMBLY_FUSED && assembly != GD_ASSEMBLY_SEPARATE) return fail(GD_E_ARG, "unknown assembly");
+    r->assembly = assembly;
+    return GD_OK;
+}
+
 int gd_renderer_set_overlays(gd_renderer *r, const gd_overlay_desc *h) {
     if (!r || !h) return fail(GD_E_ARG, "null argument");
     SIZE_CHECK(h, gd_overlay_desc);
@@ -4284,7 +4619,7 @@ int gd_renderer_set_overlays(gd_renderer *r, const gd_overlay_desc *h) {
 #define OV(field, bytes) if (rc == GD_OK) rc = copy(h->field, (bytes), reinterpret_cast<const void **>(&d.field))
     OV(weapon_atlas, wt); OV(weapon_opaque, wt); OV(weapon_w, wp * 4); OV(weapon_h, wp * 4); OV(weapon_left, wp * 4); OV(weapon_top, wp * 4);
     OV(hud_atlas, ht); OV(hud_opaque, ht); OV(hud_w, hp * 4); OV(hud_h, hp * 4); OV(hud_left, hp * 4); OV(hud_top, hp * 4);
-    r->sc.scene_depth = nullptr;
+    r->sc.scene_depth = nullptr; r->sc.frame = nullptr;
     if (h->decal_variant_count == 5) {
         OV(decal_atlas, (size_t)5 * h->decal_max_h * h->decal_max_w); OV(decal_h, 5 * 4); OV(decal_left, 5 * 4); OV(decal_top, 5 * 4);
         OV(decal_opacity_lut, 32 * 256); OV(decal_black_lut, (size_t)h->decal_black_rows * 256);
@@ -4293,12 +4628,17 @@ int gd_renderer_set_overlays(gd_renderer *r, const gd_overlay_desc *h) {
             if (hipMalloc(&ptr, (size_t)(r->chunk_lanes > 0 ? r->chunk_lanes : 1) * VH * SW * sizeof(float)) != hipSuccess) rc = fail(GD_E_HIP, "out of device memory for the decal depth buffer");
             else { r->overlay_allocations.push_back(ptr); r->sc.scene_depth = static_cast<float *>(ptr); }
         }
+        if (rc == GD_OK) {   // and the frame such frames are assembled in when the caller wants no indexed output
+            void *ptr = nullptr;
+            if (hipMalloc(&ptr, (size_t)(r->chunk_lanes > 0 ? r->chunk_lanes : 1) * GD_SCREEN_HEIGHT * SW) != hipSuccess) rc = fail(GD_E_HIP, "out of device memory for the decal frame buffer");
+            else { r->overlay_allocations.push_back(ptr); r->sc.frame = static_cast<unsigned char *>(ptr); }
+        }
     }
 #undef OV
     if (rc != GD_OK) {
         for (void *ptr : r->overlay_allocations) (void)hipFree(ptr);
         r->overlay_allocations.clear();
-        r->sc.scene_depth = nullptr;
+        r->sc.scene_depth = nullptr; r->sc.frame = nullptr;
         return rc;
     }
     r->overlays.d = d;

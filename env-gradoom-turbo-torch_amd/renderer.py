@@ -132,6 +132,16 @@ class HipRenderer:
         _lib.check(self._lib.gd_renderer_status(self._handle, C.byref(value)))
         return int(value.value)
 
+    def set_assembly(self, assembly: str) -> None:
+        """``"auto"`` (fused when a call wants no indexed frame, else separate), ``"fused"`` (every frame is put together
+        band by band in LDS and never reaches device memory unless asked for) or ``"separate"`` (kernel by kernel through
+        the frame in device memory).  Both give the same bytes."""
+
+        codes = {"auto": 0, "fused": 1, "separate": 2}
+        if assembly not in codes:
+            raise ValueError("assembly must be 'auto', 'fused' or 'separate'")
+        _lib.check(self._lib.gd_renderer_set_assembly(self._handle, codes[assembly]))
+
     def scribble(self, value: int) -> None:
         """Fill the working memory with one byte value (diagnostic: later frames must not depend on it)."""
 

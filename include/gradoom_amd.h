@@ -283,6 +283,20 @@ int gd_render_static(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_
 int gd_renderer_status(gd_renderer *r, int32_t *status);
 
 /*
+ * How a frame is put together once the walls are traversed.  GD_ASSEMBLY_SEPARATE: kernel by kernel through the
+ * 320x240 frame in device memory (needs gd_frame_out.indexed).  GD_ASSEMBLY_FUSED: band by band in LDS, where
+ * shading, billboards, overlays, PLAYPAL expansion, pooling and the stack update all happen; the frame only goes to
+ * device memory if the caller asks for it.  GD_ASSEMBLY_AUTO (the default): fused when the call wants no `indexed`
+ * frame (observations only: no 320x240 frame is ever written), separate otherwise, which measures faster when the
+ * frame has to be written anyway.  Frames that draw wall decals are always assembled separately.
+ * Both give the same bytes.  Replaces nothing in the reference.
+ */
+#define GD_ASSEMBLY_AUTO 0
+#define GD_ASSEMBLY_FUSED 1
+#define GD_ASSEMBLY_SEPARATE 2
+int gd_renderer_set_assembly(gd_renderer *r, int32_t assembly);
+
+/*
  * Fill the renderer's working memory with one byte value, asynchronously on `stream` (diagnostic: the frames
  * that follow must not depend on what the memory held before).  Replaces nothing in the reference.
  */

@@ -30,7 +30,12 @@ def test_indexed_frame_bit_exact_vs_reference_golden(name):
     count = meta["lanes"]
     indexed = torch.zeros((count, 240, 320), dtype=torch.uint8, device="cuda:0")
     obs = torch.zeros((count, 84, 84), dtype=torch.uint8, device="cuda:0")
-    for fill in (None, 0xFF):   # fresh working memory, then the same memory filled with ones: nothing is cleared between frames
+    # both ways of putting a frame together (kernel by kernel through device memory; band by band in LDS), the second one
+    # into working memory filled with ones: nothing is cleared between frames
+    for assembly, fill in (("separate", None), ("fused", 0xFF)):
+        if meta.get("decals") and assembly == "fused":
+            continue   # frames with wall decals are always assembled kernel by kernel
+        renderer.set_assembly(assembly)
         if fill is not None:
             renderer.scribble(fill)
             indexed.zero_()
@@ -40,7 +45,7 @@ def test_indexed_frame_bit_exact_vs_reference_golden(name):
         assert renderer.status() == 0
         ours = indexed.cpu().numpy()
         mismatched = int((ours != data["indexed"]).sum())
-        assert mismatched == 0, f"{mismatched} palette indices differ from the reference (working memory fill {fill})"
+        assert mismatched == 0, f"{mismatched} palette indices differ from the reference ({assembly} assembly, working memory fill {fill})"
         delta = np.abs(obs.cpu().numpy().astype(np.int32) - data["obs"].astype(np.int32))
         assert delta.max() <= 1 and delta.mean() < 0.01  # tolerance: tests/test_rendering.py:138-139
     renderer.close()
@@ -58,15 +63,20 @@ def test_observation_and_stack_bit_exact_vs_oracle(oracle, name):
     obs = torch.zeros((count, 84, 84), dtype=torch.uint8, device="cuda:0")
     frames = torch.as_tensor(start).to("cuda:0")
     rgb = torch.zeros((count, 240, 320, 3), dtype=torch.uint8, device="cuda:0")
-    renderer.render(lanes, indexed=indexed, obs=obs, frames=frames, reset_mask=torch.as_tensor(mask).to("cuda:0"), rgb=rgb)
-    torch.cuda.synchronize()
-    assert np.array_equal(indexed.cpu().numpy(), expected["indexed"])
-    assert np.array_equal(obs.cpu().numpy(), expected["obs"])
-    assert np.array_equal(frames.cpu().numpy(), expected["frames"])
-    assert np.array_equal(rgb.cpu().numpy(), expected["rgb"])
-    assert np.array_equal(rgb[0].cpu().numpy(), data["rgb_lane0"])
-    if "rgb_all" in data:   # the case with per-lane screen blends carries every lane's reference RGB24 frame
-        assert np.array_equal(rgb.cpu().numpy(), data["rgb_all"][:count])
+    for assembly in ("separate", "fused"):
+        renderer.set_assembly(assembly)
+        frames = torch.as_tensor(start).to("cuda:0")
+        for tensor in (indexed, obs, rgb):
+            tensor.zero_()
+        renderer.render(lanes, indexed=indexed, obs=obs, frames=frames, reset_mask=torch.as_tensor(mask).to("cuda:0"), rgb=rgb)
+        torch.cuda.synchronize()
+        assert np.array_equal(indexed.cpu().numpy(), expected["indexed"]), assembly
+        assert np.array_equal(obs.cpu().numpy(), expected["obs"]), assembly
+        assert np.array_equal(frames.cpu().numpy(), expected["frames"]), assembly
+        assert np.array_equal(rgb.cpu().numpy(), expected["rgb"]), assembly
+        assert np.array_equal(rgb[0].cpu().numpy(), data["rgb_lane0"])
+        if "rgb_all" in data:   # the case with per-lane screen blends carries every lane's reference RGB24 frame
+            assert np.array_equal(rgb.cpu().numpy(), data["rgb_all"][:count])
     renderer.close()
 
 
@@ -126,11 +136,16 @@ def test_final_frames_and_stack_modes_match_the_oracle(oracle):
     ):
         print(f"stack mode {mode}", flush=True)
         expected = oracle.render(tables, lane_inputs(data), data["cosine_correction"], frames=start, **oracle_kwargs)
+        # without a frame to hand out the call is assembled in LDS; with one, kernel by kernel: both must roll alike
+        scratch_frame = torch.zeros((count, 240, 320), dtype=torch.uint8, device="cuda:0")
+        separate = torch.as_tensor(start).to("cuda:0")
+        renderer.render(lanes, frames=separate, indexed=scratch_frame, **kwargs)
         frames = torch.as_tensor(start).to("cuda:0")
         final = torch.full((count, 4, 84, 84), 7, dtype=torch.uint8, device="cuda:0")
         obs = torch.zeros((count, 84, 84), dtype=torch.uint8, device="cuda:0")
         renderer.render(lanes, frames=frames, final_frames=final, obs=obs, **kwargs)
         torch.cuda.synchronize()
+        assert torch.equal(frames, separate), mode
         ours = frames.cpu().numpy()
         assert np.array_equal(ours, expected["frames"]), mode
         assert np.array_equal(final.cpu().numpy(), expected["frames"]), mode
@@ -180,6 +195,10 @@ def test_status_bar_rows_pooled_into_the_observation(oracle):
     delta = np.abs(obs.cpu().numpy().astype(np.int32) - data["obs_with_hud"].astype(np.int32))
     assert delta.max() <= 1 and delta.mean() < 0.01
     assert torch.equal(obs, again)
+    fused = torch.zeros_like(obs)
+    renderer.render(lanes, obs=fused, obs_source_rows=240)   # no frame asked for: weapon, status bar and pooling all in LDS
+    torch.cuda.synchronize()
+    assert torch.equal(obs, fused)
     oracle.set_overlays(fixture_overlays(meta))
     try:
         expected = oracle.render(tables, lane_inputs(data), data["cosine_correction"], obs_source_rows=240)

@@ -55,11 +55,15 @@ def test_random_maps_and_grazing_poses_match_the_oracle(oracle, first_seed):
         renderer = HipRenderer(smap, LANES, "cuda:0", cosine_correction=cosine, tables=tables)
         indexed = torch.zeros((LANES, 240, 320), dtype=torch.uint8, device="cuda:0")
         obs = torch.zeros((LANES, 84, 84), dtype=torch.uint8, device="cuda:0")
-        renderer.render(LaneState.from_numpy(arrays, "cuda:0"), indexed=indexed, obs=obs)
+        state = LaneState.from_numpy(arrays, "cuda:0")
+        renderer.render(state, indexed=indexed, obs=obs)
+        fused_obs = torch.zeros_like(obs)
+        renderer.render(state, obs=fused_obs)   # observations only: assembled in LDS
         torch.cuda.synchronize()
         assert renderer.status() == 0
         assert np.array_equal(indexed.cpu().numpy(), expected["indexed"]), f"seed {seed}"
         assert np.array_equal(obs.cpu().numpy(), expected["obs"]), f"seed {seed}"
+        assert torch.equal(fused_obs, obs), f"seed {seed}"
         renderer.close()
 
 
@@ -89,7 +93,8 @@ def test_random_maps_with_other_heights_and_textures_whatever_the_working_memory
         expected = oracle.render(tables, arrays, cosine)
         renderer = HipRenderer(smap, LANES, "cuda:0", cosine_correction=cosine, tables=tables)
         lanes = LaneState.from_numpy(arrays, "cuda:0")
-        for fill in (None, 0xFF, 0xA5):
+        for fill, assembly in ((None, "separate"), (0xFF, "fused"), (0xA5, "separate"), (0x5A, "fused")):
+            renderer.set_assembly(assembly)
             if fill is not None:
                 renderer.scribble(fill)
             indexed = torch.zeros((LANES, 240, 320), dtype=torch.uint8, device="cuda:0")
@@ -97,8 +102,8 @@ def test_random_maps_with_other_heights_and_textures_whatever_the_working_memory
             renderer.render(lanes, indexed=indexed, obs=obs)
             torch.cuda.synchronize()
             assert renderer.status() == 0
-            assert np.array_equal(indexed.cpu().numpy(), expected["indexed"]), f"seed {seed} fill {fill}"
-            assert np.array_equal(obs.cpu().numpy(), expected["obs"]), f"seed {seed} fill {fill}"
+            assert np.array_equal(indexed.cpu().numpy(), expected["indexed"]), f"seed {seed} fill {fill} {assembly}"
+            assert np.array_equal(obs.cpu().numpy(), expected["obs"]), f"seed {seed} fill {fill} {assembly}"
         renderer.close()
 
 
