@@ -49,6 +49,8 @@ typedef unsigned long long u64;
 #define SW 320
 #define VH 208
 #define CAND_MAX 64          // candidate linedefs kept per screen column
+#define SEG_COLS 64           // columns of a traversal segment; a wavefront takes 64 / SEG_COLS segments, of any lanes
+#define SEGS_PER_LANE (SW / SEG_COLS)
 #define GD_INF __builtin_inff()
 
 // engine.py:42-51, 139-156
@@ -174,8 +176,8 @@ struct Scratch {    // per-chunk working memory, sized at create
     unsigned char *frame;  // [L,240,320] when the caller wants no indexed output
     u64 *block_hit;        // [L,320] nearest blocking linedef of the column ray: float bits of the distance << 32 |
                            // slot in blocking_walls, all ones when no ray hits (engine.py:10534-10557)
-    unsigned char *strip_key;  // [L*5] expected traversal length of each (lane, 64-column strip)
-    int *strip_order;      // [L*5] strips, longest expected traversal first
+    unsigned char *strip_key;  // [L*SEGS_PER_LANE] expected traversal length of each (lane, segment of SEG_COLS columns)
+    int *strip_order;      // [L*SEGS_PER_LANE] segments, longest expected traversal first
     int *status;           // [1] sticky overflow flags
     float *level_reach;    // [L, floor levels + ceiling levels] lower bound of the distance from the
                            // camera to any point inside a sector with that plane level
@@ -1517,16 +1519,18 @@ struct ColumnCtx {
     const gd_map_desc *m;
     MapView mv;
     const LaneCtx *c;
-    const WallRec *recs;
-    const RecSpan *spans; // this lane's ray-test facts of every linedef
+    const WallRec *recs;  // the chunk's [L,W] records, with rec_base = lane * W
+    const RecSpan *spans; // the chunk's [L,W] ray-test facts of every linedef
     const WallRec *frags; // this lane's [split_count, fragment_slots] fragment records
-    const Cand *list;     // this lane's candidate block, entry k of column x at [k*320 + x]
+    const Cand *list;     // the chunk's candidate blocks; entry k of this column sits list_column + k * 320 * 16 bytes in
+    unsigned rec_base, list_column;
     int count;
     int x;
     float rx, ry;
+    __device__ __forceinline__ const WallRec &rec(int w) const { return recs[rec_base + (unsigned)w]; }
     __device__ __forceinline__ Cand cand(int k) const {
         union { uint4 raw; Cand c; } u;
-        u.raw = *reinterpret_cast<const uint4 *>(list + (size_t)k * SW + x);   // one 16-byte load
+        u.raw = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(list) + (list_column + (unsigned)k * (SW * 16u)));   // one 16-byte load
         return u.c;
     }
     // Entries k0 .. k0+CAND_BATCH-1 of this column's list, loaded together so that their memory
@@ -1546,7 +1550,7 @@ struct ColumnCtx {
 #pragma unroll
         for (int j = 0; j < CAND_BATCH; ++j) out[j] = cand(at[j] < 0 ? 0 : at[j]);
     }
-    __device__ Eval eval(int w) const { return eval_wall(m, *c, spans, x, w, rx, ry); }
+    __device__ Eval eval(int w) const { return eval_wall(m, *c, spans + rec_base, x, w, rx, ry); }
 };
 
 // The projection fragment of a linedef at one column (engine.py:11511-11529, 12324-12376): the first
@@ -1693,7 +1697,7 @@ __device__ __forceinline__ i64 wall_shade(float light, i64 visibility) {
 __device__ __forceinline__ void endpoint_owner(const ColumnCtx &cc, int w, const Eval &cw, int *owner_index, float *owner_distance) {
     const gd_map_desc *m = cc.m;
     const int K = m->neighbor_slots;
-    const bool subpixel = cc.spans[w].flags & WF_SUBPIXEL;
+    const bool subpixel = cc.spans[cc.rec_base + (unsigned)w].flags & WF_SUBPIXEL;
     float tol_w = tolerance_of(cw.dist);
     // the owner only matters for a linedef that does not own this column itself (engine.py:11716)
     if (cw.flags & CF_PROJ) { *owner_index = w; *owner_distance = cw.dist; return; }
@@ -1734,17 +1738,6 @@ __device__ __forceinline__ void endpoint_owner(const ColumnCtx &cc, int w, const
     *owner_distance = has ? distance : cw.dist;
 }
 
-#ifdef GD_PROFILE
-__device__ unsigned long long g_profile[16];
-__device__ unsigned int g_wave_log[3 * 32768];   // per strip: clock ticks, candidate total, passes
-#define PROF_T(var) long long var = wall_clock64()
-#define PROF_ADD(slot, t0, t1) prof_acc[slot] += (t1) - (t0)
-#define PROF_MARK(slot, tprev) do { long long tn_ = wall_clock64(); if (threadIdx.x == 0) atomicAdd(&g_profile[slot], (unsigned long long)(tn_ - tprev)); tprev = tn_; } while (0)
-#else
-#define PROF_T(var)
-#define PROF_ADD(slot, t0, t1)
-#define PROF_MARK(slot, tprev)
-#endif
 
 struct ColumnState {   // engine.py:11561-11580, 11735-11762
     int current_sector;
@@ -1816,9 +1809,6 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
     const float prev_eps = prev + 1e-3f;
     auto incident = [&](int w) { return mv.sec(w, 0) == cur || mv.sec(w, 1) == cur; };
     auto incident_c = [&](const Cand &q) { return q.s0 == cur || q.s1 == cur; };
-#ifdef GD_PROFILE
-    long long tsub = wall_clock64();
-#endif
     // a. nearest incident linedef beyond previous_distance (engine.py:11769-11780)
     float distance = GD_INF; int wi = 0x7fffffff;
     Eval cwi;
@@ -1848,7 +1838,6 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
         cwi.dist = distance; cwi.flags = wi_flags;
     }
     if (!finitef(distance)) { wi = 0; cwi = cc.eval(0); }
-    PROF_MARK(8, tsub);
     // c. selected endpoint (engine.py:11815-11871)
     bool sel_start = !(cwi.flags & CF_ALONG_HI);
     int sel_vertex = mv.vert(wi, sel_start ? 0 : 1);
@@ -1863,7 +1852,7 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
         pend_ep_has_forward_bridge = cc.eval(fb_idx).dist > distance + 1e-3f;
     bool completes_pending_endpoint_bridge = (c.flags & ST_EB) && (wi == c.pend_eb_index);
     bool sel_is_proj = cwi.flags & CF_PROJ;
-    bool sel_excl_right = cc.recs[wi].sr == x;
+    bool sel_excl_right = cc.rec(wi).sr == x;
     // d. projected solid owner (engine.py:11872-11954)
     float ps_path_distance = distance; int ps_path_index = wi;
     bool ps_path_geo = cwi.flags & CF_GEO;
@@ -1897,7 +1886,6 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
     }
     bool has_ps = finitef(psd);
     if (has_ps) { distance = psd; wi = psi; cwi.dist = psd; cwi.flags = psi_flags; }
-    PROF_MARK(9, tsub);
     // e. endpoint owner (engine.py:11960-12001)
     int eo_idx; float eo_dist;
     endpoint_owner(cc, wi, cwi, &eo_idx, &eo_dist);
@@ -1910,7 +1898,7 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
     int no_path_other = no_from_front ? mv.sec(no_path_index, 1) : mv.sec(no_path_index, 0);
     // f. near projected owner (engine.py:12002-12179)
     bool so_is_proj = cwi.flags & CF_PROJ;
-    const WallRec &so_rec = cc.recs[wi];
+    const WallRec &so_rec = cc.rec(wi);
     bool so_excl_right = so_rec.sr == x;
     i64 so_span = so_rec.sr - so_rec.sl;
     bool so_short = m->wall_len[wi] <= 32.0f;
@@ -1943,7 +1931,7 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
     int pe_other = pe_from_current ? pe_s1 : pe_s0;
     bool use_psb = false; int psb_idx = 0;
     if ((c.flags & ST_EP) && pe_incident && (pe_other >= 0) && (no_path_other >= 0) && no_path_geo && !so_is_proj && so_excl_right &&
-        (cc.recs[pe_wall].sr - cc.recs[pe_wall].sl <= 1)) {
+        (cc.rec(pe_wall).sr - cc.rec(pe_wall).sl <= 1)) {
         int pe_slot = (c.pend_ep_vertex == mv.vert(pe_wall, 1)) ? 1 : 0;
         bool psb_exists = mv.sector_bridge(pe_slot, pe_wall, no_path_index, &psb_idx);
         if (psb_exists) {
@@ -1959,7 +1947,6 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
     if (replace_np) { distance = npd; wi = npi; cwi.dist = npd; cwi.flags = npi_flags; }
     bool final_proj = cwi.flags & CF_PROJ, final_geo = cwi.flags & CF_GEO;
     bool completes_poab = (c.flags & ST_EP) && final_proj && !final_geo && mv.opposing(pe_wall, wi);
-    PROF_MARK(10, tsub);
     // g. validity (engine.py:12197-12239)
     bool valid = finitef(distance);
     bool excl_only = !so_is_proj && so_excl_right && !replace_np && (so_span <= 2) && !boundary_has_po;
@@ -1983,14 +1970,13 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
 
     r.wall = wi; r.side = side; r.render_current = render_current; r.other_sector = other_sector;
     r.distance = distance;
-    const WallRec &wr = cc.recs[wi];
+    const WallRec &wr = cc.rec(wi);
     const FragmentChoice wr_fragment = choose_fragment<SPLIT>(m, cc.frags, wr, wi, x);
     r.visibility = wall_visibility(wr_fragment.lights ? *wr_fragment.rec : wr, side, x);
     const Tables &tb = *cc.tb;
     r.view_floor = tb.floor_h(render_current); r.view_ceiling = tb.ceil_h(render_current);
     r.other_floor = tb.floor_h(safe_other); r.other_ceiling = tb.ceil_h(safe_other);
     for (int t = 0; t < 3; ++t) r.side_tex[t] = m->side_tex[(wi * 2 + side) * 3 + t];
-    PROF_MARK(11, tsub);
     // j. projection and clipping (engine.py:12607-12620)
     float one_top = 0, one_bottom = 0, lower_top = 0, upper_bottom = 0;
     // one copy of the projection code, four heights; the back sector's two only matter across a
@@ -2006,7 +1992,6 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
     r.clipped_bottom = fminf(one_bottom, c.floor_clip);
     r.clipped_upper_bottom = fmaxf(fminf(upper_bottom, c.floor_clip), r.clipped_top);
     r.clipped_lower_top = fminf(fmaxf(lower_top, c.ceiling_clip), r.clipped_bottom);
-    PROF_MARK(12, tsub);
     // k. plane marks (engine.py:12621-12636)
     bool light_differs = tb.light(render_current) != tb.light(safe_other);
     bool mark_ceiling = one_sided || (r.view_ceiling != r.other_ceiling) || (tb.ceil_tex(render_current) != tb.ceil_tex(safe_other)) || light_differs;
@@ -2023,11 +2008,20 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
              (pend_ep_has_forward_bridge ? PB_FORWARD_BRIDGE : 0) | ((cwi.flags & CF_ALONG_HI) ? PB_FINAL_ALONG_HI : 0);
 }
 
+// The per-pixel planes of a chunk of lanes and one column's place in them.  The wavefronts of the traversal hold columns of
+// several lanes, so the planes' base pointers are the same for all of them and each column keeps byte offsets: a chunk
+// is at most 4096 lanes, which keeps every offset below 4 GiB.
 struct PixelBuffers {
-    unsigned char *frame;   // [240][320]
-    unsigned int *meta;     // [208][320]
-    float *clip_depth;      // [208][320], only meaningful where the meta word names a clip linedef
-    float *scene_depth;     // [208][320] or null
+    unsigned char *frame;   // [L][240][320] or null
+    unsigned int *meta;     // [L][208][320]
+    float *clip_depth;      // [L][208][320], only meaningful where the meta word names a clip linedef
+    float *scene_depth;     // [L][208][320] or null
+    unsigned word_column;   // byte offset of (lane, row 0, column) in the four-byte planes
+    unsigned frame_column;  // and in the frame
+    __device__ __forceinline__ unsigned int &m(int y) const { return *reinterpret_cast<unsigned int *>(reinterpret_cast<char *>(meta) + (word_column + (unsigned)y * (SW * 4u))); }
+    __device__ __forceinline__ float &d(int y) const { return *reinterpret_cast<float *>(reinterpret_cast<char *>(clip_depth) + (word_column + (unsigned)y * (SW * 4u))); }
+    __device__ __forceinline__ float &s(int y) const { return *reinterpret_cast<float *>(reinterpret_cast<char *>(scene_depth) + (word_column + (unsigned)y * (SW * 4u))); }
+    __device__ __forceinline__ unsigned char &f(int y) const { return frame[frame_column + (unsigned)y * (unsigned)SW]; }
 };
 
 // Silhouette bookkeeping: every row >= bot_row holds a clip depth <= bot_depth, every row
@@ -2045,8 +2039,8 @@ __device__ __forceinline__ void clip_rows(PixelBuffers &pb, int x, int first, in
     auto load_rows = [&](int y0, float (&held)[WALL_ROWS], unsigned int (&meta)[WALL_ROWS]) {
 #pragma unroll
         for (int j = 0; j < WALL_ROWS; ++j) {
-            const size_t i = (size_t)(y0 + j < last ? y0 + j : last - 1) * SW + x;
-            held[j] = pb.clip_depth[i]; meta[j] = pb.meta[i];
+            const int y = y0 + j < last ? y0 + j : last - 1;
+            held[j] = pb.d(y); meta[j] = pb.m(y);
         }
     };
     float held[WALL_ROWS]; unsigned int meta[WALL_ROWS];
@@ -2060,8 +2054,7 @@ __device__ __forceinline__ void clip_rows(PixelBuffers &pb, int x, int first, in
         for (int j = 0; j < WALL_ROWS; ++j) {
             const float depth = (meta[j] & META_WALL_MASK) ? held[j] : GD_INF;   // no clip recorded yet: infinite
             if (y0 + j >= last || !(distance < depth)) continue;
-            const size_t i = (size_t)(y0 + j) * SW + x;
-            pb.clip_depth[i] = distance; pb.meta[i] = (meta[j] & ~META_WALL_MASK) | (unsigned)(wall + 1);
+            pb.d(y0 + j) = distance; pb.m(y0 + j) = (meta[j] & ~META_WALL_MASK) | (unsigned)(wall + 1);
         }
 #pragma unroll
         for (int j = 0; j < WALL_ROWS; ++j) { held[j] = next_held[j]; meta[j] = next_meta[j]; }
@@ -2101,14 +2094,25 @@ __device__ __forceinline__ bool silhouette_folds(const PassColumn &r) {
 // column ends.  Rows that received such a zero are the only ones that can end up without an owner: the column keeps
 // their range and lists the ownerless ones as gap pixels for the flat pass.
 struct GapRange {
-    int lo, hi;   // rows [lo, hi) hold every zero this column wrote
+    // Four row numbers (0..VH, VH < 256) in one register: the traversal holds them for the whole column.
+    //   bits 0-7 lo, 8-15 hi: rows [lo, hi) hold every zero this column wrote
+    //   bits 16-23 filled_lo, 24-31 filled_hi: rows [filled_lo, filled_hi) are known to hold wall tier pixels
+    //   (the one-sided drawseg's own)
+    unsigned int rows;
+    __device__ __forceinline__ int lo() const { return (int)(rows & 255u); }
+    __device__ __forceinline__ int hi() const { return (int)((rows >> 8) & 255u); }
+    __device__ __forceinline__ int filled_lo() const { return (int)((rows >> 16) & 255u); }
+    __device__ __forceinline__ int filled_hi() const { return (int)(rows >> 24); }
+    __device__ __forceinline__ void reset() { rows = (unsigned)VH; }
+    __device__ __forceinline__ void set_zeroed(int lo, int hi) { rows = (rows & 0xffff0000u) | (unsigned)lo | ((unsigned)hi << 8); }
+    __device__ __forceinline__ void set_filled(int lo, int hi) { rows = (rows & 0x0000ffffu) | ((unsigned)lo << 16) | ((unsigned)hi << 24); }
 };
+static_assert(VH < 256, "GapRange packs row numbers into bytes");
 __device__ __forceinline__ void zero_rows(PixelBuffers &pb, GapRange &gaps, int x, int first, int last) {
     first = first < 0 ? 0 : first; last = last > VH ? VH : last;
     if (first >= last) return;
-    for (int y = first; y < last; ++y) pb.meta[(size_t)y * SW + x] = 0u;
-    gaps.lo = first < gaps.lo ? first : gaps.lo;
-    gaps.hi = last > gaps.hi ? last : gaps.hi;
+    for (int y = first; y < last; ++y) pb.m(y) = 0u;
+    gaps.set_zeroed(min(first, gaps.lo()), max(last, gaps.hi()));
 }
 
 // engine.py:12637-12884
@@ -2130,10 +2134,10 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
     const float floor_plane_top = fmaxf(r.clipped_bottom, c.ceiling_clip);
     const float *toff = m->side_off + (wi * 2 + side) * 2;
     i64 h, swall;
-    texture_mapping(m, cc.recs[wi], wi, x, &h, &swall);
+    texture_mapping(m, cc.rec(wi), wi, x, &h, &swall);
     i64 repeat = round_to_i64(m->wall_len[wi] * 65536.0f);
     if (side != 0) h = repeat - h;
-    if (cc.recs[wi].sl > 0 && h < 0) h = 0;
+    if (cc.rec(wi).sl > 0 && h < 0) h = 0;
     if (h >= repeat) h = repeat - 1;
     i64 offx_fixed = round_to_i64(toff[0] * 65536.0f);
     i64 u_base = (h + offx_fixed) >> 16;
@@ -2170,8 +2174,8 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
                 const int e = (int)ceiling_plane_bottom;
                 const unsigned word = (claims ? claim : 0u) | (sil_top ? clip_word : 0u);
                 for (int y = y0 < 0 ? 0 : y0; y < e; ++y) {
-                    pb.meta[(size_t)y * SW + x] = word;
-                    if (sil_top) pb.clip_depth[(size_t)y * SW + x] = r.distance;
+                    pb.m(y) = word;
+                    if (sil_top) pb.d(y) = r.distance;
                 }
             }
         }
@@ -2182,8 +2186,8 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
                 const int b = (int)floor_plane_top;
                 const unsigned word = (claims ? (claim | META_FLOOR) : 0u) | (sil_bottom ? clip_word : 0u);
                 for (int y = b < 0 ? 0 : b; y < y1; ++y) {
-                    pb.meta[(size_t)y * SW + x] = word;
-                    if (sil_bottom) pb.clip_depth[(size_t)y * SW + x] = r.distance;
+                    pb.m(y) = word;
+                    if (sil_bottom) pb.d(y) = r.distance;
                 }
             }
         }
@@ -2251,23 +2255,43 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
 #pragma unroll
             for (int j = 0; j < WALL_ROWS; ++j) {
                 if (!(draw & (1u << j))) continue;
-                const size_t i = (size_t)(yb + j) * SW + x;
                 const unsigned colour = colormap[((tail & (1u << j)) ? shade_group : shade_own) * 256 + texel[j]];
-                pb.clip_depth[i] = r.distance;
-                if (DEPTH) pb.scene_depth[i] = r.distance;
-                pb.meta[i] = META_FILLED | (colour << META_SECTOR_SHIFT) | (unsigned)(wi + 1);
+                pb.d(yb + j) = r.distance;
+                if (DEPTH) pb.s(yb + j) = r.distance;
+                pb.m(yb + j) = META_FILLED | (colour << META_SECTOR_SHIFT) | (unsigned)(wi + 1);
             }
 #pragma unroll
             for (int j = 0; j < WALL_ROWS; ++j) texel[j] = next_texel[j];
             draw = next_draw; tail = next_tail;
         }
-        if (one_sided) window_dirty = true;
+        if (one_sided) {
+            window_dirty = true;
+            if (r.side_tex[0] >= 0 && t0 < t1) gaps.set_filled(max(t0, 0), min(t1, VH));   // every row of [t0, t1) was drawn just now
+        }
         return;
     }
-    for (int y = y0; y < y1; ++y) {
+    // A one-sided drawseg has painted this window.  Every row of it has been written since (GapRange), so what a later pass
+    // can still change is narrow: a tier pixel where no tier was drawn yet, which can only lie in this pass's own tier rows
+    // and outside the rows that drawseg filled, and a plane claim on a row nobody owns, which can only be one of the rows
+    // this column had to zero.  Only those rows are visited (usually none).  Few columns come here (one pass in 300 on the
+    // 4000-linedef map) but every eighth wavefront pass has one, so the loop is kept plain and light on registers.
+    int lo = VH, hi = 0;
+    if (one_sided) { lo = (int)r.clipped_top; hi = (int)r.clipped_bottom; }
+    if (lower_on) { lo = min(lo, (int)r.clipped_lower_top); hi = max(hi, (int)r.clipped_bottom); }
+    if (upper_on) { lo = min(lo, (int)r.clipped_top); hi = max(hi, (int)r.clipped_upper_bottom); }
+    if (gaps.lo() < gaps.hi()) { lo = min(lo, gaps.lo()); hi = max(hi, gaps.hi()); }
+    lo = max(lo, y0); hi = min(hi, y1);
+    const int filled_lo = gaps.filled_lo(), filled_hi = gaps.filled_hi();
+    // copies taken by value: a choice between members of `r` made per row would be a choice between addresses and
+    // would keep the whole record in private memory
+    const int side_tex0 = r.side_tex[0], side_tex1 = r.side_tex[1], side_tex2 = r.side_tex[2];
+    const float origin0 = r.view_ceiling, origin1 = r.other_floor, origin2 = r.other_ceiling;
+    const bool tail0 = group_valid[0], tail1 = group_valid[1], tail2 = group_valid[2];
+    const float tail_row0 = group_bottom[0], tail_row1 = group_bottom[1], tail_row2 = group_bottom[2];
+    for (int y = lo; y < hi; ++y) {
+        if (y >= filled_lo && y < filled_hi) { y = filled_hi - 1; continue; }   // tier pixels already: nothing to add
         const float py = (float)y;
-        const size_t i = (size_t)y * SW + x;
-        unsigned int meta = pb.meta[i];
+        unsigned int meta = pb.m(y);
         bool ceiling_span = (r.bits & PB_MARK_CEILING) && (py >= c.ceiling_clip) && (py < ceiling_plane_bottom);
         bool floor_span = (r.bits & PB_MARK_FLOOR) && (py >= floor_plane_top) && (py < c.floor_clip);
         bool meta_dirty = false;
@@ -2279,13 +2303,13 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
         bool lower_span = lower_on && (py >= r.clipped_lower_top) && (py < r.clipped_bottom);
         bool upper_span = upper_on && (py >= r.clipped_top) && (py < r.clipped_upper_bottom);
         if (one_span || lower_span || upper_span) {
-            int texture_id = one_span ? r.side_tex[0] : (lower_span ? r.side_tex[1] : r.side_tex[2]);
+            int texture_id = one_span ? side_tex0 : (lower_span ? side_tex1 : side_tex2);
             if (texture_id >= 0 && !(meta & META_FILLED)) {
-                bool bottom_tail = (one_span && group_valid[0] && py >= group_bottom[0]) ||
-                                   (lower_span && group_valid[1] && py >= group_bottom[1]) ||
-                                   (upper_span && group_valid[2] && py >= group_bottom[2]);
+                bool bottom_tail = (one_span && tail0 && py >= tail_row0) ||
+                                   (lower_span && tail1 && py >= tail_row1) ||
+                                   (upper_span && tail2 && py >= tail_row2);
                 i64 tu = tb.wrap_column(texture_id, u_base);
-                float origin_z = one_span ? r.view_ceiling : (lower_span ? r.other_floor : r.other_ceiling);
+                float origin_z = one_span ? origin0 : (lower_span ? origin1 : origin2);
                 int height_bits = tb.height_bits(texture_id);
                 i64 vertical_step = mul64(swall, shl64(1, 14 - height_bits));
                 i64 screen_delta = (i64)y * FIXED_UNIT - L.center_fixed + FIXED_UNIT;
@@ -2294,14 +2318,14 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
                 i64 tv = (fraction & UINT32_MASK) >> (32 - height_bits);
                 unsigned char texel = m->tex_atlas[((size_t)texture_id * m->tex_max_h + tv) * m->tex_max_w + tu];
                 const unsigned colour = colormap[(bottom_tail ? shade_group : shade_own) * 256 + texel];
-                if (DEPTH) pb.scene_depth[i] = r.distance;
-                const float held = (meta & META_WALL_MASK) ? pb.clip_depth[i] : GD_INF;   // no clip recorded yet
-                if (r.distance < held) { pb.clip_depth[i] = r.distance; meta = (meta & ~META_WALL_MASK) | (unsigned)(wi + 1); }
+                if (DEPTH) pb.s(y) = r.distance;
+                const float held = (meta & META_WALL_MASK) ? pb.d(y) : GD_INF;   // no clip recorded yet
+                if (r.distance < held) { pb.d(y) = r.distance; meta = (meta & ~META_WALL_MASK) | (unsigned)(wi + 1); }
                 meta = (meta & ~(META_SECTOR_MASK << META_SECTOR_SHIFT)) | (colour << META_SECTOR_SHIFT) | META_FILLED;
                 meta_dirty = true;
             }
         }
-        if (meta_dirty) pb.meta[i] = meta;
+        if (meta_dirty) pb.m(y) = meta;
     }
 }
 
@@ -2348,7 +2372,7 @@ __device__ __forceinline__ bool pass_advance(const ColumnCtx &cc, ColumnState &c
     // r. clips of the geometric portal behind a projected solid (engine.py:12969-13069)
     if (r.bits & PB_PS_KEEPS) {
         int path = r.ps_path_index;
-        const WallRec &pr = cc.recs[path];
+        const WallRec &pr = cc.rec(path);
         const FragmentChoice pr_fragment = choose_fragment<SPLIT>(m, cc.frags, pr, path, x);
         int path_safe_other = r.ps_other < 0 ? 0 : r.ps_other;
         const Tables &tb = *cc.tb;
@@ -2511,7 +2535,7 @@ __device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const Col
     bool left_edge = cand_flags & CF_LEDGE;
     bool has_saved = c.masked_wall == mw;
     if (!(has_saved || left_edge)) return;
-    const WallRec &wr = cc.recs[mw];
+    const WallRec &wr = cc.rec(mw);
     const FragmentChoice wr_fragment = choose_fragment<SPLIT>(m, cc.frags, wr, mw, x);
     int front_sector = mv.sec(mw, 0), back_sector = mv.sec(mw, 1) < 0 ? 0 : mv.sec(mw, 1);
     int light_sector = mside == 0 ? front_sector : back_sector;
@@ -2588,7 +2612,7 @@ __device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const Col
             const unsigned fraction = row_base + row_step * (unsigned)y;
             const unsigned mv_ = (fraction >> (31 - height_bits)) >> 1;
             texel[j] = m->tex_atlas[texel_base + __umul24(mv_, atlas_w)];
-            word[j] = pb.meta[(size_t)y * SW + x];
+            word[j] = pb.m(y);
         }
 #pragma unroll
         for (int j = 0; j < WALL_ROWS; ++j) {
@@ -2597,19 +2621,24 @@ __device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const Col
             // the texel goes to the frame where there is one; otherwise it waits in the sprite clip plane, which nothing
             // reads any more once a column's traversal is over, for the kernel that assembles the frame
             const unsigned char colour = colormap[shade * 256 + texel[j]];
-            if (pb.frame) pb.frame[(size_t)y * SW + x] = colour;
-            else pb.clip_depth[(size_t)y * SW + x] = __uint_as_float((unsigned)colour);
-            pb.meta[(size_t)y * SW + x] = word[j] | META_MASKED;
-            if (DEPTH) pb.scene_depth[(size_t)y * SW + x] = md;
+            if (pb.frame) pb.f(y) = colour;
+            else pb.d(y) = __uint_as_float((unsigned)colour);
+            pb.m(y) = word[j] | META_MASKED;
+            if (DEPTH) pb.s(y) = md;
         }
     }
 }
 
-// How long a strip's traversal runs is set by the column that crosses the most portals: the
-// two-sided linedefs its ray hits before the nearest blocking one.  Strips differ by a factor of
-// ten, and a launch ends with its longest wavefront, so the traversal takes the strips longest
-// first: strip_key_kernel counts (one wavefront per strip, one lane per column, a walk over the
-// column's candidate list), strip_order_kernel sorts the counts (one block, counting sort).
+// How long a column's traversal runs is set by the portals it crosses: the two-sided linedefs its ray hits before the
+// nearest blocking one.  Columns differ by a factor of ten, a wavefront runs as long as its longest column, and a launch
+// ends with its longest wavefront.  So the screen is cut into segments of SEG_COLS columns, a wavefront takes
+// 64 / SEG_COLS segments of about the same length (whatever lanes they belong to), and the longest go first:
+// strip_key_kernel counts (one lane per column, a walk over the column's candidate list, the maximum of each segment),
+// strip_order_kernel sorts the counts (one block, counting sort).
+// Narrow segments waste fewer column passes (on the 4000-linedef map 69 % of the passes a wavefront runs are useful with
+// whole 64-column strips, 80 % with two sorted 32-column segments, 89 % with four of 16), but unrelated segments share no
+// linedefs, branches or row ranges, and a pass costs what the union of its columns' paths costs: measured, the traversal
+// takes 3.86 ms with 64 or 32 columns a segment, 4.06 ms with 16 and 4.23 ms with 8.  Hence whole strips.
 __global__ void __launch_bounds__(256) strip_key_kernel(int lane_count, Scratch sc) {
     const int strip = blockIdx.x * 4 + (threadIdx.x >> 6);
     const int local = strip / (SW / 64);
@@ -2632,8 +2661,8 @@ __global__ void __launch_bounds__(256) strip_key_kernel(int lane_count, Scratch 
         }
     }
 #pragma unroll
-    for (int step = 1; step < 64; step <<= 1) portals = max(portals, __shfl_xor(portals, step));
-    if ((threadIdx.x & 63) == 0) sc.strip_key[strip] = (unsigned char)portals;   // at most CAND_MAX
+    for (int step = 1; step < SEG_COLS; step <<= 1) portals = max(portals, __shfl_xor(portals, step));
+    if ((x & (SEG_COLS - 1)) == 0) sc.strip_key[local * SEGS_PER_LANE + x / SEG_COLS] = (unsigned char)portals;   // at most CAND_MAX
 }
 
 __global__ void __launch_bounds__(1024) strip_order_kernel(int strips, Scratch sc) {
@@ -2650,51 +2679,55 @@ __global__ void __launch_bounds__(1024) strip_order_kernel(int strips, Scratch s
     for (int s = threadIdx.x; s < strips; s += blockDim.x) sc.strip_order[atomicAdd(&position[sc.strip_key[s]], 1)] = s;
 }
 
-// One wavefront per (lane, 64-column strip).  Strips share nothing but read-only tables; a
-// work-group is WALL_STRIPS_PER_GROUP strips (neighbours in the longest-first order) only so that the
-// LDS copies of those tables, 16.7 KB, are held once per group rather than once per wavefront: a CU has
-// 160 KB of LDS and room for twelve of these wavefronts (166 registers), so one strip per group would stop
-// at nine.  After the staging barrier the wavefronts never meet again.
+// One wavefront per 64 / SEG_COLS segments.  Segments share nothing but read-only tables; a work-group is
+// WALL_STRIPS_PER_GROUP wavefronts (neighbours in the longest-first order) only so that the LDS copies of those
+// tables, 16.7 KB, are held once per group rather than once per wavefront: a CU has 160 KB of LDS and room for
+// twelve of these wavefronts (168 registers), so one wavefront per group would stop at nine.  After the staging
+// barrier the wavefronts never meet again.
 #define WALL_STRIPS_PER_GROUP 2
 // DEPTH: also keep the depth of every wall pixel (frames that draw decals).  SPLIT: the map has linedefs with
 // BSP projection fragments.
 template <bool DEPTH, bool SPLIT>
 __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amdgpu_waves_per_eu(3, 3))) wall_columns_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
     const gd_map_desc *m = &dm.d;
-    __shared__ LaneCtx lane_ctxs[WALL_STRIPS_PER_GROUP];
+    __shared__ LaneCtx lane_ctxs[WALL_STRIPS_PER_GROUP][64 / SEG_COLS];
     __shared__ unsigned char colormap_lds[32 * 256];   // shade rows 0..31 are the only ones indexed
     __shared__ float4 sector_lds[LDS_SECTORS];
     __shared__ TexLds tex_lds;
     const int wave_in_group = threadIdx.x >> 6;
-    const int strip_slot = blockIdx.x * WALL_STRIPS_PER_GROUP + wave_in_group;
-    const bool live = strip_slot < lane_count * (SW / 64);
-    const int strip_index = live ? sc.strip_order[strip_slot] : 0;
-    const int local = strip_index / (SW / 64);
+    const int lane_id = threadIdx.x & 63;
+    const int segment_in_wave = lane_id / SEG_COLS;
+    const int segment_slot = (blockIdx.x * WALL_STRIPS_PER_GROUP + wave_in_group) * (64 / SEG_COLS) + segment_in_wave;
+    const bool live = segment_slot < lane_count * SEGS_PER_LANE;
+    const int segment = live ? sc.strip_order[segment_slot] : 0;
+    const int local = segment / SEGS_PER_LANE;
     Tables tb;
     stage_tables(m, sector_lds, &tex_lds, tb);
-    if ((threadIdx.x & 63) == 0 && live) lane_ctxs[wave_in_group] = sc.ctx[local];
+    if ((lane_id & (SEG_COLS - 1)) == 0 && live) lane_ctxs[wave_in_group][segment_in_wave] = sc.ctx[local];
     for (int k = threadIdx.x; k < 32 * 256 / 4; k += blockDim.x) reinterpret_cast<unsigned int *>(colormap_lds)[k] = reinterpret_cast<const unsigned int *>(m->colormap)[k];
     __syncthreads();
-    if (!live) return;
-    const LaneCtx &lane_ctx = lane_ctxs[wave_in_group];
-    const int x = (strip_index - local * (SW / 64)) * 64 + (threadIdx.x & 63);
+    if (!live) return;   // whole segments: the groups of four columns that exchange values below live or leave together
+    const LaneCtx &lane_ctx = lane_ctxs[wave_in_group][segment_in_wave];
+    const int x = (segment - local * SEGS_PER_LANE) * SEG_COLS + (lane_id & (SEG_COLS - 1));
     bool window_dirty = false;
-    GapRange gaps; gaps.lo = VH; gaps.hi = 0;
+    GapRange gaps; gaps.reset();
     ColumnCtx cc;
     cc.tb = &tb; cc.m = m; cc.mv.m = m; cc.c = &lane_ctx;
-    cc.recs = sc.rec + (size_t)local * m->wall_count;
-    cc.spans = sc.span + (size_t)local * m->wall_count;
+    cc.recs = sc.rec; cc.spans = sc.span;
+    cc.rec_base = (unsigned)local * (unsigned)m->wall_count;
     cc.frags = sc.frag_rec + (size_t)local * m->split_count * m->fragment_slots;
-    cc.list = sc.cand + (size_t)local * CAND_MAX * SW;
+    cc.list = sc.cand;
+    cc.list_column = ((unsigned)local * (CAND_MAX * SW) + (unsigned)x) * 16u;
     cc.count = sc.cand_count[(size_t)local * SW + x];
     if (cc.count > CAND_MAX) cc.count = CAND_MAX;
     cc.x = x;
     ray_direction(lane_ctx, x, &cc.rx, &cc.ry);
     PixelBuffers pb;
-    pb.frame = frame_base ? frame_base + (size_t)local * frame_stride : nullptr;
-    pb.meta = sc.meta + (size_t)local * VH * SW;
-    pb.clip_depth = sc.clip_depth + (size_t)local * VH * SW;
-    pb.scene_depth = DEPTH ? sc.scene_depth + (size_t)local * VH * SW : nullptr;
+    pb.frame = frame_base;
+    pb.meta = sc.meta; pb.clip_depth = sc.clip_depth;
+    pb.scene_depth = DEPTH ? sc.scene_depth : nullptr;
+    pb.word_column = ((unsigned)local * (VH * SW) + (unsigned)x) * 4u;
+    pb.frame_column = (unsigned)local * (unsigned)frame_stride + (unsigned)x;
     // the meta plane arrives with whatever the last frame left: see GapRange for how every row gets written
     ColumnState st;
     st.current_sector = lane_ctx.sector;
@@ -2708,21 +2741,10 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
     for (int k = 0; k < cc.count; ++k) if (cc.cand(k).flags & CF_LEDGE) { boundary_has_po = true; break; }
     PassColumn pc;
     bool done = false;
-#ifdef GD_PROFILE
-    long long prof_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    long long prof_start = wall_clock64();
-#endif
-    const int lane_id = threadIdx.x & 63;
     const int group_base = lane_id & ~3;
     const int sectors = m->sector_count;
     for (int pass = 0; pass < sectors; ++pass) {
-        PROF_T(t0);
-#ifdef GD_PROFILE
-        prof_acc[7] += 1;
-#endif
         if (!done) pass_select<SPLIT>(cc, st, boundary_has_po, pc);
-        PROF_T(t1);
-        PROF_ADD(0, t0, t1);
         // 4-column wallscan groups (engine.py:12688-12761): exchange with the aligned neighbours
         bool same_group = true;
         int w0 = __shfl(pc.wall, group_base), s0 = __shfl(pc.side, group_base);
@@ -2744,49 +2766,24 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
         bool group_valid[3];
         for (int t = 0; t < 3; ++t) group_valid[t] = same_group && all_tier[t] && (common_top[t] < common_bottom[t]);
         if (!done) {
-            PROF_T(t2);
             pass_paint<DEPTH>(cc, st, pc, pb, group_valid, common_bottom, first_group_visibility, colormap_lds, window_dirty, gaps);
-            PROF_T(t3);
-            PROF_ADD(1, t2, t3);
             bool changed = pass_advance<SPLIT>(cc, st, pc, pb, sb, !window_dirty);
-            PROF_T(t4);
-            PROF_ADD(2, t3, t4);
-#ifdef GD_PROFILE
-            prof_acc[5] += 1;
-#endif
             // A pass that found nothing and changed nothing repeats identically for ever.
             if (!(pc.bits & PB_VALID) && !changed) done = true;
         }
         if (__ballot(!done) == 0) break;
     }
-    PROF_T(t5);
-    PROF_T(t6);
     // what is left of a window no one-sided drawseg closed shows the flat pass's picture
     if (!window_dirty) zero_rows(pb, gaps, x, st.ceiling_clip <= 0.0f ? 0 : (int)st.ceiling_clip, st.floor_clip >= (float)VH ? VH : (int)st.floor_clip);
     masked_midtexture<DEPTH, SPLIT>(cc, st, pb, colormap_lds);
     // The view pixels no wall tier, plane or masked texture covers: the flat pass selects them (flat_list_kernel) and
     // flat_shade_kernel paints them.  More than the list holds: the lane is handled pixel by pixel.
-    for (int y = gaps.lo; y < gaps.hi; ++y) {
-        const unsigned int word = pb.meta[(size_t)y * SW + x];
+    for (int y = gaps.lo(), gap_end = gaps.hi(); y < gap_end; ++y) {
+        const unsigned int word = pb.m(y);
         if ((word & (META_FILLED | META_MASKED)) || ((word >> META_SECTOR_SHIFT) & META_SECTOR_MASK) != 0) continue;
         const int slot = atomicAdd(&sc.flat_list_count[local], 1);
         if (slot < FLAT_LIST_MAX) sc.flat_list[(size_t)local * FLAT_LIST_MAX + slot] = y * SW + x;
     }
-#ifdef GD_PROFILE
-    long long t7 = wall_clock64();
-    int prof_cands = cc.count;
-    for (int step = 1; step < 64; step <<= 1) prof_cands += __shfl_xor(prof_cands, step);
-    prof_acc[3] += t6 - t5; prof_acc[4] += t7 - t6; prof_acc[6] += t7 - prof_start;
-    if ((threadIdx.x & 63) == 0) {   // one sample per wave: phases are wave-synchronous
-        for (int k = 0; k < 7; ++k) atomicAdd(&g_profile[k], (unsigned long long)prof_acc[k]);
-        atomicAdd(&g_profile[7], 1ULL);
-        if (strip_index < 32768) {
-            g_wave_log[3 * strip_index] = (unsigned int)prof_acc[6];
-            g_wave_log[3 * strip_index + 1] = (unsigned int)prof_cands;
-            g_wave_log[3 * strip_index + 2] = (unsigned int)prof_acc[7];
-        }
-    }
-#endif
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -4032,8 +4029,8 @@ size_t carve_scratch(Scratch &sc, unsigned char *base, size_t L, const gd_map_de
     take(&sc.row_slope, L * (size_t)VH);
     take(&sc.step_scale, L * STEP_TABLE);
     take(&sc.block_hit, L * SW);
-    take(&sc.strip_key, L * (SW / 64));
-    take(&sc.strip_order, L * (SW / 64));
+    take(&sc.strip_key, L * SEGS_PER_LANE);
+    take(&sc.strip_order, L * SEGS_PER_LANE);
     if (depth) {   // frames that draw decals: a scene depth plane, and a frame when the caller wants none
         take(&sc.scene_depth, L * PX);
         take(&sc.frame, L * (size_t)GD_SCREEN_HEIGHT * SW);
@@ -4211,10 +4208,11 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     if (m.split_count > 0)
         hipLaunchKernelGGL(fragment_setup_kernel, dim3((m.split_count * m.fragment_slots + 63) / 64, count), dim3(64), 0, stream, r->dm, count, sc);
     hipLaunchKernelGGL(strip_key_kernel, dim3((count * (SW / 64) + 3) / 4), dim3(256), 0, stream, count, sc);
-    hipLaunchKernelGGL(strip_order_kernel, dim3(1), dim3(1024), 0, stream, count * (SW / 64), sc);
+    hipLaunchKernelGGL(strip_order_kernel, dim3(1), dim3(1024), 0, stream, count * SEGS_PER_LANE, sc);
     mark();
     {
-        const dim3 grid((count * (SW / 64) + WALL_STRIPS_PER_GROUP - 1) / WALL_STRIPS_PER_GROUP), block(64 * WALL_STRIPS_PER_GROUP);
+        const int wavefronts = (count * SEGS_PER_LANE + 64 / SEG_COLS - 1) / (64 / SEG_COLS);
+        const dim3 grid((wavefronts + WALL_STRIPS_PER_GROUP - 1) / WALL_STRIPS_PER_GROUP), block(64 * WALL_STRIPS_PER_GROUP);
         const bool split = m.split_count > 0;
         auto kernel = decals ? (split ? wall_columns_kernel<true, true> : wall_columns_kernel<true, false>)
                              : (split ? wall_columns_kernel<false, true> : wall_columns_kernel<false, false>);
@@ -4652,18 +4650,6 @@ int gd_renderer_set_sector_lights(gd_renderer *r, const float *lights, void *str
     return GD_OK;
 }
 
-#ifdef GD_PROFILE
-/* profiling build only: cumulative per-wave clock ticks of the wall kernel's phases */
-int gd_wave_log_read(unsigned int *out) {
-    HIP_TRY(hipMemcpyFromSymbol(out, HIP_SYMBOL(g_wave_log), sizeof(unsigned int) * 3 * 32768));
-    return GD_OK;
-}
-int gd_profile_read(unsigned long long *out, int reset) {
-    HIP_TRY(hipMemcpyFromSymbol(out, HIP_SYMBOL(g_profile), sizeof(unsigned long long) * 16));
-    if (reset) { unsigned long long zero[16] = {0}; HIP_TRY(hipMemcpyToSymbol(HIP_SYMBOL(g_profile), zero, sizeof(zero))); }
-    return GD_OK;
-}
-#endif
 
 int gd_observe(const uint8_t *indexed, int32_t source_rows, const uint8_t *playpal, int32_t lane_count,
                uint8_t *obs, uint8_t *frames, const uint8_t *reset_mask, int32_t stack_mode, void *stream) {
