@@ -14,6 +14,8 @@ FRAME_STACK = 4
 
 STACK_STEP = 0
 STACK_RESET = 1
+LAYOUT_CHW = 0
+LAYOUT_HWC = 1
 
 GD_OK = 0
 STATIC_SCRATCH_MIB = 64  # gd_render_static: the fixed per-GPU working memory
@@ -22,7 +24,7 @@ GD_E_ARG = -1
 GD_E_HIP = -2
 GD_E_UNSUPPORTED = -3
 
-ABI_VERSION = 2  # GD_ABI_VERSION
+ABI_VERSION = 3  # GD_ABI_VERSION
 
 _P = C.c_void_p
 
@@ -237,7 +239,8 @@ def host_overlay_desc(overlays: dict) -> tuple[OverlayDesc, list]:
 
 
 class FrameOut(_Sized):
-    _fields_ = [("struct_size", C.c_uint32)] + [(name, _P) for name in OUT_FIELDS] + [("stack_mode", C.c_int32), ("obs_source_rows", C.c_int32)]
+    _fields_ = [("struct_size", C.c_uint32)] + [(name, _P) for name in OUT_FIELDS] + [
+        ("stack_mode", C.c_int32), ("obs_source_rows", C.c_int32), ("final_frames_layout", C.c_int32)]
 
 
 def host_map_desc(tables: dict) -> tuple[MapDesc, list]:

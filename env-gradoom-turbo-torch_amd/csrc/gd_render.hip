@@ -3389,6 +3389,40 @@ __device__ __forceinline__ void stage_palette(unsigned char *pal, const unsigned
     __syncthreads();
 }
 
+// The frame stack of one lane, four pixels (one word per stacked observation) at a time: what the stack holds after
+// this call goes to `stack` (when it changes) and to the caller's copy, which is laid out either like the stack
+// ([4][84][84]) or with the four stacked values of a pixel next to each other ([84][84][4]).
+// `kept` holds the stack's words as they were (unused for a lane that resets).  env.py:678-688, engine.py:15447-15450
+__device__ __forceinline__ void store_stack_word(unsigned char *stack_lane, unsigned char *copy_lane, bool copy_hwc, bool aligned, size_t word,
+                                                 const unsigned int (&kept)[GD_FRAME_STACK], unsigned int grays, bool resets, int stack_mode) {
+    const size_t plane = (size_t)GD_OBS_SIZE * GD_OBS_SIZE;   // bytes per stacked observation
+    auto store = [&](unsigned char *p, unsigned int v) {
+        if (aligned) *reinterpret_cast<unsigned int *>(p) = v;
+        else for (int k = 0; k < 4; ++k) p[k] = (unsigned char)(v >> (8 * k));
+    };
+    const bool steps = !resets && stack_mode == GD_STACK_STEP;
+    unsigned int next[GD_FRAME_STACK];
+#pragma unroll
+    for (int k = 0; k < GD_FRAME_STACK; ++k) next[k] = resets ? grays : (steps ? (k + 1 < GD_FRAME_STACK ? kept[k + 1] : grays) : kept[k]);
+    if (resets || steps) {
+#pragma unroll
+        for (int k = 0; k < GD_FRAME_STACK; ++k) store(stack_lane + k * plane + word * 4, next[k]);
+    }
+    if (!copy_lane) return;
+    if (!copy_hwc) {
+#pragma unroll
+        for (int k = 0; k < GD_FRAME_STACK; ++k) store(copy_lane + k * plane + word * 4, next[k]);
+        return;
+    }
+    static_assert(GD_FRAME_STACK == 4, "the interleaved copy packs the four stacked values of a pixel into one word");
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {   // pixel j of the word
+        const unsigned int v = ((next[0] >> (8 * j)) & 255u) | (((next[1] >> (8 * j)) & 255u) << 8) |
+                               (((next[2] >> (8 * j)) & 255u) << 16) | (((next[3] >> (8 * j)) & 255u) << 24);
+        store(copy_lane + (word * 4 + j) * GD_FRAME_STACK, v);
+    }
+}
+
 // One block per lane and OBS_BLOCK_ROWS observation rows.  The source rows they overlap are staged in LDS with
 // word loads (a byte load per tap keeps the address units busy for 64 lanes each); taps then read LDS.
 #define OBS_BLOCK_ROWS 3
@@ -3396,7 +3430,7 @@ __device__ __forceinline__ void stage_palette(unsigned char *pal, const unsigned
 static_assert(GD_OBS_SIZE % OBS_BLOCK_ROWS == 0 && OBS_BLOCK_ROWS * GD_OBS_SIZE <= 256, "observe_kernel: rows per block");
 __global__ void __launch_bounds__(256) observe_kernel(const unsigned char *indexed, size_t lane_stride, int source_rows, const unsigned char *playpal,
                                int lane_count, unsigned char *obs, unsigned char *frames, const unsigned char *reset_mask, int stack_mode,
-                               unsigned char *final_frames, const float *blend) {
+                               unsigned char *final_frames, bool final_hwc, const float *blend) {
     __shared__ unsigned int pal[256];   // PLAYPAL after the lane's screen blend, one word per colour (red | green << 8 | blue << 16)
     __shared__ unsigned int tile[OBS_TILE_ROWS * (SW / 4)];
     int n = blockIdx.y;
@@ -3488,28 +3522,9 @@ __global__ void __launch_bounds__(256) observe_kernel(const unsigned char *index
         if ((reinterpret_cast<size_t>(obs) & 3) == 0) *reinterpret_cast<unsigned int *>(out) = grays;
         else for (int k = 0; k < 4; ++k) out[k] = (unsigned char)(grays >> (8 * k));
     }
-    if (frames) {
-        // a stack is [4][84][84] bytes, so word access only needs the tensors themselves word aligned
-        unsigned char *copy_bytes = final_frames ? final_frames + ((size_t)n * GD_FRAME_STACK * F + word) * 4 : nullptr;
-        auto store = [&](unsigned char *p, unsigned int v) {
-            if (stack_aligned) *reinterpret_cast<unsigned int *>(p) = v;
-            else for (int k = 0; k < 4; ++k) p[k] = (unsigned char)(v >> (8 * k));
-        };
-        const size_t plane = F * 4;   // bytes per stacked observation
-        if (resets) {
-            for (int k = 0; k < GD_FRAME_STACK; ++k) store(stack_bytes + k * plane, grays);
-            if (copy_bytes) for (int k = 0; k < GD_FRAME_STACK; ++k) store(copy_bytes + k * plane, grays);
-        } else if (stack_mode == GD_STACK_STEP) {
-            for (int k = 0; k < GD_FRAME_STACK - 1; ++k) store(stack_bytes + k * plane, kept[k + 1]);
-            store(stack_bytes + (GD_FRAME_STACK - 1) * plane, grays);
-            if (copy_bytes) {
-                for (int k = 0; k < GD_FRAME_STACK - 1; ++k) store(copy_bytes + k * plane, kept[k + 1]);
-                store(copy_bytes + (GD_FRAME_STACK - 1) * plane, grays);
-            }
-        } else if (copy_bytes) {
-            for (int k = 0; k < GD_FRAME_STACK; ++k) store(copy_bytes + k * plane, kept[k]);   // lane left as it was
-        }
-    }
+    // a stack is [4][84][84] bytes, so word access only needs the tensors themselves word aligned
+    if (frames) store_stack_word(frames + (size_t)n * GD_FRAME_STACK * F * 4, final_frames ? final_frames + (size_t)n * GD_FRAME_STACK * F * 4 : nullptr,
+                                 final_hwc, stack_aligned, word, kept, grays, resets, stack_mode);
 }
 
 // engine.py:15381-15384
@@ -3551,6 +3566,7 @@ struct FinishOut {   // device pointers of the chunk's first lane; null = not wa
     const unsigned char *reset_mask;
     const float *blend;
     int stack_mode, source_rows;
+    bool final_hwc;
 };
 
 __global__ void __launch_bounds__(BAND_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) band_finish_kernel(DeviceMap dm, Overlays ov, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc, FinishOut out) {
@@ -3764,24 +3780,14 @@ __global__ void __launch_bounds__(BAND_THREADS) __attribute__((amdgpu_waves_per_
         const unsigned int grays = gray_words[k];
         if (out.obs) store_word(out.obs + ((size_t)local * F + word) * 4, grays, (reinterpret_cast<size_t>(out.obs) & 3) == 0);
         if (!out.frames) continue;
-        unsigned char *stack = out.frames + ((size_t)local * GD_FRAME_STACK * F + word) * 4;
-        unsigned char *copy = out.final_frames ? out.final_frames + ((size_t)local * GD_FRAME_STACK * F + word) * 4 : nullptr;
-        const size_t plane = F * 4;   // bytes per stacked observation
-        if (resets) {
-            for (int f = 0; f < GD_FRAME_STACK; ++f) store_word(stack + f * plane, grays, stack_aligned);
-            if (copy) for (int f = 0; f < GD_FRAME_STACK; ++f) store_word(copy + f * plane, grays, stack_aligned);
-        } else if (out.stack_mode == GD_STACK_STEP) {
-            unsigned int kept[GD_FRAME_STACK];
-            for (int f = 1; f < GD_FRAME_STACK; ++f) kept[f] = load_word(stack + f * plane, stack_aligned);
-            for (int f = 0; f < GD_FRAME_STACK - 1; ++f) store_word(stack + f * plane, kept[f + 1], stack_aligned);
-            store_word(stack + (GD_FRAME_STACK - 1) * plane, grays, stack_aligned);
-            if (copy) {
-                for (int f = 0; f < GD_FRAME_STACK - 1; ++f) store_word(copy + f * plane, kept[f + 1], stack_aligned);
-                store_word(copy + (GD_FRAME_STACK - 1) * plane, grays, stack_aligned);
-            }
-        } else if (copy) {
-            for (int f = 0; f < GD_FRAME_STACK; ++f) store_word(copy + f * plane, load_word(stack + f * plane, stack_aligned), stack_aligned);   // lane left as it was
-        }
+        unsigned char *stack_lane = out.frames + (size_t)local * GD_FRAME_STACK * F * 4;
+        unsigned int kept[GD_FRAME_STACK];
+        // a lane that steps drops its oldest observation; it is only read for a copy of a stack that stays as it is
+        const bool reads = !resets, reads_oldest = reads && out.stack_mode != GD_STACK_STEP && out.final_frames;
+        for (int f = 0; f < GD_FRAME_STACK; ++f)
+            kept[f] = (reads && (f > 0 || reads_oldest)) ? load_word(stack_lane + (size_t)f * F * 4 + word * 4, stack_aligned) : 0u;
+        store_stack_word(stack_lane, out.final_frames ? out.final_frames + (size_t)local * GD_FRAME_STACK * F * 4 : nullptr, out.final_hwc,
+                         stack_aligned, word, kept, grays, resets, out.stack_mode);
     }
 }
 
@@ -4182,6 +4188,7 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     const gd_map_desc &m = r->dm.d;
     Scratch sc = chunk_scratch;
     if (out->final_frames && !out->frames) return fail(GD_E_ARG, "final_frames needs frames");
+    if (out->final_frames_layout != GD_LAYOUT_CHW && out->final_frames_layout != GD_LAYOUT_HWC) return fail(GD_E_ARG, "unknown final_frames_layout");
     const size_t frame_stride = (size_t)GD_SCREEN_HEIGHT * SW;
     const size_t F = (size_t)GD_OBS_SIZE * GD_OBS_SIZE;
     const int source_rows = out->obs_source_rows == GD_SCREEN_HEIGHT ? GD_SCREEN_HEIGHT : VH;
@@ -4245,6 +4252,7 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
         finish.reset_mask = out->reset_mask ? out->reset_mask + base : nullptr;
         finish.blend = blend;
         finish.stack_mode = out->stack_mode;
+        finish.final_hwc = out->final_frames_layout == GD_LAYOUT_HWC;
         finish.source_rows = source_rows;
         const bool sprites = lanes->sprite_slots > 0 && lanes->sprite_x;
         size_t shared = sprites ? (size_t)lanes->sprite_slots * (sizeof(SpriteRec) + sizeof(unsigned short)) : 0;
@@ -4272,7 +4280,8 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
                            frame_base, frame_stride, source_rows, m.playpal, count, out->obs ? out->obs + (size_t)base * F : nullptr,
                            out->frames ? out->frames + (size_t)base * GD_FRAME_STACK * F : nullptr,
                            out->reset_mask ? out->reset_mask + base : nullptr, out->stack_mode,
-                           out->final_frames ? out->final_frames + (size_t)base * GD_FRAME_STACK * F : nullptr, blend);
+                           out->final_frames ? out->final_frames + (size_t)base * GD_FRAME_STACK * F : nullptr,
+                           out->final_frames_layout == GD_LAYOUT_HWC, blend);
     }
     if (out->rgb) {
         size_t pixels = (size_t)count * frame_stride;
@@ -4664,7 +4673,7 @@ int gd_observe(const uint8_t *indexed, int32_t source_rows, const uint8_t *playp
         hipLaunchKernelGGL(observe_kernel, dim3(GD_OBS_SIZE / OBS_BLOCK_ROWS, count), dim3(256), 0, static_cast<hipStream_t>(stream),
                            indexed + (size_t)base * source_rows * SW, (size_t)source_rows * SW, source_rows, playpal, count,
                            obs ? obs + (size_t)base * F : nullptr, frames ? frames + (size_t)base * GD_FRAME_STACK * F : nullptr,
-                           reset_mask ? reset_mask + base : nullptr, stack_mode, nullptr, nullptr);
+                           reset_mask ? reset_mask + base : nullptr, stack_mode, nullptr, false, nullptr);
     }
     HIP_TRY(hipGetLastError());
     return GD_OK;

@@ -7,6 +7,7 @@ the render path serves:
 * ``step_device(actions) -> DeviceTransition``                                  (``env.py:851-877``)
 * ``step_and_reset_device(actions, reset_seeds) -> DeviceAutoResetTransition``  (``env.py:909-942, 998``)
 * ``render() / render_lane(i) / get_images()`` -> ``uint8 (240, 320, 3)``       (``env.py:1037-1064``)
+* ``reset(seed=, options=) / step(actions)`` with ``obs_copy`` ownership         (``env.py:750-834, 678-688``)
 
 with the same argument validation (``env.py:711-728``), the same ownership rules
 (``observations`` is the renderer-owned ``frames`` stack returned by reference;
@@ -22,6 +23,7 @@ from __future__ import annotations
 
 import dataclasses
 import operator
+from collections.abc import Sequence
 
 import numpy as np
 import torch
@@ -54,6 +56,17 @@ class DeviceAutoResetTransition:  # env.py:193-205
     final_observations: torch.Tensor
     final_signals: torch.Tensor
     final_info_histories: torch.Tensor
+
+
+def _normalize_seed(seed, num_envs: int):  # env.py:101-113
+    if seed is None:
+        return [None] * num_envs
+    if isinstance(seed, Sequence) and not isinstance(seed, (str, bytes, bytearray)):
+        values = [None if value is None else int(value) for value in seed]
+        if len(values) != num_envs:
+            raise ValueError("seed sequence length must match num_envs")
+        return values
+    return [int(seed) + lane for lane in range(num_envs)]
 
 
 class PosePoolDynamics:
@@ -122,6 +135,7 @@ class GraDoomVecEnv:
         device="cuda:0",
         render_mode: str | None = None,
         obs_layout: str = "chw",
+        obs_copy: str = "safe_view",
         dynamics=None,
         renderer=None,
         episode_timeout: int = 32,
@@ -131,6 +145,8 @@ class GraDoomVecEnv:
             raise ValueError("num_envs must be positive")
         if obs_layout not in ("chw", "hwc"):
             raise ValueError("obs_layout must be 'chw' or 'hwc'")
+        if obs_copy not in ("copy", "safe_view", "unsafe_view"):  # env.py:344-345
+            raise ValueError("obs_copy must be copy, safe_view, or unsafe_view")
         if render_mode not in (None, "rgb_array"):
             raise ValueError("render_mode must be None or 'rgb_array'")
         self.num_envs = int(num_envs)
@@ -138,6 +154,9 @@ class GraDoomVecEnv:
         self._resident_device = self.device
         self.render_mode = render_mode
         self.obs_layout = obs_layout
+        self.obs_copy = obs_copy
+        self.observation_ownership = {"copy": "owned", "safe_view": "safe_view", "unsafe_view": "unsafe_view"}[obs_copy]  # env.py:377-382
+        self.observation_buffer_depth = {"copy": None, "safe_view": 2, "unsafe_view": 1}[obs_copy]
         self.observation_renderer = "reference"
         self.closed = False
         self._renderer = renderer if renderer is not None else HipRenderer(smap, self.num_envs, self.device)
@@ -152,6 +171,16 @@ class GraDoomVecEnv:
         self._initialized = torch.zeros(n, dtype=torch.bool, device=self.device)
         self._latest_reset_seeds = torch.zeros(n, dtype=torch.int64, device=self.device)
         self._all_lanes = torch.ones(n, dtype=torch.uint8, device=self.device)
+        # obs_copy="safe_view": two buffers handed out in turn, so that the observation of the step before stays
+        # valid while this step's is written (env.py:459-472).  The renderer's observation kernel fills them.
+        view_shape = (n, self.frame_stack, 84, 84) if obs_layout == "chw" else (n, 84, 84, self.frame_stack)
+        self._view_shape = view_shape
+        self._safe_obs_buffers = (
+            tuple(torch.empty(view_shape, dtype=torch.uint8, device=self.device) for _ in range(2)) if obs_copy == "safe_view" else ()
+        )
+        self._safe_obs_index = 0
+        self._seed_values = [None] * n
+        self._reset_rngs = [np.random.default_rng() for _ in range(n)]
 
     # ------------------------------------------------------------------ helpers
     def _require_device_tensor(self, value, name, *, shape, dtypes):  # env.py:711-728
@@ -174,6 +203,9 @@ class GraDoomVecEnv:
 
     # ------------------------------------------------------------------ device API
     def reset_device(self, mask: torch.Tensor, seeds: torch.Tensor):
+        return self._reset(mask, seeds, None)
+
+    def _reset(self, mask: torch.Tensor, seeds: torch.Tensor, view):
         if self.closed:
             raise RuntimeError("cannot reset a closed environment")
         device_mask = self._require_device_tensor(mask, "mask", shape=(self.num_envs,), dtypes=(torch.bool,))
@@ -182,7 +214,8 @@ class GraDoomVecEnv:
         # engine.reset renders every lane and fills the stack of the masked ones with four copies
         # (engine.py:2443-2450); unmasked lanes keep their stack, which the fused epilogue does by
         # writing only under the mask.
-        self._renderer.render(self._dynamics.lane_state(), frames=self.frames, reset_mask=device_mask, obs=None, stack_only_masked=True)
+        self._renderer.render(self._dynamics.lane_state(), frames=self.frames, reset_mask=device_mask, obs=None, stack_only_masked=True,
+                              final_frames=view, final_layout=self.obs_layout)
         self._latest_reset_seeds.copy_(torch.where(device_mask, device_seeds, self._latest_reset_seeds))
         self._initialized |= device_mask
         self._update_signals()
@@ -191,12 +224,12 @@ class GraDoomVecEnv:
     def step_device(self, actions: torch.Tensor) -> DeviceTransition:
         return self._step(actions, None)
 
-    def _step(self, actions: torch.Tensor, final_frames) -> DeviceTransition:
+    def _step(self, actions: torch.Tensor, final_frames, final_layout: str = "chw") -> DeviceTransition:
         if self.closed:
             raise RuntimeError("cannot step a closed environment")
         indices = self._require_device_tensor(actions, "actions", shape=(self.num_envs,), dtypes=INDEX_DTYPES).to(torch.int64)
         rewards, terminated, truncated = self._dynamics.step(indices)
-        self._renderer.render(self._dynamics.lane_state(), frames=self.frames, final_frames=final_frames)
+        self._renderer.render(self._dynamics.lane_state(), frames=self.frames, final_frames=final_frames, final_layout=final_layout)
         self._update_signals()
         return DeviceTransition(
             observations=self._device_observations(self.frames), rewards=rewards, terminated=terminated, truncated=truncated,
@@ -211,7 +244,9 @@ class GraDoomVecEnv:
         final_signals = transition.signals.clone()
         final_info_histories = transition.info_histories.clone()
         done = transition.terminated | transition.truncated
-        if not bool(torch.any(done)):  # env.py:919: one host sync for the reference renderer
+        any_done = bool(torch.any(done))  # env.py:919: one host sync for the reference renderer
+        self.check_renderer_status()      # the device is idle here anyway
+        if not any_done:
             return DeviceAutoResetTransition(
                 transition.observations, transition.rewards, transition.terminated, transition.truncated,
                 transition.signals, transition.info_histories, final_observations, final_signals, final_info_histories,
@@ -224,6 +259,69 @@ class GraDoomVecEnv:
 
     def device_signals(self) -> torch.Tensor:
         return self.signal_buffer
+
+    def check_renderer_status(self) -> None:
+        """Raise if the renderer had to drop a linedef from a column's candidate list (it keeps 64 per column).
+
+        Such a frame may differ from the reference's, which has no such bound, so it must not pass for a good one.
+        Synchronises the device: called where the environment already waits for it.
+        """
+        status = getattr(self._renderer, "status", None)
+        if status is not None and status() & 1:
+            raise RuntimeError(
+                "the renderer truncated a screen column's candidate list (more than 64 linedefs overlap one column of one "
+                "lane's view): frames of this environment are not trustworthy on this map"
+            )
+
+    # ------------------------------------------------------------------ host-facing API (env.py:750-834)
+    def _view_target(self):
+        """The tensor this call's observation copy goes to, or None for ``unsafe_view`` (env.py:678-688)."""
+        if self.obs_copy == "copy":
+            return torch.empty(self._view_shape, dtype=torch.uint8, device=self.device)
+        if self.obs_copy == "safe_view":
+            buffer = self._safe_obs_buffers[self._safe_obs_index]
+            self._safe_obs_index = (self._safe_obs_index + 1) % len(self._safe_obs_buffers)
+            return buffer
+        return None
+
+    def seed(self, seed=None):
+        self._seed_values = _normalize_seed(seed, self.num_envs)
+        return list(self._seed_values)
+
+    def reset(self, *, seed=None, options=None):
+        if self.closed:
+            raise RuntimeError("cannot reset a closed environment")
+        reset_options = dict(options or {})
+        raw_mask = reset_options.pop("reset_mask", None)
+        if raw_mask is None:
+            mask = torch.ones(self.num_envs, device=self.device, dtype=torch.bool)
+        else:
+            mask = self._require_device_tensor(raw_mask, "options['reset_mask']", shape=(self.num_envs,), dtypes=(torch.bool,))
+        if not bool(torch.any(mask)):
+            raise ValueError("options['reset_mask'] must select at least one lane")
+        if reset_options:
+            raise ValueError(f"unsupported reset options: {sorted(reset_options)}")
+        seed_values = _normalize_seed(seed, self.num_envs) if seed is not None else self._seed_values
+        game_seeds = [0] * self.num_envs
+        for lane in torch.nonzero(mask, as_tuple=False).flatten().to("cpu").tolist():
+            if seed_values[lane] is not None:
+                self._reset_rngs[lane] = np.random.default_rng(seed_values[lane])
+            game_seeds[lane] = int(self._reset_rngs[lane].integers(0, np.iinfo(np.uint32).max + 1, dtype=np.uint32))
+        self._seed_values = [None] * self.num_envs
+        seeds = torch.tensor(game_seeds, device=self.device, dtype=torch.int64)
+        view = self._view_target()
+        observations, _ = self._reset(mask, seeds, view)
+        return (observations if view is None else view), {}
+
+    def step(self, actions: torch.Tensor):
+        if self.closed:
+            raise RuntimeError("cannot step a closed environment")
+        if not bool(torch.all(self._initialized)):
+            raise RuntimeError("all lanes must be reset before the first step")
+        view = self._view_target()
+        transition = self._step(actions, view, self.obs_layout)
+        observations = transition.observations if view is None else view
+        return observations, transition.rewards, transition.terminated, transition.truncated, {}
 
     # ------------------------------------------------------------------ RGB frames
     def _rgb_frames(self) -> torch.Tensor:
@@ -241,7 +339,9 @@ class GraDoomVecEnv:
             raise IndexError(f"lane must be in [0, {self.num_envs - 1}]")
         if self.render_mode != "rgb_array":
             return None
-        return self._rgb_frames()[lane_index].detach().to("cpu").numpy().copy()
+        frame = self._rgb_frames()[lane_index].detach().to("cpu").numpy().copy()
+        self.check_renderer_status()
+        return frame
 
     def render(self):
         return self.render_lane(0)
@@ -252,11 +352,18 @@ class GraDoomVecEnv:
         if self.render_mode != "rgb_array":
             return [None for _ in range(self.num_envs)]
         frames = self._rgb_frames().detach().to("cpu").numpy()
+        self.check_renderer_status()
         return [frame.copy() for frame in frames]
 
     def close(self) -> None:
         if not self.closed:
             self.closed = True
-            close = getattr(self._renderer, "close", None)
-            if close is not None:
-                close()
+            try:
+                self.check_renderer_status()
+            finally:
+                self._close_renderer()
+
+    def _close_renderer(self) -> None:
+        close = getattr(self._renderer, "close", None)
+        if close is not None:
+            close()

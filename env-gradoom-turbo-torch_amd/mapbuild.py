@@ -155,14 +155,14 @@ def build_map_tables(smap) -> dict[str, np.ndarray | int]:
 
     # engine.py:1558-1575: argmax over the start / end flags picks the first set slot (0 when none)
     direct_table = np.zeros((wall_count, 4), dtype=np.int32)
-    for w in range(wall_count):
-        start_slot = int(np.argmax(neighbor_starts[w]))
-        end_slot = int(np.argmax(neighbor_ends[w]))
-        direct_table[w, 0] = endpoint_neighbors[w, start_slot]
-        direct_table[w, 1] = endpoint_neighbors[w, end_slot]
-        direct_table[w, 2] = (
-            start_slot | (end_slot << 8) | (int(neighbor_starts[w].any()) << 16) | (int(neighbor_ends[w].any()) << 17)
-        )
+    every = np.arange(wall_count)
+    start_slot = np.argmax(neighbor_starts, axis=1)
+    end_slot = np.argmax(neighbor_ends, axis=1)
+    direct_table[:, 0] = endpoint_neighbors[every, start_slot]
+    direct_table[:, 1] = endpoint_neighbors[every, end_slot]
+    direct_table[:, 2] = (
+        start_slot | (end_slot << 8) | (neighbor_starts.any(axis=1).astype(np.int64) << 16) | (neighbor_ends.any(axis=1).astype(np.int64) << 17)
+    )
 
     # One-hop solid bridges (engine.py:787-830): bridge[w] = { k : exists j one-sided,
     # sharing w's start (resp. end), with sectors[j,0] in sectors[w], and k one-sided,
@@ -298,24 +298,31 @@ GRID_PAD = 0.5
 GRID_ALWAYS_INSIDE = 1 << 30  # flag on a grid item: every point of the cell is inside that sector
 
 
-def _any_segment_near_box(segments: np.ndarray, x0: float, y0: float, x1: float, y1: float) -> bool:
-    """True when some segment [x1,y1,x2,y2] intersects the axis-aligned box (Liang-Barsky clip)."""
+def _segments_near_boxes(segments: np.ndarray, x0, y0, x1, y1) -> np.ndarray:
+    """For every axis-aligned box (``x0..y1`` broadcast against each other with a trailing axis of length one): does
+    some segment [x1,y1,x2,y2] intersect it (Liang-Barsky clip)?  Returns the boxes' shape without the trailing axis."""
 
     px, py = segments[:, 0], segments[:, 1]
     dx, dy = segments[:, 2] - px, segments[:, 3] - py
-    t0 = np.zeros(len(segments))
-    t1 = np.ones(len(segments))
-    alive = np.ones(len(segments), dtype=bool)
+    t0, t1, alive = 0.0, 1.0, True
     for p, q in ((-dx, px - x0), (dx, x1 - px), (-dy, py - y0), (dy, y1 - py)):
         parallel = p == 0
-        alive &= ~(parallel & (q < 0))
+        alive = alive & ~(parallel & (q < 0))
         with np.errstate(divide="ignore", invalid="ignore"):
             r = np.where(parallel, 0.0, q / np.where(parallel, 1.0, p))
-        entering = (p < 0) & ~parallel
-        leaving = (p > 0) & ~parallel
-        t0 = np.where(entering, np.maximum(t0, r), t0)
-        t1 = np.where(leaving, np.minimum(t1, r), t1)
-    return bool(np.any(alive & (t0 <= t1)))
+        t0 = np.where((p < 0) & ~parallel, np.maximum(t0, r), t0)
+        t1 = np.where((p > 0) & ~parallel, np.minimum(t1, r), t1)
+    return np.any(alive & (t0 <= t1), axis=-1)
+
+
+def _points_in_polygon(segments: np.ndarray, x, y) -> np.ndarray:
+    """Even-odd test of the points (``x``, ``y`` broadcast, trailing axis of length one) against the segments."""
+
+    x1, y1, x2, y2 = segments[:, 0], segments[:, 1], segments[:, 2], segments[:, 3]
+    crosses = (y1 > y) != (y2 > y)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        crossing_x = x1 + (y - y1) * (x2 - x1) / np.where(y2 == y1, 1.0, y2 - y1)
+    return (np.count_nonzero(crosses & (x < crossing_x), axis=-1) & 1).astype(bool)
 
 
 FINE_CELL = 8.0
@@ -325,6 +332,27 @@ FINE_EMPTY = 0x40000000     # fine cell wholly outside every sector
 FINE_MIXED = 0x80000000     # crossing test needed; bits 0..14 / 15..29 = floor / ceiling levels that can win there
 FINE_UNKNOWN = 0xC0000000   # crossing test needed, nothing known about the levels
 FINE_MASK_LEVELS = 15
+
+
+def closed_boundaries(walls, sector_edge_ofs, sector_edge_idx, sector_count: int) -> np.ndarray:
+    """bool [S]: is the sector's boundary a set of closed loops (every vertex touched by an even number of its edges)?"""
+
+    counts = np.diff(sector_edge_ofs[: sector_count + 1])
+    sector = np.repeat(np.arange(sector_count), counts)
+    edges = np.asarray(sector_edge_idx[: sector_edge_ofs[sector_count]], dtype=np.int64)
+    segments = np.asarray(walls)[edges]
+    owner = np.concatenate([sector, sector])
+    x = np.concatenate([segments[:, 0], segments[:, 2]]) + 0.0   # + 0.0: -0.0 and 0.0 are one vertex
+    y = np.concatenate([segments[:, 1], segments[:, 3]]) + 0.0
+    order = np.lexsort((y, x, owner))
+    owner, x, y = owner[order], x[order], y[order]
+    starts = np.ones(len(owner), dtype=bool)
+    starts[1:] = (owner[1:] != owner[:-1]) | (x[1:] != x[:-1]) | (y[1:] != y[:-1])
+    run_start = np.nonzero(starts)[0]
+    run_length = np.diff(np.concatenate([run_start, [len(owner)]]))
+    odd = np.zeros(sector_count, dtype=bool)
+    np.logical_or.at(odd, owner[run_start], run_length % 2 == 1)
+    return ~odd
 
 
 def fine_cell_size(walls) -> float:
@@ -362,21 +390,66 @@ def build_fine_grid(walls, sector_edge_ofs, sector_edge_idx, sector_count, min_x
     level_bits = np.zeros((ny, nx), dtype=np.uint32)
     owners = np.zeros((ny, nx), dtype=np.int32)
     owner = np.full((ny, nx), FINE_EMPTY, dtype=np.uint32)
+    sector_bits = np.zeros(sector_count, dtype=np.uint32)
+    sector_level_index = np.full(sector_count, 0xFF << 16, dtype=np.uint32)  # decided cells: floor / ceiling level index in bits 16..19 / 20..23, 15 = unknown
+    if masks_known:
+        # position of each sector's height in the level lists (at most FINE_MASK_LEVELS entries, in the caller's order)
+        floor_index = np.argmax(np.asarray(floor_levels)[None, :] == sector_heights[:, 0:1], axis=1).astype(np.uint32)
+        ceil_index = np.argmax(np.asarray(ceil_levels)[None, :] == sector_heights[:, 1:2], axis=1).astype(np.uint32)
+        sector_bits = (np.uint32(1) << floor_index) | (np.uint32(1) << (np.uint32(FINE_MASK_LEVELS) + ceil_index))
+        sector_level_index = (floor_index << np.uint32(16)) | (ceil_index << np.uint32(20))
+    closed_sector = closed_boundaries(walls64, sector_edge_ofs, sector_edge_idx, sector_count)
+    edge_counts = np.diff(sector_edge_ofs)
+    pair_sector = np.repeat(np.arange(sector_count), edge_counts)       # one entry per (sector, edge of its boundary)
+    pair_edge = np.asarray(sector_edge_idx[: sector_edge_ofs[sector_count]], dtype=np.int64)
+    in_closed = closed_sector[pair_sector]
+
+    # cells that an edge of a closed sector comes near: every (edge, cell of its padded bounding box) at once
+    edges = np.unique(pair_edge[in_closed])
+    x1, y1, x2, y2 = (walls64[edges, k] for k in range(4))
+    ex0 = np.maximum(np.floor((np.minimum(x1, x2) - GRID_PAD - min_x) / cell).astype(np.int64), 0)
+    ex1 = np.minimum(np.floor((np.maximum(x1, x2) + GRID_PAD - min_x) / cell).astype(np.int64), nx - 1)
+    ey0 = np.maximum(np.floor((np.minimum(y1, y2) - GRID_PAD - min_y) / cell).astype(np.int64), 0)
+    ey1 = np.minimum(np.floor((np.maximum(y1, y2) + GRID_PAD - min_y) / cell).astype(np.int64), ny - 1)
+    box_w, box_h = np.maximum(ex1 - ex0 + 1, 0), np.maximum(ey1 - ey0 + 1, 0)
+    box_cells = box_w * box_h
+    box_start = np.concatenate([[0], np.cumsum(box_cells)])
+    of_edge = np.repeat(np.arange(len(edges)), box_cells)               # which edge each listed cell belongs to
+    local = np.arange(box_start[-1]) - box_start[of_edge]
+    cell_y = ey0[of_edge] + local // np.maximum(box_w[of_edge], 1)
+    cell_x = ex0[of_edge] + local % np.maximum(box_w[of_edge], 1)
+    # Liang-Barsky clip of the segment against the padded cell box; an edge along an axis, or whose box is one cell
+    # wide or high, is near every cell of its box
+    trivial = (ex0 == ex1) | (ey0 == ey1) | (x1 == x2) | (y1 == y2)
+    bx0 = min_x + cell_x * cell - GRID_PAD
+    by0 = min_y + cell_y * cell - GRID_PAD
+    bx1 = bx0 + cell + 2 * GRID_PAD
+    by1 = by0 + cell + 2 * GRID_PAD
+    dx, dy = (x2 - x1)[of_edge], (y2 - y1)[of_edge]
+    with np.errstate(divide="ignore", invalid="ignore"):
+        tx_a, tx_b = (bx0 - x1[of_edge]) / dx, (bx1 - x1[of_edge]) / dx
+        ty_a, ty_b = (by0 - y1[of_edge]) / dy, (by1 - y1[of_edge]) / dy
+        t_in = np.maximum(np.maximum(np.minimum(tx_a, tx_b), np.minimum(ty_a, ty_b)), 0.0)
+        t_out = np.minimum(np.minimum(np.maximum(tx_a, tx_b), np.maximum(ty_a, ty_b)), 1.0)
+        near = trivial[of_edge] | (t_in <= t_out)
+    near_flat = (cell_y * nx + cell_x)[near]
+    near_edge = of_edge[near]
+    mixed.reshape(-1)[near_flat] = True
+    if masks_known:
+        # the levels of both sectors an edge bounds (closed ones) reach every cell the edge comes near
+        edge_slot = np.full(len(walls64), -1, dtype=np.int64)
+        edge_slot[edges] = np.arange(len(edges))
+        edge_bits = np.zeros(len(edges), dtype=np.uint32)
+        np.bitwise_or.at(edge_bits, edge_slot[pair_edge[in_closed]], sector_bits[pair_sector[in_closed]])
+        np.bitwise_or.at(level_bits.reshape(-1), near_flat, edge_bits[near_edge])
+
     for s in range(sector_count):
         edges = sector_edge_idx[sector_edge_ofs[s] : sector_edge_ofs[s + 1]]
         if len(edges) == 0:
             continue
-        bits = np.uint32(0)
-        level_index = np.uint32(0xFF << 16)  # decided cells: floor / ceiling level index in bits 16..19 / 20..23, 15 = unknown
-        if masks_known:
-            floor_index = int(np.nonzero(floor_levels == sector_heights[s, 0])[0][0])
-            ceil_index = int(np.nonzero(ceil_levels == sector_heights[s, 1])[0][0])
-            bits = np.uint32((1 << floor_index) | (1 << (FINE_MASK_LEVELS + ceil_index)))
-            level_index = np.uint32((floor_index << 16) | (ceil_index << 20))
+        bits, level_index = sector_bits[s], sector_level_index[s]
         seg = walls64[edges]
-        ends = np.concatenate([seg[:, 0:2], seg[:, 2:4]]) + 0.0
-        _, counts = np.unique(ends, axis=0, return_counts=True)
-        closed = bool(np.all(counts % 2 == 0))
+        closed = bool(closed_sector[s])
         ix0 = 0 if not closed else max(int(np.floor((seg[:, (0, 2)].min() - GRID_PAD - min_x) / cell)), 0)
         ix1 = min(int(np.floor((seg[:, (0, 2)].max() + GRID_PAD - min_x) / cell)), nx - 1)
         iy0 = max(int(np.floor((seg[:, (1, 3)].min() - GRID_PAD - min_y) / cell)), 0)
@@ -387,38 +460,10 @@ def build_fine_grid(walls, sector_edge_ofs, sector_edge_idx, sector_count, min_x
             mixed[iy0 : iy1 + 1, ix0 : ix1 + 1] = True
             level_bits[iy0 : iy1 + 1, ix0 : ix1 + 1] |= bits
             continue
-        # cells that an edge of this sector comes near
-        for x1, y1, x2, y2 in seg:
-            ex0 = max(int(np.floor((min(x1, x2) - GRID_PAD - min_x) / cell)), 0)
-            ex1 = min(int(np.floor((max(x1, x2) + GRID_PAD - min_x) / cell)), nx - 1)
-            ey0 = max(int(np.floor((min(y1, y2) - GRID_PAD - min_y) / cell)), 0)
-            ey1 = min(int(np.floor((max(y1, y2) + GRID_PAD - min_y) / cell)), ny - 1)
-            if ex1 < ex0 or ey1 < ey0:
-                continue
-            if ex0 == ex1 or ey0 == ey1 or x1 == x2 or y1 == y2:
-                near = np.ones((ey1 - ey0 + 1, ex1 - ex0 + 1), dtype=bool)
-            else:
-                # Liang-Barsky clip of the segment against every padded cell box of its bounding box
-                bx0 = (min_x + np.arange(ex0, ex1 + 1) * cell - GRID_PAD)[None, :]
-                by0 = (min_y + np.arange(ey0, ey1 + 1) * cell - GRID_PAD)[:, None]
-                bx1 = bx0 + cell + 2 * GRID_PAD
-                by1 = by0 + cell + 2 * GRID_PAD
-                dx, dy = x2 - x1, y2 - y1
-                tx_a, tx_b = (bx0 - x1) / dx, (bx1 - x1) / dx
-                ty_a, ty_b = (by0 - y1) / dy, (by1 - y1) / dy
-                t_in = np.maximum(np.maximum(np.minimum(tx_a, tx_b), np.minimum(ty_a, ty_b)), 0.0)
-                t_out = np.minimum(np.minimum(np.maximum(tx_a, tx_b), np.maximum(ty_a, ty_b)), 1.0)
-                near = t_in <= t_out
-            mixed[ey0 : ey1 + 1, ex0 : ex1 + 1] |= near
-            level_bits[ey0 : ey1 + 1, ex0 : ex1 + 1] |= np.where(near, bits, np.uint32(0))
         # cells whose centre the sector contains
         cx = (min_x + (np.arange(ix0, ix1 + 1) + 0.5) * cell)[None, :, None]
         cy = (min_y + (np.arange(iy0, iy1 + 1) + 0.5) * cell)[:, None, None]
-        ex1_, ey1_, ex2_, ey2_ = (seg[:, k][None, None, :] for k in range(4))
-        crosses = (ey1_ > cy) != (ey2_ > cy)
-        with np.errstate(divide="ignore", invalid="ignore"):
-            crossing_x = ex1_ + (cy - ey1_) * (ex2_ - ex1_) / np.where(ey2_ == ey1_, 1.0, ey2_ - ey1_)
-        inside = (np.count_nonzero(crosses & (cx < crossing_x), axis=2) & 1).astype(bool)
+        inside = _points_in_polygon(seg, cx, cy)
         view_owners = owners[iy0 : iy1 + 1, ix0 : ix1 + 1]
         view_owner = owner[iy0 : iy1 + 1, ix0 : ix1 + 1]
         view_owner[inside & (view_owners == 0)] = np.uint32(s) | level_index
@@ -427,14 +472,6 @@ def build_fine_grid(walls, sector_edge_ofs, sector_edge_idx, sector_count, min_x
     mixed |= owners > 1
     owner[mixed] = (np.uint32(FINE_MIXED) | level_bits[mixed]) if masks_known else np.uint32(FINE_UNKNOWN)
     return dict(fine_nx=nx, fine_ny=ny, fine_cell=float(cell), fine_sector=np.ascontiguousarray(owner.reshape(-1)))
-
-
-def _point_in_polygon(segments: np.ndarray, x: float, y: float) -> bool:
-    x1, y1, x2, y2 = segments[:, 0], segments[:, 1], segments[:, 2], segments[:, 3]
-    crosses = (y1 > y) != (y2 > y)
-    with np.errstate(divide="ignore", invalid="ignore"):
-        crossing_x = x1 + (y - y1) * (x2 - x1) / np.where(y2 == y1, 1.0, y2 - y1)
-    return bool(np.count_nonzero(crosses & (x < crossing_x)) & 1)
 
 
 def build_sector_grid(walls, sector_edge_ofs, sector_edge_idx, sector_count, cell: float = GRID_CELL) -> dict:
@@ -458,19 +495,15 @@ def build_sector_grid(walls, sector_edge_ofs, sector_edge_idx, sector_count, cel
     min_y = float(np.floor(all_y.min() - 2 * GRID_PAD))
     nx = int(np.ceil((float(all_x.max()) + 2 * GRID_PAD - min_x) / cell)) + 1
     ny = int(np.ceil((float(all_y.max()) + 2 * GRID_PAD - min_y) / cell)) + 1
-    cell_rows: list[list[tuple[int, list[int]]]] = [[] for _ in range(nx * ny)]
+    closed_sector = closed_boundaries(walls, sector_edge_ofs, sector_edge_idx, sector_count)
+    item_cells, item_sectors, item_counts, item_edge_lists = [], [], [], []
     for s in range(sector_count):
         edges = sector_edge_idx[sector_edge_ofs[s] : sector_edge_ofs[s + 1]]
         if len(edges) == 0:
             continue
         ex = walls[edges][:, (0, 2)]
         ey = walls[edges][:, (1, 3)]
-        degree: dict[tuple[float, float], int] = {}
-        for w in edges:
-            for slot in range(2):
-                key = (float(walls[w, 2 * slot]) + 0.0, float(walls[w, 2 * slot + 1]) + 0.0)
-                degree[key] = degree.get(key, 0) + 1
-        closed = all(count % 2 == 0 for count in degree.values())
+        closed = bool(closed_sector[s])
         sx0 = -np.inf if not closed else float(ex.min()) - GRID_PAD
         sx1 = float(ex.max()) + GRID_PAD
         sy0 = float(ey.min()) - GRID_PAD
@@ -479,38 +512,56 @@ def build_sector_grid(walls, sector_edge_ofs, sector_edge_idx, sector_count, cel
         ix1 = min(int(np.floor((sx1 - min_x) / cell)), nx - 1)
         iy0 = max(int(np.floor((sy0 - min_y) / cell)), 0)
         iy1 = min(int(np.floor((sy1 - min_y) / cell)), ny - 1)
+        if ix1 < ix0 or iy1 < iy0:
+            continue
         edge_max_x = ex.max(axis=1)
         edge_min_y = ey.min(axis=1)
         edge_max_y = ey.max(axis=1)
         segments = walls[edges].astype(np.float64)
-        for iy in range(iy0, iy1 + 1):
-            cy0 = min_y + iy * cell - GRID_PAD
-            cy1 = min_y + (iy + 1) * cell + GRID_PAD
-            row_mask = (edge_max_y >= cy0) & (edge_min_y <= cy1)
-            for ix in range(ix0, ix1 + 1):
-                cx0 = (min_x + ix * cell - GRID_PAD) if ix > 0 else -np.inf
-                cx1 = min_x + (ix + 1) * cell + GRID_PAD
-                keep = row_mask & (edge_max_x >= cx0)
-                # A cell that no edge of the sector comes near (padded by GRID_PAD, far more than the
-                # float32 error of the crossing test) lies wholly inside or wholly outside the sector:
-                # decide once at its centre and spare the kernels every edge test there.
-                if closed and ix > 0 and not _any_segment_near_box(segments, cx0, cy0, cx1, cy1):
-                    centre_x = min_x + (ix + 0.5) * cell
-                    centre_y = min_y + (iy + 0.5) * cell
-                    if _point_in_polygon(segments, centre_x, centre_y):
-                        cell_rows[iy * nx + ix].append((s | GRID_ALWAYS_INSIDE, []))
-                    continue
-                cell_rows[iy * nx + ix].append((s, [int(w) for w in edges[keep]]))
-    cell_ofs = np.zeros(nx * ny + 1, dtype=np.int32)
-    item_sector: list[int] = []
-    item_edge_ofs = [0]
-    item_edges: list[int] = []
-    for c, row in enumerate(cell_rows):
-        for s, sub in row:  # sectors were appended in ascending order
-            item_sector.append(s)
-            item_edges.extend(sub)
-            item_edge_ofs.append(len(item_edges))
-        cell_ofs[c + 1] = len(item_sector)
+        # every cell of the sector's box at once: [rows, columns, edges]
+        columns = np.arange(ix0, ix1 + 1)
+        rows = np.arange(iy0, iy1 + 1)
+        cx0 = np.where(columns > 0, min_x + columns * cell - GRID_PAD, -np.inf)[None, :, None]
+        cx1 = (min_x + (columns + 1) * cell + GRID_PAD)[None, :, None]
+        cy0 = (min_y + rows * cell - GRID_PAD)[:, None, None]
+        cy1 = (min_y + (rows + 1) * cell + GRID_PAD)[:, None, None]
+        keep = ((edge_max_y[None, None, :] >= cy0) & (edge_min_y[None, None, :] <= cy1)) & (edge_max_x[None, None, :] >= cx0)
+        # A cell that no edge of the sector comes near (padded by GRID_PAD, far more than the
+        # float32 error of the crossing test) lies wholly inside or wholly outside the sector:
+        # decide once at its centre and spare the kernels every edge test there.
+        decided = np.zeros((len(rows), len(columns)), dtype=bool)
+        inside = np.zeros_like(decided)
+        if closed:
+            first = 1 if ix0 == 0 else 0   # the leftmost column of the grid stands for everything to its left
+            if len(columns) > first:
+                decided[:, first:] = ~_segments_near_boxes(segments, cx0[:, first:], cy0, cx1[:, first:], cy1)
+                centre_x = (min_x + (columns + 0.5) * cell)[None, :, None]
+                centre_y = (min_y + (rows + 0.5) * cell)[:, None, None]
+                inside = decided & _points_in_polygon(segments, centre_x, centre_y)
+        # one item per cell that lists the sector: decided cells inside it (no edges), undecided cells (their sub-list)
+        listed = ~decided | inside
+        keep &= ~decided[:, :, None]
+        cell_index = (rows[:, None] * nx + columns[None, :])[listed]
+        item_cells.append(cell_index)
+        item_sectors.append(np.where(inside[listed], s | GRID_ALWAYS_INSIDE, s))
+        item_counts.append(np.count_nonzero(keep, axis=2)[listed])
+        item_edge_lists.append(np.asarray(edges)[np.nonzero(keep)[2]])   # row-major over (row, column, edge): cell by cell
+    # gather the items cell by cell; within a cell they stay in the order they were made, ascending by sector
+    if item_cells:
+        cells = np.concatenate(item_cells)
+        order = np.argsort(cells, kind="stable")
+        counts = np.concatenate(item_counts)
+        starts = np.concatenate([[0], np.cumsum(counts)])[:-1]
+        counts_sorted = counts[order]
+        sorted_starts = np.concatenate([[0], np.cumsum(counts_sorted)])
+        gather = np.repeat(starts[order], counts_sorted) + (np.arange(sorted_starts[-1]) - np.repeat(sorted_starts[:-1], counts_sorted))
+        item_edges = np.concatenate(item_edge_lists)[gather]
+        item_sector = np.concatenate(item_sectors)[order]
+        item_edge_ofs = sorted_starts
+        cell_ofs = np.concatenate([[0], np.cumsum(np.bincount(cells, minlength=nx * ny))]).astype(np.int32)
+    else:
+        item_edges, item_sector, item_edge_ofs = np.zeros(0, np.int64), np.zeros(0, np.int64), np.zeros(1, np.int64)
+        cell_ofs = np.zeros(nx * ny + 1, dtype=np.int32)
     return dict(
         grid_nx=nx,
         grid_ny=ny,
@@ -518,7 +569,7 @@ def build_sector_grid(walls, sector_edge_ofs, sector_edge_idx, sector_count, cel
         grid_min_y=min_y,
         grid_cell=float(cell),
         grid_cell_ofs=cell_ofs,
-        grid_item_sector=np.asarray(item_sector if item_sector else [0], dtype=np.int32),  # | GRID_ALWAYS_INSIDE
+        grid_item_sector=np.asarray(item_sector if len(item_sector) else [0], dtype=np.int32),  # | GRID_ALWAYS_INSIDE
         grid_item_edge_ofs=np.asarray(item_edge_ofs, dtype=np.int32),
-        grid_item_edges=np.asarray(item_edges if item_edges else [0], dtype=np.int32),
+        grid_item_edges=np.asarray(item_edges if len(item_edges) else [0], dtype=np.int32),
     )

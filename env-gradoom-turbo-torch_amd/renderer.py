@@ -227,7 +227,8 @@ class HipRenderer:
             desc.hud_state = _require(lanes.hud_state, "hud_state", torch.int32, (count, 9), device).data_ptr()
         return desc, keep
 
-    def _out_desc(self, count, indexed, obs, frames, reset_mask, rgb, stack_only_masked=False, final_frames=None, obs_source_rows=208):
+    def _out_desc(self, count, indexed, obs, frames, reset_mask, rgb, stack_only_masked=False, final_frames=None, obs_source_rows=208,
+                  final_layout="chw"):
         device = self.device
         out = _abi.FrameOut()
         out.stack_mode = _abi.STACK_RESET if stack_only_masked else _abi.STACK_STEP
@@ -250,12 +251,16 @@ class HipRenderer:
         if final_frames is not None:
             if frames is None:
                 raise ValueError("final_frames needs frames")
-            out.final_frames = _require(final_frames, "final_frames", torch.uint8, (count, 4, 84, 84), device).data_ptr()
+            if final_layout not in ("chw", "hwc"):
+                raise ValueError("final_layout must be 'chw' or 'hwc'")
+            shape = (count, 4, 84, 84) if final_layout == "chw" else (count, 84, 84, 4)
+            out.final_frames = _require(final_frames, "final_frames", torch.uint8, shape, device).data_ptr()
+            out.final_frames_layout = _abi.LAYOUT_HWC if final_layout == "hwc" else _abi.LAYOUT_CHW
         return out, keep
 
     # ------------------------------------------------------------------ entry points
     def render(self, lanes: LaneState, *, indexed=None, obs=None, frames=None, reset_mask=None, rgb=None,
-               stack_only_masked: bool = False, final_frames=None, obs_source_rows: int = 208) -> None:
+               stack_only_masked: bool = False, final_frames=None, obs_source_rows: int = 208, final_layout: str = "chw") -> None:
         """One frame for every lane, written into the given (preallocated) tensors.
 
         ``frames`` is rolled by one and the new observation appended (``engine.py:9545-9548``); lanes
@@ -265,13 +270,16 @@ class HipRenderer:
         ``step_and_reset_device`` returns as ``final_observations`` (``env.py:915-917``), written by
         the observation kernel itself.  ``obs_source_rows=240`` pools the status bar rows into the observation
         instead of masking them black, as an environment made with ``obs_crop=None`` does (``env.py:441``,
-        ``engine.py:15440``).
+        ``engine.py:15440``).  ``final_layout="hwc"`` makes ``final_frames`` a ``(N, 84, 84, 4)`` tensor holding
+        what ``frames.permute(0, 2, 3, 1)`` shows: the buffer an ``obs_layout="hwc"`` environment hands out
+        (``env.py:678-688``).
         """
 
         if self._handle is None:
             raise RuntimeError("renderer is closed")
         desc, keep_lanes = self._lanes_desc(lanes)
-        out, keep_out = self._out_desc(desc.lane_count, indexed, obs, frames, reset_mask, rgb, stack_only_masked, final_frames, obs_source_rows)
+        out, keep_out = self._out_desc(desc.lane_count, indexed, obs, frames, reset_mask, rgb, stack_only_masked, final_frames, obs_source_rows,
+                                       final_layout)
         stream = torch.cuda.current_stream(self.device).cuda_stream
         _lib.check(self._lib.gd_render(self._handle, C.byref(desc), C.byref(out), C.c_void_p(stream)))
         del keep_lanes, keep_out

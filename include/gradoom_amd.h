@@ -32,11 +32,15 @@ extern "C" {
 #define GD_STACK_STEP 0   /* every lane: roll by one, append (engine.py:9545-9548); lanes with reset_mask set: 4 copies */
 #define GD_STACK_RESET 1  /* lanes with reset_mask set: 4 copies (engine.py:2443-2450); other lanes untouched */
 
+/* gd_frame_out.final_frames_layout: how final_frames is laid out (obs_layout of env.py:351, 678-680) */
+#define GD_LAYOUT_CHW 0   /* [N,4,84,84], like frames */
+#define GD_LAYOUT_HWC 1   /* [N,84,84,4]: what frames.permute(0, 2, 3, 1) reads, made contiguous */
+
 /*
  * Layout version of the structs below.  Every descriptor also starts with its own sizeof, which each entry
  * point checks: a caller built against another header gets GD_E_ARG instead of a wild read.
  */
-#define GD_ABI_VERSION 2
+#define GD_ABI_VERSION 3
 
 #define GD_OK 0
 #define GD_E_ARG (-1)       /* bad argument: null pointer, negative count, size over a limit */
@@ -230,6 +234,9 @@ typedef struct gd_frame_out {
                                 black (render_reference_frame with mask_hud, engine.py:15444-15450); 240 = the status bar
                                 too, as the reference does when the environment is made with obs_crop=None
                                 (env.py:441, engine.py:15440) */
+    int32_t final_frames_layout; /* GD_LAYOUT_CHW or GD_LAYOUT_HWC.  With it final_frames doubles as the observation copy
+                                    the host API hands out (obs_copy "copy" / "safe_view", env.py:678-688): the caller
+                                    passes the buffer it would have copied into and no copy kernel runs */
 } gd_frame_out;
 
 typedef struct gd_renderer gd_renderer;

@@ -15,8 +15,14 @@ class RecordingRenderer:
     def __init__(self):
         self.calls = []
 
-    def render(self, lanes, *, indexed=None, obs=None, frames=None, reset_mask=None, rgb=None, stack_only_masked=False, final_frames=None):
-        self.calls.append(dict(reset=stack_only_masked, mask=None if reset_mask is None else reset_mask.clone()))
+    status_value = 0
+
+    def status(self):
+        return self.status_value
+
+    def render(self, lanes, *, indexed=None, obs=None, frames=None, reset_mask=None, rgb=None, stack_only_masked=False, final_frames=None,
+               final_layout="chw"):
+        self.calls.append(dict(reset=stack_only_masked, mask=None if reset_mask is None else reset_mask.clone(), final=final_frames, layout=final_layout))
         value = (lanes.x.abs().to(torch.int64) % 251).to(torch.uint8)
         if frames is not None:
             new = value[:, None, None].expand(-1, 84, 84)
@@ -27,7 +33,7 @@ class RecordingRenderer:
                     frames[lane] = torch.roll(frames[lane], -1, 0)
                     frames[lane, -1] = new[lane]
             if final_frames is not None:
-                final_frames.copy_(frames)
+                final_frames.copy_(frames if final_layout == "chw" else frames.permute(0, 2, 3, 1))
         if rgb is not None:
             rgb.copy_(value[:, None, None, None].expand_as(rgb))
 
@@ -121,3 +127,90 @@ def test_render_mode_none_returns_none():
     _meta, _data, smap, _tables = load_fixture("tiny_stages")
     env = GraDoomVecEnv(smap, 2, device="cpu", renderer=RecordingRenderer())
     assert env.render() is None and env.get_images() == [None, None]
+
+
+def _host_env(obs_copy, obs_layout="chw"):
+    from gradoom_amd.env import GraDoomVecEnv
+
+    _meta, _data, smap, _tables = load_fixture("tiny_stages")
+    renderer = RecordingRenderer()
+    env = GraDoomVecEnv(smap, 4, device="cpu", renderer=renderer, episode_timeout=50, obs_copy=obs_copy, obs_layout=obs_layout)
+    return env, renderer
+
+
+def test_obs_copy_modes_follow_the_reference_ownership_rules():
+    # env.py:678-688: "copy" hands out a fresh tensor, "safe_view" two buffers in turn, "unsafe_view" the stack itself
+    from gradoom_amd.env import GraDoomVecEnv
+
+    with pytest.raises(ValueError, match="obs_copy must be copy, safe_view, or unsafe_view"):
+        GraDoomVecEnv(load_fixture("tiny_stages")[2], 4, device="cpu", renderer=RecordingRenderer(), obs_copy="view")
+    actions = torch.zeros(4, dtype=torch.int64)
+
+    env, renderer = _host_env("safe_view")
+    assert (env.observation_ownership, env.observation_buffer_depth) == ("safe_view", 2)
+    first, info = env.reset(seed=3)
+    assert info == {} and first.data_ptr() != env.frames.data_ptr() and torch.equal(first, env.frames)
+    held = first.clone()
+    second = env.step(actions)[0]
+    assert second.data_ptr() != first.data_ptr() and torch.equal(first, held), "the observation of the step before stays valid"
+    third = env.step(actions)[0]
+    assert third.data_ptr() == first.data_ptr() and torch.equal(third, env.frames)
+    assert all(call["final"] is not None for call in renderer.calls), "the renderer writes the view itself: no copy pass"
+
+    env, renderer = _host_env("copy")
+    assert (env.observation_ownership, env.observation_buffer_depth) == ("owned", None)
+    first = env.reset(seed=3)[0]
+    second = env.step(actions)[0]
+    third = env.step(actions)[0]
+    assert len({first.data_ptr(), second.data_ptr(), third.data_ptr(), env.frames.data_ptr()}) == 4
+
+    env, renderer = _host_env("unsafe_view")
+    assert (env.observation_ownership, env.observation_buffer_depth) == ("unsafe_view", 1)
+    first = env.reset(seed=3)[0]
+    assert first.data_ptr() == env.frames.data_ptr() and renderer.calls[-1]["final"] is None
+    assert env.step(actions)[0].data_ptr() == env.frames.data_ptr()
+
+
+def test_host_api_layout_seeds_and_errors():
+    env, renderer = _host_env("safe_view", "hwc")
+    actions = torch.zeros(4, dtype=torch.int64)
+    with pytest.raises(RuntimeError, match="all lanes must be reset before the first step"):
+        env.step(actions)
+    with pytest.raises(ValueError, match="must select at least one lane"):
+        env.reset(options={"reset_mask": torch.zeros(4, dtype=torch.bool)})
+    with pytest.raises(ValueError, match="unsupported reset options"):
+        env.reset(options={"difficulty": 3})
+    with pytest.raises(ValueError, match="seed sequence length must match num_envs"):
+        env.reset(seed=[1, 2])
+    observations, _ = env.reset(seed=11)
+    assert observations.shape == (4, 84, 84, 4) and renderer.calls[-1]["layout"] == "hwc"
+    assert torch.equal(observations, env.frames.permute(0, 2, 3, 1))
+    phases = env._dynamics.phase.clone()
+    env.reset(seed=11)
+    assert torch.equal(env._dynamics.phase, phases), "the same seed resets to the same lane state (env.py:785-797)"
+    assert env.seed(5) == [5, 6, 7, 8]
+    env.reset()
+    after_seed_call = env._dynamics.phase.clone()
+    env.reset(seed=5)
+    assert torch.equal(env._dynamics.phase, after_seed_call)
+    observations = env.step(actions)[0]
+    assert observations.shape == (4, 84, 84, 4) and torch.equal(observations, env.frames.permute(0, 2, 3, 1))
+    env.close()
+    with pytest.raises(RuntimeError, match="cannot step a closed environment"):
+        env.step(actions)
+    with pytest.raises(RuntimeError, match="cannot reset a closed environment"):
+        env.reset()
+
+
+def test_truncated_candidate_list_raises_instead_of_passing_a_bad_frame():
+    env, renderer = _host_env("unsafe_view")
+    mask = torch.ones(4, dtype=torch.bool)
+    env.reset_device(mask, torch.arange(4))
+    actions = torch.zeros(4, dtype=torch.int64)
+    env.step_and_reset_device(actions, torch.arange(4))
+    renderer.status_value = 1
+    with pytest.raises(RuntimeError, match="truncated a screen column's candidate list"):
+        env.step_and_reset_device(actions, torch.arange(4))
+    with pytest.raises(RuntimeError, match="truncated"):
+        env.close()
+    assert env.closed and renderer.closed

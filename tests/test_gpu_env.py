@@ -55,3 +55,54 @@ def test_step_and_reset_device_matches_oracle_frame_by_frame(oracle):
     assert np.array_equal(image, np.asarray(tables["playpal"])[third["indexed"][0]])
     assert env._renderer.status() == 0
     env.close()
+
+
+def test_host_api_safe_view_buffers_are_written_by_the_renderer():
+    # reset()/step() hand out two buffers in turn (env.py:459-472, 678-688); they hold the stack, in either layout
+    from gradoom_amd.env import GraDoomVecEnv
+
+    _meta, _data, smap, _tables = load_fixture("small_midtex_sprites")
+    lanes = 6
+    actions = torch.zeros(lanes, dtype=torch.int64, device="cuda:0")
+    for layout in ("chw", "hwc"):
+        env = GraDoomVecEnv(smap, lanes, device="cuda:0", episode_timeout=50, sprites=8, obs_layout=layout, obs_copy="safe_view")
+        view = (lambda t: t) if layout == "chw" else (lambda t: t.permute(0, 2, 3, 1))
+        first, _ = env.reset(seed=4)
+        assert first.data_ptr() != env.frames.data_ptr() and torch.equal(first, view(env.frames))
+        held = first.clone()
+        second = env.step(actions)[0]
+        assert second.data_ptr() != first.data_ptr()
+        assert torch.equal(first, held) and torch.equal(second, view(env.frames))
+        assert not torch.equal(first, second)
+        third = env.step(actions)[0]
+        assert third.data_ptr() == first.data_ptr() and torch.equal(third, view(env.frames))
+        env.close()
+
+
+def test_more_than_64_linedefs_in_one_column_raise_in_the_environment():
+    # A corridor of 80 sectors seen end on: every divider lands in the same screen columns, more than the 64 candidates
+    # the renderer keeps per column.  The environment must say so rather than hand out the frame.
+    from gradoom_amd import synthmap
+    from gradoom_amd.env import GraDoomVecEnv, PosePoolDynamics
+
+    smap = synthmap.generate_map(5, grid=(80, 1), sectors=80, linedefs=241)
+    lanes = 2
+    dynamics = PosePoolDynamics(smap, lanes, "cuda:0", pool=4)
+    quad = smap.sector_quads[0]
+    centre = quad.mean(axis=0)
+    dynamics._pool["x"].fill_(float(centre[0]))
+    dynamics._pool["y"].fill_(float(centre[1]))
+    dynamics._pool["angle_bam"].zero_()       # looking along +x, down the corridor
+    dynamics._pool["pitch_bam"].zero_()
+    dynamics._pool["view_z"].fill_(float(smap.sector_heights[0, 0]) + 41.0)
+    env = GraDoomVecEnv(smap, lanes, device="cuda:0", dynamics=dynamics, render_mode="rgb_array")
+    mask = torch.ones(lanes, dtype=torch.bool, device="cuda:0")
+    env.reset_device(mask, torch.arange(lanes, device="cuda:0"))
+    assert env._renderer.status() & 1
+    with pytest.raises(RuntimeError, match="truncated a screen column's candidate list"):
+        env.step_and_reset_device(torch.zeros(lanes, dtype=torch.int64, device="cuda:0"), torch.arange(lanes, device="cuda:0"))
+    with pytest.raises(RuntimeError, match="truncated"):
+        env.render()
+    with pytest.raises(RuntimeError, match="truncated"):
+        env.close()
+    assert env.closed

@@ -151,6 +151,16 @@ def test_final_frames_and_stack_modes_match_the_oracle(oracle):
         assert np.array_equal(final.cpu().numpy(), expected["frames"]), mode
         assert np.array_equal(obs.cpu().numpy(), expected["obs"]), mode
         assert final.data_ptr() != frames.data_ptr()
+        # the same copy with the four stacked values of a pixel side by side (obs_layout="hwc", env.py:678-680), from
+        # both assemblies
+        for with_frame in (False, True):
+            again = torch.as_tensor(start).to("cuda:0")
+            interleaved = torch.full((count, 84, 84, 4), 9, dtype=torch.uint8, device="cuda:0")
+            renderer.render(lanes, frames=again, final_frames=interleaved, final_layout="hwc",
+                            indexed=scratch_frame if with_frame else None, **kwargs)
+            torch.cuda.synchronize()
+            assert torch.equal(again, frames), (mode, with_frame)
+            assert torch.equal(interleaved, frames.permute(0, 2, 3, 1)), (mode, with_frame)
         if mode == "step":
             assert np.array_equal(ours[:, :3], start[:, 1:]) and np.array_equal(ours[:, 3], expected["obs"])
         if mode == "reset":   # lanes outside the mask keep the stack they had
