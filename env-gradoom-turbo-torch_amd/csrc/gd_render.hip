@@ -2200,69 +2200,126 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
         if (one_sided) { t0 = (int)r.clipped_top; t1 = (int)r.clipped_bottom; }
         if (lower_on) { t0 = min(t0, (int)r.clipped_lower_top); t1 = max(t1, (int)r.clipped_bottom); }
         if (upper_on) { t0 = min(t0, (int)r.clipped_top); t1 = max(t1, (int)r.clipped_upper_bottom); }
-        // what the three tiers need per row, worked out once: texture, column, vertical mapping
         // The texture row of screen row y is bits 32-height_bits .. 31 of
         //   fraction(y) = (texture_mid << (16 - height_bits)) + ((step * (y * 65536 + 65536 - center)) >> 16).
         // step * y * 65536 has no low 16 bits, so it shifts out of the floor unchanged, and only the low 32 bits of
         // the sum are looked at: they advance by the low 32 bits of step per row, whatever the 64-bit terms wrap to.
-        int tier_tex[3]; unsigned tier_frac[3], tier_step[3], tier_shift[3]; size_t tier_texel[3];
-        const float tier_origin[3] = {r.view_ceiling, r.other_floor, r.other_ceiling};
         const float toff_y = toff[1] * 65536.0f;
         const unsigned atlas_w = (unsigned)m->tex_max_w;
+        const int side_tex0 = r.side_tex[0], side_tex1 = r.side_tex[1], side_tex2 = r.side_tex[2];
+        const bool tiers_overlap = lower_on && upper_on && r.clipped_lower_top < r.clipped_upper_bottom;
+        if (!tiers_overlap) {
+            // The usual case: the rows of a tier are one run, [top, bottom) of a one-sided drawseg, or the upper tier
+            // above the lower one.  Each run is painted by a loop that knows its texture, so a row costs an add, a
+            // shift, a texel, a colormap entry and the stores.  WALL_ROWS rows at a time, one batch ahead: the texels
+            // of the next batch are asked for before the rows of this one are stored, so that a step waits for memory
+            // once, not for its stores and then for its loads.
+            auto paint_run = [&](int first, int last, int texture, float origin, bool has_tail, float tail_from) {
+                if (texture < 0 || first >= last) return;
+                const int bits = tb.height_bits(texture);
+                const i64 step64 = mul64(swall, shl64(1, 14 - bits));
+                const i64 base = shl64(round_to_i64((origin - L.view_z) * 65536.0f + toff_y), 16 - bits);
+                const unsigned shift = (unsigned)(31 - bits);   // a one-row texture (bits == 0) must shift everything out: two shifts
+                const unsigned step = (unsigned)step64;
+                unsigned frac = (unsigned)(base + (mul64(step64, FIXED_UNIT - L.center_fixed) >> 16)) + step * (unsigned)first;
+                const unsigned char *column = m->tex_atlas + ((size_t)texture * m->tex_max_h * m->tex_max_w + (size_t)tb.wrap_column(texture, u_base));
+                // rows from tail_row on take the group's shade: (float)y >= tail_from, which no row meets if that is not a number
+                const int tail_row = !has_tail || !(tail_from < (float)VH) ? VH : (tail_from <= 0.0f ? 0 : (int)ceilf(tail_from));
+                const unsigned meta_word = META_FILLED | (unsigned)(wi + 1);
+                auto load_rows = [&](int yb, unsigned char (&texel)[WALL_ROWS]) {
 #pragma unroll
-        for (int t = 0; t < 3; ++t) {
-            tier_tex[t] = r.side_tex[t];
-            const int id = tier_tex[t] < 0 ? 0 : tier_tex[t];
-            const int bits = tb.height_bits(id);
-            const i64 step = mul64(swall, shl64(1, 14 - bits));
-            const i64 base = shl64(round_to_i64((tier_origin[t] - L.view_z) * 65536.0f + toff_y), 16 - bits);
-            tier_shift[t] = (unsigned)(31 - bits);   // a one-row texture (bits == 0) must shift everything out: two shifts
-            tier_step[t] = (unsigned)step;
-            tier_frac[t] = (unsigned)(base + (mul64(step, FIXED_UNIT - L.center_fixed) >> 16)) + (unsigned)step * (unsigned)t0;
-            tier_texel[t] = (size_t)id * m->tex_max_h * m->tex_max_w + (size_t)tb.wrap_column(id, u_base);
-        }
-        // WALL_ROWS rows at a time, one batch ahead: the texels of the next batch are asked for before the rows of
-        // this one are stored, so that a step waits for memory once, not for its stores and then for its loads
-        auto load_rows = [&](int yb, unsigned char (&texel)[WALL_ROWS], unsigned &draw, unsigned &tail) {
-            draw = 0; tail = 0;
+                    for (int j = 0; j < WALL_ROWS; ++j) {
+                        texel[j] = 0;
+                        if (yb + j < last) texel[j] = column[__umul24((frac >> shift) >> 1, atlas_w)];
+                        frac += step;
+                    }
+                };
+                unsigned char texel[WALL_ROWS];
+                load_rows(first, texel);
+                for (int yb = first; yb < last; yb += WALL_ROWS) {
+                    unsigned char next_texel[WALL_ROWS];
 #pragma unroll
-            for (int j = 0; j < WALL_ROWS; ++j) {
-                const int y = yb + j;
-                const float py = (float)y;
-                const bool one_span = one_sided && (py >= r.clipped_top) && (py < r.clipped_bottom);
-                const bool lower_span = lower_on && (py >= r.clipped_lower_top) && (py < r.clipped_bottom);
-                const bool upper_span = upper_on && (py >= r.clipped_top) && (py < r.clipped_upper_bottom);
-                const int t = one_span ? 0 : (lower_span ? 1 : 2);
-                const bool draws = y < t1 && (one_span || lower_span || upper_span) && tier_tex[t] >= 0;
-                if (draws) draw |= 1u << j;
-                if (group_valid[t] && py >= group_bottom[t]) tail |= 1u << j;
-                texel[j] = 0;
-                if (draws) {
-                    const unsigned tv = (tier_frac[t] >> tier_shift[t]) >> 1;
-                    texel[j] = m->tex_atlas[tier_texel[t] + __umul24(tv, atlas_w)];
+                    for (int j = 0; j < WALL_ROWS; ++j) next_texel[j] = 0;
+                    if (yb + WALL_ROWS < last) load_rows(yb + WALL_ROWS, next_texel);
+#pragma unroll
+                    for (int j = 0; j < WALL_ROWS; ++j) {
+                        const int y = yb + j;
+                        if (y >= last) break;
+                        const unsigned colour = colormap[(y >= tail_row ? shade_group : shade_own) * 256 + texel[j]];
+                        pb.d(y) = r.distance;
+                        if (DEPTH) pb.s(y) = r.distance;
+                        pb.m(y) = meta_word | (colour << META_SECTOR_SHIFT);
+                    }
+#pragma unroll
+                    for (int j = 0; j < WALL_ROWS; ++j) texel[j] = next_texel[j];
+                }
+            };
+            // first run: a one-sided drawseg's rows, or the upper tier; second run: the lower tier
+            const bool first_run = one_sided || upper_on;
+            paint_run(first_run ? (int)r.clipped_top : 0, first_run ? (int)(one_sided ? r.clipped_bottom : r.clipped_upper_bottom) : 0,
+                      one_sided ? side_tex0 : side_tex2, one_sided ? r.view_ceiling : r.other_ceiling,
+                      one_sided ? group_valid[0] : group_valid[2], one_sided ? group_bottom[0] : group_bottom[2]);
+            paint_run(lower_on ? (int)r.clipped_lower_top : 0, lower_on ? (int)r.clipped_bottom : 0, side_tex1, r.other_floor,
+                      group_valid[1], group_bottom[1]);
+        } else {
+            // The lower and the upper tier share rows (a closed door, say): the lower tier has the say there, row by row.
+                int tier_tex[3]; unsigned tier_frac[3], tier_step[3], tier_shift[3]; size_t tier_texel[3];
+            const float tier_origin[3] = {r.view_ceiling, r.other_floor, r.other_ceiling};
+#pragma unroll
+            for (int t = 0; t < 3; ++t) {
+                tier_tex[t] = r.side_tex[t];
+                const int id = tier_tex[t] < 0 ? 0 : tier_tex[t];
+                const int bits = tb.height_bits(id);
+                const i64 step = mul64(swall, shl64(1, 14 - bits));
+                const i64 base = shl64(round_to_i64((tier_origin[t] - L.view_z) * 65536.0f + toff_y), 16 - bits);
+                tier_shift[t] = (unsigned)(31 - bits);   // a one-row texture (bits == 0) must shift everything out: two shifts
+                tier_step[t] = (unsigned)step;
+                tier_frac[t] = (unsigned)(base + (mul64(step, FIXED_UNIT - L.center_fixed) >> 16)) + (unsigned)step * (unsigned)t0;
+                tier_texel[t] = (size_t)id * m->tex_max_h * m->tex_max_w + (size_t)tb.wrap_column(id, u_base);
+            }
+            // WALL_ROWS rows at a time, one batch ahead: the texels of the next batch are asked for before the rows of
+            // this one are stored, so that a step waits for memory once, not for its stores and then for its loads
+            auto load_rows = [&](int yb, unsigned char (&texel)[WALL_ROWS], unsigned &draw, unsigned &tail) {
+                draw = 0; tail = 0;
+#pragma unroll
+                for (int j = 0; j < WALL_ROWS; ++j) {
+                    const int y = yb + j;
+                    const float py = (float)y;
+                    const bool one_span = one_sided && (py >= r.clipped_top) && (py < r.clipped_bottom);
+                    const bool lower_span = lower_on && (py >= r.clipped_lower_top) && (py < r.clipped_bottom);
+                    const bool upper_span = upper_on && (py >= r.clipped_top) && (py < r.clipped_upper_bottom);
+                    const int t = one_span ? 0 : (lower_span ? 1 : 2);
+                    const bool draws = y < t1 && (one_span || lower_span || upper_span) && tier_tex[t] >= 0;
+                    if (draws) draw |= 1u << j;
+                    if (group_valid[t] && py >= group_bottom[t]) tail |= 1u << j;
+                    texel[j] = 0;
+                    if (draws) {
+                        const unsigned tv = (tier_frac[t] >> tier_shift[t]) >> 1;
+                        texel[j] = m->tex_atlas[tier_texel[t] + __umul24(tv, atlas_w)];
+                    }
+#pragma unroll
+                    for (int k = 0; k < 3; ++k) tier_frac[k] += tier_step[k];
+                }
+            };
+            unsigned char texel[WALL_ROWS]; unsigned draw = 0, tail = 0;
+            if (t0 < t1) load_rows(t0, texel, draw, tail);
+            for (int yb = t0; yb < t1; yb += WALL_ROWS) {
+                unsigned char next_texel[WALL_ROWS]; unsigned next_draw = 0, next_tail = 0;
+#pragma unroll
+                for (int j = 0; j < WALL_ROWS; ++j) next_texel[j] = 0;
+                if (yb + WALL_ROWS < t1) load_rows(yb + WALL_ROWS, next_texel, next_draw, next_tail);
+#pragma unroll
+                for (int j = 0; j < WALL_ROWS; ++j) {
+                    if (!(draw & (1u << j))) continue;
+                    const unsigned colour = colormap[((tail & (1u << j)) ? shade_group : shade_own) * 256 + texel[j]];
+                    pb.d(yb + j) = r.distance;
+                    if (DEPTH) pb.s(yb + j) = r.distance;
+                    pb.m(yb + j) = META_FILLED | (colour << META_SECTOR_SHIFT) | (unsigned)(wi + 1);
                 }
 #pragma unroll
-                for (int k = 0; k < 3; ++k) tier_frac[k] += tier_step[k];
+                for (int j = 0; j < WALL_ROWS; ++j) texel[j] = next_texel[j];
+                draw = next_draw; tail = next_tail;
             }
-        };
-        unsigned char texel[WALL_ROWS]; unsigned draw = 0, tail = 0;
-        if (t0 < t1) load_rows(t0, texel, draw, tail);
-        for (int yb = t0; yb < t1; yb += WALL_ROWS) {
-            unsigned char next_texel[WALL_ROWS]; unsigned next_draw = 0, next_tail = 0;
-#pragma unroll
-            for (int j = 0; j < WALL_ROWS; ++j) next_texel[j] = 0;
-            if (yb + WALL_ROWS < t1) load_rows(yb + WALL_ROWS, next_texel, next_draw, next_tail);
-#pragma unroll
-            for (int j = 0; j < WALL_ROWS; ++j) {
-                if (!(draw & (1u << j))) continue;
-                const unsigned colour = colormap[((tail & (1u << j)) ? shade_group : shade_own) * 256 + texel[j]];
-                pb.d(yb + j) = r.distance;
-                if (DEPTH) pb.s(yb + j) = r.distance;
-                pb.m(yb + j) = META_FILLED | (colour << META_SECTOR_SHIFT) | (unsigned)(wi + 1);
-            }
-#pragma unroll
-            for (int j = 0; j < WALL_ROWS; ++j) texel[j] = next_texel[j];
-            draw = next_draw; tail = next_tail;
         }
         if (one_sided) {
             window_dirty = true;
