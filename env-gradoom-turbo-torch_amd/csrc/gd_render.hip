@@ -2115,6 +2115,20 @@ __device__ __forceinline__ void zero_rows(PixelBuffers &pb, GapRange &gaps, int 
     gaps.set_zeroed(min(first, gaps.lo()), max(last, gaps.hi()));
 }
 
+// Smallest / largest of a small value (0..255) over the lanes that execute the call, found by ballots: usable inside
+// divergent code, where a lane exchange would read lanes that are switched off.  The result is uniform.
+__device__ __forceinline__ int wave_min_byte(int v) {
+    u64 candidates = __ballot(true);
+    int result = 0;
+#pragma unroll
+    for (int bit = 7; bit >= 0; --bit) {
+        const u64 clear = __ballot(!((v >> bit) & 1)) & candidates;
+        if (clear) candidates = clear; else result |= 1 << bit;
+    }
+    return result;
+}
+__device__ __forceinline__ int wave_max_byte(int v) { return 255 - wave_min_byte(255 - v); }
+
 // engine.py:12637-12884
 // `window_dirty` says whether some pixel inside the open window [ceiling_clip, floor_clip) may
 // already be filled, plane-owned or carry a sprite-clip depth.  A two-sided drawseg only writes
@@ -2170,25 +2184,28 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
         {
             const bool claims = r.bits & PB_MARK_CEILING;
             const bool bare = !claims && sil_top && upper_on && (r.side_tex[2] >= 0);   // the upper tier lowers the clip past these rows
-            if (claims || bare) {
-                const int e = (int)ceiling_plane_bottom;
-                const unsigned word = (claims ? claim : 0u) | (sil_top ? clip_word : 0u);
-                for (int y = y0 < 0 ? 0 : y0; y < e; ++y) {
-                    pb.m(y) = word;
-                    if (sil_top) pb.d(y) = r.distance;
-                }
+            // The wavefront walks the rows together, each column writing where its own range has the row: neighbouring
+            // columns then store to neighbouring words, where loops that start at each column's own first row would
+            // scatter every store over as many rows as the edges' slopes spread them.
+            const bool writes = claims || bare;
+            const int first = writes ? (y0 < 0 ? 0 : y0) : VH, last = writes ? min((int)ceiling_plane_bottom, VH) : 0;
+            const unsigned word = (claims ? claim : 0u) | (sil_top ? clip_word : 0u);
+            for (int y = wave_min_byte(first), wave_last = wave_max_byte(last); y < wave_last; ++y) {
+                if (y < first || y >= last) continue;
+                pb.m(y) = word;
+                if (sil_top) pb.d(y) = r.distance;
             }
         }
         {
             const bool claims = r.bits & PB_MARK_FLOOR;
             const bool bare = !claims && sil_bottom && lower_on && (r.side_tex[1] >= 0);   // the lower tier raises the clip past these rows
-            if (claims || bare) {
-                const int b = (int)floor_plane_top;
-                const unsigned word = (claims ? (claim | META_FLOOR) : 0u) | (sil_bottom ? clip_word : 0u);
-                for (int y = b < 0 ? 0 : b; y < y1; ++y) {
-                    pb.m(y) = word;
-                    if (sil_bottom) pb.d(y) = r.distance;
-                }
+            const bool writes = claims || bare;
+            const int first = writes ? max((int)floor_plane_top, 0) : VH, last = writes ? y1 : 0;
+            const unsigned word = (claims ? (claim | META_FLOOR) : 0u) | (sil_bottom ? clip_word : 0u);
+            for (int y = wave_min_byte(min(first, VH)), wave_last = wave_max_byte(last); y < wave_last; ++y) {
+                if (y < first || y >= last) continue;
+                pb.m(y) = word;
+                if (sil_bottom) pb.d(y) = r.distance;
             }
         }
         // Rows that leave the window without being written: those the upper tier covers but that belong to a lower
@@ -2980,13 +2997,16 @@ __global__ void __launch_bounds__(128) flat_shade_kernel(DeviceMap dm, int lane_
 // sprites: engine.py:10534-10557 (blocking raycast) and 14684-14947
 // ---------------------------------------------------------------------------------------------
 #define SPRITE_ROWS 4   // rows of a sprite column in flight together
-// Columns per block.  A block lasts as long as its slowest column, so three blocks of 128 (the last one 64 wide) pack
-// the chip better than one of 320; each lists only the sprites that reach its own columns.
-#define SPRITE_COLUMNS 128
+// Columns per block.  A block lasts as long as its slowest column, so many small blocks pack the chip better than a few
+// wide ones, until the staging each block repeats for itself outweighs that; each lists only the billboards that reach its
+// own columns.  Measured on 4096 lanes with 128 billboards each, columns x row parts: 128x1 0.70 ms, 128x2 0.55, 64x2 0.49,
+// 64x4 0.51, 32x2 0.59, 32x4 0.45.
+#define SPRITE_COLUMNS 32
 struct SpriteRec {
     float x, y, depth, light;
-    i64 depth_fixed, left, right, hstep, yscale, top_fixed, texmid, iscale;
-    int id, flags;   // bit0 alive, bit1 fullbright, bits 8..15 style (signed: -1 opaque, -2 translucent, >= 0 additive)
+    i64 depth_fixed, left, right, hstep, yscale, top_fixed, fraction_base, iscale;
+    int id, flags;   // bit0 alive, bit1 fullbright, bits 8..15 style (signed: -1 opaque, -2 translucent, >= 0 additive),
+                     // bits 16..23 / 24..31 first / one past the last screen row the patch can reach
 };
 
 // A frame some kernel paints into: all of a lane's 320x240 frame in device memory, or the rows a work-group keeps in LDS.
@@ -3023,31 +3043,35 @@ __device__ __forceinline__ void stage_sprites(const DeviceMap &dm, const gd_lane
         s.right = SW / 2 + (mul64(right_fixed, xscale) >> 32);
         s.hstep = tdiv((i64)m->spr_w[s.id] << 16, max64(s.right - s.left, 1));
         s.yscale = tdiv(FOCAL_Y_FIXED << 12, max64(s.depth_fixed, SPRITE_MIN_DEPTH_FIXED));
-        s.texmid = (i64)m->spr_top[s.id] * FIXED_UNIT - round_to_i64((L.view_z - z) * 65536.0f);
-        s.top_fixed = L.center_fixed - (mul64(s.texmid, s.yscale) >> 16);
+        const i64 texmid = (i64)m->spr_top[s.id] * FIXED_UNIT - round_to_i64((L.view_z - z) * 65536.0f);
+        s.top_fixed = L.center_fixed - (mul64(texmid, s.yscale) >> 16);
         s.iscale = tdiv(UINT32_MASK, max64(s.yscale, 1));
-        bool reaches = (s.flags & 1) && (s.depth > 0) && (s.right > x_first) && (s.left < x_end) && (s.right > s.left);
-        if (reaches && s.iscale > 0 && (row_first > 0 || row_end < VH)) {
-            // the rows whose source row can fall inside the patch (the bracket sprite_column works with, a row to spare)
-            const i64 fraction_base = s.texmid - (mul64(L.center_fixed - FIXED_UNIT, s.iscale) >> 16);
-            const i64 y_lo = tdiv(-fraction_base, s.iscale) - 1, y_hi = tdiv(((i64)m->spr_h[s.id] << 16) - fraction_base, s.iscale) + 2;
-            reaches = y_hi > row_first && y_lo < row_end;
+        // Screen row y shows source row (fraction_base + y * iscale) >> 16 (engine.py:14830-14846).  The rows whose source
+        // row can fall inside the patch: a bracket from two divisions, a row too wide on either side; the exact test
+        // stays per row.
+        s.fraction_base = texmid - (mul64(L.center_fixed - FIXED_UNIT, s.iscale) >> 16);
+        int y_lo = 0, y_hi = VH;
+        if (s.iscale > 0) {
+            y_lo = (int)clampi(tdiv(-s.fraction_base, s.iscale) - 1, 0, VH);
+            y_hi = (int)clampi(tdiv(((i64)m->spr_h[s.id] << 16) - s.fraction_base, s.iscale) + 2, 0, VH);
         }
+        s.flags |= (int)(((unsigned)y_lo << 16) | ((unsigned)y_hi << 24));
+        const bool reaches = (s.flags & 1) && (s.depth > 0) && (s.right > x_first) && (s.left < x_end) && (s.right > s.left) &&
+                             y_hi > row_first && y_lo < row_end;
         s.light = reaches ? m->sector_lights[sector_at(m, s.x, s.y)] : 0.0f;
         sp[a] = s;
         if (reaches) on_screen[atomicAdd(on_screen_count, 1)] = (unsigned short)a;
     }
 }
 
-// Every billboard that shows in column x, rows [row_first, row_end), far -> near (engine.py:14762-14947).
-template <typename Frame>
-__device__ __forceinline__ void sprite_column(const DeviceMap &dm, const gd_lanes_desc &lanes, const Scratch &sc, int local, int n, const LaneCtx &L,
-                                              const SpriteRec *sp, const unsigned short *on_screen, int listed, int x, int row_first, int row_end,
-                                              const Frame &frame) {
+// The billboards that can show in column x at all (alive, in front, horizontally covering it and not hidden by the
+// column's blocking linedef), as a bit set over `on_screen` (sprite_slots <= 512): the painter's loop runs once per
+// drawn billboard and would otherwise test every slot each time.  engine.py:10534-10557, 14762-14800
+struct SpriteCover { u64 bits[8]; };
+__device__ __forceinline__ SpriteCover sprite_cover(const DeviceMap &dm, const Scratch &sc, int local, const SpriteRec *sp,
+                                                    const unsigned short *on_screen, int listed, int x) {
     const gd_map_desc *m = &dm.d;
-    const int A = lanes.sprite_slots;
     const WallRec *recs = sc.rec + (size_t)local * m->wall_count;
-    const unsigned int *meta = sc.meta + (size_t)local * VH * SW;
     // nearest blocking linedef of this column (engine.py:10534-10557), gathered by wall_setup
     const u64 hit = sc.block_hit[(size_t)local * SW + x];
     float best = hit == ~0ULL ? GD_INF : __uint_as_float((unsigned)(hit >> 32));
@@ -3059,12 +3083,10 @@ __device__ __forceinline__ void sprite_column(const DeviceMap &dm, const gd_lane
     const float4 bl = *reinterpret_cast<const float4 *>(m->walls + 4 * bw);
     float bdx = bl.z - bl.x, bdy = bl.w - bl.y;
     bool owns = (x >= bg.sl) && (x < bg.sr);
-    // The sprites that can show in this column at all (alive, in front, horizontally covering it and
-    // not hidden by the column's blocking linedef), as a bit set: the painter's loop below runs once
-    // per drawn sprite and would otherwise test every slot each time.
-    u64 cover[8] = {0, 0, 0, 0, 0, 0, 0, 0};   // sprite_slots <= 512; bit p of the set = on_screen[p]
+    SpriteCover cover;
 #pragma unroll
     for (int word = 0; word < 8; ++word) {
+        cover.bits[word] = 0;
         if (word * 64 >= listed) continue;     // the same in every thread
         u64 bits = 0;
         const int end = listed - word * 64 < 64 ? listed - word * 64 : 64;
@@ -3079,8 +3101,20 @@ __device__ __forceinline__ void sprite_column(const DeviceMap &dm, const gd_lane
             }
             if (ray_visible) bits |= 1ULL << b;
         }
-        cover[word] = bits;
+        cover.bits[word] = bits;
     }
+    return cover;
+}
+
+// Every billboard of `cover` in column x, rows [row_first, row_end), far -> near (engine.py:14762-14947).
+template <typename Frame>
+__device__ __forceinline__ void sprite_paint(const DeviceMap &dm, const gd_lanes_desc &lanes, const Scratch &sc, int local, int n, const LaneCtx &L,
+                                             const SpriteRec *sp, const unsigned short *on_screen, const SpriteCover &cover, int x, int row_first,
+                                             int row_end, const Frame &frame) {
+    const gd_map_desc *m = &dm.d;
+    const int A = lanes.sprite_slots;
+    const WallRec *recs = sc.rec + (size_t)local * m->wall_count;
+    const unsigned int *meta = sc.meta + (size_t)local * VH * SW;
     int clip_wall = -1; i64 clip_near = 0, clip_far = 0; float4 clip_line = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     // painter's order far -> near: repeatedly take the farthest candidate nearer than the last one
     float last_depth = GD_INF; int last_slot = A;
@@ -3088,7 +3122,7 @@ __device__ __forceinline__ void sprite_column(const DeviceMap &dm, const gd_lane
         float pick_depth = -GD_INF; int pick = -1;
 #pragma unroll
         for (int word = 0; word < 8; ++word) {
-            for (u64 bits = cover[word]; bits; bits &= bits - 1) {
+            for (u64 bits = cover.bits[word]; bits; bits &= bits - 1) {
                 const int a = on_screen[word * 64 + __ffsll((long long)bits) - 1];
                 const float depth = sp[a].depth;
                 // strictly before (last_depth, last_slot) in (depth, slot) order
@@ -3108,14 +3142,8 @@ __device__ __forceinline__ void sprite_column(const DeviceMap &dm, const gd_lane
         float base_shade = 61.0f - light / 4.0f;
         float visibility = fminf(1280.0f / fmaxf(s.depth, 1.0f), 24.0f);
         i64 shade = clampi((i64)floorf(base_shade - visibility), 0, 31);
-        i64 fraction_base = s.texmid - (mul64(L.center_fixed - FIXED_UNIT, s.iscale) >> 16);
-        // Rows whose source row sv = (fraction_base + y * iscale) >> 16 can fall inside the patch:
-        // a bracket from two divisions, a row too wide on either side; the exact test stays per row.
-        int y_lo = row_first, y_hi = row_end;
-        if (s.iscale > 0) {
-            y_lo = (int)clampi(tdiv(-fraction_base, s.iscale) - 1, row_first, row_end);
-            y_hi = (int)clampi(tdiv(((i64)height << 16) - fraction_base, s.iscale) + 2, row_first, row_end);
-        }
+        const i64 fraction_base = s.fraction_base;
+        const int y_lo = max((int)((unsigned)s.flags >> 16) & 255, row_first), y_hi = min((int)((unsigned)s.flags >> 24), row_end);
         // SPRITE_ROWS rows per step, each stage's loads issued together so that their latencies overlap
         for (int yb = y_lo; yb < y_hi; yb += SPRITE_ROWS) {
             i64 sv[SPRITE_ROWS]; bool live[SPRITE_ROWS]; unsigned int row_meta[SPRITE_ROWS];
@@ -3186,7 +3214,19 @@ __device__ __forceinline__ void sprite_column(const DeviceMap &dm, const gd_lane
     }
 }
 
-__global__ void __launch_bounds__(SPRITE_COLUMNS) __attribute__((amdgpu_waves_per_eu(5, 5))) sprite_columns_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc,
+template <typename Frame>
+__device__ __forceinline__ void sprite_column(const DeviceMap &dm, const gd_lanes_desc &lanes, const Scratch &sc, int local, int n, const LaneCtx &L,
+                                              const SpriteRec *sp, const unsigned short *on_screen, int listed, int x, int row_first, int row_end,
+                                              const Frame &frame) {
+    const SpriteCover cover = sprite_cover(dm, sc, local, sp, on_screen, listed, x);
+    sprite_paint(dm, lanes, sc, local, n, L, sp, on_screen, cover, x, row_first, row_end, frame);
+}
+
+// Each column's rows are shared out among SPRITE_ROW_PARTS threads (a column's time is a chain of memory round trips,
+// one row batch after another); the first of them finds the column's billboards and leaves the set in LDS for the others.
+#define SPRITE_ROW_PARTS 4
+static_assert(VH % (SPRITE_ROW_PARTS * SPRITE_ROWS) == 0, "sprite_columns_kernel: row parts hold whole row batches");
+__global__ void __launch_bounds__(SPRITE_COLUMNS * SPRITE_ROW_PARTS) __attribute__((amdgpu_waves_per_eu(4, 4))) sprite_columns_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc,
                                                             unsigned char *frame_base, size_t frame_stride) {
     extern __shared__ unsigned char shared_raw[];
     SpriteRec *sp = reinterpret_cast<SpriteRec *>(shared_raw);
@@ -3202,10 +3242,23 @@ __global__ void __launch_bounds__(SPRITE_COLUMNS) __attribute__((amdgpu_waves_pe
     const LaneCtx L = sc.ctx[local];
     stage_sprites(dm, lanes, n, L, x_first, x_end, 0, VH, sp, on_screen, &on_screen_count);
     __syncthreads();
-    const int x = x_first + threadIdx.x;
+    const int column = threadIdx.x % SPRITE_COLUMNS, part = threadIdx.x / SPRITE_COLUMNS;
+    const int x = x_first + column;
+    const int listed = on_screen_count;
+    if (listed == 0) return;                       // the same in the whole block
+    __shared__ u64 cover_bits[8][SPRITE_COLUMNS];
+    SpriteCover cover;
+    if (part == 0 && x < x_end) {
+        cover = sprite_cover(dm, sc, local, sp, on_screen, listed, x);
+#pragma unroll
+        for (int word = 0; word < 8; ++word) if (word * 64 < listed) cover_bits[word][column] = cover.bits[word];
+    }
+    __syncthreads();
     if (x >= x_end) return;
+#pragma unroll
+    for (int word = 0; word < 8; ++word) cover.bits[word] = word * 64 < listed ? cover_bits[word][column] : 0;
     GlobalFrame frame; frame.base = frame_base + (size_t)local * frame_stride;
-    sprite_column(dm, lanes, sc, local, n, L, sp, on_screen, on_screen_count, x, 0, VH, frame);
+    sprite_paint(dm, lanes, sc, local, n, L, sp, on_screen, cover, x, part * (VH / SPRITE_ROW_PARTS), (part + 1) * (VH / SPRITE_ROW_PARTS), frame);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -4324,7 +4377,7 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
         hipLaunchKernelGGL(decal_kernel, dim3(count), dim3(SW), 0, stream, r->dm, r->overlays, *lanes, base, count, sc, frame_base, frame_stride);
     if (lanes->sprite_slots > 0 && lanes->sprite_x) {
         size_t shared = (size_t)lanes->sprite_slots * (sizeof(SpriteRec) + sizeof(unsigned short));
-        hipLaunchKernelGGL(sprite_columns_kernel, dim3((SW + SPRITE_COLUMNS - 1) / SPRITE_COLUMNS, count), dim3(SPRITE_COLUMNS), shared, stream, r->dm, *lanes, base, count, sc, frame_base, frame_stride);
+        hipLaunchKernelGGL(sprite_columns_kernel, dim3((SW + SPRITE_COLUMNS - 1) / SPRITE_COLUMNS, count), dim3(SPRITE_COLUMNS * SPRITE_ROW_PARTS), shared, stream, r->dm, *lanes, base, count, sc, frame_base, frame_stride);
     }
     if (lanes->weapon_state && r->overlays.d.weapon_patch_count > 0)
         hipLaunchKernelGGL(weapon_overlay_kernel, dim3((VH * SW + 255) / 256, count), dim3(256), 0, stream, r->overlays, lanes->weapon_state, base, count,
