@@ -2706,9 +2706,10 @@ __device__ __forceinline__ void masked_midtexture(const ColumnCtx &cc, const Col
 // How long a column's traversal runs is set by the portals it crosses: the two-sided linedefs its ray hits before the
 // nearest blocking one.  Columns differ by a factor of ten, a wavefront runs as long as its longest column, and a launch
 // ends with its longest wavefront.  So the screen is cut into segments of SEG_COLS columns, a wavefront takes
-// 64 / SEG_COLS segments of about the same length (whatever lanes they belong to), and the longest go first:
-// strip_key_kernel counts (one lane per column, a walk over the column's candidate list, the maximum of each segment),
-// strip_order_kernel sorts the counts (one block, counting sort).
+// 64 / SEG_COLS segments of about the same length (whatever lanes they belong to), and the longest go first.  The length
+// is taken to be the longest candidate list of the segment, which wall_setup_kernel has counted anyway: walking the lists
+// to count the portals proper orders the segments a little better (the traversal gains 0.04 ms on the 4000-linedef map)
+// but the walk costs 0.11 ms.  strip_key_kernel takes the maxima, strip_order_kernel sorts them (one block, counting sort).
 // Narrow segments waste fewer column passes (on the 4000-linedef map 69 % of the passes a wavefront runs are useful with
 // whole 64-column strips, 80 % with two sorted 32-column segments, 89 % with four of 16), but unrelated segments share no
 // linedefs, branches or row ranges, and a pass costs what the union of its columns' paths costs: measured, the traversal
@@ -2718,25 +2719,11 @@ __global__ void __launch_bounds__(256) strip_key_kernel(int lane_count, Scratch 
     const int local = strip / (SW / 64);
     if (local >= lane_count) return;
     const int x = (strip - local * (SW / 64)) * 64 + (threadIdx.x & 63);
-    const u64 hit = sc.block_hit[(size_t)local * SW + x];
-    const float solid = hit == ~0ULL ? GD_INF : __uint_as_float((unsigned)(hit >> 32));
-    const Cand *list = sc.cand + (size_t)local * CAND_MAX * SW + x;
-    int count = sc.cand_count[(size_t)local * SW + x];
-    if (count > CAND_MAX) count = CAND_MAX;
-    int portals = 0;
-    for (int k0 = 0; k0 < count; k0 += 4) {
-        uint4 raw[4];
+    int length = sc.cand_count[(size_t)local * SW + x];
+    if (length > CAND_MAX) length = CAND_MAX;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) raw[j] = *reinterpret_cast<const uint4 *>(list + (size_t)(k0 + j < count ? k0 + j : count - 1) * SW);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            union { uint4 r; Cand c; } u; u.r = raw[j];
-            portals += (k0 + j < count && u.c.s1 >= 0 && (u.c.flags & CF_GEO) && u.c.dist < solid) ? 1 : 0;
-        }
-    }
-#pragma unroll
-    for (int step = 1; step < SEG_COLS; step <<= 1) portals = max(portals, __shfl_xor(portals, step));
-    if ((x & (SEG_COLS - 1)) == 0) sc.strip_key[local * SEGS_PER_LANE + x / SEG_COLS] = (unsigned char)portals;   // at most CAND_MAX
+    for (int step = 1; step < SEG_COLS; step <<= 1) length = max(length, __shfl_xor(length, step));
+    if ((x & (SEG_COLS - 1)) == 0) sc.strip_key[local * SEGS_PER_LANE + x / SEG_COLS] = (unsigned char)length;   // at most CAND_MAX
 }
 
 __global__ void __launch_bounds__(1024) strip_order_kernel(int strips, Scratch sc) {
@@ -4075,6 +4062,11 @@ struct gd_renderer {
     std::vector<void *> allocations;
     hipEvent_t events[16];
     bool events_ready;
+    // The flat pass (short kernels that leave most of the chip idle) runs beside the plane shading on a stream of the
+    // renderer's own: forked from the caller's stream after the walls, joined before the billboards.
+    hipStream_t side_stream;
+    hipEvent_t fork_event, join_event;
+    bool side_ready;
     Overlays overlays;                       // device pointers, counts 0 until gd_renderer_set_overlays
     std::vector<void *> overlay_allocations;
 };
@@ -4336,20 +4328,40 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
         hipLaunchKernelGGL(kernel, grid, block, 0, stream, r->dm, count, sc, frame_base, frame_stride);
     }
     mark();
-    if (!fused) {
+    // The plane shading and the flat pass do not depend on each other: the first reads the per-pixel words and writes the
+    // pixels some drawseg owns, the second reads the same words and writes its own planes and, at the end, the pixels no
+    // drawseg owns.  The flat pass is a chain of short kernels that wait more than they compute, so it runs on the
+    // renderer's side stream while the shading keeps the vector units busy.  (Not when stages are being timed.)
+    const bool beside = !fused && !timed && r->side_ready;
+    hipStream_t flat_stream = stream;
+    if (beside) {
+        HIP_TRY(hipEventRecord(r->fork_event, stream));
+        HIP_TRY(hipStreamWaitEvent(r->side_stream, r->fork_event, 0));
+        flat_stream = r->side_stream;
+    }
+    // timed (and so serial): shading, then the flat pass, each between its own marks.  Otherwise the flat pass is queued
+    // first, so that its few busy blocks find room at once and the shading fills the rest of the chip around them.
+    auto shade_planes = [&]() {
+        if (fused) return;
         const dim3 grid(((VH * SW + 255) / 256 + SHADE_TILES - 1) / SHADE_TILES, count);
         if (decals) hipLaunchKernelGGL(plane_shade_kernel<true>, grid, dim3(256), 0, stream, r->dm, count, sc, frame_base, frame_stride);
         else hipLaunchKernelGGL(plane_shade_kernel<false>, grid, dim3(256), 0, stream, r->dm, count, sc, frame_base, frame_stride);
-    }
+    };
+    if (!beside) shade_planes();
     mark();
     // the flat pass, where the walls left it something to decide
-    hipLaunchKernelGGL(flat_list_kernel, dim3(count), dim3(128), 0, stream, r->dm, *lanes, base, count, sc);
-    hipLaunchKernelGGL(flat_gap_column_kernel, dim3(count), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
-    hipLaunchKernelGGL(flat_span_select_kernel, dim3(SPAN_SELECT_BLOCKS), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
+    hipLaunchKernelGGL(flat_list_kernel, dim3(count), dim3(128), 0, flat_stream, r->dm, *lanes, base, count, sc);
+    hipLaunchKernelGGL(flat_gap_column_kernel, dim3(count), dim3(SW), 0, flat_stream, r->dm, *lanes, base, count, sc);
+    hipLaunchKernelGGL(flat_span_select_kernel, dim3(SPAN_SELECT_BLOCKS), dim3(SW), 0, flat_stream, r->dm, *lanes, base, count, sc);
     mark();
-    hipLaunchKernelGGL(flat_tail_kernel, dim3(SW / 64, count), dim3(64 * TAIL_ROWS), 0, stream, r->dm, *lanes, base, count, sc);
-    hipLaunchKernelGGL(flat_span_finish_kernel, dim3(count), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
-    if (!fused) hipLaunchKernelGGL(flat_shade_kernel, dim3(count), dim3(128), 0, stream, r->dm, count, sc, frame_base, frame_stride);
+    hipLaunchKernelGGL(flat_tail_kernel, dim3(SW / 64, count), dim3(64 * TAIL_ROWS), 0, flat_stream, r->dm, *lanes, base, count, sc);
+    hipLaunchKernelGGL(flat_span_finish_kernel, dim3(count), dim3(SW), 0, flat_stream, r->dm, *lanes, base, count, sc);
+    if (!fused) hipLaunchKernelGGL(flat_shade_kernel, dim3(count), dim3(128), 0, flat_stream, r->dm, count, sc, frame_base, frame_stride);
+    if (beside) {
+        shade_planes();
+        HIP_TRY(hipEventRecord(r->join_event, r->side_stream));
+        HIP_TRY(hipStreamWaitEvent(stream, r->join_event, 0));
+    }
     mark();
     const float *blend = lanes->screen_blend ? lanes->screen_blend + 2 * (size_t)base : nullptr;
     if (fused) {
@@ -4436,6 +4448,7 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     gd_renderer *r = new (std::nothrow) gd_renderer();
     if (!r) return fail(GD_E_ARG, "out of host memory");
     r->events_ready = false;
+    r->side_ready = false;
     r->scratch_block = nullptr; r->scratch_bytes = 0;
     r->assembly = GD_ASSEMBLY_AUTO;
     std::memset(&r->sc, 0, sizeof(r->sc));
@@ -4566,6 +4579,14 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
         for (int i = 0; i < 16; ++i) if (hipEventCreate(&r->events[i]) != hipSuccess) rc = fail(GD_E_HIP, "hipEventCreate");
         r->events_ready = rc == GD_OK;
     }
+    if (rc == GD_OK) {
+        // default priority, like the caller's stream; no implicit synchronisation with the null stream
+        if (hipStreamCreateWithFlags(&r->side_stream, hipStreamNonBlocking) != hipSuccess) rc = fail(GD_E_HIP, "hipStreamCreateWithFlags");
+        else if (hipEventCreateWithFlags(&r->fork_event, hipEventDisableTiming) != hipSuccess) { (void)hipStreamDestroy(r->side_stream); rc = fail(GD_E_HIP, "hipEventCreateWithFlags"); }
+        else if (hipEventCreateWithFlags(&r->join_event, hipEventDisableTiming) != hipSuccess) {
+            (void)hipEventDestroy(r->fork_event); (void)hipStreamDestroy(r->side_stream); rc = fail(GD_E_HIP, "hipEventCreateWithFlags");
+        } else r->side_ready = true;
+    }
     if (rc != GD_OK) { std::string keep = g_error; gd_renderer_destroy(r); g_error = keep; return rc; }
     *out = r;
     return GD_OK;
@@ -4576,6 +4597,7 @@ void gd_renderer_destroy(gd_renderer *r) {
     for (void *ptr : r->allocations) (void)hipFree(ptr);
     for (void *ptr : r->overlay_allocations) (void)hipFree(ptr);
     if (r->events_ready) for (int i = 0; i < 16; ++i) (void)hipEventDestroy(r->events[i]);
+    if (r->side_ready) { (void)hipEventDestroy(r->fork_event); (void)hipEventDestroy(r->join_event); (void)hipStreamDestroy(r->side_stream); }
     delete r;
 }
 
