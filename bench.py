@@ -1,7 +1,7 @@
 """Headline benchmark: rendered lane-frames/s (320x240 indexed + 84x84x4 observation) on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--repeats R] [--workload config4] [--heights quantised|uniform]
-                    [--lanes N] [--mode full|obs-only|rgb] [--no-cpu]
+                    [--lanes N] [--mode full|obs-only|rgb] [--assembly auto|fused|separate] [--no-cpu]
 
 A step is one pass of the whole hot path over one batch of lanes whose inputs already sit in
 HBM: sector-light flicker update, the Torch float32 ray / sprite-depth tables, the render
@@ -61,6 +61,9 @@ def main() -> int:
     parser.add_argument("--mode", choices=("full", "obs-only", "rgb"), default="full",
                         help="full: indexed frame + observation stack (the headline metric); obs-only: observation stack "
                              "only, no 320x240 frame handed to the caller; rgb: indexed + RGB24 frame, no observation")
+    parser.add_argument("--assembly", choices=("auto", "fused", "separate"), default="auto",
+                        help="how frames are put together after the walls: kernel by kernel through a frame in device memory "
+                             "(separate, what auto picks) or band by band in LDS (fused: no frame reaches device memory unless asked for)")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     parser.add_argument("--cpu-lanes", type=int, default=0, help="lanes of the same workload the CPU baseline renders (0: 24 per thread)")
     parser.add_argument("--cpu-threads", type=int, default=0, help="host threads of the CPU baseline (0: every core this process may use, at most 16)")
@@ -94,6 +97,7 @@ def main() -> int:
     tables = mapbuild.build_map_tables(smap)
     cosine = hostmath.cosine_correction("cpu").numpy()
     renderer = HipRenderer(smap, lanes, device, cosine_correction=cosine, tables=tables)
+    renderer.set_assembly(args.assembly)
 
     # Resident inputs: a few pose/sprite sets cycled step by step, plus flicker light vectors.
     states = []
@@ -201,7 +205,7 @@ def main() -> int:
         steps=args.steps, warmup=args.warmup, repeats=len(repeat_seconds), samples=samples,
         ms_per_step=round(elapsed / args.steps * 1e3, 3), higher_is_better=True,
         scaling="weak", vs_baseline=None, dtype="int64+f32", data="synthetic",
-        config=dict(mode=args.mode, workload=f"{args.workload}: {lanes} lanes, {cfg['sectors']} sectors, {cfg['linedefs']} linedefs, "
+        config=dict(mode=args.mode, assembly=args.assembly, workload=f"{args.workload}: {lanes} lanes, {cfg['sectors']} sectors, {cfg['linedefs']} linedefs, "
                     f"{sprites} sprites/lane, masked midtex p={cfg['midtex']}, per-step sector-light flicker, "
                     + ("sector heights quantised (floors 0..96, ceilings 160..256, steps of 8)" if args.heights == "quantised"
                        else "sector heights uniform (floors 0..255, ceilings 64..256 above, whole units)")),

@@ -85,7 +85,7 @@ struct LaneCtx {
     i64 view_x_fixed, view_y_fixed, vsin, vcos, center_fixed, flash_light;
     i64 upper_clip, lower_clip;   // OWallMost's view-frustum slopes at the top and bottom row (engine.py:12402-12413)
     int sector;
-    int pad;
+    int last_ceiling_row;         // rows 0 .. last_ceiling_row of the view look at ceilings, the rest at floors (-1: all floors)
 };
 
 struct WallRec {   // one linedef seen from one lane
@@ -430,6 +430,8 @@ __global__ void lane_tables_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
     const int floors = dm.d.floor_level_count, levels = floors + dm.d.ceil_level_count;
     if (local >= lane_count) return;
     const LaneCtx &c = sc.ctx[local];
+    // the lane's per-column lists start empty
+    for (int x = threadIdx.x; x < SW; x += blockDim.x) { sc.cand_count[(size_t)local * SW + x] = 0; sc.block_hit[(size_t)local * SW + x] = ~0ULL; }
     const float cx = lanes.x[lane_base + local], cy = lanes.y[lane_base + local];
     for (int l = threadIdx.x; l < levels; l += blockDim.x) {
         float reach = GD_INF, far = 0.0f;
@@ -507,13 +509,13 @@ __global__ void lane_setup_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_ba
     c.lower_clip = tdiv(shl64((i64)VH * FIXED_UNIT - c.center_fixed, 16), FOCAL_Y_FIXED);
     c.pitch_offset = (float)((tangent * 12582912LL) >> 16) / 65536.0f;
     c.sector = sector_at(&dm.d, c.x, c.y);
-    c.pad = 0;
+    c.last_ceiling_row = -1;
+    for (int y = 0; y < VH; ++y) if (!(((float)y - (103.5f + c.pitch_offset)) > 0)) c.last_ceiling_row = y;   // flat_center()
     sc.ctx[local] = c;
     int *span = sc.flat_span + (size_t)local * 4;
     span[0] = VH; span[1] = -1; span[2] = VH; span[3] = -1;
     sc.flat_list_count[local] = 0;
     if (local == 0) *sc.flat_row_count = 0;
-    for (int x = 0; x < SW; ++x) { sc.cand_count[(size_t)local * SW + x] = 0; sc.block_hit[(size_t)local * SW + x] = ~0ULL; }
 }
 
 __device__ __forceinline__ void ray_direction(const LaneCtx &c, int x, float *rx, float *ry) {
@@ -1130,8 +1132,7 @@ __global__ void __launch_bounds__(128) flat_list_kernel(DeviceMap dm, gd_lanes_d
     if (listed > FLAT_LIST_MAX) {
         // too many to list (a camera outside the map, say): every row of both halves is selected and repaired
         if (threadIdx.x == 0) {
-            int last_ceiling_row = -1;
-            for (int y = 0; y < VH; ++y) if (!(((float)y - flat_center(c)) > 0)) last_ceiling_row = y;
+            const int last_ceiling_row = c.last_ceiling_row;
             if (last_ceiling_row >= 0) { span[0] = 0; span[1] = last_ceiling_row; }
             if (last_ceiling_row + 1 < VH) { span[2] = last_ceiling_row + 1; span[3] = VH - 1; }
         }
@@ -1166,9 +1167,7 @@ __global__ void __launch_bounds__(SW) __attribute__((amdgpu_waves_per_eu(8, 8)))
     const int n = lane_base + local;
     const int lane_id = threadIdx.x & 63;
     int *span = sc.flat_span + (size_t)local * 4;
-    const float center = flat_center(c);
-    int last_ceiling_row = -1;                       // rows 0 .. last_ceiling_row look at ceilings
-    for (int y = 0; y < VH; ++y) if (!(((float)y - center) > 0)) last_ceiling_row = y;
+    const int last_ceiling_row = c.last_ceiling_row;
     const unsigned int *meta = sc.meta + (size_t)local * VH * SW;
     // the block's columns with work, both halves together, dealt out to its wavefronts in turn (the columns of a
     // gap are neighbours: taken strip by strip, one wavefront would do them all)
@@ -1408,9 +1407,7 @@ __global__ void __launch_bounds__(64 * TAIL_ROWS) flat_tail_kernel(DeviceMap dm,
     const int n = lane_base + local;
     const int slot = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int x = blockIdx.x * 64 + slot;
-    const float center = flat_center(sc.ctx[local]);
-    int last_ceiling_row = -1;                       // rows 0 .. last_ceiling_row look at ceilings
-    for (int y = 0; y < VH; ++y) if (!(((float)y - center) > 0)) last_ceiling_row = y;
+    const int last_ceiling_row = sc.ctx[local].last_ceiling_row;
     for (int half = 0; half < 2; ++half) {
         if (hi[half] < lo[half]) continue;           // the same in every thread
         const int half_end = half ? VH - 1 : last_ceiling_row;
@@ -1446,9 +1443,7 @@ __global__ void __launch_bounds__(SW) flat_span_finish_kernel(DeviceMap dm, gd_l
     unsigned short *sector = sc.flat_sector + (size_t)local * VH * SW;
     unsigned char *flags = sc.flat_flags + (size_t)local * VH * SW;
     const int x = threadIdx.x;
-    const float center = flat_center(c);
-    int last_ceiling_row = -1;                       // rows 0 .. last_ceiling_row look at ceilings
-    for (int y = 0; y < VH; ++y) if (!(((float)y - center) > 0)) last_ceiling_row = y;
+    const int last_ceiling_row = c.last_ceiling_row;
     // --- vertical (engine.py:11026-11083): floors and ceilings alike look downwards, within their own half
     for (int half = 0; half < 2; ++half) {
         if (hi[half] < lo[half]) continue;           // the same in every thread
@@ -4106,6 +4101,7 @@ __global__ void fill_words_kernel(unsigned int *words, size_t count, unsigned in
 // only measures.  `status` is not part of the block: the renderer keeps it.  `depth`: also the scene depth plane
 // of frames that draw decals.
 size_t carve_scratch(Scratch &sc, unsigned char *base, size_t L, const gd_map_desc &h, bool depth) {
+    // `depth`: frames that draw decals also need a scene depth plane
     size_t used = 0;
     auto take = [&](auto **field, size_t count) {
         typedef typename std::remove_reference<decltype(**field)>::type T;
@@ -4139,10 +4135,8 @@ size_t carve_scratch(Scratch &sc, unsigned char *base, size_t L, const gd_map_de
     take(&sc.block_hit, L * SW);
     take(&sc.strip_key, L * SEGS_PER_LANE);
     take(&sc.strip_order, L * SEGS_PER_LANE);
-    if (depth) {   // frames that draw decals: a scene depth plane, and a frame when the caller wants none
-        take(&sc.scene_depth, L * PX);
-        take(&sc.frame, L * (size_t)GD_SCREEN_HEIGHT * SW);
-    }
+    if (depth) take(&sc.scene_depth, L * PX);
+    take(&sc.frame, L * (size_t)GD_SCREEN_HEIGHT * SW);   // where a frame is put together kernel by kernel when the caller takes none
     return (used + 255) & ~(size_t)255;
 }
 
@@ -4296,15 +4290,16 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     const int source_rows = out->obs_source_rows == GD_SCREEN_HEIGHT ? GD_SCREEN_HEIGHT : VH;
     int stage = 0;
     auto mark = [&]() { if (timed) (void)hipEventRecord(r->events[stage], stream); ++stage; };
-    // After the walls and the flat selection a frame is put together in one of two ways.  Kernel by kernel through the
+    // After the walls and the flat selection a frame is put together in one of two ways.  Kernel by kernel through a
     // 320x240 frame in device memory (shade, paint the flat pass's pixels, decals, billboards, overlays, then pool the
-    // observation from it): the faster way when the caller wants that frame anyway, and the only one for frames that draw
-    // wall decals, which need a per-pixel scene depth.  Or band by band in LDS (band_finish_kernel), the frame never
-    // reaching device memory: what a caller that only wants observations gets.
+    // observation from it), the caller's `indexed` or the working memory's own: the faster way on this chip (its kernels
+    // run at full occupancy), and the only one for frames that draw wall decals, which need a per-pixel scene depth.  Or
+    // band by band in LDS (band_finish_kernel), the frame never reaching device memory: a third less traffic for a
+    // caller that only wants observations, at two thirds of the speed; chosen with gd_renderer_set_assembly.
     const bool decals = lanes->decal_slots > 0 && lanes->decal_state && lanes->decal_geom && r->overlays.d.decal_variant_count > 0;
     if (!decals) sc.scene_depth = nullptr;
     if (decals && (!sc.scene_depth || !sc.frame)) return fail(GD_E_ARG, "decal working memory missing");
-    const bool fused = !decals && (r->assembly == GD_ASSEMBLY_FUSED || (r->assembly == GD_ASSEMBLY_AUTO && !out->indexed));
+    const bool fused = !decals && (r->assembly == GD_ASSEMBLY_FUSED || (r->assembly == GD_ASSEMBLY_AUTO && !out->indexed && !sc.frame));
     unsigned char *frame_base = nullptr;
     if (!fused) {
         frame_base = out->indexed ? out->indexed + (size_t)base * frame_stride : sc.frame;
@@ -4758,7 +4753,7 @@ int gd_renderer_set_overlays(gd_renderer *r, const gd_overlay_desc *h) {
 #define OV(field, bytes) if (rc == GD_OK) rc = copy(h->field, (bytes), reinterpret_cast<const void **>(&d.field))
     OV(weapon_atlas, wt); OV(weapon_opaque, wt); OV(weapon_w, wp * 4); OV(weapon_h, wp * 4); OV(weapon_left, wp * 4); OV(weapon_top, wp * 4);
     OV(hud_atlas, ht); OV(hud_opaque, ht); OV(hud_w, hp * 4); OV(hud_h, hp * 4); OV(hud_left, hp * 4); OV(hud_top, hp * 4);
-    r->sc.scene_depth = nullptr; r->sc.frame = nullptr;
+    r->sc.scene_depth = nullptr;
     if (h->decal_variant_count == 5) {
         OV(decal_atlas, (size_t)5 * h->decal_max_h * h->decal_max_w); OV(decal_h, 5 * 4); OV(decal_left, 5 * 4); OV(decal_top, 5 * 4);
         OV(decal_opacity_lut, 32 * 256); OV(decal_black_lut, (size_t)h->decal_black_rows * 256);
@@ -4767,17 +4762,12 @@ int gd_renderer_set_overlays(gd_renderer *r, const gd_overlay_desc *h) {
             if (hipMalloc(&ptr, (size_t)(r->chunk_lanes > 0 ? r->chunk_lanes : 1) * VH * SW * sizeof(float)) != hipSuccess) rc = fail(GD_E_HIP, "out of device memory for the decal depth buffer");
             else { r->overlay_allocations.push_back(ptr); r->sc.scene_depth = static_cast<float *>(ptr); }
         }
-        if (rc == GD_OK) {   // and the frame such frames are assembled in when the caller wants no indexed output
-            void *ptr = nullptr;
-            if (hipMalloc(&ptr, (size_t)(r->chunk_lanes > 0 ? r->chunk_lanes : 1) * GD_SCREEN_HEIGHT * SW) != hipSuccess) rc = fail(GD_E_HIP, "out of device memory for the decal frame buffer");
-            else { r->overlay_allocations.push_back(ptr); r->sc.frame = static_cast<unsigned char *>(ptr); }
-        }
     }
 #undef OV
     if (rc != GD_OK) {
         for (void *ptr : r->overlay_allocations) (void)hipFree(ptr);
         r->overlay_allocations.clear();
-        r->sc.scene_depth = nullptr; r->sc.frame = nullptr;
+        r->sc.scene_depth = nullptr;
         return rc;
     }
     r->overlays.d = d;

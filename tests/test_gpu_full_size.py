@@ -147,4 +147,11 @@ def test_other_benchmark_shapes_at_full_lane_count(oracle, shape):
     if "frames" in full:   # the stack rolled: three older frames kept, no lane left blank
         assert torch.equal(full["frames"][:, :3].cpu(), torch.as_tensor(start[:, 1:]))
         assert int((full["frames"][:, 3].amax(dim=(1, 2)) > 0).sum()) == count
+    if "indexed" not in spec["outputs"]:
+        # no frame handed out: the same stacks when every frame stays in LDS and never reaches device memory
+        renderer.set_assembly("fused")
+        in_lds = render(lanes, count, start)
+        renderer.set_assembly("auto")
+        for name, ours in in_lds.items():
+            assert torch.equal(ours, full[name]), name
     renderer.close()

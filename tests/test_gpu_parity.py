@@ -136,16 +136,21 @@ def test_final_frames_and_stack_modes_match_the_oracle(oracle):
     ):
         print(f"stack mode {mode}", flush=True)
         expected = oracle.render(tables, lane_inputs(data), data["cosine_correction"], frames=start, **oracle_kwargs)
-        # without a frame to hand out the call is assembled in LDS; with one, kernel by kernel: both must roll alike
+        # kernel by kernel through the caller's frame, through the working memory's own when the caller takes none, and
+        # band by band in LDS: all must roll alike
         scratch_frame = torch.zeros((count, 240, 320), dtype=torch.uint8, device="cuda:0")
         separate = torch.as_tensor(start).to("cuda:0")
         renderer.render(lanes, frames=separate, indexed=scratch_frame, **kwargs)
+        own_frame = torch.as_tensor(start).to("cuda:0")
+        renderer.render(lanes, frames=own_frame, **kwargs)
+        renderer.set_assembly("fused")
         frames = torch.as_tensor(start).to("cuda:0")
         final = torch.full((count, 4, 84, 84), 7, dtype=torch.uint8, device="cuda:0")
         obs = torch.zeros((count, 84, 84), dtype=torch.uint8, device="cuda:0")
         renderer.render(lanes, frames=frames, final_frames=final, obs=obs, **kwargs)
+        renderer.set_assembly("auto")
         torch.cuda.synchronize()
-        assert torch.equal(frames, separate), mode
+        assert torch.equal(frames, separate) and torch.equal(own_frame, separate), mode
         ours = frames.cpu().numpy()
         assert np.array_equal(ours, expected["frames"]), mode
         assert np.array_equal(final.cpu().numpy(), expected["frames"]), mode
@@ -205,10 +210,13 @@ def test_status_bar_rows_pooled_into_the_observation(oracle):
     delta = np.abs(obs.cpu().numpy().astype(np.int32) - data["obs_with_hud"].astype(np.int32))
     assert delta.max() <= 1 and delta.mean() < 0.01
     assert torch.equal(obs, again)
-    fused = torch.zeros_like(obs)
-    renderer.render(lanes, obs=fused, obs_source_rows=240)   # no frame asked for: weapon, status bar and pooling all in LDS
+    own_frame, fused = torch.zeros_like(obs), torch.zeros_like(obs)
+    renderer.render(lanes, obs=own_frame, obs_source_rows=240)   # no frame asked for: the working memory's own
+    renderer.set_assembly("fused")
+    renderer.render(lanes, obs=fused, obs_source_rows=240)       # weapon, status bar and pooling all in LDS
+    renderer.set_assembly("auto")
     torch.cuda.synchronize()
-    assert torch.equal(obs, fused)
+    assert torch.equal(obs, fused) and torch.equal(obs, own_frame)
     oracle.set_overlays(fixture_overlays(meta))
     try:
         expected = oracle.render(tables, lane_inputs(data), data["cosine_correction"], obs_source_rows=240)

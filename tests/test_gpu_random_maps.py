@@ -57,13 +57,16 @@ def test_random_maps_and_grazing_poses_match_the_oracle(oracle, first_seed):
         obs = torch.zeros((LANES, 84, 84), dtype=torch.uint8, device="cuda:0")
         state = LaneState.from_numpy(arrays, "cuda:0")
         renderer.render(state, indexed=indexed, obs=obs)
-        fused_obs = torch.zeros_like(obs)
-        renderer.render(state, obs=fused_obs)   # observations only: assembled in LDS
+        own_frame_obs, fused_obs = torch.zeros_like(obs), torch.zeros_like(obs)
+        renderer.render(state, obs=own_frame_obs)   # observations only: through the working memory's own frame
+        renderer.set_assembly("fused")
+        renderer.render(state, obs=fused_obs)       # or assembled in LDS
+        renderer.set_assembly("auto")
         torch.cuda.synchronize()
         assert renderer.status() == 0
         assert np.array_equal(indexed.cpu().numpy(), expected["indexed"]), f"seed {seed}"
         assert np.array_equal(obs.cpu().numpy(), expected["obs"]), f"seed {seed}"
-        assert torch.equal(fused_obs, obs), f"seed {seed}"
+        assert torch.equal(fused_obs, obs) and torch.equal(own_frame_obs, obs), f"seed {seed}"
         renderer.close()
 
 
