@@ -139,8 +139,8 @@ struct DeviceMap {  // device copy of gd_map_desc (device pointers) + fixed tabl
                                          // index << 8 (or -1 when not recorded), first edge, one past the last
     const float4 *cell_edge;             // [item edges] x1, y1, x2, y2
     const int *wall_blocking_slot;       // [W] position of the linedef in blocking_walls, -1 when it does not block
-    const unsigned short *sector_level;  // [S] index of the floor in floor_levels | index of the ceiling in
-                                         // ceil_levels << 8; null when a level list is longer than PLANE_LEVELS
+    const unsigned int *sector_level;    // [S] index of the floor in floor_levels | index of the ceiling in ceil_levels << 16;
+                                         // null when some sector's height is missing from the level lists
 };
 
 struct Overlays {   // device copy of gd_overlay_desc; count 0 = layer not loaded
@@ -188,7 +188,8 @@ struct Scratch {    // per-chunk working memory, sized at create
                            // column, the fraction at screen column 0, the camera's offset
 };
 #define FLAT_LIST_MAX 1024 // listed gap pixels per lane (a gap is typically one column wide)
-#define PLANE_LEVELS 64    // level lists up to this long are shaded from the per-lane tables
+#define PLANE_LEVELS 32    // the per-lane plane tables of level lists up to this long (each) are staged in LDS by the
+                           // shading kernels; longer lists are read where lane_tables_kernel left them
 
 #define META_FILLED 0x80000000u   // an opaque wall tier owns the pixel; its palette index sits in the low byte of the
                                   // plane sector field (plane shading, which writes every other view pixel, stores it)
@@ -1051,7 +1052,7 @@ __device__ __forceinline__ int flat_select_pixel(const DeviceMap &dm, const Scra
                 for (int it = range.x; it < range.y; ++it) {
                     const int4 item = dm.cell_item[it];
                     const int s = item.x & ~GRID_ALWAYS_INSIDE;
-                    const bool same_level = item.y >= 0 ? ((floor_uniform ? (item.y & 0xFF) : (item.y >> 8)) == base + k)
+                    const bool same_level = item.y >= 0 ? ((floor_uniform ? (item.y & 0xFFFF) : (item.y >> 16)) == base + k)
                                                         : (m->sector_heights[2 * s + (floor_uniform ? 0 : 1)] == level);
                     if (!same_level) continue;
                     if (cd < best || (cd == best && s < best_sector)) {
@@ -2850,11 +2851,13 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
 // ---------------------------------------------------------------------------------------------
 #define SHADE_TILES 52   // 256-pixel tiles per block: 260 tiles per view = 5 blocks per lane (each block stages the tables once)
 #define SHADE_GROUP 4    // tiles per step
-template <bool DEPTH>   // DEPTH: also keep the depth of every pixel no wall tier covers (frames that draw decals)
+// DEPTH: also keep the depth of every pixel no wall tier covers (frames that draw decals).  STAGED: the lane's plane table
+// is short enough for LDS (the kernel then reads it with LDS instructions; a pointer that may be either costs more).
+template <bool DEPTH, bool STAGED>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) plane_shade_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
     const gd_map_desc *m = &dm.d;
     __shared__ float4 sector_lds[LDS_SECTORS];
-    __shared__ unsigned short sector_level_lds[LDS_SECTORS];
+    __shared__ unsigned int sector_level_lds[LDS_SECTORS];
     __shared__ TexLds tex_lds;
     __shared__ unsigned char colormap_lds[32 * 256];
     __shared__ i64 level_plane_lds[2 * PLANE_LEVELS * 2];
@@ -2865,14 +2868,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))
     stage_tables(m, sector_lds, &tex_lds, tb);
     for (int k = threadIdx.x; k < 32 * 256 / 4; k += blockDim.x) reinterpret_cast<unsigned int *>(colormap_lds)[k] = reinterpret_cast<const unsigned int *>(m->colormap)[k];
     const int floors = m->floor_level_count, levels = floors + m->ceil_level_count;
-    const bool tabled = dm.sector_level != nullptr;   // implies both level lists fit PLANE_LEVELS
+    const bool tabled = dm.sector_level != nullptr;
+    const bool levels_staged = STAGED;
     if (tabled) {
         for (int s = threadIdx.x; s < tb.sector_cached; s += blockDim.x) sector_level_lds[s] = dm.sector_level[s];
-        for (int k = threadIdx.x; k < 2 * levels; k += blockDim.x) level_plane_lds[k] = sc.level_plane[(size_t)local * levels * 2 + k];
+        if (levels_staged) for (int k = threadIdx.x; k < 2 * levels; k += blockDim.x) level_plane_lds[k] = sc.level_plane[(size_t)local * levels * 2 + k];
         if (threadIdx.x < STEP_TABLE) step_scale_lds[threadIdx.x] = sc.step_scale[(size_t)local * STEP_TABLE + threadIdx.x];
     }
     __syncthreads();
-    LaneTables lt; lt.level_plane = level_plane_lds; lt.step_scale = step_scale_lds; lt.floors = floors;
+    LaneTables lt; lt.step_scale = step_scale_lds; lt.floors = floors;
+    if (STAGED) lt.level_plane = level_plane_lds;
+    else lt.level_plane = sc.level_plane + (size_t)local * levels * 2;
     const LaneCtx &c = sc.ctx[local];
     unsigned char *frame = frame_base + (size_t)local * frame_stride;
     // SHADE_GROUP tiles per step and three stages per step (per-pixel words, texels, stores), each
@@ -2900,8 +2906,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))
             const int y = pixel / SW, x = pixel - y * SW;
             const bool is_floor = (meta[j] & META_FLOOR) != 0;
             const int sector = ps;
-            const unsigned short pair = sector < tb.sector_cached ? sector_level_lds[sector] : dm.sector_level[sector];
-            texel_at[j] = flat_sample_tabled(tb, c, lt, sc.row_slope[(size_t)local * VH + y], is_floor ? (pair & 0xFF) : (pair >> 8),
+            const unsigned int pair = sector < tb.sector_cached ? sector_level_lds[sector] : dm.sector_level[sector];
+            texel_at[j] = flat_sample_tabled(tb, c, lt, sc.row_slope[(size_t)local * VH + y], is_floor ? (pair & 0xFFFF) : (pair >> 16),
                                              sector, is_floor, x, y, &colormap_row[j]);
             texel[j] = m->tex_atlas[texel_at[j]];
         }
@@ -3668,7 +3674,7 @@ __global__ void __launch_bounds__(BAND_THREADS) __attribute__((amdgpu_waves_per_
     __shared__ struct { float4 sector[LDS_SECTORS]; unsigned char colormap[32 * 256]; } shading_lds;
     float4 *sector_lds = shading_lds.sector;
     unsigned char *colormap_lds = shading_lds.colormap;
-    __shared__ unsigned short sector_level_lds[LDS_SECTORS];
+    __shared__ unsigned int sector_level_lds[LDS_SECTORS];
     __shared__ TexLds tex_lds;
     __shared__ i64 level_plane_lds[2 * PLANE_LEVELS * 2];
     __shared__ i64 step_scale_lds[STEP_TABLE];
@@ -3689,10 +3695,11 @@ __global__ void __launch_bounds__(BAND_THREADS) __attribute__((amdgpu_waves_per_
     stage_tables(m, sector_lds, &tex_lds, tb);
     for (int k = tid; k < 32 * 256 / 4; k += BAND_THREADS) reinterpret_cast<unsigned int *>(colormap_lds)[k] = reinterpret_cast<const unsigned int *>(m->colormap)[k];
     const int floors = m->floor_level_count, levels = floors + m->ceil_level_count;
-    const bool tabled = dm.sector_level != nullptr;   // implies both level lists fit PLANE_LEVELS
+    const bool tabled = dm.sector_level != nullptr;
+    const bool levels_staged = levels <= 2 * PLANE_LEVELS;
     if (tabled) {
         for (int s = tid; s < tb.sector_cached; s += BAND_THREADS) sector_level_lds[s] = dm.sector_level[s];
-        for (int k = tid; k < 2 * levels; k += BAND_THREADS) level_plane_lds[k] = sc.level_plane[(size_t)local * levels * 2 + k];
+        if (levels_staged) for (int k = tid; k < 2 * levels; k += BAND_THREADS) level_plane_lds[k] = sc.level_plane[(size_t)local * levels * 2 + k];
         if (tid < STEP_TABLE) step_scale_lds[tid] = sc.step_scale[(size_t)local * STEP_TABLE + tid];
     }
     if (tid < 256) {
@@ -3709,7 +3716,8 @@ __global__ void __launch_bounds__(BAND_THREADS) __attribute__((amdgpu_waves_per_
     }
     __syncthreads();
     const LaneCtx L = sc.ctx[local];
-    LaneTables lt; lt.level_plane = level_plane_lds; lt.step_scale = step_scale_lds; lt.floors = floors;
+    LaneTables lt; lt.step_scale = step_scale_lds; lt.floors = floors;
+    lt.level_plane = levels_staged ? level_plane_lds : sc.level_plane + (size_t)local * levels * 2;
     // --- the status bar rows of this band (engine.py:15232-15267); empty without status bar patches
     for (int p = tid; p < (BAND_ROWS - view_rows) * SW; p += BAND_THREADS)
         band_bytes[view_rows * SW + p] = hud_count > 0 ? hud_pixel(ov.d, hud_list, hud_count, p % SW, row0 + view_rows + p / SW - VH) : (unsigned char)0;
@@ -3735,8 +3743,8 @@ __global__ void __launch_bounds__(BAND_THREADS) __attribute__((amdgpu_waves_per_
             texel[j] = 0; colormap_row[j] = 0;
             if (!shade[j]) continue;
             const bool is_floor = (meta[j] & META_FLOOR) != 0;
-            const unsigned short pair = ps < tb.sector_cached ? sector_level_lds[ps] : dm.sector_level[ps];
-            const size_t texel_at = flat_sample_tabled(tb, L, lt, yslope, is_floor ? (pair & 0xFF) : (pair >> 8), ps, is_floor, j * 64 + lane_id, y, &colormap_row[j]);
+            const unsigned int pair = ps < tb.sector_cached ? sector_level_lds[ps] : dm.sector_level[ps];
+            const size_t texel_at = flat_sample_tabled(tb, L, lt, yslope, is_floor ? (pair & 0xFFFF) : (pair >> 16), ps, is_floor, j * 64 + lane_id, y, &colormap_row[j]);
             texel[j] = m->tex_atlas[texel_at];
         }
 #pragma unroll
@@ -4339,8 +4347,10 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     auto shade_planes = [&]() {
         if (fused) return;
         const dim3 grid(((VH * SW + 255) / 256 + SHADE_TILES - 1) / SHADE_TILES, count);
-        if (decals) hipLaunchKernelGGL(plane_shade_kernel<true>, grid, dim3(256), 0, stream, r->dm, count, sc, frame_base, frame_stride);
-        else hipLaunchKernelGGL(plane_shade_kernel<false>, grid, dim3(256), 0, stream, r->dm, count, sc, frame_base, frame_stride);
+        const bool staged = m.floor_level_count + m.ceil_level_count <= 2 * PLANE_LEVELS;
+        auto kernel = decals ? (staged ? plane_shade_kernel<true, true> : plane_shade_kernel<true, false>)
+                             : (staged ? plane_shade_kernel<false, true> : plane_shade_kernel<false, false>);
+        hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, r->dm, count, sc, frame_base, frame_stride);
     };
     if (!beside) shade_planes();
     mark();
@@ -4517,16 +4527,15 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
         }
         if (rc == GD_OK) rc = upload(r, blocking_slot.data(), blocking_slot.size(), &r->dm.wall_blocking_slot);
         r->dm.sector_level = nullptr;
-        std::vector<unsigned short> pairs(S, 0);
-        bool listed = false;
-        if (h->floor_level_count <= PLANE_LEVELS && h->ceil_level_count <= PLANE_LEVELS) {
-            listed = true;
+        std::vector<unsigned int> pairs(S, 0);
+        bool listed = h->floor_level_count <= 65535 && h->ceil_level_count <= 65535;
+        if (listed) {
             for (size_t s = 0; s < S; ++s) {
                 int fi = -1, ci = -1;
                 for (int l = 0; l < h->floor_level_count; ++l) if (h->floor_levels[l] == h->sector_heights[2 * s]) fi = l;
                 for (int l = 0; l < h->ceil_level_count; ++l) if (h->ceil_levels[l] == h->sector_heights[2 * s + 1]) ci = l;
                 listed = listed && fi >= 0 && ci >= 0;
-                pairs[s] = (unsigned short)((fi & 0xFF) | ((ci & 0xFF) << 8));
+                pairs[s] = ((unsigned)fi & 0xFFFFu) | (((unsigned)ci & 0xFFFFu) << 16);
             }
             // a sector whose height is missing from the level lists keeps the per-pixel divisions
             if (listed && rc == GD_OK) rc = upload(r, pairs.data(), pairs.size(), &r->dm.sector_level);
@@ -4545,6 +4554,8 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
                 if (w < 0 || (size_t)w >= W) { if (rc == GD_OK) rc = fail(GD_E_ARG, "grid_item_edges holds a linedef index out of range"); continue; }
                 cell_edge.push_back(make_float4(h->walls[4 * w], h->walls[4 * w + 1], h->walls[4 * w + 2], h->walls[4 * w + 3]));
             }
+            // .y: the sector's level indices (as in sector_level), or negative: compare heights (also when the ceiling
+            // index would reach the sign bit)
             cell_item[it] = make_int4(entry, listed ? (int)pairs[s] : -1, first, (int)cell_edge.size());
         }
         if (rc == GD_OK) rc = upload(r, cell_range.data(), cell_range.size(), &r->dm.cell_range);
