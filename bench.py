@@ -33,6 +33,7 @@ POSE_SETS = 4
 # (profiles/render_chain_config4_4096lanes.md).  Measured offline; other workloads report null.
 MEASURED_TRAFFIC_PER_LANE = {
     # (workload, heights, kernel stage)
+    ("config4", "quantised", "wall_columns"): 8.823e9 / 4096,   # 5.80 GiB read + 2.57 GiB written per 4096-lane launch
 }
 
 

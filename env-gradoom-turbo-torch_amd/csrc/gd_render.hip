@@ -4302,8 +4302,8 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     // 320x240 frame in device memory (shade, paint the flat pass's pixels, decals, billboards, overlays, then pool the
     // observation from it), the caller's `indexed` or the working memory's own: the faster way on this chip (its kernels
     // run at full occupancy), and the only one for frames that draw wall decals, which need a per-pixel scene depth.  Or
-    // band by band in LDS (band_finish_kernel), the frame never reaching device memory: a third less traffic for a
-    // caller that only wants observations, at two thirds of the speed; chosen with gd_renderer_set_assembly.
+    // band by band in LDS (band_finish_kernel), the frame never reaching device memory: a fifth less traffic in the
+    // assembly for a caller that only wants observations, at nine tenths of the speed; chosen with gd_renderer_set_assembly.
     const bool decals = lanes->decal_slots > 0 && lanes->decal_state && lanes->decal_geom && r->overlays.d.decal_variant_count > 0;
     if (!decals) sc.scene_depth = nullptr;
     if (decals && (!sc.scene_depth || !sc.frame)) return fail(GD_E_ARG, "decal working memory missing");
