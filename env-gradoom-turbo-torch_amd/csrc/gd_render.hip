@@ -1068,17 +1068,41 @@ __device__ __forceinline__ int flat_select_pixel(const DeviceMap &dm, const Scra
 // One pixel's flat ray on its own (flat_select_pixel shares work between the 64 pixels of a row): the sector of
 // the nearest plane level whose probe point lies in a sector of that level, -1 if there is none
 // (engine.py:10981-11024).
-__device__ int flat_probe_pixel(const DeviceMap &dm, const Scratch &sc, int local, float rc, float rs, float cc, int y) {
+// The plane levels of the map and, per lane and level, bounds of the distance from the camera to the sectors of that
+// level: floors first, then ceilings, in all three lists.  A pixel's scan reads them level after level, each read
+// waiting for the one before (the scan may end at any level), so a block that works on one lane copies them to LDS
+// first: with a plane level per sector (several hundred) the scans otherwise spend their time waiting for device memory.
+#define FLAT_LDS_LEVELS 1024
+struct LevelLists { const float *level, *reach, *far; int floors, ceilings; };
+__device__ __forceinline__ LevelLists stage_level_lists(const DeviceMap &dm, const Scratch &sc, int local, float *lds) {
+    const gd_map_desc *m = &dm.d;
+    LevelLists lists;
+    lists.floors = m->floor_level_count; lists.ceilings = m->ceil_level_count;
+    const int total = lists.floors + lists.ceilings;
+    const float *reach = sc.level_reach + (size_t)local * total, *far = sc.level_far + (size_t)local * total;
+    if (total > FLAT_LDS_LEVELS) {        // read where they are; `level` then only serves the floors (see level_at)
+        lists.level = nullptr; lists.reach = reach; lists.far = far;
+        return lists;
+    }
+    for (int k = threadIdx.x; k < total; k += blockDim.x) {
+        lds[k] = k < lists.floors ? m->floor_levels[k] : m->ceil_levels[k - lists.floors];
+        lds[FLAT_LDS_LEVELS + k] = reach[k];
+        lds[2 * FLAT_LDS_LEVELS + k] = far[k];
+    }
+    lists.level = lds; lists.reach = lds + FLAT_LDS_LEVELS; lists.far = lds + 2 * FLAT_LDS_LEVELS;
+    return lists;   // the caller synchronises the block before the first scan
+}
+
+__device__ int flat_probe_pixel(const DeviceMap &dm, const Scratch &sc, const LevelLists &lists, int local, float rc, float rs, float cc, int y) {
     const LaneCtx &c = sc.ctx[local];
     const gd_map_desc *m = &dm.d;
     const float delta = (float)y - flat_center(c);
     const bool is_floor = delta > 0;
     const float denom = fmaxf(fabsf(delta), 0.5f);
-    const float *levels = is_floor ? m->floor_levels : m->ceil_levels;
-    const int level_count = is_floor ? m->floor_level_count : m->ceil_level_count;
-    // per lane and level: bounds of the distance from the camera to the sectors of that level
-    const size_t bounds_at = (size_t)local * (m->floor_level_count + m->ceil_level_count) + (is_floor ? 0 : m->floor_level_count);
-    const float *reach = sc.level_reach + bounds_at, *far = sc.level_far + bounds_at;
+    const int first = is_floor ? 0 : lists.floors;
+    const float *levels = lists.level ? lists.level + first : (is_floor ? m->floor_levels : m->ceil_levels);
+    const int level_count = is_floor ? lists.floors : lists.ceilings;
+    const float *reach = lists.reach + first, *far = lists.far + first;
     float best = GD_INF; int best_sector = -1;
     const bool camera_in_grid = grid_cell_of(m, c.x, c.y) >= 0;
     for (int k = 0; k < level_count; ++k) {
@@ -1140,10 +1164,14 @@ __global__ void __launch_bounds__(128) flat_list_kernel(DeviceMap dm, gd_lanes_d
         return;
     }
     const int n = lane_base + local;
+    if (listed == 0) return;                         // the same in every thread
+    __shared__ float level_lds[3 * FLAT_LDS_LEVELS];
+    const LevelLists lists = stage_level_lists(dm, sc, local, level_lds);
+    __syncthreads();
     for (int slot = threadIdx.x; slot < listed; slot += blockDim.x) {
         const int pixel = sc.flat_list[(size_t)local * FLAT_LIST_MAX + slot];
         const int y = pixel / SW, x = pixel - y * SW;
-        const int s = flat_probe_pixel(dm, sc, local, lanes.ray_cos[(size_t)n * SW + x], lanes.ray_sin[(size_t)n * SW + x], dm.cosine_correction[x], y);
+        const int s = flat_probe_pixel(dm, sc, lists, local, lanes.ray_cos[(size_t)n * SW + x], lanes.ray_sin[(size_t)n * SW + x], dm.cosine_correction[x], y);
         const size_t i = (size_t)local * VH * SW + pixel;
         sc.flat_sector[i] = (unsigned short)(s < 0 ? c.sector : s);
         sc.flat_flags[i] = s < 0 ? 1 : 0;
@@ -1186,6 +1214,12 @@ __global__ void __launch_bounds__(SW) __attribute__((amdgpu_waves_per_eu(8, 8)))
     }
     __syncthreads();
     const int columns = column_count;
+    __shared__ float level_lds[3 * FLAT_LDS_LEVELS];
+    LevelLists lists;
+    if (columns > 0) {                               // the same in every thread
+        lists = stage_level_lists(dm, sc, local, level_lds);
+        __syncthreads();
+    }
     for (int entry = threadIdx.x >> 6; entry < columns; entry += SW / 64) {
         const int packed = column_list[entry];
         const int x = packed & 511, first = (packed >> 9) & 255, half = packed >> 17;
@@ -1197,7 +1231,7 @@ __global__ void __launch_bounds__(SW) __attribute__((amdgpu_waves_per_eu(8, 8)))
         for (int chunk = chunks - 1; chunk >= 0; --chunk) {
             const int y = first + chunk * 64 + lane_id;
             const bool live = y <= half_end;
-            const int s = live ? flat_probe_pixel(dm, sc, local, rc, rs, cc, y) : -1;
+            const int s = live ? flat_probe_pixel(dm, sc, lists, local, rc, rs, cc, y) : -1;
             const u64 resolved = __ballot(live && s >= 0);
             const u64 lower = resolved & ~((2ULL << lane_id) - 1);   // resolved rows of this chunk below this one (none for lane 63)
             const int from = lower ? __ffsll((long long)lower) - 1 : lane_id;
