@@ -182,6 +182,8 @@ struct Scratch {    // per-chunk working memory, sized at create
     float *level_reach;    // [L, floor levels + ceiling levels] lower bound of the distance from the
                            // camera to any point inside a sector with that plane level
     float *level_far;      // [L, floor levels + ceiling levels] upper bound of that distance
+    unsigned int *level_masks;  // [L, LEVEL_BUCKETS, level_mask_words]: the plane levels a flat probe can reach at all, by
+                                // bucket of the probe's distance scale (see level_bucket)
     i64 *level_plane;      // [L, floor levels + ceiling levels, 2] plane height (16.16) and its visibility factor
     i64 *row_slope;        // [L, 208] plane distance per unit of plane height on each view row
     i64 *step_scale;       // [L, 3, 2, 16] per log2 texture size (widths, then heights): the flat texture step per
@@ -417,6 +419,27 @@ __device__ int sector_at(const gd_map_desc *m, float px, float py) {
     return 0;
 }
 
+// A flat probe of plane level k lands at distance cd = h_k * g from the camera, h_k the level's plane height and
+// g = 192 / |row - centre| / cos(column) the pixel's own scale, and can only hit a sector whose level is k if
+// reach_k <= cd <= far_k (level_reach / level_far): that is, if g lies in [reach_k / h_k, far_k / h_k].  With a plane
+// level per sector a pixel would test hundreds of such intervals to find the few that hold its g, so the lane keeps,
+// for each of LEVEL_BUCKETS ranges of g (6.5 to the octave from g = 0.7 up, the first and last open-ended), a bit set
+// of the levels whose interval reaches into the range, a bucket to spare on either side (far more than the rounding of
+// the logarithm or of g can move anything).  A probe then visits only the levels of its bucket, in level order, and
+// applies the exact test to those: the bit sets only spare it levels the exact test would reject as well.
+#define LEVEL_BUCKETS 64
+#define LEVEL_MASK_WORDS_MAX 32     // up to 1024 plane levels (floors and ceilings together); beyond that every level is visited,
+#define LEVEL_MASK_MIN_LEVELS 64    // and so it is with few levels, where the bit sets cost more than they spare
+__device__ __forceinline__ int level_mask_words(const gd_map_desc *m) {
+    const int levels = m->floor_level_count + m->ceil_level_count;
+    return levels > LEVEL_MASK_MIN_LEVELS && levels <= 32 * LEVEL_MASK_WORDS_MAX ? (levels + 31) / 32 : 0;
+}
+__device__ __forceinline__ int level_bucket(float g) {
+    if (!(g > 0.0f)) return 0;
+    const float b = floorf((__log2f(g) + 0.5f) * 6.5f);
+    return b <= 0.0f ? 0 : (b >= (float)(LEVEL_BUCKETS - 1) ? LEVEL_BUCKETS - 1 : (int)b);
+}
+
 // Per-lane tables for the flat kernels, one block per lane (after lane_setup):
 //  * per plane level, how far the camera is, at least, from every sector at that level: a flat
 //    probe nearer than that cannot land in such a sector (engine.py:10981-11024 tests the point
@@ -434,6 +457,10 @@ __global__ void lane_tables_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
     // the lane's per-column lists start empty
     for (int x = threadIdx.x; x < SW; x += blockDim.x) { sc.cand_count[(size_t)local * SW + x] = 0; sc.block_hit[(size_t)local * SW + x] = ~0ULL; }
     const float cx = lanes.x[lane_base + local], cy = lanes.y[lane_base + local];
+    __shared__ unsigned int masks_lds[LEVEL_BUCKETS * LEVEL_MASK_WORDS_MAX];
+    const int mask_words = level_mask_words(&dm.d);
+    for (int k = threadIdx.x; k < LEVEL_BUCKETS * mask_words; k += blockDim.x) masks_lds[k] = 0u;
+    __syncthreads();
     for (int l = threadIdx.x; l < levels; l += blockDim.x) {
         float reach = GD_INF, far = 0.0f;
         for (int k = dm.level_box_ofs[l]; k < dm.level_box_ofs[l + 1]; ++k) {
@@ -447,10 +474,17 @@ __global__ void lane_tables_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
         sc.level_reach[(size_t)local * levels + l] = reach * 0.999f - 0.5f;
         sc.level_far[(size_t)local * levels + l] = far * 1.001f + 0.5f;
         const float plane_height = l < floors ? (c.view_z - dm.d.floor_levels[l]) : (dm.d.ceil_levels[l - floors] - c.view_z);
+        if (mask_words > 0 && plane_height > 0.0f && far >= reach) {      // a level at or beyond the eye shows no plane
+            const float low = (reach * 0.999f - 0.5f) / plane_height, high = (far * 1.001f + 0.5f) / plane_height;
+            const int first = max(level_bucket(low) - 1, 0), last = min(level_bucket(high) + 1, LEVEL_BUCKETS - 1);
+            for (int b = first; b <= last; ++b) atomicOr(&masks_lds[b * mask_words + (l >> 5)], 1u << (l & 31));
+        }
         const i64 plane_height_fixed = round_to_i64(plane_height * 65536.0f);
         sc.level_plane[((size_t)local * levels + l) * 2] = plane_height_fixed;
         sc.level_plane[((size_t)local * levels + l) * 2 + 1] = min64(tdiv(FLOOR_VISIBILITY_FIXED << 16, max64(plane_height_fixed, 1)), (1LL << 31) - 1);
     }
+    __syncthreads();
+    for (int k = threadIdx.x; k < LEVEL_BUCKETS * mask_words; k += blockDim.x) sc.level_masks[(size_t)local * LEVEL_BUCKETS * mask_words + k] = masks_lds[k];
     for (int py = threadIdx.x; py < VH; py += blockDim.x) {
         i64 center_row = c.center_fixed >> 16;
         i64 pixel_y_fixed = (i64)py * FIXED_UNIT;
@@ -945,6 +979,8 @@ __device__ bool flat_ray_resolves(const DeviceMap &dm, const LaneCtx &c, float r
 // flat_select_pixel is called by whole wavefronts whose 64 lanes look at 64 pixels of ONE row of one lane's
 // screen (wanted or not: every lane takes part in the level broadcasts); it returns the sector, -1 if no
 // level's probe point lies in a sector of that level.
+// MASKS: the map has enough plane levels for the per-bucket bit sets (level_mask_words() > 0).
+template <bool MASKS>
 __device__ __forceinline__ int flat_select_pixel(const DeviceMap &dm, const Scratch &sc, const gd_lanes_desc &lanes, int local, int n,
                                                  int x, int y, bool wanted) {
     const gd_map_desc *m = &dm.d;
@@ -982,8 +1018,28 @@ __device__ __forceinline__ int flat_select_pixel(const DeviceMap &dm, const Scra
     float best = GD_INF; int best_sector = -1;
     const bool camera_in_grid = grid_cell_of(m, c.x, c.y) >= 0;
     bool done = !wanted;
+    // The levels some pixel of the wavefront can reach at all (level_bucket): the bit sets of the buckets its 64 scales
+    // fall into, joined; lane j holds word j.  Levels outside them are skipped by the whole wavefront at once.
+    const int mask_words = MASKS ? level_mask_words(m) : 0;
+    unsigned int joined_word = 0u;
+    if (MASKS) {
+        const int bucket = level_bucket((192.0f / denom) / cc);
+        int lowest = bucket, highest = bucket;
+#pragma unroll
+        for (int step = 1; step < 64; step <<= 1) { lowest = min(lowest, __shfl_xor(lowest, step)); highest = max(highest, __shfl_xor(highest, step)); }
+        const unsigned int *masks = sc.level_masks + (size_t)local * LEVEL_BUCKETS * mask_words;
+        if (slot_in_wave < mask_words) for (int b = lowest; b <= highest; ++b) joined_word |= masks[b * mask_words + slot_in_wave];
+    }
+    const int first_bit = floor_uniform ? 0 : m->floor_level_count;
     for (int base = 0; base < level_count; base += 64) {
         if (__ballot(!done) == 0) break;   // every lane takes part in the level broadcasts below, wanted or not
+        u64 chunk_levels = ~0ULL;          // bit k: level base + k is worth a look
+        if (MASKS) {
+            const int at = first_bit + base, word = at >> 5, shift = at & 31;
+            const u64 w0 = (unsigned)bcast((int)joined_word, word), w1 = (unsigned)bcast((int)joined_word, (word + 1) & 63), w2 = (unsigned)bcast((int)joined_word, (word + 2) & 63);
+            chunk_levels = ((w0 | (w1 << 32)) >> shift) | (shift ? w2 << (64 - shift) : 0ULL);   // lanes past the last word hold zeros
+            if (chunk_levels == 0ULL) continue;    // the same in every lane
+        }
         // lane k works out level base+k: its height and perpendicular distance (one division for
         // the wavefront instead of one per level per lane); a level the plane cannot show gets -1
         const int mine = base + slot_in_wave;
@@ -1005,6 +1061,7 @@ __device__ __forceinline__ int flat_select_pixel(const DeviceMap &dm, const Scra
                 const int k = k0 + j;
                 cdv[j] = -1.0f; finev[j] = 0x40000000u; cellv[j] = -1;
                 if (k >= chunk) continue;                        // the same in every lane
+                if (MASKS && !((chunk_levels >> k) & 1ULL)) continue;   // the same in every lane: no pixel here reaches the level
                 const float perpendicular = bcast(my_perpendicular, k);
                 const float nearest = bcast(my_reach, k);
                 if (!(perpendicular > 0)) continue;              // the same in every lane
@@ -1072,24 +1129,28 @@ __device__ __forceinline__ int flat_select_pixel(const DeviceMap &dm, const Scra
 // level: floors first, then ceilings, in all three lists.  A pixel's scan reads them level after level, each read
 // waiting for the one before (the scan may end at any level), so a block that works on one lane copies them to LDS
 // first: with a plane level per sector (several hundred) the scans otherwise spend their time waiting for device memory.
-#define FLAT_LDS_LEVELS 1024
-struct LevelLists { const float *level, *reach, *far; int floors, ceilings; };
-__device__ __forceinline__ LevelLists stage_level_lists(const DeviceMap &dm, const Scratch &sc, int local, float *lds) {
+#define FLAT_LDS_LEVELS (32 * LEVEL_MASK_WORDS_MAX)
+struct LevelLists { const float *level, *reach, *far; const unsigned int *masks; int floors, ceilings, mask_words; };
+struct LevelLds { float lists[3 * FLAT_LDS_LEVELS]; };
+__device__ __forceinline__ LevelLists stage_level_lists(const DeviceMap &dm, const Scratch &sc, int local, LevelLds *lds) {
     const gd_map_desc *m = &dm.d;
     LevelLists lists;
     lists.floors = m->floor_level_count; lists.ceilings = m->ceil_level_count;
+    lists.mask_words = level_mask_words(m);
     const int total = lists.floors + lists.ceilings;
     const float *reach = sc.level_reach + (size_t)local * total, *far = sc.level_far + (size_t)local * total;
-    if (total > FLAT_LDS_LEVELS) {        // read where they are; `level` then only serves the floors (see level_at)
-        lists.level = nullptr; lists.reach = reach; lists.far = far;
+    if (total > FLAT_LDS_LEVELS) {        // read where they are; `level` then only serves the floors (see flat_probe_pixel)
+        lists.level = nullptr; lists.reach = reach; lists.far = far; lists.masks = nullptr;   // more levels than the bit sets cover
         return lists;
     }
     for (int k = threadIdx.x; k < total; k += blockDim.x) {
-        lds[k] = k < lists.floors ? m->floor_levels[k] : m->ceil_levels[k - lists.floors];
-        lds[FLAT_LDS_LEVELS + k] = reach[k];
-        lds[2 * FLAT_LDS_LEVELS + k] = far[k];
+        lds->lists[k] = k < lists.floors ? m->floor_levels[k] : m->ceil_levels[k - lists.floors];
+        lds->lists[FLAT_LDS_LEVELS + k] = reach[k];
+        lds->lists[2 * FLAT_LDS_LEVELS + k] = far[k];
     }
-    lists.level = lds; lists.reach = lds + FLAT_LDS_LEVELS; lists.far = lds + 2 * FLAT_LDS_LEVELS;
+    const unsigned int *masks = sc.level_masks + (size_t)local * LEVEL_BUCKETS * lists.mask_words;
+    lists.level = lds->lists; lists.reach = lds->lists + FLAT_LDS_LEVELS; lists.far = lds->lists + 2 * FLAT_LDS_LEVELS;
+    lists.masks = masks;   // one row of a few words per pixel: read where it is
     return lists;   // the caller synchronises the block before the first scan
 }
 
@@ -1105,29 +1166,27 @@ __device__ int flat_probe_pixel(const DeviceMap &dm, const Scratch &sc, const Le
     const float *reach = lists.reach + first, *far = lists.far + first;
     float best = GD_INF; int best_sector = -1;
     const bool camera_in_grid = grid_cell_of(m, c.x, c.y) >= 0;
-    for (int k = 0; k < level_count; ++k) {
+    // one level of the scan; true ends it
+    auto visit = [&](int k) -> bool {
         const float level = levels[k];
         const float height = is_floor ? (c.view_z - level) : (level - c.view_z);
-        if (!(height > 0)) continue;
+        if (!(height > 0)) return false;
         const float cd = (height * 192.0f / denom) / cc;
-        if (!(finitef(cd) && cd > 0)) continue;
-        if (cd > best) break;                                   // later levels are at least this far
-        if (cd < reach[k] || cd > far[k]) continue;            // no sector of this level lies at that distance
+        if (!(finitef(cd) && cd > 0)) return false;
+        if (cd > best) return true;                                 // later levels are at least this far
+        if (cd < reach[k] || cd > far[k]) return false;            // no sector of this level lies at that distance
         const float px = c.x + rc * cd, py = c.y + rs * cd;
         int cell;
         const unsigned fine = fine_lookup(m, dm.fine_inverse, px, py, &cell);
         const unsigned kind = FINE_KIND(fine);
-        if (kind == FINE_EMPTY) continue;
+        if (kind == FINE_EMPTY) return false;
         if (kind == FINE_DECIDED) {
             const int s = (int)(fine & 0xFFFFu);
             if (m->sector_heights[2 * s + (is_floor ? 0 : 1)] == level && (cd < best || (cd == best && s < best_sector))) { best = cd; best_sector = s; }
-            continue;
+            return false;
         }
         if (cell < 0) cell = grid_cell_of(m, px, py);
-        if (cell < 0) {                                         // outside the grid no sector holds the point
-            if (camera_in_grid) break;                          // and this ray has left that convex region for good
-            continue;
-        }
+        if (cell < 0) return camera_in_grid;   // outside the grid no sector holds the point; seen from inside it, the ray has left that convex region for good
         const int2 range = dm.cell_range[cell];
         for (int it = range.x; it < range.y; ++it) {
             const int4 item = dm.cell_item[it];
@@ -1137,6 +1196,20 @@ __device__ int flat_probe_pixel(const DeviceMap &dm, const Scratch &sc, const Le
                 if ((item.x & GRID_ALWAYS_INSIDE) || inside_edge_copies(dm.cell_edge, item.z, item.w, px, py)) { best = cd; best_sector = s; }
             }
         }
+        return false;
+    };
+    if (lists.mask_words == 0 || !lists.masks) {
+        for (int k = 0; k < level_count; ++k) if (visit(k)) break;
+        return best_sector;
+    }
+    // only the levels whose distance bounds can hold a probe of this pixel's scale at all (level_bucket), in level order
+    const unsigned int *row = lists.masks + level_bucket((192.0f / denom) / cc) * lists.mask_words;
+    const int end = first + level_count;     // bits [first, end) of the row are this half's levels
+    for (int w = first >> 5; w <= (end - 1) >> 5; ++w) {
+        unsigned int bits = row[w];
+        if (w == first >> 5) bits &= ~0u << (first & 31);
+        if (w == (end - 1) >> 5 && (end & 31)) bits &= (1u << (end & 31)) - 1u;
+        for (; bits; bits &= bits - 1) if (visit((w << 5) + __ffs((int)bits) - 1 - first)) return best_sector;
     }
     return best_sector;
 }
@@ -1165,8 +1238,8 @@ __global__ void __launch_bounds__(128) flat_list_kernel(DeviceMap dm, gd_lanes_d
     }
     const int n = lane_base + local;
     if (listed == 0) return;                         // the same in every thread
-    __shared__ float level_lds[3 * FLAT_LDS_LEVELS];
-    const LevelLists lists = stage_level_lists(dm, sc, local, level_lds);
+    __shared__ LevelLds level_lds;
+    const LevelLists lists = stage_level_lists(dm, sc, local, &level_lds);
     __syncthreads();
     for (int slot = threadIdx.x; slot < listed; slot += blockDim.x) {
         const int pixel = sc.flat_list[(size_t)local * FLAT_LIST_MAX + slot];
@@ -1214,10 +1287,10 @@ __global__ void __launch_bounds__(SW) __attribute__((amdgpu_waves_per_eu(8, 8)))
     }
     __syncthreads();
     const int columns = column_count;
-    __shared__ float level_lds[3 * FLAT_LDS_LEVELS];
+    __shared__ LevelLds level_lds;
     LevelLists lists;
     if (columns > 0) {                               // the same in every thread
-        lists = stage_level_lists(dm, sc, local, level_lds);
+        lists = stage_level_lists(dm, sc, local, &level_lds);
         __syncthreads();
     }
     for (int entry = threadIdx.x >> 6; entry < columns; entry += SW / 64) {
@@ -1415,13 +1488,14 @@ __device__ __forceinline__ size_t flat_sample_tabled(const Tables &tb, const Lan
 // resolved pixels are never repaired.
 // Every pixel of the noted rows: the blocks take the rows of the work list in turn, so that lanes with many rows
 // and lanes with none load the chip alike.  One block per row at a time, one wavefront per 64 columns.
+template <bool MASKS>
 __global__ void __launch_bounds__(SW) __attribute__((amdgpu_waves_per_eu(8, 8))) flat_span_select_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
     const int total = *sc.flat_row_count;
     const int x = threadIdx.x;
     for (int entry = blockIdx.x; entry < total; entry += gridDim.x) {
         const int packed = sc.flat_rows[entry];
         const int local = packed >> 8, y = packed & 255;
-        const int s = flat_select_pixel(dm, sc, lanes, local, lane_base + local, x, y, true);
+        const int s = flat_select_pixel<MASKS>(dm, sc, lanes, local, lane_base + local, x, y, true);
         const size_t i = (size_t)local * VH * SW + (size_t)y * SW + x;
         sc.flat_sector[i] = (unsigned short)(s < 0 ? sc.ctx[local].sector : s);
         sc.flat_flags[i] = s < 0 ? 1 : 0;
@@ -1432,6 +1506,7 @@ __global__ void __launch_bounds__(SW) __attribute__((amdgpu_waves_per_eu(8, 8)))
 // (engine.py:11026-11083).  One block per (lane, 64-column strip); its TAIL_ROWS wavefronts select that many rows
 // at a time, while any of the strip's columns is still looking.
 #define TAIL_ROWS 8
+template <bool MASKS>
 __global__ void __launch_bounds__(64 * TAIL_ROWS) flat_tail_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
     __shared__ int found_lds[TAIL_ROWS][64];
     const int local = blockIdx.y;
@@ -1452,7 +1527,7 @@ __global__ void __launch_bounds__(64 * TAIL_ROWS) flat_tail_kernel(DeviceMap dm,
             if (!__syncthreads_or(looking)) break;   // also keeps the rows of the previous step apart from this one's
             const int y = y0 + wave;
             int s = -1;
-            if (y <= half_end) s = flat_select_pixel(dm, sc, lanes, local, n, x, y, looking);   // the same in a whole wavefront
+            if (y <= half_end) s = flat_select_pixel<MASKS>(dm, sc, lanes, local, n, x, y, looking);   // the same in a whole wavefront
             found_lds[wave][slot] = s;
             __syncthreads();
             if (looking) {
@@ -4171,6 +4246,7 @@ size_t carve_scratch(Scratch &sc, unsigned char *base, size_t L, const gd_map_de
     take(&sc.clip_depth, L * PX);
     take(&sc.level_reach, L * levels);
     take(&sc.level_far, L * levels);
+    take(&sc.level_masks, L * LEVEL_BUCKETS * (size_t)(levels <= 32 * LEVEL_MASK_WORDS_MAX ? (levels + 31) / 32 : 1));
     take(&sc.level_plane, L * levels * 2);
     take(&sc.row_slope, L * (size_t)VH);
     take(&sc.step_scale, L * STEP_TABLE);
@@ -4391,9 +4467,11 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     // the flat pass, where the walls left it something to decide
     hipLaunchKernelGGL(flat_list_kernel, dim3(count), dim3(128), 0, flat_stream, r->dm, *lanes, base, count, sc);
     hipLaunchKernelGGL(flat_gap_column_kernel, dim3(count), dim3(SW), 0, flat_stream, r->dm, *lanes, base, count, sc);
-    hipLaunchKernelGGL(flat_span_select_kernel, dim3(SPAN_SELECT_BLOCKS), dim3(SW), 0, flat_stream, r->dm, *lanes, base, count, sc);
+    const int plane_levels = m.floor_level_count + m.ceil_level_count;
+    const bool level_masks = plane_levels > LEVEL_MASK_MIN_LEVELS && plane_levels <= 32 * LEVEL_MASK_WORDS_MAX;   // level_mask_words() > 0
+    hipLaunchKernelGGL(level_masks ? flat_span_select_kernel<true> : flat_span_select_kernel<false>, dim3(SPAN_SELECT_BLOCKS), dim3(SW), 0, flat_stream, r->dm, *lanes, base, count, sc);
     mark();
-    hipLaunchKernelGGL(flat_tail_kernel, dim3(SW / 64, count), dim3(64 * TAIL_ROWS), 0, flat_stream, r->dm, *lanes, base, count, sc);
+    hipLaunchKernelGGL(level_masks ? flat_tail_kernel<true> : flat_tail_kernel<false>, dim3(SW / 64, count), dim3(64 * TAIL_ROWS), 0, flat_stream, r->dm, *lanes, base, count, sc);
     hipLaunchKernelGGL(flat_span_finish_kernel, dim3(count), dim3(SW), 0, flat_stream, r->dm, *lanes, base, count, sc);
     if (!fused) hipLaunchKernelGGL(flat_shade_kernel, dim3(count), dim3(128), 0, flat_stream, r->dm, count, sc, frame_base, frame_stride);
     if (beside) {
