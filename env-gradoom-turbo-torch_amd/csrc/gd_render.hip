@@ -169,8 +169,8 @@ struct Scratch {    // per-chunk working memory, sized at create
     int *flat_rows;        // [L*208] the noted rows of every lane as one work list, entry = lane << 8 | row
     int *flat_row_count;   // [1] its length (cleared by lane_setup_kernel, filled by flat_gap_column_kernel)
     int *flat_col_top;     // [L,2,320] per screen half and column: the topmost shown pixel the flat pass could not
-                           // resolve (any value >= 208: none).  flat_list_kernel lowers it, flat_gap_column_kernel
-                           // reads it and puts "none" back, so it is filled once, when the renderer is created.
+                           // resolve (any value >= 208: none).  flat_gap_column_kernel lowers it while it selects the
+                           // gap pixels, then reads it and puts "none" back, so it is filled once, when the renderer is created.
     unsigned int *meta;    // [L,208,320] filled | floor | plane_sector+1 | clip_wall+1
     float *clip_depth;     // [L,208,320]
     unsigned char *frame;  // [L,240,320] when the caller wants no indexed output
@@ -1198,18 +1198,28 @@ __device__ int flat_probe_pixel(const DeviceMap &dm, const Scratch &sc, const Le
         }
         return false;
     };
-    if (lists.mask_words == 0 || !lists.masks) {
-        for (int k = 0; k < level_count; ++k) if (visit(k)) break;
-        return best_sector;
-    }
-    // only the levels whose distance bounds can hold a probe of this pixel's scale at all (level_bucket), in level order
-    const unsigned int *row = lists.masks + level_bucket((192.0f / denom) / cc) * lists.mask_words;
-    const int end = first + level_count;     // bits [first, end) of the row are this half's levels
-    for (int w = first >> 5; w <= (end - 1) >> 5; ++w) {
-        unsigned int bits = row[w];
-        if (w == first >> 5) bits &= ~0u << (first & 31);
-        if (w == (end - 1) >> 5 && (end & 31)) bits &= (1u << (end & 31)) - 1u;
-        for (; bits; bits &= bits - 1) if (visit((w << 5) + __ffs((int)bits) - 1 - first)) return best_sector;
+    // With bit sets: only the levels whose distance bounds can hold a probe of this pixel's scale at all (level_bucket),
+    // in level order; bits [first, end) of the bucket's row are this half's levels.  Without: every level.
+    const bool masked = lists.mask_words > 0 && lists.masks;
+    const unsigned int *row = masked ? lists.masks + level_bucket((192.0f / denom) / cc) * lists.mask_words : nullptr;
+    const int end = first + level_count;
+    int word = (first >> 5) - 1, k = -1;
+    unsigned int bits = 0u;
+    for (;;) {
+        if (masked) {
+            while (!bits && word < ((end - 1) >> 5)) {
+                ++word;
+                bits = row[word];
+                if (word == first >> 5) bits &= ~0u << (first & 31);
+                if (word == (end - 1) >> 5 && (end & 31)) bits &= (1u << (end & 31)) - 1u;
+            }
+            if (!bits) break;
+            k = (word << 5) + __ffs((int)bits) - 1 - first;
+            bits &= bits - 1;
+        } else if (++k >= level_count) {
+            break;
+        }
+        if (visit(k)) break;
     }
     return best_sector;
 }
@@ -1218,59 +1228,53 @@ __device__ int flat_probe_pixel(const DeviceMap &dm, const Scratch &sc, const Le
 // shows it; a pixel a plane of the wall pass claimed only asks whether the flat ray resolved at all, and only
 // where a sprite stands behind the plane with no sprite clip recorded, which the sprite pass finds out for
 // itself (flat_ray_resolves); the few pixels left (columns whose traversal left a gap) show the flat pass's
-// picture.  plane_shade_kernel lists those; this kernel selects them, one thread per listed pixel, and notes,
-// per lane and screen half, the rows where one stayed unresolved: flat_span_select_kernel and
-// flat_span_finish_kernel select and repair those rows, flat_shade_kernel paints the listed pixels.
-__global__ void __launch_bounds__(128) flat_list_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
-    const int local = blockIdx.x;
-    if (local >= lane_count) return;
-    const int listed = sc.flat_list_count[local];
-    const LaneCtx &c = sc.ctx[local];
-    int *span = sc.flat_span + (size_t)local * 4;
-    if (listed > FLAT_LIST_MAX) {
-        // too many to list (a camera outside the map, say): every row of both halves is selected and repaired
-        if (threadIdx.x == 0) {
-            const int last_ceiling_row = c.last_ceiling_row;
-            if (last_ceiling_row >= 0) { span[0] = 0; span[1] = last_ceiling_row; }
-            if (last_ceiling_row + 1 < VH) { span[2] = last_ceiling_row + 1; span[3] = VH - 1; }
-        }
-        return;
-    }
-    const int n = lane_base + local;
-    if (listed == 0) return;                         // the same in every thread
-    __shared__ LevelLds level_lds;
-    const LevelLists lists = stage_level_lists(dm, sc, local, &level_lds);
-    __syncthreads();
-    for (int slot = threadIdx.x; slot < listed; slot += blockDim.x) {
-        const int pixel = sc.flat_list[(size_t)local * FLAT_LIST_MAX + slot];
-        const int y = pixel / SW, x = pixel - y * SW;
-        const int s = flat_probe_pixel(dm, sc, lists, local, lanes.ray_cos[(size_t)n * SW + x], lanes.ray_sin[(size_t)n * SW + x], dm.cosine_correction[x], y);
-        const size_t i = (size_t)local * VH * SW + pixel;
-        sc.flat_sector[i] = (unsigned short)(s < 0 ? c.sector : s);
-        sc.flat_flags[i] = s < 0 ? 1 : 0;
-        if (s < 0) {
-            const bool floor_row = ((float)y - flat_center(c)) > 0;
-            atomicMin(&sc.flat_col_top[((size_t)local * 2 + (floor_row ? 1 : 0)) * SW + x], y);
-        }
-    }
-}
-
-// The vertical repair (engine.py:11026-11083) of the listed pixels, column by column.  An unresolved pixel takes
+// picture.  wall_columns_kernel lists those.  flat_gap_column_kernel, one block per lane, first selects them, one
+// thread per listed pixel, and notes per screen half and column the topmost one that stayed unresolved.
+//
+// Then the vertical repair (engine.py:11026-11083) of the listed pixels, column by column.  An unresolved pixel takes
 // the sector of the next resolved pixel below it in its half of the screen; when that sector is not the camera's,
 // the pixel is its own left and right anchor in the horizontal repair (engine.py:11085-11135), which then leaves
 // it as it is: such a pixel is settled here and its row needs no further work.  Only the rows of the others (no
-// resolved pixel below, or the camera's own sector) are noted for the row kernels.  One block per lane; a
-// wavefront takes one column that holds an unresolved listed pixel after another, its lanes probing 64 rows of the column at a time, from the bottom of the half up to the column's topmost
-// unresolved listed pixel.
+// resolved pixel below, or the camera's own sector) are noted for the row kernels (flat_span_select_kernel,
+// flat_tail_kernel, flat_span_finish_kernel).  A wavefront takes one column that holds an unresolved listed pixel
+// after another, its lanes probing 64 rows of the column at a time, from the bottom of the half up to the column's
+// topmost unresolved listed pixel.
 __global__ void __launch_bounds__(SW) __attribute__((amdgpu_waves_per_eu(8, 8))) flat_gap_column_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
     const int local = blockIdx.x;
     if (local >= lane_count) return;
+    const int listed = sc.flat_list_count[local];
+    if (listed == 0) return;                         // the same in every thread: a lane without gap pixels has no flat pass
     const LaneCtx &c = sc.ctx[local];
     const int n = lane_base + local;
     const int lane_id = threadIdx.x & 63;
     int *span = sc.flat_span + (size_t)local * 4;
     const int last_ceiling_row = c.last_ceiling_row;
     const unsigned int *meta = sc.meta + (size_t)local * VH * SW;
+    __shared__ LevelLds level_lds;
+    const LevelLists lists = stage_level_lists(dm, sc, local, &level_lds);
+    __syncthreads();
+    if (listed > FLAT_LIST_MAX) {
+        // too many to list (a camera outside the map, say): every row of both halves is selected and repaired
+        if (threadIdx.x == 0) {
+            if (last_ceiling_row >= 0) { span[0] = 0; span[1] = last_ceiling_row; }
+            if (last_ceiling_row + 1 < VH) { span[2] = last_ceiling_row + 1; span[3] = VH - 1; }
+        }
+    } else {
+        for (int slot = threadIdx.x; slot < listed; slot += blockDim.x) {
+            const int pixel = sc.flat_list[(size_t)local * FLAT_LIST_MAX + slot];
+            const int y = pixel / SW, x = pixel - y * SW;
+            const int s = flat_probe_pixel(dm, sc, lists, local, lanes.ray_cos[(size_t)n * SW + x], lanes.ray_sin[(size_t)n * SW + x], dm.cosine_correction[x], y);
+            const size_t i = (size_t)local * VH * SW + pixel;
+            sc.flat_sector[i] = (unsigned short)(s < 0 ? c.sector : s);
+            sc.flat_flags[i] = s < 0 ? 1 : 0;
+            if (s < 0) {
+                const bool floor_row = ((float)y - flat_center(c)) > 0;
+                atomicMin(&sc.flat_col_top[((size_t)local * 2 + (floor_row ? 1 : 0)) * SW + x], y);
+            }
+        }
+    }
+    __threadfence_block();   // what the selection wrote (column tops, row ranges) is read below by other threads of the block
+    __syncthreads();
     // the block's columns with work, both halves together, dealt out to its wavefronts in turn (the columns of a
     // gap are neighbours: taken strip by strip, one wavefront would do them all)
     __shared__ int column_list[2 * SW];
@@ -1279,7 +1283,7 @@ __global__ void __launch_bounds__(SW) __attribute__((amdgpu_waves_per_eu(8, 8)))
     __syncthreads();
     for (int half = 0; half < 2; ++half) {
         int *top_at = sc.flat_col_top + ((size_t)local * 2 + half) * SW + threadIdx.x;
-        const int top = *top_at;
+        const int top = __hip_atomic_load(top_at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // where the atomics above wrote, not a cached copy
         if (top < VH) {
             *top_at = VH;
             column_list[atomicAdd(&column_count, 1)] = (int)threadIdx.x | (top << 9) | (half << 17);
@@ -1287,12 +1291,6 @@ __global__ void __launch_bounds__(SW) __attribute__((amdgpu_waves_per_eu(8, 8)))
     }
     __syncthreads();
     const int columns = column_count;
-    __shared__ LevelLds level_lds;
-    LevelLists lists;
-    if (columns > 0) {                               // the same in every thread
-        lists = stage_level_lists(dm, sc, local, &level_lds);
-        __syncthreads();
-    }
     for (int entry = threadIdx.x >> 6; entry < columns; entry += SW / 64) {
         const int packed = column_list[entry];
         const int x = packed & 511, first = (packed >> 9) & 255, half = packed >> 17;
@@ -2942,7 +2940,7 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
     // what is left of a window no one-sided drawseg closed shows the flat pass's picture
     if (!window_dirty) zero_rows(pb, gaps, x, st.ceiling_clip <= 0.0f ? 0 : (int)st.ceiling_clip, st.floor_clip >= (float)VH ? VH : (int)st.floor_clip);
     masked_midtexture<DEPTH, SPLIT>(cc, st, pb, colormap_lds);
-    // The view pixels no wall tier, plane or masked texture covers: the flat pass selects them (flat_list_kernel) and
+    // The view pixels no wall tier, plane or masked texture covers: the flat pass selects them (flat_gap_column_kernel) and
     // flat_shade_kernel paints them.  More than the list holds: the lane is handled pixel by pixel.
     for (int y = gaps.lo(), gap_end = gaps.hi(); y < gap_end; ++y) {
         const unsigned int word = pb.m(y);
@@ -4465,7 +4463,6 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     if (!beside) shade_planes();
     mark();
     // the flat pass, where the walls left it something to decide
-    hipLaunchKernelGGL(flat_list_kernel, dim3(count), dim3(128), 0, flat_stream, r->dm, *lanes, base, count, sc);
     hipLaunchKernelGGL(flat_gap_column_kernel, dim3(count), dim3(SW), 0, flat_stream, r->dm, *lanes, base, count, sc);
     const int plane_levels = m.floor_level_count + m.ceil_level_count;
     const bool level_masks = plane_levels > LEVEL_MASK_MIN_LEVELS && plane_levels <= 32 * LEVEL_MASK_WORDS_MAX;   // level_mask_words() > 0
