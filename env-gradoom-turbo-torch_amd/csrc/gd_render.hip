@@ -2508,7 +2508,7 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
 
 // engine.py:12885-13371
 template <bool SPLIT>
-__device__ __forceinline__ bool pass_advance(const ColumnCtx &cc, ColumnState &c, const PassColumn &r, PixelBuffers &pb, SilhouetteBounds &sb, bool window_untouched) {
+__device__ __forceinline__ bool pass_advance(const ColumnCtx &cc, ColumnState &c, const PassColumn &r, PixelBuffers &pb, SilhouetteBounds &sb, bool window_untouched, GapRange &gaps) {
     const gd_map_desc *m = cc.m;
     const MapView &mv = cc.mv;
     const LaneCtx &L = *cc.c;
@@ -2575,6 +2575,14 @@ __device__ __forceinline__ bool pass_advance(const ColumnCtx &cc, ColumnState &c
         float new_ceiling = c.ceiling_clip, new_floor = c.floor_clip;
         if (p_draws_upper || p_marks_ceiling) new_ceiling = p_draws_upper ? pcub : pct;
         if (p_draws_lower || p_marks_floor) new_floor = p_draws_lower ? pclt : pcb;
+        if (window_untouched) {
+            // These clips move without anything being painted or claimed: the rows they take out of an untouched
+            // window would leave it unwritten.  They show the flat pass's picture.
+            auto row_of = [](float clip) { return clip <= 0.0f ? 0 : (clip >= (float)VH ? VH : (int)clip); };
+            const int window_top = row_of(c.ceiling_clip), window_bottom = row_of(c.floor_clip);
+            zero_rows(pb, gaps, x, window_top, min(row_of(new_ceiling), window_bottom));
+            zero_rows(pb, gaps, x, max(row_of(new_floor), window_top), window_bottom);
+        }
         c.ceiling_clip = new_ceiling; c.floor_clip = new_floor;
         bool pmasked = ptex[0] >= 0;
         bool pbottom = (r.view_floor > pof) || (L.view_z < pof) || pmasked;
@@ -2931,7 +2939,7 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
         for (int t = 0; t < 3; ++t) group_valid[t] = same_group && all_tier[t] && (common_top[t] < common_bottom[t]);
         if (!done) {
             pass_paint<DEPTH>(cc, st, pc, pb, group_valid, common_bottom, first_group_visibility, colormap_lds, window_dirty, gaps);
-            bool changed = pass_advance<SPLIT>(cc, st, pc, pb, sb, !window_dirty);
+            bool changed = pass_advance<SPLIT>(cc, st, pc, pb, sb, !window_dirty, gaps);
             // A pass that found nothing and changed nothing repeats identically for ever.
             if (!(pc.bits & PB_VALID) && !changed) done = true;
         }

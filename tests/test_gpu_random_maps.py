@@ -110,6 +110,70 @@ def test_random_maps_with_other_heights_and_textures_whatever_the_working_memory
         renderer.close()
 
 
+def closed_door_case(seed: int, lanes: int):
+    """random_case plus hand-closed doors and crawl spaces on up to four sectors, then (seven times in ten) other heights,
+    texture sizes and lights over the whole map."""
+    from gradoom_amd import mapbuild, synthmap
+    from gradoom_amd.selfcheck import make_lane_arrays
+
+    rng = np.random.default_rng(seed)
+    layout, grid, sectors, linedefs, islands, pillars = SHAPES[seed % len(SHAPES)]
+    smap = synthmap.generate_map(seed, grid=grid, sectors=sectors, linedefs=linedefs, layout=layout, islands=islands, pillars=pillars,
+                                 midtex=float(rng.choice([0.0, 0.1, 0.3])))
+    if rng.random() < 0.7:
+        heights = np.array(smap.sector_heights, copy=True)
+        for sector in rng.choice(len(heights), size=min(4, len(heights)), replace=False):
+            if int(rng.choice([0, 2])) == 0:
+                heights[sector, 1] = heights[sector, 0]        # a closed door
+            else:
+                heights[sector, 0] = heights[sector, 1] - 8    # a crawl space
+        smap.sector_heights[...] = heights
+    if rng.random() < 0.7:
+        smap = synthmap.with_variant(smap, seed + 9, heights=[None, "uniform", "doors"][int(rng.integers(0, 3))],
+                                     textures=[None, "mixed", "npot"][int(rng.integers(0, 3))], lights=bool(rng.random() < 0.5))
+    if rng.random() < 0.4:
+        smap = synthmap.split_linedefs(smap, seed + 1)
+    if rng.random() < 0.5:
+        smap = synthmap.with_blend_tables(smap, seed + 2)
+    margin = float(rng.choice([0.005, 0.02, 0.15]))
+    poses = synthmap.generate_poses(smap, lanes, seed + 3, pitch=bool(rng.random() < 0.6), flash=bool(rng.random() < 0.5), margin=margin)
+    if rng.random() < 0.3:
+        poses.pitch_bam[:] = rng.integers(-30, 31, lanes) * (182 << 16)
+    sprites = synthmap.generate_sprites(smap, lanes, 24, seed + 4)
+    arrays = make_lane_arrays(smap, poses, sprites)
+    arrays["sprite_style"] = rng.choice(np.array([-1, -1, -1, -2, 0, 1], dtype=np.int8), size=sprites.x.shape)
+    return smap, mapbuild.build_map_tables(smap), arrays
+
+
+@pytest.mark.parametrize("seed", [50078, 50079, 50082])
+def test_rows_that_only_a_portal_path_clip_closes_show_the_flat_picture(oracle, seed):
+    """Seed 50078, lanes 7 and 14: a column loses its sector, picks a linedef beyond a projected solid and takes that
+    path's clips, which close the window over rows 51..97 without painting or claiming one of them (engine.py:12969-13069).
+    The reference shows the flat pass's picture there; the traversal has to hand those rows to the flat pass itself, since
+    nothing clears its working memory between frames."""
+    from gradoom_amd import hostmath
+    from gradoom_amd.renderer import HipRenderer, LaneState
+
+    lanes = 16
+    cosine = hostmath.cosine_correction("cpu").numpy()
+    smap, tables, arrays = closed_door_case(seed, lanes)
+    expected = oracle.render(tables, arrays, cosine)
+    renderer = HipRenderer(smap, lanes, "cuda:0", cosine_correction=cosine, tables=tables)
+    state = LaneState.from_numpy(arrays, "cuda:0")
+    for fill, assembly in ((None, "separate"), (0xA5, "fused"), (0xFF, "separate")):
+        renderer.set_assembly(assembly)
+        if fill is not None:
+            renderer.scribble(fill)
+        indexed = torch.zeros((lanes, 240, 320), dtype=torch.uint8, device="cuda:0")
+        obs = torch.zeros((lanes, 84, 84), dtype=torch.uint8, device="cuda:0")
+        renderer.render(state, indexed=indexed, obs=obs)
+        torch.cuda.synchronize()
+        assert renderer.status() == 0
+        assert np.array_equal(indexed.cpu().numpy(), expected["indexed"]), f"seed {seed} fill {fill} {assembly}"
+        assert np.array_equal(obs.cpu().numpy(), expected["obs"]), f"seed {seed} fill {fill} {assembly}"
+    renderer.close()
+
+
 def test_cameras_outside_the_map_match_the_oracle(oracle):
     """Cameras in the void beside the map: no wall pass claims most of the screen, so nearly every pixel shows the
     flat pass's picture (far more than the per-lane gap pixel list holds) and most of them stay unresolved."""
