@@ -381,6 +381,7 @@ __device__ __forceinline__ int grid_cell_of(const gd_map_desc *m, float px, floa
 #define FINE_UNKNOWN 3u
 #define FINE_MASK_LEVELS 15
 #define FLAT_BATCH 2       // plane levels probed together in flat_select
+#define FLAT_BATCH_MASKED 3   // ... on maps with bit sets of reachable levels, where a batch holds levels that are looked at
 
 // Fine raster lookup.  Points outside the raster (or not finite) report FINE_UNKNOWN with a
 // negative cell, and the caller locates them with grid_cell_of.  The coarse cell of a point
@@ -1021,6 +1022,7 @@ __device__ __forceinline__ int flat_select_pixel(const DeviceMap &dm, const Scra
     // The levels some pixel of the wavefront can reach at all (level_bucket): the bit sets of the buckets its 64 scales
     // fall into, joined; lane j holds word j.  Levels outside them are skipped by the whole wavefront at once.
     const int mask_words = MASKS ? level_mask_words(m) : 0;
+    constexpr int BATCH = MASKS ? FLAT_BATCH_MASKED : FLAT_BATCH;
     unsigned int joined_word = 0u;
     if (MASKS) {
         const int bucket = level_bucket((192.0f / denom) / cc);
@@ -1049,19 +1051,29 @@ __device__ __forceinline__ int flat_select_pixel(const DeviceMap &dm, const Scra
         const float my_height = floor_uniform ? (c.view_z - my_level) : (my_level - c.view_z);
         const float my_perpendicular = (mine < level_count && my_height > 0) ? my_height * 192.0f / denom : -1.0f;
         const int chunk = level_count - base < 64 ? level_count - base : 64;
-        // Levels are taken FLAT_BATCH at a time: first the probe points and raster loads of the whole
+        // Levels are taken BATCH at a time: first the probe points and raster loads of the whole
         // batch (independent, so their memory latencies overlap), then the decisions in level order.
         // A load for a level past the one that ends the scan is wasted, never wrong.
-        for (int k0 = 0; k0 < chunk && !done; k0 += FLAT_BATCH) {
-            float cdv[FLAT_BATCH];
-            unsigned finev[FLAT_BATCH];
-            int cellv[FLAT_BATCH];
+        // Only the levels whose bit is set are walked (with bit sets: the few that some pixel here can reach), so a
+        // batch holds BATCH levels that are looked at, not BATCH list positions.  `rest` is the same in every lane.
+        if (chunk < 64) chunk_levels &= (1ULL << chunk) - 1ULL;
+        u64 rest = ((u64)(unsigned)__builtin_amdgcn_readfirstlane((int)(chunk_levels >> 32)) << 32) | (u64)(unsigned)__builtin_amdgcn_readfirstlane((int)chunk_levels);
+        while (rest != 0ULL) {
+            if (__ballot(!done) == 0) break;
+            float cdv[BATCH];
+            unsigned finev[BATCH];
+            int cellv[BATCH];
+            int kv[BATCH];
 #pragma unroll
-            for (int j = 0; j < FLAT_BATCH; ++j) {
-                const int k = k0 + j;
+            for (int j = 0; j < BATCH; ++j) {
+                kv[j] = rest ? __ffsll((long long)rest) - 1 : -1;
+                rest &= rest - 1ULL;
+            }
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) {
+                const int k = kv[j];
                 cdv[j] = -1.0f; finev[j] = 0x40000000u; cellv[j] = -1;
-                if (k >= chunk) continue;                        // the same in every lane
-                if (MASKS && !((chunk_levels >> k) & 1ULL)) continue;   // the same in every lane: no pixel here reaches the level
+                if (k < 0) continue;                             // the same in every lane
                 const float perpendicular = bcast(my_perpendicular, k);
                 const float nearest = bcast(my_reach, k);
                 if (!(perpendicular > 0)) continue;              // the same in every lane
@@ -1075,13 +1087,13 @@ __device__ __forceinline__ int flat_select_pixel(const DeviceMap &dm, const Scra
                     cd = perpendicular / cc;
                 }
                 cdv[j] = cd;
-                if (!(finitef(cd) && cd > 0) || cd > best || cd < nearest) continue;   // cd < nearest: every sector at this level is farther away
+                if (done || !(finitef(cd) && cd > 0) || cd > best || cd < nearest) continue;   // cd < nearest: every sector at this level is farther away
                 finev[j] = fine_lookup_cells(m, __builtin_fmaf(cd, cell_dx, cell_x0), __builtin_fmaf(cd, cell_dy, cell_y0), &cellv[j]);
             }
 #pragma unroll
-            for (int j = 0; j < FLAT_BATCH; ++j) {
-                const int k = k0 + j;
-                if (k >= chunk || done) continue;
+            for (int j = 0; j < BATCH; ++j) {
+                const int k = kv[j];
+                if (k < 0 || done) continue;
                 const float cd = cdv[j];
                 if (!(finitef(cd) && cd > 0)) continue;
                 if (cd > best) { done = true; continue; }        // later levels are at least this far
