@@ -4461,36 +4461,37 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     mark();
     // The plane shading and the flat pass do not depend on each other: the first reads the per-pixel words and writes the
     // pixels some drawseg owns, the second reads the same words and writes its own planes and, at the end, the pixels no
-    // drawseg owns.  The flat pass is a chain of short kernels that wait more than they compute, so it runs on the
-    // renderer's side stream while the shading keeps the vector units busy.  (Not when stages are being timed.)
+    // drawseg owns.  The flat pass is a chain of short kernels that wait more than they compute; it stays on the
+    // caller's stream, where its first kernel starts the moment the traversal ends, and the shading goes to the renderer's
+    // side stream, a few microseconds behind (the other way round the shading takes every compute unit before the first
+    // block of the flat pass is placed).  (Not when stages are being timed.)
     const bool beside = !fused && !timed && r->side_ready;
-    hipStream_t flat_stream = stream;
+    hipStream_t shade_stream = stream;
     if (beside) {
         HIP_TRY(hipEventRecord(r->fork_event, stream));
         HIP_TRY(hipStreamWaitEvent(r->side_stream, r->fork_event, 0));
-        flat_stream = r->side_stream;
+        shade_stream = r->side_stream;
     }
-    // timed (and so serial): shading, then the flat pass, each between its own marks.  Otherwise the flat pass is queued
-    // first, so that its few busy blocks find room at once and the shading fills the rest of the chip around them.
+    // timed (and so serial): shading, then the flat pass, each between its own marks
     auto shade_planes = [&]() {
         if (fused) return;
         const dim3 grid(((VH * SW + 255) / 256 + SHADE_TILES - 1) / SHADE_TILES, count);
         const bool staged = m.floor_level_count + m.ceil_level_count <= 2 * PLANE_LEVELS;
         auto kernel = decals ? (staged ? plane_shade_kernel<true, true> : plane_shade_kernel<true, false>)
                              : (staged ? plane_shade_kernel<false, true> : plane_shade_kernel<false, false>);
-        hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, r->dm, count, sc, frame_base, frame_stride);
+        hipLaunchKernelGGL(kernel, grid, dim3(256), 0, shade_stream, r->dm, count, sc, frame_base, frame_stride);
     };
     if (!beside) shade_planes();
     mark();
     // the flat pass, where the walls left it something to decide
-    hipLaunchKernelGGL(flat_gap_column_kernel, dim3(count), dim3(SW), 0, flat_stream, r->dm, *lanes, base, count, sc);
+    hipLaunchKernelGGL(flat_gap_column_kernel, dim3(count), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
     const int plane_levels = m.floor_level_count + m.ceil_level_count;
     const bool level_masks = plane_levels > LEVEL_MASK_MIN_LEVELS && plane_levels <= 32 * LEVEL_MASK_WORDS_MAX;   // level_mask_words() > 0
-    hipLaunchKernelGGL(level_masks ? flat_span_select_kernel<true> : flat_span_select_kernel<false>, dim3(SPAN_SELECT_BLOCKS), dim3(SW), 0, flat_stream, r->dm, *lanes, base, count, sc);
+    hipLaunchKernelGGL(level_masks ? flat_span_select_kernel<true> : flat_span_select_kernel<false>, dim3(SPAN_SELECT_BLOCKS), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
     mark();
-    hipLaunchKernelGGL(level_masks ? flat_tail_kernel<true> : flat_tail_kernel<false>, dim3(SW / 64, count), dim3(64 * TAIL_ROWS), 0, flat_stream, r->dm, *lanes, base, count, sc);
-    hipLaunchKernelGGL(flat_span_finish_kernel, dim3(count), dim3(SW), 0, flat_stream, r->dm, *lanes, base, count, sc);
-    if (!fused) hipLaunchKernelGGL(flat_shade_kernel, dim3(count), dim3(128), 0, flat_stream, r->dm, count, sc, frame_base, frame_stride);
+    hipLaunchKernelGGL(level_masks ? flat_tail_kernel<true> : flat_tail_kernel<false>, dim3(SW / 64, count), dim3(64 * TAIL_ROWS), 0, stream, r->dm, *lanes, base, count, sc);
+    hipLaunchKernelGGL(flat_span_finish_kernel, dim3(count), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
+    if (!fused) hipLaunchKernelGGL(flat_shade_kernel, dim3(count), dim3(128), 0, stream, r->dm, count, sc, frame_base, frame_stride);
     if (beside) {
         shade_planes();
         HIP_TRY(hipEventRecord(r->join_event, r->side_stream));
