@@ -1251,7 +1251,11 @@ __device__ int flat_probe_pixel(const DeviceMap &dm, const Scratch &sc, const Le
 // flat_tail_kernel, flat_span_finish_kernel).  A wavefront takes one column that holds an unresolved listed pixel
 // after another, its lanes probing 64 rows of the column at a time, from the bottom of the half up to the column's
 // topmost unresolved listed pixel.
-__global__ void __launch_bounds__(SW) __attribute__((amdgpu_waves_per_eu(8, 8))) flat_gap_column_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
+// GAP_THREADS: three wavefronts a lane.  Most lanes have a few dozen listed pixels and one or two columns to repair, and a
+// launch lasts as many rounds of blocks as the chip needs to hold them all: with five wavefronts a block (one thread a
+// column) it took 0.05 ms longer, with one or two the lanes with many columns hold it up.
+#define GAP_THREADS 192
+__global__ void __launch_bounds__(GAP_THREADS) __attribute__((amdgpu_waves_per_eu(8, 8))) flat_gap_column_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
     const int local = blockIdx.x;
     if (local >= lane_count) return;
     const int listed = sc.flat_list_count[local];
@@ -1293,17 +1297,17 @@ __global__ void __launch_bounds__(SW) __attribute__((amdgpu_waves_per_eu(8, 8)))
     __shared__ int column_count;
     if (threadIdx.x == 0) column_count = 0;
     __syncthreads();
-    for (int half = 0; half < 2; ++half) {
-        int *top_at = sc.flat_col_top + ((size_t)local * 2 + half) * SW + threadIdx.x;
+    for (int half = 0; half < 2; ++half) for (int x = threadIdx.x; x < SW; x += blockDim.x) {
+        int *top_at = sc.flat_col_top + ((size_t)local * 2 + half) * SW + x;
         const int top = __hip_atomic_load(top_at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // where the atomics above wrote, not a cached copy
         if (top < VH) {
             *top_at = VH;
-            column_list[atomicAdd(&column_count, 1)] = (int)threadIdx.x | (top << 9) | (half << 17);
+            column_list[atomicAdd(&column_count, 1)] = x | (top << 9) | (half << 17);
         }
     }
     __syncthreads();
     const int columns = column_count;
-    for (int entry = threadIdx.x >> 6; entry < columns; entry += SW / 64) {
+    for (int entry = threadIdx.x >> 6; entry < columns; entry += blockDim.x / 64) {
         const int packed = column_list[entry];
         const int x = packed & 511, first = (packed >> 9) & 255, half = packed >> 17;
         const int half_end = half ? VH - 1 : last_ceiling_row;
@@ -1513,11 +1517,13 @@ __global__ void __launch_bounds__(SW) __attribute__((amdgpu_waves_per_eu(8, 8)))
 }
 
 // A column whose pixel in the last noted row of a half is unresolved looks further down for a resolved one
-// (engine.py:11026-11083).  One block per (lane, 64-column strip); its TAIL_ROWS wavefronts select that many rows
-// at a time, while any of the strip's columns is still looking.
-#define TAIL_ROWS 8
+// (engine.py:11026-11083).  One block per (lane, 64-column strip); its tail_rows() wavefronts select that many rows
+// at a time, while any of the strip's columns is still looking.  Eight rows a step suit maps with few plane levels, where
+// a resolved row is usually near; with a level per sector a search runs further and sixteen are quicker.
+constexpr int tail_rows(bool masks) { return masks ? 16 : 8; }
 template <bool MASKS>
-__global__ void __launch_bounds__(64 * TAIL_ROWS) flat_tail_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
+__global__ void __launch_bounds__(64 * tail_rows(MASKS)) flat_tail_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc) {
+    constexpr int TAIL_ROWS = tail_rows(MASKS);
     __shared__ int found_lds[TAIL_ROWS][64];
     const int local = blockIdx.y;
     if (local >= lane_count) return;
@@ -1572,13 +1578,25 @@ __global__ void __launch_bounds__(SW) flat_span_finish_kernel(DeviceMap dm, gd_l
         const int below = sc.flat_tail[((size_t)local * 2 + half) * SW + x];
         bool found = below >= 0;
         int span_sector = found ? below : 0;
-        for (int y = hi[half]; y >= lo[half]; --y) {
-            const size_t i = (size_t)y * SW + x;
-            if (!(flags[i] & 1)) { found = true; span_sector = sector[i]; }
-            else if (found) {
-                sector[i] = (unsigned short)span_sector;
-                // bit1: vertical span; bit2: its sector differs from the camera's (anchor)
-                flags[i] = (unsigned char)(1 | 2 | ((span_sector != c.sector) ? 4 : 0));
+        // eight rows at a time, their loads first: a column's rows are its own, so no store of the loop touches them
+        for (int y0 = hi[half]; y0 >= lo[half]; y0 -= 8) {
+            unsigned char row_flags[8]; unsigned short row_sector[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int y = y0 - j < lo[half] ? lo[half] : y0 - j;
+                row_flags[j] = flags[(size_t)y * SW + x]; row_sector[j] = sector[(size_t)y * SW + x];
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int y = y0 - j;
+                if (y < lo[half]) break;
+                const size_t i = (size_t)y * SW + x;
+                if (!(row_flags[j] & 1)) { found = true; span_sector = row_sector[j]; }
+                else if (found) {
+                    sector[i] = (unsigned short)span_sector;
+                    // bit1: vertical span; bit2: its sector differs from the camera's (anchor)
+                    flags[i] = (unsigned char)(1 | 2 | ((span_sector != c.sector) ? 4 : 0));
+                }
             }
         }
     }
@@ -4484,12 +4502,12 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     if (!beside) shade_planes();
     mark();
     // the flat pass, where the walls left it something to decide
-    hipLaunchKernelGGL(flat_gap_column_kernel, dim3(count), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
+    hipLaunchKernelGGL(flat_gap_column_kernel, dim3(count), dim3(GAP_THREADS), 0, stream, r->dm, *lanes, base, count, sc);
     const int plane_levels = m.floor_level_count + m.ceil_level_count;
     const bool level_masks = plane_levels > LEVEL_MASK_MIN_LEVELS && plane_levels <= 32 * LEVEL_MASK_WORDS_MAX;   // level_mask_words() > 0
     hipLaunchKernelGGL(level_masks ? flat_span_select_kernel<true> : flat_span_select_kernel<false>, dim3(SPAN_SELECT_BLOCKS), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
     mark();
-    hipLaunchKernelGGL(level_masks ? flat_tail_kernel<true> : flat_tail_kernel<false>, dim3(SW / 64, count), dim3(64 * TAIL_ROWS), 0, stream, r->dm, *lanes, base, count, sc);
+    hipLaunchKernelGGL(level_masks ? flat_tail_kernel<true> : flat_tail_kernel<false>, dim3(SW / 64, count), dim3(64 * tail_rows(level_masks)), 0, stream, r->dm, *lanes, base, count, sc);
     hipLaunchKernelGGL(flat_span_finish_kernel, dim3(count), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
     if (!fused) hipLaunchKernelGGL(flat_shade_kernel, dim3(count), dim3(128), 0, stream, r->dm, count, sc, frame_base, frame_stride);
     if (beside) {
