@@ -1,6 +1,6 @@
 """Headline benchmark: rendered lane-frames/s (320x240 indexed + 84x84x4 observation) on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--repeats R] [--workload config4] [--heights quantised|uniform]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--repeats R] [--workload config4] [--heights uniform|quantised]
                     [--lanes N] [--mode full|obs-only|rgb] [--assembly auto|fused|separate] [--no-cpu]
 
 A step is one pass of the whole hot path over one batch of lanes whose inputs already sit in
@@ -28,13 +28,21 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 POSE_SETS = 4
-# HBM bytes one launch of a kernel moves, per lane, on the config4 workload: rocprofv3 FETCH_SIZE + WRITE_SIZE
-# of a 4096-lane launch, each scaled by what the same counter reads for a 1 GiB copy
-# (profiles/render_chain_config4_4096lanes.md).  Measured offline; other workloads report null.
-MEASURED_TRAFFIC_PER_LANE = {
-    # (workload, heights, kernel stage)
-    ("config4", "quantised", "wall_columns"): 8.823e9 / 4096,   # 5.80 GiB read + 2.57 GiB written per 4096-lane launch
-}
+# HBM bytes one launch of a kernel moves: rocprofv3 FETCH_SIZE + WRITE_SIZE of a launch, each scaled by what the
+# same counter reads for a 1 GiB copy in the same run.  Measured offline with the commands the summaries under
+# profiles/ give and kept, per (workload, heights, mode, kernel), in profiles/hbm_traffic.json; a workload that was
+# not measured reports null.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+
+
+def measured_traffic_per_lane(workload: str, heights: str, mode: str, kernel: str):
+    try:
+        with open(TRAFFIC_FILE) as handle:
+            table = json.load(handle)["bytes_per_launch"]
+    except (OSError, KeyError, ValueError):
+        return None
+    entry = table.get(f"{workload}/{heights}/{mode}/{kernel}")
+    return None if entry is None else entry["bytes"] / entry["lanes"]
 
 
 def algorithmic_bytes_per_lane_frame(sprites: int, map_bytes: int, lanes: int, mode: str) -> float:
@@ -55,9 +63,9 @@ def main() -> int:
     parser.add_argument("--warmup", type=int, default=2)
     parser.add_argument("--repeats", type=int, default=5, help="timed repeats of --steps steps each; the median is reported")
     parser.add_argument("--workload", default="config4")
-    parser.add_argument("--heights", choices=("quantised", "uniform"), default="quantised",
-                        help="sector heights: the map generator's (floors 0..96 and ceilings 160..256 in steps of 8: 13 plane levels "
-                             "each way) or uniform (floors 0..255, ceilings 64..256 above, whole units: a plane level per sector)")
+    parser.add_argument("--heights", choices=("uniform", "quantised"), default="uniform",
+                        help="sector heights: uniform (floors 0..255, ceilings 64..256 above, whole units: a plane level per sector; the "
+                             "benchmark's distribution) or quantised (floors 0..96 and ceilings 160..256 in steps of 8: 13 plane levels each way)")
     parser.add_argument("--lanes", type=int, default=None)
     parser.add_argument("--mode", choices=("full", "obs-only", "rgb"), default="full",
                         help="full: indexed frame + observation stack (the headline metric); obs-only: observation stack "
@@ -164,7 +172,7 @@ def main() -> int:
     # render_timed sums a stage over the chunks of one frame; one launch handles `chunk` lanes
     launch_ms = stage_ms[dominant] / chunks
     achieved = bytes_per_lane * chunk / (launch_ms * 1e-3) / 1e9 if launch_ms > 0 else 0.0
-    per_lane_traffic = MEASURED_TRAFFIC_PER_LANE.get((args.workload, args.heights, dominant)) if lanes >= chunk else None
+    per_lane_traffic = measured_traffic_per_lane(args.workload, args.heights, args.mode, dominant + "_kernel") if lanes >= chunk else None
     traffic = None if per_lane_traffic is None else round(per_lane_traffic * chunk)
     roofline = dict(
         bound="hbm", kernel=dominant + "_kernel", achieved=round(achieved, 3), peak=HBM_PEAK_GBPS, unit="GB/s",

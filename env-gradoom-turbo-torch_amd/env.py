@@ -140,6 +140,7 @@ class GraDoomVecEnv:
         renderer=None,
         episode_timeout: int = 32,
         sprites: int = 0,
+        action_count: int = 17,
     ):
         if num_envs <= 0:
             raise ValueError("num_envs must be positive")
@@ -159,6 +160,9 @@ class GraDoomVecEnv:
         self.observation_buffer_depth = {"copy": None, "safe_view": 2, "unsafe_view": 1}[obs_copy]
         self.observation_renderer = "reference"
         self.closed = False
+        self.action_count = int(action_count)   # len(action_table); 17 in the reference's pinned table (actions.py:33-51)
+        if self.action_count <= 0:
+            raise ValueError("action table must contain at least one action")
         self._renderer = renderer if renderer is not None else HipRenderer(smap, self.num_envs, self.device)
         self._dynamics = dynamics if dynamics is not None else PosePoolDynamics(
             smap, self.num_envs, self.device, sprites=sprites, episode_timeout=episode_timeout
@@ -169,6 +173,7 @@ class GraDoomVecEnv:
         self.signal_buffer = torch.zeros((n, SIGNAL_COUNT), dtype=torch.float32, device=self.device)
         self._info_history = torch.zeros((n, 0, self.frame_stack), dtype=torch.float32, device=self.device)
         self._initialized = torch.zeros(n, dtype=torch.bool, device=self.device)
+        self.pending_reset = torch.ones(n, dtype=torch.bool, device=self.device)   # engine.py:1661
         self._latest_reset_seeds = torch.zeros(n, dtype=torch.int64, device=self.device)
         self._all_lanes = torch.ones(n, dtype=torch.uint8, device=self.device)
         # obs_copy="safe_view": two buffers handed out in turn, so that the observation of the step before stays
@@ -200,6 +205,7 @@ class GraDoomVecEnv:
 
     def _update_signals(self) -> None:
         self.signal_buffer[:, 17].copy_(self._dynamics.episode_time)  # episode_time, engine.py:15469
+        self.signal_buffer[:, 20].copy_(self.pending_reset)           # engine.py:15472
 
     # ------------------------------------------------------------------ device API
     def reset_device(self, mask: torch.Tensor, seeds: torch.Tensor):
@@ -218,6 +224,7 @@ class GraDoomVecEnv:
                               final_frames=view, final_layout=self.obs_layout)
         self._latest_reset_seeds.copy_(torch.where(device_mask, device_seeds, self._latest_reset_seeds))
         self._initialized |= device_mask
+        self.pending_reset.masked_fill_(device_mask, False)   # engine.py:2409
         self._update_signals()
         return self._device_observations(self.frames), self.signal_buffer
 
@@ -229,6 +236,7 @@ class GraDoomVecEnv:
             raise RuntimeError("cannot step a closed environment")
         indices = self._require_device_tensor(actions, "actions", shape=(self.num_envs,), dtypes=INDEX_DTYPES).to(torch.int64)
         rewards, terminated, truncated = self._dynamics.step(indices)
+        self.pending_reset.copy_(terminated | truncated)      # engine.py:9542
         self._renderer.render(self._dynamics.lane_state(), frames=self.frames, final_frames=final_frames, final_layout=final_layout)
         self._update_signals()
         return DeviceTransition(
@@ -318,15 +326,26 @@ class GraDoomVecEnv:
             raise RuntimeError("cannot step a closed environment")
         if not bool(torch.all(self._initialized)):
             raise RuntimeError("all lanes must be reset before the first step")
+        if bool(torch.any(self.pending_reset)):   # env.py:819-821
+            lanes = torch.nonzero(self.pending_reset).flatten().to("cpu").tolist()
+            raise RuntimeError(f"terminal lanes must be reset before step: {lanes}")
+        # every argument is checked before the observation buffer is taken: a refused call must not advance the
+        # safe_view rotation, or the next step would write into the buffer the caller still holds (env.py:459-472)
+        indices = self._require_device_tensor(actions, "actions", shape=(self.num_envs,), dtypes=INDEX_DTYPES).to(torch.int64)
+        if bool(torch.any((indices < 0) | (indices >= self.action_count))):   # env.py:828-829
+            raise ValueError("actions fall outside the declared action space")
         view = self._view_target()
-        transition = self._step(actions, view, self.obs_layout)
+        transition = self._step(indices, view, self.obs_layout)
         observations = transition.observations if view is None else view
         return observations, transition.rewards, transition.terminated, transition.truncated, {}
 
     # ------------------------------------------------------------------ RGB frames
-    def _rgb_frames(self) -> torch.Tensor:
-        rgb = torch.empty((self.num_envs, 240, 320, 3), dtype=torch.uint8, device=self.device)
-        self._renderer.render(self._dynamics.lane_state(), rgb=rgb)
+    def _rgb_frames(self, lane: int | None = None) -> torch.Tensor:
+        state = self._dynamics.lane_state()
+        if lane is not None:   # one lane's frame: only that lane is rendered
+            state = state.select(slice(lane, lane + 1))
+        rgb = torch.empty((state.x.shape[0], 240, 320, 3), dtype=torch.uint8, device=self.device)
+        self._renderer.render(state, rgb=rgb)
         return rgb
 
     def render_lane(self, lane: int):  # env.py:1037-1053
@@ -339,7 +358,7 @@ class GraDoomVecEnv:
             raise IndexError(f"lane must be in [0, {self.num_envs - 1}]")
         if self.render_mode != "rgb_array":
             return None
-        frame = self._rgb_frames()[lane_index].detach().to("cpu").numpy().copy()
+        frame = self._rgb_frames(lane_index)[0].detach().to("cpu").numpy().copy()
         self.check_renderer_status()
         return frame
 

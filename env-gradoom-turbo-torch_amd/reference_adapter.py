@@ -23,8 +23,6 @@ tensors will do); the scenario anything that carries ``CompiledScenario``'s (``s
 
 from __future__ import annotations
 
-import ctypes as C
-
 import numpy as np
 import torch
 
@@ -194,31 +192,6 @@ class HipReferenceRenderer:
         self.renderer.close()
 
 
-def policy_area_grayscale(indexed: torch.Tensor, palette: torch.Tensor) -> torch.Tensor:
-    """The 320x240 -> 84x84 area pooling and grayscale transform on palette indices.
-
-    Same arguments, result and errors as the reference's operator (``_triton_kernels.py:180-203``):
-    ``indexed`` uint8 ``[N, 208|240, 320]`` (208 rows: the status bar counts as black), ``palette`` uint8
-    ``[256, 3]``; returns uint8 ``[N, 84, 84]`` on the same device.
-    """
-
-    from . import _lib
-
-    if indexed.ndim != 3 or tuple(indexed.shape[1:]) not in ((208, 320), (240, 320)):
-        raise ValueError("indexed must have shape (N, 208, 320) or (N, 240, 320)")
-    if indexed.dtype != torch.uint8 or palette.dtype != torch.uint8:
-        raise TypeError("indexed and palette must be uint8 tensors")
-    if tuple(palette.shape) != (256, 3):
-        raise ValueError("palette must have shape (256, 3)")
-    if indexed.device.type != "cuda" or palette.device != indexed.device:
-        raise RuntimeError("policy_area_grayscale needs both tensors on one ROCm device; there is no CPU fallback")
-    library = _lib.library()
-    output = torch.empty((indexed.shape[0], 84, 84), device=indexed.device, dtype=torch.uint8)
-    if indexed.shape[0] == 0:
-        return output
-    source, colours = indexed.contiguous(), palette.contiguous()
-    with torch.cuda.device(indexed.device):
-        stream = torch.cuda.current_stream(indexed.device).cuda_stream
-        _lib.check(library.gd_observe(source.data_ptr(), int(indexed.shape[1]), colours.data_ptr(), int(indexed.shape[0]),
-                                      output.data_ptr(), None, None, 0, C.c_void_p(stream)))
-    return output
+# The stand-alone pooling operator (``_triton_kernels.py:180-203``): a registered Torch operator with a fake
+# implementation, see ``ops.py``.
+from .ops import policy_area_grayscale  # noqa: E402,F401

@@ -53,6 +53,12 @@ class LaneState:
     decal_state: torch.Tensor | None = None  # i32 [N,D,3] packed wall decals (overlay_inputs.decal_inputs)
     decal_geom: torch.Tensor | None = None  # f32 [N,D,4]
 
+    def select(self, index) -> "LaneState":
+        """The lanes ``index`` picks (a slice or an index tensor), every field cut alike and made contiguous."""
+
+        fields = {f.name: getattr(self, f.name) for f in dataclasses.fields(self)}
+        return LaneState(**{name: None if value is None else value[index].contiguous() for name, value in fields.items()})
+
     @classmethod
     def from_numpy(cls, arrays: dict, device) -> "LaneState":
         def get(name, dtype):
@@ -115,6 +121,9 @@ class HipRenderer:
             _lib.check(self._lib.gd_renderer_create(C.byref(desc), self._cosine.ctypes.data, self.max_lanes, C.byref(handle)))
         del keep
         self._handle = handle
+        from . import ops  # noqa: PLC0415
+
+        self.token = ops.register_renderer(self)   # names this renderer in torch.ops.gradoom_amd.render_ calls
 
     def close(self) -> None:
         if getattr(self, "_handle", None):

@@ -168,6 +168,12 @@ CASES = {
     "config4_subset": dict(
         map_seed=1004, grid=(21, 21), sectors=400, linedefs=4000, lanes=2, pose_seed=1, sprites=128, midtex=0.15
     ),
+    # the headline map with the benchmark's height distribution (floors U{0..255}, ceilings U{64..256} above: a plane
+    # level per sector, about 750 in all), the variant seed bench.py and the full-size GPU tests use
+    "config4_uniform_subset": dict(
+        map_seed=1004, grid=(21, 21), sectors=400, linedefs=4000, lanes=2, pose_seed=2, sprites=128, midtex=0.15, flash=True,
+        variant=dict(seed=5, heights="uniform"),
+    ),
 }
 
 

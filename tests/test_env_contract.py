@@ -214,3 +214,57 @@ def test_truncated_candidate_list_raises_instead_of_passing_a_bad_frame():
     with pytest.raises(RuntimeError, match="truncated"):
         env.close()
     assert env.closed and renderer.closed
+
+
+def test_step_preconditions_follow_the_reference():
+    # env.py:815-829: terminal lanes must be reset before the next host step; actions outside the table are refused
+    from gradoom_amd.env import GraDoomVecEnv
+
+    smap = load_fixture("tiny_stages")[2]
+    renderer = RecordingRenderer()
+    env = GraDoomVecEnv(smap, 4, device="cpu", renderer=renderer, episode_timeout=2, obs_copy="safe_view")
+    assert env.action_count == 17 and bool(env.pending_reset.all())
+    first = env.reset(seed=1)[0]
+    assert not bool(env.pending_reset.any()) and not bool(env.signal_buffer[:, 20].any())
+    actions = torch.zeros(4, dtype=torch.int64)
+    with pytest.raises(ValueError, match="actions fall outside the declared action space"):
+        env.step(torch.full((4,), 17, dtype=torch.int64))
+    with pytest.raises(ValueError, match="actions fall outside the declared action space"):
+        env.step(torch.tensor([0, -1, 0, 0], dtype=torch.int8))
+    with pytest.raises(TypeError, match="actions must have dtype"):
+        env.step(torch.zeros(4))
+    # a refused call takes no observation buffer: the next good step must not write into the one handed out last
+    held = first.clone()
+    second = env.step(actions)[0]
+    assert second.data_ptr() != first.data_ptr() and torch.equal(first, held)
+    truncated = env.step(actions)[3]
+    assert bool(truncated.all()) and bool(env.pending_reset.all()) and bool(env.signal_buffer[:, 20].all())
+    with pytest.raises(RuntimeError, match=r"terminal lanes must be reset before step: \[0, 1, 2, 3\]"):
+        env.step(actions)
+    mask = torch.tensor([True, False, True, False])
+    env.reset(options={"reset_mask": mask})
+    assert env.pending_reset.tolist() == [False, True, False, True]
+    with pytest.raises(RuntimeError, match=r"terminal lanes must be reset before step: \[1, 3\]"):
+        env.step(actions)
+    with pytest.raises(ValueError, match="action table must contain at least one action"):
+        GraDoomVecEnv(smap, 4, device="cpu", renderer=RecordingRenderer(), action_count=0)
+
+
+def test_render_lane_renders_only_the_lane_asked_for():
+    from gradoom_amd.env import GraDoomVecEnv
+
+    smap = load_fixture("tiny_stages")[2]
+    shapes = []
+
+    class ShapeRenderer(RecordingRenderer):
+        def render(self, lanes, **kwargs):
+            shapes.append(tuple(lanes.x.shape))
+            super().render(lanes, **kwargs)
+
+    env = GraDoomVecEnv(smap, 4, device="cpu", render_mode="rgb_array", renderer=ShapeRenderer())
+    env.reset_device(torch.ones(4, dtype=torch.bool), torch.arange(4))
+    state = env._dynamics.lane_state()
+    frame = env.render_lane(2)
+    assert shapes[-1] == (1,) and frame.shape == (240, 320, 3)
+    assert int(frame[0, 0, 0]) == int(state.x[2].abs().to(torch.int64) % 251)
+    assert len(env.get_images()) == 4 and shapes[-1] == (4,)

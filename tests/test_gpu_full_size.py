@@ -1,6 +1,7 @@
 """The headline shape (config4: 4096 lanes, 4000 linedefs, 128 sprites per lane) through properties that need no
 reference run: lanes are independent, batches are order free, the observation is a function of the frame, and a
-handful of lanes equal the CPU oracle."""
+handful of lanes equal the CPU oracle.  Every shape runs with both height distributions: the benchmark's (floors
+uniform over 0..255, ceilings 64..256 above: a plane level per sector) and the map generator's quantised one."""
 
 from __future__ import annotations
 
@@ -14,14 +15,26 @@ LANES = 4096
 PROBES = (0, 1337, 2048, 4095)
 
 
-@pytest.fixture(scope="module")
-def full_size():
+HEIGHTS = ("uniform", "quantised")
+
+
+def _config_map(config: str, heights: str):
+    from gradoom_amd import synthmap
+
+    smap = synthmap.generate_config_map(config)
+    if heights == "uniform":    # the variant seed bench.py uses
+        smap = synthmap.with_variant(smap, 5, heights="uniform")
+    return smap
+
+
+@pytest.fixture(scope="module", params=HEIGHTS)
+def full_size(request):
     from gradoom_amd import hostmath, mapbuild, synthmap
     from gradoom_amd.renderer import HipRenderer, LaneState
     from gradoom_amd.selfcheck import make_lane_arrays
 
-    print("full size: building the config4 map and 4096 poses", flush=True)
-    smap = synthmap.generate_config_map("config4")
+    print(f"full size: building the config4 map ({request.param} heights) and 4096 poses", flush=True)
+    smap = _config_map("config4", request.param)
     tables = mapbuild.build_map_tables(smap)
     cosine = hostmath.cosine_correction("cpu").numpy()
     poses = synthmap.generate_poses_batch(smap, LANES, 321, flash=True)
@@ -75,6 +88,21 @@ def test_a_second_frame_of_the_same_state_is_identical(full_size):
     assert torch.equal(obs, full_size["obs"])
 
 
+def test_both_assemblies_give_the_same_bytes(full_size):
+    # frames put together band by band in LDS equal the ones assembled kernel by kernel through device memory
+    renderer = full_size["renderer"]
+    again = torch.zeros_like(full_size["indexed"])
+    obs = torch.zeros_like(full_size["obs"])
+    renderer.set_assembly("fused")
+    try:
+        renderer.render(full_size["lanes"], indexed=again, obs=obs)
+        torch.cuda.synchronize()
+    finally:
+        renderer.set_assembly("auto")
+    assert torch.equal(again, full_size["indexed"])
+    assert torch.equal(obs, full_size["obs"])
+
+
 def test_observation_is_a_function_of_the_frame(full_size):
     # the standalone pooling entry point over the frames already rendered gives the fused observation
     renderer = full_size["renderer"]
@@ -98,16 +126,17 @@ SHAPES = {
 }
 
 
+@pytest.mark.parametrize("heights", HEIGHTS)
 @pytest.mark.parametrize("shape", list(SHAPES))
-def test_other_benchmark_shapes_at_full_lane_count(oracle, shape):
+def test_other_benchmark_shapes_at_full_lane_count(oracle, shape, heights):
     from gradoom_amd import hostmath, mapbuild, synthmap
     from gradoom_amd.renderer import HipRenderer, LaneState
     from gradoom_amd.selfcheck import make_lane_arrays
 
     spec = SHAPES[shape]
     count = spec["lanes"]
-    print(f"shape {shape}: building the map and {count} poses", flush=True)
-    smap = synthmap.generate_config_map(spec["config"])
+    print(f"shape {shape}, {heights} heights: building the map and {count} poses", flush=True)
+    smap = _config_map(spec["config"], heights)
     tables = mapbuild.build_map_tables(smap)
     cosine = hostmath.cosine_correction("cpu").numpy()
     poses = synthmap.generate_poses_batch(smap, count, 77, flash=True)
