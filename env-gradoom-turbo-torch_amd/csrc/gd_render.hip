@@ -8,7 +8,8 @@
 //                                             entry in the candidate list of every column it can own, and the
 //                                             nearest blocking hit of every column (64-bit atomicMin)
 //   strip_key/order 1 thread / 64-col strip   longest strip first (counting sort on the blocking distance)
-//   wall_columns    1 wave / strip            portal traversal, tiers, planes, masked mid-textures
+//   wall_select     1 wave / strip            portal traversal: which drawseg every column pass selects, one record each
+//   wall_raster     1 wave / strip            the recorded passes drawn: projection, clips, tiers, planes, masked mid-textures
 //   plane_shade     1 thread / 12 pixels      flat texel + light for every pixel a plane of the wall pass shows,
 //                                             the wall tiers' palette indices
 //   flat_list       128 threads / lane        per-pixel plane rays (fine point raster) for the listed gap pixels
@@ -16,7 +17,7 @@
 //                                             visplane repair of the rows where a gap pixel stayed unresolved
 //   flat_shade      128 threads / lane        the gap pixels' flats
 //   decal           320 threads / lane        bullet chips on the wall tiers they hit (frames that carry decals
-//                                             also keep a per-pixel scene depth: wall_columns<true>, plane_shade<true>)
+//                                             also keep a per-pixel scene depth: wall_raster<true>, plane_shade<true>)
 //   sprite_columns  320 threads / lane        billboards far -> near, opaque / additive / translucent
 //   weapon_overlay, hud                       player weapon, muzzle flash and status bar patches
 //   observe         1 thread / obs pixel      PLAYPAL + exact area pool + gray + 4-frame stack
@@ -97,6 +98,17 @@ struct WallRec {   // one linedef seen from one lane
     int flags;
 };
 
+// What the selection half of a column pass hands to the drawing half (wall_select_kernel -> wall_raster_kernel): the
+// drawseg the pass selected and, where a geometric portal path continues behind a projected solid
+// (engine.py:12969-13069), that path.  `bits` holds the PB_* flags of the selection (they fit 16 bits).
+struct __align__(16) PassRec {
+    unsigned short wall, render_current, bits, ps_path;
+    short ps_other;
+    unsigned short spare;
+    float distance;
+};
+#define PASS_MAX 96   // column passes recorded per screen column; a column that needs more sets STATUS_PASS_OVERFLOW
+
 struct RecSpan {   // what a ray test of one linedef needs (eval_segment), kept for every linedef of the map; the full record
                    // above exists only for the linedefs the camera can see at all
     short pl, pr;
@@ -159,7 +171,7 @@ struct Scratch {    // per-chunk working memory, sized at create
     unsigned short *flat_sector;// [L,208,320]
     unsigned char *flat_flags;  // [L,208,320] bit0 unresolved
     int *flat_list;        // [L,FLAT_LIST_MAX] view pixels no wall tier, plane or masked texture covers: they show the
-                           // flat pass's picture.  Listed by wall_columns_kernel, column by column.
+                           // flat pass's picture.  Listed by wall_raster_kernel, column by column.
     int *flat_list_count;  // [L] how many there are (more than FLAT_LIST_MAX: the lane is handled pixel by pixel)
     int *flat_tail;        // [L,2,320] per screen half and column: the sector of the first resolved pixel below the
                            // half's noted rows, -1 if the column was not looking for one or found none
@@ -171,6 +183,9 @@ struct Scratch {    // per-chunk working memory, sized at create
     int *flat_col_top;     // [L,2,320] per screen half and column: the topmost shown pixel the flat pass could not
                            // resolve (any value >= 208: none).  flat_gap_column_kernel lowers it while it selects the
                            // gap pixels, then reads it and puts "none" back, so it is filled once, when the renderer is created.
+    PassRec *pass_rec;     // [L,PASS_MAX,320] the drawsegs of each column's passes, in pass order
+    float *pass_path_distance;  // [L,PASS_MAX,320] distance of the portal path of a pass that carries PB_PS_KEEPS (written for those only)
+    unsigned char *pass_count;  // [L,320] passes recorded for the column: up to its last pass that draws or moves a clip
     unsigned int *meta;    // [L,208,320] filled | floor | plane_sector+1 | clip_wall+1
     float *clip_depth;     // [L,208,320]
     unsigned char *frame;  // [L,240,320] when the caller wants no indexed output
@@ -202,6 +217,7 @@ struct Scratch {    // per-chunk working memory, sized at create
 #define META_WALL_MASK 0xFFFFu    // sprite-clip linedef + 1
 
 #define STATUS_CAND_OVERFLOW 1
+#define STATUS_PASS_OVERFLOW 2
 #define SPAN_SELECT_BLOCKS 6144   // flat_span_select_kernel's grid: four times what 256 compute units hold at eight wavefronts per
                                   // SIMD, so that rows of unequal cost even out
 #define STEP_TABLE 96   // int64 entries per lane of Scratch::step_scale
@@ -1240,7 +1256,7 @@ __device__ int flat_probe_pixel(const DeviceMap &dm, const Scratch &sc, const Le
 // shows it; a pixel a plane of the wall pass claimed only asks whether the flat ray resolved at all, and only
 // where a sprite stands behind the plane with no sprite clip recorded, which the sprite pass finds out for
 // itself (flat_ray_resolves); the few pixels left (columns whose traversal left a gap) show the flat pass's
-// picture.  wall_columns_kernel lists those.  flat_gap_column_kernel, one block per lane, first selects them, one
+// picture.  wall_raster_kernel lists those.  flat_gap_column_kernel, one block per lane, first selects them, one
 // thread per listed pixel, and notes per screen half and column the topmost one that stayed unresolved.
 //
 // Then the vertical repair (engine.py:11026-11083) of the listed pixels, column by column.  An unresolved pixel takes
@@ -1907,6 +1923,13 @@ struct PassColumn {
     int ps_path_index, ps_other, no_path_other, sel_vertex, fb_idx;
     float ps_path_distance, no_path_distance;
     int bits;
+    // what the drawing half adds (pass_geometry, pass_clip)
+    int render_other;       // the sector behind the drawn side, -1 for none
+    float one_top, one_bottom, lower_top, upper_bottom;              // the four heights' projected rows, not yet clipped
+    float path_top, path_bottom, path_lower_top, path_upper_bottom;  // the same of the portal path of a PB_PS_KEEPS pass
+    i64 u_base, swall;      // texture column before wrapping, texture step (engine.py:12762-12807)
+    float offset_y;         // the side's vertical texture offset
+    float fake_contrast;    // +16 on vertical linedefs, -16 on horizontal ones (engine.py:12853-12861)
 };
 #define PB_VALID 0x1
 #define PB_RASTER 0x2
@@ -1930,7 +1953,101 @@ __device__ __forceinline__ void take_min(float v, int w, float &best, int &best_
     if (v < best || (v == best && w < best_w && finitef(v))) { best = v; best_w = w; }
 }
 
-// engine.py:11769-12636: selection of the pass's drawseg for one column
+// engine.py:12240-12620, 12762-12861, 12969-13010: what one column draws of the drawseg a pass selected, as far as it
+// depends on the selection alone (r.wall, r.render_current, r.ps_path_index, r.ps_other, PB_RASTER / PB_ONE_SIDED /
+// PB_PS_KEEPS / PB_PS_FROM_FRONT in r.bits) and not on the column's clips: the side and sectors drawn from, the wallscan
+// light, the four heights' projected rows, the texture column and step, and the projected rows of a portal path behind a
+// projected solid.  Every division of the drawing half is in here.
+template <bool SPLIT>
+__device__ __forceinline__ void pass_geometry(const ColumnCtx &cc, PassColumn &r) {
+    const gd_map_desc *m = cc.m;
+    const MapView &mv = cc.mv;
+    const LaneCtx &L = *cc.c;
+    const int x = cc.x, wi = r.wall, render_current = r.render_current;
+    const bool one_sided = r.bits & PB_ONE_SIDED;
+    // h. sides (engine.py:12240-12292)
+    const int front = mv.sec(wi, 0), back = mv.sec(wi, 1);
+    const bool render_from_front = render_current == front;
+    const int render_other = render_from_front ? back : front;
+    const int side = render_from_front ? 0 : 1;
+    const int safe_other = render_other < 0 ? 0 : render_other;
+    r.side = side; r.render_other = render_other;
+    const WallRec &wr = cc.rec(wi);
+    const FragmentChoice wr_fragment = choose_fragment<SPLIT>(m, cc.frags, wr, wi, x);
+    r.visibility = wall_visibility(wr_fragment.lights ? *wr_fragment.rec : wr, side, x);
+    const float view_floor = m->sector_heights[2 * render_current], view_ceiling = m->sector_heights[2 * render_current + 1];
+    const float other_floor = m->sector_heights[2 * safe_other], other_ceiling = m->sector_heights[2 * safe_other + 1];
+    for (int t = 0; t < 3; ++t) r.side_tex[t] = m->side_tex[(wi * 2 + side) * 3 + t];
+    // j. projection (engine.py:12607-12620): one copy of the projection code, four heights; the back sector's two only
+    // matter across a two-sided linedef (every use of them is behind !one_sided)
+    r.one_top = 0; r.one_bottom = 0; r.lower_top = 0; r.upper_bottom = 0;
+    const int heights = one_sided ? 2 : 4;
+#pragma unroll 1
+    for (int k = 0; k < heights; ++k) {
+        float z = k == 0 ? view_ceiling : (k == 1 ? view_floor : (k == 2 ? other_floor : other_ceiling));
+        float v = project(L, wr, wr_fragment, z, x);
+        if (k == 0) r.one_top = v; else if (k == 1) r.one_bottom = v; else if (k == 2) r.lower_top = v; else r.upper_bottom = v;
+    }
+    // texture column and step (engine.py:12762-12807), fake contrast (engine.py:12853-12861): only tiers use them
+    r.u_base = 0; r.swall = 0; r.offset_y = 0.0f; r.fake_contrast = 0.0f;
+    if (r.bits & PB_RASTER) {
+        const float *toff = m->side_off + (wi * 2 + side) * 2;
+        i64 h, swall;
+        texture_mapping(m, wr, wi, x, &h, &swall);
+        i64 repeat = round_to_i64(m->wall_len[wi] * 65536.0f);
+        if (side != 0) h = repeat - h;
+        if (wr.sl > 0 && h < 0) h = 0;
+        if (h >= repeat) h = repeat - 1;
+        i64 offx_fixed = round_to_i64(toff[0] * 65536.0f);
+        r.u_base = (h + offx_fixed) >> 16;
+        r.swall = swall;
+        r.offset_y = toff[1];
+        const float4 wl = *reinterpret_cast<const float4 *>(m->walls + 4 * wi);
+        bool horizontal = fabsf(wl.w - wl.y) < 1e-6f, vertical = fabsf(wl.z - wl.x) < 1e-6f;
+        r.fake_contrast = vertical ? 16.0f : (horizontal ? -16.0f : 0.0f);
+    }
+    // the portal path behind a projected solid (engine.py:12969-13010): the view sector's two heights and the path's other
+    // sector's two, projected through the path linedef
+    r.path_top = 0; r.path_bottom = 0; r.path_lower_top = 0; r.path_upper_bottom = 0;
+    if (r.bits & PB_PS_KEEPS) {
+        const int path = r.ps_path_index;
+        const WallRec &pr = cc.rec(path);
+        const FragmentChoice pr_fragment = choose_fragment<SPLIT>(m, cc.frags, pr, path, x);
+        const int path_safe_other = r.ps_other < 0 ? 0 : r.ps_other;
+        const float pof = m->sector_heights[2 * path_safe_other], poc = m->sector_heights[2 * path_safe_other + 1];
+#pragma unroll 1
+        for (int k = 0; k < 4; ++k) {
+            float z = k == 0 ? view_ceiling : (k == 1 ? view_floor : (k == 2 ? pof : poc));
+            float v = project(L, pr, pr_fragment, z, x);
+            if (k == 0) r.path_top = v; else if (k == 1) r.path_bottom = v; else if (k == 2) r.path_lower_top = v; else r.path_upper_bottom = v;
+        }
+    }
+}
+
+// engine.py:12607-12636: the projected rows of pass_geometry against the column's clips, the plane marks and the tiers.
+// r.side and r.render_other come from pass_geometry.
+__device__ __forceinline__ void pass_clip(const ColumnCtx &cc, float ceiling_clip, float floor_clip, PassColumn &r) {
+    const Tables &tb = *cc.tb;
+    const int render_current = r.render_current;
+    const int safe_other = r.render_other < 0 ? 0 : r.render_other;
+    const bool raster_valid = r.bits & PB_RASTER, one_sided = r.bits & PB_ONE_SIDED;
+    r.view_floor = tb.floor_h(render_current); r.view_ceiling = tb.ceil_h(render_current);
+    r.other_floor = tb.floor_h(safe_other); r.other_ceiling = tb.ceil_h(safe_other);
+    r.clipped_top = fmaxf(r.one_top, ceiling_clip);
+    r.clipped_bottom = fminf(r.one_bottom, floor_clip);
+    r.clipped_upper_bottom = fmaxf(fminf(r.upper_bottom, floor_clip), r.clipped_top);
+    r.clipped_lower_top = fminf(fmaxf(r.lower_top, ceiling_clip), r.clipped_bottom);
+    // k. plane marks (engine.py:12621-12636)
+    bool light_differs = tb.light(render_current) != tb.light(safe_other);
+    bool mark_ceiling = one_sided || (r.view_ceiling != r.other_ceiling) || (tb.ceil_tex(render_current) != tb.ceil_tex(safe_other)) || light_differs;
+    bool mark_floor = one_sided || (r.view_floor != r.other_floor) || (tb.floor_tex(render_current) != tb.floor_tex(safe_other)) || light_differs;
+    bool tier0 = one_sided && raster_valid && (r.side_tex[0] >= 0) && (r.clipped_top < r.clipped_bottom);
+    bool tier1 = !one_sided && raster_valid && (r.view_floor < r.other_floor) && (r.side_tex[1] >= 0) && (r.clipped_lower_top < r.clipped_bottom);
+    bool tier2 = !one_sided && raster_valid && (r.view_ceiling > r.other_ceiling) && (r.side_tex[2] >= 0) && (r.clipped_top < r.clipped_upper_bottom);
+    r.bits |= (tier0 ? PB_TIER0 : 0) | (tier1 ? PB_TIER1 : 0) | (tier2 ? PB_TIER2 : 0) | (mark_ceiling ? PB_MARK_CEILING : 0) | (mark_floor ? PB_MARK_FLOOR : 0);
+}
+
+// engine.py:11769-12239: selection of the pass's drawseg for one column
 template <bool SPLIT>
 __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnState &c, bool boundary_has_po, PassColumn &r) {
     const gd_map_desc *m = cc.m;
@@ -2098,44 +2215,13 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
     bool ps_from_front = cs == mv.sec(ps_path_index, 0);
     int ps_other = ps_from_front ? mv.sec(ps_path_index, 1) : mv.sec(ps_path_index, 0);
     bool ps_keeps = has_ps && ps_path_geo && (ps_other >= 0);
-    int safe_other = render_other < 0 ? 0 : render_other;
     bool one_sided = other_sector < 0;
 
     r.wall = wi; r.side = side; r.render_current = render_current; r.other_sector = other_sector;
     r.distance = distance;
-    const WallRec &wr = cc.rec(wi);
-    const FragmentChoice wr_fragment = choose_fragment<SPLIT>(m, cc.frags, wr, wi, x);
-    r.visibility = wall_visibility(wr_fragment.lights ? *wr_fragment.rec : wr, side, x);
-    const Tables &tb = *cc.tb;
-    r.view_floor = tb.floor_h(render_current); r.view_ceiling = tb.ceil_h(render_current);
-    r.other_floor = tb.floor_h(safe_other); r.other_ceiling = tb.ceil_h(safe_other);
-    for (int t = 0; t < 3; ++t) r.side_tex[t] = m->side_tex[(wi * 2 + side) * 3 + t];
-    // j. projection and clipping (engine.py:12607-12620)
-    float one_top = 0, one_bottom = 0, lower_top = 0, upper_bottom = 0;
-    // one copy of the projection code, four heights; the back sector's two only matter across a
-    // two-sided linedef (every use of them is behind !one_sided)
-    const int heights = one_sided ? 2 : 4;
-#pragma unroll 1
-    for (int k = 0; k < heights; ++k) {
-        float z = k == 0 ? r.view_ceiling : (k == 1 ? r.view_floor : (k == 2 ? r.other_floor : r.other_ceiling));
-        float v = project(*cc.c, wr, wr_fragment, z, x);
-        if (k == 0) one_top = v; else if (k == 1) one_bottom = v; else if (k == 2) lower_top = v; else upper_bottom = v;
-    }
-    r.clipped_top = fmaxf(one_top, c.ceiling_clip);
-    r.clipped_bottom = fminf(one_bottom, c.floor_clip);
-    r.clipped_upper_bottom = fmaxf(fminf(upper_bottom, c.floor_clip), r.clipped_top);
-    r.clipped_lower_top = fminf(fmaxf(lower_top, c.ceiling_clip), r.clipped_bottom);
-    // k. plane marks (engine.py:12621-12636)
-    bool light_differs = tb.light(render_current) != tb.light(safe_other);
-    bool mark_ceiling = one_sided || (r.view_ceiling != r.other_ceiling) || (tb.ceil_tex(render_current) != tb.ceil_tex(safe_other)) || light_differs;
-    bool mark_floor = one_sided || (r.view_floor != r.other_floor) || (tb.floor_tex(render_current) != tb.floor_tex(safe_other)) || light_differs;
-    bool tier0 = one_sided && raster_valid && (r.side_tex[0] >= 0) && (r.clipped_top < r.clipped_bottom);
-    bool tier1 = !one_sided && raster_valid && (r.view_floor < r.other_floor) && (r.side_tex[1] >= 0) && (r.clipped_lower_top < r.clipped_bottom);
-    bool tier2 = !one_sided && raster_valid && (r.view_ceiling > r.other_ceiling) && (r.side_tex[2] >= 0) && (r.clipped_top < r.clipped_upper_bottom);
     r.ps_path_index = ps_path_index; r.ps_other = ps_other; r.no_path_other = no_path_other; r.sel_vertex = sel_vertex; r.fb_idx = fb_idx;
     r.ps_path_distance = ps_path_distance; r.no_path_distance = no_path_distance;
-    r.bits = (valid ? PB_VALID : 0) | (raster_valid ? PB_RASTER : 0) | (one_sided ? PB_ONE_SIDED : 0) | (tier0 ? PB_TIER0 : 0) |
-             (tier1 ? PB_TIER1 : 0) | (tier2 ? PB_TIER2 : 0) | (mark_ceiling ? PB_MARK_CEILING : 0) | (mark_floor ? PB_MARK_FLOOR : 0) |
+    r.bits = (valid ? PB_VALID : 0) | (raster_valid ? PB_RASTER : 0) | (one_sided ? PB_ONE_SIDED : 0) |
              (ps_keeps ? PB_PS_KEEPS : 0) | (no_keeps ? PB_NO_KEEPS : 0) | (geometric_intersection ? PB_GEOMETRIC : 0) |
              (replace_np ? PB_REPLACE_NP : 0) | (ps_from_front ? PB_PS_FROM_FRONT : 0) | (continues_po_boundary ? PB_CONTINUES_PO : 0) |
              (pend_ep_has_forward_bridge ? PB_FORWARD_BRIDGE : 0) | ((cwi.flags & CF_ALONG_HI) ? PB_FINAL_ALONG_HI : 0);
@@ -2279,20 +2365,9 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
     const bool one_sided = r.bits & PB_ONE_SIDED;
     const float ceiling_plane_bottom = fminf(r.clipped_top, c.floor_clip);
     const float floor_plane_top = fmaxf(r.clipped_bottom, c.ceiling_clip);
-    const float *toff = m->side_off + (wi * 2 + side) * 2;
-    i64 h, swall;
-    texture_mapping(m, cc.rec(wi), wi, x, &h, &swall);
-    i64 repeat = round_to_i64(m->wall_len[wi] * 65536.0f);
-    if (side != 0) h = repeat - h;
-    if (cc.rec(wi).sl > 0 && h < 0) h = 0;
-    if (h >= repeat) h = repeat - 1;
-    i64 offx_fixed = round_to_i64(toff[0] * 65536.0f);
-    i64 u_base = (h + offx_fixed) >> 16;
-    const float4 wl = *reinterpret_cast<const float4 *>(m->walls + 4 * wi);
-    bool horizontal = fabsf(wl.w - wl.y) < 1e-6f, vertical = fabsf(wl.z - wl.x) < 1e-6f;
-    float fake_contrast = vertical ? 16.0f : (horizontal ? -16.0f : 0.0f);
+    const i64 u_base = r.u_base, swall = r.swall;
     const Tables &tb = *cc.tb;
-    float light = (tb.light(r.render_current) + (float)(L.flash_light * 16)) + fake_contrast;
+    float light = (tb.light(r.render_current) + (float)(L.flash_light * 16)) + r.fake_contrast;
     const i64 shade_own = wall_shade(light, r.visibility);
     const i64 shade_group = wall_shade(light, first_group_visibility);
     // every span of this pass lies inside the open window [ceiling_clip, floor_clip)
@@ -2354,7 +2429,7 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
         //   fraction(y) = (texture_mid << (16 - height_bits)) + ((step * (y * 65536 + 65536 - center)) >> 16).
         // step * y * 65536 has no low 16 bits, so it shifts out of the floor unchanged, and only the low 32 bits of
         // the sum are looked at: they advance by the low 32 bits of step per row, whatever the 64-bit terms wrap to.
-        const float toff_y = toff[1] * 65536.0f;
+        const float toff_y = r.offset_y * 65536.0f;
         const unsigned atlas_w = (unsigned)m->tex_max_w;
         const int side_tex0 = r.side_tex[0], side_tex1 = r.side_tex[1], side_tex2 = r.side_tex[2];
         const bool tiers_overlap = lower_on && upper_on && r.clipped_lower_top < r.clipped_upper_bottom;
@@ -2520,7 +2595,7 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
                 int height_bits = tb.height_bits(texture_id);
                 i64 vertical_step = mul64(swall, shl64(1, 14 - height_bits));
                 i64 screen_delta = (i64)y * FIXED_UNIT - L.center_fixed + FIXED_UNIT;
-                i64 texture_mid = round_to_i64((origin_z - L.view_z) * 65536.0f + toff[1] * 65536.0f);
+                i64 texture_mid = round_to_i64((origin_z - L.view_z) * 65536.0f + r.offset_y * 65536.0f);
                 i64 fraction = shl64(texture_mid, 16 - height_bits) + (mul64(vertical_step, screen_delta) >> 16);
                 i64 tv = (fraction & UINT32_MASK) >> (32 - height_bits);
                 unsigned char texel = m->tex_atlas[((size_t)texture_id * m->tex_max_h + tv) * m->tex_max_w + tu];
@@ -2536,8 +2611,13 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
     }
 }
 
-// engine.py:12885-13371
-template <bool SPLIT>
+// engine.py:12885-13371.  PART: ADVANCE_ALL, or only the column's clips, masked-drawseg snapshot and sprite silhouettes
+// (ADVANCE_CLIPS: what needs the projected rows and touches pixels), or only the traversal state (ADVANCE_STATE: next
+// sector, previous distance, pending boundaries; it reads neither rows nor clips).
+#define ADVANCE_ALL 0
+#define ADVANCE_STATE 1
+#define ADVANCE_CLIPS 2
+template <bool SPLIT, int PART>
 __device__ __forceinline__ bool pass_advance(const ColumnCtx &cc, ColumnState &c, const PassColumn &r, PixelBuffers &pb, SilhouetteBounds &sb, bool window_untouched, GapRange &gaps) {
     const gd_map_desc *m = cc.m;
     const MapView &mv = cc.mv;
@@ -2550,6 +2630,7 @@ __device__ __forceinline__ bool pass_advance(const ColumnCtx &cc, ColumnState &c
     const float distance = r.distance;
     const bool valid = r.bits & PB_VALID, raster_valid = r.bits & PB_RASTER, one_sided = r.bits & PB_ONE_SIDED;
     auto incident = [&](int w) { return mv.sec(w, 0) == cur || mv.sec(w, 1) == cur; };
+  if (PART != ADVANCE_STATE) {
     // o. clip updates (engine.py:12888-12913)
     bool draws_upper = (r.view_ceiling > r.other_ceiling) && (r.side_tex[2] >= 0);
     if (raster_valid && !one_sided && (draws_upper || (r.bits & PB_MARK_CEILING))) c.ceiling_clip = draws_upper ? r.clipped_upper_bottom : r.clipped_top;
@@ -2579,20 +2660,12 @@ __device__ __forceinline__ bool pass_advance(const ColumnCtx &cc, ColumnState &c
     // r. clips of the geometric portal behind a projected solid (engine.py:12969-13069)
     if (r.bits & PB_PS_KEEPS) {
         int path = r.ps_path_index;
-        const WallRec &pr = cc.rec(path);
-        const FragmentChoice pr_fragment = choose_fragment<SPLIT>(m, cc.frags, pr, path, x);
         int path_safe_other = r.ps_other < 0 ? 0 : r.ps_other;
         const Tables &tb = *cc.tb;
         float pof = tb.floor_h(path_safe_other), poc = tb.ceil_h(path_safe_other);
         int pside = (r.bits & PB_PS_FROM_FRONT) ? 0 : 1;
         const int *ptex = m->side_tex + (path * 2 + pside) * 3;
-        float path_top = 0, path_bottom = 0, path_lower_top = 0, path_upper_bottom = 0;
-#pragma unroll 1
-        for (int k = 0; k < 4; ++k) {
-            float z = k == 0 ? r.view_ceiling : (k == 1 ? r.view_floor : (k == 2 ? pof : poc));
-            float v = project(L, pr, pr_fragment, z, x);
-            if (k == 0) path_top = v; else if (k == 1) path_bottom = v; else if (k == 2) path_lower_top = v; else path_upper_bottom = v;
-        }
+        const float path_top = r.path_top, path_bottom = r.path_bottom, path_lower_top = r.path_lower_top, path_upper_bottom = r.path_upper_bottom;
         float pct = fmaxf(path_top, c.ceiling_clip);
         float pcb = fminf(path_bottom, c.floor_clip);
         float pcub = fmaxf(fminf(path_upper_bottom, c.floor_clip), pct);
@@ -2619,6 +2692,8 @@ __device__ __forceinline__ bool pass_advance(const ColumnCtx &cc, ColumnState &c
         bool ptop = (r.view_ceiling < poc) || (L.view_z > poc) || pmasked;
         apply_silhouette(pb, sb, x, pbottom, ptop, c.floor_clip, c.ceiling_clip, r.ps_path_distance, path, 0, 0);
     }
+  }
+    if (PART == ADVANCE_CLIPS) return false;
     // s. next sector (engine.py:13070-13241)
     const float prior = before.previous_distance;
     const float prior_eps = prior + 1e-3f;
@@ -2881,16 +2956,92 @@ __global__ void __launch_bounds__(1024) strip_order_kernel(int strips, Scratch s
     for (int s = threadIdx.x; s < strips; s += blockDim.x) sc.strip_order[atomicAdd(&position[sc.strip_key[s]], 1)] = s;
 }
 
-// One wavefront per 64 / SEG_COLS segments.  Segments share nothing but read-only tables; a work-group is
-// WALL_STRIPS_PER_GROUP wavefronts (neighbours in the longest-first order) only so that the LDS copies of those
-// tables, 16.7 KB, are held once per group rather than once per wavefront: a CU has 160 KB of LDS and room for
-// twelve of these wavefronts (168 registers), so one wavefront per group would stop at nine.  After the staging
-// barrier the wavefronts never meet again.
+// The traversal in two kernels.  Which drawseg a column pass selects, and where the column goes next, depends on the map,
+// the camera and the column's ray alone, never on projected rows or clips: wall_select_kernel runs that half
+// (pass_select without the projection, pass_advance's state part) and records one PassRec per pass; wall_raster_kernel
+// runs the other half over the records (pass_geometry, pass_clip, pass_paint, pass_advance's clip part, the masked mid-texture).
+// Each half is lighter in registers and in code than the two together, so more of its wavefronts share a SIMD and
+// its pass loop fits the instruction cache.  Same segment order and one wavefront per segment in both.
+#define SELECT_STRIPS_PER_GROUP 1
+template <bool SPLIT>
+__global__ void __launch_bounds__(64 * SELECT_STRIPS_PER_GROUP) wall_select_kernel(DeviceMap dm, int lane_count, Scratch sc) {
+    const gd_map_desc *m = &dm.d;
+    __shared__ LaneCtx lane_ctxs[SELECT_STRIPS_PER_GROUP][64 / SEG_COLS];
+    const int wave_in_group = threadIdx.x >> 6;
+    const int lane_id = threadIdx.x & 63;
+    const int segment_in_wave = lane_id / SEG_COLS;
+    const int segment_slot = (blockIdx.x * SELECT_STRIPS_PER_GROUP + wave_in_group) * (64 / SEG_COLS) + segment_in_wave;
+    const bool live = segment_slot < lane_count * SEGS_PER_LANE;
+    const int segment = live ? sc.strip_order[segment_slot] : 0;
+    const int local = segment / SEGS_PER_LANE;
+    if ((lane_id & (SEG_COLS - 1)) == 0 && live) lane_ctxs[wave_in_group][segment_in_wave] = sc.ctx[local];
+    __syncthreads();
+    if (!live) return;
+    const LaneCtx &lane_ctx = lane_ctxs[wave_in_group][segment_in_wave];
+    const int x = (segment - local * SEGS_PER_LANE) * SEG_COLS + (lane_id & (SEG_COLS - 1));
+    ColumnCtx cc;
+    cc.tb = nullptr; cc.m = m; cc.mv.m = m; cc.c = &lane_ctx;
+    cc.recs = sc.rec; cc.spans = sc.span;
+    cc.rec_base = (unsigned)local * (unsigned)m->wall_count;
+    cc.frags = sc.frag_rec + (size_t)local * m->split_count * m->fragment_slots;
+    cc.list = sc.cand;
+    cc.list_column = ((unsigned)local * (CAND_MAX * SW) + (unsigned)x) * 16u;
+    cc.count = sc.cand_count[(size_t)local * SW + x];
+    if (cc.count > CAND_MAX) cc.count = CAND_MAX;
+    cc.x = x;
+    ray_direction(lane_ctx, x, &cc.rx, &cc.ry);
+    ColumnState st;
+    st.current_sector = lane_ctx.sector;
+    st.ceiling_clip = 0.0f; st.floor_clip = (float)VH;
+    st.masked_ceiling_clip = 0.0f; st.masked_floor_clip = (float)VH; st.masked_distance = GD_INF; st.masked_wall = -1;
+    st.previous_distance = 0.0f;
+    st.pend_po_vertex = -1; st.pend_ep_vertex = -1; st.pend_ep_wall = 0; st.pend_eb_index = 0;
+    st.pend_pb_index = 0; st.pend_pb_sector = -1; st.pend_pb_exit = 0.0f; st.flags = 0;
+    bool boundary_has_po = false;
+    for (int k = 0; k < cc.count; ++k) if (cc.cand(k).flags & CF_LEDGE) { boundary_has_po = true; break; }
+    PassRec *records = sc.pass_rec + ((size_t)local * PASS_MAX * SW + x);
+    float *path_distances = sc.pass_path_distance + ((size_t)local * PASS_MAX * SW + x);
+    PixelBuffers no_pixels; SilhouetteBounds no_bounds; GapRange no_gaps;   // the state part of pass_advance touches none of them
+    PassColumn pc;
+    bool done = false;
+    int recorded = 0;
+    const int sectors = m->sector_count;
+    for (int pass = 0; pass < sectors; ++pass) {
+        if (!done) {
+            pass_select<SPLIT>(cc, st, boundary_has_po, pc);
+            if (pc.bits & (PB_RASTER | PB_PS_KEEPS)) {
+                if (pass < PASS_MAX) {
+                    PassRec rec;
+                    rec.wall = (unsigned short)pc.wall; rec.render_current = (unsigned short)pc.render_current;
+                    rec.bits = (unsigned short)pc.bits; rec.ps_path = (unsigned short)pc.ps_path_index;
+                    rec.ps_other = (short)pc.ps_other; rec.spare = 0; rec.distance = pc.distance;
+                    // passes between two recorded ones keep whatever the slot held: the drawing half skips them by their bits
+                    for (int skipped = recorded; skipped < pass; ++skipped) records[(size_t)skipped * SW].bits = 0;
+                    records[(size_t)pass * SW] = rec;
+                    if (pc.bits & PB_PS_KEEPS) path_distances[(size_t)pass * SW] = pc.ps_path_distance;
+                    recorded = pass + 1;
+                } else {
+                    atomicOr(sc.status, STATUS_PASS_OVERFLOW);
+                }
+            }
+            const bool changed = pass_advance<SPLIT, ADVANCE_STATE>(cc, st, pc, no_pixels, no_bounds, false, no_gaps);
+            // A pass that found nothing and changed nothing repeats identically for ever.
+            if (!(pc.bits & PB_VALID) && !changed) done = true;
+        }
+        if (__ballot(!done) == 0) break;
+    }
+    sc.pass_count[(size_t)local * SW + x] = (unsigned char)recorded;
+}
+
+// One wavefront per 64 / SEG_COLS segments.  Segments share nothing but read-only tables; a work-group of the drawing
+// half is WALL_STRIPS_PER_GROUP wavefronts (neighbours in the longest-first order) only so that the LDS copies of
+// those tables, 16.7 KB, are held once per group rather than once per wavefront (a CU has 160 KB of LDS and room for
+// sixteen of these wavefronts at 128 registers).  After the staging barrier the wavefronts never meet again.
 #define WALL_STRIPS_PER_GROUP 2
 // DEPTH: also keep the depth of every wall pixel (frames that draw decals).  SPLIT: the map has linedefs with
 // BSP projection fragments.
 template <bool DEPTH, bool SPLIT>
-__global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amdgpu_waves_per_eu(3, 3))) wall_columns_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
+__global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amdgpu_waves_per_eu(4, 4))) wall_raster_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
     const gd_map_desc *m = &dm.d;
     __shared__ LaneCtx lane_ctxs[WALL_STRIPS_PER_GROUP][64 / SEG_COLS];
     __shared__ unsigned char colormap_lds[32 * 256];   // shade rows 0..31 are the only ones indexed
@@ -2931,22 +3082,38 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
     pb.word_column = ((unsigned)local * (VH * SW) + (unsigned)x) * 4u;
     pb.frame_column = (unsigned)local * (unsigned)frame_stride + (unsigned)x;
     // the meta plane arrives with whatever the last frame left: see GapRange for how every row gets written
-    ColumnState st;
-    st.current_sector = lane_ctx.sector;
+    ColumnState st;   // only the clips and the masked-drawseg snapshot live here; the traversal state stayed in wall_select_kernel
+    st.current_sector = -1;
     st.ceiling_clip = 0.0f; st.floor_clip = (float)VH;
     st.masked_ceiling_clip = 0.0f; st.masked_floor_clip = (float)VH; st.masked_distance = GD_INF; st.masked_wall = -1;
     st.previous_distance = 0.0f;
     st.pend_po_vertex = -1; st.pend_ep_vertex = -1; st.pend_ep_wall = 0; st.pend_eb_index = 0;
     st.pend_pb_index = 0; st.pend_pb_sector = -1; st.pend_pb_exit = 0.0f; st.flags = 0;
     SilhouetteBounds sb; sb.bot_row = VH; sb.top_row = 0; sb.bot_depth = -GD_INF; sb.top_depth = -GD_INF;
-    bool boundary_has_po = false;
-    for (int k = 0; k < cc.count; ++k) if (cc.cand(k).flags & CF_LEDGE) { boundary_has_po = true; break; }
+    const int passes = sc.pass_count[(size_t)local * SW + x];
+    const PassRec *records = sc.pass_rec + ((size_t)local * PASS_MAX * SW + x);
+    const float *path_distances = sc.pass_path_distance + ((size_t)local * PASS_MAX * SW + x);
     PassColumn pc;
-    bool done = false;
+    pc.wall = 0; pc.side = 0; pc.bits = 0; pc.visibility = 0;
+    pc.clipped_top = 0.0f; pc.clipped_bottom = 0.0f; pc.clipped_upper_bottom = 0.0f; pc.clipped_lower_top = 0.0f;
     const int group_base = lane_id & ~3;
-    const int sectors = m->sector_count;
-    for (int pass = 0; pass < sectors; ++pass) {
-        if (!done) pass_select<SPLIT>(cc, st, boundary_has_po, pc);
+    for (int pass = 0; __ballot(pass < passes) != 0; ++pass) {
+        const bool mine = pass < passes;
+        bool draws = false;
+        if (mine) {
+            const PassRec rec = records[(size_t)pass * SW];
+            draws = (rec.bits & (PB_RASTER | PB_PS_KEEPS)) != 0;
+            pc.bits = draws ? (int)rec.bits : 0;
+            if (draws) {
+                pc.wall = rec.wall; pc.render_current = rec.render_current; pc.distance = rec.distance;
+                pc.ps_path_index = rec.ps_path; pc.ps_other = rec.ps_other;
+                pc.ps_path_distance = (rec.bits & PB_PS_KEEPS) ? path_distances[(size_t)pass * SW] : 0.0f;
+                pass_geometry<SPLIT>(cc, pc);
+                pass_clip(cc, st.ceiling_clip, st.floor_clip, pc);
+            }
+        } else {
+            pc.bits = 0;   // a finished column draws no tier: its group of four has no common tail
+        }
         // 4-column wallscan groups (engine.py:12688-12761): exchange with the aligned neighbours
         bool same_group = true;
         int w0 = __shfl(pc.wall, group_base), s0 = __shfl(pc.side, group_base);
@@ -2967,13 +3134,10 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
         i64 first_group_visibility = ((i64)vis_hi << 32) | (i64)(unsigned)vis_lo;
         bool group_valid[3];
         for (int t = 0; t < 3; ++t) group_valid[t] = same_group && all_tier[t] && (common_top[t] < common_bottom[t]);
-        if (!done) {
+        if (draws) {
             pass_paint<DEPTH>(cc, st, pc, pb, group_valid, common_bottom, first_group_visibility, colormap_lds, window_dirty, gaps);
-            bool changed = pass_advance<SPLIT>(cc, st, pc, pb, sb, !window_dirty, gaps);
-            // A pass that found nothing and changed nothing repeats identically for ever.
-            if (!(pc.bits & PB_VALID) && !changed) done = true;
+            pass_advance<SPLIT, ADVANCE_CLIPS>(cc, st, pc, pb, sb, !window_dirty, gaps);
         }
-        if (__ballot(!done) == 0) break;
     }
     // what is left of a window no one-sided drawseg closed shows the flat pass's picture
     if (!window_dirty) zero_rows(pb, gaps, x, st.ceiling_clip <= 0.0f ? 0 : (int)st.ceiling_clip, st.floor_clip >= (float)VH ? VH : (int)st.floor_clip);
@@ -4278,6 +4442,9 @@ size_t carve_scratch(Scratch &sc, unsigned char *base, size_t L, const gd_map_de
     take(&sc.flat_col_top, L * 2 * SW);
     take(&sc.flat_list, L * FLAT_LIST_MAX);
     take(&sc.flat_list_count, L);
+    take(&sc.pass_rec, L * PASS_MAX * SW);
+    take(&sc.pass_path_distance, L * PASS_MAX * SW);
+    take(&sc.pass_count, L * SW);
     take(&sc.meta, L * PX);
     take(&sc.clip_depth, L * PX);
     take(&sc.level_reach, L * levels);
@@ -4432,7 +4599,7 @@ int validate_map(const gd_map_desc *h) {
     return GD_OK;
 }
 
-const int STAGE_COUNT = 8;
+const int STAGE_COUNT = 9;
 
 int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_desc *lanes, const gd_frame_out *out, int base, int count, hipStream_t stream, bool timed) {
     const gd_map_desc &m = r->dm.d;
@@ -4470,10 +4637,13 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     mark();
     {
         const int wavefronts = (count * SEGS_PER_LANE + 64 / SEG_COLS - 1) / (64 / SEG_COLS);
-        const dim3 grid((wavefronts + WALL_STRIPS_PER_GROUP - 1) / WALL_STRIPS_PER_GROUP), block(64 * WALL_STRIPS_PER_GROUP);
         const bool split = m.split_count > 0;
-        auto kernel = decals ? (split ? wall_columns_kernel<true, true> : wall_columns_kernel<true, false>)
-                             : (split ? wall_columns_kernel<false, true> : wall_columns_kernel<false, false>);
+        const dim3 select_grid((wavefronts + SELECT_STRIPS_PER_GROUP - 1) / SELECT_STRIPS_PER_GROUP), select_block(64 * SELECT_STRIPS_PER_GROUP);
+        hipLaunchKernelGGL(split ? wall_select_kernel<true> : wall_select_kernel<false>, select_grid, select_block, 0, stream, r->dm, count, sc);
+        mark();
+        const dim3 grid((wavefronts + WALL_STRIPS_PER_GROUP - 1) / WALL_STRIPS_PER_GROUP), block(64 * WALL_STRIPS_PER_GROUP);
+        auto kernel = decals ? (split ? wall_raster_kernel<true, true> : wall_raster_kernel<true, false>)
+                             : (split ? wall_raster_kernel<false, true> : wall_raster_kernel<false, false>);
         hipLaunchKernelGGL(kernel, grid, block, 0, stream, r->dm, count, sc, frame_base, frame_stride);
     }
     mark();
@@ -4824,7 +4994,7 @@ int gd_render_timed(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_o
     int rc = check_render_args(r, lanes, out);
     if (rc != GD_OK) return rc;
     if (r->chunk_lanes <= 0) return fail(GD_E_ARG, "this renderer was created for 0 lanes and holds no working memory");
-    if (!ms || stage_count < STAGE_COUNT - 1 || launches <= 0) return fail(GD_E_ARG, "ms must hold 7 stage times");
+    if (!ms || stage_count < STAGE_COUNT - 1 || launches <= 0) return fail(GD_E_ARG, "ms must hold 8 stage times");
     for (int s = 0; s < stage_count; ++s) ms[s] = 0.0f;
     hipStream_t st = static_cast<hipStream_t>(stream);
     for (int it = 0; it < launches; ++it) {

@@ -275,10 +275,16 @@ class GraDoomVecEnv:
         Synchronises the device: called where the environment already waits for it.
         """
         status = getattr(self._renderer, "status", None)
-        if status is not None and status() & 1:
+        flags = status() if status is not None else 0
+        if flags & 1:
             raise RuntimeError(
                 "the renderer truncated a screen column's candidate list (more than 64 linedefs overlap one column of one "
                 "lane's view): frames of this environment are not trustworthy on this map"
+            )
+        if flags & 2:
+            raise RuntimeError(
+                "the renderer truncated a screen column's list of drawsegs (a column crossed more than 96 portals): frames of "
+                "this environment are not trustworthy on this map"
             )
 
     # ------------------------------------------------------------------ host-facing API (env.py:750-834)

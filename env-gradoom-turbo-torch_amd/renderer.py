@@ -18,7 +18,7 @@ import torch
 
 from . import _abi, _lib, hostmath, mapbuild
 
-STAGES = ("wall_setup", "wall_columns", "plane_shade", "flat_select", "flat_repair", "sprite_columns", "observe")
+STAGES = ("wall_setup", "wall_select", "wall_raster", "plane_shade", "flat_select", "flat_repair", "sprite_columns", "observe")
 
 
 @dataclasses.dataclass
