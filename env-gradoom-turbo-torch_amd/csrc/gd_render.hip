@@ -179,7 +179,10 @@ struct Scratch {    // per-chunk working memory, sized at create
                            // pixel the flat pass could not resolve and whose repair reads its row (208, -1 = none):
                            // the rows the row repairs work on
     int *flat_rows;        // [L*208] the noted rows of every lane as one work list, entry = lane << 8 | row
-    int *flat_row_count;   // [1] its length (cleared by lane_setup_kernel, filled by flat_gap_column_kernel)
+    int *flat_row_count;   // [1] its length (cleared by lane_setup_kernel, filled by flat_rows_kernel)
+    int *gap_columns;      // [L*2*320] the screen columns (of any lane, either half) that hold a shown pixel the flat pass
+                           // could not resolve, as one work list: lane << 18 | half << 17 | topmost such row << 9 | column
+    int *gap_column_count; // [1] its length (cleared by lane_setup_kernel, filled by flat_gap_column_kernel)
     int *flat_col_top;     // [L,2,320] per screen half and column: the topmost shown pixel the flat pass could not
                            // resolve (any value >= 208: none).  flat_gap_column_kernel lowers it while it selects the
                            // gap pixels, then reads it and puts "none" back, so it is filled once, when the renderer is created.
@@ -567,7 +570,7 @@ __global__ void lane_setup_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_ba
     int *span = sc.flat_span + (size_t)local * 4;
     span[0] = VH; span[1] = -1; span[2] = VH; span[3] = -1;
     sc.flat_list_count[local] = 0;
-    if (local == 0) *sc.flat_row_count = 0;
+    if (local == 0) { *sc.flat_row_count = 0; *sc.gap_column_count = 0; }
 }
 
 __device__ __forceinline__ void ray_direction(const LaneCtx &c, int x, float *rx, float *ry) {
@@ -1307,10 +1310,10 @@ __global__ void __launch_bounds__(GAP_THREADS) __attribute__((amdgpu_waves_per_e
     }
     __threadfence_block();   // what the selection wrote (column tops, row ranges) is read below by other threads of the block
     __syncthreads();
-    // the block's columns with work, both halves together, dealt out to its wavefronts in turn (the columns of a
-    // gap are neighbours: taken strip by strip, one wavefront would do them all)
+    // the lane's columns with work, both halves together, join one work list that flat_gap_repair_kernel deals out to
+    // wavefronts evenly, whichever lanes they come from
     __shared__ int column_list[2 * SW];
-    __shared__ int column_count;
+    __shared__ int column_count, list_base;
     if (threadIdx.x == 0) column_count = 0;
     __syncthreads();
     for (int half = 0; half < 2; ++half) for (int x = threadIdx.x; x < SW; x += blockDim.x) {
@@ -1318,15 +1321,41 @@ __global__ void __launch_bounds__(GAP_THREADS) __attribute__((amdgpu_waves_per_e
         const int top = __hip_atomic_load(top_at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // where the atomics above wrote, not a cached copy
         if (top < VH) {
             *top_at = VH;
-            column_list[atomicAdd(&column_count, 1)] = x | (top << 9) | (half << 17);
+            column_list[atomicAdd(&column_count, 1)] = x | (top << 9) | (half << 17) | (local << 18);
         }
     }
     __syncthreads();
     const int columns = column_count;
-    for (int entry = threadIdx.x >> 6; entry < columns; entry += blockDim.x / 64) {
-        const int packed = column_list[entry];
-        const int x = packed & 511, first = (packed >> 9) & 255, half = packed >> 17;
-        const int half_end = half ? VH - 1 : last_ceiling_row;
+    if (columns == 0) return;                        // the same in every thread
+    if (threadIdx.x == 0) list_base = atomicAdd(sc.gap_column_count, columns);
+    __syncthreads();
+    for (int k = threadIdx.x; k < columns; k += blockDim.x) sc.gap_columns[list_base + k] = column_list[k];
+}
+
+// The vertical repair (engine.py:11026-11083) of the listed gap pixels, column by column: one wavefront per listed column
+// (flat_gap_column_kernel's work list), its lanes probing 64 rows of the column at a time, from the bottom of the half up
+// to the column's topmost unresolved listed pixel.
+#define GAP_REPAIR_BLOCKS 8192
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(8, 8))) flat_gap_repair_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, Scratch sc) {
+    __shared__ LevelLds level_lds;
+    const int total = *sc.gap_column_count;
+    const int lane_id = threadIdx.x;
+    int staged = -1;
+    LevelLists lists;
+    for (int entry = blockIdx.x; entry < total; entry += gridDim.x) {
+        const int packed = sc.gap_columns[entry];
+        const int x = packed & 511, first = (packed >> 9) & 255, half = (packed >> 17) & 1, local = packed >> 18;
+        if (local != staged) {   // the same in every thread
+            __syncthreads();     // nobody reads the previous lane's lists any more
+            lists = stage_level_lists(dm, sc, local, &level_lds);
+            __syncthreads();
+            staged = local;
+        }
+        const LaneCtx &c = sc.ctx[local];
+        const int n = lane_base + local;
+        int *span = sc.flat_span + (size_t)local * 4;
+        const unsigned int *meta = sc.meta + (size_t)local * VH * SW;
+        const int half_end = half ? VH - 1 : c.last_ceiling_row;
         const float rc = lanes.ray_cos[(size_t)n * SW + x], rs = lanes.ray_sin[(size_t)n * SW + x], cc = dm.cosine_correction[x];
         // chunks of 64 rows, the lowest first: what a chunk finds serves the chunks above it
         bool below_found = false; int below_sector = 0;
@@ -1362,15 +1391,20 @@ __global__ void __launch_bounds__(GAP_THREADS) __attribute__((amdgpu_waves_per_e
             }
         }
     }
-    // The lane's row ranges are final now (only this block touches them): its rows join the work list that
-    // flat_span_select_kernel deals out evenly, whichever lanes they come from.
-    __syncthreads();
-    __shared__ int list_base;
-    const int lo0 = atomicAdd(&span[0], 0), hi0 = atomicAdd(&span[1], 0), lo1 = atomicAdd(&span[2], 0), hi1 = atomicAdd(&span[3], 0);   // read where the atomics above wrote
+}
+
+// The lanes' row ranges are final once every listed column is repaired: their rows join the work list that
+// flat_span_select_kernel deals out evenly, whichever lanes they come from.  One wavefront per lane.
+__global__ void __launch_bounds__(64) flat_rows_kernel(int lane_count, Scratch sc) {
+    const int local = blockIdx.x;
+    if (local >= lane_count) return;
+    const int *span = sc.flat_span + (size_t)local * 4;
+    const int lo0 = span[0], hi0 = span[1], lo1 = span[2], hi1 = span[3];
     const int rows0 = hi0 < lo0 ? 0 : hi0 - lo0 + 1, rows1 = hi1 < lo1 ? 0 : hi1 - lo1 + 1;
     if (rows0 + rows1 == 0) return;                  // the same in every thread
+    int list_base = 0;
     if (threadIdx.x == 0) list_base = atomicAdd(sc.flat_row_count, rows0 + rows1);
-    __syncthreads();
+    list_base = __shfl(list_base, 0);
     for (int r = threadIdx.x; r < rows0 + rows1; r += blockDim.x)
         sc.flat_rows[list_base + r] = (local << 8) | (r < rows0 ? lo0 + r : lo1 + (r - rows0));
 }
@@ -4439,6 +4473,8 @@ size_t carve_scratch(Scratch &sc, unsigned char *base, size_t L, const gd_map_de
     take(&sc.flat_tail, L * 2 * SW);
     take(&sc.flat_rows, L * (size_t)VH);
     take(&sc.flat_row_count, 1);
+    take(&sc.gap_columns, L * 2 * SW);
+    take(&sc.gap_column_count, 1);
     take(&sc.flat_col_top, L * 2 * SW);
     take(&sc.flat_list, L * FLAT_LIST_MAX);
     take(&sc.flat_list_count, L);
@@ -4673,6 +4709,8 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     mark();
     // the flat pass, where the walls left it something to decide
     hipLaunchKernelGGL(flat_gap_column_kernel, dim3(count), dim3(GAP_THREADS), 0, stream, r->dm, *lanes, base, count, sc);
+    hipLaunchKernelGGL(flat_gap_repair_kernel, dim3(GAP_REPAIR_BLOCKS), dim3(64), 0, stream, r->dm, *lanes, base, sc);
+    hipLaunchKernelGGL(flat_rows_kernel, dim3(count), dim3(64), 0, stream, count, sc);
     const int plane_levels = m.floor_level_count + m.ceil_level_count;
     const bool level_masks = plane_levels > LEVEL_MASK_MIN_LEVELS && plane_levels <= 32 * LEVEL_MASK_WORDS_MAX;   // level_mask_words() > 0
     hipLaunchKernelGGL(level_masks ? flat_span_select_kernel<true> : flat_span_select_kernel<false>, dim3(SPAN_SELECT_BLOCKS), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
