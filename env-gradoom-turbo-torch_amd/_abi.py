@@ -24,7 +24,7 @@ GD_E_ARG = -1
 GD_E_HIP = -2
 GD_E_UNSUPPORTED = -3
 
-ABI_VERSION = 3  # GD_ABI_VERSION
+ABI_VERSION = 4  # GD_ABI_VERSION
 
 _P = C.c_void_p
 
@@ -373,4 +373,21 @@ class ActorDesc(_Sized):
         [("struct_size", C.c_uint32)]
         + [(name, C.c_int32) for name in ACTOR_SCALARS] + [(name, _P) for name, _ in ACTOR_ARRAYS]
         + [(name, _P) for name, _ in ACTOR_OUTPUTS]
+    )
+
+
+WEAPON_INPUTS = (
+    "active_weapon", "weapon_state_cooldown", "weapon_fire_count", "weapon_ready_tics", "weapon_lower_cooldown",
+    "weapon_raise_cooldown", "pending_weapon", "episode_time", "player_bob_fixed", "player_dead",
+)
+WEAPON_TABLES = ("weapon_frame_ids", "weapon_flash_ids", "weapon_flash_lights", "fine_sine")
+
+
+class WeaponDesc(_Sized):
+    """``gd_weapon_desc``: the gameplay tensors ``gd_pack_weapon`` reads and the two tensors it writes."""
+
+    _fields_ = (
+        [("struct_size", C.c_uint32), ("lane_count", C.c_int32), ("cooldown_slots", C.c_int32)]
+        + [(name, _P) for name in WEAPON_INPUTS + WEAPON_TABLES]
+        + [("weapon_state", _P), ("flash_light", _P)]
     )

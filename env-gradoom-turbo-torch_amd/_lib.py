@@ -28,6 +28,7 @@ SYMBOLS = (
     "gd_observe",
     "gd_expand_rgb24",
     "gd_pack_actors",
+    "gd_pack_weapon",
 )
 
 _LIBRARY = None
@@ -81,6 +82,8 @@ def library() -> C.CDLL:
     lib.gd_expand_rgb24.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p]
     lib.gd_pack_actors.restype = C.c_int
     lib.gd_pack_actors.argtypes = [C.POINTER(_abi.ActorDesc), C.c_void_p]
+    lib.gd_pack_weapon.restype = C.c_int
+    lib.gd_pack_weapon.argtypes = [C.POINTER(_abi.WeaponDesc), C.c_void_p]
     _LIBRARY = lib
     return lib
 

@@ -130,7 +130,7 @@ def item_patches(engine) -> tuple[torch.Tensor, torch.Tensor]:
     frames = m.raw_item_animation_sprite_ids
     elapsed = engine.episode_time[:, None] + (6 - engine.item_animation_initial_tics)
     phase = torch.remainder(elapsed // 6, 6)                        # A B C D C B, six tics each; A is the still patch
-    back_and_forth = torch.tensor((-1, 0, 1, 2, 1, 0), device=phase.device)[phase]
+    back_and_forth = 2 - torch.abs(phase - 3)                       # -1 0 1 2 1 0
     health = torch.where(back_and_forth < 0, still, frames[back_and_forth.clamp_min(0)])
     armor = torch.where(back_and_forth < 0, still, frames[back_and_forth.clamp_min(0) + 3])
     patch = torch.where(kinds == 2014, health, still)

@@ -184,8 +184,8 @@ struct Scratch {    // per-chunk working memory, sized at create
                            // could not resolve, as one work list: lane << 18 | half << 17 | topmost such row << 9 | column
     int *gap_column_count; // [1] its length (cleared by lane_setup_kernel, filled by flat_gap_column_kernel)
     int *flat_col_top;     // [L,2,320] per screen half and column: the topmost shown pixel the flat pass could not
-                           // resolve (any value >= 208: none).  flat_gap_column_kernel lowers it while it selects the
-                           // gap pixels, then reads it and puts "none" back, so it is filled once, when the renderer is created.
+                           // resolve (any value >= 208: none).  lane_tables_kernel sets "none", flat_gap_column_kernel
+                           // lowers it while it selects the gap pixels.
     PassRec *pass_rec;     // [L,PASS_MAX,320] the drawsegs of each column's passes, in pass order
     float *pass_path_distance;  // [L,PASS_MAX,320] distance of the portal path of a pass that carries PB_PS_KEEPS (written for those only)
     unsigned char *pass_count;  // [L,320] passes recorded for the column: up to its last pass that draws or moves a clip
@@ -476,6 +476,8 @@ __global__ void lane_tables_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
     const LaneCtx &c = sc.ctx[local];
     // the lane's per-column lists start empty
     for (int x = threadIdx.x; x < SW; x += blockDim.x) { sc.cand_count[(size_t)local * SW + x] = 0; sc.block_hit[(size_t)local * SW + x] = ~0ULL; }
+    // and no column holds an unresolved gap pixel yet
+    for (int k = threadIdx.x; k < 2 * SW; k += blockDim.x) sc.flat_col_top[(size_t)local * 2 * SW + k] = VH;
     const float cx = lanes.x[lane_base + local], cy = lanes.y[lane_base + local];
     __shared__ unsigned int masks_lds[LEVEL_BUCKETS * LEVEL_MASK_WORDS_MAX];
     const int mask_words = level_mask_words(&dm.d);
@@ -1320,7 +1322,6 @@ __global__ void __launch_bounds__(GAP_THREADS) __attribute__((amdgpu_waves_per_e
         int *top_at = sc.flat_col_top + ((size_t)local * 2 + half) * SW + x;
         const int top = __hip_atomic_load(top_at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // where the atomics above wrote, not a cached copy
         if (top < VH) {
-            *top_at = VH;
             column_list[atomicAdd(&column_count, 1)] = x | (top << 9) | (half << 17) | (local << 18);
         }
     }
@@ -4380,6 +4381,41 @@ thread_local std::string g_error;
 
 int fail(int code, const std::string &message) { g_error = message; return code; }
 
+// gd_pack_weapon: one thread per lane.  Which patch the player's weapon shows and where (engine.py:14949-14967,
+// 15051-15092): the frame table is indexed by weapon, by a parity that alternates with every shot (an idling chainsaw
+// alternates every four tics instead) and by the tics left of the weapon's state; a weapon being lowered or raised sits
+// six map pixels lower per tic, as does one raised at the start of an episode; a ready weapon sways with the player's bob
+// along a circle of the fine sine table that advances 128 steps a tic.
+__global__ void __launch_bounds__(64) pack_weapon_kernel(gd_weapon_desc d) {
+    const int lane = blockIdx.x * blockDim.x + threadIdx.x;
+    if (lane >= d.lane_count) return;
+    const i64 slots = d.cooldown_slots;
+    const i64 weapon = clampi(d.active_weapon[lane], 0, 7);
+    const i64 state_tics = d.weapon_state_cooldown[lane];
+    const i64 tic = clampi(state_tics, 0, slots - 1);
+    i64 parity = d.weapon_fire_count[lane] % 2;
+    if (parity < 0) parity += 2;                    // torch.remainder: the sign of the divisor
+    if (weapon == 1 && tic == 0) parity = (max64(d.weapon_ready_tics[lane] - 1, 0) / 4) % 2;
+    const i64 entry = (weapon * 2 + parity) * slots + tic;
+    const i64 switching = d.pending_weapon[lane] >= 0;
+    const i64 raising = d.weapon_raise_cooldown[lane];
+    i64 lowered = switching ? clampi(16 - d.weapon_lower_cooldown[lane], 0, 16) : raising;      // engine.py:111 (16 tics to lower)
+    const i64 time = d.episode_time[lane];
+    lowered = max64(lowered, clampi(14 - (time - 1), 0, 14));                                   // engine.py:114 (14 tics to raise at spawn)
+    const bool steady = state_tics <= 0 && raising <= 0 && !switching;
+    const i64 swing = mul64(time, 128) & (FINE_ANGLES - 1);
+    const i64 bob = d.player_bob_fixed[lane];
+    const i64 sway_x = steady ? mul64(bob, d.fine_sine[(swing + FINE_ANGLES / 4) & (FINE_ANGLES - 1)]) >> 16 : 0;
+    const i64 sway_y = steady ? mul64(bob, d.fine_sine[swing & (FINE_ANGLES / 2 - 1)]) >> 16 : 0;
+    int64_t *out = d.weapon_state + (size_t)lane * 5;
+    out[0] = d.weapon_frame_ids[entry];
+    out[1] = d.weapon_flash_ids[entry];
+    out[2] = sway_x;
+    out[3] = mul64(lowered, 6 * FIXED_UNIT) + sway_y;
+    out[4] = d.player_dead[lane] ? 0 : 1;
+    if (d.flash_light) d.flash_light[lane] = d.weapon_flash_lights[entry];
+}
+
 #define HIP_TRY(expr)                                                                          \
     do {                                                                                       \
         hipError_t e_ = (expr);                                                                \
@@ -4930,8 +4966,6 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
         if (rc == GD_OK) {
             carve_scratch(sc, block, (size_t)chunk, *h, false);
             r->scratch_block = block; r->scratch_bytes = bytes;
-            hipLaunchKernelGGL(fill_words_kernel, dim3(256), dim3(256), 0, 0, reinterpret_cast<unsigned int *>(sc.flat_col_top), (size_t)chunk * 2 * SW, 0x7f7f7f7fu);
-            if (hipDeviceSynchronize() != hipSuccess) rc = fail(GD_E_HIP, "filling flat_col_top");
         }
     }
     if (rc == GD_OK) rc = scratch_alloc(r, 1, &sc.status);
@@ -5018,8 +5052,7 @@ int gd_render_static(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_
         return fail(GD_E_ARG, "gd_render_static renders at most " + std::to_string(GD_STATIC_MAX_LANES) + " lanes per call");
     carve_scratch(sc, block, (size_t)chunk, m, decals);
     hipStream_t caller = static_cast<hipStream_t>(stream);
-    // the block keeps whatever the last call left: the one buffer the kernels expect to find ready is filled here
-    hipLaunchKernelGGL(fill_words_kernel, dim3(64), dim3(256), 0, caller, reinterpret_cast<unsigned int *>(sc.flat_col_top), (size_t)chunk * 2 * SW, 0x7f7f7f7fu);
+    // the block keeps whatever the last call left: the kernels expect nothing of it
     for (int base = 0; base < lanes->lane_count; base += chunk) {
         const int count = lanes->lane_count - base < chunk ? lanes->lane_count - base : chunk;
         rc = launch_chunk(r, sc, lanes, out, base, count, caller, false);
@@ -5062,7 +5095,7 @@ int gd_renderer_status(gd_renderer *r, int32_t *status) {
     return GD_OK;
 }
 
-/* Fill the renderer's working memory with one byte value (then put back the one buffer the kernels expect ready).
+/* Fill the renderer's working memory with one byte value.
    Frames must not depend on what that memory held; this lets a caller check it.  Replaces nothing in the reference. */
 int gd_renderer_scribble(gd_renderer *r, int32_t value, void *stream) {
     if (!r) return fail(GD_E_ARG, "null argument");
@@ -5070,7 +5103,6 @@ int gd_renderer_scribble(gd_renderer *r, int32_t value, void *stream) {
     hipStream_t st = static_cast<hipStream_t>(stream);
     const unsigned int byte = (unsigned int)value & 0xFFu, word = byte * 0x01010101u;
     hipLaunchKernelGGL(fill_words_kernel, dim3(4096), dim3(256), 0, st, reinterpret_cast<unsigned int *>(r->scratch_block), r->scratch_bytes / 4, word);
-    hipLaunchKernelGGL(fill_words_kernel, dim3(256), dim3(256), 0, st, reinterpret_cast<unsigned int *>(r->sc.flat_col_top), (size_t)r->chunk_lanes * 2 * SW, 0x7f7f7f7fu);
     HIP_TRY(hipGetLastError());
     return GD_OK;
 }
@@ -5205,6 +5237,21 @@ int gd_pack_actors(const gd_actor_desc *a, void *stream) {
     if (width > 65535 * 64LL || a->lane_count > 65535) return fail(GD_E_ARG, "too many slots or lanes for one launch");
     hipLaunchKernelGGL(pack_actors_kernel, dim3((unsigned)((width + 63) / 64), (unsigned)a->lane_count), dim3(64), 0,
                        static_cast<hipStream_t>(stream), *a, (int)width);
+    HIP_TRY(hipGetLastError());
+    return GD_OK;
+}
+
+int gd_pack_weapon(const gd_weapon_desc *w, void *stream) {
+    if (!w) return fail(GD_E_ARG, "null argument");
+    SIZE_CHECK(w, gd_weapon_desc);
+    if (w->lane_count < 0 || w->cooldown_slots <= 0) return fail(GD_E_ARG, "gd_weapon_desc holds a count out of range");
+    const void *const needed[] = {w->active_weapon, w->weapon_state_cooldown, w->weapon_fire_count, w->weapon_ready_tics, w->weapon_lower_cooldown,
+                                  w->weapon_raise_cooldown, w->pending_weapon, w->episode_time, w->player_bob_fixed, w->player_dead,
+                                  w->weapon_frame_ids, w->weapon_flash_ids, w->fine_sine, w->weapon_state};
+    for (const void *p : needed) if (!p) return fail(GD_E_ARG, "null tensor in gd_weapon_desc");
+    if (w->flash_light && !w->weapon_flash_lights) return fail(GD_E_ARG, "flash_light needs weapon_flash_lights");
+    if (w->lane_count == 0) return GD_OK;
+    hipLaunchKernelGGL(pack_weapon_kernel, dim3((unsigned)((w->lane_count + 63) / 64)), dim3(64), 0, static_cast<hipStream_t>(stream), *w);
     HIP_TRY(hipGetLastError());
     return GD_OK;
 }

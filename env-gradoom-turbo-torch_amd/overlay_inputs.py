@@ -35,52 +35,104 @@ def fine_sine_fixed() -> np.ndarray:
     return table
 
 
-def weapon_state(
-    *,
-    active_weapon: torch.Tensor,
-    weapon_state_cooldown: torch.Tensor,
-    weapon_fire_count: torch.Tensor,
-    weapon_ready_tics: torch.Tensor,
-    weapon_lower_cooldown: torch.Tensor,
-    weapon_raise_cooldown: torch.Tensor,
-    pending_weapon: torch.Tensor,
-    episode_time: torch.Tensor,
-    player_bob_fixed: torch.Tensor,
-    player_dead: torch.Tensor,
-    weapon_frame_ids: torch.Tensor,
-    weapon_flash_ids: torch.Tensor,
-    fine_sine: torch.Tensor,
-) -> torch.Tensor:
+_WEAPON_INPUTS = (
+    "active_weapon", "weapon_state_cooldown", "weapon_fire_count", "weapon_ready_tics", "weapon_lower_cooldown",
+    "weapon_raise_cooldown", "pending_weapon", "episode_time", "player_bob_fixed",
+)
+
+
+def weapon_state(*, weapon_frame_ids: torch.Tensor, weapon_flash_ids: torch.Tensor, fine_sine: torch.Tensor,
+                 weapon_flash_lights: torch.Tensor | None = None, want_flash_light: bool = False, **engine: torch.Tensor):
     """``int64 [N,5]``: patch id, flash patch id, horizontal and vertical offset (16.16), visible.
 
-    ``_native_weapon_frame_selection`` (``engine.py:14949-14967``) and the offsets of
-    ``_native_render_weapon`` (``engine.py:15051-15092``).  ``weapon_frame_ids`` / ``weapon_flash_ids``
-    are the map's ``[8, 2, cooldowns]`` tables, ``fine_sine`` the table of :func:`fine_sine_fixed`.
+    The per-lane half of the reference's weapon layer: ``_native_weapon_frame_selection``
+    (``engine.py:14949-14967``) and the raise / lower / bob offsets of ``_native_render_weapon``
+    (``engine.py:15051-15092``).  ``engine`` holds the gameplay tensors by the engine's attribute names
+    (``active_weapon`` = ``_active_weapon()``, ``player_bob_fixed`` = ``_player_bob_fixed``, ``player_dead`` bool);
+    ``weapon_frame_ids`` / ``weapon_flash_ids`` / ``weapon_flash_lights`` are the map's ``[8, 2, cooldowns]`` tables,
+    ``fine_sine`` the table of :func:`fine_sine_fixed`.  With ``want_flash_light`` the muzzle flash's extra light level
+    comes back as well (``int64 [N]``).
+
+    Tensors on a ROCm device are read where they are by one kernel (``gd_pack_weapon``): no host synchronisation.
+    Host tensors (tests, fixture scripts) take the NumPy restatement below.
     """
 
-    weapon = active_weapon.to(torch.int64).clamp(0, 7)
-    cooldown = weapon_state_cooldown.to(torch.int64).clamp(0, weapon_frame_ids.shape[2] - 1)
-    parity = torch.remainder(weapon_fire_count, 2).to(torch.int64)
-    idle_chainsaw = (weapon == 1) & (cooldown == 0)
-    idle_phase = torch.remainder(torch.clamp_min(weapon_ready_tics - 1, 0) // 4, 2).to(torch.int64)
-    parity = torch.where(idle_chainsaw, idle_phase, parity)
-    frame_id = weapon_frame_ids[weapon, parity, cooldown].to(torch.int64)
-    flash_id = weapon_flash_ids[weapon, parity, cooldown].to(torch.int64)
+    if engine["episode_time"].device.type == "cuda":
+        return _weapon_state_device(engine, weapon_frame_ids, weapon_flash_ids, weapon_flash_lights, fine_sine, want_flash_light)
+    host = {name: np.asarray(value.cpu()).astype(np.int64) for name, value in engine.items() if name in _WEAPON_INPUTS}
+    words, light = _weapon_words_host(
+        host, np.asarray(engine["player_dead"].cpu()).astype(bool), np.asarray(weapon_frame_ids.cpu()).astype(np.int64),
+        np.asarray(weapon_flash_ids.cpu()).astype(np.int64),
+        None if weapon_flash_lights is None else np.asarray(weapon_flash_lights.cpu()).astype(np.int64), np.asarray(fine_sine.cpu()).astype(np.int64),
+    )
+    words = torch.as_tensor(words)
+    return (words, torch.as_tensor(light)) if want_flash_light else words
 
-    lower_vertical_tics = torch.clamp(WEAPON_LOWER_TICS - weapon_lower_cooldown, 0, WEAPON_LOWER_TICS)
-    vertical_tics = torch.where(pending_weapon >= 0, lower_vertical_tics, weapon_raise_cooldown)
-    spawn_raise_tics = torch.clamp(WEAPON_SPAWN_RAISE_TICS - (episode_time - 1), 0, WEAPON_SPAWN_RAISE_TICS)
-    vertical_tics = torch.maximum(vertical_tics, spawn_raise_tics)
-    ready = (weapon_state_cooldown <= 0) & (weapon_raise_cooldown <= 0) & (pending_weapon < 0)
-    bob_angle = (episode_time.to(torch.int64) * 128) & (FINE_ANGLES - 1)
-    bob = player_bob_fixed.to(torch.int64)
-    bob_x_fixed = (bob * fine_sine[(bob_angle + FINE_ANGLES // 4) & (FINE_ANGLES - 1)]) >> 16
-    bob_y_fixed = (bob * fine_sine[bob_angle & (FINE_ANGLES // 2 - 1)]) >> 16
-    bob_x_fixed = torch.where(ready, bob_x_fixed, torch.zeros_like(bob_x_fixed))
-    bob_y_fixed = torch.where(ready, bob_y_fixed, torch.zeros_like(bob_y_fixed))
-    vertical_offset_fixed = vertical_tics.to(torch.int64) * 6 * FIXED_UNIT + bob_y_fixed
-    visible = (~player_dead).to(torch.int64)
-    return torch.stack((frame_id, flash_id, bob_x_fixed, vertical_offset_fixed, visible), dim=1).contiguous()
+
+def _weapon_state_device(engine, frame_ids, flash_ids, flash_lights, fine_sine, want_flash_light):
+    import ctypes as C
+
+    from . import _abi, _lib
+
+    device = engine["episode_time"].device
+    count = int(engine["episode_time"].shape[0])
+    desc = _abi.WeaponDesc()
+    desc.lane_count = count
+    desc.cooldown_slots = int(frame_ids.shape[2])
+    keep = []
+
+    def pointer(tensor, dtype):
+        if tensor.device != device:
+            raise TypeError("every weapon tensor must live on the engine's device")
+        tensor = tensor.to(dtype).contiguous()   # a no-op for tensors that already are
+        keep.append(tensor)
+        return tensor.data_ptr()
+
+    for name in _WEAPON_INPUTS:
+        setattr(desc, name, pointer(engine[name], torch.int64))
+    desc.player_dead = pointer(engine["player_dead"], torch.uint8)
+    desc.weapon_frame_ids = pointer(frame_ids, torch.int64)
+    desc.weapon_flash_ids = pointer(flash_ids, torch.int64)
+    desc.fine_sine = pointer(fine_sine, torch.int64)
+    words = torch.empty((count, 5), dtype=torch.int64, device=device)
+    desc.weapon_state = words.data_ptr()
+    light = None
+    if want_flash_light:
+        if flash_lights is None:
+            raise ValueError("want_flash_light needs weapon_flash_lights")
+        desc.weapon_flash_lights = pointer(flash_lights, torch.int64)
+        light = torch.empty((count,), dtype=torch.int64, device=device)
+        desc.flash_light = light.data_ptr()
+    with torch.cuda.device(device):
+        stream = torch.cuda.current_stream(device).cuda_stream
+        _lib.check(_lib.library().gd_pack_weapon(C.byref(desc), C.c_void_p(stream)))
+    del keep
+    return (words, light) if want_flash_light else words
+
+
+def _weapon_words_host(state: dict, dead: np.ndarray, frame_table: np.ndarray, flash_table: np.ndarray, light_table, sine: np.ndarray):
+    """The words of :func:`weapon_state` for host arrays, as the kernel computes them (test infrastructure)."""
+
+    tics = state["episode_time"]
+    slot = np.clip(state["active_weapon"], 0, 7)
+    step = np.clip(state["weapon_state_cooldown"], 0, frame_table.shape[2] - 1)
+    phase = np.mod(state["weapon_fire_count"], 2)
+    idling_saw = (slot == 1) & (step == 0)             # the chainsaw's idle frames alternate every four tics
+    phase[idling_saw] = (np.maximum(state["weapon_ready_tics"][idling_saw] - 1, 0) // 4) % 2
+    words = np.zeros((len(tics), 5), dtype=np.int64)
+    words[:, 0] = frame_table[slot, phase, step]
+    words[:, 1] = flash_table[slot, phase, step]
+    switching = state["pending_weapon"] >= 0
+    drop = np.where(switching, np.clip(WEAPON_LOWER_TICS - state["weapon_lower_cooldown"], 0, WEAPON_LOWER_TICS), state["weapon_raise_cooldown"])
+    drop = np.maximum(drop, np.clip(WEAPON_SPAWN_RAISE_TICS + 1 - tics, 0, WEAPON_SPAWN_RAISE_TICS))
+    steady = (state["weapon_state_cooldown"] <= 0) & (state["weapon_raise_cooldown"] <= 0) & ~switching
+    swing = (tics * 128) % FINE_ANGLES
+    bob = state["player_bob_fixed"]
+    words[:, 2] = np.where(steady, (bob * sine[(swing + FINE_ANGLES // 4) % FINE_ANGLES]) >> 16, 0)
+    words[:, 3] = drop * (6 * FIXED_UNIT) + np.where(steady, (bob * sine[swing % (FINE_ANGLES // 2)]) >> 16, 0)
+    words[:, 4] = ~dead
+    light = None if light_table is None else light_table[slot, phase, step]
+    return words, light
 
 
 def mugshot_patch(
@@ -101,7 +153,7 @@ def mugshot_patch(
     face = 13 + pain * 3 + mugshot_face_index.to(torch.int64)
     rampage = attack_held_tics >= MUGSHOT_RAMPAGE_DELAY
     face = torch.where(rampage, 49 + pain, face)
-    direction_base = torch.tensor((44, 49, 54), dtype=torch.int64, device=health.device)[mugshot_pain_direction.to(torch.int64)]
+    direction_base = 44 + 5 * mugshot_pain_direction.to(torch.int64)   # 44, 49, 54 for directions 0, 1, 2 (no table: a device constant would be copied from the host every call)
     pained = torch.where(mugshot_ouch, 59 + pain, direction_base + pain)
     face = torch.where(mugshot_pain_tics > 0, pained, face)
     face = torch.where(mugshot_grin_tics > 0, 64 + pain, face)
@@ -164,24 +216,22 @@ def decal_inputs(serial, wall, along, impact_z, style, portal_walls, fine_sine_f
 
     ``serial, wall, along, impact_z, style`` are the engine's ``hitscan_decal_*`` tensors ``[N, slots]``
     (serial < 0 = free slot), ``portal_walls`` the map's ``[W,4]`` linedefs and ``fine_sine_fixed`` the
-    8192-entry fine sine table (``fine_sine_fixed()``).  Returns ``(decal_state i32 [N,D,3], decal_geom
-    f32 [N,D,4])`` with D the largest number of live decals in a lane, or ``None`` when no lane has one.
-    Older impacts come first so that a later chip shades an earlier one at the same texels.
+    8192-entry fine sine table (``fine_sine_fixed()``).  Returns ``(decal_state i32 [N,slots,3], decal_geom
+    f32 [N,slots,4])``, or ``None`` when the engine keeps no decal slots.  The shape is fixed: every slot is packed,
+    live ones first and older impacts before newer ones (a later chip shades an earlier one at the same texels), free
+    slots last with their ``alive`` word zero, which the decal kernel skips.  Nothing here waits for the device.
     """
 
-    active_slots = torch.nonzero(torch.any(serial >= 0, dim=0)).flatten()
-    if not active_slots.numel():
+    if serial.shape[1] == 0:
         return None
-    serial = serial[:, active_slots].to(torch.int64)
+    serial = serial.to(torch.int64)
     active = serial >= 0
-    layers = int(torch.amax(torch.sum(active, dim=1)).item())
-    order = torch.argsort(torch.where(active, serial, torch.full_like(serial, torch.iinfo(torch.int32).max)), dim=1)
-    order = order[:, :layers]
-    pick = lambda tensor: tensor[:, active_slots].gather(1, order)  # noqa: E731
-    alive = active.gather(1, order)
+    order = torch.argsort(torch.where(active, serial, torch.full_like(serial, torch.iinfo(torch.int32).max)), dim=1, stable=True)
+    pick = lambda tensor: tensor.gather(1, order)  # noqa: E731
+    alive = pick(active)
     wall_index = pick(wall).to(torch.int64).clamp(0, portal_walls.shape[0] - 1)
     style_index = pick(style).to(torch.int64)
-    side = style_index // 20
+    side = torch.div(style_index, 20, rounding_mode="floor")
     segment = portal_walls[wall_index]
     vector = segment[..., 2:] - segment[..., :2]
     # the seg runs backwards on sidedef 1; its direction goes through the fine-angle table

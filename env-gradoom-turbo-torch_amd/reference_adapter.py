@@ -113,12 +113,12 @@ class HipReferenceRenderer:
 
         e = self.engine
         contiguous = lambda t: t if t.is_contiguous() else t.contiguous()  # noqa: E731
-        flash = e._native_weapon_frame_selection()[2]   # extralight of the muzzle flash, engine.py:14949-14967
         fields = dict(
             x=contiguous(e.x), y=contiguous(e.y), angle=contiguous(e.angle), view_z=contiguous(e.view_z),
             x_fixed=contiguous(e._x_fixed), y_fixed=contiguous(e._y_fixed), angle_bam=contiguous(e._angle_bam),
-            pitch_bam=contiguous(e._pitch_bam), flash_light=flash.to(torch.int64).contiguous(),
+            pitch_bam=contiguous(e._pitch_bam),
         )
+        flash = None   # extralight of the muzzle flash, engine.py:14949-14967
         ray_cos, ray_sin = hostmath.ray_tables(e.angle, self._ray_offsets)
         fields.update(ray_cos=ray_cos, ray_sin=ray_sin)
         if self._has_actors:
@@ -128,10 +128,14 @@ class HipReferenceRenderer:
             fields["sprite_depth"] = hostmath.sprite_depth(e.x, e.y, e.angle, packed["sprite_x"], packed["sprite_y"])
         if self._overlays is not None:
             tensors = overlay_engine_tensors(e)
-            fields["weapon_state"] = overlay_inputs.weapon_state(
+            # the weapon words and, where the map carries the table, the flash's extra light: one kernel, no host round trip
+            lights = getattr(e.map, "native_weapon_flash_lights", None)
+            packed = overlay_inputs.weapon_state(
                 **{k: tensors[k] for k in WEAPON_ARGUMENTS}, weapon_frame_ids=self._weapon_frame_ids,
                 weapon_flash_ids=self._weapon_flash_ids, fine_sine=self._fine_sine,
+                weapon_flash_lights=lights, want_flash_light=lights is not None,
             )
+            fields["weapon_state"], flash = packed if lights is not None else (packed, None)
             if include_hud:
                 fields["hud_state"] = overlay_inputs.hud_state(**{k: tensors[k] for k in HUD_ARGUMENTS})
         if self._has_decals:
@@ -140,6 +144,9 @@ class HipReferenceRenderer:
                 e.map.portal_walls, self._fine_sine,
             )
             fields.update(decal_state=state, decal_geom=geometry)
+        if flash is None:
+            flash = e._native_weapon_frame_selection()[2]
+        fields["flash_light"] = flash.to(torch.int64).contiguous()
         if getattr(e, "render_screen_flashes", False):
             fields["screen_blend"] = overlay_inputs.screen_blend(e.bonus_count, e.damage_count, e._damage_to_alpha)
         return LaneState(**fields)

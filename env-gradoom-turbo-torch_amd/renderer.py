@@ -109,11 +109,13 @@ class HipRenderer:
         self.max_lanes = int(max_lanes)
         self.chunk_lanes = min(self.max_lanes, 4096)  # lanes per kernel launch (library working-memory chunk)
         if cosine_correction is None:
-            cosine_correction = hostmath.cosine_correction("cpu").numpy()
+            # the same Torch ops on the same device as the ray tables and billboard depths this renderer derives per frame
+            # (_lanes_desc): the stand-alone path is the reference's arithmetic on that device (engine.py:1527-1531, 2050-2054)
+            cosine_correction = hostmath.cosine_correction(self.device).cpu().numpy()
         self._cosine = np.ascontiguousarray(cosine_correction, dtype=np.float32)
         if self._cosine.shape != (_abi.SCREEN_WIDTH,):
             raise ValueError("cosine_correction must hold 320 floats")
-        self.ray_offsets = hostmath.native_ray_offsets("cpu").to(self.device)
+        self.ray_offsets = hostmath.native_ray_offsets(self.device)
         self.playpal = torch.as_tensor(self.tables["playpal"]).to(self.device).contiguous()
         desc, keep = _abi.host_map_desc(self.tables)
         handle = C.c_void_p()
@@ -294,15 +296,16 @@ class HipRenderer:
         del keep_lanes, keep_out
 
     def render_static(self, lanes: LaneState, *, indexed=None, obs=None, frames=None, reset_mask=None, rgb=None,
-                      stack_only_masked: bool = False, final_frames=None) -> None:
+                      stack_only_masked: bool = False, final_frames=None, obs_source_rows: int = 208, final_layout: str = "chw") -> None:
         """``render`` through the entry point that allocates nothing (``gd_render_static``): the working memory is
-        the library's fixed per-GPU array, so a renderer created with ``max_lanes=0`` can call it.  Calls that
-        overlap on one GPU race; ``ValueError`` when one lane of the map does not fit the array."""
+        the library's fixed per-GPU array, so a renderer created with ``max_lanes=0`` can call it.  Same arguments
+        as ``render``.  Calls that overlap on one GPU race; ``ValueError`` when one lane of the map does not fit the array."""
 
         if self._handle is None:
             raise RuntimeError("renderer is closed")
         desc, keep_lanes = self._lanes_desc(lanes)
-        out, keep_out = self._out_desc(desc.lane_count, indexed, obs, frames, reset_mask, rgb, stack_only_masked, final_frames)
+        out, keep_out = self._out_desc(desc.lane_count, indexed, obs, frames, reset_mask, rgb, stack_only_masked, final_frames, obs_source_rows,
+                                       final_layout)
         stream = torch.cuda.current_stream(self.device).cuda_stream
         _lib.check(self._lib.gd_render_static(self._handle, C.byref(desc), C.byref(out), C.c_void_p(stream)))
         del keep_lanes, keep_out

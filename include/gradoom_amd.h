@@ -40,7 +40,7 @@ extern "C" {
  * Layout version of the structs below.  Every descriptor also starts with its own sizeof, which each entry
  * point checks: a caller built against another header gets GD_E_ARG instead of a wild read.
  */
-#define GD_ABI_VERSION 3
+#define GD_ABI_VERSION 4
 
 #define GD_OK 0
 #define GD_E_ARG (-1)       /* bad argument: null pointer, negative count, size over a limit */
@@ -448,6 +448,42 @@ typedef struct gd_actor_desc {
 } gd_actor_desc;
 
 int gd_pack_actors(const gd_actor_desc *actors, void *stream);
+
+/*
+ * The five weapon_state words of every lane (gd_lanes_desc.weapon_state) and the muzzle flash's extra light
+ * (gd_lanes_desc.flash_light), from the gameplay tensors, in one kernel with no host synchronisation.
+ * Replaces the per-lane part of the reference's weapon layer: frame / flash selection
+ * (engine.py:14949-14967 _native_weapon_frame_selection) and the raise / lower / bob offsets of
+ * engine.py:15051-15092 (_native_render_weapon).  Every input is an int64 device array of lane_count entries (the engine's
+ * attributes of the same names; active_weapon is engine._active_weapon(), player_bob_fixed engine._player_bob_fixed),
+ * player_dead a bool array; the three tables are the map's native_weapon_frame_ids / _flash_ids / _flash_lights
+ * [8, 2, cooldown_slots] as int64, fine_sine the 8192-entry 16.16 sine table (engine.py:309-321).
+ * weapon_state receives [lane_count, 5]: patch id, flash patch id (-1: none), horizontal and vertical offset (16.16),
+ * visible.  flash_light (may be null) receives the flash's extra light level.  Returns GD_E_ARG for a null pointer or
+ * a count out of range.
+ */
+typedef struct gd_weapon_desc {
+    uint32_t struct_size;    /* sizeof(gd_weapon_desc) of the header the caller was built with */
+    int32_t lane_count, cooldown_slots;
+    const int64_t *active_weapon;
+    const int64_t *weapon_state_cooldown;
+    const int64_t *weapon_fire_count;
+    const int64_t *weapon_ready_tics;
+    const int64_t *weapon_lower_cooldown;
+    const int64_t *weapon_raise_cooldown;
+    const int64_t *pending_weapon;
+    const int64_t *episode_time;
+    const int64_t *player_bob_fixed;
+    const uint8_t *player_dead;
+    const int64_t *weapon_frame_ids;
+    const int64_t *weapon_flash_ids;
+    const int64_t *weapon_flash_lights;   /* may be null when flash_light is */
+    const int64_t *fine_sine;
+    int64_t *weapon_state;
+    int64_t *flash_light;
+} gd_weapon_desc;
+
+int gd_pack_weapon(const gd_weapon_desc *weapon, void *stream);
 
 /*
  * Time `launches` back-to-back gd_render launches with HIP events on `stream`

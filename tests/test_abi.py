@@ -60,6 +60,7 @@ def test_struct_layouts_match_header_field_order():
     assert fields("gd_frame_out") == [name for name, _ in _abi.FrameOut._fields_]
     assert fields("gd_overlay_desc") == [name for name, _ in _abi.OverlayDesc._fields_]
     assert fields("gd_actor_desc") == [name for name, _ in _abi.ActorDesc._fields_]
+    assert fields("gd_weapon_desc") == [name for name, _ in _abi.WeaponDesc._fields_]
 
 
 def test_struct_sizes_match_what_a_c_compiler_makes_of_the_header(tmp_path):
@@ -70,15 +71,15 @@ def test_struct_sizes_match_what_a_c_compiler_makes_of_the_header(tmp_path):
 
     source = tmp_path / "sizes.c"
     source.write_text(
-        '#include <stdio.h>\n#include "gradoom_amd.h"\nint main(void) { printf("%zu %zu %zu %zu %zu %d\\n", sizeof(gd_map_desc), '
-        "sizeof(gd_lanes_desc), sizeof(gd_frame_out), sizeof(gd_overlay_desc), sizeof(gd_actor_desc), GD_ABI_VERSION); return 0; }\n"
+        '#include <stdio.h>\n#include "gradoom_amd.h"\nint main(void) { printf("%zu %zu %zu %zu %zu %zu %d\\n", sizeof(gd_map_desc), '
+        "sizeof(gd_lanes_desc), sizeof(gd_frame_out), sizeof(gd_overlay_desc), sizeof(gd_actor_desc), sizeof(gd_weapon_desc), GD_ABI_VERSION); return 0; }\n"
     )
     binary = tmp_path / "sizes"
     subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(source), "-o", str(binary)], check=True)
     sizes = [int(v) for v in subprocess.run([str(binary)], check=True, capture_output=True, text=True).stdout.split()]
-    ours = [ctypes.sizeof(t) for t in (_abi.MapDesc, _abi.LanesDesc, _abi.FrameOut, _abi.OverlayDesc, _abi.ActorDesc)]
-    assert sizes[:5] == ours
-    assert sizes[5] == _abi.ABI_VERSION
+    ours = [ctypes.sizeof(t) for t in (_abi.MapDesc, _abi.LanesDesc, _abi.FrameOut, _abi.OverlayDesc, _abi.ActorDesc, _abi.WeaponDesc)]
+    assert sizes[:6] == ours
+    assert sizes[6] == _abi.ABI_VERSION
     assert _abi.LanesDesc().struct_size == ours[1]
 
 

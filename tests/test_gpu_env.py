@@ -18,7 +18,7 @@ def test_step_and_reset_device_matches_oracle_frame_by_frame(oracle):
     _meta, _data, smap, tables = load_fixture("small_midtex_sprites")
     lanes = 5
     env = GraDoomVecEnv(smap, lanes, device="cuda:0", render_mode="rgb_array", episode_timeout=2, sprites=16)
-    cosine = hostmath.cosine_correction("cpu").numpy()
+    cosine = env._renderer._cosine   # the renderer's own table (the GPU's float32 cosines, like its ray tables)
 
     def expected_obs():
         state = env._dynamics.lane_state()

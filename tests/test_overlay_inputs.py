@@ -71,3 +71,36 @@ def test_status_bar_words_match_reference_face_selection():
     for k in range(5):
         assert np.array_equal((owned >> k) & 1, (data["engine_weapons"][:, k + 1] != 0).astype(np.int64))
     assert len(set(words[:, 3].tolist())) > 3                            # several face states are exercised
+
+
+def test_decal_packing_keeps_every_slot_in_paint_order():
+    # engine.py:13756-13829: live impacts in the order they were made (serial), whatever slots they sit in; the packing
+    # has a fixed shape (free slots last, alive word zero) so that nothing has to wait for the device to size it
+    from gradoom_amd import overlay_inputs
+
+    rng = np.random.default_rng(5)
+    lanes, slots, walls = 6, 9, 12
+    serial = rng.permutation(lanes * slots).reshape(lanes, slots).astype(np.int64)
+    serial[rng.random((lanes, slots)) < 0.5] = -1
+    serial[2] = -1                                   # a lane without decals
+    wall = rng.integers(0, walls, (lanes, slots))
+    along = rng.random((lanes, slots)).astype(np.float32)
+    impact_z = rng.random((lanes, slots)).astype(np.float32) * 100
+    style = rng.integers(0, 40, (lanes, slots))
+    portal_walls = rng.integers(-500, 500, (walls, 4)).astype(np.float32)
+    table = overlay_inputs.fine_sine_fixed()
+    state, geom = overlay_inputs.decal_inputs(*(torch.as_tensor(v) for v in (serial, wall, along, impact_z, style, portal_walls)), table)
+    assert state.shape == (lanes, slots, 3) and state.dtype == torch.int32
+    assert geom.shape == (lanes, slots, 4) and geom.dtype == torch.float32
+    for lane in range(lanes):
+        live = [slot for slot in np.argsort(serial[lane], kind="stable") if serial[lane, slot] >= 0]
+        assert state[lane, :, 2].tolist() == [1] * len(live) + [0] * (slots - len(live))
+        for position, slot in enumerate(live):
+            assert int(state[lane, position, 0]) == wall[lane, slot] and int(state[lane, position, 1]) == style[lane, slot]
+            assert float(geom[lane, position, 0]) == along[lane, slot] and float(geom[lane, position, 1]) == impact_z[lane, slot]
+            x1, y1, x2, y2 = portal_walls[wall[lane, slot]]
+            sign = 1.0 if style[lane, slot] // 20 == 0 else -1.0       # the seg runs backwards on sidedef 1
+            direction = np.arctan2(np.float32(sign * (y2 - y1)), np.float32(sign * (x2 - x1)))
+            # the direction goes through the 8192-entry fine-angle table: within one table step of the true cosine / sine
+            assert abs(float(geom[lane, position, 2]) - np.cos(direction)) < 2e-3 and abs(float(geom[lane, position, 3]) - np.sin(direction)) < 2e-3
+    assert overlay_inputs.decal_inputs(*(torch.as_tensor(v[:, :0]) for v in (serial, wall, along, impact_z, style)), torch.as_tensor(portal_walls), table) is None

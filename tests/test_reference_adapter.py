@@ -275,3 +275,63 @@ def test_adapter_draws_the_weapon_and_the_status_bar_from_engine_tensors(monkeyp
     difference = np.abs(obs.cpu().numpy().astype(np.int16) - data["obs_with_hud"].astype(np.int16))
     assert int(difference.max()) <= 1
     adapter.close()
+
+
+@pytest.mark.gpu
+def test_weapon_words_come_from_one_kernel_and_equal_the_reference_selection():
+    from gradoom_amd import overlay_inputs, reference_adapter
+
+    meta, data, _smap, _tables = load_fixture("overlays")
+    overlays = fixture_overlays(meta)
+    to = lambda array: torch.as_tensor(np.ascontiguousarray(array)).to("cuda:0")  # noqa: E731
+    engine = {name: to(data[f"engine_{name}"]) for name in reference_adapter.WEAPON_ARGUMENTS}
+    words, light = overlay_inputs.weapon_state(
+        **engine, weapon_frame_ids=to(overlays["weapon_frame_ids"]), weapon_flash_ids=to(overlays["weapon_flash_ids"]),
+        weapon_flash_lights=to(overlays["weapon_flash_lights"]), fine_sine=to(overlay_inputs.fine_sine_fixed()), want_flash_light=True,
+    )
+    assert words.device.type == "cuda" and words.dtype == torch.int64
+    assert np.array_equal(words.cpu().numpy(), data["weapon_state"])            # what the reference frames were checked with
+    assert np.array_equal(words[:, 0].cpu().numpy(), data["ref_weapon_frame_id"])
+    assert np.array_equal(words[:, 1].cpu().numpy(), data["ref_weapon_flash_id"])
+    assert np.array_equal(light.cpu().numpy(), data["flash_light"])             # engine.py:14949-14967, third result
+
+
+@pytest.mark.gpu
+def test_an_adapter_step_never_waits_for_the_device():
+    # the per-lane inputs (ray tables, weapon and status bar words, wall decals) are built by kernels and Torch ops that
+    # leave the host alone: with synchronisation reported as an error, a whole step still goes through
+    from gradoom_amd import reference_adapter
+
+    meta, data, smap, _tables = load_fixture("overlays")
+    overlays = fixture_overlays(meta)
+    engine = stored_engine(data, device="cuda:0", overlays=overlays)
+    engine.map.native_weapon_flash_lights = torch.as_tensor(overlays["weapon_flash_lights"]).to("cuda:0")
+    lanes, slots = engine.num_envs, 6
+    rng = np.random.default_rng(9)
+    engine.hitscan_decal_serial = torch.as_tensor(np.where(rng.random((lanes, slots)) < 0.5, -1, rng.permutation(lanes * slots).reshape(lanes, slots))).to("cuda:0")
+    engine.hitscan_decal_wall = torch.as_tensor(rng.integers(0, len(smap.wall_segments), (lanes, slots))).to("cuda:0")
+    engine.hitscan_decal_along = torch.as_tensor(rng.random((lanes, slots)).astype(np.float32)).to("cuda:0")
+    engine.hitscan_decal_z = torch.as_tensor((rng.random((lanes, slots)) * 80).astype(np.float32)).to("cuda:0")
+    engine.hitscan_decal_style = torch.as_tensor(rng.integers(0, 40, (lanes, slots))).to("cuda:0")
+    engine.map.portal_walls = torch.as_tensor(smap.wall_segments).to("cuda:0")
+    decal_patches = dict(
+        bullet_decal_atlas=overlays["decal_atlas"], bullet_decal_heights=overlays["decal_h"], bullet_decal_left_offsets=overlays["decal_left"],
+        bullet_decal_top_offsets=overlays["decal_top"], bullet_decal_opacity_lut=overlays["decal_opacity_lut"],
+        bullet_decal_black_lut=overlays["decal_black_lut"],
+    )
+    adapter = reference_adapter.HipReferenceRenderer(engine, compiled_scenario(smap, overlays, **decal_patches))
+    assert adapter._has_decals
+    adapter.finish_observation()            # first call: whatever is built lazily
+    torch.cuda.synchronize()
+    before = engine.frames.clone()
+    torch.cuda.set_sync_debug_mode("error")
+    try:
+        adapter.finish_observation()
+        state = adapter.lane_state(include_hud=True)
+    finally:
+        torch.cuda.set_sync_debug_mode("default")
+    torch.cuda.synchronize()
+    assert state.decal_state.shape == (lanes, slots, 3) and state.flash_light.dtype == torch.int64
+    assert torch.equal(engine.frames[:, 3], before[:, 3]) and torch.equal(engine.frames[:, 2], before[:, 3])
+    assert adapter.renderer.status() == 0
+    adapter.close()
