@@ -2424,6 +2424,7 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
         const bool sil_bottom = folds && ((r.view_floor > r.other_floor) || (L.view_z < r.other_floor) || masked_texture);
         const bool sil_top = folds && ((r.view_ceiling < r.other_ceiling) || (L.view_z > r.other_ceiling) || masked_texture);
         const unsigned clip_word = (unsigned)(wi + 1);
+        int ceiling_rows_end = 0; bool ceiling_claims = false;
         {
             const bool claims = r.bits & PB_MARK_CEILING;
             const bool bare = !claims && sil_top && upper_on && (r.side_tex[2] >= 0);   // the upper tier lowers the clip past these rows
@@ -2437,7 +2438,9 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
                 if (y < first || y >= last) continue;
                 pb.m(y) = word;
                 if (sil_top) pb.d(y) = r.distance;
-            }
+                ceiling_rows_end = last; ceiling_claims = claims;
+        }
+            ceiling_rows_end = last; ceiling_claims = claims;
         }
         {
             const bool claims = r.bits & PB_MARK_FLOOR;
@@ -2449,6 +2452,17 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
                 if (y < first || y >= last) continue;
                 pb.m(y) = word;
                 if (sil_bottom) pb.d(y) = r.distance;
+            }
+            // A sector whose ceiling lies below its floor: the rows from its floor's row down to its ceiling's row
+            // belong to both runs.  There the floor's claim has the say, the ceiling's stands where the floor makes none,
+            // and the clip is recorded if either silhouette asks for it.
+            if (__any(first < ceiling_rows_end)) {
+                const int both_end = min(last, ceiling_rows_end);
+                const unsigned both = (claims ? (claim | META_FLOOR) : (ceiling_claims ? claim : 0u)) | ((sil_top || sil_bottom) ? clip_word : 0u);
+                for (int y = first; y < both_end; ++y) {
+                    pb.m(y) = both;
+                    if (sil_top || sil_bottom) pb.d(y) = r.distance;
+                }
             }
         }
         // Rows that leave the window without being written: those the upper tier covers but that belong to a lower
@@ -2551,7 +2565,9 @@ __device__ __forceinline__ void pass_paint(const ColumnCtx &cc, const ColumnStat
                     const int t = one_span ? 0 : (lower_span ? 1 : 2);
                     const bool draws = y < t1 && (one_span || lower_span || upper_span) && tier_tex[t] >= 0;
                     if (draws) draw |= 1u << j;
-                    if (group_valid[t] && py >= group_bottom[t]) tail |= 1u << j;
+                    // rows that both tiers cover take the group's shade if either tier's common bottom has been passed
+                    if ((one_span && group_valid[0] && py >= group_bottom[0]) || (lower_span && group_valid[1] && py >= group_bottom[1]) ||
+                        (upper_span && group_valid[2] && py >= group_bottom[2])) tail |= 1u << j;
                     texel[j] = 0;
                     if (draws) {
                         const unsigned tv = (tier_frac[t] >> tier_shift[t]) >> 1;
@@ -4629,8 +4645,6 @@ int validate_map(const gd_map_desc *h) {
     for (int s = 0; s < S; ++s) {
         const float floor_z = h->sector_heights[2 * s], ceiling_z = h->sector_heights[2 * s + 1];
         if (!(floor_z == floor_z) || !(ceiling_z == ceiling_z)) return fail(GD_E_ARG, "sector_heights holds a NaN");
-        if (ceiling_z < floor_z)
-            return fail(GD_E_UNSUPPORTED, "sector " + std::to_string(s) + " has its ceiling below its floor: such sectors are not rendered like the reference");
         if (h->sector_floor_tex[s] < 0 || h->sector_floor_tex[s] >= T || h->sector_ceil_tex[s] < 0 || h->sector_ceil_tex[s] >= T)
             return fail(GD_E_ARG, "a sector's flat names a texture out of range");
     }

@@ -90,12 +90,6 @@ def build_map_tables(smap) -> dict[str, np.ndarray | int]:
         raise ValueError("a map needs at least one linedef and one sector")
     if np.abs(walls).max() >= 16384:
         raise ValueError("map coordinates must stay below 16384 units (16.16 in int32)")
-    heights = np.asarray(smap.sector_heights, dtype=np.float32)
-    if (heights[:, 1] < heights[:, 0]).any():
-        # A sector whose ceiling lies below its floor makes the upper and lower wall tiers and both plane
-        # claims of one column overlap; the traversal kernels order those writes for ceilings at or above
-        # floors only (closed doors, ceiling == floor, are fine).  The reference's maps never hold one.
-        raise ValueError("sector ceilings must not lie below their floors")
 
     # rint(walls * 65536): engine.py:749-751 (float64) and engine.py:10876 (float32) agree
     # whenever the product is exact, which the int32 range check above guarantees only for

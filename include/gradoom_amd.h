@@ -45,7 +45,7 @@ extern "C" {
 #define GD_OK 0
 #define GD_E_ARG (-1)       /* bad argument: null pointer, negative count, size over a limit */
 #define GD_E_HIP (-2)       /* a HIP runtime call failed */
-#define GD_E_UNSUPPORTED (-3) /* the map needs a feature this build does not implement */
+#define GD_E_UNSUPPORTED (-3) /* reserved: a map feature this build does not implement (none at present) */
 
 /*
  * Immutable map, atlases and look-up tables.

@@ -118,18 +118,6 @@ def test_create_refuses_a_descriptor_of_another_header_version(small_tables):
     assert not handle.value
 
 
-def test_create_refuses_a_sector_with_its_ceiling_below_its_floor(small_tables):
-    from gradoom_amd import _lib
-
-    tables = dict(small_tables)
-    heights = tables["sector_heights"].copy()
-    heights[3, 1] = heights[3, 0] - 16.0
-    tables["sector_heights"] = heights
-    lib, desc, keep, cosine, handle = _create(tables)
-    with pytest.raises(NotImplementedError, match="ceiling below its floor"):
-        _lib.check(lib.gd_renderer_create(ctypes.byref(desc), cosine.ctypes.data, 4, ctypes.byref(handle)))
-
-
 @pytest.mark.parametrize(
     "field, index, value, message",
     [

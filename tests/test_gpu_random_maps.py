@@ -110,9 +110,10 @@ def test_random_maps_with_other_heights_and_textures_whatever_the_working_memory
         renderer.close()
 
 
-def closed_door_case(seed: int, lanes: int):
-    """random_case plus hand-closed doors and crawl spaces on up to four sectors, then (seven times in ten) other heights,
-    texture sizes and lights over the whole map."""
+def closed_door_case(seed: int, lanes: int, *, inverted: bool = False, variants: bool = True, eye_any: bool = False):
+    """random_case plus hand-closed doors and crawl spaces on up to four sectors (``inverted``: ceilings 16 units below
+    their floors instead), then (``variants``: seven times in ten) other heights, texture sizes and lights over the whole
+    map; ``eye_any``: six times in ten the eyes stand at any height, not between their sector's floor and ceiling."""
     from gradoom_amd import mapbuild, synthmap
     from gradoom_amd.selfcheck import make_lane_arrays
 
@@ -123,12 +124,15 @@ def closed_door_case(seed: int, lanes: int):
     if rng.random() < 0.7:
         heights = np.array(smap.sector_heights, copy=True)
         for sector in rng.choice(len(heights), size=min(4, len(heights)), replace=False):
-            if int(rng.choice([0, 2])) == 0:
+            kind = int(rng.choice([0, 2]))
+            if inverted:
+                heights[sector, 1] = heights[sector, 0] - 16   # a ceiling below its floor
+            elif kind == 0:
                 heights[sector, 1] = heights[sector, 0]        # a closed door
             else:
                 heights[sector, 0] = heights[sector, 1] - 8    # a crawl space
         smap.sector_heights[...] = heights
-    if rng.random() < 0.7:
+    if variants and rng.random() < 0.7:
         smap = synthmap.with_variant(smap, seed + 9, heights=[None, "uniform", "doors"][int(rng.integers(0, 3))],
                                      textures=[None, "mixed", "npot"][int(rng.integers(0, 3))], lights=bool(rng.random() < 0.5))
     if rng.random() < 0.4:
@@ -136,7 +140,8 @@ def closed_door_case(seed: int, lanes: int):
     if rng.random() < 0.5:
         smap = synthmap.with_blend_tables(smap, seed + 2)
     margin = float(rng.choice([0.005, 0.02, 0.15]))
-    poses = synthmap.generate_poses(smap, lanes, seed + 3, pitch=bool(rng.random() < 0.6), flash=bool(rng.random() < 0.5), margin=margin)
+    eye = {"eye": "any"} if eye_any and rng.random() < 0.6 else {}
+    poses = synthmap.generate_poses(smap, lanes, seed + 3, pitch=bool(rng.random() < 0.6), flash=bool(rng.random() < 0.5), margin=margin, **eye)
     if rng.random() < 0.3:
         poses.pitch_bam[:] = rng.integers(-30, 31, lanes) * (182 << 16)
     sprites = synthmap.generate_sprites(smap, lanes, 24, seed + 4)
@@ -161,6 +166,38 @@ def test_rows_that_only_a_portal_path_clip_closes_show_the_flat_picture(oracle, 
     renderer = HipRenderer(smap, lanes, "cuda:0", cosine_correction=cosine, tables=tables)
     state = LaneState.from_numpy(arrays, "cuda:0")
     for fill, assembly in ((None, "separate"), (0xA5, "fused"), (0xFF, "separate")):
+        renderer.set_assembly(assembly)
+        if fill is not None:
+            renderer.scribble(fill)
+        indexed = torch.zeros((lanes, 240, 320), dtype=torch.uint8, device="cuda:0")
+        obs = torch.zeros((lanes, 84, 84), dtype=torch.uint8, device="cuda:0")
+        renderer.render(state, indexed=indexed, obs=obs)
+        torch.cuda.synchronize()
+        assert renderer.status() == 0
+        assert np.array_equal(indexed.cpu().numpy(), expected["indexed"]), f"seed {seed} fill {fill} {assembly}"
+        assert np.array_equal(obs.cpu().numpy(), expected["obs"]), f"seed {seed} fill {fill} {assembly}"
+    renderer.close()
+
+
+@pytest.mark.parametrize("seed, variants, eye_any", [(70017, False, False), (70034, False, False), (70047, False, False), (80127, True, True),
+                                                    (80300, True, True), (80301, True, True), (80302, True, True), (80303, True, True)])
+def test_sectors_with_ceilings_below_their_floors_match_the_oracle(oracle, seed, variants, eye_any):
+    """Up to four sectors per map with the ceiling 16 units below the floor.  Seen from a neighbour, such a sector's upper
+    and lower tier share rows: the lower tier paints them, and they take the four-column group's shade as soon as EITHER
+    tier's common bottom row is passed (engine.py:12688-12761; seeds 70017, 70034, 70047).  Seen from inside, the ceiling's
+    and the floor's plane rows overlap: the floor's claim has the say, the ceiling's stands where the floor makes none, and
+    either silhouette records the sprite clip (engine.py:12637-12687, 12943-12964; seed 80127)."""
+    from gradoom_amd import hostmath
+    from gradoom_amd.renderer import HipRenderer, LaneState
+
+    lanes = 16
+    cosine = hostmath.cosine_correction("cpu").numpy()
+    smap, tables, arrays = closed_door_case(seed, lanes, inverted=True, variants=variants, eye_any=eye_any)
+    assert (smap.sector_heights[:, 1] < smap.sector_heights[:, 0]).any() or seed >= 80300
+    expected = oracle.render(tables, arrays, cosine)
+    renderer = HipRenderer(smap, lanes, "cuda:0", cosine_correction=cosine, tables=tables)
+    state = LaneState.from_numpy(arrays, "cuda:0")
+    for fill, assembly in ((None, "separate"), (0x5A, "fused")):
         renderer.set_assembly(assembly)
         if fill is not None:
             renderer.scribble(fill)

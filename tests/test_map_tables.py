@@ -184,13 +184,14 @@ def test_split_tables_hold_only_linedefs_whose_fragments_differ_from_the_linedef
         mapbuild.build_map_tables(dataclasses.replace(smap, wall_projection_fragments_fixed=np.zeros((48, 1, 4), np.int64)))
 
 
-def test_a_sector_with_its_ceiling_below_its_floor_is_refused():
-    """Closed doors (ceiling == floor) build; an inverted sector is outside the renderer's domain and must say so."""
+def test_closed_doors_and_ceilings_below_floors_build():
+    """The reference puts no order on a sector's two heights (``scenario.py:302-401``): closed doors (ceiling == floor)
+    and ceilings below floors build, and each height finds its own plane level."""
     from gradoom_amd import mapbuild, synthmap
 
     smap = synthmap.generate_map(5, grid=(3, 3), sectors=8, linedefs=80, layout="grid", islands=2, pillars=1)
     smap.sector_heights[2, 1] = smap.sector_heights[2, 0]
     mapbuild.build_map_tables(smap)
     smap.sector_heights[2, 1] = smap.sector_heights[2, 0] - 16
-    with pytest.raises(ValueError, match="ceilings must not lie below"):
-        mapbuild.build_map_tables(smap)
+    tables = mapbuild.build_map_tables(smap)
+    assert smap.sector_heights[2, 1] in tables["ceil_levels"] and smap.sector_heights[2, 0] in tables["floor_levels"]
