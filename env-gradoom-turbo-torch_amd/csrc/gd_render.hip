@@ -49,7 +49,14 @@ typedef unsigned long long u64;
 
 #define SW 320
 #define VH 208
-#define CAND_MAX 64          // candidate linedefs kept per screen column
+#define CAND_MAX 64          // candidate linedefs a screen column keeps in its own slots
+// A column whose ray can reach more than CAND_MAX linedefs (a long corridor seen end on) gets a slot in the chunk's spill
+// pool, where cand_spill_kernel lists all of them, up to SPILL_DEPTH.  The pool continues the candidate blocks with
+// the same layout (entry k of a column lies k * 320 entries on), SPILL_DEPTH x 320 entries per pool block, so a
+// spilled column differs from the others only in where its list starts and how long it may be.
+#define SPILL_DEPTH 256
+#define SPILL_SHIFT 12       // cand_count of a spilled column: entries | (pool slot + 1) << SPILL_SHIFT
+static_assert(SPILL_DEPTH < (1 << SPILL_SHIFT), "a spilled column's count and its pool slot share a word");
 #define SEG_COLS 64           // columns of a traversal segment; a wavefront takes 64 / SEG_COLS segments, of any lanes
 #define SEGS_PER_LANE (SW / SEG_COLS)
 #define GD_INF __builtin_inff()
@@ -166,8 +173,13 @@ struct Scratch {    // per-chunk working memory, sized at create
     WallRec *frag_rec;     // [L,split_count,fragment_slots] FWallCoords of the BSP fragments of split linedefs
     float *scene_depth;    // [L,208,320] depth of the surface each pixel shows (engine.py:11553, 12700, 13411, 13740),
                            // kept only for frames that draw wall decals, else null
-    Cand *cand;            // [L,CAND_MAX,320]
-    int *cand_count;       // [L,320] (may exceed CAND_MAX when a list overflowed)
+    Cand *cand;            // [L,CAND_MAX,320], then the spill pool [spill_slots / 320, SPILL_DEPTH, 320]
+    int *cand_count;       // [L,320] entries listed (beyond CAND_MAX: the column wanted more than its own slots hold), or for
+                           // a column with a pool slot: entries in the pool | (slot + 1) << SPILL_SHIFT
+    int *spill_columns;    // [spill_slots] the columns (lane * 320 + column) that were given pool slots, in slot order
+    int *spill_count;      // [1] columns that asked for a slot (cleared by lane_setup_kernel, counted by strip_key_kernel)
+    unsigned spill_base;   // where the pool starts in `cand`, in entries
+    int spill_slots;       // pool slots of this chunk (a multiple of 320)
     unsigned short *flat_sector;// [L,208,320]
     unsigned char *flat_flags;  // [L,208,320] bit0 unresolved
     int *flat_list;        // [L,FLAT_LIST_MAX] view pixels no wall tier, plane or masked texture covers: they show the
@@ -572,7 +584,7 @@ __global__ void lane_setup_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_ba
     int *span = sc.flat_span + (size_t)local * 4;
     span[0] = VH; span[1] = -1; span[2] = VH; span[3] = -1;
     sc.flat_list_count[local] = 0;
-    if (local == 0) { *sc.flat_row_count = 0; *sc.gap_column_count = 0; }
+    if (local == 0) { *sc.flat_row_count = 0; *sc.gap_column_count = 0; *sc.spill_count = 0; }
 }
 
 __device__ __forceinline__ void ray_direction(const LaneCtx &c, int x, float *rx, float *ry) {
@@ -659,6 +671,14 @@ __global__ void fragment_setup_kernel(DeviceMap dm, int lane_count, Scratch sc) 
     wall_coords(sc.ctx[local], m->split_fragments_fixed + 4 * (size_t)k, r);
     r.pl = 0; r.pr = 0; r.flags = 0;
     sc.frag_rec[(size_t)local * per_lane + k] = r;
+}
+
+// A column that was offered more entries than its own slots hold asks for a slot in the spill pool.  With the pool
+// used up the column keeps its first CAND_MAX entries and the renderer's status says so.
+__device__ __forceinline__ void request_spill_slot(const Scratch &sc, int column) {
+    const int slot = atomicAdd(sc.spill_count, 1);
+    if (slot < sc.spill_slots) sc.spill_columns[slot] = column;
+    else atomicOr(sc.status, STATUS_CAND_OVERFLOW);
 }
 
 // One thread owns one linedef for the per-linedef arithmetic.  The two per-column loops have
@@ -909,9 +929,7 @@ __global__ void __launch_bounds__(SETUP_WALLS) wall_setup_kernel(DeviceMap dm, i
                 entry.flags = (unsigned short)(e.flags | ((b_span & 0x200) ? CF_MASKED : 0));
                 entry.dist = e.dist;
                 list[(size_t)slot * SW + x] = entry;
-            } else {
-                atomicOr(sc.status, STATUS_CAND_OVERFLOW);
-            }
+            }   // else: the count says so, and the column is listed afresh in the spill pool (strip_key_kernel, cand_spill_kernel)
         }
     };
     shared_turns(listed && (a_hi - a_lo <= 8), 8);
@@ -937,11 +955,55 @@ __global__ void __launch_bounds__(SETUP_WALLS) wall_setup_kernel(DeviceMap dm, i
                     entry.flags = (unsigned short)(e.flags | ((b_span & 0x200) ? CF_MASKED : 0));
                     entry.dist = e.dist;
                     list[(size_t)slot * SW + x] = entry;
-                } else {
-                    atomicOr(sc.status, STATUS_CAND_OVERFLOW);
                 }
             }
         }
+    }
+}
+
+// The candidate list of every column that was given a spill slot, written afresh into the pool: one wavefront per
+// column tests the column's ray against every linedef of the map (eval_wall: the same test, on the same per-linedef
+// facts, that entered the linedef in wall_setup_kernel) and keeps those with a finite distance, in linedef order.
+// A fixed, small grid: the kernel is launched every frame and nearly always finds no column to do.
+#define SPILL_BLOCKS 1024
+__global__ void __launch_bounds__(64) cand_spill_kernel(DeviceMap dm, Scratch sc) {
+    const gd_map_desc *m = &dm.d;
+    const int wanted = *sc.spill_count;
+    const int total = wanted < sc.spill_slots ? wanted : sc.spill_slots;
+    const int walls = m->wall_count;
+    for (int slot = blockIdx.x; slot < total; slot += gridDim.x) {
+        const int column = sc.spill_columns[slot];
+        const int local = column / SW, x = column - local * SW;
+        const LaneCtx &c = sc.ctx[local];
+        float rx, ry; ray_direction(c, x, &rx, &ry);
+        const RecSpan *spans = sc.span + (size_t)local * walls;
+        Cand *list = sc.cand + sc.spill_base + ((size_t)(slot / SW) * SPILL_DEPTH * SW + (size_t)(slot % SW));
+        int listed = 0;
+        for (int w0 = 0; w0 < walls; w0 += 64) {
+            const int w = w0 + (int)threadIdx.x;
+            bool keep = false;
+            Cand entry;
+            if (w < walls) {
+                const Eval e = eval_wall(m, c, spans, x, w, rx, ry);
+                keep = finitef(e.dist);
+                const int s1 = m->wall_sectors[2 * w + 1];
+                const bool front_facing = (spans[w].flags & WF_FF) != 0;
+                const bool masked_side = s1 >= 0 && m->side_tex[(w * 2 + (front_facing ? 0 : 1)) * 3] >= 0;
+                entry.wall = (unsigned short)w;
+                entry.s0 = (short)m->wall_sectors[2 * w]; entry.s1 = (short)s1;
+                entry.v0 = (unsigned short)m->wall_vertex[2 * w]; entry.v1 = (unsigned short)m->wall_vertex[2 * w + 1];
+                entry.flags = (unsigned short)(e.flags | (masked_side ? CF_MASKED : 0));
+                entry.dist = e.dist;
+            }
+            const u64 keeps = __ballot(keep);
+            const int position = listed + __popcll(keeps & ((1ULL << threadIdx.x) - 1ULL));
+            if (keep) {
+                if (position < SPILL_DEPTH) list[(size_t)position * SW] = entry;
+                else atomicOr(sc.status, STATUS_CAND_OVERFLOW);
+            }
+            listed += __popcll(keeps);
+        }
+        if (threadIdx.x == 0) sc.cand_count[column] = (listed < SPILL_DEPTH ? listed : SPILL_DEPTH) | ((slot + 1) << SPILL_SHIFT);
     }
 }
 
@@ -1712,6 +1774,21 @@ struct ColumnCtx {
     int x;
     float rx, ry;
     __device__ __forceinline__ const WallRec &rec(int w) const { return recs[rec_base + (unsigned)w]; }
+    // Where the list of column `x` of the chunk's lane `local` starts and how many entries it has: the column's own
+    // slots, or its slot in the spill pool.
+    __device__ __forceinline__ void set_list(const Scratch &sc, int local, int column) {
+        list = sc.cand;
+        const int listed = sc.cand_count[(size_t)local * SW + column];
+        const unsigned spill = (unsigned)listed >> SPILL_SHIFT;
+        if (spill) {
+            const unsigned slot = spill - 1;
+            list_column = (sc.spill_base + (slot / SW) * (unsigned)(SPILL_DEPTH * SW) + slot % SW) * 16u;
+            count = listed & ((1 << SPILL_SHIFT) - 1);
+        } else {
+            list_column = ((unsigned)local * (CAND_MAX * SW) + (unsigned)column) * 16u;
+            count = listed < CAND_MAX ? listed : CAND_MAX;
+        }
+    }
     __device__ __forceinline__ Cand cand(int k) const {
         union { uint4 raw; Cand c; } u;
         u.raw = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(list) + (list_column + (unsigned)k * (SW * 16u)));   // one 16-byte load
@@ -2099,6 +2176,8 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
     Eval cwi;
     // List positions of the candidates incident to the current sector and beyond previous_distance: the later
     // scans of this pass ask for both (and more), so they only visit these.  Without a current sector: all.
+    // Bit b stands for the positions b, b + 64, b + 128, ... of a list longer than 64 (a spilled column's): the later
+    // scans test every candidate they visit again, so a bit that also names candidates outside the set costs a look.
     u64 incident_beyond = cc.count >= 64 ? ~0ULL : ((1ULL << cc.count) - 1);
     if (cs >= 0) {
         incident_beyond = 0;
@@ -2114,7 +2193,7 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
                 if (k0 + j >= cc.count) continue;
                 const Cand q = batch[j];
                 if (!(incident_c(q) && q.dist > prev)) continue;
-                incident_beyond |= 1ULL << (k0 + j);
+                incident_beyond |= 1ULL << ((k0 + j) & 63);
                 if (q.dist < distance || (q.dist == distance && (int)q.wall < wi)) { distance = q.dist; wi = q.wall; wi_flags = q.flags; }
                 if ((q.s1 < 0) && (q.dist < sd || (q.dist == sd && (int)q.wall < swi))) { sd = q.dist; swi = q.wall; swi_flags = q.flags; }
             }
@@ -2143,17 +2222,21 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
     bool ps_path_geo = cwi.flags & CF_GEO;
     float psd = GD_INF; int psi = 0x7fffffff; int psi_flags = 0;
     if (!sel_is_proj) {
+        auto solid_owner = [&](const Cand &q) {
+            bool owner = incident_c(q) && (q.s1 < 0) && (q.flags & CF_PROJ) && (q.flags & CF_LEDGE) && shares_sel_c(q) && (q.dist > prev_eps);
+            if (owner && (q.dist < psd || (q.dist == psd && (int)q.wall < psi))) { psd = q.dist; psi = q.wall; psi_flags = q.flags; }
+        };
         for (u64 rest = incident_beyond; rest;) {
             Cand batch[CAND_BATCH]; int at[CAND_BATCH];
             cc.cand_batch_of(rest, batch, at);
 #pragma unroll
             for (int j = 0; j < CAND_BATCH; ++j) {
                 if (at[j] < 0) continue;
-                const Cand q = batch[j];
-                bool owner = incident_c(q) && (q.s1 < 0) && (q.flags & CF_PROJ) && (q.flags & CF_LEDGE) && shares_sel_c(q) && (q.dist > prev_eps);
-                if (owner && (q.dist < psd || (q.dist == psd && (int)q.wall < psi))) { psd = q.dist; psi = q.wall; psi_flags = q.flags; }
+                solid_owner(batch[j]);
             }
         }
+        for (int k = 64; k < cc.count; ++k)   // a spilled column's further entries
+            if ((incident_beyond >> (k & 63)) & 1ULL) solid_owner(cc.cand(k));
         if (sel_excl_right) {
             const int *ofs = sel_start ? m->solid_bridge_start_ofs : m->solid_bridge_end_ofs;
             const int *idx = sel_start ? m->solid_bridge_start_idx : m->solid_bridge_end_idx;
@@ -2190,24 +2273,28 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
     float npd = GD_INF; int npi = 0x7fffffff; int npi_flags = 0;
     const int so_s0 = mv.sec(wi, 0), so_s1 = mv.sec(wi, 1);
     if (!so_is_proj) {
+        auto near_owner = [&](const Cand &q) {
+            int w = q.wall;
+            if (!(incident_c(q) && (q.s1 >= 0) && (q.flags & CF_PROJ) && (q.dist > prev_eps))) return;
+            bool le = q.flags & CF_LEDGE;
+            bool same_pair = (q.s0 == so_s0 && q.s1 == so_s1) || (q.s0 == so_s1 && q.s1 == so_s0);
+            bool close = (same_pair || (le && so_excl_right && ((so_span <= 2) || (shares_sel_c(q) && so_short)))) &&
+                         (fabsf(q.dist - distance) <= tolerance_of(q.dist));
+            bool topo = false;
+            if (!close && le && so_excl_right && so_span <= 2) { int dummy; topo = mv.sector_bridge((q.flags & CF_ALONG_HI) ? 1 : 0, w, no_path_index, &dummy); }
+            if ((close || topo) && (q.dist < npd || (q.dist == npd && w < npi))) { npd = q.dist; npi = w; npi_flags = q.flags; }
+        };
         for (u64 rest = incident_beyond; rest;) {
             Cand batch[CAND_BATCH]; int at[CAND_BATCH];
             cc.cand_batch_of(rest, batch, at);
 #pragma unroll
             for (int j = 0; j < CAND_BATCH; ++j) {
                 if (at[j] < 0) continue;
-                const Cand q = batch[j];
-                int w = q.wall;
-                if (!(incident_c(q) && (q.s1 >= 0) && (q.flags & CF_PROJ) && (q.dist > prev_eps))) continue;
-                bool le = q.flags & CF_LEDGE;
-                bool same_pair = (q.s0 == so_s0 && q.s1 == so_s1) || (q.s0 == so_s1 && q.s1 == so_s0);
-                bool close = (same_pair || (le && so_excl_right && ((so_span <= 2) || (shares_sel_c(q) && so_short)))) &&
-                             (fabsf(q.dist - distance) <= tolerance_of(q.dist));
-                bool topo = false;
-                if (!close && le && so_excl_right && so_span <= 2) { int dummy; topo = mv.sector_bridge((q.flags & CF_ALONG_HI) ? 1 : 0, w, no_path_index, &dummy); }
-                if ((close || topo) && (q.dist < npd || (q.dist == npd && w < npi))) { npd = q.dist; npi = w; npi_flags = q.flags; }
+                near_owner(batch[j]);
             }
         }
+        for (int k = 64; k < cc.count; ++k)   // a spilled column's further entries
+            if ((incident_beyond >> (k & 63)) & 1ULL) near_owner(cc.cand(k));
     }
     int pe_wall = c.pend_ep_wall;
     int pe_s0 = mv.sec(pe_wall, 0), pe_s1 = mv.sec(pe_wall, 1);
@@ -2367,6 +2454,20 @@ __device__ __forceinline__ void zero_rows(PixelBuffers &pb, GapRange &gaps, int 
     if (first >= last) return;
     for (int y = first; y < last; ++y) pb.m(y) = 0u;
     gaps.set_zeroed(min(first, gaps.lo()), max(last, gaps.hi()));
+}
+
+// Exchanges inside the aligned groups of four lanes (DPP quads): the value of the group's first lane, and the
+// conjunction, the largest and the smallest of the four.  All four lanes must be executing.
+template <int PATTERN> __device__ __forceinline__ int quad_move(int v) { return __builtin_amdgcn_mov_dpp(v, PATTERN, 0xF, 0xF, true); }
+__device__ __forceinline__ int quad_first(int v) { return quad_move<0x00>(v); }                 // lanes 0,0,0,0
+__device__ __forceinline__ int quad_and(int v) { v &= quad_move<0xB1>(v); return v & quad_move<0x4E>(v); }   // lanes 1,0,3,2 then 2,3,0,1
+__device__ __forceinline__ float quad_max(float v) {
+    v = fmaxf(v, __int_as_float(quad_move<0xB1>(__float_as_int(v))));
+    return fmaxf(v, __int_as_float(quad_move<0x4E>(__float_as_int(v))));
+}
+__device__ __forceinline__ float quad_min(float v) {
+    v = fminf(v, __int_as_float(quad_move<0xB1>(__float_as_int(v))));
+    return fminf(v, __int_as_float(quad_move<0x4E>(__float_as_int(v))));
 }
 
 // Smallest / largest of a small value (0..255) over the lanes that execute the call, found by ballots: usable inside
@@ -2987,7 +3088,7 @@ __global__ void __launch_bounds__(256) strip_key_kernel(int lane_count, Scratch 
     if (local >= lane_count) return;
     const int x = (strip - local * (SW / 64)) * 64 + (threadIdx.x & 63);
     int length = sc.cand_count[(size_t)local * SW + x];
-    if (length > CAND_MAX) length = CAND_MAX;
+    if (length > CAND_MAX) { request_spill_slot(sc, local * SW + x); length = CAND_MAX; }   // cand_spill_kernel runs next
 #pragma unroll
     for (int step = 1; step < SEG_COLS; step <<= 1) length = max(length, __shfl_xor(length, step));
     if ((x & (SEG_COLS - 1)) == 0) sc.strip_key[local * SEGS_PER_LANE + x / SEG_COLS] = (unsigned char)length;   // at most CAND_MAX
@@ -3035,10 +3136,7 @@ __global__ void __launch_bounds__(64 * SELECT_STRIPS_PER_GROUP) wall_select_kern
     cc.recs = sc.rec; cc.spans = sc.span;
     cc.rec_base = (unsigned)local * (unsigned)m->wall_count;
     cc.frags = sc.frag_rec + (size_t)local * m->split_count * m->fragment_slots;
-    cc.list = sc.cand;
-    cc.list_column = ((unsigned)local * (CAND_MAX * SW) + (unsigned)x) * 16u;
-    cc.count = sc.cand_count[(size_t)local * SW + x];
-    if (cc.count > CAND_MAX) cc.count = CAND_MAX;
+    cc.set_list(sc, local, x);
     cc.x = x;
     ray_direction(lane_ctx, x, &cc.rx, &cc.ry);
     ColumnState st;
@@ -3120,10 +3218,7 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
     cc.recs = sc.rec; cc.spans = sc.span;
     cc.rec_base = (unsigned)local * (unsigned)m->wall_count;
     cc.frags = sc.frag_rec + (size_t)local * m->split_count * m->fragment_slots;
-    cc.list = sc.cand;
-    cc.list_column = ((unsigned)local * (CAND_MAX * SW) + (unsigned)x) * 16u;
-    cc.count = sc.cand_count[(size_t)local * SW + x];
-    if (cc.count > CAND_MAX) cc.count = CAND_MAX;
+    cc.set_list(sc, local, x);
     cc.x = x;
     ray_direction(lane_ctx, x, &cc.rx, &cc.ry);
     PixelBuffers pb;
@@ -3147,7 +3242,6 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
     PassColumn pc;
     pc.wall = 0; pc.side = 0; pc.bits = 0; pc.visibility = 0;
     pc.clipped_top = 0.0f; pc.clipped_bottom = 0.0f; pc.clipped_upper_bottom = 0.0f; pc.clipped_lower_top = 0.0f;
-    const int group_base = lane_id & ~3;
     for (int pass = 0; __ballot(pass < passes) != 0; ++pass) {
         const bool mine = pass < passes;
         bool draws = false;
@@ -3165,26 +3259,23 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
         } else {
             pc.bits = 0;   // a finished column draws no tier: its group of four has no common tail
         }
-        // 4-column wallscan groups (engine.py:12688-12761): exchange with the aligned neighbours
-        bool same_group = true;
-        int w0 = __shfl(pc.wall, group_base), s0 = __shfl(pc.side, group_base);
-        bool all_tier[3] = {true, true, true};
-        float common_top[3] = {-GD_INF, -GD_INF, -GD_INF}, common_bottom[3] = {GD_INF, GD_INF, GD_INF};
-        for (int k = 0; k < 4; ++k) {
-            int src = group_base + k;
-            int qw = __shfl(pc.wall, src), qs = __shfl(pc.side, src), qb = __shfl(pc.bits, src);
-            float qt = __shfl(pc.clipped_top, src), qlt = __shfl(pc.clipped_lower_top, src);
-            float qbm = __shfl(pc.clipped_bottom, src), qub = __shfl(pc.clipped_upper_bottom, src);
-            same_group &= (qw == w0) && (qs == s0);
-            all_tier[0] &= (qb & PB_TIER0) != 0; all_tier[1] &= (qb & PB_TIER1) != 0; all_tier[2] &= (qb & PB_TIER2) != 0;
-            common_top[0] = fmaxf(common_top[0], qt); common_top[1] = fmaxf(common_top[1], qlt); common_top[2] = fmaxf(common_top[2], qt);
-            common_bottom[0] = fminf(common_bottom[0], qbm); common_bottom[1] = fminf(common_bottom[1], qbm); common_bottom[2] = fminf(common_bottom[2], qub);
-        }
-        int vis_lo = __shfl((int)(pc.visibility & 0xFFFFFFFFLL), group_base);
-        int vis_hi = __shfl((int)(pc.visibility >> 32), group_base);
-        i64 first_group_visibility = ((i64)vis_hi << 32) | (i64)(unsigned)vis_lo;
+        // 4-column wallscan groups (engine.py:12688-12761): the aligned group of four columns agrees on its drawseg, on
+        // which tiers all four draw and on the rows all four share.  The four lanes of a group are one DPP quad, so every
+        // exchange is a vector move with a lane pattern (no trip through the LDS crossbar), and the minima, maxima and
+        // conjunctions take two steps each.  Every lane of the wavefront is active here.
+        const int w0 = quad_first(pc.wall), s0 = quad_first(pc.side);
+        const int GROUP_AGREES = 0x1;   // takes PB_VALID's place in the word that is and-ed over the group
+        const int agreed = quad_and((pc.bits & (PB_TIER0 | PB_TIER1 | PB_TIER2)) | ((pc.wall == w0 && pc.side == s0) ? GROUP_AGREES : 0));
+        const bool same_group = (agreed & GROUP_AGREES) != 0;
+        // a value that is not a number never becomes a common top or bottom (std::max(-inf, nan) is -inf)
+        const float shared_top = fmaxf(-GD_INF, quad_max(pc.clipped_top)), shared_lower_top = fmaxf(-GD_INF, quad_max(pc.clipped_lower_top));
+        const float shared_bottom = fminf(GD_INF, quad_min(pc.clipped_bottom)), shared_upper_bottom = fminf(GD_INF, quad_min(pc.clipped_upper_bottom));
+        const float common_bottom[3] = {shared_bottom, shared_bottom, shared_upper_bottom};
+        const i64 first_group_visibility = ((i64)quad_first((int)(pc.visibility >> 32)) << 32) | (i64)(unsigned)quad_first((int)(pc.visibility & 0xFFFFFFFFLL));
         bool group_valid[3];
-        for (int t = 0; t < 3; ++t) group_valid[t] = same_group && all_tier[t] && (common_top[t] < common_bottom[t]);
+        group_valid[0] = same_group && (agreed & PB_TIER0) && (shared_top < shared_bottom);
+        group_valid[1] = same_group && (agreed & PB_TIER1) && (shared_lower_top < shared_bottom);
+        group_valid[2] = same_group && (agreed & PB_TIER2) && (shared_top < shared_upper_bottom);
         if (draws) {
             pass_paint<DEPTH>(cc, st, pc, pb, group_valid, common_bottom, first_group_visibility, colormap_lds, window_dirty, gaps);
             pass_advance<SPLIT, ADVANCE_CLIPS>(cc, st, pc, pb, sb, !window_dirty, gaps);
@@ -4499,11 +4590,19 @@ __global__ void fill_words_kernel(unsigned int *words, size_t count, unsigned in
     for (size_t k = (size_t)blockIdx.x * blockDim.x + threadIdx.x; k < count; k += (size_t)gridDim.x * blockDim.x) words[k] = value;
 }
 
+// Blocks of the spill pool (320 columns each, 1.25 MiB) for a chunk of `lanes` lanes: every column of up to eight
+// lanes, one column in 32 of a large chunk (160 MiB at 4096 lanes).  The static working memory has room for one.
+size_t spill_pool_blocks(int lanes) {
+    const int share = lanes / 32 > 8 ? lanes / 32 : 8;
+    return (size_t)(lanes < share ? lanes : share);
+}
+#define STATIC_SPILL_BLOCKS 1
+
 // Lay the per-chunk buffers of `sc` out in one block of device memory for `L` lanes of map `h` (every buffer
 // 256-byte aligned) and return the bytes the layout takes; with a null `base` nothing is assigned and the call
 // only measures.  `status` is not part of the block: the renderer keeps it.  `depth`: also the scene depth plane
 // of frames that draw decals.
-size_t carve_scratch(Scratch &sc, unsigned char *base, size_t L, const gd_map_desc &h, bool depth) {
+size_t carve_scratch(Scratch &sc, unsigned char *base, size_t L, const gd_map_desc &h, bool depth, size_t spill_blocks) {
     // `depth`: frames that draw decals also need a scene depth plane
     size_t used = 0;
     auto take = [&](auto **field, size_t count) {
@@ -4517,8 +4616,11 @@ size_t carve_scratch(Scratch &sc, unsigned char *base, size_t L, const gd_map_de
     take(&sc.rec, L * W);
     take(&sc.span, L * W);
     take(&sc.frag_rec, L * (size_t)(h.split_count > 0 ? h.split_count * h.fragment_slots : 1));
-    take(&sc.cand, L * CAND_MAX * SW);
+    take(&sc.cand, L * CAND_MAX * SW + spill_blocks * SPILL_DEPTH * SW);   // byte offsets into it are 32 bits wide: L <= 4096, spill_blocks <= 512
+    sc.spill_base = (unsigned)(L * CAND_MAX * SW); sc.spill_slots = (int)(spill_blocks * SW);
     take(&sc.cand_count, L * SW);
+    take(&sc.spill_columns, spill_blocks * SW);
+    take(&sc.spill_count, 1);
     take(&sc.flat_sector, L * PX);
     take(&sc.flat_flags, L * PX);
     take(&sc.flat_span, L * 4);
@@ -4719,6 +4821,8 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     if (m.split_count > 0)
         hipLaunchKernelGGL(fragment_setup_kernel, dim3((m.split_count * m.fragment_slots + 63) / 64, count), dim3(64), 0, stream, r->dm, count, sc);
     hipLaunchKernelGGL(strip_key_kernel, dim3((count * (SW / 64) + 3) / 4), dim3(256), 0, stream, count, sc);
+    if (sc.spill_slots > 0)
+        hipLaunchKernelGGL(cand_spill_kernel, dim3(sc.spill_slots < SPILL_BLOCKS ? sc.spill_slots : SPILL_BLOCKS), dim3(64), 0, stream, r->dm, sc);
     hipLaunchKernelGGL(strip_order_kernel, dim3(1), dim3(1024), 0, stream, count * SEGS_PER_LANE, sc);
     mark();
     {
@@ -4975,10 +5079,10 @@ int gd_renderer_create(const gd_map_desc *h, const float *cosine_correction, int
     Scratch &sc = r->sc;
     if (rc == GD_OK && chunk > 0) {
         unsigned char *block = nullptr;
-        const size_t bytes = carve_scratch(sc, nullptr, (size_t)chunk, *h, false);
+        const size_t bytes = carve_scratch(sc, nullptr, (size_t)chunk, *h, false, spill_pool_blocks(chunk));
         rc = scratch_alloc(r, bytes, &block);
         if (rc == GD_OK) {
-            carve_scratch(sc, block, (size_t)chunk, *h, false);
+            carve_scratch(sc, block, (size_t)chunk, *h, false, spill_pool_blocks(chunk));
             r->scratch_block = block; r->scratch_bytes = bytes;
         }
     }
@@ -5054,17 +5158,17 @@ int gd_render_static(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_
     const gd_map_desc &m = r->dm.d;
     const bool decals = lanes->decal_slots > 0 && lanes->decal_state && lanes->decal_geom && r->overlays.d.decal_variant_count > 0;
     Scratch sc = r->sc;   // keeps the renderer's status word
-    const size_t one = carve_scratch(sc, nullptr, 1, m, decals), two = carve_scratch(sc, nullptr, 2, m, decals);
+    const size_t one = carve_scratch(sc, nullptr, 1, m, decals, STATIC_SPILL_BLOCKS), two = carve_scratch(sc, nullptr, 2, m, decals, STATIC_SPILL_BLOCKS);
     if (one > STATIC_SCRATCH_BYTES)
         return fail(GD_E_ARG, "map too large for gd_render_static: one lane needs " + std::to_string(one) + " bytes of working memory, the static block holds " +
                                   std::to_string(STATIC_SCRATCH_BYTES));
     // the layout grows by a fixed amount per lane, up to the padding between its buffers
     size_t fit = 1 + (STATIC_SCRATCH_BYTES - one) / (two - one);
-    while (fit > 1 && carve_scratch(sc, nullptr, fit, m, decals) > STATIC_SCRATCH_BYTES) --fit;
+    while (fit > 1 && carve_scratch(sc, nullptr, fit, m, decals, STATIC_SPILL_BLOCKS) > STATIC_SCRATCH_BYTES) --fit;
     const int chunk = fit > 4096 ? 4096 : (int)fit;
     if (lanes->lane_count > GD_STATIC_MAX_LANES)
         return fail(GD_E_ARG, "gd_render_static renders at most " + std::to_string(GD_STATIC_MAX_LANES) + " lanes per call");
-    carve_scratch(sc, block, (size_t)chunk, m, decals);
+    carve_scratch(sc, block, (size_t)chunk, m, decals, STATIC_SPILL_BLOCKS);
     hipStream_t caller = static_cast<hipStream_t>(stream);
     // the block keeps whatever the last call left: the kernels expect nothing of it
     for (int base = 0; base < lanes->lane_count; base += chunk) {

@@ -269,7 +269,10 @@ class GraDoomVecEnv:
         return self.signal_buffer
 
     def check_renderer_status(self) -> None:
-        """Raise if the renderer had to drop a linedef from a column's candidate list (it keeps 64 per column).
+        """Raise if the renderer had to drop a linedef from a column's candidate list.
+
+        A column keeps 64 linedefs in its own slots and up to 256 in the spill pool, which holds one column in 32 of a large
+        batch (every column of up to eight lanes).
 
         Such a frame may differ from the reference's, which has no such bound, so it must not pass for a good one.
         Synchronises the device: called where the environment already waits for it.
@@ -278,8 +281,9 @@ class GraDoomVecEnv:
         flags = status() if status is not None else 0
         if flags & 1:
             raise RuntimeError(
-                "the renderer truncated a screen column's candidate list (more than 64 linedefs overlap one column of one "
-                "lane's view): frames of this environment are not trustworthy on this map"
+                "the renderer truncated a screen column's candidate list (more than 256 linedefs overlap one column of one "
+                "lane's view, or more columns than the spill pool holds see more than 64): frames of this environment are "
+                "not trustworthy on this map"
             )
         if flags & 2:
             raise RuntimeError(

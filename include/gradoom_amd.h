@@ -285,7 +285,11 @@ int gd_render_static(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_
 /*
  * Sticky status bits (synchronises the device).  bit0: some screen column had
  * more candidate linedefs than the library keeps and was truncated - the frame
- * of that lane is not trustworthy.  Replaces nothing in the reference.
+ * of that lane is not trustworthy.  A column keeps 64 in its own slots; one
+ * that sees more moves to a spill pool (up to 256 per column; every column of
+ * up to 8 lanes, one column in 32 of a 4096-lane chunk, 320 columns in
+ * gd_render_static).  bit1: a column crossed more than 96 portals.
+ * Replaces nothing in the reference.
  */
 int gd_renderer_status(gd_renderer *r, int32_t *status);
 

@@ -79,13 +79,15 @@ def test_host_api_safe_view_buffers_are_written_by_the_renderer():
         env.close()
 
 
-def test_more_than_64_linedefs_in_one_column_raise_in_the_environment():
-    # A corridor of 80 sectors seen end on: every divider lands in the same screen columns, more than the 64 candidates
-    # the renderer keeps per column.  The environment must say so rather than hand out the frame.
+def test_more_than_256_linedefs_in_one_column_raise_in_the_environment(monkeypatch):
+    # A corridor of 300 narrow sectors seen end on: every divider lands in the same few screen columns, more than the 256
+    # candidates a column can hold in the spill pool (64 in its own slots).  The environment must say so rather than hand
+    # out the frame.
     from gradoom_amd import synthmap
     from gradoom_amd.env import GraDoomVecEnv, PosePoolDynamics
 
-    smap = synthmap.generate_map(5, grid=(80, 1), sectors=80, linedefs=241)
+    monkeypatch.setattr(synthmap, "CELL", 48)   # 300 cells of the usual 256 units would leave the 16.16 coordinate range
+    smap = synthmap.generate_map(5, grid=(300, 1), sectors=300, linedefs=901)
     lanes = 2
     dynamics = PosePoolDynamics(smap, lanes, "cuda:0", pool=4)
     quad = smap.sector_quads[0]

@@ -211,6 +211,52 @@ def test_sectors_with_ceilings_below_their_floors_match_the_oracle(oracle, seed,
     renderer.close()
 
 
+def corridor_case(lanes: int):
+    """A corridor of 80 sectors and cameras in it that look along it, so that every divider lands in the same screen
+    columns: more linedefs per column ray than the 64 a column keeps in its own slots."""
+    from gradoom_amd import mapbuild, synthmap
+    from gradoom_amd.selfcheck import make_lane_arrays
+
+    smap = synthmap.generate_map(5, grid=(80, 1), sectors=80, linedefs=241, midtex=0.2)
+    poses = synthmap.generate_poses(smap, lanes, 11, pitch=True, flash=True)
+    rng = np.random.default_rng(3)
+    for lane in range(lanes):
+        sector = int(rng.integers(0, 8)) if lane % 2 == 0 else int(rng.integers(72, 80))   # either end, looking at the other
+        centre = smap.sector_quads[sector].mean(axis=0)
+        poses.x[lane], poses.y[lane] = float(centre[0]) + float(rng.uniform(-20, 20)), float(centre[1]) + float(rng.uniform(-20, 20))
+        poses.view_z[lane] = float(smap.sector_heights[sector, 0]) + 41.0
+        degrees = (0.0 if lane % 2 == 0 else 180.0) + float(rng.uniform(-12, 12))
+        poses.angle_bam[lane] = int(round(degrees / 360.0 * 4294967296.0)) & 0xFFFFFFFF
+    sprites = synthmap.generate_sprites(smap, lanes, 24, 12)
+    return smap, mapbuild.build_map_tables(smap), make_lane_arrays(smap, poses, sprites)
+
+
+def test_columns_that_see_more_than_64_linedefs_match_the_oracle(oracle):
+    """Such columns get a slot in the spill pool, where every linedef their ray can reach is listed (the reference keeps a
+    dense [columns, linedefs] table, engine.py:11446-11451, and has no limit)."""
+    from gradoom_amd import hostmath
+    from gradoom_amd.renderer import HipRenderer, LaneState
+
+    lanes = 6
+    cosine = hostmath.cosine_correction("cpu").numpy()
+    smap, tables, arrays = corridor_case(lanes)
+    expected = oracle.render(tables, arrays, cosine)
+    renderer = HipRenderer(smap, lanes, "cuda:0", cosine_correction=cosine, tables=tables)
+    state = LaneState.from_numpy(arrays, "cuda:0")
+    for fill, assembly in ((None, "separate"), (0xA5, "fused"), (None, "separate")):
+        renderer.set_assembly(assembly)
+        if fill is not None:
+            renderer.scribble(fill)
+        indexed = torch.zeros((lanes, 240, 320), dtype=torch.uint8, device="cuda:0")
+        obs = torch.zeros((lanes, 84, 84), dtype=torch.uint8, device="cuda:0")
+        renderer.render(state, indexed=indexed, obs=obs)
+        torch.cuda.synchronize()
+        assert renderer.status() == 0
+        assert np.array_equal(indexed.cpu().numpy(), expected["indexed"]), f"fill {fill} {assembly}"
+        assert np.array_equal(obs.cpu().numpy(), expected["obs"]), f"fill {fill} {assembly}"
+    renderer.close()
+
+
 def test_cameras_outside_the_map_match_the_oracle(oracle):
     """Cameras in the void beside the map: no wall pass claims most of the screen, so nearly every pixel shows the
     flat pass's picture (far more than the per-lane gap pixel list holds) and most of them stay unresolved."""
