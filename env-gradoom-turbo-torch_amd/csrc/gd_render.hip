@@ -3972,21 +3972,31 @@ __device__ __forceinline__ void store_stack_word(unsigned char *stack_lane, unsi
     }
 }
 
-// One block per lane and OBS_BLOCK_ROWS observation rows.  The source rows they overlap are staged in LDS with
-// word loads (a byte load per tap keeps the address units busy for 64 lanes each); taps then read LDS.
-#define OBS_BLOCK_ROWS 3
-#define OBS_TILE_ROWS 11   // source rows that OBS_BLOCK_ROWS observation rows can overlap (10), and one to spare
-static_assert(GD_OBS_SIZE % OBS_BLOCK_ROWS == 0 && OBS_BLOCK_ROWS * GD_OBS_SIZE <= 256, "observe_kernel: rows per block");
+// One block per lane and OBS_BLOCK_ROWS = 7 observation rows, which pool exactly OBS_SOURCE_ROWS = 20 frame rows
+// (84 observation rows x 240 / 84 frame rows each).  An observation pixel covers 240/84 frame rows and 320/84 frame
+// columns; its weights (y_overlap * x_overlap) // 48 are exactly (y_overlap / 12) * (x_overlap / 4), since row
+// overlaps are multiples of 12 and column overlaps multiples of 4 (84 = 12 * 7 = 4 * 21, 240 = 12 * 20, 320 = 4 * 80):
+// the weighted sum factors into a pass along the rows and one down the columns, all in integers.  The first pass
+// looks every frame pixel's colour up once per observation column it touches (five taps per frame row and
+// observation column), the second adds four row sums per observation pixel: 10,752 palette taps per block where a
+// pixel-by-pixel pooling takes 11,760, and a tap is a byte load, a palette load and three dot products.
+#define OBS_BLOCK_ROWS 7
+#define OBS_SOURCE_ROWS (OBS_BLOCK_ROWS * GD_SCREEN_HEIGHT / GD_OBS_SIZE)
+static_assert(GD_OBS_SIZE % OBS_BLOCK_ROWS == 0 && OBS_SOURCE_ROWS * GD_OBS_SIZE == OBS_BLOCK_ROWS * GD_SCREEN_HEIGHT, "observe_kernel: seven rows pool twenty");
+static_assert((OBS_BLOCK_ROWS * GD_OBS_SIZE) % 4 == 0 && 3 * GD_OBS_SIZE <= 256, "observe_kernel: whole words, three rows of threads");
 __global__ void __launch_bounds__(256) observe_kernel(const unsigned char *indexed, size_t lane_stride, int source_rows, const unsigned char *playpal,
                                int lane_count, unsigned char *obs, unsigned char *frames, const unsigned char *reset_mask, int stack_mode,
                                unsigned char *final_frames, bool final_hwc, const float *blend) {
     __shared__ unsigned int pal[256];   // PLAYPAL after the lane's screen blend, one word per colour (red | green << 8 | blue << 16)
-    __shared__ unsigned int tile[OBS_TILE_ROWS * (SW / 4)];
+    __shared__ unsigned int tile[OBS_SOURCE_ROWS * (SW / 4)];
+    __shared__ unsigned int along_rg[OBS_SOURCE_ROWS * GD_OBS_SIZE];      // per frame row and observation column: red | green << 16 summed along the row
+    __shared__ unsigned short along_b[OBS_SOURCE_ROWS * GD_OBS_SIZE];     // and blue (each at most 80 * 255)
+    __shared__ unsigned int gray_words[OBS_BLOCK_ROWS * GD_OBS_SIZE / 4];
     int n = blockIdx.y;
     if (n >= lane_count) return;                   // the same in the whole block
     const unsigned char *src = indexed + (size_t)n * lane_stride;
     const int first_row = blockIdx.x * OBS_BLOCK_ROWS;
-    const int tile_first = (first_row * 240) / 84;
+    const int tile_first = blockIdx.x * OBS_SOURCE_ROWS;
     // Everything the block reads from memory is asked for up front (palette entry, tile words, the stack words
     // that the roll keeps), so that the block waits for memory once.
     const size_t F = (size_t)GD_OBS_SIZE * GD_OBS_SIZE / 4;     // words per observation
@@ -4012,58 +4022,66 @@ __global__ void __launch_bounds__(256) observe_kernel(const unsigned char *index
     }
     {
         const bool aligned = (reinterpret_cast<size_t>(src) & 3) == 0;
-        for (int k = threadIdx.x; k < OBS_TILE_ROWS * (SW / 4); k += blockDim.x) {
+        for (int k = threadIdx.x; k < OBS_SOURCE_ROWS * (SW / 4); k += blockDim.x) {
             const int r = k / (SW / 4), c = k - r * (SW / 4);
-            tile[k] = load_word(src + (size_t)min(tile_first + r, source_rows - 1) * SW + 4 * c, aligned);
+            tile[k] = load_word(src + (size_t)min(tile_first + r, source_rows - 1) * SW + 4 * c, aligned);   // rows past the source weigh nothing below
         }
     }
     __syncthreads();
-    __shared__ unsigned int gray_words[OBS_BLOCK_ROWS * GD_OBS_SIZE / 4];
-    const int row_in_block = min((int)threadIdx.x / GD_OBS_SIZE, OBS_BLOCK_ROWS - 1);   // the last few threads only help staging
-    const int oy = first_row + row_in_block, ox = min((int)threadIdx.x - row_in_block * GD_OBS_SIZE, GD_OBS_SIZE - 1);
+    // three rows of 84 threads: thread (slot, ox) takes observation column ox of every third row
+    const int slot = min((int)threadIdx.x / GD_OBS_SIZE, 2), ox = min((int)threadIdx.x - slot * GD_OBS_SIZE, GD_OBS_SIZE - 1);
+    const bool works = threadIdx.x < 3 * GD_OBS_SIZE;
     const unsigned char *staged = reinterpret_cast<const unsigned char *>(tile);
-    int y_start = oy * 240, y_end = y_start + 240, x_start = ox * 320, x_end = x_start + 320;
-    int rs = 0, gs = 0, bs = 0;
-    // up to 4 x 5 source pixels overlap one observation pixel; all of them are loaded first (taps
-    // outside the overlap read a clamped address and weigh nothing), then accumulated
-    int y_overlap[4], x_overlap[5], row_offset[4], column[5];
-#pragma unroll
-    for (int sy = 0; sy < 4; ++sy) {
-        const int source_y = y_start / 84 + sy;
-        const int overlap = min(y_end, (source_y + 1) * 84) - max(y_start, source_y * 84);
-        y_overlap[sy] = (source_y >= source_rows || overlap <= 0) ? 0 : overlap;
-        row_offset[sy] = min(source_y - tile_first, OBS_TILE_ROWS - 1) * SW;   // rows past the tile weigh nothing
-    }
-#pragma unroll
-    for (int sx = 0; sx < 5; ++sx) {
-        const int source_x = x_start / 84 + sx;
-        const int overlap = min(x_end, (source_x + 1) * 84) - max(x_start, source_x * 84);
-        x_overlap[sx] = (source_x >= SW || overlap <= 0) ? 0 : overlap;
-        column[sx] = min(source_x, SW - 1);
-    }
-    unsigned char tap[4][5];
-#pragma unroll
-    for (int sy = 0; sy < 4; ++sy)
-#pragma unroll
-        for (int sx = 0; sx < 5; ++sx) tap[sy][sx] = staged[row_offset[sy] + column[sx]];
-#pragma unroll
-    for (int sy = 0; sy < 4; ++sy) {
+    {
+        // along the rows: up to five frame columns overlap an observation column, by multiples of 4 out of 84
+        const int x_start = ox * 320, x_end = x_start + 320, first_x = x_start / 84;
+        unsigned int weight_r[5], weight_g[5], weight_b[5]; int column[5];
 #pragma unroll
         for (int sx = 0; sx < 5; ++sx) {
-            // overlaps are at most 84, so the product stays below 7226 and (p * 5462) >> 18 is p / 48 exactly; every
-            // factor here fits 24 bits, and 24-bit multiplies run at full rate where 32-bit ones take four times as long
-            const unsigned weight = __umul24(__umul24((unsigned)y_overlap[sy], (unsigned)x_overlap[sx]), 5462u) >> 18;
-            const unsigned int colour = pal[tap[sy][sx]];
-            rs += (int)__umul24(colour & 0xFFu, weight); gs += (int)__umul24((colour >> 8) & 0xFFu, weight); bs += (int)__umul24(colour >> 16, weight);
+            const int source_x = first_x + sx;
+            const int over = min(x_end, (source_x + 1) * 84) - max(x_start, source_x * 84);
+            const unsigned int weight = (source_x >= SW || over <= 0) ? 0u : (unsigned)over >> 2;
+            // a colour word times a weight in byte 0, 1 or 2 is that channel times the weight (a four-byte dot product)
+            weight_r[sx] = weight; weight_g[sx] = weight << 8; weight_b[sx] = weight << 16;
+            column[sx] = min(source_x, SW - 1);
+        }
+        for (int sy = slot; sy < OBS_SOURCE_ROWS && works; sy += 3) {
+            unsigned int rs = 0, gs = 0, bs = 0;
+            if (tile_first + sy < source_rows) {
+                unsigned int colour[5];
+#pragma unroll
+                for (int sx = 0; sx < 5; ++sx) colour[sx] = pal[staged[sy * SW + column[sx]]];
+#pragma unroll
+                for (int sx = 0; sx < 5; ++sx) {
+                    rs = __builtin_amdgcn_udot4(colour[sx], weight_r[sx], rs, false);
+                    gs = __builtin_amdgcn_udot4(colour[sx], weight_g[sx], gs, false);
+                    bs = __builtin_amdgcn_udot4(colour[sx], weight_b[sx], bs, false);
+                }
+            }
+            along_rg[sy * GD_OBS_SIZE + ox] = rs | (gs << 16);
+            along_b[sy * GD_OBS_SIZE + ox] = (unsigned short)bs;
         }
     }
-    int r = (rs + 800) / 1600, g = (gs + 800) / 1600, b = (bs + 800) / 1600;
-    unsigned char gray = (unsigned char)((r * 77 + g * 150 + b * 29 + 128) >> 8);
+    __syncthreads();
+    // down the columns: up to four frame rows overlap an observation row, by multiples of 12 out of 84
+    for (int row_in_block = slot; row_in_block < OBS_BLOCK_ROWS && works; row_in_block += 3) {
+        const int y_start = row_in_block * 240, y_end = y_start + 240, first_y = y_start / 84;   // relative to the block's first frame row
+        unsigned int rs = 0, gs = 0, bs = 0;
+#pragma unroll
+        for (int sy = 0; sy < 4; ++sy) {
+            const int source_y = first_y + sy;
+            const int over = min(y_end, (source_y + 1) * 84) - max(y_start, source_y * 84);
+            const unsigned int weight = (source_y >= OBS_SOURCE_ROWS || over <= 0) ? 0u : (unsigned)over / 12u;
+            const int at = min(source_y, OBS_SOURCE_ROWS - 1) * GD_OBS_SIZE + ox;
+            const unsigned int rg = along_rg[at];
+            rs += __umul24(rg & 0xFFFFu, weight); gs += __umul24(rg >> 16, weight); bs += __umul24(along_b[at], weight);
+        }
+        const unsigned int r = (rs + 800u) / 1600u, g = (gs + 800u) / 1600u, b = (bs + 800u) / 1600u;
+        reinterpret_cast<unsigned char *>(gray_words)[row_in_block * GD_OBS_SIZE + ox] = (unsigned char)((r * 77u + g * 150u + b * 29u + 128u) >> 8);
+    }
+    __syncthreads();
     // The block's pixels are contiguous in the observation; they go out, and the stack is rolled, a word (four
     // pixels) per thread.
-    if (threadIdx.x < OBS_BLOCK_ROWS * GD_OBS_SIZE) reinterpret_cast<unsigned char *>(gray_words)[threadIdx.x] = gray;
-    __syncthreads();
-    static_assert((GD_OBS_SIZE * GD_OBS_SIZE) % 4 == 0 && (OBS_BLOCK_ROWS * GD_OBS_SIZE) % 4 == 0, "observe_kernel: whole words");
     if (!rolls) return;
     const unsigned int grays = gray_words[threadIdx.x];
     if (obs) {
