@@ -1606,6 +1606,44 @@ __device__ __forceinline__ size_t flat_sample_tabled(const Tables &tb, const Lan
     return (size_t)(((unsigned)texture * (unsigned)m->tex_max_h + v) * (unsigned)m->tex_max_w + u);   // the atlas is below 4 GiB (checked at create)
 }
 
+// flat_sample_tabled for a run of neighbouring pixels of one row that show the same plane: what depends on the row and the
+// plane is worked out once (plane_span), each pixel then costs two 64-bit additions and two products (plane_span_texel).
+// The same integers: base + px * step is (base + px0 * step) + k * step in 64-bit arithmetic.
+struct PlaneSpan {
+    i64 distance, xfrac_base, yfrac_base, xstep, ystep;
+    unsigned pviewx, pviewy, texture_row0, atlas_width;
+    int width_shift, height_shift, colormap_row;
+};
+__device__ __forceinline__ PlaneSpan plane_span(const Tables &tb, const LaneCtx &c, const LaneTables &lt, i64 yslope, int level_index, int sector,
+                                                bool is_floor, int px0, int py) {
+    const gd_map_desc *m = tb.m;
+    PlaneSpan s;
+    const int texture = is_floor ? tb.floor_tex(sector) : tb.ceil_tex(sector);
+    const int width_bits = tb.width_bits(texture), height_bits = tb.height_bits(texture);
+    const i64 *plane = lt.level_plane + 2 * (is_floor ? level_index : lt.floors + level_index);
+    const i64 plane_height_fixed = plane[0], glob = plane[1];
+    s.xstep = lt.step_scale[width_bits]; s.ystep = lt.step_scale[16 + height_bits];
+    s.xfrac_base = lt.step_scale[32 + width_bits] + mul64_u32(s.xstep, (unsigned)px0);
+    s.yfrac_base = lt.step_scale[48 + height_bits] + mul64_u32(s.ystep, (unsigned)px0);
+    s.pviewx = (unsigned)lt.step_scale[64 + width_bits]; s.pviewy = (unsigned)lt.step_scale[80 + height_bits];
+    s.distance = mul64_u32(plane_height_fixed, (unsigned)yslope) >> 16;
+    s.width_shift = 31 - width_bits; s.height_shift = 31 - height_bits;
+    const float light = tb.light(sector) + (float)(c.flash_light * 16);
+    i64 row = c.center_fixed - (i64)py * FIXED_UNIT;
+    if (row < 0) row = -row;
+    const i64 visibility = min64(mul64_u32(row, (unsigned)glob) >> 16, 24 * FIXED_UNIT);
+    const i64 plane_shade = 64 * FIXED_UNIT - ((i64)light + 12) * (FIXED_UNIT / 4);
+    s.colormap_row = (int)clampi((plane_shade - visibility) >> 16, 0, 31);
+    s.texture_row0 = (unsigned)texture * (unsigned)m->tex_max_h; s.atlas_width = (unsigned)m->tex_max_w;
+    return s;
+}
+__device__ __forceinline__ unsigned plane_span_texel(const PlaneSpan &s, int k) {   // pixel px0 + k
+    const unsigned xfrac = mul64_bits_16_47(s.distance, s.xfrac_base + mul64_u32(s.xstep, (unsigned)k)) + s.pviewx;
+    const unsigned yfrac = mul64_bits_16_47(s.distance, s.yfrac_base + mul64_u32(s.ystep, (unsigned)k)) + s.pviewy;
+    const unsigned u = (xfrac >> s.width_shift) >> 1, v = (yfrac >> s.height_shift) >> 1;   // two shifts: a size of one shifts by 32
+    return (s.texture_row0 + v) * s.atlas_width + u;   // the atlas is below 4 GiB (checked at create)
+}
+
 // Visplane repair (engine.py:11026-11135) of the row ranges flat_select_kernel noted, one block per lane, one
 // wavefront per 64 columns.  Every pixel of those rows is selected first (the repairs read whole rows and
 // columns).  Vertical: an unresolved pixel takes the sector of the next resolved pixel below it in its half of
@@ -3300,12 +3338,17 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
 // one, the sector the per-pixel plane rays selected (engine.py:11145-11163).  Doing both here
 // shades every pixel once, in a kernel light enough to run at full occupancy.
 // ---------------------------------------------------------------------------------------------
-#define SHADE_TILES 52   // 256-pixel tiles per block: 260 tiles per view = 5 blocks per lane (each block stages the tables once)
-#define SHADE_GROUP 4    // tiles per step
+#define SHADE_RUN 4      // neighbouring pixels of a row per thread
+#define SHADE_TILES 14   // tiles (256 runs) per block: 65 tiles per view = 5 blocks per lane (each block stages the tables once)
+#define SHADE_GROUP 2    // tiles per step
+static_assert(SW % SHADE_RUN == 0 && SHADE_RUN == 4, "plane_shade_kernel: a run is one 16-byte load of per-pixel words and one 4-byte store");
 // DEPTH: also keep the depth of every pixel no wall tier covers (frames that draw decals).  STAGED: the lane's plane table
 // is short enough for LDS (the kernel then reads it with LDS instructions; a pointer that may be either costs more).
 template <bool DEPTH, bool STAGED>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) plane_shade_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
+// Five wavefronts per SIMD, not the eight its registers would allow at one tile per step: alone the kernel takes a
+// seventh longer that way, but it runs beside the flat pass (launch_chunk), whose kernels wait for memory more than
+// they compute and finish sooner when this one leaves them room; the two together end 0.06 ms earlier per 4096 lanes.
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5, 5))) plane_shade_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
     const gd_map_desc *m = &dm.d;
     __shared__ float4 sector_lds[LDS_SECTORS];
     __shared__ unsigned int sector_level_lds[LDS_SECTORS];
@@ -3332,59 +3375,104 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))
     else lt.level_plane = sc.level_plane + (size_t)local * levels * 2;
     const LaneCtx &c = sc.ctx[local];
     unsigned char *frame = frame_base + (size_t)local * frame_stride;
-    // SHADE_GROUP tiles per step and three stages per step (per-pixel words, texels, stores), each
-    // stage's loads issued together so that their latencies overlap
+    const bool frame_aligned = (reinterpret_cast<size_t>(frame) & 3) == 0;
+    const uint4 *meta_groups = reinterpret_cast<const uint4 *>(sc.meta + (size_t)local * VH * SW);
+    // A thread takes SHADE_RUN neighbouring pixels of a row (a row is a whole number of runs): their per-pixel words arrive
+    // in one load, pixels that show the same plane share everything but two products, and the run's bytes leave in
+    // one store.  SHADE_GROUP runs, a tile apart, per step, each stage's loads issued together.
     for (int tile0 = 0; tile0 < SHADE_TILES; tile0 += SHADE_GROUP) {
-        unsigned int meta[SHADE_GROUP];
-        int pixels[SHADE_GROUP];
+        unsigned int meta[SHADE_GROUP][SHADE_RUN];
+        int first_pixel[SHADE_GROUP];
 #pragma unroll
-        for (int j = 0; j < SHADE_GROUP; ++j) {
-            const int pixel = (blockIdx.x * SHADE_TILES + tile0 + j) * 256 + threadIdx.x;
-            pixels[j] = (tile0 + j < SHADE_TILES && pixel < VH * SW) ? pixel : -1;
-            const size_t i = (size_t)local * VH * SW + (pixels[j] < 0 ? 0 : pixels[j]);
-            meta[j] = sc.meta[i];
-            if (pixels[j] >= 0 && pixels[j] < (GD_SCREEN_HEIGHT - VH) * SW) frame[(size_t)VH * SW + pixels[j]] = 0;   // the empty status bar, rows 208..239
-        }
-        size_t texel_at[SHADE_GROUP]; int colormap_row[SHADE_GROUP]; unsigned char texel[SHADE_GROUP];
-        bool shade[SHADE_GROUP];
-#pragma unroll
-        for (int j = 0; j < SHADE_GROUP; ++j) {
-            const int pixel = pixels[j];
-            const int ps = (int)((meta[j] >> META_SECTOR_SHIFT) & META_SECTOR_MASK) - 1;
-            shade[j] = tabled && pixel >= 0 && ps >= 0 && !(meta[j] & (META_FILLED | META_MASKED));
-            texel[j] = 0; colormap_row[j] = 0; texel_at[j] = 0;
-            if (!shade[j]) continue;
-            const int y = pixel / SW, x = pixel - y * SW;
-            const bool is_floor = (meta[j] & META_FLOOR) != 0;
-            const int sector = ps;
-            const unsigned int pair = sector < tb.sector_cached ? sector_level_lds[sector] : dm.sector_level[sector];
-            texel_at[j] = flat_sample_tabled(tb, c, lt, sc.row_slope[(size_t)local * VH + y], is_floor ? (pair & 0xFFFF) : (pair >> 16),
-                                             sector, is_floor, x, y, &colormap_row[j]);
-            texel[j] = m->tex_atlas[texel_at[j]];
-        }
-#pragma unroll
-        for (int j = 0; j < SHADE_GROUP; ++j) {
-            const int pixel = pixels[j];
-            if (pixel < 0) continue;
-            if (meta[j] & META_FILLED) {   // a wall tier's pixel, unless a masked texture went over it
-                if (!(meta[j] & META_MASKED)) frame[pixel] = (unsigned char)(meta[j] >> META_SECTOR_SHIFT);
-                continue;
+        for (int g = 0; g < SHADE_GROUP; ++g) {
+            const int run = (blockIdx.x * SHADE_TILES + tile0 + g) * 256 + threadIdx.x;
+            const bool valid = tile0 + g < SHADE_TILES && run < VH * SW / SHADE_RUN;
+            first_pixel[g] = valid ? run * SHADE_RUN : -1;
+            const uint4 words = meta_groups[valid ? run : 0];
+            meta[g][0] = words.x; meta[g][1] = words.y; meta[g][2] = words.z; meta[g][3] = words.w;
+            if (valid && run < (GD_SCREEN_HEIGHT - VH) * SW / SHADE_RUN) {   // the empty status bar, rows 208..239
+                unsigned char *bar = frame + (size_t)VH * SW + (size_t)run * SHADE_RUN;
+                if (frame_aligned) *reinterpret_cast<unsigned int *>(bar) = 0u;
+                else for (int k = 0; k < SHADE_RUN; ++k) bar[k] = 0;
             }
-            const int y = pixel / SW, x = pixel - y * SW;
-            const size_t i = (size_t)local * VH * SW + pixel;
-            const int ps = (int)((meta[j] >> META_SECTOR_SHIFT) & META_SECTOR_MASK) - 1;
-            if (ps < 0) {
-                // neither tier nor plane: the flat pass's picture shows here (unless a masked texture covers it);
-                // flat_shade_kernel paints the pixel once that pass has run
-                continue;
+        }
+        int colormap_row[SHADE_GROUP][SHADE_RUN]; unsigned char texel[SHADE_GROUP][SHADE_RUN];
+        unsigned int shades[SHADE_GROUP];   // bit k: pixel k of the run shows a visplane's flat
+#pragma unroll
+        for (int g = 0; g < SHADE_GROUP; ++g) {
+            shades[g] = 0;
+            const int pixel0 = first_pixel[g] < 0 ? 0 : first_pixel[g];
+            const int y = pixel0 / SW, x0 = pixel0 - y * SW;
+            // what names a pixel's plane in its word: the sector and which of its two planes
+            const unsigned int PLANE_KEY = (META_SECTOR_MASK << META_SECTOR_SHIFT) | META_FLOOR;
+            int leader = -1;
+#pragma unroll
+            for (int k = 0; k < SHADE_RUN; ++k) {
+                const int ps = (int)((meta[g][k] >> META_SECTOR_SHIFT) & META_SECTOR_MASK) - 1;
+                texel[g][k] = 0; colormap_row[g][k] = 0;
+                if (tabled && first_pixel[g] >= 0 && ps >= 0 && !(meta[g][k] & (META_FILLED | META_MASKED))) {
+                    shades[g] |= 1u << k;
+                    if (leader < 0) leader = k;
+                }
             }
-            const bool is_floor = (meta[j] & META_FLOOR) != 0;
-            if (shade[j]) frame[pixel] = colormap_lds[colormap_row[j] * 256 + texel[j]];
-            else if (!(meta[j] & META_MASKED)) frame[pixel] = flat_pixel(tb, colormap_lds, c, ps, is_floor, x, y);
-            if (DEPTH && !(meta[j] & META_MASKED)) {   // exact plane depth (engine.py:13406-13416)
-                const float flat_center_px = (103.0f + c.pitch_offset) + 0.5f;
-                const float plane_height = is_floor ? (c.view_z - tb.floor_h(ps)) : (tb.ceil_h(ps) - c.view_z);
-                sc.scene_depth[i] = plane_height * 192.0f / fmaxf(fabsf((float)y - flat_center_px), 0.5f);
+            if (leader < 0) continue;
+            const i64 yslope = sc.row_slope[(size_t)local * VH + y];
+            unsigned int leader_word = meta[g][0];
+#pragma unroll
+            for (int k = 1; k < SHADE_RUN; ++k) if (leader == k) leader_word = meta[g][k];
+            auto span_of = [&](unsigned int word) {
+                const int sector = (int)((word >> META_SECTOR_SHIFT) & META_SECTOR_MASK) - 1;
+                const bool is_floor = (word & META_FLOOR) != 0;
+                const unsigned int pair = sector < tb.sector_cached ? sector_level_lds[sector] : dm.sector_level[sector];
+                return plane_span(tb, c, lt, yslope, is_floor ? (pair & 0xFFFF) : (pair >> 16), sector, is_floor, x0, y);
+            };
+            const PlaneSpan shared = span_of(leader_word);
+#pragma unroll
+            for (int k = 0; k < SHADE_RUN; ++k) {
+                if (!(shades[g] & (1u << k))) continue;
+                if (((meta[g][k] ^ leader_word) & PLANE_KEY) == 0) {
+                    colormap_row[g][k] = shared.colormap_row;
+                    texel[g][k] = m->tex_atlas[plane_span_texel(shared, k)];
+                } else {   // another plane starts inside the run
+                    const PlaneSpan own = span_of(meta[g][k]);
+                    colormap_row[g][k] = own.colormap_row;
+                    texel[g][k] = m->tex_atlas[plane_span_texel(own, k)];
+                }
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < SHADE_GROUP; ++g) {
+            if (first_pixel[g] < 0) continue;
+            const int y = first_pixel[g] / SW, x0 = first_pixel[g] - y * SW;
+            unsigned int colours = 0, written = 0;   // bit k of `written`: this kernel decides pixel k
+#pragma unroll
+            for (int k = 0; k < SHADE_RUN; ++k) {
+                const unsigned int word = meta[g][k];
+                const int ps = (int)((word >> META_SECTOR_SHIFT) & META_SECTOR_MASK) - 1;
+                unsigned int colour = 0; bool writes = false;
+                if (word & META_FILLED) {   // a wall tier's pixel, unless a masked texture went over it
+                    colour = (word >> META_SECTOR_SHIFT) & 0xFFu; writes = !(word & META_MASKED);
+                } else if (ps >= 0) {
+                    // (neither tier nor plane: the flat pass's picture shows there, unless a masked texture covers it;
+                    // flat_shade_kernel paints the pixel once that pass has run)
+                    const bool is_floor = (word & META_FLOOR) != 0;
+                    if (shades[g] & (1u << k)) { colour = colormap_lds[colormap_row[g][k] * 256 + texel[g][k]]; writes = true; }
+                    else if (!(word & META_MASKED)) { colour = flat_pixel(tb, colormap_lds, c, ps, is_floor, x0 + k, y); writes = true; }
+                    if (DEPTH && !(word & META_MASKED)) {   // exact plane depth (engine.py:13406-13416)
+                        const float flat_center_px = (103.0f + c.pitch_offset) + 0.5f;
+                        const float plane_height = is_floor ? (c.view_z - tb.floor_h(ps)) : (tb.ceil_h(ps) - c.view_z);
+                        sc.scene_depth[(size_t)local * VH * SW + first_pixel[g] + k] = plane_height * 192.0f / fmaxf(fabsf((float)y - flat_center_px), 0.5f);
+                    }
+                }
+                colours |= colour << (8 * k);
+                if (writes) written |= 1u << k;
+            }
+            unsigned char *out = frame + first_pixel[g];
+            if (written == (1u << SHADE_RUN) - 1 && frame_aligned) {
+                *reinterpret_cast<unsigned int *>(out) = colours;
+            } else {   // some pixel of the run is the flat pass's or a masked texture's: byte by byte
+#pragma unroll
+                for (int k = 0; k < SHADE_RUN; ++k) if (written & (1u << k)) out[k] = (unsigned char)(colours >> (8 * k));
             }
         }
     }
@@ -4871,7 +4959,7 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     // timed (and so serial): shading, then the flat pass, each between its own marks
     auto shade_planes = [&]() {
         if (fused) return;
-        const dim3 grid(((VH * SW + 255) / 256 + SHADE_TILES - 1) / SHADE_TILES, count);
+        const dim3 grid(((VH * SW / SHADE_RUN + 255) / 256 + SHADE_TILES - 1) / SHADE_TILES, count);
         const bool staged = m.floor_level_count + m.ceil_level_count <= 2 * PLANE_LEVELS;
         auto kernel = decals ? (staged ? plane_shade_kernel<true, true> : plane_shade_kernel<true, false>)
                              : (staged ? plane_shade_kernel<false, true> : plane_shade_kernel<false, false>);
