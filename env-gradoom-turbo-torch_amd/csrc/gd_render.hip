@@ -114,7 +114,9 @@ struct __align__(16) PassRec {
     unsigned short spare;
     float distance;
 };
-#define PASS_MAX 96   // column passes recorded per screen column; a column that needs more sets STATUS_PASS_OVERFLOW
+#define PASS_MAX 255  // most column passes recorded per screen column (the count is a byte).  A chunk keeps room for as many as the
+                      // map has sectors (a column runs at most that many passes), at least 16, at most PASS_MAX: Scratch::pass_slots.
+                      // A column that needs more sets STATUS_PASS_OVERFLOW.
 
 struct RecSpan {   // what a ray test of one linedef needs (eval_segment), kept for every linedef of the map; the full record
                    // above exists only for the linedefs the camera can see at all
@@ -198,8 +200,9 @@ struct Scratch {    // per-chunk working memory, sized at create
     int *flat_col_top;     // [L,2,320] per screen half and column: the topmost shown pixel the flat pass could not
                            // resolve (any value >= 208: none).  lane_tables_kernel sets "none", flat_gap_column_kernel
                            // lowers it while it selects the gap pixels.
-    PassRec *pass_rec;     // [L,PASS_MAX,320] the drawsegs of each column's passes, in pass order
-    float *pass_path_distance;  // [L,PASS_MAX,320] distance of the portal path of a pass that carries PB_PS_KEEPS (written for those only)
+    int pass_slots;        // passes a column can record in this chunk
+    PassRec *pass_rec;     // [L,pass_slots,320] the drawsegs of each column's passes, in pass order
+    float *pass_path_distance;  // [L,pass_slots,320] distance of the portal path of a pass that carries PB_PS_KEEPS (written for those only)
     unsigned char *pass_count;  // [L,320] passes recorded for the column: up to its last pass that draws or moves a clip
     unsigned int *meta;    // [L,208,320] filled | floor | plane_sector+1 | clip_wall+1
     float *clip_depth;     // [L,208,320]
@@ -3186,8 +3189,8 @@ __global__ void __launch_bounds__(64 * SELECT_STRIPS_PER_GROUP) wall_select_kern
     st.pend_pb_index = 0; st.pend_pb_sector = -1; st.pend_pb_exit = 0.0f; st.flags = 0;
     bool boundary_has_po = false;
     for (int k = 0; k < cc.count; ++k) if (cc.cand(k).flags & CF_LEDGE) { boundary_has_po = true; break; }
-    PassRec *records = sc.pass_rec + ((size_t)local * PASS_MAX * SW + x);
-    float *path_distances = sc.pass_path_distance + ((size_t)local * PASS_MAX * SW + x);
+    PassRec *records = sc.pass_rec + ((size_t)local * sc.pass_slots * SW + x);
+    float *path_distances = sc.pass_path_distance + ((size_t)local * sc.pass_slots * SW + x);
     PixelBuffers no_pixels; SilhouetteBounds no_bounds; GapRange no_gaps;   // the state part of pass_advance touches none of them
     PassColumn pc;
     bool done = false;
@@ -3197,7 +3200,7 @@ __global__ void __launch_bounds__(64 * SELECT_STRIPS_PER_GROUP) wall_select_kern
         if (!done) {
             pass_select<SPLIT>(cc, st, boundary_has_po, pc);
             if (pc.bits & (PB_RASTER | PB_PS_KEEPS)) {
-                if (pass < PASS_MAX) {
+                if (pass < sc.pass_slots) {
                     PassRec rec;
                     rec.wall = (unsigned short)pc.wall; rec.render_current = (unsigned short)pc.render_current;
                     rec.bits = (unsigned short)pc.bits; rec.ps_path = (unsigned short)pc.ps_path_index;
@@ -3275,8 +3278,8 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
     st.pend_pb_index = 0; st.pend_pb_sector = -1; st.pend_pb_exit = 0.0f; st.flags = 0;
     SilhouetteBounds sb; sb.bot_row = VH; sb.top_row = 0; sb.bot_depth = -GD_INF; sb.top_depth = -GD_INF;
     const int passes = sc.pass_count[(size_t)local * SW + x];
-    const PassRec *records = sc.pass_rec + ((size_t)local * PASS_MAX * SW + x);
-    const float *path_distances = sc.pass_path_distance + ((size_t)local * PASS_MAX * SW + x);
+    const PassRec *records = sc.pass_rec + ((size_t)local * sc.pass_slots * SW + x);
+    const float *path_distances = sc.pass_path_distance + ((size_t)local * sc.pass_slots * SW + x);
     PassColumn pc;
     pc.wall = 0; pc.side = 0; pc.bits = 0; pc.visibility = 0;
     pc.clipped_top = 0.0f; pc.clipped_bottom = 0.0f; pc.clipped_upper_bottom = 0.0f; pc.clipped_lower_top = 0.0f;
@@ -4738,8 +4741,9 @@ size_t carve_scratch(Scratch &sc, unsigned char *base, size_t L, const gd_map_de
     take(&sc.flat_col_top, L * 2 * SW);
     take(&sc.flat_list, L * FLAT_LIST_MAX);
     take(&sc.flat_list_count, L);
-    take(&sc.pass_rec, L * PASS_MAX * SW);
-    take(&sc.pass_path_distance, L * PASS_MAX * SW);
+    sc.pass_slots = h.sector_count < 16 ? 16 : (h.sector_count > PASS_MAX ? PASS_MAX : h.sector_count);
+    take(&sc.pass_rec, L * (size_t)sc.pass_slots * SW);
+    take(&sc.pass_path_distance, L * (size_t)sc.pass_slots * SW);
     take(&sc.pass_count, L * SW);
     take(&sc.meta, L * PX);
     take(&sc.clip_depth, L * PX);

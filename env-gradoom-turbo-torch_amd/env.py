@@ -287,7 +287,7 @@ class GraDoomVecEnv:
             )
         if flags & 2:
             raise RuntimeError(
-                "the renderer truncated a screen column's list of drawsegs (a column crossed more than 96 portals): frames of "
+                "the renderer truncated a screen column's list of drawsegs (a column crossed more than 255 portals): frames of "
                 "this environment are not trustworthy on this map"
             )
 

@@ -10,6 +10,11 @@
  * host memory.  Entry points return 0 on success or a negative GD_E_* code;
  * gd_last_error() returns a message for the calling thread.
  *
+ * Host threads: the library takes no locks.  Calls that use the same renderer,
+ * and gd_render_static calls on the same GPU (its first call on a device looks
+ * up that device's working array), must come from one host thread at a time;
+ * calls on different renderers are independent.
+ *
  * Names follow the reference's domain: lanes (batched environments), linedefs
  * ("walls"), sectors, flats, visplanes, drawsegs, sprites, PLAYPAL, COLORMAP.
  */
@@ -288,7 +293,7 @@ int gd_render_static(gd_renderer *r, const gd_lanes_desc *lanes, const gd_frame_
  * of that lane is not trustworthy.  A column keeps 64 in its own slots; one
  * that sees more moves to a spill pool (up to 256 per column; every column of
  * up to 8 lanes, one column in 32 of a 4096-lane chunk, 320 columns in
- * gd_render_static).  bit1: a column crossed more than 96 portals.
+ * gd_render_static).  bit1: a column drew more than 255 passes.
  * Replaces nothing in the reference.
  */
 int gd_renderer_status(gd_renderer *r, int32_t *status);

@@ -77,8 +77,8 @@ def test_static_entry_point_rejects_more_lanes_than_its_limit():
 
 
 def test_static_entry_point_at_the_headline_map_size_in_several_chunks():
-    # the 4000-linedef map with uniform heights: a chunk of the 64 MiB array holds about thirty lanes, so 100 lanes take
-    # several; the hand-off options of gd_render (hwc final frames, status bar rows pooled) go through unchanged
+    # the 4000-linedef map with uniform heights: a chunk of the 64 MiB array holds about twenty lanes, so 100 lanes take
+    # five; the hand-off options of gd_render (hwc final frames, status bar rows pooled) go through unchanged
     from gradoom_amd import hostmath, mapbuild, synthmap
     from gradoom_amd.renderer import HipRenderer, LaneState
     from gradoom_amd.selfcheck import make_lane_arrays
