@@ -211,17 +211,17 @@ def test_sectors_with_ceilings_below_their_floors_match_the_oracle(oracle, seed,
     renderer.close()
 
 
-def corridor_case(lanes: int):
-    """A corridor of 80 sectors and cameras in it that look along it, so that every divider lands in the same screen
-    columns: more linedefs per column ray than the 64 a column keeps in its own slots."""
+def corridor_case(lanes: int, sectors: int = 80):
+    """A corridor of `sectors` sectors and cameras in it that look along it, so that every divider lands in the same
+    screen columns: more linedefs per column ray than the 64 a column keeps in its own slots."""
     from gradoom_amd import mapbuild, synthmap
     from gradoom_amd.selfcheck import make_lane_arrays
 
-    smap = synthmap.generate_map(5, grid=(80, 1), sectors=80, linedefs=241, midtex=0.2)
+    smap = synthmap.generate_map(5, grid=(sectors, 1), sectors=sectors, linedefs=3 * sectors + 1, midtex=0.2)
     poses = synthmap.generate_poses(smap, lanes, 11, pitch=True, flash=True)
     rng = np.random.default_rng(3)
     for lane in range(lanes):
-        sector = int(rng.integers(0, 8)) if lane % 2 == 0 else int(rng.integers(72, 80))   # either end, looking at the other
+        sector = int(rng.integers(0, 8)) if lane % 2 == 0 else int(rng.integers(sectors - 8, sectors))   # either end, looking at the other
         centre = smap.sector_quads[sector].mean(axis=0)
         poses.x[lane], poses.y[lane] = float(centre[0]) + float(rng.uniform(-20, 20)), float(centre[1]) + float(rng.uniform(-20, 20))
         poses.view_z[lane] = float(smap.sector_heights[sector, 0]) + 41.0
@@ -231,15 +231,17 @@ def corridor_case(lanes: int):
     return smap, mapbuild.build_map_tables(smap), make_lane_arrays(smap, poses, sprites)
 
 
-def test_columns_that_see_more_than_64_linedefs_match_the_oracle(oracle):
+@pytest.mark.parametrize("sectors", [80, 124])
+def test_columns_that_see_more_than_64_linedefs_match_the_oracle(oracle, sectors):
     """Such columns get a slot in the spill pool, where every linedef their ray can reach is listed (the reference keeps a
-    dense [columns, linedefs] table, engine.py:11446-11451, and has no limit)."""
+    dense [columns, linedefs] table, engine.py:11446-11451, and has no limit).  124 sectors: the longest corridor of
+    256-unit cells the 16.16 coordinates hold; its columns draw more than a hundred passes."""
     from gradoom_amd import hostmath
     from gradoom_amd.renderer import HipRenderer, LaneState
 
     lanes = 6
     cosine = hostmath.cosine_correction("cpu").numpy()
-    smap, tables, arrays = corridor_case(lanes)
+    smap, tables, arrays = corridor_case(lanes, sectors)
     expected = oracle.render(tables, arrays, cosine)
     renderer = HipRenderer(smap, lanes, "cuda:0", cosine_correction=cosine, tables=tables)
     state = LaneState.from_numpy(arrays, "cuda:0")
