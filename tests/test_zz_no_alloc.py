@@ -50,6 +50,30 @@ def test_static_entry_point_equals_gd_render_on_two_calls_in_a_row():
     bare.close()
 
 
+def test_static_entry_point_lists_long_columns_in_its_own_spill_pool():
+    # an 80-sector corridor seen end on: a few columns of every lane see more than 64 linedefs and move to the spill pool,
+    # of which the static array holds one block (320 columns) per chunk
+    from gradoom_amd import hostmath
+    from gradoom_amd.renderer import HipRenderer, LaneState
+    from test_gpu_random_maps import corridor_case
+
+    total = 12
+    smap, tables, arrays = corridor_case(total)
+    cosine = hostmath.cosine_correction("cpu").numpy()
+    lanes = LaneState.from_numpy(arrays, "cuda:0")
+    plain = HipRenderer(smap, total, "cuda:0", cosine_correction=cosine, tables=tables)
+    bare = HipRenderer(smap, 0, "cuda:0", cosine_correction=cosine, tables=tables)
+    rng = np.random.default_rng(5)
+    start = rng.integers(0, 256, (total, 4, 84, 84), dtype=np.uint8)
+    mask = np.zeros(total, dtype=np.uint8)
+    expected = _render(plain, plain.render, lanes, total, start, mask)
+    ours = _render(bare, bare.render_static, lanes, total, start, mask)
+    for name, a, b in zip(("indexed", "obs", "frames", "rgb"), ours, expected):
+        assert np.array_equal(a, b), name
+    plain.close()
+    bare.close()
+
+
 def test_static_entry_point_rejects_more_lanes_than_its_limit():
     import ctypes as C
 
