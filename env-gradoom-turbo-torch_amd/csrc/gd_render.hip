@@ -209,6 +209,8 @@ struct Scratch {    // per-chunk working memory, sized at create
     unsigned char *frame;  // [L,240,320] when the caller wants no indexed output
     u64 *block_hit;        // [L,320] nearest blocking linedef of the column ray: float bits of the distance << 32 |
                            // slot in blocking_walls, all ones when no ray hits (engine.py:10534-10557)
+    int *lane_blends;      // [L] does some live billboard of the lane blend with the pixel below it (sprite_style other than -1)?
+                           // lane_tables_kernel says; launch_chunk's two billboard launches split the lanes by it
     unsigned char *strip_key;  // [L*SEGS_PER_LANE] expected traversal length of each (lane, segment of SEG_COLS columns)
     int *strip_order;      // [L*SEGS_PER_LANE] segments, longest expected traversal first
     int *status;           // [1] sticky overflow flags
@@ -229,6 +231,12 @@ struct Scratch {    // per-chunk working memory, sized at create
 #define META_FILLED 0x80000000u   // an opaque wall tier owns the pixel; its palette index sits in the low byte of the
                                   // plane sector field (plane shading, which writes every other view pixel, stores it)
 #define META_FLOOR 0x40000000u    // the owning plane is a floor
+// which lanes a billboard or flat-shading launch takes (launch_chunk splits them by Scratch::lane_blends)
+#define LANES_ALL 0
+#define LANES_PLAIN 1
+#define LANES_BLENDING 2
+#define META_GAP_COVERED META_FLOOR   // in the word of a gap pixel (no tier, no plane, no masked texture: the bit above means nothing
+                                  // there): a billboard was painted over it before the flat pass's pixels were, which flat_shade_kernel respects
 #define META_MASKED 0x20000000u   // a masked mid-texture was drawn over the pixel
 #define META_SECTOR_SHIFT 16
 #define META_SECTOR_MASK 0x1FFFu  // plane sector + 1
@@ -493,6 +501,16 @@ __global__ void lane_tables_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_b
     for (int x = threadIdx.x; x < SW; x += blockDim.x) { sc.cand_count[(size_t)local * SW + x] = 0; sc.block_hit[(size_t)local * SW + x] = ~0ULL; }
     // and no column holds an unresolved gap pixel yet
     for (int k = threadIdx.x; k < 2 * SW; k += blockDim.x) sc.flat_col_top[(size_t)local * 2 * SW + k] = VH;
+    {   // does a live billboard of the lane blend with what lies under it?
+        bool blends = false;
+        if (lanes.sprite_style && lanes.sprite_alive)
+            for (int k = threadIdx.x; k < lanes.sprite_slots; k += blockDim.x) {
+                const size_t at = (size_t)(lane_base + local) * lanes.sprite_slots + k;
+                blends |= lanes.sprite_alive[at] != 0 && lanes.sprite_style[at] != -1;
+            }
+        const int any = __syncthreads_or(blends ? 1 : 0);
+        if (threadIdx.x == 0) sc.lane_blends[local] = any;
+    }
     const float cx = lanes.x[lane_base + local], cy = lanes.y[lane_base + local];
     __shared__ unsigned int masks_lds[LEVEL_BUCKETS * LEVEL_MASK_WORDS_MAX];
     const int mask_words = level_mask_words(&dm.d);
@@ -3504,21 +3522,28 @@ __device__ void flat_shade_pixel(const DeviceMap &dm, const Scratch &sc, const L
     }
 }
 
-__global__ void __launch_bounds__(128) flat_shade_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
+// lane_pick: LANES_ALL, or one half of launch_chunk's split: LANES_PLAIN for the lanes whose billboards were painted first and
+// marked the gap pixels they took, LANES_BLENDING for the others, whose billboards come after this.
+__global__ void __launch_bounds__(128) flat_shade_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride, int lane_pick) {
     const int local = blockIdx.x;
     if (local >= lane_count) return;
+    if (lane_pick != LANES_ALL && (sc.lane_blends[local] != 0) != (lane_pick == LANES_BLENDING)) return;   // the same in the whole block
+    const bool after_billboards = lane_pick == LANES_PLAIN;
     const int listed = sc.flat_list_count[local];
     const LaneCtx &c = sc.ctx[local];
     unsigned char *frame = frame_base + (size_t)local * frame_stride;
     if (listed <= FLAT_LIST_MAX) {
-        for (int slot = threadIdx.x; slot < listed; slot += blockDim.x)
-            flat_shade_pixel(dm, sc, c, local, sc.flat_list[(size_t)local * FLAT_LIST_MAX + slot], frame);
+        for (int slot = threadIdx.x; slot < listed; slot += blockDim.x) {
+            const int pixel = sc.flat_list[(size_t)local * FLAT_LIST_MAX + slot];
+            if (after_billboards && (sc.meta[(size_t)local * VH * SW + pixel] & META_GAP_COVERED)) continue;
+            flat_shade_pixel(dm, sc, c, local, pixel, frame);
+        }
         return;
     }
     // a lane with more gap pixels than the list holds: every pixel is looked at
     for (int pixel = threadIdx.x; pixel < VH * SW; pixel += blockDim.x) {
         const unsigned int meta = sc.meta[(size_t)local * VH * SW + pixel];
-        if (!(meta & (META_FILLED | META_MASKED)) && ((meta >> META_SECTOR_SHIFT) & META_SECTOR_MASK) == 0)
+        if (!(meta & (META_FILLED | META_MASKED)) && ((meta >> META_SECTOR_SHIFT) & META_SECTOR_MASK) == 0 && !(after_billboards && (meta & META_GAP_COVERED)))
             flat_shade_pixel(dm, sc, c, local, pixel, frame);
     }
 }
@@ -3640,11 +3665,11 @@ __device__ __forceinline__ SpriteCover sprite_cover(const DeviceMap &dm, const S
 template <typename Frame>
 __device__ __forceinline__ void sprite_paint(const DeviceMap &dm, const gd_lanes_desc &lanes, const Scratch &sc, int local, int n, const LaneCtx &L,
                                              const SpriteRec *sp, const unsigned short *on_screen, const SpriteCover &cover, int x, int row_first,
-                                             int row_end, const Frame &frame) {
+                                             int row_end, const Frame &frame, bool mark_gaps = false) {
     const gd_map_desc *m = &dm.d;
     const int A = lanes.sprite_slots;
     const WallRec *recs = sc.rec + (size_t)local * m->wall_count;
-    const unsigned int *meta = sc.meta + (size_t)local * VH * SW;
+    unsigned int *meta = sc.meta + (size_t)local * VH * SW;
     int clip_wall = -1; i64 clip_near = 0, clip_far = 0; float4 clip_line = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     // painter's order far -> near: repeatedly take the farthest candidate nearer than the last one
     float last_depth = GD_INF; int last_slot = A;
@@ -3739,6 +3764,9 @@ __device__ __forceinline__ void sprite_paint(const DeviceMap &dm, const gd_lanes
                 if (style == -2) lit = m->translucent_lut[(size_t)*pixel * 256 + lit];
                 else if (style >= 0) lit = m->additive_luts[((size_t)(style > 1 ? 1 : style) * 256 + *pixel) * 256 + lit];
                 *pixel = lit;
+                // painted ahead of the flat pass's pixels (launch_chunk): a gap pixel says that it is taken
+                if (mark_gaps && !(row_meta[j] & (META_FILLED | META_MASKED)) && ((row_meta[j] >> META_SECTOR_SHIFT) & META_SECTOR_MASK) == 0)
+                    meta[(size_t)y * SW + x] = row_meta[j] | META_GAP_COVERED;
             }
         }
     }
@@ -3757,11 +3785,15 @@ __device__ __forceinline__ void sprite_column(const DeviceMap &dm, const gd_lane
 #define SPRITE_ROW_PARTS 4
 static_assert(VH % (SPRITE_ROW_PARTS * SPRITE_ROWS) == 0, "sprite_columns_kernel: row parts hold whole row batches");
 __global__ void __launch_bounds__(SPRITE_COLUMNS * SPRITE_ROW_PARTS) __attribute__((amdgpu_waves_per_eu(4, 4))) sprite_columns_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, int lane_count, Scratch sc,
-                                                            unsigned char *frame_base, size_t frame_stride) {
+                                                            unsigned char *frame_base, size_t frame_stride, int lane_pick) {
     extern __shared__ unsigned char shared_raw[];
     SpriteRec *sp = reinterpret_cast<SpriteRec *>(shared_raw);
     const int local = blockIdx.y;
     if (local >= lane_count) return;
+    // lane_pick: LANES_ALL, or one half of launch_chunk's split: LANES_PLAIN (lanes whose billboards all simply cover what is
+    // under them: painted early, marking the gap pixels they take) or LANES_BLENDING (the others, after the flat pass)
+    if (lane_pick != LANES_ALL && (sc.lane_blends[local] != 0) != (lane_pick == LANES_BLENDING)) return;   // the same in the whole block
+    const bool mark_gaps = lane_pick == LANES_PLAIN;
     const int n = lane_base + local;
     const int A = lanes.sprite_slots;
     const int x_first = blockIdx.x * SPRITE_COLUMNS, x_end = x_first + SPRITE_COLUMNS < SW ? x_first + SPRITE_COLUMNS : SW;
@@ -3788,7 +3820,7 @@ __global__ void __launch_bounds__(SPRITE_COLUMNS * SPRITE_ROW_PARTS) __attribute
 #pragma unroll
     for (int word = 0; word < 8; ++word) cover.bits[word] = word * 64 < listed ? cover_bits[word][column] : 0;
     GlobalFrame frame; frame.base = frame_base + (size_t)local * frame_stride;
-    sprite_paint(dm, lanes, sc, local, n, L, sp, on_screen, cover, x, part * (VH / SPRITE_ROW_PARTS), (part + 1) * (VH / SPRITE_ROW_PARTS), frame);
+    sprite_paint(dm, lanes, sc, local, n, L, sp, on_screen, cover, x, part * (VH / SPRITE_ROW_PARTS), (part + 1) * (VH / SPRITE_ROW_PARTS), frame, mark_gaps);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -4754,6 +4786,7 @@ size_t carve_scratch(Scratch &sc, unsigned char *base, size_t L, const gd_map_de
     take(&sc.row_slope, L * (size_t)VH);
     take(&sc.step_scale, L * STEP_TABLE);
     take(&sc.block_hit, L * SW);
+    take(&sc.lane_blends, L);
     take(&sc.strip_key, L * SEGS_PER_LANE);
     take(&sc.strip_order, L * SEGS_PER_LANE);
     if (depth) take(&sc.scene_depth, L * PX);
@@ -4981,11 +5014,26 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     mark();
     hipLaunchKernelGGL(level_masks ? flat_tail_kernel<true> : flat_tail_kernel<false>, dim3(SW / 64, count), dim3(64 * tail_rows(level_masks)), 0, stream, r->dm, *lanes, base, count, sc);
     hipLaunchKernelGGL(flat_span_finish_kernel, dim3(count), dim3(SW), 0, stream, r->dm, *lanes, base, count, sc);
-    if (!fused) hipLaunchKernelGGL(flat_shade_kernel, dim3(count), dim3(128), 0, stream, r->dm, count, sc, frame_base, frame_stride);
+    // Billboards that simply cover what lies under them need not wait for the flat pass's pixels: the lanes that hold no other
+    // kind (lane_blends, decided on the device) have theirs painted right after the shading, on the side stream, where they
+    // mark the gap pixels they take; the flat pass's pixels of those lanes are painted after the join, around the marks.  The
+    // flat chain, which waits for memory most of its time, then has the billboards beside it as well as the shading.  Lanes
+    // with a billboard that blends with the pixel below (sprite_style) keep the order flat pass, then billboards; so do
+    // frames with decals, which go between the two.
+    const bool has_billboards = lanes->sprite_slots > 0 && lanes->sprite_x;
+    const bool billboards_split = beside && has_billboards && !decals;
+    const bool may_blend = lanes->sprite_style != nullptr;   // without styles no lane blends: the launches for such lanes are left out
+    auto paint_billboards = [&](hipStream_t on, int lane_pick) {
+        const size_t shared = (size_t)lanes->sprite_slots * (sizeof(SpriteRec) + sizeof(unsigned short));
+        hipLaunchKernelGGL(sprite_columns_kernel, dim3((SW + SPRITE_COLUMNS - 1) / SPRITE_COLUMNS, count), dim3(SPRITE_COLUMNS * SPRITE_ROW_PARTS), shared, on, r->dm, *lanes, base, count, sc, frame_base, frame_stride, lane_pick);
+    };
+    if (!fused && !(billboards_split && !may_blend)) hipLaunchKernelGGL(flat_shade_kernel, dim3(count), dim3(128), 0, stream, r->dm, count, sc, frame_base, frame_stride, billboards_split ? LANES_BLENDING : LANES_ALL);
     if (beside) {
         shade_planes();
+        if (billboards_split) paint_billboards(r->side_stream, LANES_PLAIN);
         HIP_TRY(hipEventRecord(r->join_event, r->side_stream));
         HIP_TRY(hipStreamWaitEvent(stream, r->join_event, 0));
+        if (billboards_split) hipLaunchKernelGGL(flat_shade_kernel, dim3(count), dim3(128), 0, stream, r->dm, count, sc, frame_base, frame_stride, LANES_PLAIN);
     }
     mark();
     const float *blend = lanes->screen_blend ? lanes->screen_blend + 2 * (size_t)base : nullptr;
@@ -5012,10 +5060,7 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     }
     if (decals)
         hipLaunchKernelGGL(decal_kernel, dim3(count), dim3(SW), 0, stream, r->dm, r->overlays, *lanes, base, count, sc, frame_base, frame_stride);
-    if (lanes->sprite_slots > 0 && lanes->sprite_x) {
-        size_t shared = (size_t)lanes->sprite_slots * (sizeof(SpriteRec) + sizeof(unsigned short));
-        hipLaunchKernelGGL(sprite_columns_kernel, dim3((SW + SPRITE_COLUMNS - 1) / SPRITE_COLUMNS, count), dim3(SPRITE_COLUMNS * SPRITE_ROW_PARTS), shared, stream, r->dm, *lanes, base, count, sc, frame_base, frame_stride);
-    }
+    if (has_billboards && !(billboards_split && !may_blend)) paint_billboards(stream, billboards_split ? LANES_BLENDING : LANES_ALL);
     if (lanes->weapon_state && r->overlays.d.weapon_patch_count > 0)
         hipLaunchKernelGGL(weapon_overlay_kernel, dim3((VH * SW + 255) / 256, count), dim3(256), 0, stream, r->overlays, lanes->weapon_state, base, count,
                            frame_base, frame_stride);

@@ -283,14 +283,25 @@ def test_cameras_outside_the_map_match_the_oracle(oracle):
         else:
             poses.x[lane] = low[0] + along * (high[0] - low[0])
             poses.y[lane] = low[1] - away if side == 2 else high[1] + away
-    arrays = make_lane_arrays(smap, poses, synthmap.generate_sprites(smap, LANES, 24, 12))
-    expected = oracle.render(tables, arrays, cosine)
+    sprites = synthmap.generate_sprites(smap, LANES, 24, 12)
+    arrays = make_lane_arrays(smap, poses, sprites)
     renderer = HipRenderer(smap, LANES, "cuda:0", cosine_correction=cosine, tables=tables)
-    indexed = torch.zeros((LANES, 240, 320), dtype=torch.uint8, device="cuda:0")
-    obs = torch.zeros((LANES, 84, 84), dtype=torch.uint8, device="cuda:0")
-    renderer.render(LaneState.from_numpy(arrays, "cuda:0"), indexed=indexed, obs=obs)
-    torch.cuda.synchronize()
-    assert renderer.status() == 0
-    assert np.array_equal(indexed.cpu().numpy(), expected["indexed"])
-    assert np.array_equal(obs.cpu().numpy(), expected["obs"])
+    # Billboards over pixels that show the flat pass's picture, three ways: no styles at all (every lane's billboards are
+    # painted ahead of the flat pass's pixels and mark the ones they take), styles on the odd lanes only (the two kinds of
+    # lane share a frame; lane 1 of them carries a style on a dead billboard only and counts as plain), styles everywhere.
+    styles = rng.choice(np.array([-1, -2, 0, 1], dtype=np.int8), size=sprites.x.shape)
+    odd_only = styles.copy()
+    odd_only[0::2] = -1
+    odd_only[1] = np.where(arrays["sprite_alive"][1] != 0, -1, -2)
+    for case in (None, odd_only, styles):
+        if case is not None:
+            arrays["sprite_style"] = case
+        expected = oracle.render(tables, arrays, cosine)
+        indexed = torch.zeros((LANES, 240, 320), dtype=torch.uint8, device="cuda:0")
+        obs = torch.zeros((LANES, 84, 84), dtype=torch.uint8, device="cuda:0")
+        renderer.render(LaneState.from_numpy(arrays, "cuda:0"), indexed=indexed, obs=obs)
+        torch.cuda.synchronize()
+        assert renderer.status() == 0
+        assert np.array_equal(indexed.cpu().numpy(), expected["indexed"])
+        assert np.array_equal(obs.cpu().numpy(), expected["obs"])
     renderer.close()
