@@ -3360,16 +3360,16 @@ __global__ void __launch_bounds__(64 * WALL_STRIPS_PER_GROUP) __attribute__((amd
 // shades every pixel once, in a kernel light enough to run at full occupancy.
 // ---------------------------------------------------------------------------------------------
 #define SHADE_RUN 4      // neighbouring pixels of a row per thread
-#define SHADE_TILES 14   // tiles (256 runs) per block: 65 tiles per view = 5 blocks per lane (each block stages the tables once)
-#define SHADE_GROUP 2    // tiles per step
+#define SHADE_TILES 13   // tiles (256 runs) per block: 65 tiles per view = 5 blocks per lane (each block stages the tables once)
+#define SHADE_GROUP 1    // tiles per step
 static_assert(SW % SHADE_RUN == 0 && SHADE_RUN == 4, "plane_shade_kernel: a run is one 16-byte load of per-pixel words and one 4-byte store");
 // DEPTH: also keep the depth of every pixel no wall tier covers (frames that draw decals).  STAGED: the lane's plane table
 // is short enough for LDS (the kernel then reads it with LDS instructions; a pointer that may be either costs more).
 template <bool DEPTH, bool STAGED>
-// Five wavefronts per SIMD, not the eight its registers would allow at one tile per step: alone the kernel takes a
-// seventh longer that way, but it runs beside the flat pass (launch_chunk), whose kernels wait for memory more than
-// they compute and finish sooner when this one leaves them room; the two together end 0.06 ms earlier per 4096 lanes.
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5, 5))) plane_shade_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
+// Eight wavefronts per SIMD.  The kernel runs beside the flat pass (launch_chunk) and the billboards follow it on the same
+// stream: the sooner it is done, the sooner they are (with the billboards still after the flat pass, five wavefronts per
+// SIMD and two tiles per step were better: the flat pass's kernels found more room beside it).
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) plane_shade_kernel(DeviceMap dm, int lane_count, Scratch sc, unsigned char *frame_base, size_t frame_stride) {
     const gd_map_desc *m = &dm.d;
     __shared__ float4 sector_lds[LDS_SECTORS];
     __shared__ unsigned int sector_level_lds[LDS_SECTORS];
