@@ -2861,9 +2861,11 @@ __device__ __forceinline__ bool pass_advance(const ColumnCtx &cc, ColumnState &c
         auto row_of = [](float clip) { return clip <= 0.0f ? 0 : (clip >= (float)VH ? VH : (int)clip); };
         const int old_floor = row_of(before.floor_clip), old_ceiling = row_of(before.ceiling_clip);
         if (window_untouched && silhouette_folds(r)) {
-            // one call per side: the rows already done differ
-            apply_silhouette(pb, sb, x, bottom_sil, false, c.floor_clip, c.ceiling_clip, distance, wi, row_of(c.floor_clip), old_floor);
-            apply_silhouette(pb, sb, x, false, top_sil, c.floor_clip, c.ceiling_clip, distance, wi, old_ceiling, row_of(c.ceiling_clip));
+            // one call per side: the rows already done differ.  pass_paint stays inside the old window, and a sector whose
+            // ceiling lies below its floor can carry a clip past the window's other end: then the rows beyond that end
+            // are not done, and the range is cut there (apply_silhouette then takes no short cut and visits them all).
+            apply_silhouette(pb, sb, x, bottom_sil, false, c.floor_clip, c.ceiling_clip, distance, wi, max(row_of(c.floor_clip), old_ceiling), old_floor);
+            apply_silhouette(pb, sb, x, false, top_sil, c.floor_clip, c.ceiling_clip, distance, wi, old_ceiling, min(row_of(c.ceiling_clip), old_floor));
         } else {
             apply_silhouette(pb, sb, x, bottom_sil, top_sil, c.floor_clip, c.ceiling_clip, distance, wi, 0, 0);
         }

@@ -110,9 +110,9 @@ def test_random_maps_with_other_heights_and_textures_whatever_the_working_memory
         renderer.close()
 
 
-def closed_door_case(seed: int, lanes: int, *, inverted: bool = False, variants: bool = True, eye_any: bool = False):
+def closed_door_case(seed: int, lanes: int, *, inverted: bool = False, variants: bool = True, eye_any: bool = False, mixed: bool = False):
     """random_case plus hand-closed doors and crawl spaces on up to four sectors (``inverted``: ceilings 16 units below
-    their floors instead), then (``variants``: seven times in ten) other heights, texture sizes and lights over the whole
+    their floors instead; ``mixed``: each of the four one of the three kinds), then (``variants``: seven times in ten) other heights, texture sizes and lights over the whole
     map; ``eye_any``: six times in ten the eyes stand at any height, not between their sector's floor and ceiling."""
     from gradoom_amd import mapbuild, synthmap
     from gradoom_amd.selfcheck import make_lane_arrays
@@ -125,7 +125,9 @@ def closed_door_case(seed: int, lanes: int, *, inverted: bool = False, variants:
         heights = np.array(smap.sector_heights, copy=True)
         for sector in rng.choice(len(heights), size=min(4, len(heights)), replace=False):
             kind = int(rng.choice([0, 2]))
-            if inverted:
+            if mixed:
+                kind = int(rng.integers(0, 3))
+            if inverted or kind == 1:
                 heights[sector, 1] = heights[sector, 0] - 16   # a ceiling below its floor
             elif kind == 0:
                 heights[sector, 1] = heights[sector, 0]        # a closed door
@@ -208,6 +210,34 @@ def test_sectors_with_ceilings_below_their_floors_match_the_oracle(oracle, seed,
         assert renderer.status() == 0
         assert np.array_equal(indexed.cpu().numpy(), expected["indexed"]), f"seed {seed} fill {fill} {assembly}"
         assert np.array_equal(obs.cpu().numpy(), expected["obs"]), f"seed {seed} fill {fill} {assembly}"
+    renderer.close()
+
+
+def test_a_ceiling_clip_carried_below_the_floor_clip_still_records_its_silhouette(oracle):
+    """A zero-height sector closes a column's window at row 94; behind it a sector with its ceiling below its floor moves
+    the ceiling clip on to row 130, past the floor clip.  Nothing is painted in the rows between, yet the pass's top
+    silhouette reaches over them, and being nearer by a rounding error (three linedefs meet in that column) than the
+    bottom silhouette of the pass before, it decides whether a billboard behind shows there (engine.py:12943-12964)."""
+    from gradoom_amd import hostmath
+    from gradoom_amd.renderer import HipRenderer, LaneState
+
+    lanes = 16
+    cosine = hostmath.cosine_correction("cpu").numpy()
+    smap, tables, arrays = closed_door_case(503259, lanes, mixed=True, variants=True, eye_any=True)
+    heights = np.asarray(smap.sector_heights)
+    assert (heights[:, 1] < heights[:, 0]).any() and (heights[:, 1] == heights[:, 0]).any()
+    expected = oracle.render(tables, arrays, cosine)
+    renderer = HipRenderer(smap, lanes, "cuda:0", cosine_correction=cosine, tables=tables)
+    state = LaneState.from_numpy(arrays, "cuda:0")
+    for assembly in ("separate", "fused"):
+        renderer.set_assembly(assembly)
+        indexed = torch.zeros((lanes, 240, 320), dtype=torch.uint8, device="cuda:0")
+        obs = torch.zeros((lanes, 84, 84), dtype=torch.uint8, device="cuda:0")
+        renderer.render(state, indexed=indexed, obs=obs)
+        torch.cuda.synchronize()
+        assert renderer.status() == 0
+        assert np.array_equal(indexed.cpu().numpy(), expected["indexed"]), assembly
+        assert np.array_equal(obs.cpu().numpy(), expected["obs"]), assembly
     renderer.close()
 
 
