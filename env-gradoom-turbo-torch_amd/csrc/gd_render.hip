@@ -1832,6 +1832,12 @@ struct ColumnCtx {
     int count;
     int x;
     float rx, ry;
+    // wall_select_kernel's staged launch: this column's list copied to LDS (entry k at staged + k * 1024 bytes: a row of
+    // 64 columns), null everywhere else.  (One or the other for a whole kernel: a choice per load would become one flat
+    // load of a selected address.)
+    typedef __attribute__((address_space(3))) const char LdsByte;
+    LdsByte *staged;
+    bool use_staged = false;
     __device__ __forceinline__ const WallRec &rec(int w) const { return recs[rec_base + (unsigned)w]; }
     // Where the list of column `x` of the chunk's lane `local` starts and how many entries it has: the column's own
     // slots, or its slot in the spill pool.
@@ -1849,8 +1855,11 @@ struct ColumnCtx {
         }
     }
     __device__ __forceinline__ Cand cand(int k) const {
-        union { uint4 raw; Cand c; } u;
-        u.raw = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(list) + (list_column + (unsigned)k * (SW * 16u)));   // one 16-byte load
+        typedef unsigned int Words4 __attribute__((ext_vector_type(4)));
+        typedef __attribute__((address_space(3))) const Words4 LdsEntry;
+        union { uint4 raw; Words4 words; Cand c; } u;
+        if (use_staged) u.words = *(LdsEntry *)(staged + (unsigned)k * (64 * 16u));   // all of the list is there
+        else u.raw = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(list) + (list_column + (unsigned)k * (SW * 16u)));   // one 16-byte load
         return u.c;
     }
     // Entries k0 .. k0+CAND_BATCH-1 of this column's list, loaded together so that their memory
@@ -3176,15 +3185,23 @@ __global__ void __launch_bounds__(1024) strip_order_kernel(int strips, Scratch s
 // Each half is lighter in registers and in code than the two together, so more of its wavefronts share a SIMD and
 // its pass loop fits the instruction cache.  Same segment order and one wavefront per segment in both.
 #define SELECT_STRIPS_PER_GROUP 1
-template <bool SPLIT>
-__global__ void __launch_bounds__(64 * SELECT_STRIPS_PER_GROUP) wall_select_kernel(DeviceMap dm, int lane_count, Scratch sc) {
+// The kernel lasts as long as its longest strips: on the 4000-linedef map the 256 longest of 20,480 take 0.94 ms with the
+// chip to themselves, all of them together 1.22 ms, all but the 4096 longest 0.53 ms.  What a lone wavefront waits for is
+// its candidate scans, each a chain of trips to device memory.  So the SELECT_STAGED_STRIPS longest strips (they lead the
+// order) go to a launch of their own (STAGED) that first copies each column's list to LDS, 64 KB a wavefront, and scans
+// it there; it runs on the renderer's side stream beside the launch for all other strips.
+#define SELECT_STAGED_STRIPS 512
+static_assert(SEG_COLS == 64 && SELECT_STRIPS_PER_GROUP == 1, "wall_select_kernel's staged launch: one whole strip per work-group");
+template <bool SPLIT, bool STAGED>
+__global__ void __launch_bounds__(64 * SELECT_STRIPS_PER_GROUP) wall_select_kernel(DeviceMap dm, int lane_count, Scratch sc, int staged_slots) {
     const gd_map_desc *m = &dm.d;
     __shared__ LaneCtx lane_ctxs[SELECT_STRIPS_PER_GROUP][64 / SEG_COLS];
+    __shared__ uint4 staged_entries[STAGED ? CAND_MAX * 64 : 1];   // [CAND_MAX][64] in the staged launch
     const int wave_in_group = threadIdx.x >> 6;
     const int lane_id = threadIdx.x & 63;
     const int segment_in_wave = lane_id / SEG_COLS;
     const int segment_slot = (blockIdx.x * SELECT_STRIPS_PER_GROUP + wave_in_group) * (64 / SEG_COLS) + segment_in_wave;
-    const bool live = segment_slot < lane_count * SEGS_PER_LANE;
+    const bool live = segment_slot < (STAGED ? staged_slots : lane_count * SEGS_PER_LANE);
     const int segment = live ? sc.strip_order[segment_slot] : 0;
     const int local = segment / SEGS_PER_LANE;
     if ((lane_id & (SEG_COLS - 1)) == 0 && live) lane_ctxs[wave_in_group][segment_in_wave] = sc.ctx[local];
@@ -3200,6 +3217,27 @@ __global__ void __launch_bounds__(64 * SELECT_STRIPS_PER_GROUP) wall_select_kern
     cc.set_list(sc, local, x);
     cc.x = x;
     ray_direction(lane_ctx, x, &cc.rx, &cc.ry);
+    // A strip with a column in the spill pool (more entries than the LDS copy holds) is left to the other launch, which
+    // covers the staged launch's slots as well and otherwise leaves them alone.
+    const bool long_lists = __ballot(cc.count > CAND_MAX) != 0;
+    if (STAGED ? long_lists : (segment_slot < staged_slots && !long_lists)) return;   // the same in the whole wavefront
+    if (STAGED) {
+        // every lane copies its own column's entries and reads only those: no barrier
+        char *mine = reinterpret_cast<char *>(staged_entries) + lane_id * 16;
+        const int depth = cc.count;
+        for (int k0 = 0; k0 < depth; k0 += CAND_BATCH) {
+            Cand batch[CAND_BATCH];
+            cc.cand_batch(k0, batch);
+#pragma unroll
+            for (int j = 0; j < CAND_BATCH; ++j) {
+                union { uint4 raw; Cand c; } u;
+                u.c = batch[j];
+                if (k0 + j < depth) *reinterpret_cast<uint4 *>(mine + (k0 + j) * (64 * 16)) = u.raw;
+            }
+        }
+        cc.staged = (ColumnCtx::LdsByte *)mine;
+        cc.use_staged = true;
+    }
     ColumnState st;
     st.current_sector = lane_ctx.sector;
     st.ceiling_clip = 0.0f; st.floor_clip = (float)VH;
@@ -4973,8 +5011,25 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     {
         const int wavefronts = (count * SEGS_PER_LANE + 64 / SEG_COLS - 1) / (64 / SEG_COLS);
         const bool split = m.split_count > 0;
-        const dim3 select_grid((wavefronts + SELECT_STRIPS_PER_GROUP - 1) / SELECT_STRIPS_PER_GROUP), select_block(64 * SELECT_STRIPS_PER_GROUP);
-        hipLaunchKernelGGL(split ? wall_select_kernel<true> : wall_select_kernel<false>, select_grid, select_block, 0, stream, r->dm, count, sc);
+        const dim3 select_block(64 * SELECT_STRIPS_PER_GROUP);
+        // The longest strips here with their lists in LDS, the others on the side stream, both at once.  This way round: the
+        // side stream starts a few microseconds behind, time enough for the staged launch's work-groups (64 KB of LDS each,
+        // two to a compute unit) to be placed; started together, the other launch's 20,000 take every wavefront slot first
+        // and the strips that decide how long the pair lasts begin last.
+        const int strips = count * SEGS_PER_LANE;
+        const int staged_strips = r->side_ready ? (strips < SELECT_STAGED_STRIPS ? strips : SELECT_STAGED_STRIPS) : 0;
+        auto select_kernel = split ? wall_select_kernel<true, false> : wall_select_kernel<false, false>;
+        if (staged_strips > 0) {
+            HIP_TRY(hipEventRecord(r->fork_event, stream));
+            HIP_TRY(hipStreamWaitEvent(r->side_stream, r->fork_event, 0));
+            auto staged_kernel = split ? wall_select_kernel<true, true> : wall_select_kernel<false, true>;
+            hipLaunchKernelGGL(staged_kernel, dim3(staged_strips), select_block, 0, stream, r->dm, count, sc, staged_strips);
+            hipLaunchKernelGGL(select_kernel, dim3(strips), select_block, 0, r->side_stream, r->dm, count, sc, staged_strips);
+            HIP_TRY(hipEventRecord(r->join_event, r->side_stream));
+            HIP_TRY(hipStreamWaitEvent(stream, r->join_event, 0));
+        } else {
+            hipLaunchKernelGGL(select_kernel, dim3(strips), select_block, 0, stream, r->dm, count, sc, 0);
+        }
         mark();
         const dim3 grid((wavefronts + WALL_STRIPS_PER_GROUP - 1) / WALL_STRIPS_PER_GROUP), block(64 * WALL_STRIPS_PER_GROUP);
         auto kernel = decals ? (split ? wall_raster_kernel<true, true> : wall_raster_kernel<true, false>)
