@@ -126,11 +126,19 @@ struct RecSpan {   // what a ray test of one linedef needs (eval_segment), kept 
 
 struct __align__(16) Cand {      // one linedef with a finite ray distance at one column, with the static
                    // linedef facts every scan needs packed in so that scans do no gathers
-    unsigned short wall, flags;
+    unsigned short flags, wall;   // in this order: the entry's first word under its last is the key below
     short s0, s1;            // front / back sector (-1 = none)
     unsigned short v0, v1;   // vertex ids of start / end
     float dist;
 };
+// (distance, linedef, flags) of a candidate as one unsigned number.  Listed distances are positive, so their bit patterns
+// order as they do: the smallest key is the nearest candidate, the lowest linedef on ties, which is how every scan of the
+// traversal breaks them (no column lists a linedef twice).  CAND_KEY_NONE, greater than any entry's, stands for "none".
+#define CAND_KEY_NONE 0x7F800000FFFFFFFFULL
+__device__ __forceinline__ u64 cand_key(const Cand &q) { return ((u64)__float_as_uint(q.dist) << 32) | ((u64)q.wall << 16) | (u64)q.flags; }
+__device__ __forceinline__ float cand_key_distance(u64 key) { return __uint_as_float((unsigned)(key >> 32)); }
+__device__ __forceinline__ int cand_key_wall(u64 key) { return key == CAND_KEY_NONE ? 0x7fffffff : (int)((unsigned)key >> 16); }
+__device__ __forceinline__ int cand_key_flags(u64 key) { return key == CAND_KEY_NONE ? 0 : (int)((unsigned)key & 0xFFFFu); }
 
 struct Eval {      // distances/along/geometric/projected/left-edge of one linedef at one column;
                    // CF_ALONG_HI in flags carries (along > 0.5), the only use the traversal makes of along
@@ -1818,6 +1826,8 @@ __global__ void __launch_bounds__(SW) flat_span_finish_kernel(DeviceMap dm, gd_l
 // walls: engine.py:11462-13745
 // ---------------------------------------------------------------------------------------------
 #define CAND_BATCH 8
+#define SELECT_STAGED_STRIPS 512   // wall_select_kernel's launch for the longest strips: how many strips,
+#define SELECT_STAGED_PARTS 4      // and over how many wavefronts each is shared out
 #define WALL_ROWS 8          // rows painted / clipped per step of the wall traversal
 struct ColumnCtx {
     const Tables *tb;
@@ -1832,8 +1842,8 @@ struct ColumnCtx {
     int count;
     int x;
     float rx, ry;
-    // wall_select_kernel's staged launch: this column's list copied to LDS (entry k at staged + k * 1024 bytes: a row of
-    // 64 columns), null everywhere else.  (One or the other for a whole kernel: a choice per load would become one flat
+    // wall_select_kernel's staged launch: this column's list copied to LDS (entry k at staged + k * 256 bytes: a row of
+    // the wavefront's 16 columns), unused everywhere else.  (One or the other for a whole kernel: a choice per load would become one flat
     // load of a selected address.)
     typedef __attribute__((address_space(3))) const char LdsByte;
     LdsByte *staged;
@@ -1858,7 +1868,7 @@ struct ColumnCtx {
         typedef unsigned int Words4 __attribute__((ext_vector_type(4)));
         typedef __attribute__((address_space(3))) const Words4 LdsEntry;
         union { uint4 raw; Words4 words; Cand c; } u;
-        if (use_staged) u.words = *(LdsEntry *)(staged + (unsigned)k * (64 * 16u));   // all of the list is there
+        if (use_staged) u.words = *(LdsEntry *)(staged + (unsigned)k * (64 / SELECT_STAGED_PARTS * 16u));   // all of the list is there
         else u.raw = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(list) + (list_column + (unsigned)k * (SW * 16u)));   // one 16-byte load
         return u.c;
     }
@@ -2251,23 +2261,27 @@ __device__ __forceinline__ void pass_select(const ColumnCtx &cc, const ColumnSta
         incident_beyond = 0;
         // b. equal-depth solid (engine.py:11784-11807): the nearest one-sided candidate replaces
         // the selection when it lies within 1e-3 of the nearest candidate, found in the same scan.
-        float sd = GD_INF; int swi = 0x7fffffff;
-        int wi_flags = 0, swi_flags = 0;
+        u64 nearest = CAND_KEY_NONE, nearest_solid = CAND_KEY_NONE;
         for (int k0 = 0; k0 < cc.count; k0 += CAND_BATCH) {
             Cand batch[CAND_BATCH];
             cc.cand_batch(k0, batch);
+            unsigned batch_bits = 0u;
 #pragma unroll
             for (int j = 0; j < CAND_BATCH; ++j) {
-                if (k0 + j >= cc.count) continue;
                 const Cand q = batch[j];
-                if (!(incident_c(q) && q.dist > prev)) continue;
-                incident_beyond |= 1ULL << ((k0 + j) & 63);
-                if (q.dist < distance || (q.dist == distance && (int)q.wall < wi)) { distance = q.dist; wi = q.wall; wi_flags = q.flags; }
-                if ((q.s1 < 0) && (q.dist < sd || (q.dist == sd && (int)q.wall < swi))) { sd = q.dist; swi = q.wall; swi_flags = q.flags; }
+                const bool hit = k0 + j < cc.count && incident_c(q) && q.dist > prev;
+                batch_bits |= hit ? 1u << j : 0u;
+                const u64 key = hit ? cand_key(q) : CAND_KEY_NONE;
+                nearest = key < nearest ? key : nearest;
+                const u64 solid_key = q.s1 < 0 ? key : CAND_KEY_NONE;
+                nearest_solid = solid_key < nearest_solid ? solid_key : nearest_solid;
             }
+            incident_beyond |= (u64)batch_bits << (k0 & 63);
         }
-        if (finitef(sd) && (fabsf(sd - distance) <= 1e-3f)) { distance = sd; wi = swi; wi_flags = swi_flags; }
-        cwi.dist = distance; cwi.flags = wi_flags;
+        const float sd = cand_key_distance(nearest_solid);
+        if (finitef(sd) && (fabsf(sd - cand_key_distance(nearest)) <= 1e-3f)) nearest = nearest_solid;
+        distance = cand_key_distance(nearest); wi = cand_key_wall(nearest);
+        cwi.dist = distance; cwi.flags = cand_key_flags(nearest);
     }
     if (!finitef(distance)) { wi = 0; cwi = cc.eval(0); }
     // c. selected endpoint (engine.py:11815-11871)
@@ -3186,21 +3200,25 @@ __global__ void __launch_bounds__(1024) strip_order_kernel(int strips, Scratch s
 // its pass loop fits the instruction cache.  Same segment order and one wavefront per segment in both.
 #define SELECT_STRIPS_PER_GROUP 1
 // The kernel lasts as long as its longest strips: on the 4000-linedef map the 256 longest of 20,480 take 0.94 ms with the
-// chip to themselves, all of them together 1.22 ms, all but the 4096 longest 0.53 ms.  What a lone wavefront waits for is
-// its candidate scans, each a chain of trips to device memory.  So the SELECT_STAGED_STRIPS longest strips (they lead the
-// order) go to a launch of their own (STAGED) that first copies each column's list to LDS, 64 KB a wavefront, and scans
-// it there; it runs on the renderer's side stream beside the launch for all other strips.
-#define SELECT_STAGED_STRIPS 512
-static_assert(SEG_COLS == 64 && SELECT_STRIPS_PER_GROUP == 1, "wall_select_kernel's staged launch: one whole strip per work-group");
+// chip to themselves, all of them together 1.22 ms, all but the 4096 longest 0.53 ms.  Such a strip's wavefront is held
+// up by its candidate scans (the longest lists, read from device memory beside 20,000 other wavefronts) and by running,
+// pass after pass, every rule that any of its 64 columns takes.  So the SELECT_STAGED_STRIPS longest strips (they lead
+// the order) go to a launch of their own (STAGED): a strip is shared out over SELECT_STAGED_PARTS wavefronts of 16 columns
+// each, which first copy their columns' lists to LDS (16 KB a wavefront) and scan them there.  It runs beside the
+// launch for all other strips: 1.22 -> 0.99 ms.  (Measured: 256 to 1024 strips, 1, 2, 4 or 8 parts; lists left in device
+// memory: no gain.)
+static_assert(SEG_COLS == 64 && SELECT_STRIPS_PER_GROUP == 1, "wall_select_kernel's staged launch: parts of one whole strip per work-group");
 template <bool SPLIT, bool STAGED>
 __global__ void __launch_bounds__(64 * SELECT_STRIPS_PER_GROUP) wall_select_kernel(DeviceMap dm, int lane_count, Scratch sc, int staged_slots) {
     const gd_map_desc *m = &dm.d;
     __shared__ LaneCtx lane_ctxs[SELECT_STRIPS_PER_GROUP][64 / SEG_COLS];
-    __shared__ uint4 staged_entries[STAGED ? CAND_MAX * 64 : 1];   // [CAND_MAX][64] in the staged launch
+    constexpr int PARTS = STAGED ? SELECT_STAGED_PARTS : 1, PART_COLS = 64 / PARTS;
+    __shared__ uint4 staged_entries[STAGED ? CAND_MAX * PART_COLS : 1];   // [CAND_MAX][PART_COLS] in the staged launch
     const int wave_in_group = threadIdx.x >> 6;
     const int lane_id = threadIdx.x & 63;
     const int segment_in_wave = lane_id / SEG_COLS;
-    const int segment_slot = (blockIdx.x * SELECT_STRIPS_PER_GROUP + wave_in_group) * (64 / SEG_COLS) + segment_in_wave;
+    const int segment_slot = (blockIdx.x / PARTS * SELECT_STRIPS_PER_GROUP + wave_in_group) * (64 / SEG_COLS) + segment_in_wave;
+    const int part = blockIdx.x % PARTS;
     const bool live = segment_slot < (STAGED ? staged_slots : lane_count * SEGS_PER_LANE);
     const int segment = live ? sc.strip_order[segment_slot] : 0;
     const int local = segment / SEGS_PER_LANE;
@@ -3208,7 +3226,13 @@ __global__ void __launch_bounds__(64 * SELECT_STRIPS_PER_GROUP) wall_select_kern
     __syncthreads();
     if (!live) return;
     const LaneCtx &lane_ctx = lane_ctxs[wave_in_group][segment_in_wave];
-    const int x = (segment - local * SEGS_PER_LANE) * SEG_COLS + (lane_id & (SEG_COLS - 1));
+    // A strip with a column in the spill pool (more entries than the LDS copy holds) is left to the other launch, which
+    // covers the staged launch's slots as well and otherwise leaves them alone.  Both ask all 64 columns of the strip.
+    const int strip_x = (segment - local * SEGS_PER_LANE) * SEG_COLS;
+    const bool long_lists = __ballot(((unsigned)sc.cand_count[(size_t)local * SW + strip_x + lane_id] >> SPILL_SHIFT) != 0) != 0;
+    if (STAGED ? long_lists : (segment_slot < staged_slots && !long_lists)) return;   // the same in the whole wavefront
+    if (lane_id >= PART_COLS) return;
+    const int x = strip_x + part * PART_COLS + lane_id;
     ColumnCtx cc;
     cc.tb = nullptr; cc.m = m; cc.mv.m = m; cc.c = &lane_ctx;
     cc.recs = sc.rec; cc.spans = sc.span;
@@ -3217,10 +3241,6 @@ __global__ void __launch_bounds__(64 * SELECT_STRIPS_PER_GROUP) wall_select_kern
     cc.set_list(sc, local, x);
     cc.x = x;
     ray_direction(lane_ctx, x, &cc.rx, &cc.ry);
-    // A strip with a column in the spill pool (more entries than the LDS copy holds) is left to the other launch, which
-    // covers the staged launch's slots as well and otherwise leaves them alone.
-    const bool long_lists = __ballot(cc.count > CAND_MAX) != 0;
-    if (STAGED ? long_lists : (segment_slot < staged_slots && !long_lists)) return;   // the same in the whole wavefront
     if (STAGED) {
         // every lane copies its own column's entries and reads only those: no barrier
         char *mine = reinterpret_cast<char *>(staged_entries) + lane_id * 16;
@@ -3232,7 +3252,7 @@ __global__ void __launch_bounds__(64 * SELECT_STRIPS_PER_GROUP) wall_select_kern
             for (int j = 0; j < CAND_BATCH; ++j) {
                 union { uint4 raw; Cand c; } u;
                 u.c = batch[j];
-                if (k0 + j < depth) *reinterpret_cast<uint4 *>(mine + (k0 + j) * (64 * 16)) = u.raw;
+                if (k0 + j < depth) *reinterpret_cast<uint4 *>(mine + (k0 + j) * (PART_COLS * 16)) = u.raw;
             }
         }
         cc.staged = (ColumnCtx::LdsByte *)mine;
@@ -5013,9 +5033,9 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
         const bool split = m.split_count > 0;
         const dim3 select_block(64 * SELECT_STRIPS_PER_GROUP);
         // The longest strips here with their lists in LDS, the others on the side stream, both at once.  This way round: the
-        // side stream starts a few microseconds behind, time enough for the staged launch's work-groups (64 KB of LDS each,
-        // two to a compute unit) to be placed; started together, the other launch's 20,000 take every wavefront slot first
-        // and the strips that decide how long the pair lasts begin last.
+        // side stream starts a few microseconds behind, time enough for the staged launch's work-groups to be placed;
+        // started together, the other launch's 20,000 take every wavefront slot first and the strips that decide how long
+        // the pair lasts begin last.
         const int strips = count * SEGS_PER_LANE;
         const int staged_strips = r->side_ready ? (strips < SELECT_STAGED_STRIPS ? strips : SELECT_STAGED_STRIPS) : 0;
         auto select_kernel = split ? wall_select_kernel<true, false> : wall_select_kernel<false, false>;
@@ -5023,7 +5043,7 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
             HIP_TRY(hipEventRecord(r->fork_event, stream));
             HIP_TRY(hipStreamWaitEvent(r->side_stream, r->fork_event, 0));
             auto staged_kernel = split ? wall_select_kernel<true, true> : wall_select_kernel<false, true>;
-            hipLaunchKernelGGL(staged_kernel, dim3(staged_strips), select_block, 0, stream, r->dm, count, sc, staged_strips);
+            hipLaunchKernelGGL(staged_kernel, dim3(staged_strips * SELECT_STAGED_PARTS), select_block, 0, stream, r->dm, count, sc, staged_strips);
             hipLaunchKernelGGL(select_kernel, dim3(strips), select_block, 0, r->side_stream, r->dm, count, sc, staged_strips);
             HIP_TRY(hipEventRecord(r->join_event, r->side_stream));
             HIP_TRY(hipStreamWaitEvent(stream, r->join_event, 0));
