@@ -1424,62 +1424,64 @@ __global__ void __launch_bounds__(GAP_THREADS) __attribute__((amdgpu_waves_per_e
     for (int k = threadIdx.x; k < columns; k += blockDim.x) sc.gap_columns[list_base + k] = column_list[k];
 }
 
-// The vertical repair (engine.py:11026-11083) of the listed gap pixels, column by column: one wavefront per listed column
-// (flat_gap_column_kernel's work list), its lanes probing 64 rows of the column at a time, from the bottom of the half up
-// to the column's topmost unresolved listed pixel.
+// The vertical repair (engine.py:11026-11083) of the listed gap pixels, column by column: one work-group per listed column
+// (flat_gap_column_kernel's work list), one wavefront per chunk of 64 rows between the column's topmost unresolved listed
+// pixel and the bottom of its half, all chunks probed at once.  What a chunk needs from the chunks below it (the sector of
+// the next resolved pixel down) goes through LDS once every chunk has probed: a column lasts as long as its slowest
+// pixel's walk over the plane levels, not as long as one such walk per chunk.
 #define GAP_REPAIR_BLOCKS 8192
-__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(8, 8))) flat_gap_repair_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, Scratch sc) {
+#define GAP_REPAIR_CHUNKS ((VH + 63) / 64)
+__global__ void __launch_bounds__(64 * GAP_REPAIR_CHUNKS) __attribute__((amdgpu_waves_per_eu(8, 8))) flat_gap_repair_kernel(DeviceMap dm, gd_lanes_desc lanes, int lane_base, Scratch sc) {
     __shared__ LevelLds level_lds;
+    __shared__ int chunk_found[GAP_REPAIR_CHUNKS], chunk_sector[GAP_REPAIR_CHUNKS];
     const int total = *sc.gap_column_count;
-    const int lane_id = threadIdx.x;
+    const int lane_id = threadIdx.x & 63, chunk = threadIdx.x >> 6;
     int staged = -1;
     LevelLists lists;
     for (int entry = blockIdx.x; entry < total; entry += gridDim.x) {
         const int packed = sc.gap_columns[entry];
         const int x = packed & 511, first = (packed >> 9) & 255, half = (packed >> 17) & 1, local = packed >> 18;
+        __syncthreads();         // nobody reads the previous column's chunk results or the previous lane's lists any more
         if (local != staged) {   // the same in every thread
-            __syncthreads();     // nobody reads the previous lane's lists any more
             lists = stage_level_lists(dm, sc, local, &level_lds);
-            __syncthreads();
             staged = local;
         }
+        __syncthreads();
         const LaneCtx &c = sc.ctx[local];
         const int n = lane_base + local;
         int *span = sc.flat_span + (size_t)local * 4;
         const unsigned int *meta = sc.meta + (size_t)local * VH * SW;
         const int half_end = half ? VH - 1 : c.last_ceiling_row;
         const float rc = lanes.ray_cos[(size_t)n * SW + x], rs = lanes.ray_sin[(size_t)n * SW + x], cc = dm.cosine_correction[x];
-        // chunks of 64 rows, the lowest first: what a chunk finds serves the chunks above it
+        const int chunks = (half_end - first) / 64 + 1;   // at most GAP_REPAIR_CHUNKS
+        const int y = first + chunk * 64 + lane_id;
+        const bool live = chunk < chunks && y <= half_end;
+        const int s = live ? flat_probe_pixel(dm, sc, lists, local, rc, rs, cc, y) : -1;
+        const u64 resolved = __ballot(live && s >= 0);
+        const int first_sector = __shfl(s, resolved ? __ffsll((long long)resolved) - 1 : 0);
+        if (lane_id == 0) { chunk_found[chunk] = resolved != 0; chunk_sector[chunk] = first_sector; }
+        __syncthreads();
+        // the next resolved pixel below: in this chunk, else the topmost one of the nearest chunk below that has any
         bool below_found = false; int below_sector = 0;
-        const int chunks = (half_end - first) / 64 + 1;
-        for (int chunk = chunks - 1; chunk >= 0; --chunk) {
-            const int y = first + chunk * 64 + lane_id;
-            const bool live = y <= half_end;
-            const int s = live ? flat_probe_pixel(dm, sc, lists, local, rc, rs, cc, y) : -1;
-            const u64 resolved = __ballot(live && s >= 0);
-            const u64 lower = resolved & ~((2ULL << lane_id) - 1);   // resolved rows of this chunk below this one (none for lane 63)
-            const int from = lower ? __ffsll((long long)lower) - 1 : lane_id;
-            const int taken = __shfl(s, from);
-            const bool found = lower ? true : below_found;
-            const int sector = lower ? taken : below_sector;
-            if (live && s < 0) {
-                const size_t i = (size_t)y * SW + x;
-                const unsigned int word = meta[i];
-                const bool listed = !(word & (META_FILLED | META_MASKED)) && ((word >> META_SECTOR_SHIFT) & META_SECTOR_MASK) == 0;
-                if (listed) {
-                    if (found && sector != c.sector) {
-                        sc.flat_sector[(size_t)local * VH * SW + i] = (unsigned short)sector;
-                        sc.flat_flags[(size_t)local * VH * SW + i] = (unsigned char)(1 | 2 | 4 | 8);
-                    } else {
-                        atomicMin(&span[half ? 2 : 0], y);
-                        atomicMax(&span[half ? 3 : 1], y);
-                    }
+        for (int lower_chunk = chunk + 1; lower_chunk < chunks && !below_found; ++lower_chunk)
+            if (chunk_found[lower_chunk]) { below_found = true; below_sector = chunk_sector[lower_chunk]; }
+        const u64 lower = resolved & ~((2ULL << lane_id) - 1);   // resolved rows of this chunk below this one (none for lane 63)
+        const int from = lower ? __ffsll((long long)lower) - 1 : lane_id;
+        const int taken = __shfl(s, from);
+        const bool found = lower ? true : below_found;
+        const int sector = lower ? taken : below_sector;
+        if (live && s < 0) {
+            const size_t i = (size_t)y * SW + x;
+            const unsigned int word = meta[i];
+            const bool listed = !(word & (META_FILLED | META_MASKED)) && ((word >> META_SECTOR_SHIFT) & META_SECTOR_MASK) == 0;
+            if (listed) {
+                if (found && sector != c.sector) {
+                    sc.flat_sector[(size_t)local * VH * SW + i] = (unsigned short)sector;
+                    sc.flat_flags[(size_t)local * VH * SW + i] = (unsigned char)(1 | 2 | 4 | 8);
+                } else {
+                    atomicMin(&span[half ? 2 : 0], y);
+                    atomicMax(&span[half ? 3 : 1], y);
                 }
-            }
-            if (resolved) {
-                const int first_resolved = __ffsll((long long)resolved) - 1;
-                below_sector = __shfl(s, first_resolved);
-                below_found = true;
             }
         }
     }
@@ -5083,7 +5085,7 @@ int launch_chunk(gd_renderer *r, const Scratch &chunk_scratch, const gd_lanes_de
     mark();
     // the flat pass, where the walls left it something to decide
     hipLaunchKernelGGL(flat_gap_column_kernel, dim3(count), dim3(GAP_THREADS), 0, stream, r->dm, *lanes, base, count, sc);
-    hipLaunchKernelGGL(flat_gap_repair_kernel, dim3(GAP_REPAIR_BLOCKS), dim3(64), 0, stream, r->dm, *lanes, base, sc);
+    hipLaunchKernelGGL(flat_gap_repair_kernel, dim3(GAP_REPAIR_BLOCKS), dim3(64 * GAP_REPAIR_CHUNKS), 0, stream, r->dm, *lanes, base, sc);
     hipLaunchKernelGGL(flat_rows_kernel, dim3(count), dim3(64), 0, stream, count, sc);
     const int plane_levels = m.floor_level_count + m.ceil_level_count;
     const bool level_masks = plane_levels > LEVEL_MASK_MIN_LEVELS && plane_levels <= 32 * LEVEL_MASK_WORDS_MAX;   // level_mask_words() > 0
