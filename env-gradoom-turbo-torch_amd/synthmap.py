@@ -619,12 +619,14 @@ def generate_picked_poses(
     flash_light = np.zeros(lanes, dtype=np.int64)
     sector = np.zeros(lanes, dtype=np.int32)
     sector_count = len(smap.sector_heights)
+    if lanes and not np.any(smap.sector_heights[:, 1] - smap.sector_heights[:, 0] >= 56.0):
+        raise ValueError("no sector of the map is high enough for a camera to stand in (56 units)")
     for slot, (seed, lane) in enumerate(picks):
         rng = np.random.default_rng((seed * 65536 + lane) * 4096 + frame)
         s = int(rng.integers(0, sector_count))
         while smap.sector_heights[s, 1] - smap.sector_heights[s, 0] < 56.0:   # no room to stand (closed doors, crawl spaces)
             s = int(rng.integers(0, sector_count))
-        while True:
+        for attempt in range(10000):
             u, v = rng.uniform(margin, 1.0 - margin, 2)
             px, py = _point_in_cell(smap, s, float(u), float(v))
             if smap.void_boxes is None or not np.any(
@@ -632,6 +634,8 @@ def generate_picked_poses(
                 & (py > smap.void_boxes[:, 1] - 4) & (py < smap.void_boxes[:, 3] + 4)
             ):
                 break
+        else:
+            raise ValueError(f"sector {s} has no spot clear of the map's void boxes for a camera")
         x[slot], y[slot] = px, py
         angle_bam[slot] = int(rng.integers(0, 1 << 32))
         view_z[slot] = smap.sector_heights[s, 0] + 41.0

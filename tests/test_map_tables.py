@@ -195,3 +195,13 @@ def test_closed_doors_and_ceilings_below_floors_build():
     smap.sector_heights[2, 1] = smap.sector_heights[2, 0] - 16
     tables = mapbuild.build_map_tables(smap)
     assert smap.sector_heights[2, 1] in tables["ceil_levels"] and smap.sector_heights[2, 0] in tables["floor_levels"]
+
+
+def test_pose_generator_refuses_a_map_with_no_room_to_stand():
+    # every sector lower than a standing camera: the generator says so instead of drawing sectors for ever
+    from gradoom_amd import synthmap
+
+    smap = synthmap.generate_map(3, grid=(3, 3), sectors=8, linedefs=80)
+    smap.sector_heights[:, 1] = smap.sector_heights[:, 0] + 40.0
+    with pytest.raises(ValueError, match="high enough"):
+        synthmap.generate_poses(smap, 2, 1)
