@@ -40,6 +40,13 @@ def load_fixture(name: str):
 
     data = dict(np.load(os.path.join(FIXTURE_DIR, f"{name}.npz")))
     meta = ast.literal_eval(str(data.pop("meta")))
+    if meta.get("recipe"):   # a case of tests/random_cases.py
+        import random_cases
+
+        recipe = dict(meta["recipe"])
+        smap = random_cases.closed_door_parts(recipe.pop("seed"), meta["lanes"], **recipe)[0]
+        assert map_digest(smap) == meta["map_sha256"], "random case generator drifted from the golden fixtures"
+        return meta, data, smap, mapbuild.build_map_tables(smap)
     smap = synthmap.generate_map(
         meta["map_seed"], grid=tuple(meta["grid"]), sectors=meta["sectors"], linedefs=meta["linedefs"],
         midtex=meta.get("midtex", 0.0), layout=meta.get("layout", "grid"), islands=meta.get("islands", 0),

@@ -33,6 +33,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
 sys.path.insert(0, ROOT)
 sys.path.insert(0, HERE)
+sys.path.insert(0, os.path.dirname(HERE))
 
 import __graft_entry__ as entry  # noqa: E402
 
@@ -174,14 +175,34 @@ CASES = {
         map_seed=1004, grid=(21, 21), sectors=400, linedefs=4000, lanes=2, pose_seed=2, sprites=128, midtex=0.15, flash=True,
         variant=dict(seed=5, heights="uniform"),
     ),
+    # Sectors with the ceiling BELOW the floor, which no map of the reference holds: three seeds of the random-map tests
+    # (tests/random_cases.py), each the first found to show one way such a sector differs from an ordinary one.  Seen from a
+    # neighbour its wall tiers share rows (the four-column group's shade applies once either tier's common bottom is passed);
+    "inverted_shared_tier_rows": dict(recipe=dict(seed=70017, inverted=True, variants=False), lanes=16),
+    # seen from inside, the ceiling's and the floor's plane rows overlap;
+    "inverted_plane_rows_overlap": dict(recipe=dict(seed=80127, inverted=True, variants=True, eye_any=True), lanes=16),
+    # behind a window that a zero-height sector closed, its ceiling clip passes the floor clip and the silhouette over the
+    # rows between decides whether a billboard behind shows.
+    "inverted_clip_past_window": dict(recipe=dict(seed=503259, mixed=True, variants=True, eye_any=True), lanes=16),
 }
 
 
 def build_case(name: str, cfg: dict, do_time: bool) -> dict:
-    smap = synthmap.generate_map(
-        cfg["map_seed"], grid=cfg["grid"], sectors=cfg["sectors"], linedefs=cfg["linedefs"], midtex=cfg.get("midtex", 0.0),
-        layout=cfg.get("layout", "grid"), islands=cfg.get("islands", 0), pillars=cfg.get("pillars", 0),
-    )
+    recipe_parts = None
+    if cfg.get("recipe"):
+        # map, poses and billboards as tests/random_cases.py builds them (heights edited by hand, maybe a variant, split
+        # linedefs or blend tables on top); the billboards' patches are then whatever the reference's actors show
+        import random_cases
+
+        recipe = dict(cfg["recipe"])
+        recipe_parts = random_cases.closed_door_parts(recipe.pop("seed"), cfg["lanes"], **recipe)
+        smap = recipe_parts[0]
+        cfg = dict(cfg, flash=True, sectors=len(smap.sector_heights), linedefs=len(smap.wall_segments))
+    else:
+        smap = synthmap.generate_map(
+            cfg["map_seed"], grid=cfg["grid"], sectors=cfg["sectors"], linedefs=cfg["linedefs"], midtex=cfg.get("midtex", 0.0),
+            layout=cfg.get("layout", "grid"), islands=cfg.get("islands", 0), pillars=cfg.get("pillars", 0),
+        )
     base_digest = map_digest(smap)
     if cfg.get("variant"):
         smap = synthmap.with_variant(smap, **cfg["variant"])
@@ -197,12 +218,15 @@ def build_case(name: str, cfg: dict, do_time: bool) -> dict:
         actors=cfg.get("actors", 0),
     )
     ctor_seconds = time.time() - started
-    picks = cfg.get("picks") or [(cfg["pose_seed"], lane) for lane in range(lanes)]
-    assert len(picks) == lanes
-    poses = synthmap.generate_picked_poses(
-        smap, picks, pitch=cfg.get("pitch", False), flash=cfg.get("flash", False), margin=cfg.get("margin", 0.15),
-        eye=cfg.get("eye", "standing"),
-    )
+    if recipe_parts is not None:
+        poses = recipe_parts[1]
+    else:
+        picks = cfg.get("picks") or [(cfg["pose_seed"], lane) for lane in range(lanes)]
+        assert len(picks) == lanes
+        poses = synthmap.generate_picked_poses(
+            smap, picks, pitch=cfg.get("pitch", False), flash=cfg.get("flash", False), margin=cfg.get("margin", 0.15),
+            eye=cfg.get("eye", "standing"),
+        )
     refdrive.set_poses(engine, poses)
     offsets = hostmath.native_ray_offsets("cpu")
     assert torch.equal(offsets, engine._native_ray_offsets)
@@ -230,7 +254,13 @@ def build_case(name: str, cfg: dict, do_time: bool) -> dict:
         data["sprite_depth"] = hostmath.sprite_depth(
             engine.x, engine.y, engine.angle, torch.as_tensor(packed["sprite_x"]), torch.as_tensor(packed["sprite_y"])
         ).numpy()
-    if cfg.get("sprites", 0):
+    if recipe_parts is not None:
+        packed = refdrive.set_sprites(engine, recipe_parts[2], cfg["recipe"]["seed"])
+        data.update(packed)
+        data["sprite_depth"] = hostmath.sprite_depth(
+            engine.x, engine.y, engine.angle, torch.as_tensor(packed["sprite_x"]), torch.as_tensor(packed["sprite_y"])
+        ).numpy()
+    elif cfg.get("sprites", 0):
         sprites = synthmap.generate_sprites(smap, lanes, cfg["sprites"], cfg["pose_seed"])
         effects = synthmap.generate_sprites(smap, lanes, cfg["effects"], cfg["pose_seed"] + 50) if cfg.get("effects") else None
         packed = refdrive.set_sprites(engine, sprites, cfg["pose_seed"], effects)

@@ -10,11 +10,8 @@ import torch
 
 pytestmark = pytest.mark.gpu
 
-SHAPES = (
-    ("grid", (4, 3), 10, 60, 0, 0), ("grid", (5, 4), 17, 140, 4, 2), ("brick", (5, 4), 18, 170, 6, 0),
-    ("brick", (4, 3), 10, 90, 3, 2), ("grid", (6, 5), 26, 240, 10, 0), ("brick", (6, 5), 26, 260, 10, 3),
-    ("grid", (3, 3), 8, 80, 2, 1), ("brick", (3, 3), 8, 100, 2, 0),
-)
+from random_cases import SHAPES, closed_door_case  # noqa: E402,F401  (other test modules import corridor_case and this from here)
+
 LANES = 8
 
 
@@ -108,48 +105,6 @@ def test_random_maps_with_other_heights_and_textures_whatever_the_working_memory
             assert np.array_equal(indexed.cpu().numpy(), expected["indexed"]), f"seed {seed} fill {fill} {assembly}"
             assert np.array_equal(obs.cpu().numpy(), expected["obs"]), f"seed {seed} fill {fill} {assembly}"
         renderer.close()
-
-
-def closed_door_case(seed: int, lanes: int, *, inverted: bool = False, variants: bool = True, eye_any: bool = False, mixed: bool = False):
-    """random_case plus hand-closed doors and crawl spaces on up to four sectors (``inverted``: ceilings 16 units below
-    their floors instead; ``mixed``: each of the four one of the three kinds), then (``variants``: seven times in ten) other heights, texture sizes and lights over the whole
-    map; ``eye_any``: six times in ten the eyes stand at any height, not between their sector's floor and ceiling."""
-    from gradoom_amd import mapbuild, synthmap
-    from gradoom_amd.selfcheck import make_lane_arrays
-
-    rng = np.random.default_rng(seed)
-    layout, grid, sectors, linedefs, islands, pillars = SHAPES[seed % len(SHAPES)]
-    smap = synthmap.generate_map(seed, grid=grid, sectors=sectors, linedefs=linedefs, layout=layout, islands=islands, pillars=pillars,
-                                 midtex=float(rng.choice([0.0, 0.1, 0.3])))
-    if rng.random() < 0.7:
-        heights = np.array(smap.sector_heights, copy=True)
-        for sector in rng.choice(len(heights), size=min(4, len(heights)), replace=False):
-            kind = int(rng.choice([0, 2]))
-            if mixed:
-                kind = int(rng.integers(0, 3))
-            if inverted or kind == 1:
-                heights[sector, 1] = heights[sector, 0] - 16   # a ceiling below its floor
-            elif kind == 0:
-                heights[sector, 1] = heights[sector, 0]        # a closed door
-            else:
-                heights[sector, 0] = heights[sector, 1] - 8    # a crawl space
-        smap.sector_heights[...] = heights
-    if variants and rng.random() < 0.7:
-        smap = synthmap.with_variant(smap, seed + 9, heights=[None, "uniform", "doors"][int(rng.integers(0, 3))],
-                                     textures=[None, "mixed", "npot"][int(rng.integers(0, 3))], lights=bool(rng.random() < 0.5))
-    if rng.random() < 0.4:
-        smap = synthmap.split_linedefs(smap, seed + 1)
-    if rng.random() < 0.5:
-        smap = synthmap.with_blend_tables(smap, seed + 2)
-    margin = float(rng.choice([0.005, 0.02, 0.15]))
-    eye = {"eye": "any"} if eye_any and rng.random() < 0.6 else {}
-    poses = synthmap.generate_poses(smap, lanes, seed + 3, pitch=bool(rng.random() < 0.6), flash=bool(rng.random() < 0.5), margin=margin, **eye)
-    if rng.random() < 0.3:
-        poses.pitch_bam[:] = rng.integers(-30, 31, lanes) * (182 << 16)
-    sprites = synthmap.generate_sprites(smap, lanes, 24, seed + 4)
-    arrays = make_lane_arrays(smap, poses, sprites)
-    arrays["sprite_style"] = rng.choice(np.array([-1, -1, -1, -2, 0, 1], dtype=np.int8), size=sprites.x.shape)
-    return smap, mapbuild.build_map_tables(smap), arrays
 
 
 @pytest.mark.parametrize("seed", [50078, 50079, 50082])
