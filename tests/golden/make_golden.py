@@ -184,6 +184,11 @@ CASES = {
     # behind a window that a zero-height sector closed, its ceiling clip passes the floor clip and the silhouette over the
     # rows between decides whether a billboard behind shows.
     "inverted_clip_past_window": dict(recipe=dict(seed=503259, mixed=True, variants=True, eye_any=True), lanes=16),
+    # An 80-sector corridor seen end on: up to 85 linedefs in one column ray, more than a column of the HIP path keeps in
+    # its own list (the reference's dense loops have no list to overflow).
+    "corridor_80": dict(recipe=dict(kind="corridor", sectors=80), lanes=6),
+    # Cameras in the void beside the map: hardly a pixel that a wall pass claims, most flat rays unresolved.
+    "cameras_outside": dict(recipe=dict(kind="outside"), lanes=8),
 }
 
 
@@ -194,8 +199,7 @@ def build_case(name: str, cfg: dict, do_time: bool) -> dict:
         # linedefs or blend tables on top); the billboards' patches are then whatever the reference's actors show
         import random_cases
 
-        recipe = dict(cfg["recipe"])
-        recipe_parts = random_cases.closed_door_parts(recipe.pop("seed"), cfg["lanes"], **recipe)
+        recipe_parts = random_cases.build_parts(cfg["recipe"], cfg["lanes"])
         smap = recipe_parts[0]
         cfg = dict(cfg, flash=True, sectors=len(smap.sector_heights), linedefs=len(smap.wall_segments))
     else:
@@ -255,7 +259,7 @@ def build_case(name: str, cfg: dict, do_time: bool) -> dict:
             engine.x, engine.y, engine.angle, torch.as_tensor(packed["sprite_x"]), torch.as_tensor(packed["sprite_y"])
         ).numpy()
     if recipe_parts is not None:
-        packed = refdrive.set_sprites(engine, recipe_parts[2], cfg["recipe"]["seed"])
+        packed = refdrive.set_sprites(engine, recipe_parts[2], cfg["recipe"].get("seed", 1))
         data.update(packed)
         data["sprite_depth"] = hostmath.sprite_depth(
             engine.x, engine.y, engine.angle, torch.as_tensor(packed["sprite_x"]), torch.as_tensor(packed["sprite_y"])

@@ -62,3 +62,69 @@ def closed_door_case(seed: int, lanes: int, **options):
     arrays = make_lane_arrays(smap, poses, sprites)
     arrays["sprite_style"] = styles
     return smap, mapbuild.build_map_tables(smap), arrays
+
+
+def corridor_parts(lanes: int, sectors: int = 80):
+    """A corridor of `sectors` sectors and cameras in it that look along it, so that every divider lands in the same
+    screen columns: more linedefs per column ray than the 64 a column keeps in its own slots.  (map, poses, sprites)"""
+    from gradoom_amd import synthmap
+
+    smap = synthmap.generate_map(5, grid=(sectors, 1), sectors=sectors, linedefs=3 * sectors + 1, midtex=0.2)
+    poses = synthmap.generate_poses(smap, lanes, 11, pitch=True, flash=True)
+    rng = np.random.default_rng(3)
+    for lane in range(lanes):
+        sector = int(rng.integers(0, 8)) if lane % 2 == 0 else int(rng.integers(sectors - 8, sectors))   # either end, looking at the other
+        centre = smap.sector_quads[sector].mean(axis=0)
+        poses.x[lane], poses.y[lane] = float(centre[0]) + float(rng.uniform(-20, 20)), float(centre[1]) + float(rng.uniform(-20, 20))
+        poses.view_z[lane] = float(smap.sector_heights[sector, 0]) + 41.0
+        degrees = (0.0 if lane % 2 == 0 else 180.0) + float(rng.uniform(-12, 12))
+        poses.angle_bam[lane] = int(round(degrees / 360.0 * 4294967296.0)) & 0xFFFFFFFF
+    sprites = synthmap.generate_sprites(smap, lanes, 24, 12)
+    return smap, poses, sprites
+
+
+def corridor_case(lanes: int, sectors: int = 80):
+    """corridor_parts as (map, derived tables, lane arrays)."""
+    from gradoom_amd import mapbuild
+    from gradoom_amd.selfcheck import make_lane_arrays
+
+    smap, poses, sprites = corridor_parts(lanes, sectors)
+    return smap, mapbuild.build_map_tables(smap), make_lane_arrays(smap, poses, sprites)
+
+
+def outside_parts(lanes: int):
+    """Cameras in the void beside a small map, 8 to 200 units off one of its four sides, looking wherever the generator
+    turned them: no wall pass claims most of the screen.  (map, poses, sprites)"""
+    from gradoom_amd import synthmap
+
+    smap = synthmap.generate_map(7001, grid=(5, 4), sectors=17, linedefs=140, layout="grid", islands=4, pillars=2, midtex=0.1)
+    poses = synthmap.generate_poses(smap, lanes, 11, pitch=True)
+    segments = np.asarray(smap.wall_segments, dtype=np.float64)
+    low = np.array([segments[:, [0, 2]].min(), segments[:, [1, 3]].min()])
+    high = np.array([segments[:, [0, 2]].max(), segments[:, [1, 3]].max()])
+    rng = np.random.default_rng(5)
+    for lane in range(lanes):
+        along, away = rng.uniform(0.1, 0.9), rng.uniform(8, 200)
+        side = lane % 4
+        if side < 2:
+            poses.x[lane] = low[0] - away if side == 0 else high[0] + away
+            poses.y[lane] = low[1] + along * (high[1] - low[1])
+        else:
+            poses.x[lane] = low[0] + along * (high[0] - low[0])
+            poses.y[lane] = low[1] - away if side == 2 else high[1] + away
+    sprites = synthmap.generate_sprites(smap, lanes, 24, 12)
+    return smap, poses, sprites
+
+
+def build_parts(recipe: dict, lanes: int):
+    """(map, poses, sprites) of a recipe as the golden fixtures name it: {"kind": "closed_door" (the default) | "corridor"
+    | "outside", ...the builder's own arguments}."""
+    recipe = dict(recipe)
+    kind = recipe.pop("kind", "closed_door")
+    if kind == "closed_door":
+        return closed_door_parts(recipe.pop("seed"), lanes, **recipe)[:3]
+    if kind == "corridor":
+        return corridor_parts(lanes, **recipe)
+    if kind == "outside":
+        return outside_parts(lanes, **recipe)
+    raise ValueError(f"unknown recipe kind {kind!r}")

@@ -10,7 +10,7 @@ import torch
 
 pytestmark = pytest.mark.gpu
 
-from random_cases import SHAPES, closed_door_case  # noqa: E402,F401  (other test modules import corridor_case and this from here)
+from random_cases import SHAPES, closed_door_case, corridor_case, outside_parts  # noqa: E402,F401  (other test modules import corridor_case from here)
 
 LANES = 8
 
@@ -196,26 +196,6 @@ def test_a_ceiling_clip_carried_below_the_floor_clip_still_records_its_silhouett
     renderer.close()
 
 
-def corridor_case(lanes: int, sectors: int = 80):
-    """A corridor of `sectors` sectors and cameras in it that look along it, so that every divider lands in the same
-    screen columns: more linedefs per column ray than the 64 a column keeps in its own slots."""
-    from gradoom_amd import mapbuild, synthmap
-    from gradoom_amd.selfcheck import make_lane_arrays
-
-    smap = synthmap.generate_map(5, grid=(sectors, 1), sectors=sectors, linedefs=3 * sectors + 1, midtex=0.2)
-    poses = synthmap.generate_poses(smap, lanes, 11, pitch=True, flash=True)
-    rng = np.random.default_rng(3)
-    for lane in range(lanes):
-        sector = int(rng.integers(0, 8)) if lane % 2 == 0 else int(rng.integers(sectors - 8, sectors))   # either end, looking at the other
-        centre = smap.sector_quads[sector].mean(axis=0)
-        poses.x[lane], poses.y[lane] = float(centre[0]) + float(rng.uniform(-20, 20)), float(centre[1]) + float(rng.uniform(-20, 20))
-        poses.view_z[lane] = float(smap.sector_heights[sector, 0]) + 41.0
-        degrees = (0.0 if lane % 2 == 0 else 180.0) + float(rng.uniform(-12, 12))
-        poses.angle_bam[lane] = int(round(degrees / 360.0 * 4294967296.0)) & 0xFFFFFFFF
-    sprites = synthmap.generate_sprites(smap, lanes, 24, 12)
-    return smap, mapbuild.build_map_tables(smap), make_lane_arrays(smap, poses, sprites)
-
-
 @pytest.mark.parametrize("sectors", [80, 124])
 def test_columns_that_see_more_than_64_linedefs_match_the_oracle(oracle, sectors):
     """Such columns get a slot in the spill pool, where every linedef their ray can reach is listed (the reference keeps a
@@ -252,23 +232,9 @@ def test_cameras_outside_the_map_match_the_oracle(oracle):
     from gradoom_amd.selfcheck import make_lane_arrays
 
     cosine = hostmath.cosine_correction("cpu").numpy()
-    smap = synthmap.generate_map(7001, grid=(5, 4), sectors=17, linedefs=140, layout="grid", islands=4, pillars=2, midtex=0.1)
+    smap, poses, sprites = outside_parts(LANES)
     tables = mapbuild.build_map_tables(smap)
-    poses = synthmap.generate_poses(smap, LANES, 11, pitch=True)
-    segments = np.asarray(smap.wall_segments, dtype=np.float64)
-    low = np.array([segments[:, [0, 2]].min(), segments[:, [1, 3]].min()])
-    high = np.array([segments[:, [0, 2]].max(), segments[:, [1, 3]].max()])
-    rng = np.random.default_rng(5)
-    for lane in range(LANES):
-        along, away = rng.uniform(0.1, 0.9), rng.uniform(8, 200)
-        side = lane % 4
-        if side < 2:
-            poses.x[lane] = low[0] - away if side == 0 else high[0] + away
-            poses.y[lane] = low[1] + along * (high[1] - low[1])
-        else:
-            poses.x[lane] = low[0] + along * (high[0] - low[0])
-            poses.y[lane] = low[1] - away if side == 2 else high[1] + away
-    sprites = synthmap.generate_sprites(smap, LANES, 24, 12)
+    rng = np.random.default_rng(6)
     arrays = make_lane_arrays(smap, poses, sprites)
     renderer = HipRenderer(smap, LANES, "cuda:0", cosine_correction=cosine, tables=tables)
     # Billboards over pixels that show the flat pass's picture, three ways: no styles at all (every lane's billboards are
