@@ -189,6 +189,12 @@ CASES = {
     "corridor_80": dict(recipe=dict(kind="corridor", sectors=80), lanes=6),
     # Cameras in the void beside the map: hardly a pixel that a wall pass claims, most flat rays unresolved.
     "cameras_outside": dict(recipe=dict(kind="outside"), lanes=8),
+    # Seed 50078 of the random-map tests, lanes 7 and 14: a column loses its sector, picks a linedef beyond a projected solid
+    # and takes that path's clips, which close the window over rows that no drawseg painted or claimed.
+    "portal_path_clip_closes_window": dict(recipe=dict(seed=50078), lanes=16),
+    # Billboards in awkward places: at the eye, a step from it, on vertices and linedefs, far outside the map, lifted or
+    # sunk.  No two at exactly the same depth: among those the reference's order is torch.topk's, which is not defined.
+    "awkward_billboards": dict(recipe=dict(kind="awkward_billboards", seed=1200007, ties=False), lanes=16),
 }
 
 

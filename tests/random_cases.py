@@ -116,13 +116,62 @@ def outside_parts(lanes: int):
     return smap, poses, sprites
 
 
+def awkward_billboard_parts(seed: int, lanes: int, ties: bool = True):
+    """closed_door_parts with its billboards moved to awkward places: exact depth ties with an earlier slot, at the eye,
+    within a few units of it, far outside the map, on a vertex, on a linedef, lifted or sunk.  (map, poses, sprites)
+
+    ``ties=False`` leaves out what puts two billboards at exactly the same depth (a shared spot, a second billboard at the
+    eye).  The reference paints the billboards of a column in the order ``torch.topk`` returns them
+    (``engine.py:14768-14780``), which among equal depths is whatever that routine's partial sort leaves: its CPU build
+    paints five billboards at one spot in slot order in 319 columns of a frame and in another order in the 320th.  The
+    oracle and the HIP path paint equal depths in slot order; only cases without ties can be compared with the reference."""
+    smap, poses, sprites, _styles = closed_door_parts(seed, lanes, mixed=True, eye_any=True)
+    rng = np.random.default_rng(seed * 13 + 5)
+    segments = np.asarray(smap.wall_segments, dtype=np.float32)
+    vertices = segments.reshape(-1, 2)
+    for lane in range(lanes):
+        at_the_eye = 0
+        for slot in range(sprites.x.shape[1]):
+            kind = int(rng.integers(0, 12))
+            if kind == 0:
+                sprites.z[lane, slot] += np.float32(rng.uniform(-60, 140))
+            elif kind == 1 and slot > 0:
+                other = int(rng.integers(0, slot))
+                moved = bool(rng.random() < 0.5)
+                lift = np.float32(rng.integers(-16, 17))
+                if ties:
+                    sprites.x[lane, slot], sprites.y[lane, slot] = sprites.x[lane, other], sprites.y[lane, other]
+                    if moved:
+                        sprites.z[lane, slot] = sprites.z[lane, other] + lift
+            elif kind == 2:
+                if ties or at_the_eye == 0:
+                    sprites.x[lane, slot], sprites.y[lane, slot] = poses.x[lane], poses.y[lane]
+                at_the_eye += 1
+            elif kind == 3:
+                angle, reach = float(rng.uniform(0, 6.283)), float(rng.choice([0.01, 0.5, 2.0, 6.0]))
+                sprites.x[lane, slot] = poses.x[lane] + np.float32(reach * np.cos(angle))
+                sprites.y[lane, slot] = poses.y[lane] + np.float32(reach * np.sin(angle))
+            elif kind == 4:
+                sprites.x[lane, slot] += np.float32(rng.uniform(-3000, 3000))
+                sprites.y[lane, slot] += np.float32(rng.uniform(-3000, 3000))
+            elif kind == 5:
+                sprites.x[lane, slot], sprites.y[lane, slot] = vertices[int(rng.integers(0, len(vertices)))]
+            elif kind == 6:
+                wall, along = segments[int(rng.integers(0, len(segments)))], np.float32(rng.random())
+                sprites.x[lane, slot] = wall[0] + along * (wall[2] - wall[0])
+                sprites.y[lane, slot] = wall[1] + along * (wall[3] - wall[1])
+    return smap, poses, sprites
+
+
 def build_parts(recipe: dict, lanes: int):
-    """(map, poses, sprites) of a recipe as the golden fixtures name it: {"kind": "closed_door" (the default) | "corridor"
-    | "outside", ...the builder's own arguments}."""
+    """(map, poses, sprites) of a recipe as the golden fixtures name it: {"kind": "closed_door" (the default) | "awkward_billboards" |
+    "corridor" | "outside", ...the builder's own arguments}."""
     recipe = dict(recipe)
     kind = recipe.pop("kind", "closed_door")
     if kind == "closed_door":
         return closed_door_parts(recipe.pop("seed"), lanes, **recipe)[:3]
+    if kind == "awkward_billboards":
+        return awkward_billboard_parts(recipe.pop("seed"), lanes, **recipe)
     if kind == "corridor":
         return corridor_parts(lanes, **recipe)
     if kind == "outside":

@@ -10,7 +10,7 @@ import torch
 
 pytestmark = pytest.mark.gpu
 
-from random_cases import SHAPES, closed_door_case, corridor_case, outside_parts  # noqa: E402,F401  (other test modules import corridor_case from here)
+from random_cases import SHAPES, awkward_billboard_parts, closed_door_case, corridor_case, outside_parts  # noqa: E402,F401  (other test modules import corridor_case from here)
 
 LANES = 8
 
@@ -181,6 +181,37 @@ def test_a_ceiling_clip_carried_below_the_floor_clip_still_records_its_silhouett
     smap, tables, arrays = closed_door_case(503259, lanes, mixed=True, variants=True, eye_any=True)
     heights = np.asarray(smap.sector_heights)
     assert (heights[:, 1] < heights[:, 0]).any() and (heights[:, 1] == heights[:, 0]).any()
+    expected = oracle.render(tables, arrays, cosine)
+    renderer = HipRenderer(smap, lanes, "cuda:0", cosine_correction=cosine, tables=tables)
+    state = LaneState.from_numpy(arrays, "cuda:0")
+    for assembly in ("separate", "fused"):
+        renderer.set_assembly(assembly)
+        indexed = torch.zeros((lanes, 240, 320), dtype=torch.uint8, device="cuda:0")
+        obs = torch.zeros((lanes, 84, 84), dtype=torch.uint8, device="cuda:0")
+        renderer.render(state, indexed=indexed, obs=obs)
+        torch.cuda.synchronize()
+        assert renderer.status() == 0
+        assert np.array_equal(indexed.cpu().numpy(), expected["indexed"]), assembly
+        assert np.array_equal(obs.cpu().numpy(), expected["obs"]), assembly
+    renderer.close()
+
+
+@pytest.mark.parametrize("seed", [1200007, 1200011, 1200018])
+def test_billboards_in_awkward_places_match_the_oracle(oracle, seed):
+    """Billboards at exactly the same depth (the oracle and the HIP path paint those in slot order; the reference's order
+    among them is torch.topk's and not defined), at the eye, a step from it, on vertices and linedefs, far outside the map,
+    lifted or sunk, some of them blending with what is under them."""
+    from gradoom_amd import hostmath, mapbuild
+    from gradoom_amd.renderer import HipRenderer, LaneState
+    from gradoom_amd.selfcheck import make_lane_arrays
+
+    lanes = 16
+    cosine = hostmath.cosine_correction("cpu").numpy()
+    smap, poses, sprites = awkward_billboard_parts(seed, lanes)
+    tables = mapbuild.build_map_tables(smap)
+    arrays = make_lane_arrays(smap, poses, sprites)
+    arrays["sprite_style"] = np.random.default_rng(seed).choice(np.array([-1, -1, -2, 0, 1], dtype=np.int8), size=sprites.x.shape)
+    arrays["sprite_style"][::2] = -1    # every other lane's billboards all plain: painted beside the flat pass
     expected = oracle.render(tables, arrays, cosine)
     renderer = HipRenderer(smap, lanes, "cuda:0", cosine_correction=cosine, tables=tables)
     state = LaneState.from_numpy(arrays, "cuda:0")
