@@ -1477,7 +1477,9 @@ struct Oracle {
                 if (inside && s.alive && (s.depth > 0) && ray_visible) order[count++] = a;
             }
             if (!count) continue;
-            // topk(largest=False, sorted=True): ascending depth; ties keep slot order
+            // topk(largest=False, sorted=True): ascending depth.  Among exactly equal depths the reference's order is
+            // whatever torch.topk's partial sort leaves (it varies from column to column of one frame); here, and in the
+            // HIP path, equal depths keep slot order.
             std::stable_sort(order.begin(), order.begin() + count, [&](int a, int b) { return sp[a].depth < sp[b].depth; });
             for (int layer = count - 1; layer >= 0; --layer) {
                 const Spr &s = sp[order[layer]];
