@@ -1,6 +1,6 @@
 """Compare the CPU oracle with the reference's own Torch CPU render path on seeded random cases (build container only).
 
-Usage:  python tests/golden/reference_sweep.py FIRST_SEED COUNT [doors|billboards] [--keep]
+Usage:  python tests/golden/reference_sweep.py FIRST_SEED COUNT [doors|billboards|layers] [--keep]
 
 Each case is a recipe of ``tests/random_cases.py`` (8 lanes), rendered by the reference through ``make_golden.build_case``
 and by the oracle from the same lane inputs.  Indexed frames must be equal and observations within one, the bar of
@@ -39,18 +39,26 @@ def main() -> int:
     differing = 0
     for seed in range(first, first + count):
         rng = np.random.default_rng(seed)
-        if kind == "doors":
+        layers = {}
+        if kind in ("doors", "layers"):
             recipe = dict(seed=seed, mixed=True, variants=True, eye_any=True, inverted=bool(rng.random() < 0.3))
+            if kind == "layers":   # weapon, status bar and bullet chips over the view, projectiles and puffs that blend
+                layers = dict(overlays=seed % 50 + 1, decals=seed % 97 + 1, effects=24)
         else:
             recipe = dict(kind="awkward_billboards", seed=seed, ties=False)
         try:
-            data = make_golden.build_case(f"sweep_{seed}", dict(recipe=recipe, lanes=LANES), False)
+            data = make_golden.build_case(f"sweep_{seed}", dict(recipe=recipe, lanes=LANES, **layers), False)
         except ValueError as error:   # a map the pose generator refuses
             print("seed", seed, "skipped:", error, flush=True)
             continue
         tables = mapbuild.build_map_tables(random_cases.build_parts(recipe, LANES)[0])
         arrays = conftest.lane_inputs(data)
+        if layers:
+            from gradoom_amd import synthmap
+
+            oracle.set_overlays(synthmap.generate_overlays(layers["overlays"]))
         result = oracle.render(tables, arrays, data["cosine_correction"])
+        oracle.set_overlays(None)
         tied = np.zeros(LANES, dtype=bool)
         for lane in range(LANES):
             depths = arrays["sprite_depth"][lane][arrays["sprite_alive"][lane] != 0]
