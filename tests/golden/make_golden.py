@@ -264,7 +264,7 @@ def build_case(name: str, cfg: dict, do_time: bool) -> dict:
         data["sprite_depth"] = hostmath.sprite_depth(
             engine.x, engine.y, engine.angle, torch.as_tensor(packed["sprite_x"]), torch.as_tensor(packed["sprite_y"])
         ).numpy()
-    if recipe_parts is not None:
+    if recipe_parts is not None and not cfg.get("actors"):
         effects = synthmap.generate_sprites(smap, lanes, cfg["effects"], cfg["recipe"].get("seed", 1) + 50) if cfg.get("effects") else None
         packed = refdrive.set_sprites(engine, recipe_parts[2], cfg["recipe"].get("seed", 1), effects)
         data.update(packed)

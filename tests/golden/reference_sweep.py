@@ -1,6 +1,6 @@
 """Compare the CPU oracle with the reference's own Torch CPU render path on seeded random cases (build container only).
 
-Usage:  python tests/golden/reference_sweep.py FIRST_SEED COUNT [doors|billboards|layers] [--keep]
+Usage:  python tests/golden/reference_sweep.py FIRST_SEED COUNT [doors|billboards|layers|actors] [--keep]
 
 Each case is a recipe of ``tests/random_cases.py`` (8 lanes), rendered by the reference through ``make_golden.build_case``
 and by the oracle from the same lane inputs.  Indexed frames must be equal and observations within one, the bar of
@@ -40,10 +40,12 @@ def main() -> int:
     for seed in range(first, first + count):
         rng = np.random.default_rng(seed)
         layers = {}
-        if kind in ("doors", "layers"):
+        if kind in ("doors", "layers", "actors"):
             recipe = dict(seed=seed, mixed=True, variants=True, eye_any=True, inverted=bool(rng.random() < 0.3))
             if kind == "layers":   # weapon, status bar and bullet chips over the view, projectiles and puffs that blend
                 layers = dict(overlays=seed % 50 + 1, decals=seed % 97 + 1, effects=24)
+            if kind == "actors":   # every kind of actor from randomised gameplay tensors, packed by actor_inputs.pack_actors
+                layers = dict(actors=seed % 1000 + 1)
         else:
             recipe = dict(kind="awkward_billboards", seed=seed, ties=False)
         try:
@@ -53,7 +55,7 @@ def main() -> int:
             continue
         tables = mapbuild.build_map_tables(random_cases.build_parts(recipe, LANES)[0])
         arrays = conftest.lane_inputs(data)
-        if layers:
+        if layers.get("overlays"):
             from gradoom_amd import synthmap
 
             oracle.set_overlays(synthmap.generate_overlays(layers["overlays"]))
