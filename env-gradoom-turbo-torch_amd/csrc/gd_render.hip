@@ -5356,8 +5356,9 @@ static int check_render_args(gd_renderer *r, const gd_lanes_desc *lanes, const g
     if (out->obs_source_rows != 0 && out->obs_source_rows != VH && out->obs_source_rows != GD_SCREEN_HEIGHT)
         return fail(GD_E_ARG, "obs_source_rows must be 208 (or 0) or 240");
     if (lanes->lane_count < 0) return fail(GD_E_ARG, "negative lane count");
-    if (!lanes->x || !lanes->y || !lanes->angle || !lanes->view_z || !lanes->x_fixed || !lanes->y_fixed || !lanes->angle_bam ||
-        !lanes->pitch_bam || !lanes->ray_cos || !lanes->ray_sin)
+    // an empty batch is a call that does nothing: its tensors hold no element and may have no address
+    if (lanes->lane_count > 0 && (!lanes->x || !lanes->y || !lanes->angle || !lanes->view_z || !lanes->x_fixed || !lanes->y_fixed ||
+                                  !lanes->angle_bam || !lanes->pitch_bam || !lanes->ray_cos || !lanes->ray_sin))
         return fail(GD_E_ARG, "missing lane tensor");
     if (out->stack_mode != GD_STACK_STEP && out->stack_mode != GD_STACK_RESET) return fail(GD_E_ARG, "unknown stack_mode");
     if (lanes->sprite_slots < 0 || lanes->sprite_slots > 512) return fail(GD_E_ARG, "sprite_slots must be in [0, 512]");
@@ -5535,11 +5536,12 @@ int gd_renderer_set_sector_lights(gd_renderer *r, const float *lights, void *str
 
 int gd_observe(const uint8_t *indexed, int32_t source_rows, const uint8_t *playpal, int32_t lane_count,
                uint8_t *obs, uint8_t *frames, const uint8_t *reset_mask, int32_t stack_mode, void *stream) {
-    if (!indexed || !playpal) return fail(GD_E_ARG, "null argument");
     if (stack_mode != GD_STACK_STEP && stack_mode != GD_STACK_RESET) return fail(GD_E_ARG, "unknown stack_mode");
     if (source_rows != 208 && source_rows != 240) return fail(GD_E_ARG, "indexed must have 208 or 240 rows");
     if (lane_count < 0) return fail(GD_E_ARG, "negative lane count");
-    if (lane_count == 0 || (!obs && !frames)) return GD_OK;
+    if (lane_count == 0) return GD_OK;    // an empty batch: its tensors may have no address
+    if (!indexed || !playpal) return fail(GD_E_ARG, "null argument");
+    if (!obs && !frames) return GD_OK;
     for (int base = 0; base < lane_count; base += 32768) {
         int count = lane_count - base < 32768 ? lane_count - base : 32768;
         const size_t F = (size_t)GD_OBS_SIZE * GD_OBS_SIZE;
@@ -5553,10 +5555,10 @@ int gd_observe(const uint8_t *indexed, int32_t source_rows, const uint8_t *playp
 }
 
 int gd_expand_rgb24(const uint8_t *indexed, int32_t rows, const uint8_t *playpal, int32_t lane_count, uint8_t *rgb, void *stream) {
-    if (!indexed || !playpal || !rgb) return fail(GD_E_ARG, "null argument");
     if (rows <= 0 || lane_count < 0) return fail(GD_E_ARG, "bad shape");
     size_t pixels = (size_t)lane_count * rows * SW;
-    if (pixels == 0) return GD_OK;
+    if (pixels == 0) return GD_OK;        // an empty batch: its tensors may have no address
+    if (!indexed || !playpal || !rgb) return fail(GD_E_ARG, "null argument");
     const size_t step = (size_t)1 << 30;
     for (size_t base = 0; base < pixels; base += step) {
         size_t count = pixels - base < step ? pixels - base : step;

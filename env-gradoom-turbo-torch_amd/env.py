@@ -185,6 +185,7 @@ class GraDoomVecEnv:
         )
         self._safe_obs_index = 0
         self._seed_values = [None] * n
+        self._deferred_actions = None   # the one-element tuple step_async leaves for step_wait
         self._reset_rngs = [np.random.default_rng() for _ in range(n)]
 
     # ------------------------------------------------------------------ helpers
@@ -348,6 +349,18 @@ class GraDoomVecEnv:
         transition = self._step(indices, view, self.obs_layout)
         observations = transition.observations if view is None else view
         return observations, transition.rewards, transition.terminated, transition.truncated, {}
+
+    def step_async(self, actions: torch.Tensor) -> None:  # env.py:839-842
+        """Hand in the actions of a step that ``step_wait`` will run; nothing is checked or rendered yet."""
+        if self._deferred_actions is not None:
+            raise RuntimeError("an asynchronous step is already pending")
+        self._deferred_actions = (actions,)
+
+    def step_wait(self):  # env.py:844-849
+        if self._deferred_actions is None:
+            raise RuntimeError("no asynchronous step is pending")
+        (actions,), self._deferred_actions = self._deferred_actions, None
+        return self.step(actions)
 
     # ------------------------------------------------------------------ RGB frames
     def _rgb_frames(self, lane: int | None = None) -> torch.Tensor:

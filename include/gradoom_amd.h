@@ -156,7 +156,7 @@ typedef struct gd_map_desc {
  */
 typedef struct gd_lanes_desc {
     uint32_t struct_size;    /* sizeof(gd_lanes_desc) of the header the caller was built with */
-    int32_t lane_count;       /* N */
+    int32_t lane_count;       /* N; 0 is allowed: the call checks its arguments and does nothing */
     int32_t sprite_slots;     /* A sprites per lane (0 = none) */
     int32_t decal_slots;      /* D packed wall decals per lane (0 = none) */
     const float *x, *y;       /* [N] */

@@ -268,3 +268,25 @@ def test_render_lane_renders_only_the_lane_asked_for():
     assert shapes[-1] == (1,) and frame.shape == (240, 320, 3)
     assert int(frame[0, 0, 0]) == int(state.x[2].abs().to(torch.int64) % 251)
     assert len(env.get_images()) == 4 and shapes[-1] == (4,)
+
+
+def test_deferred_step_runs_when_waited_for(env):
+    # tests/test_turbo_api_contract.py:345-347 and env.py:839-849: one step may be pending; waiting without one is an error
+    env.reset(seed=5)
+    with pytest.raises(RuntimeError, match="no asynchronous step is pending"):
+        env.step_wait()
+    calls = len(env._renderer.calls)
+    env.step_async(torch.zeros(4, dtype=torch.int64))
+    assert len(env._renderer.calls) == calls   # nothing rendered yet
+    with pytest.raises(RuntimeError, match="already pending"):
+        env.step_async(torch.zeros(4, dtype=torch.int64))
+    transition = env.step_wait()
+    assert len(env._renderer.calls) == calls + 1
+    assert all(isinstance(value, torch.Tensor) for value in transition[:4]) and transition[0].shape == (4, 4, 84, 84)
+    with pytest.raises(RuntimeError, match="no asynchronous step is pending"):
+        env.step_wait()
+    env.step_async(torch.zeros(4))   # a bad argument is refused when the step runs, and leaves nothing pending
+    with pytest.raises(TypeError, match="actions must have dtype"):
+        env.step_wait()
+    env.step_async(torch.zeros(4, dtype=torch.int64))
+    env.step_wait()

@@ -119,6 +119,42 @@ def test_chunked_batches_render_every_lane_like_the_golden():
         renderer.close()
 
 
+def test_empty_single_lane_and_billboard_free_batches(oracle):
+    # the ragged ends of the input domain: a batch of no lanes (the call does nothing and writes nothing), one lane on its
+    # own, lanes whose billboards are all dead, and the same lanes handed over without any billboard tensor
+    import dataclasses
+
+    meta, data, tables, renderer, lanes = _renderer("small_midtex_sprites")
+    count = meta["lanes"]
+    arrays = lane_inputs(data)
+    none = lanes.select(slice(0, 0))
+    guard = torch.full((1, 240, 320), 7, dtype=torch.uint8, device="cuda:0")
+    for call in (renderer.render, renderer.render_static):
+        call(none, indexed=guard[:0], obs=torch.empty((0, 84, 84), dtype=torch.uint8, device="cuda:0"),
+             frames=torch.empty((0, 4, 84, 84), dtype=torch.uint8, device="cuda:0"))
+    renderer.observe(guard[:0, :208], obs=torch.empty((0, 84, 84), dtype=torch.uint8, device="cuda:0"))
+    torch.cuda.synchronize()
+    assert renderer.status() == 0 and bool((guard == 7).all())
+    for lane in (0, count - 1):
+        indexed = torch.zeros((1, 240, 320), dtype=torch.uint8, device="cuda:0")
+        renderer.render(lanes.select(slice(lane, lane + 1)), indexed=indexed)
+        assert np.array_equal(indexed.cpu().numpy(), data["indexed"][lane:lane + 1])
+    dead = dict(arrays, sprite_alive=np.zeros_like(arrays["sprite_alive"]))
+    expected = oracle.render(tables, dead, data["cosine_correction"])
+    indexed = torch.zeros((count, 240, 320), dtype=torch.uint8, device="cuda:0")
+    obs = torch.zeros((count, 84, 84), dtype=torch.uint8, device="cuda:0")
+    bare = {f.name: None for f in dataclasses.fields(lanes) if f.name.startswith("sprite_")}
+    for variant in (dataclasses.replace(lanes, sprite_alive=torch.zeros_like(lanes.sprite_alive)), dataclasses.replace(lanes, **bare)):
+        for assembly in ("separate", "fused"):
+            renderer.set_assembly(assembly)
+            indexed.zero_()
+            obs.zero_()
+            renderer.render(variant, indexed=indexed, obs=obs)
+            assert np.array_equal(indexed.cpu().numpy(), expected["indexed"]), assembly
+            assert np.array_equal(obs.cpu().numpy(), expected["obs"]), assembly
+    renderer.close()
+
+
 def test_final_frames_and_stack_modes_match_the_oracle(oracle):
     # the three ways a call leaves the stack (step; step with some lanes reset; reset of the masked lanes only), each
     # against the oracle's stack, with the fused final-observation clone (env.py:915-917) equal to it
