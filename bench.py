@@ -59,8 +59,8 @@ def algorithmic_bytes_per_lane_frame(sprites: int, map_bytes: int, lanes: int, m
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
-    parser.add_argument("--steps", type=int, default=10)
-    parser.add_argument("--warmup", type=int, default=2)
+    parser.add_argument("--steps", type=int, default=100)
+    parser.add_argument("--warmup", type=int, default=20)
     parser.add_argument("--repeats", type=int, default=5, help="timed repeats of --steps steps each; the median is reported")
     parser.add_argument("--workload", default="config4")
     parser.add_argument("--heights", choices=("uniform", "quantised"), default="uniform",
