@@ -3757,7 +3757,9 @@ __device__ __forceinline__ void sprite_paint(const DeviceMap &dm, const gd_lanes
         float light = s.light + (float)(L.flash_light * 16);
         if (s.flags & 2) light = 255.0f;
         float base_shade = 61.0f - light / 4.0f;
-        float visibility = fminf(1280.0f / fmaxf(s.depth, 1.0f), 24.0f);
+        // engine.py:10583 divides a Python number by a tensor, which Torch evaluates as reciprocal(distance) * 1280
+        // (Tensor.__rtruediv__): two roundings, not one division
+        float visibility = fminf((1.0f / fmaxf(s.depth, 1.0f)) * 1280.0f, 24.0f);
         i64 shade = clampi((i64)floorf(base_shade - visibility), 0, 31);
         const i64 fraction_base = s.fraction_base;
         const int y_lo = max((int)((unsigned)s.flags >> 16) & 255, row_first), y_hi = min((int)((unsigned)s.flags >> 24), row_end);
@@ -3951,7 +3953,8 @@ __global__ void __launch_bounds__(SW) decal_kernel(DeviceMap dm, Overlays ov, gd
         i64 tu = clampi((i64)floorf(decal_along * (float)width), 0, width - 1);
         if (flip_x) tu = width - 1 - tu;
         const float safe_distance = fmaxf(distance, 1e-6f);
-        const float vertical_scale = 96.0f / safe_distance;
+        // engine.py:13909 divides a Python number by a tensor: reciprocal(distance) * 96 in Torch (Tensor.__rtruediv__)
+        const float vertical_scale = (1.0f / safe_distance) * 96.0f;
         const float top = center - ((impact_z + (float)o.decal_top[variant] * 0.5f) - L.view_z) * 192.0f / safe_distance;
         int sector = m->wall_sectors[2 * wall_index + (side > 1 ? 1 : side)];
         if (sector < 0) sector = 0;

@@ -1490,7 +1490,9 @@ struct Oracle {
                 if (s.fullbright) light = 255.0f;
                 // engine.py:10576-10586 (float shade)
                 float base_shade = 61.0f - light / 4.0f;
-                float visibility = std::min(1280.0f / std::max(s.depth, 1.0f), 24.0f);
+                // `1280.0 / distance` divides a Python number by a tensor: Torch evaluates it as reciprocal(distance) * 1280
+                // (Tensor.__rtruediv__), two roundings, not one division
+                float visibility = std::min((1.0f / std::max(s.depth, 1.0f)) * 1280.0f, 24.0f);
                 i64 shade = clampi((i64)std::floor(base_shade - visibility), 0, 31);
                 for (int y = 0; y < VH; ++y) {
                     size_t i = size_t(y) * SW + x;
@@ -1596,7 +1598,9 @@ void render_decals(Oracle &o, const gd_overlay_desc &ov, const gd_lanes_desc *la
             i64 tu = clampi(i64(std::floor(decal_along * float(width))), 0, width - 1);
             if (flip_x) tu = width - 1 - tu;
             float safe_distance = std::max(distance, 1e-6f);
-            float vertical_scale = 96.0f / safe_distance;
+            // `focal_length * _BULLET_DECAL_SCALE / distance` divides a Python number by a tensor, which Torch evaluates as
+            // reciprocal(distance) * 96 (Tensor.__rtruediv__): two roundings, not one division
+            float vertical_scale = (1.0f / safe_distance) * 96.0f;
             float top = center - ((impact_z + top_offset * 0.5f) - L.view_z) * focal_length / safe_distance;
             i64 depth_fixed = round_to_i64(safe_distance * 4096.0f);
             i64 visibility = tdiv(WALL_VISIBILITY_FIXED << 12, std::max<i64>(depth_fixed, 1));

@@ -195,6 +195,11 @@ CASES = {
     # Billboards in awkward places: at the eye, a step from it, on vertices and linedefs, far outside the map, lifted or
     # sunk.  No two at exactly the same depth: among those the reference's order is torch.topk's, which is not defined.
     "awkward_billboards": dict(recipe=dict(kind="awkward_billboards", seed=1200007, ties=False), lanes=16),
+    # Seed 7045 of reference_sweep.py's layers kind: a bullet chip on a wall eight units from the eye whose texel row
+    # boundary falls on a screen row, (y - top) / vertical_scale a rounding step from a whole number in lane 3.  The
+    # reference's `96.0 / distance` is a Python number over a tensor, which Torch evaluates as reciprocal(distance) * 96.
+    "decal_row_on_a_rounding_step": dict(recipe=dict(seed=7045, mixed=True, variants=True, eye_any=True, inverted=False), lanes=8,
+                                         overlays=46, decals=62, effects=24),
 }
 
 
